@@ -1,0 +1,229 @@
+// Shared device and host helpers for the gfx950 axis-primitive kernels.
+//
+// Everything here assumes CDNA4: 64-lane wavefronts, DPP row operations and
+// row broadcasts, 160 KB of LDS per compute unit.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/dlfx.h"
+
+namespace dlfx {
+
+constexpr int kWave = 64;
+constexpr int kMaxRank = DLFX_MAX_RANK;
+
+// ------------------------------------------------------------------ views
+// A group of merged dimensions: flat index -> element offset by a div/mod walk
+// from the innermost extent outwards.  rank 0 maps every index to 0.
+struct DimMap {
+    int rank;
+    int64_t dims[kMaxRank];
+    int64_t strides[kMaxRank];
+
+    __host__ __device__ int64_t at(int64_t flat) const {
+        if (rank == 1) return flat * strides[0];
+        int64_t off = 0;
+        for (int i = rank - 1; i > 0; --i) {
+            int64_t d = dims[i];
+            int64_t q = flat / d;
+            off += (flat - q * d) * strides[i];
+            flat = q;
+        }
+        if (rank > 0) off += flat * strides[0];
+        return off;
+    }
+    __host__ __device__ int64_t size() const {
+        int64_t s = 1;
+        for (int i = 0; i < rank; ++i) s *= dims[i];
+        return s;
+    }
+};
+
+// Host side: copy dims [b, e) of a view into a DimMap, dropping extent-1
+// dimensions and merging neighbours that walk memory as one dimension.
+// Returns false when more than kMaxRank dimensions remain.
+inline bool make_dim_map(const int64_t* dims, const int64_t* strides, int b, int e, DimMap* out) {
+    int r = 0;
+    int64_t d[64], s[64];
+    for (int i = b; i < e; ++i) {
+        if (dims[i] == 1) continue;
+        if (r > 0 && s[r - 1] == strides[i] * dims[i]) {
+            d[r - 1] *= dims[i];
+            s[r - 1] = strides[i];
+        } else {
+            if (r == 64) return false;
+            d[r] = dims[i];
+            s[r] = strides[i];
+            ++r;
+        }
+    }
+    if (r > kMaxRank) return false;
+    out->rank = r;
+    for (int i = 0; i < kMaxRank; ++i) {
+        out->dims[i] = i < r ? d[i] : 1;
+        out->strides[i] = i < r ? s[i] : 0;
+    }
+    return true;
+}
+
+// ------------------------------------------------------------------ bit casts / DPP
+template <typename To, typename From>
+__device__ __forceinline__ To bit_cast(const From& f) {
+    static_assert(sizeof(To) == sizeof(From), "size mismatch");
+    return __builtin_bit_cast(To, f);
+}
+
+template <int N>
+struct Words {
+    int w[N];
+};
+
+// Value of `v` in the lane the DPP control selects; lanes whose source is
+// outside the row (or masked off by ROW_MASK) receive `fill`.
+template <int CTRL, int ROW_MASK = 0xf, typename T>
+__device__ __forceinline__ T dpp_fetch(T v, T fill) {
+    static_assert(sizeof(T) % 4 == 0, "whole 32-bit words only");
+    constexpr int N = sizeof(T) / 4;
+    Words<N> a = bit_cast<Words<N>>(v), f = bit_cast<Words<N>>(fill), r;
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+        r.w[i] = __builtin_amdgcn_update_dpp(f.w[i], a.w[i], CTRL, ROW_MASK, 0xf, false);
+    return bit_cast<T>(r);
+}
+
+template <typename T>
+__device__ __forceinline__ T lane_xor(T v, int mask) {
+    constexpr int N = sizeof(T) / 4;
+    Words<N> a = bit_cast<Words<N>>(v);
+#pragma unroll
+    for (int i = 0; i < N; ++i) a.w[i] = __shfl_xor(a.w[i], mask, kWave);
+    return bit_cast<T>(a);
+}
+
+template <typename T>
+__device__ __forceinline__ T lane_get(T v, int lane) {
+    constexpr int N = sizeof(T) / 4;
+    Words<N> a = bit_cast<Words<N>>(v);
+#pragma unroll
+    for (int i = 0; i < N; ++i) a.w[i] = __shfl(a.w[i], lane, kWave);
+    return bit_cast<T>(a);
+}
+
+// Broadcast of one lane's value through a scalar register (lane is uniform).
+template <typename T>
+__device__ __forceinline__ T lane_read(T v, int lane) {
+    constexpr int N = sizeof(T) / 4;
+    Words<N> a = bit_cast<Words<N>>(v);
+#pragma unroll
+    for (int i = 0; i < N; ++i) a.w[i] = __builtin_amdgcn_readlane(a.w[i], lane);
+    return bit_cast<T>(a);
+}
+
+// DPP controls used below.
+constexpr int kQuadXor1 = 0xB1;      // quad_perm [1,0,3,2]
+constexpr int kQuadXor2 = 0x4E;      // quad_perm [2,3,0,1]
+constexpr int kRowHalfMirror = 0x141;
+constexpr int kRowMirror = 0x140;
+constexpr int kRowShr1 = 0x111, kRowShr2 = 0x112, kRowShr4 = 0x114, kRowShr8 = 0x118;
+constexpr int kRowBcast15 = 0x142, kRowBcast31 = 0x143;
+
+// All-lanes reduction over a wavefront with a commutative `join`.
+template <typename T, typename Join>
+__device__ __forceinline__ T wave_reduce(T v, Join join) {
+    v = join(v, dpp_fetch<kQuadXor1>(v, v));
+    v = join(v, dpp_fetch<kQuadXor2>(v, v));
+    v = join(v, dpp_fetch<kRowHalfMirror>(v, v));
+    v = join(v, dpp_fetch<kRowMirror>(v, v));
+    v = join(v, lane_xor(v, 16));
+    v = join(v, lane_xor(v, 32));
+    return v;
+}
+
+// Reduction over aligned groups of `width` lanes (power of two, <= 64); every
+// lane of a group ends with the group's result.
+template <typename T, typename Join>
+__device__ __forceinline__ T group_reduce(T v, int width, Join join) {
+    if (width > 1) v = join(v, dpp_fetch<kQuadXor1>(v, v));
+    if (width > 2) v = join(v, dpp_fetch<kQuadXor2>(v, v));
+    if (width > 4) v = join(v, dpp_fetch<kRowHalfMirror>(v, v));
+    if (width > 8) v = join(v, dpp_fetch<kRowMirror>(v, v));
+    if (width > 16) v = join(v, lane_xor(v, 16));
+    if (width > 32) v = join(v, lane_xor(v, 32));
+    return v;
+}
+
+// Inclusive scan over a wavefront: lane i receives op(v0, ..., vi) with the
+// operands in lane order.  `id` is the operator's identity.
+template <typename T, typename Op>
+__device__ __forceinline__ T wave_scan_inclusive(T v, T id, Op op) {
+    v = op(dpp_fetch<kRowShr1>(v, id), v);
+    v = op(dpp_fetch<kRowShr2>(v, id), v);
+    v = op(dpp_fetch<kRowShr4>(v, id), v);
+    v = op(dpp_fetch<kRowShr8>(v, id), v);
+    v = op(dpp_fetch<kRowBcast15, 0xa>(v, id), v);
+    v = op(dpp_fetch<kRowBcast31, 0xc>(v, id), v);
+    return v;
+}
+
+__device__ __forceinline__ int lane_id() { return __lane_id(); }
+
+// ------------------------------------------------------------------ vectors
+template <typename T, int N>
+struct alignas(sizeof(T) * N) Vec {
+    T v[N];
+};
+
+// Elements per 128-bit load.
+template <typename T>
+constexpr int vec_width() { return 16 / sizeof(T); }
+
+// ------------------------------------------------------------------ host launch helpers
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Records a HIP failure for dlfx_last_hip_error and returns DLFX_ERR_LAUNCH.
+int record_hip_error(hipError_t e);
+
+#define DLFX_CHECK_LAUNCH()                                      \
+    do {                                                         \
+        hipError_t e_ = hipGetLastError();                       \
+        if (e_ != hipSuccess) return dlfx::record_hip_error(e_); \
+    } while (0)
+
+// Common argument validation for a strided view.
+inline bool view_ok(int rank, const int64_t* dims, const int64_t* strides) {
+    if (rank < 0 || rank > 64) return false;
+    if (rank > 0 && (!dims || !strides)) return false;
+    for (int i = 0; i < rank; ++i)
+        if (dims[i] <= 0) return false;
+    return true;
+}
+
+inline int64_t view_size(int rank, const int64_t* dims) {
+    int64_t s = 1;
+    for (int i = 0; i < rank; ++i) s *= dims[i];
+    return s;
+}
+
+template <typename F>
+inline int dispatch_dtype(int dtype, F&& f) {
+    switch (dtype) {
+    case DLFX_F32: return f(float());
+    case DLFX_F64: return f(double());
+    case DLFX_I32: return f(int32_t());
+    case DLFX_I64: return f(int64_t());
+    default: return DLFX_ERR_UNSUPPORTED_DTYPE;
+    }
+}
+
+inline size_t dtype_size(int dtype) {
+    switch (dtype) {
+    case DLFX_F32: case DLFX_I32: return 4;
+    case DLFX_F64: case DLFX_I64: return 8;
+    default: return 0;
+    }
+}
+
+}  // namespace dlfx

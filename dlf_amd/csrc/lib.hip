@@ -1,0 +1,31 @@
+// Library-level entry points: version, status text, last HIP error.
+#include "common.hip.h"
+
+namespace dlfx {
+
+static thread_local int g_last_hip_error = 0;
+
+int record_hip_error(hipError_t e) {
+    g_last_hip_error = static_cast<int>(e);
+    return DLFX_ERR_LAUNCH;
+}
+
+}  // namespace dlfx
+
+extern "C" int dlfx_version(void) { return 100; }
+
+extern "C" int dlfx_last_hip_error(void) { return dlfx::g_last_hip_error; }
+
+extern "C" const char* dlfx_status_string(int status) {
+    switch (status) {
+    case DLFX_OK: return "ok";
+    case DLFX_ERR_INVALID_ARGUMENT: return "invalid argument";
+    case DLFX_ERR_UNSUPPORTED_DTYPE: return "unsupported element type for this operation";
+    case DLFX_ERR_UNKNOWN_OP: return "unknown operation name";
+    case DLFX_ERR_SCRATCH_TOO_SMALL: return "scratch buffer too small";
+    case DLFX_ERR_RANK: return "view rank exceeds DLFX_MAX_RANK";
+    case DLFX_ERR_LAUNCH: return "HIP launch failed";
+    case DLFX_ERR_TOO_LARGE: return "extent too large for this kernel";
+    default: return "unknown status";
+    }
+}

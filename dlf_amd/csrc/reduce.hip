@@ -1,0 +1,573 @@
+// reduce / arg_reduce over strided views for gfx950.
+//
+// Three row shapes get their own kernels:
+//   * rows whose reduced elements are contiguous in memory: 128-bit loads, a
+//     group of 1..64 lanes per row (short rows), or one or more 256-thread
+//     workgroups per row (long rows) with a small second stage;
+//   * reductions across a strided axis while a kept axis is contiguous
+//     ("columns"): lanes run along the contiguous kept axis so every load
+//     instruction is a contiguous 256-byte segment, four waves split the
+//     reduced axis and combine through LDS;
+//   * anything else: the row kernels with per-element address computation.
+// All of them are bandwidth bound; fp32 sums accumulate in fp64 registers.
+#include <cmath>
+#include <cstring>
+#include <limits>
+#include <type_traits>
+
+#include "common.hip.h"
+
+namespace dlfx {
+namespace {
+
+enum JoinKind { kAdd = 0, kMul = 1, kMax = 2, kMin = 3 };
+enum MapKind { kMapId = 0, kMapExp = 1, kMapAbs = 2, kMapSquare = 3 };
+enum FinalKind { kFinalId = 0, kFinalMean = 1, kFinalLog = 2, kFinalSqrt = 3 };
+
+constexpr int kBlock = 256;
+
+template <typename T, int J>
+struct AccType { using type = T; };
+template <> struct AccType<float, kAdd> { using type = double; };
+template <> struct AccType<float, kMul> { using type = double; };
+
+template <typename T>
+__device__ __forceinline__ T wrap_add(T a, T b) {
+    if constexpr (std::is_integral<T>::value) {
+        using U = typename std::make_unsigned<T>::type;
+        return static_cast<T>(static_cast<U>(a) + static_cast<U>(b));
+    } else {
+        return a + b;
+    }
+}
+template <typename T>
+__device__ __forceinline__ T wrap_mul(T a, T b) {
+    if constexpr (std::is_integral<T>::value) {
+        using U = typename std::make_unsigned<T>::type;
+        return static_cast<T>(static_cast<U>(a) * static_cast<U>(b));
+    } else {
+        return a * b;
+    }
+}
+
+// Map -> fold -> Final of the reducer table (dlf/include/tensor/xfn.h:661-805).
+template <typename T, int J, int M>
+struct ValueReducer {
+    using in_t = T;
+    using acc_t = typename AccType<T, J>::type;
+    using out_t = T;
+
+    __device__ static __forceinline__ acc_t identity() {
+        if constexpr (J == kAdd) return acc_t(0);
+        else if constexpr (J == kMul) return acc_t(1);
+        else if constexpr (J == kMax) return (M == kMapAbs) ? acc_t(0) : std::numeric_limits<T>::lowest();
+        else return std::numeric_limits<T>::max();
+    }
+    __device__ static __forceinline__ acc_t map(T x, int64_t) {
+        if constexpr (M == kMapExp) {
+            if constexpr (std::is_same<T, float>::value) return static_cast<acc_t>(expf(x));
+            else return static_cast<acc_t>(exp(static_cast<double>(x)));
+        } else if constexpr (M == kMapAbs) {
+            if constexpr (std::is_integral<T>::value) {
+                using U = typename std::make_unsigned<T>::type;
+                return x < 0 ? static_cast<T>(U(0) - static_cast<U>(x)) : x;
+            } else {
+                return static_cast<acc_t>(x < 0 ? -x : x);
+            }
+        } else if constexpr (M == kMapSquare) {
+            acc_t v = static_cast<acc_t>(x);
+            return wrap_mul(v, v);
+        } else {
+            return static_cast<acc_t>(x);
+        }
+    }
+    __device__ static __forceinline__ acc_t join(acc_t a, acc_t b) {
+        if constexpr (J == kAdd) return wrap_add(a, b);
+        else if constexpr (J == kMul) return wrap_mul(a, b);
+        else if constexpr (J == kMax) return (a < b) ? b : a;
+        else return (b < a) ? b : a;
+    }
+    __device__ static __forceinline__ out_t finish(acc_t a, int64_t n, int final_op) {
+        if constexpr (std::is_integral<T>::value) {
+            if (final_op == kFinalMean) return static_cast<T>(a / static_cast<T>(n));
+            return static_cast<T>(a);
+        } else {
+            double v = static_cast<double>(a);
+            if (final_op == kFinalMean) v = v / static_cast<double>(n);
+            else if (final_op == kFinalLog) v = log(v);
+            else if (final_op == kFinalSqrt) v = sqrt(v);
+            return static_cast<T>(v);
+        }
+    }
+};
+
+template <typename T>
+struct ArgAcc {
+    T v;
+    int32_t i;
+};
+
+// argmax / argmin with the serial loop's semantics
+// (dlf/include/tensor/reduce_detail.h:107-132): strict comparison, so the first
+// occurrence wins; a NaN in position 0 is never displaced, a NaN elsewhere
+// never wins.
+template <typename T, bool MAX, typename I>
+struct ArgReducer {
+    using in_t = T;
+    using acc_t = ArgAcc<T>;
+    using out_t = I;
+
+    __device__ static __forceinline__ acc_t identity() {
+        return {MAX ? std::numeric_limits<T>::lowest() : std::numeric_limits<T>::max(),
+                std::numeric_limits<int32_t>::max()};
+    }
+    __device__ static __forceinline__ acc_t map(T x, int64_t j) {
+        if constexpr (!std::is_integral<T>::value) {
+            if (x != x) {
+                if (j == 0)
+                    return {MAX ? std::numeric_limits<T>::infinity() : -std::numeric_limits<T>::infinity(), -1};
+                return identity();
+            }
+        }
+        return {x, static_cast<int32_t>(j)};
+    }
+    __device__ static __forceinline__ acc_t join(acc_t a, acc_t b) {
+        bool take_b = MAX ? (b.v > a.v) : (b.v < a.v);
+        take_b = take_b || (b.v == a.v && b.i < a.i);
+        return take_b ? b : a;
+    }
+    __device__ static __forceinline__ out_t finish(acc_t a, int64_t, int) {
+        return static_cast<I>(a.i < 0 ? 0 : a.i);
+    }
+};
+
+// --------------------------------------------------------------------------
+// One row's contiguous elements, visited by `width` cooperating lanes (lane
+// `g` of the group) restricted to 128-bit vectors [v_lo, v_hi) of the aligned
+// body; with_head / with_tail add the unaligned ends of the row.
+template <typename R>
+__device__ __forceinline__ typename R::acc_t
+row_partial_contig(const typename R::in_t* __restrict__ p, int64_t n, int g, int width,
+                   int64_t part, int64_t parts) {
+    using T = typename R::in_t;
+    using acc_t = typename R::acc_t;
+    constexpr int V = vec_width<T>();
+    using VecT = Vec<T, V>;
+
+    acc_t acc = R::identity();
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(p) / sizeof(T);
+    int64_t head = (V - static_cast<int64_t>(addr % V)) % V;
+    if (head > n) head = n;
+    const int64_t nv = (n - head) / V;
+    const int64_t tail_start = head + nv * V;
+
+    const int64_t per = (nv + parts - 1) / parts;
+    const int64_t v_lo = part * per;
+    const int64_t v_hi = (v_lo + per < nv) ? v_lo + per : nv;
+
+    const VecT* __restrict__ pv = reinterpret_cast<const VecT*>(p + head);
+    int64_t v = v_lo + g;
+    // four independent 128-bit loads in flight per lane
+    for (; v + 3 * static_cast<int64_t>(width) < v_hi; v += 4 * static_cast<int64_t>(width)) {
+        VecT a = pv[v], b = pv[v + width], c = pv[v + 2 * width], d = pv[v + 3 * width];
+        const int64_t j0 = head + v * V;
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(a.v[e], j0 + e));
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(b.v[e], j0 + static_cast<int64_t>(width) * V + e));
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(c.v[e], j0 + 2 * static_cast<int64_t>(width) * V + e));
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(d.v[e], j0 + 3 * static_cast<int64_t>(width) * V + e));
+    }
+    for (; v < v_hi; v += width) {
+        VecT a = pv[v];
+        const int64_t j0 = head + v * V;
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(a.v[e], j0 + e));
+    }
+    if (part == 0)
+        for (int64_t j = g; j < head; j += width) acc = R::join(acc, R::map(p[j], j));
+    if (part == parts - 1)
+        for (int64_t j = tail_start + g; j < n; j += width) acc = R::join(acc, R::map(p[j], j));
+    return acc;
+}
+
+template <typename R>
+__device__ __forceinline__ typename R::acc_t
+row_partial_strided(const typename R::in_t* __restrict__ p, const DimMap& red, int64_t n, int g,
+                    int width, int64_t part, int64_t parts) {
+    typename R::acc_t acc = R::identity();
+    const int64_t per = (n + parts - 1) / parts;
+    const int64_t lo = part * per;
+    const int64_t hi = (lo + per < n) ? lo + per : n;
+    for (int64_t j = lo + g; j < hi; j += width) acc = R::join(acc, R::map(p[red.at(j)], j));
+    return acc;
+}
+
+// Short rows: 2^log2g lanes per row, 256 >> log2g rows per workgroup.
+template <typename R, bool CONTIG>
+__global__ __launch_bounds__(kBlock) void reduce_rows_group(
+    const typename R::in_t* __restrict__ x, DimMap kept, DimMap red, int64_t m, int64_t n, int log2g,
+    typename R::out_t* __restrict__ y, DimMap ymap, int final_op) {
+    const int width = 1 << log2g;
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * (kBlock >> log2g) + (threadIdx.x >> log2g);
+    const int g = threadIdx.x & (width - 1);
+    typename R::acc_t acc = R::identity();
+    if (row < m) {
+        const typename R::in_t* p = x + kept.at(row);
+        if constexpr (CONTIG) acc = row_partial_contig<R>(p, n, g, width, 0, 1);
+        else acc = row_partial_strided<R>(p, red, n, g, width, 0, 1);
+    }
+    acc = group_reduce(acc, width, [](typename R::acc_t a, typename R::acc_t b) { return R::join(a, b); });
+    if (row < m && g == 0) y[ymap.at(row)] = R::finish(acc, n, final_op);
+}
+
+template <typename R>
+__device__ __forceinline__ typename R::acc_t block_reduce(typename R::acc_t acc) {
+    using acc_t = typename R::acc_t;
+    __shared__ acc_t sm[kBlock / kWave];
+    acc = wave_reduce(acc, [](acc_t a, acc_t b) { return R::join(a, b); });
+    const int w = threadIdx.x / kWave;
+    if (lane_id() == 0) sm[w] = acc;
+    __syncthreads();
+    acc_t r = sm[0];
+#pragma unroll
+    for (int i = 1; i < kBlock / kWave; ++i) r = R::join(r, sm[i]);
+    return r;
+}
+
+// Long rows: `parts` workgroups per row.  parts == 1 writes the result,
+// otherwise each workgroup leaves one partial accumulator in `partial`.
+template <typename R, bool CONTIG>
+__global__ __launch_bounds__(kBlock) void reduce_rows_block(
+    const typename R::in_t* __restrict__ x, DimMap kept, DimMap red, int64_t n, int64_t parts,
+    typename R::out_t* __restrict__ y, DimMap ymap, int final_op,
+    typename R::acc_t* __restrict__ partial) {
+    const int64_t row = blockIdx.x / parts;
+    const int64_t part = blockIdx.x - row * parts;
+    const typename R::in_t* p = x + kept.at(row);
+    typename R::acc_t acc;
+    if constexpr (CONTIG) acc = row_partial_contig<R>(p, n, threadIdx.x, kBlock, part, parts);
+    else acc = row_partial_strided<R>(p, red, n, threadIdx.x, kBlock, part, parts);
+    acc = block_reduce<R>(acc);
+    if (threadIdx.x == 0) {
+        if (parts == 1) y[ymap.at(row)] = R::finish(acc, n, final_op);
+        else partial[blockIdx.x] = acc;
+    }
+}
+
+// Second stage: one wave per row folds that row's `parts` partials.
+template <typename R>
+__global__ __launch_bounds__(kBlock) void reduce_finalize(
+    const typename R::acc_t* __restrict__ partial, int64_t m, int64_t n, int64_t parts,
+    typename R::out_t* __restrict__ y, DimMap ymap, int final_op) {
+    using acc_t = typename R::acc_t;
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + threadIdx.x / kWave;
+    acc_t acc = R::identity();
+    if (row < m)
+        for (int64_t i = lane_id(); i < parts; i += kWave) acc = R::join(acc, partial[row * parts + i]);
+    acc = wave_reduce(acc, [](acc_t a, acc_t b) { return R::join(a, b); });
+    if (row < m && lane_id() == 0) y[ymap.at(row)] = R::finish(acc, n, final_op);
+}
+
+// Columns: kept axis of extent L is contiguous, lanes run along it; the four
+// waves of a workgroup take reduced indices ty, ty+4, ... of slice `part`.
+template <typename R>
+__global__ __launch_bounds__(kBlock) void reduce_cols(
+    const typename R::in_t* __restrict__ x, DimMap outer, int64_t L, DimMap red, int64_t n,
+    int64_t col_blocks, int64_t parts, typename R::out_t* __restrict__ y, DimMap ymap, int final_op,
+    typename R::acc_t* __restrict__ partial) {
+    using acc_t = typename R::acc_t;
+    constexpr int TY = kBlock / kWave;
+    __shared__ acc_t sm[TY][kWave];
+    const int lx = threadIdx.x & (kWave - 1);
+    const int ty = threadIdx.x / kWave;
+    int64_t b = blockIdx.x;
+    const int64_t part = b % parts;
+    b /= parts;
+    const int64_t cb = b % col_blocks;
+    const int64_t o = b / col_blocks;
+    const int64_t c = cb * kWave + lx;
+
+    const int64_t per = (n + parts - 1) / parts;
+    const int64_t lo = part * per;
+    const int64_t hi = (lo + per < n) ? lo + per : n;
+
+    acc_t acc = R::identity();
+    if (c < L) {
+        const typename R::in_t* __restrict__ p = x + outer.at(o) + c;
+        if (red.rank == 1) {
+            const int64_t s = red.strides[0];
+            int64_t j = lo + ty;
+            for (; j + 7 * TY < hi; j += 8 * TY) {
+                typename R::in_t v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = p[(j + u * TY) * s];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) acc = R::join(acc, R::map(v[u], j + u * TY));
+            }
+            for (; j < hi; j += TY) acc = R::join(acc, R::map(p[j * s], j));
+        } else {
+            for (int64_t j = lo + ty; j < hi; j += TY) acc = R::join(acc, R::map(p[red.at(j)], j));
+        }
+    }
+    sm[ty][lx] = acc;
+    __syncthreads();
+    if (ty == 0 && c < L) {
+#pragma unroll
+        for (int i = 1; i < TY; ++i) acc = R::join(acc, sm[i][lx]);
+        const int64_t row = o * L + c;
+        if (parts == 1) y[ymap.at(row)] = R::finish(acc, n, final_op);
+        else partial[row * parts + part] = acc;
+    }
+}
+
+// --------------------------------------------------------------------------
+// Host-side planning.
+
+struct ReducePlan {
+    DimMap kept, red, ymap;
+    int64_t m, n;
+};
+
+int next_pow2_log(int64_t v) {
+    int l = 0;
+    while ((int64_t(1) << l) < v) ++l;
+    return l;
+}
+
+// Workgroups per row for the long-row kernel; a function of (m, n) only so the
+// scratch query and the launch agree.
+int64_t row_parts(int64_t m, int64_t n) {
+    if (m >= 1024) return 1;
+    int64_t want = ceil_div(2048, m);
+    int64_t cap = n / 16384;
+    if (cap < 1) cap = 1;
+    return want < cap ? want : cap;
+}
+
+int64_t col_parts(int64_t base_blocks, int64_t n) {
+    if (base_blocks >= 1024) return 1;
+    int64_t want = ceil_div(2048, base_blocks);
+    int64_t cap = n / 64;
+    if (cap < 1) cap = 1;
+    return want < cap ? want : cap;
+}
+
+size_t partial_bound_bytes(int64_t m) {
+    if (m >= 65536) return 0;
+    return static_cast<size_t>(m + 133120) * 16;
+}
+
+template <typename R>
+int launch_reduce(hipStream_t stream, const ReducePlan& pl, const typename R::in_t* x,
+                  typename R::out_t* y, int final_op, void* scratch, size_t scratch_bytes) {
+    using acc_t = typename R::acc_t;
+    using T = typename R::in_t;
+    const int64_t m = pl.m, n = pl.n;
+    acc_t* partial = static_cast<acc_t*>(scratch);
+
+    const bool contig = pl.red.rank == 0 || (pl.red.rank == 1 && pl.red.strides[0] == 1);
+    const bool cols = !contig && pl.kept.rank >= 1 && pl.kept.strides[pl.kept.rank - 1] == 1 &&
+                      pl.kept.dims[pl.kept.rank - 1] >= 16;
+
+    if (cols) {
+        DimMap outer = pl.kept;
+        const int64_t L = outer.dims[outer.rank - 1];
+        outer.rank -= 1;
+        outer.dims[outer.rank] = 1;
+        outer.strides[outer.rank] = 0;
+        const int64_t col_blocks = ceil_div(L, kWave);
+        const int64_t base_blocks = (m / L) * col_blocks;
+        const int64_t parts = col_parts(base_blocks, n);
+        if (base_blocks * parts > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+        if (parts > 1 && scratch_bytes < static_cast<size_t>(m * parts) * sizeof(acc_t))
+            return DLFX_ERR_SCRATCH_TOO_SMALL;
+        reduce_cols<R><<<dim3(static_cast<unsigned>(base_blocks * parts)), dim3(kBlock), 0, stream>>>(
+            x, outer, L, pl.red, n, col_blocks, parts, y, pl.ymap, final_op, partial);
+        DLFX_CHECK_LAUNCH();
+        if (parts > 1) {
+            reduce_finalize<R><<<dim3(static_cast<unsigned>(ceil_div(m, kBlock / kWave))), dim3(kBlock), 0, stream>>>(
+                partial, m, n, parts, y, pl.ymap, final_op);
+            DLFX_CHECK_LAUNCH();
+        }
+        return DLFX_OK;
+    }
+
+    const int64_t short_limit = 8192;
+    if (n <= short_limit) {
+        const int per_lane = contig ? vec_width<T>() * 4 : 8;
+        int log2g = next_pow2_log(ceil_div(n, per_lane));
+        if (log2g > 6) log2g = 6;
+        const int64_t blocks = ceil_div(m, kBlock >> log2g);
+        if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+        if (contig)
+            reduce_rows_group<R, true><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
+                x, pl.kept, pl.red, m, n, log2g, y, pl.ymap, final_op);
+        else
+            reduce_rows_group<R, false><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
+                x, pl.kept, pl.red, m, n, log2g, y, pl.ymap, final_op);
+        DLFX_CHECK_LAUNCH();
+        return DLFX_OK;
+    }
+
+    const int64_t parts = row_parts(m, n);
+    if (m * parts > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+    if (parts > 1 && scratch_bytes < static_cast<size_t>(m * parts) * sizeof(acc_t))
+        return DLFX_ERR_SCRATCH_TOO_SMALL;
+    if (contig)
+        reduce_rows_block<R, true><<<dim3(static_cast<unsigned>(m * parts)), dim3(kBlock), 0, stream>>>(
+            x, pl.kept, pl.red, n, parts, y, pl.ymap, final_op, partial);
+    else
+        reduce_rows_block<R, false><<<dim3(static_cast<unsigned>(m * parts)), dim3(kBlock), 0, stream>>>(
+            x, pl.kept, pl.red, n, parts, y, pl.ymap, final_op, partial);
+    DLFX_CHECK_LAUNCH();
+    if (parts > 1) {
+        reduce_finalize<R><<<dim3(static_cast<unsigned>(ceil_div(m, kBlock / kWave))), dim3(kBlock), 0, stream>>>(
+            partial, m, n, parts, y, pl.ymap, final_op);
+        DLFX_CHECK_LAUNCH();
+    }
+    return DLFX_OK;
+}
+
+struct ReduceOp {
+    const char* name;
+    int join, map, final_op;
+    bool float_only;
+};
+
+const ReduceOp kReduceOps[] = {
+    {"reduce_sum", kAdd, kMapId, kFinalId, false},
+    {"reduce_mean", kAdd, kMapId, kFinalMean, false},
+    {"reduce_max", kMax, kMapId, kFinalId, false},
+    {"reduce_min", kMin, kMapId, kFinalId, false},
+    {"reduce_log_sum_exp", kAdd, kMapExp, kFinalLog, true},
+    {"reduce_sum_exp", kAdd, kMapExp, kFinalId, true},
+    {"reduce_log_sum", kAdd, kMapId, kFinalLog, true},
+    {"reduce_prod", kMul, kMapId, kFinalId, false},
+    {"reduce_asum", kAdd, kMapAbs, kFinalId, false},
+    {"reduce_sum_square", kAdd, kMapSquare, kFinalId, false},
+    {"reduce_nrm2", kAdd, kMapSquare, kFinalSqrt, true},
+    {"reduce_amax", kMax, kMapAbs, kFinalId, false},
+    {"reduce_amin", kMin, kMapAbs, kFinalId, false},
+};
+
+template <typename T>
+int launch_reduce_typed(hipStream_t stream, const ReduceOp& op, const ReducePlan& pl, const T* x, T* y,
+                        void* scratch, size_t scratch_bytes) {
+#define DLFX_CASE(J, M)                                                                       \
+    if (op.join == J && op.map == M)                                                          \
+        return launch_reduce<ValueReducer<T, J, M>>(stream, pl, x, y, op.final_op, scratch, scratch_bytes);
+    DLFX_CASE(kAdd, kMapId)
+    DLFX_CASE(kAdd, kMapAbs)
+    DLFX_CASE(kAdd, kMapSquare)
+    DLFX_CASE(kMul, kMapId)
+    DLFX_CASE(kMax, kMapId)
+    DLFX_CASE(kMin, kMapId)
+    DLFX_CASE(kMax, kMapAbs)
+    DLFX_CASE(kMin, kMapAbs)
+    if constexpr (!std::is_integral<T>::value) {
+        DLFX_CASE(kAdd, kMapExp)
+    }
+#undef DLFX_CASE
+    return DLFX_ERR_UNKNOWN_OP;
+}
+
+}  // namespace
+}  // namespace dlfx
+
+using namespace dlfx;
+
+extern "C" size_t dlfx_reduce_scratch_bytes(int dtype, int64_t m, int64_t n) {
+    (void)dtype;
+    (void)n;
+    if (m <= 0) return 0;
+    return partial_bound_bytes(m);
+}
+
+extern "C" int dlfx_reduce(dlfx_stream_t stream, const char* name, int dtype, int64_t m, int64_t n,
+                           int x_rank, const int64_t* x_dims, const int64_t* x_strides,
+                           const void* x, int64_t x_offset,
+                           int y_rank, const int64_t* y_dims, const int64_t* y_strides,
+                           void* y, int64_t y_offset, void* scratch, size_t scratch_bytes) {
+    if (!name || !x || !y || m <= 0 || n <= 0) return DLFX_ERR_INVALID_ARGUMENT;
+    if (!view_ok(x_rank, x_dims, x_strides) || !view_ok(y_rank, y_dims, y_strides))
+        return DLFX_ERR_INVALID_ARGUMENT;
+    if (view_size(x_rank, x_dims) != m * n || view_size(y_rank, y_dims) != m) return DLFX_ERR_INVALID_ARGUMENT;
+    const ReduceOp* op = nullptr;
+    for (const auto& o : kReduceOps)
+        if (!std::strcmp(o.name, name)) op = &o;
+    if (!op) return DLFX_ERR_UNKNOWN_OP;
+    if (op->float_only && (dtype == DLFX_I32 || dtype == DLFX_I64)) return DLFX_ERR_UNSUPPORTED_DTYPE;
+
+    // the reduced extents are the trailing dimensions whose product is n
+    int split = x_rank;
+    int64_t prod = 1;
+    while (split > 0 && prod < n) prod *= x_dims[--split];
+    if (prod != n) return DLFX_ERR_INVALID_ARGUMENT;
+
+    ReducePlan pl;
+    pl.m = m;
+    pl.n = n;
+    if (!make_dim_map(x_dims, x_strides, 0, split, &pl.kept) ||
+        !make_dim_map(x_dims, x_strides, split, x_rank, &pl.red) ||
+        !make_dim_map(y_dims, y_strides, 0, y_rank, &pl.ymap))
+        return DLFX_ERR_RANK;
+
+    return dispatch_dtype(dtype, [&](auto tag) {
+        using T = decltype(tag);
+        return launch_reduce_typed<T>(static_cast<hipStream_t>(stream), *op, pl,
+                                      static_cast<const T*>(x) + x_offset, static_cast<T*>(y) + y_offset,
+                                      scratch, scratch_bytes);
+    });
+}
+
+extern "C" size_t dlfx_arg_reduce_scratch_bytes(int dtype, int64_t n_rows, int64_t k) {
+    (void)dtype;
+    (void)k;
+    if (n_rows <= 0) return 0;
+    return partial_bound_bytes(n_rows);
+}
+
+extern "C" int dlfx_arg_reduce(dlfx_stream_t stream, const char* name, int dtype, int index_dtype,
+                               int64_t n_rows, int64_t k,
+                               int x_rank, const int64_t* x_dims, const int64_t* x_strides,
+                               const void* x, int64_t x_offset,
+                               int y_rank, const int64_t* y_dims, const int64_t* y_strides,
+                               void* y, int64_t y_offset, void* scratch, size_t scratch_bytes) {
+    if (!name || !x || !y || n_rows <= 0 || k <= 0) return DLFX_ERR_INVALID_ARGUMENT;
+    if (!view_ok(x_rank, x_dims, x_strides) || !view_ok(y_rank, y_dims, y_strides))
+        return DLFX_ERR_INVALID_ARGUMENT;
+    if (x_rank < 1 || x_dims[x_rank - 1] != k) return DLFX_ERR_INVALID_ARGUMENT;
+    if (view_size(x_rank, x_dims) != n_rows * k || view_size(y_rank, y_dims) != n_rows)
+        return DLFX_ERR_INVALID_ARGUMENT;
+    if (k > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+    bool want_max;
+    if (!std::strcmp(name, "argmax")) want_max = true;
+    else if (!std::strcmp(name, "argmin")) want_max = false;
+    else return DLFX_ERR_UNKNOWN_OP;
+    if (index_dtype != DLFX_I32 && index_dtype != DLFX_I64) return DLFX_ERR_UNSUPPORTED_DTYPE;
+
+    ReducePlan pl;
+    pl.m = n_rows;
+    pl.n = k;
+    if (!make_dim_map(x_dims, x_strides, 0, x_rank - 1, &pl.kept) ||
+        !make_dim_map(x_dims, x_strides, x_rank - 1, x_rank, &pl.red) ||
+        !make_dim_map(y_dims, y_strides, 0, y_rank, &pl.ymap))
+        return DLFX_ERR_RANK;
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dispatch_dtype(dtype, [&](auto tag) {
+        using T = decltype(tag);
+        const T* xp = static_cast<const T*>(x) + x_offset;
+        if (index_dtype == DLFX_I32) {
+            int32_t* yp = static_cast<int32_t*>(y) + y_offset;
+            if (want_max) return launch_reduce<ArgReducer<T, true, int32_t>>(s, pl, xp, yp, 0, scratch, scratch_bytes);
+            return launch_reduce<ArgReducer<T, false, int32_t>>(s, pl, xp, yp, 0, scratch, scratch_bytes);
+        }
+        int64_t* yp = static_cast<int64_t*>(y) + y_offset;
+        if (want_max) return launch_reduce<ArgReducer<T, true, int64_t>>(s, pl, xp, yp, 0, scratch, scratch_bytes);
+        return launch_reduce<ArgReducer<T, false, int64_t>>(s, pl, xp, yp, 0, scratch, scratch_bytes);
+    });
+}

@@ -1,0 +1,208 @@
+"""ctypes binding of libdlfx.so (the C ABI in include/dlfx.h) plus the backend
+object the front-ends call.  PyTorch is used only to own device memory and to
+name the HIP stream work is enqueued on.
+
+There is no fallback: if the library is missing or a call fails, this raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p, POINTER
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libdlfx.so")
+
+_I64P = POINTER(c_int64)
+
+
+class DlfxError(RuntimeError):
+    def __init__(self, status: int, text: str, where: str):
+        super().__init__("%s: %s (status %d)" % (where, text, status))
+        self.status = status
+
+
+def _declare(lib):
+    view = [c_int, _I64P, _I64P]
+    lib.dlfx_version.restype = c_int
+    lib.dlfx_status_string.restype = c_char_p
+    lib.dlfx_status_string.argtypes = [c_int]
+    lib.dlfx_last_hip_error.restype = c_int
+
+    lib.dlfx_reduce_scratch_bytes.restype = c_size_t
+    lib.dlfx_reduce_scratch_bytes.argtypes = [c_int, c_int64, c_int64]
+    lib.dlfx_reduce.restype = c_int
+    lib.dlfx_reduce.argtypes = ([c_void_p, c_char_p, c_int, c_int64, c_int64] + view + [c_void_p, c_int64]
+                                + view + [c_void_p, c_int64, c_void_p, c_size_t])
+
+    lib.dlfx_arg_reduce_scratch_bytes.restype = c_size_t
+    lib.dlfx_arg_reduce_scratch_bytes.argtypes = [c_int, c_int64, c_int64]
+    lib.dlfx_arg_reduce.restype = c_int
+    lib.dlfx_arg_reduce.argtypes = ([c_void_p, c_char_p, c_int, c_int, c_int64, c_int64] + view
+                                    + [c_void_p, c_int64] + view + [c_void_p, c_int64, c_void_p, c_size_t])
+
+    lib.dlfx_scan_scratch_bytes.restype = c_size_t
+    lib.dlfx_scan_scratch_bytes.argtypes = [c_int, c_int64, c_int64]
+    lib.dlfx_scan.restype = c_int
+    lib.dlfx_scan.argtypes = [c_void_p, c_char_p, c_int, c_int64, c_int64, c_int, c_int, _I64P,
+                              c_void_p, c_int64, _I64P, c_void_p, c_int64, _I64P, c_void_p, c_size_t]
+
+    lib.dlfx_sort_scratch_bytes.restype = c_size_t
+    lib.dlfx_sort_scratch_bytes.argtypes = [c_int, c_int64, c_int64]
+    lib.dlfx_sort.restype = c_int
+    lib.dlfx_sort.argtypes = [c_void_p, c_int, c_int, c_int, _I64P, c_void_p, c_int64, _I64P,
+                              c_void_p, c_int64, _I64P, c_void_p, c_size_t]
+
+    lib.dlfx_argsort_scratch_bytes.restype = c_size_t
+    lib.dlfx_argsort_scratch_bytes.argtypes = [c_int, c_int64, c_int64]
+    lib.dlfx_argsort.restype = c_int
+    lib.dlfx_argsort.argtypes = [c_void_p, c_int, c_int, c_int, c_int, _I64P, c_void_p, c_int64, _I64P,
+                                 c_void_p, c_int64, _I64P, c_void_p, c_int64, _I64P, c_void_p, c_size_t]
+
+    lib.dlfx_top_k_scratch_bytes.restype = c_size_t
+    lib.dlfx_top_k_scratch_bytes.argtypes = [c_int, c_int64, c_int64, c_int64]
+    lib.dlfx_top_k.restype = c_int
+    lib.dlfx_top_k.argtypes = [c_void_p, c_int64, c_int, c_int, c_int, c_int, _I64P, _I64P,
+                               c_void_p, c_int64, _I64P, c_void_p, c_int64, _I64P,
+                               c_void_p, c_int64, _I64P, c_void_p, c_size_t]
+    return lib
+
+
+_lib = None
+
+# Every symbol include/dlfx.h declares.
+EXPORTS = ("dlfx_version", "dlfx_status_string", "dlfx_last_hip_error",
+           "dlfx_reduce_scratch_bytes", "dlfx_reduce",
+           "dlfx_arg_reduce_scratch_bytes", "dlfx_arg_reduce",
+           "dlfx_scan_scratch_bytes", "dlfx_scan",
+           "dlfx_sort_scratch_bytes", "dlfx_sort",
+           "dlfx_argsort_scratch_bytes", "dlfx_argsort",
+           "dlfx_top_k_scratch_bytes", "dlfx_top_k")
+
+
+def load_library():
+    """Loads libdlfx.so; raises when it has not been built (no fallback exists)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libdlfx.so is not built: run `python -m dlf_amd.build` "
+                               "(or __graft_entry__.build()) first; expected at " + LIB_PATH)
+        _lib = _declare(ctypes.CDLL(LIB_PATH))
+    return _lib
+
+
+def _arr(values):
+    values = list(values)
+    return (c_int64 * max(1, len(values)))(*values)
+
+
+def _check(status: int, where: str):
+    if status != 0:
+        lib = load_library()
+        text = lib.dlfx_status_string(status).decode()
+        if status == -6:
+            text += " (hipError %d)" % lib.dlfx_last_hip_error()
+        raise DlfxError(status, text, where)
+
+
+_NP_TO_TORCH = None
+
+
+def _torch_dtype(np_dtype):
+    global _NP_TO_TORCH
+    import torch
+    if _NP_TO_TORCH is None:
+        _NP_TO_TORCH = {np.dtype(np.float32): torch.float32, np.dtype(np.float64): torch.float64,
+                        np.dtype(np.int32): torch.int32, np.dtype(np.int64): torch.int64}
+    return _NP_TO_TORCH[np.dtype(np_dtype)]
+
+
+class HipBackend:
+    """Backend whose six boundary calls go through the C ABI onto the current HIP stream."""
+
+    name = "hip"
+
+    def __init__(self, device: str = "cuda:0"):
+        import torch
+        if not torch.cuda.is_available():
+            raise RuntimeError("no HIP device visible to PyTorch")
+        self.torch = torch
+        self.device = torch.device(device)
+        self.lib = load_library()
+        self._scratch = None
+
+    # -- storage ------------------------------------------------------------
+    def alloc(self, dtype, count: int):
+        return self.torch.empty(max(1, count), dtype=_torch_dtype(dtype), device=self.device)
+
+    def upload(self, flat: np.ndarray):
+        return self.torch.from_numpy(np.ascontiguousarray(flat)).to(self.device)
+
+    def download(self, storage) -> np.ndarray:
+        return storage.cpu().numpy()
+
+    def wrap(self, tensor):
+        """Use an existing contiguous 1-D device tensor as storage."""
+        return tensor
+
+    def scratch(self, nbytes: int):
+        if nbytes == 0:
+            return None, 0
+        if self._scratch is None or self._scratch.numel() < nbytes:
+            self._scratch = self.torch.empty(nbytes, dtype=self.torch.uint8, device=self.device)
+        return self._scratch.data_ptr(), nbytes
+
+    def _stream(self):
+        return self.torch.cuda.current_stream(self.device).cuda_stream
+
+    # -- boundary calls -----------------------------------------------------
+    def reduce(self, name, dtype, m, n, xs, x, ys, y):
+        sp, sb = self.scratch(self.lib.dlfx_reduce_scratch_bytes(dtype, m, n))
+        _check(self.lib.dlfx_reduce(self._stream(), name.encode(), dtype, m, n,
+                                    xs.rank, _arr(xs.extents), _arr(xs.strides), x.data_ptr(), xs.offset,
+                                    ys.rank, _arr(ys.extents), _arr(ys.strides), y.data_ptr(), ys.offset,
+                                    sp, sb), "dlfx_reduce(%s)" % name)
+
+    def arg_reduce(self, name, dtype, index_dtype, rows, k, xs, x, ys, y):
+        sp, sb = self.scratch(self.lib.dlfx_arg_reduce_scratch_bytes(dtype, rows, k))
+        _check(self.lib.dlfx_arg_reduce(self._stream(), name.encode(), dtype, index_dtype, rows, k,
+                                        xs.rank, _arr(xs.extents), _arr(xs.strides), x.data_ptr(), xs.offset,
+                                        ys.rank, _arr(ys.extents), _arr(ys.strides), y.data_ptr(), ys.offset,
+                                        sp, sb), "dlfx_arg_reduce(%s)" % name)
+
+    def scan(self, name, dtype, m, n, exclusive, xs, x, ys, y):
+        sp, sb = self.scratch(self.lib.dlfx_scan_scratch_bytes(dtype, m, n))
+        _check(self.lib.dlfx_scan(self._stream(), name.encode(), dtype, m, n, int(bool(exclusive)),
+                                  xs.rank, _arr(xs.extents), x.data_ptr(), xs.offset, _arr(xs.strides),
+                                  y.data_ptr(), ys.offset, _arr(ys.strides), sp, sb), "dlfx_scan(%s)" % name)
+
+    def sort(self, direction, dtype, xs, x, ys, y):
+        n = xs.extents[-1]
+        sp, sb = self.scratch(self.lib.dlfx_sort_scratch_bytes(dtype, xs.size // n, n))
+        _check(self.lib.dlfx_sort(self._stream(), direction, dtype, xs.rank, _arr(xs.extents),
+                                  x.data_ptr(), xs.offset, _arr(xs.strides),
+                                  y.data_ptr(), ys.offset, _arr(ys.strides), sp, sb), "dlfx_sort")
+
+    def argsort(self, direction, dtype, index_dtype, xs, x, ys, y, is_, i):
+        n = xs.extents[-1]
+        sp, sb = self.scratch(self.lib.dlfx_argsort_scratch_bytes(dtype, xs.size // n, n))
+        _check(self.lib.dlfx_argsort(self._stream(), direction, dtype, index_dtype, xs.rank, _arr(xs.extents),
+                                     x.data_ptr(), xs.offset, _arr(xs.strides),
+                                     y.data_ptr() if y is not None else None,
+                                     ys.offset if ys is not None else 0,
+                                     _arr(ys.strides) if ys is not None else None,
+                                     i.data_ptr(), is_.offset, _arr(is_.strides), sp, sb), "dlfx_argsort")
+
+    def top_k(self, limit, direction, dtype, index_dtype, xs, x, ys, y, is_, i):
+        n = xs.extents[-1]
+        sp, sb = self.scratch(self.lib.dlfx_top_k_scratch_bytes(dtype, xs.size // n, n, limit))
+        _check(self.lib.dlfx_top_k(self._stream(), limit, direction, dtype, index_dtype, xs.rank,
+                                   _arr(xs.extents), _arr(ys.extents),
+                                   x.data_ptr(), xs.offset, _arr(xs.strides),
+                                   y.data_ptr(), ys.offset, _arr(ys.strides),
+                                   i.data_ptr(), is_.offset, _arr(is_.strides), sp, sb), "dlfx_top_k")
+
+    def synchronize(self):
+        self.torch.cuda.synchronize(self.device)

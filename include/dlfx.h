@@ -1,0 +1,165 @@
+/*
+ * dlfx -- C ABI of the MI355X (gfx950) axis primitives: reduce, arg_reduce,
+ * scan, sort, argsort, top_k over strided N-d views.
+ *
+ * This is the boundary a dlf build binds in place of the gpgpu::dnn routines
+ * for these operations (reference declarations: gpgpu/include/gdnn.h:108-182,
+ * bodies gpgpu/src/gdnn.cpp:833-1347).  Each entry point below names the
+ * reference function it replaces.
+ *
+ * Conventions shared by every call
+ *   stream     a hipStream_t passed as void*; work is enqueued asynchronously on
+ *              it and the call returns without synchronising.
+ *   dtype      DLFX_F32 / DLFX_F64 / DLFX_I32 / DLFX_I64 -- the element type T
+ *              of the reference template instantiation.
+ *   dims       extents of the (already axis-moved) view, `rank` entries.
+ *   strides    element strides, signed: a reference stride that wrapped as
+ *              size_t (negative step) is passed as the negative number it means.
+ *   offset     element offset of the view's first element from the pointer.
+ *   x, y, idx  device pointers to the start of the buffers (Buffer<T>::data()).
+ *              Outputs may alias inputs where the reference allows it
+ *              (in-place scan / sort / argsort).
+ *   scratch    device memory owned by the caller, at least the number of bytes
+ *              the matching *_scratch_bytes() query returns (256-byte aligned);
+ *              may be NULL when that number is 0.  Its contents are undefined
+ *              on entry and on return; two calls that overlap in time must not
+ *              share it.
+ *   return     DLFX_OK or a negative dlfx_status; nothing is enqueued when the
+ *              status is an argument error.
+ * Ranks above DLFX_MAX_RANK (after merging mergeable dimensions) are rejected.
+ * No call allocates or frees device memory.
+ */
+#ifndef DLFX_H_
+#define DLFX_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DLFX_MAX_RANK 8
+
+typedef void* dlfx_stream_t; /* hipStream_t */
+
+typedef enum dlfx_dtype {
+    DLFX_F32 = 0,
+    DLFX_F64 = 1,
+    DLFX_I32 = 2,
+    DLFX_I64 = 3
+} dlfx_dtype;
+
+typedef enum dlfx_status {
+    DLFX_OK = 0,
+    DLFX_ERR_INVALID_ARGUMENT = -1,  /* null pointer, negative extent, m*n mismatch ... */
+    DLFX_ERR_UNSUPPORTED_DTYPE = -2,
+    DLFX_ERR_UNKNOWN_OP = -3,        /* `name` is not one this library implements */
+    DLFX_ERR_SCRATCH_TOO_SMALL = -4,
+    DLFX_ERR_RANK = -5,              /* view rank above DLFX_MAX_RANK */
+    DLFX_ERR_LAUNCH = -6,            /* HIP reported an error; see dlfx_last_hip_error */
+    DLFX_ERR_TOO_LARGE = -7          /* an extent exceeds what the kernels index */
+} dlfx_status;
+
+/* Library version: major*10000 + minor*100 + patch. */
+int dlfx_version(void);
+/* Static, human-readable text for a dlfx_status. */
+const char* dlfx_status_string(int status);
+/* hipError_t of the last DLFX_ERR_LAUNCH on the calling thread (0 if none). */
+int dlfx_last_hip_error(void);
+
+/* ---------------------------------------------------------------- reduce
+ * Replaces gpgpu::dnn::reduce<T> (gdnn.h:108-114; caller
+ * dlf/include/tensor/reduce_detail.h:91-101).  x_dims lists the kept extents
+ * followed by the reduced extents (the transposed view prepare_reduce builds);
+ * m = product of kept, n = product of reduced; output element r (row-major
+ * over y_dims) receives Final(fold(Map(x[r, 0..n)))).
+ * name: reduce_sum, reduce_mean, reduce_max, reduce_min, reduce_log_sum_exp,
+ *       reduce_sum_exp, reduce_log_sum, reduce_prod, reduce_asum,
+ *       reduce_sum_square, reduce_nrm2, reduce_amax, reduce_amin
+ *       (dlf/include/tensor/xfn.h:661-805).  The exp/log/sqrt reducers accept
+ *       floating dtypes only.
+ */
+size_t dlfx_reduce_scratch_bytes(int dtype, int64_t m, int64_t n);
+int dlfx_reduce(dlfx_stream_t stream, const char* name, int dtype, int64_t m, int64_t n,
+                int x_rank, const int64_t* x_dims, const int64_t* x_strides,
+                const void* x, int64_t x_offset,
+                int y_rank, const int64_t* y_dims, const int64_t* y_strides,
+                void* y, int64_t y_offset,
+                void* scratch, size_t scratch_bytes);
+
+/* ---------------------------------------------------------------- arg_reduce
+ * Replaces gpgpu::dnn::arg_reduce<T> (gdnn.h:138-144; caller
+ * reduce_detail.h:134-147).  The reduced axis is the last one of x_dims
+ * (extent k, n_rows = size / k).  name: "argmax" | "argmin".  The first
+ * occurrence wins ties (reduce_detail.h:120-128).  index_dtype DLFX_I32 is the
+ * reference's Buffer<int>; DLFX_I64 writes 64-bit indices.
+ */
+size_t dlfx_arg_reduce_scratch_bytes(int dtype, int64_t n_rows, int64_t k);
+int dlfx_arg_reduce(dlfx_stream_t stream, const char* name, int dtype, int index_dtype,
+                    int64_t n_rows, int64_t k,
+                    int x_rank, const int64_t* x_dims, const int64_t* x_strides,
+                    const void* x, int64_t x_offset,
+                    int y_rank, const int64_t* y_dims, const int64_t* y_strides,
+                    void* y, int64_t y_offset,
+                    void* scratch, size_t scratch_bytes);
+
+/* ---------------------------------------------------------------- scan
+ * Replaces gpgpu::dnn::scan<T> (gdnn.h:124-129; caller
+ * reduce_detail.h:244-253).  The scanned axis is the last one of dims (extent
+ * n, m rows); x and y share dims and have independent strides; a reverse scan
+ * arrives as flipped views (negative last strides).
+ * name: "cumsum" | "cumprod" | "cummax" | "cummin".
+ */
+size_t dlfx_scan_scratch_bytes(int dtype, int64_t m, int64_t n);
+int dlfx_scan(dlfx_stream_t stream, const char* name, int dtype, int64_t m, int64_t n,
+              int exclusive, int rank, const int64_t* dims,
+              const void* x, int64_t x_offset, const int64_t* x_strides,
+              void* y, int64_t y_offset, const int64_t* y_strides,
+              void* scratch, size_t scratch_bytes);
+
+/* ---------------------------------------------------------------- sort
+ * Replaces gpgpu::dnn::sort<T> (gdnn.h:157-161; caller
+ * dlf/include/tensor/reorder_detail.h:617-627).  Sorts every row of the last
+ * axis; dir 0 ascending, 1 descending.
+ */
+size_t dlfx_sort_scratch_bytes(int dtype, int64_t m, int64_t n);
+int dlfx_sort(dlfx_stream_t stream, int dir, int dtype, int rank, const int64_t* dims,
+              const void* x, int64_t x_offset, const int64_t* x_strides,
+              void* y, int64_t y_offset, const int64_t* y_strides,
+              void* scratch, size_t scratch_bytes);
+
+/* ---------------------------------------------------------------- argsort
+ * Replaces both gpgpu::dnn::argsort<T> overloads (gdnn.h:163-174; callers
+ * reorder_detail.h:667-677, 951-963).  y == NULL is the index-only overload.
+ * The order is stable: equal keys keep ascending source index, for both
+ * directions.  index_dtype DLFX_I32 is the reference's Buffer<int32_t>.
+ */
+size_t dlfx_argsort_scratch_bytes(int dtype, int64_t m, int64_t n);
+int dlfx_argsort(dlfx_stream_t stream, int dir, int dtype, int index_dtype,
+                 int rank, const int64_t* dims,
+                 const void* x, int64_t x_offset, const int64_t* x_strides,
+                 void* y, int64_t y_offset, const int64_t* y_strides,
+                 void* idx, int64_t i_offset, const int64_t* i_strides,
+                 void* scratch, size_t scratch_bytes);
+
+/* ---------------------------------------------------------------- top_k
+ * Replaces gpgpu::dnn::top_k<T> (gdnn.h:176-182; caller
+ * reorder_detail.h:1062-1073).  Selects `limit` elements per row of the last
+ * axis of x (dir 1: largest, 0: smallest), written in sorted order; among equal
+ * values the lowest source index is taken first.  y and idx share y_dims
+ * (last extent == limit <= last extent of x_dims).
+ */
+size_t dlfx_top_k_scratch_bytes(int dtype, int64_t m, int64_t n, int64_t limit);
+int dlfx_top_k(dlfx_stream_t stream, int64_t limit, int dir, int dtype, int index_dtype,
+               int rank, const int64_t* x_dims, const int64_t* y_dims,
+               const void* x, int64_t x_offset, const int64_t* x_strides,
+               void* y, int64_t y_offset, const int64_t* y_strides,
+               void* idx, int64_t i_offset, const int64_t* i_strides,
+               void* scratch, size_t scratch_bytes);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+
+#endif /* DLFX_H_ */

@@ -1,0 +1,200 @@
+"""Pins the CPU oracle against independent library routines (numpy) and closed
+forms, on strided / transposed / flipped views, so that a dropped term, wrong
+index or transposed operand in the restatement fails here."""
+import numpy as np
+import pytest
+
+from dlf_amd import frontend as F
+from dlf_amd.frontend import Tensor
+from helpers import normal, randint, full_range_i64, uniform01
+
+
+def T(be, a):
+    return Tensor.from_numpy(be, a)
+
+
+@pytest.mark.parametrize("axes,keep", [((), False), ((0,), False), ((1,), True), ((2,), False),
+                                       ((0, 2), False), ((1, 2), True), ((-1,), False)])
+def test_reduce_int_matches_numpy(oracle_backend, axes, keep):
+    x = randint(11, 7 * 9 * 300, -50, 50).astype(np.int64).reshape(7, 9, 300)
+    X = T(oracle_backend, x)
+    ax = tuple(a % 3 for a in axes) or None
+    assert np.array_equal(F.reduce_sum(X, axes, keep).numpy(), x.sum(axis=ax, keepdims=keep))
+    assert np.array_equal(F.reduce_max(X, axes, keep).numpy(), x.max(axis=ax, keepdims=keep))
+    assert np.array_equal(F.reduce_min(X, axes, keep).numpy(), x.min(axis=ax, keepdims=keep))
+    n = x.size // x.sum(axis=ax, keepdims=keep).size
+    # integer mean truncates toward zero (C++ division), unlike numpy's floor division
+    want = np.trunc(x.sum(axis=ax, keepdims=keep) / n).astype(np.int64)
+    assert np.array_equal(F.reduce_mean(X, axes, keep).numpy(), want)
+
+
+def test_reduce_int32_sum_wraps(oracle_backend):
+    x = np.full((3, 5000), 2**30, dtype=np.int32)
+    got = F.reduce_sum(T(oracle_backend, x), [1]).numpy()
+    assert np.array_equal(got, x.astype(np.int64).sum(axis=1).astype(np.int32))
+
+
+def test_reduce_float_close_to_numpy_f64(oracle_backend):
+    x = normal(12, 40 * 5000).astype(np.float32).reshape(40, 5000)
+    X = T(oracle_backend, x)
+    x64 = x.astype(np.float64)
+    np.testing.assert_allclose(F.reduce_sum(X, [1]).numpy(), x64.sum(axis=1), rtol=0, atol=1e-3)
+    np.testing.assert_allclose(F.reduce_mean(X, [0]).numpy(), x64.mean(axis=0), rtol=0, atol=1e-5)
+    np.testing.assert_allclose(F.reduce_log_sum_exp(X, [1]).numpy(), np.log(np.exp(x64).sum(axis=1)), rtol=1e-5)
+    np.testing.assert_allclose(F.reduce_sum_square(X, [1]).numpy(), (x64 * x64).sum(axis=1), rtol=1e-5)
+    np.testing.assert_allclose(F.reduce_nrm2(X, [1]).numpy(), np.sqrt((x64 * x64).sum(axis=1)), rtol=1e-5)
+    np.testing.assert_allclose(F.reduce_asum(X, [1]).numpy(), np.abs(x64).sum(axis=1), rtol=1e-5)
+    assert np.array_equal(F.reduce_amax(X, [1]).numpy(), np.abs(x).max(axis=1))
+    assert np.array_equal(F.reduce_amin(X, [1]).numpy(), np.abs(x).min(axis=1))
+
+
+def test_log_sum_exp_is_naive_and_overflows(oracle_backend):
+    # xfn.h:779-791: log(sum(exp(x))) without a max shift
+    x = np.array([[1.0, 2.0, 3.0], [100.0, 0.0, 0.0]], dtype=np.float32)
+    got = F.reduce_log_sum_exp(T(oracle_backend, x), [1]).numpy()
+    assert np.isclose(got[0], np.log(np.exp(1.0) + np.exp(2.0) + np.exp(3.0)), rtol=1e-6)
+    assert np.isposinf(got[1])
+
+
+def test_reduce_f64_evaluator(oracle_backend):
+    from oracle import oracle as O
+    x = normal(13, 6 * 4000).astype(np.float32).reshape(6, 4000)
+    X = T(oracle_backend, x)
+    view, _, m, n = F.prepare_reduce(X.shape, [1], False)
+    got = O.reduce_f64("reduce_sum", 0, m, n, view, X.storage)
+    np.testing.assert_allclose(got, x.astype(np.float64).sum(axis=1), rtol=1e-13)
+    view, _, m, n = F.prepare_reduce(X.shape, [0], False)
+    got = O.reduce_f64("reduce_mean", 0, m, n, view, X.storage)
+    np.testing.assert_allclose(got, x.astype(np.float64).mean(axis=0), rtol=1e-13)
+
+
+@pytest.mark.parametrize("axis", [0, 1, 2, -1])
+@pytest.mark.parametrize("keep", [True, False])
+def test_argmax_argmin_match_numpy_first_occurrence(oracle_backend, axis, keep):
+    x = randint(14, 6 * 7 * 50, 0, 5).astype(np.int32).reshape(6, 7, 50)   # many ties
+    X = T(oracle_backend, x)
+    want_max = np.argmax(x, axis=axis)
+    want_min = np.argmin(x, axis=axis)
+    if keep:
+        want_max, want_min = np.expand_dims(want_max, axis), np.expand_dims(want_min, axis)
+    assert np.array_equal(F.argmax(X, axis, keep).numpy(), want_max)
+    assert np.array_equal(F.argmin(X, axis, keep).numpy(), want_min)
+
+
+def test_argmax_transposed_view(oracle_backend):
+    # DNNTest.cpp:1011-1017: argmax(X.transpose(), 0) == argmax(X, -1).transpose()
+    x = randint(15, 4 * 5 * 6, 0, 100).astype(np.int32).reshape(4, 5, 6)
+    X = T(oracle_backend, x)
+    a = F.argmax(X.transpose(), 0).numpy()
+    b = F.argmax(X, -1).numpy().transpose()
+    assert np.array_equal(a, b)
+
+
+def test_argmax_nan_rule(oracle_backend):
+    x = np.array([[1.0, np.nan, 2.0], [np.nan, 5.0, 7.0]], dtype=np.float32)
+    assert F.argmax(T(oracle_backend, x), 1, False).numpy().tolist() == [2, 0]
+
+
+@pytest.mark.parametrize("axis", [0, 1, 2])
+@pytest.mark.parametrize("exclusive", [False, True])
+@pytest.mark.parametrize("reverse", [False, True])
+def test_cumsum_int_matches_numpy(oracle_backend, axis, exclusive, reverse):
+    x = randint(16, 5 * 3000 * 4, 0, 100).astype(np.int32).reshape(5, 3000, 4)
+    got = F.cumsum(T(oracle_backend, x), axis, exclusive, reverse).numpy()
+    xx = np.flip(x, axis) if reverse else x
+    want = np.cumsum(xx, axis=axis, dtype=np.int32)
+    if exclusive:
+        want = want - xx
+    if reverse:
+        want = np.flip(want, axis)
+    assert np.array_equal(got, want)
+
+
+def test_cumprod_cummax_cummin(oracle_backend):
+    x = randint(17, 3 * 2500, 1, 3).astype(np.int64).reshape(3, 2500)
+    assert np.array_equal(F.cumprod(T(oracle_backend, x), 1).numpy(), np.cumprod(x, axis=1))
+    y = normal(18, 3 * 2500).astype(np.float32).reshape(3, 2500)
+    assert np.array_equal(F.cummax(T(oracle_backend, y), 1).numpy(), np.maximum.accumulate(y, axis=1))
+    assert np.array_equal(F.cummin(T(oracle_backend, y), 1).numpy(), np.minimum.accumulate(y, axis=1))
+
+
+def test_cumsum_in_place_and_random_int_property(oracle_backend):
+    # UniformTest.cpp:2188-2189 uses a [2, 100000] random int tensor
+    x = full_range_i64(19, 2 * 100000).astype(np.int32).reshape(2, 100000)
+    X = T(oracle_backend, x)
+    F.cumsum(X, 1, out=X)
+    assert np.array_equal(X.numpy(), np.cumsum(x, axis=1, dtype=np.int32))
+
+
+def test_scan_f64_evaluator(oracle_backend):
+    from oracle import oracle as O
+    x = normal(20, 3 * 5000).astype(np.float32).reshape(3, 5000)
+    X = T(oracle_backend, x)
+    y, mag = O.scan_f64("cumsum", 0, 3, 5000, False, X.shape, X.storage)
+    np.testing.assert_allclose(y, np.cumsum(x.astype(np.float64), axis=1), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(mag, np.cumsum(np.abs(x.astype(np.float64)), axis=1), rtol=1e-12)
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.int64, np.float32, np.float64])
+@pytest.mark.parametrize("axis", [0, 1, 2])
+@pytest.mark.parametrize("desc", [False, True])
+def test_sort_matches_numpy(oracle_backend, dtype, axis, desc):
+    x = randint(21, 4 * 1500 * 3, -1000, 1000).astype(dtype).reshape(4, 1500, 3)
+    got = F.sort(T(oracle_backend, x), axis, desc).numpy()
+    want = np.sort(x, axis=axis)
+    if desc:
+        want = np.flip(want, axis)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("n", [1, 2, 10, 99, 100, 101, 500, 501, 1000, 1001, 2500, 10000])
+def test_sort_sizes_and_in_place(oracle_backend, n):
+    x = randint(22 + n, 2 * n, 0, 2000).astype(np.int32).reshape(2, n)
+    X = T(oracle_backend, x)
+    F.sort(X, -1, out=X)
+    assert np.array_equal(X.numpy(), np.sort(x, axis=-1))
+
+
+@pytest.mark.parametrize("axis", [0, 1])
+@pytest.mark.parametrize("desc", [False, True])
+def test_argsort_is_stable_like_numpy(oracle_backend, axis, desc):
+    x = randint(23, 300 * 7, 0, 8).astype(np.int32).reshape(300, 7)          # heavy duplicates
+    X = T(oracle_backend, x)
+    I = F.argsort(X, axis, desc).numpy()
+    key = -x.astype(np.int64) if desc else x
+    want = np.argsort(key, axis=axis, kind="stable")
+    assert np.array_equal(I, want)
+    Y, I2 = F.argsort(X, axis, desc, with_values=True)
+    assert np.array_equal(I2.numpy(), want)
+    assert np.array_equal(Y.numpy(), np.take_along_axis(x, want, axis=axis))
+
+
+def test_argsort_long_rows_stable(oracle_backend):
+    x = (uniform01(24, 3 * 20000) * 64).astype(np.float32).astype(np.int64).astype(np.float32).reshape(3, 20000)
+    I = F.argsort(T(oracle_backend, x), -1).numpy()
+    assert np.array_equal(I, np.argsort(x, axis=-1, kind="stable"))
+
+
+@pytest.mark.parametrize("largest", [True, False])
+@pytest.mark.parametrize("k", [1, 5, 50, 256])
+def test_top_k_spec_and_heap_agree_on_values(oracle_backend, largest, k):
+    from oracle.oracle import OracleBackend
+    x = np.round(normal(25, 20 * 3000) * 2 * 256) / 256          # ties occur
+    x = x.astype(np.float32).reshape(20, 3000)
+    ys, is_ = F.top_k(T(oracle_backend, x), k, -1, largest)
+    yh, ih = F.top_k(T(OracleBackend(topk_mode=0), x), k, -1, largest)
+    ys, is_, yh, ih = ys.numpy(), is_.numpy(), yh.numpy(), ih.numpy()
+    key = -x.astype(np.float64) if largest else x.astype(np.float64)
+    order = np.argsort(key, axis=-1, kind="stable")[:, :k]
+    assert np.array_equal(is_, order)                                   # lowest index on ties
+    assert np.array_equal(ys, np.take_along_axis(x, order, axis=-1))
+    assert np.array_equal(yh, ys)                                       # reference heap: same values
+    assert np.array_equal(np.take_along_axis(x, ih.astype(np.int64), axis=-1), yh)
+
+
+def test_top_k_axis_and_clamp(oracle_backend):
+    x = randint(26, 6 * 9, 0, 1000).astype(np.int64).reshape(6, 9)
+    y, i = F.top_k(T(oracle_backend, x), 100, 0, True, index_dtype=np.int64)
+    assert y.numpy().shape == (6, 9)                                    # k clamps to the extent
+    assert np.array_equal(y.numpy(), np.flip(np.sort(x, axis=0), 0))
+    assert i.numpy().dtype == np.int64
