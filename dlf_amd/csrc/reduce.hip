@@ -118,8 +118,14 @@ struct ArgReducer {
     using out_t = I;
 
     __device__ static __forceinline__ acc_t identity() {
-        return {MAX ? std::numeric_limits<T>::lowest() : std::numeric_limits<T>::max(),
-                std::numeric_limits<int32_t>::max()};
+        // weakest possible value, so that any element (even -inf / +inf) ties or wins;
+        // ties go to the lower index, and every real index is below this one
+        if constexpr (std::is_integral<T>::value)
+            return {MAX ? std::numeric_limits<T>::lowest() : std::numeric_limits<T>::max(),
+                    std::numeric_limits<int32_t>::max()};
+        else
+            return {MAX ? -std::numeric_limits<T>::infinity() : std::numeric_limits<T>::infinity(),
+                    std::numeric_limits<int32_t>::max()};
     }
     __device__ static __forceinline__ acc_t map(T x, int64_t j) {
         if constexpr (!std::is_integral<T>::value) {

@@ -1,0 +1,485 @@
+// scan (cumsum / cumprod / cummax / cummin) over strided views for gfx950.
+//
+// Two kernels:
+//   * scan_rows: the scanned axis is walked by whole workgroups.  A row is cut
+//     into tiles of 256 x ITEMS elements; every tile is read once and written
+//     once.  Inside a tile each wave owns a contiguous segment that it loads
+//     with 128-bit accesses and scans with DPP row shifts / broadcasts; tiles of
+//     one row are chained with decoupled look-back (aggregate / inclusive-prefix
+//     words published with agent-scope atomics), tile ids come from an atomic
+//     ticket so a tile only ever waits for tiles that already started.
+//   * scan_cols: many rows, scanned axis strided, a kept axis contiguous (e.g.
+//     cumsum over C of NCHW).  Lanes run along the kept axis so each load is a
+//     contiguous segment, the four waves of a workgroup take consecutive
+//     chunks of the scanned axis and exchange chunk totals through LDS.
+#include <cstring>
+#include <limits>
+#include <type_traits>
+
+#include "common.hip.h"
+
+namespace dlfx {
+namespace {
+
+enum ScanKind { kScanAdd = 0, kScanMul = 1, kScanMax = 2, kScanMin = 3 };
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / kWave;
+
+template <typename T, int K>
+struct ScanOp {
+    __device__ static __forceinline__ T identity() {
+        if constexpr (K == kScanAdd) return T(0);
+        else if constexpr (K == kScanMul) return T(1);
+        else if constexpr (K == kScanMax) return std::numeric_limits<T>::lowest();
+        else return std::numeric_limits<T>::max();
+    }
+    __device__ static __forceinline__ T apply(T a, T b) {
+        if constexpr (K == kScanAdd) {
+            if constexpr (std::is_integral<T>::value) {
+                using U = typename std::make_unsigned<T>::type;
+                return static_cast<T>(static_cast<U>(a) + static_cast<U>(b));
+            } else return a + b;
+        } else if constexpr (K == kScanMul) {
+            if constexpr (std::is_integral<T>::value) {
+                using U = typename std::make_unsigned<T>::type;
+                return static_cast<T>(static_cast<U>(a) * static_cast<U>(b));
+            } else return a * b;
+        } else if constexpr (K == kScanMax) {
+            return (a < b) ? b : a;
+        } else {
+            return (b < a) ? b : a;
+        }
+    }
+};
+
+// ------------------------------------------------------------------ look-back state
+constexpr uint32_t kInvalid = 0, kAggregate = 1, kInclusive = 2;
+
+// 4-byte values travel with their flag in one 64-bit word.
+template <typename T, int SIZE = sizeof(T)>
+struct TileState;
+
+template <typename T>
+struct TileState<T, 4> {
+    unsigned long long* words;
+    static size_t bytes(int64_t tiles) { return static_cast<size_t>(tiles) * 8; }
+    __host__ __device__ void bind(void* base, int64_t) { words = static_cast<unsigned long long*>(base); }
+    __device__ __forceinline__ void clear(int64_t i) { words[i] = 0ull; }
+    __device__ __forceinline__ void publish(int64_t i, uint32_t flag, T v) {
+        unsigned long long w = (static_cast<unsigned long long>(flag) << 32) | bit_cast<uint32_t>(v);
+        __hip_atomic_store(&words[i], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __device__ __forceinline__ uint32_t read(int64_t i, T* v) {
+        unsigned long long w = __hip_atomic_load(&words[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *v = bit_cast<T>(static_cast<uint32_t>(w));
+        return static_cast<uint32_t>(w >> 32);
+    }
+};
+
+// 8-byte values: value arrays plus a flag written with release / read with acquire.
+template <typename T>
+struct TileState<T, 8> {
+    uint32_t* flags;
+    unsigned long long* agg;
+    unsigned long long* incl;
+    static size_t bytes(int64_t tiles) { return align_up(static_cast<size_t>(tiles) * 4, 256) + static_cast<size_t>(tiles) * 16; }
+    __host__ __device__ void bind(void* base, int64_t tiles) {
+        flags = static_cast<uint32_t*>(base);
+        size_t off = (static_cast<size_t>(tiles) * 4 + 255) / 256 * 256;
+        agg = reinterpret_cast<unsigned long long*>(static_cast<char*>(base) + off);
+        incl = agg + tiles;
+    }
+    __device__ __forceinline__ void clear(int64_t i) { flags[i] = 0u; }
+    __device__ __forceinline__ void publish(int64_t i, uint32_t flag, T v) {
+        unsigned long long* dst = (flag == kAggregate) ? agg : incl;
+        __hip_atomic_store(&dst[i], bit_cast<unsigned long long>(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&flags[i], flag, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __device__ __forceinline__ uint32_t read(int64_t i, T* v) {
+        uint32_t f = __hip_atomic_load(&flags[i], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+        if (f != kInvalid) {
+            unsigned long long* src = (f == kAggregate) ? agg : incl;
+            *v = bit_cast<T>(__hip_atomic_load(&src[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        }
+        return f;
+    }
+};
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void scan_init(unsigned* ticket, TileState<T> st, int64_t tiles) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i == 0) *ticket = 0u;
+    if (i < tiles) st.clear(i);
+}
+
+// ------------------------------------------------------------------ row kernel
+// Element order inside a tile: wave w owns [w*64*ITEMS, (w+1)*64*ITEMS); within
+// it, vector k of lane l covers elements (k*64 + l)*V .. +V.
+template <typename T, int K, int ITEMS>
+__global__ __launch_bounds__(kBlock) void scan_rows(
+    const T* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
+    int64_t n, int64_t tiles_per_row, int exclusive, unsigned* ticket, TileState<T> st) {
+    using Op = ScanOp<T, K>;
+    constexpr int V = (vec_width<T>() < ITEMS) ? vec_width<T>() : ITEMS;
+    constexpr int KV = ITEMS / V;
+    constexpr int64_t TILE = static_cast<int64_t>(kBlock) * ITEMS;
+    using VecT = Vec<T, V>;
+
+    __shared__ T wave_total[kWaves];
+    __shared__ T tile_prefix_sm;
+    __shared__ unsigned tile_id_sm;
+
+    const int lane = lane_id();
+    const int w = threadIdx.x / kWave;
+
+    int64_t tile_id;
+    if (tiles_per_row > 1) {
+        if (threadIdx.x == 0) tile_id_sm = atomicAdd(ticket, 1u);
+        __syncthreads();
+        tile_id = tile_id_sm;
+    } else {
+        tile_id = blockIdx.x;
+    }
+    const int64_t row = tile_id / tiles_per_row;
+    const int64_t t = tile_id - row * tiles_per_row;
+    const int64_t tile_base = t * TILE;
+    const int64_t avail = (n - tile_base < TILE) ? n - tile_base : TILE;   // valid elements in this tile
+
+    const T* xr = x + xmap.at(row);
+    T* yr = y + ymap.at(row);
+    const int64_t seg = tile_base + static_cast<int64_t>(w) * kWave * ITEMS;
+
+    // ---- load
+    T vals[ITEMS];
+    const bool full = avail == TILE;
+    const bool x_vec = full && sx == 1 && (reinterpret_cast<uintptr_t>(xr + seg) % (sizeof(T) * V) == 0);
+    if (x_vec) {
+        const VecT* pv = reinterpret_cast<const VecT*>(xr + seg);
+#pragma unroll
+        for (int k = 0; k < KV; ++k) {
+            VecT a = pv[k * kWave + lane];
+#pragma unroll
+            for (int e = 0; e < V; ++e) vals[k * V + e] = a.v[e];
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < KV; ++k)
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const int64_t i = seg + static_cast<int64_t>(k * kWave + lane) * V + e;
+                vals[k * V + e] = (i < n) ? xr[i * sx] : Op::identity();
+            }
+    }
+
+    // ---- scan inside the wave: vals[] become inclusive prefixes within the wave segment
+    T carry = Op::identity();
+#pragma unroll
+    for (int k = 0; k < KV; ++k) {
+#pragma unroll
+        for (int e = 1; e < V; ++e) vals[k * V + e] = Op::apply(vals[k * V + e - 1], vals[k * V + e]);
+        const T lane_total = vals[k * V + V - 1];
+        const T incl = wave_scan_inclusive(lane_total, Op::identity(), [](T a, T b) { return Op::apply(a, b); });
+        T excl = lane_get(incl, lane - 1 < 0 ? 0 : lane - 1);
+        if (lane == 0) excl = Op::identity();
+        const T base = Op::apply(carry, excl);
+#pragma unroll
+        for (int e = 0; e < V; ++e) vals[k * V + e] = Op::apply(base, vals[k * V + e]);
+        carry = Op::apply(carry, lane_read(incl, kWave - 1));
+    }
+    if (lane == 0) wave_total[w] = carry;
+    __syncthreads();
+
+    T wave_prefix = Op::identity();
+    T aggregate = Op::identity();
+#pragma unroll
+    for (int i = 0; i < kWaves; ++i) {
+        const T wt = wave_total[i];
+        if (i < w) wave_prefix = Op::apply(wave_prefix, wt);
+        aggregate = Op::apply(aggregate, wt);
+    }
+
+    // ---- chain tiles of this row
+    T tile_prefix = Op::identity();
+    if (tiles_per_row > 1) {
+        if (w == 0) {
+            const int64_t sbase = row * tiles_per_row;
+            if (lane == 0) st.publish(sbase + t, t == 0 ? kInclusive : kAggregate, aggregate);
+            T excl = Op::identity();
+            if (t > 0) {
+                int64_t pos = t - 1;
+                for (;;) {
+                    const int64_t idx = pos - lane;
+                    T v = Op::identity();
+                    uint32_t f = kInclusive;          // before the row: an inclusive identity
+                    if (idx >= 0) {
+                        f = st.read(sbase + idx, &v);
+                        while (f == kInvalid) {
+                            __builtin_amdgcn_s_sleep(1);
+                            f = st.read(sbase + idx, &v);
+                        }
+                    }
+                    const unsigned long long incl_mask = __ballot(f == kInclusive);
+                    const int first = __ffsll(static_cast<long long>(incl_mask)) - 1;   // >= 0: some lane is inclusive
+                    const T contrib = (first < 0 || lane <= first) ? v : Op::identity();
+                    const T red = wave_reduce(contrib, [](T a, T b) { return Op::apply(a, b); });
+                    excl = Op::apply(red, excl);
+                    if (incl_mask != 0ull) break;
+                    pos -= kWave;
+                }
+                if (lane == 0) st.publish(sbase + t, kInclusive, Op::apply(excl, aggregate));
+            }
+            if (lane == 0) tile_prefix_sm = excl;
+        }
+        __syncthreads();
+        tile_prefix = tile_prefix_sm;
+    }
+
+    // ---- combine and store
+    const T pre = Op::apply(tile_prefix, wave_prefix);
+    if (exclusive) {
+        // element i receives the prefix of everything before it: shift by one element
+        // inside the lane's vector, and take the previous lane / vector / wave for e == 0
+#pragma unroll
+        for (int k = KV - 1; k >= 0; --k) {
+            const T last = vals[k * V + V - 1];
+            T prev = lane_get(last, lane - 1 < 0 ? 0 : lane - 1);      // inclusive prefix up to the previous lane's vector
+            T prev_vec_end = (k > 0) ? lane_read(vals[(k > 0 ? k - 1 : 0) * V + V - 1], kWave - 1) : Op::identity();
+            if (lane == 0) prev = prev_vec_end;
+#pragma unroll
+            for (int e = V - 1; e > 0; --e) vals[k * V + e] = vals[k * V + e - 1];
+            vals[k * V] = prev;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) vals[i] = Op::apply(pre, vals[i]);
+
+    const bool y_vec = full && sy == 1 && (reinterpret_cast<uintptr_t>(yr + seg) % (sizeof(T) * V) == 0);
+    if (y_vec) {
+        VecT* pv = reinterpret_cast<VecT*>(yr + seg);
+#pragma unroll
+        for (int k = 0; k < KV; ++k) {
+            VecT a;
+#pragma unroll
+            for (int e = 0; e < V; ++e) a.v[e] = vals[k * V + e];
+            pv[k * kWave + lane] = a;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < KV; ++k)
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const int64_t i = seg + static_cast<int64_t>(k * kWave + lane) * V + e;
+                if (i < n) yr[i * sy] = vals[k * V + e];
+            }
+    }
+}
+
+// ------------------------------------------------------------------ column kernel
+// One lane per row ("column"), four waves along the scanned axis.  Each pass of
+// the loop covers kWaves * chunk positions of the axis: thread (lx, ty) scans
+// positions [s + ty*chunk, s + (ty+1)*chunk) in registers.
+template <typename T, int K>
+__global__ __launch_bounds__(kBlock) void scan_cols(
+    const T* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
+    int64_t m, int64_t n, int chunk, int exclusive) {
+    using Op = ScanOp<T, K>;
+    constexpr int R = 16;
+    __shared__ T totals[2][kWaves][kWave];
+
+    const int lx = threadIdx.x & (kWave - 1);
+    const int ty = threadIdx.x / kWave;
+    const int64_t col = static_cast<int64_t>(blockIdx.x) * kWave + lx;
+    const bool live = col < m;
+    const T* xc = x + (live ? xmap.at(col) : 0);
+    T* yc = y + (live ? ymap.at(col) : 0);
+
+    T carry = Op::identity();
+    int buf = 0;
+    for (int64_t s = 0; s < n; s += static_cast<int64_t>(kWaves) * chunk, buf ^= 1) {
+        const int64_t p0 = s + static_cast<int64_t>(ty) * chunk;
+        T v[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t p = p0 + r;
+            v[r] = (live && r < chunk && p < n) ? xc[p * sx] : Op::identity();
+        }
+#pragma unroll
+        for (int r = 1; r < R; ++r) v[r] = Op::apply(v[r - 1], v[r]);
+        totals[buf][ty][lx] = v[R - 1];
+        __syncthreads();
+        T pre = carry;
+        T all = Op::identity();
+#pragma unroll
+        for (int i = 0; i < kWaves; ++i) {
+            const T tv = totals[buf][i][lx];
+            if (i < ty) pre = Op::apply(pre, tv);
+            all = Op::apply(all, tv);
+        }
+        carry = Op::apply(carry, all);
+        if (live) {
+            if (exclusive) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const int64_t p = p0 + r;
+                    const T prev = (r == 0) ? pre : Op::apply(pre, v[r > 0 ? r - 1 : 0]);
+                    if (r < chunk && p < n) yc[p * sy] = prev;
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const int64_t p = p0 + r;
+                    if (r < chunk && p < n) yc[p * sy] = Op::apply(pre, v[r]);
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ host side
+// Joint merge of the leading dimensions [0, e) of two stride sets that share
+// extents: neighbours merge only when both walks allow it.
+bool make_dim_map2(const int64_t* dims, const int64_t* sx, const int64_t* sy, int e, DimMap* mx, DimMap* my) {
+    int r = 0;
+    int64_t d[64], a[64], b[64];
+    for (int i = 0; i < e; ++i) {
+        if (dims[i] == 1) continue;
+        if (r > 0 && a[r - 1] == sx[i] * dims[i] && b[r - 1] == sy[i] * dims[i]) {
+            d[r - 1] *= dims[i];
+            a[r - 1] = sx[i];
+            b[r - 1] = sy[i];
+        } else {
+            if (r == 64) return false;
+            d[r] = dims[i];
+            a[r] = sx[i];
+            b[r] = sy[i];
+            ++r;
+        }
+    }
+    if (r > kMaxRank) return false;
+    mx->rank = my->rank = r;
+    for (int i = 0; i < kMaxRank; ++i) {
+        mx->dims[i] = my->dims[i] = i < r ? d[i] : 1;
+        mx->strides[i] = i < r ? a[i] : 0;
+        my->strides[i] = i < r ? b[i] : 0;
+    }
+    return true;
+}
+
+template <typename T>
+constexpr int items_full() { return 64 / sizeof(T); }   // 64 bytes per thread
+
+int64_t tile_elems(size_t elem_size, int64_t n) {
+    const int64_t full = 256 * (64 / static_cast<int64_t>(elem_size));
+    if (n > 1024) return full;
+    if (n > 256) return 1024;
+    return 256;
+}
+
+struct ScanLayout {
+    int64_t tiles_per_row, tiles;
+    size_t ticket_off, state_off, total;
+};
+
+ScanLayout scan_layout(size_t elem_size, int64_t m, int64_t n) {
+    ScanLayout l;
+    l.tiles_per_row = ceil_div(n, tile_elems(elem_size, n));
+    l.tiles = m * l.tiles_per_row;
+    l.ticket_off = 0;
+    l.state_off = 256;
+    if (l.tiles_per_row <= 1) {
+        l.total = 0;
+    } else {
+        size_t sb = elem_size == 4 ? static_cast<size_t>(l.tiles) * 8
+                                   : align_up(static_cast<size_t>(l.tiles) * 4, 256) + static_cast<size_t>(l.tiles) * 16;
+        l.total = 256 + align_up(sb, 256);
+    }
+    return l;
+}
+
+template <typename T, int K>
+int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int rank, const int64_t* dims,
+                const T* x, const int64_t* x_strides, T* y, const int64_t* y_strides,
+                void* scratch, size_t scratch_bytes) {
+    DimMap xmap, ymap;
+    if (!make_dim_map2(dims, x_strides, y_strides, rank - 1, &xmap, &ymap)) return DLFX_ERR_RANK;
+    const int64_t sx = rank ? x_strides[rank - 1] : 1;
+    const int64_t sy = rank ? y_strides[rank - 1] : 1;
+
+    // Many rows with a contiguous kept axis and a strided scanned axis: column kernel.
+    const bool axis_unit = (sx == 1 || sx == -1 || n == 1) && (sy == 1 || sy == -1 || n == 1);
+    const bool inner_unit = xmap.rank >= 1 && xmap.strides[xmap.rank - 1] == 1 && ymap.strides[ymap.rank - 1] == 1 &&
+                            xmap.dims[xmap.rank - 1] >= 16;
+    const bool short_rows = n <= 64 && m >= 256;
+    const bool use_cols = short_rows || (!axis_unit && m >= 64 && (inner_unit || n < 4096));
+    if (use_cols) {
+        int chunk = static_cast<int>(ceil_div(n, kWaves) < 16 ? ceil_div(n, kWaves) : 16);
+        const int64_t blocks = ceil_div(m, kWave);
+        if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+        scan_cols<T, K><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
+            x, y, xmap, ymap, sx, sy, m, n, chunk, exclusive);
+        DLFX_CHECK_LAUNCH();
+        return DLFX_OK;
+    }
+
+    const ScanLayout l = scan_layout(sizeof(T), m, n);
+    if (l.tiles > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+    if (scratch_bytes < l.total || (l.total && !scratch)) return DLFX_ERR_SCRATCH_TOO_SMALL;
+    unsigned* ticket = nullptr;
+    TileState<T> st;
+    st.bind(nullptr, 0);
+    if (l.tiles_per_row > 1) {
+        ticket = reinterpret_cast<unsigned*>(static_cast<char*>(scratch) + l.ticket_off);
+        st.bind(static_cast<char*>(scratch) + l.state_off, l.tiles);
+        scan_init<T><<<dim3(static_cast<unsigned>(ceil_div(l.tiles, kBlock))), dim3(kBlock), 0, stream>>>(ticket, st, l.tiles);
+        DLFX_CHECK_LAUNCH();
+    }
+    const int64_t tile = tile_elems(sizeof(T), n);
+    const dim3 grid(static_cast<unsigned>(l.tiles)), block(kBlock);
+    if (tile == 256)
+        scan_rows<T, K, 1><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, n, l.tiles_per_row, exclusive, ticket, st);
+    else if (tile == 1024)
+        scan_rows<T, K, 4><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, n, l.tiles_per_row, exclusive, ticket, st);
+    else
+        scan_rows<T, K, items_full<T>()><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, n, l.tiles_per_row, exclusive, ticket, st);
+    DLFX_CHECK_LAUNCH();
+    return DLFX_OK;
+}
+
+}  // namespace
+}  // namespace dlfx
+
+using namespace dlfx;
+
+extern "C" size_t dlfx_scan_scratch_bytes(int dtype, int64_t m, int64_t n) {
+    const size_t es = dtype_size(dtype);
+    if (!es || m <= 0 || n <= 0) return 0;
+    return scan_layout(es, m, n).total;
+}
+
+extern "C" int dlfx_scan(dlfx_stream_t stream, const char* name, int dtype, int64_t m, int64_t n,
+                         int exclusive, int rank, const int64_t* dims,
+                         const void* x, int64_t x_offset, const int64_t* x_strides,
+                         void* y, int64_t y_offset, const int64_t* y_strides,
+                         void* scratch, size_t scratch_bytes) {
+    if (!name || !x || !y || m <= 0 || n <= 0) return DLFX_ERR_INVALID_ARGUMENT;
+    if (!view_ok(rank, dims, x_strides) || !view_ok(rank, dims, y_strides)) return DLFX_ERR_INVALID_ARGUMENT;
+    if (rank < 1 || dims[rank - 1] != n || view_size(rank, dims) != m * n) return DLFX_ERR_INVALID_ARGUMENT;
+    int kind;
+    if (!std::strcmp(name, "cumsum")) kind = kScanAdd;
+    else if (!std::strcmp(name, "cumprod")) kind = kScanMul;
+    else if (!std::strcmp(name, "cummax")) kind = kScanMax;
+    else if (!std::strcmp(name, "cummin")) kind = kScanMin;
+    else return DLFX_ERR_UNKNOWN_OP;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dispatch_dtype(dtype, [&](auto tag) {
+        using T = decltype(tag);
+        const T* xp = static_cast<const T*>(x) + x_offset;
+        T* yp = static_cast<T*>(y) + y_offset;
+        switch (kind) {
+        case kScanAdd: return launch_scan<T, kScanAdd>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
+        case kScanMul: return launch_scan<T, kScanMul>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
+        case kScanMax: return launch_scan<T, kScanMax>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
+        default:       return launch_scan<T, kScanMin>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
+        }
+    });
+}

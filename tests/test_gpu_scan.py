@@ -1,0 +1,114 @@
+"""scan: HIP path vs the CPU oracle on the same seeded inputs.
+
+Integers are bit-exact (sums wrap).  fp32 prefixes are compared with the fp64
+scan: |got - o64| <= 4 ulp(fp32) * log2(n) * max(|o64|, running sum of |x|).
+cummax / cummin are exact for every dtype.
+"""
+import numpy as np
+import pytest
+
+from dlf_amd import frontend as F
+from dlf_amd.frontend import Tensor
+from helpers import normal, randint, full_range_i64, ulp_bound
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [1, 2, 63, 64, 65, 255, 256, 257, 1000, 1024, 1025, 4095, 4096, 4097, 8192, 12289, 100000]
+
+
+def both(hip, orc, x):
+    return Tensor.from_numpy(hip, x), Tensor.from_numpy(orc, x)
+
+
+@pytest.mark.parametrize("n", SIZES)
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_cumsum_rows_bit_exact(hip_backend, oracle_backend, n, dtype):
+    x = randint(41 + n, 3 * n, 0, 100).astype(dtype).reshape(3, n)
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    for exclusive in (False, True):
+        for reverse in (False, True):
+            g = F.cumsum(Xh, 1, exclusive, reverse).numpy()
+            w = F.cumsum(Xo, 1, exclusive, reverse).numpy()
+            assert np.array_equal(g, w), (exclusive, reverse)
+
+
+@pytest.mark.parametrize("shape,axis", [((5, 7, 300), 0), ((5, 7, 300), 1), ((5, 7, 300), 2),
+                                        ((4, 33, 20, 20), 1), ((2, 5000, 3), 1), ((300, 40), 0),
+                                        ((1000, 8), 1), ((70, 5000), 0), ((64, 2, 2), 1)])
+@pytest.mark.parametrize("dtype", [np.int32, np.int64, np.float64])
+def test_scan_any_axis(hip_backend, oracle_backend, shape, axis, dtype):
+    x = randint(42, int(np.prod(shape)), -50, 50).astype(dtype).reshape(shape)   # exact in every dtype
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    for exclusive in (False, True):
+        for reverse in (False, True):
+            g = F.cumsum(Xh, axis, exclusive, reverse).numpy()
+            w = F.cumsum(Xo, axis, exclusive, reverse).numpy()
+            assert np.array_equal(g, w), (exclusive, reverse)
+    assert np.array_equal(F.cummax(Xh, axis).numpy(), F.cummax(Xo, axis).numpy())
+    assert np.array_equal(F.cummin(Xh, axis, reverse=True).numpy(), F.cummin(Xo, axis, reverse=True).numpy())
+
+
+def test_cumprod_int_and_wrap(hip_backend, oracle_backend):
+    x = randint(43, 4 * 3000, 1, 4).astype(np.int64).reshape(4, 3000)
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    assert np.array_equal(F.cumprod(Xh, 1).numpy(), F.cumprod(Xo, 1).numpy())
+    y = full_range_i64(44, 2 * 100000).astype(np.int32).reshape(2, 100000)    # UniformTest.cpp:2188-2189 shape
+    Yh, Yo = both(hip_backend, oracle_backend, y)
+    assert np.array_equal(F.cumsum(Yh).numpy(), F.cumsum(Yo).numpy())
+    assert np.array_equal(F.cumsum(Yh).numpy(), np.cumsum(y, axis=1, dtype=np.int32))
+
+
+def test_in_place_and_views(hip_backend, oracle_backend):
+    x = randint(45, 6 * 5000, -9, 9).astype(np.int32).reshape(6, 5000)
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    F.cumsum(Xh, 1, out=Xh)
+    F.cumsum(Xo, 1, out=Xo)
+    assert np.array_equal(Xh.numpy(), Xo.numpy())
+    # sliced / stepped / transposed inputs written to fresh outputs
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    for args in (([1, 3], [5, 4999]), ([0, 4999], [6, 0], None, [2, -3])):
+        for axis in (0, 1):
+            g = F.cumsum(Xh.slice(*args), axis).numpy()
+            w = F.cumsum(Xo.slice(*args), axis).numpy()
+            assert np.array_equal(g, w)
+    g = F.cumsum(Xh.transpose(), 0, True).numpy()
+    assert np.array_equal(g, F.cumsum(Xo.transpose(), 0, True).numpy())
+
+
+@pytest.mark.parametrize("shape,axis", [((4, 100000), 1), ((3, 4097), 1), ((8, 64, 30, 30), 1), ((2, 1 << 20), 1)])
+def test_float_cumsum_tolerance(hip_backend, oracle_backend, shape, axis):
+    x = normal(46, int(np.prod(shape))).astype(np.float32).reshape(shape)
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    for exclusive in (False, True):
+        g = np.moveaxis(F.cumsum(Xh, axis, exclusive).numpy(), axis, -1).astype(np.float64)
+        n = shape[axis]
+        m = x.size // n
+        xs = Xo.shape.moveaxis(axis, -1)
+        want, mag = O.scan_f64("cumsum", 0, m, n, exclusive, xs, Xo.storage)
+        g = g.reshape(m, n)
+        bound = ulp_bound(n, np.maximum(np.abs(want), mag)) + 1e-30
+        err = np.abs(g - want)
+        assert (err <= bound).all(), "worst ratio %g" % (err / bound).max()
+        # the reference-association restatement satisfies the same bound
+        ref = np.moveaxis(F.cumsum(Xo, axis, exclusive).numpy(), axis, -1).reshape(m, n).astype(np.float64)
+        assert (np.abs(ref - want) <= bound).all()
+
+
+def test_float_cummax_exact_and_cumprod_close(hip_backend, oracle_backend):
+    x = normal(47, 5 * 20000).astype(np.float32).reshape(5, 20000)
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    assert np.array_equal(F.cummax(Xh, 1).numpy(), F.cummax(Xo, 1).numpy())
+    assert np.array_equal(F.cummin(Xh, 1).numpy(), F.cummin(Xo, 1).numpy())
+    y = (1.0 + 1e-3 * normal(48, 3 * 5000)).astype(np.float32).reshape(3, 5000)
+    Yh, Yo = both(hip_backend, oracle_backend, y)
+    np.testing.assert_allclose(F.cumprod(Yh, 1).numpy(), F.cumprod(Yo, 1).numpy(), rtol=2e-4)
+
+
+def test_many_rows_of_one_tile_and_long_single_row(hip_backend, oracle_backend):
+    x = randint(49, 3000 * 300, 0, 100).astype(np.int32).reshape(3000, 300)
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    assert np.array_equal(F.cumsum(Xh, 1).numpy(), F.cumsum(Xo, 1).numpy())
+    y = randint(50, 3_000_001, 0, 100).astype(np.int32).reshape(1, 3_000_001)
+    Yh = Tensor.from_numpy(hip_backend, y)
+    assert np.array_equal(F.cumsum(Yh, 1).numpy(), np.cumsum(y, axis=1, dtype=np.int32))
