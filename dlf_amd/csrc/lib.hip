@@ -12,6 +12,16 @@ int record_hip_error(hipError_t e) {
 
 }  // namespace dlfx
 
+namespace dlfx {
+bool set_scan_tuning(const char* key, int64_t value);
+}
+
+extern "C" int dlfx_set_tuning(const char* key, int64_t value) {
+    if (!key) return DLFX_ERR_INVALID_ARGUMENT;
+    if (dlfx::set_scan_tuning(key, value)) return DLFX_OK;
+    return DLFX_ERR_UNKNOWN_OP;
+}
+
 extern "C" int dlfx_version(void) { return 100; }
 
 extern "C" int dlfx_last_hip_error(void) { return dlfx::g_last_hip_error; }

@@ -6,8 +6,11 @@
 //     once.  Inside a tile each wave owns a contiguous segment that it loads
 //     with 128-bit accesses and scans with DPP row shifts / broadcasts; tiles of
 //     one row are chained with decoupled look-back (aggregate / inclusive-prefix
-//     words published with agent-scope atomics), tile ids come from an atomic
-//     ticket so a tile only ever waits for tiles that already started.
+//     words published with agent-scope atomics).  No wait is unbounded: when the
+//     output does not overlap the input, a tile that polled a predecessor's
+//     state too long computes that predecessor's aggregate from the input
+//     itself; when it does overlap (in-place scan) tile numbers are drawn from a
+//     per-row atomic ticket, so a tile only waits for tiles that are running.
 //   * scan_cols: many rows, scanned axis strided, a kept axis contiguous (e.g.
 //     cumsum over C of NCHW).  Lanes run along the kept axis so each load is a
 //     contiguous segment, the four waves of a workgroup take consecutive
@@ -54,6 +57,8 @@ struct ScanOp {
 
 // ------------------------------------------------------------------ look-back state
 constexpr uint32_t kInvalid = 0, kAggregate = 1, kInclusive = 2;
+// polls of one predecessor's state before a tile stops waiting for it (dlfx_set_tuning "scan_poll_limit")
+int g_poll_limit = 2048;
 
 // 4-byte values travel with their flag in one 64-bit word.
 template <typename T, int SIZE = sizeof(T)>
@@ -106,42 +111,36 @@ struct TileState<T, 8> {
 };
 
 template <typename T>
-__global__ __launch_bounds__(kBlock) void scan_init(unsigned* ticket, TileState<T> st, int64_t tiles) {
+__global__ __launch_bounds__(kBlock) void scan_init(unsigned* ticket, int64_t rows, TileState<T> st, int64_t tiles) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (i == 0) *ticket = 0u;
+    if (i < rows) ticket[i] = 0u;
     if (i < tiles) st.clear(i);
 }
 
-// ------------------------------------------------------------------ row kernel
-// Element order inside a tile: wave w owns [w*64*ITEMS, (w+1)*64*ITEMS); within
-// it, vector k of lane l covers elements (k*64 + l)*V .. +V.
-template <typename T, int K, int ITEMS>
-__global__ __launch_bounds__(kBlock) void scan_rows(
-    const T* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
-    int64_t n, int64_t tiles_per_row, int exclusive, unsigned* ticket, TileState<T> st) {
+// ------------------------------------------------------------------ row kernels
+template <typename T>
+struct RowScanShared {
+    T wave_total[kWaves];
+    T tile_prefix;
+    unsigned next_tile;
+};
+
+// One tile: tile `t` of row `row`.  Element order inside a tile: wave w owns
+// [w*64*ITEMS, (w+1)*64*ITEMS); within it, vector k of lane l covers elements
+// (k*64 + l)*V .. +V.  CHAINED tiles publish / look back through `st`.
+template <typename T, int K, int ITEMS, bool CHAINED, bool SELF_HELP>
+__device__ __forceinline__ void scan_tile(
+    const T* __restrict__ x, T* __restrict__ y, const DimMap& xmap, const DimMap& ymap, int64_t sx, int64_t sy,
+    int64_t n, int64_t tiles_per_row, int exclusive, int64_t row, int64_t t, int poll_limit,
+    TileState<T>& st, RowScanShared<T>& sm) {
     using Op = ScanOp<T, K>;
     constexpr int V = (vec_width<T>() < ITEMS) ? vec_width<T>() : ITEMS;
     constexpr int KV = ITEMS / V;
     constexpr int64_t TILE = static_cast<int64_t>(kBlock) * ITEMS;
     using VecT = Vec<T, V>;
 
-    __shared__ T wave_total[kWaves];
-    __shared__ T tile_prefix_sm;
-    __shared__ unsigned tile_id_sm;
-
     const int lane = lane_id();
     const int w = threadIdx.x / kWave;
-
-    int64_t tile_id;
-    if (tiles_per_row > 1) {
-        if (threadIdx.x == 0) tile_id_sm = atomicAdd(ticket, 1u);
-        __syncthreads();
-        tile_id = tile_id_sm;
-    } else {
-        tile_id = blockIdx.x;
-    }
-    const int64_t row = tile_id / tiles_per_row;
-    const int64_t t = tile_id - row * tiles_per_row;
     const int64_t tile_base = t * TILE;
     const int64_t avail = (n - tile_base < TILE) ? n - tile_base : TILE;   // valid elements in this tile
 
@@ -170,7 +169,6 @@ __global__ __launch_bounds__(kBlock) void scan_rows(
                 vals[k * V + e] = (i < n) ? xr[i * sx] : Op::identity();
             }
     }
-
     // ---- scan inside the wave: vals[] become inclusive prefixes within the wave segment
     T carry = Op::identity();
 #pragma unroll
@@ -186,21 +184,21 @@ __global__ __launch_bounds__(kBlock) void scan_rows(
         for (int e = 0; e < V; ++e) vals[k * V + e] = Op::apply(base, vals[k * V + e]);
         carry = Op::apply(carry, lane_read(incl, kWave - 1));
     }
-    if (lane == 0) wave_total[w] = carry;
+    if (lane == 0) sm.wave_total[w] = carry;
     __syncthreads();
 
     T wave_prefix = Op::identity();
     T aggregate = Op::identity();
 #pragma unroll
     for (int i = 0; i < kWaves; ++i) {
-        const T wt = wave_total[i];
+        const T wt = sm.wave_total[i];
         if (i < w) wave_prefix = Op::apply(wave_prefix, wt);
         aggregate = Op::apply(aggregate, wt);
     }
 
     // ---- chain tiles of this row
     T tile_prefix = Op::identity();
-    if (tiles_per_row > 1) {
+    if (CHAINED) {
         if (w == 0) {
             const int64_t sbase = row * tiles_per_row;
             if (lane == 0) st.publish(sbase + t, t == 0 ? kInclusive : kAggregate, aggregate);
@@ -213,9 +211,34 @@ __global__ __launch_bounds__(kBlock) void scan_rows(
                     uint32_t f = kInclusive;          // before the row: an inclusive identity
                     if (idx >= 0) {
                         f = st.read(sbase + idx, &v);
-                        while (f == kInvalid) {
-                            __builtin_amdgcn_s_sleep(1);
-                            f = st.read(sbase + idx, &v);
+                        if constexpr (SELF_HELP) {
+                            for (int polls = 0; f == kInvalid && polls < poll_limit; ++polls) {
+                                __builtin_amdgcn_s_sleep(1);
+                                f = st.read(sbase + idx, &v);
+                            }
+                        } else {
+                            while (f == kInvalid) {
+                                __builtin_amdgcn_s_sleep(1);
+                                f = st.read(sbase + idx, &v);
+                            }
+                        }
+                    }
+                    if constexpr (SELF_HELP) {
+                        // predecessors that still have nothing published: fold their tile of
+                        // the input here (the input is not being overwritten in this mode)
+                        unsigned long long stuck = __ballot(f == kInvalid);
+                        while (stuck != 0ull) {
+                            const int l = __ffsll(static_cast<long long>(stuck)) - 1;
+                            stuck &= stuck - 1;
+                            const int64_t pbase = (pos - l) * TILE;
+                            const int64_t cnt = (n - pbase < TILE) ? n - pbase : TILE;
+                            T a = Op::identity();
+                            for (int64_t i = lane; i < cnt; i += kWave) a = Op::apply(a, xr[(pbase + i) * sx]);
+                            a = wave_reduce(a, [](T p, T q) { return Op::apply(p, q); });
+                            if (lane == l) {
+                                v = a;
+                                f = kAggregate;
+                            }
                         }
                     }
                     const unsigned long long incl_mask = __ballot(f == kInclusive);
@@ -228,21 +251,21 @@ __global__ __launch_bounds__(kBlock) void scan_rows(
                 }
                 if (lane == 0) st.publish(sbase + t, kInclusive, Op::apply(excl, aggregate));
             }
-            if (lane == 0) tile_prefix_sm = excl;
+            if (lane == 0) sm.tile_prefix = excl;
         }
         __syncthreads();
-        tile_prefix = tile_prefix_sm;
+        tile_prefix = sm.tile_prefix;
     }
 
     // ---- combine and store
     const T pre = Op::apply(tile_prefix, wave_prefix);
     if (exclusive) {
         // element i receives the prefix of everything before it: shift by one element
-        // inside the lane's vector, and take the previous lane / vector / wave for e == 0
+        // inside the lane's vector, and take the previous lane / vector for e == 0
 #pragma unroll
         for (int k = KV - 1; k >= 0; --k) {
             const T last = vals[k * V + V - 1];
-            T prev = lane_get(last, lane - 1 < 0 ? 0 : lane - 1);      // inclusive prefix up to the previous lane's vector
+            T prev = lane_get(last, lane - 1 < 0 ? 0 : lane - 1);
             T prev_vec_end = (k > 0) ? lane_read(vals[(k > 0 ? k - 1 : 0) * V + V - 1], kWave - 1) : Op::identity();
             if (lane == 0) prev = prev_vec_end;
 #pragma unroll
@@ -272,6 +295,35 @@ __global__ __launch_bounds__(kBlock) void scan_rows(
                 if (i < n) yr[i * sy] = vals[k * V + e];
             }
     }
+}
+
+// Rows of a single tile: workgroup b scans row b.
+template <typename T, int K, int ITEMS>
+__global__ __launch_bounds__(kBlock) void scan_rows_single(
+    const T* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
+    int64_t n, int exclusive) {
+    __shared__ RowScanShared<T> sm;
+    TileState<T> st;
+    scan_tile<T, K, ITEMS, false, false>(x, y, xmap, ymap, sx, sy, n, 1, exclusive, blockIdx.x, 0, 0, st, sm);
+}
+
+// Rows of several tiles.  Workgroup b belongs to row b / tiles_per_row.  With
+// TICKET the tile of the row is drawn from that row's atomic counter (in-place
+// scans); without, it is the workgroup's position in the row and waits are
+// bounded by self-help.
+template <typename T, int K, int ITEMS, bool TICKET>
+__global__ __launch_bounds__(kBlock) void scan_rows_chained(
+    const T* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
+    int64_t n, int64_t tiles_per_row, int exclusive, int poll_limit, unsigned* ticket, TileState<T> st) {
+    __shared__ RowScanShared<T> sm;
+    const int64_t row = blockIdx.x / tiles_per_row;
+    int64_t t = blockIdx.x - row * tiles_per_row;
+    if constexpr (TICKET) {
+        if (threadIdx.x == 0) sm.next_tile = atomicAdd(&ticket[row], 1u);
+        __syncthreads();
+        t = sm.next_tile;
+    }
+    scan_tile<T, K, ITEMS, true, !TICKET>(x, y, xmap, ymap, sx, sy, n, tiles_per_row, exclusive, row, t, poll_limit, st, sm);
 }
 
 // ------------------------------------------------------------------ column kernel
@@ -365,12 +417,11 @@ bool make_dim_map2(const int64_t* dims, const int64_t* sx, const int64_t* sy, in
     return true;
 }
 
-template <typename T>
-constexpr int items_full() { return 64 / sizeof(T); }   // 64 bytes per thread
-
+// Elements per tile: 256 bytes per thread for chained rows, less for short rows.
 int64_t tile_elems(size_t elem_size, int64_t n) {
-    const int64_t full = 256 * (64 / static_cast<int64_t>(elem_size));
-    if (n > 1024) return full;
+    const int64_t full = 256 * (256 / static_cast<int64_t>(elem_size));
+    if (n > full / 4) return full;
+    if (n > 1024) return full / 4;
     if (n > 256) return 1024;
     return 256;
 }
@@ -385,15 +436,27 @@ ScanLayout scan_layout(size_t elem_size, int64_t m, int64_t n) {
     l.tiles_per_row = ceil_div(n, tile_elems(elem_size, n));
     l.tiles = m * l.tiles_per_row;
     l.ticket_off = 0;
-    l.state_off = 256;
+    l.state_off = align_up(static_cast<size_t>(m) * 4, 256);
     if (l.tiles_per_row <= 1) {
         l.total = 0;
     } else {
         size_t sb = elem_size == 4 ? static_cast<size_t>(l.tiles) * 8
                                    : align_up(static_cast<size_t>(l.tiles) * 4, 256) + static_cast<size_t>(l.tiles) * 16;
-        l.total = 256 + align_up(sb, 256);
+        l.total = l.state_off + align_up(sb, 256);
     }
     return l;
+}
+
+// True when the element ranges the two views touch intersect.
+template <typename T>
+bool views_overlap(int rank, const int64_t* dims, const T* x, const int64_t* sx, const T* y, const int64_t* sy) {
+    int64_t xlo = 0, xhi = 0, ylo = 0, yhi = 0;
+    for (int i = 0; i < rank; ++i) {
+        const int64_t ex = (dims[i] - 1) * sx[i], ey = (dims[i] - 1) * sy[i];
+        if (ex > 0) xhi += ex; else xlo += ex;
+        if (ey > 0) yhi += ey; else ylo += ey;
+    }
+    return !(x + xhi < y + ylo || y + yhi < x + xlo);
 }
 
 template <typename T, int K>
@@ -424,23 +487,34 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     const ScanLayout l = scan_layout(sizeof(T), m, n);
     if (l.tiles > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
     if (scratch_bytes < l.total || (l.total && !scratch)) return DLFX_ERR_SCRATCH_TOO_SMALL;
-    unsigned* ticket = nullptr;
-    TileState<T> st;
-    st.bind(nullptr, 0);
-    if (l.tiles_per_row > 1) {
-        ticket = reinterpret_cast<unsigned*>(static_cast<char*>(scratch) + l.ticket_off);
-        st.bind(static_cast<char*>(scratch) + l.state_off, l.tiles);
-        scan_init<T><<<dim3(static_cast<unsigned>(ceil_div(l.tiles, kBlock))), dim3(kBlock), 0, stream>>>(ticket, st, l.tiles);
-        DLFX_CHECK_LAUNCH();
-    }
     const int64_t tile = tile_elems(sizeof(T), n);
-    const dim3 grid(static_cast<unsigned>(l.tiles)), block(kBlock);
-    if (tile == 256)
-        scan_rows<T, K, 1><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, n, l.tiles_per_row, exclusive, ticket, st);
-    else if (tile == 1024)
-        scan_rows<T, K, 4><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, n, l.tiles_per_row, exclusive, ticket, st);
+    constexpr int FULL = 256 / sizeof(T);
+    const dim3 block(kBlock);
+    if (l.tiles_per_row == 1) {
+        const dim3 grid(static_cast<unsigned>(m));
+        if (tile == 256)
+            scan_rows_single<T, K, 1><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, n, exclusive);
+        else if (tile == 1024)
+            scan_rows_single<T, K, 4><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, n, exclusive);
+        else if (tile == 256 * (FULL / 4))
+            scan_rows_single<T, K, FULL / 4><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, n, exclusive);
+        else
+            scan_rows_single<T, K, FULL><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, n, exclusive);
+        DLFX_CHECK_LAUNCH();
+        return DLFX_OK;
+    }
+    unsigned* ticket = reinterpret_cast<unsigned*>(static_cast<char*>(scratch) + l.ticket_off);
+    TileState<T> st;
+    st.bind(static_cast<char*>(scratch) + l.state_off, l.tiles);
+    scan_init<T><<<dim3(static_cast<unsigned>(ceil_div(l.tiles, kBlock))), block, 0, stream>>>(ticket, m, st, l.tiles);
+    DLFX_CHECK_LAUNCH();
+    const dim3 grid(static_cast<unsigned>(l.tiles));
+    if (views_overlap(rank, dims, x, x_strides, y, y_strides))
+        scan_rows_chained<T, K, FULL, true><<<grid, block, 0, stream>>>(
+            x, y, xmap, ymap, sx, sy, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st);
     else
-        scan_rows<T, K, items_full<T>()><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, n, l.tiles_per_row, exclusive, ticket, st);
+        scan_rows_chained<T, K, FULL, false><<<grid, block, 0, stream>>>(
+            x, y, xmap, ymap, sx, sy, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st);
     DLFX_CHECK_LAUNCH();
     return DLFX_OK;
 }
@@ -449,6 +523,16 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
 }  // namespace dlfx
 
 using namespace dlfx;
+
+namespace dlfx {
+bool set_scan_tuning(const char* key, int64_t value) {
+    if (!std::strcmp(key, "scan_poll_limit") && value >= 0 && value <= (1 << 30)) {
+        g_poll_limit = static_cast<int>(value);
+        return true;
+    }
+    return false;
+}
+}  // namespace dlfx
 
 extern "C" size_t dlfx_scan_scratch_bytes(int dtype, int64_t m, int64_t n) {
     const size_t es = dtype_size(dtype);

@@ -30,6 +30,8 @@ def _declare(lib):
     lib.dlfx_status_string.restype = c_char_p
     lib.dlfx_status_string.argtypes = [c_int]
     lib.dlfx_last_hip_error.restype = c_int
+    lib.dlfx_set_tuning.restype = c_int
+    lib.dlfx_set_tuning.argtypes = [c_char_p, c_int64]
 
     lib.dlfx_reduce_scratch_bytes.restype = c_size_t
     lib.dlfx_reduce_scratch_bytes.argtypes = [c_int, c_int64, c_int64]
@@ -73,7 +75,7 @@ def _declare(lib):
 _lib = None
 
 # Every symbol include/dlfx.h declares.
-EXPORTS = ("dlfx_version", "dlfx_status_string", "dlfx_last_hip_error",
+EXPORTS = ("dlfx_version", "dlfx_status_string", "dlfx_last_hip_error", "dlfx_set_tuning",
            "dlfx_reduce_scratch_bytes", "dlfx_reduce",
            "dlfx_arg_reduce_scratch_bytes", "dlfx_arg_reduce",
            "dlfx_scan_scratch_bytes", "dlfx_scan",
@@ -203,6 +205,9 @@ class HipBackend:
                                    x.data_ptr(), xs.offset, _arr(xs.strides),
                                    y.data_ptr(), ys.offset, _arr(ys.strides),
                                    i.data_ptr(), is_.offset, _arr(is_.strides), sp, sb), "dlfx_top_k")
+
+    def set_tuning(self, key: str, value: int):
+        _check(self.lib.dlfx_set_tuning(key.encode(), value), "dlfx_set_tuning(%s)" % key)
 
     def synchronize(self):
         self.torch.cuda.synchronize(self.device)

@@ -68,6 +68,14 @@ const char* dlfx_status_string(int status);
 /* hipError_t of the last DLFX_ERR_LAUNCH on the calling thread (0 if none). */
 int dlfx_last_hip_error(void);
 
+/* Process-wide tuning knobs (not thread-safe against running calls).  Keys:
+ *   "scan_poll_limit"  how many times a scan tile polls a predecessor's published
+ *                      state before it folds that predecessor's input itself
+ *                      (default 2048; 0 makes every tile help itself at once).
+ * Returns DLFX_ERR_UNKNOWN_OP for an unknown key or out-of-range value.  No
+ * counterpart in the reference (its database/ tuning tables play this role). */
+int dlfx_set_tuning(const char* key, int64_t value);
+
 /* ---------------------------------------------------------------- reduce
  * Replaces gpgpu::dnn::reduce<T> (gdnn.h:108-114; caller
  * dlf/include/tensor/reduce_detail.h:91-101).  x_dims lists the kept extents

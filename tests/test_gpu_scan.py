@@ -112,3 +112,38 @@ def test_many_rows_of_one_tile_and_long_single_row(hip_backend, oracle_backend):
     y = randint(50, 3_000_001, 0, 100).astype(np.int32).reshape(1, 3_000_001)
     Yh = Tensor.from_numpy(hip_backend, y)
     assert np.array_equal(F.cumsum(Yh, 1).numpy(), np.cumsum(y, axis=1, dtype=np.int32))
+
+
+def test_bounded_wait_self_help_path(hip_backend, oracle_backend):
+    # With a poll limit of 0 a tile never waits: whatever predecessor has not
+    # published yet is folded from the input by the waiting tile itself.
+    x = randint(51, 5 * 200000, -100, 100).astype(np.int32).reshape(5, 200000)
+    y = randint(52, 3 * 70000, -10**9, 10**9).astype(np.int64).reshape(3, 70000)
+    hip_backend.set_tuning("scan_poll_limit", 0)
+    try:
+        for a in (x, y):
+            Xh, Xo = both(hip_backend, oracle_backend, a)
+            for exclusive in (False, True):
+                for reverse in (False, True):
+                    g = F.cumsum(Xh, 1, exclusive, reverse).numpy()
+                    assert np.array_equal(g, F.cumsum(Xo, 1, exclusive, reverse).numpy())
+            assert np.array_equal(F.cummax(Xh, 1).numpy(), F.cummax(Xo, 1).numpy())
+    finally:
+        hip_backend.set_tuning("scan_poll_limit", 2048)
+
+
+def test_in_place_long_rows_use_tickets(hip_backend, oracle_backend):
+    x = randint(53, 4 * 300000, -100, 100).astype(np.int32).reshape(4, 300000)
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    F.cumsum(Xh, 1, out=Xh)
+    F.cumsum(Xo, 1, out=Xo)
+    assert np.array_equal(Xh.numpy(), Xo.numpy())
+    # In-place *exclusive* scans: the reference's CPU loop stores the running value
+    # into y before it reads x (reduce_detail.h:183-187), so with y aliasing x it
+    # loses the input it has yet to read.  That is a read-after-write slip, not a
+    # specification; the HIP path must equal the out-of-place answer.
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    F.cumsum(Xh, 1, True, True, out=Xh)
+    assert np.array_equal(Xh.numpy(), F.cumsum(Xo, 1, True, True).numpy())
+    F.cumsum(Xo, 1, True, True, out=Xo)
+    assert not np.array_equal(Xo.numpy(), Xh.numpy())     # the restated reference loop reproduces the slip
