@@ -72,6 +72,7 @@ int dlfx_last_hip_error(void);
  *   "scan_poll_limit"  how many times a scan tile polls a predecessor's published
  *                      state before it folds that predecessor's input itself
  *                      (default 2048; 0 makes every tile help itself at once).
+ *   "sort_poll_limit"  the same bound for the per-digit tile chaining of a radix pass.
  * Returns DLFX_ERR_UNKNOWN_OP for an unknown key or out-of-range value.  No
  * counterpart in the reference (its database/ tuning tables play this role). */
 int dlfx_set_tuning(const char* key, int64_t value);

@@ -1,0 +1,132 @@
+"""sort / argsort: HIP path vs the CPU oracle, bit-exact.
+
+Values must equal the restated reference merge sort; argsort indices must equal
+the stable order (lowest source index first among equal keys, both directions),
+which no reference test pins -- it is pinned against numpy's stable argsort in
+the CPU suite -- and gather(X, I) must reproduce the sorted values.
+"""
+import numpy as np
+import pytest
+
+from dlf_amd import frontend as F
+from dlf_amd.frontend import Tensor
+from helpers import normal, randint, full_range_i64, uniform01
+
+pytestmark = pytest.mark.gpu
+
+
+def both(hip, orc, x):
+    return Tensor.from_numpy(hip, x), Tensor.from_numpy(orc, x)
+
+
+def make(dtype, seed, count, dup):
+    if dup:
+        return randint(seed, count, -6, 6).astype(dtype)
+    if np.dtype(dtype) == np.int64:
+        return full_range_i64(seed, count)
+    if np.dtype(dtype) == np.int32:
+        return full_range_i64(seed, count).astype(np.int32)
+    return (normal(seed, count) * 1e3).astype(dtype)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.int32, np.int64, np.float64])
+@pytest.mark.parametrize("n", [2, 3, 10, 100, 1000, 4095, 4096, 4097, 10000, 70001])
+def test_sort_rows_sizes(hip_backend, oracle_backend, dtype, n):
+    for dup in (False, True):
+        x = make(dtype, 60 + n, 2 * n, dup).reshape(2, n)
+        Xh, Xo = both(hip_backend, oracle_backend, x)
+        for desc in (False, True):
+            g = F.sort(Xh, -1, desc).numpy()
+            assert np.array_equal(g, F.sort(Xo, -1, desc).numpy()), (desc, dup)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.int64])
+@pytest.mark.parametrize("axis", [0, 1, 2])
+def test_sort_any_axis_and_in_place(hip_backend, oracle_backend, dtype, axis):
+    x = make(dtype, 61, 6 * 50 * 40, True).reshape(6, 50, 40)
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    for desc in (False, True):
+        assert np.array_equal(F.sort(Xh, axis, desc).numpy(), F.sort(Xo, axis, desc).numpy())
+    F.sort(Xh, axis, out=Xh)
+    assert np.array_equal(Xh.numpy(), np.sort(x, axis=axis))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.int32, np.int64, np.float64])
+@pytest.mark.parametrize("n", [2, 10, 257, 1000, 4096, 4097, 10000, 70001])
+def test_argsort_stable_both_directions(hip_backend, oracle_backend, dtype, n):
+    for dup in (True, False):
+        x = make(dtype, 62 + n, 2 * n, dup).reshape(2, n)
+        Xh, Xo = both(hip_backend, oracle_backend, x)
+        for desc in (False, True):
+            Ih = F.argsort(Xh, -1, desc).numpy()
+            Io = F.argsort(Xo, -1, desc).numpy()
+            assert Ih.dtype == np.int32 and np.array_equal(Ih, Io), (desc, dup)
+            Yh, Ih2 = F.argsort(Xh, -1, desc, with_values=True)
+            Yo, _ = F.argsort(Xo, -1, desc, with_values=True)
+            assert np.array_equal(Ih2.numpy(), Io)
+            assert np.array_equal(Yh.numpy(), Yo.numpy())
+            assert np.array_equal(F.gather_elements(x, Ih, -1), Yo.numpy())
+
+
+@pytest.mark.parametrize("axis", [0, 1, 2])
+def test_argsort_axes_int64_indices_and_in_place_values(hip_backend, oracle_backend, axis):
+    x = make(np.int32, 63, 5 * 30 * 20, True).reshape(5, 30, 20)
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    I64 = F.argsort(Xh, axis, index_dtype=np.int64).numpy()
+    assert I64.dtype == np.int64 and np.array_equal(I64, F.argsort(Xo, axis).numpy())
+    # values written over the input (UniformTest.cpp:2419: argsort(Y, Y, I, axis))
+    Yh, Ih = F.argsort(Xh, axis, values=Xh)
+    assert np.array_equal(Yh.numpy(), np.sort(x, axis=axis))
+    assert np.array_equal(F.gather_elements(x, Ih.numpy(), axis), np.sort(x, axis=axis))
+
+
+def test_argsort_signed_zeros_are_one_key(hip_backend):
+    x = np.array([[0.0, -0.0, 1.0, -0.0, 0.0, -1.0, -0.0]], dtype=np.float32)
+    X = Tensor.from_numpy(hip_backend, x)
+    Y, I = F.argsort(X, -1, with_values=True)
+    assert I.numpy().tolist() == [[5, 0, 1, 3, 4, 6, 2]]
+    assert np.array_equal(np.signbit(Y.numpy()), np.signbit(x[0][I.numpy()[0]])[None, :])
+    Y, I = F.argsort(X, -1, True, with_values=True)
+    assert I.numpy().tolist() == [[2, 0, 1, 3, 4, 6, 5]]
+
+
+def test_extent_one_axis_copies(hip_backend):
+    x = make(np.float32, 64, 7, False).reshape(7, 1)
+    X = Tensor.from_numpy(hip_backend, x)
+    assert np.array_equal(F.sort(X, 1).numpy(), x)
+    Y, I = F.argsort(X, 1, with_values=True)
+    assert np.array_equal(Y.numpy(), x) and not I.numpy().any()
+
+
+def test_quantised_heavy_duplicates_and_full_range(hip_backend, oracle_backend):
+    # the two benchmark input families at reduced size
+    x = (np.floor(uniform01(65, 8 * 65536) * 4096) / 4096).astype(np.float32).reshape(8, 65536)
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    for desc in (False, True):
+        assert np.array_equal(F.sort(Xh, -1, desc).numpy(), F.sort(Xo, -1, desc).numpy())
+        assert np.array_equal(F.argsort(Xh, -1, desc).numpy(), F.argsort(Xo, -1, desc).numpy())
+    y = full_range_i64(66, 2 * (1 << 18)).reshape(2, 1 << 18)
+    Yh, Yo = both(hip_backend, oracle_backend, y)
+    for desc in (False, True):
+        assert np.array_equal(F.sort(Yh, -1, desc).numpy(), F.sort(Yo, -1, desc).numpy())
+        assert np.array_equal(F.argsort(Yh, -1, desc).numpy(), F.argsort(Yo, -1, desc).numpy())
+
+
+def test_bounded_wait_self_help_path(hip_backend, oracle_backend):
+    x = make(np.int32, 67, 3 * 50000, True).reshape(3, 50000)
+    y = full_range_i64(68, 2 * 30000).reshape(2, 30000)
+    hip_backend.set_tuning("sort_poll_limit", 0)
+    try:
+        for a in (x, y):
+            Xh, Xo = both(hip_backend, oracle_backend, a)
+            assert np.array_equal(F.sort(Xh, -1, True).numpy(), F.sort(Xo, -1, True).numpy())
+            assert np.array_equal(F.argsort(Xh, -1).numpy(), F.argsort(Xo, -1).numpy())
+    finally:
+        hip_backend.set_tuning("sort_poll_limit", 2048)
+
+
+def test_many_short_rows(hip_backend, oracle_backend):
+    x = make(np.float32, 69, 3000 * 17, True).reshape(3000, 17)
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    assert np.array_equal(F.sort(Xh, -1).numpy(), F.sort(Xo, -1).numpy())
+    assert np.array_equal(F.argsort(Xh, 0).numpy(), F.argsort(Xo, 0).numpy())
