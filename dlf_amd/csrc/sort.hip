@@ -523,7 +523,34 @@ bool set_sort_tuning(const char* key, int64_t value) {
     return false;
 }
 
-// Used by top_k for rows or limits its selection kernel does not take.
+// Used by top_k for rows or limits its selection kernel does not take: stable
+// argsort of a strided view into contiguous value and int32 index arrays.
+int argsort_contiguous(hipStream_t stream, int dir, int dtype, int rank, const int64_t* dims,
+                       const void* x, const int64_t* x_strides, void* y_contig, int32_t* idx_contig,
+                       void* scratch, size_t scratch_bytes) {
+    if (rank < 1 || rank > 64) return DLFX_ERR_INVALID_ARGUMENT;
+    int64_t cs[64];
+    int64_t acc = 1;
+    for (int i = rank - 1; i >= 0; --i) {
+        cs[i] = acc;
+        acc *= dims[i];
+    }
+    SortArgs a{};
+    a.dir = dir;
+    a.rank = rank;
+    a.dims = dims;
+    a.x = x;
+    a.xs = x_strides;
+    a.y = y_contig;
+    a.ys = cs;
+    a.idx = idx_contig;
+    a.is = cs;
+    a.idx64 = 0;
+    a.pairs = true;
+    return sort_entry(stream, dtype, a, scratch, scratch_bytes);
+}
+
+
 size_t argsort_scratch_bytes_impl(int dtype, int64_t m, int64_t n) {
     const size_t es = dtype_size(dtype);
     if (!es || m <= 0 || n <= 0) return 0;

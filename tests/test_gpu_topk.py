@@ -1,0 +1,108 @@
+"""top_k: HIP path vs the CPU oracle, bit-exact.
+
+Values must equal what the reference's heap algorithm returns (restated in the
+oracle, mode 0).  Indices must equal the specification order -- first `limit`
+entries of a stable sort, so the lowest index wins ties (oracle mode 1; the
+reference's own tie order is implementation-defined and its test concedes the
+indices may differ) -- and gather(X, I) must reproduce the values.
+"""
+import numpy as np
+import pytest
+
+from dlf_amd import frontend as F
+from dlf_amd.frontend import Tensor
+from helpers import normal, randint, full_range_i64
+from oracle.oracle import OracleBackend
+
+pytestmark = pytest.mark.gpu
+
+
+def check(hip, x, k, axis=-1, largest=True, index_dtype=np.int32):
+    spec, heap = OracleBackend(topk_mode=1), OracleBackend(topk_mode=0)
+    Yh, Ih = F.top_k(Tensor.from_numpy(hip, x), k, axis, largest, index_dtype)
+    Ys, Is = F.top_k(Tensor.from_numpy(spec, x), k, axis, largest, index_dtype)
+    Yr, _ = F.top_k(Tensor.from_numpy(heap, x), k, axis, largest, index_dtype)
+    yh, ih = Yh.numpy(), Ih.numpy()
+    assert ih.dtype == np.dtype(index_dtype)
+    assert np.array_equal(yh, Ys.numpy()) and np.array_equal(yh, Yr.numpy())
+    assert np.array_equal(ih, Is.numpy())
+    assert np.array_equal(F.gather_elements(x, ih, axis), yh)
+
+
+def quantised(seed, shape):
+    return (np.round(normal(seed, int(np.prod(shape))) * 2 * 256) / 256).astype(np.float32).reshape(shape)
+
+
+@pytest.mark.parametrize("k", [1, 5, 50, 256])
+@pytest.mark.parametrize("largest", [True, False])
+def test_quantised_rows_with_ties(hip_backend, k, largest):
+    check(hip_backend, quantised(70, (24, 32000)), k, -1, largest)           # benchmark row shape
+    check(hip_backend, quantised(71, (40, 1000)), k, -1, largest, np.int64)  # logits-head shape
+
+
+@pytest.mark.parametrize("n", [1, 2, 10, 255, 256, 257, 1000, 1024, 1025, 2048, 4097, 8192, 10000, 16385, 32769, 65536])
+def test_row_lengths(hip_backend, n):
+    x = randint(72 + n, 3 * n, 0, 50).astype(np.int32).reshape(3, n)       # heavy ties
+    for k in sorted({1, min(n, 7), min(n, 200), min(n, 1024)}):
+        check(hip_backend, x, k, -1, True)
+        check(hip_backend, x, k, -1, False)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int64])
+def test_dtypes_and_axes(hip_backend, dtype):
+    if np.dtype(dtype).kind == "f":
+        x = (normal(73, 6 * 40 * 30) * 100).astype(dtype).reshape(6, 40, 30)
+    else:
+        x = full_range_i64(73, 6 * 40 * 30).astype(dtype).reshape(6, 40, 30)
+    for axis in (0, 1, 2):
+        check(hip_backend, x, 5, axis, True)
+        check(hip_backend, x, 3, axis, False, np.int64)
+
+
+def test_reference_test_shapes(hip_backend):
+    # UniformTest.cpp:2494-2535: [2, n] ints, k = 10 / 200 / 500 / 1000
+    for n in (10, 500, 1000):
+        check(hip_backend, randint(74 + n, 2 * n, 0, 10000).astype(np.int32).reshape(2, n), 10)
+    for n in (1000, 5000, 10000):
+        x = randint(75 + n, 2 * n, 0, 100000).astype(np.int32).reshape(2, n)
+        for k in (200, 500, 1000):
+            check(hip_backend, x, k)
+
+
+def test_all_equal_rows_and_k_equals_n(hip_backend):
+    x = np.full((4, 3000), 7, dtype=np.int64)
+    Y, I = F.top_k(Tensor.from_numpy(hip_backend, x), 100)
+    assert np.array_equal(I.numpy(), np.tile(np.arange(100, dtype=np.int32), (4, 1)))
+    assert (Y.numpy() == 7).all()
+    y = randint(76, 5 * 300, -5, 5).astype(np.int32).reshape(5, 300)
+    check(hip_backend, y, 300)
+    check(hip_backend, y, 1000)          # limit clamps to the extent
+
+
+def test_long_rows_and_large_limits_take_the_sort_path(hip_backend):
+    check(hip_backend, quantised(77, (3, 100000)), 50)
+    check(hip_backend, randint(78, 2 * 20000, 0, 1000).astype(np.int32).reshape(2, 20000), 3000, -1, False)
+    check(hip_backend, full_range_i64(79, 2 * 40000).reshape(2, 40000), 10, -1, True, np.int64)
+
+
+def test_signed_zeros_and_infinities(hip_backend):
+    x = np.array([[0.0, -0.0, -1.0, -0.0, np.inf, -np.inf, 0.0, 3.0]], dtype=np.float32)
+    Y, I = F.top_k(Tensor.from_numpy(hip_backend, x), 5)
+    assert I.numpy().tolist() == [[4, 7, 0, 1, 3]]
+    assert np.array_equal(np.signbit(Y.numpy()[0]), np.signbit(x[0][I.numpy()[0]]))
+    Y, I = F.top_k(Tensor.from_numpy(hip_backend, x), 4, largest=False)
+    assert I.numpy().tolist() == [[5, 2, 0, 1]]
+
+
+def test_strided_views(hip_backend):
+    x = randint(80, 40 * 700, 0, 30).astype(np.int32).reshape(40, 700)
+    X = Tensor.from_numpy(hip_backend, x)
+    from oracle.oracle import OracleBackend as OB
+    Xo = Tensor.from_numpy(OB(1), x)
+    for args in (([3, 5], [37, 690]), ([0, 699], [40, 0], None, [3, -2])):
+        Yh, Ih = F.top_k(X.slice(*args), 9, -1)
+        Yo, Io = F.top_k(Xo.slice(*args), 9, -1)
+        assert np.array_equal(Yh.numpy(), Yo.numpy()) and np.array_equal(Ih.numpy(), Io.numpy())
+        Yh, Ih = F.top_k(X.slice(*args), 4, 0, False)
+        Yo, Io = F.top_k(Xo.slice(*args), 4, 0, False)
+        assert np.array_equal(Yh.numpy(), Yo.numpy()) and np.array_equal(Ih.numpy(), Io.numpy())
