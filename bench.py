@@ -1,0 +1,409 @@
+#!/usr/bin/env python3
+"""Benchmark of the axis primitives on one MI355X.
+
+A step is one pass of the scan / long-reduce configuration (BASELINE.json
+configs[1]): inclusive cumsum along the last axis of int32 [64, 2^20] and of
+fp32 [64, 2^20], then a 1-D fp32 reduce_sum over 2^30 elements, all inputs
+resident in HBM before the timed region starts.  `value` is the algorithmic
+bytes of the step (every input element read once, every output element written
+once) divided by the wall time of the K timed steps.
+
+Per-operation figures for every configuration (Gelem/s, GB/s, fraction of the
+8 TB/s HBM peak) are reported in `per_op`; `roofline` describes the kernel that
+dominates the step; `cpu_baseline` times the CPU restatement of the reference's
+algorithm on this box's host cores on a bounded sample of the same workload.
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs all|step] [--no-cpu]
+Prints ONE JSON line on stdout.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+METRIC = "HBM GB/s (% of ~8 TB/s peak) + Gelem/s per op: reduce, scan, top_k, sort"
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+class Op:
+    """One measured operation: a list of prepared calls over rotated input buffers."""
+
+    def __init__(self, config, name, elems, alg_bytes, calls, verify=None, kernel=None):
+        self.config, self.name, self.elems, self.alg_bytes = config, name, elems, alg_bytes
+        self.calls, self.verify, self.kernel = calls, verify, kernel
+        self._i = 0
+
+    def issue(self):
+        self.calls[self._i % len(self.calls)]()
+        self._i += 1
+
+
+def make_ops(be, which):
+    import numpy as np
+    import torch
+    from dlf_amd import frontend as F
+    from dlf_amd import synth
+    from dlf_amd.frontend import Tensor, dtype_code, prepare_reduce
+    from dlf_amd.shape import Shape
+
+    dev = be.device
+    np_of = {torch.float32: np.float32, torch.int32: np.int32, torch.int64: np.int64, torch.float64: np.float64}
+
+    def tensor(t):
+        return Tensor(be, Shape(list(t.shape)), t.view(-1), np_of[t.dtype])
+
+    def gen(shape, dtype, fn, copies):
+        out = []
+        for c in range(copies):
+            t = torch.empty(shape, dtype=dtype, device=dev)
+            synth.fill(t, fn(c))
+            out.append(t)
+        return out
+
+    def empty(shape, dtype):
+        return torch.empty(shape, dtype=dtype, device=dev)
+
+    def reduce_calls(name, xs, axes):
+        calls, outs = [], []
+        for x in xs:
+            X = tensor(x)
+            view, out_dims, m, n = prepare_reduce(X.shape, list(axes), False)
+            Y = Tensor.empty(be, out_dims, X.dtype)
+            calls.append(be.reduce(name, dtype_code(X.dtype), m, n, view, X.storage, Y.shape, Y.storage, defer=True))
+            outs.append(Y)
+        return calls, outs
+
+    def argmax_calls(xs, axis):
+        calls, outs = [], []
+        for x in xs:
+            X = tensor(x)
+            view = X.shape.moveaxis(axis, -1)
+            y_dims = [e for i, e in enumerate(X.shape.extents) if i != axis]
+            Y = Tensor.empty(be, y_dims, np.int32)
+            k = view.extents[-1]
+            calls.append(be.arg_reduce("argmax", dtype_code(X.dtype), 2, view.size // k, k, view, X.storage,
+                                       Y.shape, Y.storage, defer=True))
+            outs.append(Y)
+        return calls, outs
+
+    def scan_calls(xs, axis):
+        y = empty(xs[0].shape, xs[0].dtype)
+        Y = tensor(y)
+        calls = []
+        for x in xs:
+            X = tensor(x)
+            n = X.shape.extents[axis]
+            calls.append(be.scan("cumsum", dtype_code(X.dtype), X.size // n, n, False,
+                                 X.shape.moveaxis(axis, -1), X.storage, Y.shape.moveaxis(axis, -1), Y.storage, defer=True))
+        return calls, y
+
+    ops = []
+
+    # ---------------- C2: scans and the long reduce (the step)
+    if which in ("all", "step", "c2"):
+        xi = gen((64, 1 << 20), torch.int32, lambda c: synth.randint(2 + 100 * c, 0, 100), 4)
+        calls, y = scan_calls(xi, 1)
+
+        def v_c2a(xi=xi, y=y, call=calls[0]):
+            call()
+            assert torch.equal(y, torch.cumsum(xi[0], 1, dtype=torch.int32)), "C2a cumsum int32 not bit-exact"
+        ops.append(Op("C2a", "cumsum_i32_[64,2^20]", 64 << 20, 2 * 4 * (64 << 20), calls, v_c2a, "scan_rows_chained"))
+
+        xf = gen((64, 1 << 20), torch.float32, lambda c: synth.normal(3 + 100 * c), 4)
+        calls, yf = scan_calls(xf, 1)
+
+        def v_c2b(xf=xf, y=yf, call=calls[0]):
+            call()
+            want = torch.cumsum(xf[0].double(), 1)
+            mag = torch.cumsum(xf[0].double().abs(), 1)
+            tol = 4 * 20 * float(np.finfo(np.float32).eps) * torch.maximum(want.abs(), mag)
+            assert bool(((y.double() - want).abs() <= tol).all()), "C2b cumsum fp32 out of tolerance"
+        ops.append(Op("C2b", "cumsum_f32_[64,2^20]", 64 << 20, 2 * 4 * (64 << 20), calls, v_c2b, "scan_rows_chained"))
+
+        xl = gen((1 << 30,), torch.float32, lambda c: synth.unit_interval_exact(4), 1)
+        calls, outs = reduce_calls("reduce_sum", xl, [])
+
+        def v_c2c(xl=xl, out=outs[0], call=calls[0]):
+            call()
+            # every element is a multiple of 2^-23 below 1 in magnitude: the fp64 sum is exact
+            want = float(xl[0].double().sum())
+            got = float(out.storage[0])
+            assert abs(got - want) <= 4 * 30 * float(np.finfo(np.float32).eps) * max(abs(want), 1.0), (got, want)
+        ops.append(Op("C2c", "reduce_sum_f32_[2^30]", 1 << 30, 4 * (1 << 30) + 4, calls, v_c2c, "reduce_rows_block"))
+
+    # ---------------- C1: logits head
+    if which in ("all", "c1"):
+        x1 = gen((256, 1000), torch.float32, lambda c: synth.normal(1 + 100 * c), 8)
+        for name in ("reduce_sum", "reduce_max", "reduce_log_sum_exp"):
+            calls, outs = reduce_calls(name, x1, [1])
+
+            def v(name=name, x=x1[0], out=outs[0], call=calls[0]):
+                call()
+                ref = {"reduce_sum": lambda t: t.double().sum(1), "reduce_max": lambda t: t.double().amax(1),
+                       "reduce_log_sum_exp": lambda t: torch.logsumexp(t.double(), 1)}[name](x)
+                assert torch.allclose(out.storage[:256].double(), ref, rtol=1e-5, atol=1e-5), name
+            ops.append(Op("C1", name + "_f32_[256,1000]", 256000, 1024000 + 1024, calls, v))
+        calls, outs = argmax_calls(x1, 1)
+
+        def v_am(x=x1[0], out=outs[0], call=calls[0]):
+            call()
+            assert torch.equal(out.storage[:256].long(), torch.argmax(x, 1))
+        ops.append(Op("C1", "argmax_f32_[256,1000]", 256000, 1024000 + 1024, calls, v_am))
+        ops += topk_ops(be, tensor, x1, [5], "C1", "[256,1000]")
+
+    # ---------------- C3: top_k
+    if which in ("all", "c3"):
+        x3 = gen((4096, 32000), torch.float32, lambda c: synth.quantised_normal(5 + 100 * c), 4)
+        ops += topk_ops(be, tensor, x3, [1, 5, 50, 256], "C3", "[4096,32000]")
+
+    # ---------------- C4: sort / argsort
+    if which in ("all", "c4"):
+        x4a = gen((1024, 65536), torch.float32, lambda c: synth.quantised_uniform(6 + 100 * c), 4)
+        ops += sort_ops(be, tensor, x4a, "C4a", "f32_[1024,65536]")
+        x4b = gen((256, 1 << 20), torch.int64, lambda c: synth.full_range_i64(7), 1)
+        ops += sort_ops(be, tensor, x4b, "C4b", "i64_[256,2^20]")
+
+    # ---------------- C5: strided NCHW
+    if which in ("all", "c5"):
+        x5 = gen((32, 512, 56, 56), torch.float32, lambda c: synth.normal(8 + 100 * c), 6)
+        n5 = 32 * 512 * 56 * 56
+        calls, outs = reduce_calls("reduce_mean", x5, [2, 3])
+
+        def v_mean(x=x5[0], out=outs[0], call=calls[0]):
+            call()
+            assert torch.allclose(out.storage[:16384].double(), x.double().mean((2, 3)).view(-1), rtol=1e-5, atol=1e-6)
+        ops.append(Op("C5", "reduce_mean{2,3}_f32_[32,512,56,56]", n5, 4 * n5 + 65536, calls, v_mean))
+        calls, outs = reduce_calls("reduce_max", x5, [1])
+
+        def v_max(x=x5[0], out=outs[0], call=calls[0]):
+            call()
+            assert torch.equal(out.storage[:100352], x.amax(1).reshape(-1))
+        ops.append(Op("C5", "reduce_max{1}_f32_[32,512,56,56]", n5, 4 * n5 + 401408, calls, v_max))
+        calls, outs = argmax_calls(x5, 1)
+
+        def v_arg(x=x5[0], out=outs[0], call=calls[0]):
+            call()
+            assert torch.equal(out.storage[:100352].long(), torch.argmax(x, 1).reshape(-1))
+        ops.append(Op("C5", "argmax{1}_f32_[32,512,56,56]", n5, 4 * n5 + 401408, calls, v_arg))
+        calls, y5 = scan_calls(x5, 1)
+
+        def v_cs(x=x5[0], y=y5, call=calls[0]):
+            call()
+            want = torch.cumsum(x.double(), 1)
+            mag = torch.cumsum(x.double().abs(), 1)
+            tol = 4 * 9 * float(np.finfo(np.float32).eps) * torch.maximum(want.abs(), mag)
+            assert bool(((y.double() - want).abs() <= tol).all())
+        ops.append(Op("C5", "cumsum{1}_f32_[32,512,56,56]", n5, 8 * n5, calls, v_cs))
+    return ops
+
+
+def topk_ops(be, tensor, xs, ks, config, shape_text):
+    import numpy as np
+    import torch
+    from dlf_amd.frontend import Tensor, dtype_code
+    ops = []
+    rows, n = xs[0].shape
+    for k in ks:
+        Y = Tensor.empty(be, [rows, k], np.float32)
+        I = Tensor.empty(be, [rows, k], np.int64)
+        calls = []
+        for x in xs:
+            X = tensor(x)
+            calls.append(be.top_k(k, 1, dtype_code(np.float32), 3, X.shape, X.storage, Y.shape, Y.storage,
+                                  I.shape, I.storage, defer=True))
+
+        def v(x=xs[0], Y=Y, I=I, k=k, call=calls[0], rows=rows):
+            call()
+            y = Y.storage[:rows * k].view(rows, k)
+            i = I.storage[:rows * k].view(rows, k)
+            want = torch.topk(x, k, dim=1, largest=True, sorted=True).values
+            assert torch.equal(y, want), "top_k values"
+            assert torch.equal(torch.gather(x, 1, i), y), "top_k gather"
+            # lowest index on ties: compare against a stable descending sort on a slice of rows
+            sub = x[:64]
+            order = torch.sort(sub, dim=1, descending=True, stable=True).indices[:, :k]
+            assert torch.equal(i[:64], order), "top_k tie order"
+        ops.append(Op(config, "top_k%d_f32_%s" % (k, shape_text), rows * n, 4 * rows * n + rows * k * 12, calls, v,
+                      "topk_select"))
+    return ops
+
+
+def sort_ops(be, tensor, xs, config, text):
+    import numpy as np
+    import torch
+    from dlf_amd.frontend import Tensor, dtype_code
+    ops = []
+    rows, n = xs[0].shape
+    es = xs[0].element_size()
+    npd = np.float32 if xs[0].dtype == torch.float32 else np.int64
+    y = torch.empty_like(xs[0])
+    Y = tensor(y)
+    I = Tensor.empty(be, [rows, n], np.int32)
+    for desc in (0, 1):
+        calls = []
+        for x in xs:
+            X = tensor(x)
+            calls.append(be.sort(desc, dtype_code(npd), X.shape, X.storage, Y.shape, Y.storage, defer=True))
+
+        def v(x=xs[0], y=y, desc=desc, call=calls[0]):
+            call()
+            assert torch.equal(y, torch.sort(x, dim=1, descending=bool(desc)).values), "sort"
+        ops.append(Op(config, "sort_%s_%s" % ("desc" if desc else "asc", text), rows * n, 2 * es * rows * n, calls, v,
+                      "sort_pass"))
+        calls = []
+        for x in xs:
+            X = tensor(x)
+            calls.append(be.argsort(desc, dtype_code(npd), 2, X.shape, X.storage, None, None, I.shape, I.storage, defer=True))
+
+        def va(x=xs[0], I=I, desc=desc, call=calls[0], rows=rows, n=n):
+            call()
+            i = I.storage[:rows * n].view(rows, n).long()
+            sub = slice(0, 16)
+            want = torch.sort(x[sub], dim=1, descending=bool(desc), stable=True).indices
+            assert torch.equal(i[sub], want), "argsort stable order"
+            g = torch.gather(x, 1, i)
+            d = g[:, 1:] - g[:, :-1] if x.dtype != torch.int64 else None
+            if d is not None:
+                assert bool((d <= 0).all() if desc else (d >= 0).all()), "argsort sortedness"
+            else:
+                assert bool((g[:, 1:] <= g[:, :-1]).all() if desc else (g[:, 1:] >= g[:, :-1]).all())
+        ops.append(Op(config, "argsort_%s_%s" % ("desc" if desc else "asc", text), rows * n, (es + 4) * rows * n,
+                      calls, va, "sort_pass"))
+    return ops
+
+
+def time_op(torch, op, iters, warm=3):
+    for _ in range(warm):
+        op.issue()
+    torch.cuda.synchronize()
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(iters + 1)]
+    evs[0].record()
+    for i in range(iters):
+        op.issue()
+        evs[i + 1].record()
+    torch.cuda.synchronize()
+    ts = sorted(evs[i].elapsed_time(evs[i + 1]) * 1e3 for i in range(iters))   # us
+    return ts[len(ts) // 2], sum(ts) / len(ts)
+
+
+def cpu_baseline():
+    """The CPU restatement of the reference's algorithms, timed on this box's host cores."""
+    import numpy as np
+    from dlf_amd import frontend as F
+    from dlf_amd.frontend import Tensor
+    from oracle import oracle as O
+    be = O.OracleBackend()
+    rng = np.random.default_rng(2)
+    xi = rng.integers(0, 100, size=(64, 1 << 20), dtype=np.int32)
+    xf = rng.standard_normal((64, 1 << 20), dtype=np.float32)
+    xl = (rng.integers(0, 1 << 24, size=1 << 28).astype(np.float32) * np.float32(2.0 ** -23)) - np.float32(1.0)
+    Xi, Xf, Xl = (Tensor.from_numpy(be, a) for a in (xi, xf, xl))
+    Yi, Yf = Tensor.empty(be, xi.shape, np.int32), Tensor.empty(be, xf.shape, np.float32)
+    F.cumsum(Xi, 1, out=Yi)                       # warm the pages
+    t0 = time.perf_counter()
+    reps = 3
+    for _ in range(reps):
+        F.cumsum(Xi, 1, out=Yi)
+        F.cumsum(Xf, 1, out=Yf)
+        F.reduce_sum(Xl, [])
+    dt = (time.perf_counter() - t0) / reps
+    nbytes = 2 * 4 * (64 << 20) * 2 + 4 * (1 << 28)
+    return {"value": round(nbytes / dt / 1e9, 2), "unit": "GB/s", "cores": O.threads(), "kind": "port",
+            "sample": "cumsum int32 + fp32 [64,2^20] in full and reduce_sum over 2^28 of the 2^30 fp32 elements, "
+                      "3 repetitions, OpenMP rows/chunks in parallel"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--configs", default="all", help="all | step | c1 | c2 | c3 | c4 | c5")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-verify", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
+
+    import torch
+    from dlf_amd.hip_backend import HipBackend
+    be = HipBackend("cuda:0")
+    ops = make_ops(be, args.configs)
+    log("inputs resident: %d operations" % len(ops))
+
+    if not args.no_verify:
+        for op in ops:
+            if op.verify:
+                op.verify()
+        torch.cuda.synchronize()
+        log("parity gates passed")
+
+    # ---- the step: C2a + C2b + C2c back to back
+    step_ops = [op for op in ops if op.config in ("C2a", "C2b", "C2c")]
+    result = {"metric": METRIC, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+              "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int32+f32 (fp32 sums accumulate in f64)",
+              "data": "synthetic"}
+    if step_ops:
+        for _ in range(args.warmup):
+            for op in step_ops:
+                op.issue()
+        torch.cuda.synchronize()
+        per_kernel = {op.name: [] for op in step_ops}
+        evs = []
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            row = [torch.cuda.Event(enable_timing=True)]
+            row[0].record()
+            for op in step_ops:
+                op.issue()
+                e = torch.cuda.Event(enable_timing=True)
+                e.record()
+                row.append(e)
+            evs.append(row)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        for row in evs:
+            for j, op in enumerate(step_ops):
+                per_kernel[op.name].append(row[j].elapsed_time(row[j + 1]) * 1e3)
+        step_bytes = sum(op.alg_bytes for op in step_ops)
+        ms = wall / args.steps * 1e3
+        result.update({"value": round(step_bytes / (wall / args.steps) / 1e9, 1), "ms_per_step": round(ms, 4),
+                       "config": {"workload": "configs[1]: cumsum int32 [64,2^20] + cumsum fp32 [64,2^20] + "
+                                              "reduce_sum fp32 [2^30], last axis, contiguous",
+                                  "algorithmic_bytes_per_step": step_bytes}})
+        dom = max(step_ops, key=lambda op: sum(per_kernel[op.name]))
+        avg_us = sum(per_kernel[dom.name]) / len(per_kernel[dom.name])
+        achieved = dom.alg_bytes / avg_us / 1e3
+        result["roofline"] = {"bound": "hbm", "kernel": dom.kernel, "op": dom.name, "achieved": round(achieved, 1),
+                              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                              "avg_launch_us": round(avg_us, 2), "traffic": None}
+    else:
+        result.update({"value": None, "ms_per_step": None, "config": {"workload": args.configs}})
+
+    # ---- every operation on its own
+    per_op = []
+    for op in ops:
+        iters = 20 if op.alg_bytes < (1 << 31) else 8
+        med, avg = time_op(torch, op, iters)
+        gbs = op.alg_bytes / med / 1e3
+        per_op.append({"config": op.config, "op": op.name, "us": round(med, 2), "gelem_s": round(op.elems / med / 1e3, 2),
+                       "gb_s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)})
+        log("%-4s %-44s %10.1f us %9.1f GB/s %6.1f%%" % (op.config, op.name, med, gbs, 100 * gbs / HBM_PEAK_GBS))
+    result["per_op"] = per_op
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -70,5 +70,27 @@ def build_all(force=False, jobs=None):
     return LIB
 
 
+VENEER_TEST_SRC = os.path.join(HERE, "..", "tests", "cpp", "veneer_test.cpp")
+VENEER_TEST_BIN = os.path.join(HERE, "..", "tests", "cpp", "veneer_test.bin")
+
+
+def build_veneer_test(force=False):
+    """Compiles the C++ host veneer's test program (host code + HIP runtime only)."""
+    src, out = os.path.abspath(VENEER_TEST_SRC), os.path.abspath(VENEER_TEST_BIN)
+    if not os.path.exists(src):
+        return None
+    inc = os.path.join(HERE, "include")
+    newest = max([os.path.getmtime(src)] + [os.path.getmtime(os.path.join(inc, f)) for f in os.listdir(inc)])
+    if not force and os.path.exists(out) and os.path.getmtime(out) > newest:
+        return out
+    cmd = [_hipcc(), "-O2", "-std=c++17", "-I", inc, "-I", os.path.join(HERE, "..", "include"), src, "-o", out,
+           "-L", os.path.dirname(LIB), "-ldlfx", "-Wl,-rpath,$ORIGIN/../../dlf_amd/lib"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("veneer test build failed:\n" + r.stderr)
+    return out
+
+
 if __name__ == "__main__":
     print(build_all(force="--force" in sys.argv))
+    print(build_veneer_test(force="--force" in sys.argv))

@@ -57,9 +57,20 @@ struct View {
     const int64_t* dims;
     const int64_t* strides;
     int64_t offset;
+    bool contiguous;   // row-major dense: the reference then walks a raw pointer (map.h:5-41)
+
+    View(int r, const int64_t* d, const int64_t* s, int64_t o) : rank(r), dims(d), strides(s), offset(o) {
+        contiguous = true;
+        int64_t size = 1;
+        for (int i = rank - 1; i >= 0; --i) {
+            if (dims[i] != 1 && strides[i] != size) contiguous = false;
+            size *= dims[i];
+        }
+    }
 
     // Shape::linear_offset: row-major unravel of a flat index, then dot with strides.
     int64_t at(int64_t flat) const {
+        if (contiguous) return offset + flat;
         int64_t off = offset;
         for (int i = rank - 1; i >= 0; --i) {
             int64_t d = dims[i];
@@ -563,7 +574,7 @@ int dlf_oracle_reduce(const char* name, int dtype, int64_t m, int64_t n,
                       void* y, int64_t y_offset) {
     Red r;
     if (!parse_reduce(name, &r)) return -1;
-    View xv{x_rank, x_dims, x_strides, x_offset}, yv{y_rank, y_dims, y_strides, y_offset};
+    View xv(x_rank, x_dims, x_strides, x_offset), yv(y_rank, y_dims, y_strides, y_offset);
     return by_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
         return do_reduce<T>(r, m, n, xv, static_cast<const T*>(x), yv, static_cast<T*>(y));
@@ -575,7 +586,7 @@ int dlf_oracle_reduce_f64(const char* name, int dtype, int64_t m, int64_t n,
                           const void* x, int64_t x_offset, double* y) {
     Red r;
     if (!parse_reduce(name, &r)) return -1;
-    View xv{x_rank, x_dims, x_strides, x_offset};
+    View xv(x_rank, x_dims, x_strides, x_offset);
     return by_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
         return do_reduce_f64<T>(r, m, n, xv, static_cast<const T*>(x), y);
@@ -591,7 +602,7 @@ int dlf_oracle_arg_reduce(const char* name, int dtype, int64_t rows, int64_t k,
     if (!std::strcmp(name, "argmax")) want_max = true;
     else if (!std::strcmp(name, "argmin")) want_max = false;
     else return -1;
-    View xv{x_rank, x_dims, x_strides, x_offset}, yv{y_rank, y_dims, y_strides, y_offset};
+    View xv(x_rank, x_dims, x_strides, x_offset), yv(y_rank, y_dims, y_strides, y_offset);
     return by_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
         return do_arg_reduce<T>(want_max, rows, k, xv, static_cast<const T*>(x), yv, y);
@@ -604,7 +615,7 @@ int dlf_oracle_scan(const char* name, int dtype, int64_t m, int64_t n, int exclu
                     void* y, int64_t y_offset, const int64_t* y_strides) {
     Scn s;
     if (!parse_scan(name, &s)) return -1;
-    View xv{rank, dims, x_strides, x_offset}, yv{rank, dims, y_strides, y_offset};
+    View xv(rank, dims, x_strides, x_offset), yv(rank, dims, y_strides, y_offset);
     return by_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
         return do_scan<T>(s, m, n, exclusive != 0, xv, static_cast<const T*>(x), yv, static_cast<T*>(y));
@@ -618,7 +629,7 @@ int dlf_oracle_scan_f64(const char* name, int dtype, int64_t m, int64_t n, int e
                         double* y, double* abs_prefix) {
     Scn s;
     if (!parse_scan(name, &s)) return -1;
-    View xv{rank, dims, x_strides, x_offset};
+    View xv(rank, dims, x_strides, x_offset);
     return by_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
         return do_scan_f64<T>(s, m, n, exclusive != 0, xv, static_cast<const T*>(x), y, abs_prefix);
@@ -628,7 +639,7 @@ int dlf_oracle_scan_f64(const char* name, int dtype, int64_t m, int64_t n, int e
 int dlf_oracle_sort(int dir, int dtype, int rank, const int64_t* dims,
                     const void* x, int64_t x_offset, const int64_t* x_strides,
                     void* y, int64_t y_offset, const int64_t* y_strides) {
-    View xv{rank, dims, x_strides, x_offset}, yv{rank, dims, y_strides, y_offset};
+    View xv(rank, dims, x_strides, x_offset), yv(rank, dims, y_strides, y_offset);
     return by_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
         return do_sort<T>(dir, xv, static_cast<const T*>(x), yv, static_cast<T*>(y));
@@ -640,8 +651,8 @@ int dlf_oracle_argsort(int dir, int dtype, int rank, const int64_t* dims,
                        const void* x, int64_t x_offset, const int64_t* x_strides,
                        void* y, int64_t y_offset, const int64_t* y_strides,
                        int32_t* idx, int64_t i_offset, const int64_t* i_strides) {
-    View xv{rank, dims, x_strides, x_offset}, iv{rank, dims, i_strides, i_offset};
-    View yv{rank, dims, y_strides ? y_strides : x_strides, y_offset};
+    View xv(rank, dims, x_strides, x_offset), iv(rank, dims, i_strides, i_offset);
+    View yv(rank, dims, y_strides ? y_strides : x_strides, y_offset);
     return by_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
         return do_argsort<T>(dir, xv, static_cast<const T*>(x), y ? &yv : nullptr,
@@ -657,8 +668,8 @@ int dlf_oracle_top_k(int mode, int64_t limit, int largest, int sorted, int dtype
                      const void* x, int64_t x_offset, const int64_t* x_strides,
                      void* y, int64_t y_offset, const int64_t* y_strides,
                      void* idx, int64_t i_offset, const int64_t* i_strides, int index_bytes) {
-    View xv{rank, x_dims, x_strides, x_offset}, yv{rank, y_dims, y_strides, y_offset},
-         iv{rank, y_dims, i_strides, i_offset};
+    View xv(rank, x_dims, x_strides, x_offset), yv(rank, y_dims, y_strides, y_offset),
+         iv(rank, y_dims, i_strides, i_offset);
     if (limit > xv.last_extent() || limit != yv.last_extent()) return -3;
     return by_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
