@@ -1,0 +1,178 @@
+// Host veneer: dlf's gpgpu::dnn entry points for the axis primitives, forwarding
+// to the C ABI in dlfx.h.  Signatures follow gpgpu/include/gdnn.h:108-182 so
+// that dlf's tensor front-ends (dlf/include/tensor/reduce_detail.h:91-101,
+// 134-147, 244-253; reorder_detail.h:617-627, 667-677, 951-963, 1062-1073)
+// compile against it unchanged: sizes and strides are std::vector<size_t>
+// (negative steps wrapped), scratch comes from the context's temporary-buffer
+// stack, failures surface as exceptions, and `event`, when given, brackets the
+// work of the call.
+#pragma once
+
+#include <cstdint>
+#include <string>
+#include <type_traits>
+#include <vector>
+
+#include "dlfx.h"
+#include "gpgpu.h"
+
+namespace gpgpu { namespace dnn {
+
+namespace detail {
+
+template <typename T> struct dtype_of;
+template <> struct dtype_of<float>   { static constexpr int value = DLFX_F32; };
+template <> struct dtype_of<double>  { static constexpr int value = DLFX_F64; };
+template <> struct dtype_of<int32_t> { static constexpr int value = DLFX_I32; };
+template <> struct dtype_of<int64_t> { static constexpr int value = DLFX_I64; };
+
+// size_t strides that wrapped for a negative step come back as the negative number
+inline std::vector<int64_t> signed_vec(const std::vector<size_t>& v) {
+    std::vector<int64_t> r(v.size());
+    for (size_t i = 0; i < v.size(); ++i) r[i] = static_cast<int64_t>(v[i]);
+    return r;
+}
+
+struct EventScope {
+    const Queue& q;
+    Event* e;
+    EventScope(const Queue& queue, Event* event) : q(queue), e(event) {
+        if (e) check_hip(hipEventRecord(e->start(), q.stream()), "hipEventRecord");
+    }
+    void done() { if (e) check_hip(hipEventRecord(e->end(), q.stream()), "hipEventRecord"); }
+};
+
+}  // namespace detail
+
+template <typename T>
+void reduce(const std::string& name, const size_t m, const size_t n,
+            const std::vector<size_t>& x_dims, const std::vector<size_t>& x_strides,
+            const Buffer<T>& x_buffer, const size_t x_offset,
+            const std::vector<size_t>& y_dims, const std::vector<size_t>& y_strides,
+            Buffer<T>& y_buffer, const size_t y_offset,
+            const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    const int dt = detail::dtype_of<T>::value;
+    auto xd = detail::signed_vec(x_dims), xs = detail::signed_vec(x_strides);
+    auto yd = detail::signed_vec(y_dims), ys = detail::signed_vec(y_strides);
+    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_reduce_scratch_bytes(dt, m, n));
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_reduce(queue.stream(), name.c_str(), dt, m, n,
+                             static_cast<int>(xd.size()), xd.data(), xs.data(), x_buffer.data(), x_offset,
+                             static_cast<int>(yd.size()), yd.data(), ys.data(), y_buffer.data(), y_offset,
+                             tmp.bytes(), tmp.byte_size()), "gpgpu::dnn::reduce");
+    ev.done();
+}
+
+template <typename T>
+void arg_reduce(const std::string& name, const size_t n, const size_t k,
+                const std::vector<size_t>& x_dims, const std::vector<size_t>& x_strides,
+                const Buffer<T>& x_buffer, const size_t x_offset,
+                const std::vector<size_t>& y_dims, const std::vector<size_t>& y_strides,
+                Buffer<int>& y_buffer, const size_t y_offset,
+                const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    const int dt = detail::dtype_of<T>::value;
+    auto xd = detail::signed_vec(x_dims), xs = detail::signed_vec(x_strides);
+    auto yd = detail::signed_vec(y_dims), ys = detail::signed_vec(y_strides);
+    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_arg_reduce_scratch_bytes(dt, n, k));
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_arg_reduce(queue.stream(), name.c_str(), dt, DLFX_I32, n, k,
+                                 static_cast<int>(xd.size()), xd.data(), xs.data(), x_buffer.data(), x_offset,
+                                 static_cast<int>(yd.size()), yd.data(), ys.data(), y_buffer.data(), y_offset,
+                                 tmp.bytes(), tmp.byte_size()), "gpgpu::dnn::arg_reduce");
+    ev.done();
+}
+
+template <typename T>
+void scan(const std::string& name, const size_t m, const size_t n,
+          const bool exclusive, const std::vector<size_t>& dims,
+          const Buffer<T>& x_buffer, const size_t x_offset, const std::vector<size_t>& x_strides,
+          Buffer<T>& y_buffer, const size_t y_offset, const std::vector<size_t>& y_strides,
+          const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    const int dt = detail::dtype_of<T>::value;
+    auto d = detail::signed_vec(dims), xs = detail::signed_vec(x_strides), ys = detail::signed_vec(y_strides);
+    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_scan_scratch_bytes(dt, m, n));
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_scan(queue.stream(), name.c_str(), dt, m, n, exclusive ? 1 : 0,
+                           static_cast<int>(d.size()), d.data(), x_buffer.data(), x_offset, xs.data(),
+                           y_buffer.data(), y_offset, ys.data(), tmp.bytes(), tmp.byte_size()), "gpgpu::dnn::scan");
+    ev.done();
+}
+
+template <typename T>
+void sort(const int dir, const std::vector<size_t>& dims,
+          const Buffer<T>& x_buffer, const size_t x_offset, const std::vector<size_t>& x_strides,
+          Buffer<T>& y_buffer, const size_t y_offset, const std::vector<size_t>& y_strides,
+          const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    const int dt = detail::dtype_of<T>::value;
+    auto d = detail::signed_vec(dims), xs = detail::signed_vec(x_strides), ys = detail::signed_vec(y_strides);
+    const int64_t n = d.empty() ? 1 : d.back();
+    int64_t m = 1;
+    for (size_t i = 0; i + 1 < d.size(); ++i) m *= d[i];
+    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_sort_scratch_bytes(dt, m, n));
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_sort(queue.stream(), dir, dt, static_cast<int>(d.size()), d.data(),
+                           x_buffer.data(), x_offset, xs.data(), y_buffer.data(), y_offset, ys.data(),
+                           tmp.bytes(), tmp.byte_size()), "gpgpu::dnn::sort");
+    ev.done();
+}
+
+template <typename T>
+void argsort(const int dir, const std::vector<size_t>& dims,
+             const Buffer<T>& x_buffer, const size_t x_offset, const std::vector<size_t>& x_strides,
+             Buffer<int32_t>& i_buffer, const size_t i_offset, const std::vector<size_t>& i_strides,
+             const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    const int dt = detail::dtype_of<T>::value;
+    auto d = detail::signed_vec(dims), xs = detail::signed_vec(x_strides), is = detail::signed_vec(i_strides);
+    const int64_t n = d.empty() ? 1 : d.back();
+    int64_t m = 1;
+    for (size_t i = 0; i + 1 < d.size(); ++i) m *= d[i];
+    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_argsort_scratch_bytes(dt, m, n));
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_argsort(queue.stream(), dir, dt, DLFX_I32, static_cast<int>(d.size()), d.data(),
+                              x_buffer.data(), x_offset, xs.data(), nullptr, 0, nullptr,
+                              i_buffer.data(), i_offset, is.data(), tmp.bytes(), tmp.byte_size()), "gpgpu::dnn::argsort");
+    ev.done();
+}
+
+template <typename T>
+void argsort(const int dir, const std::vector<size_t>& dims,
+             const Buffer<T>& x_buffer, const size_t x_offset, const std::vector<size_t>& x_strides,
+             Buffer<T>& y_buffer, const size_t y_offset, const std::vector<size_t>& y_strides,
+             Buffer<int32_t>& i_buffer, const size_t i_offset, const std::vector<size_t>& i_strides,
+             const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    const int dt = detail::dtype_of<T>::value;
+    auto d = detail::signed_vec(dims), xs = detail::signed_vec(x_strides), ys = detail::signed_vec(y_strides),
+         is = detail::signed_vec(i_strides);
+    const int64_t n = d.empty() ? 1 : d.back();
+    int64_t m = 1;
+    for (size_t i = 0; i + 1 < d.size(); ++i) m *= d[i];
+    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_argsort_scratch_bytes(dt, m, n));
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_argsort(queue.stream(), dir, dt, DLFX_I32, static_cast<int>(d.size()), d.data(),
+                              x_buffer.data(), x_offset, xs.data(), y_buffer.data(), y_offset, ys.data(),
+                              i_buffer.data(), i_offset, is.data(), tmp.bytes(), tmp.byte_size()), "gpgpu::dnn::argsort");
+    ev.done();
+}
+
+template <typename T>
+void top_k(const size_t limit, const int dir,
+           const std::vector<size_t>& x_dims, const std::vector<size_t>& y_dims,
+           const Buffer<T>& x_buffer, const size_t x_offset, const std::vector<size_t>& x_strides,
+           Buffer<T>& y_buffer, const size_t y_offset, const std::vector<size_t>& y_strides,
+           Buffer<int32_t>& i_buffer, const size_t i_offset, const std::vector<size_t>& i_strides,
+           const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    const int dt = detail::dtype_of<T>::value;
+    auto xd = detail::signed_vec(x_dims), yd = detail::signed_vec(y_dims);
+    auto xs = detail::signed_vec(x_strides), ys = detail::signed_vec(y_strides), is = detail::signed_vec(i_strides);
+    const int64_t n = xd.empty() ? 1 : xd.back();
+    int64_t m = 1;
+    for (size_t i = 0; i + 1 < xd.size(); ++i) m *= xd[i];
+    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_top_k_scratch_bytes(dt, m, n, limit));
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_top_k(queue.stream(), limit, dir, dt, DLFX_I32, static_cast<int>(xd.size()), xd.data(), yd.data(),
+                            x_buffer.data(), x_offset, xs.data(), y_buffer.data(), y_offset, ys.data(),
+                            i_buffer.data(), i_offset, is.data(), tmp.bytes(), tmp.byte_size()), "gpgpu::dnn::top_k");
+    ev.done();
+}
+
+}}  // namespace gpgpu::dnn

@@ -1,0 +1,223 @@
+// Host veneer: the subset of dlf's gpgpu runtime objects that the axis
+// primitives' call surface touches, implemented directly on HIP.
+//
+// Mirrors gpgpu/include/gpgpu.h (exceptions :21-121, Queue/Event :593-637,
+// Buffer<T> :639-698, TemporaryBuffer<T> :710-746, current:: :828-857) and
+// gpgpu/src/gpgpu.cpp:139-229 (thread-local current queue, LIFO temporary
+// buffers).  Only HIP is behind it: no OpenCL/CUDA back-ends, no run-time
+// kernel compilation, no program cache.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "dlfx.h"
+
+namespace gpgpu {
+
+// ---------------------------------------------------------------- errors
+class Error : public std::runtime_error {
+public:
+    explicit Error(const std::string& what) : std::runtime_error(what) {}
+};
+
+// A HIP runtime call failed (reference: APIError).
+class APIError : public Error {
+    int status_;
+public:
+    APIError(int status, const std::string& where)
+        : Error("HIP error " + std::to_string(status) + " (" + hipGetErrorString(static_cast<hipError_t>(status)) +
+                ") in " + where), status_(status) {}
+    int status() const noexcept { return status_; }
+};
+
+// A routine rejected its arguments or failed to launch (reference: RuntimeErrorCode).
+class RuntimeErrorCode : public Error {
+    int status_;
+public:
+    RuntimeErrorCode(int status, const std::string& where)
+        : Error(where + ": " + dlfx_status_string(status)), status_(status) {}
+    int status() const noexcept { return status_; }
+};
+
+// Misuse of the veneer itself, e.g. temporary buffers released out of order (reference: LogicError).
+class LogicError : public Error {
+public:
+    explicit LogicError(const std::string& what) : Error(what) {}
+};
+
+inline void check_hip(hipError_t e, const char* where) {
+    if (e != hipSuccess) throw APIError(static_cast<int>(e), where);
+}
+
+inline void check_status(int status, const char* where) {
+    if (status == DLFX_OK) return;
+    if (status == DLFX_ERR_LAUNCH) throw APIError(dlfx_last_hip_error(), where);
+    throw RuntimeErrorCode(status, where);
+}
+
+// ---------------------------------------------------------------- queue / event
+// An in-order stream of work on one device.
+class Queue {
+    struct Holder {
+        hipStream_t stream = nullptr;
+        bool owned = false;
+        ~Holder() { if (owned && stream) (void)hipStreamDestroy(stream); }
+    };
+    std::shared_ptr<Holder> h_;
+public:
+    Queue() : h_(std::make_shared<Holder>()) {
+        check_hip(hipStreamCreate(&h_->stream), "hipStreamCreate");
+        h_->owned = true;
+    }
+    // Wraps an existing stream without taking ownership (nullptr = the default stream).
+    explicit Queue(hipStream_t s) : h_(std::make_shared<Holder>()) { h_->stream = s; }
+    hipStream_t stream() const noexcept { return h_->stream; }
+    void finish() const { check_hip(hipStreamSynchronize(h_->stream), "hipStreamSynchronize"); }
+};
+
+// Start/end markers around the last kernel of a routine.
+class Event {
+    struct Holder {
+        hipEvent_t start = nullptr, end = nullptr;
+        Holder() {
+            check_hip(hipEventCreate(&start), "hipEventCreate");
+            check_hip(hipEventCreate(&end), "hipEventCreate");
+        }
+        ~Holder() { (void)hipEventDestroy(start); (void)hipEventDestroy(end); }
+    };
+    std::shared_ptr<Holder> h_ = std::make_shared<Holder>();
+public:
+    hipEvent_t start() const noexcept { return h_->start; }
+    hipEvent_t end() const noexcept { return h_->end; }
+    void waitForCompletion() const { check_hip(hipEventSynchronize(h_->end), "hipEventSynchronize"); }
+    float getElapsedTime() const {          // milliseconds
+        waitForCompletion();
+        float ms = 0;
+        check_hip(hipEventElapsedTime(&ms, h_->start, h_->end), "hipEventElapsedTime");
+        return ms;
+    }
+};
+
+// ---------------------------------------------------------------- buffers
+class Context;
+
+// Typed device memory shared by reference; offset() is non-zero only for
+// temporary buffers carved out of a context's scratch arena.
+template <typename T>
+class Buffer {
+protected:
+    std::shared_ptr<void> mem_;
+    size_t size_ = 0;      // elements
+    size_t offset_ = 0;    // elements from mem_
+public:
+    Buffer() = default;
+    explicit Buffer(size_t size) : size_(size) {
+        void* p = nullptr;
+        check_hip(hipMalloc(&p, (size ? size : 1) * sizeof(T)), "hipMalloc");
+        mem_ = std::shared_ptr<void>(p, [](void* q) { (void)hipFree(q); });
+    }
+    Buffer(std::shared_ptr<void> mem, size_t size, size_t offset) : mem_(std::move(mem)), size_(size), offset_(offset) {}
+
+    size_t size() const noexcept { return size_; }
+    size_t offset() const noexcept { return offset_; }
+    T* data() const noexcept { return static_cast<T*>(mem_.get()); }       // start of the allocation
+    explicit operator bool() const noexcept { return static_cast<bool>(mem_); }
+
+    void read(const Queue& q, T* host, size_t n, size_t offset = 0) const {
+        if (offset + n > size_ + offset_) throw LogicError("Buffer::read: range exceeds the buffer");
+        check_hip(hipMemcpyAsync(host, data() + offset, n * sizeof(T), hipMemcpyDeviceToHost, q.stream()), "hipMemcpyAsync");
+        q.finish();
+    }
+    void write(const Queue& q, const T* host, size_t n, size_t offset = 0) {
+        if (offset + n > size_ + offset_) throw LogicError("Buffer::write: range exceeds the buffer");
+        check_hip(hipMemcpyAsync(data() + offset, host, n * sizeof(T), hipMemcpyHostToDevice, q.stream()), "hipMemcpyAsync");
+        q.finish();
+    }
+    void copyTo(const Queue& q, Buffer<T>& dst, size_t n, size_t src_offset = 0, size_t dst_offset = 0) const {
+        check_hip(hipMemcpyAsync(dst.data() + dst_offset, data() + src_offset, n * sizeof(T), hipMemcpyDeviceToDevice,
+                                 q.stream()), "hipMemcpyAsync");
+    }
+};
+
+// A bump allocation from the context's arena, released in LIFO order when it
+// goes out of scope; releasing out of order throws (gpgpu.cpp:208-214).
+template <typename T>
+class TemporaryBuffer : public Buffer<T> {
+    Context* ctx_ = nullptr;
+    size_t bytes_begin_ = 0, bytes_end_ = 0;
+public:
+    TemporaryBuffer(Context* ctx, std::shared_ptr<void> mem, size_t size, size_t byte_begin, size_t byte_end)
+        : Buffer<T>(std::move(mem), size, byte_begin / sizeof(T)), ctx_(ctx), bytes_begin_(byte_begin), bytes_end_(byte_end) {}
+    TemporaryBuffer(const TemporaryBuffer&) = delete;
+    TemporaryBuffer& operator=(const TemporaryBuffer&) = delete;
+    TemporaryBuffer(TemporaryBuffer&& o) noexcept
+        : Buffer<T>(std::move(o)), ctx_(o.ctx_), bytes_begin_(o.bytes_begin_), bytes_end_(o.bytes_end_) { o.ctx_ = nullptr; }
+    ~TemporaryBuffer() noexcept(false);
+    void* bytes() const noexcept { return static_cast<char*>(this->mem_.get()) + bytes_begin_; }
+    size_t byte_size() const noexcept { return bytes_end_ - bytes_begin_; }
+};
+
+// One device, one scratch arena.
+class Context {
+    int device_ = 0;
+    std::shared_ptr<void> arena_;
+    size_t capacity_ = 0, top_ = 0;
+    std::vector<std::shared_ptr<void>> retired_;   // arenas outgrown while temporaries were live
+    template <typename T> friend class TemporaryBuffer;
+
+    void release(size_t begin, size_t end) {
+        if (end != top_) throw LogicError("TemporaryBuffer: released out of order");
+        top_ = begin;
+        if (top_ == 0) retired_.clear();
+    }
+public:
+    explicit Context(int device = 0) : device_(device) { check_hip(hipSetDevice(device), "hipSetDevice"); }
+    int device() const noexcept { return device_; }
+
+    template <typename T>
+    TemporaryBuffer<T> getTemporaryBuffer(size_t size) {
+        const size_t align = 256;
+        const size_t begin = (top_ + align - 1) / align * align;
+        const size_t end = begin + (size ? size : 1) * sizeof(T);
+        if (end > capacity_) {
+            // grow: earlier temporaries keep their (retired) arena alive through their shared_ptr
+            size_t cap = capacity_ ? capacity_ : (size_t(1) << 20);
+            while (cap < end) cap *= 2;
+            void* p = nullptr;
+            check_hip(hipMalloc(&p, cap), "hipMalloc");
+            if (arena_) retired_.push_back(arena_);
+            arena_ = std::shared_ptr<void>(p, [](void* q) { (void)hipFree(q); });
+            capacity_ = cap;
+        }
+        top_ = end;
+        return TemporaryBuffer<T>(this, arena_, size, begin, end);
+    }
+};
+
+template <typename T>
+TemporaryBuffer<T>::~TemporaryBuffer() noexcept(false) {
+    if (ctx_) ctx_->release(bytes_begin_, bytes_end_);
+}
+
+// ---------------------------------------------------------------- thread-local current objects
+namespace current {
+
+inline Context& context() {
+    thread_local Context ctx(0);
+    return ctx;
+}
+
+inline const Queue& queue() {
+    thread_local Queue q = (context(), Queue());
+    return q;
+}
+
+}  // namespace current
+}  // namespace gpgpu
