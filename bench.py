@@ -330,6 +330,9 @@ def main():
     ap.add_argument("--configs", default="all", help="all | step | c1 | c2 | c3 | c4 | c5")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy (read 1 GiB, write 1 GiB) so that byte counters "
+                         "collected by a profiler can be scaled against a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
@@ -399,6 +402,13 @@ def main():
                        "gb_s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)})
         log("%-4s %-44s %10.1f us %9.1f GB/s %6.1f%%" % (op.config, op.name, med, gbs, 100 * gbs / HBM_PEAK_GBS))
     result["per_op"] = per_op
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=be.device).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
