@@ -32,8 +32,8 @@ enum KeyKind { kKeyInt = 0, kKeyFloat = 1 };
 
 template <typename K>
 struct KeyBits;
-template <> struct KeyBits<uint32_t> { static constexpr int kBytes = 4; static constexpr uint32_t kSign = 0x80000000u; };
-template <> struct KeyBits<uint64_t> { static constexpr int kBytes = 8; static constexpr uint64_t kSign = 0x8000000000000000ull; };
+template <> struct KeyBits<uint32_t> { static constexpr uint32_t kSign = 0x80000000u; };
+template <> struct KeyBits<uint64_t> { static constexpr uint64_t kSign = 0x8000000000000000ull; };
 
 // Larger image <=> better candidate.
 template <typename K>
@@ -64,32 +64,35 @@ struct TopkIo {
     int idx64, kind, largest;
 };
 
+constexpr int kCandCap = 4096;     // candidates kept in LDS after the pre-filter
+
 template <typename K>
 struct TopkShared {
     uint32_t hist[kRadix];
     uint32_t wave_tot[kRadix / kWave];
+    uint32_t scan_tot[16];
     uint32_t sel_digit, sel_k, sel_ties, count;
     K out_ord[kMaxLimit];
     uint32_t out_idx[kMaxLimit];
+    K cand_ord[kCandCap];
+    uint32_t cand_idx[kCandCap];
 };
 
 // One radix-select step over the values val(i) of the items for which part(i)
 // holds: picks the digit (at `shift`) that contains the kk-th largest
 // participating value.  Results: sm.sel_digit, sm.sel_k (rank inside that
-// digit), sm.sel_ties (its population).
-template <int BLOCK, int ITEMS, typename K, typename Val, typename Part>
+// digit), sm.sel_ties (its population).  sm.hist must be all zero on entry and is
+// all zero again on return.
+template <int BLOCK, int ITEMS, bool ROLLED, typename K, typename Val, typename Part>
 __device__ __forceinline__ void select_digit(TopkShared<K>& sm, int shift, uint32_t kk, Val val, Part part) {
     const int tid = threadIdx.x;
     const int lane = lane_id();
-    for (int i = tid; i < kRadix; i += BLOCK) sm.hist[i] = 0;
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < ITEMS; ++i) {
+    auto count_item = [&](int i) {
         const bool in = part(i);
         const uint32_t d = static_cast<uint32_t>(val(i) >> shift) & 0xffu;
         // a wave whose participants all share the digit adds once
         const unsigned long long in_mask = __ballot(in);
-        if (in_mask == 0ull) continue;
+        if (in_mask == 0ull) return;
         const int first = __ffsll(static_cast<long long>(in_mask)) - 1;
         const uint32_t d0 = __shfl(d, first, kWave);
         if (__ballot(in && d != d0) == 0ull) {
@@ -97,107 +100,102 @@ __device__ __forceinline__ void select_digit(TopkShared<K>& sm, int shift, uint3
         } else if (in) {
             atomicAdd(&sm.hist[d], 1u);
         }
+    };
+    if constexpr (ROLLED) {
+#pragma unroll 1
+        for (int i = 0; i < ITEMS; ++i) count_item(i);
+    } else {
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) count_item(i);
     }
     __syncthreads();
-    // thread t < 256 looks at digit 255 - t, so an inclusive scan over t is a suffix sum over digits
-    const uint32_t d = kRadix - 1 - tid;
-    const int w = tid / kWave;
-    uint32_t h = 0, incl = 0;
-    if (tid < kRadix) {
-        h = sm.hist[d];
-        incl = wave_scan_inclusive(h, 0u, [](uint32_t a, uint32_t b) { return a + b; });
-        if (lane == kWave - 1) sm.wave_tot[w] = incl;
-    }
-    __syncthreads();
-    if (tid < kRadix) {
-        for (int i = 0; i < w; ++i) incl += sm.wave_tot[i];
-        const uint32_t above = incl - h;              // participants with a larger digit
-        if (incl >= kk && above < kk) {
-            sm.sel_digit = d;
-            sm.sel_k = kk - above;
-            sm.sel_ties = h;
+    if (tid < kWave) {
+        // lane l owns digits 255-4l .. 252-4l (descending), so a scan over lanes is a suffix sum over digits
+        uint32_t h[4], run = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int d = kRadix - 1 - (4 * lane + j);
+            h[j] = sm.hist[d];
+            sm.hist[d] = 0;
+            run += h[j];
+        }
+        const uint32_t incl = wave_scan_inclusive(run, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+        uint32_t above = incl - run;                  // participants with a digit above this lane's four
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (above < kk && above + h[j] >= kk) {
+                sm.sel_digit = kRadix - 1 - (4 * lane + j);
+                sm.sel_k = kk - above;
+                sm.sel_ties = h[j];
+            }
+            above += h[j];
         }
     }
     __syncthreads();
 }
 
-template <typename K, int BLOCK, int ITEMS>
-__global__ __launch_bounds__(BLOCK) void topk_select(TopkIo<K> io, int64_t n, int limit) {
-    constexpr int V = (16 / sizeof(K) < ITEMS) ? 16 / sizeof(K) : ITEMS;
-    constexpr int G = ITEMS / V;
-    using VecT = Vec<K, V>;
-    __shared__ TopkShared<K> sm;
-
-    const int tid = threadIdx.x;
-    const int64_t row = blockIdx.x;
-    const K* xr = io.x + io.xmap.at(row);
-
-    // item (g, e) of thread t is element ((g*BLOCK + t)*V + e) of the row
-    K ord[ITEMS];
-    const bool vec_ok = io.sx == 1 && (reinterpret_cast<uintptr_t>(xr) % (sizeof(K) * V) == 0);
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-        const int64_t i0 = (static_cast<int64_t>(g) * BLOCK + tid) * V;
-        if (vec_ok && i0 + V <= n) {
-            const VecT a = *reinterpret_cast<const VecT*>(xr + i0);
-#pragma unroll
-            for (int e = 0; e < V; ++e) ord[g * V + e] = to_ord<K>(a.v[e], io.kind, io.largest);
-        } else {
-#pragma unroll
-            for (int e = 0; e < V; ++e)
-                ord[g * V + e] = (i0 + e < n) ? to_ord<K>(xr[(i0 + e) * io.sx], io.kind, io.largest) : K(0);
-        }
+// The kk-th largest of the values val(i) over the items with part(i): most significant
+// byte first.  Returns the value; *rank_in_ties / *ties describe how many of the elements
+// equal to it still have to be taken and how many there are.
+template <int BLOCK, int ITEMS, bool ROLLED, typename V, typename K, typename Val, typename Valid>
+__device__ __forceinline__ V kth_largest(TopkShared<K>& sm, uint32_t kk, Val val, Valid valid,
+                                         uint32_t* rank_in_ties, uint32_t* ties) {
+    V prefix = 0;
+#pragma unroll 1
+    for (int pass = static_cast<int>(sizeof(V)) - 1; pass >= 0; --pass) {
+        const int shift = 8 * pass;
+        const V hi_mask = (pass == static_cast<int>(sizeof(V)) - 1) ? V(0) : static_cast<V>(~V(0) << (shift + 8));
+        select_digit<BLOCK, ITEMS, ROLLED>(sm, shift, kk, val, [&](int i) {
+            return valid(i) && ((val(i) ^ prefix) & hi_mask) == 0;
+        });
+        prefix |= static_cast<V>(sm.sel_digit) << shift;
+        kk = sm.sel_k;
+        *ties = sm.sel_ties;
     }
-    auto index_of = [&](int i) -> uint32_t {
-        return static_cast<uint32_t>((static_cast<int64_t>(i / V) * BLOCK + tid) * V + (i % V));
-    };
+    *rank_in_ties = kk;
+    return prefix;
+}
+
+// Exact selection of the `limit` best of the items (ord(i), idx(i)), best = larger image,
+// then lower index; writes them in that order.  Padding items carry image 0 and an index
+// that is not below the row length: they lose every tie, and limit <= row length, so no
+// validity test is needed.
+template <int BLOCK, int ITEMS, bool ROLLED, typename K, typename Ord, typename Idx>
+__device__ __forceinline__ void select_and_emit(TopkShared<K>& sm, const TopkIo<K>& io, int64_t row, const K* xr,
+                                                int limit, Ord ord, Idx idx) {
+    const int tid = threadIdx.x;
     if (tid == 0) sm.count = 0;
 
-    // ---- threshold key: the limit-th largest image
-    K prefix = 0;
-    uint32_t kk = static_cast<uint32_t>(limit);
-    uint32_t ties = 0;
-#pragma unroll 1
-    for (int pass = KeyBits<K>::kBytes - 1; pass >= 0; --pass) {
-        const int shift = 8 * pass;
-        const K hi_mask = (pass == KeyBits<K>::kBytes - 1) ? K(0) : (~K(0) << (shift + 8));
-        select_digit<BLOCK, ITEMS>(sm, shift, kk, [&](int i) { return ord[i]; }, [&](int i) {
-            return index_of(i) < n && ((ord[i] ^ prefix) & hi_mask) == 0;
-        });
-        prefix |= static_cast<K>(sm.sel_digit) << shift;
-        kk = sm.sel_k;
-        ties = sm.sel_ties;
-        __syncthreads();
-    }
-    // kk of the `ties` elements equal to the threshold are taken: those with the lowest indices
+    uint32_t kk = 0, ties = 0;
+    const K threshold = kth_largest<BLOCK, ITEMS, ROLLED, K>(sm, static_cast<uint32_t>(limit), ord, [](int) { return true; }, &kk, &ties);
+    // kk of the `ties` elements equal to the threshold are taken: those with the lowest indices,
+    // i.e. the kk largest images of ~index
     uint32_t idx_limit = 0xffffffffu;
     if (kk < ties) {
-        uint32_t iprefix = 0;        // select over ~index: the largest images are the lowest indices
-#pragma unroll 1
-        for (int pass = 3; pass >= 0; --pass) {
-            const int shift = 8 * pass;
-            const uint32_t hi_mask = (pass == 3) ? 0u : (~0u << (shift + 8));
-            select_digit<BLOCK, ITEMS>(sm, shift, kk, [&](int i) { return ~index_of(i); }, [&](int i) {
-                return index_of(i) < n && ord[i] == prefix && ((~index_of(i) ^ iprefix) & hi_mask) == 0;
-            });
-            iprefix |= sm.sel_digit << shift;
-            kk = sm.sel_k;
-            __syncthreads();
-        }
-        idx_limit = ~iprefix;
+        uint32_t k2 = 0, t2 = 0;
+        const uint32_t inv = kth_largest<BLOCK, ITEMS, ROLLED, uint32_t>(
+            sm, kk, [&](int i) { return ~idx(i); }, [&](int i) { return ord(i) == threshold; }, &k2, &t2);
+        idx_limit = ~inv;
     }
 
     // ---- compact the winners
-#pragma unroll
-    for (int i = 0; i < ITEMS; ++i) {
-        const uint32_t ix = index_of(i);
-        if (ix < n && (ord[i] > prefix || (ord[i] == prefix && ix <= idx_limit))) {
+    auto take = [&](int i) {
+        const uint32_t ix = idx(i);
+        const K o = ord(i);
+        if (o > threshold || (o == threshold && ix <= idx_limit)) {
             const uint32_t slot = atomicAdd(&sm.count, 1u);
             if (slot < kMaxLimit) {
-                sm.out_ord[slot] = ord[i];
+                sm.out_ord[slot] = o;
                 sm.out_idx[slot] = ix;
             }
         }
+    };
+    if constexpr (ROLLED) {
+#pragma unroll 1
+        for (int i = 0; i < ITEMS; ++i) take(i);
+    } else {
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) take(i);
     }
     int kp = 1;
     while (kp < limit) kp <<= 1;
@@ -217,8 +215,8 @@ __global__ __launch_bounds__(BLOCK) void topk_select(TopkIo<K> io, int64_t n, in
                 const K oi = sm.out_ord[i], oj = sm.out_ord[j];
                 const uint32_t xi = sm.out_idx[i], xj = sm.out_idx[j];
                 const bool j_better = oj > oi || (oj == oi && xj < xi);
-                const bool descending_block = (i & size) == 0;      // best first in this block
-                if (j_better == descending_block) {
+                const bool best_first = (i & size) == 0;
+                if (j_better == best_first) {
                     sm.out_ord[i] = oj; sm.out_ord[j] = oi;
                     sm.out_idx[i] = xj; sm.out_idx[j] = xi;
                 }
@@ -237,6 +235,133 @@ __global__ __launch_bounds__(BLOCK) void topk_select(TopkIo<K> io, int64_t n, in
         yr[j * io.sy] = bits;
         if (io.idx64) static_cast<int64_t*>(io.idx)[ir + j * io.si] = static_cast<int64_t>(ix);
         else static_cast<int32_t*>(io.idx)[ir + j * io.si] = static_cast<int32_t>(ix);
+    }
+}
+
+// ALIGNED: the axis is contiguous and every row starts on a 16-byte boundary (checked on the
+// host), so rows are read with 128-bit loads off one base register.
+template <typename K, int BLOCK, int ITEMS, bool ALIGNED>
+__global__ __launch_bounds__(BLOCK) void topk_select(TopkIo<K> io, int64_t n, int limit) {
+    constexpr int V = (16 / sizeof(K) < ITEMS) ? 16 / sizeof(K) : ITEMS;
+    constexpr int G = ITEMS / V;
+    constexpr int WAVES = BLOCK / kWave;
+    using VecT = Vec<K, V>;
+    __shared__ TopkShared<K> sm;
+
+    const int tid = threadIdx.x;
+    const int lane = lane_id();
+    const int w = tid / kWave;
+    const int64_t row = blockIdx.x;
+    const K* xr = io.x + io.xmap.at(row);
+    if (tid < kRadix) sm.hist[tid] = 0;
+
+    // item (g, e) of thread t is element ((g*BLOCK + t)*V + e) of the row
+    const uint32_t n32 = static_cast<uint32_t>(n);        // rows here have at most 65536 elements
+    const uint32_t tid_v = static_cast<uint32_t>(tid) * V;
+    auto index_of = [&](int i) -> uint32_t {
+        return tid_v + static_cast<uint32_t>((i / V) * (BLOCK * V) + (i % V));
+    };
+    auto in_row = [&](int i) -> bool { return index_of(i) < n32; };
+
+    if constexpr (BLOCK * ITEMS <= kCandCap) {
+        // short rows: select straight from registers
+        K ord[ITEMS];
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i)
+            ord[i] = in_row(i) ? to_ord<K>(xr[static_cast<int64_t>(index_of(i)) * io.sx], io.kind, io.largest) : K(0);
+        __syncthreads();
+        select_and_emit<BLOCK, ITEMS, false>(sm, io, row, xr, limit, [&](int i) { return ord[i]; }, index_of);
+    } else {
+        K ord[ITEMS];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const uint32_t i0 = tid_v + static_cast<uint32_t>(g * (BLOCK * V));
+            if (ALIGNED && i0 + V <= n32) {
+                const VecT a = *reinterpret_cast<const VecT*>(xr + i0);
+#pragma unroll
+                for (int e = 0; e < V; ++e) ord[g * V + e] = to_ord<K>(a.v[e], io.kind, io.largest);
+            } else {
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    const int64_t at = ALIGNED ? static_cast<int64_t>(i0 + e) : static_cast<int64_t>(i0 + e) * io.sx;
+                    ord[g * V + e] = (i0 + e < n32) ? to_ord<K>(xr[at], io.kind, io.largest) : K(0);
+                }
+            }
+        }
+        // ---- pre-filter.  Split the threads into `groups` >= limit groups; the largest
+        // element each group holds gives `groups` distinct elements, so the smallest of those
+        // maxima cannot exceed the limit-th largest element of the row: everything below it is
+        // out.  What is left is usually a few times `limit` elements.
+        K tmax = 0;
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) tmax = ord[i] > tmax ? ord[i] : tmax;      // padding is 0
+        int groups = 1;
+        while (groups < limit && groups < BLOCK) groups <<= 1;
+        const int span = BLOCK / groups;               // threads per group, a power of two
+        auto kmax = [](K a, K b) { return a > b ? a : b; };
+        auto kmin = [](K a, K b) { return a < b ? a : b; };
+        K bound;
+        if (span >= kWave) {
+            const K wmax = wave_reduce(tmax, kmax);
+            if (lane == 0) sm.cand_ord[w] = wmax;
+            __syncthreads();
+            bound = ~K(0);
+            const int wpg = span / kWave;              // waves per group
+            for (int g0 = 0; g0 < WAVES; g0 += wpg) {
+                K gm = 0;
+                for (int j = 0; j < wpg; ++j) gm = kmax(gm, sm.cand_ord[g0 + j]);
+                bound = kmin(bound, gm);
+            }
+        } else {
+            const K gmax = group_reduce(tmax, span, kmax);
+            const K wmin = wave_reduce(gmax, kmin);
+            if (lane == 0) sm.cand_ord[w] = wmin;
+            __syncthreads();
+            bound = ~K(0);
+            for (int j = 0; j < WAVES; ++j) bound = kmin(bound, sm.cand_ord[j]);
+        }
+        uint32_t mine = 0;
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) mine += (ord[i] >= bound) ? 1u : 0u;
+        const uint32_t incl = wave_scan_inclusive(mine, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+        if (lane == kWave - 1) sm.scan_tot[w] = incl;
+        __syncthreads();
+        uint32_t before = incl - mine, total = 0;
+        for (int i = 0; i < WAVES; ++i) {
+            const uint32_t t = sm.scan_tot[i];
+            if (i < w) before += t;
+            total += t;
+        }
+        if (total <= kCandCap && limit <= BLOCK) {
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) {
+                if (ord[i] >= bound) {
+                    sm.cand_ord[before] = ord[i];
+                    sm.cand_idx[before] = index_of(i);
+                    ++before;
+                }
+            }
+            __syncthreads();
+            constexpr int CI = kCandCap / BLOCK;
+            K cord[CI];
+            uint32_t cidx[CI];
+#pragma unroll
+            for (int j = 0; j < CI; ++j) {
+                const uint32_t slot = j * BLOCK + tid;
+                cord[j] = slot < total ? sm.cand_ord[slot] : K(0);
+                cidx[j] = slot < total ? sm.cand_idx[slot] : 0xffffffffu;
+            }
+            select_and_emit<BLOCK, CI, false>(sm, io, row, xr, limit, [&](int j) { return cord[j]; },
+                                       [&](int j) { return cidx[j]; });
+        } else {
+            // the filter kept too much (e.g. long runs of equal values): exact selection over the
+            // whole row, re-reading elements (they are cache resident) instead of holding them
+            __syncthreads();
+            select_and_emit<BLOCK, ITEMS, true>(
+                sm, io, row, xr, limit,
+                [&](int i) { return in_row(i) ? to_ord<K>(xr[static_cast<int64_t>(index_of(i)) * io.sx], io.kind, io.largest) : K(0); },
+                index_of);
+        }
     }
 }
 
@@ -284,15 +409,23 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int kind, int dtype, i
     if (selection_fits(sizeof(K), n, limit)) {
         const dim3 grid(static_cast<unsigned>(m));
         const int lim = static_cast<int>(limit);
-#define DLFX_TOPK(BLOCK, ITEMS) topk_select<K, BLOCK, ITEMS><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim)
+        bool aligned = io.sx == 1 && reinterpret_cast<uintptr_t>(io.x) % 16 == 0;
+        for (int i = 0; i < io.xmap.rank; ++i) aligned = aligned && io.xmap.strides[i] % (16 / static_cast<int64_t>(sizeof(K))) == 0;
+#define DLFX_TOPK(BLOCK, ITEMS)                                                                     \
+    do {                                                                                            \
+        if (aligned) topk_select<K, BLOCK, ITEMS, true><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim); \
+        else topk_select<K, BLOCK, ITEMS, false><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim);      \
+    } while (0)
         if (n <= 256) DLFX_TOPK(256, 1);
         else if (n <= 1024) DLFX_TOPK(256, 4);
         else if (n <= 2048) DLFX_TOPK(1024, 2);
         else if (n <= 4096) DLFX_TOPK(1024, 4);
         else if (n <= 8192) DLFX_TOPK(1024, 8);
         else if (n <= 16384) DLFX_TOPK(1024, 16);
-        else if (n <= 32768) DLFX_TOPK(1024, 32);
-        else {
+        else if (n <= 32768) {
+            if (lim <= 512) DLFX_TOPK(512, 64);
+            else DLFX_TOPK(1024, 32);
+        } else {
             if constexpr (sizeof(K) == 4) DLFX_TOPK(1024, 64);
             else return DLFX_ERR_TOO_LARGE;
         }
