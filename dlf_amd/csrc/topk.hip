@@ -11,6 +11,7 @@
 // Anything larger goes through the stable segmented argsort and keeps the first
 // `limit` entries of each row.
 #include <cstring>
+#include <limits>
 #include <type_traits>
 
 #include "common.hip.h"
@@ -64,19 +65,54 @@ struct TopkIo {
     int idx64, kind, largest;
 };
 
-constexpr int kCandCap = 4096;     // candidates kept in LDS after the pre-filter
+constexpr int kCandCap = 4096;     // candidates kept after the pre-filter (4-byte keys; half for 8-byte keys)
+template <typename K> constexpr int cand_cap() { return sizeof(K) == 4 ? kCandCap : kCandCap / 2; }
+constexpr int kAmbMax = 64;        // members of the deciding digit that are ranked directly
+constexpr int kSelectThreads = 256; // threads that run the exact selection among candidates
+constexpr uint32_t kRowDone = 0u, kRowWhole = 0xffffffffu;   // per-row hand-over state (else: candidate count)
 
 template <typename K>
 struct TopkShared {
     uint32_t hist[kRadix];
     uint32_t wave_tot[kRadix / kWave];
-    uint32_t scan_tot[16];
+    uint32_t scan_tot[32];
     uint32_t sel_digit, sel_k, sel_ties, count;
     K out_ord[kMaxLimit];
     uint32_t out_idx[kMaxLimit];
-    K cand_ord[kCandCap];
-    uint32_t cand_idx[kCandCap];
+    uint32_t rank[kMaxLimit];
+    K amb_ord[kAmbMax];
+    uint32_t amb_idx[kAmbMax];
+    K and_bits[16], or_bits[16];
+    uint32_t amb_count;
+    K cand_ord[cand_cap<K>()];
+    uint32_t cand_idx[cand_cap<K>()];
 };
+
+// Synchronises the TEAM threads that run a selection.  A single wave needs no hardware
+// barrier: its LDS accesses execute in program order, the fence only stops the compiler
+// from moving them across this point.
+template <int TEAM>
+__device__ __forceinline__ void team_sync() {
+    if constexpr (TEAM <= kWave) {
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    } else {
+        __syncthreads();
+    }
+}
+
+// Appends the items flagged `take` of the calling wave to an LDS list whose length is
+// *counter: one atomic per wave, slots in lane order.  Returns the slot (valid when take).
+__device__ __forceinline__ uint32_t wave_append(uint32_t* counter, bool take) {
+    const unsigned long long m = __ballot(take);
+    if (m == 0ull) return 0u;
+    const int lane = lane_id();
+    const int first = __ffsll(static_cast<long long>(m)) - 1;
+    uint32_t base = 0;
+    if (lane == first) base = atomicAdd(counter, static_cast<uint32_t>(__popcll(m)));
+    base = __shfl(base, first, kWave);
+    return base + static_cast<uint32_t>(__popcll(m & ((1ull << lane) - 1ull)));
+}
 
 // One radix-select step over the values val(i) of the items for which part(i)
 // holds: picks the digit (at `shift`) that contains the kk-th largest
@@ -84,31 +120,23 @@ struct TopkShared {
 // digit), sm.sel_ties (its population).  sm.hist must be all zero on entry and is
 // all zero again on return.
 template <int BLOCK, int ITEMS, bool ROLLED, typename K, typename Val, typename Part>
-__device__ __forceinline__ void select_digit(TopkShared<K>& sm, int shift, uint32_t kk, Val val, Part part) {
+__device__ __forceinline__ void select_digit(TopkShared<K>& sm, int nitems, int shift, uint32_t kk, Val val, Part part) {
     const int tid = threadIdx.x;
     const int lane = lane_id();
+    (void)lane;
     auto count_item = [&](int i) {
-        const bool in = part(i);
-        const uint32_t d = static_cast<uint32_t>(val(i) >> shift) & 0xffu;
-        // a wave whose participants all share the digit adds once
-        const unsigned long long in_mask = __ballot(in);
-        if (in_mask == 0ull) return;
-        const int first = __ffsll(static_cast<long long>(in_mask)) - 1;
-        const uint32_t d0 = __shfl(d, first, kWave);
-        if (__ballot(in && d != d0) == 0ull) {
-            if (lane == first) atomicAdd(&sm.hist[d0], static_cast<uint32_t>(__popcll(in_mask)));
-        } else if (in) {
-            atomicAdd(&sm.hist[d], 1u);
-        }
+        // callers skip bytes in which all items agree, so a digit shared by everyone (the one
+        // case that would serialise these adds) does not reach this point
+        if (part(i)) atomicAdd(&sm.hist[static_cast<uint32_t>(val(i) >> shift) & 0xffu], 1u);
     };
     if constexpr (ROLLED) {
 #pragma unroll 1
-        for (int i = 0; i < ITEMS; ++i) count_item(i);
+        for (int i = 0; i < nitems; ++i) count_item(i);
     } else {
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) count_item(i);
     }
-    __syncthreads();
+    team_sync<BLOCK>();
     if (tid < kWave) {
         // lane l owns digits 255-4l .. 252-4l (descending), so a scan over lanes is a suffix sum over digits
         uint32_t h[4], run = 0;
@@ -131,21 +159,23 @@ __device__ __forceinline__ void select_digit(TopkShared<K>& sm, int shift, uint3
             above += h[j];
         }
     }
-    __syncthreads();
+    team_sync<BLOCK>();
 }
 
 // The kk-th largest of the values val(i) over the items with part(i): most significant
 // byte first.  Returns the value; *rank_in_ties / *ties describe how many of the elements
 // equal to it still have to be taken and how many there are.
 template <int BLOCK, int ITEMS, bool ROLLED, typename V, typename K, typename Val, typename Valid>
-__device__ __forceinline__ V kth_largest(TopkShared<K>& sm, uint32_t kk, Val val, Valid valid,
-                                         uint32_t* rank_in_ties, uint32_t* ties) {
-    V prefix = 0;
+__device__ __forceinline__ V kth_largest(TopkShared<K>& sm, int nitems, uint32_t kk, Val val, Valid valid,
+                                         uint32_t* rank_in_ties, uint32_t* ties,
+                                         int first_pass = static_cast<int>(sizeof(V)) - 1, V known_high = 0) {
+    // bytes above first_pass are the same (known_high) in every participating value
+    V prefix = known_high;
 #pragma unroll 1
-    for (int pass = static_cast<int>(sizeof(V)) - 1; pass >= 0; --pass) {
+    for (int pass = first_pass; pass >= 0; --pass) {
         const int shift = 8 * pass;
         const V hi_mask = (pass == static_cast<int>(sizeof(V)) - 1) ? V(0) : static_cast<V>(~V(0) << (shift + 8));
-        select_digit<BLOCK, ITEMS, ROLLED>(sm, shift, kk, val, [&](int i) {
+        select_digit<BLOCK, ITEMS, ROLLED>(sm, nitems, shift, kk, val, [&](int i) {
             return valid(i) && ((val(i) ^ prefix) & hi_mask) == 0;
         });
         prefix |= static_cast<V>(sm.sel_digit) << shift;
@@ -156,57 +186,237 @@ __device__ __forceinline__ V kth_largest(TopkShared<K>& sm, uint32_t kk, Val val
     return prefix;
 }
 
+template <typename K>
+__device__ __forceinline__ void emit_one(const TopkIo<K>& io, K* yr, int64_t ir, const K* xr, int j, K ord, uint32_t ix) {
+    K bits = from_ord<K>(ord, io.kind, io.largest);
+    if (io.kind == kKeyFloat && (bits << 1) == 0) bits = xr[static_cast<int64_t>(ix) * io.sx];   // keep the zero's sign
+    yr[j * io.sy] = bits;
+    if (io.idx64) static_cast<int64_t*>(io.idx)[ir + j * io.si] = static_cast<int64_t>(ix);
+    else static_cast<int32_t*>(io.idx)[ir + j * io.si] = static_cast<int32_t>(ix);
+}
+
+// "entry j beats (o, x)": larger image, then lower index.
+template <typename K>
+__device__ __forceinline__ uint32_t beats(K oj, uint32_t xj, K o, uint32_t x) {
+    if constexpr (sizeof(K) == 4) {
+        // one 64-bit comparison of (image, ~index)
+        const uint64_t a = (static_cast<uint64_t>(oj) << 32) | static_cast<uint32_t>(~xj);
+        const uint64_t b = (static_cast<uint64_t>(o) << 32) | static_cast<uint32_t>(~x);
+        return a > b ? 1u : 0u;
+    } else {
+        return (oj > o || (oj == o && xj < x)) ? 1u : 0u;
+    }
+}
+
+// For each of `count` (image, index) entries held in LDS: sm.rank[e] = number of entries that
+// beat it (entries are distinct).  Quadratic: small counts.  Ends with a barrier.
+template <int BLOCK, typename K>
+__device__ __forceinline__ void compute_ranks(TopkShared<K>& sm, const K* e_ord, const uint32_t* e_idx, int count) {
+    const int tid = threadIdx.x;
+    for (int i = tid; i < count; i += BLOCK) sm.rank[i] = 0;
+    team_sync<BLOCK>();
+    int cp = 1;
+    while (cp < count) cp <<= 1;
+    // BLOCK / cp threads share one entry (one thread when there are more entries than threads),
+    // each scanning a slice of the others; eight independent LDS reads in flight
+    const int parts = cp <= BLOCK ? BLOCK / cp : 1;
+    const int per = (count + parts - 1) / parts;
+    for (int e0 = 0; e0 < count; e0 += BLOCK) {
+        const int e = e0 + (parts > 1 ? (tid & (cp - 1)) : tid);
+        const int part = parts > 1 ? tid / cp : 0;
+        if (e < count) {
+            const K o = e_ord[e];
+            const uint32_t x = e_idx[e];
+            const int lo = part * per;
+            const int hi = lo + per < count ? lo + per : count;
+            uint32_t r = 0;
+            int j = lo;
+            for (; j + 8 <= hi; j += 8) {
+                K oj[8];
+                uint32_t xj[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) { oj[u] = e_ord[j + u]; xj[u] = e_idx[j + u]; }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) r += beats<K>(oj[u], xj[u], o, x);
+            }
+            for (; j < hi; ++j) r += beats<K>(e_ord[j], e_idx[j], o, x);
+            if (parts > 1) { if (r) atomicAdd(&sm.rank[e], r); }
+            else sm.rank[e] = r;
+        }
+        if (parts > 1) break;
+    }
+    team_sync<BLOCK>();
+}
+
+// Writes the entries ranked below `limit` to their place in the outputs.
+template <int BLOCK, typename K>
+__device__ __forceinline__ void rank_emit(TopkShared<K>& sm, const K* e_ord, const uint32_t* e_idx, int count, int limit,
+                                          const TopkIo<K>& io, int64_t row, const K* xr) {
+    compute_ranks<BLOCK, K>(sm, e_ord, e_idx, count);
+    K* yr = io.y + io.ymap.at(row);
+    const int64_t ir = io.imap.at(row);
+    for (int e = threadIdx.x; e < count; e += BLOCK) {
+        const int r = static_cast<int>(sm.rank[e]);
+        if (r < limit) emit_one<K>(io, yr, ir, xr, r, e_ord[e], e_idx[e]);
+    }
+}
+
+constexpr int kRankSortMax = 64;     // winners up to which counting ranks beats a bitonic network
+
 // Exact selection of the `limit` best of the items (ord(i), idx(i)), best = larger image,
 // then lower index; writes them in that order.  Padding items carry image 0 and an index
 // that is not below the row length: they lose every tie, and limit <= row length, so no
 // validity test is needed.
+//
+// Radix select from the first byte in which the items differ; as soon as the digit that
+// holds the limit-th best has at most kAmbMax members, those members are ranked
+// directly (by image, then index) instead of refining further.
 template <int BLOCK, int ITEMS, bool ROLLED, typename K, typename Ord, typename Idx>
 __device__ __forceinline__ void select_and_emit(TopkShared<K>& sm, const TopkIo<K>& io, int64_t row, const K* xr,
-                                                int limit, Ord ord, Idx idx) {
+                                                int limit, int nitems, Ord ord, Idx idx) {
     const int tid = threadIdx.x;
-    if (tid == 0) sm.count = 0;
+    const int lane = lane_id();
+    const int w = tid / kWave;
+    constexpr int WAVES = BLOCK / kWave;
+    auto for_items = [&](auto&& body) {
+        if constexpr (ROLLED) {
+#pragma unroll 1
+            for (int i = 0; i < nitems; ++i) body(i);
+        } else {
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) body(i);
+        }
+    };
+    if (tid == 0) { sm.count = 0; sm.amb_count = 0; }
 
-    uint32_t kk = 0, ties = 0;
-    const K threshold = kth_largest<BLOCK, ITEMS, ROLLED, K>(sm, static_cast<uint32_t>(limit), ord, [](int) { return true; }, &kk, &ties);
-    // kk of the `ties` elements equal to the threshold are taken: those with the lowest indices,
-    // i.e. the kk largest images of ~index
-    uint32_t idx_limit = 0xffffffffu;
-    if (kk < ties) {
-        uint32_t k2 = 0, t2 = 0;
-        const uint32_t inv = kth_largest<BLOCK, ITEMS, ROLLED, uint32_t>(
-            sm, kk, [&](int i) { return ~idx(i); }, [&](int i) { return ord(i) == threshold; }, &k2, &t2);
-        idx_limit = ~inv;
-    }
-
-    // ---- compact the winners
-    auto take = [&](int i) {
-        const uint32_t ix = idx(i);
+    // ---- bytes in which every item agrees need no pass.  Padding (image 0) is left out of
+    // the comparison; should the limit reach into the padding-valued items, nothing is skipped.
+    K all_and = ~K(0), all_or = 0;
+    uint32_t nonzero = 0;
+    for_items([&](int i) {
         const K o = ord(i);
-        if (o > threshold || (o == threshold && ix <= idx_limit)) {
-            const uint32_t slot = atomicAdd(&sm.count, 1u);
-            if (slot < kMaxLimit) {
+        if (o != 0) { all_and &= o; all_or |= o; }
+        nonzero += static_cast<uint32_t>(__popcll(__ballot(o != 0)));
+    });
+    all_and = wave_reduce(all_and, [](K a, K b) { return a & b; });
+    all_or = wave_reduce(all_or, [](K a, K b) { return a | b; });
+    if (lane == 0) { sm.and_bits[w] = all_and; sm.or_bits[w] = all_or; sm.scan_tot[w] = nonzero; }
+    team_sync<BLOCK>();
+    nonzero = 0;
+    for (int i = 0; i < WAVES; ++i) { all_and &= sm.and_bits[i]; all_or |= sm.or_bits[i]; nonzero += sm.scan_tot[i]; }
+    team_sync<BLOCK>();            // scan_tot is reused below
+    const K differ = (nonzero >= static_cast<uint32_t>(limit)) ? static_cast<K>(all_and ^ all_or) : ~K(0);
+
+    K prefix = 0, decided = 0;
+    uint32_t kk = static_cast<uint32_t>(limit), ties = nonzero;
+#pragma unroll 1
+    for (int pass = static_cast<int>(sizeof(K)) - 1; pass >= 0; --pass) {
+        const int shift = 8 * pass;
+        if (((differ >> shift) & 0xffu) == 0) {
+            // all (non-padding) items share this byte
+            prefix |= all_and & (static_cast<K>(0xffu) << shift);
+            decided = static_cast<K>(~K(0) << shift);
+            continue;
+        }
+        select_digit<BLOCK, ITEMS, ROLLED>(sm, nitems, shift, kk, ord, [&](int i) { return ((ord(i) ^ prefix) & decided) == 0; });
+        prefix |= static_cast<K>(sm.sel_digit) << shift;
+        decided = static_cast<K>(~K(0) << shift);
+        kk = sm.sel_k;
+        ties = sm.sel_ties;
+        if (ties <= kAmbMax) break;
+    }
+    // now: (image & decided) > prefix  -> in;  == prefix -> one of `ties` items of which kk are in;  < prefix -> out
+
+    if (ties <= kAmbMax) {
+        // two sweeps, no atomics: every wave counts its winners / deciding-digit members with
+        // ballots, the counts are prefix-summed over the team's waves, then each item is placed
+        // at wave offset + number of such items before it in the wave
+        const unsigned long long lt_mask = (1ull << lane) - 1ull;
+        uint32_t n_in = 0, n_amb = 0;
+        for_items([&](int i) {
+            const K hi = ord(i) & decided;
+            n_in += static_cast<uint32_t>(__popcll(__ballot(hi > prefix)));
+            n_amb += static_cast<uint32_t>(__popcll(__ballot(hi == prefix)));
+        });
+        if (lane == 0) { sm.scan_tot[w] = n_in; sm.scan_tot[WAVES + w] = n_amb; }
+        team_sync<BLOCK>();
+        uint32_t b_in = 0, b_amb = 0;
+        for (int i = 0; i < w; ++i) { b_in += sm.scan_tot[i]; b_amb += sm.scan_tot[WAVES + i]; }
+        for_items([&](int i) {
+            const K o = ord(i);
+            const K hi = o & decided;
+            const bool in = hi > prefix, maybe = hi == prefix;
+            const unsigned long long m_in = __ballot(in), m_amb = __ballot(maybe);
+            if (in) {
+                const uint32_t slot = b_in + static_cast<uint32_t>(__popcll(m_in & lt_mask));
+                if (slot < kMaxLimit) { sm.out_ord[slot] = o; sm.out_idx[slot] = idx(i); }
+            }
+            if (maybe) {
+                const uint32_t slot = b_amb + static_cast<uint32_t>(__popcll(m_amb & lt_mask));
+                if (slot < kAmbMax) { sm.amb_ord[slot] = o; sm.amb_idx[slot] = idx(i); }
+            }
+            b_in += static_cast<uint32_t>(__popcll(m_in));
+            b_amb += static_cast<uint32_t>(__popcll(m_amb));
+        });
+        if (tid == 0) sm.count = static_cast<uint32_t>(limit) - kk;     // winners above the deciding digit
+        team_sync<BLOCK>();
+        if (kk == ties) {
+            // the whole digit is in
+            for (int e0 = 0; e0 < static_cast<int>(ties); e0 += BLOCK) {
+                const int e = e0 + tid;
+                const bool in = e < static_cast<int>(ties);
+                const uint32_t slot = wave_append(&sm.count, in);
+                if (in && slot < kMaxLimit) {
+                    sm.out_ord[slot] = sm.amb_ord[e];
+                    sm.out_idx[slot] = sm.amb_idx[e];
+                }
+            }
+        } else {
+            compute_ranks<BLOCK, K>(sm, sm.amb_ord, sm.amb_idx, static_cast<int>(ties));
+            for (int e0 = 0; e0 < static_cast<int>(ties); e0 += BLOCK) {
+                const int e = e0 + tid;
+                const bool in = e < static_cast<int>(ties) && sm.rank[e] < kk;
+                const uint32_t slot = wave_append(&sm.count, in);
+                if (in && slot < kMaxLimit) {
+                    sm.out_ord[slot] = sm.amb_ord[e];
+                    sm.out_idx[slot] = sm.amb_idx[e];
+                }
+            }
+        }
+    } else {
+        // more than kAmbMax items share the threshold image: take the kk lowest indices
+        // among them, i.e. the kk largest images of ~index (indices are below 2^24 here)
+        uint32_t k2 = 0, t2 = 0;
+        const K threshold = prefix;
+        const uint32_t inv = kth_largest<BLOCK, ITEMS, ROLLED, uint32_t>(
+            sm, nitems, kk, [&](int i) { return ~idx(i); }, [&](int i) { return ord(i) == threshold && idx(i) < (1u << 24); },
+            &k2, &t2, 2, 0xff000000u);
+        const uint32_t idx_limit = ~inv;
+        for_items([&](int i) {
+            const uint32_t ix = idx(i);
+            const K o = ord(i);
+            const bool in = o > threshold || (o == threshold && ix <= idx_limit);
+            const uint32_t slot = wave_append(&sm.count, in);
+            if (in && slot < kMaxLimit) {
                 sm.out_ord[slot] = o;
                 sm.out_idx[slot] = ix;
             }
-        }
-    };
-    if constexpr (ROLLED) {
-#pragma unroll 1
-        for (int i = 0; i < ITEMS; ++i) take(i);
-    } else {
-#pragma unroll
-        for (int i = 0; i < ITEMS; ++i) take(i);
+        });
+    }
+    team_sync<BLOCK>();
+
+    // ---- order the winners: best first
+    if (limit <= kRankSortMax) {
+        rank_emit<BLOCK, K>(sm, sm.out_ord, sm.out_idx, limit, limit, io, row, xr);
+        return;
     }
     int kp = 1;
     while (kp < limit) kp <<= 1;
-    __syncthreads();
     for (int i = limit + tid; i < kp; i += BLOCK) {
         sm.out_ord[i] = 0;
         sm.out_idx[i] = 0xffffffffu;      // padding: worse than any real entry
     }
-    __syncthreads();
-
-    // ---- bitonic network: best first (larger image, then lower index)
+    team_sync<BLOCK>();
     for (int size = 2; size <= kp; size <<= 1) {
         for (int stride = size >> 1; stride > 0; stride >>= 1) {
             for (int t = tid; t < kp / 2; t += BLOCK) {
@@ -221,27 +431,33 @@ __device__ __forceinline__ void select_and_emit(TopkShared<K>& sm, const TopkIo<
                     sm.out_idx[i] = xj; sm.out_idx[j] = xi;
                 }
             }
-            __syncthreads();
+            team_sync<BLOCK>();
         }
     }
-
-    // ---- write
     K* yr = io.y + io.ymap.at(row);
     const int64_t ir = io.imap.at(row);
-    for (int j = tid; j < limit; j += BLOCK) {
-        const uint32_t ix = sm.out_idx[j];
-        K bits = from_ord<K>(sm.out_ord[j], io.kind, io.largest);
-        if (io.kind == kKeyFloat && (bits << 1) == 0) bits = xr[static_cast<int64_t>(ix) * io.sx];   // keep the zero's sign
-        yr[j * io.sy] = bits;
-        if (io.idx64) static_cast<int64_t*>(io.idx)[ir + j * io.si] = static_cast<int64_t>(ix);
-        else static_cast<int32_t*>(io.idx)[ir + j * io.si] = static_cast<int32_t>(ix);
-    }
+    for (int j = tid; j < limit; j += BLOCK) emit_one<K>(io, yr, ir, xr, j, sm.out_ord[j], sm.out_idx[j]);
 }
 
-// ALIGNED: the axis is contiguous and every row starts on a 16-byte boundary (checked on the
-// host), so rows are read with 128-bit loads off one base register.
-template <typename K, int BLOCK, int ITEMS, bool ALIGNED>
-__global__ __launch_bounds__(BLOCK) void topk_select(TopkIo<K> io, int64_t n, int limit) {
+template <typename T> struct BitsOf;
+template <> struct BitsOf<float>   { using type = uint32_t; static constexpr int kind = kKeyFloat; };
+template <> struct BitsOf<int32_t> { using type = uint32_t; static constexpr int kind = kKeyInt; };
+template <> struct BitsOf<double>  { using type = uint64_t; static constexpr int kind = kKeyFloat; };
+template <> struct BitsOf<int64_t> { using type = uint64_t; static constexpr int kind = kKeyInt; };
+
+// T: the element type.  ALIGNED: the axis is contiguous and every row starts on a 16-byte
+// boundary (checked on the host), so rows are read with 128-bit loads off one base register.
+//
+// Elements are held as scores of type T: the element itself when the largest are wanted,
+// its order-reversing image otherwise (sign flip for floats, complement for integers), so
+// the kernel always looks for the largest scores and compares them natively.
+template <typename T, int BLOCK, int ITEMS, bool ALIGNED>
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(BLOCK >= 1024 && sizeof(T) == 4 && ITEMS <= 32 ? 8 : 1)))
+void topk_select(TopkIo<typename BitsOf<T>::type> io, int64_t n, int limit,
+                 uint32_t* __restrict__ row_state, typename BitsOf<T>::type* __restrict__ spill_ord,
+                 uint32_t* __restrict__ spill_idx) {
+    using K = typename BitsOf<T>::type;
+    constexpr int kind = BitsOf<T>::kind;
     constexpr int V = (16 / sizeof(K) < ITEMS) ? 16 / sizeof(K) : ITEMS;
     constexpr int G = ITEMS / V;
     constexpr int WAVES = BLOCK / kWave;
@@ -261,30 +477,39 @@ __global__ __launch_bounds__(BLOCK) void topk_select(TopkIo<K> io, int64_t n, in
     auto index_of = [&](int i) -> uint32_t {
         return tid_v + static_cast<uint32_t>((i / V) * (BLOCK * V) + (i % V));
     };
-    auto in_row = [&](int i) -> bool { return index_of(i) < n32; };
+    const K flip = io.largest ? K(0) : (kind == kKeyFloat ? KeyBits<K>::kSign : ~K(0));
+    const T worst = std::is_integral<T>::value ? std::numeric_limits<T>::lowest() : -std::numeric_limits<T>::infinity();
+    auto score_of = [&](K bits) -> T { return bit_cast<T>(static_cast<K>(bits ^ flip)); };
+    // order-preserving unsigned image of a score (scores are always maximised)
+    auto ord_of = [&](T sc) -> K { return to_ord<K>(bit_cast<K>(sc), kind, 1); };
+    auto load_ord = [&](int i) -> K {        // straight from memory; padding -> 0
+        const uint32_t ix = index_of(i);
+        return ix < n32 ? ord_of(score_of(xr[static_cast<int64_t>(ix) * io.sx])) : K(0);
+    };
 
-    if constexpr (BLOCK * ITEMS <= kCandCap) {
+    constexpr int CAP = cand_cap<K>();
+    if constexpr (BLOCK * ITEMS <= CAP) {
         // short rows: select straight from registers
         K ord[ITEMS];
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i)
-            ord[i] = in_row(i) ? to_ord<K>(xr[static_cast<int64_t>(index_of(i)) * io.sx], io.kind, io.largest) : K(0);
+        for (int i = 0; i < ITEMS; ++i) ord[i] = load_ord(i);
         __syncthreads();
-        select_and_emit<BLOCK, ITEMS, false>(sm, io, row, xr, limit, [&](int i) { return ord[i]; }, index_of);
+        if (tid == 0) row_state[row] = kRowDone;
+        select_and_emit<BLOCK, ITEMS, false>(sm, io, row, xr, limit, ITEMS, [&](int i) { return ord[i]; }, index_of);
     } else {
-        K ord[ITEMS];
+        T sc[ITEMS];
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             const uint32_t i0 = tid_v + static_cast<uint32_t>(g * (BLOCK * V));
             if (ALIGNED && i0 + V <= n32) {
                 const VecT a = *reinterpret_cast<const VecT*>(xr + i0);
 #pragma unroll
-                for (int e = 0; e < V; ++e) ord[g * V + e] = to_ord<K>(a.v[e], io.kind, io.largest);
+                for (int e = 0; e < V; ++e) sc[g * V + e] = score_of(a.v[e]);
             } else {
 #pragma unroll
                 for (int e = 0; e < V; ++e) {
                     const int64_t at = ALIGNED ? static_cast<int64_t>(i0 + e) : static_cast<int64_t>(i0 + e) * io.sx;
-                    ord[g * V + e] = (i0 + e < n32) ? to_ord<K>(xr[at], io.kind, io.largest) : K(0);
+                    sc[g * V + e] = (i0 + e < n32) ? score_of(xr[at]) : worst;
                 }
             }
         }
@@ -292,76 +517,143 @@ __global__ __launch_bounds__(BLOCK) void topk_select(TopkIo<K> io, int64_t n, in
         // element each group holds gives `groups` distinct elements, so the smallest of those
         // maxima cannot exceed the limit-th largest element of the row: everything below it is
         // out.  What is left is usually a few times `limit` elements.
-        K tmax = 0;
+        T tmax = worst;
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) tmax = ord[i] > tmax ? ord[i] : tmax;      // padding is 0
+        for (int i = 0; i < ITEMS; ++i) tmax = sc[i] > tmax ? sc[i] : tmax;
         int groups = 1;
         while (groups < limit && groups < BLOCK) groups <<= 1;
         const int span = BLOCK / groups;               // threads per group, a power of two
-        auto kmax = [](K a, K b) { return a > b ? a : b; };
-        auto kmin = [](K a, K b) { return a < b ? a : b; };
-        K bound;
+        auto tmaxf = [](T a, T b) { return a > b ? a : b; };
+        auto tminf = [](T a, T b) { return a < b ? a : b; };
+        T* red = reinterpret_cast<T*>(sm.out_ord);
+        T bound;
         if (span >= kWave) {
-            const K wmax = wave_reduce(tmax, kmax);
-            if (lane == 0) sm.cand_ord[w] = wmax;
+            const T wmax = wave_reduce(tmax, tmaxf);
+            if (lane == 0) red[w] = wmax;
             __syncthreads();
-            bound = ~K(0);
             const int wpg = span / kWave;              // waves per group
-            for (int g0 = 0; g0 < WAVES; g0 += wpg) {
-                K gm = 0;
-                for (int j = 0; j < wpg; ++j) gm = kmax(gm, sm.cand_ord[g0 + j]);
-                bound = kmin(bound, gm);
+            bound = red[0];
+            for (int j = 1; j < wpg; ++j) bound = tmaxf(bound, red[j]);
+            for (int g0 = wpg; g0 < WAVES; g0 += wpg) {
+                T gm = red[g0];
+                for (int j = 1; j < wpg; ++j) gm = tmaxf(gm, red[g0 + j]);
+                bound = tminf(bound, gm);
             }
         } else {
-            const K gmax = group_reduce(tmax, span, kmax);
-            const K wmin = wave_reduce(gmax, kmin);
-            if (lane == 0) sm.cand_ord[w] = wmin;
+            const T gmax = group_reduce(tmax, span, tmaxf);
+            const T wmin = wave_reduce(gmax, tminf);
+            if (lane == 0) red[w] = wmin;
             __syncthreads();
-            bound = ~K(0);
-            for (int j = 0; j < WAVES; ++j) bound = kmin(bound, sm.cand_ord[j]);
+            bound = red[0];
+            for (int j = 1; j < WAVES; ++j) bound = tminf(bound, red[j]);
         }
-        uint32_t mine = 0;
+        // ---- survivors go to LDS as (image, index), in element order: each wave counts its
+        // survivors with ballots, the waves' counts are prefix-summed through LDS, and a second
+        // sweep places every survivor at wave offset + number of survivors before it in the wave
+        uint32_t wave_count = 0;
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) mine += (ord[i] >= bound) ? 1u : 0u;
-        const uint32_t incl = wave_scan_inclusive(mine, 0u, [](uint32_t a, uint32_t b) { return a + b; });
-        if (lane == kWave - 1) sm.scan_tot[w] = incl;
+        for (int i = 0; i < ITEMS; ++i) wave_count += static_cast<uint32_t>(__popcll(__ballot(sc[i] >= bound)));
+        if (lane == 0) sm.scan_tot[w] = wave_count;
         __syncthreads();
-        uint32_t before = incl - mine, total = 0;
+        uint32_t wave_base = 0, total = 0;
         for (int i = 0; i < WAVES; ++i) {
             const uint32_t t = sm.scan_tot[i];
-            if (i < w) before += t;
+            if (i < w) wave_base += t;
             total += t;
         }
-        if (total <= kCandCap && limit <= BLOCK) {
+        if (total <= CAP) {
+            const unsigned long long lt_mask = (1ull << lane) - 1ull;
 #pragma unroll
             for (int i = 0; i < ITEMS; ++i) {
-                if (ord[i] >= bound) {
-                    sm.cand_ord[before] = ord[i];
-                    sm.cand_idx[before] = index_of(i);
-                    ++before;
+                const bool pass = sc[i] >= bound;
+                const unsigned long long m = __ballot(pass);
+                if (m != 0ull) {
+                    if (pass) {
+                        const uint32_t slot = wave_base + static_cast<uint32_t>(__popcll(m & lt_mask));
+                        sm.cand_ord[slot] = ord_of(sc[i]);
+                        sm.cand_idx[slot] = index_of(i);
+                    }
+                    wave_base += static_cast<uint32_t>(__popcll(m));
                 }
             }
-            __syncthreads();
-            constexpr int CI = kCandCap / BLOCK;
-            K cord[CI];
-            uint32_t cidx[CI];
-#pragma unroll
-            for (int j = 0; j < CI; ++j) {
-                const uint32_t slot = j * BLOCK + tid;
-                cord[j] = slot < total ? sm.cand_ord[slot] : K(0);
-                cidx[j] = slot < total ? sm.cand_idx[slot] : 0xffffffffu;
-            }
-            select_and_emit<BLOCK, CI, false>(sm, io, row, xr, limit, [&](int j) { return cord[j]; },
-                                       [&](int j) { return cidx[j]; });
-        } else {
-            // the filter kept too much (e.g. long runs of equal values): exact selection over the
-            // whole row, re-reading elements (they are cache resident) instead of holding them
-            __syncthreads();
-            select_and_emit<BLOCK, ITEMS, true>(
-                sm, io, row, xr, limit,
-                [&](int i) { return in_row(i) ? to_ord<K>(xr[static_cast<int64_t>(index_of(i)) * io.sx], io.kind, io.largest) : K(0); },
-                index_of);
         }
+        __syncthreads();
+        // What happens next depends on how many survived:
+        //   * at most one per lane of a wave: the first wave ranks them and writes the answer;
+        //   * up to kCandCap: they are handed, through global memory, to topk_finish, whose
+        //     small workgroups hide the latency of the exact selection much better than this
+        //     one (which holds a whole row) could;
+        //   * more (long runs of equal values, adversarial order), or a limit the bound does
+        //     not hold for: topk_finish selects from the row itself.
+        if (total <= kWave && limit <= BLOCK) {
+            if (tid == 0) row_state[row] = kRowDone;
+            if (tid >= kWave) return;
+            const int cnt = static_cast<int>(total);
+            if (tid < cnt) {
+                const K o = sm.cand_ord[tid];
+                const uint32_t x = sm.cand_idx[tid];
+                uint32_t r = 0;
+                for (int j = 0; j < cnt; ++j) r += beats<K>(sm.cand_ord[j], sm.cand_idx[j], o, x);
+                if (static_cast<int>(r) < limit)
+                    emit_one<K>(io, io.y + io.ymap.at(row), io.imap.at(row), xr, static_cast<int>(r), o, x);
+            }
+        } else if (total <= CAP && limit <= BLOCK) {
+            if (tid == 0) row_state[row] = total;
+            K* so = spill_ord + row * CAP;
+            uint32_t* si = spill_idx + row * CAP;
+            for (uint32_t i = tid; i < total; i += BLOCK) {
+                so[i] = sm.cand_ord[i];
+                si[i] = sm.cand_idx[i];
+            }
+        } else {
+            if (tid == 0) row_state[row] = kRowWhole;
+        }
+    }
+}
+
+// Second stage of the selection for rows topk_select did not finish: exact selection among the
+// row's spilled candidates, or over the whole row when it has to be.
+template <typename T>
+__global__ __launch_bounds__(kSelectThreads) void topk_finish(
+    TopkIo<typename BitsOf<T>::type> io, int64_t n, int limit, const uint32_t* __restrict__ row_state,
+    const typename BitsOf<T>::type* __restrict__ spill_ord, const uint32_t* __restrict__ spill_idx) {
+    using K = typename BitsOf<T>::type;
+    constexpr int kind = BitsOf<T>::kind;
+    constexpr int SEL = kSelectThreads;
+    __shared__ TopkShared<K> sm;
+    const int tid = threadIdx.x;
+    const int64_t row = blockIdx.x;
+    const uint32_t state = row_state[row];
+    if (state == kRowDone) return;
+    const K* xr = io.x + io.xmap.at(row);
+    if (tid < kRadix) sm.hist[tid] = 0;
+    if (state != kRowWhole) {
+        const uint32_t total = state;
+        constexpr int CAP = cand_cap<K>();
+        const K* so = spill_ord + row * CAP;
+        const uint32_t* si = spill_idx + row * CAP;
+        for (uint32_t i = tid; i < total; i += SEL) {
+            sm.cand_ord[i] = so[i];
+            sm.cand_idx[i] = si[i];
+        }
+        __syncthreads();
+        const int per_thread = static_cast<int>((total + SEL - 1) / SEL);
+        select_and_emit<SEL, CAP / SEL, true>(
+            sm, io, row, xr, limit, per_thread,
+            [&](int j) { const uint32_t s2 = j * SEL + tid; return s2 < total ? sm.cand_ord[s2] : K(0); },
+            [&](int j) { const uint32_t s2 = j * SEL + tid; return s2 < total ? sm.cand_idx[s2] : 0xffffffffu; });
+    } else {
+        __syncthreads();
+        const uint32_t n32 = static_cast<uint32_t>(n);
+        const K flip = io.largest ? K(0) : (kind == kKeyFloat ? KeyBits<K>::kSign : ~K(0));
+        const int per_thread = static_cast<int>((n32 + SEL - 1) / SEL);
+        select_and_emit<SEL, 1, true>(
+            sm, io, row, xr, limit, per_thread,
+            [&](int j) {
+                const uint32_t ix = j * SEL + tid;
+                return ix < n32 ? to_ord<K>(static_cast<K>(xr[static_cast<int64_t>(ix) * io.sx] ^ flip), kind, 1) : K(0);
+            },
+            [&](int j) { return static_cast<uint32_t>(j * SEL + tid); });
     }
 }
 
@@ -378,16 +670,36 @@ __global__ __launch_bounds__(256) void topk_take(const K* __restrict__ ys, const
     else static_cast<int32_t*>(io.idx)[io.imap.at(row) + j * io.si] = ix;
 }
 
+// Scratch of the selection path: one state word per row and room for kCandCap spilled
+// candidates per row (rows no longer than kCandCap finish in one kernel and need none).
+struct SelectLayout {
+    size_t state_off, ord_off, idx_off, total;
+};
+SelectLayout select_layout(size_t key_size, int64_t m, int64_t n) {
+    SelectLayout l{0, 0, 0, 0};
+    const int64_t cap = key_size == 4 ? kCandCap : kCandCap / 2;
+    l.ord_off = align_up(static_cast<size_t>(m) * 4, 256);
+    if (n <= cap) {
+        l.idx_off = l.ord_off;
+        l.total = l.ord_off;
+        return l;
+    }
+    l.idx_off = l.ord_off + align_up(static_cast<size_t>(m) * cap * key_size, 256);
+    l.total = l.idx_off + align_up(static_cast<size_t>(m) * cap * 4, 256);
+    return l;
+}
+
 bool selection_fits(size_t key_size, int64_t n, int64_t limit) {
     if (limit > kMaxLimit) return false;
     return n <= (key_size == 4 ? 65536 : 32768);
 }
 
-template <typename K>
-int run_top_k(hipStream_t stream, int64_t limit, int dir, int kind, int dtype, int index_dtype,
+template <typename T>
+int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_dtype,
               int rank, const int64_t* x_dims, const int64_t* y_dims,
               const void* x, const int64_t* xs, void* y, const int64_t* ys, void* idx, const int64_t* is,
               void* scratch, size_t scratch_bytes) {
+    using K = typename BitsOf<T>::type;
     const int64_t n = x_dims[rank - 1];
     const int64_t m = view_size(rank, x_dims) / n;
     TopkIo<K> io;
@@ -402,7 +714,7 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int kind, int dtype, i
     io.sy = ys[rank - 1];
     io.si = is[rank - 1];
     io.idx64 = index_dtype == DLFX_I64;
-    io.kind = kind;
+    io.kind = BitsOf<T>::kind;
     io.largest = dir ? 1 : 0;
     if (m > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
 
@@ -411,10 +723,16 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int kind, int dtype, i
         const int lim = static_cast<int>(limit);
         bool aligned = io.sx == 1 && reinterpret_cast<uintptr_t>(io.x) % 16 == 0;
         for (int i = 0; i < io.xmap.rank; ++i) aligned = aligned && io.xmap.strides[i] % (16 / static_cast<int64_t>(sizeof(K))) == 0;
+        const SelectLayout sl = select_layout(sizeof(K), m, n);
+        if (sl.total && (!scratch || scratch_bytes < sl.total)) return DLFX_ERR_SCRATCH_TOO_SMALL;
+        char* sbase = static_cast<char*>(scratch);
+        uint32_t* row_state = reinterpret_cast<uint32_t*>(sbase + sl.state_off);
+        K* spill_ord = reinterpret_cast<K*>(sbase + sl.ord_off);
+        uint32_t* spill_idx = reinterpret_cast<uint32_t*>(sbase + sl.idx_off);
 #define DLFX_TOPK(BLOCK, ITEMS)                                                                     \
     do {                                                                                            \
-        if (aligned) topk_select<K, BLOCK, ITEMS, true><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim); \
-        else topk_select<K, BLOCK, ITEMS, false><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim);      \
+        if (aligned) topk_select<T, BLOCK, ITEMS, true><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx); \
+        else topk_select<T, BLOCK, ITEMS, false><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx);      \
     } while (0)
         if (n <= 256) DLFX_TOPK(256, 1);
         else if (n <= 1024) DLFX_TOPK(256, 4);
@@ -423,14 +741,17 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int kind, int dtype, i
         else if (n <= 8192) DLFX_TOPK(1024, 8);
         else if (n <= 16384) DLFX_TOPK(1024, 16);
         else if (n <= 32768) {
-            if (lim <= 512) DLFX_TOPK(512, 64);
-            else DLFX_TOPK(1024, 32);
+            DLFX_TOPK(1024, 32);
         } else {
             if constexpr (sizeof(K) == 4) DLFX_TOPK(1024, 64);
             else return DLFX_ERR_TOO_LARGE;
         }
 #undef DLFX_TOPK
         DLFX_CHECK_LAUNCH();
+        if (n > cand_cap<K>()) {
+            topk_finish<T><<<grid, dim3(kSelectThreads), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx);
+            DLFX_CHECK_LAUNCH();
+        }
         return DLFX_OK;
     }
 
@@ -460,7 +781,7 @@ using namespace dlfx;
 extern "C" size_t dlfx_top_k_scratch_bytes(int dtype, int64_t m, int64_t n, int64_t limit) {
     const size_t es = dtype_size(dtype);
     if (!es || m <= 0 || n <= 0) return 0;
-    if (selection_fits(es, n, limit)) return 0;
+    if (selection_fits(es, n, limit)) return select_layout(es, m, n).total;
     return align_up(static_cast<size_t>(m) * n * es, 256) + align_up(static_cast<size_t>(m) * n * 4, 256) +
            argsort_scratch_bytes_impl(dtype, m, n);
 }
@@ -486,10 +807,10 @@ extern "C" int dlfx_top_k(dlfx_stream_t stream, int64_t limit, int dir, int dtyp
     void* ip = static_cast<char*>(idx) + i_offset * (index_dtype == DLFX_I64 ? 8 : 4);
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (dtype) {
-    case DLFX_F32: return run_top_k<uint32_t>(s, limit, dir, kKeyFloat, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
-    case DLFX_I32: return run_top_k<uint32_t>(s, limit, dir, kKeyInt, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
-    case DLFX_F64: return run_top_k<uint64_t>(s, limit, dir, kKeyFloat, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
-    case DLFX_I64: return run_top_k<uint64_t>(s, limit, dir, kKeyInt, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
+    case DLFX_F32: return run_top_k<float>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
+    case DLFX_I32: return run_top_k<int32_t>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
+    case DLFX_F64: return run_top_k<double>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
+    case DLFX_I64: return run_top_k<int64_t>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
     default: return DLFX_ERR_UNSUPPORTED_DTYPE;
     }
 }
