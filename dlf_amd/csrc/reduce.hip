@@ -175,7 +175,8 @@ row_partial_contig(const typename R::in_t* __restrict__ p, int64_t n, int g, int
     int64_t v = v_lo + g;
     // four independent 128-bit loads in flight per lane
     for (; v + 3 * static_cast<int64_t>(width) < v_hi; v += 4 * static_cast<int64_t>(width)) {
-        VecT a = pv[v], b = pv[v + width], c = pv[v + 2 * width], d = pv[v + 3 * width];
+        VecT a = load_stream(&pv[v]), b = load_stream(&pv[v + width]), c = load_stream(&pv[v + 2 * width]),
+             d = load_stream(&pv[v + 3 * width]);
         const int64_t j0 = head + v * V;
 #pragma unroll
         for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(a.v[e], j0 + e));
@@ -187,7 +188,7 @@ row_partial_contig(const typename R::in_t* __restrict__ p, int64_t n, int g, int
         for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(d.v[e], j0 + 3 * static_cast<int64_t>(width) * V + e));
     }
     for (; v < v_hi; v += width) {
-        VecT a = pv[v];
+        VecT a = load_stream(&pv[v]);
         const int64_t j0 = head + v * V;
 #pragma unroll
         for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(a.v[e], j0 + e));
@@ -309,11 +310,11 @@ __global__ __launch_bounds__(kBlock) void reduce_cols(
             for (; j + 7 * TY < hi; j += 8 * TY) {
                 typename R::in_t v[8];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) v[u] = p[(j + u * TY) * s];
+                for (int u = 0; u < 8; ++u) v[u] = load_stream(&p[(j + u * TY) * s]);
 #pragma unroll
                 for (int u = 0; u < 8; ++u) acc = R::join(acc, R::map(v[u], j + u * TY));
             }
-            for (; j < hi; j += TY) acc = R::join(acc, R::map(p[j * s], j));
+            for (; j < hi; j += TY) acc = R::join(acc, R::map(load_stream(&p[j * s]), j));
         } else {
             for (int64_t j = lo + ty; j < hi; j += TY) acc = R::join(acc, R::map(p[red.at(j)], j));
         }

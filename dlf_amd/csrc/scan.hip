@@ -156,7 +156,7 @@ __device__ __forceinline__ void scan_tile(
         const VecT* pv = reinterpret_cast<const VecT*>(xr + seg);
 #pragma unroll
         for (int k = 0; k < KV; ++k) {
-            VecT a = pv[k * kWave + lane];
+            VecT a = load_stream(&pv[k * kWave + lane]);
 #pragma unroll
             for (int e = 0; e < V; ++e) vals[k * V + e] = a.v[e];
         }
@@ -284,7 +284,7 @@ __device__ __forceinline__ void scan_tile(
             VecT a;
 #pragma unroll
             for (int e = 0; e < V; ++e) a.v[e] = vals[k * V + e];
-            pv[k * kWave + lane] = a;
+            store_stream(&pv[k * kWave + lane], a);
         }
     } else {
 #pragma unroll
@@ -353,7 +353,7 @@ __global__ __launch_bounds__(kBlock) void scan_cols(
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int64_t p = p0 + r;
-            v[r] = (live && r < chunk && p < n) ? xc[p * sx] : Op::identity();
+            v[r] = (live && r < chunk && p < n) ? load_stream(&xc[p * sx]) : Op::identity();
         }
 #pragma unroll
         for (int r = 1; r < R; ++r) v[r] = Op::apply(v[r - 1], v[r]);
@@ -374,13 +374,13 @@ __global__ __launch_bounds__(kBlock) void scan_cols(
                 for (int r = 0; r < R; ++r) {
                     const int64_t p = p0 + r;
                     const T prev = (r == 0) ? pre : Op::apply(pre, v[r > 0 ? r - 1 : 0]);
-                    if (r < chunk && p < n) yc[p * sy] = prev;
+                    if (r < chunk && p < n) store_stream(&yc[p * sy], prev);
                 }
             } else {
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const int64_t p = p0 + r;
-                    if (r < chunk && p < n) yc[p * sy] = Op::apply(pre, v[r]);
+                    if (r < chunk && p < n) store_stream(&yc[p * sy], Op::apply(pre, v[r]));
                 }
             }
         }

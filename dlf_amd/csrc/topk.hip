@@ -502,7 +502,7 @@ void topk_select(TopkIo<typename BitsOf<T>::type> io, int64_t n, int limit,
         for (int g = 0; g < G; ++g) {
             const uint32_t i0 = tid_v + static_cast<uint32_t>(g * (BLOCK * V));
             if (ALIGNED && i0 + V <= n32) {
-                const VecT a = *reinterpret_cast<const VecT*>(xr + i0);
+                const VecT a = load_stream(reinterpret_cast<const VecT*>(xr + i0));
 #pragma unroll
                 for (int e = 0; e < V; ++e) sc[g * V + e] = score_of(a.v[e]);
             } else {
