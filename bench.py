@@ -48,6 +48,9 @@ class Op:
 
 
 def make_ops(be, which):
+    want = set(which.split(","))
+    def on(*names):
+        return bool(want & set(names))
     import numpy as np
     import torch
     from dlf_amd import frontend as F
@@ -109,7 +112,7 @@ def make_ops(be, which):
     ops = []
 
     # ---------------- C2: scans and the long reduce (the step)
-    if which in ("all", "step", "c2"):
+    if on("all", "step", "c2"):
         xi = gen((64, 1 << 20), torch.int32, lambda c: synth.randint(2 + 100 * c, 0, 100), 4)
         calls, y = scan_calls(xi, 1)
 
@@ -141,7 +144,7 @@ def make_ops(be, which):
         ops.append(Op("C2c", "reduce_sum_f32_[2^30]", 1 << 30, 4 * (1 << 30) + 4, calls, v_c2c, "reduce_rows_block"))
 
     # ---------------- C1: logits head
-    if which in ("all", "c1"):
+    if on("all", "c1"):
         x1 = gen((256, 1000), torch.float32, lambda c: synth.normal(1 + 100 * c), 8)
         for name in ("reduce_sum", "reduce_max", "reduce_log_sum_exp"):
             calls, outs = reduce_calls(name, x1, [1])
@@ -161,19 +164,19 @@ def make_ops(be, which):
         ops += topk_ops(be, tensor, x1, [5], "C1", "[256,1000]")
 
     # ---------------- C3: top_k
-    if which in ("all", "c3"):
+    if on("all", "c3"):
         x3 = gen((4096, 32000), torch.float32, lambda c: synth.quantised_normal(5 + 100 * c), 4)
         ops += topk_ops(be, tensor, x3, [1, 5, 50, 256], "C3", "[4096,32000]")
 
     # ---------------- C4: sort / argsort
-    if which in ("all", "c4"):
+    if on("all", "c4"):
         x4a = gen((1024, 65536), torch.float32, lambda c: synth.quantised_uniform(6 + 100 * c), 4)
         ops += sort_ops(be, tensor, x4a, "C4a", "f32_[1024,65536]")
         x4b = gen((256, 1 << 20), torch.int64, lambda c: synth.full_range_i64(7), 1)
         ops += sort_ops(be, tensor, x4b, "C4b", "i64_[256,2^20]")
 
     # ---------------- C5: strided NCHW
-    if which in ("all", "c5"):
+    if on("all", "c5"):
         x5 = gen((32, 512, 56, 56), torch.float32, lambda c: synth.normal(8 + 100 * c), 6)
         n5 = 32 * 512 * 56 * 56
         calls, outs = reduce_calls("reduce_mean", x5, [2, 3])
@@ -327,7 +330,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--configs", default="all", help="all | step | c1 | c2 | c3 | c4 | c5")
+    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",

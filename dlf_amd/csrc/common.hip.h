@@ -7,6 +7,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/dlfx.h"
 
 namespace dlfx {
@@ -82,14 +84,14 @@ struct Words {
 
 // Value of `v` in the lane the DPP control selects; lanes whose source is
 // outside the row (or masked off by ROW_MASK) receive `fill`.
-template <int CTRL, int ROW_MASK = 0xf, typename T>
+template <int CTRL, int ROW_MASK = 0xf, int BANK_MASK = 0xf, typename T>
 __device__ __forceinline__ T dpp_fetch(T v, T fill) {
     static_assert(sizeof(T) % 4 == 0, "whole 32-bit words only");
     constexpr int N = sizeof(T) / 4;
     Words<N> a = bit_cast<Words<N>>(v), f = bit_cast<Words<N>>(fill), r;
 #pragma unroll
     for (int i = 0; i < N; ++i)
-        r.w[i] = __builtin_amdgcn_update_dpp(f.w[i], a.w[i], CTRL, ROW_MASK, 0xf, false);
+        r.w[i] = __builtin_amdgcn_update_dpp(f.w[i], a.w[i], CTRL, ROW_MASK, BANK_MASK, false);
     return bit_cast<T>(r);
 }
 
@@ -128,6 +130,52 @@ constexpr int kRowHalfMirror = 0x141;
 constexpr int kRowMirror = 0x140;
 constexpr int kRowShr1 = 0x111, kRowShr2 = 0x112, kRowShr4 = 0x114, kRowShr8 = 0x118;
 constexpr int kRowBcast15 = 0x142, kRowBcast31 = 0x143;
+
+// Value of `v` in lane (lane ^ J), J a power of two.  Distances below 16 stay inside a DPP
+// row and cost one or two moves; 16 and 32 cross rows and go through the LDS crossbar.
+template <int J, typename T>
+__device__ __forceinline__ T lane_xor_const(T v) {
+    if constexpr (J == 1) return dpp_fetch<kQuadXor1>(v, v);
+    else if constexpr (J == 2) return dpp_fetch<kQuadXor2>(v, v);
+    else if constexpr (J == 4) {
+        // banks are groups of four lanes: even banks take lane + 4, odd banks lane - 4
+        const T up = dpp_fetch<0x104, 0xf, 0x5>(v, v);        // row_shl:4 into banks 0 and 2
+        return dpp_fetch<0x114, 0xf, 0xa>(v, up);             // row_shr:4 into banks 1 and 3
+    } else if constexpr (J == 8) return dpp_fetch<0x128>(v, v);   // row_ror:8
+    else return lane_xor(v, J);
+}
+
+// Bitonic network over aligned groups of WIDTH lanes (a power of two, at most 64); the group
+// that starts at lane 0 ends up best-first.  `exchange(J, keep_better)` must replace the lane's
+// item by the item of lane ^ J when that one is better and keep_better holds, or when it is not
+// better and keep_better does not hold.
+template <int WIDTH, typename Exchange>
+__device__ __forceinline__ void wave_bitonic(Exchange exchange) {
+    const int lane = __lane_id();
+    auto step = [&](auto jc, int k) {
+        constexpr int J = decltype(jc)::value;
+        exchange(jc, ((lane & J) == 0) == ((lane & k) == 0));
+    };
+#pragma unroll
+    for (int k = 2; k <= WIDTH; k <<= 1) {
+        if (k >= 64) step(std::integral_constant<int, 32>(), k);
+        if (k >= 32) step(std::integral_constant<int, 16>(), k);
+        if (k >= 16) step(std::integral_constant<int, 8>(), k);
+        if (k >= 8) step(std::integral_constant<int, 4>(), k);
+        if (k >= 4) step(std::integral_constant<int, 2>(), k);
+        step(std::integral_constant<int, 1>(), k);
+    }
+}
+
+// Sorts one value per lane, largest in lane 0 of each even group of WIDTH lanes.
+template <int WIDTH = kWave, typename T>
+__device__ __forceinline__ T wave_sort_descending(T v) {
+    wave_bitonic<WIDTH>([&](auto jc, bool keep_better) {
+        const T other = lane_xor_const<decltype(jc)::value>(v);
+        v = (keep_better == (other > v)) ? other : v;
+    });
+    return v;
+}
 
 // All-lanes reduction over a wavefront with a commutative `join`.
 template <typename T, typename Join>

@@ -120,7 +120,7 @@ __global__ __launch_bounds__(kBlock) void scan_init(unsigned* ticket, int64_t ro
 // ------------------------------------------------------------------ row kernels
 template <typename T>
 struct RowScanShared {
-    T wave_total[kWaves];
+    T wave_total[16];
     T tile_prefix;
     unsigned next_tile;
 };
@@ -128,7 +128,7 @@ struct RowScanShared {
 // One tile: tile `t` of row `row`.  Element order inside a tile: wave w owns
 // [w*64*ITEMS, (w+1)*64*ITEMS); within it, vector k of lane l covers elements
 // (k*64 + l)*V .. +V.  CHAINED tiles publish / look back through `st`.
-template <typename T, int K, int ITEMS, bool CHAINED, bool SELF_HELP>
+template <typename T, int K, int ITEMS, bool CHAINED, bool SELF_HELP, int BLOCK = kBlock>
 __device__ __forceinline__ void scan_tile(
     const T* __restrict__ x, T* __restrict__ y, const DimMap& xmap, const DimMap& ymap, int64_t sx, int64_t sy,
     int64_t n, int64_t tiles_per_row, int exclusive, int64_t row, int64_t t, int poll_limit,
@@ -136,7 +136,7 @@ __device__ __forceinline__ void scan_tile(
     using Op = ScanOp<T, K>;
     constexpr int V = (vec_width<T>() < ITEMS) ? vec_width<T>() : ITEMS;
     constexpr int KV = ITEMS / V;
-    constexpr int64_t TILE = static_cast<int64_t>(kBlock) * ITEMS;
+    constexpr int64_t TILE = static_cast<int64_t>(BLOCK) * ITEMS;
     using VecT = Vec<T, V>;
 
     const int lane = lane_id();
@@ -190,7 +190,7 @@ __device__ __forceinline__ void scan_tile(
     T wave_prefix = Op::identity();
     T aggregate = Op::identity();
 #pragma unroll
-    for (int i = 0; i < kWaves; ++i) {
+    for (int i = 0; i < BLOCK / kWave; ++i) {
         const T wt = sm.wave_total[i];
         if (i < w) wave_prefix = Op::apply(wave_prefix, wt);
         aggregate = Op::apply(aggregate, wt);
@@ -311,8 +311,8 @@ __global__ __launch_bounds__(kBlock) void scan_rows_single(
 // TICKET the tile of the row is drawn from that row's atomic counter (in-place
 // scans); without, it is the workgroup's position in the row and waits are
 // bounded by self-help.
-template <typename T, int K, int ITEMS, bool TICKET>
-__global__ __launch_bounds__(kBlock) void scan_rows_chained(
+template <typename T, int K, int ITEMS, bool TICKET, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void scan_rows_chained(
     const T* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
     int64_t n, int64_t tiles_per_row, int exclusive, int poll_limit, unsigned* ticket, TileState<T> st) {
     __shared__ RowScanShared<T> sm;
@@ -323,7 +323,7 @@ __global__ __launch_bounds__(kBlock) void scan_rows_chained(
         __syncthreads();
         t = sm.next_tile;
     }
-    scan_tile<T, K, ITEMS, true, !TICKET>(x, y, xmap, ymap, sx, sy, n, tiles_per_row, exclusive, row, t, poll_limit, st, sm);
+    scan_tile<T, K, ITEMS, true, !TICKET, BLOCK>(x, y, xmap, ymap, sx, sy, n, tiles_per_row, exclusive, row, t, poll_limit, st, sm);
 }
 
 // ------------------------------------------------------------------ column kernel
@@ -417,9 +417,19 @@ bool make_dim_map2(const int64_t* dims, const int64_t* sx, const int64_t* sy, in
     return true;
 }
 
+#ifndef DLFX_SCAN_CHAIN_BLOCK
+#define DLFX_SCAN_CHAIN_BLOCK 256
+#endif
+#ifndef DLFX_SCAN_CHAIN_BYTES
+#define DLFX_SCAN_CHAIN_BYTES 65536
+#endif
+constexpr int kChainBlock = DLFX_SCAN_CHAIN_BLOCK;
+constexpr int64_t kChainTileBytes = DLFX_SCAN_CHAIN_BYTES;
+
 // Elements per tile: 256 bytes per thread for chained rows, less for short rows.
 int64_t tile_elems(size_t elem_size, int64_t n) {
     const int64_t full = 256 * (256 / static_cast<int64_t>(elem_size));
+    if (n > full) return kChainTileBytes / static_cast<int64_t>(elem_size);
     if (n > full / 4) return full;
     if (n > 1024) return full / 4;
     if (n > 256) return 1024;
@@ -509,11 +519,13 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     scan_init<T><<<dim3(static_cast<unsigned>(ceil_div(l.tiles, kBlock))), block, 0, stream>>>(ticket, m, st, l.tiles);
     DLFX_CHECK_LAUNCH();
     const dim3 grid(static_cast<unsigned>(l.tiles));
+    constexpr int CI = static_cast<int>(kChainTileBytes / sizeof(T) / kChainBlock);
+    const dim3 cblock(kChainBlock);
     if (views_overlap(rank, dims, x, x_strides, y, y_strides))
-        scan_rows_chained<T, K, FULL, true><<<grid, block, 0, stream>>>(
+        scan_rows_chained<T, K, CI, true, kChainBlock><<<grid, cblock, 0, stream>>>(
             x, y, xmap, ymap, sx, sy, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st);
     else
-        scan_rows_chained<T, K, FULL, false><<<grid, block, 0, stream>>>(
+        scan_rows_chained<T, K, CI, false, kChainBlock><<<grid, cblock, 0, stream>>>(
             x, y, xmap, ymap, sx, sy, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st);
     DLFX_CHECK_LAUNCH();
     return DLFX_OK;

@@ -248,20 +248,105 @@ __device__ __forceinline__ void compute_ranks(TopkShared<K>& sm, const K* e_ord,
     team_sync<BLOCK>();
 }
 
-// Writes the entries ranked below `limit` to their place in the outputs.
+// Sorts one (image, index) entry per lane across the wavefront, best entry in lane 0.
+template <typename K>
+__device__ __forceinline__ void wave_sort_entries(K& o, uint32_t& x) {
+    wave_bitonic<kWave>([&](auto jc, bool keep_better) {
+        constexpr int J = decltype(jc)::value;
+        const K oo = lane_xor_const<J>(o);
+        const uint32_t xo = lane_xor_const<J>(x);
+        if (keep_better == (beats<K>(oo, xo, o, x) != 0u)) {
+            o = oo;
+            x = xo;
+        }
+    });
+}
+
+constexpr int kMergeMax = 512;       // entries up to which sorted runs are merged by rank
+
+// Orders `count` distinct (image, index) entries held in LDS, best first, and writes those
+// ranked below `limit` to the outputs.  The arrays must have room for count rounded up to a
+// multiple of 64 and are overwritten.  Each wave sorts runs of 64 entries in registers; the
+// rank of an entry is its position in its run plus, for every other run, the number of that
+// run's entries that beat it, found by bisection.  All threads of the team must call.
 template <int BLOCK, typename K>
-__device__ __forceinline__ void rank_emit(TopkShared<K>& sm, const K* e_ord, const uint32_t* e_idx, int count, int limit,
-                                          const TopkIo<K>& io, int64_t row, const K* xr) {
-    compute_ranks<BLOCK, K>(sm, e_ord, e_idx, count);
+__device__ __forceinline__ void merge_rank_emit(K* e_ord, uint32_t* e_idx, int count, int limit,
+                                                const TopkIo<K>& io, int64_t row, const K* xr) {
+    constexpr int WAVES = BLOCK / kWave;
+    const int tid = threadIdx.x;
+    const int lane = lane_id();
+    const int w = tid / kWave;
+    const int runs = (count + kWave - 1) / kWave;
     K* yr = io.y + io.ymap.at(row);
     const int64_t ir = io.imap.at(row);
-    for (int e = threadIdx.x; e < count; e += BLOCK) {
-        const int r = static_cast<int>(sm.rank[e]);
-        if (r < limit) emit_one<K>(io, yr, ir, xr, r, e_ord[e], e_idx[e]);
+    for (int r = w; r < runs; r += WAVES) {
+        const int e = r * kWave + lane;
+        K o = e < count ? e_ord[e] : K(0);
+        uint32_t x = e < count ? e_idx[e] : 0xffffffffu;      // padding: beaten by every entry
+        wave_sort_entries<K>(o, x);
+        if (runs == 1) {
+            if (lane < limit && lane < count) emit_one<K>(io, yr, ir, xr, lane, o, x);
+        } else {
+            e_ord[e] = o;
+            e_idx[e] = x;
+        }
+    }
+    if (runs == 1) return;
+    team_sync<BLOCK>();
+    for (int e = tid; e < count; e += BLOCK) {
+        const K o = e_ord[e];
+        const uint32_t x = e_idx[e];
+        const int mine = e / kWave;
+        uint32_t rank = static_cast<uint32_t>(e % kWave);
+        // U bisections at a time keep U independent LDS reads in flight; indices are only
+        // read in the steps where some image ties with this entry's
+        auto bisect = [&](auto uc, int first_other) {
+            constexpr int U = decltype(uc)::value;
+            int base[U];
+            uint32_t c[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int other = first_other + u;
+                base[u] = (other < mine ? other : other + 1) * kWave;
+                c[u] = 0u;
+            }
+            auto probe = [&](int step) {      // step 0: the last probe, which decides 63 against 64
+                K oj[U];
+                uint32_t xj[U];
+                bool tie = false;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    oj[u] = e_ord[base[u] + static_cast<int>(c[u]) + (step ? step - 1 : 0)];
+                    xj[u] = 0xffffffffu;
+                    tie = tie || oj[u] == o;
+                }
+                if (tie) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) xj[u] = e_idx[base[u] + static_cast<int>(c[u]) + (step ? step - 1 : 0)];
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    c[u] += (oj[u] > o || (oj[u] == o && xj[u] < x)) ? static_cast<uint32_t>(step ? step : 1) : 0u;
+            };
+#pragma unroll
+            for (int step = 32; step >= 1; step >>= 1) probe(step);
+            probe(0);
+#pragma unroll
+            for (int u = 0; u < U; ++u) rank += c[u];
+        };
+        const int others = runs - 1;
+        int r0 = 0;
+        for (; r0 + 4 <= others; r0 += 4) bisect(std::integral_constant<int, 4>(), r0);
+        switch (others - r0) {
+        case 3: bisect(std::integral_constant<int, 3>(), r0); break;
+        case 2: bisect(std::integral_constant<int, 2>(), r0); break;
+        case 1: bisect(std::integral_constant<int, 1>(), r0); break;
+        default: break;
+        }
+        if (rank < static_cast<uint32_t>(limit)) emit_one<K>(io, yr, ir, xr, static_cast<int>(rank), o, x);
     }
 }
 
-constexpr int kRankSortMax = 64;     // winners up to which counting ranks beats a bitonic network
 
 // Exact selection of the `limit` best of the items (ord(i), idx(i)), best = larger image,
 // then lower index; writes them in that order.  Padding items carry image 0 and an index
@@ -406,8 +491,8 @@ __device__ __forceinline__ void select_and_emit(TopkShared<K>& sm, const TopkIo<
     team_sync<BLOCK>();
 
     // ---- order the winners: best first
-    if (limit <= kRankSortMax) {
-        rank_emit<BLOCK, K>(sm, sm.out_ord, sm.out_idx, limit, limit, io, row, xr);
+    if (limit <= kMergeMax) {
+        merge_rank_emit<BLOCK, K>(sm.out_ord, sm.out_idx, limit, limit, io, row, xr);
         return;
     }
     int kp = 1;
@@ -513,40 +598,38 @@ void topk_select(TopkIo<typename BitsOf<T>::type> io, int64_t n, int limit,
                 }
             }
         }
-        // ---- pre-filter.  Split the threads into `groups` >= limit groups; the largest
-        // element each group holds gives `groups` distinct elements, so the smallest of those
-        // maxima cannot exceed the limit-th largest element of the row: everything below it is
-        // out.  What is left is usually a few times `limit` elements.
+        // ---- pre-filter.  The largest element of each thread is a distinct element of the
+        // row.  Every wave sorts its 64 of them; the value at position p*s - 1 of a wave has
+        // p*s elements of the row at or above it.  Four such samples per wave (p = 1..4) are
+        // sorted together: the m-th largest sample has at least m*s elements at or above it
+        // (q samples of one wave among the first m stand for q*s elements of that wave), so
+        // with m*s >= limit it cannot exceed the limit-th largest element of the row and
+        // everything below it is out.  What is left is usually 1 to 1.5 times `limit` elements.
+        static_assert(WAVES == 16, "four samples from each of sixteen waves fill one wave");
         T tmax = worst;
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) tmax = sc[i] > tmax ? sc[i] : tmax;
-        int groups = 1;
-        while (groups < limit && groups < BLOCK) groups <<= 1;
-        const int span = BLOCK / groups;               // threads per group, a power of two
-        auto tmaxf = [](T a, T b) { return a > b ? a : b; };
-        auto tminf = [](T a, T b) { return a < b ? a : b; };
         T* red = reinterpret_cast<T*>(sm.out_ord);
-        T bound;
-        if (span >= kWave) {
-            const T wmax = wave_reduce(tmax, tmaxf);
+        int samples, mth;
+        if (limit <= WAVES) {
+            const T wmax = wave_reduce(tmax, [](T a, T b) { return a > b ? a : b; });
             if (lane == 0) red[w] = wmax;
-            __syncthreads();
-            const int wpg = span / kWave;              // waves per group
-            bound = red[0];
-            for (int j = 1; j < wpg; ++j) bound = tmaxf(bound, red[j]);
-            for (int g0 = wpg; g0 < WAVES; g0 += wpg) {
-                T gm = red[g0];
-                for (int j = 1; j < wpg; ++j) gm = tmaxf(gm, red[g0 + j]);
-                bound = tminf(bound, gm);
-            }
+            samples = WAVES;
+            mth = limit;
         } else {
-            const T gmax = group_reduce(tmax, span, tmaxf);
-            const T wmin = wave_reduce(gmax, tminf);
-            if (lane == 0) red[w] = wmin;
-            __syncthreads();
-            bound = red[0];
-            for (int j = 1; j < WAVES; ++j) bound = tminf(bound, red[j]);
+            const int stride = limit <= 512 ? (limit + 31) / 32 : (limit + 63) / 64;     // <= 16
+            tmax = wave_sort_descending(tmax);
+            const int p = (lane + 1) / stride;
+            if (p * stride == lane + 1 && p <= 4) red[w * 4 + p - 1] = tmax;
+            samples = 4 * WAVES;
+            mth = (limit + stride - 1) / stride;                                       // <= 64
         }
+        __syncthreads();
+        T bound = lane < samples ? red[lane] : worst;
+        if (limit <= WAVES) bound = wave_sort_descending<16>(bound);
+        else bound = wave_sort_descending(bound);
+        bound = lane_get(bound, mth - 1);
+        if (limit > BLOCK) bound = worst;
         // ---- survivors go to LDS as (image, index), in element order: each wave counts its
         // survivors with ballots, the waves' counts are prefix-summed through LDS, and a second
         // sweep places every survivor at wave offset + number of survivors before it in the wave
@@ -579,24 +662,15 @@ void topk_select(TopkIo<typename BitsOf<T>::type> io, int64_t n, int limit,
         }
         __syncthreads();
         // What happens next depends on how many survived:
-        //   * at most one per lane of a wave: the first wave ranks them and writes the answer;
+        //   * up to kMergeMax: ordered here by sorted runs and ranks, answer written;
         //   * up to kCandCap: they are handed, through global memory, to topk_finish, whose
-        //     small workgroups hide the latency of the exact selection much better than this
-        //     one (which holds a whole row) could;
+        //     small workgroups hide the latency of an exact radix selection much better than
+        //     this one (which holds a whole row) could;
         //   * more (long runs of equal values, adversarial order), or a limit the bound does
         //     not hold for: topk_finish selects from the row itself.
-        if (total <= kWave && limit <= BLOCK) {
+        if (total <= static_cast<uint32_t>(kMergeMax) && limit <= BLOCK) {
             if (tid == 0) row_state[row] = kRowDone;
-            if (tid >= kWave) return;
-            const int cnt = static_cast<int>(total);
-            if (tid < cnt) {
-                const K o = sm.cand_ord[tid];
-                const uint32_t x = sm.cand_idx[tid];
-                uint32_t r = 0;
-                for (int j = 0; j < cnt; ++j) r += beats<K>(sm.cand_ord[j], sm.cand_idx[j], o, x);
-                if (static_cast<int>(r) < limit)
-                    emit_one<K>(io, io.y + io.ymap.at(row), io.imap.at(row), xr, static_cast<int>(r), o, x);
-            }
+            merge_rank_emit<BLOCK, K>(sm.cand_ord, sm.cand_idx, static_cast<int>(total), limit, io, row, xr);
         } else if (total <= CAP && limit <= BLOCK) {
             if (tid == 0) row_state[row] = total;
             K* so = spill_ord + row * CAP;
@@ -637,6 +711,10 @@ __global__ __launch_bounds__(kSelectThreads) void topk_finish(
             sm.cand_idx[i] = si[i];
         }
         __syncthreads();
+        if (total <= static_cast<uint32_t>(kMergeMax)) {
+            merge_rank_emit<SEL, K>(sm.cand_ord, sm.cand_idx, static_cast<int>(total), limit, io, row, xr);
+            return;
+        }
         const int per_thread = static_cast<int>((total + SEL - 1) / SEL);
         select_and_emit<SEL, CAP / SEL, true>(
             sm, io, row, xr, limit, per_thread,
