@@ -28,12 +28,26 @@
 namespace dlfx {
 namespace {
 
+#ifndef DLFX_SORT_WAVES
+#define DLFX_SORT_WAVES 4
+#endif
 constexpr int kBlock = 256;
 constexpr int kWaves = kBlock / kWave;
 constexpr int kRadix = 256;
 constexpr int64_t kMaxRow = (int64_t(1) << 27) - 1;   // counts share a status word with 5 tag bits
 
 int g_sort_poll_limit = 2048;
+
+#ifdef DLFX_SORT_TIMING
+// Debug builds only: shader-clock cycles spent by thread 0 of every workgroup in each phase.
+constexpr int kPhaseSlots = 16384;
+__device__ unsigned long long g_phase_cycles[kPhaseSlots * 8];
+#define DLFX_PHASE(i) do { if (threadIdx.x == 0) { const long long now_ = clock64(); g_phase_cycles[(blockIdx.x % kPhaseSlots) * 8 + (i)] += static_cast<unsigned long long>(now_ - phase_t_); phase_t_ = now_; } } while (0)
+#define DLFX_PHASE_BEGIN() long long phase_t_ = clock64()
+#else
+#define DLFX_PHASE(i) do { } while (0)
+#define DLFX_PHASE_BEGIN() do { } while (0)
+#endif
 
 enum KeyKind { kKeyInt = 0, kKeyFloat = 1 };
 
@@ -63,18 +77,14 @@ __device__ __forceinline__ K decode_key(K k, int kind, int descending) {
     return (kind == kKeyFloat) ? ((k & S) ? (k & ~S) : ~k) : (k ^ S);
 }
 
-// Where a pass reads its keys and writes them.
+// What the passes of one sort read and write.
 template <typename K>
 struct PassIo {
-    // input
-    const K* src_keys;        // contiguous [m][n] (null on the first pass)
-    const uint32_t* src_vals; // contiguous [m][n] (null on the first pass / keys only)
-    const K* x;               // strided input, read on the first pass
+    const K* x;               // strided input, read by the first pass that runs
     DimMap xmap;
     int64_t sx;
-    // output
-    K* dst_keys;              // contiguous [m][n] (null on the last pass)
-    uint32_t* dst_vals;
+    K* kbuf[2];               // contiguous [m][n] ping-pong buffers between passes
+    uint32_t* vbuf[2];        // ... and their index payloads (argsort)
     K* y;                     // strided value output of the last pass (may be null)
     DimMap ymap;
     int64_t sy;
@@ -82,29 +92,31 @@ struct PassIo {
     DimMap imap;
     int64_t si;
     int idx64;
-    int first, last;
     int kind, descending;
     int canon_zero;           // argsort of floats: -0.0 and +0.0 are one key
     int restore_zero;         // ... and the value written for a zero key is re-read from x
 };
 
 template <typename K>
-__device__ __forceinline__ K load_key(const PassIo<K>& io, int64_t row, int64_t row_n, const K* xrow, int64_t i) {
-    if (io.first) {
-        K bits = xrow[i * io.sx];
-        if (io.canon_zero && (bits << 1) == 0) bits = 0;      // -0.0 -> +0.0
-        return encode_key<K>(bits, io.kind, io.descending);
-    }
-    return io.src_keys[row * row_n + i];
+__device__ __forceinline__ K key_of_element(const PassIo<K>& io, K bits) {
+    if (io.canon_zero && (bits << 1) == 0) bits = 0;      // -0.0 -> +0.0
+    return encode_key<K>(bits, io.kind, io.descending);
 }
 
 // ------------------------------------------------------------------ histograms
+// One read of the input builds the digit histograms of every pass for a chunk of a row.
+// Each workgroup keeps kHistCopies interleaved copies of every histogram (a lane adds to copy
+// lane % kHistCopies), so that the few distinct values of a low-entropy digit do not
+// serialise all 64 lanes on one LDS word; a digit that is the same in a whole batch of
+// keys (constant bytes: small integers, narrow float ranges) is added once per wave.
 template <typename K>
 __global__ __launch_bounds__(kBlock) void sort_histogram(PassIo<K> io, int64_t n, int64_t chunk, int64_t chunks_per_row,
                                                          uint32_t* __restrict__ ghist) {
     constexpr int P = KeyTraits<K>::kPasses;
-    __shared__ uint32_t hist[P][kRadix];
-    for (int i = threadIdx.x; i < P * kRadix; i += kBlock) (&hist[0][0])[i] = 0;
+    constexpr int U = 32 / sizeof(K);                 // keys in flight per thread
+    constexpr int R = 32 / P;                         // copies: 8 (32-bit keys) or 4 (64-bit keys): 32 KB
+    __shared__ uint32_t hist[P * kRadix * R];
+    for (int i = threadIdx.x; i < P * kRadix * R; i += kBlock) hist[i] = 0;
     __syncthreads();
     const int64_t row = blockIdx.x / chunks_per_row;
     const int64_t c = blockIdx.x - row * chunks_per_row;
@@ -112,45 +124,72 @@ __global__ __launch_bounds__(kBlock) void sort_histogram(PassIo<K> io, int64_t n
     const int64_t lo = c * chunk;
     const int64_t hi = (lo + chunk < n) ? lo + chunk : n;
     const int lane = lane_id();
-    for (int64_t i0 = lo + (threadIdx.x - lane); i0 < hi; i0 += kBlock) {
-        const int64_t i = i0 + lane;
-        const bool live = i < hi;
-        K key = 0;
-        if (live) key = load_key<K>(io, row, n, xrow, i);
-        const unsigned long long live_mask = __ballot(live);
+    const int copy = lane % R;
+    // wave-uniform trip count: every wave walks whole batches of U * 256 keys
+    for (int64_t b0 = lo; b0 < hi; b0 += static_cast<int64_t>(kBlock) * U) {
+        const int64_t i0 = b0 + threadIdx.x;
+        K key[U];
+        const bool whole = b0 + static_cast<int64_t>(kBlock) * U <= hi;
+        if (whole) {
 #pragma unroll
-        for (int p = 0; p < P; ++p) {
-            const uint32_t d = static_cast<uint32_t>(key >> (8 * p)) & 0xffu;
-            // a wave whose live keys share the digit adds once instead of 64 times to one word
-            const uint32_t d0 = __builtin_amdgcn_readfirstlane(d);
-            const bool uniform = __ballot(live && d != d0) == 0ull && (live_mask & 1ull);
-            if (uniform) {
-                if (lane == 0) atomicAdd(&hist[p][d0], static_cast<uint32_t>(__popcll(live_mask)));
-            } else if (live) {
-                atomicAdd(&hist[p][d], 1u);
+            for (int u = 0; u < U; ++u) key[u] = xrow[(i0 + static_cast<int64_t>(u) * kBlock) * io.sx];
+#pragma unroll
+            for (int u = 0; u < U; ++u) key[u] = key_of_element<K>(io, key[u]);
+            const K key0 = lane_read(key[0], 0);
+            K diff = 0;
+#pragma unroll
+            for (int u = 0; u < U; ++u) diff |= key[u] ^ key0;
+#pragma unroll
+            for (int p = 0; p < P; ++p) {
+                uint32_t* h = hist + p * kRadix * R;
+                if (__ballot(((diff >> (8 * p)) & 0xffu) != 0) == 0ull) {
+                    if (lane == 0) atomicAdd(&h[(static_cast<uint32_t>(key0 >> (8 * p)) & 0xffu) * R], static_cast<uint32_t>(U * kWave));
+                } else {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) atomicAdd(&h[(static_cast<uint32_t>(key[u] >> (8 * p)) & 0xffu) * R + copy], 1u);
+                }
+            }
+        } else {
+            for (int u = 0; u < U; ++u) {
+                const int64_t i = i0 + static_cast<int64_t>(u) * kBlock;
+                if (i < hi) {
+                    const K k1 = key_of_element<K>(io, xrow[i * io.sx]);
+#pragma unroll
+                    for (int p = 0; p < P; ++p)
+                        atomicAdd(&hist[p * kRadix * R + (static_cast<uint32_t>(k1 >> (8 * p)) & 0xffu) * R + copy], 1u);
+                }
             }
         }
     }
     __syncthreads();
     uint32_t* g = ghist + row * (P * kRadix);
     for (int i = threadIdx.x; i < P * kRadix; i += kBlock) {
-        const uint32_t v = (&hist[0][0])[i];
+        uint32_t v = 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) v += hist[i * R + r];
         if (v) atomicAdd(&g[i], v);
     }
 }
 
-// In place: histogram -> exclusive prefix (start of each digit's run in the row).
-__global__ __launch_bounds__(kRadix) void sort_bases(uint32_t* __restrict__ ghist) {
+// In place: histogram -> exclusive prefix (start of each digit's run in the row).  Workgroup
+// b handles one (row, pass) pair.  moves[b] tells whether that pass changes the order of that
+// row: when all n keys of the row share the digit it does not, and the row skips the pass.
+__global__ __launch_bounds__(kRadix) void sort_bases(uint32_t* __restrict__ ghist, uint32_t* __restrict__ moves, uint32_t n) {
     __shared__ uint32_t wave_tot[kRadix / kWave];
+    __shared__ uint32_t one_digit;
+    if (threadIdx.x == 0) one_digit = 0u;
     uint32_t* g = ghist + static_cast<int64_t>(blockIdx.x) * kRadix;
     const uint32_t v = g[threadIdx.x];
     const uint32_t incl = wave_scan_inclusive(v, 0u, [](uint32_t a, uint32_t b) { return a + b; });
     const int w = threadIdx.x / kWave;
+    __syncthreads();
     if (lane_id() == kWave - 1) wave_tot[w] = incl;
+    if (v == n) one_digit = 1u;
     __syncthreads();
     uint32_t pre = 0;
     for (int i = 0; i < w; ++i) pre += wave_tot[i];
     g[threadIdx.x] = pre + incl - v;
+    if (threadIdx.x == 0) moves[blockIdx.x] = one_digit ? 0u : 1u;
 }
 
 __global__ __launch_bounds__(kBlock) void sort_clear(uint32_t* __restrict__ p, int64_t words) {
@@ -170,116 +209,239 @@ template <typename K, bool PAIRS, int ITEMS>
 struct PassShared {
     uint32_t wave_hist[kWaves][kRadix];       // per-wave digit counts, then per-wave offsets
     uint32_t help_hist[kRadix];               // digits of an earlier tile counted here when it is late
-    uint32_t digit_start[kRadix];             // first tile-local position of each digit
-    int64_t dst_base[kRadix];                 // global position of that digit's run start minus digit_start
+    int32_t dst_base[kRadix];                 // row position of that digit's run start minus digit_start
     uint32_t scan_tmp[kWaves];
     int help_tile;
     K keys[kBlock * ITEMS];
     uint32_t vals[PAIRS ? kBlock * ITEMS : 1];
 };
 
-template <typename K, bool PAIRS, int ITEMS>
-__global__ __launch_bounds__(kBlock) void sort_pass(PassIo<K> io, int pass, int64_t n, int64_t tiles_per_row,
+// Pass `pass` of the sort (digit = bits [8 pass, 8 pass + 8) of the key).  LAST: the pass of
+// the most significant digit, which every row runs and which writes the strided outputs.
+// Rows are independent: a row leaves out the passes that would not move its keys, the first
+// pass it runs reads the strided input, and its place in the ping-pong buffers alternates
+// over the passes it does run.
+template <typename K, bool PAIRS, int ITEMS, bool LAST>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SORT_WAVES))) void sort_pass(PassIo<K> io, int pass, int64_t rows, int64_t n, int64_t tiles_per_row,
                                                     const uint32_t* __restrict__ gbase,
+                                                    const uint32_t* __restrict__ moves,
                                                     uint32_t* __restrict__ status, int poll_limit) {
     constexpr int P = KeyTraits<K>::kPasses;
     constexpr int TILE = kBlock * ITEMS;
     constexpr int W = 4;    // status words of earlier tiles fetched per look-back step
     __shared__ PassShared<K, PAIRS, ITEMS> sm;
 
+    // workgroups are handed out in index order and dealt round-robin over the chip's eight
+    // parts: tile t of every row comes before tile t + 1 of any row, so a tile's predecessors
+    // in its row have usually finished when it looks back, and the tiles of a row share a
+    // second-level cache when the number of rows is a multiple of eight
+    const int64_t t = blockIdx.x / rows;
+    const int64_t row = blockIdx.x - t * rows;
+    const uint32_t* row_moves = moves + row * P;
+    int ran = 0;            // passes before this one that this row ran
+    for (int p = 0; p < pass; ++p) ran += row_moves[p] ? 1 : 0;
+    if (!LAST && row_moves[pass] == 0u) return;
+    const bool first = ran == 0;
+    const K* __restrict__ src_keys = first ? nullptr : io.kbuf[(ran - 1) & 1];
+    const uint32_t* __restrict__ src_vals = first ? nullptr : io.vbuf[(ran - 1) & 1];
+    K* __restrict__ dst_keys = io.kbuf[ran & 1];
+    uint32_t* __restrict__ dst_vals = io.vbuf[ran & 1];
+
     const int tid = threadIdx.x;
     const int lane = lane_id();
     const int w = tid / kWave;
-    const int64_t row = blockIdx.x / tiles_per_row;
-    const int64_t t = blockIdx.x - row * tiles_per_row;
     const int64_t tile_base = t * TILE;
     const int valid = static_cast<int>((n - tile_base < TILE) ? n - tile_base : TILE);
-    const K* xrow = io.first ? io.x + io.xmap.at(row) : nullptr;
+    const bool full = valid == TILE;
+    const K* xrow = io.x + io.xmap.at(row);
+    const int64_t row_off = row * n;
     const int shift = 8 * pass;
 
+    DLFX_PHASE_BEGIN();
     for (int i = tid; i < kWaves * kRadix; i += kBlock) (&sm.wave_hist[0][0])[i] = 0;
     if (tid == 0) sm.help_tile = -1;
 
-    // ---- load: wave w owns [w*64*ITEMS, ...), item k of lane l is element k*64 + l of it
+    // ---- load: wave w owns [w*64*ITEMS, ...), item k of lane l is element k*64 + l of it.
+    // All loads are issued before the first key is used.
     K key[ITEMS];
     uint32_t val[PAIRS ? ITEMS : 1];
-    const int seg = w * kWave * ITEMS;
+    const int seg = w * kWave * ITEMS + lane;
+    if (first) {
+        const K* src = xrow + (tile_base + seg) * io.sx;
+        const int64_t step = io.sx * kWave;
+        if (full) {
 #pragma unroll
-    for (int k = 0; k < ITEMS; ++k) {
-        const int li = seg + k * kWave + lane;
-        const int64_t i = tile_base + li;
-        if (li < valid) {
-            key[k] = load_key<K>(io, row, n, xrow, i);
-            if constexpr (PAIRS) val[k] = io.first ? static_cast<uint32_t>(i) : io.src_vals[row * n + i];
+            for (int k = 0; k < ITEMS; ++k) key[k] = src[k * step];
         } else {
-            key[k] = ~K(0);      // padding sorts last and is never stored
-            if constexpr (PAIRS) val[k] = 0;
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) {
+                key[k] = 0;
+                if (seg + k * kWave < valid) key[k] = src[k * step];
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            key[k] = key_of_element<K>(io, key[k]);
+            if constexpr (PAIRS) val[k] = static_cast<uint32_t>(tile_base) + static_cast<uint32_t>(seg + k * kWave);
+        }
+    } else {
+        const K* src = src_keys + row_off + tile_base + seg;
+        if (full) {
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) key[k] = src[k * kWave];
+        } else {
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) {
+                key[k] = 0;
+                if (seg + k * kWave < valid) key[k] = src[k * kWave];
+            }
+        }
+        if constexpr (PAIRS) {
+            const uint32_t* vsrc = src_vals + row_off + tile_base + seg;
+            if (full) {
+#pragma unroll
+                for (int k = 0; k < ITEMS; ++k) val[k] = vsrc[k * kWave];
+            } else {
+#pragma unroll
+                for (int k = 0; k < ITEMS; ++k) {
+                    val[k] = 0;
+                    if (seg + k * kWave < valid) val[k] = vsrc[k * kWave];
+                }
+            }
         }
     }
-    __syncthreads();
-
-    // ---- rank inside the wave, in element order (stable)
-    uint32_t rank[ITEMS];
-    const unsigned long long lt_mask = (1ull << lane) - 1ull;
+    if (!full) {
 #pragma unroll
-    for (int k = 0; k < ITEMS; ++k) {
-        const uint32_t d = static_cast<uint32_t>(key[k] >> shift) & 0xffu;
-        unsigned long long peers = ~0ull;
+        for (int k = 0; k < ITEMS; ++k)
+            if (seg + k * kWave >= valid) key[k] = ~K(0);      // padding sorts last and is never stored
+    }
+    __syncthreads();
+    DLFX_PHASE(0);
+
+    // ---- rank inside the wave, in element order (stable).  The lanes whose digit equals this
+    // lane's are found with one ballot per digit bit; two items at a time, so that the two
+    // independent chains fill each other's wait states.  The items then take their ranks from
+    // the wave's running digit counts one after the other: the first lane of each group of
+    // equal digits moves the count on.
+    uint32_t rank[ITEMS];
+    static_assert(ITEMS % 2 == 0, "items are ranked in pairs");
+#pragma unroll
+    for (int k0 = 0; k0 < ITEMS; k0 += 2) {
+        uint32_t d[2], before[2], cnt[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) d[j] = static_cast<uint32_t>(key[k0 + j] >> shift) & 0xffu;
+        uint32_t peers_lo[2] = {0xffffffffu, 0xffffffffu}, peers_hi[2] = {0xffffffffu, 0xffffffffu};
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
-            const bool bit = (d >> b) & 1u;
-            const unsigned long long vote = __ballot(bit);
-            peers &= bit ? vote : ~vote;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int32_t ones = static_cast<int32_t>(d[j] << (31 - b)) >> 31;       // all ones when the bit is set
+                const unsigned long long vote = __ballot(ones < 0);
+                peers_lo[j] &= ~(static_cast<uint32_t>(vote) ^ static_cast<uint32_t>(ones));
+                peers_hi[j] &= ~(static_cast<uint32_t>(vote >> 32) ^ static_cast<uint32_t>(ones));
+            }
         }
-        const uint32_t before = static_cast<uint32_t>(__popcll(peers & lt_mask));
-        const uint32_t cnt = static_cast<uint32_t>(__popcll(peers));
-        const uint32_t seen = sm.wave_hist[w][d];          // same word for all peers: a broadcast read
-        rank[k] = seen + before;
-        __builtin_amdgcn_wave_barrier();
-        if (before == 0) sm.wave_hist[w][d] = seen + cnt;
-        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            before[j] = __builtin_amdgcn_mbcnt_hi(peers_hi[j], __builtin_amdgcn_mbcnt_lo(peers_lo[j], 0u));
+            cnt[j] = static_cast<uint32_t>(__popc(peers_lo[j]) + __popc(peers_hi[j]));
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t seen = sm.wave_hist[w][d[j]];          // same word for all peers: a broadcast read
+            rank[k0 + j] = seen + before[j];
+            __builtin_amdgcn_wave_barrier();
+            if (before[j] == 0) sm.wave_hist[w][d[j]] = seen + cnt[j];
+            __builtin_amdgcn_wave_barrier();
+        }
     }
+#ifdef DLFX_SORT_DOUBLE_RANK
+    // timing experiment only: the ballot work of the ranking a second time, on other bits
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const uint32_t d = static_cast<uint32_t>(key[k] >> (shift ^ 8)) & 0xffu;
+        uint32_t peers_lo = 0xffffffffu, peers_hi = 0xffffffffu;
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const uint32_t ones = 0u - ((d >> b) & 1u);
+            const unsigned long long vote = __ballot(ones != 0u);
+            peers_lo &= ~(static_cast<uint32_t>(vote) ^ ones);
+            peers_hi &= ~(static_cast<uint32_t>(vote >> 32) ^ ones);
+        }
+        const uint32_t before = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
+        if (before == 0xffffu) rank[k] += 1;
+    }
+#endif
     __syncthreads();
+    DLFX_PHASE(1);
 
-    // ---- thread d owns digit d: wave offsets, tile count, position of the digit in the tile
+    // ---- thread d owns digit d: tile count, position of the digit in the tile, wave offsets
+    uint32_t wave_count[kWaves];
     uint32_t count = 0;
 #pragma unroll
     for (int i = 0; i < kWaves; ++i) {
-        const uint32_t c = sm.wave_hist[i][tid];
-        sm.wave_hist[i][tid] = count;
-        count += c;
+        wave_count[i] = sm.wave_hist[i][tid];
+        count += wave_count[i];
     }
+    const uint32_t padded = count;
     if (tid == kRadix - 1) count -= static_cast<uint32_t>(TILE - valid);     // padding is not part of the row
     const int64_t srow = (row * tiles_per_row) * kRadix;
     uint32_t* my_status = status + srow + t * kRadix + tid;
     if (t + 1 < tiles_per_row)
         __hip_atomic_store(my_status, make_status(pass, t == 0, count), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // the status words of the W tiles before this one are requested now and looked at after
+    // the tile has been gathered, so that their latency is not waited for
+    uint32_t sw[W];
+    int64_t p = t - 1;
+    auto fetch = [&]() {
+#pragma unroll
+        for (int i = 0; i < W; ++i) {
+            const int64_t q = p - i;
+            sw[i] = (q >= 0) ? __hip_atomic_load(status + srow + q * kRadix + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                             : make_status(pass, true, 0u);
+        }
+    };
+    bool done = (t == 0);
+    if (!done) fetch();
+    uint32_t start;
     {
-        uint32_t padded = count + (tid == kRadix - 1 ? static_cast<uint32_t>(TILE - valid) : 0u);
         const uint32_t incl = wave_scan_inclusive(padded, 0u, [](uint32_t a, uint32_t b) { return a + b; });
         if (lane == kWave - 1) sm.scan_tmp[w] = incl;
         __syncthreads();
         uint32_t pre = 0;
         for (int i = 0; i < w; ++i) pre += sm.scan_tmp[i];
-        sm.digit_start[tid] = pre + incl - padded;
+        start = pre + incl - padded;
+        uint32_t run = start;
+#pragma unroll
+        for (int i = 0; i < kWaves; ++i) {
+            sm.wave_hist[i][tid] = run;        // tile position of the first key of wave i with this digit
+            run += wave_count[i];
+        }
     }
+    __syncthreads();
+    DLFX_PHASE(2);
+
+    // ---- gather the tile in its locally sorted order
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const uint32_t d = static_cast<uint32_t>(key[k] >> shift) & 0xffu;
+        const uint32_t pos = sm.wave_hist[w][d] + rank[k];
+        sm.keys[pos] = key[k];
+        if constexpr (PAIRS) sm.vals[pos] = val[k];
+    }
+    DLFX_PHASE(3);
 
     // ---- look back over the row's earlier tiles for digit `tid`
     uint32_t before_tiles = 0;
     {
-        int64_t p = t - 1;
-        bool done = (t == 0);
+        bool refetch = false;
         const uint32_t want_tag = static_cast<uint32_t>(pass + 1);
         for (;;) {
             int stuck = -1;
             while (!done) {
-                uint32_t sw[W];
-#pragma unroll
-                for (int i = 0; i < W; ++i) {
-                    const int64_t q = p - i;
-                    sw[i] = (q >= 0) ? __hip_atomic_load(status + srow + q * kRadix + tid, __ATOMIC_RELAXED,
-                                                         __HIP_MEMORY_SCOPE_AGENT)
-                                     : make_status(pass, true, 0u);
+                if (refetch) {
+                    fetch();
+                    refetch = false;
                 }
 #pragma unroll
                 for (int i = 0; i < W; ++i) {
@@ -292,13 +454,16 @@ __global__ __launch_bounds__(kBlock) void sort_pass(PassIo<K> io, int pass, int6
                     }
                     if ((s >> 28) != want_tag) {
                         stuck = static_cast<int>(q);
-                        p = q;                    // resume at this tile
                     } else {
                         before_tiles += s & kCountMask;
                         if (s & (1u << 27)) done = true;
                     }
                 }
-                if (stuck >= 0) break;
+                refetch = true;
+                if (stuck >= 0) {
+                    p = stuck;                    // resume at this tile
+                    break;
+                }
                 p -= W;
             }
             // anyone still waiting?  then the whole workgroup counts that tile's digits itself
@@ -312,7 +477,7 @@ __global__ __launch_bounds__(kBlock) void sort_pass(PassIo<K> io, int pass, int6
                 const int64_t hb = static_cast<int64_t>(help) * TILE;
                 const int hv = static_cast<int>((n - hb < TILE) ? n - hb : TILE);
                 for (int li = tid; li < hv; li += kBlock) {
-                    const K hk = load_key<K>(io, row, n, xrow, hb + li);
+                    const K hk = first ? key_of_element<K>(io, xrow[(hb + li) * io.sx]) : src_keys[row_off + hb + li];
                     atomicAdd(&sm.help_hist[static_cast<uint32_t>(hk >> shift) & 0xffu], 1u);
                 }
             }
@@ -329,69 +494,84 @@ __global__ __launch_bounds__(kBlock) void sort_pass(PassIo<K> io, int pass, int6
     }
     if (t > 0 && t + 1 < tiles_per_row)
         __hip_atomic_store(my_status, make_status(pass, true, before_tiles + count), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    sm.dst_base[tid] = static_cast<int64_t>(gbase[(row * P + pass) * kRadix + tid]) + before_tiles -
-                       static_cast<int64_t>(sm.digit_start[tid]);
+    sm.dst_base[tid] = static_cast<int32_t>(gbase[(row * P + pass) * kRadix + tid] + before_tiles) - static_cast<int32_t>(start);
     __syncthreads();
+    DLFX_PHASE(4);
 
-    // ---- gather the tile in its locally sorted order
+    // ---- write runs: thread t takes tile positions t, t + 256, ...
+    K out[ITEMS];
+    int32_t at[ITEMS];
+    uint32_t pay[PAIRS ? ITEMS : 1];
 #pragma unroll
-    for (int k = 0; k < ITEMS; ++k) {
-        const uint32_t d = static_cast<uint32_t>(key[k] >> shift) & 0xffu;
-        const uint32_t pos = sm.digit_start[d] + sm.wave_hist[w][d] + rank[k];
-        sm.keys[pos] = key[k];
-        if constexpr (PAIRS) sm.vals[pos] = val[k];
+    for (int k = 0; k < ITEMS; ++k) out[k] = sm.keys[k * kBlock + tid];
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) at[k] = sm.dst_base[static_cast<uint32_t>(out[k] >> shift) & 0xffu] + (k * kBlock + tid);
+    if constexpr (PAIRS) {
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) pay[k] = sm.vals[k * kBlock + tid];
     }
-    __syncthreads();
-
-    // ---- write runs
-    const int64_t row_off = row * n;
-    K* yrow = (io.last && io.y) ? io.y + io.ymap.at(row) : nullptr;
-    const int64_t irow = (io.last && io.idx) ? io.imap.at(row) : 0;
+    if constexpr (!LAST) {
+        K* dk = dst_keys + row_off;
 #pragma unroll
-    for (int k = 0; k < ITEMS; ++k) {
-        const int lp = k * kBlock + tid;
-        if (lp >= valid) continue;
-        const K kk = sm.keys[lp];
-        const uint32_t d = static_cast<uint32_t>(kk >> shift) & 0xffu;
-        const int64_t dst = sm.dst_base[d] + lp;
-        if (!io.last) {
-            io.dst_keys[row_off + dst] = kk;
-            if constexpr (PAIRS) io.dst_vals[row_off + dst] = sm.vals[lp];
-        } else {
-            uint32_t v = 0;
-            if constexpr (PAIRS) v = sm.vals[lp];
-            if (yrow) {
-                K bits = decode_key<K>(kk, io.kind, io.descending);
+        for (int k = 0; k < ITEMS; ++k)
+            if (full || k * kBlock + tid < valid) dk[at[k]] = out[k];
+        if constexpr (PAIRS) {
+            uint32_t* dv = dst_vals + row_off;
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k)
+                if (full || k * kBlock + tid < valid) dv[at[k]] = pay[k];
+        }
+    } else {
+        if (io.y) {
+            K* yrow = io.y + io.ymap.at(row);
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) {
+                K bits = decode_key<K>(out[k], io.kind, io.descending);
                 if constexpr (PAIRS) {
-                    if (io.restore_zero && (bits << 1) == 0) bits = io.x[io.xmap.at(row) + static_cast<int64_t>(v) * io.sx];
+                    if (io.restore_zero && (bits << 1) == 0 && (full || k * kBlock + tid < valid))
+                        bits = xrow[static_cast<int64_t>(pay[k]) * io.sx];
                 }
-                yrow[dst * io.sy] = bits;
+                if (full || k * kBlock + tid < valid) yrow[at[k] * io.sy] = bits;
             }
-            if constexpr (PAIRS) {
-                if (io.idx) {
-                    if (io.idx64) static_cast<int64_t*>(io.idx)[irow + dst * io.si] = static_cast<int64_t>(v);
-                    else static_cast<int32_t*>(io.idx)[irow + dst * io.si] = static_cast<int32_t>(v);
+        }
+        if constexpr (PAIRS) {
+            if (io.idx) {
+                const int64_t irow = io.imap.at(row);
+                if (io.idx64) {
+                    int64_t* ip = static_cast<int64_t*>(io.idx) + irow;
+#pragma unroll
+                    for (int k = 0; k < ITEMS; ++k)
+                        if (full || k * kBlock + tid < valid) ip[at[k] * io.si] = static_cast<int64_t>(pay[k]);
+                } else {
+                    int32_t* ip = static_cast<int32_t*>(io.idx) + irow;
+#pragma unroll
+                    for (int k = 0; k < ITEMS; ++k)
+                        if (full || k * kBlock + tid < valid) ip[at[k] * io.si] = static_cast<int32_t>(pay[k]);
                 }
             }
         }
     }
+    DLFX_PHASE(5);
 }
 
 // ------------------------------------------------------------------ host side
-template <typename K>
-constexpr int tile_items() { return 64 / sizeof(K); }       // 16 x u32 or 8 x u64 per thread
+// Keys per thread: 16, or 8 for 64-bit keys that carry an index (LDS and registers then
+// still allow four workgroups per compute unit).
+constexpr int tile_items(size_t key_size, bool pairs) { return (key_size == 8 && pairs) ? 8 : 16; }
 
 struct SortLayout {
     int64_t tiles_per_row;
-    size_t hist_off, hist_bytes, status_off, status_bytes, keys_off[2], vals_off[2], total;
+    size_t moves_off, hist_off, hist_bytes, status_off, status_bytes, keys_off[2], vals_off[2], total;
 };
 
 SortLayout sort_layout(size_t key_size, bool pairs, int64_t m, int64_t n) {
     SortLayout l;
     const int passes = key_size == 4 ? 4 : 8;
-    const int64_t tile = kBlock * (64 / static_cast<int64_t>(key_size));
+    const int64_t tile = kBlock * tile_items(key_size, pairs);
     l.tiles_per_row = ceil_div(n, tile);
     size_t off = 0;
+    l.moves_off = off;           // one word per (row, pass): does the pass move the row's keys
+    off += align_up(static_cast<size_t>(m) * passes * 4, 256);
     l.hist_off = off;
     l.hist_bytes = static_cast<size_t>(m) * passes * kRadix * 4;
     off += align_up(l.hist_bytes, 256);
@@ -434,7 +614,7 @@ struct SortArgs {
 template <typename K>
 int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratch_bytes) {
     constexpr int P = KeyTraits<K>::kPasses;
-    constexpr int ITEMS = tile_items<K>();
+    constexpr int IK = tile_items(sizeof(K), false), IP = tile_items(sizeof(K), true);
     const int64_t n = a.dims[a.rank - 1];
     const int64_t m = view_size(a.rank, a.dims) / n;
     if (n > kMaxRow) return DLFX_ERR_TOO_LARGE;
@@ -468,35 +648,41 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     io.canon_zero = (a.pairs && a.kind == kKeyFloat && !y_over_x) ? 1 : 0;
     io.restore_zero = (io.canon_zero && a.y) ? 1 : 0;
 
+    uint32_t* moves = reinterpret_cast<uint32_t*>(base + l.moves_off);
     uint32_t* ghist = reinterpret_cast<uint32_t*>(base + l.hist_off);
     uint32_t* status = reinterpret_cast<uint32_t*>(base + l.status_off);
-    const int64_t clear_words = static_cast<int64_t>((l.status_off + l.status_bytes) / 4);   // histograms + status
+    const int64_t clear_words = static_cast<int64_t>((l.status_off + l.status_bytes - l.hist_off) / 4);   // histograms + status
     sort_clear<<<dim3(static_cast<unsigned>(ceil_div(clear_words, kBlock))), dim3(kBlock), 0, stream>>>(ghist, clear_words);
     DLFX_CHECK_LAUNCH();
 
-    io.first = 1;
     const int64_t chunk = 32768;
     const int64_t chunks_per_row = ceil_div(n, chunk);
     if (m * chunks_per_row > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
     sort_histogram<K><<<dim3(static_cast<unsigned>(m * chunks_per_row)), dim3(kBlock), 0, stream>>>(io, n, chunk, chunks_per_row, ghist);
     DLFX_CHECK_LAUNCH();
-    sort_bases<<<dim3(static_cast<unsigned>(m * P)), dim3(kRadix), 0, stream>>>(ghist);
+    // a pass that moves nothing may only be left out when no pass reads the input while
+    // another tile of the same pass writes the output over it
+    sort_bases<<<dim3(static_cast<unsigned>(m * P)), dim3(kRadix), 0, stream>>>(
+        ghist, moves, y_over_x ? 0xffffffffu : static_cast<uint32_t>(n));
     DLFX_CHECK_LAUNCH();
 
-    K* kbuf[2] = {reinterpret_cast<K*>(base + l.keys_off[0]), reinterpret_cast<K*>(base + l.keys_off[1])};
-    uint32_t* vbuf[2] = {reinterpret_cast<uint32_t*>(base + l.vals_off[0]), reinterpret_cast<uint32_t*>(base + l.vals_off[1])};
+    io.kbuf[0] = reinterpret_cast<K*>(base + l.keys_off[0]);
+    io.kbuf[1] = reinterpret_cast<K*>(base + l.keys_off[1]);
+    io.vbuf[0] = a.pairs ? reinterpret_cast<uint32_t*>(base + l.vals_off[0]) : nullptr;
+    io.vbuf[1] = a.pairs ? reinterpret_cast<uint32_t*>(base + l.vals_off[1]) : nullptr;
     const dim3 grid(static_cast<unsigned>(m * l.tiles_per_row));
     for (int p = 0; p < P; ++p) {
-        io.first = (p == 0);
-        io.last = (p == P - 1);
-        io.src_keys = io.first ? nullptr : kbuf[(p - 1) & 1];
-        io.src_vals = (io.first || !a.pairs) ? nullptr : vbuf[(p - 1) & 1];
-        io.dst_keys = io.last ? nullptr : kbuf[p & 1];
-        io.dst_vals = (io.last || !a.pairs) ? nullptr : vbuf[p & 1];
-        if (a.pairs)
-            sort_pass<K, true, ITEMS><<<grid, dim3(kBlock), 0, stream>>>(io, p, n, l.tiles_per_row, ghist, status, g_sort_poll_limit);
-        else
-            sort_pass<K, false, ITEMS><<<grid, dim3(kBlock), 0, stream>>>(io, p, n, l.tiles_per_row, ghist, status, g_sort_poll_limit);
+        if (p < P - 1) {
+            if (a.pairs)
+                sort_pass<K, true, IP, false><<<grid, dim3(kBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
+            else
+                sort_pass<K, false, IK, false><<<grid, dim3(kBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
+        } else {
+            if (a.pairs)
+                sort_pass<K, true, IP, true><<<grid, dim3(kBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
+            else
+                sort_pass<K, false, IK, true><<<grid, dim3(kBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
+        }
         DLFX_CHECK_LAUNCH();
     }
     return DLFX_OK;
@@ -617,3 +803,19 @@ extern "C" int dlfx_argsort(dlfx_stream_t stream, int dir, int dtype, int index_
     a.pairs = true;
     return sort_entry(static_cast<hipStream_t>(stream), dtype, a, scratch, scratch_bytes);
 }
+
+#ifdef DLFX_SORT_TIMING
+extern "C" void dlfx_debug_sort_phases(unsigned long long* out, int reset) {
+    static unsigned long long host[dlfx::kPhaseSlots * 8];
+    if (out) {
+        (void)hipMemcpyFromSymbol(host, HIP_SYMBOL(dlfx::g_phase_cycles), sizeof(host));
+        for (int i = 0; i < 8; ++i) out[i] = 0;
+        for (int b = 0; b < dlfx::kPhaseSlots; ++b)
+            for (int i = 0; i < 8; ++i) out[i] += host[b * 8 + i];
+    }
+    if (reset) {
+        for (auto& v : host) v = 0;
+        (void)hipMemcpyToSymbol(HIP_SYMBOL(dlfx::g_phase_cycles), host, sizeof(host));
+    }
+}
+#endif

@@ -130,3 +130,32 @@ def test_many_short_rows(hip_backend, oracle_backend):
     Xh, Xo = both(hip_backend, oracle_backend, x)
     assert np.array_equal(F.sort(Xh, -1).numpy(), F.sort(Xo, -1).numpy())
     assert np.array_equal(F.argsort(Xh, 0).numpy(), F.argsort(Xo, 0).numpy())
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.int64, np.float32, np.float64])
+def test_rows_leave_out_passes_that_move_nothing(hip_backend, oracle_backend, dtype):
+    # digits that are the same in a whole row are not sorted on; rows decide independently, so
+    # neighbouring rows take different routes through the scratch buffers
+    n = 10000
+    small = randint(70, n, 0, 200).astype(dtype)                      # only the lowest digit varies
+    medium = randint(71, n, 0, 50000).astype(dtype)                   # two digits vary
+    constant = np.full(n, 7, dtype=dtype)                             # nothing varies: one pass, input -> output
+    if np.dtype(dtype).kind == "i":
+        wide = full_range_i64(72, n).astype(dtype)
+    else:
+        wide = (normal(72, n) * 1e3).astype(dtype)
+    x = np.stack([small, wide, constant, medium, small[::-1].copy(), constant])
+    Xh, Xo = both(hip_backend, oracle_backend, x)
+    for desc in (False, True):
+        assert np.array_equal(F.sort(Xh, -1, desc).numpy(), F.sort(Xo, -1, desc).numpy()), desc
+        Yh, Ih = F.argsort(Xh, -1, desc, with_values=True)
+        Yo, Io = F.argsort(Xo, -1, desc, with_values=True)
+        assert np.array_equal(Ih.numpy(), Io.numpy()), desc
+        assert np.array_equal(Yh.numpy(), Yo.numpy()), desc
+    # written over the input: every pass runs, none may read the input while it is overwritten
+    F.sort(Xh, -1, out=Xh)
+    assert np.array_equal(Xh.numpy(), np.sort(x, axis=-1))
+    Xh = Tensor.from_numpy(hip_backend, x)
+    Yh, Ih = F.argsort(Xh, -1, values=Xh)
+    assert np.array_equal(Yh.numpy(), np.sort(x, axis=-1))
+    assert np.array_equal(Ih.numpy(), np.argsort(x, axis=-1, kind="stable"))
