@@ -33,6 +33,11 @@ namespace {
 #endif
 constexpr int kBlock = 256;
 constexpr int kWaves = kBlock / kWave;
+#ifndef DLFX_SORT_PASS_BLOCK
+#define DLFX_SORT_PASS_BLOCK 256
+#endif
+constexpr int kPassBlock = DLFX_SORT_PASS_BLOCK;       // threads of a sort_pass workgroup
+constexpr int kPassWaves = kPassBlock / kWave;
 constexpr int kRadix = 256;
 constexpr int64_t kMaxRow = (int64_t(1) << 27) - 1;   // counts share a status word with 5 tag bits
 
@@ -172,24 +177,36 @@ __global__ __launch_bounds__(kBlock) void sort_histogram(PassIo<K> io, int64_t n
 }
 
 // In place: histogram -> exclusive prefix (start of each digit's run in the row).  Workgroup
-// b handles one (row, pass) pair.  moves[b] tells whether that pass changes the order of that
-// row: when all n keys of the row share the digit it does not, and the row skips the pass.
-__global__ __launch_bounds__(kRadix) void sort_bases(uint32_t* __restrict__ ghist, uint32_t* __restrict__ moves, uint32_t n) {
+// b handles one (row, pass) pair.  moves[b] receives the bits of the digit that are not the
+// same in all keys of the row: none means the pass would not change the order of the row (the
+// row then skips it), and the ranking only needs to look at those bits.  `all_bits` forces
+// every pass of every row to run.
+__global__ __launch_bounds__(kRadix) void sort_bases(uint32_t* __restrict__ ghist, uint32_t* __restrict__ moves, int all_bits) {
     __shared__ uint32_t wave_tot[kRadix / kWave];
-    __shared__ uint32_t one_digit;
-    if (threadIdx.x == 0) one_digit = 0u;
+    __shared__ uint32_t wave_or[kRadix / kWave], wave_and[kRadix / kWave];
     uint32_t* g = ghist + static_cast<int64_t>(blockIdx.x) * kRadix;
     const uint32_t v = g[threadIdx.x];
     const uint32_t incl = wave_scan_inclusive(v, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+    const uint32_t ors = wave_reduce(v ? threadIdx.x : 0u, [](uint32_t a, uint32_t b) { return a | b; });
+    const uint32_t ands = wave_reduce(v ? threadIdx.x : 0xffu, [](uint32_t a, uint32_t b) { return a & b; });
     const int w = threadIdx.x / kWave;
-    __syncthreads();
-    if (lane_id() == kWave - 1) wave_tot[w] = incl;
-    if (v == n) one_digit = 1u;
+    if (lane_id() == kWave - 1) {
+        wave_tot[w] = incl;
+        wave_or[w] = ors;
+        wave_and[w] = ands;
+    }
     __syncthreads();
     uint32_t pre = 0;
     for (int i = 0; i < w; ++i) pre += wave_tot[i];
     g[threadIdx.x] = pre + incl - v;
-    if (threadIdx.x == 0) moves[blockIdx.x] = one_digit ? 0u : 1u;
+    if (threadIdx.x == 0) {
+        uint32_t o = 0, a = 0xffu;
+        for (int i = 0; i < kRadix / kWave; ++i) {
+            o |= wave_or[i];
+            a &= wave_and[i];
+        }
+        moves[blockIdx.x] = all_bits ? 0xffu : (o ^ a);
+    }
 }
 
 __global__ __launch_bounds__(kBlock) void sort_clear(uint32_t* __restrict__ p, int64_t words) {
@@ -207,13 +224,13 @@ __device__ __forceinline__ uint32_t make_status(int pass, bool inclusive, uint32
 
 template <typename K, bool PAIRS, int ITEMS>
 struct PassShared {
-    uint32_t wave_hist[kWaves][kRadix];       // per-wave digit counts, then per-wave offsets
+    uint32_t wave_hist[kPassWaves][kRadix];       // per-wave digit counts, then per-wave offsets
     uint32_t help_hist[kRadix];               // digits of an earlier tile counted here when it is late
     int32_t dst_base[kRadix];                 // row position of that digit's run start minus digit_start
-    uint32_t scan_tmp[kWaves];
+    uint32_t scan_tmp[kPassWaves];
     int help_tile;
-    K keys[kBlock * ITEMS];
-    uint32_t vals[PAIRS ? kBlock * ITEMS : 1];
+    K keys[kPassBlock * ITEMS];
+    uint32_t vals[PAIRS ? kPassBlock * ITEMS : 1];
 };
 
 // Pass `pass` of the sort (digit = bits [8 pass, 8 pass + 8) of the key).  LAST: the pass of
@@ -222,12 +239,12 @@ struct PassShared {
 // pass it runs reads the strided input, and its place in the ping-pong buffers alternates
 // over the passes it does run.
 template <typename K, bool PAIRS, int ITEMS, bool LAST>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SORT_WAVES))) void sort_pass(PassIo<K> io, int pass, int64_t rows, int64_t n, int64_t tiles_per_row,
+__global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SORT_WAVES))) void sort_pass(PassIo<K> io, int pass, int64_t rows, int64_t n, int64_t tiles_per_row,
                                                     const uint32_t* __restrict__ gbase,
                                                     const uint32_t* __restrict__ moves,
                                                     uint32_t* __restrict__ status, int poll_limit) {
     constexpr int P = KeyTraits<K>::kPasses;
-    constexpr int TILE = kBlock * ITEMS;
+    constexpr int TILE = kPassBlock * ITEMS;
     constexpr int W = 4;    // status words of earlier tiles fetched per look-back step
     __shared__ PassShared<K, PAIRS, ITEMS> sm;
 
@@ -258,7 +275,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SOR
     const int shift = 8 * pass;
 
     DLFX_PHASE_BEGIN();
-    for (int i = tid; i < kWaves * kRadix; i += kBlock) (&sm.wave_hist[0][0])[i] = 0;
+    for (int i = tid; i < kPassWaves * kRadix; i += kPassBlock) (&sm.wave_hist[0][0])[i] = 0;
     if (tid == 0) sm.help_tile = -1;
 
     // ---- load: wave w owns [w*64*ITEMS, ...), item k of lane l is element k*64 + l of it.
@@ -319,10 +336,12 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SOR
     DLFX_PHASE(0);
 
     // ---- rank inside the wave, in element order (stable).  The lanes whose digit equals this
-    // lane's are found with one ballot per digit bit; two items at a time, so that the two
-    // independent chains fill each other's wait states.  The items then take their ranks from
+    // lane's are found with one ballot per digit bit that varies in the row (padding differs
+    // in other bits too, so a tile with padding looks at all of them); two items at a time, so
+    // that the two independent chains fill each other's wait states.  The items then take their ranks from
     // the wave's running digit counts one after the other: the first lane of each group of
     // equal digits moves the count on.
+    const uint32_t vary = full ? row_moves[pass] : 0xffu;
     uint32_t rank[ITEMS];
     static_assert(ITEMS % 2 == 0, "items are ranked in pairs");
 #pragma unroll
@@ -331,11 +350,11 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SOR
 #pragma unroll
         for (int j = 0; j < 2; ++j) d[j] = static_cast<uint32_t>(key[k0 + j] >> shift) & 0xffu;
         uint32_t peers_lo[2] = {0xffffffffu, 0xffffffffu}, peers_hi[2] = {0xffffffffu, 0xffffffffu};
-#pragma unroll
-        for (int b = 0; b < 8; ++b) {
+        for (uint32_t bits = vary; bits != 0u; bits &= bits - 1u) {
+            const uint32_t b = static_cast<uint32_t>(__builtin_ctz(bits));
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const int32_t ones = static_cast<int32_t>(d[j] << (31 - b)) >> 31;       // all ones when the bit is set
+                const int32_t ones = __builtin_amdgcn_sbfe(static_cast<int32_t>(d[j]), b, 1u);     // all ones when the bit is set
                 const unsigned long long vote = __ballot(ones < 0);
                 peers_lo[j] &= ~(static_cast<uint32_t>(vote) ^ static_cast<uint32_t>(ones));
                 peers_hi[j] &= ~(static_cast<uint32_t>(vote >> 32) ^ static_cast<uint32_t>(ones));
@@ -355,39 +374,25 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SOR
             __builtin_amdgcn_wave_barrier();
         }
     }
-#ifdef DLFX_SORT_DOUBLE_RANK
-    // timing experiment only: the ballot work of the ranking a second time, on other bits
-#pragma unroll
-    for (int k = 0; k < ITEMS; ++k) {
-        const uint32_t d = static_cast<uint32_t>(key[k] >> (shift ^ 8)) & 0xffu;
-        uint32_t peers_lo = 0xffffffffu, peers_hi = 0xffffffffu;
-#pragma unroll
-        for (int b = 0; b < 8; ++b) {
-            const uint32_t ones = 0u - ((d >> b) & 1u);
-            const unsigned long long vote = __ballot(ones != 0u);
-            peers_lo &= ~(static_cast<uint32_t>(vote) ^ ones);
-            peers_hi &= ~(static_cast<uint32_t>(vote >> 32) ^ ones);
-        }
-        const uint32_t before = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
-        if (before == 0xffffu) rank[k] += 1;
-    }
-#endif
     __syncthreads();
     DLFX_PHASE(1);
 
     // ---- thread d owns digit d: tile count, position of the digit in the tile, wave offsets
-    uint32_t wave_count[kWaves];
+    // (threads beyond the 256 digits idle through this part, except at the barriers)
+    const bool owner = tid < kRadix;
+    const int dg = owner ? tid : 0;
+    uint32_t wave_count[kPassWaves];
     uint32_t count = 0;
 #pragma unroll
-    for (int i = 0; i < kWaves; ++i) {
-        wave_count[i] = sm.wave_hist[i][tid];
+    for (int i = 0; i < kPassWaves; ++i) {
+        wave_count[i] = sm.wave_hist[i][dg];
         count += wave_count[i];
     }
     const uint32_t padded = count;
     if (tid == kRadix - 1) count -= static_cast<uint32_t>(TILE - valid);     // padding is not part of the row
     const int64_t srow = (row * tiles_per_row) * kRadix;
-    uint32_t* my_status = status + srow + t * kRadix + tid;
-    if (t + 1 < tiles_per_row)
+    uint32_t* my_status = status + srow + t * kRadix + dg;
+    if (owner && t + 1 < tiles_per_row)
         __hip_atomic_store(my_status, make_status(pass, t == 0, count), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // the status words of the W tiles before this one are requested now and looked at after
     // the tile has been gathered, so that their latency is not waited for
@@ -397,25 +402,27 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SOR
 #pragma unroll
         for (int i = 0; i < W; ++i) {
             const int64_t q = p - i;
-            sw[i] = (q >= 0) ? __hip_atomic_load(status + srow + q * kRadix + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+            sw[i] = (q >= 0) ? __hip_atomic_load(status + srow + q * kRadix + dg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
                              : make_status(pass, true, 0u);
         }
     };
-    bool done = (t == 0);
+    bool done = (t == 0) || !owner;
     if (!done) fetch();
     uint32_t start;
     {
         const uint32_t incl = wave_scan_inclusive(padded, 0u, [](uint32_t a, uint32_t b) { return a + b; });
-        if (lane == kWave - 1) sm.scan_tmp[w] = incl;
+        if (owner && lane == kWave - 1) sm.scan_tmp[w] = incl;
         __syncthreads();
         uint32_t pre = 0;
-        for (int i = 0; i < w; ++i) pre += sm.scan_tmp[i];
+        for (int i = 0; i < w && i < kRadix / kWave; ++i) pre += sm.scan_tmp[i];
         start = pre + incl - padded;
         uint32_t run = start;
+        if (owner) {
 #pragma unroll
-        for (int i = 0; i < kWaves; ++i) {
-            sm.wave_hist[i][tid] = run;        // tile position of the first key of wave i with this digit
-            run += wave_count[i];
+            for (int i = 0; i < kPassWaves; ++i) {
+                sm.wave_hist[i][tid] = run;        // tile position of the first key of wave i with this digit
+                run += wave_count[i];
+            }
         }
     }
     __syncthreads();
@@ -450,7 +457,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SOR
                     uint32_t s = sw[i];
                     for (int polls = 0; (s >> 28) != want_tag && polls < poll_limit; ++polls) {
                         __builtin_amdgcn_s_sleep(1);
-                        s = __hip_atomic_load(status + srow + q * kRadix + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        s = __hip_atomic_load(status + srow + q * kRadix + dg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     }
                     if ((s >> 28) != want_tag) {
                         stuck = static_cast<int>(q);
@@ -471,19 +478,19 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SOR
             __syncthreads();
             const int help = sm.help_tile;
             if (help < 0) break;
-            sm.help_hist[tid] = 0;
+            if (owner) sm.help_hist[tid] = 0;
             __syncthreads();
             {
                 const int64_t hb = static_cast<int64_t>(help) * TILE;
                 const int hv = static_cast<int>((n - hb < TILE) ? n - hb : TILE);
-                for (int li = tid; li < hv; li += kBlock) {
+                for (int li = tid; li < hv; li += kPassBlock) {
                     const K hk = first ? key_of_element<K>(io, xrow[(hb + li) * io.sx]) : src_keys[row_off + hb + li];
                     atomicAdd(&sm.help_hist[static_cast<uint32_t>(hk >> shift) & 0xffu], 1u);
                 }
             }
             __syncthreads();
             if (stuck == help) {
-                before_tiles += sm.help_hist[tid];
+                before_tiles += sm.help_hist[dg];
                 p = static_cast<int64_t>(help) - 1;
                 if (p < 0) done = true;
             }
@@ -492,9 +499,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SOR
             __syncthreads();
         }
     }
-    if (t > 0 && t + 1 < tiles_per_row)
+    if (owner && t > 0 && t + 1 < tiles_per_row)
         __hip_atomic_store(my_status, make_status(pass, true, before_tiles + count), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    sm.dst_base[tid] = static_cast<int32_t>(gbase[(row * P + pass) * kRadix + tid] + before_tiles) - static_cast<int32_t>(start);
+    if (owner) sm.dst_base[tid] = static_cast<int32_t>(gbase[(row * P + pass) * kRadix + tid] + before_tiles) - static_cast<int32_t>(start);
     __syncthreads();
     DLFX_PHASE(4);
 
@@ -503,23 +510,23 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SOR
     int32_t at[ITEMS];
     uint32_t pay[PAIRS ? ITEMS : 1];
 #pragma unroll
-    for (int k = 0; k < ITEMS; ++k) out[k] = sm.keys[k * kBlock + tid];
+    for (int k = 0; k < ITEMS; ++k) out[k] = sm.keys[k * kPassBlock + tid];
 #pragma unroll
-    for (int k = 0; k < ITEMS; ++k) at[k] = sm.dst_base[static_cast<uint32_t>(out[k] >> shift) & 0xffu] + (k * kBlock + tid);
+    for (int k = 0; k < ITEMS; ++k) at[k] = sm.dst_base[static_cast<uint32_t>(out[k] >> shift) & 0xffu] + (k * kPassBlock + tid);
     if constexpr (PAIRS) {
 #pragma unroll
-        for (int k = 0; k < ITEMS; ++k) pay[k] = sm.vals[k * kBlock + tid];
+        for (int k = 0; k < ITEMS; ++k) pay[k] = sm.vals[k * kPassBlock + tid];
     }
     if constexpr (!LAST) {
         K* dk = dst_keys + row_off;
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k)
-            if (full || k * kBlock + tid < valid) dk[at[k]] = out[k];
+            if (full || k * kPassBlock + tid < valid) dk[at[k]] = out[k];
         if constexpr (PAIRS) {
             uint32_t* dv = dst_vals + row_off;
 #pragma unroll
             for (int k = 0; k < ITEMS; ++k)
-                if (full || k * kBlock + tid < valid) dv[at[k]] = pay[k];
+                if (full || k * kPassBlock + tid < valid) dv[at[k]] = pay[k];
         }
     } else {
         if (io.y) {
@@ -528,10 +535,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SOR
             for (int k = 0; k < ITEMS; ++k) {
                 K bits = decode_key<K>(out[k], io.kind, io.descending);
                 if constexpr (PAIRS) {
-                    if (io.restore_zero && (bits << 1) == 0 && (full || k * kBlock + tid < valid))
+                    if (io.restore_zero && (bits << 1) == 0 && (full || k * kPassBlock + tid < valid))
                         bits = xrow[static_cast<int64_t>(pay[k]) * io.sx];
                 }
-                if (full || k * kBlock + tid < valid) yrow[at[k] * io.sy] = bits;
+                if (full || k * kPassBlock + tid < valid) yrow[at[k] * io.sy] = bits;
             }
         }
         if constexpr (PAIRS) {
@@ -541,12 +548,12 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SOR
                     int64_t* ip = static_cast<int64_t*>(io.idx) + irow;
 #pragma unroll
                     for (int k = 0; k < ITEMS; ++k)
-                        if (full || k * kBlock + tid < valid) ip[at[k] * io.si] = static_cast<int64_t>(pay[k]);
+                        if (full || k * kPassBlock + tid < valid) ip[at[k] * io.si] = static_cast<int64_t>(pay[k]);
                 } else {
                     int32_t* ip = static_cast<int32_t*>(io.idx) + irow;
 #pragma unroll
                     for (int k = 0; k < ITEMS; ++k)
-                        if (full || k * kBlock + tid < valid) ip[at[k] * io.si] = static_cast<int32_t>(pay[k]);
+                        if (full || k * kPassBlock + tid < valid) ip[at[k] * io.si] = static_cast<int32_t>(pay[k]);
                 }
             }
         }
@@ -557,7 +564,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SOR
 // ------------------------------------------------------------------ host side
 // Keys per thread: 16, or 8 for 64-bit keys that carry an index (LDS and registers then
 // still allow four workgroups per compute unit).
-constexpr int tile_items(size_t key_size, bool pairs) { return (key_size == 8 && pairs) ? 8 : 16; }
+constexpr int tile_items(size_t key_size, bool pairs) { return ((key_size == 8 && pairs) ? 8 : 16) * 256 / kPassBlock; }
 
 struct SortLayout {
     int64_t tiles_per_row;
@@ -567,7 +574,7 @@ struct SortLayout {
 SortLayout sort_layout(size_t key_size, bool pairs, int64_t m, int64_t n) {
     SortLayout l;
     const int passes = key_size == 4 ? 4 : 8;
-    const int64_t tile = kBlock * tile_items(key_size, pairs);
+    const int64_t tile = kPassBlock * tile_items(key_size, pairs);
     l.tiles_per_row = ceil_div(n, tile);
     size_t off = 0;
     l.moves_off = off;           // one word per (row, pass): does the pass move the row's keys
@@ -662,8 +669,7 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     DLFX_CHECK_LAUNCH();
     // a pass that moves nothing may only be left out when no pass reads the input while
     // another tile of the same pass writes the output over it
-    sort_bases<<<dim3(static_cast<unsigned>(m * P)), dim3(kRadix), 0, stream>>>(
-        ghist, moves, y_over_x ? 0xffffffffu : static_cast<uint32_t>(n));
+    sort_bases<<<dim3(static_cast<unsigned>(m * P)), dim3(kRadix), 0, stream>>>(ghist, moves, y_over_x ? 1 : 0);
     DLFX_CHECK_LAUNCH();
 
     io.kbuf[0] = reinterpret_cast<K*>(base + l.keys_off[0]);
@@ -674,14 +680,14 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     for (int p = 0; p < P; ++p) {
         if (p < P - 1) {
             if (a.pairs)
-                sort_pass<K, true, IP, false><<<grid, dim3(kBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
+                sort_pass<K, true, IP, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
             else
-                sort_pass<K, false, IK, false><<<grid, dim3(kBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
+                sort_pass<K, false, IK, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
         } else {
             if (a.pairs)
-                sort_pass<K, true, IP, true><<<grid, dim3(kBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
+                sort_pass<K, true, IP, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
             else
-                sort_pass<K, false, IK, true><<<grid, dim3(kBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
+                sort_pass<K, false, IK, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
         }
         DLFX_CHECK_LAUNCH();
     }
