@@ -27,6 +27,14 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the step's kernels, from two profiler runs of this script with
+# --copy-calibration (rocprofv3 --pmc FETCH_SIZE, then --pmc WRITE_SIZE; KiB per dispatch, each
+# scaled by what the counter reads for the 1 GiB device copy: 2.000 and 1.000).  A counter cannot
+# be read from inside the timed run, so the figures are constants of the kernels as committed.
+MEASURED_TRAFFIC_BYTES = {
+    "reduce_rows_block": 4295003390,      # 2^30 fp32: 1.0000 x the algorithmic bytes
+    "scan_rows_chained": 539300000,       # [64, 2^20] 4-byte elements: 1.0045 x
+}
 METRIC = "HBM GB/s (% of ~8 TB/s peak) + Gelem/s per op: reduce, scan, top_k, sort"
 
 
@@ -391,7 +399,8 @@ def main():
         achieved = dom.alg_bytes / avg_us / 1e3
         result["roofline"] = {"bound": "hbm", "kernel": dom.kernel, "op": dom.name, "achieved": round(achieved, 1),
                               "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                              "avg_launch_us": round(avg_us, 2), "traffic": None}
+                              "avg_launch_us": round(avg_us, 2),
+                              "traffic": next((v for k, v in MEASURED_TRAFFIC_BYTES.items() if k in dom.kernel), None)}
     else:
         result.update({"value": None, "ms_per_step": None, "config": {"workload": args.configs}})
 
