@@ -214,6 +214,50 @@ def make_ops(be, which):
             tol = 4 * 9 * float(np.finfo(np.float32).eps) * torch.maximum(want.abs(), mag)
             assert bool(((y.double() - want).abs() <= tol).all())
         ops.append(Op("C5", "cumsum{1}_f32_[32,512,56,56]", n5, 8 * n5, calls, v_cs))
+
+    # ---------------- N1: count and nonzero (the callers next to reduce and scan)
+    if on("all", "n1"):
+        rows_n, cols_n = 4096, 16384
+        xn = gen((rows_n, cols_n), torch.float32, lambda c: (lambda idx, f=synth.randint(9 + 100 * c, 0, 4): f(idx) // 3), 4)   # a quarter ones, the rest zeros
+        nn = rows_n * cols_n
+        zero = np.zeros(1, dtype=np.float32)
+        calls, outs = [], []
+        for x in xn:
+            X = tensor(x)
+            view, out_dims, m, n = prepare_reduce(X.shape, [1], False)
+            Y = Tensor.empty(be, out_dims, np.int32)
+            calls.append(be.count(dtype_code(X.dtype), m, n, 0.0, view, X.storage, Y.shape, Y.storage, defer=True))
+            outs.append(Y)
+
+        def v_count(x=xn[0], out=outs[0], call=calls[0]):
+            call()
+            assert torch.equal(out.storage[:rows_n].long(), (x == 0).sum(1))
+        ops.append(Op("N1", "count0{1}_f32_[4096,16384]", nn, 4 * nn + 4 * rows_n, calls, v_count))
+
+        counts = Tensor.empty(be, [nn], np.int32)
+        flat = Shape([nn])
+        calls = [be.scan_nonzero(dtype_code(np.float32), 1, nn, False, tensor(x).shape, tensor(x).storage,
+                                 Shape([rows_n, cols_n]), counts.storage, defer=True) for x in xn]
+
+        def v_scan_nz(x=xn[0], call=calls[0]):
+            call()
+            assert torch.equal(counts.storage[:nn].long(), torch.cumsum((x.view(-1) != 0).long(), 0))
+        ops.append(Op("N1", "scan_nonzero_f32_[2^26]", nn, 8 * nn, calls, v_scan_nz))
+
+        # gather_indices reads counts that must match its n: it gets its own copy of the
+        # first input's counts, which the timed scan_nonzero calls (other inputs) never touch
+        counts0 = Tensor.empty(be, [nn], np.int32)
+        be.scan_nonzero(dtype_code(np.float32), 1, nn, False, tensor(xn[0]).shape, tensor(xn[0]).storage,
+                        Shape([rows_n, cols_n]), counts0.storage)
+        torch.cuda.synchronize()
+        total = int(counts0.storage[nn - 1].item())
+        coords = Tensor.empty(be, [total, 2], np.int32)
+        gcall = be.gather_indices(nn, total, False, [rows_n, cols_n], counts0.storage, coords.storage, defer=True)
+
+        def v_gather(x=xn[0]):
+            gcall()
+            assert torch.equal(coords.storage[:2 * total].view(total, 2).long(), torch.nonzero(x))
+        ops.append(Op("N1", "gather_indices_[2^26]->[%d,2]" % total, nn, 4 * nn + 8 * total, [gcall], v_gather))
     return ops
 
 
@@ -338,7 +382,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5")
+    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",

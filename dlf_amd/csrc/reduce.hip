@@ -56,6 +56,7 @@ struct ValueReducer {
     using in_t = T;
     using acc_t = typename AccType<T, J>::type;
     using out_t = T;
+    using param_t = int;      // no run-time parameter
 
     __device__ static __forceinline__ acc_t identity() {
         if constexpr (J == kAdd) return acc_t(0);
@@ -63,7 +64,7 @@ struct ValueReducer {
         else if constexpr (J == kMax) return (M == kMapAbs) ? acc_t(0) : std::numeric_limits<T>::lowest();
         else return std::numeric_limits<T>::max();
     }
-    __device__ static __forceinline__ acc_t map(T x, int64_t) {
+    __device__ static __forceinline__ acc_t map(T x, int64_t, param_t) {
         if constexpr (M == kMapExp) {
             if constexpr (std::is_same<T, float>::value) return static_cast<acc_t>(expf(x));
             else return static_cast<acc_t>(exp(static_cast<double>(x)));
@@ -116,6 +117,7 @@ struct ArgReducer {
     using in_t = T;
     using acc_t = ArgAcc<T>;
     using out_t = I;
+    using param_t = int;
 
     __device__ static __forceinline__ acc_t identity() {
         // weakest possible value, so that any element (even -inf / +inf) ties or wins;
@@ -127,7 +129,7 @@ struct ArgReducer {
             return {MAX ? -std::numeric_limits<T>::infinity() : std::numeric_limits<T>::infinity(),
                     std::numeric_limits<int32_t>::max()};
     }
-    __device__ static __forceinline__ acc_t map(T x, int64_t j) {
+    __device__ static __forceinline__ acc_t map(T x, int64_t j, param_t) {
         if constexpr (!std::is_integral<T>::value) {
             if (x != x) {
                 if (j == 0)
@@ -147,6 +149,21 @@ struct ArgReducer {
     }
 };
 
+// count: number of elements equal to a value (dlf/include/tensor/reduce.h:151-158: Map
+// x == value ? 1 : 0, fold +).  The value is the reducer's run-time parameter.
+template <typename T>
+struct CountReducer {
+    using in_t = T;
+    using acc_t = int32_t;
+    using out_t = int32_t;
+    using param_t = T;
+
+    __device__ static __forceinline__ acc_t identity() { return 0; }
+    __device__ static __forceinline__ acc_t map(T x, int64_t, param_t value) { return x == value ? 1 : 0; }
+    __device__ static __forceinline__ acc_t join(acc_t a, acc_t b) { return wrap_add(a, b); }
+    __device__ static __forceinline__ out_t finish(acc_t a, int64_t, int) { return a; }
+};
+
 // --------------------------------------------------------------------------
 // One row's contiguous elements, visited by `width` cooperating lanes (lane
 // `g` of the group) restricted to 128-bit vectors [v_lo, v_hi) of the aligned
@@ -154,7 +171,7 @@ struct ArgReducer {
 template <typename R>
 __device__ __forceinline__ typename R::acc_t
 row_partial_contig(const typename R::in_t* __restrict__ p, int64_t n, int g, int width,
-                   int64_t part, int64_t parts) {
+                   int64_t part, int64_t parts, typename R::param_t prm) {
     using T = typename R::in_t;
     using acc_t = typename R::acc_t;
     constexpr int V = vec_width<T>();
@@ -179,36 +196,36 @@ row_partial_contig(const typename R::in_t* __restrict__ p, int64_t n, int g, int
              d = load_stream(&pv[v + 3 * width]);
         const int64_t j0 = head + v * V;
 #pragma unroll
-        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(a.v[e], j0 + e));
+        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(a.v[e], j0 + e, prm));
 #pragma unroll
-        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(b.v[e], j0 + static_cast<int64_t>(width) * V + e));
+        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(b.v[e], j0 + static_cast<int64_t>(width) * V + e, prm));
 #pragma unroll
-        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(c.v[e], j0 + 2 * static_cast<int64_t>(width) * V + e));
+        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(c.v[e], j0 + 2 * static_cast<int64_t>(width) * V + e, prm));
 #pragma unroll
-        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(d.v[e], j0 + 3 * static_cast<int64_t>(width) * V + e));
+        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(d.v[e], j0 + 3 * static_cast<int64_t>(width) * V + e, prm));
     }
     for (; v < v_hi; v += width) {
         VecT a = load_stream(&pv[v]);
         const int64_t j0 = head + v * V;
 #pragma unroll
-        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(a.v[e], j0 + e));
+        for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(a.v[e], j0 + e, prm));
     }
     if (part == 0)
-        for (int64_t j = g; j < head; j += width) acc = R::join(acc, R::map(p[j], j));
+        for (int64_t j = g; j < head; j += width) acc = R::join(acc, R::map(p[j], j, prm));
     if (part == parts - 1)
-        for (int64_t j = tail_start + g; j < n; j += width) acc = R::join(acc, R::map(p[j], j));
+        for (int64_t j = tail_start + g; j < n; j += width) acc = R::join(acc, R::map(p[j], j, prm));
     return acc;
 }
 
 template <typename R>
 __device__ __forceinline__ typename R::acc_t
 row_partial_strided(const typename R::in_t* __restrict__ p, const DimMap& red, int64_t n, int g,
-                    int width, int64_t part, int64_t parts) {
+                    int width, int64_t part, int64_t parts, typename R::param_t prm) {
     typename R::acc_t acc = R::identity();
     const int64_t per = (n + parts - 1) / parts;
     const int64_t lo = part * per;
     const int64_t hi = (lo + per < n) ? lo + per : n;
-    for (int64_t j = lo + g; j < hi; j += width) acc = R::join(acc, R::map(p[red.at(j)], j));
+    for (int64_t j = lo + g; j < hi; j += width) acc = R::join(acc, R::map(p[red.at(j)], j, prm));
     return acc;
 }
 
@@ -216,15 +233,15 @@ row_partial_strided(const typename R::in_t* __restrict__ p, const DimMap& red, i
 template <typename R, bool CONTIG>
 __global__ __launch_bounds__(kBlock) void reduce_rows_group(
     const typename R::in_t* __restrict__ x, DimMap kept, DimMap red, int64_t m, int64_t n, int log2g,
-    typename R::out_t* __restrict__ y, DimMap ymap, int final_op) {
+    typename R::out_t* __restrict__ y, DimMap ymap, int final_op, typename R::param_t prm) {
     const int width = 1 << log2g;
     const int64_t row = static_cast<int64_t>(blockIdx.x) * (kBlock >> log2g) + (threadIdx.x >> log2g);
     const int g = threadIdx.x & (width - 1);
     typename R::acc_t acc = R::identity();
     if (row < m) {
         const typename R::in_t* p = x + kept.at(row);
-        if constexpr (CONTIG) acc = row_partial_contig<R>(p, n, g, width, 0, 1);
-        else acc = row_partial_strided<R>(p, red, n, g, width, 0, 1);
+        if constexpr (CONTIG) acc = row_partial_contig<R>(p, n, g, width, 0, 1, prm);
+        else acc = row_partial_strided<R>(p, red, n, g, width, 0, 1, prm);
     }
     acc = group_reduce(acc, width, [](typename R::acc_t a, typename R::acc_t b) { return R::join(a, b); });
     if (row < m && g == 0) y[ymap.at(row)] = R::finish(acc, n, final_op);
@@ -250,13 +267,13 @@ template <typename R, bool CONTIG>
 __global__ __launch_bounds__(kBlock) void reduce_rows_block(
     const typename R::in_t* __restrict__ x, DimMap kept, DimMap red, int64_t n, int64_t parts,
     typename R::out_t* __restrict__ y, DimMap ymap, int final_op,
-    typename R::acc_t* __restrict__ partial) {
+    typename R::acc_t* __restrict__ partial, typename R::param_t prm) {
     const int64_t row = blockIdx.x / parts;
     const int64_t part = blockIdx.x - row * parts;
     const typename R::in_t* p = x + kept.at(row);
     typename R::acc_t acc;
-    if constexpr (CONTIG) acc = row_partial_contig<R>(p, n, threadIdx.x, kBlock, part, parts);
-    else acc = row_partial_strided<R>(p, red, n, threadIdx.x, kBlock, part, parts);
+    if constexpr (CONTIG) acc = row_partial_contig<R>(p, n, threadIdx.x, kBlock, part, parts, prm);
+    else acc = row_partial_strided<R>(p, red, n, threadIdx.x, kBlock, part, parts, prm);
     acc = block_reduce<R>(acc);
     if (threadIdx.x == 0) {
         if (parts == 1) y[ymap.at(row)] = R::finish(acc, n, final_op);
@@ -284,7 +301,7 @@ template <typename R>
 __global__ __launch_bounds__(kBlock) void reduce_cols(
     const typename R::in_t* __restrict__ x, DimMap outer, int64_t L, DimMap red, int64_t n,
     int64_t col_blocks, int64_t parts, typename R::out_t* __restrict__ y, DimMap ymap, int final_op,
-    typename R::acc_t* __restrict__ partial) {
+    typename R::acc_t* __restrict__ partial, typename R::param_t prm) {
     using acc_t = typename R::acc_t;
     constexpr int TY = kBlock / kWave;
     __shared__ acc_t sm[TY][kWave];
@@ -312,11 +329,11 @@ __global__ __launch_bounds__(kBlock) void reduce_cols(
 #pragma unroll
                 for (int u = 0; u < 8; ++u) v[u] = load_stream(&p[(j + u * TY) * s]);
 #pragma unroll
-                for (int u = 0; u < 8; ++u) acc = R::join(acc, R::map(v[u], j + u * TY));
+                for (int u = 0; u < 8; ++u) acc = R::join(acc, R::map(v[u], j + u * TY, prm));
             }
-            for (; j < hi; j += TY) acc = R::join(acc, R::map(load_stream(&p[j * s]), j));
+            for (; j < hi; j += TY) acc = R::join(acc, R::map(load_stream(&p[j * s]), j, prm));
         } else {
-            for (int64_t j = lo + ty; j < hi; j += TY) acc = R::join(acc, R::map(p[red.at(j)], j));
+            for (int64_t j = lo + ty; j < hi; j += TY) acc = R::join(acc, R::map(p[red.at(j)], j, prm));
         }
     }
     sm[ty][lx] = acc;
@@ -369,7 +386,8 @@ size_t partial_bound_bytes(int64_t m) {
 
 template <typename R>
 int launch_reduce(hipStream_t stream, const ReducePlan& pl, const typename R::in_t* x,
-                  typename R::out_t* y, int final_op, void* scratch, size_t scratch_bytes) {
+                  typename R::out_t* y, int final_op, void* scratch, size_t scratch_bytes,
+                  typename R::param_t prm = typename R::param_t()) {
     using acc_t = typename R::acc_t;
     using T = typename R::in_t;
     const int64_t m = pl.m, n = pl.n;
@@ -392,7 +410,7 @@ int launch_reduce(hipStream_t stream, const ReducePlan& pl, const typename R::in
         if (parts > 1 && scratch_bytes < static_cast<size_t>(m * parts) * sizeof(acc_t))
             return DLFX_ERR_SCRATCH_TOO_SMALL;
         reduce_cols<R><<<dim3(static_cast<unsigned>(base_blocks * parts)), dim3(kBlock), 0, stream>>>(
-            x, outer, L, pl.red, n, col_blocks, parts, y, pl.ymap, final_op, partial);
+            x, outer, L, pl.red, n, col_blocks, parts, y, pl.ymap, final_op, partial, prm);
         DLFX_CHECK_LAUNCH();
         if (parts > 1) {
             reduce_finalize<R><<<dim3(static_cast<unsigned>(ceil_div(m, kBlock / kWave))), dim3(kBlock), 0, stream>>>(
@@ -411,10 +429,10 @@ int launch_reduce(hipStream_t stream, const ReducePlan& pl, const typename R::in
         if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
         if (contig)
             reduce_rows_group<R, true><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
-                x, pl.kept, pl.red, m, n, log2g, y, pl.ymap, final_op);
+                x, pl.kept, pl.red, m, n, log2g, y, pl.ymap, final_op, prm);
         else
             reduce_rows_group<R, false><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
-                x, pl.kept, pl.red, m, n, log2g, y, pl.ymap, final_op);
+                x, pl.kept, pl.red, m, n, log2g, y, pl.ymap, final_op, prm);
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
     }
@@ -425,10 +443,10 @@ int launch_reduce(hipStream_t stream, const ReducePlan& pl, const typename R::in
         return DLFX_ERR_SCRATCH_TOO_SMALL;
     if (contig)
         reduce_rows_block<R, true><<<dim3(static_cast<unsigned>(m * parts)), dim3(kBlock), 0, stream>>>(
-            x, pl.kept, pl.red, n, parts, y, pl.ymap, final_op, partial);
+            x, pl.kept, pl.red, n, parts, y, pl.ymap, final_op, partial, prm);
     else
         reduce_rows_block<R, false><<<dim3(static_cast<unsigned>(m * parts)), dim3(kBlock), 0, stream>>>(
-            x, pl.kept, pl.red, n, parts, y, pl.ymap, final_op, partial);
+            x, pl.kept, pl.red, n, parts, y, pl.ymap, final_op, partial, prm);
     DLFX_CHECK_LAUNCH();
     if (parts > 1) {
         reduce_finalize<R><<<dim3(static_cast<unsigned>(ceil_div(m, kBlock / kWave))), dim3(kBlock), 0, stream>>>(
@@ -576,5 +594,46 @@ extern "C" int dlfx_arg_reduce(dlfx_stream_t stream, const char* name, int dtype
         int64_t* yp = static_cast<int64_t*>(y) + y_offset;
         if (want_max) return launch_reduce<ArgReducer<T, true, int64_t>>(s, pl, xp, yp, 0, scratch, scratch_bytes);
         return launch_reduce<ArgReducer<T, false, int64_t>>(s, pl, xp, yp, 0, scratch, scratch_bytes);
+    });
+}
+
+extern "C" size_t dlfx_count_scratch_bytes(int dtype, int64_t m, int64_t n) {
+    (void)dtype;
+    (void)n;
+    if (m <= 0) return 0;
+    return partial_bound_bytes(m);
+}
+
+extern "C" int dlfx_count(dlfx_stream_t stream, int dtype, int64_t m, int64_t n, const void* value,
+                          int x_rank, const int64_t* x_dims, const int64_t* x_strides,
+                          const void* x, int64_t x_offset,
+                          int y_rank, const int64_t* y_dims, const int64_t* y_strides,
+                          int32_t* y, int64_t y_offset, void* scratch, size_t scratch_bytes) {
+    if (!value || !x || !y || m <= 0 || n <= 0) return DLFX_ERR_INVALID_ARGUMENT;
+    if (!view_ok(x_rank, x_dims, x_strides) || !view_ok(y_rank, y_dims, y_strides))
+        return DLFX_ERR_INVALID_ARGUMENT;
+    if (view_size(x_rank, x_dims) != m * n || view_size(y_rank, y_dims) != m) return DLFX_ERR_INVALID_ARGUMENT;
+    if (n > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;       // counts are 32-bit, as in the reference
+
+    int split = x_rank;
+    int64_t prod = 1;
+    while (split > 0 && prod < n) prod *= x_dims[--split];
+    if (prod != n) return DLFX_ERR_INVALID_ARGUMENT;
+
+    ReducePlan pl;
+    pl.m = m;
+    pl.n = n;
+    if (!make_dim_map(x_dims, x_strides, 0, split, &pl.kept) ||
+        !make_dim_map(x_dims, x_strides, split, x_rank, &pl.red) ||
+        !make_dim_map(y_dims, y_strides, 0, y_rank, &pl.ymap))
+        return DLFX_ERR_RANK;
+
+    return dispatch_dtype(dtype, [&](auto tag) {
+        using T = decltype(tag);
+        T v;
+        std::memcpy(&v, value, sizeof(T));
+        return launch_reduce<CountReducer<T>>(static_cast<hipStream_t>(stream), pl,
+                                              static_cast<const T*>(x) + x_offset, y + y_offset, kFinalId,
+                                              scratch, scratch_bytes, v);
     });
 }

@@ -117,6 +117,14 @@ __global__ __launch_bounds__(kBlock) void scan_init(unsigned* ticket, int64_t ro
     if (i < tiles) st.clear(i);
 }
 
+// What a scan folds for an input element: the element itself, or (scan_nonzero,
+// gpgpu/include/gdnn.h:131-136) one for every element that is not zero.
+template <typename T, typename X, bool NZ>
+__device__ __forceinline__ T scan_input(X x) {
+    if constexpr (NZ) return x != X(0) ? T(1) : T(0);
+    else return static_cast<T>(x);
+}
+
 // ------------------------------------------------------------------ row kernels
 template <typename T>
 struct RowScanShared {
@@ -128,37 +136,44 @@ struct RowScanShared {
 // One tile: tile `t` of row `row`.  Element order inside a tile: wave w owns
 // [w*64*ITEMS, (w+1)*64*ITEMS); within it, vector k of lane l covers elements
 // (k*64 + l)*V .. +V.  CHAINED tiles publish / look back through `st`.
-template <typename T, int K, int ITEMS, bool CHAINED, bool SELF_HELP, int BLOCK = kBlock>
+template <typename T, int K, int ITEMS, bool CHAINED, bool SELF_HELP, int BLOCK = kBlock, typename X = T, bool NZ = false>
 __device__ __forceinline__ void scan_tile(
-    const T* __restrict__ x, T* __restrict__ y, const DimMap& xmap, const DimMap& ymap, int64_t sx, int64_t sy,
-    int64_t n, int64_t tiles_per_row, int exclusive, int64_t row, int64_t t, int poll_limit,
+    const X* __restrict__ x, T* __restrict__ y, const DimMap& xmap, const DimMap& ymap, int64_t sx, int64_t sy,
+    const DimMap& xaxis, int64_t n, int64_t tiles_per_row, int exclusive, int64_t row, int64_t t, int poll_limit,
     TileState<T>& st, RowScanShared<T>& sm) {
+    // where element i of a row lives: i * sx, or (scan_nonzero over a flattened view whose
+    // dimensions do not merge) wherever the row-major walk of `xaxis` puts it
+    auto x_at = [&](int64_t i) -> int64_t {
+        if constexpr (NZ) return xaxis.at(i);
+        else return i * sx;
+    };
     using Op = ScanOp<T, K>;
     constexpr int V = (vec_width<T>() < ITEMS) ? vec_width<T>() : ITEMS;
     constexpr int KV = ITEMS / V;
     constexpr int64_t TILE = static_cast<int64_t>(BLOCK) * ITEMS;
     using VecT = Vec<T, V>;
+    using VecX = Vec<X, V>;
 
     const int lane = lane_id();
     const int w = threadIdx.x / kWave;
     const int64_t tile_base = t * TILE;
     const int64_t avail = (n - tile_base < TILE) ? n - tile_base : TILE;   // valid elements in this tile
 
-    const T* xr = x + xmap.at(row);
+    const X* xr = x + xmap.at(row);
     T* yr = y + ymap.at(row);
     const int64_t seg = tile_base + static_cast<int64_t>(w) * kWave * ITEMS;
 
     // ---- load
     T vals[ITEMS];
     const bool full = avail == TILE;
-    const bool x_vec = full && sx == 1 && (reinterpret_cast<uintptr_t>(xr + seg) % (sizeof(T) * V) == 0);
+    const bool x_vec = full && sx == 1 && (reinterpret_cast<uintptr_t>(xr + seg) % (sizeof(X) * V) == 0);
     if (x_vec) {
-        const VecT* pv = reinterpret_cast<const VecT*>(xr + seg);
+        const VecX* pv = reinterpret_cast<const VecX*>(xr + seg);
 #pragma unroll
         for (int k = 0; k < KV; ++k) {
-            VecT a = load_stream(&pv[k * kWave + lane]);
+            VecX a = load_stream(&pv[k * kWave + lane]);
 #pragma unroll
-            for (int e = 0; e < V; ++e) vals[k * V + e] = a.v[e];
+            for (int e = 0; e < V; ++e) vals[k * V + e] = scan_input<T, X, NZ>(a.v[e]);
         }
     } else {
 #pragma unroll
@@ -166,7 +181,7 @@ __device__ __forceinline__ void scan_tile(
 #pragma unroll
             for (int e = 0; e < V; ++e) {
                 const int64_t i = seg + static_cast<int64_t>(k * kWave + lane) * V + e;
-                vals[k * V + e] = (i < n) ? xr[i * sx] : Op::identity();
+                vals[k * V + e] = (i < n) ? scan_input<T, X, NZ>(xr[x_at(i)]) : Op::identity();
             }
     }
     // ---- scan inside the wave: vals[] become inclusive prefixes within the wave segment
@@ -233,7 +248,7 @@ __device__ __forceinline__ void scan_tile(
                             const int64_t pbase = (pos - l) * TILE;
                             const int64_t cnt = (n - pbase < TILE) ? n - pbase : TILE;
                             T a = Op::identity();
-                            for (int64_t i = lane; i < cnt; i += kWave) a = Op::apply(a, xr[(pbase + i) * sx]);
+                            for (int64_t i = lane; i < cnt; i += kWave) a = Op::apply(a, scan_input<T, X, NZ>(xr[x_at(pbase + i)]));
                             a = wave_reduce(a, [](T p, T q) { return Op::apply(p, q); });
                             if (lane == l) {
                                 v = a;
@@ -298,22 +313,22 @@ __device__ __forceinline__ void scan_tile(
 }
 
 // Rows of a single tile: workgroup b scans row b.
-template <typename T, int K, int ITEMS>
+template <typename T, int K, int ITEMS, typename X, bool NZ>
 __global__ __launch_bounds__(kBlock) void scan_rows_single(
-    const T* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
+    const X* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy, DimMap xaxis,
     int64_t n, int exclusive) {
     __shared__ RowScanShared<T> sm;
     TileState<T> st;
-    scan_tile<T, K, ITEMS, false, false>(x, y, xmap, ymap, sx, sy, n, 1, exclusive, blockIdx.x, 0, 0, st, sm);
+    scan_tile<T, K, ITEMS, false, false, kBlock, X, NZ>(x, y, xmap, ymap, sx, sy, xaxis, n, 1, exclusive, blockIdx.x, 0, 0, st, sm);
 }
 
 // Rows of several tiles.  Workgroup b belongs to row b / tiles_per_row.  With
 // TICKET the tile of the row is drawn from that row's atomic counter (in-place
 // scans); without, it is the workgroup's position in the row and waits are
 // bounded by self-help.
-template <typename T, int K, int ITEMS, bool TICKET, int BLOCK>
+template <typename T, int K, int ITEMS, bool TICKET, int BLOCK, typename X, bool NZ>
 __global__ __launch_bounds__(BLOCK) void scan_rows_chained(
-    const T* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
+    const X* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy, DimMap xaxis,
     int64_t n, int64_t tiles_per_row, int exclusive, int poll_limit, unsigned* ticket, TileState<T> st) {
     __shared__ RowScanShared<T> sm;
     const int64_t row = blockIdx.x / tiles_per_row;
@@ -323,16 +338,16 @@ __global__ __launch_bounds__(BLOCK) void scan_rows_chained(
         __syncthreads();
         t = sm.next_tile;
     }
-    scan_tile<T, K, ITEMS, true, !TICKET, BLOCK>(x, y, xmap, ymap, sx, sy, n, tiles_per_row, exclusive, row, t, poll_limit, st, sm);
+    scan_tile<T, K, ITEMS, true, !TICKET, BLOCK, X, NZ>(x, y, xmap, ymap, sx, sy, xaxis, n, tiles_per_row, exclusive, row, t, poll_limit, st, sm);
 }
 
 // ------------------------------------------------------------------ column kernel
 // One lane per row ("column"), four waves along the scanned axis.  Each pass of
 // the loop covers kWaves * chunk positions of the axis: thread (lx, ty) scans
 // positions [s + ty*chunk, s + (ty+1)*chunk) in registers.
-template <typename T, int K>
+template <typename T, int K, typename X, bool NZ>
 __global__ __launch_bounds__(kBlock) void scan_cols(
-    const T* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
+    const X* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
     int64_t m, int64_t n, int chunk, int exclusive) {
     using Op = ScanOp<T, K>;
     constexpr int R = 16;
@@ -342,7 +357,7 @@ __global__ __launch_bounds__(kBlock) void scan_cols(
     const int ty = threadIdx.x / kWave;
     const int64_t col = static_cast<int64_t>(blockIdx.x) * kWave + lx;
     const bool live = col < m;
-    const T* xc = x + (live ? xmap.at(col) : 0);
+    const X* xc = x + (live ? xmap.at(col) : 0);
     T* yc = y + (live ? ymap.at(col) : 0);
 
     T carry = Op::identity();
@@ -353,7 +368,7 @@ __global__ __launch_bounds__(kBlock) void scan_cols(
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int64_t p = p0 + r;
-            v[r] = (live && r < chunk && p < n) ? load_stream(&xc[p * sx]) : Op::identity();
+            v[r] = (live && r < chunk && p < n) ? scan_input<T, X, NZ>(load_stream(&xc[p * sx])) : Op::identity();
         }
 #pragma unroll
         for (int r = 1; r < R; ++r) v[r] = Op::apply(v[r - 1], v[r]);
@@ -457,25 +472,42 @@ ScanLayout scan_layout(size_t elem_size, int64_t m, int64_t n) {
     return l;
 }
 
-// True when the element ranges the two views touch intersect.
-template <typename T>
-bool views_overlap(int rank, const int64_t* dims, const T* x, const int64_t* sx, const T* y, const int64_t* sy) {
+// True when the byte ranges the two views touch intersect.
+template <typename X, typename T>
+bool views_overlap(int rank, const int64_t* dims, const X* x, const int64_t* sx, const T* y, const int64_t* sy) {
     int64_t xlo = 0, xhi = 0, ylo = 0, yhi = 0;
     for (int i = 0; i < rank; ++i) {
         const int64_t ex = (dims[i] - 1) * sx[i], ey = (dims[i] - 1) * sy[i];
         if (ex > 0) xhi += ex; else xlo += ex;
         if (ey > 0) yhi += ey; else ylo += ey;
     }
-    return !(x + xhi < y + ylo || y + yhi < x + xlo);
+    const char* xb = reinterpret_cast<const char*>(x + xlo);
+    const char* xe = reinterpret_cast<const char*>(x + xhi + 1);
+    const char* yb = reinterpret_cast<const char*>(y + ylo);
+    const char* ye = reinterpret_cast<const char*>(y + yhi + 1);
+    return xb < ye && yb < xe;
 }
 
-template <typename T, int K>
+template <typename T, int K, typename X = T, bool NZ = false>
 int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int rank, const int64_t* dims,
-                const T* x, const int64_t* x_strides, T* y, const int64_t* y_strides,
-                void* scratch, size_t scratch_bytes) {
+                const X* x, const int64_t* x_strides, T* y, const int64_t* y_strides,
+                void* scratch, size_t scratch_bytes, const DimMap* x_axis = nullptr) {
     DimMap xmap, ymap;
     if (!make_dim_map2(dims, x_strides, y_strides, rank - 1, &xmap, &ymap)) return DLFX_ERR_RANK;
-    const int64_t sx = rank ? x_strides[rank - 1] : 1;
+    DimMap xaxis;
+    if (x_axis) {
+        xaxis = *x_axis;
+    } else {
+        const int64_t one_dim[1] = {n}, one_stride[1] = {rank ? x_strides[rank - 1] : 1};
+        make_dim_map(one_dim, one_stride, 0, 1, &xaxis);
+        if (xaxis.rank == 0) {          // n == 1
+            xaxis.rank = 1;
+            xaxis.dims[0] = 1;
+            xaxis.strides[0] = one_stride[0];
+        }
+    }
+    const bool axis_general = xaxis.rank > 1;
+    const int64_t sx = axis_general ? 0 : xaxis.strides[0];
     const int64_t sy = rank ? y_strides[rank - 1] : 1;
 
     // Many rows with a contiguous kept axis and a strided scanned axis: column kernel.
@@ -483,12 +515,12 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     const bool inner_unit = xmap.rank >= 1 && xmap.strides[xmap.rank - 1] == 1 && ymap.strides[ymap.rank - 1] == 1 &&
                             xmap.dims[xmap.rank - 1] >= 16;
     const bool short_rows = n <= 64 && m >= 256;
-    const bool use_cols = short_rows || (!axis_unit && m >= 64 && (inner_unit || n < 4096));
+    const bool use_cols = !axis_general && (short_rows || (!axis_unit && m >= 64 && (inner_unit || n < 4096)));
     if (use_cols) {
         int chunk = static_cast<int>(ceil_div(n, kWaves) < 16 ? ceil_div(n, kWaves) : 16);
         const int64_t blocks = ceil_div(m, kWave);
         if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
-        scan_cols<T, K><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
+        scan_cols<T, K, X, NZ><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
             x, y, xmap, ymap, sx, sy, m, n, chunk, exclusive);
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
@@ -503,13 +535,13 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     if (l.tiles_per_row == 1) {
         const dim3 grid(static_cast<unsigned>(m));
         if (tile == 256)
-            scan_rows_single<T, K, 1><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, n, exclusive);
+            scan_rows_single<T, K, 1, X, NZ><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
         else if (tile == 1024)
-            scan_rows_single<T, K, 4><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, n, exclusive);
+            scan_rows_single<T, K, 4, X, NZ><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
         else if (tile == 256 * (FULL / 4))
-            scan_rows_single<T, K, FULL / 4><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, n, exclusive);
+            scan_rows_single<T, K, FULL / 4, X, NZ><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
         else
-            scan_rows_single<T, K, FULL><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, n, exclusive);
+            scan_rows_single<T, K, FULL, X, NZ><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
     }
@@ -522,11 +554,11 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     constexpr int CI = static_cast<int>(kChainTileBytes / sizeof(T) / kChainBlock);
     const dim3 cblock(kChainBlock);
     if (views_overlap(rank, dims, x, x_strides, y, y_strides))
-        scan_rows_chained<T, K, CI, true, kChainBlock><<<grid, cblock, 0, stream>>>(
-            x, y, xmap, ymap, sx, sy, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st);
+        scan_rows_chained<T, K, CI, true, kChainBlock, X, NZ><<<grid, cblock, 0, stream>>>(
+            x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st);
     else
-        scan_rows_chained<T, K, CI, false, kChainBlock><<<grid, cblock, 0, stream>>>(
-            x, y, xmap, ymap, sx, sy, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st);
+        scan_rows_chained<T, K, CI, false, kChainBlock, X, NZ><<<grid, cblock, 0, stream>>>(
+            x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st);
     DLFX_CHECK_LAUNCH();
     return DLFX_OK;
 }
@@ -577,5 +609,52 @@ extern "C" int dlfx_scan(dlfx_stream_t stream, const char* name, int dtype, int6
         case kScanMax: return launch_scan<T, kScanMax>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
         default:       return launch_scan<T, kScanMin>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
         }
+    });
+}
+
+extern "C" size_t dlfx_scan_nonzero_scratch_bytes(int dtype, int64_t m, int64_t n) {
+    if (!dtype_size(dtype) || m <= 0 || n <= 0) return 0;
+    return scan_layout(4, m, n).total;
+}
+
+extern "C" int dlfx_scan_nonzero(dlfx_stream_t stream, int dtype, int64_t m, int64_t n,
+                                 int exclusive, int rank, const int64_t* dims,
+                                 const void* x, int64_t x_offset, const int64_t* x_strides,
+                                 int32_t* y, int64_t y_offset, const int64_t* y_strides,
+                                 void* scratch, size_t scratch_bytes) {
+    if (!x || !y || m <= 0 || n <= 0) return DLFX_ERR_INVALID_ARGUMENT;
+    if (!view_ok(rank, dims, x_strides) || !view_ok(rank, dims, y_strides)) return DLFX_ERR_INVALID_ARGUMENT;
+    if (rank < 1 || rank > 64 || view_size(rank, dims) != m * n) return DLFX_ERR_INVALID_ARGUMENT;
+    if (n > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;       // counts are 32-bit, as in the reference
+    // the scanned elements are the trailing dimensions whose product is n, walked in row-major
+    // order (nonzero() scans a whole tensor as one row: reduce.h:426-429)
+    int split = rank;
+    int64_t prod = 1;
+    while (split > 0 && prod < n) prod *= dims[--split];
+    if (prod != n) return DLFX_ERR_INVALID_ARGUMENT;
+    if (split == rank) split = rank - 1;                   // n == 1
+    DimMap xaxis, yaxis;
+    if (!make_dim_map(dims, x_strides, split, rank, &xaxis) || !make_dim_map(dims, y_strides, split, rank, &yaxis))
+        return DLFX_ERR_RANK;
+    if (yaxis.rank > 1) return DLFX_ERR_RANK;              // the counts must be walked with one stride
+    if (xaxis.rank == 0) {
+        xaxis.rank = 1;
+        xaxis.dims[0] = 1;
+        xaxis.strides[0] = 1;
+    }
+    int64_t d2[64], xs2[64], ys2[64];
+    for (int i = 0; i < split; ++i) {
+        d2[i] = dims[i];
+        xs2[i] = x_strides[i];
+        ys2[i] = y_strides[i];
+    }
+    d2[split] = n;
+    xs2[split] = xaxis.rank == 1 ? xaxis.strides[0] : 0;
+    ys2[split] = yaxis.rank == 1 ? yaxis.strides[0] : 1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dispatch_dtype(dtype, [&](auto tag) {
+        using X = decltype(tag);
+        return launch_scan<int32_t, kScanAdd, X, true>(s, m, n, exclusive, split + 1, d2, static_cast<const X*>(x) + x_offset,
+                                                       xs2, y + y_offset, ys2, scratch, scratch_bytes, &xaxis);
     });
 }

@@ -32,7 +32,6 @@ namespace {
 #define DLFX_SORT_WAVES 4
 #endif
 constexpr int kBlock = 256;
-constexpr int kWaves = kBlock / kWave;
 #ifndef DLFX_SORT_PASS_BLOCK
 #define DLFX_SORT_PASS_BLOCK 256
 #endif

@@ -129,6 +129,39 @@ def reduce(name: str, X: Tensor, axes: Sequence[int] = (), keepdims: bool = Fals
     return Y
 
 
+def count(X: Tensor, value, axes: Sequence[int] = (), keepdims: bool = False) -> Tensor:
+    """Number of elements equal to `value` over `axes` (reduce.h:160-198); int32 result."""
+    if isinstance(axes, int):
+        axes = [axes]
+    view, out_dims, m, n = prepare_reduce(X.shape, list(axes), keepdims)
+    Y = Tensor.empty(X.backend, out_dims, np.int32)
+    X.backend.count(dtype_code(X.dtype), m, n, value, view, X.storage, Y.shape, Y.storage)
+    return Y
+
+
+def nonzero(X: Tensor, row_major: bool = False) -> Optional[Tensor]:
+    """Coordinates of the non-zero elements (reduce.h:419-450): an [n, rank] int32 tensor, or
+    [rank, n] when row_major; None when there is none (the reference clears the output)."""
+    size = X.size
+    counts = Tensor.empty(X.backend, [size], np.int32)
+    counts_shape = Shape(X.shape.extents)           # contiguous, the input's extents
+    X.backend.scan_nonzero(dtype_code(X.dtype), 1, size, False,
+                           _as_row(X.shape), X.storage, _as_row(counts_shape), counts.storage)
+    n = int(X.backend.read_element(counts.storage, size - 1))
+    if n == 0:
+        return None
+    rank = X.rank
+    Y = Tensor.empty(X.backend, [rank, n] if row_major else [n, rank], np.int32)
+    X.backend.gather_indices(size, n, row_major, list(X.shape.extents), counts.storage, Y.storage)
+    return Y
+
+
+def _as_row(shape: Shape) -> Shape:
+    """The view itself: scan_nonzero(1, size, ...) walks all of it as one row, in row-major
+    order of the extents, which is how the reference passes it (reduce.h:426-429)."""
+    return shape
+
+
 def _make_reduce(name):
     def f(X: Tensor, axes: Sequence[int] = (), keepdims: bool = False) -> Tensor:
         return reduce(name, X, axes, keepdims)

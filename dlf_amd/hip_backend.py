@@ -69,6 +69,21 @@ def _declare(lib):
     lib.dlfx_top_k.argtypes = [c_void_p, c_int64, c_int, c_int, c_int, c_int, _I64P, _I64P,
                                c_void_p, c_int64, _I64P, c_void_p, c_int64, _I64P,
                                c_void_p, c_int64, _I64P, c_void_p, c_size_t]
+    lib.dlfx_count_scratch_bytes.restype = c_size_t
+    lib.dlfx_count_scratch_bytes.argtypes = [c_int, c_int64, c_int64]
+    lib.dlfx_count.restype = c_int
+    lib.dlfx_count.argtypes = ([c_void_p, c_int, c_int64, c_int64, c_void_p] + view + [c_void_p, c_int64]
+                               + view + [c_void_p, c_int64, c_void_p, c_size_t])
+
+    lib.dlfx_scan_nonzero_scratch_bytes.restype = c_size_t
+    lib.dlfx_scan_nonzero_scratch_bytes.argtypes = [c_int, c_int64, c_int64]
+    lib.dlfx_scan_nonzero.restype = c_int
+    lib.dlfx_scan_nonzero.argtypes = [c_void_p, c_int, c_int64, c_int64, c_int, c_int, _I64P,
+                                      c_void_p, c_int64, _I64P, c_void_p, c_int64, _I64P, c_void_p, c_size_t]
+
+    lib.dlfx_gather_indices.restype = c_int
+    lib.dlfx_gather_indices.argtypes = [c_void_p, c_int64, c_int64, c_int, c_int, _I64P,
+                                        c_void_p, c_int64, c_void_p, c_int64]
     return lib
 
 
@@ -81,7 +96,9 @@ EXPORTS = ("dlfx_version", "dlfx_status_string", "dlfx_last_hip_error", "dlfx_se
            "dlfx_scan_scratch_bytes", "dlfx_scan",
            "dlfx_sort_scratch_bytes", "dlfx_sort",
            "dlfx_argsort_scratch_bytes", "dlfx_argsort",
-           "dlfx_top_k_scratch_bytes", "dlfx_top_k")
+           "dlfx_top_k_scratch_bytes", "dlfx_top_k",
+           "dlfx_count_scratch_bytes", "dlfx_count",
+           "dlfx_scan_nonzero_scratch_bytes", "dlfx_scan_nonzero", "dlfx_gather_indices")
 
 
 def load_library():
@@ -223,6 +240,31 @@ class HipBackend:
                             x.data_ptr(), xs.offset, _arr(xs.strides),
                             y.data_ptr(), ys.offset, _arr(ys.strides),
                             i.data_ptr(), is_.offset, _arr(is_.strides), sp, sb), defer)
+
+    def count(self, dtype, m, n, value, xs, x, ys, y, defer=False):
+        sp, sb = self.scratch(self.lib.dlfx_count_scratch_bytes(dtype, m, n))
+        v = np.array([value], dtype=(np.float32, np.float64, np.int32, np.int64)[dtype])   # one host element of the input's type
+        keep = v.ctypes.data_as(c_void_p)
+        call = self._issue(self.lib.dlfx_count, "dlfx_count", (dtype, m, n, keep),
+                           (xs.rank, _arr(xs.extents), _arr(xs.strides), x.data_ptr(), xs.offset,
+                            ys.rank, _arr(ys.extents), _arr(ys.strides), y.data_ptr(), ys.offset, sp, sb), defer)
+        if call is None:
+            return None
+        return lambda v=v: call()      # the closure keeps the host value alive
+
+    def scan_nonzero(self, dtype, m, n, exclusive, xs, x, ys, y, defer=False):
+        sp, sb = self.scratch(self.lib.dlfx_scan_nonzero_scratch_bytes(dtype, m, n))
+        return self._issue(self.lib.dlfx_scan_nonzero, "dlfx_scan_nonzero", (dtype, m, n, int(bool(exclusive))),
+                           (xs.rank, _arr(xs.extents), x.data_ptr(), xs.offset, _arr(xs.strides),
+                            y.data_ptr(), ys.offset, _arr(ys.strides), sp, sb), defer)
+
+    def gather_indices(self, m, n, row_major, dims, counts, out, defer=False):
+        return self._issue(self.lib.dlfx_gather_indices, "dlfx_gather_indices", (m, n, int(bool(row_major))),
+                           (len(dims), _arr(dims), counts.data_ptr(), 0, out.data_ptr(), 0), defer)
+
+    def read_element(self, storage, index):
+        """One element of a device buffer on the host (synchronises the stream)."""
+        return storage[index].item()
 
     def set_tuning(self, key: str, value: int):
         _check(self.lib.dlfx_set_tuning(key.encode(), value), "dlfx_set_tuning(%s)" % key)

@@ -171,6 +171,12 @@ public:
         if (!data_ || data_.size() < shape.size()) data_ = gpgpu::Buffer<T>(shape.size());
         shape_ = Shape(shape.extents());
     }
+    // Drops the storage; the tensor is empty afterwards (device.h: DevTensor::clear).
+    void clear() {
+        data_ = gpgpu::Buffer<T>();
+        shape_ = Shape();
+    }
+    bool empty() const noexcept { return !data_; }
     DevTensor view(Shape shape) const { return DevTensor(std::move(shape), data_); }
     DevTensor transpose() const { return view(shape_.transpose()); }
     DevTensor transpose(const std::vector<size_t>& perm) const { return view(shape_.transpose(perm)); }
@@ -262,6 +268,51 @@ DLF_DEFINE_REDUCE_OP(reduce_sum_exp)
 DLF_DEFINE_REDUCE_OP(reduce_log_sum_exp)
 DLF_DEFINE_REDUCE_OP(reduce_prod)
 #undef DLF_DEFINE_REDUCE_OP
+
+// ---------------------------------------------------------------- count / nonzero
+// dlf/include/tensor/reduce.h:160-198
+template <typename T>
+void count(const DevTensor<T>& X, DevTensor<int>& Y, const T& value, std::vector<int> axes = {}, bool keepdims = false) {
+    size_t m, n;
+    DevTensor<T> shape_only;       // prepare_reduce sizes an output of X's type; only its shape is used
+    const Shape xs = detail::prepare_reduce(X, shape_only, std::move(axes), keepdims, &m, &n);
+    Y.resize(shape_only.shape());
+    gpgpu::dnn::count(m, n, value, xs.extents(), xs.strides(), X.data(), xs.offset(),
+                      Y.shape().extents(), Y.shape().strides(), Y.data(), Y.shape().offset());
+}
+template <typename T>
+inline DevTensor<int> count(const DevTensor<T>& X, const T& value, std::vector<int> axes = {}, bool keepdims = false) {
+    DevTensor<int> Y;
+    count(X, Y, value, std::move(axes), keepdims);
+    return Y;
+}
+
+// dlf/include/tensor/reduce.h:419-450: running count of the non-zero elements of the whole
+// tensor, one read of the total, then the coordinates.  Y becomes [n, rank], or [rank, n] when
+// row_major; an input without non-zero elements leaves Y empty.
+template <typename T>
+void nonzero(const DevTensor<T>& X, DevTensor<int32_t>& Y, bool row_major = false) {
+    auto counts = gpgpu::current::context().getTemporaryBuffer<int32_t>(X.size());
+    const Shape counts_shape(X.shape().extents());
+    gpgpu::dnn::scan_nonzero(1, X.size(), false, X.shape().extents(), X.data(), X.shape().offset(), X.shape().strides(),
+                             counts, counts.offset(), counts_shape.strides());
+    int32_t n = 0;
+    counts.read(gpgpu::current::queue(), &n, 1, counts.offset() + X.size() - 1);
+    if (n == 0) {
+        Y.clear();
+        return;
+    }
+    if (row_major) Y.resize(Shape({X.rank(), static_cast<size_t>(n)}));
+    else Y.resize(Shape({static_cast<size_t>(n), X.rank()}));
+    gpgpu::dnn::gather_indices(X.size(), n, row_major, X.shape().extents(), counts, counts.offset(),
+                               Y.data(), Y.shape().offset());
+}
+template <typename T>
+inline DevTensor<int32_t> nonzero(const DevTensor<T>& X, bool row_major = false) {
+    DevTensor<int32_t> Y;
+    nonzero(X, Y, row_major);
+    return Y;
+}
 
 // ---------------------------------------------------------------- argmax / argmin
 namespace detail {

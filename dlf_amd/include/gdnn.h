@@ -175,4 +175,56 @@ void top_k(const size_t limit, const int dir,
     ev.done();
 }
 
+// gpgpu/include/gdnn.h:116-122
+template <typename T>
+void count(const size_t m, const size_t n, const T value,
+           const std::vector<size_t>& x_dims, const std::vector<size_t>& x_strides,
+           const Buffer<T>& x_buffer, const size_t x_offset,
+           const std::vector<size_t>& y_dims, const std::vector<size_t>& y_strides,
+           Buffer<int>& y_buffer, const size_t y_offset,
+           const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    const int dt = detail::dtype_of<T>::value;
+    auto xd = detail::signed_vec(x_dims), xs = detail::signed_vec(x_strides);
+    auto yd = detail::signed_vec(y_dims), ys = detail::signed_vec(y_strides);
+    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_count_scratch_bytes(dt, m, n));
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_count(queue.stream(), dt, m, n, &value,
+                            static_cast<int>(xd.size()), xd.data(), xs.data(), x_buffer.data(), x_offset,
+                            static_cast<int>(yd.size()), yd.data(), ys.data(), y_buffer.data(), y_offset,
+                            tmp.bytes(), tmp.byte_size()), "gpgpu::dnn::count");
+    ev.done();
+}
+
+// gpgpu/include/gdnn.h:131-136
+template <typename T>
+void scan_nonzero(const size_t m, const size_t n,
+                  const bool exclusive, const std::vector<size_t>& dims,
+                  const Buffer<T>& x_buffer, const size_t x_offset, const std::vector<size_t>& x_strides,
+                  Buffer<int32_t>& y_buffer, const size_t y_offset, const std::vector<size_t>& y_strides,
+                  const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    const int dt = detail::dtype_of<T>::value;
+    auto d = detail::signed_vec(dims), xs = detail::signed_vec(x_strides), ys = detail::signed_vec(y_strides);
+    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_scan_nonzero_scratch_bytes(dt, m, n));
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_scan_nonzero(queue.stream(), dt, m, n, exclusive ? 1 : 0,
+                                   static_cast<int>(d.size()), d.data(), x_buffer.data(), x_offset, xs.data(),
+                                   y_buffer.data(), y_offset, ys.data(), tmp.bytes(), tmp.byte_size()),
+                 "gpgpu::dnn::scan_nonzero");
+    ev.done();
+}
+
+// gpgpu/include/gdnn.h:328-332
+inline void gather_indices(const size_t m, const size_t n, const bool row_major,
+                           const std::vector<size_t>& dims,
+                           const Buffer<int32_t>& indices, const size_t indices_offset,
+                           Buffer<int32_t>& output, const size_t output_offset,
+                           const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    auto d = detail::signed_vec(dims);
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_gather_indices(queue.stream(), m, n, row_major ? 1 : 0, static_cast<int>(d.size()), d.data(),
+                                     indices.data(), indices_offset, output.data(), output_offset),
+                 "gpgpu::dnn::gather_indices");
+    ev.done();
+}
+
 }}  // namespace gpgpu::dnn

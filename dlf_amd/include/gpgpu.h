@@ -151,14 +151,17 @@ public:
 template <typename T>
 class TemporaryBuffer : public Buffer<T> {
     Context* ctx_ = nullptr;
-    size_t bytes_begin_ = 0, bytes_end_ = 0;
+    size_t bytes_begin_ = 0, bytes_end_ = 0, prev_top_ = 0;   // prev_top_: the arena's top before this allocation
 public:
-    TemporaryBuffer(Context* ctx, std::shared_ptr<void> mem, size_t size, size_t byte_begin, size_t byte_end)
-        : Buffer<T>(std::move(mem), size, byte_begin / sizeof(T)), ctx_(ctx), bytes_begin_(byte_begin), bytes_end_(byte_end) {}
+    TemporaryBuffer(Context* ctx, std::shared_ptr<void> mem, size_t size, size_t byte_begin, size_t byte_end, size_t prev_top)
+        : Buffer<T>(std::move(mem), size, byte_begin / sizeof(T)), ctx_(ctx), bytes_begin_(byte_begin), bytes_end_(byte_end),
+          prev_top_(prev_top) {}
     TemporaryBuffer(const TemporaryBuffer&) = delete;
     TemporaryBuffer& operator=(const TemporaryBuffer&) = delete;
     TemporaryBuffer(TemporaryBuffer&& o) noexcept
-        : Buffer<T>(std::move(o)), ctx_(o.ctx_), bytes_begin_(o.bytes_begin_), bytes_end_(o.bytes_end_) { o.ctx_ = nullptr; }
+        : Buffer<T>(std::move(o)), ctx_(o.ctx_), bytes_begin_(o.bytes_begin_), bytes_end_(o.bytes_end_), prev_top_(o.prev_top_) {
+        o.ctx_ = nullptr;
+    }
     ~TemporaryBuffer() noexcept(false);
     void* bytes() const noexcept { return static_cast<char*>(this->mem_.get()) + bytes_begin_; }
     size_t byte_size() const noexcept { return bytes_end_ - bytes_begin_; }
@@ -172,9 +175,9 @@ class Context {
     std::vector<std::shared_ptr<void>> retired_;   // arenas outgrown while temporaries were live
     template <typename T> friend class TemporaryBuffer;
 
-    void release(size_t begin, size_t end) {
+    void release(size_t prev_top, size_t end) {
         if (end != top_) throw LogicError("TemporaryBuffer: released out of order");
-        top_ = begin;
+        top_ = prev_top;
         if (top_ == 0) retired_.clear();
     }
 public:
@@ -184,6 +187,7 @@ public:
     template <typename T>
     TemporaryBuffer<T> getTemporaryBuffer(size_t size) {
         const size_t align = 256;
+        const size_t prev_top = top_;
         const size_t begin = (top_ + align - 1) / align * align;
         const size_t end = begin + (size ? size : 1) * sizeof(T);
         if (end > capacity_) {
@@ -197,13 +201,13 @@ public:
             capacity_ = cap;
         }
         top_ = end;
-        return TemporaryBuffer<T>(this, arena_, size, begin, end);
+        return TemporaryBuffer<T>(this, arena_, size, begin, end, prev_top);
     }
 };
 
 template <typename T>
 TemporaryBuffer<T>::~TemporaryBuffer() noexcept(false) {
-    if (ctx_) ctx_->release(bytes_begin_, bytes_end_);
+    if (ctx_) ctx_->release(prev_top_, bytes_end_);
 }
 
 // ---------------------------------------------------------------- thread-local current objects

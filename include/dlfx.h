@@ -167,6 +167,43 @@ int dlfx_top_k(dlfx_stream_t stream, int64_t limit, int dir, int dtype, int inde
                void* idx, int64_t i_offset, const int64_t* i_strides,
                void* scratch, size_t scratch_bytes);
 
+/* ---------------------------------------------------------------- count
+ * Replaces gpgpu::dnn::count<T> (gdnn.h:116-122; caller reduce.h:160-175): the number of
+ * elements of each row that equal *value.  Views as for dlfx_reduce (kept dims then reduced
+ * dims); y holds 32-bit counts.  `value` points to one element of `dtype` in host memory.
+ */
+size_t dlfx_count_scratch_bytes(int dtype, int64_t m, int64_t n);
+int dlfx_count(dlfx_stream_t stream, int dtype, int64_t m, int64_t n, const void* value,
+               int x_rank, const int64_t* x_dims, const int64_t* x_strides,
+               const void* x, int64_t x_offset,
+               int y_rank, const int64_t* y_dims, const int64_t* y_strides,
+               int32_t* y, int64_t y_offset,
+               void* scratch, size_t scratch_bytes);
+
+/* ---------------------------------------------------------------- scan_nonzero
+ * Replaces gpgpu::dnn::scan_nonzero<T> (gdnn.h:131-136; caller reduce.h:426-429): running
+ * count of the elements that are not zero along the last axis, as 32-bit integers.  Views as
+ * for dlfx_scan.
+ */
+size_t dlfx_scan_nonzero_scratch_bytes(int dtype, int64_t m, int64_t n);
+int dlfx_scan_nonzero(dlfx_stream_t stream, int dtype, int64_t m, int64_t n,
+                      int exclusive, int rank, const int64_t* dims,
+                      const void* x, int64_t x_offset, const int64_t* x_strides,
+                      int32_t* y, int64_t y_offset, const int64_t* y_strides,
+                      void* scratch, size_t scratch_bytes);
+
+/* ---------------------------------------------------------------- gather_indices
+ * Replaces gpgpu::dnn::gather_indices (gdnn.h:328-332; caller reduce.h:446-449): `indices`
+ * holds the inclusive running count of non-zero elements over the m elements of a tensor of
+ * extents `dims` in row-major order, n is the total.  For every element that raised the
+ * count, its coordinates are written to column (count - 1) of a [rank, n] matrix
+ * (row_major) or to row (count - 1) of an [n, rank] matrix.
+ */
+int dlfx_gather_indices(dlfx_stream_t stream, int64_t m, int64_t n, int row_major,
+                        int rank, const int64_t* dims,
+                        const int32_t* indices, int64_t indices_offset,
+                        int32_t* output, int64_t output_offset);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

@@ -681,4 +681,75 @@ int dlf_oracle_top_k(int mode, int64_t limit, int largest, int sorted, int dtype
     });
 }
 
+// count (dlf/include/tensor/reduce.h:151-158): reduce with identity 0, Map x == value ? 1 : 0,
+// fold +, over the permuted view that prepare_reduce builds; integer addition, so the order
+// of the fold does not matter.
+int dlf_oracle_count(int dtype, int64_t m, int64_t n, const void* value,
+                     int x_rank, const int64_t* x_dims, const int64_t* x_strides,
+                     const void* x, int64_t x_offset,
+                     int y_rank, const int64_t* y_dims, const int64_t* y_strides,
+                     int32_t* y, int64_t y_offset) {
+    View xv(x_rank, x_dims, x_strides, x_offset), yv(y_rank, y_dims, y_strides, y_offset);
+    return by_dtype(dtype, [&](auto tag) {
+        using T = decltype(tag);
+        T v;
+        std::memcpy(&v, value, sizeof(T));
+        const T* xp = static_cast<const T*>(x);
+#pragma omp parallel for schedule(static)
+        for (int64_t i = 0; i < m; ++i) {
+            int32_t acc = 0;
+            for (int64_t j = 0; j < n; ++j) acc += xp[xv.at(i * n + j)] == v ? 1 : 0;
+            y[yv.at(i)] = acc;
+        }
+        return 0;
+    });
+}
+
+// First half of nonzero() (dlf/include/tensor/reduce.h:383-386): indices = (x != 0), then
+// cumsum(indices, indices) along the last axis.
+int dlf_oracle_scan_nonzero(int dtype, int64_t m, int64_t n, int exclusive,
+                            int rank, const int64_t* dims,
+                            const void* x, int64_t x_offset, const int64_t* x_strides,
+                            int32_t* y, int64_t y_offset, const int64_t* y_strides) {
+    View xv(rank, dims, x_strides, x_offset), yv(rank, dims, y_strides, y_offset);
+    return by_dtype(dtype, [&](auto tag) {
+        using T = decltype(tag);
+        const T* xp = static_cast<const T*>(x);
+        for (int64_t i = 0; i < m; ++i) {
+            int32_t acc = 0;
+            for (int64_t j = 0; j < n; ++j) {
+                const int32_t flag = xp[xv.at(i * n + j)] != T(0) ? 1 : 0;
+                if (exclusive) {
+                    y[yv.at(i * n + j)] = acc;
+                    acc += flag;
+                } else {
+                    acc += flag;
+                    y[yv.at(i * n + j)] = acc;
+                }
+            }
+        }
+        return 0;
+    });
+}
+
+// Second half of nonzero() (dlf/include/tensor/reduce.h:404-417): for every element i whose
+// running count differs from its predecessor's, the coordinates of flat index i go to column
+// prev of a [rank, n] matrix (row_major) or to row prev of an [n, rank] matrix.
+int dlf_oracle_gather_indices(int64_t m, int64_t n, int row_major, int rank, const int64_t* dims,
+                              const int32_t* idx, int32_t* out) {
+    for (int64_t i = 0; i < m; ++i) {
+        const int32_t curr = idx[i];
+        const int32_t prev = i == 0 ? 0 : idx[i - 1];
+        if (curr != prev) {
+            int64_t temp = i;
+            for (int j = rank; --j >= 0;) {
+                const int64_t id = row_major ? (n * j + prev) : (static_cast<int64_t>(prev) * rank + j);
+                out[id] = static_cast<int32_t>(temp % dims[j]);
+                temp /= dims[j];
+            }
+        }
+    }
+    return 0;
+}
+
 }  // extern "C"

@@ -116,6 +116,27 @@ class OracleBackend:
             _ptr(y), c_int64(ys.offset), _arr(ys.strides),
             _ptr(i), c_int64(is_.offset), _arr(is_.strides), c_int(i.dtype.itemsize)), "oracle top_k")
 
+    def count(self, dtype, m, n, value, xs, x, ys, y):
+        v = np.array([value], dtype=x.dtype)
+        _check(self.lib.dlf_oracle_count(
+            c_int(dtype), c_int64(m), c_int64(n), _ptr(v),
+            c_int(xs.rank), _arr(xs.extents), _arr(xs.strides), _ptr(x), c_int64(xs.offset),
+            c_int(ys.rank), _arr(ys.extents), _arr(ys.strides), _ptr(y), c_int64(ys.offset)), "oracle count")
+
+    def scan_nonzero(self, dtype, m, n, exclusive, xs, x, ys, y):
+        _check(self.lib.dlf_oracle_scan_nonzero(
+            c_int(dtype), c_int64(m), c_int64(n), c_int(int(bool(exclusive))),
+            c_int(xs.rank), _arr(xs.extents), _ptr(x), c_int64(xs.offset), _arr(xs.strides),
+            _ptr(y), c_int64(ys.offset), _arr(ys.strides)), "oracle scan_nonzero")
+
+    def gather_indices(self, m, n, row_major, dims, counts, out):
+        _check(self.lib.dlf_oracle_gather_indices(
+            c_int64(m), c_int64(n), c_int(int(bool(row_major))), c_int(len(dims)), _arr(dims),
+            _ptr(counts), _ptr(out)), "oracle gather_indices")
+
+    def read_element(self, storage, index):
+        return storage[index]
+
     def synchronize(self):
         pass
 

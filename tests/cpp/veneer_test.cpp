@@ -5,7 +5,8 @@
 //
 // Vectors: dlf/test/UniformTest.cpp:1857-1965 (reduce), :2106-2189 (scan),
 // :2304-2377 (sort), dlf/test/DNNTest.cpp:861-1019 (argmax/argmin),
-// dlf/test/model/PredictTest.cpp:609-637 (top_k).
+// dlf/test/model/PredictTest.cpp:609-637 (top_k), dlf/test/UniformTest.cpp:2065-2080
+// (count) and :2553-2561 (nonzero).
 #include <cmath>
 #include <cstdio>
 #include <random>
@@ -160,6 +161,24 @@ static void test_top_k() {
     CHECK(top_k(dev(T), 4).second.read() == Tensor<int32_t>({1, 4}, {1, 3, 5, 0}));   // lowest index first among ties
 }
 
+static void test_count_nonzero() {
+    auto A = Tensor<float>({3, 3}, {1, 0, 3, 0, 2, 4, 0, 0, 3});
+    auto dA = dev(A);
+    CHECK(count(dA, 0.0f, {0}).read() == Tensor<int>({3}, {2, 2, 0}));
+    CHECK(count(dA, 0.0f, {1}).read() == Tensor<int>({3}, {1, 1, 2}));
+    CHECK(count(dA, 0.0f).read() == Tensor<int>(Shape(std::vector<size_t>{}), {4}));
+    CHECK(count(dA.transpose(), 0.0f, {1}).read() == Tensor<int>({3}, {2, 2, 0}));
+
+    auto X = Tensor<float>({2, 2, 2}, {1, 0, 0, 2, 5, 6, 0, 0});
+    auto Y = Tensor<int32_t>({3, 4}, {0, 0, 1, 1, 0, 1, 0, 0, 0, 1, 0, 1});
+    CHECK(nonzero(dev(X), true).read() == Y);
+    CHECK(nonzero(dev(X)).transpose().read() == Y);
+    CHECK(nonzero(dev(Tensor<float>({2, 2}, {0, 0, 0, 0}))).empty());
+    // a transposed input is walked in the row-major order of the view
+    auto Xt = dev(Tensor<int64_t>({2, 3}, {0, 7, 0, 8, 0, 9})).transpose();
+    CHECK(nonzero(Xt).read() == Tensor<int32_t>({3, 2}, {0, 1, 1, 0, 2, 1}));
+}
+
 static void test_errors_and_temporaries() {
     auto X = dev(Tensor<float>({2, 3}).range());
     bool threw = false;
@@ -181,6 +200,14 @@ static void test_errors_and_temporaries() {
         delete b;
     }
     CHECK(threw);
+    // nested temporaries of odd sizes release cleanly in stack order
+    threw = false;
+    try {
+        auto outer = ctx.getTemporaryBuffer<int32_t>(7);
+        { auto inner = ctx.getTemporaryBuffer<char>(0); }
+        { auto inner = ctx.getTemporaryBuffer<double>(3); auto innermost = ctx.getTemporaryBuffer<char>(5); }
+    } catch (const gpgpu::LogicError&) { threw = true; }
+    CHECK(!threw);
     // event timing brackets a call
     gpgpu::Event ev;
     auto big = DevTensor<float>(Shape({64, 1 << 16}));
@@ -197,6 +224,7 @@ int main() {
     test_scan();
     test_sort();
     test_top_k();
+    test_count_nonzero();
     test_errors_and_temporaries();
     std::printf("veneer_test: %d checks, %d failed\n", g_checked, g_failed);
     return g_failed ? 1 : 0;

@@ -50,6 +50,12 @@ def run_golden_case(backend, case):
         elif op == "top_k":
             y, i = F.top_k(X, call["k"], call["axis"], call["largest"])
             outs = [(y, call["y_shape"], call["y"]), (i, call["y_shape"], call["i"])]
+        elif op == "count":
+            got = F.count(X, call["value"], call["axes"], call["keepdims"])
+            outs = [(got, call["y_shape"], call["y"])]
+        elif op == "nonzero":
+            got = F.nonzero(X, call["row_major"])
+            outs = [(got, call["y_shape"], call["y"])]
         else:
             raise AssertionError("unknown op " + op)
         backend.synchronize()

@@ -198,3 +198,34 @@ def test_top_k_axis_and_clamp(oracle_backend):
     assert y.numpy().shape == (6, 9)                                    # k clamps to the extent
     assert np.array_equal(y.numpy(), np.flip(np.sort(x, axis=0), 0))
     assert i.numpy().dtype == np.int64
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int64])
+@pytest.mark.parametrize("axes,keep", [((), False), ((0,), False), ((1,), True), ((0, 2), False), ((-1,), True)])
+def test_count_matches_numpy(oracle_backend, dtype, axes, keep):
+    x = randint(31, 5 * 6 * 70, -3, 4).astype(dtype).reshape(5, 6, 70)
+    ax = tuple(a % 3 for a in axes) or None
+    for view, ref in ((T(oracle_backend, x), x), (T(oracle_backend, x).transpose([2, 0, 1]), x.transpose(2, 0, 1))):
+        for value in (0, 2, -3, 9):
+            got = F.count(view, value, axes, keep).numpy()
+            assert got.dtype == np.int32
+            assert np.array_equal(got, (ref == value).sum(axis=ax, keepdims=keep))
+
+
+def test_count_float_special_values(oracle_backend):
+    x = np.array([0.0, -0.0, np.nan, 1.5, np.inf, -0.0], dtype=np.float32)
+    X = T(oracle_backend, x)
+    assert F.count(X, 0.0).numpy() == 3              # -0.0 == 0.0
+    assert F.count(X, np.nan).numpy() == 0           # NaN equals nothing
+    assert F.count(X, np.inf).numpy() == 1
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.int64])
+def test_nonzero_matches_numpy(oracle_backend, dtype):
+    x = (randint(32, 4 * 5 * 37, 0, 3) * (randint(33, 4 * 5 * 37, 0, 2))).astype(dtype).reshape(4, 5, 37)
+    for view, ref in ((T(oracle_backend, x), x), (T(oracle_backend, x).transpose([1, 2, 0]), x.transpose(1, 2, 0)),
+                      (T(oracle_backend, x).slice([1], [36], [2], [3]), x[:, :, 1:36:3])):
+        want = np.argwhere(ref != 0).astype(np.int32)           # row-major order of the view
+        assert np.array_equal(F.nonzero(view).numpy(), want)
+        assert np.array_equal(F.nonzero(view, True).numpy(), want.T)
+    assert F.nonzero(T(oracle_backend, np.zeros((3, 4), dtype=dtype))) is None
