@@ -258,6 +258,21 @@ def make_ops(be, which):
             gcall()
             assert torch.equal(coords.storage[:2 * total].view(total, 2).long(), torch.nonzero(x))
         ops.append(Op("N1", "gather_indices_[2^26]->[%d,2]" % total, nn, 4 * nn + 8 * total, [gcall], v_gather))
+
+    # ---------------- N2: merge of sorted rows
+    if on("all", "n2"):
+        half = 1 << 19
+        am = [torch.sort(t, dim=1).values for t in gen((64, half), torch.float32, lambda c: synth.normal(10 + 100 * c), 2)]
+        bm = [torch.sort(t, dim=1).values for t in gen((64, half), torch.float32, lambda c: synth.normal(11 + 100 * c), 2)]
+        zm = empty((64, 2 * half), torch.float32)
+        Z = tensor(zm)
+        calls = [be.merge(0, dtype_code(np.float32), tensor(a).shape, tensor(a).storage, tensor(b).shape, tensor(b).storage,
+                          Z.shape, Z.storage, defer=True) for a, b in zip(am, bm)]
+
+        def v_merge(a=am[0], b=bm[0], call=calls[0]):
+            call()
+            assert torch.equal(zm, torch.sort(torch.cat([a, b], dim=1), dim=1).values)
+        ops.append(Op("N2", "merge_f32_[64,2^19]+[64,2^19]", 64 * 2 * half, 2 * 4 * 64 * 2 * half, calls, v_merge))
     return ops
 
 
@@ -382,7 +397,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1")
+    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",

@@ -288,6 +288,29 @@ def top_k(X: Tensor, k: int, axis: int = -1, largest: bool = True, index_dtype=n
     return Y, I
 
 
+def merge(A: Tensor, B: Tensor, axis: int = -1, descending: bool = False, out: Optional[Tensor] = None) -> Tensor:
+    """Merges two tensors sorted along `axis` into one sorted tensor (reorder.h:1061-1114):
+    the other extents must agree; equal elements keep A's before B's."""
+    rank = A.rank
+    if B.rank != rank:
+        raise ShapeError("merge: incompatible shape")
+    axis = norm_axis(rank, axis)
+    dims = []
+    for i in range(rank):
+        if i == axis:
+            dims.append(A.extent(i) + B.extent(i))
+        elif A.extent(i) != B.extent(i):
+            raise ShapeError("merge: incompatible shape")
+        else:
+            dims.append(A.extent(i))
+    C = out if out is not None else Tensor.empty(A.backend, dims, A.dtype)
+    if list(C.shape.extents) != dims:
+        raise ShapeError("merge: output shape")
+    a, b, c = A.shape.moveaxis(axis, -1), B.shape.moveaxis(axis, -1), C.shape.moveaxis(axis, -1)
+    A.backend.merge(1 if descending else 0, dtype_code(A.dtype), a, A.storage, b, B.storage, c, C.storage)
+    return C
+
+
 def gather_elements(X: np.ndarray, I: np.ndarray, axis: int) -> np.ndarray:
     """Host helper of the reference's property tests (reorder_detail.h:190-207)."""
     return np.take_along_axis(X, I.astype(np.int64), axis=axis)

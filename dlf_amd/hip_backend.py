@@ -81,6 +81,12 @@ def _declare(lib):
     lib.dlfx_scan_nonzero.argtypes = [c_void_p, c_int, c_int64, c_int64, c_int, c_int, _I64P,
                                       c_void_p, c_int64, _I64P, c_void_p, c_int64, _I64P, c_void_p, c_size_t]
 
+    lib.dlfx_merge_scratch_bytes.restype = c_size_t
+    lib.dlfx_merge_scratch_bytes.argtypes = [c_int, c_int64, c_int64]
+    lib.dlfx_merge.restype = c_int
+    lib.dlfx_merge.argtypes = [c_void_p, c_int, c_int, c_int, _I64P, _I64P, c_void_p, c_int64,
+                               _I64P, _I64P, c_void_p, c_int64, _I64P, _I64P, c_void_p, c_int64, c_void_p, c_size_t]
+
     lib.dlfx_gather_indices.restype = c_int
     lib.dlfx_gather_indices.argtypes = [c_void_p, c_int64, c_int64, c_int, c_int, _I64P,
                                         c_void_p, c_int64, c_void_p, c_int64]
@@ -98,7 +104,8 @@ EXPORTS = ("dlfx_version", "dlfx_status_string", "dlfx_last_hip_error", "dlfx_se
            "dlfx_argsort_scratch_bytes", "dlfx_argsort",
            "dlfx_top_k_scratch_bytes", "dlfx_top_k",
            "dlfx_count_scratch_bytes", "dlfx_count",
-           "dlfx_scan_nonzero_scratch_bytes", "dlfx_scan_nonzero", "dlfx_gather_indices")
+           "dlfx_scan_nonzero_scratch_bytes", "dlfx_scan_nonzero", "dlfx_gather_indices",
+           "dlfx_merge_scratch_bytes", "dlfx_merge")
 
 
 def load_library():
@@ -261,6 +268,14 @@ class HipBackend:
     def gather_indices(self, m, n, row_major, dims, counts, out, defer=False):
         return self._issue(self.lib.dlfx_gather_indices, "dlfx_gather_indices", (m, n, int(bool(row_major))),
                            (len(dims), _arr(dims), counts.data_ptr(), 0, out.data_ptr(), 0), defer)
+
+    def merge(self, direction, dtype, xs, x, ys, y, zs, z, defer=False):
+        n = zs.extents[-1]
+        sp, sb = self.scratch(self.lib.dlfx_merge_scratch_bytes(dtype, zs.size // n, n))
+        return self._issue(self.lib.dlfx_merge, "dlfx_merge", (direction, dtype, zs.rank),
+                           (_arr(xs.extents), _arr(xs.strides), x.data_ptr(), xs.offset,
+                            _arr(ys.extents), _arr(ys.strides), y.data_ptr(), ys.offset,
+                            _arr(zs.extents), _arr(zs.strides), z.data_ptr(), zs.offset, sp, sb), defer)
 
     def read_element(self, storage, index):
         """One element of a device buffer on the host (synchronises the stream)."""

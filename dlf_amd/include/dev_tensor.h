@@ -466,4 +466,32 @@ inline std::pair<DevTensor<T>, DevTensor<int32_t>> top_k(const DevTensor<T>& X, 
     return {std::move(Y), std::move(I)};
 }
 
+// ---------------------------------------------------------------- merge
+// dlf/include/tensor/reorder.h:1061-1114: A and B are sorted along `axis`; C receives the
+// merged rows (descending: both inputs sorted descending, the reference's comp = greater).
+template <typename T>
+void merge(const DevTensor<T>& A, const DevTensor<T>& B, DevTensor<T>& C, int axis = -1, bool descending = false) {
+    const int rank = static_cast<int>(A.rank());
+    if (static_cast<int>(B.rank()) != rank) throw shape_error("merge: incompatible shape");
+    detail::norm_axis(rank, axis);
+    std::vector<size_t> dims(rank);
+    for (int i = 0; i < rank; ++i) {
+        if (i == axis) dims[i] = A.extent(i) + B.extent(i);
+        else if (A.extent(i) != B.extent(i)) throw shape_error("merge: incompatible shape");
+        else dims[i] = A.extent(i);
+    }
+    C.resize(Shape(dims));
+    const auto a = moveaxis(A, axis, -1), b = moveaxis(B, axis, -1), c = moveaxis(C, axis, -1);
+    gpgpu::dnn::merge(descending ? 1 : 0,
+                      a.shape().extents(), a.shape().strides(), a.data(), a.shape().offset(),
+                      b.shape().extents(), b.shape().strides(), b.data(), b.shape().offset(),
+                      c.shape().extents(), c.shape().strides(), C.data(), c.shape().offset());
+}
+template <typename T>
+inline DevTensor<T> merge(const DevTensor<T>& A, const DevTensor<T>& B, int axis = -1, bool descending = false) {
+    DevTensor<T> C;
+    merge(A, B, C, axis, descending);
+    return C;
+}
+
 }  // namespace dlf

@@ -175,6 +175,35 @@ void top_k(const size_t limit, const int dir,
     ev.done();
 }
 
+// gpgpu/include/gdnn.h:147-155
+template <typename T>
+void merge(const int dir,
+           const std::vector<size_t>& x_dims, const std::vector<size_t>& x_strides,
+           const Buffer<T>& x_buffer, const size_t x_offset,
+           const std::vector<size_t>& y_dims, const std::vector<size_t>& y_strides,
+           const Buffer<T>& y_buffer, const size_t y_offset,
+           const std::vector<size_t>& z_dims, const std::vector<size_t>& z_strides,
+           Buffer<T>& z_buffer, const size_t z_offset,
+           const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    const int dt = detail::dtype_of<T>::value;
+    if (x_dims.size() != z_dims.size() || y_dims.size() != z_dims.size() || z_dims.empty())
+        throw LogicError("gpgpu::dnn::merge: ranks differ");
+    auto xd = detail::signed_vec(x_dims), xs = detail::signed_vec(x_strides);
+    auto yd = detail::signed_vec(y_dims), ys = detail::signed_vec(y_strides);
+    auto zd = detail::signed_vec(z_dims), zs = detail::signed_vec(z_strides);
+    const size_t n = z_dims.back();
+    size_t m = 1;
+    for (size_t i = 0; i + 1 < z_dims.size(); ++i) m *= z_dims[i];
+    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_merge_scratch_bytes(dt, m, n));
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_merge(queue.stream(), dir, dt, static_cast<int>(zd.size()),
+                            xd.data(), xs.data(), x_buffer.data(), x_offset,
+                            yd.data(), ys.data(), y_buffer.data(), y_offset,
+                            zd.data(), zs.data(), z_buffer.data(), z_offset,
+                            tmp.bytes(), tmp.byte_size()), "gpgpu::dnn::merge");
+    ev.done();
+}
+
 // gpgpu/include/gdnn.h:116-122
 template <typename T>
 void count(const size_t m, const size_t n, const T value,

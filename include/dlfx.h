@@ -192,6 +192,19 @@ int dlfx_scan_nonzero(dlfx_stream_t stream, int dtype, int64_t m, int64_t n,
                       int32_t* y, int64_t y_offset, const int64_t* y_strides,
                       void* scratch, size_t scratch_bytes);
 
+/* ---------------------------------------------------------------- merge
+ * Replaces gpgpu::dnn::merge<T> (gdnn.h:147-155; caller reorder_detail.h:496-506).  x and y
+ * are sorted along their last axis (dir 0 ascending, 1 descending) and share z's leading
+ * extents; z's last extent is the sum of theirs.  Equal elements keep "x before y".
+ * m = number of rows of z, n = its last extent.
+ */
+size_t dlfx_merge_scratch_bytes(int dtype, int64_t m, int64_t n);
+int dlfx_merge(dlfx_stream_t stream, int dir, int dtype, int rank,
+               const int64_t* x_dims, const int64_t* x_strides, const void* x, int64_t x_offset,
+               const int64_t* y_dims, const int64_t* y_strides, const void* y, int64_t y_offset,
+               const int64_t* z_dims, const int64_t* z_strides, void* z, int64_t z_offset,
+               void* scratch, size_t scratch_bytes);
+
 /* ---------------------------------------------------------------- gather_indices
  * Replaces gpgpu::dnn::gather_indices (gdnn.h:328-332; caller reduce.h:446-449): `indices`
  * holds the inclusive running count of non-zero elements over the m elements of a tensor of

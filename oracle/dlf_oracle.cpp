@@ -752,4 +752,37 @@ int dlf_oracle_gather_indices(int64_t m, int64_t n, int row_major, int rank, con
     return 0;
 }
 
+// merge (dlf/include/tensor/reorder_detail.h:346-368, 470-494): per row, the serial merge that
+// takes y's element only when comp(y, x); the parallel split of longer rows produces the same
+// sequence because it cuts x at a pivot and y at lower_bound of that pivot (394-449).
+int dlf_oracle_merge(int dir, int dtype, int rank,
+                     const int64_t* x_dims, const int64_t* x_strides, const void* x, int64_t x_offset,
+                     const int64_t* y_dims, const int64_t* y_strides, const void* y, int64_t y_offset,
+                     const int64_t* z_dims, const int64_t* z_strides, void* z, int64_t z_offset) {
+    View xv(rank, x_dims, x_strides, x_offset), yv(rank, y_dims, y_strides, y_offset), zv(rank, z_dims, z_strides, z_offset);
+    const int64_t na = x_dims[rank - 1], nb = y_dims[rank - 1], n = na + nb;
+    if (n != z_dims[rank - 1]) return -3;
+    const int64_t rows = zv.size() / n;
+    return by_dtype(dtype, [&](auto tag) {
+        using T = decltype(tag);
+        const T* xp = static_cast<const T*>(x);
+        const T* yp = static_cast<const T*>(y);
+        T* zp = static_cast<T*>(z);
+        auto comp = [dir](T a, T b) { return dir ? a > b : a < b; };
+#pragma omp parallel for schedule(static)
+        for (int64_t r = 0; r < rows; ++r) {
+            int64_t i = 0, j = 0, k = 0;
+            const int64_t xb = na ? xv.at(r * na) : 0, yb = nb ? yv.at(r * nb) : 0, zb = zv.at(r * n);
+            const int64_t sx = xv.last_stride(), sy = yv.last_stride(), sz = zv.last_stride();
+            while (i < na && j < nb) {
+                if (comp(yp[yb + j * sy], xp[xb + i * sx])) zp[zb + (k++) * sz] = yp[yb + (j++) * sy];
+                else zp[zb + (k++) * sz] = xp[xb + (i++) * sx];
+            }
+            while (i < na) zp[zb + (k++) * sz] = xp[xb + (i++) * sx];
+            while (j < nb) zp[zb + (k++) * sz] = yp[yb + (j++) * sy];
+        }
+        return 0;
+    });
+}
+
 }  // extern "C"

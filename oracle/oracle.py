@@ -134,6 +134,13 @@ class OracleBackend:
             c_int64(m), c_int64(n), c_int(int(bool(row_major))), c_int(len(dims)), _arr(dims),
             _ptr(counts), _ptr(out)), "oracle gather_indices")
 
+    def merge(self, direction, dtype, xs, x, ys, y, zs, z):
+        _check(self.lib.dlf_oracle_merge(
+            c_int(direction), c_int(dtype), c_int(zs.rank),
+            _arr(xs.extents), _arr(xs.strides), _ptr(x), c_int64(xs.offset),
+            _arr(ys.extents), _arr(ys.strides), _ptr(y), c_int64(ys.offset),
+            _arr(zs.extents), _arr(zs.strides), _ptr(z), c_int64(zs.offset)), "oracle merge")
+
     def read_element(self, storage, index):
         return storage[index]
 

@@ -6,7 +6,8 @@
 // Vectors: dlf/test/UniformTest.cpp:1857-1965 (reduce), :2106-2189 (scan),
 // :2304-2377 (sort), dlf/test/DNNTest.cpp:861-1019 (argmax/argmin),
 // dlf/test/model/PredictTest.cpp:609-637 (top_k), dlf/test/UniformTest.cpp:2065-2080
-// (count) and :2553-2561 (nonzero).
+// (count), :2553-2561 (nonzero) and :2250-2283 (merge).
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <random>
@@ -179,6 +180,26 @@ static void test_count_nonzero() {
     CHECK(nonzero(Xt).read() == Tensor<int32_t>({3, 2}, {0, 1, 1, 0, 2, 1}));
 }
 
+static void test_merge() {
+    // UniformTest.cpp:2250-2283: merge of two sorted vectors == std::merge
+    std::mt19937 rng(7);
+    std::vector<int> a(2000), b(3000), want(5000);
+    for (auto& v : a) v = static_cast<int>(rng() % 100000);
+    for (auto& v : b) v = static_cast<int>(rng() % 100000);
+    std::sort(a.begin(), a.end());
+    std::sort(b.begin(), b.end());
+    std::merge(a.begin(), a.end(), b.begin(), b.end(), want.begin());
+    auto C = merge(dev(Tensor<int>({2000}, a)), dev(Tensor<int>({3000}, b)));
+    CHECK(C.read() == Tensor<int>({5000}, want));
+    // along the first axis of matrices (a strided axis)
+    auto A2 = dev(Tensor<float>({3, 2}, {1, 10, 3, 20, 5, 30}));
+    auto B2 = dev(Tensor<float>({2, 2}, {2, 15, 4, 25}));
+    CHECK(merge(A2, B2, 0).read() == Tensor<float>({5, 2}, {1, 10, 2, 15, 3, 20, 4, 25, 5, 30}));
+    bool threw = false;
+    try { merge(A2, dev(Tensor<float>({2, 3}).range()), 0); } catch (const shape_error&) { threw = true; }
+    CHECK(threw);
+}
+
 static void test_errors_and_temporaries() {
     auto X = dev(Tensor<float>({2, 3}).range());
     bool threw = false;
@@ -225,6 +246,7 @@ int main() {
     test_sort();
     test_top_k();
     test_count_nonzero();
+    test_merge();
     test_errors_and_temporaries();
     std::printf("veneer_test: %d checks, %d failed\n", g_checked, g_failed);
     return g_failed ? 1 : 0;

@@ -229,3 +229,32 @@ def test_nonzero_matches_numpy(oracle_backend, dtype):
         assert np.array_equal(F.nonzero(view).numpy(), want)
         assert np.array_equal(F.nonzero(view, True).numpy(), want.T)
     assert F.nonzero(T(oracle_backend, np.zeros((3, 4), dtype=dtype))) is None
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.float64])
+@pytest.mark.parametrize("desc", [False, True])
+def test_merge_matches_numpy(oracle_backend, dtype, desc):
+    # UniformTest.cpp:2250-2283: merge of sorted inputs == std::merge (one sorted sequence)
+    for na, nb in ((2000, 3000), (1, 7), (500, 0 + 1), (1500, 1500)):
+        a = np.sort(randint(40, 3 * na, -1000, 1000).astype(dtype).reshape(3, na), axis=1)
+        b = np.sort(randint(41, 3 * nb, -1000, 1000).astype(dtype).reshape(3, nb), axis=1)
+        if desc:
+            a, b = a[:, ::-1].copy(), b[:, ::-1].copy()
+        want = np.sort(np.concatenate([a, b], axis=1), axis=1)
+        if desc:
+            want = want[:, ::-1]
+        got = F.merge(T(oracle_backend, a), T(oracle_backend, b), -1, desc).numpy()
+        assert np.array_equal(got, want)
+    # along axis 0 of transposed data
+    a = np.sort(randint(42, 40 * 6, 0, 50).astype(dtype).reshape(40, 6), axis=0)
+    b = np.sort(randint(43, 25 * 6, 0, 50).astype(dtype).reshape(25, 6), axis=0)
+    got = F.merge(T(oracle_backend, a), T(oracle_backend, b), 0).numpy()
+    assert np.array_equal(got, np.sort(np.concatenate([a, b], axis=0), axis=0))
+
+
+def test_merge_keeps_first_input_first_on_ties(oracle_backend):
+    a = np.array([-1.0, 0.0, 0.0, 2.0], dtype=np.float32)
+    b = np.array([-0.0, -0.0, 2.0], dtype=np.float32)
+    got = F.merge(T(oracle_backend, a), T(oracle_backend, b)).numpy()
+    assert got.tolist() == [-1.0, 0.0, 0.0, 0.0, 0.0, 2.0, 2.0]
+    assert np.signbit(got).tolist() == [True, False, False, True, True, False, False]
