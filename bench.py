@@ -259,6 +259,25 @@ def make_ops(be, which):
             assert torch.equal(coords.storage[:2 * total].view(total, 2).long(), torch.nonzero(x))
         ops.append(Op("N1", "gather_indices_[2^26]->[%d,2]" % total, nn, 4 * nn + 8 * total, [gcall], v_gather))
 
+    # ---------------- N3: softmax family on the top_k shape and the logits head
+    if on("all", "n3"):
+        for rows_s, cols_s, copies in ((4096, 32000, 3), (256, 1000, 4)):
+            xs_ = gen((rows_s, cols_s), torch.float32, lambda c: synth.normal(12 + 100 * c), copies)
+            ys_ = empty((rows_s, cols_s), torch.float32)
+            for nm in ("softmax", "logsoftmax", "hardmax"):
+                calls = [be.softmax(nm, dtype_code(np.float32), rows_s, cols_s, x.view(-1), 0, ys_.view(-1), 0, defer=True)
+                         for x in xs_]
+
+                def v_soft(x=xs_[0], call=calls[0], nm=nm, ys_=ys_, rows_s=rows_s):
+                    call()
+                    if nm == "softmax":
+                        assert torch.allclose(ys_.double(), torch.softmax(x.double(), 1), rtol=1e-5, atol=1e-12)
+                    elif nm == "logsoftmax":
+                        assert torch.allclose(ys_.double(), torch.log_softmax(x.double(), 1), rtol=1e-5, atol=1e-5)
+                    else:
+                        assert torch.equal(ys_.argmax(1), x.argmax(1)) and float(ys_.sum()) == rows_s
+                ops.append(Op("N3", "%s_f32_[%d,%d]" % (nm, rows_s, cols_s), rows_s * cols_s, 8 * rows_s * cols_s, calls, v_soft))
+
     # ---------------- N2: merge of sorted rows
     if on("all", "n2"):
         half = 1 << 19
@@ -397,7 +416,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2")
+    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",

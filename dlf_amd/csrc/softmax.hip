@@ -1,0 +1,272 @@
+// softmax / logsoftmax / hardmax over the rows of a contiguous [m, n] matrix
+// (gpgpu/include/gdnn.h:253-264; host semantics dlf/include/tensor/dnn_detail.h:266-350:
+// subtract the row maximum, exponentiate, divide by the sum; logsoftmax x - max - log(sum);
+// hardmax a one at the first occurrence of the maximum and zeros elsewhere).
+//
+// A row is read once: it lives in the registers of a team of threads (one wavefront for rows
+// up to 2048 elements, a 1024-thread workgroup up to 32768 four-byte elements) between the
+// load, the two team-wide reductions and the store.  Longer rows are streamed twice (running
+// maximum and rescaled sum first, then the outputs).  Bandwidth bound; exp and log in the
+// element type, sums in it as well (tree order), as the reference's row loops do.
+#include <cmath>
+#include <cstring>
+#include <limits>
+#include <type_traits>
+
+#include "common.hip.h"
+
+namespace dlfx {
+namespace {
+
+enum SoftKind { kSoftmax = 0, kLogSoftmax = 1, kHardmax = 2 };
+
+template <typename T> __device__ __forceinline__ T exp_of(T v);
+template <> __device__ __forceinline__ float exp_of<float>(float v) { return expf(v); }
+template <> __device__ __forceinline__ double exp_of<double>(double v) { return exp(v); }
+template <typename T> __device__ __forceinline__ T log_of(T v);
+template <> __device__ __forceinline__ float log_of<float>(float v) { return logf(v); }
+template <> __device__ __forceinline__ double log_of<double>(double v) { return log(v); }
+
+// (maximum, first index holding it) with the serial loop's rules (dnn_detail.h:334-346):
+// strict comparison, so the first occurrence wins; a NaN in position 0 is never displaced and
+// a NaN elsewhere never wins.
+template <typename T>
+struct MaxAt {
+    T v;
+    int32_t i;
+};
+template <typename T>
+__device__ __forceinline__ MaxAt<T> max_at_of(T x, int64_t j) {
+    if (x != x) {
+        if (j == 0) return {std::numeric_limits<T>::infinity(), -1};
+        return {-std::numeric_limits<T>::infinity(), std::numeric_limits<int32_t>::max()};
+    }
+    return {x, static_cast<int32_t>(j)};
+}
+template <typename T>
+__device__ __forceinline__ MaxAt<T> max_at_join(MaxAt<T> a, MaxAt<T> b) {
+    const bool take_b = b.v > a.v || (b.v == a.v && b.i < a.i);
+    return take_b ? b : a;
+}
+
+// Reduction over the TEAM threads that share a row (a wavefront, or a whole workgroup through
+// LDS); every thread receives the result.  `slot` separates the teams of a workgroup.
+template <int TEAM, typename V, typename Join>
+__device__ __forceinline__ V team_reduce(V v, Join join, V* lds) {
+    v = wave_reduce(v, join);
+    if constexpr (TEAM > kWave) {
+        constexpr int WAVES = TEAM / kWave;
+        const int w = threadIdx.x / kWave;
+        __syncthreads();                       // the previous use of `lds` is over
+        if (lane_id() == 0) lds[w] = v;
+        __syncthreads();
+        v = lds[0];
+#pragma unroll
+        for (int i = 1; i < WAVES; ++i) v = join(v, lds[i]);
+    }
+    return v;
+}
+
+// Rows held in registers.  TEAM threads per row, ITEMS elements per thread; element (k, t) of
+// the row is ((k / V) * TEAM + t) * V + k % V with V elements per 128-bit access when VEC.
+template <typename T, int TEAM, int ITEMS, int KIND, bool VEC>
+__global__ __launch_bounds__(TEAM > 256 ? TEAM : 256)
+__attribute__((amdgpu_waves_per_eu(TEAM >= 1024 && sizeof(T) * ITEMS <= 128 ? 8 : 1)))      // two 1024-thread rows per CU
+void softmax_rows(const T* __restrict__ x, T* __restrict__ y,
+                                                                        int64_t m, int64_t n) {
+    constexpr int BLOCK = TEAM > 256 ? TEAM : 256;
+    constexpr int V = VEC ? 16 / static_cast<int>(sizeof(T)) : 1;
+    static_assert(ITEMS % V == 0, "whole vectors per thread");
+    constexpr int G = ITEMS / V;
+    using VecT = Vec<T, V>;
+    __shared__ alignas(16) unsigned char lds_raw[(TEAM > kWave ? TEAM / kWave : 1) * sizeof(MaxAt<T>)];
+
+    const int t = threadIdx.x % TEAM;
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * (BLOCK / TEAM) + threadIdx.x / TEAM;
+    const bool live = row < m;                           // whole teams are live or not
+    const T* xr = x + (live ? row : 0) * n;
+    T* yr = y + (live ? row : 0) * n;
+    const T lowest = -std::numeric_limits<T>::infinity();
+    const int32_t n32 = static_cast<int32_t>(n);          // rows here have at most 32768 elements
+    auto index_of = [&](int k) -> int32_t { return ((k / V) * TEAM + t) * V + k % V; };
+
+    T v[ITEMS];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int64_t i0 = (static_cast<int64_t>(g) * TEAM + t) * V;
+        if (VEC) {
+            if (live && i0 < n) {                         // n is a multiple of V here
+                const VecT a = load_stream(reinterpret_cast<const VecT*>(xr + i0));
+#pragma unroll
+                for (int e = 0; e < V; ++e) v[g * V + e] = a.v[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < V; ++e) v[g * V + e] = lowest;
+            }
+        } else {
+            v[g] = (live && i0 < n) ? load_stream(&xr[i0]) : lowest;
+        }
+    }
+
+    if constexpr (KIND == kHardmax) {
+        // the serial loop (dnn_detail.h:334-346) keeps the first element that is strictly larger
+        // than everything before it: the first occurrence of the largest non-NaN value, or
+        // position 0 when the row starts with a NaN (nothing compares larger than a NaN)
+        T mx = lowest;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) mx = (mx < v[k]) ? v[k] : mx;
+        mx = team_reduce<TEAM>(mx, [](T a, T b) { return (a < b) ? b : a; }, reinterpret_cast<T*>(lds_raw));
+        int32_t hot = std::numeric_limits<int32_t>::max();
+#pragma unroll
+        for (int k = ITEMS - 1; k >= 0; --k)
+            if (v[k] == mx && index_of(k) < n32) hot = index_of(k);      // this thread's indices grow with k
+        hot = team_reduce<TEAM>(hot, [](int32_t a, int32_t b) { return a < b ? a : b; }, reinterpret_cast<int32_t*>(lds_raw));
+        if (hot >= n32 || (live && xr[0] != xr[0])) hot = 0;               // all NaN or -inf, or a leading NaN
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) v[k] = index_of(k) == hot ? T(1) : T(0);
+    } else {
+        // the reference starts from px[0] and uses std::max, which keeps its first argument when
+        // the comparison fails: a NaN spreads only from position 0; other NaNs are skipped
+        T mx = lowest;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) mx = (mx < v[k]) ? v[k] : mx;
+        mx = team_reduce<TEAM>(mx, [](T a, T b) { return (a < b) ? b : a; }, reinterpret_cast<T*>(lds_raw));
+        if (live && xr[0] != xr[0]) mx = xr[0];
+        T sum = T(0);
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const T e = index_of(k) < n32 ? exp_of<T>(v[k] - mx) : T(0);
+            if constexpr (KIND == kSoftmax) v[k] = e;
+            sum += e;
+        }
+        sum = team_reduce<TEAM>(sum, [](T a, T b) { return a + b; }, reinterpret_cast<T*>(lds_raw));
+        if constexpr (KIND == kSoftmax) {
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) v[k] = v[k] / sum;
+        } else {
+            // (x - max) - log(sum) in this order: x - max is exact for nearby values, max + log(sum)
+            // would round at the magnitude of max
+            const T lsum = log_of<T>(sum);
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) v[k] = (v[k] - mx) - lsum;
+        }
+    }
+
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int64_t i0 = (static_cast<int64_t>(g) * TEAM + t) * V;
+        if (live && i0 < n) {
+            if (VEC) {
+                VecT a;
+#pragma unroll
+                for (int e = 0; e < V; ++e) a.v[e] = v[g * V + e];
+                store_stream(reinterpret_cast<VecT*>(yr + i0), a);
+            } else {
+                store_stream(&yr[i0], v[g]);
+            }
+        }
+    }
+}
+
+// Rows too long for registers: one 1024-thread workgroup per row, two passes over the row.
+template <typename T, int KIND>
+__global__ __launch_bounds__(1024) void softmax_rows_streamed(const T* __restrict__ x, T* __restrict__ y, int64_t n) {
+    constexpr int TEAM = 1024;
+    __shared__ alignas(16) unsigned char lds_raw[(TEAM / kWave) * sizeof(MaxAt<T>)];
+    const int t = threadIdx.x;
+    const T* xr = x + static_cast<int64_t>(blockIdx.x) * n;
+    T* yr = y + static_cast<int64_t>(blockIdx.x) * n;
+    const T lowest = -std::numeric_limits<T>::infinity();
+    if constexpr (KIND == kHardmax) {
+        MaxAt<T> best = {lowest, std::numeric_limits<int32_t>::max()};
+        for (int64_t i = t; i < n; i += TEAM) best = max_at_join(best, max_at_of(xr[i], i));
+        best = team_reduce<TEAM>(best, [](MaxAt<T> a, MaxAt<T> b) { return max_at_join(a, b); },
+                                 reinterpret_cast<MaxAt<T>*>(lds_raw));
+        const int64_t hot = best.i < 0 ? 0 : best.i;
+        for (int64_t i = t; i < n; i += TEAM) yr[i] = i == hot ? T(1) : T(0);
+    } else {
+        // running maximum and the sum of exp(x - maximum), rescaled whenever the maximum moves
+        T mx = lowest, sum = T(0);
+        for (int64_t i = t; i < n; i += TEAM) {
+            const T xv = xr[i];
+            if (mx < xv) {
+                sum = sum * exp_of<T>(mx - xv);          // exp(-inf) = 0 on the first element
+                mx = xv;
+            }
+            if (xv != lowest || mx != lowest) sum += exp_of<T>(xv - mx);     // -inf before any finite element adds nothing
+        }
+        T row_max = team_reduce<TEAM>(mx, [](T a, T b) { return (a < b) ? b : a; }, reinterpret_cast<T*>(lds_raw));
+        sum = (mx == lowest) ? T(0) : sum * exp_of<T>(mx - row_max);
+        if (xr[0] != xr[0]) row_max = xr[0];             // a NaN in position 0 is the reference's maximum
+        sum = team_reduce<TEAM>(sum, [](T a, T b) { return a + b; }, reinterpret_cast<T*>(lds_raw));
+        const T lsum = log_of<T>(sum);
+        for (int64_t i = t; i < n; i += TEAM) {
+            const T xv = xr[i];
+            yr[i] = KIND == kSoftmax ? exp_of<T>(xv - row_max) / sum : (xv - row_max) - lsum;
+        }
+    }
+}
+
+template <typename T, int KIND>
+int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y) {
+    constexpr int V = 16 / static_cast<int>(sizeof(T));
+    const bool vec = n % V == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
+    // wavefront teams: 4 rows per workgroup
+#define DLFX_WAVE_ROWS(ITEMS)                                                                                   \
+    do {                                                                                                        \
+        const dim3 grid(static_cast<unsigned>(ceil_div(m, 4)));                                                 \
+        if (vec) softmax_rows<T, kWave, ITEMS, KIND, true><<<grid, dim3(256), 0, stream>>>(x, y, m, n);         \
+        else softmax_rows<T, kWave, ITEMS, KIND, false><<<grid, dim3(256), 0, stream>>>(x, y, m, n);            \
+        DLFX_CHECK_LAUNCH();                                                                                    \
+        return DLFX_OK;                                                                                         \
+    } while (0)
+#define DLFX_BLOCK_ROWS(ITEMS)                                                                                  \
+    do {                                                                                                        \
+        const dim3 grid(static_cast<unsigned>(m));                                                              \
+        if (vec) softmax_rows<T, 1024, ITEMS, KIND, true><<<grid, dim3(1024), 0, stream>>>(x, y, m, n);         \
+        else softmax_rows<T, 1024, ITEMS, KIND, false><<<grid, dim3(1024), 0, stream>>>(x, y, m, n);            \
+        DLFX_CHECK_LAUNCH();                                                                                    \
+        return DLFX_OK;                                                                                         \
+    } while (0)
+    if (ceil_div(m, 4) > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+    if (n <= kWave * V) DLFX_WAVE_ROWS(V);
+    if (n <= kWave * 4 * V) DLFX_WAVE_ROWS(4 * V);
+    if (n <= kWave * 32) DLFX_WAVE_ROWS(32);
+    if (n <= 1024 * 8) DLFX_BLOCK_ROWS(8);
+    if (n <= 1024 * 16) DLFX_BLOCK_ROWS(16);
+    if (n <= 1024 * 32 && sizeof(T) == 4) DLFX_BLOCK_ROWS(32);
+#undef DLFX_WAVE_ROWS
+#undef DLFX_BLOCK_ROWS
+    softmax_rows_streamed<T, KIND><<<dim3(static_cast<unsigned>(m)), dim3(1024), 0, stream>>>(x, y, n);
+    DLFX_CHECK_LAUNCH();
+    return DLFX_OK;
+}
+
+}  // namespace
+}  // namespace dlfx
+
+using namespace dlfx;
+
+extern "C" int dlfx_softmax(dlfx_stream_t stream, const char* name, int dtype, int64_t m, int64_t n,
+                            const void* x, int64_t x_offset, void* y, int64_t y_offset) {
+    if (!name || !x || !y || m <= 0 || n <= 0) return DLFX_ERR_INVALID_ARGUMENT;
+    if (m > 0x7fffffffLL || n > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+    int kind;
+    if (!std::strcmp(name, "softmax")) kind = kSoftmax;
+    else if (!std::strcmp(name, "logsoftmax")) kind = kLogSoftmax;
+    else if (!std::strcmp(name, "hardmax")) kind = kHardmax;
+    else return DLFX_ERR_UNKNOWN_OP;
+    if (dtype != DLFX_F32 && dtype != DLFX_F64) return DLFX_ERR_UNSUPPORTED_DTYPE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    auto run = [&](auto tag) {
+        using T = decltype(tag);
+        const T* xp = static_cast<const T*>(x) + x_offset;
+        T* yp = static_cast<T*>(y) + y_offset;
+        switch (kind) {
+        case kSoftmax: return launch_softmax<T, kSoftmax>(s, m, n, xp, yp);
+        case kLogSoftmax: return launch_softmax<T, kLogSoftmax>(s, m, n, xp, yp);
+        default: return launch_softmax<T, kHardmax>(s, m, n, xp, yp);
+        }
+    };
+    return dtype == DLFX_F32 ? run(float()) : run(double());
+}

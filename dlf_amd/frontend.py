@@ -311,6 +311,33 @@ def merge(A: Tensor, B: Tensor, axis: int = -1, descending: bool = False, out: O
     return C
 
 
+def _softmax_family(name: str, X: Tensor, axis: int) -> Tensor:
+    """dlf/include/tensor/dnn.h:447-531: the tensor is flattened to [m, n] with m the product
+    of the extents before `axis` (default 1) and each row is normalised.  A non-contiguous
+    input is copied first, as the reference's reorder(X, Y) does."""
+    axis = norm_axis(X.rank, axis)
+    m = 1
+    for i in range(axis):
+        m *= X.extent(i)
+    n = X.size // m
+    src = X if X.shape.is_contiguous() else X.contiguous()
+    Y = Tensor.empty(X.backend, list(X.shape.extents), X.dtype)
+    X.backend.softmax(name, dtype_code(X.dtype), m, n, src.storage, src.shape.offset, Y.storage, 0)
+    return Y
+
+
+def softmax(X: Tensor, axis: int = 1) -> Tensor:
+    return _softmax_family("softmax", X, axis)
+
+
+def logsoftmax(X: Tensor, axis: int = 1) -> Tensor:
+    return _softmax_family("logsoftmax", X, axis)
+
+
+def hardmax(X: Tensor, axis: int = 1) -> Tensor:
+    return _softmax_family("hardmax", X, axis)
+
+
 def gather_elements(X: np.ndarray, I: np.ndarray, axis: int) -> np.ndarray:
     """Host helper of the reference's property tests (reorder_detail.h:190-207)."""
     return np.take_along_axis(X, I.astype(np.int64), axis=axis)

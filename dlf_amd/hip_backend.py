@@ -81,6 +81,9 @@ def _declare(lib):
     lib.dlfx_scan_nonzero.argtypes = [c_void_p, c_int, c_int64, c_int64, c_int, c_int, _I64P,
                                       c_void_p, c_int64, _I64P, c_void_p, c_int64, _I64P, c_void_p, c_size_t]
 
+    lib.dlfx_softmax.restype = c_int
+    lib.dlfx_softmax.argtypes = [c_void_p, c_char_p, c_int, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64]
+
     lib.dlfx_merge_scratch_bytes.restype = c_size_t
     lib.dlfx_merge_scratch_bytes.argtypes = [c_int, c_int64, c_int64]
     lib.dlfx_merge.restype = c_int
@@ -105,7 +108,7 @@ EXPORTS = ("dlfx_version", "dlfx_status_string", "dlfx_last_hip_error", "dlfx_se
            "dlfx_top_k_scratch_bytes", "dlfx_top_k",
            "dlfx_count_scratch_bytes", "dlfx_count",
            "dlfx_scan_nonzero_scratch_bytes", "dlfx_scan_nonzero", "dlfx_gather_indices",
-           "dlfx_merge_scratch_bytes", "dlfx_merge")
+           "dlfx_merge_scratch_bytes", "dlfx_merge", "dlfx_softmax")
 
 
 def load_library():
@@ -268,6 +271,10 @@ class HipBackend:
     def gather_indices(self, m, n, row_major, dims, counts, out, defer=False):
         return self._issue(self.lib.dlfx_gather_indices, "dlfx_gather_indices", (m, n, int(bool(row_major))),
                            (len(dims), _arr(dims), counts.data_ptr(), 0, out.data_ptr(), 0), defer)
+
+    def softmax(self, name, dtype, m, n, x, x_offset, y, y_offset, defer=False):
+        return self._issue(self.lib.dlfx_softmax, "dlfx_softmax(%s)" % name, (name.encode(), dtype, m, n),
+                           (x.data_ptr(), x_offset, y.data_ptr(), y_offset), defer)
 
     def merge(self, direction, dtype, xs, x, ys, y, zs, z, defer=False):
         n = zs.extents[-1]

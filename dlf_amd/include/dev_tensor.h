@@ -75,6 +75,15 @@ public:
     size_t stride(int i) const { return strides_[i < 0 ? i + rank() : i]; }
     bool operator==(const Shape& o) const noexcept { return extents_ == o.extents_; }
     bool operator!=(const Shape& o) const noexcept { return !(*this == o); }
+    // Row-major dense: every stride is the product of the extents after it (shape.cpp:126-135).
+    bool is_contiguous() const noexcept {
+        size_t size = 1;
+        for (size_t i = rank(); i-- != 0;) {
+            if (extents_[i] != 1 && strides_[i] != size) return false;
+            size *= extents_[i];
+        }
+        return true;
+    }
 
     size_t linear_offset(size_t index) const noexcept {
         size_t off = offset_;
@@ -465,6 +474,42 @@ inline std::pair<DevTensor<T>, DevTensor<int32_t>> top_k(const DevTensor<T>& X, 
     top_k(X, Y, I, k, axis, largest);
     return {std::move(Y), std::move(I)};
 }
+
+// ---------------------------------------------------------------- softmax family
+// dlf/include/tensor/dnn.h:447-531: rows are everything from `axis` on (default 1); the input
+// is first copied into Y in row-major order (the reference's reorder(X, Y)), then normalised
+// in place.
+namespace dnn {
+namespace detail {
+template <typename T, typename Fn>
+void normalize_rows(const DevTensor<T>& X, DevTensor<T>& Y, int axis, Fn fn) {
+    dlf::detail::norm_axis(static_cast<int>(X.rank()), axis);
+    size_t m = 1;
+    for (int i = 0; i < axis; ++i) m *= X.extent(i);
+    const size_t n = X.size() / m;
+    if (&X != &Y || !X.shape().is_contiguous()) Y = dev(X.read());       // row-major copy of the viewed elements
+    fn(m, n, Y.data(), Y.shape().offset());
+}
+}  // namespace detail
+template <typename T>
+void softmax(const DevTensor<T>& X, DevTensor<T>& Y, int axis = 1) {
+    detail::normalize_rows(X, Y, axis, [](size_t m, size_t n, gpgpu::Buffer<T>& b, size_t off) { gpgpu::dnn::softmax(m, n, b, off); });
+}
+template <typename T>
+void logsoftmax(const DevTensor<T>& X, DevTensor<T>& Y, int axis = 1) {
+    detail::normalize_rows(X, Y, axis, [](size_t m, size_t n, gpgpu::Buffer<T>& b, size_t off) { gpgpu::dnn::logsoftmax(m, n, b, off); });
+}
+template <typename T>
+void hardmax(const DevTensor<T>& X, DevTensor<T>& Y, int axis = 1) {
+    detail::normalize_rows(X, Y, axis, [](size_t m, size_t n, gpgpu::Buffer<T>& b, size_t off) { gpgpu::dnn::hardmax(m, n, b, off); });
+}
+template <typename T>
+inline DevTensor<T> softmax(const DevTensor<T>& X, int axis = 1) { DevTensor<T> Y; softmax(X, Y, axis); return Y; }
+template <typename T>
+inline DevTensor<T> logsoftmax(const DevTensor<T>& X, int axis = 1) { DevTensor<T> Y; logsoftmax(X, Y, axis); return Y; }
+template <typename T>
+inline DevTensor<T> hardmax(const DevTensor<T>& X, int axis = 1) { DevTensor<T> Y; hardmax(X, Y, axis); return Y; }
+}  // namespace dnn
 
 // ---------------------------------------------------------------- merge
 // dlf/include/tensor/reorder.h:1061-1114: A and B are sorted along `axis`; C receives the

@@ -175,6 +175,33 @@ void top_k(const size_t limit, const int dir,
     ev.done();
 }
 
+// gpgpu/include/gdnn.h:253-264: in place on the rows of a contiguous [m, n] matrix
+namespace detail {
+template <typename T>
+void softmax_family(const char* name, const size_t m, const size_t n, Buffer<T>& x_buffer, const size_t x_offset,
+                    const Queue& queue, Event* event) {
+    EventScope ev(queue, event);
+    check_status(dlfx_softmax(queue.stream(), name, dtype_of<T>::value, m, n, x_buffer.data(), x_offset,
+                              x_buffer.data(), x_offset), name);
+    ev.done();
+}
+}  // namespace detail
+template <typename T>
+void softmax(const size_t m, const size_t n, Buffer<T>& x_buffer, const size_t x_offset,
+             const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    detail::softmax_family("softmax", m, n, x_buffer, x_offset, queue, event);
+}
+template <typename T>
+void logsoftmax(const size_t m, const size_t n, Buffer<T>& x_buffer, const size_t x_offset,
+                const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    detail::softmax_family("logsoftmax", m, n, x_buffer, x_offset, queue, event);
+}
+template <typename T>
+void hardmax(const size_t m, const size_t n, Buffer<T>& x_buffer, const size_t x_offset,
+             const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    detail::softmax_family("hardmax", m, n, x_buffer, x_offset, queue, event);
+}
+
 // gpgpu/include/gdnn.h:147-155
 template <typename T>
 void merge(const int dir,

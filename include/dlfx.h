@@ -192,6 +192,15 @@ int dlfx_scan_nonzero(dlfx_stream_t stream, int dtype, int64_t m, int64_t n,
                       int32_t* y, int64_t y_offset, const int64_t* y_strides,
                       void* scratch, size_t scratch_bytes);
 
+/* ---------------------------------------------------------------- softmax family
+ * Replaces gpgpu::dnn::softmax / logsoftmax / hardmax<T> (gdnn.h:253-264; callers
+ * dnn_detail.h:292-295, 324-327, 352-355) on the rows of a contiguous [m, n] matrix.  The
+ * reference works in place on x; here y may be x (in place) or another buffer.
+ * name: "softmax" | "logsoftmax" | "hardmax".  Floating-point types only.  No scratch.
+ */
+int dlfx_softmax(dlfx_stream_t stream, const char* name, int dtype, int64_t m, int64_t n,
+                 const void* x, int64_t x_offset, void* y, int64_t y_offset);
+
 /* ---------------------------------------------------------------- merge
  * Replaces gpgpu::dnn::merge<T> (gdnn.h:147-155; caller reorder_detail.h:496-506).  x and y
  * are sorted along their last axis (dir 0 ascending, 1 descending) and share z's leading

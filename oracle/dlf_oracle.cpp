@@ -785,4 +785,48 @@ int dlf_oracle_merge(int dir, int dtype, int rank,
     });
 }
 
+// softmax / logsoftmax / hardmax on the rows of a contiguous [m, n] matrix, in place, as the
+// reference's row loops (dlf/include/tensor/dnn_detail.h:266-350): serial maximum from px[0]
+// with std::max, serial sum in the element type.  kind: 0 softmax, 1 logsoftmax, 2 hardmax.
+int dlf_oracle_softmax(int kind, int dtype, int64_t m, int64_t n, void* x) {
+    if (dtype != 0 && dtype != 1) return -2;
+    auto run = [&](auto tag) {
+        using T = decltype(tag);
+        T* base = static_cast<T*>(x);
+#pragma omp parallel for schedule(static)
+        for (int64_t b = 0; b < m; ++b) {
+            T* px = base + b * n;
+            if (kind == 2) {
+                T amax = px[0];
+                int64_t imax = 0;
+                for (int64_t i = 0; i < n; ++i) {
+                    if (px[i] > amax) {
+                        amax = px[i];
+                        imax = i;
+                    }
+                    px[i] = 0;
+                }
+                px[imax] = 1;
+                continue;
+            }
+            T amax = px[0];
+            for (int64_t i = 1; i < n; ++i) amax = std::max(amax, px[i]);
+            T asum = 0;
+            if (kind == 0) {
+                for (int64_t i = 0; i < n; ++i) {
+                    px[i] = std::exp(px[i] - amax);
+                    asum += px[i];
+                }
+                for (int64_t i = 0; i < n; ++i) px[i] /= asum;
+            } else {
+                for (int64_t i = 0; i < n; ++i) asum += std::exp(px[i] - amax);
+                asum = std::log(asum);
+                for (int64_t i = 0; i < n; ++i) px[i] = px[i] - amax - asum;
+            }
+        }
+        return 0;
+    };
+    return dtype == 0 ? run(float()) : run(double());
+}
+
 }  // extern "C"

@@ -134,6 +134,13 @@ class OracleBackend:
             c_int64(m), c_int64(n), c_int(int(bool(row_major))), c_int(len(dims)), _arr(dims),
             _ptr(counts), _ptr(out)), "oracle gather_indices")
 
+    def softmax(self, name, dtype, m, n, x, x_offset, y, y_offset):
+        kind = {"softmax": 0, "logsoftmax": 1, "hardmax": 2}[name]
+        if y is not x or y_offset != x_offset:
+            y[y_offset:y_offset + m * n] = x[x_offset:x_offset + m * n]
+        rows = y[y_offset:y_offset + m * n]
+        _check(self.lib.dlf_oracle_softmax(c_int(kind), c_int(dtype), c_int64(m), c_int64(n), _ptr(rows)), "oracle " + name)
+
     def merge(self, direction, dtype, xs, x, ys, y, zs, z):
         _check(self.lib.dlf_oracle_merge(
             c_int(direction), c_int(dtype), c_int(zs.rank),

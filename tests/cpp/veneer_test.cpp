@@ -6,7 +6,8 @@
 // Vectors: dlf/test/UniformTest.cpp:1857-1965 (reduce), :2106-2189 (scan),
 // :2304-2377 (sort), dlf/test/DNNTest.cpp:861-1019 (argmax/argmin),
 // dlf/test/model/PredictTest.cpp:609-637 (top_k), dlf/test/UniformTest.cpp:2065-2080
-// (count), :2553-2561 (nonzero) and :2250-2283 (merge).
+// (count), :2553-2561 (nonzero), :2250-2283 (merge), dlf/test/DNNTest.cpp:796-858
+// (softmax, logsoftmax, hardmax).
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
@@ -180,6 +181,23 @@ static void test_count_nonzero() {
     CHECK(nonzero(Xt).read() == Tensor<int32_t>({3, 2}, {0, 1, 1, 0, 2, 1}));
 }
 
+static void test_softmax_family() {
+    // DNNTest.cpp:796-858
+    auto X = Tensor<float>({2, 4}, {0, 1, 2, 3, 10000, 10001, 10002, 10003});
+    CHECK(near(dnn::softmax(dev(X)).read(), Tensor<float>({2, 4}, {0.0320586f, 0.08714432f, 0.23688284f, 0.64391428f,
+                                                                   0.0320586f, 0.08714432f, 0.23688284f, 0.64391428f})));
+    CHECK(near(dnn::logsoftmax(dev(X)).read(), Tensor<float>({2, 4}, {-3.4401896f, -2.4401896f, -1.44018972f, -0.44018969f,
+                                                                      -3.4401896f, -2.4401896f, -1.44018972f, -0.44018969f})));
+    auto H = Tensor<float>({4, 4}, {3, 0, 1, 2, 2, 5, 1, 0, 0, 1, 3, 2, 0, 1, 2, 3});
+    CHECK(dnn::hardmax(dev(H)).read() == Tensor<float>({4, 4}, {1, 0, 0, 0, 0, 1, 0, 0, 0, 0, 1, 0, 0, 0, 0, 1}));
+    CHECK(dnn::hardmax(dev(Tensor<float>({1, 4}, {3, 3, 3, 1}))).read() == Tensor<float>({1, 4}, {1, 0, 0, 0}));
+    // in place, and a transposed input (copied to row-major order first)
+    auto D = dev(H);
+    dnn::hardmax(D, D);
+    CHECK(D.read() == Tensor<float>({4, 4}, {1, 0, 0, 0, 0, 1, 0, 0, 0, 0, 1, 0, 0, 0, 0, 1}));
+    CHECK(dnn::hardmax(dev(H).transpose()).read() == Tensor<float>({4, 4}, {1, 0, 0, 0, 0, 1, 0, 0, 0, 0, 1, 0, 0, 0, 0, 1}));
+}
+
 static void test_merge() {
     // UniformTest.cpp:2250-2283: merge of two sorted vectors == std::merge
     std::mt19937 rng(7);
@@ -247,6 +265,7 @@ int main() {
     test_top_k();
     test_count_nonzero();
     test_merge();
+    test_softmax_family();
     test_errors_and_temporaries();
     std::printf("veneer_test: %d checks, %d failed\n", g_checked, g_failed);
     return g_failed ? 1 : 0;

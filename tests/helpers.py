@@ -50,6 +50,9 @@ def run_golden_case(backend, case):
         elif op == "top_k":
             y, i = F.top_k(X, call["k"], call["axis"], call["largest"])
             outs = [(y, call["y_shape"], call["y"]), (i, call["y_shape"], call["i"])]
+        elif op in ("softmax", "logsoftmax", "hardmax"):
+            got = getattr(F, op)(X, call["axis"])
+            outs = [(got, call["y_shape"], call["y"])]
         elif op == "count":
             got = F.count(X, call["value"], call["axes"], call["keepdims"])
             outs = [(got, call["y_shape"], call["y"])]

@@ -1,0 +1,79 @@
+"""softmax / logsoftmax / hardmax: HIP path vs the CPU oracle (the reference's row loops).
+
+hardmax is exact.  softmax and logsoftmax: the reference sums a row serially in the element
+type, which for long fp32 rows is itself several hundred ulp away from the exact value, so
+fp32 results are held to |got - exact| <= 4 * log2(n) * eps32 * |exact| (softmax: all terms
+are non-negative, no cancellation; logsoftmax: scaled by max(1, |exact|)) against an fp64
+evaluation of the same formula, and the oracle is checked to lie within its own serial-sum
+error of that value.  fp64 results are compared with the oracle within
+(4 * log2(n) + sqrt(n)) * eps64."""
+import numpy as np
+import pytest
+from scipy.special import log_softmax as sp_log_softmax, softmax as sp_softmax
+
+from dlf_amd import frontend as F
+from dlf_amd.frontend import Tensor
+from helpers import normal, randint
+
+pytestmark = pytest.mark.gpu
+
+
+def check_rows(hip, orc, x, axis):
+    Xh, Xo = Tensor.from_numpy(hip, x), Tensor.from_numpy(orc, x)
+    m = int(np.prod(x.shape[:axis]))
+    n = x.size // m
+    eps = float(np.finfo(x.dtype).eps)
+    tiny = float(np.finfo(x.dtype).tiny)
+    gs = F.softmax(Xh, axis).numpy().astype(np.float64).reshape(m, n)
+    gl = F.logsoftmax(Xh, axis).numpy().astype(np.float64).reshape(m, n)
+    ws = F.softmax(Xo, axis).numpy().astype(np.float64).reshape(m, n)
+    wl = F.logsoftmax(Xo, axis).numpy().astype(np.float64).reshape(m, n)
+    if x.dtype == np.float32:
+        flat = x.reshape(m, n).astype(np.float64)
+        es, el = sp_softmax(flat, axis=1), sp_log_softmax(flat, axis=1)
+        bound = 4 * max(1.0, np.log2(n)) * eps
+        assert (np.abs(gs - es) <= bound * np.maximum(es, tiny)).all()
+        assert (np.abs(gl - el) <= bound * np.maximum(1.0, np.abs(el))).all()
+        serial = (n + 8) * eps                          # what a serial fp32 sum may be off by
+        assert (np.abs(ws - es) <= serial * np.maximum(es, tiny)).all()
+        assert (np.abs(wl - el) <= serial * np.maximum(1.0, np.abs(el))).all()
+    else:
+        bound = (4 * max(1.0, np.log2(n)) + np.sqrt(n)) * eps
+        assert (np.abs(gs - ws) <= bound * np.maximum(ws, tiny)).all()
+        assert (np.abs(gl - wl) <= bound * np.maximum(1.0, np.abs(wl))).all()
+    assert np.array_equal(F.hardmax(Xh, axis).numpy(), F.hardmax(Xo, axis).numpy())
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n", [1, 2, 7, 64, 65, 256, 1000, 1023, 2048, 2049, 8191, 16384, 32000, 32768, 40000, 100003])
+def test_rows_of_every_size_class(hip_backend, oracle_backend, dtype, n):
+    x = (normal(100 + n, 5 * n) * 4).astype(dtype).reshape(5, n)
+    check_rows(hip_backend, oracle_backend, x, 1)
+
+
+def test_axes_views_and_special_values(hip_backend, oracle_backend):
+    x = (normal(101, 6 * 10 * 33) * 2).astype(np.float32).reshape(6, 10, 33)
+    for axis in (0, 1, 2):
+        check_rows(hip_backend, oracle_backend, x, axis)
+    Xh, Xo = Tensor.from_numpy(hip_backend, x).transpose([1, 0, 2]), Tensor.from_numpy(oracle_backend, x).transpose([1, 0, 2])
+    assert np.allclose(F.softmax(Xh, 2).numpy(), F.softmax(Xo, 2).numpy(), rtol=1e-5, atol=1e-9)
+    # large magnitudes do not overflow (the row maximum is subtracted), -inf entries get weight 0
+    s = np.array([[10000.0, 10001.0, -np.inf, 10003.0], [-5.0, -np.inf, -np.inf, -5.0]], dtype=np.float32)
+    g = F.softmax(Tensor.from_numpy(hip_backend, s), 1).numpy()
+    w = F.softmax(Tensor.from_numpy(oracle_backend, s), 1).numpy()
+    assert np.allclose(g, w, rtol=1e-6) and g[0, 2] == 0 and np.allclose(g[1], [0.5, 0, 0, 0.5])
+    # rows far from zero: x - max must be formed before log(sum) is subtracted
+    big = (normal(103, 4 * 1000) * 2 + 30000).astype(np.float32).reshape(4, 1000)
+    check_rows(hip_backend, oracle_backend, big, 1)
+    # ties: the first maximum is the hot one (DNNTest.cpp:848-858); long rows of equal values too
+    t = np.full((3, 5000), 2.5, dtype=np.float32)
+    h = F.hardmax(Tensor.from_numpy(hip_backend, t), 1).numpy()
+    assert (h[:, 0] == 1).all() and h.sum() == 3
+
+
+def test_large_matrix_property(hip_backend):
+    # the benchmark shape at reduced height: rows sum to one, order is preserved
+    x = (normal(102, 64 * 32000) * 2).astype(np.float32).reshape(64, 32000)
+    y = F.softmax(Tensor.from_numpy(hip_backend, x), 1).numpy().astype(np.float64)
+    assert np.allclose(y.sum(axis=1), 1.0, atol=1e-5)
+    assert np.array_equal(np.argmax(y, axis=1), np.argmax(x, axis=1))

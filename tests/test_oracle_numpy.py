@@ -258,3 +258,26 @@ def test_merge_keeps_first_input_first_on_ties(oracle_backend):
     got = F.merge(T(oracle_backend, a), T(oracle_backend, b)).numpy()
     assert got.tolist() == [-1.0, 0.0, 0.0, 0.0, 0.0, 2.0, 2.0]
     assert np.signbit(got).tolist() == [True, False, False, True, True, False, False]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_softmax_family_matches_closed_forms(oracle_backend, dtype):
+    from scipy.special import softmax as sp_softmax, log_softmax as sp_log_softmax
+    x = (normal(50, 6 * 5 * 40) * 3).astype(dtype).reshape(6, 5, 40)
+    X = T(oracle_backend, x)
+    tol = 2e-6 if dtype == np.float32 else 1e-13
+    for axis in (0, 1, 2, -1):
+        a = axis % 3
+        m = int(np.prod(x.shape[:a]))
+        flat = x.reshape(m, -1).astype(np.float64)
+        assert np.allclose(F.softmax(X, axis).numpy().reshape(m, -1), sp_softmax(flat, axis=1), rtol=tol * 50, atol=tol)
+        assert np.allclose(F.logsoftmax(X, axis).numpy().reshape(m, -1), sp_log_softmax(flat, axis=1), rtol=tol * 50, atol=tol * 50)
+        hm = F.hardmax(X, axis).numpy().reshape(m, -1)
+        want = np.zeros_like(flat)
+        want[np.arange(m), flat.argmax(axis=1)] = 1
+        assert np.array_equal(hm, want)
+    # a transposed input is copied to row-major order first (dnn.h:452: reorder(X, Y))
+    Xt = X.transpose([2, 0, 1])
+    xt = x.transpose(2, 0, 1)
+    assert np.allclose(F.softmax(Xt, 1).numpy().reshape(40, -1), sp_softmax(xt.reshape(40, -1).astype(np.float64), axis=1),
+                       rtol=tol * 50, atol=tol)
