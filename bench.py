@@ -411,12 +411,55 @@ def cpu_baseline():
                       "3 repetitions, OpenMP rows/chunks in parallel"}
 
 
+def cpu_per_config():
+    """The CPU restatement timed on a bounded sample of every other configuration (--cpu-all):
+    the same shapes with fewer rows where a full run would take minutes."""
+    import numpy as np
+    from dlf_amd import frontend as F
+    from dlf_amd.frontend import Tensor
+    from oracle import oracle as O
+    be = O.OracleBackend()
+    rng = np.random.default_rng(3)
+    out = []
+
+    def timed(label, sample, nbytes, fn, reps=3):
+        fn()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        dt = (time.perf_counter() - t0) / reps
+        out.append({"op": label, "sample": sample, "us": round(dt * 1e6, 1), "gb_s": round(nbytes / dt / 1e9, 2)})
+
+    x1 = Tensor.from_numpy(be, rng.standard_normal((256, 1000), dtype=np.float32))
+    timed("C1 reduce_sum+max+lse+argmax+top_k5 [256,1000]", "full", 5 * 1024000,
+          lambda: (F.reduce_sum(x1, [1]), F.reduce_max(x1, [1]), F.reduce_log_sum_exp(x1, [1]), F.argmax(x1, 1),
+                   F.top_k(x1, 5, 1)), reps=20)
+    x3 = Tensor.from_numpy(be, (np.round(rng.standard_normal((512, 32000)) * 512) / 256).astype(np.float32))
+    for k in (1, 5, 50, 256):
+        timed("C3 top_k%d [4096,32000]" % k, "512 of 4096 rows", 4 * 512 * 32000, lambda k=k: F.top_k(x3, k, 1))
+    x4 = Tensor.from_numpy(be, (np.floor(rng.random((128, 65536)) * 4096) / 4096).astype(np.float32))
+    timed("C4a sort f32 [1024,65536]", "128 of 1024 rows", 8 * 128 * 65536, lambda: F.sort(x4, 1))
+    timed("C4a argsort f32 [1024,65536]", "128 of 1024 rows", 8 * 128 * 65536, lambda: F.argsort(x4, 1))
+    x4b = Tensor.from_numpy(be, rng.integers(-2 ** 63, 2 ** 63 - 1, size=(16, 1 << 20), dtype=np.int64))
+    timed("C4b sort i64 [256,2^20]", "16 of 256 rows", 16 * 16 * (1 << 20), lambda: F.sort(x4b, 1), reps=2)
+    timed("C4b argsort i64 [256,2^20]", "16 of 256 rows", 12 * 16 * (1 << 20), lambda: F.argsort(x4b, 1), reps=2)
+    x5 = Tensor.from_numpy(be, rng.standard_normal((8, 512, 56, 56), dtype=np.float32))
+    n5 = 8 * 512 * 56 * 56
+    timed("C5 reduce_mean{2,3} [32,512,56,56]", "8 of 32 images", 4 * n5, lambda: F.reduce_mean(x5, [2, 3]))
+    timed("C5 reduce_max{1}", "8 of 32 images", 4 * n5, lambda: F.reduce_max(x5, [1]))
+    timed("C5 argmax{1}", "8 of 32 images", 4 * n5, lambda: F.argmax(x5, 1))
+    timed("C5 cumsum{1}", "8 of 32 images", 8 * n5, lambda: F.cumsum(x5, 1))
+    return {"cores": O.threads(), "kind": "port", "ops": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3")
+    ap.add_argument("--cpu-all", action="store_true",
+                    help="also time the CPU restatement on a bounded sample of every configuration")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -502,6 +545,8 @@ def main():
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
+    if args.cpu_all:
+        result["cpu_per_config"] = cpu_per_config()
     print(json.dumps(result), flush=True)
 
 
