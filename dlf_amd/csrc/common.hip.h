@@ -82,10 +82,24 @@ struct Words {
     int w[N];
 };
 
+// Cross-lane helpers move whole 32-bit words; a 2-byte value rides in the low half of one.
+template <typename T>
+__device__ __forceinline__ int widen16(T v) {
+    static_assert(sizeof(T) == 2, "2-byte values only");
+    return static_cast<int>(bit_cast<unsigned short>(v));
+}
+template <typename T>
+__device__ __forceinline__ T narrow16(int w) {
+    return bit_cast<T>(static_cast<unsigned short>(w));
+}
+
 // Value of `v` in the lane the DPP control selects; lanes whose source is
 // outside the row (or masked off by ROW_MASK) receive `fill`.
 template <int CTRL, int ROW_MASK = 0xf, int BANK_MASK = 0xf, typename T>
 __device__ __forceinline__ T dpp_fetch(T v, T fill) {
+    if constexpr (sizeof(T) == 2) {
+        return narrow16<T>(__builtin_amdgcn_update_dpp(widen16(fill), widen16(v), CTRL, ROW_MASK, BANK_MASK, false));
+    } else {
     static_assert(sizeof(T) % 4 == 0, "whole 32-bit words only");
     constexpr int N = sizeof(T) / 4;
     Words<N> a = bit_cast<Words<N>>(v), f = bit_cast<Words<N>>(fill), r;
@@ -93,34 +107,47 @@ __device__ __forceinline__ T dpp_fetch(T v, T fill) {
     for (int i = 0; i < N; ++i)
         r.w[i] = __builtin_amdgcn_update_dpp(f.w[i], a.w[i], CTRL, ROW_MASK, BANK_MASK, false);
     return bit_cast<T>(r);
+    }
 }
 
 template <typename T>
 __device__ __forceinline__ T lane_xor(T v, int mask) {
-    constexpr int N = sizeof(T) / 4;
-    Words<N> a = bit_cast<Words<N>>(v);
+    if constexpr (sizeof(T) == 2) {
+        return narrow16<T>(__shfl_xor(widen16(v), mask, kWave));
+    } else {
+        constexpr int N = sizeof(T) / 4;
+        Words<N> a = bit_cast<Words<N>>(v);
 #pragma unroll
-    for (int i = 0; i < N; ++i) a.w[i] = __shfl_xor(a.w[i], mask, kWave);
-    return bit_cast<T>(a);
+        for (int i = 0; i < N; ++i) a.w[i] = __shfl_xor(a.w[i], mask, kWave);
+        return bit_cast<T>(a);
+    }
 }
 
 template <typename T>
 __device__ __forceinline__ T lane_get(T v, int lane) {
-    constexpr int N = sizeof(T) / 4;
-    Words<N> a = bit_cast<Words<N>>(v);
+    if constexpr (sizeof(T) == 2) {
+        return narrow16<T>(__shfl(widen16(v), lane, kWave));
+    } else {
+        constexpr int N = sizeof(T) / 4;
+        Words<N> a = bit_cast<Words<N>>(v);
 #pragma unroll
-    for (int i = 0; i < N; ++i) a.w[i] = __shfl(a.w[i], lane, kWave);
-    return bit_cast<T>(a);
+        for (int i = 0; i < N; ++i) a.w[i] = __shfl(a.w[i], lane, kWave);
+        return bit_cast<T>(a);
+    }
 }
 
 // Broadcast of one lane's value through a scalar register (lane is uniform).
 template <typename T>
 __device__ __forceinline__ T lane_read(T v, int lane) {
-    constexpr int N = sizeof(T) / 4;
-    Words<N> a = bit_cast<Words<N>>(v);
+    if constexpr (sizeof(T) == 2) {
+        return narrow16<T>(__builtin_amdgcn_readlane(widen16(v), lane));
+    } else {
+        constexpr int N = sizeof(T) / 4;
+        Words<N> a = bit_cast<Words<N>>(v);
 #pragma unroll
-    for (int i = 0; i < N; ++i) a.w[i] = __builtin_amdgcn_readlane(a.w[i], lane);
-    return bit_cast<T>(a);
+        for (int i = 0; i < N; ++i) a.w[i] = __builtin_amdgcn_readlane(a.w[i], lane);
+        return bit_cast<T>(a);
+    }
 }
 
 // DPP controls used below.
@@ -301,10 +328,31 @@ inline int dispatch_dtype(int dtype, F&& f) {
     }
 }
 
+using half_t = _Float16;      // IEEE half as a native scalar type
+
+// The four wide types plus half.
+template <typename F>
+inline int dispatch_dtype_half(int dtype, F&& f) {
+    if (dtype == DLFX_F16) return f(half_t());
+    return dispatch_dtype(dtype, f);
+}
+
+// The four wide types plus the two 16-bit ones.
+template <typename F>
+inline int dispatch_dtype16(int dtype, F&& f) {
+    switch (dtype) {
+    case DLFX_F16: return f(half_t());
+    case DLFX_I16: return f(int16_t());
+    default: return dispatch_dtype(dtype, f);
+    }
+}
+
 inline size_t dtype_size(int dtype) {
     switch (dtype) {
     case DLFX_F32: case DLFX_I32: return 4;
     case DLFX_F64: case DLFX_I64: return 8;
+    case DLFX_F16: case DLFX_I16: return 2;
+    case DLFX_BOOL: return 1;
     default: return 0;
     }
 }

@@ -215,7 +215,7 @@ int launch_merge(hipStream_t stream, int dir, int64_t m, const MergeViews& v, co
 using namespace dlfx;
 
 extern "C" size_t dlfx_merge_scratch_bytes(int dtype, int64_t m, int64_t n) {
-    if (!dtype_size(dtype) || m <= 0 || n <= 0) return 0;
+    if (!dtype_size(dtype) || dtype == DLFX_BOOL || m <= 0 || n <= 0) return 0;
     return merge_layout(dtype_size(dtype), m, n).total;
 }
 
@@ -243,7 +243,8 @@ extern "C" int dlfx_merge(dlfx_stream_t stream, int dir, int dtype, int rank,
     v.na = na;
     v.nb = nb;
     const int64_t m = view_size(rank, z_dims) / z_dims[rank - 1];
-    return dispatch_dtype(dtype, [&](auto tag) {
+    if (dtype == DLFX_BOOL) return DLFX_ERR_UNSUPPORTED_DTYPE;
+    return dispatch_dtype16(dtype, [&](auto tag) {
         using T = decltype(tag);
         return launch_merge<T>(static_cast<hipStream_t>(stream), dir, m, v, static_cast<const T*>(x) + x_offset,
                                static_cast<const T*>(y) + y_offset, static_cast<T*>(z) + z_offset, scratch, scratch_bytes);

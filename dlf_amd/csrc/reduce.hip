@@ -30,6 +30,19 @@ template <typename T, int J>
 struct AccType { using type = T; };
 template <> struct AccType<float, kAdd> { using type = double; };
 template <> struct AccType<float, kMul> { using type = double; };
+template <int J> struct AccType<half_t, J> { using type = float; };       // half: every fold in fp32, one rounding at the end
+
+// numeric_limits for the element types (the host library has none for half)
+template <typename T> struct Limits {
+    __host__ __device__ static constexpr T lowest() { return std::numeric_limits<T>::lowest(); }
+    __host__ __device__ static constexpr T max() { return std::numeric_limits<T>::max(); }
+    __host__ __device__ static constexpr T infinity() { return std::numeric_limits<T>::infinity(); }
+};
+template <> struct Limits<half_t> {
+    __host__ __device__ static constexpr half_t lowest() { return static_cast<half_t>(-65504.0f); }
+    __host__ __device__ static constexpr half_t max() { return static_cast<half_t>(65504.0f); }
+    __host__ __device__ static constexpr half_t infinity() { return static_cast<half_t>(__builtin_inff()); }
+};
 
 template <typename T>
 __device__ __forceinline__ T wrap_add(T a, T b) {
@@ -61,19 +74,19 @@ struct ValueReducer {
     __device__ static __forceinline__ acc_t identity() {
         if constexpr (J == kAdd) return acc_t(0);
         else if constexpr (J == kMul) return acc_t(1);
-        else if constexpr (J == kMax) return (M == kMapAbs) ? acc_t(0) : std::numeric_limits<T>::lowest();
-        else return std::numeric_limits<T>::max();
+        else if constexpr (J == kMax) return (M == kMapAbs) ? acc_t(0) : static_cast<acc_t>(Limits<T>::lowest());
+        else return static_cast<acc_t>(Limits<T>::max());
     }
     __device__ static __forceinline__ acc_t map(T x, int64_t, param_t) {
         if constexpr (M == kMapExp) {
-            if constexpr (std::is_same<T, float>::value) return static_cast<acc_t>(expf(x));
+            if constexpr (std::is_same<T, float>::value || std::is_same<T, half_t>::value) return static_cast<acc_t>(expf(static_cast<float>(x)));
             else return static_cast<acc_t>(exp(static_cast<double>(x)));
         } else if constexpr (M == kMapAbs) {
             if constexpr (std::is_integral<T>::value) {
                 using U = typename std::make_unsigned<T>::type;
                 return x < 0 ? static_cast<T>(U(0) - static_cast<U>(x)) : x;
             } else {
-                return static_cast<acc_t>(x < 0 ? -x : x);
+                return x < T(0) ? -static_cast<acc_t>(x) : static_cast<acc_t>(x);
             }
         } else if constexpr (M == kMapSquare) {
             acc_t v = static_cast<acc_t>(x);
@@ -126,14 +139,14 @@ struct ArgReducer {
             return {MAX ? std::numeric_limits<T>::lowest() : std::numeric_limits<T>::max(),
                     std::numeric_limits<int32_t>::max()};
         else
-            return {MAX ? -std::numeric_limits<T>::infinity() : std::numeric_limits<T>::infinity(),
+            return {MAX ? static_cast<T>(-Limits<T>::infinity()) : Limits<T>::infinity(),
                     std::numeric_limits<int32_t>::max()};
     }
     __device__ static __forceinline__ acc_t map(T x, int64_t j, param_t) {
         if constexpr (!std::is_integral<T>::value) {
             if (x != x) {
                 if (j == 0)
-                    return {MAX ? std::numeric_limits<T>::infinity() : -std::numeric_limits<T>::infinity(), -1};
+                    return {MAX ? Limits<T>::infinity() : static_cast<T>(-Limits<T>::infinity()), -1};
                 return identity();
             }
         }
@@ -525,6 +538,7 @@ extern "C" int dlfx_reduce(dlfx_stream_t stream, const char* name, int dtype, in
         if (!std::strcmp(o.name, name)) op = &o;
     if (!op) return DLFX_ERR_UNKNOWN_OP;
     if (op->float_only && (dtype == DLFX_I32 || dtype == DLFX_I64)) return DLFX_ERR_UNSUPPORTED_DTYPE;
+    if (dtype == DLFX_I16 || dtype == DLFX_BOOL) return DLFX_ERR_UNSUPPORTED_DTYPE;        // as the reference's instantiations
 
     // the reduced extents are the trailing dimensions whose product is n
     int split = x_rank;
@@ -540,7 +554,7 @@ extern "C" int dlfx_reduce(dlfx_stream_t stream, const char* name, int dtype, in
         !make_dim_map(y_dims, y_strides, 0, y_rank, &pl.ymap))
         return DLFX_ERR_RANK;
 
-    return dispatch_dtype(dtype, [&](auto tag) {
+    return dispatch_dtype_half(dtype, [&](auto tag) {
         using T = decltype(tag);
         return launch_reduce_typed<T>(static_cast<hipStream_t>(stream), *op, pl,
                                       static_cast<const T*>(x) + x_offset, static_cast<T*>(y) + y_offset,
@@ -573,6 +587,7 @@ extern "C" int dlfx_arg_reduce(dlfx_stream_t stream, const char* name, int dtype
     else if (!std::strcmp(name, "argmin")) want_max = false;
     else return DLFX_ERR_UNKNOWN_OP;
     if (index_dtype != DLFX_I32 && index_dtype != DLFX_I64) return DLFX_ERR_UNSUPPORTED_DTYPE;
+    if (dtype == DLFX_BOOL) return DLFX_ERR_UNSUPPORTED_DTYPE;
 
     ReducePlan pl;
     pl.m = n_rows;
@@ -583,7 +598,7 @@ extern "C" int dlfx_arg_reduce(dlfx_stream_t stream, const char* name, int dtype
         return DLFX_ERR_RANK;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return dispatch_dtype(dtype, [&](auto tag) {
+    return dispatch_dtype16(dtype, [&](auto tag) {
         using T = decltype(tag);
         const T* xp = static_cast<const T*>(x) + x_offset;
         if (index_dtype == DLFX_I32) {
@@ -614,6 +629,7 @@ extern "C" int dlfx_count(dlfx_stream_t stream, int dtype, int64_t m, int64_t n,
         return DLFX_ERR_INVALID_ARGUMENT;
     if (view_size(x_rank, x_dims) != m * n || view_size(y_rank, y_dims) != m) return DLFX_ERR_INVALID_ARGUMENT;
     if (n > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;       // counts are 32-bit, as in the reference
+    if (dtype == DLFX_I16 || dtype == DLFX_BOOL) return DLFX_ERR_UNSUPPORTED_DTYPE;
 
     int split = x_rank;
     int64_t prod = 1;
@@ -628,7 +644,7 @@ extern "C" int dlfx_count(dlfx_stream_t stream, int dtype, int64_t m, int64_t n,
         !make_dim_map(y_dims, y_strides, 0, y_rank, &pl.ymap))
         return DLFX_ERR_RANK;
 
-    return dispatch_dtype(dtype, [&](auto tag) {
+    return dispatch_dtype_half(dtype, [&](auto tag) {
         using T = decltype(tag);
         T v;
         std::memcpy(&v, value, sizeof(T));

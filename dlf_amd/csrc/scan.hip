@@ -136,9 +136,10 @@ struct RowScanShared {
 // One tile: tile `t` of row `row`.  Element order inside a tile: wave w owns
 // [w*64*ITEMS, (w+1)*64*ITEMS); within it, vector k of lane l covers elements
 // (k*64 + l)*V .. +V.  CHAINED tiles publish / look back through `st`.
-template <typename T, int K, int ITEMS, bool CHAINED, bool SELF_HELP, int BLOCK = kBlock, typename X = T, bool NZ = false>
+template <typename T, int K, int ITEMS, bool CHAINED, bool SELF_HELP, int BLOCK = kBlock, typename X = T, bool NZ = false,
+          typename Y = T>
 __device__ __forceinline__ void scan_tile(
-    const X* __restrict__ x, T* __restrict__ y, const DimMap& xmap, const DimMap& ymap, int64_t sx, int64_t sy,
+    const X* __restrict__ x, Y* __restrict__ y, const DimMap& xmap, const DimMap& ymap, int64_t sx, int64_t sy,
     const DimMap& xaxis, int64_t n, int64_t tiles_per_row, int exclusive, int64_t row, int64_t t, int poll_limit,
     TileState<T>& st, RowScanShared<T>& sm) {
     // where element i of a row lives: i * sx, or (scan_nonzero over a flattened view whose
@@ -151,7 +152,6 @@ __device__ __forceinline__ void scan_tile(
     constexpr int V = (vec_width<T>() < ITEMS) ? vec_width<T>() : ITEMS;
     constexpr int KV = ITEMS / V;
     constexpr int64_t TILE = static_cast<int64_t>(BLOCK) * ITEMS;
-    using VecT = Vec<T, V>;
     using VecX = Vec<X, V>;
 
     const int lane = lane_id();
@@ -160,7 +160,7 @@ __device__ __forceinline__ void scan_tile(
     const int64_t avail = (n - tile_base < TILE) ? n - tile_base : TILE;   // valid elements in this tile
 
     const X* xr = x + xmap.at(row);
-    T* yr = y + ymap.at(row);
+    Y* yr = y + ymap.at(row);
     const int64_t seg = tile_base + static_cast<int64_t>(w) * kWave * ITEMS;
 
     // ---- load
@@ -291,14 +291,15 @@ __device__ __forceinline__ void scan_tile(
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) vals[i] = Op::apply(pre, vals[i]);
 
-    const bool y_vec = full && sy == 1 && (reinterpret_cast<uintptr_t>(yr + seg) % (sizeof(T) * V) == 0);
+    using VecY = Vec<Y, V>;
+    const bool y_vec = full && sy == 1 && (reinterpret_cast<uintptr_t>(yr + seg) % (sizeof(Y) * V) == 0);
     if (y_vec) {
-        VecT* pv = reinterpret_cast<VecT*>(yr + seg);
+        VecY* pv = reinterpret_cast<VecY*>(yr + seg);
 #pragma unroll
         for (int k = 0; k < KV; ++k) {
-            VecT a;
+            VecY a;
 #pragma unroll
-            for (int e = 0; e < V; ++e) a.v[e] = vals[k * V + e];
+            for (int e = 0; e < V; ++e) a.v[e] = static_cast<Y>(vals[k * V + e]);
             store_stream(&pv[k * kWave + lane], a);
         }
     } else {
@@ -307,28 +308,28 @@ __device__ __forceinline__ void scan_tile(
 #pragma unroll
             for (int e = 0; e < V; ++e) {
                 const int64_t i = seg + static_cast<int64_t>(k * kWave + lane) * V + e;
-                if (i < n) yr[i * sy] = vals[k * V + e];
+                if (i < n) yr[i * sy] = static_cast<Y>(vals[k * V + e]);
             }
     }
 }
 
 // Rows of a single tile: workgroup b scans row b.
-template <typename T, int K, int ITEMS, typename X, bool NZ>
+template <typename T, int K, int ITEMS, typename X, bool NZ, typename Y>
 __global__ __launch_bounds__(kBlock) void scan_rows_single(
-    const X* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy, DimMap xaxis,
+    const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy, DimMap xaxis,
     int64_t n, int exclusive) {
     __shared__ RowScanShared<T> sm;
     TileState<T> st;
-    scan_tile<T, K, ITEMS, false, false, kBlock, X, NZ>(x, y, xmap, ymap, sx, sy, xaxis, n, 1, exclusive, blockIdx.x, 0, 0, st, sm);
+    scan_tile<T, K, ITEMS, false, false, kBlock, X, NZ, Y>(x, y, xmap, ymap, sx, sy, xaxis, n, 1, exclusive, blockIdx.x, 0, 0, st, sm);
 }
 
 // Rows of several tiles.  Workgroup b belongs to row b / tiles_per_row.  With
 // TICKET the tile of the row is drawn from that row's atomic counter (in-place
 // scans); without, it is the workgroup's position in the row and waits are
 // bounded by self-help.
-template <typename T, int K, int ITEMS, bool TICKET, int BLOCK, typename X, bool NZ>
+template <typename T, int K, int ITEMS, bool TICKET, int BLOCK, typename X, bool NZ, typename Y>
 __global__ __launch_bounds__(BLOCK) void scan_rows_chained(
-    const X* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy, DimMap xaxis,
+    const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy, DimMap xaxis,
     int64_t n, int64_t tiles_per_row, int exclusive, int poll_limit, unsigned* ticket, TileState<T> st) {
     __shared__ RowScanShared<T> sm;
     const int64_t row = blockIdx.x / tiles_per_row;
@@ -338,16 +339,16 @@ __global__ __launch_bounds__(BLOCK) void scan_rows_chained(
         __syncthreads();
         t = sm.next_tile;
     }
-    scan_tile<T, K, ITEMS, true, !TICKET, BLOCK, X, NZ>(x, y, xmap, ymap, sx, sy, xaxis, n, tiles_per_row, exclusive, row, t, poll_limit, st, sm);
+    scan_tile<T, K, ITEMS, true, !TICKET, BLOCK, X, NZ, Y>(x, y, xmap, ymap, sx, sy, xaxis, n, tiles_per_row, exclusive, row, t, poll_limit, st, sm);
 }
 
 // ------------------------------------------------------------------ column kernel
 // One lane per row ("column"), four waves along the scanned axis.  Each pass of
 // the loop covers kWaves * chunk positions of the axis: thread (lx, ty) scans
 // positions [s + ty*chunk, s + (ty+1)*chunk) in registers.
-template <typename T, int K, typename X, bool NZ>
+template <typename T, int K, typename X, bool NZ, typename Y>
 __global__ __launch_bounds__(kBlock) void scan_cols(
-    const X* __restrict__ x, T* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
+    const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
     int64_t m, int64_t n, int chunk, int exclusive) {
     using Op = ScanOp<T, K>;
     constexpr int R = 16;
@@ -358,7 +359,7 @@ __global__ __launch_bounds__(kBlock) void scan_cols(
     const int64_t col = static_cast<int64_t>(blockIdx.x) * kWave + lx;
     const bool live = col < m;
     const X* xc = x + (live ? xmap.at(col) : 0);
-    T* yc = y + (live ? ymap.at(col) : 0);
+    Y* yc = y + (live ? ymap.at(col) : 0);
 
     T carry = Op::identity();
     int buf = 0;
@@ -389,13 +390,13 @@ __global__ __launch_bounds__(kBlock) void scan_cols(
                 for (int r = 0; r < R; ++r) {
                     const int64_t p = p0 + r;
                     const T prev = (r == 0) ? pre : Op::apply(pre, v[r > 0 ? r - 1 : 0]);
-                    if (r < chunk && p < n) store_stream(&yc[p * sy], prev);
+                    if (r < chunk && p < n) store_stream(&yc[p * sy], static_cast<Y>(prev));
                 }
             } else {
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const int64_t p = p0 + r;
-                    if (r < chunk && p < n) store_stream(&yc[p * sy], Op::apply(pre, v[r]));
+                    if (r < chunk && p < n) store_stream(&yc[p * sy], static_cast<Y>(Op::apply(pre, v[r])));
                 }
             }
         }
@@ -488,9 +489,9 @@ bool views_overlap(int rank, const int64_t* dims, const X* x, const int64_t* sx,
     return xb < ye && yb < xe;
 }
 
-template <typename T, int K, typename X = T, bool NZ = false>
+template <typename T, int K, typename X = T, bool NZ = false, typename Y = T>
 int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int rank, const int64_t* dims,
-                const X* x, const int64_t* x_strides, T* y, const int64_t* y_strides,
+                const X* x, const int64_t* x_strides, Y* y, const int64_t* y_strides,
                 void* scratch, size_t scratch_bytes, const DimMap* x_axis = nullptr) {
     DimMap xmap, ymap;
     if (!make_dim_map2(dims, x_strides, y_strides, rank - 1, &xmap, &ymap)) return DLFX_ERR_RANK;
@@ -520,7 +521,7 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
         int chunk = static_cast<int>(ceil_div(n, kWaves) < 16 ? ceil_div(n, kWaves) : 16);
         const int64_t blocks = ceil_div(m, kWave);
         if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
-        scan_cols<T, K, X, NZ><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
+        scan_cols<T, K, X, NZ, Y><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
             x, y, xmap, ymap, sx, sy, m, n, chunk, exclusive);
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
@@ -535,13 +536,13 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     if (l.tiles_per_row == 1) {
         const dim3 grid(static_cast<unsigned>(m));
         if (tile == 256)
-            scan_rows_single<T, K, 1, X, NZ><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
+            scan_rows_single<T, K, 1, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
         else if (tile == 1024)
-            scan_rows_single<T, K, 4, X, NZ><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
+            scan_rows_single<T, K, 4, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
         else if (tile == 256 * (FULL / 4))
-            scan_rows_single<T, K, FULL / 4, X, NZ><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
+            scan_rows_single<T, K, FULL / 4, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
         else
-            scan_rows_single<T, K, FULL, X, NZ><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
+            scan_rows_single<T, K, FULL, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
     }
@@ -554,10 +555,10 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     constexpr int CI = static_cast<int>(kChainTileBytes / sizeof(T) / kChainBlock);
     const dim3 cblock(kChainBlock);
     if (views_overlap(rank, dims, x, x_strides, y, y_strides))
-        scan_rows_chained<T, K, CI, true, kChainBlock, X, NZ><<<grid, cblock, 0, stream>>>(
+        scan_rows_chained<T, K, CI, true, kChainBlock, X, NZ, Y><<<grid, cblock, 0, stream>>>(
             x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st);
     else
-        scan_rows_chained<T, K, CI, false, kChainBlock, X, NZ><<<grid, cblock, 0, stream>>>(
+        scan_rows_chained<T, K, CI, false, kChainBlock, X, NZ, Y><<<grid, cblock, 0, stream>>>(
             x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st);
     DLFX_CHECK_LAUNCH();
     return DLFX_OK;
@@ -579,8 +580,9 @@ bool set_scan_tuning(const char* key, int64_t value) {
 }  // namespace dlfx
 
 extern "C" size_t dlfx_scan_scratch_bytes(int dtype, int64_t m, int64_t n) {
-    const size_t es = dtype_size(dtype);
-    if (!es || m <= 0 || n <= 0) return 0;
+    size_t es = dtype_size(dtype);
+    if (dtype == DLFX_F16) es = 4;                  // scanned as fp32
+    if (es < 4 || m <= 0 || n <= 0) return 0;
     return scan_layout(es, m, n).total;
 }
 
@@ -599,6 +601,17 @@ extern "C" int dlfx_scan(dlfx_stream_t stream, const char* name, int dtype, int6
     else if (!std::strcmp(name, "cummin")) kind = kScanMin;
     else return DLFX_ERR_UNKNOWN_OP;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == DLFX_F16) {
+        // half elements are scanned in fp32: one rounding per output instead of one per step
+        const half_t* xp = static_cast<const half_t*>(x) + x_offset;
+        half_t* yp = static_cast<half_t*>(y) + y_offset;
+        switch (kind) {
+        case kScanAdd: return launch_scan<float, kScanAdd, half_t, false, half_t>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
+        case kScanMul: return launch_scan<float, kScanMul, half_t, false, half_t>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
+        case kScanMax: return launch_scan<float, kScanMax, half_t, false, half_t>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
+        default:       return launch_scan<float, kScanMin, half_t, false, half_t>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
+        }
+    }
     return dispatch_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
         const T* xp = static_cast<const T*>(x) + x_offset;
@@ -652,9 +665,13 @@ extern "C" int dlfx_scan_nonzero(dlfx_stream_t stream, int dtype, int64_t m, int
     xs2[split] = xaxis.rank == 1 ? xaxis.strides[0] : 0;
     ys2[split] = yaxis.rank == 1 ? yaxis.strides[0] : 1;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return dispatch_dtype(dtype, [&](auto tag) {
+    auto run = [&](auto tag) {
         using X = decltype(tag);
         return launch_scan<int32_t, kScanAdd, X, true>(s, m, n, exclusive, split + 1, d2, static_cast<const X*>(x) + x_offset,
                                                        xs2, y + y_offset, ys2, scratch, scratch_bytes, &xaxis);
-    });
+    };
+    if (dtype == DLFX_F16) return run(half_t());
+    if (dtype == DLFX_BOOL) return run(uint8_t());
+    if (dtype == DLFX_I16) return DLFX_ERR_UNSUPPORTED_DTYPE;
+    return dispatch_dtype(dtype, run);
 }

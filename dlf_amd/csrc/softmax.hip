@@ -7,7 +7,8 @@
 // up to 2048 elements, a 1024-thread workgroup up to 32768 four-byte elements) between the
 // load, the two team-wide reductions and the store.  Longer rows are streamed twice (running
 // maximum and rescaled sum first, then the outputs).  Bandwidth bound; exp and log in the
-// element type, sums in it as well (tree order), as the reference's row loops do.
+// element type, sums in it as well (tree order), as the reference's row loops do.  IEEE half
+// rows are widened to float at the load and rounded once at the store.
 #include <cmath>
 #include <cstring>
 #include <limits>
@@ -19,6 +20,10 @@ namespace dlfx {
 namespace {
 
 enum SoftKind { kSoftmax = 0, kLogSoftmax = 1, kHardmax = 2 };
+
+// The arithmetic type for rows stored as S.
+template <typename S> struct ComputeOf { using type = S; };
+template <> struct ComputeOf<half_t> { using type = float; };
 
 template <typename T> __device__ __forceinline__ T exp_of(T v);
 template <> __device__ __forceinline__ float exp_of<float>(float v) { return expf(v); }
@@ -69,23 +74,23 @@ __device__ __forceinline__ V team_reduce(V v, Join join, V* lds) {
 
 // Rows held in registers.  TEAM threads per row, ITEMS elements per thread; element (k, t) of
 // the row is ((k / V) * TEAM + t) * V + k % V with V elements per 128-bit access when VEC.
-template <typename T, int TEAM, int ITEMS, int KIND, bool VEC>
+template <typename S, int TEAM, int ITEMS, int KIND, bool VEC>
 __global__ __launch_bounds__(TEAM > 256 ? TEAM : 256)
-__attribute__((amdgpu_waves_per_eu(TEAM >= 1024 && sizeof(T) * ITEMS <= 128 ? 8 : 1)))      // two 1024-thread rows per CU
-void softmax_rows(const T* __restrict__ x, T* __restrict__ y,
-                                                                        int64_t m, int64_t n) {
+__attribute__((amdgpu_waves_per_eu(TEAM >= 1024 && sizeof(typename ComputeOf<S>::type) * ITEMS <= 128 ? 8 : 1)))      // two 1024-thread rows per CU
+void softmax_rows(const S* __restrict__ x, S* __restrict__ y, int64_t m, int64_t n) {
+    using T = typename ComputeOf<S>::type;
     constexpr int BLOCK = TEAM > 256 ? TEAM : 256;
-    constexpr int V = VEC ? 16 / static_cast<int>(sizeof(T)) : 1;
+    constexpr int V = VEC ? 16 / static_cast<int>(sizeof(S)) : 1;
     static_assert(ITEMS % V == 0, "whole vectors per thread");
     constexpr int G = ITEMS / V;
-    using VecT = Vec<T, V>;
+    using VecT = Vec<S, V>;
     __shared__ alignas(16) unsigned char lds_raw[(TEAM > kWave ? TEAM / kWave : 1) * sizeof(MaxAt<T>)];
 
     const int t = threadIdx.x % TEAM;
     const int64_t row = static_cast<int64_t>(blockIdx.x) * (BLOCK / TEAM) + threadIdx.x / TEAM;
     const bool live = row < m;                           // whole teams are live or not
-    const T* xr = x + (live ? row : 0) * n;
-    T* yr = y + (live ? row : 0) * n;
+    const S* xr = x + (live ? row : 0) * n;
+    S* yr = y + (live ? row : 0) * n;
     const T lowest = -std::numeric_limits<T>::infinity();
     const int32_t n32 = static_cast<int32_t>(n);          // rows here have at most 32768 elements
     auto index_of = [&](int k) -> int32_t { return ((k / V) * TEAM + t) * V + k % V; };
@@ -98,13 +103,13 @@ void softmax_rows(const T* __restrict__ x, T* __restrict__ y,
             if (live && i0 < n) {                         // n is a multiple of V here
                 const VecT a = load_stream(reinterpret_cast<const VecT*>(xr + i0));
 #pragma unroll
-                for (int e = 0; e < V; ++e) v[g * V + e] = a.v[e];
+                for (int e = 0; e < V; ++e) v[g * V + e] = static_cast<T>(a.v[e]);
             } else {
 #pragma unroll
                 for (int e = 0; e < V; ++e) v[g * V + e] = lowest;
             }
         } else {
-            v[g] = (live && i0 < n) ? load_stream(&xr[i0]) : lowest;
+            v[g] = (live && i0 < n) ? static_cast<T>(load_stream(&xr[i0])) : lowest;
         }
     }
 
@@ -131,7 +136,7 @@ void softmax_rows(const T* __restrict__ x, T* __restrict__ y,
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) mx = (mx < v[k]) ? v[k] : mx;
         mx = team_reduce<TEAM>(mx, [](T a, T b) { return (a < b) ? b : a; }, reinterpret_cast<T*>(lds_raw));
-        if (live && xr[0] != xr[0]) mx = xr[0];
+        if (live && xr[0] != xr[0]) mx = static_cast<T>(xr[0]);
         T sum = T(0);
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
@@ -159,36 +164,37 @@ void softmax_rows(const T* __restrict__ x, T* __restrict__ y,
             if (VEC) {
                 VecT a;
 #pragma unroll
-                for (int e = 0; e < V; ++e) a.v[e] = v[g * V + e];
+                for (int e = 0; e < V; ++e) a.v[e] = static_cast<S>(v[g * V + e]);
                 store_stream(reinterpret_cast<VecT*>(yr + i0), a);
             } else {
-                store_stream(&yr[i0], v[g]);
+                store_stream(&yr[i0], static_cast<S>(v[g]));
             }
         }
     }
 }
 
 // Rows too long for registers: one 1024-thread workgroup per row, two passes over the row.
-template <typename T, int KIND>
-__global__ __launch_bounds__(1024) void softmax_rows_streamed(const T* __restrict__ x, T* __restrict__ y, int64_t n) {
+template <typename S, int KIND>
+__global__ __launch_bounds__(1024) void softmax_rows_streamed(const S* __restrict__ x, S* __restrict__ y, int64_t n) {
+    using T = typename ComputeOf<S>::type;
     constexpr int TEAM = 1024;
     __shared__ alignas(16) unsigned char lds_raw[(TEAM / kWave) * sizeof(MaxAt<T>)];
     const int t = threadIdx.x;
-    const T* xr = x + static_cast<int64_t>(blockIdx.x) * n;
-    T* yr = y + static_cast<int64_t>(blockIdx.x) * n;
+    const S* xr = x + static_cast<int64_t>(blockIdx.x) * n;
+    S* yr = y + static_cast<int64_t>(blockIdx.x) * n;
     const T lowest = -std::numeric_limits<T>::infinity();
     if constexpr (KIND == kHardmax) {
         MaxAt<T> best = {lowest, std::numeric_limits<int32_t>::max()};
-        for (int64_t i = t; i < n; i += TEAM) best = max_at_join(best, max_at_of(xr[i], i));
+        for (int64_t i = t; i < n; i += TEAM) best = max_at_join(best, max_at_of(static_cast<T>(xr[i]), i));
         best = team_reduce<TEAM>(best, [](MaxAt<T> a, MaxAt<T> b) { return max_at_join(a, b); },
                                  reinterpret_cast<MaxAt<T>*>(lds_raw));
         const int64_t hot = best.i < 0 ? 0 : best.i;
-        for (int64_t i = t; i < n; i += TEAM) yr[i] = i == hot ? T(1) : T(0);
+        for (int64_t i = t; i < n; i += TEAM) yr[i] = i == hot ? S(1) : S(0);
     } else {
         // running maximum and the sum of exp(x - maximum), rescaled whenever the maximum moves
         T mx = lowest, sum = T(0);
         for (int64_t i = t; i < n; i += TEAM) {
-            const T xv = xr[i];
+            const T xv = static_cast<T>(xr[i]);
             if (mx < xv) {
                 sum = sum * exp_of<T>(mx - xv);          // exp(-inf) = 0 on the first element
                 mx = xv;
@@ -197,12 +203,12 @@ __global__ __launch_bounds__(1024) void softmax_rows_streamed(const T* __restric
         }
         T row_max = team_reduce<TEAM>(mx, [](T a, T b) { return (a < b) ? b : a; }, reinterpret_cast<T*>(lds_raw));
         sum = (mx == lowest) ? T(0) : sum * exp_of<T>(mx - row_max);
-        if (xr[0] != xr[0]) row_max = xr[0];             // a NaN in position 0 is the reference's maximum
+        if (xr[0] != xr[0]) row_max = static_cast<T>(xr[0]);             // a NaN in position 0 is the reference's maximum
         sum = team_reduce<TEAM>(sum, [](T a, T b) { return a + b; }, reinterpret_cast<T*>(lds_raw));
         const T lsum = log_of<T>(sum);
         for (int64_t i = t; i < n; i += TEAM) {
-            const T xv = xr[i];
-            yr[i] = KIND == kSoftmax ? exp_of<T>(xv - row_max) / sum : (xv - row_max) - lsum;
+            const T xv = static_cast<T>(xr[i]);
+            yr[i] = static_cast<S>(KIND == kSoftmax ? exp_of<T>(xv - row_max) / sum : (xv - row_max) - lsum);
         }
     }
 }
@@ -210,6 +216,7 @@ __global__ __launch_bounds__(1024) void softmax_rows_streamed(const T* __restric
 template <typename T, int KIND>
 int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y) {
     constexpr int V = 16 / static_cast<int>(sizeof(T));
+    constexpr int kRegisterBytes = static_cast<int>(sizeof(typename ComputeOf<T>::type));
     const bool vec = n % V == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
     // wavefront teams: 4 rows per workgroup
 #define DLFX_WAVE_ROWS(ITEMS)                                                                                   \
@@ -234,7 +241,7 @@ int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y) {
     if (n <= kWave * 32) DLFX_WAVE_ROWS(32);
     if (n <= 1024 * 8) DLFX_BLOCK_ROWS(8);
     if (n <= 1024 * 16) DLFX_BLOCK_ROWS(16);
-    if (n <= 1024 * 32 && sizeof(T) == 4) DLFX_BLOCK_ROWS(32);
+    if (n <= 1024 * 32 && kRegisterBytes == 4) DLFX_BLOCK_ROWS(32);
 #undef DLFX_WAVE_ROWS
 #undef DLFX_BLOCK_ROWS
     softmax_rows_streamed<T, KIND><<<dim3(static_cast<unsigned>(m)), dim3(1024), 0, stream>>>(x, y, n);
@@ -256,7 +263,7 @@ extern "C" int dlfx_softmax(dlfx_stream_t stream, const char* name, int dtype, i
     else if (!std::strcmp(name, "logsoftmax")) kind = kLogSoftmax;
     else if (!std::strcmp(name, "hardmax")) kind = kHardmax;
     else return DLFX_ERR_UNKNOWN_OP;
-    if (dtype != DLFX_F32 && dtype != DLFX_F64) return DLFX_ERR_UNSUPPORTED_DTYPE;
+    if (dtype != DLFX_F32 && dtype != DLFX_F64 && dtype != DLFX_F16) return DLFX_ERR_UNSUPPORTED_DTYPE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     auto run = [&](auto tag) {
         using T = decltype(tag);
@@ -268,5 +275,5 @@ extern "C" int dlfx_softmax(dlfx_stream_t stream, const char* name, int dtype, i
         default: return launch_softmax<T, kHardmax>(s, m, n, xp, yp);
         }
     };
-    return dtype == DLFX_F32 ? run(float()) : run(double());
+    return dtype == DLFX_F32 ? run(float()) : dtype == DLFX_F64 ? run(double()) : run(half_t());
 }

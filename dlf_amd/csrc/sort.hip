@@ -58,6 +58,11 @@ enum KeyKind { kKeyInt = 0, kKeyFloat = 1 };
 template <typename K>
 struct KeyTraits;
 template <>
+struct KeyTraits<uint16_t> {
+    static constexpr int kPasses = 2;
+    static constexpr uint16_t kSign = 0x8000u;
+};
+template <>
 struct KeyTraits<uint32_t> {
     static constexpr int kPasses = 4;
     static constexpr uint32_t kSign = 0x80000000u;
@@ -103,7 +108,7 @@ struct PassIo {
 
 template <typename K>
 __device__ __forceinline__ K key_of_element(const PassIo<K>& io, K bits) {
-    if (io.canon_zero && (bits << 1) == 0) bits = 0;      // -0.0 -> +0.0
+    if (io.canon_zero && static_cast<K>(bits << 1) == 0) bits = 0;      // -0.0 -> +0.0
     return encode_key<K>(bits, io.kind, io.descending);
 }
 
@@ -534,7 +539,7 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
             for (int k = 0; k < ITEMS; ++k) {
                 K bits = decode_key<K>(out[k], io.kind, io.descending);
                 if constexpr (PAIRS) {
-                    if (io.restore_zero && (bits << 1) == 0 && (full || k * kPassBlock + tid < valid))
+                    if (io.restore_zero && static_cast<K>(bits << 1) == 0 && (full || k * kPassBlock + tid < valid))
                         bits = xrow[static_cast<int64_t>(pay[k]) * io.sx];
                 }
                 if (full || k * kPassBlock + tid < valid) yrow[at[k] * io.sy] = bits;
@@ -572,7 +577,7 @@ struct SortLayout {
 
 SortLayout sort_layout(size_t key_size, bool pairs, int64_t m, int64_t n) {
     SortLayout l;
-    const int passes = key_size == 4 ? 4 : 8;
+    const int passes = static_cast<int>(key_size);          // one per key byte
     const int64_t tile = kPassBlock * tile_items(key_size, pairs);
     l.tiles_per_row = ceil_div(n, tile);
     size_t off = 0;
@@ -700,6 +705,8 @@ int sort_entry(hipStream_t stream, int dtype, const SortArgs& a0, void* scratch,
     case DLFX_I32: a.kind = kKeyInt;   return run_sort<uint32_t>(stream, a, scratch, scratch_bytes);
     case DLFX_F64: a.kind = kKeyFloat; return run_sort<uint64_t>(stream, a, scratch, scratch_bytes);
     case DLFX_I64: a.kind = kKeyInt;   return run_sort<uint64_t>(stream, a, scratch, scratch_bytes);
+    case DLFX_F16: a.kind = kKeyFloat; return run_sort<uint16_t>(stream, a, scratch, scratch_bytes);
+    case DLFX_I16: a.kind = kKeyInt;   return run_sort<uint16_t>(stream, a, scratch, scratch_bytes);
     default: return DLFX_ERR_UNSUPPORTED_DTYPE;
     }
 }
@@ -743,7 +750,7 @@ int argsort_contiguous(hipStream_t stream, int dir, int dtype, int rank, const i
 
 
 size_t argsort_scratch_bytes_impl(int dtype, int64_t m, int64_t n) {
-    const size_t es = dtype_size(dtype);
+    const size_t es = dtype == DLFX_BOOL ? 0 : dtype_size(dtype);
     if (!es || m <= 0 || n <= 0) return 0;
     return sort_layout(es, true, m, n).total;
 }
@@ -753,7 +760,7 @@ size_t argsort_scratch_bytes_impl(int dtype, int64_t m, int64_t n) {
 using namespace dlfx;
 
 extern "C" size_t dlfx_sort_scratch_bytes(int dtype, int64_t m, int64_t n) {
-    const size_t es = dtype_size(dtype);
+    const size_t es = dtype == DLFX_BOOL ? 0 : dtype_size(dtype);
     if (!es || m <= 0 || n <= 0) return 0;
     return sort_layout(es, false, m, n).total;
 }
@@ -764,7 +771,7 @@ extern "C" int dlfx_sort(dlfx_stream_t stream, int dir, int dtype, int rank, con
                          void* scratch, size_t scratch_bytes) {
     if (!x || !y || rank < 1) return DLFX_ERR_INVALID_ARGUMENT;
     if (!view_ok(rank, dims, x_strides) || !view_ok(rank, dims, y_strides)) return DLFX_ERR_INVALID_ARGUMENT;
-    const size_t es = dtype_size(dtype);
+    const size_t es = dtype == DLFX_BOOL ? 0 : dtype_size(dtype);
     if (!es) return DLFX_ERR_UNSUPPORTED_DTYPE;
     SortArgs a{};
     a.dir = dir;
@@ -792,7 +799,7 @@ extern "C" int dlfx_argsort(dlfx_stream_t stream, int dir, int dtype, int index_
     if (!view_ok(rank, dims, x_strides) || !view_ok(rank, dims, i_strides)) return DLFX_ERR_INVALID_ARGUMENT;
     if (y && !view_ok(rank, dims, y_strides)) return DLFX_ERR_INVALID_ARGUMENT;
     if (index_dtype != DLFX_I32 && index_dtype != DLFX_I64) return DLFX_ERR_UNSUPPORTED_DTYPE;
-    const size_t es = dtype_size(dtype);
+    const size_t es = dtype == DLFX_BOOL ? 0 : dtype_size(dtype);
     if (!es) return DLFX_ERR_UNSUPPORTED_DTYPE;
     SortArgs a{};
     a.dir = dir;

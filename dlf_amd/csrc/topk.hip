@@ -51,12 +51,34 @@ __device__ __forceinline__ K from_ord(K k, int kind, int largest) {
     return (kind == kKeyFloat) ? ((k & S) ? (k & ~S) : ~k) : (k ^ S);
 }
 
-template <typename K>
+// Elements are stored as S and handled as K-wide bit patterns: S is K itself for four- and
+// eight-byte types; IEEE half and int16 are stored as 16 bits and widened (exactly, order
+// preserved) to the bits of a float or an int32 at the load, narrowed again at the store.
+template <typename K, typename S>
+__device__ __forceinline__ K widen_bits(S s, int kind) {
+    if constexpr (sizeof(S) == sizeof(K)) {
+        return s;
+    } else {
+        if (kind == kKeyFloat) return bit_cast<uint32_t>(static_cast<float>(bit_cast<half_t>(s)));
+        return static_cast<uint32_t>(static_cast<int32_t>(static_cast<int16_t>(s)));
+    }
+}
+template <typename S, typename K>
+__device__ __forceinline__ S narrow_bits(K bits, int kind) {
+    if constexpr (sizeof(S) == sizeof(K)) {
+        return bits;
+    } else {
+        if (kind == kKeyFloat) return bit_cast<uint16_t>(static_cast<half_t>(bit_cast<float>(bits)));
+        return static_cast<uint16_t>(bits);
+    }
+}
+
+template <typename K, typename S = K>
 struct TopkIo {
-    const K* x;
+    const S* x;
     DimMap xmap;
     int64_t sx;
-    K* y;
+    S* y;
     DimMap ymap;
     int64_t sy;
     void* idx;
@@ -186,11 +208,12 @@ __device__ __forceinline__ V kth_largest(TopkShared<K>& sm, int nitems, uint32_t
     return prefix;
 }
 
-template <typename K>
-__device__ __forceinline__ void emit_one(const TopkIo<K>& io, K* yr, int64_t ir, const K* xr, int j, K ord, uint32_t ix) {
+template <typename K, typename S>
+__device__ __forceinline__ void emit_one(const TopkIo<K, S>& io, S* yr, int64_t ir, const S* xr, int j, K ord, uint32_t ix) {
     K bits = from_ord<K>(ord, io.kind, io.largest);
-    if (io.kind == kKeyFloat && (bits << 1) == 0) bits = xr[static_cast<int64_t>(ix) * io.sx];   // keep the zero's sign
-    yr[j * io.sy] = bits;
+    S out = narrow_bits<S, K>(bits, io.kind);
+    if (io.kind == kKeyFloat && (bits << 1) == 0) out = xr[static_cast<int64_t>(ix) * io.sx];   // keep the zero's sign
+    yr[j * io.sy] = out;
     if (io.idx64) static_cast<int64_t*>(io.idx)[ir + j * io.si] = static_cast<int64_t>(ix);
     else static_cast<int32_t*>(io.idx)[ir + j * io.si] = static_cast<int32_t>(ix);
 }
@@ -269,15 +292,15 @@ constexpr int kMergeMax = 512;       // entries up to which sorted runs are merg
 // multiple of 64 and are overwritten.  Each wave sorts runs of 64 entries in registers; the
 // rank of an entry is its position in its run plus, for every other run, the number of that
 // run's entries that beat it, found by bisection.  All threads of the team must call.
-template <int BLOCK, typename K>
+template <int BLOCK, typename K, typename S>
 __device__ __forceinline__ void merge_rank_emit(K* e_ord, uint32_t* e_idx, int count, int limit,
-                                                const TopkIo<K>& io, int64_t row, const K* xr) {
+                                                const TopkIo<K, S>& io, int64_t row, const S* xr) {
     constexpr int WAVES = BLOCK / kWave;
     const int tid = threadIdx.x;
     const int lane = lane_id();
     const int w = tid / kWave;
     const int runs = (count + kWave - 1) / kWave;
-    K* yr = io.y + io.ymap.at(row);
+    S* yr = io.y + io.ymap.at(row);
     const int64_t ir = io.imap.at(row);
     for (int r = w; r < runs; r += WAVES) {
         const int e = r * kWave + lane;
@@ -356,8 +379,8 @@ __device__ __forceinline__ void merge_rank_emit(K* e_ord, uint32_t* e_idx, int c
 // Radix select from the first byte in which the items differ; as soon as the digit that
 // holds the limit-th best has at most kAmbMax members, those members are ranked
 // directly (by image, then index) instead of refining further.
-template <int BLOCK, int ITEMS, bool ROLLED, typename K, typename Ord, typename Idx>
-__device__ __forceinline__ void select_and_emit(TopkShared<K>& sm, const TopkIo<K>& io, int64_t row, const K* xr,
+template <int BLOCK, int ITEMS, bool ROLLED, typename K, typename S, typename Ord, typename Idx>
+__device__ __forceinline__ void select_and_emit(TopkShared<K>& sm, const TopkIo<K, S>& io, int64_t row, const S* xr,
                                                 int limit, int nitems, Ord ord, Idx idx) {
     const int tid = threadIdx.x;
     const int lane = lane_id();
@@ -519,41 +542,47 @@ __device__ __forceinline__ void select_and_emit(TopkShared<K>& sm, const TopkIo<
             team_sync<BLOCK>();
         }
     }
-    K* yr = io.y + io.ymap.at(row);
+    S* yr = io.y + io.ymap.at(row);
     const int64_t ir = io.imap.at(row);
     for (int j = tid; j < limit; j += BLOCK) emit_one<K>(io, yr, ir, xr, j, sm.out_ord[j], sm.out_idx[j]);
 }
 
-template <typename T> struct BitsOf;
-template <> struct BitsOf<float>   { using type = uint32_t; static constexpr int kind = kKeyFloat; };
-template <> struct BitsOf<int32_t> { using type = uint32_t; static constexpr int kind = kKeyInt; };
-template <> struct BitsOf<double>  { using type = uint64_t; static constexpr int kind = kKeyFloat; };
-template <> struct BitsOf<int64_t> { using type = uint64_t; static constexpr int kind = kKeyInt; };
+// E: the element type in memory.  type: its K-wide bit pattern; storage: its bits in memory;
+// score: the arithmetic type elements are compared in.
+template <typename E> struct BitsOf;
+template <> struct BitsOf<float>   { using type = uint32_t; using storage = uint32_t; using score = float;   static constexpr int kind = kKeyFloat; };
+template <> struct BitsOf<int32_t> { using type = uint32_t; using storage = uint32_t; using score = int32_t; static constexpr int kind = kKeyInt; };
+template <> struct BitsOf<double>  { using type = uint64_t; using storage = uint64_t; using score = double;  static constexpr int kind = kKeyFloat; };
+template <> struct BitsOf<int64_t> { using type = uint64_t; using storage = uint64_t; using score = int64_t; static constexpr int kind = kKeyInt; };
+template <> struct BitsOf<half_t>  { using type = uint32_t; using storage = uint16_t; using score = float;   static constexpr int kind = kKeyFloat; };
+template <> struct BitsOf<int16_t> { using type = uint32_t; using storage = uint16_t; using score = int32_t; static constexpr int kind = kKeyInt; };
 
-// T: the element type.  ALIGNED: the axis is contiguous and every row starts on a 16-byte
+// E: the element type.  ALIGNED: the axis is contiguous and every row starts on a 16-byte
 // boundary (checked on the host), so rows are read with 128-bit loads off one base register.
 //
 // Elements are held as scores of type T: the element itself when the largest are wanted,
 // its order-reversing image otherwise (sign flip for floats, complement for integers), so
 // the kernel always looks for the largest scores and compares them natively.
-template <typename T, int BLOCK, int ITEMS, bool ALIGNED>
-__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(BLOCK >= 1024 && sizeof(T) == 4 && ITEMS <= 32 ? 8 : 1)))
-void topk_select(TopkIo<typename BitsOf<T>::type> io, int64_t n, int limit,
-                 uint32_t* __restrict__ row_state, typename BitsOf<T>::type* __restrict__ spill_ord,
+template <typename E, int BLOCK, int ITEMS, bool ALIGNED>
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(BLOCK >= 1024 && sizeof(typename BitsOf<E>::type) == 4 && ITEMS <= 32 ? 8 : 1)))
+void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> io, int64_t n, int limit,
+                 uint32_t* __restrict__ row_state, typename BitsOf<E>::type* __restrict__ spill_ord,
                  uint32_t* __restrict__ spill_idx) {
-    using K = typename BitsOf<T>::type;
-    constexpr int kind = BitsOf<T>::kind;
-    constexpr int V = (16 / sizeof(K) < ITEMS) ? 16 / sizeof(K) : ITEMS;
+    using K = typename BitsOf<E>::type;
+    using S = typename BitsOf<E>::storage;
+    using T = typename BitsOf<E>::score;
+    constexpr int kind = BitsOf<E>::kind;
+    constexpr int V = (16 / sizeof(S) < ITEMS) ? 16 / sizeof(S) : ITEMS;
     constexpr int G = ITEMS / V;
     constexpr int WAVES = BLOCK / kWave;
-    using VecT = Vec<K, V>;
+    using VecT = Vec<S, V>;
     __shared__ TopkShared<K> sm;
 
     const int tid = threadIdx.x;
     const int lane = lane_id();
     const int w = tid / kWave;
     const int64_t row = blockIdx.x;
-    const K* xr = io.x + io.xmap.at(row);
+    const S* xr = io.x + io.xmap.at(row);
     if (tid < kRadix) sm.hist[tid] = 0;
 
     // item (g, e) of thread t is element ((g*BLOCK + t)*V + e) of the row
@@ -564,7 +593,7 @@ void topk_select(TopkIo<typename BitsOf<T>::type> io, int64_t n, int limit,
     };
     const K flip = io.largest ? K(0) : (kind == kKeyFloat ? KeyBits<K>::kSign : ~K(0));
     const T worst = std::is_integral<T>::value ? std::numeric_limits<T>::lowest() : -std::numeric_limits<T>::infinity();
-    auto score_of = [&](K bits) -> T { return bit_cast<T>(static_cast<K>(bits ^ flip)); };
+    auto score_of = [&](S stored) -> T { return bit_cast<T>(static_cast<K>(widen_bits<K, S>(stored, kind) ^ flip)); };
     // order-preserving unsigned image of a score (scores are always maximised)
     auto ord_of = [&](T sc) -> K { return to_ord<K>(bit_cast<K>(sc), kind, 1); };
     auto load_ord = [&](int i) -> K {        // straight from memory; padding -> 0
@@ -687,19 +716,20 @@ void topk_select(TopkIo<typename BitsOf<T>::type> io, int64_t n, int limit,
 
 // Second stage of the selection for rows topk_select did not finish: exact selection among the
 // row's spilled candidates, or over the whole row when it has to be.
-template <typename T>
+template <typename E>
 __global__ __launch_bounds__(kSelectThreads) void topk_finish(
-    TopkIo<typename BitsOf<T>::type> io, int64_t n, int limit, const uint32_t* __restrict__ row_state,
-    const typename BitsOf<T>::type* __restrict__ spill_ord, const uint32_t* __restrict__ spill_idx) {
-    using K = typename BitsOf<T>::type;
-    constexpr int kind = BitsOf<T>::kind;
+    TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> io, int64_t n, int limit, const uint32_t* __restrict__ row_state,
+    const typename BitsOf<E>::type* __restrict__ spill_ord, const uint32_t* __restrict__ spill_idx) {
+    using K = typename BitsOf<E>::type;
+    using S = typename BitsOf<E>::storage;
+    constexpr int kind = BitsOf<E>::kind;
     constexpr int SEL = kSelectThreads;
     __shared__ TopkShared<K> sm;
     const int tid = threadIdx.x;
     const int64_t row = blockIdx.x;
     const uint32_t state = row_state[row];
     if (state == kRowDone) return;
-    const K* xr = io.x + io.xmap.at(row);
+    const S* xr = io.x + io.xmap.at(row);
     if (tid < kRadix) sm.hist[tid] = 0;
     if (state != kRowWhole) {
         const uint32_t total = state;
@@ -729,16 +759,16 @@ __global__ __launch_bounds__(kSelectThreads) void topk_finish(
             sm, io, row, xr, limit, per_thread,
             [&](int j) {
                 const uint32_t ix = j * SEL + tid;
-                return ix < n32 ? to_ord<K>(static_cast<K>(xr[static_cast<int64_t>(ix) * io.sx] ^ flip), kind, 1) : K(0);
+                return ix < n32 ? to_ord<K>(static_cast<K>(widen_bits<K, S>(xr[static_cast<int64_t>(ix) * io.sx], kind) ^ flip), kind, 1) : K(0);
             },
             [&](int j) { return static_cast<uint32_t>(j * SEL + tid); });
     }
 }
 
 // Fallback epilogue: first `limit` entries of each row of a full stable argsort.
-template <typename K>
-__global__ __launch_bounds__(256) void topk_take(const K* __restrict__ ys, const int32_t* __restrict__ is,
-                                                  int64_t m, int64_t n, int64_t limit, TopkIo<K> io) {
+template <typename K, typename S>
+__global__ __launch_bounds__(256) void topk_take(const S* __restrict__ ys, const int32_t* __restrict__ is,
+                                                  int64_t m, int64_t n, int64_t limit, TopkIo<K, S> io) {
     const int64_t g = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (g >= m * limit) return;
     const int64_t row = g / limit, j = g - row * limit;
@@ -778,12 +808,13 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
               const void* x, const int64_t* xs, void* y, const int64_t* ys, void* idx, const int64_t* is,
               void* scratch, size_t scratch_bytes) {
     using K = typename BitsOf<T>::type;
+    using S = typename BitsOf<T>::storage;
     const int64_t n = x_dims[rank - 1];
     const int64_t m = view_size(rank, x_dims) / n;
-    TopkIo<K> io;
+    TopkIo<K, S> io;
     std::memset(&io, 0, sizeof(io));
-    io.x = static_cast<const K*>(x);
-    io.y = static_cast<K*>(y);
+    io.x = static_cast<const S*>(x);
+    io.y = static_cast<S*>(y);
     io.idx = idx;
     if (!make_dim_map(x_dims, xs, 0, rank - 1, &io.xmap) || !make_dim_map(y_dims, ys, 0, rank - 1, &io.ymap) ||
         !make_dim_map(y_dims, is, 0, rank - 1, &io.imap))
@@ -800,7 +831,7 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
         const dim3 grid(static_cast<unsigned>(m));
         const int lim = static_cast<int>(limit);
         bool aligned = io.sx == 1 && reinterpret_cast<uintptr_t>(io.x) % 16 == 0;
-        for (int i = 0; i < io.xmap.rank; ++i) aligned = aligned && io.xmap.strides[i] % (16 / static_cast<int64_t>(sizeof(K))) == 0;
+        for (int i = 0; i < io.xmap.rank; ++i) aligned = aligned && io.xmap.strides[i] % (16 / static_cast<int64_t>(sizeof(S))) == 0;
         const SelectLayout sl = select_layout(sizeof(K), m, n);
         if (sl.total && (!scratch || scratch_bytes < sl.total)) return DLFX_ERR_SCRATCH_TOO_SMALL;
         char* sbase = static_cast<char*>(scratch);
@@ -834,19 +865,19 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
     }
 
     // full stable argsort into scratch, then keep the head of each row
-    const size_t ysz = align_up(static_cast<size_t>(m) * n * sizeof(K), 256);
+    const size_t ysz = align_up(static_cast<size_t>(m) * n * sizeof(S), 256);
     const size_t isz = align_up(static_cast<size_t>(m) * n * 4, 256);
     const size_t need = ysz + isz + argsort_scratch_bytes_impl(dtype, m, n);
     if (!scratch || scratch_bytes < need) return DLFX_ERR_SCRATCH_TOO_SMALL;
     char* base = static_cast<char*>(scratch);
-    K* ysorted = reinterpret_cast<K*>(base);
+    S* ysorted = reinterpret_cast<S*>(base);
     int32_t* isorted = reinterpret_cast<int32_t*>(base + ysz);
     int st = argsort_contiguous(stream, dir ? 1 : 0, dtype, rank, x_dims, x, xs, ysorted, isorted,
                                 base + ysz + isz, scratch_bytes - ysz - isz);
     if (st != DLFX_OK) return st;
     const int64_t total = m * limit;
     if (ceil_div(total, 256) > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
-    topk_take<K><<<dim3(static_cast<unsigned>(ceil_div(total, 256))), dim3(256), 0, stream>>>(ysorted, isorted, m, n, limit, io);
+    topk_take<K, S><<<dim3(static_cast<unsigned>(ceil_div(total, 256))), dim3(256), 0, stream>>>(ysorted, isorted, m, n, limit, io);
     DLFX_CHECK_LAUNCH();
     return DLFX_OK;
 }
@@ -858,8 +889,9 @@ using namespace dlfx;
 
 extern "C" size_t dlfx_top_k_scratch_bytes(int dtype, int64_t m, int64_t n, int64_t limit) {
     const size_t es = dtype_size(dtype);
-    if (!es || m <= 0 || n <= 0) return 0;
-    if (selection_fits(es, n, limit)) return select_layout(es, m, n).total;
+    if (!es || dtype == DLFX_BOOL || m <= 0 || n <= 0) return 0;
+    const size_t ks = es < 4 ? 4 : es;            // 16-bit elements are selected as 32-bit keys
+    if (selection_fits(ks, n, limit)) return select_layout(ks, m, n).total;
     return align_up(static_cast<size_t>(m) * n * es, 256) + align_up(static_cast<size_t>(m) * n * 4, 256) +
            argsort_scratch_bytes_impl(dtype, m, n);
 }
@@ -889,6 +921,8 @@ extern "C" int dlfx_top_k(dlfx_stream_t stream, int64_t limit, int dir, int dtyp
     case DLFX_I32: return run_top_k<int32_t>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
     case DLFX_F64: return run_top_k<double>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
     case DLFX_I64: return run_top_k<int64_t>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
+    case DLFX_F16: return run_top_k<half_t>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
+    case DLFX_I16: return run_top_k<int16_t>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
     default: return DLFX_ERR_UNSUPPORTED_DTYPE;
     }
 }

@@ -144,7 +144,9 @@ def _torch_dtype(np_dtype):
     import torch
     if _NP_TO_TORCH is None:
         _NP_TO_TORCH = {np.dtype(np.float32): torch.float32, np.dtype(np.float64): torch.float64,
-                        np.dtype(np.int32): torch.int32, np.dtype(np.int64): torch.int64}
+                        np.dtype(np.int32): torch.int32, np.dtype(np.int64): torch.int64,
+                        np.dtype(np.float16): torch.float16, np.dtype(np.int16): torch.int16,
+                        np.dtype(np.bool_): torch.bool}
     return _NP_TO_TORCH[np.dtype(np_dtype)]
 
 
@@ -253,7 +255,7 @@ class HipBackend:
 
     def count(self, dtype, m, n, value, xs, x, ys, y, defer=False):
         sp, sb = self.scratch(self.lib.dlfx_count_scratch_bytes(dtype, m, n))
-        v = np.array([value], dtype=(np.float32, np.float64, np.int32, np.int64)[dtype])   # one host element of the input's type
+        v = np.array([value], dtype=(np.float32, np.float64, np.int32, np.int64, np.float16, np.int16)[dtype])   # one host element of the input's type
         keep = v.ctypes.data_as(c_void_p)
         call = self._issue(self.lib.dlfx_count, "dlfx_count", (dtype, m, n, keep),
                            (xs.rank, _arr(xs.extents), _arr(xs.strides), x.data_ptr(), xs.offset,

@@ -14,6 +14,7 @@
 #include <vector>
 
 #include "dlfx.h"
+#include "gblas_half.h"
 #include "gpgpu.h"
 
 namespace gpgpu { namespace dnn {
@@ -25,6 +26,8 @@ template <> struct dtype_of<float>   { static constexpr int value = DLFX_F32; };
 template <> struct dtype_of<double>  { static constexpr int value = DLFX_F64; };
 template <> struct dtype_of<int32_t> { static constexpr int value = DLFX_I32; };
 template <> struct dtype_of<int64_t> { static constexpr int value = DLFX_I64; };
+template <> struct dtype_of<int16_t> { static constexpr int value = DLFX_I16; };
+template <> struct dtype_of<blas::half> { static constexpr int value = DLFX_F16; };
 
 // size_t strides that wrapped for a negative step come back as the negative number
 inline std::vector<int64_t> signed_vec(const std::vector<size_t>& v) {

@@ -10,8 +10,8 @@
  * Conventions shared by every call
  *   stream     a hipStream_t passed as void*; work is enqueued asynchronously on
  *              it and the call returns without synchronising.
- *   dtype      DLFX_F32 / DLFX_F64 / DLFX_I32 / DLFX_I64 -- the element type T
- *              of the reference template instantiation.
+ *   dtype      a dlfx_dtype -- the element type T of the reference template
+ *              instantiation (gdnn.cpp:847-1347, 1851-1894).
  *   dims       extents of the (already axis-moved) view, `rank` entries.
  *   strides    element strides, signed: a reference stride that wrapped as
  *              size_t (negative step) is passed as the negative number it means.
@@ -47,7 +47,10 @@ typedef enum dlfx_dtype {
     DLFX_F32 = 0,
     DLFX_F64 = 1,
     DLFX_I32 = 2,
-    DLFX_I64 = 3
+    DLFX_I64 = 3,
+    DLFX_F16 = 4,   /* IEEE half: every entry point (sums and scans accumulate in fp32, rounded once) */
+    DLFX_I16 = 5,   /* arg_reduce, sort, argsort, top_k (the reference's int16 instantiations) and merge */
+    DLFX_BOOL = 6   /* one byte per element; input of scan_nonzero only */
 } dlfx_dtype;
 
 typedef enum dlfx_status {

@@ -64,6 +64,31 @@ class OracleBackend:
     def alloc(self, dtype, count):
         return np.zeros(max(1, count), dtype=dtype)
 
+    @staticmethod
+    def _wide(dtype, inputs, outputs, fn):
+        """16-bit and bool elements go through the 32-bit restatement: half -> float and
+        int16 / bool -> int32 are exact and order preserving, and every result that is an
+        element (not an index or a count) converts back exactly or, for sums, with the one
+        rounding the 16-bit result type requires.  fn(code, inputs, outputs) makes the call."""
+        if dtype not in (4, 5, 6):
+            return fn(dtype, list(inputs), list(outputs))
+        to, code = (np.float32, 0) if dtype == 4 else (np.int32, 2)
+        cache = {}
+
+        def widen(a):
+            if a is None:
+                return None
+            if id(a) not in cache:
+                cache[id(a)] = a.astype(to)
+            return cache[id(a)]
+        ins = [widen(a) for a in inputs]
+        outs = [widen(a) for a in outputs]
+        r = fn(code, ins, outs)
+        for a, b in zip(outputs, outs):
+            if a is not None:
+                a[...] = b.astype(a.dtype)
+        return r
+
     def upload(self, flat):
         return np.array(flat, copy=True).reshape(-1)
 
@@ -71,12 +96,18 @@ class OracleBackend:
         return storage
 
     def reduce(self, name, dtype, m, n, xs, x, ys, y):
+        return self._wide(dtype, [x], [y], lambda dtype, i, o: self._reduce_impl(name, dtype, m, n, xs, i[0], ys, o[0]))
+
+    def _reduce_impl(self, name, dtype, m, n, xs, x, ys, y):
         _check(self.lib.dlf_oracle_reduce(
             c_char_p(name.encode()), c_int(dtype), c_int64(m), c_int64(n),
             c_int(xs.rank), _arr(xs.extents), _arr(xs.strides), _ptr(x), c_int64(xs.offset),
             c_int(ys.rank), _arr(ys.extents), _arr(ys.strides), _ptr(y), c_int64(ys.offset)), "oracle reduce")
 
     def arg_reduce(self, name, dtype, index_dtype, rows, k, xs, x, ys, y):
+        return self._wide(dtype, [x], [], lambda dtype, i, o: self._arg_reduce_impl(name, dtype, index_dtype, rows, k, xs, i[0], ys, y))
+
+    def _arg_reduce_impl(self, name, dtype, index_dtype, rows, k, xs, x, ys, y):
         out = y if y.dtype == np.int32 else np.zeros(y.shape, dtype=np.int32)
         _check(self.lib.dlf_oracle_arg_reduce(
             c_char_p(name.encode()), c_int(dtype), c_int64(rows), c_int64(k),
@@ -86,18 +117,27 @@ class OracleBackend:
             y[...] = out
 
     def scan(self, name, dtype, m, n, exclusive, xs, x, ys, y):
+        return self._wide(dtype, [x], [y], lambda dtype, i, o: self._scan_impl(name, dtype, m, n, exclusive, xs, i[0], ys, o[0]))
+
+    def _scan_impl(self, name, dtype, m, n, exclusive, xs, x, ys, y):
         _check(self.lib.dlf_oracle_scan(
             c_char_p(name.encode()), c_int(dtype), c_int64(m), c_int64(n), c_int(int(bool(exclusive))),
             c_int(xs.rank), _arr(xs.extents), _ptr(x), c_int64(xs.offset), _arr(xs.strides),
             _ptr(y), c_int64(ys.offset), _arr(ys.strides)), "oracle scan")
 
     def sort(self, direction, dtype, xs, x, ys, y):
+        return self._wide(dtype, [x], [y], lambda dtype, i, o: self._sort_impl(direction, dtype, xs, i[0], ys, o[0]))
+
+    def _sort_impl(self, direction, dtype, xs, x, ys, y):
         _check(self.lib.dlf_oracle_sort(
             c_int(direction), c_int(dtype), c_int(xs.rank), _arr(xs.extents),
             _ptr(x), c_int64(xs.offset), _arr(xs.strides),
             _ptr(y), c_int64(ys.offset), _arr(ys.strides)), "oracle sort")
 
     def argsort(self, direction, dtype, index_dtype, xs, x, ys, y, is_, i):
+        return self._wide(dtype, [x], [y], lambda dtype, ins, o, idx=i: self._argsort_impl(direction, dtype, index_dtype, xs, ins[0], ys, o[0], is_, idx))
+
+    def _argsort_impl(self, direction, dtype, index_dtype, xs, x, ys, y, is_, i):
         out = i if i.dtype == np.int32 else np.zeros(i.shape, dtype=np.int32)
         _check(self.lib.dlf_oracle_argsort(
             c_int(direction), c_int(dtype), c_int(xs.rank), _arr(xs.extents),
@@ -109,6 +149,9 @@ class OracleBackend:
             i[...] = out
 
     def top_k(self, limit, direction, dtype, index_dtype, xs, x, ys, y, is_, i):
+        return self._wide(dtype, [x], [y], lambda dtype, ins, o, idx=i: self._top_k_impl(limit, direction, dtype, index_dtype, xs, ins[0], ys, o[0], is_, idx))
+
+    def _top_k_impl(self, limit, direction, dtype, index_dtype, xs, x, ys, y, is_, i):
         _check(self.lib.dlf_oracle_top_k(
             c_int(self.topk_mode), c_int64(limit), c_int(direction), c_int(1), c_int(dtype),
             c_int(xs.rank), _arr(xs.extents), _arr(ys.extents),
@@ -117,6 +160,9 @@ class OracleBackend:
             _ptr(i), c_int64(is_.offset), _arr(is_.strides), c_int(i.dtype.itemsize)), "oracle top_k")
 
     def count(self, dtype, m, n, value, xs, x, ys, y):
+        return self._wide(dtype, [x], [], lambda dtype, i, o: self._count_impl(dtype, m, n, value, xs, i[0], ys, y))
+
+    def _count_impl(self, dtype, m, n, value, xs, x, ys, y):
         v = np.array([value], dtype=x.dtype)
         _check(self.lib.dlf_oracle_count(
             c_int(dtype), c_int64(m), c_int64(n), _ptr(v),
@@ -124,6 +170,9 @@ class OracleBackend:
             c_int(ys.rank), _arr(ys.extents), _arr(ys.strides), _ptr(y), c_int64(ys.offset)), "oracle count")
 
     def scan_nonzero(self, dtype, m, n, exclusive, xs, x, ys, y):
+        return self._wide(dtype, [x], [], lambda dtype, i, o: self._scan_nonzero_impl(dtype, m, n, exclusive, xs, i[0], ys, y))
+
+    def _scan_nonzero_impl(self, dtype, m, n, exclusive, xs, x, ys, y):
         _check(self.lib.dlf_oracle_scan_nonzero(
             c_int(dtype), c_int64(m), c_int64(n), c_int(int(bool(exclusive))),
             c_int(xs.rank), _arr(xs.extents), _ptr(x), c_int64(xs.offset), _arr(xs.strides),
@@ -135,6 +184,9 @@ class OracleBackend:
             _ptr(counts), _ptr(out)), "oracle gather_indices")
 
     def softmax(self, name, dtype, m, n, x, x_offset, y, y_offset):
+        return self._wide(dtype, [x], [y], lambda dtype, i, o: self._softmax_impl(name, dtype, m, n, i[0], x_offset, o[0], y_offset))
+
+    def _softmax_impl(self, name, dtype, m, n, x, x_offset, y, y_offset):
         kind = {"softmax": 0, "logsoftmax": 1, "hardmax": 2}[name]
         if y is not x or y_offset != x_offset:
             y[y_offset:y_offset + m * n] = x[x_offset:x_offset + m * n]
@@ -142,6 +194,9 @@ class OracleBackend:
         _check(self.lib.dlf_oracle_softmax(c_int(kind), c_int(dtype), c_int64(m), c_int64(n), _ptr(rows)), "oracle " + name)
 
     def merge(self, direction, dtype, xs, x, ys, y, zs, z):
+        return self._wide(dtype, [x, y], [z], lambda dtype, i, o: self._merge_impl(direction, dtype, xs, i[0], ys, i[1], zs, o[0]))
+
+    def _merge_impl(self, direction, dtype, xs, x, ys, y, zs, z):
         _check(self.lib.dlf_oracle_merge(
             c_int(direction), c_int(dtype), c_int(zs.rank),
             _arr(xs.extents), _arr(xs.strides), _ptr(x), c_int64(xs.offset),
@@ -157,6 +212,8 @@ class OracleBackend:
 
 def reduce_f64(name, dtype, m, n, xs, x) -> np.ndarray:
     """fp64 evaluation of a reducer over the same view: one double per output row."""
+    if dtype == 4:
+        dtype, x = 0, x.astype(np.float32)
     out = np.zeros(m, dtype=np.float64)
     _check(lib().dlf_oracle_reduce_f64(
         c_char_p(name.encode()), c_int(dtype), c_int64(m), c_int64(n),
@@ -167,6 +224,8 @@ def reduce_f64(name, dtype, m, n, xs, x) -> np.ndarray:
 
 def scan_f64(name, dtype, m, n, exclusive, xs, x, with_abs=True):
     """fp64 scan of the view, contiguous [m, n]; also the running sum of |x| when asked."""
+    if dtype == 4:
+        dtype, x = 0, x.astype(np.float32)
     out = np.zeros((m, n), dtype=np.float64)
     mag = np.zeros((m, n), dtype=np.float64) if with_abs else None
     _check(lib().dlf_oracle_scan_f64(

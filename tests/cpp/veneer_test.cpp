@@ -218,6 +218,43 @@ static void test_merge() {
     CHECK(threw);
 }
 
+// 16-bit element types through the same front-ends: order-based results are exact, half sums
+// are formed in float and rounded once.
+static void test_16bit_types() {
+    using gpgpu::blas::half;
+    auto S = Tensor<int16_t>({2, 6}, {5, -3, 300, -30000, 7, 5, 1, 1, 0, -1, 32767, -32768});
+    DevTensor<int16_t> SS;
+    sort(dev(S), SS, -1);
+    CHECK(SS.read() == Tensor<int16_t>({2, 6}, {-30000, -3, 5, 5, 7, 300, -32768, -1, 0, 1, 1, 32767}));
+    DevTensor<int16_t> SV;
+    DevTensor<int32_t> SI;
+    argsort(dev(S), SV, SI, -1, true);
+    CHECK(SI.read() == Tensor<int32_t>({2, 6}, {2, 4, 0, 5, 1, 3, 4, 0, 1, 2, 3, 5}));
+    CHECK(argmax(dev(S), 1, false).read() == Tensor<int>({2}, {2, 4}));
+    DevTensor<int16_t> TV;
+    DevTensor<int32_t> TI;
+    top_k(dev(S), TV, TI, 2, -1, true);
+    CHECK(TV.read() == Tensor<int16_t>({2, 2}, {300, 7, 32767, 1}));
+    CHECK(TI.read() == Tensor<int32_t>({2, 2}, {2, 4, 4, 0}));
+
+    std::vector<half> hv;
+    for (float f : {1.5f, -2.25f, 0.0f, 1024.0f, 0.5f, -0.125f, 3.0f, 3.0f}) hv.push_back(half(f));
+    auto H = Tensor<half>({2, 4}, hv);
+    auto sum = reduce_sum(dev(H), {1}).read();
+    CHECK(static_cast<float>(sum.values()[0]) == 1023.0f);                // 1023.25 rounds to the even neighbour 1023
+    CHECK(static_cast<float>(sum.values()[1]) == 6.375f);
+    auto mx = reduce_max(dev(H), {1}).read();
+    CHECK(static_cast<float>(mx.values()[0]) == 1024.0f && static_cast<float>(mx.values()[1]) == 3.0f);
+    DevTensor<half> HS;
+    sort(dev(H), HS, -1);
+    auto hs = HS.read();
+    CHECK(static_cast<float>(hs.values()[0]) == -2.25f && static_cast<float>(hs.values()[3]) == 1024.0f);
+    CHECK(argmax(dev(H), 1, false).read() == Tensor<int>({2}, {3, 2}));
+    auto sm = dnn::hardmax(dev(H), 1).read();
+    CHECK(static_cast<float>(sm.values()[3]) == 1.0f && static_cast<float>(sm.values()[6]) == 1.0f &&
+          static_cast<float>(sm.values()[7]) == 0.0f);
+}
+
 static void test_errors_and_temporaries() {
     auto X = dev(Tensor<float>({2, 3}).range());
     bool threw = false;
@@ -266,6 +303,7 @@ int main() {
     test_count_nonzero();
     test_merge();
     test_softmax_family();
+    test_16bit_types();
     test_errors_and_temporaries();
     std::printf("veneer_test: %d checks, %d failed\n", g_checked, g_failed);
     return g_failed ? 1 : 0;

@@ -281,3 +281,48 @@ def test_softmax_family_matches_closed_forms(oracle_backend, dtype):
     xt = x.transpose(2, 0, 1)
     assert np.allclose(F.softmax(Xt, 1).numpy().reshape(40, -1), sp_softmax(xt.reshape(40, -1).astype(np.float64), axis=1),
                        rtol=tol * 50, atol=tol)
+
+
+# ---------------------------------------------------------------- 16-bit element types
+# The oracle widens float16 / int16 / bool exactly to float / int32 and narrows the result:
+# checked here against numpy on the 16-bit arrays themselves (stable sorts: numpy's default
+# float16 sort returned unsorted rows on this host).
+@pytest.mark.parametrize("dtype", [np.float16, np.int16])
+def test_sixteen_bit_order_ops_match_numpy(oracle_backend, dtype):
+    x = (normal(140, 4 * 500) * 20).astype(dtype).reshape(4, 500)
+    X = Tensor.from_numpy(oracle_backend, x)
+    assert np.array_equal(F.sort(X, -1).numpy(), np.sort(x, axis=1, kind="stable"))
+    assert F.sort(X, -1).numpy().dtype == dtype
+    assert np.array_equal(F.argsort(X, -1).numpy(), np.argsort(x, axis=1, kind="stable"))
+    assert np.array_equal(F.argsort(X, -1, True).numpy(), np.argsort(-x.astype(np.float64), axis=1, kind="stable"))
+    assert np.array_equal(F.argmax(X, 1, False).numpy(), x.argmax(axis=1))
+    assert np.array_equal(F.argmin(X, 0, False).numpy(), x.argmin(axis=0))
+    assert np.array_equal(F.reduce("reduce_max", X, (1,)).numpy(), x.max(axis=1))
+    Y, I = F.top_k(X, 7, -1)
+    want = np.argsort(-x.astype(np.float64), axis=1, kind="stable")[:, :7]
+    assert np.array_equal(I.numpy(), want) and np.array_equal(Y.numpy(), np.take_along_axis(x, want, 1))
+    a, b = np.sort(x, axis=1, kind="stable"), np.sort(x[::-1] * 1, axis=1, kind="stable")
+    assert np.array_equal(F.merge(Tensor.from_numpy(oracle_backend, a), Tensor.from_numpy(oracle_backend, b)).numpy(),
+                          np.sort(np.concatenate([a, b], 1), axis=1, kind="stable"))
+    assert np.array_equal(F.count(X, dtype(3), (1,)).numpy(), (x == dtype(3)).sum(axis=1))
+    assert np.array_equal(F.nonzero(X).numpy(), np.argwhere(x != 0))
+
+
+def test_half_sums_round_once(oracle_backend):
+    x = (normal(141, 3 * 200) * 0.5).astype(np.float16).reshape(3, 200)
+    X = Tensor.from_numpy(oracle_backend, x)
+    got = F.reduce("reduce_sum", X, (1,)).numpy()
+    assert got.dtype == np.float16
+    # the float sum of 200 halves of this size is within an ulp32 or two of exact; its half
+    # rounding is one of the two halves around the exact sum
+    exact = x.astype(np.float64).sum(axis=1)
+    assert (np.abs(got.astype(np.float64) - exact) <= np.abs(exact) * 2.0 ** -10 + 2.0 ** -24).all()
+    cs = F.cumsum(X, 1).numpy().astype(np.float64)
+    ce = np.cumsum(x.astype(np.float64), axis=1)
+    assert (np.abs(cs - ce) <= np.abs(ce) * 2.0 ** -10 + 1e-4).all()
+    assert np.array_equal(F.cummax(X, 1).numpy(), np.maximum.accumulate(x, axis=1))
+
+
+def test_bool_nonzero(oracle_backend):
+    b = randint(142, 6 * 40, 0, 3).reshape(6, 40) == 0
+    assert np.array_equal(F.nonzero(Tensor.from_numpy(oracle_backend, b)).numpy(), np.argwhere(b))
