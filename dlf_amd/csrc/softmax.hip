@@ -1,7 +1,8 @@
 // softmax / logsoftmax / hardmax over the rows of a contiguous [m, n] matrix
 // (gpgpu/include/gdnn.h:253-264; host semantics dlf/include/tensor/dnn_detail.h:266-350:
 // subtract the row maximum, exponentiate, divide by the sum; logsoftmax x - max - log(sum);
-// hardmax a one at the first occurrence of the maximum and zeros elsewhere).
+// hardmax a one at the first occurrence of the maximum and zeros elsewhere; hardmax also takes
+// int32 / int64 rows, gpgpu/src/gdnn.cpp:1888-1900).
 //
 // A row is read once: it lives in the registers of a team of threads (one wavefront for rows
 // up to 2048 elements, a 1024-thread workgroup up to 32768 four-byte elements) between the
@@ -91,7 +92,7 @@ void softmax_rows(const S* __restrict__ x, S* __restrict__ y, int64_t m, int64_t
     const bool live = row < m;                           // whole teams are live or not
     const S* xr = x + (live ? row : 0) * n;
     S* yr = y + (live ? row : 0) * n;
-    const T lowest = -std::numeric_limits<T>::infinity();
+    const T lowest = std::is_integral<T>::value ? std::numeric_limits<T>::lowest() : -std::numeric_limits<T>::infinity();
     const int32_t n32 = static_cast<int32_t>(n);          // rows here have at most 32768 elements
     auto index_of = [&](int k) -> int32_t { return ((k / V) * TEAM + t) * V + k % V; };
 
@@ -182,7 +183,7 @@ __global__ __launch_bounds__(1024) void softmax_rows_streamed(const S* __restric
     const int t = threadIdx.x;
     const S* xr = x + static_cast<int64_t>(blockIdx.x) * n;
     S* yr = y + static_cast<int64_t>(blockIdx.x) * n;
-    const T lowest = -std::numeric_limits<T>::infinity();
+    const T lowest = std::is_integral<T>::value ? std::numeric_limits<T>::lowest() : -std::numeric_limits<T>::infinity();
     if constexpr (KIND == kHardmax) {
         MaxAt<T> best = {lowest, std::numeric_limits<int32_t>::max()};
         for (int64_t i = t; i < n; i += TEAM) best = max_at_join(best, max_at_of(static_cast<T>(xr[i]), i));
@@ -263,17 +264,25 @@ extern "C" int dlfx_softmax(dlfx_stream_t stream, const char* name, int dtype, i
     else if (!std::strcmp(name, "logsoftmax")) kind = kLogSoftmax;
     else if (!std::strcmp(name, "hardmax")) kind = kHardmax;
     else return DLFX_ERR_UNKNOWN_OP;
-    if (dtype != DLFX_F32 && dtype != DLFX_F64 && dtype != DLFX_F16) return DLFX_ERR_UNSUPPORTED_DTYPE;
+    const bool integer = dtype == DLFX_I32 || dtype == DLFX_I64;
+    if (dtype != DLFX_F32 && dtype != DLFX_F64 && dtype != DLFX_F16 && !(integer && kind == kHardmax))
+        return DLFX_ERR_UNSUPPORTED_DTYPE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     auto run = [&](auto tag) {
         using T = decltype(tag);
         const T* xp = static_cast<const T*>(x) + x_offset;
         T* yp = static_cast<T*>(y) + y_offset;
-        switch (kind) {
-        case kSoftmax: return launch_softmax<T, kSoftmax>(s, m, n, xp, yp);
-        case kLogSoftmax: return launch_softmax<T, kLogSoftmax>(s, m, n, xp, yp);
-        default: return launch_softmax<T, kHardmax>(s, m, n, xp, yp);
+        if constexpr (!std::is_integral<T>::value) {
+            if (kind == kSoftmax) return launch_softmax<T, kSoftmax>(s, m, n, xp, yp);
+            if (kind == kLogSoftmax) return launch_softmax<T, kLogSoftmax>(s, m, n, xp, yp);
         }
+        return launch_softmax<T, kHardmax>(s, m, n, xp, yp);
     };
-    return dtype == DLFX_F32 ? run(float()) : dtype == DLFX_F64 ? run(double()) : run(half_t());
+    switch (dtype) {
+    case DLFX_F32: return run(float());
+    case DLFX_F64: return run(double());
+    case DLFX_F16: return run(half_t());
+    case DLFX_I32: return run(int32_t());
+    default: return run(int64_t());
+    }
 }

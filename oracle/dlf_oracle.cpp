@@ -789,9 +789,10 @@ int dlf_oracle_merge(int dir, int dtype, int rank,
 // reference's row loops (dlf/include/tensor/dnn_detail.h:266-350): serial maximum from px[0]
 // with std::max, serial sum in the element type.  kind: 0 softmax, 1 logsoftmax, 2 hardmax.
 int dlf_oracle_softmax(int kind, int dtype, int64_t m, int64_t n, void* x) {
-    if (dtype != 0 && dtype != 1) return -2;
+    if (dtype != 0 && dtype != 1 && !(kind == 2 && (dtype == 2 || dtype == 3))) return -2;
     auto run = [&](auto tag) {
         using T = decltype(tag);
+        using F = std::conditional_t<std::is_integral<T>::value, double, T>;     // integers reach hardmax only
         T* base = static_cast<T*>(x);
 #pragma omp parallel for schedule(static)
         for (int64_t b = 0; b < m; ++b) {
@@ -811,22 +812,27 @@ int dlf_oracle_softmax(int kind, int dtype, int64_t m, int64_t n, void* x) {
             }
             T amax = px[0];
             for (int64_t i = 1; i < n; ++i) amax = std::max(amax, px[i]);
-            T asum = 0;
+            F asum = 0;
             if (kind == 0) {
                 for (int64_t i = 0; i < n; ++i) {
-                    px[i] = std::exp(px[i] - amax);
+                    px[i] = static_cast<T>(std::exp(static_cast<F>(px[i] - amax)));
                     asum += px[i];
                 }
-                for (int64_t i = 0; i < n; ++i) px[i] /= asum;
+                for (int64_t i = 0; i < n; ++i) px[i] = static_cast<T>(px[i] / asum);
             } else {
-                for (int64_t i = 0; i < n; ++i) asum += std::exp(px[i] - amax);
+                for (int64_t i = 0; i < n; ++i) asum += std::exp(static_cast<F>(px[i] - amax));
                 asum = std::log(asum);
-                for (int64_t i = 0; i < n; ++i) px[i] = px[i] - amax - asum;
+                for (int64_t i = 0; i < n; ++i) px[i] = static_cast<T>(px[i] - amax - asum);
             }
         }
         return 0;
     };
-    return dtype == 0 ? run(float()) : run(double());
+    switch (dtype) {
+    case 0: return run(float());
+    case 1: return run(double());
+    case 2: return run(int32_t());
+    default: return run(int64_t());
+    }
 }
 
 }  // extern "C"

@@ -77,3 +77,19 @@ def test_large_matrix_property(hip_backend):
     y = F.softmax(Tensor.from_numpy(hip_backend, x), 1).numpy().astype(np.float64)
     assert np.allclose(y.sum(axis=1), 1.0, atol=1e-5)
     assert np.array_equal(np.argmax(y, axis=1), np.argmax(x, axis=1))
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+@pytest.mark.parametrize("n", [1, 9, 300, 5000, 20000, 40000])
+def test_hardmax_of_integer_rows(hip_backend, oracle_backend, dtype, n):
+    # the reference instantiates hardmax (only) for int32 / int64 as well (gdnn.cpp:1897-1902)
+    x = randint(150 + n, 6 * n, -40, 40).astype(dtype).reshape(6, n)
+    x[3] = np.iinfo(dtype).min                      # a row of the lowest value: the first element is hot
+    got = F.hardmax(Tensor.from_numpy(hip_backend, x), 1).numpy()
+    assert got.dtype == dtype
+    assert np.array_equal(got, F.hardmax(Tensor.from_numpy(oracle_backend, x), 1).numpy())
+    want = np.zeros_like(x)
+    want[np.arange(6), x.argmax(axis=1)] = 1
+    assert np.array_equal(got, want)
+    with pytest.raises(Exception):
+        F.softmax(Tensor.from_numpy(hip_backend, x), 1)
