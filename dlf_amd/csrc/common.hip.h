@@ -82,6 +82,28 @@ struct Words {
     int w[N];
 };
 
+// Complex element (the reference's float2 / double2, std::complex on the host): real part first.
+template <typename F>
+struct alignas(2 * sizeof(F)) Cx {
+    F re, im;
+    Cx() = default;
+    __host__ __device__ constexpr Cx(F r, F i = F(0)) : re(r), im(i) {}
+    template <typename G>
+    __host__ __device__ explicit constexpr Cx(const Cx<G>& o) : re(static_cast<F>(o.re)), im(static_cast<F>(o.im)) {}
+};
+template <typename F>
+__host__ __device__ __forceinline__ Cx<F> operator+(Cx<F> a, Cx<F> b) { return {a.re + b.re, a.im + b.im}; }
+template <typename F>
+__host__ __device__ __forceinline__ Cx<F> operator*(Cx<F> a, Cx<F> b) {
+    return {a.re * b.re - a.im * b.im, a.re * b.im + a.im * b.re};
+}
+template <typename F>
+__host__ __device__ __forceinline__ bool operator==(Cx<F> a, Cx<F> b) { return a.re == b.re && a.im == b.im; }
+template <typename F>
+__host__ __device__ __forceinline__ bool operator!=(Cx<F> a, Cx<F> b) { return !(a == b); }
+template <typename T> struct IsComplex : std::false_type {};
+template <typename F> struct IsComplex<Cx<F>> : std::true_type {};
+
 // Cross-lane helpers move whole 32-bit words; a 2-byte value rides in the low half of one.
 template <typename T>
 __device__ __forceinline__ int widen16(T v) {
@@ -259,7 +281,11 @@ constexpr int vec_width() { return 16 / sizeof(T); }
 // lifts a read-only stream from about 5.9 to 6.6 TB/s.
 template <typename T, int N>
 __device__ __forceinline__ Vec<T, N> load_stream(const Vec<T, N>* p) {
-    if constexpr (N == 1) {
+    if constexpr (std::is_class<T>::value) {
+        // structs travel as the 32-bit words they are made of
+        constexpr int W = N * static_cast<int>(sizeof(T)) / 4;
+        return bit_cast<Vec<T, N>>(load_stream(reinterpret_cast<const Vec<uint32_t, W>*>(p)));
+    } else if constexpr (N == 1) {
         Vec<T, 1> r;
         r.v[0] = __builtin_nontemporal_load(reinterpret_cast<const T*>(p));
         return r;
@@ -274,7 +300,10 @@ __device__ __forceinline__ Vec<T, N> load_stream(const Vec<T, N>* p) {
 }
 template <typename T, int N>
 __device__ __forceinline__ void store_stream(Vec<T, N>* p, const Vec<T, N>& v) {
-    if constexpr (N == 1) {
+    if constexpr (std::is_class<T>::value) {
+        constexpr int W = N * static_cast<int>(sizeof(T)) / 4;
+        store_stream(reinterpret_cast<Vec<uint32_t, W>*>(p), bit_cast<Vec<uint32_t, W>>(v));
+    } else if constexpr (N == 1) {
         __builtin_nontemporal_store(v.v[0], reinterpret_cast<T*>(p));
     } else {
         typedef T NV __attribute__((ext_vector_type(N)));
@@ -285,9 +314,20 @@ __device__ __forceinline__ void store_stream(Vec<T, N>* p, const Vec<T, N>& v) {
     }
 }
 template <typename T>
-__device__ __forceinline__ T load_stream(const T* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ T load_stream(const T* p) {
+    if constexpr (std::is_class<T>::value) return load_stream(reinterpret_cast<const Vec<T, 1>*>(p)).v[0];
+    else return __builtin_nontemporal_load(p);
+}
 template <typename T>
-__device__ __forceinline__ void store_stream(T* p, T v) { __builtin_nontemporal_store(v, p); }
+__device__ __forceinline__ void store_stream(T* p, T v) {
+    if constexpr (std::is_class<T>::value) {
+        Vec<T, 1> one;
+        one.v[0] = v;
+        store_stream(reinterpret_cast<Vec<T, 1>*>(p), one);
+    } else {
+        __builtin_nontemporal_store(v, p);
+    }
+}
 
 // ------------------------------------------------------------------ host launch helpers
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -350,7 +390,8 @@ inline int dispatch_dtype16(int dtype, F&& f) {
 inline size_t dtype_size(int dtype) {
     switch (dtype) {
     case DLFX_F32: case DLFX_I32: return 4;
-    case DLFX_F64: case DLFX_I64: return 8;
+    case DLFX_F64: case DLFX_I64: case DLFX_C64: return 8;
+    case DLFX_C128: return 16;
     case DLFX_F16: case DLFX_I16: return 2;
     case DLFX_BOOL: return 1;
     default: return 0;

@@ -21,7 +21,7 @@ namespace dlfx {
 namespace {
 
 enum JoinKind { kAdd = 0, kMul = 1, kMax = 2, kMin = 3 };
-enum MapKind { kMapId = 0, kMapExp = 1, kMapAbs = 2, kMapSquare = 3 };
+enum MapKind { kMapId = 0, kMapExp = 1, kMapAbs = 2, kMapSquare = 3, kMapNorm = 4 };     // norm: |x|^2, x*x for reals
 enum FinalKind { kFinalId = 0, kFinalMean = 1, kFinalLog = 2, kFinalSqrt = 3 };
 
 constexpr int kBlock = 256;
@@ -112,6 +112,60 @@ struct ValueReducer {
             else if (final_op == kFinalSqrt) v = sqrt(v);
             return static_cast<T>(v);
         }
+    }
+};
+
+// The same table over complex elements (std::complex on the reference's host side: abs and
+// norm give a real value held in a complex, exp / log / sqrt are the principal complex
+// functions, mean divides by (n, 0)).  Both parts accumulate in fp64.  Ordering reducers
+// (max, min, amax, amin) have no meaning here and are rejected by the caller.
+template <typename F, int J, int M>
+struct ComplexReducer {
+    using in_t = Cx<F>;
+    using acc_t = Cx<double>;
+    using out_t = Cx<F>;
+    using param_t = int;
+
+    __device__ static __forceinline__ acc_t identity() { return J == kMul ? acc_t(1.0, 0.0) : acc_t(0.0, 0.0); }
+    __device__ static __forceinline__ acc_t map(in_t x, int64_t, param_t) {
+        if constexpr (M == kMapExp) {
+            if constexpr (std::is_same<F, float>::value) {
+                const float e = expf(x.re);
+                float s, c;
+                sincosf(x.im, &s, &c);
+                return acc_t(static_cast<double>(e * c), static_cast<double>(e * s));
+            } else {
+                const double e = exp(x.re);
+                double s, c;
+                sincos(x.im, &s, &c);
+                return acc_t(e * c, e * s);
+            }
+        } else if constexpr (M == kMapAbs) {
+            return acc_t(hypot(static_cast<double>(x.re), static_cast<double>(x.im)), 0.0);
+        } else if constexpr (M == kMapSquare) {
+            const acc_t v(x);
+            return v * v;
+        } else if constexpr (M == kMapNorm) {
+            const acc_t v(x);
+            return acc_t(v.re * v.re + v.im * v.im, 0.0);
+        } else {
+            return acc_t(x);
+        }
+    }
+    __device__ static __forceinline__ acc_t join(acc_t a, acc_t b) { return J == kMul ? a * b : a + b; }
+    __device__ static __forceinline__ out_t finish(acc_t a, int64_t n, int final_op) {
+        if (final_op == kFinalMean) {
+            a = acc_t(a.re / static_cast<double>(n), a.im / static_cast<double>(n));
+        } else if (final_op == kFinalLog) {
+            a = acc_t(log(hypot(a.re, a.im)), atan2(a.im, a.re));
+        } else if (final_op == kFinalSqrt) {
+            // principal square root: non-negative real part, imaginary part with the sign of a.im
+            const double mod = hypot(a.re, a.im);
+            const double big = sqrt((mod + fabs(a.re)) * 0.5);
+            const double small = big > 0.0 ? fabs(a.im) / (2.0 * big) : 0.0;
+            a = a.re >= 0.0 ? acc_t(big, copysign(small, a.im)) : acc_t(small, copysign(big, a.im));
+        }
+        return out_t(a);
     }
 };
 
@@ -486,7 +540,7 @@ const ReduceOp kReduceOps[] = {
     {"reduce_prod", kMul, kMapId, kFinalId, false},
     {"reduce_asum", kAdd, kMapAbs, kFinalId, false},
     {"reduce_sum_square", kAdd, kMapSquare, kFinalId, false},
-    {"reduce_nrm2", kAdd, kMapSquare, kFinalSqrt, true},
+    {"reduce_nrm2", kAdd, kMapNorm, kFinalSqrt, true},
     {"reduce_amax", kMax, kMapAbs, kFinalId, false},
     {"reduce_amin", kMin, kMapAbs, kFinalId, false},
 };
@@ -500,6 +554,8 @@ int launch_reduce_typed(hipStream_t stream, const ReduceOp& op, const ReducePlan
     DLFX_CASE(kAdd, kMapId)
     DLFX_CASE(kAdd, kMapAbs)
     DLFX_CASE(kAdd, kMapSquare)
+    if (op.join == kAdd && op.map == kMapNorm)           // |x|^2 of a real is its square
+        return launch_reduce<ValueReducer<T, kAdd, kMapSquare>>(stream, pl, x, y, op.final_op, scratch, scratch_bytes);
     DLFX_CASE(kMul, kMapId)
     DLFX_CASE(kMax, kMapId)
     DLFX_CASE(kMin, kMapId)
@@ -510,6 +566,22 @@ int launch_reduce_typed(hipStream_t stream, const ReduceOp& op, const ReducePlan
     }
 #undef DLFX_CASE
     return DLFX_ERR_UNKNOWN_OP;
+}
+
+template <typename F>
+int launch_reduce_complex(hipStream_t stream, const ReduceOp& op, const ReducePlan& pl, const Cx<F>* x, Cx<F>* y,
+                          void* scratch, size_t scratch_bytes) {
+#define DLFX_CASE(J, M)                                                                       \
+    if (op.join == J && op.map == M)                                                          \
+        return launch_reduce<ComplexReducer<F, J, M>>(stream, pl, x, y, op.final_op, scratch, scratch_bytes);
+    DLFX_CASE(kAdd, kMapId)
+    DLFX_CASE(kAdd, kMapAbs)
+    DLFX_CASE(kAdd, kMapSquare)
+    DLFX_CASE(kAdd, kMapNorm)
+    DLFX_CASE(kAdd, kMapExp)
+    DLFX_CASE(kMul, kMapId)
+#undef DLFX_CASE
+    return DLFX_ERR_UNSUPPORTED_DTYPE;      // max / min / amax / amin: complex numbers are not ordered
 }
 
 }  // namespace
@@ -554,6 +626,12 @@ extern "C" int dlfx_reduce(dlfx_stream_t stream, const char* name, int dtype, in
         !make_dim_map(y_dims, y_strides, 0, y_rank, &pl.ymap))
         return DLFX_ERR_RANK;
 
+    if (dtype == DLFX_C64)
+        return launch_reduce_complex<float>(static_cast<hipStream_t>(stream), *op, pl, static_cast<const Cx<float>*>(x) + x_offset,
+                                            static_cast<Cx<float>*>(y) + y_offset, scratch, scratch_bytes);
+    if (dtype == DLFX_C128)
+        return launch_reduce_complex<double>(static_cast<hipStream_t>(stream), *op, pl, static_cast<const Cx<double>*>(x) + x_offset,
+                                             static_cast<Cx<double>*>(y) + y_offset, scratch, scratch_bytes);
     return dispatch_dtype_half(dtype, [&](auto tag) {
         using T = decltype(tag);
         return launch_reduce_typed<T>(static_cast<hipStream_t>(stream), *op, pl,
@@ -644,12 +722,15 @@ extern "C" int dlfx_count(dlfx_stream_t stream, int dtype, int64_t m, int64_t n,
         !make_dim_map(y_dims, y_strides, 0, y_rank, &pl.ymap))
         return DLFX_ERR_RANK;
 
-    return dispatch_dtype_half(dtype, [&](auto tag) {
+    auto count_as = [&](auto tag) {
         using T = decltype(tag);
         T v;
         std::memcpy(&v, value, sizeof(T));
         return launch_reduce<CountReducer<T>>(static_cast<hipStream_t>(stream), pl,
                                               static_cast<const T*>(x) + x_offset, y + y_offset, kFinalId,
                                               scratch, scratch_bytes, v);
-    });
+    };
+    if (dtype == DLFX_C64) return count_as(Cx<float>());
+    if (dtype == DLFX_C128) return count_as(Cx<double>());
+    return dispatch_dtype_half(dtype, count_as);
 }

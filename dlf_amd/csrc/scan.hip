@@ -110,6 +110,43 @@ struct TileState<T, 8> {
     }
 };
 
+// 16-byte values (complex of doubles): as the 8-byte case with two words per value.
+template <typename T>
+struct TileState<T, 16> {
+    struct Pair {
+        unsigned long long lo, hi;
+    };
+    uint32_t* flags;
+    unsigned long long* agg;
+    unsigned long long* incl;
+    static size_t bytes(int64_t tiles) { return align_up(static_cast<size_t>(tiles) * 4, 256) + static_cast<size_t>(tiles) * 32; }
+    __host__ __device__ void bind(void* base, int64_t tiles) {
+        flags = static_cast<uint32_t*>(base);
+        size_t off = (static_cast<size_t>(tiles) * 4 + 255) / 256 * 256;
+        agg = reinterpret_cast<unsigned long long*>(static_cast<char*>(base) + off);
+        incl = agg + 2 * tiles;
+    }
+    __device__ __forceinline__ void clear(int64_t i) { flags[i] = 0u; }
+    __device__ __forceinline__ void publish(int64_t i, uint32_t flag, T v) {
+        unsigned long long* dst = (flag == kAggregate) ? agg : incl;
+        const Pair p = bit_cast<Pair>(v);
+        __hip_atomic_store(&dst[2 * i], p.lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&dst[2 * i + 1], p.hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&flags[i], flag, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __device__ __forceinline__ uint32_t read(int64_t i, T* v) {
+        uint32_t f = __hip_atomic_load(&flags[i], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+        if (f != kInvalid) {
+            unsigned long long* src = (f == kAggregate) ? agg : incl;
+            Pair p;
+            p.lo = __hip_atomic_load(&src[2 * i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            p.hi = __hip_atomic_load(&src[2 * i + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *v = bit_cast<T>(p);
+        }
+        return f;
+    }
+};
+
 template <typename T>
 __global__ __launch_bounds__(kBlock) void scan_init(unsigned* ticket, int64_t rows, TileState<T> st, int64_t tiles) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
@@ -467,7 +504,7 @@ ScanLayout scan_layout(size_t elem_size, int64_t m, int64_t n) {
         l.total = 0;
     } else {
         size_t sb = elem_size == 4 ? static_cast<size_t>(l.tiles) * 8
-                                   : align_up(static_cast<size_t>(l.tiles) * 4, 256) + static_cast<size_t>(l.tiles) * 16;
+                                   : align_up(static_cast<size_t>(l.tiles) * 4, 256) + static_cast<size_t>(l.tiles) * 2 * elem_size;
         l.total = l.state_off + align_up(sb, 256);
     }
     return l;
@@ -611,6 +648,18 @@ extern "C" int dlfx_scan(dlfx_stream_t stream, const char* name, int dtype, int6
         case kScanMax: return launch_scan<float, kScanMax, half_t, false, half_t>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
         default:       return launch_scan<float, kScanMin, half_t, false, half_t>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
         }
+    }
+    if (dtype == DLFX_C64 || dtype == DLFX_C128) {
+        // running sums and products of complex elements; complex numbers are not ordered
+        if (kind != kScanAdd && kind != kScanMul) return DLFX_ERR_UNSUPPORTED_DTYPE;
+        auto run = [&](auto tag) {
+            using T = decltype(tag);
+            const T* xp = static_cast<const T*>(x) + x_offset;
+            T* yp = static_cast<T*>(y) + y_offset;
+            if (kind == kScanAdd) return launch_scan<T, kScanAdd>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
+            return launch_scan<T, kScanMul>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
+        };
+        return dtype == DLFX_C64 ? run(Cx<float>()) : run(Cx<double>());
     }
     return dispatch_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);

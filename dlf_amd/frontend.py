@@ -19,7 +19,8 @@ from .shape import Shape, ShapeError, norm_axes, norm_axis
 
 DTYPE_CODES = {np.dtype(np.float32): 0, np.dtype(np.float64): 1,
                np.dtype(np.int32): 2, np.dtype(np.int64): 3,
-               np.dtype(np.float16): 4, np.dtype(np.int16): 5, np.dtype(np.bool_): 6}
+               np.dtype(np.float16): 4, np.dtype(np.int16): 5, np.dtype(np.bool_): 6,
+               np.dtype(np.complex64): 7, np.dtype(np.complex128): 8}
 
 REDUCE_NAMES = ("reduce_sum", "reduce_mean", "reduce_max", "reduce_min", "reduce_log_sum_exp",
                 "reduce_sum_exp", "reduce_log_sum", "reduce_prod", "reduce_asum",

@@ -146,7 +146,8 @@ def _torch_dtype(np_dtype):
         _NP_TO_TORCH = {np.dtype(np.float32): torch.float32, np.dtype(np.float64): torch.float64,
                         np.dtype(np.int32): torch.int32, np.dtype(np.int64): torch.int64,
                         np.dtype(np.float16): torch.float16, np.dtype(np.int16): torch.int16,
-                        np.dtype(np.bool_): torch.bool}
+                        np.dtype(np.bool_): torch.bool,
+                        np.dtype(np.complex64): torch.complex64, np.dtype(np.complex128): torch.complex128}
     return _NP_TO_TORCH[np.dtype(np_dtype)]
 
 
@@ -255,7 +256,9 @@ class HipBackend:
 
     def count(self, dtype, m, n, value, xs, x, ys, y, defer=False):
         sp, sb = self.scratch(self.lib.dlfx_count_scratch_bytes(dtype, m, n))
-        v = np.array([value], dtype=(np.float32, np.float64, np.int32, np.int64, np.float16, np.int16)[dtype])   # one host element of the input's type
+        host_types = {0: np.float32, 1: np.float64, 2: np.int32, 3: np.int64, 4: np.float16, 5: np.int16,
+                      7: np.complex64, 8: np.complex128}
+        v = np.array([value], dtype=host_types[dtype])       # one host element of the input's type
         keep = v.ctypes.data_as(c_void_p)
         call = self._issue(self.lib.dlfx_count, "dlfx_count", (dtype, m, n, keep),
                            (xs.rank, _arr(xs.extents), _arr(xs.strides), x.data_ptr(), xs.offset,

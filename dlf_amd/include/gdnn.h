@@ -13,6 +13,8 @@
 #include <type_traits>
 #include <vector>
 
+#include <complex>
+
 #include "dlfx.h"
 #include "gblas_half.h"
 #include "gpgpu.h"
@@ -28,6 +30,8 @@ template <> struct dtype_of<int32_t> { static constexpr int value = DLFX_I32; };
 template <> struct dtype_of<int64_t> { static constexpr int value = DLFX_I64; };
 template <> struct dtype_of<int16_t> { static constexpr int value = DLFX_I16; };
 template <> struct dtype_of<blas::half> { static constexpr int value = DLFX_F16; };
+template <> struct dtype_of<std::complex<float>>  { static constexpr int value = DLFX_C64; };     // float2
+template <> struct dtype_of<std::complex<double>> { static constexpr int value = DLFX_C128; };    // double2
 
 // size_t strides that wrapped for a negative step come back as the negative number
 inline std::vector<int64_t> signed_vec(const std::vector<size_t>& v) {

@@ -50,7 +50,9 @@ typedef enum dlfx_dtype {
     DLFX_I64 = 3,
     DLFX_F16 = 4,   /* IEEE half: every entry point (sums and scans accumulate in fp32, rounded once) */
     DLFX_I16 = 5,   /* arg_reduce, sort, argsort, top_k (the reference's int16 instantiations) and merge */
-    DLFX_BOOL = 6   /* one byte per element; input of scan_nonzero only */
+    DLFX_BOOL = 6,  /* one byte per element; input of scan_nonzero only */
+    DLFX_C64 = 7,   /* complex of two floats (the reference's float2): reduce, count, scan */
+    DLFX_C128 = 8   /* complex of two doubles (double2): reduce, count, scan */
 } dlfx_dtype;
 
 typedef enum dlfx_status {

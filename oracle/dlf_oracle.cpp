@@ -35,6 +35,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <complex>
 #include <cstdint>
 #include <cstring>
 #include <functional>
@@ -104,6 +105,13 @@ bool parse_reduce(const char* name, Red* r) {
     return false;
 }
 
+// std::complex elements (float2 / double2 on the device side): the reducer table instantiated
+// with T = std::complex<F> as the reference's host templates do (abs and norm yield a real
+// value converted back to T, exp / log / sqrt are the std::complex functions, mean divides by
+// T(n)); the ordering reducers do not compile there and are rejected here.
+template <typename T> struct is_complex : std::false_type {};
+template <typename F> struct is_complex<std::complex<F>> : std::true_type {};
+
 template <typename T> T t_abs(T x) { return x < 0 ? T(-x) : x; }
 template <typename T> T t_exp(T x) { return static_cast<T>(std::exp(static_cast<double>(x))); }
 template <> float  t_exp<float>(float x)   { return std::exp(x); }
@@ -115,6 +123,8 @@ template <typename T> T t_sqrt(T x) { return static_cast<T>(std::sqrt(static_cas
 template <> float  t_sqrt<float>(float x)  { return std::sqrt(x); }
 
 template <typename T> T red_identity(Red r) {
+    if constexpr (is_complex<T>::value) return r == Red::Prod ? T(1) : T(0);
+    else
     switch (r) {
     case Red::Max: return std::numeric_limits<T>::lowest();
     case Red::Min: case Red::AMin: return std::numeric_limits<T>::max();
@@ -123,6 +133,15 @@ template <typename T> T red_identity(Red r) {
     }
 }
 template <typename T> T red_map(Red r, T x) {
+    if constexpr (is_complex<T>::value) {
+        switch (r) {
+        case Red::LogSumExp: case Red::SumExp: return std::exp(x);
+        case Red::ASum: return T(std::abs(x));
+        case Red::SumSquare: return x * x;
+        case Red::Nrm2: return T(std::norm(x));
+        default: return x;
+        }
+    } else
     switch (r) {
     case Red::LogSumExp: case Red::SumExp: return t_exp(x);
     case Red::ASum: case Red::AMax: case Red::AMin: return t_abs(x);
@@ -131,6 +150,8 @@ template <typename T> T red_map(Red r, T x) {
     }
 }
 template <typename T> T red_join(Red r, T a, T b) {
+    if constexpr (is_complex<T>::value) return r == Red::Prod ? a * b : a + b;
+    else
     switch (r) {
     case Red::Max: return std::max(a, b);
     case Red::Min: return std::min(a, b);
@@ -141,6 +162,14 @@ template <typename T> T red_join(Red r, T a, T b) {
     }
 }
 template <typename T> T red_final(Red r, T acc, int64_t n) {
+    if constexpr (is_complex<T>::value) {
+        switch (r) {
+        case Red::Mean: return acc / T(static_cast<typename T::value_type>(n));
+        case Red::LogSumExp: case Red::LogSum: return std::log(acc);
+        case Red::Nrm2: return std::sqrt(acc);
+        default: return acc;
+        }
+    } else
     switch (r) {
     case Red::Mean: return T(acc / static_cast<T>(n));
     case Red::LogSumExp: case Red::LogSum: return t_log(acc);
@@ -274,6 +303,8 @@ bool parse_scan(const char* name, Scn* s) {
     return false;
 }
 template <typename T> T scan_identity(Scn s) {
+    if constexpr (is_complex<T>::value) return s == Scn::Prod ? T(1) : T(0);
+    else
     switch (s) {
     case Scn::Prod: return T(1);
     case Scn::Max: return std::numeric_limits<T>::lowest();
@@ -282,6 +313,8 @@ template <typename T> T scan_identity(Scn s) {
     }
 }
 template <typename T> T scan_op(Scn s, T a, T b) {
+    if constexpr (is_complex<T>::value) return s == Scn::Prod ? a * b : a + b;
+    else
     switch (s) {
     case Scn::Prod: return T(a * b);
     case Scn::Max: return std::max(a, b);
@@ -547,6 +580,16 @@ int by_dtype(int dtype, F&& f) {
     }
 }
 
+// dtype codes 7 / 8: complex of floats / doubles (reduce, count and scan only)
+template <typename F>
+int by_dtype_complex(int dtype, F&& f) {
+    if (dtype == 7) return f(std::complex<float>());
+    if (dtype == 8) return f(std::complex<double>());
+    return by_dtype(dtype, f);
+}
+bool complex_dtype(int dtype) { return dtype == 7 || dtype == 8; }
+bool ordered_only(Red r) { return r == Red::Max || r == Red::Min || r == Red::AMax || r == Red::AMin; }
+
 }  // namespace
 
 extern "C" {
@@ -575,7 +618,8 @@ int dlf_oracle_reduce(const char* name, int dtype, int64_t m, int64_t n,
     Red r;
     if (!parse_reduce(name, &r)) return -1;
     View xv(x_rank, x_dims, x_strides, x_offset), yv(y_rank, y_dims, y_strides, y_offset);
-    return by_dtype(dtype, [&](auto tag) {
+    if (complex_dtype(dtype) && ordered_only(r)) return -2;
+    return by_dtype_complex(dtype, [&](auto tag) {
         using T = decltype(tag);
         return do_reduce<T>(r, m, n, xv, static_cast<const T*>(x), yv, static_cast<T*>(y));
     });
@@ -616,7 +660,8 @@ int dlf_oracle_scan(const char* name, int dtype, int64_t m, int64_t n, int exclu
     Scn s;
     if (!parse_scan(name, &s)) return -1;
     View xv(rank, dims, x_strides, x_offset), yv(rank, dims, y_strides, y_offset);
-    return by_dtype(dtype, [&](auto tag) {
+    if (complex_dtype(dtype) && (s == Scn::Max || s == Scn::Min)) return -2;
+    return by_dtype_complex(dtype, [&](auto tag) {
         using T = decltype(tag);
         return do_scan<T>(s, m, n, exclusive != 0, xv, static_cast<const T*>(x), yv, static_cast<T*>(y));
     });
@@ -690,7 +735,7 @@ int dlf_oracle_count(int dtype, int64_t m, int64_t n, const void* value,
                      int y_rank, const int64_t* y_dims, const int64_t* y_strides,
                      int32_t* y, int64_t y_offset) {
     View xv(x_rank, x_dims, x_strides, x_offset), yv(y_rank, y_dims, y_strides, y_offset);
-    return by_dtype(dtype, [&](auto tag) {
+    return by_dtype_complex(dtype, [&](auto tag) {
         using T = decltype(tag);
         T v;
         std::memcpy(&v, value, sizeof(T));

@@ -10,6 +10,7 @@
 // (softmax, logsoftmax, hardmax).
 #include <algorithm>
 #include <cmath>
+#include <complex>
 #include <cstdio>
 #include <random>
 
@@ -255,6 +256,18 @@ static void test_16bit_types() {
           static_cast<float>(sm.values()[7]) == 0.0f);
 }
 
+// dlf/test/UniformTest.cpp:2060-2063 through the device front-end, plus a complex running sum
+static void test_complex() {
+    using C = std::complex<float>;
+    auto X = Tensor<C>({2}, {C(3, 4), C(5, 12)});
+    auto nrm = reduce_nrm2(dev(X), {0}).read();
+    CHECK(std::abs(nrm.values()[0] - C(std::sqrt(194.f))) < 1e-5f);
+    auto Y = Tensor<C>({2, 3}, {C(1, 1), C(2, -1), C(0, 3), C(-1, 0), C(0, 0), C(4, 4)});
+    CHECK(reduce_sum(dev(Y), {1}).read() == Tensor<C>({2}, {C(3, 3), C(3, 4)}));
+    CHECK(cumsum(dev(Y), 1).read() == Tensor<C>({2, 3}, {C(1, 1), C(3, 0), C(3, 3), C(-1, 0), C(-1, 0), C(3, 4)}));
+    CHECK(count(dev(Y), C(0, 0), {}).read() == Tensor<int>({}, {1}));
+}
+
 static void test_errors_and_temporaries() {
     auto X = dev(Tensor<float>({2, 3}).range());
     bool threw = false;
@@ -304,6 +317,7 @@ int main() {
     test_merge();
     test_softmax_family();
     test_16bit_types();
+    test_complex();
     test_errors_and_temporaries();
     std::printf("veneer_test: %d checks, %d failed\n", g_checked, g_failed);
     return g_failed ? 1 : 0;

@@ -326,3 +326,43 @@ def test_half_sums_round_once(oracle_backend):
 def test_bool_nonzero(oracle_backend):
     b = randint(142, 6 * 40, 0, 3).reshape(6, 40) == 0
     assert np.array_equal(F.nonzero(Tensor.from_numpy(oracle_backend, b)).numpy(), np.argwhere(b))
+
+
+# ---------------------------------------------------------------- complex elements
+@pytest.mark.parametrize("dtype", [np.complex64, np.complex128])
+def test_complex_reduce_count_scan_match_numpy(oracle_backend, dtype):
+    n = 4 * 9 * 50
+    x = ((normal(143, n) + 1j * normal(144, n)) * 0.7).astype(dtype).reshape(4, 9, 50)
+    X = Tensor.from_numpy(oracle_backend, x)
+    x128 = x.astype(np.complex128)
+    rtol = 200 * np.finfo(dtype).eps
+    for axes in ((), (1,), (0, 2)):
+        ax = axes if axes else None
+        cases = {"reduce_sum": x128.sum(axis=ax), "reduce_mean": x128.mean(axis=ax),
+                 "reduce_asum": np.abs(x128).sum(axis=ax), "reduce_sum_square": (x128 * x128).sum(axis=ax),
+                 "reduce_nrm2": np.sqrt((np.abs(x128) ** 2).sum(axis=ax)),
+                 "reduce_sum_exp": np.exp(x128).sum(axis=ax), "reduce_log_sum": np.log(x128.sum(axis=ax)),
+                 "reduce_log_sum_exp": np.log(np.exp(x128).sum(axis=ax))}
+        for name, want in cases.items():
+            got = F.reduce(name, X, axes).numpy()
+            assert got.dtype == dtype
+            assert np.allclose(got.reshape(-1), np.asarray(want).reshape(-1), rtol=rtol, atol=rtol * 50), name
+    u = np.exp(1j * normal(145, 3 * 40).reshape(3, 40)).astype(dtype)
+    U = Tensor.from_numpy(oracle_backend, u)
+    assert np.allclose(F.reduce("reduce_prod", U, (1,)).numpy(), u.astype(np.complex128).prod(axis=1), rtol=rtol, atol=rtol)
+    assert np.allclose(F.cumprod(U, 1).numpy(), np.cumprod(u.astype(np.complex128), axis=1), rtol=rtol, atol=rtol)
+    assert np.allclose(F.cumsum(X, 1, exclusive=True).numpy()[:, 1:], np.cumsum(x128, axis=1)[:, :-1], rtol=rtol, atol=rtol * 50)
+    y = (randint(146, 200, 0, 2) + 1j * randint(147, 200, 0, 2)).astype(dtype).reshape(4, 50)
+    assert np.array_equal(F.count(Tensor.from_numpy(oracle_backend, y), 1 + 1j, (1,)).numpy(), (y == 1 + 1j).sum(axis=1))
+    for name in ("reduce_max", "reduce_amin"):
+        with pytest.raises(Exception):
+            F.reduce(name, X, ())
+    with pytest.raises(Exception):
+        F.cummax(X, 1)
+
+
+def test_complex_nrm2_reference_vector(oracle_backend):
+    # dlf/test/UniformTest.cpp:2060-2063
+    x = np.array([3 + 4j, 5 + 12j], dtype=np.complex64)
+    got = F.reduce("reduce_nrm2", Tensor.from_numpy(oracle_backend, x), (0,)).numpy()
+    assert got.reshape(-1)[0] == np.complex64(np.sqrt(np.float32(194.0)))
