@@ -181,7 +181,7 @@ constexpr int kRowShr1 = 0x111, kRowShr2 = 0x112, kRowShr4 = 0x114, kRowShr8 = 0
 constexpr int kRowBcast15 = 0x142, kRowBcast31 = 0x143;
 
 // Value of `v` in lane (lane ^ J), J a power of two.  Distances below 16 stay inside a DPP
-// row and cost one or two moves; 16 and 32 cross rows and go through the LDS crossbar.
+// row and cost one or two moves; 16 and 32 cross rows with one lane-swap instruction and a select.
 template <int J, typename T>
 __device__ __forceinline__ T lane_xor_const(T v) {
     if constexpr (J == 1) return dpp_fetch<kQuadXor1>(v, v);
@@ -191,7 +191,33 @@ __device__ __forceinline__ T lane_xor_const(T v) {
         const T up = dpp_fetch<0x104, 0xf, 0x5>(v, v);        // row_shl:4 into banks 0 and 2
         return dpp_fetch<0x114, 0xf, 0xa>(v, up);             // row_shr:4 into banks 1 and 3
     } else if constexpr (J == 8) return dpp_fetch<0x128>(v, v);   // row_ror:8
-    else return lane_xor(v, J);
+    else {
+        // v_permlane16_swap exchanges the odd rows of its first operand with the even rows of
+        // its second, v_permlane32_swap the upper half of the first with the lower half of the
+        // second: with both operands holding v, the first result carries v's even rows (lower
+        // half) twice and the second its odd rows (upper half) twice.
+        static_assert(J == 16 || J == 32, "power-of-two distance inside a wavefront");
+        const bool upper = (__lane_id() & J) != 0;
+        auto word = [&](int w) -> int {
+            const unsigned u = static_cast<unsigned>(w);
+            if constexpr (J == 16) {
+                const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+                return static_cast<int>(upper ? r[0] : r[1]);
+            } else {
+                const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+                return static_cast<int>(upper ? r[0] : r[1]);
+            }
+        };
+        if constexpr (sizeof(T) == 2) {
+            return narrow16<T>(word(widen16(v)));
+        } else {
+            constexpr int N = sizeof(T) / 4;
+            Words<N> a = bit_cast<Words<N>>(v);
+#pragma unroll
+            for (int i = 0; i < N; ++i) a.w[i] = word(a.w[i]);
+            return bit_cast<T>(a);
+        }
+    }
 }
 
 // Bitonic network over aligned groups of WIDTH lanes (a power of two, at most 64); the group

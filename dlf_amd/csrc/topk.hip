@@ -29,6 +29,17 @@ namespace {
 constexpr int kRadix = 256;
 constexpr int kMaxLimit = 1024;
 
+#ifdef DLFX_TOPK_TIMING
+// Debug builds only: shader-clock cycles spent by thread 0 of every workgroup in each phase.
+constexpr int kPhaseSlots = 8192;
+__device__ unsigned long long g_topk_cycles[kPhaseSlots * 8];
+#define DLFX_PHASE(i) do { if (threadIdx.x == 0) { const long long now_ = clock64(); g_topk_cycles[(blockIdx.x % kPhaseSlots) * 8 + (i)] += static_cast<unsigned long long>(now_ - phase_t_); phase_t_ = now_; } } while (0)
+#define DLFX_PHASE_BEGIN() long long phase_t_ = clock64()
+#else
+#define DLFX_PHASE(i) do { } while (0)
+#define DLFX_PHASE_BEGIN() do { } while (0)
+#endif
+
 enum KeyKind { kKeyInt = 0, kKeyFloat = 1 };
 
 template <typename K>
@@ -286,15 +297,24 @@ __device__ __forceinline__ void wave_sort_entries(K& o, uint32_t& x) {
 }
 
 constexpr int kMergeMax = 512;       // entries up to which sorted runs are merged by rank
+constexpr int kCountMax = 20;        // entries up to which ranks are counted directly
 
 // Orders `count` distinct (image, index) entries held in LDS, best first, and writes those
 // ranked below `limit` to the outputs.  The arrays must have room for count rounded up to a
 // multiple of 64 and are overwritten.  Each wave sorts runs of 64 entries in registers; the
 // rank of an entry is its position in its run plus, for every other run, the number of that
 // run's entries that beat it, found by bisection.  All threads of the team must call.
-template <int BLOCK, typename K, typename S>
+struct KeepImage {
+    template <typename K>
+    __device__ __forceinline__ K operator()(K v) const { return v; }
+};
+
+// `image_of` maps what e_ord holds to the image (the identity unless the caller stored
+// something cheaper to produce).
+template <int BLOCK, typename K, typename S, typename ImageOf = KeepImage>
 __device__ __forceinline__ void merge_rank_emit(K* e_ord, uint32_t* e_idx, int count, int limit,
-                                                const TopkIo<K, S>& io, int64_t row, const S* xr) {
+                                                const TopkIo<K, S>& io, int64_t row, const S* xr,
+                                                ImageOf image_of = ImageOf()) {
     constexpr int WAVES = BLOCK / kWave;
     const int tid = threadIdx.x;
     const int lane = lane_id();
@@ -302,9 +322,20 @@ __device__ __forceinline__ void merge_rank_emit(K* e_ord, uint32_t* e_idx, int c
     const int runs = (count + kWave - 1) / kWave;
     S* yr = io.y + io.ymap.at(row);
     const int64_t ir = io.imap.at(row);
+    if (count <= kCountMax) {
+        // a handful of entries: the first wave counts, for each, the entries that beat it
+        if (w == 0) {
+            const K o = lane < count ? image_of(e_ord[lane]) : K(0);
+            const uint32_t x = lane < count ? e_idx[lane] : 0xffffffffu;
+            uint32_t rank = 0;
+            for (int j = 0; j < count; ++j) rank += beats<K>(lane_read(o, j), lane_read(x, j), o, x);
+            if (lane < count && rank < static_cast<uint32_t>(limit)) emit_one<K>(io, yr, ir, xr, static_cast<int>(rank), o, x);
+        }
+        return;
+    }
     for (int r = w; r < runs; r += WAVES) {
         const int e = r * kWave + lane;
-        K o = e < count ? e_ord[e] : K(0);
+        K o = e < count ? image_of(e_ord[e]) : K(0);
         uint32_t x = e < count ? e_idx[e] : 0xffffffffu;      // padding: beaten by every entry
         wave_sort_entries<K>(o, x);
         if (runs == 1) {
@@ -357,13 +388,16 @@ __device__ __forceinline__ void merge_rank_emit(K* e_ord, uint32_t* e_idx, int c
 #pragma unroll
             for (int u = 0; u < U; ++u) rank += c[u];
         };
-        const int others = runs - 1;
-        int r0 = 0;
-        for (; r0 + 4 <= others; r0 += 4) bisect(std::integral_constant<int, 4>(), r0);
-        switch (others - r0) {
-        case 3: bisect(std::integral_constant<int, 3>(), r0); break;
-        case 2: bisect(std::integral_constant<int, 2>(), r0); break;
-        case 1: bisect(std::integral_constant<int, 1>(), r0); break;
+        // all the other runs (at most seven: kMergeMax / 64 - 1) are bisected side by side
+        static_assert(kMergeMax / kWave - 1 == 7, "one case per possible number of other runs");
+        switch (runs - 1) {
+        case 7: bisect(std::integral_constant<int, 7>(), 0); break;
+        case 6: bisect(std::integral_constant<int, 6>(), 0); break;
+        case 5: bisect(std::integral_constant<int, 5>(), 0); break;
+        case 4: bisect(std::integral_constant<int, 4>(), 0); break;
+        case 3: bisect(std::integral_constant<int, 3>(), 0); break;
+        case 2: bisect(std::integral_constant<int, 2>(), 0); break;
+        case 1: bisect(std::integral_constant<int, 1>(), 0); break;
         default: break;
         }
         if (rank < static_cast<uint32_t>(limit)) emit_one<K>(io, yr, ir, xr, static_cast<int>(rank), o, x);
@@ -584,6 +618,7 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
     const int64_t row = blockIdx.x;
     const S* xr = io.x + io.xmap.at(row);
     if (tid < kRadix) sm.hist[tid] = 0;
+    DLFX_PHASE_BEGIN();
 
     // item (g, e) of thread t is element ((g*BLOCK + t)*V + e) of the row
     const uint32_t n32 = static_cast<uint32_t>(n);        // rows here have at most 65536 elements
@@ -628,70 +663,111 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
             }
         }
         // ---- pre-filter.  The largest element of each thread is a distinct element of the
-        // row.  Every wave sorts its 64 of them; the value at position p*s - 1 of a wave has
-        // p*s elements of the row at or above it.  Four such samples per wave (p = 1..4) are
-        // sorted together: the m-th largest sample has at least m*s elements at or above it
-        // (q samples of one wave among the first m stand for q*s elements of that wave), so
-        // with m*s >= limit it cannot exceed the limit-th largest element of the row and
-        // everything below it is out.  What is left is usually 1 to 1.5 times `limit` elements.
+        // row, and so is the largest of any group of threads.  A bound that provably has at
+        // least `limit` elements at or above it comes from 16 or 64 such samples:
+        //   * limit <= 16: the limit-th largest of the 16 wave maxima;
+        //   * limit <= 64: the limit-th largest of the 64 maxima of 16-lane rows;
+        //   * above: every wave sorts its 64 thread maxima; the value at position p*s - 1 of a
+        //     wave has p*s elements at or above it.  Four such samples per wave (p = 1..4) are
+        //     sorted together: the m-th largest sample has at least m*s elements at or above
+        //     it (q samples of one wave among the first m stand for q*s elements of that
+        //     wave), so with m*s >= limit it cannot exceed the limit-th largest element.
+        // Everything below the bound is out; what is left is usually 1 to 2 times `limit`.
         static_assert(WAVES == 16, "four samples from each of sixteen waves fill one wave");
         T tmax = worst;
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) tmax = sc[i] > tmax ? sc[i] : tmax;
         T* red = reinterpret_cast<T*>(sm.out_ord);
+        if (tid == 0) sm.count = 0u;
+        DLFX_PHASE(0);            // loads and thread maxima
+        auto larger = [](T a, T b) { return a > b ? a : b; };
         int samples, mth;
         if (limit <= WAVES) {
-            const T wmax = wave_reduce(tmax, [](T a, T b) { return a > b ? a : b; });
+            const T wmax = wave_reduce(tmax, larger);
             if (lane == 0) red[w] = wmax;
             samples = WAVES;
             mth = limit;
+        } else if (limit <= 4 * WAVES) {
+            const T rmax = group_reduce(tmax, 16, larger);
+            if ((lane & 15) == 0) red[w * 4 + (lane >> 4)] = rmax;
+            samples = 4 * WAVES;
+            mth = limit;
         } else {
             const int stride = limit <= 512 ? (limit + 31) / 32 : (limit + 63) / 64;     // <= 16
-            tmax = wave_sort_descending(tmax);
-            const int p = (lane + 1) / stride;
-            if (p * stride == lane + 1 && p <= 4) red[w * 4 + p - 1] = tmax;
+            const T sorted = wave_sort_descending(tmax);
+#pragma unroll
+            for (int p = 1; p <= 4; ++p)
+                if (lane + 1 == p * stride) red[w * 4 + p - 1] = sorted;
             samples = 4 * WAVES;
             mth = (limit + stride - 1) / stride;                                       // <= 64
         }
         __syncthreads();
-        T bound = lane < samples ? red[lane] : worst;
-        if (limit <= WAVES) bound = wave_sort_descending<16>(bound);
-        else bound = wave_sort_descending(bound);
-        bound = lane_get(bound, mth - 1);
-        if (limit > BLOCK) bound = worst;
-        // ---- survivors go to LDS as (image, index), in element order: each wave counts its
-        // survivors with ballots, the waves' counts are prefix-summed through LDS, and a second
-        // sweep places every survivor at wave offset + number of survivors before it in the wave
-        uint32_t wave_count = 0;
-#pragma unroll
-        for (int i = 0; i < ITEMS; ++i) wave_count += static_cast<uint32_t>(__popcll(__ballot(sc[i] >= bound)));
-        if (lane == 0) sm.scan_tot[w] = wave_count;
-        __syncthreads();
-        uint32_t wave_base = 0, total = 0;
-        for (int i = 0; i < WAVES; ++i) {
-            const uint32_t t = sm.scan_tot[i];
-            if (i < w) wave_base += t;
-            total += t;
+        T bound;
+        if (samples == WAVES) {
+            // sixteen samples: every wave orders them itself (ten exchange steps)
+            bound = lane < WAVES ? red[lane] : worst;
+            bound = lane_get(wave_sort_descending<16>(bound), mth - 1);
+        } else {
+            // one wave orders the samples; the others wait (sixteen waves sorting the same
+            // samples would only compete for the issue slots of the row that shares this
+            // compute unit)
+            if (w == 0) {
+                T b = wave_sort_descending(red[lane]);
+                b = lane_get(b, mth - 1);
+                if (limit > BLOCK) b = worst;
+                if (lane == 0) red[4 * WAVES] = b;
+            }
+            __syncthreads();
+            bound = red[4 * WAVES];
         }
-        if (total <= CAP) {
-            const unsigned long long lt_mask = (1ull << lane) - 1ull;
+        DLFX_PHASE(1);            // bound
+        // ---- survivors go to LDS as (image, index).  A wave counts its survivors with one
+        // ballot per item, reserves that many slots with one atomic and places every survivor
+        // at the wave's base + the number of the wave's survivors before it; their order in
+        // LDS does not matter (they are ranked by image and index afterwards).  The ballots
+        // are kept in scalar registers for the second sweep while there are few enough.  What
+        // is stored is the score's bit pattern; its image is formed when the few survivors
+        // are read back.  A wave none of whose thread maxima reaches the bound has none.
+        constexpr uint32_t kCap = static_cast<uint32_t>(CAP);
+        constexpr bool kKeepMasks = ITEMS <= 32;
+        unsigned long long masks[kKeepMasks ? ITEMS : 1];
+        uint32_t wave_count = 0;
+        if (__ballot(tmax >= bound) != 0ull) {
 #pragma unroll
             for (int i = 0; i < ITEMS; ++i) {
-                const bool pass = sc[i] >= bound;
-                const unsigned long long m = __ballot(pass);
-                if (m != 0ull) {
-                    if (pass) {
-                        const uint32_t slot = wave_base + static_cast<uint32_t>(__popcll(m & lt_mask));
-                        sm.cand_ord[slot] = ord_of(sc[i]);
-                        sm.cand_idx[slot] = index_of(i);
+                const unsigned long long m = __ballot(sc[i] >= bound);
+                if constexpr (kKeepMasks) masks[i] = m;
+                wave_count += static_cast<uint32_t>(__popcll(m));
+            }
+        }
+        if (wave_count != 0u) {
+            uint32_t base = 0;
+            if (lane == 0) base = atomicAdd(&sm.count, wave_count);
+            base = lane_read(base, 0);
+            if (base + wave_count <= kCap) {
+                const unsigned long long lt_mask = (1ull << lane) - 1ull;
+#pragma unroll
+                for (int i = 0; i < ITEMS; ++i) {
+                    unsigned long long m;
+                    if constexpr (kKeepMasks) m = masks[i];
+                    else m = __ballot(sc[i] >= bound);
+                    if (m != 0ull) {
+                        if (sc[i] >= bound) {
+                            const uint32_t slot = base + static_cast<uint32_t>(__popcll(m & lt_mask));
+                            sm.cand_ord[slot] = bit_cast<K>(sc[i]);
+                            sm.cand_idx[slot] = index_of(i);
+                        }
+                        base += static_cast<uint32_t>(__popcll(m));
                     }
-                    wave_base += static_cast<uint32_t>(__popcll(m));
                 }
             }
         }
         __syncthreads();
+        const uint32_t total = sm.count;              // above the capacity: not all were stored
+        DLFX_PHASE(2);            // compaction
         // What happens next depends on how many survived:
-        //   * up to kMergeMax: ordered here by sorted runs and ranks, answer written;
+        //   * up to kMergeMax: ordered here by sorted runs and ranks, answer written (handing
+        //     them to a second kernel with small workgroups was measured: slower);
         //   * up to kCandCap: they are handed, through global memory, to topk_finish, whose
         //     small workgroups hide the latency of an exact radix selection much better than
         //     this one (which holds a whole row) could;
@@ -699,13 +775,15 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
         //     not hold for: topk_finish selects from the row itself.
         if (total <= static_cast<uint32_t>(kMergeMax) && limit <= BLOCK) {
             if (tid == 0) row_state[row] = kRowDone;
-            merge_rank_emit<BLOCK, K>(sm.cand_ord, sm.cand_idx, static_cast<int>(total), limit, io, row, xr);
+            merge_rank_emit<BLOCK, K>(sm.cand_ord, sm.cand_idx, static_cast<int>(total), limit, io, row, xr,
+                                      [&](K bits) { return ord_of(bit_cast<T>(bits)); });
+            DLFX_PHASE(3);        // ordering and output
         } else if (total <= CAP && limit <= BLOCK) {
             if (tid == 0) row_state[row] = total;
             K* so = spill_ord + row * CAP;
             uint32_t* si = spill_idx + row * CAP;
             for (uint32_t i = tid; i < total; i += BLOCK) {
-                so[i] = sm.cand_ord[i];
+                so[i] = ord_of(bit_cast<T>(sm.cand_ord[i]));
                 si[i] = sm.cand_idx[i];
             }
         } else {
@@ -714,8 +792,8 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
     }
 }
 
-// Second stage of the selection for rows topk_select did not finish: exact selection among the
-// row's spilled candidates, or over the whole row when it has to be.
+// Second stage of the selection for rows topk_select did not finish: exact selection among the row's
+// spilled candidates, or over the whole row when it has to be.
 template <typename E>
 __global__ __launch_bounds__(kSelectThreads) void topk_finish(
     TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> io, int64_t n, int limit, const uint32_t* __restrict__ row_state,
@@ -886,6 +964,22 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
 }  // namespace dlfx
 
 using namespace dlfx;
+
+#ifdef DLFX_TOPK_TIMING
+extern "C" void dlfx_debug_topk_phases(unsigned long long* out, int reset) {
+    static unsigned long long host[dlfx::kPhaseSlots * 8];
+    if (out) {
+        (void)hipMemcpyFromSymbol(host, HIP_SYMBOL(dlfx::g_topk_cycles), sizeof(host));
+        for (int i = 0; i < 8; ++i) out[i] = 0;
+        for (int b = 0; b < dlfx::kPhaseSlots; ++b)
+            for (int i = 0; i < 8; ++i) out[i] += host[b * 8 + i];
+    }
+    if (reset) {
+        std::memset(host, 0, sizeof(host));
+        (void)hipMemcpyToSymbol(HIP_SYMBOL(dlfx::g_topk_cycles), host, sizeof(host));
+    }
+}
+#endif
 
 extern "C" size_t dlfx_top_k_scratch_bytes(int dtype, int64_t m, int64_t n, int64_t limit) {
     const size_t es = dtype_size(dtype);
