@@ -259,8 +259,8 @@ __device__ __forceinline__ T wave_reduce(T v, Join join) {
     v = join(v, dpp_fetch<kQuadXor2>(v, v));
     v = join(v, dpp_fetch<kRowHalfMirror>(v, v));
     v = join(v, dpp_fetch<kRowMirror>(v, v));
-    v = join(v, lane_xor(v, 16));
-    v = join(v, lane_xor(v, 32));
+    v = join(v, lane_xor_const<16>(v));
+    v = join(v, lane_xor_const<32>(v));
     return v;
 }
 
@@ -272,8 +272,8 @@ __device__ __forceinline__ T group_reduce(T v, int width, Join join) {
     if (width > 2) v = join(v, dpp_fetch<kQuadXor2>(v, v));
     if (width > 4) v = join(v, dpp_fetch<kRowHalfMirror>(v, v));
     if (width > 8) v = join(v, dpp_fetch<kRowMirror>(v, v));
-    if (width > 16) v = join(v, lane_xor(v, 16));
-    if (width > 32) v = join(v, lane_xor(v, 32));
+    if (width > 16) v = join(v, lane_xor_const<16>(v));
+    if (width > 32) v = join(v, lane_xor_const<32>(v));
     return v;
 }
 
