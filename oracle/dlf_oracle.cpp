@@ -18,6 +18,12 @@
 //   argsort       dlf/include/tensor/reorder_detail.h:681-772 (serial leaves
 //                 and serial merge, which are stable)
 //   top_k (heap)  dlf/include/tensor/reorder_detail.h:969-1060
+//   count         dlf/include/tensor/reduce.h:151-158
+//   scan_nonzero, gather_indices   dlf/include/tensor/reduce.h:381-418
+//   merge         dlf/include/tensor/reorder_detail.h:346-368
+//   softmax, logsoftmax, hardmax   dlf/include/tensor/dnn_detail.h:266-350
+//   complex elements: the same reduce / scan / count templates instantiated with
+//                 std::complex<float|double> (functors dlf/include/tensor/xfn.h:73-170)
 //
 // Pinning status (what independent evidence fixes each function):
 //   reduce, arg_reduce, scan, sort, top_k values+indices on tie-free input:
@@ -28,6 +34,13 @@
 //       "lowest index first" (std::stable_sort); it is pinned against numpy's
 //       stable argsort, not against the reference.  parity unpinned w.r.t. the
 //       reference for tie order only.
+//   count, nonzero, merge, softmax family: literal vectors of the reference's tests
+//       (tests/golden/reference_vectors.json) and numpy / scipy closed forms.
+//   complex reduce / scan / count: the reference's literal nrm2 vector
+//       (dlf/test/UniformTest.cpp:2060-2063) and numpy complex128 closed forms; the
+//       reference holds no other complex vector for this path.
+//   16-bit elements never reach this file: the Python wrapper widens them exactly to the
+//       32-bit types (oracle.py), which numpy on the 16-bit arrays pins.
 //   fp32 sum/scan rounding: the reference's association depends on TBB's
 //       run-time range splitting; the restatement uses one valid schedule
 //       (recursive halving down to 1024-element leaves) and parity is judged
