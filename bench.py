@@ -536,6 +536,30 @@ def main():
         log("%-4s %-44s %10.1f us %9.1f GB/s %6.1f%%" % (op.config, op.name, med, gbs, 100 * gbs / HBM_PEAK_GBS))
     result["per_op"] = per_op
 
+    # ---- the launch-bound configuration recorded once and replayed as a HIP graph
+    c1 = [op for op in ops if op.config == "C1"]
+    if c1:
+        for op in c1:
+            op.calls[0]()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for op in c1:
+                op.calls[0]()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        reps = 50
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / reps
+        result["c1_graph"] = {"ops": len(c1), "us_per_replay": round(us, 2), "us_per_op": round(us / len(c1), 2)}
+        log("C1   %d ops replayed as one HIP graph: %.1f us per replay, %.1f us per op" % (len(c1), us, us / len(c1)))
+
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device=be.device).normal_()
         dst = torch.empty_like(src)
