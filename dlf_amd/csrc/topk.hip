@@ -677,6 +677,18 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
         T tmax = worst;
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) tmax = sc[i] > tmax ? sc[i] : tmax;
+        // NaNs compare false with everything, so the comparisons below would drop them, while
+        // the radix selection (and the sort) place them by their bit pattern, above +inf or
+        // below -inf.  A row that holds one is therefore selected by topk_finish from the row
+        // itself; the sum of a thread's scores is NaN exactly when one of them is, or when
+        // infinities of both signs meet, which only costs that row the slower path.
+        bool nan_seen = false;
+        if constexpr (!std::is_integral<T>::value) {
+            T sum = T(0);
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) sum += sc[i];
+            nan_seen = sum != sum;
+        }
         T* red = reinterpret_cast<T*>(sm.out_ord);
         if (tid == 0) sm.count = 0u;
         DLFX_PHASE(0);            // loads and thread maxima
@@ -740,6 +752,7 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
                 wave_count += static_cast<uint32_t>(__popcll(m));
             }
         }
+        if (__ballot(nan_seen) != 0ull) wave_count = kCap + 1u;       // more than fits: the row goes to topk_finish
         if (wave_count != 0u) {
             uint32_t base = 0;
             if (lane == 0) base = atomicAdd(&sm.count, wave_count);

@@ -106,3 +106,31 @@ def test_strided_views(hip_backend):
         Yh, Ih = F.top_k(X.slice(*args), 4, 0, False)
         Yo, Io = F.top_k(Xo.slice(*args), 4, 0, False)
         assert np.array_equal(Yh.numpy(), Yo.numpy()) and np.array_equal(Ih.numpy(), Io.numpy())
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.float16])
+@pytest.mark.parametrize("n,k", [(700, 5), (5000, 50), (32000, 5), (32000, 256), (40000, 17)])
+def test_top_k_with_nans_agrees_with_the_sort(hip_backend, dtype, n, k):
+    """The reference leaves the place of NaNs open (its comparisons are not an order on them).
+    Here they are ordered by their bit pattern everywhere - positive NaNs above +inf, negative
+    ones below -inf - so top_k must return the head of the stable argsort, bit for bit, whatever
+    path selects the row."""
+    if dtype == np.float64 and n > 32768:
+        pytest.skip("rows this long take the argsort path for 8-byte elements anyway")
+    x = (normal(190 + n + k, 4 * n) * 3).astype(dtype).reshape(4, n)
+    bits = {np.float32: np.uint32, np.float64: np.uint64, np.float16: np.uint16}[dtype]
+    pos_nan = np.array([np.nan], dtype=dtype)
+    neg_nan = (pos_nan.view(bits) | (bits(1) << bits(8 * dtype().itemsize - 1))).view(dtype)
+    x[0, [3, n // 2, n - 1]] = pos_nan[0]
+    x[1, [0, n // 3]] = neg_nan[0]
+    x[1, [5, n - 2]] = pos_nan[0]
+    x[2, n // 7] = np.inf
+    x[2, n // 5] = -np.inf                       # infinities of both signs, no NaN
+    X = Tensor.from_numpy(hip_backend, x)
+    for largest in (True, False):
+        Y, I = F.top_k(X, k, -1, largest)
+        SV, SI = F.argsort(X, -1, largest, with_values=True)
+        assert np.array_equal(I.numpy(), SI.numpy()[:, :k]), largest
+        assert np.array_equal(Y.numpy().view(bits), SV.numpy()[:, :k].view(bits)), largest
+    top = F.top_k(X, 3, -1, True)[0].numpy()
+    assert np.isnan(top[0]).all() and np.isnan(top[1][:2]).all() and top[2, 0] == np.inf
