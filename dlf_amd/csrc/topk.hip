@@ -119,6 +119,7 @@ struct TopkShared {
     uint32_t amb_count;
     K cand_ord[cand_cap<K>()];
     uint32_t cand_idx[cand_cap<K>()];
+    unsigned long long pack[sizeof(K) == 4 ? 512 : 1];      // sorted runs of (image, ~index) words, 4-byte keys
 };
 
 // Synchronises the TEAM threads that run a selection.  A single wave needs no hardware
@@ -297,6 +298,7 @@ __device__ __forceinline__ void wave_sort_entries(K& o, uint32_t& x) {
 }
 
 constexpr int kMergeMax = 512;       // entries up to which sorted runs are merged by rank
+static_assert(sizeof(TopkShared<uint32_t>::pack) == kMergeMax * 8, "room for kMergeMax packed entries");
 constexpr int kCountMax = 20;        // entries up to which ranks are counted directly
 
 // Orders `count` distinct (image, index) entries held in LDS, best first, and writes those
@@ -311,10 +313,14 @@ struct KeepImage {
 
 // `image_of` maps what e_ord holds to the image (the identity unless the caller stored
 // something cheaper to produce).
+// 4-byte images travel through the ranking as one 64-bit word (image, ~index) in `e_pack`
+// (room for kMergeMax words): an entry beats another exactly when its word is larger, one
+// LDS read and one comparison per probe.  8-byte images keep the two arrays.
 template <int BLOCK, typename K, typename S, typename ImageOf = KeepImage>
-__device__ __forceinline__ void merge_rank_emit(K* e_ord, uint32_t* e_idx, int count, int limit,
+__device__ __forceinline__ void merge_rank_emit(K* e_ord, uint32_t* e_idx, unsigned long long* e_pack, int count, int limit,
                                                 const TopkIo<K, S>& io, int64_t row, const S* xr,
                                                 ImageOf image_of = ImageOf()) {
+    constexpr bool PACKED = sizeof(K) == 4;
     constexpr int WAVES = BLOCK / kWave;
     const int tid = threadIdx.x;
     const int lane = lane_id();
@@ -340,6 +346,8 @@ __device__ __forceinline__ void merge_rank_emit(K* e_ord, uint32_t* e_idx, int c
         wave_sort_entries<K>(o, x);
         if (runs == 1) {
             if (lane < limit && lane < count) emit_one<K>(io, yr, ir, xr, lane, o, x);
+        } else if constexpr (PACKED) {
+            e_pack[e] = (static_cast<unsigned long long>(o) << 32) | static_cast<uint32_t>(~x);
         } else {
             e_ord[e] = o;
             e_idx[e] = x;
@@ -348,8 +356,17 @@ __device__ __forceinline__ void merge_rank_emit(K* e_ord, uint32_t* e_idx, int c
     if (runs == 1) return;
     team_sync<BLOCK>();
     for (int e = tid; e < count; e += BLOCK) {
-        const K o = e_ord[e];
-        const uint32_t x = e_idx[e];
+        K o;
+        uint32_t x;
+        unsigned long long mine_word = 0ull;
+        if constexpr (PACKED) {
+            mine_word = e_pack[e];
+            o = static_cast<K>(mine_word >> 32);
+            x = ~static_cast<uint32_t>(mine_word);
+        } else {
+            o = e_ord[e];
+            x = e_idx[e];
+        }
         const int mine = e / kWave;
         uint32_t rank = static_cast<uint32_t>(e % kWave);
         // U bisections at a time keep U independent LDS reads in flight; indices are only
@@ -365,6 +382,14 @@ __device__ __forceinline__ void merge_rank_emit(K* e_ord, uint32_t* e_idx, int c
                 c[u] = 0u;
             }
             auto probe = [&](int step) {      // step 0: the last probe, which decides 63 against 64
+                if constexpr (PACKED) {
+                    unsigned long long pj[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) pj[u] = e_pack[base[u] + static_cast<int>(c[u]) + (step ? step - 1 : 0)];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) c[u] += pj[u] > mine_word ? static_cast<uint32_t>(step ? step : 1) : 0u;
+                    return;
+                }
                 K oj[U];
                 uint32_t xj[U];
                 bool tie = false;
@@ -549,7 +574,7 @@ __device__ __forceinline__ void select_and_emit(TopkShared<K>& sm, const TopkIo<
 
     // ---- order the winners: best first
     if (limit <= kMergeMax) {
-        merge_rank_emit<BLOCK, K>(sm.out_ord, sm.out_idx, limit, limit, io, row, xr);
+        merge_rank_emit<BLOCK, K>(sm.out_ord, sm.out_idx, sm.pack, limit, limit, io, row, xr);
         return;
     }
     int kp = 1;
@@ -788,7 +813,7 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
         //     not hold for: topk_finish selects from the row itself.
         if (total <= static_cast<uint32_t>(kMergeMax) && limit <= BLOCK) {
             if (tid == 0) row_state[row] = kRowDone;
-            merge_rank_emit<BLOCK, K>(sm.cand_ord, sm.cand_idx, static_cast<int>(total), limit, io, row, xr,
+            merge_rank_emit<BLOCK, K>(sm.cand_ord, sm.cand_idx, sm.pack, static_cast<int>(total), limit, io, row, xr,
                                       [&](K bits) { return ord_of(bit_cast<T>(bits)); });
             DLFX_PHASE(3);        // ordering and output
         } else if (total <= CAP && limit <= BLOCK) {
@@ -833,7 +858,7 @@ __global__ __launch_bounds__(kSelectThreads) void topk_finish(
         }
         __syncthreads();
         if (total <= static_cast<uint32_t>(kMergeMax)) {
-            merge_rank_emit<SEL, K>(sm.cand_ord, sm.cand_idx, static_cast<int>(total), limit, io, row, xr);
+            merge_rank_emit<SEL, K>(sm.cand_ord, sm.cand_idx, sm.pack, static_cast<int>(total), limit, io, row, xr);
             return;
         }
         const int per_thread = static_cast<int>((total + SEL - 1) / SEL);
