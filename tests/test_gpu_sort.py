@@ -159,3 +159,25 @@ def test_rows_leave_out_passes_that_move_nothing(hip_backend, oracle_backend, dt
     Yh, Ih = F.argsort(Xh, -1, values=Xh)
     assert np.array_equal(Yh.numpy(), np.sort(x, axis=-1))
     assert np.array_equal(Ih.numpy(), np.argsort(x, axis=-1, kind="stable"))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.float16])
+def test_nans_take_the_place_of_their_bit_pattern(hip_backend, dtype):
+    """The reference's comparisons do not order NaNs (std::sort on them is undefined).  The radix
+    key places them by bit pattern: negative NaNs first, positive NaNs last, ascending."""
+    bits = {np.float32: np.uint32, np.float64: np.uint64, np.float16: np.uint16}[dtype]
+    pos = np.array([np.nan], dtype=dtype)
+    neg = (pos.view(bits) | (bits(1) << bits(8 * dtype().itemsize - 1))).view(dtype)
+    row = np.array([1.5, pos[0], -np.inf, neg[0], np.inf, -2.0, pos[0], 0.0], dtype=dtype)
+    x = np.tile(row, (3, 200))                      # rows of 1600 elements
+    X = Tensor.from_numpy(hip_backend, x)
+    asc = F.sort(X, -1).numpy()
+    assert np.signbit(asc[:, :200]).all() and np.isnan(asc[:, :200]).all()          # negative NaNs
+    assert np.isnan(asc[:, -400:]).all() and not np.signbit(asc[:, -400:]).any()    # positive NaNs
+    mid = asc[:, 200:-400]
+    assert not np.isnan(mid).any() and (mid[:, 1:] >= mid[:, :-1]).all()
+    desc = F.sort(X, -1, True).numpy()
+    assert np.array_equal(desc.view(bits), asc[:, ::-1].view(bits))
+    idx = F.argsort(X, -1).numpy()
+    assert np.array_equal(np.take_along_axis(x, idx, 1).view(bits), asc.view(bits))
+    assert (np.diff(idx[:, :200], axis=1) > 0).all()                                # equal keys keep their order
