@@ -565,6 +565,185 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
     DLFX_PHASE(5);
 }
 
+// ------------------------------------------------------------------ rows that fit one workgroup
+// A row of at most 256 * ITEMS keys is read once, sorted through all its passes in LDS and
+// registers and written once: no histogram pass, no scratch traffic, no chaining between
+// tiles.  The passes are those of sort_pass without the parts that connect tiles: rank inside
+// the wave with ballots over the digit bits that vary in the row, digit starts from the four
+// waves' counts, scatter through LDS, reload in element order.  Digits that are the same in
+// the whole row are skipped.  Element e of the row is item e / 64 % ITEMS of lane e % 64 of
+// wave e / (64 * ITEMS), before and after every pass.
+template <typename K, bool PAIRS, int ITEMS>
+struct SmallShared {
+    uint32_t wave_hist[4][kRadix];
+    uint32_t scan_tmp[4];
+    K wave_or[4], wave_and[4];
+    K keys[256 * ITEMS];
+    uint32_t vals[PAIRS ? 256 * ITEMS : 1];
+};
+
+template <typename K, bool PAIRS, int ITEMS>
+__global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t n) {
+    constexpr int P = KeyTraits<K>::kPasses;
+    constexpr int CAP = 256 * ITEMS;
+    static_assert(ITEMS % 2 == 0, "items are ranked in pairs");
+    __shared__ SmallShared<K, PAIRS, ITEMS> sm;
+    const int tid = threadIdx.x;
+    const int lane = lane_id();
+    const int w = tid / kWave;
+    const int64_t row = blockIdx.x;
+    const K* xrow = io.x + io.xmap.at(row);
+    const int valid = static_cast<int>(n);
+    const bool padded = valid < CAP;
+    const int seg = w * kWave * ITEMS + lane;
+
+    K key[ITEMS];
+    uint32_t val[PAIRS ? ITEMS : 1];
+    K ors = 0, ands = ~K(0);
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const int e = seg + k * kWave;
+        key[k] = ~K(0);                                   // padding sorts last in every pass that runs
+        if (e < valid) {
+            key[k] = key_of_element<K>(io, xrow[static_cast<int64_t>(e) * io.sx]);
+            ors |= key[k];
+            ands &= key[k];
+        }
+        if constexpr (PAIRS) val[k] = static_cast<uint32_t>(e);
+    }
+    ors = wave_reduce(ors, [](K a, K b) { return static_cast<K>(a | b); });
+    ands = wave_reduce(ands, [](K a, K b) { return static_cast<K>(a & b); });
+    if (lane == 0) {
+        sm.wave_or[w] = ors;
+        sm.wave_and[w] = ands;
+    }
+    __syncthreads();
+    const K differ = static_cast<K>((sm.wave_or[0] | sm.wave_or[1] | sm.wave_or[2] | sm.wave_or[3]) &
+                                    ~(sm.wave_and[0] & sm.wave_and[1] & sm.wave_and[2] & sm.wave_and[3]));
+
+    for (int pass = 0; pass < P; ++pass) {
+        const int shift = 8 * pass;
+        const uint32_t moves = static_cast<uint32_t>(differ >> shift) & 0xffu;
+        if (moves == 0u) continue;                        // this digit is the same in the whole row
+        const uint32_t vary = padded ? 0xffu : moves;     // padding differs from the row in other bits too
+        for (int i = tid; i < 4 * kRadix; i += 256) (&sm.wave_hist[0][0])[i] = 0;
+        __syncthreads();
+
+        // ---- rank inside the wave, in element order
+        uint32_t rank[ITEMS];
+#pragma unroll
+        for (int k0 = 0; k0 < ITEMS; k0 += 2) {
+            uint32_t d[2], before[2], cnt[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) d[j] = static_cast<uint32_t>(key[k0 + j] >> shift) & 0xffu;
+            uint32_t peers_lo[2] = {0xffffffffu, 0xffffffffu}, peers_hi[2] = {0xffffffffu, 0xffffffffu};
+            for (uint32_t bits = vary; bits != 0u; bits &= bits - 1u) {
+                const uint32_t b = static_cast<uint32_t>(__builtin_ctz(bits));
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int32_t ones = __builtin_amdgcn_sbfe(static_cast<int32_t>(d[j]), b, 1u);
+                    const unsigned long long vote = __ballot(ones < 0);
+                    peers_lo[j] &= ~(static_cast<uint32_t>(vote) ^ static_cast<uint32_t>(ones));
+                    peers_hi[j] &= ~(static_cast<uint32_t>(vote >> 32) ^ static_cast<uint32_t>(ones));
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                before[j] = __builtin_amdgcn_mbcnt_hi(peers_hi[j], __builtin_amdgcn_mbcnt_lo(peers_lo[j], 0u));
+                cnt[j] = static_cast<uint32_t>(__popc(peers_lo[j]) + __popc(peers_hi[j]));
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const uint32_t seen = sm.wave_hist[w][d[j]];
+                rank[k0 + j] = seen + before[j];
+                __builtin_amdgcn_wave_barrier();
+                if (before[j] == 0) sm.wave_hist[w][d[j]] = seen + cnt[j];
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+        __syncthreads();
+
+        // ---- thread d owns digit d: where the digit starts in the row, and each wave's share of it
+        {
+            uint32_t wave_count[4];
+            uint32_t count = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                wave_count[i] = sm.wave_hist[i][tid];
+                count += wave_count[i];
+            }
+            const uint32_t incl = wave_scan_inclusive(count, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+            if (lane == kWave - 1) sm.scan_tmp[w] = incl;
+            __syncthreads();
+            uint32_t run = incl - count;
+            for (int i = 0; i < w; ++i) run += sm.scan_tmp[i];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                sm.wave_hist[i][tid] = run;
+                run += wave_count[i];
+            }
+        }
+        __syncthreads();
+
+        // ---- scatter to the sorted position, reload in element order
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const uint32_t pos = sm.wave_hist[w][static_cast<uint32_t>(key[k] >> shift) & 0xffu] + rank[k];
+            sm.keys[pos] = key[k];
+            if constexpr (PAIRS) sm.vals[pos] = val[k];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            key[k] = sm.keys[seg + k * kWave];
+            if constexpr (PAIRS) val[k] = sm.vals[seg + k * kWave];
+        }
+        // (the three barriers of the next pass lie between these reads and its scatter)
+    }
+
+    // ---- write
+    if (io.y) {
+        K* yrow = io.y + io.ymap.at(row);
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const int e = seg + k * kWave;
+            if (e < valid) {
+                K bits = decode_key<K>(key[k], io.kind, io.descending);
+                if constexpr (PAIRS) {
+                    if (io.restore_zero && static_cast<K>(bits << 1) == 0) bits = xrow[static_cast<int64_t>(val[k]) * io.sx];
+                }
+                yrow[static_cast<int64_t>(e) * io.sy] = bits;
+            }
+        }
+    }
+    if constexpr (PAIRS) {
+        if (io.idx) {
+            const int64_t irow = io.imap.at(row);
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) {
+                const int e = seg + k * kWave;
+                if (e < valid) {
+                    if (io.idx64) static_cast<int64_t*>(io.idx)[irow + static_cast<int64_t>(e) * io.si] = static_cast<int64_t>(val[k]);
+                    else static_cast<int32_t*>(io.idx)[irow + static_cast<int64_t>(e) * io.si] = static_cast<int32_t>(val[k]);
+                }
+            }
+        }
+    }
+}
+
+constexpr int64_t kSmallRow = 4096;      // longest row sort_rows_small takes
+
+template <typename K, bool PAIRS>
+int launch_small(hipStream_t stream, const PassIo<K>& io, int64_t m, int64_t n) {
+    const dim3 grid(static_cast<unsigned>(m)), block(256);
+    if (n <= 512) sort_rows_small<K, PAIRS, 2><<<grid, block, 0, stream>>>(io, n);
+    else if (n <= 1024) sort_rows_small<K, PAIRS, 4><<<grid, block, 0, stream>>>(io, n);
+    else if (n <= 2048) sort_rows_small<K, PAIRS, 8><<<grid, block, 0, stream>>>(io, n);
+    else sort_rows_small<K, PAIRS, 16><<<grid, block, 0, stream>>>(io, n);
+    DLFX_CHECK_LAUNCH();
+    return DLFX_OK;
+}
+
 // ------------------------------------------------------------------ host side
 // Keys per thread: 16, or 8 for 64-bit keys that carry an index (LDS and registers then
 // still allow four workgroups per compute unit).
@@ -631,7 +810,6 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     if (n > kMaxRow) return DLFX_ERR_TOO_LARGE;
     const SortLayout l = sort_layout(sizeof(K), a.pairs, m, n);
     if (m * l.tiles_per_row > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
-    if (!scratch || scratch_bytes < l.total) return DLFX_ERR_SCRATCH_TOO_SMALL;
     char* base = static_cast<char*>(scratch);
 
     PassIo<K> io;
@@ -658,6 +836,17 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     const bool y_over_x = a.y && ranges_overlap<K>(a.rank, a.dims, static_cast<const K*>(a.x), a.xs, static_cast<const K*>(a.y), a.ys);
     io.canon_zero = (a.pairs && a.kind == kKeyFloat && !y_over_x) ? 1 : 0;
     io.restore_zero = (io.canon_zero && a.y) ? 1 : 0;
+
+    // short rows: one workgroup sorts a row on chip.  A workgroup reads its whole row before it
+    // writes, so sorting in place is fine; an output that overlaps the input in any other way
+    // (one row's output over another row's input) takes the general path.
+    bool same_view = a.y == a.x;
+    for (int i = 0; i < a.rank && same_view; ++i) same_view = a.xs[i] == a.ys[i] || a.dims[i] == 1;
+    if (n <= kSmallRow && (!y_over_x || same_view)) {
+        if (m > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+        return a.pairs ? launch_small<K, true>(stream, io, m, n) : launch_small<K, false>(stream, io, m, n);
+    }
+    if (!scratch || scratch_bytes < l.total) return DLFX_ERR_SCRATCH_TOO_SMALL;
 
     uint32_t* moves = reinterpret_cast<uint32_t*>(base + l.moves_off);
     uint32_t* ghist = reinterpret_cast<uint32_t*>(base + l.hist_off);

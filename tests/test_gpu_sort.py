@@ -181,3 +181,49 @@ def test_nans_take_the_place_of_their_bit_pattern(hip_backend, dtype):
     idx = F.argsort(X, -1).numpy()
     assert np.array_equal(np.take_along_axis(x, idx, 1).view(bits), asc.view(bits))
     assert (np.diff(idx[:, :200], axis=1) > 0).all()                                # equal keys keep their order
+
+
+@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 511, 512, 513, 1023, 1024, 1025, 2047, 2048, 2049, 4095, 4096, 4097])
+def test_rows_around_the_one_workgroup_limits(hip_backend, oracle_backend, n):
+    """Rows of up to 4096 elements are sorted by one workgroup on chip (512, 1024, 2048 or 4096
+    slots); longer rows take the tiled passes.  Every boundary, all key widths, both directions,
+    values, indices (32- and 64-bit) and in place."""
+    for dtype in (np.float32, np.int64, np.float64, np.int16, np.float16, np.int32):
+        x = (normal(200 + n, 5 * n) * 50).astype(dtype).reshape(5, n)
+        x[1] = x[1, 0]                                   # a constant row: no pass runs
+        x[2] = np.sort(x[2])[::-1]
+        if n > 4:
+            x[3, : n // 2] = x[3, n // 2: 2 * (n // 2)]  # every key twice: stability matters
+        Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
+        for desc in (False, True):
+            want = np.sort(x, axis=1, kind="stable")
+            want = want[:, ::-1] if desc else want
+            assert np.array_equal(F.sort(Xh, -1, desc).numpy(), want)
+            Y, I = F.argsort(Xh, -1, desc, with_values=True)
+            Yo, Io = F.argsort(Xo, -1, desc, with_values=True)
+            assert np.array_equal(I.numpy(), Io.numpy()) and np.array_equal(Y.numpy(), Yo.numpy())
+            I64 = F.argsort(Xh, -1, desc, index_dtype=np.int64)
+            assert I64.numpy().dtype == np.int64 and np.array_equal(I64.numpy(), Io.numpy())
+        Z = Tensor.from_numpy(hip_backend, x)
+        F.sort(Z, -1, False, out=Z)                      # in place
+        assert np.array_equal(Z.numpy(), np.sort(x, axis=1, kind="stable"))
+
+
+def test_short_rows_on_strided_views(hip_backend, oracle_backend):
+    a = (normal(201, 40 * 9 * 300) * 20).astype(np.float32).reshape(40, 9, 300)
+    T, O = Tensor.from_numpy(hip_backend, a), Tensor.from_numpy(oracle_backend, a)
+    for V, W, v in ((T.transpose(), O.transpose(), a.transpose()),
+                    (T.slice([0, 1, 3], [40, 9, 300], None, [3, 2, 7]), O.slice([0, 1, 3], [40, 9, 300], None, [3, 2, 7]), a[::3, 1::2, 3::7]),
+                    (T.flip([2]), O.flip([2]), a[:, :, ::-1])):
+        for axis in range(3):
+            assert np.array_equal(F.sort(V, axis).numpy(), np.sort(v, axis=axis, kind="stable"))
+            assert np.array_equal(F.argsort(V, axis, True).numpy(), F.argsort(W, axis, True).numpy())
+    # sorted into a strided output view
+    out = Tensor.from_numpy(hip_backend, np.zeros((300, 9, 40), dtype=np.float32))
+    F.sort(T, 2, False, out=out.transpose())
+    assert np.array_equal(out.numpy(), np.sort(a, axis=2).transpose())
+    # zeros of both signs in a short row: values keep their sign, equal keys keep their order
+    z = np.array([[0.0, -0.0, 1.0, -0.0, 0.0, -1.0]], dtype=np.float32)
+    Y, I = F.argsort(Tensor.from_numpy(hip_backend, z), -1, with_values=True)
+    assert I.numpy().tolist() == [[5, 0, 1, 3, 4, 2]]
+    assert np.array_equal(np.signbit(Y.numpy()), np.signbit(z[0][I.numpy()[0]])[None, :])
