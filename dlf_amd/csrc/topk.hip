@@ -616,6 +616,111 @@ template <> struct BitsOf<int64_t> { using type = uint64_t; using storage = uint
 template <> struct BitsOf<half_t>  { using type = uint32_t; using storage = uint16_t; using score = float;   static constexpr int kind = kKeyFloat; };
 template <> struct BitsOf<int16_t> { using type = uint32_t; using storage = uint16_t; using score = int32_t; static constexpr int kind = kKeyInt; };
 
+// Short rows and small limits: one wavefront per row, four rows per workgroup, no workgroup
+// barrier.  A row of at most 64 * ITEMS elements lives in the wave's registers as images.  The
+// limit-th largest of the 64 lane maxima (distinct elements of the row) has at least `limit`
+// elements at or above it; what reaches it - usually a few more than `limit` entries - is
+// gathered through a 64-entry LDS buffer of the wave and ordered by one wave sort (or by
+// counting, when there is only a handful).  When more than 64 elements reach the bound (long
+// runs of equal values), the wave takes the `limit` best one after the other instead: exact
+// for any input, and only slow where it is needed.
+constexpr int kWaveRowMax = 4096;       // longest row topk_rows_wave takes
+constexpr int kWaveRowLimit = 64;       // largest limit
+
+template <typename E, int ITEMS>
+__global__ __launch_bounds__(256) void topk_rows_wave(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> io,
+                                                      int64_t rows, int64_t n, int limit) {
+    using K = typename BitsOf<E>::type;
+    using S = typename BitsOf<E>::storage;
+    constexpr int kind = BitsOf<E>::kind;
+    __shared__ K cand_ord[4][kWave];
+    __shared__ uint32_t cand_idx[4][kWave];
+    const int lane = lane_id();
+    const int w = threadIdx.x / kWave;
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + w;
+    if (row >= rows) return;                               // whole waves leave; nothing below synchronises the workgroup
+    const S* xr = io.x + io.xmap.at(row);
+    S* yr = io.y + io.ymap.at(row);
+    const int64_t ir = io.imap.at(row);
+    const uint32_t n32 = static_cast<uint32_t>(n);
+    const K flip = io.largest ? K(0) : (kind == kKeyFloat ? KeyBits<K>::kSign : ~K(0));
+
+    // element i * 64 + lane is item i of the lane; padding carries image 0 and an index past the row
+    K ord[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        const uint32_t e = static_cast<uint32_t>(i * kWave + lane);
+        ord[i] = e < n32 ? to_ord<K>(static_cast<K>(widen_bits<K, S>(xr[static_cast<int64_t>(e) * io.sx], kind) ^ flip), kind, 1) : K(0);
+    }
+    K best = 0;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) best = ord[i] > best ? ord[i] : best;
+    const K bound = lane_get(wave_sort_descending(best), limit - 1);
+    uint32_t count = 0;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) count += static_cast<uint32_t>(__popcll(__ballot(ord[i] >= bound)));
+
+    if (count <= static_cast<uint32_t>(kWave)) {
+        const unsigned long long lt_mask = (1ull << lane) - 1ull;
+        uint32_t base = 0;
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const bool pass = ord[i] >= bound;
+            const unsigned long long m = __ballot(pass);
+            if (m != 0ull) {
+                if (pass) {
+                    const uint32_t slot = base + static_cast<uint32_t>(__popcll(m & lt_mask));
+                    cand_ord[w][slot] = ord[i];
+                    cand_idx[w][slot] = static_cast<uint32_t>(i * kWave + lane);
+                }
+                base += static_cast<uint32_t>(__popcll(m));
+            }
+        }
+        team_sync<kWave>();
+        const bool live = static_cast<uint32_t>(lane) < count;
+        K o = live ? cand_ord[w][lane] : K(0);
+        uint32_t x = live ? cand_idx[w][lane] : 0xffffffffu;
+        uint32_t rank;
+        if (count <= static_cast<uint32_t>(kCountMax)) {
+            rank = 0;
+            for (uint32_t j = 0; j < count; ++j) rank += beats<K>(lane_read(o, static_cast<int>(j)), lane_read(x, static_cast<int>(j)), o, x);
+        } else {
+            wave_sort_entries<K>(o, x);
+            rank = static_cast<uint32_t>(lane);
+        }
+        if (live && rank < static_cast<uint32_t>(limit)) emit_one<K>(io, yr, ir, xr, static_cast<int>(rank), o, x);
+        return;
+    }
+
+    // more than a wave's worth of entries reach the bound: take the best entry that comes
+    // after the one taken last, `limit` times (entries are ordered by image, then by lower index)
+    K last_o = ~K(0);
+    uint32_t last_x = 0;
+    bool first = true;
+    for (int j = 0; j < limit; ++j) {
+        K bo = 0;
+        uint32_t bx = 0xffffffffu;
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const uint32_t e = static_cast<uint32_t>(i * kWave + lane);
+            const bool after = first || beats<K>(last_o, last_x, ord[i], e) != 0u;      // not taken yet
+            if (e < n32 && after && beats<K>(ord[i], e, bo, bx) != 0u) {
+                bo = ord[i];
+                bx = e;
+            }
+        }
+        struct Entry {
+            K o;
+            uint32_t x;
+        };
+        const Entry top = wave_reduce(Entry{bo, bx}, [](Entry a, Entry b) { return beats<K>(b.o, b.x, a.o, a.x) ? b : a; });
+        if (lane == 0) emit_one<K>(io, yr, ir, xr, j, top.o, top.x);
+        last_o = top.o;
+        last_x = top.x;
+        first = false;
+    }
+}
+
 // E: the element type.  ALIGNED: the axis is contiguous and every row starts on a 16-byte
 // boundary (checked on the host), so rows are read with 128-bit loads off one base register.
 //
@@ -954,6 +1059,20 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
         uint32_t* row_state = reinterpret_cast<uint32_t*>(sbase + sl.state_off);
         K* spill_ord = reinterpret_cast<K*>(sbase + sl.ord_off);
         uint32_t* spill_idx = reinterpret_cast<uint32_t*>(sbase + sl.idx_off);
+        if (n <= kWaveRowMax && lim <= kWaveRowLimit) {
+            const dim3 wgrid(static_cast<unsigned>(ceil_div(m, 4)));
+#define DLFX_TOPK_WAVE(ITEMS) topk_rows_wave<T, ITEMS><<<wgrid, dim3(256), 0, stream>>>(io, m, n, lim)
+            if (n <= 64) DLFX_TOPK_WAVE(1);
+            else if (n <= 128) DLFX_TOPK_WAVE(2);
+            else if (n <= 256) DLFX_TOPK_WAVE(4);
+            else if (n <= 512) DLFX_TOPK_WAVE(8);
+            else if (n <= 1024) DLFX_TOPK_WAVE(16);
+            else if (n <= 2048) DLFX_TOPK_WAVE(32);
+            else DLFX_TOPK_WAVE(64);
+#undef DLFX_TOPK_WAVE
+            DLFX_CHECK_LAUNCH();
+            return DLFX_OK;
+        }
 #define DLFX_TOPK(BLOCK, ITEMS)                                                                     \
     do {                                                                                            \
         if (aligned) topk_select<T, BLOCK, ITEMS, true><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx); \

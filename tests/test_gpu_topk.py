@@ -134,3 +134,33 @@ def test_top_k_with_nans_agrees_with_the_sort(hip_backend, dtype, n, k):
         assert np.array_equal(Y.numpy().view(bits), SV.numpy()[:, :k].view(bits)), largest
     top = F.top_k(X, 3, -1, True)[0].numpy()
     assert np.isnan(top[0]).all() and np.isnan(top[1][:2]).all() and top[2, 0] == np.inf
+
+
+@pytest.mark.parametrize("n", [1, 5, 63, 64, 65, 128, 129, 1000, 1024, 2048, 2049, 4096])
+def test_short_rows_one_wave_per_row(hip_backend, oracle_backend, n):
+    """Rows of up to 4096 elements with limits up to 64 are selected by one wavefront each.
+    Every size class, limits up to the cap, both directions, all element types, and the rows
+    that defeat the bound (all equal, few distinct values, sorted either way)."""
+    for dtype in (np.float32, np.int32, np.float64, np.int64, np.float16, np.int16):
+        x = (normal(210 + n, 7 * n) * 40).astype(dtype).reshape(7, n)
+        x[1] = 3                                               # all equal: every element reaches the bound
+        x[2] = randint(211 + n, n, 0, 3).astype(dtype)         # three distinct values
+        x[3] = np.sort(x[3])
+        x[4] = np.sort(x[4])[::-1]
+        Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
+        for k in sorted({1, min(n, 5), min(n, 21), min(n, 64)}):
+            for largest in (True, False):
+                Yh, Ih = F.top_k(Xh, k, -1, largest)
+                Yo, Io = F.top_k(Xo, k, -1, largest)
+                assert np.array_equal(Ih.numpy(), Io.numpy()), (dtype, k, largest)
+                assert np.array_equal(Yh.numpy().view(np.uint8), Yo.numpy().view(np.uint8))
+    # 64-bit indices and a strided view
+    a = (normal(212, 33 * 5 * max(n, 2)) * 9).astype(np.float32).reshape(33, 5, max(n, 2))
+    T, O = Tensor.from_numpy(hip_backend, a), Tensor.from_numpy(oracle_backend, a)
+    k = min(3, a.shape[2])
+    Yh, Ih = F.top_k(T.flip([2]), k, 2, True, index_dtype=np.int64)
+    Yo, Io = F.top_k(O.flip([2]), k, 2, True)
+    assert Ih.numpy().dtype == np.int64 and np.array_equal(Ih.numpy(), Io.numpy()) and np.array_equal(Yh.numpy(), Yo.numpy())
+    Yh, Ih = F.top_k(T, min(4, a.shape[0]), 0, False)
+    Yo, Io = F.top_k(O, min(4, a.shape[0]), 0, False)
+    assert np.array_equal(Ih.numpy(), Io.numpy()) and np.array_equal(Yh.numpy(), Yo.numpy())
