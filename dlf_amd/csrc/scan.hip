@@ -360,6 +360,90 @@ __global__ __launch_bounds__(kBlock) void scan_rows_single(
     scan_tile<T, K, ITEMS, false, false, kBlock, X, NZ, Y>(x, y, xmap, ymap, sx, sy, xaxis, n, 1, exclusive, blockIdx.x, 0, 0, st, sm);
 }
 
+// Short rows: LANES lanes per row (a DPP row of 16 lanes, or a whole wavefront), ITEMS elements
+// per lane in vectors of V, no workgroup barrier and no LDS; a 256-thread workgroup takes
+// 256 / LANES rows.  Element (v * LANES + l) * V + j is item (v, j) of lane l of the group.
+template <typename T, int K, int LANES, int ITEMS, typename X, bool NZ, typename Y>
+__global__ __launch_bounds__(kBlock) void scan_rows_group(
+    const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
+    int64_t rows, int64_t n, int exclusive) {
+    static_assert(LANES == 16 || LANES == kWave, "a DPP row or a wavefront");
+    using Op = ScanOp<T, K>;
+    constexpr int V = (vec_width<T>() < ITEMS) ? vec_width<T>() : ITEMS;
+    constexpr int KV = ITEMS / V;
+    using VecX = Vec<X, V>;
+    using VecY = Vec<Y, V>;
+    const int lane = lane_id();
+    const int l = lane & (LANES - 1);
+    const int64_t row = (static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x) / LANES;
+    const bool live = row < rows;                       // whole groups are live or not
+    const X* xr = x + (live ? xmap.at(row) : 0);
+    Y* yr = y + (live ? ymap.at(row) : 0);
+    const int64_t count = live ? n : 0;
+
+    // whole vectors of an aligned unit-stride row move as one access, the row's last, partial
+    // vector element by element
+    const bool x_vec = sx == 1 && reinterpret_cast<uintptr_t>(xr) % (sizeof(X) * V) == 0;
+    const bool y_vec = sy == 1 && reinterpret_cast<uintptr_t>(yr) % (sizeof(Y) * V) == 0;
+    T vals[ITEMS];
+#pragma unroll
+    for (int v = 0; v < KV; ++v) {
+        const int64_t e0 = static_cast<int64_t>(v * LANES + l) * V;
+        if (x_vec && e0 + V <= count) {
+            const VecX a = load_stream(reinterpret_cast<const VecX*>(xr + e0));
+#pragma unroll
+            for (int j = 0; j < V; ++j) vals[v * V + j] = scan_input<T, X, NZ>(a.v[j]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < V; ++j) vals[v * V + j] = (e0 + j < count) ? scan_input<T, X, NZ>(xr[(e0 + j) * sx]) : Op::identity();
+        }
+    }
+    auto combine = [](T a, T b) { return Op::apply(a, b); };
+    T carry = Op::identity();
+#pragma unroll
+    for (int v = 0; v < KV; ++v) {
+#pragma unroll
+        for (int j = 1; j < V; ++j) vals[v * V + j] = Op::apply(vals[v * V + j - 1], vals[v * V + j]);
+        const T lane_total = vals[v * V + V - 1];
+        T incl;
+        if constexpr (LANES == 16) {
+            incl = combine(dpp_fetch<kRowShr1>(lane_total, Op::identity()), lane_total);
+            incl = combine(dpp_fetch<kRowShr2>(incl, Op::identity()), incl);
+            incl = combine(dpp_fetch<kRowShr4>(incl, Op::identity()), incl);
+            incl = combine(dpp_fetch<kRowShr8>(incl, Op::identity()), incl);
+        } else {
+            incl = wave_scan_inclusive(lane_total, Op::identity(), combine);
+        }
+        T before = lane_get(incl, lane - 1 < 0 ? 0 : lane - 1);     // the lanes before this one in the group
+        if (l == 0) before = Op::identity();
+        const T base = Op::apply(carry, before);
+        const T group_total = lane_get(incl, lane | (LANES - 1));
+        if (exclusive) {
+#pragma unroll
+            for (int j = V - 1; j > 0; --j) vals[v * V + j] = Op::apply(base, vals[v * V + j - 1]);
+            vals[v * V] = base;
+        } else {
+#pragma unroll
+            for (int j = 0; j < V; ++j) vals[v * V + j] = Op::apply(base, vals[v * V + j]);
+        }
+        carry = Op::apply(carry, group_total);
+    }
+#pragma unroll
+    for (int v = 0; v < KV; ++v) {
+        const int64_t e0 = static_cast<int64_t>(v * LANES + l) * V;
+        if (y_vec && e0 + V <= count) {
+            VecY a;
+#pragma unroll
+            for (int j = 0; j < V; ++j) a.v[j] = static_cast<Y>(vals[v * V + j]);
+            store_stream(reinterpret_cast<VecY*>(yr + e0), a);
+        } else {
+#pragma unroll
+            for (int j = 0; j < V; ++j)
+                if (e0 + j < count) yr[(e0 + j) * sy] = static_cast<Y>(vals[v * V + j]);
+        }
+    }
+}
+
 // Rows of several tiles.  Workgroup b belongs to row b / tiles_per_row.  With
 // TICKET the tile of the row is drawn from that row's atomic counter (in-place
 // scans); without, it is the workgroup's position in the row and waits are
@@ -552,6 +636,23 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     const bool axis_unit = (sx == 1 || sx == -1 || n == 1) && (sy == 1 || sy == -1 || n == 1);
     const bool inner_unit = xmap.rank >= 1 && xmap.strides[xmap.rank - 1] == 1 && ymap.strides[ymap.rank - 1] == 1 &&
                             xmap.dims[xmap.rank - 1] >= 16;
+    // Short rows along a unit-stride axis: a group of lanes per row (rows of up to 512 elements;
+    // a workgroup per row would leave most of its threads, or of the chip, idle).
+    if (!axis_general && axis_unit && n <= 512 && m >= 4) {
+        const int64_t lanes = n <= 64 ? 16 : kWave;
+        const int64_t blocks = ceil_div(m * lanes, kBlock);
+        if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+        const dim3 grid(static_cast<unsigned>(blocks)), block(kBlock);
+#define DLFX_SCAN_GROUP(LANES, ITEMS) \
+    scan_rows_group<T, K, LANES, ITEMS, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, m, n, exclusive)
+        if (n <= 16) DLFX_SCAN_GROUP(16, 1);
+        else if (n <= 64) DLFX_SCAN_GROUP(16, 4);
+        else if (n <= 256) DLFX_SCAN_GROUP(kWave, 4);
+        else DLFX_SCAN_GROUP(kWave, 8);
+#undef DLFX_SCAN_GROUP
+        DLFX_CHECK_LAUNCH();
+        return DLFX_OK;
+    }
     const bool short_rows = n <= 64 && m >= 256;
     const bool use_cols = !axis_general && (short_rows || (!axis_unit && m >= 64 && (inner_unit || n < 4096)));
     if (use_cols) {

@@ -147,3 +147,44 @@ def test_in_place_long_rows_use_tickets(hip_backend, oracle_backend):
     assert np.array_equal(Xh.numpy(), F.cumsum(Xo, 1, True, True).numpy())
     F.cumsum(Xo, 1, True, True, out=Xo)
     assert not np.array_equal(Xo.numpy(), Xh.numpy())     # the restated reference loop reproduces the slip
+
+
+@pytest.mark.parametrize("n", [1, 2, 15, 16, 17, 63, 64, 65, 255, 256, 257, 511, 512, 513])
+def test_short_rows_one_lane_group_per_row(hip_backend, oracle_backend, n):
+    """Rows of up to 512 elements along a unit-stride axis are scanned by a group of 16 or 64
+    lanes each.  Every size class; all four scans; exclusive and reversed; integer results are
+    exact, floating ones within the usual bound of the fp64 evaluation."""
+    m = 37
+    xi = randint(220 + n, m * n, -9, 10).astype(np.int32).reshape(m, n)
+    Xi = Tensor.from_numpy(hip_backend, xi)
+    for exclusive in (False, True):
+        for reverse in (False, True):
+            src = xi[:, ::-1] if reverse else xi
+            want = np.cumsum(src, axis=1, dtype=np.int32)
+            if exclusive:
+                want = np.concatenate([np.zeros((m, 1), np.int32), want[:, :-1]], axis=1)
+            want = want[:, ::-1] if reverse else want
+            assert np.array_equal(F.cumsum(Xi, 1, exclusive, reverse).numpy(), want), (exclusive, reverse)
+    assert np.array_equal(F.cummax(Xi, 1).numpy(), np.maximum.accumulate(xi, axis=1))
+    assert np.array_equal(F.cummin(Xi, 1, True).numpy(), np.minimum.accumulate(xi[:, ::-1], axis=1)[:, ::-1])
+    small = randint(221 + n, m * n, 1, 3).astype(np.int64).reshape(m, n)
+    assert np.array_equal(F.cumprod(Tensor.from_numpy(hip_backend, small), 1).numpy(), np.cumprod(small, axis=1))   # wraps like numpy
+    for dtype in (np.float32, np.float64, np.float16):
+        xf = (normal(222 + n, m * n) * 0.5).astype(dtype).reshape(m, n)
+        got = F.cumsum(Tensor.from_numpy(hip_backend, xf), 1).numpy().astype(np.float64)
+        x64 = xf.astype(np.float64)
+        want, mag = np.cumsum(x64, axis=1), np.cumsum(np.abs(x64), axis=1)
+        eps = np.finfo(np.float32 if dtype == np.float16 else dtype).eps
+        out_ulp = 2.0 ** -10 if dtype == np.float16 else 0.0
+        assert (np.abs(got - want) <= 4 * max(1.0, np.log2(n)) * eps * mag + out_ulp * np.abs(want) + 1e-30).all(), dtype
+    xc = ((normal(223 + n, m * n) + 1j * normal(224 + n, m * n)) * 0.5).astype(np.complex64).reshape(m, n)
+    assert np.allclose(F.cumsum(Tensor.from_numpy(hip_backend, xc), 1, True).numpy()[:, 1:], np.cumsum(xc.astype(np.complex128), axis=1)[:, :-1], rtol=1e-5, atol=1e-5)
+    # in place, and rows that are not 16-byte aligned (a sliced view)
+    Z = Tensor.from_numpy(hip_backend, xi)
+    F.cumsum(Z, 1, out=Z)
+    assert np.array_equal(Z.numpy(), np.cumsum(xi, axis=1, dtype=np.int32))
+    if n > 3:
+        V = Xi.slice([1], [n], [1])
+        assert np.array_equal(F.cumsum(V, 1).numpy(), np.cumsum(xi[:, 1:], axis=1, dtype=np.int32))
+    # the same rows as columns of the transposed view: the axis is no longer unit-stride
+    assert np.array_equal(F.cumsum(Xi.transpose(), 0).numpy(), np.cumsum(xi, axis=1, dtype=np.int32).T)
