@@ -59,7 +59,8 @@ __device__ __forceinline__ MaxAt<T> max_at_join(MaxAt<T> a, MaxAt<T> b) {
 // LDS); every thread receives the result.  `slot` separates the teams of a workgroup.
 template <int TEAM, typename V, typename Join>
 __device__ __forceinline__ V team_reduce(V v, Join join, V* lds) {
-    v = wave_reduce(v, join);
+    if constexpr (TEAM < kWave) v = group_reduce(v, TEAM, join);      // a DPP row of 16 lanes
+    else v = wave_reduce(v, join);
     if constexpr (TEAM > kWave) {
         constexpr int WAVES = TEAM / kWave;
         const int w = threadIdx.x / kWave;
@@ -237,9 +238,20 @@ int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y) {
         return DLFX_OK;                                                                                         \
     } while (0)
     if (ceil_div(m, 4) > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+    if (n <= 16 * V) {
+        // very short rows: sixteen lanes per row, sixteen rows per workgroup
+        const dim3 grid(static_cast<unsigned>(ceil_div(m, 16)));
+        if (vec) softmax_rows<T, 16, V, KIND, true><<<grid, dim3(256), 0, stream>>>(x, y, m, n);
+        else softmax_rows<T, 16, V, KIND, false><<<grid, dim3(256), 0, stream>>>(x, y, m, n);
+        DLFX_CHECK_LAUNCH();
+        return DLFX_OK;
+    }
     if (n <= kWave * V) DLFX_WAVE_ROWS(V);
     if (n <= kWave * 4 * V) DLFX_WAVE_ROWS(4 * V);
     if (n <= kWave * 32) DLFX_WAVE_ROWS(32);
+    if constexpr (V <= 4) {
+        if (n <= 1024 * 4) DLFX_BLOCK_ROWS(4);
+    }
     if (n <= 1024 * 8) DLFX_BLOCK_ROWS(8);
     if (n <= 1024 * 16) DLFX_BLOCK_ROWS(16);
     if (n <= 1024 * 32 && kRegisterBytes == 4) DLFX_BLOCK_ROWS(32);

@@ -93,3 +93,27 @@ def test_hardmax_of_integer_rows(hip_backend, oracle_backend, dtype, n):
     assert np.array_equal(got, want)
     with pytest.raises(Exception):
         F.softmax(Tensor.from_numpy(hip_backend, x), 1)
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 15, 16, 17, 31, 32, 33, 63, 64, 65, 4095, 4096, 4097])
+def test_row_lengths_around_the_team_sizes(hip_backend, oracle_backend, n):
+    """Sixteen lanes per row up to 64 (fp32) / 32 (fp64) / 128 (half) elements, a wavefront up to
+    2048, a workgroup of 1024 threads with 4 elements each up to 4096: the boundaries of each."""
+    m = 70 if n < 1000 else 9
+    for dtype in (np.float32, np.float64, np.float16):
+        x = (normal(230 + n, m * n) * 2).astype(dtype).reshape(m, n)
+        x[1] = x[1, 0]                                   # a constant row
+        if n > 2:
+            x[2, n // 2] = np.nan                        # a NaN that is not in position 0 is skipped
+        Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
+        x64 = np.delete(x, 2, axis=0).astype(np.float64) if n > 2 else x.astype(np.float64)
+        keep = [r for r in range(m) if not (n > 2 and r == 2)]
+        eps = np.finfo(np.float32 if dtype == np.float16 else dtype).eps
+        out_ulp = 2.0 ** -10 if dtype == np.float16 else 0.0
+        slack = 8 * max(1.0, np.log2(n)) * eps + out_ulp
+        got = F.softmax(Xh).numpy().astype(np.float64)[keep]
+        assert (np.abs(got - sp_softmax(x64, axis=1)) <= sp_softmax(x64, axis=1) * slack + 1e-30 + (2.0 ** -24 if dtype == np.float16 else 0)).all(), dtype
+        got = F.logsoftmax(Xh).numpy().astype(np.float64)[keep]
+        want = sp_log_softmax(x64, axis=1)
+        assert (np.abs(got - want) <= slack * (1 + np.abs(want)) + out_ulp * np.abs(want)).all(), dtype
+        assert np.array_equal(F.hardmax(Xh).numpy(), F.hardmax(Xo).numpy()), dtype
