@@ -731,12 +731,57 @@ __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t n) 
     }
 }
 
+// Rows of at most 64 elements: one wavefront per row, one element per lane, a bitonic network
+// over (key, index) pairs - a total order, so the result is the stable one.  Four rows per
+// workgroup, no LDS, no barrier.
+template <typename K, bool PAIRS>
+__global__ __launch_bounds__(256) void sort_rows_wave(PassIo<K> io, int64_t rows, int64_t n) {
+    const int lane = lane_id();
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+    if (row >= rows) return;
+    const K* xrow = io.x + io.xmap.at(row);
+    const bool live = lane < n;
+    K key = live ? key_of_element<K>(io, xrow[static_cast<int64_t>(lane) * io.sx]) : ~K(0);   // padding sorts last
+    uint32_t idx = static_cast<uint32_t>(lane);
+    wave_bitonic<kWave>([&](auto jc, bool keep_first) {
+        constexpr int J = decltype(jc)::value;
+        const K other_key = lane_xor_const<J>(key);
+        bool other_first = other_key < key;
+        if constexpr (PAIRS) {
+            const uint32_t other_idx = lane_xor_const<J>(idx);
+            other_first = other_first || (other_key == key && other_idx < idx);
+            if (keep_first == other_first) {
+                key = other_key;
+                idx = other_idx;
+            }
+        } else {
+            if (keep_first == other_first) key = other_key;
+        }
+    });
+    if (!live) return;                                     // the first n lanes hold the row in order
+    if (io.y) {
+        K bits = decode_key<K>(key, io.kind, io.descending);
+        if constexpr (PAIRS) {
+            if (io.restore_zero && static_cast<K>(bits << 1) == 0) bits = xrow[static_cast<int64_t>(idx) * io.sx];
+        }
+        io.y[io.ymap.at(row) + static_cast<int64_t>(lane) * io.sy] = bits;
+    }
+    if constexpr (PAIRS) {
+        if (io.idx) {
+            const int64_t at = io.imap.at(row) + static_cast<int64_t>(lane) * io.si;
+            if (io.idx64) static_cast<int64_t*>(io.idx)[at] = static_cast<int64_t>(idx);
+            else static_cast<int32_t*>(io.idx)[at] = static_cast<int32_t>(idx);
+        }
+    }
+}
+
 constexpr int64_t kSmallRow = 4096;      // longest row sort_rows_small takes
 
 template <typename K, bool PAIRS>
 int launch_small(hipStream_t stream, const PassIo<K>& io, int64_t m, int64_t n) {
     const dim3 grid(static_cast<unsigned>(m)), block(256);
-    if (n <= 512) sort_rows_small<K, PAIRS, 2><<<grid, block, 0, stream>>>(io, n);
+    if (n <= kWave) sort_rows_wave<K, PAIRS><<<dim3(static_cast<unsigned>(ceil_div(m, 4))), block, 0, stream>>>(io, m, n);
+    else if (n <= 512) sort_rows_small<K, PAIRS, 2><<<grid, block, 0, stream>>>(io, n);
     else if (n <= 1024) sort_rows_small<K, PAIRS, 4><<<grid, block, 0, stream>>>(io, n);
     else if (n <= 2048) sort_rows_small<K, PAIRS, 8><<<grid, block, 0, stream>>>(io, n);
     else sort_rows_small<K, PAIRS, 16><<<grid, block, 0, stream>>>(io, n);
