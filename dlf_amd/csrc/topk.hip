@@ -625,7 +625,7 @@ template <> struct BitsOf<int16_t> { using type = uint32_t; using storage = uint
 // runs of equal values), the wave takes the `limit` best one after the other instead: exact
 // for any input, and only slow where it is needed.
 constexpr int kWaveRowMax = 4096;       // longest row topk_rows_wave takes
-constexpr int kWaveRowLimit = 64;       // largest limit
+constexpr int kWaveRowLimit = 16;       // largest limit (the limit-th of 64 lane maxima is a weak bound beyond)
 
 template <typename E, int ITEMS>
 __global__ __launch_bounds__(256) void topk_rows_wave(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> io,
@@ -1059,7 +1059,7 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
         uint32_t* row_state = reinterpret_cast<uint32_t*>(sbase + sl.state_off);
         K* spill_ord = reinterpret_cast<K*>(sbase + sl.ord_off);
         uint32_t* spill_idx = reinterpret_cast<uint32_t*>(sbase + sl.idx_off);
-        if (n <= kWaveRowMax && lim <= kWaveRowLimit) {
+        if (n <= kWaveRowMax && (lim <= kWaveRowLimit || n <= kWave)) {      // at most 64 elements: one wave sort, whatever the limit
             const dim3 wgrid(static_cast<unsigned>(ceil_div(m, 4)));
 #define DLFX_TOPK_WAVE(ITEMS) topk_rows_wave<T, ITEMS><<<wgrid, dim3(256), 0, stream>>>(io, m, n, lim)
             if (n <= 64) DLFX_TOPK_WAVE(1);

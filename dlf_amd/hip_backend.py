@@ -176,6 +176,12 @@ class HipBackend:
     def download(self, storage) -> np.ndarray:
         return storage.cpu().numpy()
 
+    def copy_view(self, storage, shape):
+        """Row-major device copy of a strided view with non-negative strides (a layout copy, done
+        by torch: it is not one of the axis primitives)."""
+        view = self.torch.as_strided(storage, list(shape.extents), list(shape.strides), shape.offset)
+        return view.clone(memory_format=self.torch.contiguous_format).view(-1)
+
     def wrap(self, tensor):
         """Use an existing contiguous 1-D device tensor as storage."""
         return tensor

@@ -95,3 +95,21 @@ def test_half_scans_and_softmax_on_views(hip_backend):
             assert np.array_equal(F.cummax(V, axis).numpy(), np.maximum.accumulate(v, axis=axis))
         got = F.reduce("reduce_max", V, (1,)).numpy()
         assert np.array_equal(got, v.max(axis=1))
+
+
+def test_contiguous_copy_of_views(hip_backend):
+    """Tensor.contiguous(): transposed, sliced, broadcast and flipped views come back in
+    row-major order in storage of their own (the layout copy softmax makes of a view)."""
+    a = randint(211, 5 * 7 * 9, -1000, 1000).astype(np.int32).reshape(5, 7, 9)
+    T = Tensor.from_numpy(hip_backend, a)
+    for view, want in ((T.transpose([2, 0, 1]), a.transpose(2, 0, 1)),
+                       (T.transpose([1, 0, 2]), a.transpose(1, 0, 2)),
+                       (T.flip([1]), a[:, ::-1, :]),
+                       (T, a)):
+        C = view.contiguous()
+        assert C.shape.is_contiguous() and C.storage is not view.storage
+        assert (C.numpy() == want).all()
+    before = T.numpy().copy()
+    C = T.contiguous()
+    C.storage.zero_()
+    assert (T.numpy() == before).all()
