@@ -9,6 +9,8 @@
 // with coalesced loads, every thread finds its own split by a search in LDS, merges kItems
 // outputs serially, and the tile leaves through LDS again so that stores are coalesced.
 // Bandwidth bound: every input element is read once and every output element written once.
+// Output rows of up to 2048 elements skip the partition: merge_rows_small packs several rows
+// into a workgroup.
 #include <type_traits>
 
 #include "common.hip.h"
@@ -172,6 +174,97 @@ __global__ __launch_bounds__(kBlock) void merge_tiles(const T* __restrict__ x, c
         if (e * kBlock + tid < total) store_stream(&zr[static_cast<int64_t>(e * kBlock + tid) * v.sz], out[e]);
 }
 
+// Short rows: several rows per workgroup.  A row of n <= 256 * ITEMS outputs belongs to a team
+// of 2^lg consecutive threads (ITEMS outputs each), a workgroup holds 256 >> lg rows, each in
+// its own slab of LDS.  No partition pass and no scratch: a row is one tile whose split is
+// known (all of x, all of y).  The steps are those of merge_tiles.
+template <typename T, bool DESC, int ITEMS>
+__global__ __launch_bounds__(kBlock) void merge_rows_small(const T* __restrict__ x, const T* __restrict__ y, T* __restrict__ z,
+                                                           MergeViews v, int64_t rows, int lg) {
+    __shared__ T buf[kBlock * ITEMS + kBlock * ITEMS / 32];
+    auto at = [](int p) { return p + (p >> 5); };
+    const int tid = threadIdx.x;
+    const int team = 1 << lg;
+    const int sub = tid & (team - 1);
+    const int base = (tid - sub) * ITEMS;                         // the row's slab
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * (kBlock >> lg) + (tid >> lg);
+    const bool live = row < rows;
+    const int na = static_cast<int>(v.na), nb = static_cast<int>(v.nb), n = na + nb;
+    const T* xr = x + (live ? v.xrows.at(row) : 0);
+    const T* yr = y + (live ? v.yrows.at(row) : 0);
+
+    T in[ITEMS];
+#pragma unroll
+    for (int e = 0; e < ITEMS; ++e) {
+        const int k = e * team + sub;
+        if (live && k < n) in[e] = load_stream(k < na ? xr + k * v.sx : yr + (k - na) * v.sy);
+    }
+#pragma unroll
+    for (int e = 0; e < ITEMS; ++e) {
+        const int k = e * team + sub;
+        if (live && k < n) buf[at(base + k)] = in[e];
+    }
+    __syncthreads();
+
+    int diag = sub * ITEMS;
+    if (diag > n) diag = n;
+    int i = 0;
+    if (live)
+        i = static_cast<int>(merge_split<T, DESC>(
+            diag, na, nb, [&](int64_t k) { return buf[at(base + static_cast<int>(k))]; },
+            [&](int64_t k) { return buf[at(base + na + static_cast<int>(k))]; }));
+    int j = diag - i;
+    T out[ITEMS];
+    T xv = buf[at(base + (i < na ? i : 0))], yv = buf[at(base + (j < nb ? na + j : 0))];
+#pragma unroll
+    for (int e = 0; e < ITEMS; ++e) {
+        const bool has_x = i < na, has_y = j < nb;
+        const bool take_y = has_y && (!has_x || before<T, DESC>(yv, xv));
+        out[e] = take_y ? yv : xv;
+        i += take_y ? 0 : 1;
+        j += take_y ? 1 : 0;
+        int next = take_y ? na + j : i;
+        if (next >= n) next = 0;
+        const T nv = buf[at(base + next)];
+        if (take_y) yv = nv;
+        else xv = nv;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < ITEMS; ++e)
+        if (sub * ITEMS + e < n) buf[at(base + sub * ITEMS + e)] = out[e];
+    __syncthreads();
+    if (!live) return;
+    T* zr = z + v.zrows.at(row);
+#pragma unroll
+    for (int e = 0; e < ITEMS; ++e) {
+        const int k = e * team + sub;
+        if (k < n) out[e] = buf[at(base + k)];
+    }
+#pragma unroll
+    for (int e = 0; e < ITEMS; ++e) {
+        const int k = e * team + sub;
+        if (k < n) store_stream(&zr[static_cast<int64_t>(k) * v.sz], out[e]);
+    }
+}
+
+constexpr int kSmallRowMax = kBlock * 8;        // longest output row merge_rows_small takes
+
+template <typename T, bool DESC>
+int launch_merge_small(hipStream_t stream, int64_t m, const MergeViews& v, const T* x, const T* y, T* z) {
+    const int n = static_cast<int>(v.na + v.nb);
+    const int items = n <= 256 ? 4 : 8;
+    int lg = 0;
+    while ((items << lg) < n) ++lg;                               // team = 2^lg threads, at most 256
+    const int64_t blocks = ceil_div(m, static_cast<int64_t>(kBlock >> lg));
+    if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+    const dim3 grid(static_cast<unsigned>(blocks));
+    if (items == 4) merge_rows_small<T, DESC, 4><<<grid, dim3(kBlock), 0, stream>>>(x, y, z, v, m, lg);
+    else merge_rows_small<T, DESC, 8><<<grid, dim3(kBlock), 0, stream>>>(x, y, z, v, m, lg);
+    DLFX_CHECK_LAUNCH();
+    return DLFX_OK;
+}
+
 struct MergeLayout {
     int64_t tiles_per_row;
     size_t total;
@@ -190,6 +283,7 @@ int launch_merge(hipStream_t stream, int dir, int64_t m, const MergeViews& v, co
                  void* scratch, size_t scratch_bytes) {
     const int64_t n = v.na + v.nb;
     if (n > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;       // splits are 32-bit
+    if (n <= kSmallRowMax) return dir ? launch_merge_small<T, true>(stream, m, v, x, y, z) : launch_merge_small<T, false>(stream, m, v, x, y, z);
     const MergeLayout l = merge_layout(sizeof(T), m, n);
     if (m * l.tiles_per_row > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
     if (!scratch || scratch_bytes < l.total) return DLFX_ERR_SCRATCH_TOO_SMALL;
