@@ -721,6 +721,94 @@ __global__ __launch_bounds__(256) void topk_rows_wave(TopkIo<typename BitsOf<E>:
     }
 }
 
+// Rows that lie side by side in memory (the axis is an outer dimension of the tensor, the
+// innermost row dimension has stride 1) and a limit of at most 8: one thread per row and
+// segment of the axis, so the 64 lanes of a wave read 64 neighbouring elements whatever the
+// stride along the axis.  A thread keeps the KMAX best (image, index) entries it has seen in
+// registers, ordered; an element enters only when it beats the last of them.  SEG waves share
+// 64 rows, each scanning a contiguous piece of the axis; their lists meet in LDS and the first
+// wave merges and writes them.  No scratch, any row length.
+constexpr int kColsLimit = 8;
+
+template <typename K, int KMAX>
+__device__ __forceinline__ void cols_insert(K (&lo)[KMAX], uint32_t (&li)[KMAX], K o, uint32_t x) {
+    if (beats<K>(o, x, lo[KMAX - 1], li[KMAX - 1]) == 0u) return;
+#pragma unroll
+    for (int p = 0; p < KMAX; ++p) {
+        const bool b = beats<K>(o, x, lo[p], li[p]) != 0u;
+        const K to = lo[p];
+        const uint32_t tx = li[p];
+        lo[p] = b ? o : to;
+        li[p] = b ? x : tx;
+        o = b ? to : o;
+        x = b ? tx : x;
+    }
+}
+
+template <typename E, int KMAX, int SEG>
+__global__ __launch_bounds__(kWave * SEG) void topk_cols(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> io,
+                                                         int64_t rows, int64_t n, int limit) {
+    using K = typename BitsOf<E>::type;
+    using S = typename BitsOf<E>::storage;
+    constexpr int kind = BitsOf<E>::kind;
+    constexpr int kUnroll = 8;
+    __shared__ K s_ord[SEG > 1 ? SEG - 1 : 1][KMAX][kWave];
+    __shared__ uint32_t s_idx[SEG > 1 ? SEG - 1 : 1][KMAX][kWave];
+    const int lane = threadIdx.x % kWave;
+    const int seg = threadIdx.x / kWave;
+    // workgroups are dealt to the 8 XCDs in turn: give each XCD one contiguous range of rows,
+    // so that the pieces of a page (and of a cache line) are fetched through one L2 and TLB
+    const int64_t per_xcd = gridDim.x / 8;                 // the grid is a multiple of 8
+    const int64_t block = static_cast<int64_t>(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    const int64_t row = block * kWave + lane;
+    const bool live = row < rows;
+    const S* xr = io.x + (live ? io.xmap.at(row) : 0);
+    const K flip = io.largest ? K(0) : (kind == kKeyFloat ? KeyBits<K>::kSign : ~K(0));
+
+    K lo[KMAX];
+    uint32_t li[KMAX];
+#pragma unroll
+    for (int p = 0; p < KMAX; ++p) {
+        lo[p] = K(0);                    // beaten by every element of the row (lower index)
+        li[p] = 0xffffffffu;
+    }
+    const int64_t chunk = (n + SEG - 1) / SEG;
+    const int64_t j0 = seg * chunk;
+    const int64_t j1 = j0 + chunk < n ? j0 + chunk : n;
+    for (int64_t j = j0; j < j1; j += kUnroll) {
+        K o[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const bool in = live && j + u < j1;
+            o[u] = in ? to_ord<K>(static_cast<K>(widen_bits<K, S>(load_stream(xr + (j + u) * io.sx), kind) ^ flip), kind, 1) : K(0);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+            cols_insert<K, KMAX>(lo, li, o[u], (live && j + u < j1) ? static_cast<uint32_t>(j + u) : 0xffffffffu);
+    }
+    if constexpr (SEG > 1) {
+        if (seg > 0) {
+#pragma unroll
+            for (int p = 0; p < KMAX; ++p) {
+                s_ord[seg - 1][p][lane] = lo[p];
+                s_idx[seg - 1][p][lane] = li[p];
+            }
+        }
+        __syncthreads();
+        if (seg > 0) return;
+        for (int s = 0; s < SEG - 1; ++s) {
+#pragma unroll
+            for (int p = 0; p < KMAX; ++p) cols_insert<K, KMAX>(lo, li, s_ord[s][p][lane], s_idx[s][p][lane]);
+        }
+    }
+    if (!live) return;
+    S* yr = io.y + io.ymap.at(row);
+    const int64_t ir = io.imap.at(row);
+#pragma unroll
+    for (int p = 0; p < KMAX; ++p)
+        if (p < limit) emit_one<K>(io, yr, ir, xr, p, lo[p], li[p]);
+}
+
 // E: the element type.  ALIGNED: the axis is contiguous and every row starts on a 16-byte
 // boundary (checked on the host), so rows are read with 128-bit loads off one base register.
 //
@@ -1047,6 +1135,28 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
     io.kind = BitsOf<T>::kind;
     io.largest = dir ? 1 : 0;
     if (m > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+
+    // rows side by side in memory, small limit: one thread per row (and segment of the axis)
+    if (limit <= kColsLimit && io.sx != 1 && io.sx != -1 && m >= 16384 && n <= 0x7fffffffLL && io.xmap.rank >= 1 &&
+        io.xmap.strides[io.xmap.rank - 1] == 1 && io.xmap.dims[io.xmap.rank - 1] >= kWave) {
+        const int lim = static_cast<int>(limit);
+        const int64_t blocks = ceil_div(m, static_cast<int64_t>(kWave));
+        const int seg = (blocks >= 8192 || n < 64) ? 1 : (blocks >= 2048 || n < 512) ? 4 : 8;
+        const dim3 cgrid(static_cast<unsigned>(ceil_div(blocks, 8) * 8));
+#define DLFX_TOPK_COLS(KMAX)                                                                        \
+    do {                                                                                            \
+        if (seg == 1) topk_cols<T, KMAX, 1><<<cgrid, dim3(kWave), 0, stream>>>(io, m, n, lim);      \
+        else if (seg == 4) topk_cols<T, KMAX, 4><<<cgrid, dim3(kWave * 4), 0, stream>>>(io, m, n, lim); \
+        else topk_cols<T, KMAX, 8><<<cgrid, dim3(kWave * 8), 0, stream>>>(io, m, n, lim);           \
+    } while (0)
+        if (lim <= 1) DLFX_TOPK_COLS(1);
+        else if (lim <= 2) DLFX_TOPK_COLS(2);
+        else if (lim <= 4) DLFX_TOPK_COLS(4);
+        else DLFX_TOPK_COLS(8);
+#undef DLFX_TOPK_COLS
+        DLFX_CHECK_LAUNCH();
+        return DLFX_OK;
+    }
 
     if (selection_fits(sizeof(K), n, limit)) {
         const dim3 grid(static_cast<unsigned>(m));

@@ -164,3 +164,47 @@ def test_short_rows_one_wave_per_row(hip_backend, oracle_backend, n):
     Yh, Ih = F.top_k(T, min(4, a.shape[0]), 0, False)
     Yo, Io = F.top_k(O, min(4, a.shape[0]), 0, False)
     assert np.array_equal(Ih.numpy(), Io.numpy()) and np.array_equal(Yh.numpy(), Yo.numpy())
+
+
+@pytest.mark.parametrize("n", [1, 2, 7, 63, 64, 100, 511, 512, 700])
+def test_rows_side_by_side_in_memory(hip_backend, oracle_backend, n):
+    """top_k along an outer axis with a limit of at most 8: one thread per row, several waves
+    per row segment.  Every list length, both directions, all element types, rows that are all
+    ties, row counts that leave lanes idle, and a middle axis."""
+    cols = 16400 + n % 50
+    for dtype in (np.float32, np.int32, np.float64, np.int64, np.float16, np.int16):
+        x = (normal(230 + n, n * cols) * 40).astype(dtype).reshape(n, cols)
+        x[:, 1] = 3                                                   # all equal
+        x[:, 2] = randint(231 + n, n, 0, 3).astype(dtype)             # three distinct values
+        x[:, 3] = np.sort(x[:, 3], kind="stable")
+        x[:, 4] = np.sort(x[:, 4], kind="stable")[::-1]
+        Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
+        for k in sorted({1, min(n, 2), min(n, 3), min(n, 4), min(n, 5), min(n, 8)}):
+            for largest in (True, False):
+                Yh, Ih = F.top_k(Xh, k, 0, largest)
+                Yo, Io = F.top_k(Xo, k, 0, largest)
+                assert np.array_equal(Ih.numpy(), Io.numpy()), (dtype, k, largest)
+                assert np.array_equal(Yh.numpy().view(np.uint8), Yo.numpy().view(np.uint8))
+    a = (normal(232, 3 * n * 6000) * 9).astype(np.float32).reshape(3, n, 6000)
+    a[1, :, 17] = np.nan                                              # ordered by bit pattern, as in the sort
+    a[2, n // 2, :] = -0.0
+    a[2, 0, :] = 0.0
+    T, O = Tensor.from_numpy(hip_backend, a), Tensor.from_numpy(oracle_backend, a)
+    k = min(5, n)
+    Yh, Ih = F.top_k(T, k, 1, True, index_dtype=np.int64)
+    SV, SI = F.argsort(T, 1, True, with_values=True)
+    assert Ih.numpy().dtype == np.int64 and np.array_equal(Ih.numpy(), SI.numpy()[:, :k, :])
+    assert np.array_equal(Yh.numpy().view(np.uint32), SV.numpy()[:, :k, :].view(np.uint32))
+    Yh, Ih = F.top_k(T.flip([1]), k, 1, False)
+    Yo, Io = F.top_k(O.flip([1]), k, 1, False)
+    ok = ~np.isnan(Yo.numpy())
+    assert np.array_equal(Ih.numpy()[ok], Io.numpy()[ok]) and np.array_equal(Yh.numpy()[ok], Yo.numpy()[ok])
+
+
+def test_many_rows_side_by_side_one_wave_per_block(hip_backend, oracle_backend):
+    x = (normal(240, 64 * 524291) * 5).astype(np.float32).reshape(64, 524291)
+    Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
+    for k, largest in ((5, True), (8, False)):
+        Yh, Ih = F.top_k(Xh, k, 0, largest)
+        Yo, Io = F.top_k(Xo, k, 0, largest)
+        assert np.array_equal(Ih.numpy(), Io.numpy()) and np.array_equal(Yh.numpy(), Yo.numpy())
