@@ -137,3 +137,45 @@ def test_nchw_reductions_full_size(hip_backend):
     want = torch.cumsum(x.double(), 1)
     mag = torch.cumsum(x.double().abs(), 1)
     assert bool(((cs.double() - want).abs() <= 4 * 9 * EPS32 * mag).all())
+
+
+def test_tensors_of_more_than_2_32_elements(hip_backend):
+    """Element offsets beyond 32 bits (HBM holds 2^36 fp32 elements): totals above 2^32 are
+    served, single rows above 2^32 elements by reduce and scan; the routines whose results are
+    32-bit positions or counts refuse such a row with the too-large status."""
+    import torch
+    from dlf_amd.hip_backend import DlfxError
+    g = torch.Generator(device="cuda").manual_seed(16)
+    N = 4_400_000_000
+    x = torch.randint(-100, 100, (N,), dtype=torch.int32, device="cuda", generator=g)
+    X = wrap(hip_backend, x)
+    total = x.sum(dtype=torch.int64).to(torch.int32)
+    assert int(F.reduce("reduce_sum", X, ()).storage[0]) == int(total)
+    assert int(F.reduce("reduce_max", X, ()).storage[0]) == int(x.max())
+    y = dev(F.cumsum(X, 0))
+    for lo in (0, (1 << 31) - 5000, (1 << 32) - 5000, N - 6000):
+        base = int(x[:lo].sum(dtype=torch.int64)) if lo else 0
+        want = (torch.cumsum(x[lo:lo + 6000].long(), 0) + base).to(torch.int32)
+        assert torch.equal(y[lo:lo + 6000], want), lo
+    del y
+    for call in (lambda: F.argmax(wrap(hip_backend, x.view(1, N)), 1), lambda: F.count(wrap(hip_backend, x.view(1, N)), np.int32(3), (1,)),
+                 lambda: F.nonzero(X)):
+        with pytest.raises(DlfxError, match="too large"):
+            call()
+    xr = x[:1025 * (1 << 22)].view(1025, 1 << 22)
+    assert torch.equal(dev(F.cumsum(wrap(hip_backend, xr), 1))[-3:], torch.cumsum(xr[-3:], 1, dtype=torch.int32))
+    assert torch.equal(dev(F.reduce("reduce_sum", wrap(hip_backend, xr), (1,))), xr.sum(dim=1, dtype=torch.int64).to(torch.int32))
+    assert torch.equal(dev(F.reduce("reduce_sum", wrap(hip_backend, xr), (0,))), xr.sum(dim=0, dtype=torch.int64).to(torch.int32))
+    am = dev(F.argmax(wrap(hip_backend, xr), 1)).long().reshape(-1)
+    first = (xr == xr.amax(dim=1, keepdim=True)).to(torch.int8).argmax(dim=1)
+    assert torch.equal(am, first)
+    xt = x[:135000 * 32000].view(135000, 32000)
+    Y, I = F.top_k(wrap(hip_backend, xt), 5, 1, True)
+    for rows in (slice(0, 32), slice(-32, None)):
+        w = torch.sort(xt[rows], dim=1, descending=True, stable=True)
+        assert torch.equal(dev(Y)[rows], w.values[:, :5]) and torch.equal(dev(I)[rows].long(), w.indices[:, :5])
+    del Y, I, xt
+    xs = x[:66000 * 65536].view(66000, 65536)
+    ys = dev(F.sort(wrap(hip_backend, xs), 1))
+    for rows in (slice(0, 8), slice(32768, 32776), slice(-8, None)):
+        assert torch.equal(ys[rows], torch.sort(xs[rows], dim=1).values)
