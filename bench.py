@@ -292,6 +292,53 @@ def make_ops(be, which):
             call()
             assert torch.equal(zm, torch.sort(torch.cat([a, b], dim=1), dim=1).values)
         ops.append(Op("N2", "merge_f32_[64,2^19]+[64,2^19]", 64 * 2 * half, 2 * 4 * 64 * 2 * half, calls, v_merge))
+    # ---------------- S1 (only on request): many short rows, and top_k along an outer axis
+    if on("short"):
+        for rows_s, n_s in ((1 << 20, 64), (1 << 18, 256), (1 << 16, 1024)):
+            text = "[%d,%d]" % (rows_s, n_s)
+            xs_ = gen((rows_s, n_s), torch.float32, lambda c: synth.normal(20 + 100 * c), 2)
+            ops += [op for op in sort_ops(be, tensor, xs_, "S1", "f32_" + text) if "_asc_" in op.name]
+            ops += topk_ops(be, tensor, xs_, (5,), "S1", text)
+            calls, ycs = scan_calls(xs_, 1)
+
+            def v_cs(x=xs_[0], y=ycs, call=calls[0]):
+                call()
+                want = torch.cumsum(x.double(), 1)
+                tol = 4 * 10 * float(np.finfo(np.float32).eps) * torch.cumsum(x.double().abs(), 1)
+                assert bool(((y.double() - want).abs() <= tol).all()), "short-row cumsum out of tolerance"
+            ops.append(Op("S1", "cumsum_f32_" + text, rows_s * n_s, 8 * rows_s * n_s, calls, v_cs))
+            ysm = empty((rows_s, n_s), torch.float32)
+            calls = [be.softmax("softmax", dtype_code(np.float32), rows_s, n_s, x.view(-1), 0, ysm.view(-1), 0, defer=True)
+                     for x in xs_]
+
+            def v_sm(x=xs_[0], y=ysm, call=calls[0]):
+                call()
+                assert torch.allclose(y.double(), torch.softmax(x.double(), 1), rtol=1e-5, atol=1e-12)
+            ops.append(Op("S1", "softmax_f32_" + text, rows_s * n_s, 8 * rows_s * n_s, calls, v_sm))
+            ha = [torch.sort(x[:, :n_s // 2], dim=1).values.contiguous() for x in xs_]
+            hb = [torch.sort(x[:, n_s // 2:], dim=1).values.contiguous() for x in xs_]
+            zs = empty((rows_s, n_s), torch.float32)
+            Z = tensor(zs)
+            calls = [be.merge(0, dtype_code(np.float32), tensor(a).shape, tensor(a).storage, tensor(b).shape, tensor(b).storage,
+                              Z.shape, Z.storage, defer=True) for a, b in zip(ha, hb)]
+
+            def v_mg(x=xs_[0], z=zs, call=calls[0]):
+                call()
+                assert torch.equal(z, torch.sort(x, dim=1).values)
+            ops.append(Op("S1", "merge_f32_%s/2+%s/2" % (text, text), rows_s * n_s, 8 * rows_s * n_s, calls, v_mg))
+        xo = gen((64, 1 << 20), torch.float32, lambda c: synth.normal(21 + 100 * c), 2)
+        for k in (1, 5):
+            Y = Tensor.empty(be, [k, 1 << 20], np.float32)
+            I = Tensor.empty(be, [k, 1 << 20], np.int32)
+            calls = [be.top_k(k, 1, dtype_code(np.float32), 2, tensor(x).shape.moveaxis(0, -1), tensor(x).storage,
+                              Y.shape.moveaxis(0, -1), Y.storage, I.shape.moveaxis(0, -1), I.storage, defer=True) for x in xo]
+
+            def v_tc(x=xo[0], Y=Y, I=I, k=k, call=calls[0]):
+                call()
+                w = torch.sort(x, dim=0, descending=True, stable=True)
+                assert torch.equal(Y.storage[:k << 20].view(k, 1 << 20), w.values[:k]), "outer-axis top_k values"
+                assert torch.equal(I.storage[:k << 20].view(k, 1 << 20).long(), w.indices[:k]), "outer-axis top_k indices"
+            ops.append(Op("S1", "top_k%d_axis0_f32_[64,2^20]" % k, 64 << 20, 4 * (64 << 20) + 8 * (k << 20), calls, v_tc))
     return ops
 
 
@@ -460,7 +507,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3")
+    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3 | short (many short rows and an outer axis; not part of all)")
     ap.add_argument("--cpu-all", action="store_true",
                     help="also time the CPU restatement on a bounded sample of every configuration")
     ap.add_argument("--no-cpu", action="store_true")

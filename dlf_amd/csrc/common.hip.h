@@ -252,6 +252,70 @@ __device__ __forceinline__ T wave_sort_descending(T v) {
     return v;
 }
 
+template <typename T>
+__device__ __forceinline__ T lane_xor_any(T v, int j) {      // j is a constant after unrolling
+    switch (j) {
+        case 1: return lane_xor_const<1>(v);
+        case 2: return lane_xor_const<2>(v);
+        case 4: return lane_xor_const<4>(v);
+        case 8: return lane_xor_const<8>(v);
+        case 16: return lane_xor_const<16>(v);
+        default: return lane_xor_const<32>(v);
+    }
+}
+
+// Bitonic network over the 64 * ITEMS (key, index) entries of a wavefront; entry i * 64 + lane
+// is item i of the lane and ends up holding the entry of that rank in the order `first`
+// (first(ka, ia, kb, ib): entry a comes strictly before entry b).  Exchanges at a distance
+// below 64 cross lanes; the others pair two items of one lane, with a direction known at
+// compile time.  The indices travel only when PAIRS is set.
+template <bool PAIRS, int ITEMS, typename K, typename First>
+__device__ __forceinline__ void wave_bitonic_items(K (&key)[ITEMS], uint32_t (&idx)[ITEMS], First first) {
+    constexpr int N = kWave * ITEMS;
+    const int lane = __lane_id();
+#pragma unroll
+    for (int k = 2; k <= N; k <<= 1) {
+#pragma unroll
+        for (int j = k >> 1; j >= 1; j >>= 1) {
+            if (j >= kWave) {
+                const int jj = j / kWave;
+#pragma unroll
+                for (int i = 0; i < ITEMS; ++i) {
+                    if (i & jj) continue;
+                    const int o = i | jj;
+                    const bool ascending = ((i * kWave) & k) == 0;
+                    const bool swap = ascending ? first(key[o], idx[o], key[i], idx[i]) : first(key[i], idx[i], key[o], idx[o]);
+                    const K ka = key[i], kb = key[o];
+                    key[i] = swap ? kb : ka;
+                    key[o] = swap ? ka : kb;
+                    if constexpr (PAIRS) {
+                        const uint32_t ia = idx[i], ib = idx[o];
+                        idx[i] = swap ? ib : ia;
+                        idx[o] = swap ? ia : ib;
+                    }
+                }
+            } else {
+                const bool low = (lane & j) == 0;
+#pragma unroll
+                for (int i = 0; i < ITEMS; ++i) {
+                    const bool ascending = k < kWave ? (lane & k) == 0 : ((i * kWave) & k) == 0;
+                    const bool keep_first = low == ascending;
+                    const K other_key = lane_xor_any(key[i], j);
+                    if constexpr (PAIRS) {
+                        const uint32_t other_idx = lane_xor_any(idx[i], j);
+                        if (keep_first == first(other_key, other_idx, key[i], idx[i])) {
+                            key[i] = other_key;
+                            idx[i] = other_idx;
+                        }
+                    } else {
+                        if (keep_first == first(other_key, 0u, key[i], 0u)) key[i] = other_key;
+                    }
+                }
+            }
+        }
+    }
+}
+
 // All-lanes reduction over a wavefront with a commutative `join`.
 template <typename T, typename Join>
 __device__ __forceinline__ T wave_reduce(T v, Join join) {

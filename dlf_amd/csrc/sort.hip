@@ -775,12 +775,66 @@ __global__ __launch_bounds__(256) void sort_rows_wave(PassIo<K> io, int64_t rows
     }
 }
 
+// Rows of 65 to 64 * ITEMS elements: still one wavefront per row and no LDS.  Element
+// i * 64 + lane is item i of the lane (coalesced loads and stores); the bitonic network runs
+// over that index: exchanges at a distance below 64 cross lanes, the others pair two items of
+// one lane, with a direction known at compile time.
+template <typename K, bool PAIRS, int ITEMS>
+__global__ __launch_bounds__(256) void sort_rows_wave_items(PassIo<K> io, int64_t rows, int64_t n) {
+    const int lane = lane_id();
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+    if (row >= rows) return;
+    const K* xrow = io.x + io.xmap.at(row);
+    const int n32 = static_cast<int>(n);
+    K key[ITEMS];
+    uint32_t idx[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        const int e = i * kWave + lane;
+        key[i] = e < n32 ? key_of_element<K>(io, xrow[static_cast<int64_t>(e) * io.sx]) : ~K(0);   // padding sorts last
+        idx[i] = static_cast<uint32_t>(e);
+    }
+    wave_bitonic_items<PAIRS, ITEMS>(key, idx, [](K ka, uint32_t ia, K kb, uint32_t ib) {      // a strictly before b
+        if constexpr (PAIRS) return ka < kb || (ka == kb && ia < ib);
+        else return ka < kb;
+    });
+    K* yrow = io.y ? io.y + io.ymap.at(row) : nullptr;
+    const int64_t irow = (PAIRS && io.idx) ? io.imap.at(row) : 0;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        const int e = i * kWave + lane;
+        if (e >= n32) continue;                            // the first n places hold the row in order
+        if (yrow) {
+            K bits = decode_key<K>(key[i], io.kind, io.descending);
+            if constexpr (PAIRS) {
+                if (io.restore_zero && static_cast<K>(bits << 1) == 0) bits = xrow[static_cast<int64_t>(idx[i]) * io.sx];
+            }
+            yrow[static_cast<int64_t>(e) * io.sy] = bits;
+        }
+        if constexpr (PAIRS) {
+            if (io.idx) {
+                const int64_t at = irow + static_cast<int64_t>(e) * io.si;
+                if (io.idx64) static_cast<int64_t*>(io.idx)[at] = static_cast<int64_t>(idx[i]);
+                else static_cast<int32_t*>(io.idx)[at] = static_cast<int32_t>(idx[i]);
+            }
+        }
+    }
+}
+
+// longest row sorted by one wavefront (dlfx_set_tuning "sort_wave_rows": 64, 128, 256 or 512)
+int g_sort_wave_rows = 512;
+
 constexpr int64_t kSmallRow = 4096;      // longest row sort_rows_small takes
 
 template <typename K, bool PAIRS>
 int launch_small(hipStream_t stream, const PassIo<K>& io, int64_t m, int64_t n) {
     const dim3 grid(static_cast<unsigned>(m)), block(256);
+    // eight items per lane pay off except for 4-byte keys that carry an index
+    const bool wave_items8 = g_sort_wave_rows >= 8 * kWave && !(PAIRS && sizeof(K) == 4);
     if (n <= kWave) sort_rows_wave<K, PAIRS><<<dim3(static_cast<unsigned>(ceil_div(m, 4))), block, 0, stream>>>(io, m, n);
+    else if (n <= 2 * kWave && g_sort_wave_rows >= 2 * kWave) sort_rows_wave_items<K, PAIRS, 2><<<dim3(static_cast<unsigned>(ceil_div(m, 4))), block, 0, stream>>>(io, m, n);
+    else if (n <= 4 * kWave && g_sort_wave_rows >= 4 * kWave) sort_rows_wave_items<K, PAIRS, 4><<<dim3(static_cast<unsigned>(ceil_div(m, 4))), block, 0, stream>>>(io, m, n);
+    else if (n <= 8 * kWave && wave_items8) sort_rows_wave_items<K, PAIRS, 8><<<dim3(static_cast<unsigned>(ceil_div(m, 4))), block, 0, stream>>>(io, m, n);
     else if (n <= 512) sort_rows_small<K, PAIRS, 2><<<grid, block, 0, stream>>>(io, n);
     else if (n <= 1024) sort_rows_small<K, PAIRS, 4><<<grid, block, 0, stream>>>(io, n);
     else if (n <= 2048) sort_rows_small<K, PAIRS, 8><<<grid, block, 0, stream>>>(io, n);
@@ -950,6 +1004,10 @@ int sort_entry(hipStream_t stream, int dtype, const SortArgs& a0, void* scratch,
 bool set_sort_tuning(const char* key, int64_t value) {
     if (!std::strcmp(key, "sort_poll_limit") && value >= 0 && value <= (1 << 30)) {
         g_sort_poll_limit = static_cast<int>(value);
+        return true;
+    }
+    if (!std::strcmp(key, "sort_wave_rows") && value >= 0 && value <= 512) {
+        g_sort_wave_rows = static_cast<int>(value);
         return true;
     }
     return false;

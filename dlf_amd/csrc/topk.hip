@@ -626,6 +626,7 @@ template <> struct BitsOf<int16_t> { using type = uint32_t; using storage = uint
 // for any input, and only slow where it is needed.
 constexpr int kWaveRowMax = 4096;       // longest row topk_rows_wave takes
 constexpr int kWaveRowLimit = 16;       // largest limit (the limit-th of 64 lane maxima is a weak bound beyond)
+constexpr int kWaveSortItems = 4;       // rows of up to 64 * this many elements can be ordered whole by the wave
 
 template <typename E, int ITEMS>
 __global__ __launch_bounds__(256) void topk_rows_wave(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> io,
@@ -651,6 +652,25 @@ __global__ __launch_bounds__(256) void topk_rows_wave(TopkIo<typename BitsOf<E>:
     for (int i = 0; i < ITEMS; ++i) {
         const uint32_t e = static_cast<uint32_t>(i * kWave + lane);
         ord[i] = e < n32 ? to_ord<K>(static_cast<K>(widen_bits<K, S>(xr[static_cast<int64_t>(e) * io.sx], kind) ^ flip), kind, 1) : K(0);
+    }
+    // rows of up to 256 elements and a limit for which the bound below is weak (or cannot be
+    // formed: it is one of 64 lane maxima), and rows the bound fails on: order the whole row
+    auto order_row = [&]() {
+        uint32_t ix[ITEMS];
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) ix[i] = static_cast<uint32_t>(i * kWave + lane);      // padding: image 0, index past the row
+        wave_bitonic_items<true, ITEMS>(ord, ix, [](K ka, uint32_t ia, K kb, uint32_t ib) { return beats<K>(ka, ia, kb, ib) != 0u; });
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const int e = i * kWave + lane;
+            if (e < limit) emit_one<K>(io, yr, ir, xr, e, ord[i], ix[i]);
+        }
+    };
+    if constexpr (ITEMS <= kWaveSortItems) {
+        if (limit > kWaveRowLimit) {
+            order_row();
+            return;
+        }
     }
     K best = 0;
 #pragma unroll
@@ -692,6 +712,10 @@ __global__ __launch_bounds__(256) void topk_rows_wave(TopkIo<typename BitsOf<E>:
         return;
     }
 
+    if constexpr (ITEMS <= kWaveSortItems) {
+        order_row();
+        return;
+    }
     // more than a wave's worth of entries reach the bound: take the best entry that comes
     // after the one taken last, `limit` times (entries are ordered by image, then by lower index)
     K last_o = ~K(0);
@@ -1169,7 +1193,7 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
         uint32_t* row_state = reinterpret_cast<uint32_t*>(sbase + sl.state_off);
         K* spill_ord = reinterpret_cast<K*>(sbase + sl.ord_off);
         uint32_t* spill_idx = reinterpret_cast<uint32_t*>(sbase + sl.idx_off);
-        if (n <= kWaveRowMax && (lim <= kWaveRowLimit || n <= kWave)) {      // at most 64 elements: one wave sort, whatever the limit
+        if (n <= kWaveRowMax && (lim <= kWaveRowLimit || n <= kWaveSortItems * kWave)) {      // at most 256 elements: a wave can order the whole row, whatever the limit
             const dim3 wgrid(static_cast<unsigned>(ceil_div(m, 4)));
 #define DLFX_TOPK_WAVE(ITEMS) topk_rows_wave<T, ITEMS><<<wgrid, dim3(256), 0, stream>>>(io, m, n, lim)
             if (n <= 64) DLFX_TOPK_WAVE(1);

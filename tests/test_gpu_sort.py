@@ -183,10 +183,12 @@ def test_nans_take_the_place_of_their_bit_pattern(hip_backend, dtype):
     assert (np.diff(idx[:, :200], axis=1) > 0).all()                                # equal keys keep their order
 
 
-@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 511, 512, 513, 1023, 1024, 1025, 2047, 2048, 2049, 4095, 4096, 4097])
+@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 100, 127, 128, 129, 255, 256, 257, 300, 511, 512, 513, 1023, 1024, 1025, 2047, 2048, 2049, 4095,
+                               4096, 4097])
 def test_rows_around_the_one_workgroup_limits(hip_backend, oracle_backend, n):
-    """Rows of up to 4096 elements are sorted by one workgroup on chip (512, 1024, 2048 or 4096
-    slots); longer rows take the tiled passes.  Every boundary, all key widths, both directions,
+    """Rows of up to 64, 128, 256 (512 for values only or 8-byte keys) elements are sorted by one
+    wavefront in registers, rows of up to 4096 elements by one workgroup on chip (512, 1024, 2048
+    or 4096 slots); longer rows take the tiled passes.  Every boundary, all key widths, both directions,
     values, indices (32- and 64-bit) and in place."""
     for dtype in (np.float32, np.int64, np.float64, np.int16, np.float16, np.int32):
         x = (normal(200 + n, 5 * n) * 50).astype(dtype).reshape(5, n)
@@ -227,3 +229,22 @@ def test_short_rows_on_strided_views(hip_backend, oracle_backend):
     Y, I = F.argsort(Tensor.from_numpy(hip_backend, z), -1, with_values=True)
     assert I.numpy().tolist() == [[5, 0, 1, 3, 4, 2]]
     assert np.array_equal(np.signbit(Y.numpy()), np.signbit(z[0][I.numpy()[0]])[None, :])
+
+
+@pytest.mark.parametrize("n", [65, 128, 200, 256, 400, 512])
+def test_short_rows_sorted_by_one_workgroup_when_the_wave_sort_is_switched_off(hip_backend, oracle_backend, n):
+    """The one-workgroup kernel still serves rows of 65 to 512 elements when the knob that bounds
+    the wave sort says so (and always for 4-byte keys with indices above 256)."""
+    hip_backend.set_tuning("sort_wave_rows", 64)
+    try:
+        for dtype in (np.float32, np.int64, np.int16):
+            x = (normal(220 + n, 300 * n) * 50).astype(dtype).reshape(300, n)
+            x[3, : n // 2] = x[3, n // 2: 2 * (n // 2)]
+            Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
+            for desc in (False, True):
+                Y, I = F.argsort(Xh, -1, desc, with_values=True)
+                Yo, Io = F.argsort(Xo, -1, desc, with_values=True)
+                assert np.array_equal(I.numpy(), Io.numpy()) and np.array_equal(Y.numpy(), Yo.numpy())
+                assert np.array_equal(F.sort(Xh, -1, desc).numpy(), Yo.numpy())
+    finally:
+        hip_backend.set_tuning("sort_wave_rows", 512)
