@@ -15,11 +15,12 @@ int record_hip_error(hipError_t e) {
 namespace dlfx {
 bool set_scan_tuning(const char* key, int64_t value);
 bool set_sort_tuning(const char* key, int64_t value);
+bool set_topk_tuning(const char* key, int64_t value);
 }
 
 extern "C" int dlfx_set_tuning(const char* key, int64_t value) {
     if (!key) return DLFX_ERR_INVALID_ARGUMENT;
-    if (dlfx::set_scan_tuning(key, value) || dlfx::set_sort_tuning(key, value)) return DLFX_OK;
+    if (dlfx::set_scan_tuning(key, value) || dlfx::set_sort_tuning(key, value) || dlfx::set_topk_tuning(key, value)) return DLFX_OK;
     return DLFX_ERR_UNKNOWN_OP;
 }
 

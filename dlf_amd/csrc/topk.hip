@@ -753,6 +753,9 @@ __global__ __launch_bounds__(256) void topk_rows_wave(TopkIo<typename BitsOf<E>:
 // 64 rows, each scanning a contiguous piece of the axis; their lists meet in LDS and the first
 // wave merges and writes them.  No scratch, any row length.
 constexpr int kColsLimit = 8;
+// longest row topk_rows_thread takes with 4-byte keys, half of it with 8-byte keys
+// (dlfx_set_tuning "topk_thread_rows"); beyond, a wave per row has enough rows in flight and wins
+int g_topk_thread_rows = 256;
 
 template <typename K, int KMAX>
 __device__ __forceinline__ void cols_insert(K (&lo)[KMAX], uint32_t (&li)[KMAX], K o, uint32_t x) {
@@ -826,6 +829,68 @@ __global__ __launch_bounds__(kWave * SEG) void topk_cols(TopkIo<typename BitsOf<
         }
     }
     if (!live) return;
+    S* yr = io.y + io.ymap.at(row);
+    const int64_t ir = io.imap.at(row);
+#pragma unroll
+    for (int p = 0; p < KMAX; ++p)
+        if (p < limit) emit_one<K>(io, yr, ir, xr, p, lo[p], li[p]);
+}
+
+// Many short contiguous rows and a limit of at most 8: one thread per row again, but the rows
+// lie one after the other in memory, so a wavefront reads its 64 rows in pieces of 32 elements
+// with coalesced loads (a half-wave per row piece), passes them through its own slab of LDS
+// (row pitch 33: no bank conflicts either way), and every lane then walks its own row and
+// keeps the KMAX best entries in the ordered register list of topk_cols.  The work per element
+// does not depend on the row length, where a wave per row pays its fixed cost for every row.
+constexpr int kThreadRowChunk = 32;
+
+template <typename E, int KMAX>
+__global__ __launch_bounds__(256) void topk_rows_thread(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> io,
+                                                        int64_t rows, int64_t n, int limit, int64_t row_pitch) {
+    using K = typename BitsOf<E>::type;
+    using S = typename BitsOf<E>::storage;
+    constexpr int kind = BitsOf<E>::kind;
+    constexpr int C = kThreadRowChunk;
+    __shared__ S slab[4][kWave * (C + 1)];
+    const int lane = lane_id();
+    const int w = threadIdx.x / kWave;
+    const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * 4 + w) * kWave;
+    if (row0 >= rows) return;                              // whole waves leave; nothing below synchronises the workgroup
+    const int64_t row = row0 + lane;
+    const bool live = row < rows;
+    const int n32 = static_cast<int>(n);
+    const K flip = io.largest ? K(0) : (kind == kKeyFloat ? KeyBits<K>::kSign : ~K(0));
+    S* mine = slab[w];
+
+    K lo[KMAX];
+    uint32_t li[KMAX];
+#pragma unroll
+    for (int p = 0; p < KMAX; ++p) {
+        lo[p] = K(0);                    // beaten by every element of the row (lower index)
+        li[p] = 0xffffffffu;
+    }
+    const int half = lane / C, col = lane % C;             // C == 32: lanes 0-31 one row piece, lanes 32-63 the next
+    for (int c0 = 0; c0 < n32; c0 += C) {
+        S in[C];
+#pragma unroll
+        for (int t = 0; t < C; ++t) {
+            const int r = 2 * t + half;
+            const bool ok = row0 + r < rows && c0 + col < n32;
+            in[t] = ok ? load_stream(io.x + (row0 + r) * row_pitch + (c0 + col)) : S(0);
+        }
+#pragma unroll
+        for (int t = 0; t < C; ++t) mine[(2 * t + half) * (C + 1) + col] = in[t];
+        team_sync<kWave>();
+#pragma unroll
+        for (int j = 0; j < C; ++j) {
+            const bool ok = live && c0 + j < n32;
+            const K o = ok ? to_ord<K>(static_cast<K>(widen_bits<K, S>(mine[lane * (C + 1) + j], kind) ^ flip), kind, 1) : K(0);
+            cols_insert<K, KMAX>(lo, li, o, ok ? static_cast<uint32_t>(c0 + j) : 0xffffffffu);
+        }
+        team_sync<kWave>();
+    }
+    if (!live) return;
+    const S* xr = io.x + row * row_pitch;
     S* yr = io.y + io.ymap.at(row);
     const int64_t ir = io.imap.at(row);
 #pragma unroll
@@ -1182,6 +1247,21 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
         return DLFX_OK;
     }
 
+    // many short rows one after the other in memory, small limit: one thread per row
+    if (limit <= kColsLimit && io.sx == 1 && io.xmap.rank <= 1 && m >= 16384 &&
+        n <= (sizeof(K) == 4 ? g_topk_thread_rows : g_topk_thread_rows / 2)) {
+        const int lim = static_cast<int>(limit);
+        const int64_t pitch = io.xmap.rank ? io.xmap.strides[0] : 0;
+        const int64_t blocks = ceil_div(m, static_cast<int64_t>(4 * kWave));
+        const dim3 rgrid(static_cast<unsigned>(blocks));
+        if (lim <= 1) topk_rows_thread<T, 1><<<rgrid, dim3(256), 0, stream>>>(io, m, n, lim, pitch);
+        else if (lim <= 2) topk_rows_thread<T, 2><<<rgrid, dim3(256), 0, stream>>>(io, m, n, lim, pitch);
+        else if (lim <= 4) topk_rows_thread<T, 4><<<rgrid, dim3(256), 0, stream>>>(io, m, n, lim, pitch);
+        else topk_rows_thread<T, 8><<<rgrid, dim3(256), 0, stream>>>(io, m, n, lim, pitch);
+        DLFX_CHECK_LAUNCH();
+        return DLFX_OK;
+    }
+
     if (selection_fits(sizeof(K), n, limit)) {
         const dim3 grid(static_cast<unsigned>(m));
         const int lim = static_cast<int>(limit);
@@ -1252,6 +1332,14 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
 }
 
 }  // namespace
+
+bool set_topk_tuning(const char* key, int64_t value) {
+    if (!std::strcmp(key, "topk_thread_rows") && value >= 0 && value <= 65536) {
+        g_topk_thread_rows = static_cast<int>(value);
+        return true;
+    }
+    return false;
+}
 }  // namespace dlfx
 
 using namespace dlfx;

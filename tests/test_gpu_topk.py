@@ -209,3 +209,47 @@ def test_many_rows_side_by_side_one_wave_per_block(hip_backend, oracle_backend):
         Yh, Ih = F.top_k(Xh, k, 0, largest)
         Yo, Io = F.top_k(Xo, k, 0, largest)
         assert np.array_equal(Ih.numpy(), Io.numpy()) and np.array_equal(Yh.numpy(), Yo.numpy())
+
+
+@pytest.mark.parametrize("n", [1, 5, 31, 32, 33, 64, 100, 257, 1000, 1024])
+def test_many_short_rows_one_thread_per_row(hip_backend, oracle_backend, n):
+    """At least 16384 contiguous rows of up to 1024 elements with a limit of at most 8: a thread
+    per row behind a coalesced, LDS-transposed load.  Piece boundaries (32 elements), row counts
+    that leave lanes and waves idle, every list length, ties, all element types, a row pitch
+    above the row length."""
+    hip_backend.set_tuning("topk_thread_rows", 2048)          # by default only rows of up to 256 (8-byte keys: 128) go this way
+    try:
+        _many_short_rows(hip_backend, oracle_backend, n)
+    finally:
+        hip_backend.set_tuning("topk_thread_rows", 256)
+    if n <= 100:
+        _many_short_rows(hip_backend, oracle_backend, n, dtypes=(np.float32, np.int64))
+
+
+def _many_short_rows(hip_backend, oracle_backend, n, dtypes=None):
+    rows = 16384 + 70 + n % 7
+    dtypes = dtypes or ((np.float32, np.int32, np.float64, np.int64, np.float16, np.int16) if n <= 100 else (np.float32, np.int64))
+    for dtype in dtypes:
+        x = (normal(250 + n, rows * n) * 40).astype(dtype).reshape(rows, n)
+        x[1] = 3                                                      # all equal
+        x[2] = randint(251 + n, n, 0, 3).astype(dtype)                # three distinct values
+        x[3] = np.sort(x[3], kind="stable")
+        x[4] = np.sort(x[4], kind="stable")[::-1]
+        Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
+        for k in sorted({1, min(n, 2), min(n, 3), min(n, 5), min(n, 8)}):
+            for largest in (True, False):
+                Yh, Ih = F.top_k(Xh, k, -1, largest)
+                Yo, Io = F.top_k(Xo, k, -1, largest)
+                assert np.array_equal(Ih.numpy(), Io.numpy()), (dtype, k, largest)
+                assert np.array_equal(Yh.numpy().view(np.uint8), Yo.numpy().view(np.uint8))
+    if n >= 5:
+        a = (normal(252, rows * n) * 9).astype(np.float32).reshape(rows, n)
+        a[7, 1] = np.nan
+        a[9, :] = 0.0
+        a[9, n // 2] = -0.0
+        T = Tensor.from_numpy(hip_backend, a).slice([0, 1], [rows, n - 1])      # pitch n, rows of n - 2
+        k = min(4, n - 2)
+        Yh, Ih = F.top_k(T, k, 1, True, index_dtype=np.int64)
+        SV, SI = F.argsort(T, 1, True, with_values=True)
+        assert Ih.numpy().dtype == np.int64 and np.array_equal(Ih.numpy(), SI.numpy()[:, :k])
+        assert np.array_equal(Yh.numpy().view(np.uint32), SV.numpy()[:, :k].view(np.uint32))
