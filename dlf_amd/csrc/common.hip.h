@@ -224,12 +224,15 @@ __device__ __forceinline__ T lane_xor_const(T v) {
 // that starts at lane 0 ends up best-first.  `exchange(J, keep_better)` must replace the lane's
 // item by the item of lane ^ J when that one is better and keep_better holds, or when it is not
 // better and keep_better does not hold.
-template <int WIDTH, typename Exchange>
+// SAME_WAY: every group of WIDTH lanes ends in the same direction (first item in its lowest
+// lane); otherwise neighbouring groups end in opposite directions, as a later merge wants.
+template <int WIDTH, bool SAME_WAY = false, typename Exchange>
 __device__ __forceinline__ void wave_bitonic(Exchange exchange) {
     const int lane = __lane_id();
     auto step = [&](auto jc, int k) {
         constexpr int J = decltype(jc)::value;
-        exchange(jc, ((lane & J) == 0) == ((lane & k) == 0));
+        const bool up = (SAME_WAY && k == WIDTH) ? true : (lane & k) == 0;
+        exchange(jc, ((lane & J) == 0) == up);
     };
 #pragma unroll
     for (int k = 2; k <= WIDTH; k <<= 1) {

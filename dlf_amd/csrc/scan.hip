@@ -367,7 +367,7 @@ template <typename T, int K, int LANES, int ITEMS, typename X, bool NZ, typename
 __global__ __launch_bounds__(kBlock) void scan_rows_group(
     const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
     int64_t rows, int64_t n, int exclusive) {
-    static_assert(LANES == 16 || LANES == kWave, "a DPP row or a wavefront");
+    static_assert(LANES == 1 || LANES == 4 || LANES == 16 || LANES == kWave, "a thread, a quad, a DPP row or a wavefront");
     using Op = ScanOp<T, K>;
     constexpr int V = (vec_width<T>() < ITEMS) ? vec_width<T>() : ITEMS;
     constexpr int KV = ITEMS / V;
@@ -406,7 +406,15 @@ __global__ __launch_bounds__(kBlock) void scan_rows_group(
         for (int j = 1; j < V; ++j) vals[v * V + j] = Op::apply(vals[v * V + j - 1], vals[v * V + j]);
         const T lane_total = vals[v * V + V - 1];
         T incl;
-        if constexpr (LANES == 16) {
+        if constexpr (LANES == 1) {
+            incl = lane_total;
+        } else if constexpr (LANES == 4) {
+            // shifts within a DPP row cross quads: what comes from another quad is dropped
+            const T s1 = dpp_fetch<kRowShr1>(lane_total, Op::identity());
+            incl = combine(l >= 1 ? s1 : Op::identity(), lane_total);
+            const T s2 = dpp_fetch<kRowShr2>(incl, Op::identity());
+            incl = combine(l >= 2 ? s2 : Op::identity(), incl);
+        } else if constexpr (LANES == 16) {
             incl = combine(dpp_fetch<kRowShr1>(lane_total, Op::identity()), lane_total);
             incl = combine(dpp_fetch<kRowShr2>(incl, Op::identity()), incl);
             incl = combine(dpp_fetch<kRowShr4>(incl, Op::identity()), incl);
@@ -639,13 +647,15 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     // Short rows along a unit-stride axis: a group of lanes per row (rows of up to 512 elements;
     // a workgroup per row would leave most of its threads, or of the chip, idle).
     if (!axis_general && axis_unit && n <= 512 && m >= 4) {
-        const int64_t lanes = n <= 64 ? 16 : kWave;
+        const int64_t lanes = n <= 4 ? 1 : n <= 32 ? 4 : n <= 64 ? 16 : kWave;
         const int64_t blocks = ceil_div(m * lanes, kBlock);
         if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
         const dim3 grid(static_cast<unsigned>(blocks)), block(kBlock);
 #define DLFX_SCAN_GROUP(LANES, ITEMS) \
     scan_rows_group<T, K, LANES, ITEMS, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, m, n, exclusive)
-        if (n <= 16) DLFX_SCAN_GROUP(16, 1);
+        if (n <= 4) DLFX_SCAN_GROUP(1, 4);
+        else if (n <= 16) DLFX_SCAN_GROUP(4, 4);
+        else if (n <= 32) DLFX_SCAN_GROUP(4, 8);
         else if (n <= 64) DLFX_SCAN_GROUP(16, 4);
         else if (n <= 256) DLFX_SCAN_GROUP(kWave, 4);
         else DLFX_SCAN_GROUP(kWave, 8);

@@ -238,14 +238,19 @@ int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y) {
         return DLFX_OK;                                                                                         \
     } while (0)
     if (ceil_div(m, 4) > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
-    if (n <= 16 * V) {
-        // very short rows: sixteen lanes per row, sixteen rows per workgroup
-        const dim3 grid(static_cast<unsigned>(ceil_div(m, 16)));
-        if (vec) softmax_rows<T, 16, V, KIND, true><<<grid, dim3(256), 0, stream>>>(x, y, m, n);
-        else softmax_rows<T, 16, V, KIND, false><<<grid, dim3(256), 0, stream>>>(x, y, m, n);
-        DLFX_CHECK_LAUNCH();
-        return DLFX_OK;
-    }
+    // very short rows: one, four or sixteen lanes per row (V elements each), 256, 64 or 16 rows per workgroup
+#define DLFX_LANE_ROWS(TEAM)                                                                                    \
+    do {                                                                                                        \
+        const dim3 grid(static_cast<unsigned>(ceil_div(m, 256 / TEAM)));                                        \
+        if (vec) softmax_rows<T, TEAM, V, KIND, true><<<grid, dim3(256), 0, stream>>>(x, y, m, n);              \
+        else softmax_rows<T, TEAM, V, KIND, false><<<grid, dim3(256), 0, stream>>>(x, y, m, n);                 \
+        DLFX_CHECK_LAUNCH();                                                                                    \
+        return DLFX_OK;                                                                                         \
+    } while (0)
+    if (n <= V) DLFX_LANE_ROWS(1);
+    if (n <= 4 * V) DLFX_LANE_ROWS(4);
+    if (n <= 16 * V) DLFX_LANE_ROWS(16);
+#undef DLFX_LANE_ROWS
     if (n <= kWave * V) DLFX_WAVE_ROWS(V);
     if (n <= kWave * 4 * V) DLFX_WAVE_ROWS(4 * V);
     if (n <= kWave * 32) DLFX_WAVE_ROWS(32);

@@ -731,19 +731,19 @@ __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t n) 
     }
 }
 
-// Rows of at most 64 elements: one wavefront per row, one element per lane, a bitonic network
-// over (key, index) pairs - a total order, so the result is the stable one.  Four rows per
-// workgroup, no LDS, no barrier.
-template <typename K, bool PAIRS>
+// Rows of at most 64 elements: a group of WIDTH = 4, 8, 16, 32 or 64 lanes per row, one element
+// per lane, a bitonic network over (key, index) pairs - a total order, so the result is the
+// stable one.  256 / WIDTH rows per workgroup, no LDS, no barrier.
+template <typename K, bool PAIRS, int WIDTH>
 __global__ __launch_bounds__(256) void sort_rows_wave(PassIo<K> io, int64_t rows, int64_t n) {
-    const int lane = lane_id();
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
-    if (row >= rows) return;
-    const K* xrow = io.x + io.xmap.at(row);
-    const bool live = lane < n;
-    K key = live ? key_of_element<K>(io, xrow[static_cast<int64_t>(lane) * io.sx]) : ~K(0);   // padding sorts last
-    uint32_t idx = static_cast<uint32_t>(lane);
-    wave_bitonic<kWave>([&](auto jc, bool keep_first) {
+    const int at = lane_id() % WIDTH;
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * (256 / WIDTH) + threadIdx.x / WIDTH;
+    const bool row_live = row < rows;                      // lanes of absent rows still take part in the exchanges
+    const K* xrow = io.x + (row_live ? io.xmap.at(row) : 0);
+    const bool live = row_live && at < n;
+    K key = live ? key_of_element<K>(io, xrow[static_cast<int64_t>(at) * io.sx]) : ~K(0);   // padding sorts last
+    uint32_t idx = static_cast<uint32_t>(at);
+    wave_bitonic<WIDTH, true>([&](auto jc, bool keep_first) {
         constexpr int J = decltype(jc)::value;
         const K other_key = lane_xor_const<J>(key);
         bool other_first = other_key < key;
@@ -758,19 +758,19 @@ __global__ __launch_bounds__(256) void sort_rows_wave(PassIo<K> io, int64_t rows
             if (keep_first == other_first) key = other_key;
         }
     });
-    if (!live) return;                                     // the first n lanes hold the row in order
+    if (!live) return;                                     // the first n lanes of the group hold the row in order
     if (io.y) {
         K bits = decode_key<K>(key, io.kind, io.descending);
         if constexpr (PAIRS) {
             if (io.restore_zero && static_cast<K>(bits << 1) == 0) bits = xrow[static_cast<int64_t>(idx) * io.sx];
         }
-        io.y[io.ymap.at(row) + static_cast<int64_t>(lane) * io.sy] = bits;
+        io.y[io.ymap.at(row) + static_cast<int64_t>(at) * io.sy] = bits;
     }
     if constexpr (PAIRS) {
         if (io.idx) {
-            const int64_t at = io.imap.at(row) + static_cast<int64_t>(lane) * io.si;
-            if (io.idx64) static_cast<int64_t*>(io.idx)[at] = static_cast<int64_t>(idx);
-            else static_cast<int32_t*>(io.idx)[at] = static_cast<int32_t>(idx);
+            const int64_t where = io.imap.at(row) + static_cast<int64_t>(at) * io.si;
+            if (io.idx64) static_cast<int64_t*>(io.idx)[where] = static_cast<int64_t>(idx);
+            else static_cast<int32_t*>(io.idx)[where] = static_cast<int32_t>(idx);
         }
     }
 }
@@ -831,7 +831,11 @@ int launch_small(hipStream_t stream, const PassIo<K>& io, int64_t m, int64_t n) 
     const dim3 grid(static_cast<unsigned>(m)), block(256);
     // eight items per lane pay off except for 4-byte keys that carry an index
     const bool wave_items8 = g_sort_wave_rows >= 8 * kWave && !(PAIRS && sizeof(K) == 4);
-    if (n <= kWave) sort_rows_wave<K, PAIRS><<<dim3(static_cast<unsigned>(ceil_div(m, 4))), block, 0, stream>>>(io, m, n);
+    if (n <= 4) sort_rows_wave<K, PAIRS, 4><<<dim3(static_cast<unsigned>(ceil_div(m, 64))), block, 0, stream>>>(io, m, n);
+    else if (n <= 8) sort_rows_wave<K, PAIRS, 8><<<dim3(static_cast<unsigned>(ceil_div(m, 32))), block, 0, stream>>>(io, m, n);
+    else if (n <= 16) sort_rows_wave<K, PAIRS, 16><<<dim3(static_cast<unsigned>(ceil_div(m, 16))), block, 0, stream>>>(io, m, n);
+    else if (n <= 32) sort_rows_wave<K, PAIRS, 32><<<dim3(static_cast<unsigned>(ceil_div(m, 8))), block, 0, stream>>>(io, m, n);
+    else if (n <= kWave) sort_rows_wave<K, PAIRS, kWave><<<dim3(static_cast<unsigned>(ceil_div(m, 4))), block, 0, stream>>>(io, m, n);
     else if (n <= 2 * kWave && g_sort_wave_rows >= 2 * kWave) sort_rows_wave_items<K, PAIRS, 2><<<dim3(static_cast<unsigned>(ceil_div(m, 4))), block, 0, stream>>>(io, m, n);
     else if (n <= 4 * kWave && g_sort_wave_rows >= 4 * kWave) sort_rows_wave_items<K, PAIRS, 4><<<dim3(static_cast<unsigned>(ceil_div(m, 4))), block, 0, stream>>>(io, m, n);
     else if (n <= 8 * kWave && wave_items8) sort_rows_wave_items<K, PAIRS, 8><<<dim3(static_cast<unsigned>(ceil_div(m, 4))), block, 0, stream>>>(io, m, n);

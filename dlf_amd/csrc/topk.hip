@@ -844,7 +844,7 @@ __global__ __launch_bounds__(kWave * SEG) void topk_cols(TopkIo<typename BitsOf<
 // does not depend on the row length, where a wave per row pays its fixed cost for every row.
 constexpr int kThreadRowChunk = 32;
 
-template <typename E, int KMAX>
+template <typename E, int KMAX, bool ONE_RUN>
 __global__ __launch_bounds__(256) void topk_rows_thread(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> io,
                                                         int64_t rows, int64_t n, int limit, int64_t row_pitch) {
     using K = typename BitsOf<E>::type;
@@ -870,22 +870,42 @@ __global__ __launch_bounds__(256) void topk_rows_thread(TopkIo<typename BitsOf<E
         li[p] = 0xffffffffu;
     }
     const int half = lane / C, col = lane % C;             // C == 32: lanes 0-31 one row piece, lanes 32-63 the next
+    // rows shorter than a piece that follow each other without a gap: the wave's 64 rows are
+    // one run of 64 * n elements, read 64 at a time (a piece per row would leave most lanes idle)
+    // (ONE_RUN, chosen by the host: n < 32 and the row pitch equals n)
+    const int run = static_cast<int>((rows - row0 < kWave ? rows - row0 : kWave) * n);
+    const float inv_n = 1.0f / static_cast<float>(n32);
     for (int c0 = 0; c0 < n32; c0 += C) {
         S in[C];
+        if constexpr (ONE_RUN) {
 #pragma unroll
-        for (int t = 0; t < C; ++t) {
-            const int r = 2 * t + half;
-            const bool ok = row0 + r < rows && c0 + col < n32;
-            in[t] = ok ? load_stream(io.x + (row0 + r) * row_pitch + (c0 + col)) : S(0);
+            for (int t = 0; t < C; ++t) {
+                const int f = t * kWave + lane;
+                in[t] = (t < n32 && f < run) ? load_stream(io.x + row0 * row_pitch + f) : S(0);
+            }
+#pragma unroll
+            for (int t = 0; t < C; ++t) {
+                const int f = t * kWave + lane;
+                const int r = static_cast<int>((static_cast<float>(f) + 0.5f) * inv_n);      // f / n, exact for f < 2048
+                if (t < n32 && f < run) mine[r * (C + 1) + (f - r * n32)] = in[t];
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < C; ++t) {
+                const int r = 2 * t + half;
+                const bool ok = row0 + r < rows && c0 + col < n32;
+                in[t] = ok ? load_stream(io.x + (row0 + r) * row_pitch + (c0 + col)) : S(0);
+            }
+#pragma unroll
+            for (int t = 0; t < C; ++t) mine[(2 * t + half) * (C + 1) + col] = in[t];
         }
-#pragma unroll
-        for (int t = 0; t < C; ++t) mine[(2 * t + half) * (C + 1) + col] = in[t];
         team_sync<kWave>();
 #pragma unroll
         for (int j = 0; j < C; ++j) {
-            const bool ok = live && c0 + j < n32;
-            const K o = ok ? to_ord<K>(static_cast<K>(widen_bits<K, S>(mine[lane * (C + 1) + j], kind) ^ flip), kind, 1) : K(0);
-            cols_insert<K, KMAX>(lo, li, o, ok ? static_cast<uint32_t>(c0 + j) : 0xffffffffu);
+            if (c0 + j < n32) {                            // the same for every lane: a scalar branch past the row's end
+                const K o = live ? to_ord<K>(static_cast<K>(widen_bits<K, S>(mine[lane * (C + 1) + j], kind) ^ flip), kind, 1) : K(0);
+                cols_insert<K, KMAX>(lo, li, o, live ? static_cast<uint32_t>(c0 + j) : 0xffffffffu);
+            }
         }
         team_sync<kWave>();
     }
@@ -1254,10 +1274,17 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
         const int64_t pitch = io.xmap.rank ? io.xmap.strides[0] : 0;
         const int64_t blocks = ceil_div(m, static_cast<int64_t>(4 * kWave));
         const dim3 rgrid(static_cast<unsigned>(blocks));
-        if (lim <= 1) topk_rows_thread<T, 1><<<rgrid, dim3(256), 0, stream>>>(io, m, n, lim, pitch);
-        else if (lim <= 2) topk_rows_thread<T, 2><<<rgrid, dim3(256), 0, stream>>>(io, m, n, lim, pitch);
-        else if (lim <= 4) topk_rows_thread<T, 4><<<rgrid, dim3(256), 0, stream>>>(io, m, n, lim, pitch);
-        else topk_rows_thread<T, 8><<<rgrid, dim3(256), 0, stream>>>(io, m, n, lim, pitch);
+        const bool one_run = n < kThreadRowChunk && pitch == n;
+#define DLFX_TOPK_THREAD(KMAX)                                                                      \
+    do {                                                                                            \
+        if (one_run) topk_rows_thread<T, KMAX, true><<<rgrid, dim3(256), 0, stream>>>(io, m, n, lim, pitch);  \
+        else topk_rows_thread<T, KMAX, false><<<rgrid, dim3(256), 0, stream>>>(io, m, n, lim, pitch);         \
+    } while (0)
+        if (lim <= 1) DLFX_TOPK_THREAD(1);
+        else if (lim <= 2) DLFX_TOPK_THREAD(2);
+        else if (lim <= 4) DLFX_TOPK_THREAD(4);
+        else DLFX_TOPK_THREAD(8);
+#undef DLFX_TOPK_THREAD
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
     }

@@ -149,12 +149,12 @@ def test_in_place_long_rows_use_tickets(hip_backend, oracle_backend):
     assert not np.array_equal(Xo.numpy(), Xh.numpy())     # the restated reference loop reproduces the slip
 
 
-@pytest.mark.parametrize("n", [1, 2, 15, 16, 17, 63, 64, 65, 255, 256, 257, 511, 512, 513])
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 7, 8, 9, 13, 15, 16, 17, 63, 64, 65, 255, 256, 257, 511, 512, 513])
 def test_short_rows_one_lane_group_per_row(hip_backend, oracle_backend, n):
-    """Rows of up to 512 elements along a unit-stride axis are scanned by a group of 16 or 64
-    lanes each.  Every size class; all four scans; exclusive and reversed; integer results are
+    """Rows of up to 512 elements along a unit-stride axis are scanned by a group of 1, 4, 16 or
+    64 lanes each.  Every size class; all four scans; exclusive and reversed; integer results are
     exact, floating ones within the usual bound of the fp64 evaluation."""
-    m = 37
+    m = 37 if n > 16 else 1037                       # several workgroups of thread- and quad-sized groups
     xi = randint(220 + n, m * n, -9, 10).astype(np.int32).reshape(m, n)
     Xi = Tensor.from_numpy(hip_backend, xi)
     for exclusive in (False, True):

@@ -95,11 +95,12 @@ def test_hardmax_of_integer_rows(hip_backend, oracle_backend, dtype, n):
         F.softmax(Tensor.from_numpy(hip_backend, x), 1)
 
 
-@pytest.mark.parametrize("n", [1, 2, 3, 15, 16, 17, 31, 32, 33, 63, 64, 65, 4095, 4096, 4097])
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8, 10, 15, 16, 17, 31, 32, 33, 63, 64, 65, 4095, 4096, 4097])
 def test_row_lengths_around_the_team_sizes(hip_backend, oracle_backend, n):
-    """Sixteen lanes per row up to 64 (fp32) / 32 (fp64) / 128 (half) elements, a wavefront up to
+    """One lane per row up to 4 (fp32) / 2 (fp64) / 8 (half) elements, four lanes up to four times
+    that, sixteen lanes per row up to 64 (fp32) / 32 (fp64) / 128 (half) elements, a wavefront up to
     2048, a workgroup of 1024 threads with 4 elements each up to 4096: the boundaries of each."""
-    m = 70 if n < 1000 else 9
+    m = 700 if n <= 16 else 70 if n < 1000 else 9     # several workgroups of one- and four-lane teams
     for dtype in (np.float32, np.float64, np.float16):
         x = (normal(230 + n, m * n) * 2).astype(dtype).reshape(m, n)
         x[1] = x[1, 0]                                   # a constant row

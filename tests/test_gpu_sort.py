@@ -183,7 +183,7 @@ def test_nans_take_the_place_of_their_bit_pattern(hip_backend, dtype):
     assert (np.diff(idx[:, :200], axis=1) > 0).all()                                # equal keys keep their order
 
 
-@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 100, 127, 128, 129, 255, 256, 257, 300, 511, 512, 513, 1023, 1024, 1025, 2047, 2048, 2049, 4095,
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8, 9, 16, 17, 32, 33, 63, 64, 65, 100, 127, 128, 129, 255, 256, 257, 300, 511, 512, 513, 1023, 1024, 1025, 2047, 2048, 2049, 4095,
                                4096, 4097])
 def test_rows_around_the_one_workgroup_limits(hip_backend, oracle_backend, n):
     """Rows of up to 64, 128, 256 (512 for values only or 8-byte keys) elements are sorted by one
