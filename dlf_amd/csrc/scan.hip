@@ -360,7 +360,7 @@ __global__ __launch_bounds__(kBlock) void scan_rows_single(
     scan_tile<T, K, ITEMS, false, false, kBlock, X, NZ, Y>(x, y, xmap, ymap, sx, sy, xaxis, n, 1, exclusive, blockIdx.x, 0, 0, st, sm);
 }
 
-// Short rows: LANES lanes per row (a DPP row of 16 lanes, or a whole wavefront), ITEMS elements
+// Short rows: LANES lanes per row (one lane, a quad, a DPP row of 16 lanes, or a whole wavefront), ITEMS elements
 // per lane in vectors of V, no workgroup barrier and no LDS; a 256-thread workgroup takes
 // 256 / LANES rows.  Element (v * LANES + l) * V + j is item (v, j) of lane l of the group.
 template <typename T, int K, int LANES, int ITEMS, typename X, bool NZ, typename Y>

@@ -55,11 +55,11 @@ __device__ __forceinline__ MaxAt<T> max_at_join(MaxAt<T> a, MaxAt<T> b) {
     return take_b ? b : a;
 }
 
-// Reduction over the TEAM threads that share a row (a wavefront, or a whole workgroup through
+// Reduction over the TEAM threads that share a row (part of a wavefront, one, or a whole workgroup through
 // LDS); every thread receives the result.  `slot` separates the teams of a workgroup.
 template <int TEAM, typename V, typename Join>
 __device__ __forceinline__ V team_reduce(V v, Join join, V* lds) {
-    if constexpr (TEAM < kWave) v = group_reduce(v, TEAM, join);      // a DPP row of 16 lanes
+    if constexpr (TEAM < kWave) v = group_reduce(v, TEAM, join);      // one lane, a quad, or a DPP row of 16 lanes
     else v = wave_reduce(v, join);
     if constexpr (TEAM > kWave) {
         constexpr int WAVES = TEAM / kWave;
