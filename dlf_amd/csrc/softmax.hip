@@ -215,8 +215,131 @@ __global__ __launch_bounds__(1024) void softmax_rows_streamed(const S* __restric
     }
 }
 
+// Few long rows: a row is cut into tiles so that the whole device works on it.  A first kernel
+// leaves one record per tile in scratch, a second one folds a row's records (every workgroup of
+// the row does, they are few) and writes its own tile.  A workgroup only ever writes the tile
+// it read, and what the second kernel needs from other places of the row (the first element,
+// for the NaN rule) travels in the records, so y may be x.
+template <typename T>
+struct SoftPartial {
+    T mx, sum, first;          // soft kinds: running maximum, sum of exp(x - mx), the row's first element (tile 0)
+    MaxAt<T> best;             // hardmax
+};
+
+struct SplitPlan {
+    int64_t tiles, tile_len;
+};
+
+// about 2048 workgroups in all, tiles of at least 8192 elements
+inline SplitPlan split_plan(int64_t m, int64_t n) {
+    int64_t tiles = ceil_div(2048, m);
+    const int64_t most = ceil_div(n, 8192);
+    if (tiles > most) tiles = most;
+    if (tiles < 1) tiles = 1;
+    SplitPlan p;
+    p.tile_len = ceil_div(n, tiles);
+    p.tiles = ceil_div(n, p.tile_len);
+    return p;
+}
+
+template <typename S, int KIND>
+__global__ __launch_bounds__(1024) void softmax_split_partials(const S* __restrict__ x, int64_t n, int64_t tiles, int64_t tile_len,
+                                                               SoftPartial<typename ComputeOf<S>::type>* __restrict__ part) {
+    using T = typename ComputeOf<S>::type;
+    constexpr int TEAM = 1024;
+    __shared__ alignas(16) unsigned char lds_raw[(TEAM / kWave) * sizeof(MaxAt<T>)];
+    const int t = threadIdx.x;
+    const int64_t row = blockIdx.x / tiles, tile = blockIdx.x - row * tiles;
+    const S* xr = x + row * n;
+    const int64_t i0 = tile * tile_len, i1 = i0 + tile_len < n ? i0 + tile_len : n;
+    const T lowest = std::is_integral<T>::value ? std::numeric_limits<T>::lowest() : -std::numeric_limits<T>::infinity();
+    SoftPartial<T> out;
+    out.mx = lowest;
+    out.sum = T(0);
+    out.first = static_cast<T>(xr[0]);
+    out.best = {lowest, std::numeric_limits<int32_t>::max()};
+    if constexpr (KIND == kHardmax) {
+        MaxAt<T> best = out.best;
+        for (int64_t i = i0 + t; i < i1; i += TEAM) best = max_at_join(best, max_at_of(static_cast<T>(xr[i]), i));
+        out.best = team_reduce<TEAM>(best, [](MaxAt<T> a, MaxAt<T> b) { return max_at_join(a, b); },
+                                     reinterpret_cast<MaxAt<T>*>(lds_raw));
+    } else {
+        T mx = lowest, sum = T(0);
+        for (int64_t i = i0 + t; i < i1; i += TEAM) {
+            const T xv = static_cast<T>(xr[i]);
+            if (mx < xv) {
+                sum = sum * exp_of<T>(mx - xv);
+                mx = xv;
+            }
+            if (xv != lowest || mx != lowest) sum += exp_of<T>(xv - mx);
+        }
+        const T tile_max = team_reduce<TEAM>(mx, [](T a, T b) { return (a < b) ? b : a; }, reinterpret_cast<T*>(lds_raw));
+        sum = (mx == lowest) ? T(0) : sum * exp_of<T>(mx - tile_max);
+        out.mx = tile_max;
+        out.sum = team_reduce<TEAM>(sum, [](T a, T b) { return a + b; }, reinterpret_cast<T*>(lds_raw));
+    }
+    if (t == 0) part[blockIdx.x] = out;
+}
+
+template <typename S, int KIND>
+__global__ __launch_bounds__(1024) void softmax_split_apply(const S* __restrict__ x, S* __restrict__ y, int64_t n, int64_t tiles,
+                                                            int64_t tile_len,
+                                                            const SoftPartial<typename ComputeOf<S>::type>* __restrict__ part) {
+    using T = typename ComputeOf<S>::type;
+    constexpr int TEAM = 1024;
+    __shared__ alignas(16) unsigned char lds_raw[(TEAM / kWave) * sizeof(MaxAt<T>)];
+    const int t = threadIdx.x;
+    const int64_t row = blockIdx.x / tiles, tile = blockIdx.x - row * tiles;
+    const S* xr = x + row * n;
+    S* yr = y + row * n;
+    const SoftPartial<T>* pr = part + row * tiles;
+    const int64_t i0 = tile * tile_len, i1 = i0 + tile_len < n ? i0 + tile_len : n;
+    const T lowest = std::is_integral<T>::value ? std::numeric_limits<T>::lowest() : -std::numeric_limits<T>::infinity();
+    if constexpr (KIND == kHardmax) {
+        MaxAt<T> best = {lowest, std::numeric_limits<int32_t>::max()};
+        for (int64_t p = t; p < tiles; p += TEAM) best = max_at_join(best, pr[p].best);
+        best = team_reduce<TEAM>(best, [](MaxAt<T> a, MaxAt<T> b) { return max_at_join(a, b); },
+                                 reinterpret_cast<MaxAt<T>*>(lds_raw));
+        const int64_t hot = best.i < 0 ? 0 : best.i;
+        for (int64_t i = i0 + t; i < i1; i += TEAM) yr[i] = i == hot ? S(1) : S(0);
+    } else {
+        T mx = lowest, sum = T(0);
+        for (int64_t p = t; p < tiles; p += TEAM) {
+            const T pm = pr[p].mx, ps = pr[p].sum;
+            if (mx < pm) {
+                sum = sum * exp_of<T>(mx - pm);
+                mx = pm;
+            }
+            if (pm != lowest) sum += ps * exp_of<T>(pm - mx);
+        }
+        T row_max = team_reduce<TEAM>(mx, [](T a, T b) { return (a < b) ? b : a; }, reinterpret_cast<T*>(lds_raw));
+        sum = (mx == lowest) ? T(0) : sum * exp_of<T>(mx - row_max);
+        const T first = pr[0].first;
+        if (first != first) row_max = first;                      // a NaN in position 0 is the reference's maximum
+        sum = team_reduce<TEAM>(sum, [](T a, T b) { return a + b; }, reinterpret_cast<T*>(lds_raw));
+        const T lsum = log_of<T>(sum);
+        for (int64_t i = i0 + t; i < i1; i += TEAM) {
+            const T xv = static_cast<T>(xr[i]);
+            yr[i] = static_cast<S>(KIND == kSoftmax ? exp_of<T>(xv - row_max) / sum : (xv - row_max) - lsum);
+        }
+    }
+}
+
+// rows at most this long are held in registers by one workgroup
+template <typename T>
+constexpr int64_t register_row_limit() { return sizeof(typename ComputeOf<T>::type) == 4 ? 1024 * 32 : 1024 * 16; }
+constexpr int64_t kSplitMaxRows = 512;        // from this many rows on, a workgroup per row fills the device
+
+template <typename T>
+size_t split_scratch_bytes(int64_t m, int64_t n) {
+    if (n <= register_row_limit<T>() || m >= kSplitMaxRows) return 0;
+    const SplitPlan p = split_plan(m, n);
+    if (p.tiles < 2) return 0;
+    return static_cast<size_t>(m * p.tiles) * sizeof(SoftPartial<typename ComputeOf<T>::type>);
+}
+
 template <typename T, int KIND>
-int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y) {
+int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y, void* scratch, size_t scratch_bytes) {
     constexpr int V = 16 / static_cast<int>(sizeof(T));
     constexpr int kRegisterBytes = static_cast<int>(sizeof(typename ComputeOf<T>::type));
     const bool vec = n % V == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
@@ -262,6 +385,17 @@ int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y) {
     if (n <= 1024 * 32 && kRegisterBytes == 4) DLFX_BLOCK_ROWS(32);
 #undef DLFX_WAVE_ROWS
 #undef DLFX_BLOCK_ROWS
+    const size_t need = split_scratch_bytes<T>(m, n);
+    if (need && scratch && scratch_bytes >= need && reinterpret_cast<uintptr_t>(scratch) % 16 == 0) {
+        using P = SoftPartial<typename ComputeOf<T>::type>;
+        const SplitPlan p = split_plan(m, n);
+        const dim3 grid(static_cast<unsigned>(m * p.tiles));
+        softmax_split_partials<T, KIND><<<grid, dim3(1024), 0, stream>>>(x, n, p.tiles, p.tile_len, static_cast<P*>(scratch));
+        DLFX_CHECK_LAUNCH();
+        softmax_split_apply<T, KIND><<<grid, dim3(1024), 0, stream>>>(x, y, n, p.tiles, p.tile_len, static_cast<const P*>(scratch));
+        DLFX_CHECK_LAUNCH();
+        return DLFX_OK;
+    }
     softmax_rows_streamed<T, KIND><<<dim3(static_cast<unsigned>(m)), dim3(1024), 0, stream>>>(x, y, n);
     DLFX_CHECK_LAUNCH();
     return DLFX_OK;
@@ -272,8 +406,21 @@ int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y) {
 
 using namespace dlfx;
 
+extern "C" size_t dlfx_softmax_scratch_bytes(int dtype, int64_t m, int64_t n) {
+    if (m <= 0 || n <= 0 || m > 0x7fffffffLL || n > 0x7fffffffLL) return 0;
+    switch (dtype) {
+    case DLFX_F32: return split_scratch_bytes<float>(m, n);
+    case DLFX_F64: return split_scratch_bytes<double>(m, n);
+    case DLFX_F16: return split_scratch_bytes<half_t>(m, n);
+    case DLFX_I32: return split_scratch_bytes<int32_t>(m, n);
+    case DLFX_I64: return split_scratch_bytes<int64_t>(m, n);
+    default: return 0;
+    }
+}
+
 extern "C" int dlfx_softmax(dlfx_stream_t stream, const char* name, int dtype, int64_t m, int64_t n,
-                            const void* x, int64_t x_offset, void* y, int64_t y_offset) {
+                            const void* x, int64_t x_offset, void* y, int64_t y_offset,
+                            void* scratch, size_t scratch_bytes) {
     if (!name || !x || !y || m <= 0 || n <= 0) return DLFX_ERR_INVALID_ARGUMENT;
     if (m > 0x7fffffffLL || n > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
     int kind;
@@ -290,10 +437,10 @@ extern "C" int dlfx_softmax(dlfx_stream_t stream, const char* name, int dtype, i
         const T* xp = static_cast<const T*>(x) + x_offset;
         T* yp = static_cast<T*>(y) + y_offset;
         if constexpr (!std::is_integral<T>::value) {
-            if (kind == kSoftmax) return launch_softmax<T, kSoftmax>(s, m, n, xp, yp);
-            if (kind == kLogSoftmax) return launch_softmax<T, kLogSoftmax>(s, m, n, xp, yp);
+            if (kind == kSoftmax) return launch_softmax<T, kSoftmax>(s, m, n, xp, yp, scratch, scratch_bytes);
+            if (kind == kLogSoftmax) return launch_softmax<T, kLogSoftmax>(s, m, n, xp, yp, scratch, scratch_bytes);
         }
-        return launch_softmax<T, kHardmax>(s, m, n, xp, yp);
+        return launch_softmax<T, kHardmax>(s, m, n, xp, yp, scratch, scratch_bytes);
     };
     switch (dtype) {
     case DLFX_F32: return run(float());

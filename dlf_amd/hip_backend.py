@@ -82,7 +82,9 @@ def _declare(lib):
                                       c_void_p, c_int64, _I64P, c_void_p, c_int64, _I64P, c_void_p, c_size_t]
 
     lib.dlfx_softmax.restype = c_int
-    lib.dlfx_softmax.argtypes = [c_void_p, c_char_p, c_int, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64]
+    lib.dlfx_softmax.argtypes = [c_void_p, c_char_p, c_int, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_size_t]
+    lib.dlfx_softmax_scratch_bytes.restype = c_size_t
+    lib.dlfx_softmax_scratch_bytes.argtypes = [c_int, c_int64, c_int64]
 
     lib.dlfx_merge_scratch_bytes.restype = c_size_t
     lib.dlfx_merge_scratch_bytes.argtypes = [c_int, c_int64, c_int64]
@@ -108,7 +110,7 @@ EXPORTS = ("dlfx_version", "dlfx_status_string", "dlfx_last_hip_error", "dlfx_se
            "dlfx_top_k_scratch_bytes", "dlfx_top_k",
            "dlfx_count_scratch_bytes", "dlfx_count",
            "dlfx_scan_nonzero_scratch_bytes", "dlfx_scan_nonzero", "dlfx_gather_indices",
-           "dlfx_merge_scratch_bytes", "dlfx_merge", "dlfx_softmax")
+           "dlfx_merge_scratch_bytes", "dlfx_merge", "dlfx_softmax_scratch_bytes", "dlfx_softmax")
 
 
 def load_library():
@@ -284,8 +286,9 @@ class HipBackend:
                            (len(dims), _arr(dims), counts.data_ptr(), 0, out.data_ptr(), 0), defer, (counts, out))
 
     def softmax(self, name, dtype, m, n, x, x_offset, y, y_offset, defer=False):
+        sp, sb = self.scratch(self.lib.dlfx_softmax_scratch_bytes(dtype, m, n))
         return self._issue(self.lib.dlfx_softmax, "dlfx_softmax(%s)" % name, (name.encode(), dtype, m, n),
-                           (x.data_ptr(), x_offset, y.data_ptr(), y_offset), defer, (x, y))
+                           (x.data_ptr(), x_offset, y.data_ptr(), y_offset, sp, sb), defer, (x, y))
 
     def merge(self, direction, dtype, xs, x, ys, y, zs, z, defer=False):
         n = zs.extents[-1]

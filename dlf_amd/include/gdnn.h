@@ -188,8 +188,10 @@ template <typename T>
 void softmax_family(const char* name, const size_t m, const size_t n, Buffer<T>& x_buffer, const size_t x_offset,
                     const Queue& queue, Event* event) {
     EventScope ev(queue, event);
-    check_status(dlfx_softmax(queue.stream(), name, dtype_of<T>::value, m, n, x_buffer.data(), x_offset,
-                              x_buffer.data(), x_offset), name);
+    const int dt = dtype_of<T>::value;
+    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_softmax_scratch_bytes(dt, m, n));      // only few, long rows need any
+    check_status(dlfx_softmax(queue.stream(), name, dt, m, n, x_buffer.data(), x_offset,
+                              x_buffer.data(), x_offset, tmp.data(), tmp.size()), name);
     ev.done();
 }
 }  // namespace detail

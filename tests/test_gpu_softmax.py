@@ -118,3 +118,56 @@ def test_row_lengths_around_the_team_sizes(hip_backend, oracle_backend, n):
         want = sp_log_softmax(x64, axis=1)
         assert (np.abs(got - want) <= slack * (1 + np.abs(want)) + out_ulp * np.abs(want)).all(), dtype
         assert np.array_equal(F.hardmax(Xh).numpy(), F.hardmax(Xo).numpy()), dtype
+
+
+@pytest.mark.parametrize("m,n,dtype", [(1, 200000, np.float32), (3, 70001, np.float32), (7, 40000, np.float64), (2, 32769, np.float32),
+                                       (5, 16385, np.float64), (2, 100000, np.float16), (300, 33000, np.float32)])
+def test_few_long_rows_are_cut_into_tiles(hip_backend, oracle_backend, m, n, dtype):
+    """Fewer than 512 rows that are too long for one workgroup's registers: every row is cut
+    into tiles that the whole device works on (two kernels, one record per tile in scratch).
+    All three kinds, in place and out of place, a NaN in position 0 and elsewhere, -inf entries,
+    an all -inf row, and the same call without scratch (one workgroup per row)."""
+    import ctypes
+    x = (normal(260 + n, m * n) * 3).astype(dtype).reshape(m, n)
+    x[0, n // 3] = -np.inf
+    if m > 1:
+        x[1, 0] = np.nan                                 # the reference's maximum: the whole row becomes NaN
+    if m > 2:
+        x[2, n - 5] = np.nan                             # poisons the sum, not the maximum
+    if m > 4:
+        x[4] = -np.inf
+    Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
+    eps = float(np.finfo(np.float32 if dtype == np.float16 else dtype).eps)
+    out_ulp = 2.0 ** -10 if dtype == np.float16 else 0.0
+    slack = 8 * np.log2(n) * eps + out_ulp
+    clean = [r for r in range(m) if r not in (1, 2, 4)]
+    x64 = x[clean].astype(np.float64)
+    results = {}
+    for name, fn, want in (("softmax", F.softmax, sp_softmax(x64, axis=1)), ("logsoftmax", F.logsoftmax, sp_log_softmax(x64, axis=1))):
+        got = fn(Xh).numpy().astype(np.float64)
+        results[name] = got
+        if name == "softmax":
+            assert (np.abs(got[clean] - want) <= want * slack + 1e-30 + (2.0 ** -24 if dtype == np.float16 else 0)).all()
+        else:
+            fin = np.isfinite(want)
+            assert (np.abs(got[clean][fin] - want[fin]) <= slack * (1 + np.abs(want[fin])) + out_ulp * np.abs(want[fin])).all()
+            assert (got[clean][~fin] == -np.inf).all()
+        ref = fn(Xo).numpy().astype(np.float64)
+        for r in (1, 2, 4):                              # NaN rows and the all -inf row: the same non-finite pattern as the reference's loop
+            if r < m:
+                assert np.array_equal(np.isnan(got[r]), np.isnan(ref[r])), (name, r)
+    assert np.array_equal(F.hardmax(Xh).numpy(), F.hardmax(Xo).numpy())
+    # in place (the reference's calling convention)
+    Z = Tensor.from_numpy(hip_backend, x)
+    hip_backend.softmax("softmax", F.dtype_code(Z.dtype), m, n, Z.storage, 0, Z.storage, 0)
+    assert np.array_equal(np.nan_to_num(Z.numpy().astype(np.float64), nan=-7.0), np.nan_to_num(results["softmax"], nan=-7.0))
+    # no scratch given: one workgroup per row, the same values up to the order of the sums
+    lib = hip_backend.lib
+    assert lib.dlfx_softmax_scratch_bytes(F.dtype_code(x.dtype), m, n) > 0
+    Y = Tensor.empty(hip_backend, [m, n], x.dtype)
+    import torch
+    st = lib.dlfx_softmax(torch.cuda.current_stream().cuda_stream, b"softmax", F.dtype_code(x.dtype), m, n,
+                          Xh.storage.data_ptr(), 0, Y.storage.data_ptr(), 0, None, 0)
+    assert st == 0
+    a, b = Y.numpy().astype(np.float64)[clean], results["softmax"][clean]
+    assert (np.abs(a - b) <= b * 2 * slack + 1e-30 + (2.0 ** -23 if dtype == np.float16 else 0)).all()
