@@ -96,6 +96,9 @@ struct TopkIo {
     DimMap imap;
     int64_t si;
     int idx64, kind, largest;
+    // segmented rows (first stage of long rows): row r of the launch is segment r % segs of a
+    // longer row; the last segment of each has last_n elements instead of n.  0 or 1: plain rows.
+    int64_t segs, last_n;
 };
 
 constexpr int kCandCap = 4096;     // candidates kept after the pre-filter (4-byte keys; half for 8-byte keys)
@@ -943,6 +946,7 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
     const int lane = lane_id();
     const int w = tid / kWave;
     const int64_t row = blockIdx.x;
+    if (io.segs > 1 && row % io.segs == io.segs - 1) n = io.last_n;
     const S* xr = io.x + io.xmap.at(row);
     if (tid < kRadix) sm.hist[tid] = 0;
     DLFX_PHASE_BEGIN();
@@ -1147,6 +1151,7 @@ __global__ __launch_bounds__(kSelectThreads) void topk_finish(
     const int64_t row = blockIdx.x;
     const uint32_t state = row_state[row];
     if (state == kRowDone) return;
+    if (io.segs > 1 && row % io.segs == io.segs - 1) n = io.last_n;
     const S* xr = io.x + io.xmap.at(row);
     if (tid < kRadix) sm.hist[tid] = 0;
     if (state != kRowWhole) {
@@ -1220,6 +1225,111 @@ bool selection_fits(size_t key_size, int64_t n, int64_t limit) {
     return n <= (key_size == 4 ? 65536 : 32768);
 }
 
+// The selection kernels over `m` rows of `n` elements (n within selection_fits).
+template <typename T>
+int launch_select(hipStream_t stream, const TopkIo<typename BitsOf<T>::type, typename BitsOf<T>::storage>& io, int64_t m, int64_t n,
+                  int64_t limit, void* scratch, size_t scratch_bytes) {
+    using K = typename BitsOf<T>::type;
+    using S = typename BitsOf<T>::storage;
+    const dim3 grid(static_cast<unsigned>(m));
+    const int lim = static_cast<int>(limit);
+    bool aligned = io.sx == 1 && reinterpret_cast<uintptr_t>(io.x) % 16 == 0;
+    for (int i = 0; i < io.xmap.rank; ++i) aligned = aligned && io.xmap.strides[i] % (16 / static_cast<int64_t>(sizeof(S))) == 0;
+    const SelectLayout sl = select_layout(sizeof(K), m, n);
+    if (sl.total && (!scratch || scratch_bytes < sl.total)) return DLFX_ERR_SCRATCH_TOO_SMALL;
+    char* sbase = static_cast<char*>(scratch);
+    uint32_t* row_state = reinterpret_cast<uint32_t*>(sbase + sl.state_off);
+    K* spill_ord = reinterpret_cast<K*>(sbase + sl.ord_off);
+    uint32_t* spill_idx = reinterpret_cast<uint32_t*>(sbase + sl.idx_off);
+    if (n <= kWaveRowMax && (lim <= kWaveRowLimit || n <= kWaveSortItems * kWave)) {      // at most 256 elements: a wave can order the whole row, whatever the limit
+        const dim3 wgrid(static_cast<unsigned>(ceil_div(m, 4)));
+#define DLFX_TOPK_WAVE(ITEMS) topk_rows_wave<T, ITEMS><<<wgrid, dim3(256), 0, stream>>>(io, m, n, lim)
+        if (n <= 64) DLFX_TOPK_WAVE(1);
+        else if (n <= 128) DLFX_TOPK_WAVE(2);
+        else if (n <= 256) DLFX_TOPK_WAVE(4);
+        else if (n <= 512) DLFX_TOPK_WAVE(8);
+        else if (n <= 1024) DLFX_TOPK_WAVE(16);
+        else if (n <= 2048) DLFX_TOPK_WAVE(32);
+        else DLFX_TOPK_WAVE(64);
+#undef DLFX_TOPK_WAVE
+        DLFX_CHECK_LAUNCH();
+        return DLFX_OK;
+    }
+#define DLFX_TOPK(BLOCK, ITEMS)                                                                     \
+do {                                                                                            \
+    if (aligned) topk_select<T, BLOCK, ITEMS, true><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx); \
+    else topk_select<T, BLOCK, ITEMS, false><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx);      \
+} while (0)
+    if (n <= 256) DLFX_TOPK(256, 1);
+    else if (n <= 1024) DLFX_TOPK(256, 4);
+    else if (n <= 2048) DLFX_TOPK(1024, 2);
+    else if (n <= 4096) DLFX_TOPK(1024, 4);
+    else if (n <= 8192) DLFX_TOPK(1024, 8);
+    else if (n <= 16384) DLFX_TOPK(1024, 16);
+    else if (n <= 32768) {
+        DLFX_TOPK(1024, 32);
+    } else {
+        if constexpr (sizeof(K) == 4) DLFX_TOPK(1024, 64);
+        else return DLFX_ERR_TOO_LARGE;
+    }
+#undef DLFX_TOPK
+    DLFX_CHECK_LAUNCH();
+    if (n > cand_cap<K>()) {
+        topk_finish<T><<<grid, dim3(kSelectThreads), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx);
+        DLFX_CHECK_LAUNCH();
+    }
+    return DLFX_OK;
+}
+
+// ---------------------------------------------------------------- rows longer than the selection kernel takes
+// A long row is cut into segments the selection kernel takes (a launch of m * segs "rows"); each
+// leaves its `limit` best as (value, index within the segment) in scratch, ordered, so that
+// among equal values a lower place in the candidate array means a lower index in the row.
+// top_k of the m rows of segs * limit candidates (this routine again) then yields the values
+// and the places of the winners, and topk_places_to_indices turns places into row indices.
+struct LongPlan {
+    bool ok;
+    int64_t seg_len, segs, last_n;
+    size_t val_off, idx_off, pos_off, rest_off, total;
+};
+
+size_t top_k_scratch_impl(int dtype, int64_t m, int64_t n, int64_t limit);
+
+LongPlan long_plan(int dtype, size_t elem_size, size_t key_size, int64_t m, int64_t n, int64_t limit) {
+    LongPlan p{};
+    const int64_t cap = key_size == 4 ? 65536 : 32768;
+    if (n <= cap || limit > kMaxLimit) return p;
+    int64_t segs = ceil_div(n, cap);
+    p.seg_len = align_up(static_cast<size_t>(ceil_div(n, segs)), 8);      // segments start on 16-byte boundaries when the row does
+    p.segs = ceil_div(n, p.seg_len);
+    p.last_n = n - (p.segs - 1) * p.seg_len;
+    if (p.segs < 2 || p.last_n < limit || p.segs * limit > n / 2 || m * p.segs > 0x7fffffffLL) return p;
+    const size_t cands = static_cast<size_t>(m) * p.segs * limit;
+    p.val_off = 0;
+    p.idx_off = align_up(cands * elem_size, 256);
+    p.pos_off = p.idx_off + align_up(cands * 4, 256);
+    p.rest_off = p.pos_off + align_up(static_cast<size_t>(m) * limit * 4, 256);
+    const size_t first = select_layout(key_size, m * p.segs, p.seg_len).total;
+    const size_t second = top_k_scratch_impl(dtype, m, p.segs * limit, limit);
+    p.total = p.rest_off + (first > second ? first : second);
+    p.ok = true;
+    return p;
+}
+
+__global__ __launch_bounds__(256) void topk_places_to_indices(const int32_t* __restrict__ place, const uint32_t* __restrict__ cand_idx,
+                                                              int64_t rows, int limit, int64_t segs, int64_t seg_len,
+                                                              void* idx, DimMap imap, int64_t si, int idx64) {
+    const int64_t g = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (g >= rows * limit) return;
+    const int64_t row = g / limit;
+    const int j = static_cast<int>(g - row * limit);
+    const int64_t p = place[g];
+    const int64_t ix = (p / limit) * seg_len + cand_idx[row * segs * limit + p];
+    const int64_t at = imap.at(row) + j * si;
+    if (idx64) static_cast<int64_t*>(idx)[at] = ix;
+    else static_cast<int32_t*>(idx)[at] = static_cast<int32_t>(ix);
+}
+
 template <typename T>
 int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_dtype,
               int rank, const int64_t* x_dims, const int64_t* y_dims,
@@ -1289,54 +1399,49 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
         return DLFX_OK;
     }
 
-    if (selection_fits(sizeof(K), n, limit)) {
-        const dim3 grid(static_cast<unsigned>(m));
+    if (selection_fits(sizeof(K), n, limit)) return launch_select<T>(stream, io, m, n, limit, scratch, scratch_bytes);
+
+    // rows too long for the selection kernel: select within segments, then among their winners
+    const LongPlan lp = long_plan(dtype, sizeof(S), sizeof(K), m, n, limit);
+    if (lp.ok && io.xmap.rank < kMaxRank) {
+        if (!scratch || scratch_bytes < lp.total) return DLFX_ERR_SCRATCH_TOO_SMALL;
         const int lim = static_cast<int>(limit);
-        bool aligned = io.sx == 1 && reinterpret_cast<uintptr_t>(io.x) % 16 == 0;
-        for (int i = 0; i < io.xmap.rank; ++i) aligned = aligned && io.xmap.strides[i] % (16 / static_cast<int64_t>(sizeof(S))) == 0;
-        const SelectLayout sl = select_layout(sizeof(K), m, n);
-        if (sl.total && (!scratch || scratch_bytes < sl.total)) return DLFX_ERR_SCRATCH_TOO_SMALL;
-        char* sbase = static_cast<char*>(scratch);
-        uint32_t* row_state = reinterpret_cast<uint32_t*>(sbase + sl.state_off);
-        K* spill_ord = reinterpret_cast<K*>(sbase + sl.ord_off);
-        uint32_t* spill_idx = reinterpret_cast<uint32_t*>(sbase + sl.idx_off);
-        if (n <= kWaveRowMax && (lim <= kWaveRowLimit || n <= kWaveSortItems * kWave)) {      // at most 256 elements: a wave can order the whole row, whatever the limit
-            const dim3 wgrid(static_cast<unsigned>(ceil_div(m, 4)));
-#define DLFX_TOPK_WAVE(ITEMS) topk_rows_wave<T, ITEMS><<<wgrid, dim3(256), 0, stream>>>(io, m, n, lim)
-            if (n <= 64) DLFX_TOPK_WAVE(1);
-            else if (n <= 128) DLFX_TOPK_WAVE(2);
-            else if (n <= 256) DLFX_TOPK_WAVE(4);
-            else if (n <= 512) DLFX_TOPK_WAVE(8);
-            else if (n <= 1024) DLFX_TOPK_WAVE(16);
-            else if (n <= 2048) DLFX_TOPK_WAVE(32);
-            else DLFX_TOPK_WAVE(64);
-#undef DLFX_TOPK_WAVE
-            DLFX_CHECK_LAUNCH();
-            return DLFX_OK;
+        char* base = static_cast<char*>(scratch);
+        S* cand_val = reinterpret_cast<S*>(base + lp.val_off);
+        uint32_t* cand_idx = reinterpret_cast<uint32_t*>(base + lp.idx_off);
+        int32_t* place = reinterpret_cast<int32_t*>(base + lp.pos_off);
+        TopkIo<K, S> io1 = io;
+        io1.xmap.dims[io1.xmap.rank] = lp.segs;                    // innermost: row r of the launch is segment r % segs
+        io1.xmap.strides[io1.xmap.rank] = lp.seg_len * io.sx;
+        io1.xmap.rank += 1;
+        io1.y = cand_val;
+        io1.idx = cand_idx;
+        io1.ymap.rank = io1.imap.rank = 1;
+        io1.ymap.dims[0] = io1.imap.dims[0] = m * lp.segs;
+        io1.ymap.strides[0] = io1.imap.strides[0] = limit;
+        io1.sy = io1.si = 1;
+        io1.idx64 = 0;
+        io1.segs = lp.segs;
+        io1.last_n = lp.last_n;
+        int st = launch_select<T>(stream, io1, m * lp.segs, lp.seg_len, limit, base + lp.rest_off, scratch_bytes - lp.rest_off);
+        if (st != DLFX_OK) return st;
+        int64_t c_dims[64], c_strides[64], p_strides[64];
+        for (int i = 0; i < rank; ++i) c_dims[i] = x_dims[i];
+        c_dims[rank - 1] = lp.segs * limit;
+        int64_t cs = 1, ps = 1;
+        for (int i = rank - 1; i >= 0; --i) {
+            c_strides[i] = cs;
+            cs *= c_dims[i];
+            p_strides[i] = ps;
+            ps *= y_dims[i];
         }
-#define DLFX_TOPK(BLOCK, ITEMS)                                                                     \
-    do {                                                                                            \
-        if (aligned) topk_select<T, BLOCK, ITEMS, true><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx); \
-        else topk_select<T, BLOCK, ITEMS, false><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx);      \
-    } while (0)
-        if (n <= 256) DLFX_TOPK(256, 1);
-        else if (n <= 1024) DLFX_TOPK(256, 4);
-        else if (n <= 2048) DLFX_TOPK(1024, 2);
-        else if (n <= 4096) DLFX_TOPK(1024, 4);
-        else if (n <= 8192) DLFX_TOPK(1024, 8);
-        else if (n <= 16384) DLFX_TOPK(1024, 16);
-        else if (n <= 32768) {
-            DLFX_TOPK(1024, 32);
-        } else {
-            if constexpr (sizeof(K) == 4) DLFX_TOPK(1024, 64);
-            else return DLFX_ERR_TOO_LARGE;
-        }
-#undef DLFX_TOPK
+        st = run_top_k<T>(stream, limit, dir, dtype, DLFX_I32, rank, c_dims, y_dims, cand_val, c_strides, y, ys, place, p_strides,
+                          base + lp.rest_off, scratch_bytes - lp.rest_off);
+        if (st != DLFX_OK) return st;
+        const int64_t outs = m * limit;
+        topk_places_to_indices<<<dim3(static_cast<unsigned>(ceil_div(outs, 256))), dim3(256), 0, stream>>>(
+            place, cand_idx, m, lim, lp.segs, lp.seg_len, idx, io.imap, io.si, io.idx64);
         DLFX_CHECK_LAUNCH();
-        if (n > cand_cap<K>()) {
-            topk_finish<T><<<grid, dim3(kSelectThreads), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx);
-            DLFX_CHECK_LAUNCH();
-        }
         return DLFX_OK;
     }
 
@@ -1387,13 +1492,23 @@ extern "C" void dlfx_debug_topk_phases(unsigned long long* out, int reset) {
 }
 #endif
 
-extern "C" size_t dlfx_top_k_scratch_bytes(int dtype, int64_t m, int64_t n, int64_t limit) {
+namespace dlfx {
+namespace {
+size_t top_k_scratch_impl(int dtype, int64_t m, int64_t n, int64_t limit) {
     const size_t es = dtype_size(dtype);
     if (!es || dtype == DLFX_BOOL || m <= 0 || n <= 0) return 0;
     const size_t ks = es < 4 ? 4 : es;            // 16-bit elements are selected as 32-bit keys
     if (selection_fits(ks, n, limit)) return select_layout(ks, m, n).total;
+    const LongPlan lp = long_plan(dtype, es, ks, m, n, limit);
+    if (lp.ok) return lp.total;
     return align_up(static_cast<size_t>(m) * n * es, 256) + align_up(static_cast<size_t>(m) * n * 4, 256) +
            argsort_scratch_bytes_impl(dtype, m, n);
+}
+}  // namespace
+}  // namespace dlfx
+
+extern "C" size_t dlfx_top_k_scratch_bytes(int dtype, int64_t m, int64_t n, int64_t limit) {
+    return top_k_scratch_impl(dtype, m, n, limit);
 }
 
 extern "C" int dlfx_top_k(dlfx_stream_t stream, int64_t limit, int dir, int dtype, int index_dtype,

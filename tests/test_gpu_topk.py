@@ -253,3 +253,35 @@ def _many_short_rows(hip_backend, oracle_backend, n, dtypes=None):
         SV, SI = F.argsort(T, 1, True, with_values=True)
         assert Ih.numpy().dtype == np.int64 and np.array_equal(Ih.numpy(), SI.numpy()[:, :k])
         assert np.array_equal(Yh.numpy().view(np.uint32), SV.numpy()[:, :k].view(np.uint32))
+
+
+@pytest.mark.parametrize("shape,axis", [((1, 200000), 1), ((3, 70001), 1), ((2, 1 << 20), 1), ((70001, 3), 0), ((2, 65537), 1),
+                                        ((1, 5_000_000), 1)])
+def test_rows_longer_than_the_selection_kernel_takes(hip_backend, shape, axis):
+    """Rows of more than 65536 (8-byte keys: 32768) elements: selection within segments, then
+    among the segments' winners (and again, when those are still too many), places turned back
+    into row indices.  Ties across segment boundaries, every element type, both directions,
+    64-bit indices, a strided axis, NaNs by bit pattern."""
+    n = shape[axis]
+    x = quantised(270 + n, shape)                               # ties everywhere, also across segments
+    ks = (1, 5, 100, 1024) if n < 1_000_000 else (5, 1000)
+    for k in ks:
+        check(hip_backend, x, k, axis, True)
+    check(hip_backend, x, 7, axis, False, np.int64)
+    if n <= 200000:
+        for dtype in (np.int64, np.float64, np.float16, np.int16, np.int32):
+            xd = (normal(271 + n, int(np.prod(shape))) * 300).astype(dtype).reshape(shape)
+            check(hip_backend, xd, 33, axis, True)
+            check(hip_backend, xd, 2, axis, False)
+        xn = (normal(272 + n, int(np.prod(shape))) * 3).astype(np.float32).reshape(shape)
+        flat = np.moveaxis(xn, axis, -1)
+        flat[0, [3, n // 2, n - 1]] = np.nan
+        flat[0, 70000 if n > 70000 else 11] = np.inf
+        X = Tensor.from_numpy(hip_backend, xn)
+        for largest in (True, False):
+            Y, I = F.top_k(X, 6, axis, largest)
+            SV, SI = F.argsort(X, axis, largest, with_values=True)
+            take = [slice(None)] * 2
+            take[axis] = slice(0, 6)
+            assert np.array_equal(I.numpy(), SI.numpy()[tuple(take)]), largest
+            assert np.array_equal(Y.numpy().view(np.uint32), SV.numpy()[tuple(take)].view(np.uint32)), largest
