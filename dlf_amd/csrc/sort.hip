@@ -104,7 +104,17 @@ struct PassIo {
     int kind, descending;
     int canon_zero;           // argsort of floats: -0.0 and +0.0 are one key
     int restore_zero;         // ... and the value written for a zero key is re-read from x
+    // rows side by side in memory (the axis is an outer dimension): workgroups are dealt to the
+    // 8 XCDs in turn, so workgroup b takes block (b % 8) * xcd_blocks + b / 8 and neighbouring
+    // rows, which share cache lines, meet in one L2 (0: workgroup b takes block b)
+    int64_t xcd_blocks;
 };
+
+template <typename K>
+__device__ __forceinline__ int64_t block_of(const PassIo<K>& io) {
+    if (io.xcd_blocks == 0) return blockIdx.x;
+    return static_cast<int64_t>(blockIdx.x % 8) * io.xcd_blocks + blockIdx.x / 8;
+}
 
 template <typename K>
 __device__ __forceinline__ K key_of_element(const PassIo<K>& io, K bits) {
@@ -583,7 +593,7 @@ struct SmallShared {
 };
 
 template <typename K, bool PAIRS, int ITEMS>
-__global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t n) {
+__global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t rows, int64_t n) {
     constexpr int P = KeyTraits<K>::kPasses;
     constexpr int CAP = 256 * ITEMS;
     static_assert(ITEMS % 2 == 0, "items are ranked in pairs");
@@ -591,7 +601,8 @@ __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t n) 
     const int tid = threadIdx.x;
     const int lane = lane_id();
     const int w = tid / kWave;
-    const int64_t row = blockIdx.x;
+    const int64_t row = block_of(io);
+    if (row >= rows) return;                               // (the grid is rounded up to a multiple of 8)
     const K* xrow = io.x + io.xmap.at(row);
     const int valid = static_cast<int>(n);
     const bool padded = valid < CAP;
@@ -737,7 +748,7 @@ __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t n) 
 template <typename K, bool PAIRS, int WIDTH>
 __global__ __launch_bounds__(256) void sort_rows_wave(PassIo<K> io, int64_t rows, int64_t n) {
     const int at = lane_id() % WIDTH;
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * (256 / WIDTH) + threadIdx.x / WIDTH;
+    const int64_t row = block_of(io) * (256 / WIDTH) + threadIdx.x / WIDTH;
     const bool row_live = row < rows;                      // lanes of absent rows still take part in the exchanges
     const K* xrow = io.x + (row_live ? io.xmap.at(row) : 0);
     const bool live = row_live && at < n;
@@ -782,7 +793,7 @@ __global__ __launch_bounds__(256) void sort_rows_wave(PassIo<K> io, int64_t rows
 template <typename K, bool PAIRS, int ITEMS>
 __global__ __launch_bounds__(256) void sort_rows_wave_items(PassIo<K> io, int64_t rows, int64_t n) {
     const int lane = lane_id();
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+    const int64_t row = block_of(io) * 4 + threadIdx.x / kWave;
     if (row >= rows) return;
     const K* xrow = io.x + io.xmap.at(row);
     const int n32 = static_cast<int>(n);
@@ -821,28 +832,107 @@ __global__ __launch_bounds__(256) void sort_rows_wave_items(PassIo<K> io, int64_
     }
 }
 
+// Rows of at most 64 elements that lie side by side in memory (the axis is an outer
+// dimension): a workgroup takes 64 neighbouring rows, reads them with coalesced loads (64
+// rows wide, one axis position at a time) into LDS, each wavefront sorts sixteen of them with the
+// network of sort_rows_wave (lane l holds element l; pitch 65 keeps both access patterns
+// free of bank conflicts), and the tile leaves the way it came.
+template <typename K, bool PAIRS>
+__global__ __launch_bounds__(256) void sort_cols_wave(PassIo<K> io, int64_t rows, int64_t n) {
+    constexpr int kPitch = kWave + 1;
+    __shared__ K keys[kWave * kPitch];
+    __shared__ uint32_t places[PAIRS ? kWave * kPitch : 1];
+    const int lane = lane_id();
+    const int w = threadIdx.x / kWave;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kWave;
+    const int r = lane;                                    // this thread's row of the tile in the load and store phases
+    const bool row_live = row0 + r < rows;
+    const int n32 = static_cast<int>(n);
+    const K* xrow = io.x + (row_live ? io.xmap.at(row0 + r) : 0);
+    for (int a = w; a < n32; a += 4)
+        keys[a * kPitch + r] = row_live ? key_of_element<K>(io, xrow[static_cast<int64_t>(a) * io.sx]) : ~K(0);
+    __syncthreads();
+    for (int q = w; q < kWave; q += 4) {                   // row q of the tile, element `lane`
+        K key = lane < n32 ? keys[lane * kPitch + q] : ~K(0);      // padding sorts last
+        uint32_t idx = static_cast<uint32_t>(lane);
+        wave_bitonic<kWave, true>([&](auto jc, bool keep_first) {
+            constexpr int J = decltype(jc)::value;
+            const K other_key = lane_xor_const<J>(key);
+            bool other_first = other_key < key;
+            if constexpr (PAIRS) {
+                const uint32_t other_idx = lane_xor_const<J>(idx);
+                other_first = other_first || (other_key == key && other_idx < idx);
+                if (keep_first == other_first) {
+                    key = other_key;
+                    idx = other_idx;
+                }
+            } else {
+                if (keep_first == other_first) key = other_key;
+            }
+        });
+        if (lane < n32) {
+            K bits = decode_key<K>(key, io.kind, io.descending);
+            if constexpr (PAIRS) {
+                if (io.restore_zero && static_cast<K>(bits << 1) == 0 && row0 + q < rows)
+                    bits = io.x[io.xmap.at(row0 + q) + static_cast<int64_t>(idx) * io.sx];
+                places[lane * kPitch + q] = idx;
+            }
+            keys[lane * kPitch + q] = bits;
+        }
+    }
+    __syncthreads();
+    if (!row_live) return;
+    if (io.y) {
+        K* yrow = io.y + io.ymap.at(row0 + r);
+        for (int a = w; a < n32; a += 4) yrow[static_cast<int64_t>(a) * io.sy] = keys[a * kPitch + r];
+    }
+    if constexpr (PAIRS) {
+        if (io.idx) {
+            const int64_t irow = io.imap.at(row0 + r);
+            for (int a = w; a < n32; a += 4) {
+                const int64_t at = irow + static_cast<int64_t>(a) * io.si;
+                if (io.idx64) static_cast<int64_t*>(io.idx)[at] = static_cast<int64_t>(places[a * kPitch + r]);
+                else static_cast<int32_t*>(io.idx)[at] = static_cast<int32_t>(places[a * kPitch + r]);
+            }
+        }
+    }
+}
+
 // longest row sorted by one wavefront (dlfx_set_tuning "sort_wave_rows": 64, 128, 256 or 512)
 int g_sort_wave_rows = 512;
 
 constexpr int64_t kSmallRow = 4096;      // longest row sort_rows_small takes
 
 template <typename K, bool PAIRS>
-int launch_small(hipStream_t stream, const PassIo<K>& io, int64_t m, int64_t n) {
-    const dim3 grid(static_cast<unsigned>(m)), block(256);
+int launch_small(hipStream_t stream, const PassIo<K>& io_in, int64_t m, int64_t n) {
+    PassIo<K> io = io_in;
+    const dim3 block(256);
+    // rows side by side in memory: neighbouring rows to the same XCD
+    const bool side_by_side = io.sx != 1 && io.sx != -1 && io.xmap.rank >= 1 && io.xmap.strides[io.xmap.rank - 1] == 1;
+    auto grid_for = [&](int64_t rows_per_block) {
+        int64_t blocks = ceil_div(m, rows_per_block);
+        io.xcd_blocks = 0;
+        if (side_by_side && blocks >= 64) {
+            io.xcd_blocks = ceil_div(blocks, 8);
+            blocks = io.xcd_blocks * 8;
+        }
+        return dim3(static_cast<unsigned>(blocks));
+    };
     // eight items per lane pay off except for 4-byte keys that carry an index
     const bool wave_items8 = g_sort_wave_rows >= 8 * kWave && !(PAIRS && sizeof(K) == 4);
-    if (n <= 4) sort_rows_wave<K, PAIRS, 4><<<dim3(static_cast<unsigned>(ceil_div(m, 64))), block, 0, stream>>>(io, m, n);
-    else if (n <= 8) sort_rows_wave<K, PAIRS, 8><<<dim3(static_cast<unsigned>(ceil_div(m, 32))), block, 0, stream>>>(io, m, n);
-    else if (n <= 16) sort_rows_wave<K, PAIRS, 16><<<dim3(static_cast<unsigned>(ceil_div(m, 16))), block, 0, stream>>>(io, m, n);
-    else if (n <= 32) sort_rows_wave<K, PAIRS, 32><<<dim3(static_cast<unsigned>(ceil_div(m, 8))), block, 0, stream>>>(io, m, n);
-    else if (n <= kWave) sort_rows_wave<K, PAIRS, kWave><<<dim3(static_cast<unsigned>(ceil_div(m, 4))), block, 0, stream>>>(io, m, n);
-    else if (n <= 2 * kWave && g_sort_wave_rows >= 2 * kWave) sort_rows_wave_items<K, PAIRS, 2><<<dim3(static_cast<unsigned>(ceil_div(m, 4))), block, 0, stream>>>(io, m, n);
-    else if (n <= 4 * kWave && g_sort_wave_rows >= 4 * kWave) sort_rows_wave_items<K, PAIRS, 4><<<dim3(static_cast<unsigned>(ceil_div(m, 4))), block, 0, stream>>>(io, m, n);
-    else if (n <= 8 * kWave && wave_items8) sort_rows_wave_items<K, PAIRS, 8><<<dim3(static_cast<unsigned>(ceil_div(m, 4))), block, 0, stream>>>(io, m, n);
-    else if (n <= 512) sort_rows_small<K, PAIRS, 2><<<grid, block, 0, stream>>>(io, n);
-    else if (n <= 1024) sort_rows_small<K, PAIRS, 4><<<grid, block, 0, stream>>>(io, n);
-    else if (n <= 2048) sort_rows_small<K, PAIRS, 8><<<grid, block, 0, stream>>>(io, n);
-    else sort_rows_small<K, PAIRS, 16><<<grid, block, 0, stream>>>(io, n);
+    if (side_by_side && n <= kWave && m >= 4096) sort_cols_wave<K, PAIRS><<<dim3(static_cast<unsigned>(ceil_div(m, kWave))), block, 0, stream>>>(io, m, n);
+    else if (n <= 4) { const dim3 g = grid_for(64); sort_rows_wave<K, PAIRS, 4><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 8) { const dim3 g = grid_for(32); sort_rows_wave<K, PAIRS, 8><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 16) { const dim3 g = grid_for(16); sort_rows_wave<K, PAIRS, 16><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 32) { const dim3 g = grid_for(8); sort_rows_wave<K, PAIRS, 32><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= kWave) { const dim3 g = grid_for(4); sort_rows_wave<K, PAIRS, kWave><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 2 * kWave && g_sort_wave_rows >= 2 * kWave) { const dim3 g = grid_for(4); sort_rows_wave_items<K, PAIRS, 2><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 4 * kWave && g_sort_wave_rows >= 4 * kWave) { const dim3 g = grid_for(4); sort_rows_wave_items<K, PAIRS, 4><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 8 * kWave && wave_items8) { const dim3 g = grid_for(4); sort_rows_wave_items<K, PAIRS, 8><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 512) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 2><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 1024) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 4><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 2048) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 8><<<g, block, 0, stream>>>(io, m, n); }
+    else { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 16><<<g, block, 0, stream>>>(io, m, n); }
     DLFX_CHECK_LAUNCH();
     return DLFX_OK;
 }

@@ -248,3 +248,36 @@ def test_short_rows_sorted_by_one_workgroup_when_the_wave_sort_is_switched_off(h
                 assert np.array_equal(F.sort(Xh, -1, desc).numpy(), Yo.numpy())
     finally:
         hip_backend.set_tuning("sort_wave_rows", 512)
+
+
+@pytest.mark.parametrize("n", [1, 2, 7, 33, 63, 64])
+def test_short_rows_side_by_side_in_memory(hip_backend, oracle_backend, n):
+    """sort / argsort along an outer axis of at most 64 elements with thousands of rows side by
+    side: tiles of 64 rows pass through LDS.  All key widths, both directions, 64-bit indices,
+    a middle axis, a row count that leaves part of the last tile empty, in place, signed zeros."""
+    for dtype in (np.float32, np.int64, np.float64, np.int16, np.float16, np.int32):
+        x = (normal(280 + n, n * 5003) * 50).astype(dtype).reshape(n, 5003)
+        x[:, 1] = x[0, 1]
+        if n > 4:
+            x[: n // 2, 3] = x[n // 2: 2 * (n // 2), 3]            # every key twice: stability matters
+        Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
+        for desc in (False, True):
+            want = np.sort(x, axis=0, kind="stable")
+            want = want[::-1] if desc else want
+            assert np.array_equal(F.sort(Xh, 0, desc).numpy(), want)
+            Y, I = F.argsort(Xh, 0, desc, with_values=True)
+            Yo, Io = F.argsort(Xo, 0, desc, with_values=True)
+            assert np.array_equal(I.numpy(), Io.numpy()) and np.array_equal(Y.numpy(), Yo.numpy())
+        I64 = F.argsort(Xh, 0, False, index_dtype=np.int64)
+        assert I64.numpy().dtype == np.int64 and np.array_equal(I64.numpy(), F.argsort(Xo, 0).numpy())
+        Z = Tensor.from_numpy(hip_backend, x)
+        F.sort(Z, 0, False, out=Z)
+        assert np.array_equal(Z.numpy(), np.sort(x, axis=0, kind="stable"))
+    a = (normal(281 + n, 3 * n * 2100) * 9).astype(np.float32).reshape(3, n, 2100)
+    a[1, 0, :] = 0.0
+    if n > 1:
+        a[1, n - 1, :] = -0.0
+    T, O = Tensor.from_numpy(hip_backend, a), Tensor.from_numpy(oracle_backend, a)
+    Y, I = F.argsort(T, 1, True, with_values=True)
+    Yo, Io = F.argsort(O, 1, True, with_values=True)
+    assert np.array_equal(I.numpy(), Io.numpy()) and np.array_equal(Y.numpy().view(np.uint32), Yo.numpy().view(np.uint32))
