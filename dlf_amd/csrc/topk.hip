@@ -99,6 +99,9 @@ struct TopkIo {
     // segmented rows (first stage of long rows): row r of the launch is segment r % segs of a
     // longer row; the last segment of each has last_n elements instead of n.  0 or 1: plain rows.
     int64_t segs, last_n;
+    // rows side by side in memory: workgroup b takes block (b % 8) * xcd_blocks + b / 8, so that
+    // neighbouring rows, which share cache lines, run on one XCD (0: workgroup b takes block b)
+    int64_t xcd_blocks;
 };
 
 constexpr int kCandCap = 4096;     // candidates kept after the pre-filter (4-byte keys; half for 8-byte keys)
@@ -641,7 +644,8 @@ __global__ __launch_bounds__(256) void topk_rows_wave(TopkIo<typename BitsOf<E>:
     __shared__ uint32_t cand_idx[4][kWave];
     const int lane = lane_id();
     const int w = threadIdx.x / kWave;
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + w;
+    const int64_t block = io.xcd_blocks ? static_cast<int64_t>(blockIdx.x % 8) * io.xcd_blocks + blockIdx.x / 8 : blockIdx.x;
+    const int64_t row = block * 4 + w;
     if (row >= rows) return;                               // whole waves leave; nothing below synchronises the workgroup
     const S* xr = io.x + io.xmap.at(row);
     S* yr = io.y + io.ymap.at(row);
@@ -749,13 +753,14 @@ __global__ __launch_bounds__(256) void topk_rows_wave(TopkIo<typename BitsOf<E>:
 }
 
 // Rows that lie side by side in memory (the axis is an outer dimension of the tensor, the
-// innermost row dimension has stride 1) and a limit of at most 8: one thread per row and
+// innermost row dimension has stride 1) and a limit of at most 16: one thread per row and
 // segment of the axis, so the 64 lanes of a wave read 64 neighbouring elements whatever the
 // stride along the axis.  A thread keeps the KMAX best (image, index) entries it has seen in
 // registers, ordered; an element enters only when it beats the last of them.  SEG waves share
 // 64 rows, each scanning a contiguous piece of the axis; their lists meet in LDS and the first
 // wave merges and writes them.  No scratch, any row length.
-constexpr int kColsLimit = 8;
+constexpr int kColsLimit = 16;         // largest limit topk_cols takes
+constexpr int kThreadRowLimit = 8;     // ... and topk_rows_thread
 // longest row topk_rows_thread takes with 4-byte keys, half of it with 8-byte keys
 // (dlfx_set_tuning "topk_thread_rows"); beyond, a wave per row has enough rows in flight and wins
 int g_topk_thread_rows = 256;
@@ -1242,8 +1247,14 @@ int launch_select(hipStream_t stream, const TopkIo<typename BitsOf<T>::type, typ
     K* spill_ord = reinterpret_cast<K*>(sbase + sl.ord_off);
     uint32_t* spill_idx = reinterpret_cast<uint32_t*>(sbase + sl.idx_off);
     if (n <= kWaveRowMax && (lim <= kWaveRowLimit || n <= kWaveSortItems * kWave)) {      // at most 256 elements: a wave can order the whole row, whatever the limit
-        const dim3 wgrid(static_cast<unsigned>(ceil_div(m, 4)));
-#define DLFX_TOPK_WAVE(ITEMS) topk_rows_wave<T, ITEMS><<<wgrid, dim3(256), 0, stream>>>(io, m, n, lim)
+        TopkIo<K, S> wio = io;
+        int64_t wblocks = ceil_div(m, 4);
+        if (io.sx != 1 && io.sx != -1 && io.xmap.rank >= 1 && io.xmap.strides[io.xmap.rank - 1] == 1 && wblocks >= 64) {
+            wio.xcd_blocks = ceil_div(wblocks, 8);
+            wblocks = wio.xcd_blocks * 8;
+        }
+        const dim3 wgrid(static_cast<unsigned>(wblocks));
+#define DLFX_TOPK_WAVE(ITEMS) topk_rows_wave<T, ITEMS><<<wgrid, dim3(256), 0, stream>>>(wio, m, n, lim)
         if (n <= 64) DLFX_TOPK_WAVE(1);
         else if (n <= 128) DLFX_TOPK_WAVE(2);
         else if (n <= 256) DLFX_TOPK_WAVE(4);
@@ -1356,7 +1367,8 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
     if (m > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
 
     // rows side by side in memory, small limit: one thread per row (and segment of the axis)
-    if (limit <= kColsLimit && io.sx != 1 && io.sx != -1 && m >= 16384 && n <= 0x7fffffffLL && io.xmap.rank >= 1 &&
+    // (limits of 9 to 16 only on rows of up to 256 elements: beyond, a wave per row with neighbouring rows on one XCD is faster)
+    if (limit <= kColsLimit && (limit <= 8 || n <= 256) && io.sx != 1 && io.sx != -1 && m >= 16384 && n <= 0x7fffffffLL && io.xmap.rank >= 1 &&
         io.xmap.strides[io.xmap.rank - 1] == 1 && io.xmap.dims[io.xmap.rank - 1] >= kWave) {
         const int lim = static_cast<int>(limit);
         const int64_t blocks = ceil_div(m, static_cast<int64_t>(kWave));
@@ -1371,14 +1383,15 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
         if (lim <= 1) DLFX_TOPK_COLS(1);
         else if (lim <= 2) DLFX_TOPK_COLS(2);
         else if (lim <= 4) DLFX_TOPK_COLS(4);
-        else DLFX_TOPK_COLS(8);
+        else if (lim <= 8) DLFX_TOPK_COLS(8);
+        else DLFX_TOPK_COLS(16);
 #undef DLFX_TOPK_COLS
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
     }
 
     // many short rows one after the other in memory, small limit: one thread per row
-    if (limit <= kColsLimit && io.sx == 1 && io.xmap.rank <= 1 && m >= 16384 &&
+    if (limit <= kThreadRowLimit && io.sx == 1 && io.xmap.rank <= 1 && m >= 16384 &&
         n <= (sizeof(K) == 4 ? g_topk_thread_rows : g_topk_thread_rows / 2)) {
         const int lim = static_cast<int>(limit);
         const int64_t pitch = io.xmap.rank ? io.xmap.strides[0] : 0;

@@ -169,7 +169,7 @@ def test_short_rows_one_wave_per_row(hip_backend, oracle_backend, n):
 
 @pytest.mark.parametrize("n", [1, 2, 7, 63, 64, 100, 511, 512, 700])
 def test_rows_side_by_side_in_memory(hip_backend, oracle_backend, n):
-    """top_k along an outer axis with a limit of at most 8: one thread per row, several waves
+    """top_k along an outer axis with a limit of at most 16: one thread per row, several waves
     per row segment.  Every list length, both directions, all element types, rows that are all
     ties, row counts that leave lanes idle, and a middle axis."""
     cols = 16400 + n % 50
@@ -180,7 +180,7 @@ def test_rows_side_by_side_in_memory(hip_backend, oracle_backend, n):
         x[:, 3] = np.sort(x[:, 3], kind="stable")
         x[:, 4] = np.sort(x[:, 4], kind="stable")[::-1]
         Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
-        for k in sorted({1, min(n, 2), min(n, 3), min(n, 4), min(n, 5), min(n, 8)}):
+        for k in sorted({1, min(n, 2), min(n, 3), min(n, 4), min(n, 5), min(n, 8), min(n, 9), min(n, 16)}):
             for largest in (True, False):
                 Yh, Ih = F.top_k(Xh, k, 0, largest)
                 Yo, Io = F.top_k(Xo, k, 0, largest)
