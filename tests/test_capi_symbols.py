@@ -36,10 +36,24 @@ def test_host_only_calls():
     assert lib.dlfx_scan_scratch_bytes(0, 64, 100) == 0
     assert 0 < lib.dlfx_top_k_scratch_bytes(0, 4096, 32000, 256) <= 4096 * (4096 * 8 + 4) + 1024
     assert lib.dlfx_top_k_scratch_bytes(0, 256, 1000, 5) <= 1024
-    assert lib.dlfx_top_k_scratch_bytes(0, 8, 1 << 20, 5) > 8 * (1 << 20) * 8
+    # rows longer than the selection kernel takes: winners of 16 segments per row, far below a full argsort
+    assert 0 < lib.dlfx_top_k_scratch_bytes(0, 8, 1 << 20, 5) < 8 * (1 << 20)
+    # limits the selection does not take still need room for the argsort
+    assert lib.dlfx_top_k_scratch_bytes(0, 8, 1 << 20, 5000) > 8 * (1 << 20) * 8
+    # the softmax family needs scratch only for few rows that are too long for one workgroup's registers
+    assert lib.dlfx_softmax_scratch_bytes(0, 4096, 32000) == 0
+    assert lib.dlfx_softmax_scratch_bytes(0, 8, 32768) == 0
+    assert 0 < lib.dlfx_softmax_scratch_bytes(0, 8, 262144) <= 8 * 32 * 32
+    assert lib.dlfx_softmax_scratch_bytes(1, 8, 20000) > 0
+    assert lib.dlfx_softmax_scratch_bytes(0, 512, 262144) == 0
+    assert lib.dlfx_softmax_scratch_bytes(2, 8, 262144) > 0            # hardmax of int32
+    assert lib.dlfx_softmax_scratch_bytes(5, 8, 262144) == 0           # no int16 softmax family
     assert lib.dlfx_sort_scratch_bytes(3, 256, 1 << 20) >= 2 * 256 * (1 << 20) * 8
     assert lib.dlfx_set_tuning(b"no_such_knob", 1) == -3
     assert lib.dlfx_set_tuning(b"scan_poll_limit", 2048) == 0
+    for knob, value in ((b"sort_poll_limit", 2048), (b"sort_wave_rows", 512), (b"topk_thread_rows", 256)):
+        assert lib.dlfx_set_tuning(knob, value) == 0
+    assert lib.dlfx_set_tuning(b"sort_wave_rows", 100000) == -3
 
 
 def test_argument_errors_are_reported_without_a_gpu():
