@@ -78,6 +78,11 @@ int dlfx_last_hip_error(void);
  *                      state before it folds that predecessor's input itself
  *                      (default 2048; 0 makes every tile help itself at once).
  *   "sort_poll_limit"  the same bound for the per-digit tile chaining of a radix pass.
+ *   "sort_wave_rows"   longest row (64, 128, 256 or 512; default 512) sorted by one wavefront
+ *                      in registers; longer rows of up to 4096 elements take one workgroup.
+ *   "topk_thread_rows" longest row (default 256; half of it for 8-byte keys) for which top_k
+ *                      with a limit of at most 8 over at least 16384 contiguous rows gives
+ *                      each row to one thread.
  * Returns DLFX_ERR_UNKNOWN_OP for an unknown key or out-of-range value.  No
  * counterpart in the reference (its database/ tuning tables play this role). */
 int dlfx_set_tuning(const char* key, int64_t value);
