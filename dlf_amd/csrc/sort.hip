@@ -742,6 +742,25 @@ __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t row
     }
 }
 
+// One exchange of the (key, index) networks below: the lane takes the entry of lane ^ J when
+// that entry comes first (smaller key, then smaller index - a total order, hence stable) and
+// this lane keeps the first of the two, or when it does not and this lane keeps the second.
+template <bool PAIRS, int J, typename K>
+__device__ __forceinline__ void exchange_entry(K& key, uint32_t& idx, bool keep_first) {
+    const K other_key = lane_xor_const<J>(key);
+    bool other_first = other_key < key;
+    if constexpr (PAIRS) {
+        const uint32_t other_idx = lane_xor_const<J>(idx);
+        other_first = other_first || (other_key == key && other_idx < idx);
+        if (keep_first == other_first) {
+            key = other_key;
+            idx = other_idx;
+        }
+    } else {
+        if (keep_first == other_first) key = other_key;
+    }
+}
+
 // Rows of at most 64 elements: a group of WIDTH = 4, 8, 16, 32 or 64 lanes per row, one element
 // per lane, a bitonic network over (key, index) pairs - a total order, so the result is the
 // stable one.  256 / WIDTH rows per workgroup, no LDS, no barrier.
@@ -754,21 +773,7 @@ __global__ __launch_bounds__(256) void sort_rows_wave(PassIo<K> io, int64_t rows
     const bool live = row_live && at < n;
     K key = live ? key_of_element<K>(io, xrow[static_cast<int64_t>(at) * io.sx]) : ~K(0);   // padding sorts last
     uint32_t idx = static_cast<uint32_t>(at);
-    wave_bitonic<WIDTH, true>([&](auto jc, bool keep_first) {
-        constexpr int J = decltype(jc)::value;
-        const K other_key = lane_xor_const<J>(key);
-        bool other_first = other_key < key;
-        if constexpr (PAIRS) {
-            const uint32_t other_idx = lane_xor_const<J>(idx);
-            other_first = other_first || (other_key == key && other_idx < idx);
-            if (keep_first == other_first) {
-                key = other_key;
-                idx = other_idx;
-            }
-        } else {
-            if (keep_first == other_first) key = other_key;
-        }
-    });
+    wave_bitonic<WIDTH, true>([&](auto jc, bool keep_first) { exchange_entry<PAIRS, decltype(jc)::value>(key, idx, keep_first); });
     if (!live) return;                                     // the first n lanes of the group hold the row in order
     if (io.y) {
         K bits = decode_key<K>(key, io.kind, io.descending);
@@ -855,21 +860,7 @@ __global__ __launch_bounds__(256) void sort_cols_wave(PassIo<K> io, int64_t rows
     for (int q = w; q < kWave; q += 4) {                   // row q of the tile, element `lane`
         K key = lane < n32 ? keys[lane * kPitch + q] : ~K(0);      // padding sorts last
         uint32_t idx = static_cast<uint32_t>(lane);
-        wave_bitonic<kWave, true>([&](auto jc, bool keep_first) {
-            constexpr int J = decltype(jc)::value;
-            const K other_key = lane_xor_const<J>(key);
-            bool other_first = other_key < key;
-            if constexpr (PAIRS) {
-                const uint32_t other_idx = lane_xor_const<J>(idx);
-                other_first = other_first || (other_key == key && other_idx < idx);
-                if (keep_first == other_first) {
-                    key = other_key;
-                    idx = other_idx;
-                }
-            } else {
-                if (keep_first == other_first) key = other_key;
-            }
-        });
+        wave_bitonic<kWave, true>([&](auto jc, bool keep_first) { exchange_entry<PAIRS, decltype(jc)::value>(key, idx, keep_first); });
         if (lane < n32) {
             K bits = decode_key<K>(key, io.kind, io.descending);
             if constexpr (PAIRS) {
