@@ -179,3 +179,35 @@ def test_tensors_of_more_than_2_32_elements(hip_backend):
     ys = dev(F.sort(wrap(hip_backend, xs), 1))
     for rows in (slice(0, 8), slice(32768, 32776), slice(-8, None)):
         assert torch.equal(ys[rows], torch.sort(xs[rows], dim=1).values)
+
+
+def test_one_row_of_2_26_elements(hip_backend):
+    """A single long row (global sort / top-k / softmax over one vector): the routines that cut
+    a row into tiles or segments, checked against an independent device implementation."""
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(17)
+    n = 1 << 26
+    x = (torch.randn(1, n, device="cuda", generator=g) * 1024).round() / 64            # ties
+    X = wrap(hip_backend, x)
+    want = torch.sort(x, dim=1, descending=True, stable=True)
+    assert torch.equal(dev(F.sort(X, 1, True)), want.values)
+    assert torch.equal(dev(F.argsort(X, 1, True)).long(), want.indices)
+    for k in (1, 100, 1024):
+        Y, I = F.top_k(X, k, 1, True)
+        assert torch.equal(dev(Y), want.values[:, :k]) and torch.equal(dev(I).long(), want.indices[:, :k])
+    Y, I = F.top_k(X, 7, 1, False, index_dtype=np.int64)
+    up = torch.sort(x, dim=1, descending=False, stable=True)
+    assert torch.equal(dev(Y), up.values[:, :7]) and torch.equal(dev(I), up.indices[:, :7])
+    del want, up
+    z = x / 16
+    sm = dev(F.softmax(wrap(hip_backend, z), 1)).double()
+    ref = torch.softmax(z.double(), 1)
+    assert bool(((sm - ref).abs() <= 8 * 26 * EPS32 * ref + 1e-300).all())
+    assert abs(float(sm.sum()) - 1.0) < 1e-5
+    ls = dev(F.logsoftmax(wrap(hip_backend, z), 1)).double()
+    refl = torch.log_softmax(z.double(), 1)
+    assert bool(((ls - refl).abs() <= 8 * 26 * EPS32 * (1 + refl.abs())).all())
+    hm = dev(F.hardmax(wrap(hip_backend, z), 1))
+    assert float(hm.sum()) == 1.0 and int(hm.argmax()) == int((z == z.max()).to(torch.int8).argmax())
+    xi = torch.randint(-1000, 1000, (1, n), dtype=torch.int32, device="cuda", generator=g)
+    assert torch.equal(dev(F.cumsum(wrap(hip_backend, xi), 1)), torch.cumsum(xi, 1, dtype=torch.int32))
