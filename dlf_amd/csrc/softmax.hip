@@ -175,6 +175,8 @@ void softmax_rows(const S* __restrict__ x, S* __restrict__ y, int64_t m, int64_t
     }
 }
 
+constexpr int kStreamBatch = 8;
+
 // Rows too long for registers: one 1024-thread workgroup per row, two passes over the row.
 template <typename S, int KIND>
 __global__ __launch_bounds__(1024) void softmax_rows_streamed(const S* __restrict__ x, S* __restrict__ y, int64_t n) {
@@ -195,22 +197,43 @@ __global__ __launch_bounds__(1024) void softmax_rows_streamed(const S* __restric
     } else {
         // running maximum and the sum of exp(x - maximum), rescaled whenever the maximum moves
         T mx = lowest, sum = T(0);
-        for (int64_t i = t; i < n; i += TEAM) {
-            const T xv = static_cast<T>(xr[i]);
-            if (mx < xv) {
-                sum = sum * exp_of<T>(mx - xv);          // exp(-inf) = 0 on the first element
-                mx = xv;
+        for (int64_t i = t; i < n; i += TEAM * kStreamBatch) {              // kStreamBatch loads in flight per thread
+            S in[kStreamBatch];
+#pragma unroll
+            for (int u = 0; u < kStreamBatch; ++u) {
+                const int64_t j = i + static_cast<int64_t>(u) * TEAM;
+                if (j < n) in[u] = load_stream(&xr[j]);
             }
-            if (xv != lowest || mx != lowest) sum += exp_of<T>(xv - mx);     // -inf before any finite element adds nothing
+#pragma unroll
+            for (int u = 0; u < kStreamBatch; ++u) {
+                if (i + static_cast<int64_t>(u) * TEAM >= n) break;
+                const T xv = static_cast<T>(in[u]);
+                if (mx < xv) {
+                    sum = sum * exp_of<T>(mx - xv);          // exp(-inf) = 0 on the first element
+                    mx = xv;
+                }
+                if (xv != lowest || mx != lowest) sum += exp_of<T>(xv - mx);     // -inf before any finite element adds nothing
+            }
         }
         T row_max = team_reduce<TEAM>(mx, [](T a, T b) { return (a < b) ? b : a; }, reinterpret_cast<T*>(lds_raw));
         sum = (mx == lowest) ? T(0) : sum * exp_of<T>(mx - row_max);
         if (xr[0] != xr[0]) row_max = static_cast<T>(xr[0]);             // a NaN in position 0 is the reference's maximum
         sum = team_reduce<TEAM>(sum, [](T a, T b) { return a + b; }, reinterpret_cast<T*>(lds_raw));
         const T lsum = log_of<T>(sum);
-        for (int64_t i = t; i < n; i += TEAM) {
-            const T xv = static_cast<T>(xr[i]);
-            yr[i] = static_cast<S>(KIND == kSoftmax ? exp_of<T>(xv - row_max) / sum : (xv - row_max) - lsum);
+        for (int64_t i = t; i < n; i += TEAM * kStreamBatch) {
+            S in[kStreamBatch];
+#pragma unroll
+            for (int u = 0; u < kStreamBatch; ++u) {
+                const int64_t j = i + static_cast<int64_t>(u) * TEAM;
+                if (j < n) in[u] = load_stream(&xr[j]);
+            }
+#pragma unroll
+            for (int u = 0; u < kStreamBatch; ++u) {
+                const int64_t j = i + static_cast<int64_t>(u) * TEAM;
+                if (j >= n) break;
+                const T xv = static_cast<T>(in[u]);
+                store_stream(&yr[j], static_cast<S>(KIND == kSoftmax ? exp_of<T>(xv - row_max) / sum : (xv - row_max) - lsum));
+            }
         }
     }
 }
@@ -225,6 +248,8 @@ struct SoftPartial {
     T mx, sum, first;          // soft kinds: running maximum, sum of exp(x - mx), the row's first element (tile 0)
     MaxAt<T> best;             // hardmax
 };
+
+constexpr int kSplitBatch = 8;
 
 struct SplitPlan {
     int64_t tiles, tile_len;
@@ -265,13 +290,23 @@ __global__ __launch_bounds__(1024) void softmax_split_partials(const S* __restri
                                      reinterpret_cast<MaxAt<T>*>(lds_raw));
     } else {
         T mx = lowest, sum = T(0);
-        for (int64_t i = i0 + t; i < i1; i += TEAM) {
-            const T xv = static_cast<T>(xr[i]);
-            if (mx < xv) {
-                sum = sum * exp_of<T>(mx - xv);
-                mx = xv;
+        for (int64_t i = i0 + t; i < i1; i += TEAM * kSplitBatch) {           // kSplitBatch loads in flight per thread
+            S in[kSplitBatch];
+#pragma unroll
+            for (int u = 0; u < kSplitBatch; ++u) {
+                const int64_t j = i + static_cast<int64_t>(u) * TEAM;
+                if (j < i1) in[u] = load_stream(&xr[j]);
             }
-            if (xv != lowest || mx != lowest) sum += exp_of<T>(xv - mx);
+#pragma unroll
+            for (int u = 0; u < kSplitBatch; ++u) {
+                if (i + static_cast<int64_t>(u) * TEAM >= i1) break;
+                const T xv = static_cast<T>(in[u]);
+                if (mx < xv) {
+                    sum = sum * exp_of<T>(mx - xv);
+                    mx = xv;
+                }
+                if (xv != lowest || mx != lowest) sum += exp_of<T>(xv - mx);
+            }
         }
         const T tile_max = team_reduce<TEAM>(mx, [](T a, T b) { return (a < b) ? b : a; }, reinterpret_cast<T*>(lds_raw));
         sum = (mx == lowest) ? T(0) : sum * exp_of<T>(mx - tile_max);
@@ -318,9 +353,20 @@ __global__ __launch_bounds__(1024) void softmax_split_apply(const S* __restrict_
         if (first != first) row_max = first;                      // a NaN in position 0 is the reference's maximum
         sum = team_reduce<TEAM>(sum, [](T a, T b) { return a + b; }, reinterpret_cast<T*>(lds_raw));
         const T lsum = log_of<T>(sum);
-        for (int64_t i = i0 + t; i < i1; i += TEAM) {
-            const T xv = static_cast<T>(xr[i]);
-            yr[i] = static_cast<S>(KIND == kSoftmax ? exp_of<T>(xv - row_max) / sum : (xv - row_max) - lsum);
+        for (int64_t i = i0 + t; i < i1; i += TEAM * kSplitBatch) {
+            S in[kSplitBatch];
+#pragma unroll
+            for (int u = 0; u < kSplitBatch; ++u) {
+                const int64_t j = i + static_cast<int64_t>(u) * TEAM;
+                if (j < i1) in[u] = load_stream(&xr[j]);
+            }
+#pragma unroll
+            for (int u = 0; u < kSplitBatch; ++u) {
+                const int64_t j = i + static_cast<int64_t>(u) * TEAM;
+                if (j >= i1) break;
+                const T xv = static_cast<T>(in[u]);
+                store_stream(&yr[j], static_cast<S>(KIND == kSoftmax ? exp_of<T>(xv - row_max) / sum : (xv - row_max) - lsum));
+            }
         }
     }
 }
@@ -328,7 +374,7 @@ __global__ __launch_bounds__(1024) void softmax_split_apply(const S* __restrict_
 // rows at most this long are held in registers by one workgroup
 template <typename T>
 constexpr int64_t register_row_limit() { return sizeof(typename ComputeOf<T>::type) == 4 ? 1024 * 32 : 1024 * 16; }
-constexpr int64_t kSplitMaxRows = 512;        // from this many rows on, a workgroup per row fills the device
+constexpr int64_t kSplitMaxRows = 256;        // from this many rows on (one per compute unit), a workgroup per row is as fast
 
 template <typename T>
 size_t split_scratch_bytes(int64_t m, int64_t n) {

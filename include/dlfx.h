@@ -207,7 +207,7 @@ int dlfx_scan_nonzero(dlfx_stream_t stream, int dtype, int64_t m, int64_t n,
  * dnn_detail.h:292-295, 324-327, 352-355) on the rows of a contiguous [m, n] matrix.  The
  * reference works in place on x; here y may be x (in place) or another buffer.
  * name: "softmax" | "logsoftmax" | "hardmax".  Floating-point types (hardmax: int32, int64 too).
- * Scratch is optional: fewer than 512 rows that are too long for one workgroup's registers
+ * Scratch is optional: fewer than 256 rows that are too long for one workgroup's registers
  * (more than 32768 4-byte or 16384 8-byte elements) are cut into tiles that the whole device
  * works on when scratch of dlfx_softmax_scratch_bytes() bytes (16-byte aligned) is given, and
  * are walked by one workgroup per row when it is not (scratch NULL); every other shape needs none.

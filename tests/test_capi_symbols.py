@@ -45,7 +45,8 @@ def test_host_only_calls():
     assert lib.dlfx_softmax_scratch_bytes(0, 8, 32768) == 0
     assert 0 < lib.dlfx_softmax_scratch_bytes(0, 8, 262144) <= 8 * 32 * 32
     assert lib.dlfx_softmax_scratch_bytes(1, 8, 20000) > 0
-    assert lib.dlfx_softmax_scratch_bytes(0, 512, 262144) == 0
+    assert lib.dlfx_softmax_scratch_bytes(0, 255, 262144) > 0
+    assert lib.dlfx_softmax_scratch_bytes(0, 256, 262144) == 0
     assert lib.dlfx_softmax_scratch_bytes(2, 8, 262144) > 0            # hardmax of int32
     assert lib.dlfx_softmax_scratch_bytes(5, 8, 262144) == 0           # no int16 softmax family
     assert lib.dlfx_sort_scratch_bytes(3, 256, 1 << 20) >= 2 * 256 * (1 << 20) * 8

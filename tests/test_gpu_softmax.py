@@ -121,9 +121,9 @@ def test_row_lengths_around_the_team_sizes(hip_backend, oracle_backend, n):
 
 
 @pytest.mark.parametrize("m,n,dtype", [(1, 200000, np.float32), (3, 70001, np.float32), (7, 40000, np.float64), (2, 32769, np.float32),
-                                       (5, 16385, np.float64), (2, 100000, np.float16), (300, 33000, np.float32)])
+                                       (5, 16385, np.float64), (2, 100000, np.float16), (200, 33000, np.float32)])
 def test_few_long_rows_are_cut_into_tiles(hip_backend, oracle_backend, m, n, dtype):
-    """Fewer than 512 rows that are too long for one workgroup's registers: every row is cut
+    """Fewer than 256 rows that are too long for one workgroup's registers: every row is cut
     into tiles that the whole device works on (two kernels, one record per tile in scratch).
     All three kinds, in place and out of place, a NaN in position 0 and elsewhere, -inf entries,
     an all -inf row, and the same call without scratch (one workgroup per row)."""
