@@ -81,71 +81,50 @@ struct TileState<T, 4> {
     }
 };
 
-// 8-byte values: value arrays plus a flag written with release / read with acquire.
-template <typename T>
-struct TileState<T, 8> {
-    uint32_t* flags;
-    unsigned long long* agg;
-    unsigned long long* incl;
-    static size_t bytes(int64_t tiles) { return align_up(static_cast<size_t>(tiles) * 4, 256) + static_cast<size_t>(tiles) * 16; }
-    __host__ __device__ void bind(void* base, int64_t tiles) {
-        flags = static_cast<uint32_t*>(base);
-        size_t off = (static_cast<size_t>(tiles) * 4 + 255) / 256 * 256;
-        agg = reinterpret_cast<unsigned long long*>(static_cast<char*>(base) + off);
-        incl = agg + tiles;
-    }
-    __device__ __forceinline__ void clear(int64_t i) { flags[i] = 0u; }
-    __device__ __forceinline__ void publish(int64_t i, uint32_t flag, T v) {
-        unsigned long long* dst = (flag == kAggregate) ? agg : incl;
-        __hip_atomic_store(&dst[i], bit_cast<unsigned long long>(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&flags[i], flag, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __device__ __forceinline__ uint32_t read(int64_t i, T* v) {
-        uint32_t f = __hip_atomic_load(&flags[i], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
-        if (f != kInvalid) {
-            unsigned long long* src = (f == kAggregate) ? agg : incl;
-            *v = bit_cast<T>(__hip_atomic_load(&src[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        }
-        return f;
-    }
-};
-
-// 16-byte values (complex of doubles): as the 8-byte case with two words per value.
-template <typename T>
-struct TileState<T, 16> {
-    struct Pair {
-        unsigned long long lo, hi;
+// 8- and 16-byte values: one 64-bit word per 32 bits of the value, each carrying the flag in
+// its upper half, all written and read with relaxed atomics (no fences, so no cache
+// write-backs or invalidations on the polling path).  A value is taken only when all of its
+// words carry the same flag: every state of a tile is written once and the states follow one
+// another, so equal flags mean the words belong to one state; anything else reads as "not
+// there yet" and is polled again.
+template <typename T, int WORDS>
+struct TileStateWords {
+    struct Parts {
+        uint32_t w[WORDS];
     };
-    uint32_t* flags;
-    unsigned long long* agg;
-    unsigned long long* incl;
-    static size_t bytes(int64_t tiles) { return align_up(static_cast<size_t>(tiles) * 4, 256) + static_cast<size_t>(tiles) * 32; }
-    __host__ __device__ void bind(void* base, int64_t tiles) {
-        flags = static_cast<uint32_t*>(base);
-        size_t off = (static_cast<size_t>(tiles) * 4 + 255) / 256 * 256;
-        agg = reinterpret_cast<unsigned long long*>(static_cast<char*>(base) + off);
-        incl = agg + 2 * tiles;
+    unsigned long long* words;
+    static size_t bytes(int64_t tiles) { return static_cast<size_t>(tiles) * WORDS * 8; }
+    __host__ __device__ void bind(void* base, int64_t) { words = static_cast<unsigned long long*>(base); }
+    __device__ __forceinline__ void clear(int64_t i) {
+#pragma unroll
+        for (int k = 0; k < WORDS; ++k) words[i * WORDS + k] = 0ull;
     }
-    __device__ __forceinline__ void clear(int64_t i) { flags[i] = 0u; }
     __device__ __forceinline__ void publish(int64_t i, uint32_t flag, T v) {
-        unsigned long long* dst = (flag == kAggregate) ? agg : incl;
-        const Pair p = bit_cast<Pair>(v);
-        __hip_atomic_store(&dst[2 * i], p.lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&dst[2 * i + 1], p.hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&flags[i], flag, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        const Parts p = bit_cast<Parts>(v);
+#pragma unroll
+        for (int k = 0; k < WORDS; ++k)
+            __hip_atomic_store(&words[i * WORDS + k], (static_cast<unsigned long long>(flag) << 32) | p.w[k], __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
     }
     __device__ __forceinline__ uint32_t read(int64_t i, T* v) {
-        uint32_t f = __hip_atomic_load(&flags[i], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
-        if (f != kInvalid) {
-            unsigned long long* src = (f == kAggregate) ? agg : incl;
-            Pair p;
-            p.lo = __hip_atomic_load(&src[2 * i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            p.hi = __hip_atomic_load(&src[2 * i + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            *v = bit_cast<T>(p);
+        unsigned long long w[WORDS];
+#pragma unroll
+        for (int k = 0; k < WORDS; ++k) w[k] = __hip_atomic_load(&words[i * WORDS + k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t f = static_cast<uint32_t>(w[0] >> 32);
+        Parts p;
+        bool whole = true;
+#pragma unroll
+        for (int k = 0; k < WORDS; ++k) {
+            whole = whole && static_cast<uint32_t>(w[k] >> 32) == f;
+            p.w[k] = static_cast<uint32_t>(w[k]);
         }
+        if (!whole) return kInvalid;
+        *v = bit_cast<T>(p);
         return f;
     }
 };
+template <typename T> struct TileState<T, 8> : TileStateWords<T, 2> {};
+template <typename T> struct TileState<T, 16> : TileStateWords<T, 4> {};
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void scan_init(unsigned* ticket, int64_t rows, TileState<T> st, int64_t tiles) {
@@ -153,6 +132,11 @@ __global__ __launch_bounds__(kBlock) void scan_init(unsigned* ticket, int64_t ro
     if (i < rows) ticket[i] = 0u;
     if (i < tiles) st.clear(i);
 }
+
+// Elements per memory access: 16 bytes of the arithmetic type, or of the stored type when input
+// and output are both 16-bit (half scans compute in fp32 but should still move 16 bytes at a time).
+template <typename T, typename X, typename Y>
+constexpr int scan_vec() { return (sizeof(X) == 2 && sizeof(Y) == 2) ? 8 : vec_width<T>(); }
 
 // What a scan folds for an input element: the element itself, or (scan_nonzero,
 // gpgpu/include/gdnn.h:131-136) one for every element that is not zero.
@@ -186,7 +170,7 @@ __device__ __forceinline__ void scan_tile(
         else return i * sx;
     };
     using Op = ScanOp<T, K>;
-    constexpr int V = (vec_width<T>() < ITEMS) ? vec_width<T>() : ITEMS;
+    constexpr int V = (scan_vec<T, X, Y>() < ITEMS) ? scan_vec<T, X, Y>() : ITEMS;
     constexpr int KV = ITEMS / V;
     constexpr int64_t TILE = static_cast<int64_t>(BLOCK) * ITEMS;
     using VecX = Vec<X, V>;
@@ -194,7 +178,6 @@ __device__ __forceinline__ void scan_tile(
     const int lane = lane_id();
     const int w = threadIdx.x / kWave;
     const int64_t tile_base = t * TILE;
-    const int64_t avail = (n - tile_base < TILE) ? n - tile_base : TILE;   // valid elements in this tile
 
     const X* xr = x + xmap.at(row);
     Y* yr = y + ymap.at(row);
@@ -202,24 +185,21 @@ __device__ __forceinline__ void scan_tile(
 
     // ---- load
     T vals[ITEMS];
-    const bool full = avail == TILE;
-    const bool x_vec = full && sx == 1 && (reinterpret_cast<uintptr_t>(xr + seg) % (sizeof(X) * V) == 0);
-    if (x_vec) {
-        const VecX* pv = reinterpret_cast<const VecX*>(xr + seg);
+    // whole vectors of an aligned unit-stride row move as one access; the row's last, partial
+    // vector (and what lies past the row in its last tile) element by element
+    const bool x_vec = sx == 1 && (reinterpret_cast<uintptr_t>(xr + seg) % (sizeof(X) * V) == 0);
+    const VecX* pv = reinterpret_cast<const VecX*>(xr + seg);
 #pragma unroll
-        for (int k = 0; k < KV; ++k) {
+    for (int k = 0; k < KV; ++k) {
+        const int64_t i0 = seg + static_cast<int64_t>(k * kWave + lane) * V;
+        if (x_vec && i0 + V <= n) {
             VecX a = load_stream(&pv[k * kWave + lane]);
 #pragma unroll
             for (int e = 0; e < V; ++e) vals[k * V + e] = scan_input<T, X, NZ>(a.v[e]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < V; ++e) vals[k * V + e] = (i0 + e < n) ? scan_input<T, X, NZ>(xr[x_at(i0 + e)]) : Op::identity();
         }
-    } else {
-#pragma unroll
-        for (int k = 0; k < KV; ++k)
-#pragma unroll
-            for (int e = 0; e < V; ++e) {
-                const int64_t i = seg + static_cast<int64_t>(k * kWave + lane) * V + e;
-                vals[k * V + e] = (i < n) ? scan_input<T, X, NZ>(xr[x_at(i)]) : Op::identity();
-            }
     }
     // ---- scan inside the wave: vals[] become inclusive prefixes within the wave segment
     T carry = Op::identity();
@@ -329,24 +309,21 @@ __device__ __forceinline__ void scan_tile(
     for (int i = 0; i < ITEMS; ++i) vals[i] = Op::apply(pre, vals[i]);
 
     using VecY = Vec<Y, V>;
-    const bool y_vec = full && sy == 1 && (reinterpret_cast<uintptr_t>(yr + seg) % (sizeof(Y) * V) == 0);
-    if (y_vec) {
-        VecY* pv = reinterpret_cast<VecY*>(yr + seg);
+    const bool y_vec = sy == 1 && (reinterpret_cast<uintptr_t>(yr + seg) % (sizeof(Y) * V) == 0);
+    VecY* qv = reinterpret_cast<VecY*>(yr + seg);
 #pragma unroll
-        for (int k = 0; k < KV; ++k) {
+    for (int k = 0; k < KV; ++k) {
+        const int64_t i0 = seg + static_cast<int64_t>(k * kWave + lane) * V;
+        if (y_vec && i0 + V <= n) {
             VecY a;
 #pragma unroll
             for (int e = 0; e < V; ++e) a.v[e] = static_cast<Y>(vals[k * V + e]);
-            store_stream(&pv[k * kWave + lane], a);
+            store_stream(&qv[k * kWave + lane], a);
+        } else {
+#pragma unroll
+            for (int e = 0; e < V; ++e)
+                if (i0 + e < n) yr[(i0 + e) * sy] = static_cast<Y>(vals[k * V + e]);
         }
-    } else {
-#pragma unroll
-        for (int k = 0; k < KV; ++k)
-#pragma unroll
-            for (int e = 0; e < V; ++e) {
-                const int64_t i = seg + static_cast<int64_t>(k * kWave + lane) * V + e;
-                if (i < n) yr[i * sy] = static_cast<Y>(vals[k * V + e]);
-            }
     }
 }
 
@@ -369,7 +346,7 @@ __global__ __launch_bounds__(kBlock) void scan_rows_group(
     int64_t rows, int64_t n, int exclusive) {
     static_assert(LANES == 1 || LANES == 4 || LANES == 16 || LANES == kWave, "a thread, a quad, a DPP row or a wavefront");
     using Op = ScanOp<T, K>;
-    constexpr int V = (vec_width<T>() < ITEMS) ? vec_width<T>() : ITEMS;
+    constexpr int V = (scan_vec<T, X, Y>() < ITEMS) ? scan_vec<T, X, Y>() : ITEMS;
     constexpr int KV = ITEMS / V;
     using VecX = Vec<X, V>;
     using VecY = Vec<Y, V>;
@@ -575,10 +552,10 @@ constexpr int64_t kChainTileBytes = DLFX_SCAN_CHAIN_BYTES;
 int64_t tile_elems(size_t elem_size, int64_t n) {
     const int64_t full = 256 * (256 / static_cast<int64_t>(elem_size));
     if (n > full) return kChainTileBytes / static_cast<int64_t>(elem_size);
-    if (n > full / 4) return full;
-    if (n > 1024) return full / 4;
-    if (n > 256) return 1024;
-    return 256;
+    // the smallest of 1, 4, 8, 16, 32, 64 elements per thread that holds the row
+    for (int64_t tile = 256; tile < full; tile *= (tile == 256 ? 4 : 2))
+        if (n <= tile) return tile;
+    return full;
 }
 
 struct ScanLayout {
@@ -595,8 +572,7 @@ ScanLayout scan_layout(size_t elem_size, int64_t m, int64_t n) {
     if (l.tiles_per_row <= 1) {
         l.total = 0;
     } else {
-        size_t sb = elem_size == 4 ? static_cast<size_t>(l.tiles) * 8
-                                   : align_up(static_cast<size_t>(l.tiles) * 4, 256) + static_cast<size_t>(l.tiles) * 2 * elem_size;
+        const size_t sb = static_cast<size_t>(l.tiles) * 2 * elem_size;      // a 64-bit word per 32 bits of the value
         l.total = l.state_off + align_up(sb, 256);
     }
     return l;
@@ -683,14 +659,19 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     const dim3 block(kBlock);
     if (l.tiles_per_row == 1) {
         const dim3 grid(static_cast<unsigned>(m));
-        if (tile == 256)
-            scan_rows_single<T, K, 1, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
-        else if (tile == 1024)
-            scan_rows_single<T, K, 4, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
-        else if (tile == 256 * (FULL / 4))
-            scan_rows_single<T, K, FULL / 4, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
-        else
-            scan_rows_single<T, K, FULL, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
+        auto single = [&](auto items) {
+            constexpr int ITEMS = decltype(items)::value;
+            if constexpr (ITEMS <= FULL)
+                scan_rows_single<T, K, ITEMS, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
+        };
+        switch (tile / 256) {
+        case 1: single(std::integral_constant<int, 1>()); break;
+        case 4: single(std::integral_constant<int, 4>()); break;
+        case 8: single(std::integral_constant<int, 8>()); break;
+        case 16: single(std::integral_constant<int, 16>()); break;
+        case 32: single(std::integral_constant<int, 32>()); break;
+        default: single(std::integral_constant<int, 64>()); break;
+        }
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
     }
