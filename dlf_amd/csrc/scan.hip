@@ -189,6 +189,16 @@ __device__ __forceinline__ void scan_tile(
     // vector (and what lies past the row in its last tile) element by element
     const bool x_vec = sx == 1 && (reinterpret_cast<uintptr_t>(xr + seg) % (sizeof(X) * V) == 0);
     const VecX* pv = reinterpret_cast<const VecX*>(xr + seg);
+    const bool full = n - tile_base >= TILE;               // every element of the tile lies in the row
+    if (full && x_vec) {
+        // the common case apart: all loads issued back to back, nothing to test per vector
+#pragma unroll
+        for (int k = 0; k < KV; ++k) {
+            VecX a = load_stream(&pv[k * kWave + lane]);
+#pragma unroll
+            for (int e = 0; e < V; ++e) vals[k * V + e] = scan_input<T, X, NZ>(a.v[e]);
+        }
+    } else
 #pragma unroll
     for (int k = 0; k < KV; ++k) {
         const int64_t i0 = seg + static_cast<int64_t>(k * kWave + lane) * V;
@@ -311,6 +321,15 @@ __device__ __forceinline__ void scan_tile(
     using VecY = Vec<Y, V>;
     const bool y_vec = sy == 1 && (reinterpret_cast<uintptr_t>(yr + seg) % (sizeof(Y) * V) == 0);
     VecY* qv = reinterpret_cast<VecY*>(yr + seg);
+    if (full && y_vec) {
+#pragma unroll
+        for (int k = 0; k < KV; ++k) {
+            VecY a;
+#pragma unroll
+            for (int e = 0; e < V; ++e) a.v[e] = static_cast<Y>(vals[k * V + e]);
+            store_stream(&qv[k * kWave + lane], a);
+        }
+    } else
 #pragma unroll
     for (int k = 0; k < KV; ++k) {
         const int64_t i0 = seg + static_cast<int64_t>(k * kWave + lane) * V;
