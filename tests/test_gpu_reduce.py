@@ -172,3 +172,30 @@ def test_error_statuses(hip_backend):
     with pytest.raises(DlfxError) as e:
         F.reduce("reduce_log_sum_exp", Xi, [1])
     assert e.value.status == -2
+
+
+def test_int64_mean_of_many_short_rows_truncates_exactly(hip_backend, oracle_backend):
+    """The mean of int64 rows divides the (wrapping) sum by the row length, truncating toward
+    zero.  Sums of every magnitude and sign, including the extremes, over row lengths from 1 to
+    thousands."""
+    from helpers import full_range_i64
+    for n in (1, 2, 3, 7, 64, 1000, 4097):
+        rows = 3000
+        x = full_range_i64(300 + n, rows * n).reshape(rows, n)
+        x[0] = 0
+        x[0, 0] = np.iinfo(np.int64).min                                  # sum = INT64_MIN
+        x[1] = 0
+        x[1, 0] = np.iinfo(np.int64).max
+        x[2] = -1
+        x[3] = 1
+        x[4] = 0
+        x[4, 0] = -(n - 1) if n > 1 else -1                               # a quotient just above -1
+        small = randint(301 + n, (rows - 5) * n // 2, -50, 50).astype(np.int64)
+        x[5:5 + (rows - 5) // 2] = small[: ((rows - 5) // 2) * n].reshape(-1, n)      # quotients near zero, both signs
+        got = F.reduce_mean(Tensor.from_numpy(hip_backend, x), [1]).numpy()
+        want = F.reduce_mean(Tensor.from_numpy(oracle_backend, x), [1]).numpy()
+        assert np.array_equal(got, want), n
+        sums = [int(v) for v in x[5:50].astype(object).sum(axis=1)]
+        wrapped = [((s + 2**63) % 2**64) - 2**63 for s in sums]
+        exact = [abs(s) // n * (1 if s >= 0 else -1) for s in wrapped]
+        assert got[5:50].tolist() == exact
