@@ -926,6 +926,45 @@ __global__ __launch_bounds__(256) void topk_rows_thread(TopkIo<typename BitsOf<E
         if (p < limit) emit_one<K>(io, yr, ir, xr, p, lo[p], li[p]);
 }
 
+// Rows of at most 64 elements side by side in memory and a limit the register lists of
+// topk_cols do not take: a workgroup reads 64 neighbouring rows with coalesced loads (64 rows
+// wide, one axis position at a time) into an LDS tile of images (pitch 65: no bank conflicts
+// either way), each wavefront orders sixteen of them whole (lane l holds element l), and the
+// winners leave the way the rows came, `limit` axis positions deep.
+template <typename E>
+__global__ __launch_bounds__(256) void topk_cols_wave(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> io,
+                                                      int64_t rows, int64_t n, int limit) {
+    using K = typename BitsOf<E>::type;
+    using S = typename BitsOf<E>::storage;
+    constexpr int kind = BitsOf<E>::kind;
+    constexpr int kPitch = kWave + 1;
+    __shared__ K images[kWave * kPitch];
+    __shared__ uint32_t places[kWave * kPitch];
+    const int lane = lane_id();
+    const int w = threadIdx.x / kWave;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kWave;
+    const int r = lane;                                    // this thread's row of the tile in the load and store phases
+    const bool row_live = row0 + r < rows;
+    const int n32 = static_cast<int>(n);
+    const K flip = io.largest ? K(0) : (kind == kKeyFloat ? KeyBits<K>::kSign : ~K(0));
+    const S* xr = io.x + (row_live ? io.xmap.at(row0 + r) : 0);
+    for (int a = w; a < n32; a += 4)
+        images[a * kPitch + r] = row_live ? to_ord<K>(static_cast<K>(widen_bits<K, S>(load_stream(xr + static_cast<int64_t>(a) * io.sx), kind) ^ flip), kind, 1) : K(0);
+    __syncthreads();
+    for (int q = w; q < kWave; q += 4) {                   // row q of the tile, element `lane`
+        K ord[1] = {lane < n32 ? images[lane * kPitch + q] : K(0)};
+        uint32_t ix[1] = {static_cast<uint32_t>(lane)};    // padding: image 0 and an index past the row
+        wave_bitonic_items<true, 1>(ord, ix, [](K ka, uint32_t ia, K kb, uint32_t ib) { return beats<K>(ka, ia, kb, ib) != 0u; });
+        images[lane * kPitch + q] = ord[0];
+        places[lane * kPitch + q] = ix[0];
+    }
+    __syncthreads();
+    if (!row_live) return;
+    S* yr = io.y + io.ymap.at(row0 + r);
+    const int64_t ir = io.imap.at(row0 + r);
+    for (int a = w; a < limit; a += 4) emit_one<K>(io, yr, ir, xr, a, images[a * kPitch + r], places[a * kPitch + r]);
+}
+
 // E: the element type.  ALIGNED: the axis is contiguous and every row starts on a 16-byte
 // boundary (checked on the host), so rows are read with 128-bit loads off one base register.
 //
@@ -1386,6 +1425,15 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
         else if (lim <= 8) DLFX_TOPK_COLS(8);
         else DLFX_TOPK_COLS(16);
 #undef DLFX_TOPK_COLS
+        DLFX_CHECK_LAUNCH();
+        return DLFX_OK;
+    }
+
+    // short rows side by side in memory, a limit beyond the register lists: LDS tiles of 64 rows
+    if (n <= kWave && m >= 4096 && io.sx != 1 && io.sx != -1 && io.xmap.rank >= 1 && io.xmap.strides[io.xmap.rank - 1] == 1 &&
+        io.xmap.dims[io.xmap.rank - 1] >= kWave) {
+        topk_cols_wave<T><<<dim3(static_cast<unsigned>(ceil_div(m, static_cast<int64_t>(kWave)))), dim3(256), 0, stream>>>(
+            io, m, n, static_cast<int>(limit));
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
     }

@@ -202,6 +202,33 @@ def test_rows_side_by_side_in_memory(hip_backend, oracle_backend, n):
     assert np.array_equal(Ih.numpy()[ok], Io.numpy()[ok]) and np.array_equal(Yh.numpy()[ok], Yo.numpy()[ok])
 
 
+@pytest.mark.parametrize("n", [17, 33, 63, 64])
+def test_short_rows_side_by_side_with_a_long_list(hip_backend, oracle_backend, n):
+    """top_k along an outer axis of at most 64 elements with a limit beyond the register lists:
+    tiles of 64 neighbouring rows, one wavefront orders a row whole.  Every element type, both
+    directions, tied columns, a row count that leaves the last tile ragged, a middle axis."""
+    cols = 4096 + 37
+    for dtype in (np.float32, np.int32, np.float64, np.int64, np.float16, np.int16):
+        x = (normal(250 + n, n * cols) * 40).astype(dtype).reshape(n, cols)
+        x[:, 1] = 3
+        x[:, 2] = randint(251 + n, n, 0, 3).astype(dtype)
+        x[:, cols - 1] = np.sort(x[:, cols - 1], kind="stable")
+        Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
+        for k in sorted({17, min(n, 20), n}):
+            for largest in (True, False):
+                Yh, Ih = F.top_k(Xh, k, 0, largest)
+                Yo, Io = F.top_k(Xo, k, 0, largest)
+                assert np.array_equal(Ih.numpy(), Io.numpy()), (dtype, k, largest)
+                assert np.array_equal(Yh.numpy().view(np.uint8), Yo.numpy().view(np.uint8))
+    a = (normal(252, 2 * n * 2100) * 9).astype(np.float32).reshape(2, n, 2100)
+    a[1, n // 2, :] = -0.0
+    a[1, 0, :] = 0.0
+    T, O = Tensor.from_numpy(hip_backend, a), Tensor.from_numpy(oracle_backend, a)
+    Yh, Ih = F.top_k(T, 17, 1, True, index_dtype=np.int64)
+    Yo, Io = F.top_k(O, 17, 1, True, index_dtype=np.int64)
+    assert np.array_equal(Ih.numpy(), Io.numpy()) and np.array_equal(Yh.numpy().view(np.uint32), Yo.numpy().view(np.uint32))
+
+
 def test_many_rows_side_by_side_one_wave_per_block(hip_backend, oracle_backend):
     x = (normal(240, 64 * 524291) * 5).astype(np.float32).reshape(64, 524291)
     Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
