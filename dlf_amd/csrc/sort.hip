@@ -194,38 +194,64 @@ __global__ __launch_bounds__(kBlock) void sort_histogram(PassIo<K> io, int64_t n
 // b handles one (row, pass) pair.  moves[b] receives the bits of the digit that are not the
 // same in all keys of the row: none means the pass would not change the order of the row (the
 // row then skips it), and the ranking only needs to look at those bits.  `all_bits` forces
-// every pass of every row to run.
-__global__ __launch_bounds__(kRadix) void sort_bases(uint32_t* __restrict__ ghist, uint32_t* __restrict__ moves, int all_bits) {
+// every pass of every row to run.  largest[b] receives the count of the most frequent digit.
+__global__ __launch_bounds__(kRadix) void sort_bases(uint32_t* __restrict__ ghist, uint32_t* __restrict__ moves,
+                                                     uint32_t* __restrict__ largest, int all_bits) {
     __shared__ uint32_t wave_tot[kRadix / kWave];
-    __shared__ uint32_t wave_or[kRadix / kWave], wave_and[kRadix / kWave];
+    __shared__ uint32_t wave_or[kRadix / kWave], wave_and[kRadix / kWave], wave_max[kRadix / kWave];
     uint32_t* g = ghist + static_cast<int64_t>(blockIdx.x) * kRadix;
     const uint32_t v = g[threadIdx.x];
     const uint32_t incl = wave_scan_inclusive(v, 0u, [](uint32_t a, uint32_t b) { return a + b; });
     const uint32_t ors = wave_reduce(v ? threadIdx.x : 0u, [](uint32_t a, uint32_t b) { return a | b; });
     const uint32_t ands = wave_reduce(v ? threadIdx.x : 0xffu, [](uint32_t a, uint32_t b) { return a & b; });
+    const uint32_t most = wave_reduce(v, [](uint32_t a, uint32_t b) { return a > b ? a : b; });
     const int w = threadIdx.x / kWave;
     if (lane_id() == kWave - 1) {
         wave_tot[w] = incl;
         wave_or[w] = ors;
         wave_and[w] = ands;
+        wave_max[w] = most;
     }
     __syncthreads();
     uint32_t pre = 0;
     for (int i = 0; i < w; ++i) pre += wave_tot[i];
     g[threadIdx.x] = pre + incl - v;
     if (threadIdx.x == 0) {
-        uint32_t o = 0, a = 0xffu;
+        uint32_t o = 0, a = 0xffu, mx = 0;
         for (int i = 0; i < kRadix / kWave; ++i) {
             o |= wave_or[i];
             a &= wave_and[i];
+            mx = wave_max[i] > mx ? wave_max[i] : mx;
         }
         moves[blockIdx.x] = all_bits ? 0xffu : (o ^ a);
+        largest[blockIdx.x] = mx;                         // keys of the row that share the most frequent digit
     }
 }
 
 __global__ __launch_bounds__(kBlock) void sort_clear(uint32_t* __restrict__ p, int64_t words) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     if (i < words) p[i] = 0u;
+}
+
+// Rows whose keys the most significant varying digit spreads into runs ("buckets") of at most
+// `cap` keys are sorted most significant digit first: one tiled pass on that digit leaves the
+// buckets, in source order, in the first ping-pong buffer, and a workgroup then sorts each
+// bucket by its lower digits on chip (sort_buckets) and writes the outputs: the keys cross HBM
+// five times instead of 2 * passes + 1 times.  Returns that digit's pass for such a row, -1
+// for a row that takes the least-significant-digit-first passes (cap 0: every row).
+template <int P>
+__device__ __forceinline__ int msd_digit(const uint32_t* __restrict__ row_moves, const uint32_t* __restrict__ row_largest, uint32_t cap) {
+    if (cap == 0u) return -1;
+    int q = -1, varying = 0;
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        if (row_moves[p] != 0u) {
+            q = p;
+            ++varying;
+        }
+    }
+    if (varying < 2 || row_largest[q] > cap) return -1;
+    return q;
 }
 
 // ------------------------------------------------------------------ one pass
@@ -256,6 +282,7 @@ template <typename K, bool PAIRS, int ITEMS, bool LAST>
 __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SORT_WAVES))) void sort_pass(PassIo<K> io, int pass, int64_t rows, int64_t n, int64_t tiles_per_row,
                                                     const uint32_t* __restrict__ gbase,
                                                     const uint32_t* __restrict__ moves,
+                                                    const uint32_t* __restrict__ largest, uint32_t bucket_cap,
                                                     uint32_t* __restrict__ status, int poll_limit) {
     constexpr int P = KeyTraits<K>::kPasses;
     constexpr int TILE = kPassBlock * ITEMS;
@@ -269,8 +296,14 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
     const int64_t t = blockIdx.x / rows;
     const int64_t row = blockIdx.x - t * rows;
     const uint32_t* row_moves = moves + row * P;
+    // a row sorted most significant digit first runs that digit's pass only, from the input
+    // into the first buffer
+    const int msd = msd_digit<P>(row_moves, largest + row * P, bucket_cap);
+    const bool to_buckets = msd >= 0;
+    if (to_buckets && pass != msd) return;
     int ran = 0;            // passes before this one that this row ran
-    for (int p = 0; p < pass; ++p) ran += row_moves[p] ? 1 : 0;
+    if (!to_buckets)
+        for (int p = 0; p < pass; ++p) ran += row_moves[p] ? 1 : 0;
     if (!LAST && row_moves[pass] == 0u) return;
     const bool first = ran == 0;
     const K* __restrict__ src_keys = first ? nullptr : io.kbuf[(ran - 1) & 1];
@@ -531,7 +564,7 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) pay[k] = sm.vals[k * kPassBlock + tid];
     }
-    if constexpr (!LAST) {
+    if (!LAST || to_buckets) {
         K* dk = dst_keys + row_off;
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k)
@@ -542,7 +575,7 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
             for (int k = 0; k < ITEMS; ++k)
                 if (full || k * kPassBlock + tid < valid) dv[at[k]] = pay[k];
         }
-    } else {
+    } else if constexpr (LAST) {
         if (io.y) {
             K* yrow = io.y + io.ymap.at(row);
 #pragma unroll
@@ -583,45 +616,27 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
 // waves' counts, scatter through LDS, reload in element order.  Digits that are the same in
 // the whole row are skipped.  Element e of the row is item e / 64 % ITEMS of lane e % 64 of
 // wave e / (64 * ITEMS), before and after every pass.
-template <typename K, bool PAIRS, int ITEMS>
+template <typename K, bool PAIRS, int ITEMS, int WAVES = 4>
 struct SmallShared {
-    uint32_t wave_hist[4][kRadix];
-    uint32_t scan_tmp[4];
-    K wave_or[4], wave_and[4];
-    K keys[256 * ITEMS];
-    uint32_t vals[PAIRS ? 256 * ITEMS : 1];
+    uint32_t wave_hist[WAVES][kRadix];
+    uint32_t scan_tmp[kRadix / kWave];
+    K wave_or[WAVES], wave_and[WAVES];
+    K keys[WAVES * kWave * ITEMS];
+    uint32_t vals[PAIRS ? WAVES * kWave * ITEMS : 1];
 };
 
-template <typename K, bool PAIRS, int ITEMS>
-__global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t rows, int64_t n) {
-    constexpr int P = KeyTraits<K>::kPasses;
-    constexpr int CAP = 256 * ITEMS;
-    static_assert(ITEMS % 2 == 0, "items are ranked in pairs");
-    __shared__ SmallShared<K, PAIRS, ITEMS> sm;
+// The passes of a workgroup-resident sort: key[] / val[] hold the row (or bucket) in element
+// order before and after; `ors` / `ands` are this thread's OR / AND over its valid keys, `top`
+// the number of low digits that may differ (digits from `top` up are known to be equal).
+// The workgroup has WAVES wavefronts (4 or 8).
+template <typename K, bool PAIRS, int ITEMS, int WAVES = 4>
+__device__ __forceinline__ void sort_in_workgroup(SmallShared<K, PAIRS, ITEMS, WAVES>& sm, K (&key)[ITEMS], uint32_t (&val)[PAIRS ? ITEMS : 1],
+                                                  K ors, K ands, bool padded, int top) {
+    static_assert(WAVES * kWave >= kRadix, "a thread per digit");
     const int tid = threadIdx.x;
     const int lane = lane_id();
     const int w = tid / kWave;
-    const int64_t row = block_of(io);
-    if (row >= rows) return;                               // (the grid is rounded up to a multiple of 8)
-    const K* xrow = io.x + io.xmap.at(row);
-    const int valid = static_cast<int>(n);
-    const bool padded = valid < CAP;
     const int seg = w * kWave * ITEMS + lane;
-
-    K key[ITEMS];
-    uint32_t val[PAIRS ? ITEMS : 1];
-    K ors = 0, ands = ~K(0);
-#pragma unroll
-    for (int k = 0; k < ITEMS; ++k) {
-        const int e = seg + k * kWave;
-        key[k] = ~K(0);                                   // padding sorts last in every pass that runs
-        if (e < valid) {
-            key[k] = key_of_element<K>(io, xrow[static_cast<int64_t>(e) * io.sx]);
-            ors |= key[k];
-            ands &= key[k];
-        }
-        if constexpr (PAIRS) val[k] = static_cast<uint32_t>(e);
-    }
     ors = wave_reduce(ors, [](K a, K b) { return static_cast<K>(a | b); });
     ands = wave_reduce(ands, [](K a, K b) { return static_cast<K>(a & b); });
     if (lane == 0) {
@@ -629,15 +644,21 @@ __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t row
         sm.wave_and[w] = ands;
     }
     __syncthreads();
-    const K differ = static_cast<K>((sm.wave_or[0] | sm.wave_or[1] | sm.wave_or[2] | sm.wave_or[3]) &
-                                    ~(sm.wave_and[0] & sm.wave_and[1] & sm.wave_and[2] & sm.wave_and[3]));
+    K any = 0, all = ~K(0);
+#pragma unroll
+    for (int i = 0; i < WAVES; ++i) {
+        any |= sm.wave_or[i];
+        all &= sm.wave_and[i];
+    }
+    const K differ = static_cast<K>(any & ~all);
+    const bool owner = tid < kRadix;                       // thread d < 256 owns digit d
 
-    for (int pass = 0; pass < P; ++pass) {
+    for (int pass = 0; pass < top; ++pass) {
         const int shift = 8 * pass;
         const uint32_t moves = static_cast<uint32_t>(differ >> shift) & 0xffu;
         if (moves == 0u) continue;                        // this digit is the same in the whole row
         const uint32_t vary = padded ? 0xffu : moves;     // padding differs from the row in other bits too
-        for (int i = tid; i < 4 * kRadix; i += 256) (&sm.wave_hist[0][0])[i] = 0;
+        for (int i = tid; i < WAVES * kRadix; i += WAVES * kWave) (&sm.wave_hist[0][0])[i] = 0;
         __syncthreads();
 
         // ---- rank inside the wave, in element order
@@ -676,22 +697,26 @@ __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t row
 
         // ---- thread d owns digit d: where the digit starts in the row, and each wave's share of it
         {
-            uint32_t wave_count[4];
+            uint32_t wave_count[WAVES];
             uint32_t count = 0;
+            if (owner) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                wave_count[i] = sm.wave_hist[i][tid];
-                count += wave_count[i];
+                for (int i = 0; i < WAVES; ++i) {
+                    wave_count[i] = sm.wave_hist[i][tid];
+                    count += wave_count[i];
+                }
             }
             const uint32_t incl = wave_scan_inclusive(count, 0u, [](uint32_t a, uint32_t b) { return a + b; });
-            if (lane == kWave - 1) sm.scan_tmp[w] = incl;
+            if (owner && lane == kWave - 1) sm.scan_tmp[w] = incl;
             __syncthreads();
-            uint32_t run = incl - count;
-            for (int i = 0; i < w; ++i) run += sm.scan_tmp[i];
+            if (owner) {
+                uint32_t run = incl - count;
+                for (int i = 0; i < w; ++i) run += sm.scan_tmp[i];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                sm.wave_hist[i][tid] = run;
-                run += wave_count[i];
+                for (int i = 0; i < WAVES; ++i) {
+                    sm.wave_hist[i][tid] = run;
+                    run += wave_count[i];
+                }
             }
         }
         __syncthreads();
@@ -711,6 +736,40 @@ __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t row
         }
         // (the three barriers of the next pass lie between these reads and its scatter)
     }
+
+}
+
+template <typename K, bool PAIRS, int ITEMS>
+__global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t rows, int64_t n) {
+    constexpr int P = KeyTraits<K>::kPasses;
+    constexpr int CAP = 256 * ITEMS;
+    static_assert(ITEMS % 2 == 0, "items are ranked in pairs");
+    __shared__ SmallShared<K, PAIRS, ITEMS> sm;
+    const int tid = threadIdx.x;
+    const int lane = lane_id();
+    const int w = tid / kWave;
+    const int64_t row = block_of(io);
+    if (row >= rows) return;                               // (the grid is rounded up to a multiple of 8)
+    const K* xrow = io.x + io.xmap.at(row);
+    const int valid = static_cast<int>(n);
+    const bool padded = valid < CAP;
+    const int seg = w * kWave * ITEMS + lane;
+
+    K key[ITEMS];
+    uint32_t val[PAIRS ? ITEMS : 1];
+    K ors = 0, ands = ~K(0);
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const int e = seg + k * kWave;
+        key[k] = ~K(0);                                   // padding sorts last in every pass that runs
+        if (e < valid) {
+            key[k] = key_of_element<K>(io, xrow[static_cast<int64_t>(e) * io.sx]);
+            ors |= key[k];
+            ands &= key[k];
+        }
+        if constexpr (PAIRS) val[k] = static_cast<uint32_t>(e);
+    }
+    sort_in_workgroup<K, PAIRS, ITEMS>(sm, key, val, ors, ands, padded, P);
 
     // ---- write
     if (io.y) {
@@ -736,6 +795,80 @@ __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t row
                 if (e < valid) {
                     if (io.idx64) static_cast<int64_t*>(io.idx)[irow + static_cast<int64_t>(e) * io.si] = static_cast<int64_t>(val[k]);
                     else static_cast<int32_t*>(io.idx)[irow + static_cast<int64_t>(e) * io.si] = static_cast<int32_t>(val[k]);
+                }
+            }
+        }
+    }
+}
+
+// Second half of the most-significant-digit-first sort: workgroup (row, d) takes the run of
+// keys whose digit `msd` is d - at most 64 * WAVES * ITEMS keys, in source order, in the first
+// ping-pong buffer - sorts it by the lower digits on chip and writes it to the strided outputs
+// at the run's place in the row.  Rows that took the other way leave at once.
+template <typename K, bool PAIRS, int ITEMS, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void sort_buckets(PassIo<K> io, int64_t n, const uint32_t* __restrict__ gbase,
+                                                    const uint32_t* __restrict__ moves, const uint32_t* __restrict__ largest) {
+    constexpr int P = KeyTraits<K>::kPasses;
+    constexpr int CAP = WAVES * kWave * ITEMS;
+    __shared__ SmallShared<K, PAIRS, ITEMS, WAVES> sm;
+    const int tid = threadIdx.x;
+    const int lane = lane_id();
+    const int w = tid / kWave;
+    const int64_t row = blockIdx.x / kRadix;
+    const int d = static_cast<int>(blockIdx.x % kRadix);
+    const int msd = msd_digit<P>(moves + row * P, largest + row * P, static_cast<uint32_t>(CAP));
+    if (msd < 0) return;
+    const uint32_t* starts = gbase + (row * P + msd) * kRadix;
+    const int64_t begin = starts[d];
+    const int64_t end = d + 1 < kRadix ? static_cast<int64_t>(starts[d + 1]) : n;
+    const int valid = static_cast<int>(end - begin);
+    if (valid <= 0 || valid > CAP) return;                 // (never more than CAP: msd_digit saw the largest run)
+    const bool padded = valid < CAP;
+    const int seg = w * kWave * ITEMS + lane;
+    const K* src = io.kbuf[0] + row * n + begin;
+    const uint32_t* vsrc = PAIRS ? io.vbuf[0] + row * n + begin : nullptr;
+
+    K key[ITEMS];
+    uint32_t val[PAIRS ? ITEMS : 1];
+    K ors = 0, ands = ~K(0);
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const int e = seg + k * kWave;
+        key[k] = ~K(0);                                   // padding sorts last in every pass that runs
+        if constexpr (PAIRS) val[k] = 0u;
+        if (e < valid) {
+            key[k] = src[e];
+            if constexpr (PAIRS) val[k] = vsrc[e];
+            ors |= key[k];
+            ands &= key[k];
+        }
+    }
+    sort_in_workgroup<K, PAIRS, ITEMS, WAVES>(sm, key, val, ors, ands, padded, msd);
+
+    if (io.y) {
+        K* yrow = io.y + io.ymap.at(row);
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const int e = seg + k * kWave;
+            if (e < valid) {
+                K bits = decode_key<K>(key[k], io.kind, io.descending);
+                if constexpr (PAIRS) {
+                    if (io.restore_zero && static_cast<K>(bits << 1) == 0)
+                        bits = (io.x + io.xmap.at(row))[static_cast<int64_t>(val[k]) * io.sx];
+                }
+                yrow[(begin + e) * io.sy] = bits;
+            }
+        }
+    }
+    if constexpr (PAIRS) {
+        if (io.idx) {
+            const int64_t irow = io.imap.at(row);
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) {
+                const int e = seg + k * kWave;
+                if (e < valid) {
+                    if (io.idx64) static_cast<int64_t*>(io.idx)[irow + (begin + e) * io.si] = static_cast<int64_t>(val[k]);
+                    else static_cast<int32_t*>(io.idx)[irow + (begin + e) * io.si] = static_cast<int32_t>(val[k]);
                 }
             }
         }
@@ -894,6 +1027,20 @@ int g_sort_wave_rows = 512;
 
 constexpr int64_t kSmallRow = 4096;      // longest row sort_rows_small takes
 
+// Most significant digit first: capacities (keys per thread) of the two bucket kernels, and the
+// mean run length above which a row may go that way.
+// The large kernel holds 18 keys per thread in 4 wavefronts; with indices that many registers
+// leave one wavefront per SIMD, so pairs take 10 per thread in 8 wavefronts.
+constexpr int kBucketItemsSmall = 8, kBucketWavesSmall = 4;
+constexpr int bucket_items_large(bool pairs) { return pairs ? 10 : 18; }
+constexpr int bucket_waves_large(bool pairs) { return pairs ? 8 : 4; }
+constexpr int kBucketCapSmall = kBucketItemsSmall * kBucketWavesSmall * kWave;
+constexpr int bucket_cap_large(bool pairs) { return bucket_items_large(pairs) * bucket_waves_large(pairs) * kWave; }
+constexpr int64_t kBucketMinMean = 1024;
+int g_sort_buckets = 1;
+template <typename K>
+constexpr bool kBucketKeys = sizeof(K) >= 4;     // two-digit keys gain nothing
+
 template <typename K, bool PAIRS>
 int launch_small(hipStream_t stream, const PassIo<K>& io_in, int64_t m, int64_t n) {
     PassIo<K> io = io_in;
@@ -935,7 +1082,7 @@ constexpr int tile_items(size_t key_size, bool pairs) { return ((key_size == 8 &
 
 struct SortLayout {
     int64_t tiles_per_row;
-    size_t moves_off, hist_off, hist_bytes, status_off, status_bytes, keys_off[2], vals_off[2], total;
+    size_t moves_off, largest_off, hist_off, hist_bytes, status_off, status_bytes, keys_off[2], vals_off[2], total;
 };
 
 SortLayout sort_layout(size_t key_size, bool pairs, int64_t m, int64_t n) {
@@ -945,6 +1092,8 @@ SortLayout sort_layout(size_t key_size, bool pairs, int64_t m, int64_t n) {
     l.tiles_per_row = ceil_div(n, tile);
     size_t off = 0;
     l.moves_off = off;           // one word per (row, pass): does the pass move the row's keys
+    off += align_up(static_cast<size_t>(m) * passes * 4, 256);
+    l.largest_off = off;         // one word per (row, pass): keys sharing the most frequent digit
     off += align_up(static_cast<size_t>(m) * passes * 4, 256);
     l.hist_off = off;
     l.hist_bytes = static_cast<size_t>(m) * passes * kRadix * 4;
@@ -1046,8 +1195,18 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     DLFX_CHECK_LAUNCH();
     // a pass that moves nothing may only be left out when no pass reads the input while
     // another tile of the same pass writes the output over it
-    sort_bases<<<dim3(static_cast<unsigned>(m * P)), dim3(kRadix), 0, stream>>>(ghist, moves, y_over_x ? 1 : 0);
+    uint32_t* largest = reinterpret_cast<uint32_t*>(base + l.largest_off);
+    sort_bases<<<dim3(static_cast<unsigned>(m * P)), dim3(kRadix), 0, stream>>>(ghist, moves, largest, y_over_x ? 1 : 0);
     DLFX_CHECK_LAUNCH();
+    // rows long enough for an even leading digit to leave runs of 1024 to 4096 keys may go most
+    // significant digit first (each row decides on the device from its histogram); the bucket
+    // kernel's capacity is picked from the mean run length with an eighth of headroom
+    uint32_t bucket_cap = 0;
+    if (kBucketKeys<K> && !y_over_x && g_sort_buckets && m * kRadix <= 0x7fffffffLL) {
+        const int64_t mean = ceil_div(n, static_cast<int64_t>(kRadix));
+        if (mean > kBucketMinMean && mean + mean / 8 <= bucket_cap_large(a.pairs))
+            bucket_cap = static_cast<uint32_t>(mean + mean / 8 <= kBucketCapSmall ? kBucketCapSmall : bucket_cap_large(a.pairs));
+    }
 
     io.kbuf[0] = reinterpret_cast<K*>(base + l.keys_off[0]);
     io.kbuf[1] = reinterpret_cast<K*>(base + l.keys_off[1]);
@@ -1057,14 +1216,28 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     for (int p = 0; p < P; ++p) {
         if (p < P - 1) {
             if (a.pairs)
-                sort_pass<K, true, IP, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
+                sort_pass<K, true, IP, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
             else
-                sort_pass<K, false, IK, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
+                sort_pass<K, false, IK, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
         } else {
             if (a.pairs)
-                sort_pass<K, true, IP, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
+                sort_pass<K, true, IP, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
             else
-                sort_pass<K, false, IK, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
+                sort_pass<K, false, IK, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
+        }
+        DLFX_CHECK_LAUNCH();
+    }
+    if constexpr (kBucketKeys<K>) if (bucket_cap != 0u) {
+        const dim3 bgrid(static_cast<unsigned>(m * kRadix));
+        if (bucket_cap == kBucketCapSmall) {
+            constexpr int I = kBucketItemsSmall, W = kBucketWavesSmall;
+            if (a.pairs) sort_buckets<K, true, I, W><<<bgrid, dim3(W * kWave), 0, stream>>>(io, n, ghist, moves, largest);
+            else sort_buckets<K, false, I, W><<<bgrid, dim3(W * kWave), 0, stream>>>(io, n, ghist, moves, largest);
+        } else {
+            constexpr int BIP = bucket_items_large(true), BWP = bucket_waves_large(true);
+            constexpr int BIK = bucket_items_large(false), BWK = bucket_waves_large(false);
+            if (a.pairs) sort_buckets<K, true, BIP, BWP><<<bgrid, dim3(BWP * kWave), 0, stream>>>(io, n, ghist, moves, largest);
+            else sort_buckets<K, false, BIK, BWK><<<bgrid, dim3(BWK * kWave), 0, stream>>>(io, n, ghist, moves, largest);
         }
         DLFX_CHECK_LAUNCH();
     }
@@ -1089,6 +1262,10 @@ int sort_entry(hipStream_t stream, int dtype, const SortArgs& a0, void* scratch,
 bool set_sort_tuning(const char* key, int64_t value) {
     if (!std::strcmp(key, "sort_poll_limit") && value >= 0 && value <= (1 << 30)) {
         g_sort_poll_limit = static_cast<int>(value);
+        return true;
+    }
+    if (!std::strcmp(key, "sort_buckets") && value >= 0 && value <= 1) {
+        g_sort_buckets = static_cast<int>(value);
         return true;
     }
     if (!std::strcmp(key, "sort_wave_rows") && value >= 0 && value <= 512) {

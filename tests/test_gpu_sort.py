@@ -161,6 +161,50 @@ def test_rows_leave_out_passes_that_move_nothing(hip_backend, oracle_backend, dt
     assert np.array_equal(Ih.numpy(), np.argsort(x, axis=-1, kind="stable"))
 
 
+@pytest.mark.parametrize("dtype", [np.int64, np.float32, np.int32, np.float64])
+@pytest.mark.parametrize("n", [300000, 1 << 20])
+def test_long_rows_sorted_leading_digit_first(hip_backend, dtype, n):
+    """Rows of 2^18 to 2^20 keys whose leading digit spreads them evenly take one tiled pass on
+    that digit and finish every run of equal digits on chip; rows it does not spread (or that
+    vary in one digit only) take the least-significant-digit-first passes in the same call.
+    Checked against numpy's stable sort and against the same call with that route switched off."""
+    if np.dtype(dtype).kind == "i":
+        wide = full_range_i64(300, n).astype(dtype)                   # even leading digit
+        lopsided = (full_range_i64(301, n) >> 40).astype(dtype)       # (int64) three digits vary, the top one in two values
+        narrow = randint(302, n, 0, 60000).astype(dtype)              # two low digits vary: leading digit of those spreads evenly
+    else:
+        wide = np.ldexp(uniform01(300, n) + 1.0, randint(303, n, -100, 100).astype(np.int32)).astype(dtype) * np.where(randint(304, n, 0, 2) > 0, 1, -1).astype(dtype)
+        lopsided = (normal(301, n) * 1e3).astype(dtype)               # the sign and exponent byte takes few values
+        narrow = (1.0 + randint(302, n, 0, 60000) / 65536.0).astype(dtype)
+    ties = wide.copy()
+    ties[1::2] = ties[0::2][: ties[1::2].size]                        # every key twice: the order of equals shows
+    one_digit = randint(305, n, 0, 200).astype(dtype)
+    x = np.stack([wide, lopsided, ties, one_digit, narrow, wide[::-1].copy()])
+    Xh = Tensor.from_numpy(hip_backend, x)
+    want = np.sort(x, axis=-1, kind="stable")
+    order = np.argsort(x, axis=-1, kind="stable")
+    assert np.array_equal(F.sort(Xh, -1).numpy().view(np.uint8), want.view(np.uint8))
+    Yh, Ih = F.argsort(Xh, -1, False, with_values=True, index_dtype=np.int64)
+    assert np.array_equal(Ih.numpy(), order) and np.array_equal(Yh.numpy().view(np.uint8), want.view(np.uint8))
+    got = {}
+    for route in (1, 0):
+        hip_backend.set_tuning("sort_buckets", route)
+        try:
+            Yd, Id = F.argsort(Xh, -1, True, with_values=True)
+            got[route] = (F.sort(Xh, -1, True).numpy(), Yd.numpy(), Id.numpy(), F.argsort(Xh, -1).numpy())
+        finally:
+            hip_backend.set_tuning("sort_buckets", 1)
+    for a, b in zip(got[1], got[0]):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+    assert np.array_equal(got[1][0].view(np.uint8), np.ascontiguousarray(want[:, ::-1]).view(np.uint8))
+    assert np.array_equal(np.take_along_axis(x, got[1][2].astype(np.int64), -1).view(np.uint8), got[1][1].view(np.uint8))
+    assert np.array_equal(got[1][3], order)
+    # strided outputs (a transposed destination) and an input view with a step
+    Zh = Tensor.from_numpy(hip_backend, np.zeros((n // 2, 6), dtype=dtype)).transpose([1, 0])
+    F.sort(Xh.slice([0], [n], [1], [2]).flip([1]), -1, out=Zh)
+    assert np.array_equal(np.ascontiguousarray(Zh.numpy()).view(np.uint8), np.sort(x[:, 0:n:2], axis=-1).view(np.uint8))
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64, np.float16])
 def test_nans_take_the_place_of_their_bit_pattern(hip_backend, dtype):
     """The reference's comparisons do not order NaNs (std::sort on them is undefined).  The radix
