@@ -627,12 +627,19 @@ struct SmallShared {
 
 // The passes of a workgroup-resident sort: key[] / val[] hold the row (or bucket) in element
 // order before and after; `ors` / `ands` are this thread's OR / AND over its valid keys, `top`
-// the number of low digits that may differ (digits from `top` up are known to be equal).
-// The workgroup has WAVES wavefronts (4 or 8).
+// the number of low digits that may differ (digits from `top` up are known to be equal),
+// `valid` the number of keys that are not padding.  The workgroup has WAVES wavefronts (4 or 8).
+//
+// When more digits vary than `valid` distinct keys need to tell them apart (with 2^6 to spare
+// over the square of `valid`, so that evenly spread keys rarely collide), the leading ones of
+// the varying digits are sorted first: if no two neighbours of the result agree in all of
+// them, the order is final and the lower digits never ran.  Otherwise every digit runs from
+// that arrangement, which the passes so far left in source order among equal keys.
 template <typename K, bool PAIRS, int ITEMS, int WAVES = 4>
 __device__ __forceinline__ void sort_in_workgroup(SmallShared<K, PAIRS, ITEMS, WAVES>& sm, K (&key)[ITEMS], uint32_t (&val)[PAIRS ? ITEMS : 1],
-                                                  K ors, K ands, bool padded, int top) {
+                                                  K ors, K ands, int valid, int top) {
     static_assert(WAVES * kWave >= kRadix, "a thread per digit");
+    const bool padded = valid < WAVES * kWave * ITEMS;
     const int tid = threadIdx.x;
     const int lane = lane_id();
     const int w = tid / kWave;
@@ -653,96 +660,116 @@ __device__ __forceinline__ void sort_in_workgroup(SmallShared<K, PAIRS, ITEMS, W
     const K differ = static_cast<K>(any & ~all);
     const bool owner = tid < kRadix;                       // thread d < 256 owns digit d
 
-    for (int pass = 0; pass < top; ++pass) {
-        const int shift = 8 * pass;
-        const uint32_t moves = static_cast<uint32_t>(differ >> shift) & 0xffu;
-        if (moves == 0u) continue;                        // this digit is the same in the whole row
-        const uint32_t vary = padded ? 0xffu : moves;     // padding differs from the row in other bits too
-        for (int i = tid; i < WAVES * kRadix; i += WAVES * kWave) (&sm.wave_hist[0][0])[i] = 0;
-        __syncthreads();
-
-        // ---- rank inside the wave, in element order
-        uint32_t rank[ITEMS];
-#pragma unroll
-        for (int k0 = 0; k0 < ITEMS; k0 += 2) {
-            uint32_t d[2], before[2], cnt[2];
-#pragma unroll
-            for (int j = 0; j < 2; ++j) d[j] = static_cast<uint32_t>(key[k0 + j] >> shift) & 0xffu;
-            uint32_t peers_lo[2] = {0xffffffffu, 0xffffffffu}, peers_hi[2] = {0xffffffffu, 0xffffffffu};
-            for (uint32_t bits = vary; bits != 0u; bits &= bits - 1u) {
-                const uint32_t b = static_cast<uint32_t>(__builtin_ctz(bits));
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const int32_t ones = __builtin_amdgcn_sbfe(static_cast<int32_t>(d[j]), b, 1u);
-                    const unsigned long long vote = __ballot(ones < 0);
-                    peers_lo[j] &= ~(static_cast<uint32_t>(vote) ^ static_cast<uint32_t>(ones));
-                    peers_hi[j] &= ~(static_cast<uint32_t>(vote >> 32) ^ static_cast<uint32_t>(ones));
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                before[j] = __builtin_amdgcn_mbcnt_hi(peers_hi[j], __builtin_amdgcn_mbcnt_lo(peers_lo[j], 0u));
-                cnt[j] = static_cast<uint32_t>(__popc(peers_lo[j]) + __popc(peers_hi[j]));
-            }
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const uint32_t seen = sm.wave_hist[w][d[j]];
-                rank[k0 + j] = seen + before[j];
-                __builtin_amdgcn_wave_barrier();
-                if (before[j] == 0) sm.wave_hist[w][d[j]] = seen + cnt[j];
-                __builtin_amdgcn_wave_barrier();
-            }
+    int first = 0;                                         // lowest digit of this round of passes
+    if constexpr (sizeof(K) > 4) {
+        const int enough = (2 * (32 - __builtin_clz(static_cast<uint32_t>(valid > 1 ? valid - 1 : 1))) + 6 + 7) / 8;
+        int varying = 0;
+        for (int p = top - 1; p >= 0; --p) {
+            if ((static_cast<uint32_t>(differ >> (8 * p)) & 0xffu) != 0u && ++varying == enough) first = p;
         }
-        __syncthreads();
-
-        // ---- thread d owns digit d: where the digit starts in the row, and each wave's share of it
-        {
-            uint32_t wave_count[WAVES];
-            uint32_t count = 0;
-            if (owner) {
-#pragma unroll
-                for (int i = 0; i < WAVES; ++i) {
-                    wave_count[i] = sm.wave_hist[i][tid];
-                    count += wave_count[i];
-                }
-            }
-            const uint32_t incl = wave_scan_inclusive(count, 0u, [](uint32_t a, uint32_t b) { return a + b; });
-            if (owner && lane == kWave - 1) sm.scan_tmp[w] = incl;
-            __syncthreads();
-            if (owner) {
-                uint32_t run = incl - count;
-                for (int i = 0; i < w; ++i) run += sm.scan_tmp[i];
-#pragma unroll
-                for (int i = 0; i < WAVES; ++i) {
-                    sm.wave_hist[i][tid] = run;
-                    run += wave_count[i];
-                }
-            }
-        }
-        __syncthreads();
-
-        // ---- scatter to the sorted position, reload in element order
-#pragma unroll
-        for (int k = 0; k < ITEMS; ++k) {
-            const uint32_t pos = sm.wave_hist[w][static_cast<uint32_t>(key[k] >> shift) & 0xffu] + rank[k];
-            sm.keys[pos] = key[k];
-            if constexpr (PAIRS) sm.vals[pos] = val[k];
-        }
-        __syncthreads();
-#pragma unroll
-        for (int k = 0; k < ITEMS; ++k) {
-            key[k] = sm.keys[seg + k * kWave];
-            if constexpr (PAIRS) val[k] = sm.vals[seg + k * kWave];
-        }
-        // (the three barriers of the next pass lie between these reads and its scatter)
+        if (varying <= enough) first = 0;
     }
 
+    for (;;) {
+        for (int pass = first; pass < top; ++pass) {
+            const int shift = 8 * pass;
+            const uint32_t moves = static_cast<uint32_t>(differ >> shift) & 0xffu;
+            if (moves == 0u) continue;                        // this digit is the same in the whole row
+            const uint32_t vary = padded ? 0xffu : moves;     // padding differs from the row in other bits too
+            for (int i = tid; i < WAVES * kRadix; i += WAVES * kWave) (&sm.wave_hist[0][0])[i] = 0;
+            __syncthreads();
+
+            // ---- rank inside the wave, in element order
+            uint32_t rank[ITEMS];
+#pragma unroll
+            for (int k0 = 0; k0 < ITEMS; k0 += 2) {
+                uint32_t d[2], before[2], cnt[2];
+#pragma unroll
+                for (int j = 0; j < 2; ++j) d[j] = static_cast<uint32_t>(key[k0 + j] >> shift) & 0xffu;
+                uint32_t peers_lo[2] = {0xffffffffu, 0xffffffffu}, peers_hi[2] = {0xffffffffu, 0xffffffffu};
+                for (uint32_t bits = vary; bits != 0u; bits &= bits - 1u) {
+                    const uint32_t b = static_cast<uint32_t>(__builtin_ctz(bits));
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        const int32_t ones = __builtin_amdgcn_sbfe(static_cast<int32_t>(d[j]), b, 1u);
+                        const unsigned long long vote = __ballot(ones < 0);
+                        peers_lo[j] &= ~(static_cast<uint32_t>(vote) ^ static_cast<uint32_t>(ones));
+                        peers_hi[j] &= ~(static_cast<uint32_t>(vote >> 32) ^ static_cast<uint32_t>(ones));
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    before[j] = __builtin_amdgcn_mbcnt_hi(peers_hi[j], __builtin_amdgcn_mbcnt_lo(peers_lo[j], 0u));
+                    cnt[j] = static_cast<uint32_t>(__popc(peers_lo[j]) + __popc(peers_hi[j]));
+                }
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const uint32_t seen = sm.wave_hist[w][d[j]];
+                    rank[k0 + j] = seen + before[j];
+                    __builtin_amdgcn_wave_barrier();
+                    if (before[j] == 0) sm.wave_hist[w][d[j]] = seen + cnt[j];
+                    __builtin_amdgcn_wave_barrier();
+                }
+            }
+            __syncthreads();
+
+            // ---- thread d owns digit d: where the digit starts in the row, and each wave's share of it
+            {
+                uint32_t wave_count[WAVES];
+                uint32_t count = 0;
+                if (owner) {
+#pragma unroll
+                    for (int i = 0; i < WAVES; ++i) {
+                        wave_count[i] = sm.wave_hist[i][tid];
+                        count += wave_count[i];
+                    }
+                }
+                const uint32_t incl = wave_scan_inclusive(count, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+                if (owner && lane == kWave - 1) sm.scan_tmp[w] = incl;
+                __syncthreads();
+                if (owner) {
+                    uint32_t run = incl - count;
+                    for (int i = 0; i < w; ++i) run += sm.scan_tmp[i];
+#pragma unroll
+                    for (int i = 0; i < WAVES; ++i) {
+                        sm.wave_hist[i][tid] = run;
+                        run += wave_count[i];
+                    }
+                }
+            }
+            __syncthreads();
+
+            // ---- scatter to the sorted position, reload in element order
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) {
+                const uint32_t pos = sm.wave_hist[w][static_cast<uint32_t>(key[k] >> shift) & 0xffu] + rank[k];
+                sm.keys[pos] = key[k];
+                if constexpr (PAIRS) sm.vals[pos] = val[k];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) {
+                key[k] = sm.keys[seg + k * kWave];
+                if constexpr (PAIRS) val[k] = sm.vals[seg + k * kWave];
+            }
+            // (the three barriers of the next pass lie between these reads and its scatter)
+        }
+        if (first == 0) break;
+        // do any two neighbours agree in every digit sorted so far?
+        bool same = false;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const int e = seg + k * kWave;
+            if (e > 0 && e < valid) same |= (sm.keys[e - 1] >> (8 * first)) == (key[k] >> (8 * first));
+        }
+        if (!__syncthreads_or(same ? 1 : 0)) break;
+        first = 0;
+    }
 }
 
 template <typename K, bool PAIRS, int ITEMS>
 __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t rows, int64_t n) {
     constexpr int P = KeyTraits<K>::kPasses;
-    constexpr int CAP = 256 * ITEMS;
     static_assert(ITEMS % 2 == 0, "items are ranked in pairs");
     __shared__ SmallShared<K, PAIRS, ITEMS> sm;
     const int tid = threadIdx.x;
@@ -752,7 +779,6 @@ __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t row
     if (row >= rows) return;                               // (the grid is rounded up to a multiple of 8)
     const K* xrow = io.x + io.xmap.at(row);
     const int valid = static_cast<int>(n);
-    const bool padded = valid < CAP;
     const int seg = w * kWave * ITEMS + lane;
 
     K key[ITEMS];
@@ -769,7 +795,7 @@ __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t row
         }
         if constexpr (PAIRS) val[k] = static_cast<uint32_t>(e);
     }
-    sort_in_workgroup<K, PAIRS, ITEMS>(sm, key, val, ors, ands, padded, P);
+    sort_in_workgroup<K, PAIRS, ITEMS>(sm, key, val, ors, ands, valid, P);
 
     // ---- write
     if (io.y) {
@@ -823,7 +849,6 @@ __global__ __launch_bounds__(WAVES * kWave) void sort_buckets(PassIo<K> io, int6
     const int64_t end = d + 1 < kRadix ? static_cast<int64_t>(starts[d + 1]) : n;
     const int valid = static_cast<int>(end - begin);
     if (valid <= 0 || valid > CAP) return;                 // (never more than CAP: msd_digit saw the largest run)
-    const bool padded = valid < CAP;
     const int seg = w * kWave * ITEMS + lane;
     const K* src = io.kbuf[0] + row * n + begin;
     const uint32_t* vsrc = PAIRS ? io.vbuf[0] + row * n + begin : nullptr;
@@ -843,7 +868,7 @@ __global__ __launch_bounds__(WAVES * kWave) void sort_buckets(PassIo<K> io, int6
             ands &= key[k];
         }
     }
-    sort_in_workgroup<K, PAIRS, ITEMS, WAVES>(sm, key, val, ors, ands, padded, msd);
+    sort_in_workgroup<K, PAIRS, ITEMS, WAVES>(sm, key, val, ors, ands, valid, msd);
 
     if (io.y) {
         K* yrow = io.y + io.ymap.at(row);

@@ -179,7 +179,12 @@ def test_long_rows_sorted_leading_digit_first(hip_backend, dtype, n):
     ties = wide.copy()
     ties[1::2] = ties[0::2][: ties[1::2].size]                        # every key twice: the order of equals shows
     one_digit = randint(305, n, 0, 200).astype(dtype)
-    x = np.stack([wide, lopsided, ties, one_digit, narrow, wide[::-1].copy()])
+    # every key beside one that differs from it in its low 20 bits only: the leading digits of a
+    # run do not settle the order
+    close = wide.copy()
+    bits = close.view(np.uint64 if close.itemsize == 8 else np.uint32)
+    bits[1::2] = bits[0::2][: bits[1::2].size] ^ randint(306, bits[1::2].size, 0, 1 << 20).astype(bits.dtype)
+    x = np.stack([wide, lopsided, ties, one_digit, narrow, wide[::-1].copy(), close])
     Xh = Tensor.from_numpy(hip_backend, x)
     want = np.sort(x, axis=-1, kind="stable")
     order = np.argsort(x, axis=-1, kind="stable")
@@ -200,9 +205,47 @@ def test_long_rows_sorted_leading_digit_first(hip_backend, dtype, n):
     assert np.array_equal(np.take_along_axis(x, got[1][2].astype(np.int64), -1).view(np.uint8), got[1][1].view(np.uint8))
     assert np.array_equal(got[1][3], order)
     # strided outputs (a transposed destination) and an input view with a step
-    Zh = Tensor.from_numpy(hip_backend, np.zeros((n // 2, 6), dtype=dtype)).transpose([1, 0])
+    Zh = Tensor.from_numpy(hip_backend, np.zeros((n // 2, x.shape[0]), dtype=dtype)).transpose([1, 0])
     F.sort(Xh.slice([0], [n], [1], [2]).flip([1]), -1, out=Zh)
     assert np.array_equal(np.ascontiguousarray(Zh.numpy()).view(np.uint8), np.sort(x[:, 0:n:2], axis=-1).view(np.uint8))
+
+
+@pytest.mark.parametrize("dtype", [np.int64, np.float64])
+@pytest.mark.parametrize("n", [100, 700, 2048, 4096])
+def test_wide_keys_in_short_rows_settle_on_their_leading_digits_or_run_every_digit(hip_backend, dtype, n):
+    """Rows sorted whole on chip order 8-byte keys by as many leading digits as their count needs
+    and run the lower digits only when two neighbours still agree.  Rows where they never do,
+    rows where every key has a neighbour differing in low bits only, exact duplicates, and keys
+    that differ in the lowest digit alone, against numpy's stable sort."""
+    m = 24
+    spread = full_range_i64(310, m * n).reshape(m, n)
+    near = spread.copy()
+    near[:, 1::2] = near[:, 0::2][:, : near[:, 1::2].shape[1]] ^ randint(311, m * (n // 2), 0, 1 << 24).reshape(m, n // 2)
+    twice = spread.copy()
+    twice[:, 1::2] = twice[:, 0::2][:, : twice[:, 1::2].shape[1]]
+    low = (spread & ~np.int64(0xff)) [:, :1] | randint(312, m * n, 0, 256).reshape(m, n)
+    raw = np.concatenate([spread, near, twice, low])
+    if np.dtype(dtype).kind == "f":
+        x = raw.view(np.float64).copy()
+        x[np.isnan(x)] = 0.0
+    else:
+        x = raw
+    Xh = Tensor.from_numpy(hip_backend, x)
+    for descending in (False, True):
+        want = np.sort(x, axis=-1, kind="stable")
+        order = np.argsort(x, axis=-1, kind="stable")
+        if descending:
+            want = np.ascontiguousarray(want[:, ::-1])
+        assert np.array_equal(F.sort(Xh, -1, descending).numpy().view(np.uint8), want.view(np.uint8))
+        Yh, Ih = F.argsort(Xh, -1, descending, with_values=True)
+        assert np.array_equal(Yh.numpy().view(np.uint8), want.view(np.uint8))
+        got = Ih.numpy().astype(np.int64)
+        assert np.array_equal(np.take_along_axis(x, got, -1).view(np.uint8), want.view(np.uint8))
+        # equal keys keep their source order in both directions
+        same = np.take_along_axis(x, got, -1)[:, 1:] == np.take_along_axis(x, got, -1)[:, :-1]
+        assert np.all(got[:, 1:][same] > got[:, :-1][same])
+        if not descending:
+            assert np.array_equal(got, order)
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64, np.float16])
