@@ -832,16 +832,16 @@ __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t row
 // ping-pong buffer - sorts it by the lower digits on chip and writes it to the strided outputs
 // at the run's place in the row.  Rows that took the other way leave at once.
 template <typename K, bool PAIRS, int ITEMS, int WAVES>
-__global__ __launch_bounds__(WAVES * kWave) void sort_buckets(PassIo<K> io, int64_t n, const uint32_t* __restrict__ gbase,
-                                                    const uint32_t* __restrict__ moves, const uint32_t* __restrict__ largest) {
+__device__ __forceinline__ void sort_one_bucket(SmallShared<K, PAIRS, ITEMS, WAVES>& sm, const PassIo<K>& io, int64_t n, int64_t bucket,
+                                                const uint32_t* __restrict__ gbase, const uint32_t* __restrict__ moves,
+                                                const uint32_t* __restrict__ largest) {
     constexpr int P = KeyTraits<K>::kPasses;
     constexpr int CAP = WAVES * kWave * ITEMS;
-    __shared__ SmallShared<K, PAIRS, ITEMS, WAVES> sm;
     const int tid = threadIdx.x;
     const int lane = lane_id();
     const int w = tid / kWave;
-    const int64_t row = blockIdx.x / kRadix;
-    const int d = static_cast<int>(blockIdx.x % kRadix);
+    const int64_t row = bucket / kRadix;
+    const int d = static_cast<int>(bucket % kRadix);
     const int msd = msd_digit<P>(moves + row * P, largest + row * P, static_cast<uint32_t>(CAP));
     if (msd < 0) return;
     const uint32_t* starts = gbase + (row * P + msd) * kRadix;
@@ -898,6 +898,13 @@ __global__ __launch_bounds__(WAVES * kWave) void sort_buckets(PassIo<K> io, int6
             }
         }
     }
+}
+
+template <typename K, bool PAIRS, int ITEMS, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void sort_buckets(PassIo<K> io, int64_t n, const uint32_t* __restrict__ gbase,
+                                                    const uint32_t* __restrict__ moves, const uint32_t* __restrict__ largest) {
+    __shared__ SmallShared<K, PAIRS, ITEMS, WAVES> sm;
+    sort_one_bucket<K, PAIRS, ITEMS, WAVES>(sm, io, n, blockIdx.x, gbase, moves, largest);
 }
 
 // One exchange of the (key, index) networks below: the lane takes the entry of lane ^ J when
@@ -1056,13 +1063,35 @@ constexpr int64_t kSmallRow = 4096;      // longest row sort_rows_small takes
 // mean run length above which a row may go that way.
 // The large kernel holds 18 keys per thread in 4 wavefronts; with indices that many registers
 // leave one wavefront per SIMD, so pairs take 10 per thread in 8 wavefronts.
-constexpr int kBucketItemsSmall = 8, kBucketWavesSmall = 4;
+// Smaller runs take 2, 4, 8 or 12 keys per thread in 4 wavefronts (512 to 3072 keys).
 constexpr int bucket_items_large(bool pairs) { return pairs ? 10 : 18; }
 constexpr int bucket_waves_large(bool pairs) { return pairs ? 8 : 4; }
-constexpr int kBucketCapSmall = kBucketItemsSmall * kBucketWavesSmall * kWave;
 constexpr int bucket_cap_large(bool pairs) { return bucket_items_large(pairs) * bucket_waves_large(pairs) * kWave; }
-constexpr int64_t kBucketMinMean = 1024;
 int g_sort_buckets = 1;
+int g_sort_bucket_min = 0;               // shortest mean run that goes this way (0: bucket_min_mean below)
+
+// Integers: the measured break-even against the least-significant-digit-first passes on evenly
+// spread keys.  Floating-point rows seldom spread evenly over the sign and exponent byte, and
+// a row that does not go this way still pays for the dispatch of its 256 bucket workgroups
+// (about 8 % of a sort of 65536-key rows, under 2 % from 262144 keys on).
+constexpr int64_t bucket_min_mean(size_t key_size, bool pairs, int kind) {
+    if (kind == kKeyFloat) return 1024;
+    return key_size == 8 ? (pairs ? 64 : 128) : (pairs ? 128 : 512);
+}
+
+// Capacity of the bucket kernel for rows of n keys (0: none): the mean run with a quarter of
+// headroom (an eighth from 2048 keys on) has to fit; each row then decides on the device from
+// its own histogram.  `min_mean` is the shortest mean run worth the detour.
+uint32_t bucket_capacity(int64_t n, bool pairs, int64_t min_mean) {
+    const int64_t mean = ceil_div(n, static_cast<int64_t>(kRadix));
+    if (mean < min_mean) return 0u;
+    if (mean + mean / 4 <= 512) return 512u;
+    if (mean + mean / 4 <= 1024) return 1024u;
+    if (mean + mean / 8 <= 2048) return 2048u;
+    if (mean + mean / 8 <= 3072) return 3072u;
+    if (mean + mean / 8 <= bucket_cap_large(pairs)) return static_cast<uint32_t>(bucket_cap_large(pairs));
+    return 0u;
+}
 template <typename K>
 constexpr bool kBucketKeys = sizeof(K) >= 4;     // two-digit keys gain nothing
 
@@ -1223,15 +1252,10 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     uint32_t* largest = reinterpret_cast<uint32_t*>(base + l.largest_off);
     sort_bases<<<dim3(static_cast<unsigned>(m * P)), dim3(kRadix), 0, stream>>>(ghist, moves, largest, y_over_x ? 1 : 0);
     DLFX_CHECK_LAUNCH();
-    // rows long enough for an even leading digit to leave runs of 1024 to 4096 keys may go most
-    // significant digit first (each row decides on the device from its histogram); the bucket
-    // kernel's capacity is picked from the mean run length with an eighth of headroom
+    // rows whose leading digit leaves runs that a workgroup can hold may go most significant
+    // digit first
     uint32_t bucket_cap = 0;
-    if (kBucketKeys<K> && !y_over_x && g_sort_buckets && m * kRadix <= 0x7fffffffLL) {
-        const int64_t mean = ceil_div(n, static_cast<int64_t>(kRadix));
-        if (mean > kBucketMinMean && mean + mean / 8 <= bucket_cap_large(a.pairs))
-            bucket_cap = static_cast<uint32_t>(mean + mean / 8 <= kBucketCapSmall ? kBucketCapSmall : bucket_cap_large(a.pairs));
-    }
+    if (kBucketKeys<K> && !y_over_x && g_sort_buckets && m * kRadix <= 0x7fffffffLL) bucket_cap = bucket_capacity(n, a.pairs, g_sort_bucket_min ? g_sort_bucket_min : bucket_min_mean(sizeof(K), a.pairs, a.kind));
 
     io.kbuf[0] = reinterpret_cast<K*>(base + l.keys_off[0]);
     io.kbuf[1] = reinterpret_cast<K*>(base + l.keys_off[1]);
@@ -1254,15 +1278,21 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     }
     if constexpr (kBucketKeys<K>) if (bucket_cap != 0u) {
         const dim3 bgrid(static_cast<unsigned>(m * kRadix));
-        if (bucket_cap == kBucketCapSmall) {
-            constexpr int I = kBucketItemsSmall, W = kBucketWavesSmall;
-            if (a.pairs) sort_buckets<K, true, I, W><<<bgrid, dim3(W * kWave), 0, stream>>>(io, n, ghist, moves, largest);
-            else sort_buckets<K, false, I, W><<<bgrid, dim3(W * kWave), 0, stream>>>(io, n, ghist, moves, largest);
-        } else {
-            constexpr int BIP = bucket_items_large(true), BWP = bucket_waves_large(true);
-            constexpr int BIK = bucket_items_large(false), BWK = bucket_waves_large(false);
-            if (a.pairs) sort_buckets<K, true, BIP, BWP><<<bgrid, dim3(BWP * kWave), 0, stream>>>(io, n, ghist, moves, largest);
-            else sort_buckets<K, false, BIK, BWK><<<bgrid, dim3(BWK * kWave), 0, stream>>>(io, n, ghist, moves, largest);
+        constexpr int BIP = bucket_items_large(true), BWP = bucket_waves_large(true);
+        constexpr int BIK = bucket_items_large(false), BWK = bucket_waves_large(false);
+        switch (bucket_cap) {
+#define DLFX_BUCKETS(I)                                                                                             \
+    if (a.pairs) sort_buckets<K, true, I, 4><<<bgrid, dim3(4 * kWave), 0, stream>>>(io, n, ghist, moves, largest); \
+    else sort_buckets<K, false, I, 4><<<bgrid, dim3(4 * kWave), 0, stream>>>(io, n, ghist, moves, largest);        \
+    break
+            case 512u: DLFX_BUCKETS(2);
+            case 1024u: DLFX_BUCKETS(4);
+            case 2048u: DLFX_BUCKETS(8);
+            case 3072u: DLFX_BUCKETS(12);
+#undef DLFX_BUCKETS
+            default:
+                if (a.pairs) sort_buckets<K, true, BIP, BWP><<<bgrid, dim3(BWP * kWave), 0, stream>>>(io, n, ghist, moves, largest);
+                else sort_buckets<K, false, BIK, BWK><<<bgrid, dim3(BWK * kWave), 0, stream>>>(io, n, ghist, moves, largest);
         }
         DLFX_CHECK_LAUNCH();
     }
@@ -1291,6 +1321,10 @@ bool set_sort_tuning(const char* key, int64_t value) {
     }
     if (!std::strcmp(key, "sort_buckets") && value >= 0 && value <= 1) {
         g_sort_buckets = static_cast<int>(value);
+        return true;
+    }
+    if (!std::strcmp(key, "sort_bucket_min") && value >= 0 && value <= 65536) {
+        g_sort_bucket_min = static_cast<int>(value);
         return true;
     }
     if (!std::strcmp(key, "sort_wave_rows") && value >= 0 && value <= 512) {

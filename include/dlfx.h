@@ -80,6 +80,13 @@ int dlfx_last_hip_error(void);
  *   "sort_poll_limit"  the same bound for the per-digit tile chaining of a radix pass.
  *   "sort_wave_rows"   longest row (64, 128, 256 or 512; default 512) sorted by one wavefront
  *                      in registers; longer rows of up to 4096 elements take one workgroup.
+ *   "sort_buckets"     1 (default): rows of 4- and 8-byte keys whose most significant varying
+ *                      digit spreads them evenly are sorted on that digit first and each run
+ *                      of equal digits is finished on chip; 0: every row takes the
+ *                      least-significant-digit-first passes.  Same results either way.
+ *   "sort_bucket_min"  shortest mean run (row length / 256) for which "sort_buckets" applies;
+ *                      0 (default): 128 / 512 for 8- / 4-byte integers, 64 / 128 when
+ *                      indices travel with them, 1024 for floating-point keys.
  *   "topk_thread_rows" longest row (default 256; half of it for 8-byte keys) for which top_k
  *                      with a limit of at most 8 over at least 16384 contiguous rows gives
  *                      each row to one thread.

@@ -162,9 +162,17 @@ def test_rows_leave_out_passes_that_move_nothing(hip_backend, oracle_backend, dt
 
 
 @pytest.mark.parametrize("dtype", [np.int64, np.float32, np.int32, np.float64])
-@pytest.mark.parametrize("n", [300000, 1 << 20])
+@pytest.mark.parametrize("n", [5000, 40000, 150000, 300000, 600000, 1 << 20])
 def test_long_rows_sorted_leading_digit_first(hip_backend, dtype, n):
-    """Rows of 2^18 to 2^20 keys whose leading digit spreads them evenly take one tiled pass on
+    hip_backend.set_tuning("sort_bucket_min", 1)     # every run length takes the route (the lengths cover each bucket kernel)
+    try:
+        _leading_digit_first(hip_backend, dtype, n)
+    finally:
+        hip_backend.set_tuning("sort_bucket_min", 0)
+
+
+def _leading_digit_first(hip_backend, dtype, n):
+    """Rows whose leading digit spreads them evenly take one tiled pass on
     that digit and finish every run of equal digits on chip; rows it does not spread (or that
     vary in one digit only) take the least-significant-digit-first passes in the same call.
     Checked against numpy's stable sort and against the same call with that route switched off."""
