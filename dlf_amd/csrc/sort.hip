@@ -616,8 +616,12 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
 // waves' counts, scatter through LDS, reload in element order.  Digits that are the same in
 // the whole row are skipped.  Element e of the row is item e / 64 % ITEMS of lane e % 64 of
 // wave e / (64 * ITEMS), before and after every pass.
+constexpr int kSmallMoves = 256;         // keys that the run walk of sort_in_workgroup may move (one thread each)
+
 template <typename K, bool PAIRS, int ITEMS, int WAVES = 4>
 struct SmallShared {
+    uint32_t n_moves;
+    uint2 moves[kSmallMoves];
     uint32_t wave_hist[WAVES][kRadix];
     uint32_t scan_tmp[kRadix / kWave];
     K wave_or[WAVES], wave_and[WAVES];
@@ -630,11 +634,13 @@ struct SmallShared {
 // the number of low digits that may differ (digits from `top` up are known to be equal),
 // `valid` the number of keys that are not padding.  The workgroup has WAVES wavefronts (4 or 8).
 //
-// When more digits vary than `valid` distinct keys need to tell them apart (with 2^6 to spare
-// over the square of `valid`, so that evenly spread keys rarely collide), the leading ones of
-// the varying digits are sorted first: if no two neighbours of the result agree in all of
-// them, the order is final and the lower digits never ran.  Otherwise every digit runs from
-// that arrangement, which the passes so far left in source order among equal keys.
+// When more digits vary than `valid` distinct keys need to tell most of them apart (about as
+// many bits as the square of `valid` has, so that evenly spread keys leave a few pairs that
+// agree), the leading ones of the varying digits are sorted first.  Keys that then agree with
+// a neighbour in all of those digits form short runs, in source order; every key of such a run
+// finds its place by comparing whole keys with the run's other members (at most kNear to
+// either side), and the lower digits never ran.  A longer run makes every digit run from that
+// arrangement, which the passes so far left in source order among equal keys.
 template <typename K, bool PAIRS, int ITEMS, int WAVES = 4>
 __device__ __forceinline__ void sort_in_workgroup(SmallShared<K, PAIRS, ITEMS, WAVES>& sm, K (&key)[ITEMS], uint32_t (&val)[PAIRS ? ITEMS : 1],
                                                   K ors, K ands, int valid, int top) {
@@ -650,6 +656,7 @@ __device__ __forceinline__ void sort_in_workgroup(SmallShared<K, PAIRS, ITEMS, W
         sm.wave_or[w] = ors;
         sm.wave_and[w] = ands;
     }
+    if (tid == 0) sm.n_moves = 0u;
     __syncthreads();
     K any = 0, all = ~K(0);
 #pragma unroll
@@ -662,7 +669,7 @@ __device__ __forceinline__ void sort_in_workgroup(SmallShared<K, PAIRS, ITEMS, W
 
     int first = 0;                                         // lowest digit of this round of passes
     if constexpr (sizeof(K) > 4) {
-        const int enough = (2 * (32 - __builtin_clz(static_cast<uint32_t>(valid > 1 ? valid - 1 : 1))) + 6 + 7) / 8;
+        const int enough = (2 * (32 - __builtin_clz(static_cast<uint32_t>(valid > 1 ? valid - 1 : 1))) - 2 + 7) / 8;
         int varying = 0;
         for (int p = top - 1; p >= 0; --p) {
             if ((static_cast<uint32_t>(differ >> (8 * p)) & 0xffu) != 0u && ++varying == enough) first = p;
@@ -755,15 +762,76 @@ __device__ __forceinline__ void sort_in_workgroup(SmallShared<K, PAIRS, ITEMS, W
             // (the three barriers of the next pass lie between these reads and its scatter)
         }
         if (first == 0) break;
-        // do any two neighbours agree in every digit sorted so far?
-        bool same = false;
+        // Runs of neighbours that agree in every digit sorted so far.  Keys with such a neighbour
+        // are few: each walks its run (the tile holds what the registers hold), and the ones that
+        // have to move are listed.
+        constexpr int kNear = 3;
+        const int sh = 8 * first;
+        uint32_t near = 0;                                 // bit k: item k has a neighbour of its run
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
             const int e = seg + k * kWave;
-            if (e > 0 && e < valid) same |= (sm.keys[e - 1] >> (8 * first)) == (key[k] >> (8 * first));
+            if (e < valid) {
+                const K lead = key[k] >> sh;
+                const bool left = e > 0 && (sm.keys[e - 1] >> sh) == lead;
+                const bool right = e + 1 < valid && (sm.keys[e + 1] >> sh) == lead;
+                if (left || right) near |= 1u << k;
+            }
         }
-        if (!__syncthreads_or(same ? 1 : 0)) break;
-        first = 0;
+        bool longer = false;
+        for (; near != 0u; near &= near - 1u) {
+            const int e = seg + __builtin_ctz(near) * kWave;
+            const K mine = sm.keys[e];
+            const K lead = mine >> sh;
+            int before = 0, ahead = 0;                     // members of the run to the left; of the whole run that come first
+            int j = e - 1;
+            for (; j >= 0 && before < kNear; --j, ++before) {
+                const K other = sm.keys[j];
+                if ((other >> sh) != lead) break;
+                ahead += other <= mine ? 1 : 0;
+            }
+            if (before == kNear && j >= 0 && (sm.keys[j] >> sh) == lead) longer = true;
+            int after = 0;
+            for (j = e + 1; j < valid && after < kNear; ++j, ++after) {
+                const K other = sm.keys[j];
+                if ((other >> sh) != lead) break;
+                ahead += other < mine ? 1 : 0;
+            }
+            if (after == kNear && j < valid && (sm.keys[j] >> sh) == lead) longer = true;
+            const int dest = e - before + ahead;
+            if (dest != e) {
+                const uint32_t slot = atomicAdd(&sm.n_moves, 1u);
+                if (slot < static_cast<uint32_t>(kSmallMoves)) sm.moves[slot] = make_uint2(static_cast<uint32_t>(e), static_cast<uint32_t>(dest));
+                else longer = true;
+            }
+        }
+        if (__syncthreads_or(longer ? 1 : 0)) {            // a run too long, or too many moves: every digit runs
+            first = 0;
+            continue;
+        }
+        const int n_moves = static_cast<int>(sm.n_moves);
+        if (n_moves != 0) {
+            uint2 mv = make_uint2(0u, 0u);
+            K moved_key = 0;
+            uint32_t moved_val = 0;
+            if (tid < n_moves) {
+                mv = sm.moves[tid];
+                moved_key = sm.keys[mv.x];
+                if constexpr (PAIRS) moved_val = sm.vals[mv.x];
+            }
+            __syncthreads();
+            if (tid < n_moves) {
+                sm.keys[mv.y] = moved_key;
+                if constexpr (PAIRS) sm.vals[mv.y] = moved_val;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) {
+                key[k] = sm.keys[seg + k * kWave];
+                if constexpr (PAIRS) val[k] = sm.vals[seg + k * kWave];
+            }
+        }
+        break;
     }
 }
 

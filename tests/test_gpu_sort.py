@@ -192,7 +192,15 @@ def _leading_digit_first(hip_backend, dtype, n):
     close = wide.copy()
     bits = close.view(np.uint64 if close.itemsize == 8 else np.uint32)
     bits[1::2] = bits[0::2][: bits[1::2].size] ^ randint(306, bits[1::2].size, 0, 1 << 20).astype(bits.dtype)
-    x = np.stack([wide, lopsided, ties, one_digit, narrow, wide[::-1].copy(), close])
+    # the same for one key in 64 (a few per run, which move within the run without the lower
+    # digits being sorted), and groups of 4 and of 6 such keys
+    few = wide.copy()
+    bits = few.view(np.uint64 if few.itemsize == 8 else np.uint32)
+    for group, step in ((2, 64), (4, 1000), (6, 1777)):
+        for j in range(1, group):
+            at = np.arange(0, n - group, step) + j
+            bits[at] = bits[at - j] ^ randint(307 + j, at.size, 0, 1 << 20).astype(bits.dtype)
+    x = np.stack([wide, lopsided, ties, one_digit, narrow, wide[::-1].copy(), close, few])
     Xh = Tensor.from_numpy(hip_backend, x)
     want = np.sort(x, axis=-1, kind="stable")
     order = np.argsort(x, axis=-1, kind="stable")
@@ -232,7 +240,15 @@ def test_wide_keys_in_short_rows_settle_on_their_leading_digits_or_run_every_dig
     twice = spread.copy()
     twice[:, 1::2] = twice[:, 0::2][:, : twice[:, 1::2].shape[1]]
     low = (spread & ~np.int64(0xff)) [:, :1] | randint(312, m * n, 0, 256).reshape(m, n)
-    raw = np.concatenate([spread, near, twice, low])
+    # a few groups of 2 to 4 keys that differ in their low 16 bits (they find their places among
+    # themselves), and the same with groups of 6 (too long for that: every digit runs)
+    some, long_runs = spread.copy(), spread.copy()
+    for rows, sizes in ((some, (2, 3, 4)), (long_runs, (2, 6))):
+        for g, group in enumerate(sizes):
+            for j in range(1, group):
+                at = np.arange(7 * g, n - group, 97) + j
+                rows[:, at] = rows[:, at - j] ^ randint(313 + j, m * at.size, 0, 1 << 16).reshape(m, at.size)
+    raw = np.concatenate([spread, near, twice, low, some, long_runs])
     if np.dtype(dtype).kind == "f":
         x = raw.view(np.float64).copy()
         x[np.isnan(x)] = 0.0
