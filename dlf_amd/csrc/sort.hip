@@ -257,6 +257,10 @@ __device__ __forceinline__ int msd_digit(const uint32_t* __restrict__ row_moves,
 // ------------------------------------------------------------------ one pass
 // Status word of (tile, digit): [tag:4 | inclusive:1 | count:27]; a word is valid
 // for pass p when its tag is p + 1, so the array is cleared once per sort.
+// Values of sort_pass's pass argument beside a pass number: the launch that takes only the
+// rows sorted most significant digit first (each on its own digit), and the flag on a pass
+// number that says those rows have such a launch.
+constexpr int kLeadingPass = -1, kLeadingPassElsewhere = 64;
 constexpr uint32_t kCountMask = (1u << 27) - 1;
 __device__ __forceinline__ uint32_t make_status(int pass, bool inclusive, uint32_t count) {
     return (static_cast<uint32_t>(pass + 1) << 28) | (inclusive ? (1u << 27) : 0u) | count;
@@ -279,7 +283,7 @@ struct PassShared {
 // pass it runs reads the strided input, and its place in the ping-pong buffers alternates
 // over the passes it does run.
 template <typename K, bool PAIRS, int ITEMS, bool LAST>
-__global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SORT_WAVES))) void sort_pass(PassIo<K> io, int pass, int64_t rows, int64_t n, int64_t tiles_per_row,
+__global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(sizeof(K) == 8 && PAIRS && ITEMS > 8 ? 2 : DLFX_SORT_WAVES))) void sort_pass(PassIo<K> io, int pass_arg, int64_t rows, int64_t n, int64_t tiles_per_row,
                                                     const uint32_t* __restrict__ gbase,
                                                     const uint32_t* __restrict__ moves,
                                                     const uint32_t* __restrict__ largest, uint32_t bucket_cap,
@@ -297,10 +301,16 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
     const int64_t row = blockIdx.x - t * rows;
     const uint32_t* row_moves = moves + row * P;
     // a row sorted most significant digit first runs that digit's pass only, from the input
-    // into the first buffer
+    // into the first buffer: in the launch of that pass, or - when `pass_arg` is kLeadingPass
+    // or kLeadingPassElsewhere - in a launch of its own that takes those rows only (with its
+    // own tile size, hence its own status tag: the words of its tiles lie where other rows'
+    // tiles of the other launches lie)
     const int msd = msd_digit<P>(row_moves, largest + row * P, bucket_cap);
     const bool to_buckets = msd >= 0;
-    if (to_buckets && pass != msd) return;
+    const bool own_launch = pass_arg == kLeadingPass;
+    if (own_launch ? !to_buckets : to_buckets && (pass_arg >= kLeadingPassElsewhere || (pass_arg & ~kLeadingPassElsewhere) != msd)) return;
+    const int pass = own_launch ? msd : (pass_arg & ~kLeadingPassElsewhere);
+    const int tag = own_launch ? P : pass;
     int ran = 0;            // passes before this one that this row ran
     if (!to_buckets)
         for (int p = 0; p < pass; ++p) ran += row_moves[p] ? 1 : 0;
@@ -440,7 +450,7 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
     const int64_t srow = (row * tiles_per_row) * kRadix;
     uint32_t* my_status = status + srow + t * kRadix + dg;
     if (owner && t + 1 < tiles_per_row)
-        __hip_atomic_store(my_status, make_status(pass, t == 0, count), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(my_status, make_status(tag, t == 0, count), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // the status words of the W tiles before this one are requested now and looked at after
     // the tile has been gathered, so that their latency is not waited for
     uint32_t sw[W];
@@ -450,7 +460,7 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
         for (int i = 0; i < W; ++i) {
             const int64_t q = p - i;
             sw[i] = (q >= 0) ? __hip_atomic_load(status + srow + q * kRadix + dg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                             : make_status(pass, true, 0u);
+                             : make_status(tag, true, 0u);
         }
     };
     bool done = (t == 0) || !owner;
@@ -489,7 +499,7 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
     uint32_t before_tiles = 0;
     {
         bool refetch = false;
-        const uint32_t want_tag = static_cast<uint32_t>(pass + 1);
+        const uint32_t want_tag = static_cast<uint32_t>(tag + 1);
         for (;;) {
             int stuck = -1;
             while (!done) {
@@ -547,7 +557,7 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
         }
     }
     if (owner && t > 0 && t + 1 < tiles_per_row)
-        __hip_atomic_store(my_status, make_status(pass, true, before_tiles + count), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(my_status, make_status(tag, true, before_tiles + count), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (owner) sm.dst_base[tid] = static_cast<int32_t>(gbase[(row * P + pass) * kRadix + tid] + before_tiles) - static_cast<int32_t>(start);
     __syncthreads();
     DLFX_PHASE(4);
@@ -1136,6 +1146,7 @@ constexpr int bucket_items_large(bool pairs) { return pairs ? 10 : 18; }
 constexpr int bucket_waves_large(bool pairs) { return pairs ? 8 : 4; }
 constexpr int bucket_cap_large(bool pairs) { return bucket_items_large(pairs) * bucket_waves_large(pairs) * kWave; }
 int g_sort_buckets = 1;
+int g_sort_leading_launch = 1;
 int g_sort_bucket_min = 0;               // shortest mean run that goes this way (0: bucket_min_mean below)
 
 // Integers: the measured break-even against the least-significant-digit-first passes on evenly
@@ -1330,17 +1341,30 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     io.vbuf[0] = a.pairs ? reinterpret_cast<uint32_t*>(base + l.vals_off[0]) : nullptr;
     io.vbuf[1] = a.pairs ? reinterpret_cast<uint32_t*>(base + l.vals_off[1]) : nullptr;
     const dim3 grid(static_cast<unsigned>(m * l.tiles_per_row));
+    // 8-byte keys with indices: the tiled passes take 2048 keys per tile, which cuts a tile's share
+    // of a digit into runs of 8 keys (64 + 32 bytes: twice the bytes written).  The rows sorted most
+    // significant digit first run their one pass in a launch of their own with 4096-key tiles.
+    int elsewhere = 0;
+    if constexpr (sizeof(K) == 8) {
+        if (a.pairs && bucket_cap != 0u && g_sort_leading_launch) {
+            constexpr int IL = tile_items(sizeof(K), false);
+            const int64_t tiles = ceil_div(n, static_cast<int64_t>(kPassBlock) * IL);
+            sort_pass<K, true, IL, false><<<dim3(static_cast<unsigned>(m * tiles)), dim3(kPassBlock), 0, stream>>>(io, kLeadingPass, m, n, tiles, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
+            DLFX_CHECK_LAUNCH();
+            elsewhere = kLeadingPassElsewhere;
+        }
+    }
     for (int p = 0; p < P; ++p) {
         if (p < P - 1) {
             if (a.pairs)
-                sort_pass<K, true, IP, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
+                sort_pass<K, true, IP, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p | elsewhere, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
             else
-                sort_pass<K, false, IK, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
+                sort_pass<K, false, IK, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p | elsewhere, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
         } else {
             if (a.pairs)
-                sort_pass<K, true, IP, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
+                sort_pass<K, true, IP, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p | elsewhere, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
             else
-                sort_pass<K, false, IK, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
+                sort_pass<K, false, IK, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p | elsewhere, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
         }
         DLFX_CHECK_LAUNCH();
     }
@@ -1389,6 +1413,10 @@ bool set_sort_tuning(const char* key, int64_t value) {
     }
     if (!std::strcmp(key, "sort_buckets") && value >= 0 && value <= 1) {
         g_sort_buckets = static_cast<int>(value);
+        return true;
+    }
+    if (!std::strcmp(key, "sort_leading_launch") && value >= 0 && value <= 1) {
+        g_sort_leading_launch = static_cast<int>(value);
         return true;
     }
     if (!std::strcmp(key, "sort_bucket_min") && value >= 0 && value <= 65536) {

@@ -87,6 +87,10 @@ int dlfx_last_hip_error(void);
  *   "sort_bucket_min"  shortest mean run (row length / 256) for which "sort_buckets" applies;
  *                      0 (default): 128 / 512 for 8- / 4-byte integers, 64 / 128 when
  *                      indices travel with them, 1024 for floating-point keys.
+ *   "sort_leading_launch" 1 (default): rows of 8-byte keys with indices that "sort_buckets" sends
+ *                      most significant digit first run that digit's pass in a launch of
+ *                      their own with 4096-key tiles; 0: inside the launch of that pass, with
+ *                      the 2048-key tiles of the other rows.  Same results either way.
  *   "topk_thread_rows" longest row (default 256; half of it for 8-byte keys) for which top_k
  *                      with a limit of at most 8 over at least 16384 contiguous rows gives
  *                      each row to one thread.

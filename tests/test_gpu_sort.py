@@ -227,6 +227,38 @@ def _leading_digit_first(hip_backend, dtype, n):
 
 
 @pytest.mark.parametrize("dtype", [np.int64, np.float64])
+@pytest.mark.parametrize("n", [40000, 300000, 1 << 20])
+def test_leading_digit_pass_in_its_own_launch_or_not(hip_backend, dtype, n):
+    """Stable argsort of 8-byte keys: the rows sorted most significant digit first run their one
+    tiled pass in a launch of their own (larger tiles) beside rows that take every pass; the same
+    indices and values come out when that launch is switched off, and both match numpy."""
+    spread = full_range_i64(320, 3 * n).reshape(3, n)
+    spread[1, 1::2] = spread[1, 0::2][: spread[1, 1::2].size]                   # every key twice
+    lopsided = (full_range_i64(321, 2 * n).reshape(2, n) >> 40)
+    raw = np.concatenate([spread, lopsided])
+    if np.dtype(dtype).kind == "f":
+        x = raw.view(np.float64).copy()
+        x[np.isnan(x)] = 0.0
+    else:
+        x = raw
+    Xh = Tensor.from_numpy(hip_backend, x)
+    order = np.argsort(x, axis=-1, kind="stable")
+    want = np.take_along_axis(x, order, -1)
+    for own in (0, 1):
+        hip_backend.set_tuning("sort_leading_launch", own)
+        try:
+            Yh, Ih = F.argsort(Xh, -1, False, with_values=True)
+            Id = F.argsort(Xh, -1, True).numpy().astype(np.int64)
+        finally:
+            hip_backend.set_tuning("sort_leading_launch", 1)
+        assert np.array_equal(Ih.numpy(), order) and np.array_equal(Yh.numpy().view(np.uint8), want.view(np.uint8))
+        got = np.take_along_axis(x, Id, -1)
+        assert np.array_equal(got.view(np.uint8), np.ascontiguousarray(want[:, ::-1]).view(np.uint8))
+        same = got[:, 1:] == got[:, :-1]
+        assert np.all(Id[:, 1:][same] > Id[:, :-1][same])
+
+
+@pytest.mark.parametrize("dtype", [np.int64, np.float64])
 @pytest.mark.parametrize("n", [100, 700, 2048, 4096])
 def test_wide_keys_in_short_rows_settle_on_their_leading_digits_or_run_every_digit(hip_backend, dtype, n):
     """Rows sorted whole on chip order 8-byte keys by as many leading digits as their count needs
