@@ -10,6 +10,7 @@
 //     reduced axis and combine through LDS;
 //   * anything else: the row kernels with per-element address computation.
 // All of them are bandwidth bound; fp32 sums accumulate in fp64 registers.
+#include <atomic>
 #include <cmath>
 #include <cstring>
 #include <limits>
@@ -596,11 +597,13 @@ extern "C" size_t dlfx_reduce_scratch_bytes(int dtype, int64_t m, int64_t n) {
     return partial_bound_bytes(m);
 }
 
-extern "C" int dlfx_reduce(dlfx_stream_t stream, const char* name, int dtype, int64_t m, int64_t n,
-                           int x_rank, const int64_t* x_dims, const int64_t* x_strides,
-                           const void* x, int64_t x_offset,
-                           int y_rank, const int64_t* y_dims, const int64_t* y_strides,
-                           void* y, int64_t y_offset, void* scratch, size_t scratch_bytes) {
+namespace {
+
+int reduce_entry(dlfx_stream_t stream, const char* name, int dtype, int64_t m, int64_t n,
+                 int x_rank, const int64_t* x_dims, const int64_t* x_strides,
+                 const void* x, int64_t x_offset,
+                 int y_rank, const int64_t* y_dims, const int64_t* y_strides,
+                 void* y, int64_t y_offset, void* scratch, size_t scratch_bytes) {
     if (!name || !x || !y || m <= 0 || n <= 0) return DLFX_ERR_INVALID_ARGUMENT;
     if (!view_ok(x_rank, x_dims, x_strides) || !view_ok(y_rank, y_dims, y_strides))
         return DLFX_ERR_INVALID_ARGUMENT;
@@ -638,6 +641,63 @@ extern "C" int dlfx_reduce(dlfx_stream_t stream, const char* name, int dtype, in
                                       static_cast<const T*>(x) + x_offset, static_cast<T*>(y) + y_offset,
                                       scratch, scratch_bytes);
     });
+}
+
+// Partial accumulators of dlfx_reduce_static: one copy of this array lives on every device the
+// library runs on, from the load of the code object to the end of the process.  The size is
+// partial_bound_bytes() of the largest row count that needs partials (65535), rounded up to 256.
+constexpr size_t kStaticScratchBytes = 3178496;
+static_assert(kStaticScratchBytes == DLFX_REDUCE_STATIC_SCRATCH_BYTES, "header and array disagree");
+static_assert(kStaticScratchBytes % 256 == 0 && kStaticScratchBytes >= (65535 + 133120) * 16, "array too small");
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// The array's address on each device.  In host code the name `scratch` is only a handle for
+// hipGetSymbolAddress: every device has its own copy at its own address, looked up once with
+// that device current and kept here; kernels are only ever given these pointers.
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_static_scratch[kMaxDevices];
+
+int static_scratch_of_current_device(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return record_hip_error(e);
+    if (dev < 0 || dev >= kMaxDevices) return DLFX_ERR_INVALID_ARGUMENT;
+    void* p = g_static_scratch[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return record_hip_error(e);
+        if (!p) return record_hip_error(hipErrorInvalidSymbol);
+        g_static_scratch[dev].store(p, std::memory_order_release);   // racing threads store the same address
+    }
+    *out = p;
+    return DLFX_OK;
+}
+
+}  // namespace
+
+extern "C" int dlfx_reduce(dlfx_stream_t stream, const char* name, int dtype, int64_t m, int64_t n,
+                           int x_rank, const int64_t* x_dims, const int64_t* x_strides,
+                           const void* x, int64_t x_offset,
+                           int y_rank, const int64_t* y_dims, const int64_t* y_strides,
+                           void* y, int64_t y_offset, void* scratch_arg, size_t scratch_bytes) {
+    return reduce_entry(stream, name, dtype, m, n, x_rank, x_dims, x_strides, x, x_offset,
+                        y_rank, y_dims, y_strides, y, y_offset, scratch_arg, scratch_bytes);
+}
+
+extern "C" int dlfx_reduce_static(dlfx_stream_t stream, const char* name, int dtype, int64_t m, int64_t n,
+                                  int x_rank, const int64_t* x_dims, const int64_t* x_strides,
+                                  const void* x, int64_t x_offset,
+                                  int y_rank, const int64_t* y_dims, const int64_t* y_strides,
+                                  void* y, int64_t y_offset) {
+    if (m <= 0 || n <= 0) return DLFX_ERR_INVALID_ARGUMENT;
+    // Same bound as the caller of dlfx_reduce would have to provide; beyond the array: refuse.
+    if (partial_bound_bytes(m) > kStaticScratchBytes) return DLFX_ERR_TOO_LARGE;
+    void* ptr = nullptr;
+    const int st = static_scratch_of_current_device(&ptr);
+    if (st != DLFX_OK) return st;
+    // Partials are written by the first kernel before the second reads them: nothing to clear.
+    return reduce_entry(stream, name, dtype, m, n, x_rank, x_dims, x_strides, x, x_offset,
+                        y_rank, y_dims, y_strides, y, y_offset, ptr, kStaticScratchBytes);
 }
 
 extern "C" size_t dlfx_arg_reduce_scratch_bytes(int dtype, int64_t n_rows, int64_t k) {

@@ -39,6 +39,10 @@ def _declare(lib):
     lib.dlfx_reduce.argtypes = ([c_void_p, c_char_p, c_int, c_int64, c_int64] + view + [c_void_p, c_int64]
                                 + view + [c_void_p, c_int64, c_void_p, c_size_t])
 
+    lib.dlfx_reduce_static.restype = c_int
+    lib.dlfx_reduce_static.argtypes = ([c_void_p, c_char_p, c_int, c_int64, c_int64] + view + [c_void_p, c_int64]
+                                       + view + [c_void_p, c_int64])
+
     lib.dlfx_arg_reduce_scratch_bytes.restype = c_size_t
     lib.dlfx_arg_reduce_scratch_bytes.argtypes = [c_int, c_int64, c_int64]
     lib.dlfx_arg_reduce.restype = c_int
@@ -102,7 +106,7 @@ _lib = None
 
 # Every symbol include/dlfx.h declares.
 EXPORTS = ("dlfx_version", "dlfx_status_string", "dlfx_last_hip_error", "dlfx_set_tuning",
-           "dlfx_reduce_scratch_bytes", "dlfx_reduce",
+           "dlfx_reduce_scratch_bytes", "dlfx_reduce", "dlfx_reduce_static",
            "dlfx_arg_reduce_scratch_bytes", "dlfx_arg_reduce",
            "dlfx_scan_scratch_bytes", "dlfx_scan",
            "dlfx_sort_scratch_bytes", "dlfx_sort",
@@ -221,6 +225,13 @@ class HipBackend:
                            (name.encode(), dtype, m, n),
                            (xs.rank, _arr(xs.extents), _arr(xs.strides), x.data_ptr(), xs.offset,
                             ys.rank, _arr(ys.extents), _arr(ys.strides), y.data_ptr(), ys.offset, sp, sb), defer, (x, y))
+
+    def reduce_static(self, name, dtype, m, n, xs, x, ys, y, defer=False):
+        """dlfx_reduce_static: the same reduction with the library's own static device scratch."""
+        return self._issue(self.lib.dlfx_reduce_static, "dlfx_reduce_static(%s)" % name,
+                           (name.encode(), dtype, m, n),
+                           (xs.rank, _arr(xs.extents), _arr(xs.strides), x.data_ptr(), xs.offset,
+                            ys.rank, _arr(ys.extents), _arr(ys.strides), y.data_ptr(), ys.offset), defer, (x, y))
 
     def arg_reduce(self, name, dtype, index_dtype, rows, k, xs, x, ys, y, defer=False):
         sp, sb = self.scratch(self.lib.dlfx_arg_reduce_scratch_bytes(dtype, rows, k))

@@ -118,6 +118,27 @@ int dlfx_reduce(dlfx_stream_t stream, const char* name, int dtype, int64_t m, in
                 void* y, int64_t y_offset,
                 void* scratch, size_t scratch_bytes);
 
+/* ---------------------------------------------------------------- reduce, allocation-free
+ * No counterpart in the reference.  For callers that cannot allocate device memory or carry a
+ * scratch buffer: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  Same arguments, results and status codes as dlfx_reduce, without the scratch
+ * pair: the partial accumulators of long-row and strided-axis reductions live in an array of
+ * DLFX_REDUCE_STATIC_SCRATCH_BYTES bytes that is part of the library's device code (every GPU
+ * the library runs on holds one copy until the process ends).  The call allocates and frees
+ * nothing.  The array covers every shape dlfx_reduce accepts (its scratch query never asks for
+ * more); a shape whose partials would not fit is refused with DLFX_ERR_TOO_LARGE and nothing
+ * is enqueued.  The first call on a device looks the array's address up (the device that is
+ * current must be the one the stream belongs to).  All calls on one GPU share that GPU's
+ * array: calls that overlap in time on one GPU -- different streams, or different host threads
+ * -- race on it and must be serialised by the caller.
+ */
+#define DLFX_REDUCE_STATIC_SCRATCH_BYTES 3178496
+int dlfx_reduce_static(dlfx_stream_t stream, const char* name, int dtype, int64_t m, int64_t n,
+                       int x_rank, const int64_t* x_dims, const int64_t* x_strides,
+                       const void* x, int64_t x_offset,
+                       int y_rank, const int64_t* y_dims, const int64_t* y_strides,
+                       void* y, int64_t y_offset);
+
 /* ---------------------------------------------------------------- arg_reduce
  * Replaces gpgpu::dnn::arg_reduce<T> (gdnn.h:138-144; caller
  * reduce_detail.h:134-147).  The reduced axis is the last one of x_dims
