@@ -79,7 +79,7 @@ __device__ __forceinline__ V team_reduce(V v, Join join, V* lds) {
 template <typename S, int TEAM, int ITEMS, int KIND, bool VEC>
 __global__ __launch_bounds__(TEAM > 256 ? TEAM : 256)
 __attribute__((amdgpu_waves_per_eu(TEAM >= 1024 && sizeof(typename ComputeOf<S>::type) * ITEMS <= 128 ? 8 : 1)))      // two 1024-thread rows per CU
-void softmax_rows(const S* __restrict__ x, S* __restrict__ y, int64_t m, int64_t n) {
+void softmax_rows(const S* x, S* y, int64_t m, int64_t n) {          // y may be x: no restrict
     using T = typename ComputeOf<S>::type;
     constexpr int BLOCK = TEAM > 256 ? TEAM : 256;
     constexpr int V = VEC ? 16 / static_cast<int>(sizeof(S)) : 1;
@@ -115,6 +115,10 @@ void softmax_rows(const S* __restrict__ x, S* __restrict__ y, int64_t m, int64_t
         }
     }
 
+    // Whether the row starts with a NaN, read now: in place, another wave of the team may store
+    // element 0 as soon as it has left the last team reduction.
+    const bool leading_nan = live && xr[0] != xr[0];
+
     if constexpr (KIND == kHardmax) {
         // the serial loop (dnn_detail.h:334-346) keeps the first element that is strictly larger
         // than everything before it: the first occurrence of the largest non-NaN value, or
@@ -128,7 +132,7 @@ void softmax_rows(const S* __restrict__ x, S* __restrict__ y, int64_t m, int64_t
         for (int k = ITEMS - 1; k >= 0; --k)
             if (v[k] == mx && index_of(k) < n32) hot = index_of(k);      // this thread's indices grow with k
         hot = team_reduce<TEAM>(hot, [](int32_t a, int32_t b) { return a < b ? a : b; }, reinterpret_cast<int32_t*>(lds_raw));
-        if (hot >= n32 || (live && xr[0] != xr[0])) hot = 0;               // all NaN or -inf, or a leading NaN
+        if (hot >= n32 || leading_nan) hot = 0;                            // all NaN or -inf, or a leading NaN
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) v[k] = index_of(k) == hot ? T(1) : T(0);
     } else {
@@ -138,7 +142,7 @@ void softmax_rows(const S* __restrict__ x, S* __restrict__ y, int64_t m, int64_t
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) mx = (mx < v[k]) ? v[k] : mx;
         mx = team_reduce<TEAM>(mx, [](T a, T b) { return (a < b) ? b : a; }, reinterpret_cast<T*>(lds_raw));
-        if (live && xr[0] != xr[0]) mx = static_cast<T>(xr[0]);
+        if (leading_nan) mx = static_cast<T>(xr[0]);           // stores only follow the next team reduction
         T sum = T(0);
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
@@ -179,7 +183,7 @@ constexpr int kStreamBatch = 8;
 
 // Rows too long for registers: one 1024-thread workgroup per row, two passes over the row.
 template <typename S, int KIND>
-__global__ __launch_bounds__(1024) void softmax_rows_streamed(const S* __restrict__ x, S* __restrict__ y, int64_t n) {
+__global__ __launch_bounds__(1024) void softmax_rows_streamed(const S* x, S* y, int64_t n) {
     using T = typename ComputeOf<S>::type;
     constexpr int TEAM = 1024;
     __shared__ alignas(16) unsigned char lds_raw[(TEAM / kWave) * sizeof(MaxAt<T>)];
@@ -317,7 +321,7 @@ __global__ __launch_bounds__(1024) void softmax_split_partials(const S* __restri
 }
 
 template <typename S, int KIND>
-__global__ __launch_bounds__(1024) void softmax_split_apply(const S* __restrict__ x, S* __restrict__ y, int64_t n, int64_t tiles,
+__global__ __launch_bounds__(1024) void softmax_split_apply(const S* x, S* y, int64_t n, int64_t tiles,
                                                             int64_t tile_len,
                                                             const SoftPartial<typename ComputeOf<S>::type>* __restrict__ part) {
     using T = typename ComputeOf<S>::type;

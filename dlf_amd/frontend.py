@@ -97,7 +97,7 @@ class Tensor:
         """The viewed elements in row-major order in storage of their own (the reference's
         reorder(X, Y)); on the device when the backend can copy a strided view there."""
         copy = getattr(self.backend, "copy_view", None)
-        if copy is not None and all(s >= 0 for s in self.shape.strides):
+        if copy is not None:
             return Tensor(self.backend, Shape(list(self.shape.extents)), copy(self.storage, self.shape), self.dtype)
         return Tensor.from_numpy(self.backend, self.numpy())
 

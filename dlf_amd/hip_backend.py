@@ -99,6 +99,10 @@ def _declare(lib):
     lib.dlfx_gather_indices.restype = c_int
     lib.dlfx_gather_indices.argtypes = [c_void_p, c_int64, c_int64, c_int, c_int, _I64P,
                                         c_void_p, c_int64, c_void_p, c_int64]
+    lib.dlfx_copy.restype = c_int
+    lib.dlfx_copy.argtypes = [c_void_p, c_int, c_int, _I64P, c_void_p, c_int64, _I64P, c_void_p, c_int64, _I64P]
+    lib.dlfx_fill.restype = c_int
+    lib.dlfx_fill.argtypes = [c_void_p, c_int, c_int, _I64P, _I64P, c_void_p, c_int64, c_void_p]
     return lib
 
 
@@ -114,7 +118,8 @@ EXPORTS = ("dlfx_version", "dlfx_status_string", "dlfx_last_hip_error", "dlfx_se
            "dlfx_top_k_scratch_bytes", "dlfx_top_k",
            "dlfx_count_scratch_bytes", "dlfx_count",
            "dlfx_scan_nonzero_scratch_bytes", "dlfx_scan_nonzero", "dlfx_gather_indices",
-           "dlfx_merge_scratch_bytes", "dlfx_merge", "dlfx_softmax_scratch_bytes", "dlfx_softmax")
+           "dlfx_merge_scratch_bytes", "dlfx_merge", "dlfx_softmax_scratch_bytes", "dlfx_softmax",
+           "dlfx_copy", "dlfx_fill")
 
 
 def load_library():
@@ -157,6 +162,11 @@ def _torch_dtype(np_dtype):
     return _NP_TO_TORCH[np.dtype(np_dtype)]
 
 
+def _dtype_code_of(torch_dtype, torch):
+    return {torch.float32: 0, torch.float64: 1, torch.int32: 2, torch.int64: 3, torch.float16: 4, torch.int16: 5,
+            torch.bool: 6, torch.complex64: 7, torch.complex128: 8}[torch_dtype]
+
+
 class HipBackend:
     """Backend whose six boundary calls go through the C ABI onto the current HIP stream."""
 
@@ -183,10 +193,29 @@ class HipBackend:
         return storage.cpu().numpy()
 
     def copy_view(self, storage, shape):
-        """Row-major device copy of a strided view with non-negative strides (a layout copy, done
-        by torch: it is not one of the axis primitives)."""
-        view = self.torch.as_strided(storage, list(shape.extents), list(shape.strides), shape.offset)
-        return view.clone(memory_format=self.torch.contiguous_format).view(-1)
+        """Row-major device copy of a strided view (dlfx_copy: the reference's reorder(X, Y))."""
+        out = self.torch.empty(max(1, shape.size), dtype=storage.dtype, device=self.device)
+        dense = []
+        size = 1
+        for e in reversed(shape.extents):
+            dense.insert(0, size)
+            size *= e
+        self.copy(_dtype_code_of(storage.dtype, self.torch), shape.extents, storage, shape.offset, shape.strides, out, 0, dense)
+        return out
+
+    def copy(self, dtype, extents, x, x_offset, x_strides, y, y_offset, y_strides, defer=False):
+        return self._issue(self.lib.dlfx_copy, "dlfx_copy", (dtype, len(extents), _arr(extents)),
+                           (x.data_ptr(), x_offset, _arr(x_strides), y.data_ptr(), y_offset, _arr(y_strides)), defer, (x, y))
+
+    def fill(self, dtype, extents, strides, x, x_offset, value, defer=False):
+        host_types = {0: np.float32, 1: np.float64, 2: np.int32, 3: np.int64, 4: np.float16, 5: np.int16,
+                      6: np.bool_, 7: np.complex64, 8: np.complex128}
+        v = np.array([value], dtype=host_types[dtype])
+        call = self._issue(self.lib.dlfx_fill, "dlfx_fill", (dtype, len(extents), _arr(extents), _arr(strides)),
+                           (x.data_ptr(), x_offset, v.ctypes.data_as(c_void_p)), defer, (x,))
+        if call is None:
+            return None
+        return lambda v=v: call()
 
     def wrap(self, tensor):
         """Use an existing contiguous 1-D device tensor as storage."""

@@ -380,14 +380,29 @@ inline void cumsum(const DevTensor<T>& X, DevTensor<T>& Y, int axis = -1, bool e
     scan("cumsum", X, Y, axis, exclusive, reverse);
 }
 
+// ---------------------------------------------------------------- reorder
+// dlf/include/tensor/reorder.h reorder(X, Y) on device tensors: the viewed elements of X in
+// row-major order in Y, copied on the device (gpgpu::dnn::copy).
+template <typename T>
+void reorder(const DevTensor<T>& X, DevTensor<T>& Y) {
+    if (&X == &Y && X.shape().is_contiguous()) return;
+    DevTensor<T> out;
+    DevTensor<T>& dst = (&X == &Y) ? out : Y;
+    dst.resize(X.shape());
+    gpgpu::dnn::copy(X.size(), X.shape().extents(), X.data(), X.shape().offset(), X.shape().strides(),
+                     dst.data(), dst.shape().offset(), dst.shape().strides());
+    if (&X == &Y) Y = std::move(out);
+}
+
 // ---------------------------------------------------------------- sort / argsort / top_k
 namespace detail {
 template <typename T>
 void copy_dense(const DevTensor<T>& X, DevTensor<T>& Y) {
     if (&X == &Y) return;
-    const Tensor<T> h = X.read();
-    Y.resize(X.shape());
-    Y.data().write(gpgpu::current::queue(), h.data(), h.size());
+    reorder(X, Y);
+}
+inline void zero_indices(DevTensor<int32_t>& I) {
+    gpgpu::dnn::fill(I.size(), I.data(), I.shape().offset(), int32_t(0));
 }
 }  // namespace detail
 
@@ -422,8 +437,7 @@ void argsort(const DevTensor<T>& X, DevTensor<int32_t>& I, int axis = -1, bool d
         gpgpu::dnn::argsort(descending ? 1 : 0, xv.shape().extents(), xv.data(), xv.shape().offset(), xv.shape().strides(),
                             iv.data(), iv.shape().offset(), iv.shape().strides());
     } else {
-        std::vector<int32_t> zeros(I.size(), 0);
-        I.data().write(gpgpu::current::queue(), zeros.data(), zeros.size());
+        detail::zero_indices(I);
     }
 }
 template <typename T>
@@ -440,8 +454,7 @@ void argsort(const DevTensor<T>& X, DevTensor<T>& Y, DevTensor<int32_t>& I, int 
                             iv.data(), iv.shape().offset(), iv.shape().strides());
     } else {
         detail::copy_dense(X, Y);
-        std::vector<int32_t> zeros(I.size(), 0);
-        I.data().write(gpgpu::current::queue(), zeros.data(), zeros.size());
+        detail::zero_indices(I);
     }
 }
 template <typename T>
@@ -481,28 +494,33 @@ inline std::pair<DevTensor<T>, DevTensor<int32_t>> top_k(const DevTensor<T>& X, 
 // in place.
 namespace dnn {
 namespace detail {
+// A dense input goes straight through the out-of-place routine; any other view is first laid out
+// row-major in Y on the device (the reference's reorder(X, Y)) and normalised in place there.
 template <typename T, typename Fn>
 void normalize_rows(const DevTensor<T>& X, DevTensor<T>& Y, int axis, Fn fn) {
     dlf::detail::norm_axis(static_cast<int>(X.rank()), axis);
     size_t m = 1;
     for (int i = 0; i < axis; ++i) m *= X.extent(i);
     const size_t n = X.size() / m;
-    if (&X != &Y || !X.shape().is_contiguous()) Y = dev(X.read());       // row-major copy of the viewed elements
-    fn(m, n, Y.data(), Y.shape().offset());
+    if (X.shape().is_contiguous()) {
+        if (&X != &Y) Y.resize(X.shape());
+        fn(m, n, X.data(), X.shape().offset(), Y.data(), Y.shape().offset());
+    } else {
+        reorder(X, Y);
+        fn(m, n, Y.data(), Y.shape().offset(), Y.data(), Y.shape().offset());
+    }
 }
 }  // namespace detail
-template <typename T>
-void softmax(const DevTensor<T>& X, DevTensor<T>& Y, int axis = 1) {
-    detail::normalize_rows(X, Y, axis, [](size_t m, size_t n, gpgpu::Buffer<T>& b, size_t off) { gpgpu::dnn::softmax(m, n, b, off); });
-}
-template <typename T>
-void logsoftmax(const DevTensor<T>& X, DevTensor<T>& Y, int axis = 1) {
-    detail::normalize_rows(X, Y, axis, [](size_t m, size_t n, gpgpu::Buffer<T>& b, size_t off) { gpgpu::dnn::logsoftmax(m, n, b, off); });
-}
-template <typename T>
-void hardmax(const DevTensor<T>& X, DevTensor<T>& Y, int axis = 1) {
-    detail::normalize_rows(X, Y, axis, [](size_t m, size_t n, gpgpu::Buffer<T>& b, size_t off) { gpgpu::dnn::hardmax(m, n, b, off); });
-}
+#define DLF_DEFINE_ROW_NORMALIZER(fn)                                                                     \
+    template <typename T>                                                                                 \
+    void fn(const DevTensor<T>& X, DevTensor<T>& Y, int axis = 1) {                                       \
+        detail::normalize_rows(X, Y, axis, [](size_t m, size_t n, const gpgpu::Buffer<T>& x, size_t xo,  \
+                                              gpgpu::Buffer<T>& y, size_t yo) { gpgpu::dnn::fn(m, n, x, xo, y, yo); }); \
+    }
+DLF_DEFINE_ROW_NORMALIZER(softmax)
+DLF_DEFINE_ROW_NORMALIZER(logsoftmax)
+DLF_DEFINE_ROW_NORMALIZER(hardmax)
+#undef DLF_DEFINE_ROW_NORMALIZER
 template <typename T>
 inline DevTensor<T> softmax(const DevTensor<T>& X, int axis = 1) { DevTensor<T> Y; softmax(X, Y, axis); return Y; }
 template <typename T>

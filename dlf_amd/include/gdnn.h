@@ -61,7 +61,7 @@ void reduce(const std::string& name, const size_t m, const size_t n,
     const int dt = detail::dtype_of<T>::value;
     auto xd = detail::signed_vec(x_dims), xs = detail::signed_vec(x_strides);
     auto yd = detail::signed_vec(y_dims), ys = detail::signed_vec(y_strides);
-    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_reduce_scratch_bytes(dt, m, n));
+    auto tmp = queue.context().getTemporaryBuffer<char>(dlfx_reduce_scratch_bytes(dt, m, n));
     detail::EventScope ev(queue, event);
     check_status(dlfx_reduce(queue.stream(), name.c_str(), dt, m, n,
                              static_cast<int>(xd.size()), xd.data(), xs.data(), x_buffer.data(), x_offset,
@@ -80,7 +80,7 @@ void arg_reduce(const std::string& name, const size_t n, const size_t k,
     const int dt = detail::dtype_of<T>::value;
     auto xd = detail::signed_vec(x_dims), xs = detail::signed_vec(x_strides);
     auto yd = detail::signed_vec(y_dims), ys = detail::signed_vec(y_strides);
-    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_arg_reduce_scratch_bytes(dt, n, k));
+    auto tmp = queue.context().getTemporaryBuffer<char>(dlfx_arg_reduce_scratch_bytes(dt, n, k));
     detail::EventScope ev(queue, event);
     check_status(dlfx_arg_reduce(queue.stream(), name.c_str(), dt, DLFX_I32, n, k,
                                  static_cast<int>(xd.size()), xd.data(), xs.data(), x_buffer.data(), x_offset,
@@ -97,7 +97,7 @@ void scan(const std::string& name, const size_t m, const size_t n,
           const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
     const int dt = detail::dtype_of<T>::value;
     auto d = detail::signed_vec(dims), xs = detail::signed_vec(x_strides), ys = detail::signed_vec(y_strides);
-    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_scan_scratch_bytes(dt, m, n));
+    auto tmp = queue.context().getTemporaryBuffer<char>(dlfx_scan_scratch_bytes(dt, m, n));
     detail::EventScope ev(queue, event);
     check_status(dlfx_scan(queue.stream(), name.c_str(), dt, m, n, exclusive ? 1 : 0,
                            static_cast<int>(d.size()), d.data(), x_buffer.data(), x_offset, xs.data(),
@@ -115,7 +115,7 @@ void sort(const int dir, const std::vector<size_t>& dims,
     const int64_t n = d.empty() ? 1 : d.back();
     int64_t m = 1;
     for (size_t i = 0; i + 1 < d.size(); ++i) m *= d[i];
-    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_sort_scratch_bytes(dt, m, n));
+    auto tmp = queue.context().getTemporaryBuffer<char>(dlfx_sort_scratch_bytes(dt, m, n));
     detail::EventScope ev(queue, event);
     check_status(dlfx_sort(queue.stream(), dir, dt, static_cast<int>(d.size()), d.data(),
                            x_buffer.data(), x_offset, xs.data(), y_buffer.data(), y_offset, ys.data(),
@@ -133,7 +133,7 @@ void argsort(const int dir, const std::vector<size_t>& dims,
     const int64_t n = d.empty() ? 1 : d.back();
     int64_t m = 1;
     for (size_t i = 0; i + 1 < d.size(); ++i) m *= d[i];
-    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_argsort_scratch_bytes(dt, m, n));
+    auto tmp = queue.context().getTemporaryBuffer<char>(dlfx_argsort_scratch_bytes(dt, m, n));
     detail::EventScope ev(queue, event);
     check_status(dlfx_argsort(queue.stream(), dir, dt, DLFX_I32, static_cast<int>(d.size()), d.data(),
                               x_buffer.data(), x_offset, xs.data(), nullptr, 0, nullptr,
@@ -153,7 +153,7 @@ void argsort(const int dir, const std::vector<size_t>& dims,
     const int64_t n = d.empty() ? 1 : d.back();
     int64_t m = 1;
     for (size_t i = 0; i + 1 < d.size(); ++i) m *= d[i];
-    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_argsort_scratch_bytes(dt, m, n));
+    auto tmp = queue.context().getTemporaryBuffer<char>(dlfx_argsort_scratch_bytes(dt, m, n));
     detail::EventScope ev(queue, event);
     check_status(dlfx_argsort(queue.stream(), dir, dt, DLFX_I32, static_cast<int>(d.size()), d.data(),
                               x_buffer.data(), x_offset, xs.data(), y_buffer.data(), y_offset, ys.data(),
@@ -174,7 +174,7 @@ void top_k(const size_t limit, const int dir,
     const int64_t n = xd.empty() ? 1 : xd.back();
     int64_t m = 1;
     for (size_t i = 0; i + 1 < xd.size(); ++i) m *= xd[i];
-    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_top_k_scratch_bytes(dt, m, n, limit));
+    auto tmp = queue.context().getTemporaryBuffer<char>(dlfx_top_k_scratch_bytes(dt, m, n, limit));
     detail::EventScope ev(queue, event);
     check_status(dlfx_top_k(queue.stream(), limit, dir, dt, DLFX_I32, static_cast<int>(xd.size()), xd.data(), yd.data(),
                             x_buffer.data(), x_offset, xs.data(), y_buffer.data(), y_offset, ys.data(),
@@ -185,30 +185,124 @@ void top_k(const size_t limit, const int dir,
 // gpgpu/include/gdnn.h:253-264: in place on the rows of a contiguous [m, n] matrix
 namespace detail {
 template <typename T>
-void softmax_family(const char* name, const size_t m, const size_t n, Buffer<T>& x_buffer, const size_t x_offset,
-                    const Queue& queue, Event* event) {
-    EventScope ev(queue, event);
+void softmax_family(const char* name, const size_t m, const size_t n, const Buffer<T>& x_buffer, const size_t x_offset,
+                    Buffer<T>& y_buffer, const size_t y_offset, const Queue& queue, Event* event) {
     const int dt = dtype_of<T>::value;
-    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_softmax_scratch_bytes(dt, m, n));      // only few, long rows need any
+    auto tmp = queue.context().getTemporaryBuffer<char>(dlfx_softmax_scratch_bytes(dt, m, n));      // only few, long rows need any
+    EventScope ev(queue, event);
     check_status(dlfx_softmax(queue.stream(), name, dt, m, n, x_buffer.data(), x_offset,
-                              x_buffer.data(), x_offset, tmp.data(), tmp.size()), name);
+                              y_buffer.data(), y_offset, tmp.bytes(), tmp.byte_size()), name);
     ev.done();
 }
 }  // namespace detail
 template <typename T>
 void softmax(const size_t m, const size_t n, Buffer<T>& x_buffer, const size_t x_offset,
              const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
-    detail::softmax_family("softmax", m, n, x_buffer, x_offset, queue, event);
+    detail::softmax_family("softmax", m, n, x_buffer, x_offset, x_buffer, x_offset, queue, event);
+}
+// Out of place (no counterpart in the reference, whose routine works in place only): rows of the
+// contiguous [m, n] matrix at x go to y, which may be the same buffer.
+template <typename T>
+void softmax(const size_t m, const size_t n, const Buffer<T>& x_buffer, const size_t x_offset,
+        Buffer<T>& y_buffer, const size_t y_offset,
+        const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    detail::softmax_family("softmax", m, n, x_buffer, x_offset, y_buffer, y_offset, queue, event);
 }
 template <typename T>
 void logsoftmax(const size_t m, const size_t n, Buffer<T>& x_buffer, const size_t x_offset,
                 const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
-    detail::softmax_family("logsoftmax", m, n, x_buffer, x_offset, queue, event);
+    detail::softmax_family("logsoftmax", m, n, x_buffer, x_offset, x_buffer, x_offset, queue, event);
+}
+// Out of place (no counterpart in the reference, whose routine works in place only): rows of the
+// contiguous [m, n] matrix at x go to y, which may be the same buffer.
+template <typename T>
+void logsoftmax(const size_t m, const size_t n, const Buffer<T>& x_buffer, const size_t x_offset,
+        Buffer<T>& y_buffer, const size_t y_offset,
+        const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    detail::softmax_family("logsoftmax", m, n, x_buffer, x_offset, y_buffer, y_offset, queue, event);
 }
 template <typename T>
 void hardmax(const size_t m, const size_t n, Buffer<T>& x_buffer, const size_t x_offset,
              const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
-    detail::softmax_family("hardmax", m, n, x_buffer, x_offset, queue, event);
+    detail::softmax_family("hardmax", m, n, x_buffer, x_offset, x_buffer, x_offset, queue, event);
+}
+// Out of place (no counterpart in the reference, whose routine works in place only): rows of the
+// contiguous [m, n] matrix at x go to y, which may be the same buffer.
+template <typename T>
+void hardmax(const size_t m, const size_t n, const Buffer<T>& x_buffer, const size_t x_offset,
+        Buffer<T>& y_buffer, const size_t y_offset,
+        const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    detail::softmax_family("hardmax", m, n, x_buffer, x_offset, y_buffer, y_offset, queue, event);
+}
+
+// gpgpu/include/gdnn.h:14-17 (routine xcopy.cpp:59-81): strided view to strided view
+template <typename T>
+void copy(const size_t n, const std::vector<size_t>& dims,
+          const Buffer<T>& x_buffer, const size_t x_offset, const std::vector<size_t>& x_stride,
+          Buffer<T>& y_buffer, const size_t y_offset, const std::vector<size_t>& y_stride,
+          const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    auto d = detail::signed_vec(dims), xs = detail::signed_vec(x_stride), ys = detail::signed_vec(y_stride);
+    size_t size = 1;
+    for (auto e : dims) size *= e;
+    if (size != n || x_stride.size() != dims.size() || y_stride.size() != dims.size())
+        throw LogicError("gpgpu::dnn::copy: extents, strides and n disagree");
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_copy(queue.stream(), detail::dtype_of<T>::value, static_cast<int>(d.size()), d.data(),
+                           x_buffer.data(), x_offset, xs.data(), y_buffer.data(), y_offset, ys.data()), "gpgpu::dnn::copy");
+    ev.done();
+}
+
+// gpgpu/include/gdnn.h:9-11 (xcopy.cpp:15-55, kernel xcopy.cl:8-26): y_size elements; a shorter x repeats
+template <typename T>
+void copy(const size_t x_size, const Buffer<T>& x_buffer, const size_t x_offset,
+          const size_t y_size, Buffer<T>& y_buffer, const size_t y_offset,
+          const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    if (x_size == 0 || y_size == 0) throw RuntimeErrorCode(DLFX_ERR_INVALID_ARGUMENT, "gpgpu::dnn::copy");
+    detail::EventScope ev(queue, event);
+    const int dt = detail::dtype_of<T>::value;
+    if (x_size >= y_size) {
+        const int64_t d[1] = {static_cast<int64_t>(y_size)}, one[1] = {1};
+        check_status(dlfx_copy(queue.stream(), dt, 1, d, x_buffer.data(), x_offset, one, y_buffer.data(), y_offset, one),
+                     "gpgpu::dnn::copy");
+    } else {
+        const size_t reps = y_size / x_size, rest = y_size % x_size;
+        const int64_t d[2] = {static_cast<int64_t>(reps), static_cast<int64_t>(x_size)};
+        const int64_t xs[2] = {0, 1}, ys[2] = {static_cast<int64_t>(x_size), 1};
+        check_status(dlfx_copy(queue.stream(), dt, 2, d, x_buffer.data(), x_offset, xs, y_buffer.data(), y_offset, ys),
+                     "gpgpu::dnn::copy");
+        if (rest) {
+            const int64_t dr[1] = {static_cast<int64_t>(rest)}, one[1] = {1};
+            check_status(dlfx_copy(queue.stream(), dt, 1, dr, x_buffer.data(), x_offset, one, y_buffer.data(),
+                                   y_offset + reps * x_size, one), "gpgpu::dnn::copy");
+        }
+    }
+    ev.done();
+}
+
+// gpgpu/include/gdnn.h:20-22
+template <typename T>
+void fill(const size_t n, Buffer<T>& x_buffer, const size_t x_offset, const T value,
+          const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    const int64_t d[1] = {static_cast<int64_t>(n)}, one[1] = {1};
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_fill(queue.stream(), detail::dtype_of<T>::value, 1, d, one, x_buffer.data(), x_offset, &value),
+                 "gpgpu::dnn::fill");
+    ev.done();
+}
+
+// gpgpu/include/gdnn.h:24-26
+template <typename T>
+void fill(const size_t n, const std::vector<size_t>& dims, const std::vector<size_t>& strides,
+          Buffer<T>& x_buffer, const size_t x_offset, const T value,
+          const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    auto d = detail::signed_vec(dims), st = detail::signed_vec(strides);
+    size_t size = 1;
+    for (auto e : dims) size *= e;
+    if (size != n || strides.size() != dims.size()) throw LogicError("gpgpu::dnn::fill: extents, strides and n disagree");
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_fill(queue.stream(), detail::dtype_of<T>::value, static_cast<int>(d.size()), d.data(), st.data(),
+                           x_buffer.data(), x_offset, &value), "gpgpu::dnn::fill");
+    ev.done();
 }
 
 // gpgpu/include/gdnn.h:147-155
@@ -230,7 +324,7 @@ void merge(const int dir,
     const size_t n = z_dims.back();
     size_t m = 1;
     for (size_t i = 0; i + 1 < z_dims.size(); ++i) m *= z_dims[i];
-    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_merge_scratch_bytes(dt, m, n));
+    auto tmp = queue.context().getTemporaryBuffer<char>(dlfx_merge_scratch_bytes(dt, m, n));
     detail::EventScope ev(queue, event);
     check_status(dlfx_merge(queue.stream(), dir, dt, static_cast<int>(zd.size()),
                             xd.data(), xs.data(), x_buffer.data(), x_offset,
@@ -251,7 +345,7 @@ void count(const size_t m, const size_t n, const T value,
     const int dt = detail::dtype_of<T>::value;
     auto xd = detail::signed_vec(x_dims), xs = detail::signed_vec(x_strides);
     auto yd = detail::signed_vec(y_dims), ys = detail::signed_vec(y_strides);
-    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_count_scratch_bytes(dt, m, n));
+    auto tmp = queue.context().getTemporaryBuffer<char>(dlfx_count_scratch_bytes(dt, m, n));
     detail::EventScope ev(queue, event);
     check_status(dlfx_count(queue.stream(), dt, m, n, &value,
                             static_cast<int>(xd.size()), xd.data(), xs.data(), x_buffer.data(), x_offset,
@@ -269,7 +363,7 @@ void scan_nonzero(const size_t m, const size_t n,
                   const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
     const int dt = detail::dtype_of<T>::value;
     auto d = detail::signed_vec(dims), xs = detail::signed_vec(x_strides), ys = detail::signed_vec(y_strides);
-    auto tmp = current::context().getTemporaryBuffer<char>(dlfx_scan_nonzero_scratch_bytes(dt, m, n));
+    auto tmp = queue.context().getTemporaryBuffer<char>(dlfx_scan_nonzero_scratch_bytes(dt, m, n));
     detail::EventScope ev(queue, event);
     check_status(dlfx_scan_nonzero(queue.stream(), dt, m, n, exclusive ? 1 : 0,
                                    static_cast<int>(d.size()), d.data(), x_buffer.data(), x_offset, xs.data(),

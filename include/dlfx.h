@@ -274,6 +274,25 @@ int dlfx_gather_indices(dlfx_stream_t stream, int64_t m, int64_t n, int row_majo
                         const int32_t* indices, int64_t indices_offset,
                         int32_t* output, int64_t output_offset);
 
+/* ---------------------------------------------------------------- copy
+ * Replaces the strided gpgpu::dnn::copy<T> (gdnn.h:14-17; routine xcopy.cpp:59-81): element
+ * (i0, ..., ik) of the view (dims, x_strides) of x goes to the same element of the view
+ * (dims, y_strides) of y.  A stride of 0 on the x side repeats elements.  The views must not
+ * overlap unless they are the same dense view.  Every dtype (elements move as opaque words).
+ * This is the device-side reorder(X, Y) the front-ends use before the in-place softmax family
+ * and for sort / argsort along an axis of extent 1.
+ */
+int dlfx_copy(dlfx_stream_t stream, int dtype, int rank, const int64_t* dims,
+              const void* x, int64_t x_offset, const int64_t* x_strides,
+              void* y, int64_t y_offset, const int64_t* y_strides);
+
+/* ---------------------------------------------------------------- fill
+ * Replaces gpgpu::dnn::fill<T> (gdnn.h:20-26): every element of the view becomes *value (one
+ * element of `dtype` in host memory, read before the call returns).
+ */
+int dlfx_fill(dlfx_stream_t stream, int dtype, int rank, const int64_t* dims, const int64_t* strides,
+              void* x, int64_t x_offset, const void* value);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

@@ -7,7 +7,8 @@
 // :2304-2377 (sort), dlf/test/DNNTest.cpp:861-1019 (argmax/argmin),
 // dlf/test/model/PredictTest.cpp:609-637 (top_k), dlf/test/UniformTest.cpp:2065-2080
 // (count), :2553-2561 (nonzero), :2250-2283 (merge), dlf/test/DNNTest.cpp:796-858
-// (softmax, logsoftmax, hardmax).
+// (softmax, logsoftmax, hardmax), dlf/test/model/PredictTest.cpp:290-319 (Reduce nodes),
+// :609-637 (TopK node).
 #include <algorithm>
 #include <cmath>
 #include <complex>
@@ -15,6 +16,7 @@
 #include <random>
 
 #include "dev_tensor.h"
+#include "onnx_nodes.h"
 
 using namespace dlf;
 
@@ -307,6 +309,281 @@ static void test_errors_and_temporaries() {
     CHECK(ev.getElapsedTime() > 0.0f);
 }
 
+// Scratch comes from the context of the queue a routine is given (xreduce.cpp:78, xscan.cpp:82),
+// not from the calling thread's: a call on another queue leaves this thread's arena alone.
+static void test_queue_contexts() {
+    const gpgpu::Queue& mine = gpgpu::current::queue();
+    CHECK(mine.context() == gpgpu::current::context());
+    gpgpu::Queue other;                                   // a context and arena of its own
+    CHECK(other.context() != mine.context());
+    gpgpu::Queue sibling = mine.context().createQueue(); // shares this thread's context, as in the reference
+    CHECK(sibling.context() == mine.context() && sibling != mine);
+
+    // a live temporary of this thread's context with known contents
+    const size_t words = 1 << 16;
+    auto held = mine.context().getTemporaryBuffer<int32_t>(words);
+    std::vector<int32_t> pattern(words);
+    for (size_t i = 0; i < words; ++i) pattern[i] = static_cast<int32_t>(i * 2654435761u);
+    held.write(mine, pattern.data(), words, held.offset());
+
+    // long rows on the other queue: both routines need scratch (partials, tile states)
+    const size_t m = 3, n = 1 << 20;
+    std::vector<int32_t> xs(m * n);
+    std::mt19937 rng(11);
+    for (auto& v : xs) v = static_cast<int32_t>(rng() % 100);
+    auto X = dev(Tensor<int32_t>({m, n}, xs));
+    DevTensor<int32_t> S(Shape({m})), C(Shape({m, n}));
+    const size_t in_use = mine.context().temporary_bytes_in_use();
+    gpgpu::dnn::reduce<int32_t>("reduce_sum", m, n, {m, n}, {n, 1}, X.data(), 0, {m}, {1}, S.data(), 0, other);
+    gpgpu::dnn::scan<int32_t>("cumsum", m, n, false, {m, n}, X.data(), 0, {n, 1}, C.data(), 0, {n, 1}, other);
+    other.finish();
+    CHECK(mine.context().temporary_bytes_in_use() == in_use);
+    CHECK(other.context().temporary_bytes_in_use() == 0);
+    auto sums = S.read(), scan = C.read();
+    bool ok = true;
+    for (size_t r = 0; r < m; ++r) {
+        int32_t acc = 0;
+        for (size_t j = 0; j < n; ++j) {
+            acc += xs[r * n + j];
+            ok = ok && scan.values()[r * n + j] == acc;
+        }
+        ok = ok && sums.values()[r] == acc;
+    }
+    CHECK(ok);
+    std::vector<int32_t> back(words);
+    held.read(mine, back.data(), words, held.offset());
+    CHECK(back == pattern);
+}
+
+// A live temporary survives a softmax that needs scratch of its own from the same arena
+// (few rows, too long for one workgroup's registers).
+static void test_softmax_scratch_is_its_own_slice() {
+    const gpgpu::Queue& q = gpgpu::current::queue();
+    const size_t words = 1 << 14;
+    auto held = q.context().getTemporaryBuffer<float>(words);
+    std::vector<float> pattern(words);
+    for (size_t i = 0; i < words; ++i) pattern[i] = static_cast<float>(i) * 0.5f - 7.0f;
+    held.write(q, pattern.data(), words, held.offset());
+    const size_t m = 4, n = 1 << 20;
+    CHECK(dlfx_softmax_scratch_bytes(DLFX_F32, m, n) > 0);
+    std::vector<float> xs(m * n);
+    std::mt19937 rng(12);
+    for (auto& v : xs) v = static_cast<float>(rng() % 2000) * 0.001f;
+    auto X = dev(Tensor<float>({m, n}, xs));
+    auto Y = dnn::softmax(X, 1).read();
+    bool ok = true;
+    for (size_t r = 0; r < m; ++r) {
+        double sum = 0;
+        for (size_t j = 0; j < n; ++j) sum += Y.values()[r * n + j];
+        ok = ok && std::fabs(sum - 1.0) < 1e-4;
+    }
+    CHECK(ok);
+    std::vector<float> back(words);
+    held.read(q, back.data(), words, held.offset());
+    CHECK(back == pattern);
+}
+
+// Out-of-place and strided row normalisation, extent-1 sort / argsort: no host round trip.
+static void test_layout_steps_stay_on_the_device() {
+    auto host = Tensor<float>({2, 3}, {-1, 0, 1, 2, 4, 8});
+    auto X = dev(host);
+    DevTensor<float> Y;
+    size_t& reads = gpgpu::detail::device_to_host_reads();
+    const size_t before = reads;
+    dnn::softmax(X, Y, 1);                                   // dense input, out of place
+    DevTensor<float> Z;
+    dnn::logsoftmax(X.transpose(), Z, 1);                    // strided view: device copy, then in place
+    DevTensor<float> S;
+    auto col = dev(Tensor<float>({4, 1}, {3, 1, 2, 0}));
+    sort(col, S, 1);                                         // extent 1: a copy
+    DevTensor<float> AV;
+    DevTensor<int32_t> AI;
+    argsort(col.transpose(), AV, AI, 0);                     // [1, 4] along axis 0: copy + zero indices
+    CHECK(reads == before);
+    CHECK(near(Y.read(), Tensor<float>({2, 3}, {0.09003057f, 0.24472848f, 0.66524094f, 0.00242826f, 0.01794253f, 0.97962922f})));
+    // rows of the transposed view are (-1, 2), (0, 4), (1, 8)
+    auto z = Z.read();
+    CHECK(z.shape() == Shape({3, 2}));
+    CHECK(std::fabs(z.values()[0] - (-3.0485873f)) < 1e-4 && std::fabs(z.values()[1] - (-0.0485873f)) < 1e-4);
+    CHECK(std::fabs(z.values()[5] - (-0.00091147f)) < 1e-5);
+    CHECK(X.read() == host);                                 // the input is untouched
+    CHECK(S.read() == Tensor<float>({4, 1}, {3, 1, 2, 0}));
+    CHECK(AV.read() == Tensor<float>({1, 4}, {3, 1, 2, 0}));
+    CHECK(AI.read() == Tensor<int32_t>({1, 4}, {0, 0, 0, 0}));
+    // reorder of a flipped, sliced view
+    auto R = dev(Tensor<int32_t>({3, 4}).range());
+    DevTensor<int32_t> RR;
+    reorder(flip(R, 1).slice(0, 1, 3), RR);
+    CHECK(RR.read() == Tensor<int32_t>({2, 4}, {7, 6, 5, 4, 11, 10, 9, 8}));
+    // the flat copy repeats a shorter source (xcopy.cl:8-26); fill writes a strided view
+    auto src = dev(Tensor<int32_t>({3}, {1, 2, 3}));
+    DevTensor<int32_t> dst(Shape({8}));
+    gpgpu::dnn::copy<int32_t>(3, src.data(), 0, 8, dst.data(), 0);
+    CHECK(dst.read() == Tensor<int32_t>({8}, {1, 2, 3, 1, 2, 3, 1, 2}));
+    gpgpu::dnn::fill<int32_t>(4, {4}, {2}, dst.data(), 1, -5);
+    CHECK(dst.read() == Tensor<int32_t>({8}, {1, -5, 3, -5, 2, -5, 1, -5}));
+}
+
+// ONNX nodes as the interpreter binds them (predict.h:1078-1201, 1486-1510, 2031-2044):
+// attribute defaults, output shapes and order.
+static void test_onnx_nodes() {
+    using namespace dlf::predict;
+    // PredictTest.cpp:290-319
+    auto X = dev(Tensor<float>({3, 2, 2}).range(1));
+    DevTensor<float> A, B, C;
+    Node<float> n;
+    n.op_type = "ReduceSum";
+    n.inputs = {&X};
+    n.outputs = {&A};
+    evaluate(n);                                                        // every axis, keepdims 1
+    CHECK(A.read() == Tensor<float>({1, 1, 1}, {78}));
+    n.attrs.set_is("axes", {1});
+    n.outputs = {&B};
+    evaluate(n);
+    CHECK(B.read() == Tensor<float>({3, 1, 2}, {4, 6, 12, 14, 20, 22}));
+    n.attrs.set_i("keepdims", 0);
+    n.outputs = {&C};
+    evaluate(n);
+    CHECK(C.read() == Tensor<float>({3, 2}, {4, 6, 12, 14, 20, 22}));
+    // every reduction node kind against a host loop over axis -1
+    const char* kinds[] = {"ReduceMax", "ReduceMin", "ReduceSum", "ReduceSumSquare", "ReduceMean", "ReduceProd",
+                           "ReduceLogSum", "ReduceLogSumExp", "ReduceL1", "ReduceL2"};
+    auto P = Tensor<float>({2, 3}, {1.5f, 0.5f, 2.0f, 3.0f, 0.25f, 1.0f});
+    auto dP = dev(P);
+    for (const char* kind : kinds) {
+        Node<float> r;
+        DevTensor<float> out;
+        r.op_type = kind;
+        r.inputs = {&dP};
+        r.outputs = {&out};
+        r.attrs.set_is("axes", {-1}).set_i("keepdims", 0);
+        evaluate(r);
+        std::vector<float> want;
+        for (int row = 0; row < 2; ++row) {
+            const float* v = P.data() + row * 3;
+            const std::string k = kind;
+            double acc = (k == "ReduceProd") ? 1 : 0, mx = v[0], mn = v[0];
+            for (int j = 0; j < 3; ++j) {
+                mx = std::max<double>(mx, v[j]);
+                mn = std::min<double>(mn, v[j]);
+                if (k == "ReduceProd") acc *= v[j];
+                else if (k == "ReduceSumSquare" || k == "ReduceL2") acc += double(v[j]) * v[j];
+                else if (k == "ReduceLogSumExp") acc += std::exp(double(v[j]));
+                else if (k == "ReduceL1") acc += std::fabs(v[j]);
+                else acc += v[j];
+            }
+            if (k == "ReduceMax") acc = mx;
+            if (k == "ReduceMin") acc = mn;
+            if (k == "ReduceMean") acc /= 3;
+            if (k == "ReduceLogSum" || k == "ReduceLogSumExp") acc = std::log(acc);
+            if (k == "ReduceL2") acc = std::sqrt(acc);
+            want.push_back(static_cast<float>(acc));
+        }
+        CHECK(near(out.read(), Tensor<float>({2}, want), 1e-5));
+    }
+
+    // ArgMax / ArgMin: axis 0 and keepdims 1 by default (DNNTest.cpp:861-1019 vectors)
+    auto M = dev(Tensor<float>({2, 3, 4}, {21, 22, 2, 15, 16, 7, 14, 0, 18, 20, 6, 9, 23, 4, 12, 11, 10, 5, 3, 8, 17, 19, 13, 1}));
+    DevTensor<int32_t> I;
+    Node<float> am;
+    am.op_type = "ArgMax";
+    am.inputs = {&M};
+    am.index_outputs = {&I};
+    evaluate(am);
+    CHECK(I.read() == Tensor<int32_t>({1, 3, 4}, {1, 0, 1, 0, 0, 0, 0, 1, 0, 0, 1, 0}));
+    am.attrs.set_i("axis", 2).set_i("keepdims", 0);
+    evaluate(am);
+    CHECK(I.read() == Tensor<int32_t>({2, 3}, {1, 0, 1, 0, 0, 1}));
+    am.op_type = "ArgMin";
+    am.attrs.set_i("axis", 1).set_i("keepdims", 1);
+    evaluate(am);
+    CHECK(I.read() == Tensor<int32_t>({2, 1, 4}, {1, 1, 0, 1, 1, 0, 1, 2}));
+
+    // CumSum: the axis is a tensor read on the host; exclusive / reverse default to 0; in place
+    auto S = dev(Tensor<int32_t>({2, 3}, {1, 2, 3, 4, 5, 6}));
+    Tensor<int64_t> axis({}, {1});
+    DevTensor<int32_t> CS;
+    Node<int32_t> cs;
+    cs.op_type = "CumSum";
+    cs.inputs = {&S};
+    cs.host_inputs = {&axis};
+    cs.outputs = {&CS};
+    evaluate(cs);
+    CHECK(CS.read() == Tensor<int32_t>({2, 3}, {1, 3, 6, 4, 9, 15}));
+    cs.attrs.set_i("exclusive", 1).set_i("reverse", 1);
+    evaluate(cs);
+    CHECK(CS.read() == Tensor<int32_t>({2, 3}, {5, 3, 0, 11, 6, 0}));
+    cs.attrs = Attributes();
+    cs.outputs = {&S};                                                  // allocInplace: output is the input
+    evaluate(cs);
+    CHECK(S.read() == Tensor<int32_t>({2, 3}, {1, 3, 6, 4, 9, 15}));
+
+    // TopK (PredictTest.cpp:609-637): K is an int64 tensor; axis -1, largest 1 by default
+    auto T = dev(Tensor<float>({3, 4}, {0, 1, 2, 3, 7, 6, 5, 4, 10, 11, 9, 8}));
+    Tensor<int64_t> K({1}, {3});
+    DevTensor<float> TV;
+    DevTensor<int32_t> TI;
+    Node<float> tk;
+    tk.op_type = "TopK";
+    tk.inputs = {&T};
+    tk.host_inputs = {&K};
+    tk.outputs = {&TV};
+    tk.index_outputs = {&TI};
+    evaluate(tk);
+    CHECK(TV.read() == Tensor<float>({3, 3}, {3, 2, 1, 7, 6, 5, 11, 10, 9}));
+    CHECK(TI.read() == Tensor<int32_t>({3, 3}, {3, 2, 1, 0, 1, 2, 1, 0, 2}));
+    tk.attrs.set_i("axis", 0).set_i("largest", 0);
+    Tensor<int64_t> K1({1}, {1});
+    tk.host_inputs = {&K1};
+    evaluate(tk);
+    CHECK(TV.read() == Tensor<float>({1, 4}, {0, 1, 2, 3}));
+    CHECK(TI.read() == Tensor<int32_t>({1, 4}, {0, 0, 0, 0}));
+
+    // NonZero: [rank, n] (UniformTest.cpp:2553-2561 layout)
+    auto Z = dev(Tensor<float>({2, 3}, {1, 0, 0, 0, 2, 3}));
+    DevTensor<int32_t> NZ;
+    Node<float> nz;
+    nz.op_type = "NonZero";
+    nz.inputs = {&Z};
+    nz.index_outputs = {&NZ};
+    evaluate(nz);
+    CHECK(NZ.read() == Tensor<int32_t>({2, 3}, {0, 1, 1, 0, 1, 2}));
+
+    // Softmax family: axis 1 by default; rows are everything from the axis on
+    auto L = dev(Tensor<float>({2, 3}, {-1, 0, 1, 2, 4, 8}));
+    DevTensor<float> SO;
+    Node<float> sm;
+    sm.op_type = "Softmax";
+    sm.inputs = {&L};
+    sm.outputs = {&SO};
+    evaluate(sm);
+    CHECK(near(SO.read(), Tensor<float>({2, 3}, {0.09003057f, 0.24472848f, 0.66524094f, 0.00242826f, 0.01794253f, 0.97962922f})));
+    sm.op_type = "Hardmax";
+    sm.attrs.set_i("axis", 0);                                          // one row of six
+    evaluate(sm);
+    CHECK(SO.read() == Tensor<float>({2, 3}, {0, 0, 0, 0, 0, 1}));
+    sm.op_type = "LogSoftmax";
+    sm.attrs.set_i("axis", 1);
+    auto op = make_operator(sm);                                        // bound once, run twice
+    op->evaluate();
+    op->evaluate();
+    CHECK(std::fabs(SO.read().values()[2] - std::log(0.66524094f)) < 1e-5);
+
+    bool threw = false;
+    Node<float> conv;
+    conv.op_type = "Conv";
+    conv.inputs = {&L};
+    conv.outputs = {&SO};
+    try { evaluate(conv); } catch (const unsupported_operator&) { threw = true; }
+    CHECK(threw);
+    threw = false;
+    Node<float> bad;
+    bad.op_type = "TopK";
+    bad.inputs = {&T};
+    try { evaluate(bad); } catch (const std::invalid_argument&) { threw = true; }
+    CHECK(threw);
+}
+
 int main() {
     test_reduce();
     test_arg_reduce();
@@ -319,6 +596,10 @@ int main() {
     test_16bit_types();
     test_complex();
     test_errors_and_temporaries();
+    test_queue_contexts();
+    test_softmax_scratch_is_its_own_slice();
+    test_layout_steps_stay_on_the_device();
+    test_onnx_nodes();
     std::printf("veneer_test: %d checks, %d failed\n", g_checked, g_failed);
     return g_failed ? 1 : 0;
 }

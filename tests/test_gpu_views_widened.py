@@ -113,3 +113,32 @@ def test_contiguous_copy_of_views(hip_backend):
     C = T.contiguous()
     C.storage.zero_()
     assert (T.numpy() == before).all()
+
+
+@pytest.mark.parametrize("dtype", [np.int16, np.float32, np.int64, np.complex128, np.bool_])
+def test_copy_and_fill_over_views(hip_backend, dtype):
+    """dlfx_copy / dlfx_fill (gdnn.h:14-26): strided view to strided view, every element width."""
+    rng = np.random.default_rng(212)
+    a = rng.integers(0, 2 if dtype == np.bool_ else 1000, size=(6, 5, 8, 3)).astype(dtype)
+    T = Tensor.from_numpy(hip_backend, a)
+    for view, want in ((T.transpose([3, 1, 0, 2]), a.transpose(3, 1, 0, 2)),
+                       (T.flip([0, 2]), a[::-1, :, ::-1, :]),
+                       (T.slice([1, 2], [5, 7], [0, 2], [2, 3]), a[1:5:2, :, 2:7:3, :]),
+                       (T.transpose([1, 0, 2, 3]).slice([0], [1], [3]), a.transpose(1, 0, 2, 3)[:, :, :, 0:1])):
+        assert np.array_equal(view.contiguous().numpy(), want)
+    # into a strided destination: the transposed view of a second tensor
+    D = Tensor.from_numpy(hip_backend, np.zeros((8, 6), dtype=dtype))
+    src = Tensor.from_numpy(hip_backend, a[:, 0, :, 0].copy())             # [6, 8]
+    dv = D.transpose([1, 0])
+    hip_backend.copy(F.dtype_code(dtype), src.shape.extents, src.storage, 0, src.shape.strides,
+                     D.storage, dv.shape.offset, dv.shape.strides)
+    assert np.array_equal(D.numpy(), a[:, 0, :, 0].T)
+    # a stride of 0 on the source repeats it
+    row = Tensor.from_numpy(hip_backend, a[0, 0, :, 0].copy())             # [8]
+    hip_backend.copy(F.dtype_code(dtype), [6, 8], row.storage, 0, [0, 1], src.storage, 0, [8, 1])
+    assert np.array_equal(src.numpy(), np.broadcast_to(a[0, 0, :, 0], (6, 8)))
+    # fill of every other column
+    value = a.reshape(-1)[7]
+    hip_backend.fill(F.dtype_code(dtype), [6, 4], [8, 2], src.storage, 1, value)
+    got = src.numpy()
+    assert (got[:, 1::2] == value).all() and np.array_equal(got[:, 0::2], np.broadcast_to(a[0, 0, 0::2, 0], (6, 4)))
