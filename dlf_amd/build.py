@@ -13,7 +13,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "obj")
 LIB = os.path.join(HERE, "lib", "libdlfx.so")
 
-SOURCES = ["lib.hip", "reduce.hip", "scan.hip", "sort.hip", "topk.hip", "nonzero.hip", "merge.hip", "softmax.hip", "copy.hip"]
+SOURCES = ["lib.hip", "reduce.hip", "scan.hip", "sort.hip", "sort_split.hip", "topk.hip", "nonzero.hip", "merge.hip", "softmax.hip", "copy.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

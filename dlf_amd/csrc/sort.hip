@@ -23,7 +23,7 @@
 #include <cstring>
 #include <type_traits>
 
-#include "common.hip.h"
+#include "sort_common.hip.h"
 
 namespace dlfx {
 namespace {
@@ -37,7 +37,6 @@ constexpr int kBlock = 256;
 #endif
 constexpr int kPassBlock = DLFX_SORT_PASS_BLOCK;       // threads of a sort_pass workgroup
 constexpr int kPassWaves = kPassBlock / kWave;
-constexpr int kRadix = 256;
 constexpr int64_t kMaxRow = (int64_t(1) << 27) - 1;   // counts share a status word with 5 tag bits
 
 int g_sort_poll_limit = 2048;
@@ -53,74 +52,16 @@ __device__ unsigned long long g_phase_cycles[kPhaseSlots * 8];
 #define DLFX_PHASE_BEGIN() do { } while (0)
 #endif
 
-enum KeyKind { kKeyInt = 0, kKeyFloat = 1 };
-
-template <typename K>
-struct KeyTraits;
-template <>
-struct KeyTraits<uint16_t> {
-    static constexpr int kPasses = 2;
-    static constexpr uint16_t kSign = 0x8000u;
+// Which rows of a call the digit passes take: the bucket route (sort_split.hip) marks the rows
+// it sorts with a first word of 1 in its per-row records and counts the others; with no
+// records every row is taken here.
+struct RowRoutes {
+    const uint32_t* records;      // null: every row
+    size_t stride_words;
+    const uint32_t* other_rows;   // how many rows the bucket route left
+    __device__ __forceinline__ bool none_here() const { return records && *other_rows == 0u; }
+    __device__ __forceinline__ bool elsewhere(int64_t row) const { return records && records[row * stride_words] == 1u; }
 };
-template <>
-struct KeyTraits<uint32_t> {
-    static constexpr int kPasses = 4;
-    static constexpr uint32_t kSign = 0x80000000u;
-};
-template <>
-struct KeyTraits<uint64_t> {
-    static constexpr int kPasses = 8;
-    static constexpr uint64_t kSign = 0x8000000000000000ull;
-};
-
-template <typename K>
-__device__ __forceinline__ K encode_key(K bits, int kind, int descending) {
-    constexpr K S = KeyTraits<K>::kSign;
-    K k = (kind == kKeyFloat) ? ((bits & S) ? ~bits : (bits | S)) : (bits ^ S);
-    return descending ? ~k : k;
-}
-template <typename K>
-__device__ __forceinline__ K decode_key(K k, int kind, int descending) {
-    constexpr K S = KeyTraits<K>::kSign;
-    if (descending) k = ~k;
-    return (kind == kKeyFloat) ? ((k & S) ? (k & ~S) : ~k) : (k ^ S);
-}
-
-// What the passes of one sort read and write.
-template <typename K>
-struct PassIo {
-    const K* x;               // strided input, read by the first pass that runs
-    DimMap xmap;
-    int64_t sx;
-    K* kbuf[2];               // contiguous [m][n] ping-pong buffers between passes
-    uint32_t* vbuf[2];        // ... and their index payloads (argsort)
-    K* y;                     // strided value output of the last pass (may be null)
-    DimMap ymap;
-    int64_t sy;
-    void* idx;                // strided index output of the last pass (may be null)
-    DimMap imap;
-    int64_t si;
-    int idx64;
-    int kind, descending;
-    int canon_zero;           // argsort of floats: -0.0 and +0.0 are one key
-    int restore_zero;         // ... and the value written for a zero key is re-read from x
-    // rows side by side in memory (the axis is an outer dimension): workgroups are dealt to the
-    // 8 XCDs in turn, so workgroup b takes block (b % 8) * xcd_blocks + b / 8 and neighbouring
-    // rows, which share cache lines, meet in one L2 (0: workgroup b takes block b)
-    int64_t xcd_blocks;
-};
-
-template <typename K>
-__device__ __forceinline__ int64_t block_of(const PassIo<K>& io) {
-    if (io.xcd_blocks == 0) return blockIdx.x;
-    return static_cast<int64_t>(blockIdx.x % 8) * io.xcd_blocks + blockIdx.x / 8;
-}
-
-template <typename K>
-__device__ __forceinline__ K key_of_element(const PassIo<K>& io, K bits) {
-    if (io.canon_zero && static_cast<K>(bits << 1) == 0) bits = 0;      // -0.0 -> +0.0
-    return encode_key<K>(bits, io.kind, io.descending);
-}
 
 // ------------------------------------------------------------------ histograms
 // One read of the input builds the digit histograms of every pass for a chunk of a row.
@@ -130,14 +71,16 @@ __device__ __forceinline__ K key_of_element(const PassIo<K>& io, K bits) {
 // keys (constant bytes: small integers, narrow float ranges) is added once per wave.
 template <typename K>
 __global__ __launch_bounds__(kBlock) void sort_histogram(PassIo<K> io, int64_t n, int64_t chunk, int64_t chunks_per_row,
-                                                         uint32_t* __restrict__ ghist) {
+                                                         RowRoutes routes, uint32_t* __restrict__ ghist) {
     constexpr int P = KeyTraits<K>::kPasses;
     constexpr int U = 32 / sizeof(K);                 // keys in flight per thread
     constexpr int R = 32 / P;                         // copies: 8 (32-bit keys) or 4 (64-bit keys): 32 KB
     __shared__ uint32_t hist[P * kRadix * R];
+    if (routes.none_here()) return;
+    const int64_t row = blockIdx.x / chunks_per_row;
+    if (routes.elsewhere(row)) return;
     for (int i = threadIdx.x; i < P * kRadix * R; i += kBlock) hist[i] = 0;
     __syncthreads();
-    const int64_t row = blockIdx.x / chunks_per_row;
     const int64_t c = blockIdx.x - row * chunks_per_row;
     const K* xrow = io.x + io.xmap.at(row);
     const int64_t lo = c * chunk;
@@ -194,78 +137,45 @@ __global__ __launch_bounds__(kBlock) void sort_histogram(PassIo<K> io, int64_t n
 // b handles one (row, pass) pair.  moves[b] receives the bits of the digit that are not the
 // same in all keys of the row: none means the pass would not change the order of the row (the
 // row then skips it), and the ranking only needs to look at those bits.  `all_bits` forces
-// every pass of every row to run.  largest[b] receives the count of the most frequent digit.
-__global__ __launch_bounds__(kRadix) void sort_bases(uint32_t* __restrict__ ghist, uint32_t* __restrict__ moves,
-                                                     uint32_t* __restrict__ largest, int all_bits) {
+// every pass of every row to run.
+__global__ __launch_bounds__(kRadix) void sort_bases(uint32_t* __restrict__ ghist, uint32_t* __restrict__ moves, int all_bits,
+                                                     RowRoutes routes) {
     __shared__ uint32_t wave_tot[kRadix / kWave];
-    __shared__ uint32_t wave_or[kRadix / kWave], wave_and[kRadix / kWave], wave_max[kRadix / kWave];
+    __shared__ uint32_t wave_or[kRadix / kWave], wave_and[kRadix / kWave];
+    if (routes.none_here()) return;
     uint32_t* g = ghist + static_cast<int64_t>(blockIdx.x) * kRadix;
     const uint32_t v = g[threadIdx.x];
     const uint32_t incl = wave_scan_inclusive(v, 0u, [](uint32_t a, uint32_t b) { return a + b; });
     const uint32_t ors = wave_reduce(v ? threadIdx.x : 0u, [](uint32_t a, uint32_t b) { return a | b; });
     const uint32_t ands = wave_reduce(v ? threadIdx.x : 0xffu, [](uint32_t a, uint32_t b) { return a & b; });
-    const uint32_t most = wave_reduce(v, [](uint32_t a, uint32_t b) { return a > b ? a : b; });
     const int w = threadIdx.x / kWave;
     if (lane_id() == kWave - 1) {
         wave_tot[w] = incl;
         wave_or[w] = ors;
         wave_and[w] = ands;
-        wave_max[w] = most;
     }
     __syncthreads();
     uint32_t pre = 0;
     for (int i = 0; i < w; ++i) pre += wave_tot[i];
     g[threadIdx.x] = pre + incl - v;
     if (threadIdx.x == 0) {
-        uint32_t o = 0, a = 0xffu, mx = 0;
+        uint32_t o = 0, a = 0xffu;
         for (int i = 0; i < kRadix / kWave; ++i) {
             o |= wave_or[i];
             a &= wave_and[i];
-            mx = wave_max[i] > mx ? wave_max[i] : mx;
         }
         moves[blockIdx.x] = all_bits ? 0xffu : (o ^ a);
-        largest[blockIdx.x] = mx;                         // keys of the row that share the most frequent digit
     }
 }
 
-__global__ __launch_bounds__(kBlock) void sort_clear(uint32_t* __restrict__ p, int64_t words) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (i < words) p[i] = 0u;
-}
-
-// Rows whose keys the most significant varying digit spreads into runs ("buckets") of at most
-// `cap` keys are sorted most significant digit first: one tiled pass on that digit leaves the
-// buckets, in source order, in the first ping-pong buffer, and a workgroup then sorts each
-// bucket by its lower digits on chip (sort_buckets) and writes the outputs: the keys cross HBM
-// five times instead of 2 * passes + 1 times.  Returns that digit's pass for such a row, -1
-// for a row that takes the least-significant-digit-first passes (cap 0: every row).
-template <int P>
-__device__ __forceinline__ int msd_digit(const uint32_t* __restrict__ row_moves, const uint32_t* __restrict__ row_largest, uint32_t cap) {
-    if (cap == 0u) return -1;
-    int q = -1, varying = 0;
-#pragma unroll
-    for (int p = 0; p < P; ++p) {
-        if (row_moves[p] != 0u) {
-            q = p;
-            ++varying;
-        }
-    }
-    if (varying < 2 || row_largest[q] > cap) return -1;
-    return q;
+__global__ __launch_bounds__(kBlock) void sort_clear(uint32_t* __restrict__ p, int64_t words, RowRoutes routes) {
+    if (routes.none_here()) return;
+    const int64_t i = (static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x) * 4;
+    if (i + 4 <= words) *reinterpret_cast<uint4*>(p + i) = make_uint4(0u, 0u, 0u, 0u);
+    else for (int64_t j = i; j < words; ++j) p[j] = 0u;
 }
 
 // ------------------------------------------------------------------ one pass
-// Status word of (tile, digit): [tag:4 | inclusive:1 | count:27]; a word is valid
-// for pass p when its tag is p + 1, so the array is cleared once per sort.
-// Values of sort_pass's pass argument beside a pass number: the launch that takes only the
-// rows sorted most significant digit first (each on its own digit), and the flag on a pass
-// number that says those rows have such a launch.
-constexpr int kLeadingPass = -1, kLeadingPassElsewhere = 64;
-constexpr uint32_t kCountMask = (1u << 27) - 1;
-__device__ __forceinline__ uint32_t make_status(int pass, bool inclusive, uint32_t count) {
-    return (static_cast<uint32_t>(pass + 1) << 28) | (inclusive ? (1u << 27) : 0u) | count;
-}
-
 template <typename K, bool PAIRS, int ITEMS>
 struct PassShared {
     uint32_t wave_hist[kPassWaves][kRadix];       // per-wave digit counts, then per-wave offsets
@@ -283,37 +193,28 @@ struct PassShared {
 // pass it runs reads the strided input, and its place in the ping-pong buffers alternates
 // over the passes it does run.
 template <typename K, bool PAIRS, int ITEMS, bool LAST>
-__global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(sizeof(K) == 8 && PAIRS && ITEMS > 8 ? 2 : DLFX_SORT_WAVES))) void sort_pass(PassIo<K> io, int pass_arg, int64_t rows, int64_t n, int64_t tiles_per_row,
+__global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SORT_WAVES))) void sort_pass(PassIo<K> io, int pass, int64_t rows, int64_t n, int64_t tiles_per_row,
                                                     const uint32_t* __restrict__ gbase,
                                                     const uint32_t* __restrict__ moves,
-                                                    const uint32_t* __restrict__ largest, uint32_t bucket_cap,
+                                                    RowRoutes routes,
                                                     uint32_t* __restrict__ status, int poll_limit) {
     constexpr int P = KeyTraits<K>::kPasses;
     constexpr int TILE = kPassBlock * ITEMS;
     constexpr int W = 4;    // status words of earlier tiles fetched per look-back step
     __shared__ PassShared<K, PAIRS, ITEMS> sm;
 
+    if (routes.none_here()) return;
     // workgroups are handed out in index order and dealt round-robin over the chip's eight
     // parts: tile t of every row comes before tile t + 1 of any row, so a tile's predecessors
     // in its row have usually finished when it looks back, and the tiles of a row share a
     // second-level cache when the number of rows is a multiple of eight
     const int64_t t = blockIdx.x / rows;
     const int64_t row = blockIdx.x - t * rows;
+    if (routes.elsewhere(row)) return;
     const uint32_t* row_moves = moves + row * P;
-    // a row sorted most significant digit first runs that digit's pass only, from the input
-    // into the first buffer: in the launch of that pass, or - when `pass_arg` is kLeadingPass
-    // or kLeadingPassElsewhere - in a launch of its own that takes those rows only (with its
-    // own tile size, hence its own status tag: the words of its tiles lie where other rows'
-    // tiles of the other launches lie)
-    const int msd = msd_digit<P>(row_moves, largest + row * P, bucket_cap);
-    const bool to_buckets = msd >= 0;
-    const bool own_launch = pass_arg == kLeadingPass;
-    if (own_launch ? !to_buckets : to_buckets && (pass_arg >= kLeadingPassElsewhere || (pass_arg & ~kLeadingPassElsewhere) != msd)) return;
-    const int pass = own_launch ? msd : (pass_arg & ~kLeadingPassElsewhere);
-    const int tag = own_launch ? P : pass;
+    const int tag = pass;
     int ran = 0;            // passes before this one that this row ran
-    if (!to_buckets)
-        for (int p = 0; p < pass; ++p) ran += row_moves[p] ? 1 : 0;
+    for (int p = 0; p < pass; ++p) ran += row_moves[p] ? 1 : 0;
     if (!LAST && row_moves[pass] == 0u) return;
     const bool first = ran == 0;
     const K* __restrict__ src_keys = first ? nullptr : io.kbuf[(ran - 1) & 1];
@@ -574,7 +475,7 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(size
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) pay[k] = sm.vals[k * kPassBlock + tid];
     }
-    if (!LAST || to_buckets) {
+    if (!LAST) {
         K* dk = dst_keys + row_off;
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k)
@@ -626,225 +527,6 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(size
 // waves' counts, scatter through LDS, reload in element order.  Digits that are the same in
 // the whole row are skipped.  Element e of the row is item e / 64 % ITEMS of lane e % 64 of
 // wave e / (64 * ITEMS), before and after every pass.
-constexpr int kSmallMoves = 256;         // keys that the run walk of sort_in_workgroup may move (one thread each)
-
-template <typename K, bool PAIRS, int ITEMS, int WAVES = 4>
-struct SmallShared {
-    uint32_t n_moves;
-    uint2 moves[kSmallMoves];
-    uint32_t wave_hist[WAVES][kRadix];
-    uint32_t scan_tmp[kRadix / kWave];
-    K wave_or[WAVES], wave_and[WAVES];
-    K keys[WAVES * kWave * ITEMS];
-    uint32_t vals[PAIRS ? WAVES * kWave * ITEMS : 1];
-};
-
-// The passes of a workgroup-resident sort: key[] / val[] hold the row (or bucket) in element
-// order before and after; `ors` / `ands` are this thread's OR / AND over its valid keys, `top`
-// the number of low digits that may differ (digits from `top` up are known to be equal),
-// `valid` the number of keys that are not padding.  The workgroup has WAVES wavefronts (4 or 8).
-//
-// When more digits vary than `valid` distinct keys need to tell most of them apart (about as
-// many bits as the square of `valid` has, so that evenly spread keys leave a few pairs that
-// agree), the leading ones of the varying digits are sorted first.  Keys that then agree with
-// a neighbour in all of those digits form short runs, in source order; every key of such a run
-// finds its place by comparing whole keys with the run's other members (at most kNear to
-// either side), and the lower digits never ran.  A longer run makes every digit run from that
-// arrangement, which the passes so far left in source order among equal keys.
-template <typename K, bool PAIRS, int ITEMS, int WAVES = 4>
-__device__ __forceinline__ void sort_in_workgroup(SmallShared<K, PAIRS, ITEMS, WAVES>& sm, K (&key)[ITEMS], uint32_t (&val)[PAIRS ? ITEMS : 1],
-                                                  K ors, K ands, int valid, int top) {
-    static_assert(WAVES * kWave >= kRadix, "a thread per digit");
-    const bool padded = valid < WAVES * kWave * ITEMS;
-    const int tid = threadIdx.x;
-    const int lane = lane_id();
-    const int w = tid / kWave;
-    const int seg = w * kWave * ITEMS + lane;
-    ors = wave_reduce(ors, [](K a, K b) { return static_cast<K>(a | b); });
-    ands = wave_reduce(ands, [](K a, K b) { return static_cast<K>(a & b); });
-    if (lane == 0) {
-        sm.wave_or[w] = ors;
-        sm.wave_and[w] = ands;
-    }
-    if (tid == 0) sm.n_moves = 0u;
-    __syncthreads();
-    K any = 0, all = ~K(0);
-#pragma unroll
-    for (int i = 0; i < WAVES; ++i) {
-        any |= sm.wave_or[i];
-        all &= sm.wave_and[i];
-    }
-    const K differ = static_cast<K>(any & ~all);
-    const bool owner = tid < kRadix;                       // thread d < 256 owns digit d
-
-    int first = 0;                                         // lowest digit of this round of passes
-    if constexpr (sizeof(K) > 4) {
-        const int enough = (2 * (32 - __builtin_clz(static_cast<uint32_t>(valid > 1 ? valid - 1 : 1))) - 2 + 7) / 8;
-        int varying = 0;
-        for (int p = top - 1; p >= 0; --p) {
-            if ((static_cast<uint32_t>(differ >> (8 * p)) & 0xffu) != 0u && ++varying == enough) first = p;
-        }
-        if (varying <= enough) first = 0;
-    }
-
-    for (;;) {
-        for (int pass = first; pass < top; ++pass) {
-            const int shift = 8 * pass;
-            const uint32_t moves = static_cast<uint32_t>(differ >> shift) & 0xffu;
-            if (moves == 0u) continue;                        // this digit is the same in the whole row
-            const uint32_t vary = padded ? 0xffu : moves;     // padding differs from the row in other bits too
-            for (int i = tid; i < WAVES * kRadix; i += WAVES * kWave) (&sm.wave_hist[0][0])[i] = 0;
-            __syncthreads();
-
-            // ---- rank inside the wave, in element order
-            uint32_t rank[ITEMS];
-#pragma unroll
-            for (int k0 = 0; k0 < ITEMS; k0 += 2) {
-                uint32_t d[2], before[2], cnt[2];
-#pragma unroll
-                for (int j = 0; j < 2; ++j) d[j] = static_cast<uint32_t>(key[k0 + j] >> shift) & 0xffu;
-                uint32_t peers_lo[2] = {0xffffffffu, 0xffffffffu}, peers_hi[2] = {0xffffffffu, 0xffffffffu};
-                for (uint32_t bits = vary; bits != 0u; bits &= bits - 1u) {
-                    const uint32_t b = static_cast<uint32_t>(__builtin_ctz(bits));
-#pragma unroll
-                    for (int j = 0; j < 2; ++j) {
-                        const int32_t ones = __builtin_amdgcn_sbfe(static_cast<int32_t>(d[j]), b, 1u);
-                        const unsigned long long vote = __ballot(ones < 0);
-                        peers_lo[j] &= ~(static_cast<uint32_t>(vote) ^ static_cast<uint32_t>(ones));
-                        peers_hi[j] &= ~(static_cast<uint32_t>(vote >> 32) ^ static_cast<uint32_t>(ones));
-                    }
-                }
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    before[j] = __builtin_amdgcn_mbcnt_hi(peers_hi[j], __builtin_amdgcn_mbcnt_lo(peers_lo[j], 0u));
-                    cnt[j] = static_cast<uint32_t>(__popc(peers_lo[j]) + __popc(peers_hi[j]));
-                }
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const uint32_t seen = sm.wave_hist[w][d[j]];
-                    rank[k0 + j] = seen + before[j];
-                    __builtin_amdgcn_wave_barrier();
-                    if (before[j] == 0) sm.wave_hist[w][d[j]] = seen + cnt[j];
-                    __builtin_amdgcn_wave_barrier();
-                }
-            }
-            __syncthreads();
-
-            // ---- thread d owns digit d: where the digit starts in the row, and each wave's share of it
-            {
-                uint32_t wave_count[WAVES];
-                uint32_t count = 0;
-                if (owner) {
-#pragma unroll
-                    for (int i = 0; i < WAVES; ++i) {
-                        wave_count[i] = sm.wave_hist[i][tid];
-                        count += wave_count[i];
-                    }
-                }
-                const uint32_t incl = wave_scan_inclusive(count, 0u, [](uint32_t a, uint32_t b) { return a + b; });
-                if (owner && lane == kWave - 1) sm.scan_tmp[w] = incl;
-                __syncthreads();
-                if (owner) {
-                    uint32_t run = incl - count;
-                    for (int i = 0; i < w; ++i) run += sm.scan_tmp[i];
-#pragma unroll
-                    for (int i = 0; i < WAVES; ++i) {
-                        sm.wave_hist[i][tid] = run;
-                        run += wave_count[i];
-                    }
-                }
-            }
-            __syncthreads();
-
-            // ---- scatter to the sorted position, reload in element order
-#pragma unroll
-            for (int k = 0; k < ITEMS; ++k) {
-                const uint32_t pos = sm.wave_hist[w][static_cast<uint32_t>(key[k] >> shift) & 0xffu] + rank[k];
-                sm.keys[pos] = key[k];
-                if constexpr (PAIRS) sm.vals[pos] = val[k];
-            }
-            __syncthreads();
-#pragma unroll
-            for (int k = 0; k < ITEMS; ++k) {
-                key[k] = sm.keys[seg + k * kWave];
-                if constexpr (PAIRS) val[k] = sm.vals[seg + k * kWave];
-            }
-            // (the three barriers of the next pass lie between these reads and its scatter)
-        }
-        if (first == 0) break;
-        // Runs of neighbours that agree in every digit sorted so far.  Keys with such a neighbour
-        // are few: each walks its run (the tile holds what the registers hold), and the ones that
-        // have to move are listed.
-        constexpr int kNear = 3;
-        const int sh = 8 * first;
-        uint32_t near = 0;                                 // bit k: item k has a neighbour of its run
-#pragma unroll
-        for (int k = 0; k < ITEMS; ++k) {
-            const int e = seg + k * kWave;
-            if (e < valid) {
-                const K lead = key[k] >> sh;
-                const bool left = e > 0 && (sm.keys[e - 1] >> sh) == lead;
-                const bool right = e + 1 < valid && (sm.keys[e + 1] >> sh) == lead;
-                if (left || right) near |= 1u << k;
-            }
-        }
-        bool longer = false;
-        for (; near != 0u; near &= near - 1u) {
-            const int e = seg + __builtin_ctz(near) * kWave;
-            const K mine = sm.keys[e];
-            const K lead = mine >> sh;
-            int before = 0, ahead = 0;                     // members of the run to the left; of the whole run that come first
-            int j = e - 1;
-            for (; j >= 0 && before < kNear; --j, ++before) {
-                const K other = sm.keys[j];
-                if ((other >> sh) != lead) break;
-                ahead += other <= mine ? 1 : 0;
-            }
-            if (before == kNear && j >= 0 && (sm.keys[j] >> sh) == lead) longer = true;
-            int after = 0;
-            for (j = e + 1; j < valid && after < kNear; ++j, ++after) {
-                const K other = sm.keys[j];
-                if ((other >> sh) != lead) break;
-                ahead += other < mine ? 1 : 0;
-            }
-            if (after == kNear && j < valid && (sm.keys[j] >> sh) == lead) longer = true;
-            const int dest = e - before + ahead;
-            if (dest != e) {
-                const uint32_t slot = atomicAdd(&sm.n_moves, 1u);
-                if (slot < static_cast<uint32_t>(kSmallMoves)) sm.moves[slot] = make_uint2(static_cast<uint32_t>(e), static_cast<uint32_t>(dest));
-                else longer = true;
-            }
-        }
-        if (__syncthreads_or(longer ? 1 : 0)) {            // a run too long, or too many moves: every digit runs
-            first = 0;
-            continue;
-        }
-        const int n_moves = static_cast<int>(sm.n_moves);
-        if (n_moves != 0) {
-            uint2 mv = make_uint2(0u, 0u);
-            K moved_key = 0;
-            uint32_t moved_val = 0;
-            if (tid < n_moves) {
-                mv = sm.moves[tid];
-                moved_key = sm.keys[mv.x];
-                if constexpr (PAIRS) moved_val = sm.vals[mv.x];
-            }
-            __syncthreads();
-            if (tid < n_moves) {
-                sm.keys[mv.y] = moved_key;
-                if constexpr (PAIRS) sm.vals[mv.y] = moved_val;
-            }
-            __syncthreads();
-#pragma unroll
-            for (int k = 0; k < ITEMS; ++k) {
-                key[k] = sm.keys[seg + k * kWave];
-                if constexpr (PAIRS) val[k] = sm.vals[seg + k * kWave];
-            }
-        }
-        break;
-    }
-}
-
 template <typename K, bool PAIRS, int ITEMS>
 __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t rows, int64_t n) {
     constexpr int P = KeyTraits<K>::kPasses;
@@ -903,86 +585,6 @@ __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t row
             }
         }
     }
-}
-
-// Second half of the most-significant-digit-first sort: workgroup (row, d) takes the run of
-// keys whose digit `msd` is d - at most 64 * WAVES * ITEMS keys, in source order, in the first
-// ping-pong buffer - sorts it by the lower digits on chip and writes it to the strided outputs
-// at the run's place in the row.  Rows that took the other way leave at once.
-template <typename K, bool PAIRS, int ITEMS, int WAVES>
-__device__ __forceinline__ void sort_one_bucket(SmallShared<K, PAIRS, ITEMS, WAVES>& sm, const PassIo<K>& io, int64_t n, int64_t bucket,
-                                                const uint32_t* __restrict__ gbase, const uint32_t* __restrict__ moves,
-                                                const uint32_t* __restrict__ largest) {
-    constexpr int P = KeyTraits<K>::kPasses;
-    constexpr int CAP = WAVES * kWave * ITEMS;
-    const int tid = threadIdx.x;
-    const int lane = lane_id();
-    const int w = tid / kWave;
-    const int64_t row = bucket / kRadix;
-    const int d = static_cast<int>(bucket % kRadix);
-    const int msd = msd_digit<P>(moves + row * P, largest + row * P, static_cast<uint32_t>(CAP));
-    if (msd < 0) return;
-    const uint32_t* starts = gbase + (row * P + msd) * kRadix;
-    const int64_t begin = starts[d];
-    const int64_t end = d + 1 < kRadix ? static_cast<int64_t>(starts[d + 1]) : n;
-    const int valid = static_cast<int>(end - begin);
-    if (valid <= 0 || valid > CAP) return;                 // (never more than CAP: msd_digit saw the largest run)
-    const int seg = w * kWave * ITEMS + lane;
-    const K* src = io.kbuf[0] + row * n + begin;
-    const uint32_t* vsrc = PAIRS ? io.vbuf[0] + row * n + begin : nullptr;
-
-    K key[ITEMS];
-    uint32_t val[PAIRS ? ITEMS : 1];
-    K ors = 0, ands = ~K(0);
-#pragma unroll
-    for (int k = 0; k < ITEMS; ++k) {
-        const int e = seg + k * kWave;
-        key[k] = ~K(0);                                   // padding sorts last in every pass that runs
-        if constexpr (PAIRS) val[k] = 0u;
-        if (e < valid) {
-            key[k] = src[e];
-            if constexpr (PAIRS) val[k] = vsrc[e];
-            ors |= key[k];
-            ands &= key[k];
-        }
-    }
-    sort_in_workgroup<K, PAIRS, ITEMS, WAVES>(sm, key, val, ors, ands, valid, msd);
-
-    if (io.y) {
-        K* yrow = io.y + io.ymap.at(row);
-#pragma unroll
-        for (int k = 0; k < ITEMS; ++k) {
-            const int e = seg + k * kWave;
-            if (e < valid) {
-                K bits = decode_key<K>(key[k], io.kind, io.descending);
-                if constexpr (PAIRS) {
-                    if (io.restore_zero && static_cast<K>(bits << 1) == 0)
-                        bits = (io.x + io.xmap.at(row))[static_cast<int64_t>(val[k]) * io.sx];
-                }
-                yrow[(begin + e) * io.sy] = bits;
-            }
-        }
-    }
-    if constexpr (PAIRS) {
-        if (io.idx) {
-            const int64_t irow = io.imap.at(row);
-#pragma unroll
-            for (int k = 0; k < ITEMS; ++k) {
-                const int e = seg + k * kWave;
-                if (e < valid) {
-                    if (io.idx64) static_cast<int64_t*>(io.idx)[irow + (begin + e) * io.si] = static_cast<int64_t>(val[k]);
-                    else static_cast<int32_t*>(io.idx)[irow + (begin + e) * io.si] = static_cast<int32_t>(val[k]);
-                }
-            }
-        }
-    }
-}
-
-template <typename K, bool PAIRS, int ITEMS, int WAVES>
-__global__ __launch_bounds__(WAVES * kWave) void sort_buckets(PassIo<K> io, int64_t n, const uint32_t* __restrict__ gbase,
-                                                    const uint32_t* __restrict__ moves, const uint32_t* __restrict__ largest) {
-    __shared__ SmallShared<K, PAIRS, ITEMS, WAVES> sm;
-    sort_one_bucket<K, PAIRS, ITEMS, WAVES>(sm, io, n, blockIdx.x, gbase, moves, largest);
 }
 
 // One exchange of the (key, index) networks below: the lane takes the entry of lane ^ J when
@@ -1137,42 +739,8 @@ int g_sort_wave_rows = 512;
 
 constexpr int64_t kSmallRow = 4096;      // longest row sort_rows_small takes
 
-// Most significant digit first: capacities (keys per thread) of the two bucket kernels, and the
-// mean run length above which a row may go that way.
-// The large kernel holds 18 keys per thread in 4 wavefronts; with indices that many registers
-// leave one wavefront per SIMD, so pairs take 10 per thread in 8 wavefronts.
-// Smaller runs take 2, 4, 8 or 12 keys per thread in 4 wavefronts (512 to 3072 keys).
-constexpr int bucket_items_large(bool pairs) { return pairs ? 10 : 18; }
-constexpr int bucket_waves_large(bool pairs) { return pairs ? 8 : 4; }
-constexpr int bucket_cap_large(bool pairs) { return bucket_items_large(pairs) * bucket_waves_large(pairs) * kWave; }
-int g_sort_buckets = 1;
-int g_sort_leading_launch = 1;
-int g_sort_bucket_min = 0;               // shortest mean run that goes this way (0: bucket_min_mean below)
-
-// Integers: the measured break-even against the least-significant-digit-first passes on evenly
-// spread keys.  Floating-point rows seldom spread evenly over the sign and exponent byte, and
-// a row that does not go this way still pays for the dispatch of its 256 bucket workgroups
-// (about 8 % of a sort of 65536-key rows, under 2 % from 262144 keys on).
-constexpr int64_t bucket_min_mean(size_t key_size, bool pairs, int kind) {
-    if (kind == kKeyFloat) return 1024;
-    return key_size == 8 ? (pairs ? 64 : 128) : (pairs ? 128 : 512);
-}
-
-// Capacity of the bucket kernel for rows of n keys (0: none): the mean run with a quarter of
-// headroom (an eighth from 2048 keys on) has to fit; each row then decides on the device from
-// its own histogram.  `min_mean` is the shortest mean run worth the detour.
-uint32_t bucket_capacity(int64_t n, bool pairs, int64_t min_mean) {
-    const int64_t mean = ceil_div(n, static_cast<int64_t>(kRadix));
-    if (mean < min_mean) return 0u;
-    if (mean + mean / 4 <= 512) return 512u;
-    if (mean + mean / 4 <= 1024) return 1024u;
-    if (mean + mean / 8 <= 2048) return 2048u;
-    if (mean + mean / 8 <= 3072) return 3072u;
-    if (mean + mean / 8 <= bucket_cap_large(pairs)) return static_cast<uint32_t>(bucket_cap_large(pairs));
-    return 0u;
-}
-template <typename K>
-constexpr bool kBucketKeys = sizeof(K) >= 4;     // two-digit keys gain nothing
+int g_sort_buckets = 1;                  // 1: rows the bucket route takes go that way (dlfx_set_tuning "sort_buckets")
+int g_sort_compare_max = 96;             // fullest counting bin of a bucket that is still ranked by comparison
 
 template <typename K, bool PAIRS>
 int launch_small(hipStream_t stream, const PassIo<K>& io_in, int64_t m, int64_t n) {
@@ -1215,7 +783,7 @@ constexpr int tile_items(size_t key_size, bool pairs) { return ((key_size == 8 &
 
 struct SortLayout {
     int64_t tiles_per_row;
-    size_t moves_off, largest_off, hist_off, hist_bytes, status_off, status_bytes, keys_off[2], vals_off[2], total;
+    size_t moves_off, hist_off, hist_bytes, status_off, status_bytes, split_off, split_bytes, keys_off[2], vals_off[2], total;
 };
 
 SortLayout sort_layout(size_t key_size, bool pairs, int64_t m, int64_t n) {
@@ -1226,14 +794,15 @@ SortLayout sort_layout(size_t key_size, bool pairs, int64_t m, int64_t n) {
     size_t off = 0;
     l.moves_off = off;           // one word per (row, pass): does the pass move the row's keys
     off += align_up(static_cast<size_t>(m) * passes * 4, 256);
-    l.largest_off = off;         // one word per (row, pass): keys sharing the most frequent digit
-    off += align_up(static_cast<size_t>(m) * passes * 4, 256);
     l.hist_off = off;
     l.hist_bytes = static_cast<size_t>(m) * passes * kRadix * 4;
     off += align_up(l.hist_bytes, 256);
     l.status_off = off;
     l.status_bytes = l.tiles_per_row > 1 ? static_cast<size_t>(m) * l.tiles_per_row * kRadix * 4 : 0;
     off += align_up(l.status_bytes, 256);
+    l.split_off = off;           // tables of the bucket route (rows longer than one workgroup sorts on chip)
+    l.split_bytes = (n > kSmallRow && split_route_takes(key_size, m, n)) ? split_scratch_bytes(key_size, pairs, m, n) : 0;
+    off += align_up(l.split_bytes, 256);
     for (int i = 0; i < 2; ++i) {
         l.keys_off[i] = off;
         off += align_up(static_cast<size_t>(m) * n * key_size, 256);
@@ -1314,77 +883,54 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     }
     if (!scratch || scratch_bytes < l.total) return DLFX_ERR_SCRATCH_TOO_SMALL;
 
+    io.kbuf[0] = reinterpret_cast<K*>(base + l.keys_off[0]);
+    io.kbuf[1] = reinterpret_cast<K*>(base + l.keys_off[1]);
+    io.vbuf[0] = a.pairs ? reinterpret_cast<uint32_t*>(base + l.vals_off[0]) : nullptr;
+    io.vbuf[1] = a.pairs ? reinterpret_cast<uint32_t*>(base + l.vals_off[1]) : nullptr;
+
+    // The bucket route first: every row it can take goes that way (decided on the device, row by
+    // row); the digit passes below take the others and leave at once when there are none.  The
+    // routes share the first ping-pong buffer: their rows are different rows.
+    RowRoutes routes = {nullptr, 0, nullptr};
+    if constexpr (sizeof(K) >= 4) {
+        if (l.split_bytes != 0 && g_sort_buckets) {
+            size_t stride = 0;
+            const int st = run_split<K>(stream, io, a.pairs, m, n, base + l.split_off, g_sort_poll_limit, g_sort_compare_max,
+                                        &routes.other_rows, &routes.records, &stride);
+            if (st != DLFX_OK) return st;
+            routes.stride_words = stride / 4;
+        }
+    }
+
     uint32_t* moves = reinterpret_cast<uint32_t*>(base + l.moves_off);
     uint32_t* ghist = reinterpret_cast<uint32_t*>(base + l.hist_off);
     uint32_t* status = reinterpret_cast<uint32_t*>(base + l.status_off);
     const int64_t clear_words = static_cast<int64_t>((l.status_off + l.status_bytes - l.hist_off) / 4);   // histograms + status
-    sort_clear<<<dim3(static_cast<unsigned>(ceil_div(clear_words, kBlock))), dim3(kBlock), 0, stream>>>(ghist, clear_words);
+    sort_clear<<<dim3(static_cast<unsigned>(ceil_div(clear_words, kBlock * 4))), dim3(kBlock), 0, stream>>>(ghist, clear_words, routes);
     DLFX_CHECK_LAUNCH();
 
     const int64_t chunk = 32768;
     const int64_t chunks_per_row = ceil_div(n, chunk);
     if (m * chunks_per_row > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
-    sort_histogram<K><<<dim3(static_cast<unsigned>(m * chunks_per_row)), dim3(kBlock), 0, stream>>>(io, n, chunk, chunks_per_row, ghist);
+    sort_histogram<K><<<dim3(static_cast<unsigned>(m * chunks_per_row)), dim3(kBlock), 0, stream>>>(io, n, chunk, chunks_per_row, routes, ghist);
     DLFX_CHECK_LAUNCH();
     // a pass that moves nothing may only be left out when no pass reads the input while
     // another tile of the same pass writes the output over it
-    uint32_t* largest = reinterpret_cast<uint32_t*>(base + l.largest_off);
-    sort_bases<<<dim3(static_cast<unsigned>(m * P)), dim3(kRadix), 0, stream>>>(ghist, moves, largest, y_over_x ? 1 : 0);
+    sort_bases<<<dim3(static_cast<unsigned>(m * P)), dim3(kRadix), 0, stream>>>(ghist, moves, y_over_x ? 1 : 0, routes);
     DLFX_CHECK_LAUNCH();
-    // rows whose leading digit leaves runs that a workgroup can hold may go most significant
-    // digit first
-    uint32_t bucket_cap = 0;
-    if (kBucketKeys<K> && !y_over_x && g_sort_buckets && m * kRadix <= 0x7fffffffLL) bucket_cap = bucket_capacity(n, a.pairs, g_sort_bucket_min ? g_sort_bucket_min : bucket_min_mean(sizeof(K), a.pairs, a.kind));
 
-    io.kbuf[0] = reinterpret_cast<K*>(base + l.keys_off[0]);
-    io.kbuf[1] = reinterpret_cast<K*>(base + l.keys_off[1]);
-    io.vbuf[0] = a.pairs ? reinterpret_cast<uint32_t*>(base + l.vals_off[0]) : nullptr;
-    io.vbuf[1] = a.pairs ? reinterpret_cast<uint32_t*>(base + l.vals_off[1]) : nullptr;
     const dim3 grid(static_cast<unsigned>(m * l.tiles_per_row));
-    // 8-byte keys with indices: the tiled passes take 2048 keys per tile, which cuts a tile's share
-    // of a digit into runs of 8 keys (64 + 32 bytes: twice the bytes written).  The rows sorted most
-    // significant digit first run their one pass in a launch of their own with 4096-key tiles.
-    int elsewhere = 0;
-    if constexpr (sizeof(K) == 8) {
-        if (a.pairs && bucket_cap != 0u && g_sort_leading_launch) {
-            constexpr int IL = tile_items(sizeof(K), false);
-            const int64_t tiles = ceil_div(n, static_cast<int64_t>(kPassBlock) * IL);
-            sort_pass<K, true, IL, false><<<dim3(static_cast<unsigned>(m * tiles)), dim3(kPassBlock), 0, stream>>>(io, kLeadingPass, m, n, tiles, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
-            DLFX_CHECK_LAUNCH();
-            elsewhere = kLeadingPassElsewhere;
-        }
-    }
     for (int p = 0; p < P; ++p) {
         if (p < P - 1) {
             if (a.pairs)
-                sort_pass<K, true, IP, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p | elsewhere, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
+                sort_pass<K, true, IP, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, routes, status, g_sort_poll_limit);
             else
-                sort_pass<K, false, IK, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p | elsewhere, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
+                sort_pass<K, false, IK, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, routes, status, g_sort_poll_limit);
         } else {
             if (a.pairs)
-                sort_pass<K, true, IP, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p | elsewhere, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
+                sort_pass<K, true, IP, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, routes, status, g_sort_poll_limit);
             else
-                sort_pass<K, false, IK, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p | elsewhere, m, n, l.tiles_per_row, ghist, moves, largest, bucket_cap, status, g_sort_poll_limit);
-        }
-        DLFX_CHECK_LAUNCH();
-    }
-    if constexpr (kBucketKeys<K>) if (bucket_cap != 0u) {
-        const dim3 bgrid(static_cast<unsigned>(m * kRadix));
-        constexpr int BIP = bucket_items_large(true), BWP = bucket_waves_large(true);
-        constexpr int BIK = bucket_items_large(false), BWK = bucket_waves_large(false);
-        switch (bucket_cap) {
-#define DLFX_BUCKETS(I)                                                                                             \
-    if (a.pairs) sort_buckets<K, true, I, 4><<<bgrid, dim3(4 * kWave), 0, stream>>>(io, n, ghist, moves, largest); \
-    else sort_buckets<K, false, I, 4><<<bgrid, dim3(4 * kWave), 0, stream>>>(io, n, ghist, moves, largest);        \
-    break
-            case 512u: DLFX_BUCKETS(2);
-            case 1024u: DLFX_BUCKETS(4);
-            case 2048u: DLFX_BUCKETS(8);
-            case 3072u: DLFX_BUCKETS(12);
-#undef DLFX_BUCKETS
-            default:
-                if (a.pairs) sort_buckets<K, true, BIP, BWP><<<bgrid, dim3(BWP * kWave), 0, stream>>>(io, n, ghist, moves, largest);
-                else sort_buckets<K, false, BIK, BWK><<<bgrid, dim3(BWK * kWave), 0, stream>>>(io, n, ghist, moves, largest);
+                sort_pass<K, false, IK, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, routes, status, g_sort_poll_limit);
         }
         DLFX_CHECK_LAUNCH();
     }
@@ -1415,12 +961,8 @@ bool set_sort_tuning(const char* key, int64_t value) {
         g_sort_buckets = static_cast<int>(value);
         return true;
     }
-    if (!std::strcmp(key, "sort_leading_launch") && value >= 0 && value <= 1) {
-        g_sort_leading_launch = static_cast<int>(value);
-        return true;
-    }
-    if (!std::strcmp(key, "sort_bucket_min") && value >= 0 && value <= 65536) {
-        g_sort_bucket_min = static_cast<int>(value);
+    if (!std::strcmp(key, "sort_compare_max") && value >= 0 && value <= 4096) {
+        g_sort_compare_max = static_cast<int>(value);
         return true;
     }
     if (!std::strcmp(key, "sort_wave_rows") && value >= 0 && value <= 512) {

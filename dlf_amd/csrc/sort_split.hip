@@ -1,0 +1,967 @@
+// The bucket route of sort / argsort for rows longer than one workgroup holds (gfx950).
+//
+// A row is cut into at most 256 buckets of at most 5120 (shorter rows: 2560) keys by value, each bucket is then
+// sorted on chip, so the keys cross HBM four times (plus one read for the histogram) however
+// wide they are:
+//   1. split_sample     1024 keys of every row, evenly spaced, give the range of its keys (a few
+//                       stray keys at either end left aside); 4096 "fine bins" resolve that range.
+//   2. split_histogram  one read of the input: fine-bin histogram of every row (LDS atomics)
+//                       and the OR / AND of all its keys.
+//   3. split_plan       per row: neighbouring fine bins are merged into buckets of equal depth
+//                       (bucket of a bin = keys before it / target), so skewed rows - floats
+//                       with their exponents, clustered integers - still give even buckets.
+//                       A row whose sample missed a varying bit, whose largest fine bin does
+//                       not fit a workgroup, or that would need more than 256 buckets keeps
+//                       the least-significant-digit-first passes of sort.hip (decided here, on
+//                       the device, row by row).
+//   4. split_pass       a tile of 4096 keys finds each key's bucket (table in LDS) and its slot
+//                       among the tile's keys of that bucket with one LDS atomic, lays the tile
+//                       out by bucket in LDS and writes it as runs; a tile's offset inside each
+//                       bucket comes from the earlier tiles of the row through chained status
+//                       words (decoupled look-back, bounded waits).  The order inside a run is
+//                       whatever the atomics gave: not stable, and it need not be.
+//   5. split_finish     one workgroup per bucket: the keys' offsets from the bucket minimum,
+//                       scaled to 8192 bins, are counted and placed with LDS atomics; what
+//                       shares a bin (about one other key) is ranked by comparing whole
+//                       (key, index) entries, which also restores the stable order of equal
+//                       keys; the bucket leaves for the strided outputs.  Bins too crowded for
+//                       that (many equal or clustered keys) fall back to the stable digit
+//                       passes of sort_in_workgroup, for pairs first by index, then by key.
+// Ranking with an LDS atomic costs a few instructions per key where wave-wide digit matching
+// costs about fifty per digit, which is what bounded the digit passes.
+#include <cstddef>
+#include <cstring>
+
+#include "sort_common.hip.h"
+
+namespace dlfx {
+namespace {
+
+#ifdef SPLIT_TIMING
+// Debug builds only: shader-clock cycles spent by thread 0 of every workgroup in each phase.
+constexpr int kPhaseSlots = 4096;
+__device__ unsigned long long g_split_cycles[kPhaseSlots * 16];
+#define SPLIT_PHASE(i) do { if (threadIdx.x == 0) { const long long now_ = clock64(); g_split_cycles[(blockIdx.x % kPhaseSlots) * 16 + (i)] += static_cast<unsigned long long>(now_ - phase_t_); phase_t_ = now_; } } while (0)
+#define SPLIT_PHASE_BEGIN() long long phase_t_ = clock64()
+#else
+#define SPLIT_PHASE(i) do { } while (0)
+#define SPLIT_PHASE_BEGIN() do { } while (0)
+#endif
+
+constexpr int kFineBits = 12;
+constexpr int kFine = 1 << kFineBits;                 // fine bins per row
+constexpr int kMaxBuckets = 256;
+constexpr int kSplitBlock = 256;
+constexpr int kSplitItems = 16;                       // keys per thread of a split_pass tile
+constexpr int kSplitTile = kSplitBlock * kSplitItems;
+constexpr int kChunk = 8 * kSplitTile;                // keys one split_pass workgroup takes (32768)
+// split_finish comes in two sizes: eight wavefronts for buckets of up to 5120 keys (rows of up
+// to about 1.2 M keys), four wavefronts for buckets of up to 2560 (rows of up to 131072 keys:
+// more, smaller workgroups on a compute unit hide each other's waits better).
+constexpr int kFinishItems = 10;
+constexpr int finish_cap(int waves) { return waves * kWave * kFinishItems; }      // keys a bucket may hold
+constexpr int finish_bins(int waves) { return waves * 1024; }                     // counting bins, two 16-bit counters a word
+constexpr int kCapLarge = finish_cap(8), kCapSmall = finish_cap(4);
+constexpr int64_t kSmallCapRows = 131072;             // longest row that takes the small size
+constexpr int kNear = 2;                              // entries of a bin compared without a loop
+
+// What split_sample and split_plan decide for a row.
+struct alignas(16) SplitRow {
+    uint32_t route;                        // 1: this row takes the bucket route, 0: the digit passes
+    uint32_t shift;                        // fine bin of a key: min((key - base) >> shift, kFine - 1), 0 below base
+    unsigned long long base;
+    uint32_t n_buckets;
+    uint32_t reserved[3];
+    uint32_t begin[kMaxBuckets + 4];       // first position of each bucket in the row; begin[n_buckets] = n
+    uint8_t bucket_of[kFine];              // fine bin -> bucket (16-byte aligned: tiles load it as vectors)
+};
+static_assert(offsetof(SplitRow, bucket_of) % 16 == 0 && sizeof(SplitRow) % 16 == 0, "vector loads of the table");
+
+// Monotone in the key whatever the key: keys outside the sampled range land in the first or
+// last bins, so nothing has to be verified afterwards - a poor sample costs balance, not order.
+template <typename K>
+__device__ __forceinline__ uint32_t fine_bin(K key, K base, uint32_t shift) {
+    const K off = static_cast<K>(key - base) >> shift;
+    const uint32_t f = off < static_cast<K>(kFine - 1) ? static_cast<uint32_t>(off) : static_cast<uint32_t>(kFine - 1);
+    return key < base ? 0u : f;
+}
+
+template <typename T, typename Join>
+__device__ __forceinline__ T block_reduce(T v, Join join, T* lds, int waves) {
+    v = wave_reduce(v, join);
+    __syncthreads();                                   // the previous use of `lds` is over
+    if (lane_id() == 0) lds[threadIdx.x / kWave] = v;
+    __syncthreads();
+    T r = lds[0];
+    for (int i = 1; i < waves; ++i) r = join(r, lds[i]);
+    return r;
+}
+
+// ------------------------------------------------------------------ 1. the range of a row's keys
+template <typename K>
+__global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_t n, SplitRow* __restrict__ rows) {
+    __shared__ K red[kSplitBlock / kWave];
+    const int64_t row = blockIdx.x;
+    const K* xrow = io.x + io.xmap.at(row);
+    // 1024 evenly spaced keys, each wave's 256 spread over the whole row (the last one is the
+    // row's last key: a sorted row shows its whole range)
+    K key[4];
+    uint32_t unused[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t j = static_cast<int64_t>(threadIdx.x) + u * kSplitBlock;
+        int64_t e = n >= 1024 ? (j * n) / 1024 : (j < n ? j : n - 1);
+        if (j == 1023) e = n - 1;
+        key[u] = key_of_element<K>(io, xrow[e * io.sx]);
+    }
+    // every wave orders its 256 keys and offers its 4th smallest and 4th largest: three stray
+    // keys per wave at either end (a few zeros among positive values, a few huge ones) do not
+    // stretch the range the fine bins resolve
+    wave_bitonic_items<false, 4>(key, unused, [](K ka, uint32_t, K kb, uint32_t) { return ka < kb; });
+    K lo = lane_read(key[0], 3), hi = lane_read(key[3], kWave - 4);
+    if (n < 64) {                                      // too few keys for that: the plain range
+        lo = lane_read(key[0], 0);
+        hi = lane_read(key[3], kWave - 1);
+    }
+    lo = block_reduce(lo, [](K a, K b) { return a < b ? a : b; }, red, kSplitBlock / kWave);
+    hi = block_reduce(hi, [](K a, K b) { return a > b ? a : b; }, red, kSplitBlock / kWave);
+    if (threadIdx.x == 0) {
+        // that range takes the middle half of the fine bins; a quarter on either side is left for
+        // keys outside it (beyond those, keys share the first or last bin)
+        const unsigned long long range = static_cast<unsigned long long>(static_cast<K>(hi - lo));
+        const int width = range ? 64 - __builtin_clzll(range) : 0;
+        const uint32_t shift = width > kFineBits - 1 ? static_cast<uint32_t>(width - (kFineBits - 1)) : 0u;
+        const K margin = static_cast<K>(K(kFine / 4) << shift);
+        rows[row].route = 0u;
+        rows[row].shift = shift;
+        rows[row].base = static_cast<unsigned long long>(lo > margin ? static_cast<K>(lo - margin) : K(0));
+    }
+}
+
+__global__ __launch_bounds__(256) void split_clear(uint32_t* __restrict__ p, int64_t words) {
+    const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+    if (i + 4 <= words) *reinterpret_cast<uint4*>(p + i) = make_uint4(0u, 0u, 0u, 0u);
+    else for (int64_t j = i; j < words; ++j) p[j] = 0u;
+}
+
+// ------------------------------------------------------------------ 2. fine-bin histograms
+// One workgroup per chunk of kChunk keys of a row: the chunk's fine-bin histogram, two 16-bit
+// counts a word (a count is at most kChunk).  split_plan adds the chunks up for the row's
+// histogram and turns each chunk's into its keys per bucket, so that split_pass needs no
+// communication between workgroups.
+template <typename K>
+__global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int64_t n, int64_t chunks_per_row,
+                                                               const SplitRow* __restrict__ rows, uint32_t* __restrict__ chunk_fine) {
+    constexpr int U = 32 / sizeof(K);                 // keys in flight per thread
+    __shared__ uint32_t hist[kFine];
+    for (int i = threadIdx.x; i < kFine; i += kSplitBlock) hist[i] = 0;
+    __syncthreads();
+    const int64_t row = blockIdx.x / chunks_per_row;
+    const int64_t c = blockIdx.x - row * chunks_per_row;
+    const K* xrow = io.x + io.xmap.at(row);
+    const uint32_t shift = rows[row].shift;
+    const K base = static_cast<K>(rows[row].base);
+    const int64_t lo = c * kChunk;
+    const int64_t hi = (lo + kChunk < n) ? lo + kChunk : n;
+    for (int64_t b0 = lo; b0 < hi; b0 += static_cast<int64_t>(kSplitBlock) * U) {
+        const int64_t i0 = b0 + threadIdx.x;
+        if (b0 + static_cast<int64_t>(kSplitBlock) * U <= hi) {
+            K key[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) key[u] = xrow[(i0 + static_cast<int64_t>(u) * kSplitBlock) * io.sx];
+            uint32_t f[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) f[u] = fine_bin(key_of_element<K>(io, key[u]), base, shift);
+            // a wave whose keys all share one fine bin (narrow ranges, few distinct values) adds once
+            const uint32_t f0 = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(f[0])));
+            bool same = true;
+#pragma unroll
+            for (int u = 0; u < U; ++u) same = same && f[u] == f0;
+            if (__ballot(!same) == 0ull) {
+                if (lane_id() == 0) atomicAdd(&hist[f0], static_cast<uint32_t>(U * kWave));
+            } else {
+#pragma unroll
+                for (int u = 0; u < U; ++u) atomicAdd(&hist[f[u]], 1u);
+            }
+        } else {
+            for (int u = 0; u < U; ++u) {
+                const int64_t i = i0 + static_cast<int64_t>(u) * kSplitBlock;
+                if (i < hi) atomicAdd(&hist[fine_bin(key_of_element<K>(io, xrow[i * io.sx]), base, shift)], 1u);
+            }
+        }
+    }
+    __syncthreads();
+    uint32_t* g = chunk_fine + static_cast<int64_t>(blockIdx.x) * (kFine / 2);
+    for (int i = threadIdx.x; i < kFine / 2; i += kSplitBlock) g[i] = hist[2 * i] | (hist[2 * i + 1] << 16);
+}
+
+// ------------------------------------------------------------------ 3. buckets of equal depth
+// One workgroup per row; thread t owns fine bins [16 t, 16 t + 16).  counters[0] counts the rows
+// that keep the digit passes, counters[2] the buckets listed for split_finish.  For a row that
+// takes the route, chunk_base[chunk][b] receives the row position where that chunk's keys of
+// bucket b go: the bucket's start plus what the row's earlier chunks hold of it.
+__global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t cap, int64_t chunks_per_row, const uint32_t* __restrict__ chunk_fine,
+                                                          SplitRow* __restrict__ rows, uint32_t* __restrict__ counters,
+                                                          uint4* __restrict__ bucket_list, uint32_t* __restrict__ chunk_base) {
+    constexpr int PER = kFine / kSplitBlock;          // 16
+    __shared__ uint32_t red[kSplitBlock / kWave];
+    __shared__ uint32_t listed[2];                    // buckets of this row, and where they go in the list
+    __shared__ uint32_t per_bucket[kMaxBuckets];
+    const int64_t row = blockIdx.x;
+    const uint32_t* f = chunk_fine + row * chunks_per_row * (kFine / 2) + threadIdx.x * (PER / 2);
+    SplitRow& info = rows[row];
+    uint32_t cnt[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) cnt[i] = 0;
+    for (int64_t c = 0; c < chunks_per_row; ++c) {
+        const uint4 a = reinterpret_cast<const uint4*>(f + c * (kFine / 2))[0], b = reinterpret_cast<const uint4*>(f + c * (kFine / 2))[1];
+        const uint32_t w[PER / 2] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int i = 0; i < PER / 2; ++i) {
+            cnt[2 * i] += w[i] & 0xffffu;
+            cnt[2 * i + 1] += w[i] >> 16;
+        }
+    }
+    uint32_t sum = 0, biggest = 0;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        sum += cnt[i];
+        biggest = cnt[i] > biggest ? cnt[i] : biggest;
+    }
+    biggest = block_reduce(biggest, [](uint32_t a, uint32_t b) { return a > b ? a : b; }, red, kSplitBlock / kWave);
+    // exclusive prefix of the thread sums
+    const uint32_t incl = wave_scan_inclusive(sum, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+    __syncthreads();
+    if (lane_id() == kWave - 1) red[threadIdx.x / kWave] = incl;
+    __syncthreads();
+    uint32_t before = incl - sum;
+    for (int i = 0; i < static_cast<int>(threadIdx.x / kWave); ++i) before += red[i];
+
+    // every fine bin leaves room in a bucket, and 256 buckets are enough
+    bool ok = biggest < cap;
+    uint32_t target = 1;
+    if (ok) {
+        target = cap - biggest;
+        ok = static_cast<uint64_t>(n) / target + 1 <= static_cast<uint64_t>(kMaxBuckets);
+    }
+    if (!ok) {
+        if (threadIdx.x == 0) {
+            info.route = 0u;
+            atomicAdd(&counters[0], 1u);
+        }
+        return;
+    }
+    // a bin goes to bucket (keys before it) / target: every bucket then holds fewer than
+    // target + biggest = cap keys; a bin opens every bucket after its predecessor's up to its own
+    uint32_t prev_bucket = 0;                          // bucket of the bin before this thread's first
+    {
+        // (the last count of the thread before this one: the prefix before this thread's first bin minus that count)
+        const uint32_t prev_cnt = __shfl_up(cnt[PER - 1], 1, kWave);
+        uint32_t carried = prev_cnt;
+        if (lane_id() == 0 && threadIdx.x != 0) {
+            // first lane of a wave: the count lives in the wave before; take it from the chunk histograms again
+            carried = 0;
+            const uint32_t* g = chunk_fine + row * chunks_per_row * (kFine / 2) + (threadIdx.x * PER - 1) / 2;
+            for (int64_t c = 0; c < chunks_per_row; ++c) carried += g[c * (kFine / 2)] >> 16;
+        }
+        if (threadIdx.x != 0) prev_bucket = (before - carried) / target;
+        else info.begin[0] = 0u;
+    }
+    uint32_t bucket[PER];
+    uint32_t run = before;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const uint32_t b = run / target;
+        bucket[i] = b;
+        info.bucket_of[threadIdx.x * PER + i] = static_cast<uint8_t>(b);
+        for (uint32_t k = prev_bucket + 1; k <= b; ++k) info.begin[k] = run;
+        prev_bucket = b;
+        run += cnt[i];
+    }
+    if (threadIdx.x == kSplitBlock - 1) {
+        // (run == n here) the last bin's bucket is the last one
+        info.n_buckets = prev_bucket + 1;
+        info.begin[prev_bucket + 1] = static_cast<uint32_t>(n);
+        info.route = 1u;
+        listed[0] = prev_bucket + 1;
+        listed[1] = atomicAdd(&counters[2], prev_bucket + 1);
+    }
+    per_bucket[threadIdx.x] = 0u;
+    __syncthreads();
+    // the buckets of every such row, in no particular order: what split_finish walks
+    uint32_t next = 0;                                 // where the coming chunk's keys of bucket threadIdx.x go
+    if (threadIdx.x < listed[0]) {
+        const uint32_t b0 = info.begin[threadIdx.x], b1 = info.begin[threadIdx.x + 1];
+        bucket_list[listed[1] + threadIdx.x] = make_uint4(static_cast<uint32_t>(row), b0, b1 - b0, static_cast<uint32_t>(row) * kMaxBuckets + threadIdx.x);
+        next = b0;
+    }
+    // each chunk's keys per bucket, and from them where the chunk writes each bucket
+    for (int64_t c = 0; c < chunks_per_row; ++c) {
+        const uint4 a = reinterpret_cast<const uint4*>(f + c * (kFine / 2))[0], b = reinterpret_cast<const uint4*>(f + c * (kFine / 2))[1];
+        const uint32_t w[PER / 2] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        // this thread's bins lie in few buckets: sum runs of equal buckets before touching LDS
+        uint32_t acc = 0;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            acc += (i & 1) ? (w[i / 2] >> 16) : (w[i / 2] & 0xffffu);
+            if (i == PER - 1 || bucket[i + 1] != bucket[i]) {
+                if (acc) atomicAdd(&per_bucket[bucket[i]], acc);
+                acc = 0;
+            }
+        }
+        __syncthreads();
+        chunk_base[(row * chunks_per_row + c) * kMaxBuckets + threadIdx.x] = next;
+        next += per_bucket[threadIdx.x];
+        per_bucket[threadIdx.x] = 0u;
+        __syncthreads();
+    }
+}
+
+// ------------------------------------------------------------------ 4. one pass: chunk -> buckets
+template <typename K, bool PAIRS>
+struct SplitShared {
+    uint32_t table[kFine / 4];                 // bucket_of, four fine bins a word
+    uint32_t hist[kMaxBuckets];                // keys of the tile per bucket
+    uint32_t start[kMaxBuckets];               // where each bucket begins in the tile
+    int32_t dst_base[kMaxBuckets];             // row position of a bucket's share of this tile minus start
+    uint32_t scan_tmp[kSplitBlock / kWave];
+    K keys[kSplitTile];
+    uint32_t vals[PAIRS ? kSplitTile : 1];
+};
+
+// One workgroup per chunk (kChunk keys, tiles of 4096): where the chunk's keys of each bucket
+// go is known (chunk_base), so the workgroup carries the running positions itself from tile to
+// tile and nothing passes between workgroups.  A tile's keys find their bucket (table in LDS)
+// and their slot among the tile's keys of that bucket with one LDS atomic each, the tile is laid
+// out by bucket in LDS and written as runs; once it lies in LDS the registers already receive
+// the next tile's keys.  The order inside a run is whatever the atomics gave.
+template <typename K, bool PAIRS>
+__global__ __launch_bounds__(kSplitBlock) __attribute__((amdgpu_waves_per_eu(4))) void split_pass(PassIo<K> io, int64_t n, int64_t chunks_per_row,
+                                                          const SplitRow* __restrict__ infos, const uint32_t* __restrict__ chunk_base) {
+    constexpr int ITEMS = kSplitItems;
+    constexpr int TILE = kSplitTile;
+    __shared__ SplitShared<K, PAIRS> sm;
+    const int tid = threadIdx.x;
+    const int lane = lane_id();
+    const int w = tid / kWave;
+    const int64_t row = blockIdx.x / chunks_per_row;
+    const int64_t c = blockIdx.x - row * chunks_per_row;
+    const SplitRow& info = infos[row];
+    if (info.route != 1u) return;
+    const uint32_t shift = info.shift;
+    const K base = static_cast<K>(info.base);
+    const K* xrow = io.x + io.xmap.at(row);
+    const int64_t row_off = row * n;
+    const int64_t chunk_lo = c * kChunk;
+    const int64_t chunk_hi = (chunk_lo + kChunk < n) ? chunk_lo + kChunk : n;
+
+    // (no branches: an element beyond the chunk's end reads the tile's first element instead and is never used)
+    auto load_tile = [&](int64_t tile_base, K (&key)[ITEMS]) __attribute__((always_inline)) {
+        const int valid = static_cast<int>((chunk_hi - tile_base < TILE) ? chunk_hi - tile_base : TILE);
+        const K* src = xrow + tile_base * io.sx;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const int e = tid + k * kSplitBlock;
+            key[k] = src[static_cast<int64_t>(e < valid ? e : 0) * io.sx];
+        }
+    };
+
+    K key[ITEMS];
+    load_tile(chunk_lo, key);
+    reinterpret_cast<uint4*>(sm.table)[tid] = reinterpret_cast<const uint4*>(info.bucket_of)[tid];   // 256 threads x 16 bytes
+    sm.hist[tid] = 0u;
+    uint32_t next = chunk_base[static_cast<int64_t>(blockIdx.x) * kMaxBuckets + tid];   // where this chunk's coming keys of bucket tid go
+    __syncthreads();
+
+    for (int64_t tile_base = chunk_lo; tile_base < chunk_hi; tile_base += TILE) {
+        const int valid = static_cast<int>((chunk_hi - tile_base < TILE) ? chunk_hi - tile_base : TILE);
+        const bool full = valid == TILE;
+        SPLIT_PHASE_BEGIN();
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) key[k] = key_of_element<K>(io, key[k]);
+        SPLIT_PHASE(0);
+
+        // ---- bucket of every key (table), then its slot among the tile's keys of that bucket:
+        // one LDS atomic each, eight lookups issued before their eight atomics
+        uint32_t where[ITEMS];                     // bucket << 16 | slot, later the key's place in the tile
+#pragma unroll
+        for (int k0 = 0; k0 < ITEMS; k0 += 8) {
+#pragma unroll
+            for (int k = k0; k < k0 + 8; ++k) {
+                const uint32_t f = fine_bin(key[k], base, shift);
+                where[k] = (sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu;
+            }
+#pragma unroll
+            for (int k = k0; k < k0 + 8; ++k)
+                if (full || tid + k * kSplitBlock < valid) where[k] = (where[k] << 16) | atomicAdd(&sm.hist[where[k]], 1u);
+        }
+        __syncthreads();
+        SPLIT_PHASE(1);
+
+        // ---- thread b owns bucket b: its place in the tile and in the row
+        {
+            const uint32_t count = sm.hist[tid];
+            const uint32_t incl = wave_scan_inclusive(count, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+            if (lane == kWave - 1) sm.scan_tmp[w] = incl;
+            sm.hist[tid] = 0u;                             // for the next tile
+            __syncthreads();
+            uint32_t pre = 0;
+            for (int i = 0; i < w; ++i) pre += sm.scan_tmp[i];
+            const uint32_t start = pre + incl - count;
+            sm.start[tid] = start;
+            sm.dst_base[tid] = static_cast<int32_t>(next) - static_cast<int32_t>(start);
+            next += count;
+        }
+        __syncthreads();
+        SPLIT_PHASE(2);
+
+        // ---- lay the tile out by bucket (bucket starts read first, then the stores)
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) where[k] = sm.start[where[k] >> 16] + (where[k] & 0xffffu);
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            if (full || tid + k * kSplitBlock < valid) {
+                sm.keys[where[k]] = key[k];
+                if constexpr (PAIRS) sm.vals[where[k]] = static_cast<uint32_t>(tile_base) + static_cast<uint32_t>(tid + k * kSplitBlock);
+            }
+        }
+        __syncthreads();
+        SPLIT_PHASE(3);
+        // the tile is in LDS: the registers take the next tile, whose keys arrive while this one is written
+        if (tile_base + TILE < chunk_hi) load_tile(tile_base + TILE, key);
+
+        // ---- write runs: thread tid takes tile positions tid, tid + 256, ...; eight at a time, the
+        // reads of each step issued for all eight before the next step uses them
+        {
+            K* dk = io.kbuf[0] + row_off;
+            uint32_t* dv = PAIRS ? io.vbuf[0] + row_off : nullptr;
+#pragma unroll
+            for (int k0 = 0; k0 < ITEMS; k0 += 8) {
+                K out[8];
+                int32_t at[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) out[j] = sm.keys[(k0 + j) * kSplitBlock + tid];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t f = fine_bin(out[j], base, shift);
+                    at[j] = static_cast<int32_t>((sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu);
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) at[j] = sm.dst_base[at[j]] + ((k0 + j) * kSplitBlock + tid);
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (full || (k0 + j) * kSplitBlock + tid < valid) dk[at[j]] = out[j];
+                if constexpr (PAIRS) {
+                    uint32_t pay[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) pay[j] = sm.vals[(k0 + j) * kSplitBlock + tid];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (full || (k0 + j) * kSplitBlock + tid < valid) dv[at[j]] = pay[j];
+                }
+            }
+        }
+        SPLIT_PHASE(5);
+        __syncthreads();                                   // the tile in LDS has left
+    }
+}
+
+// ------------------------------------------------------------------ 5. a bucket, on chip
+// Whether split_finish keeps every entry's bin beside it in LDS (two bytes an entry) instead of
+// working it out again from the key when the entry is ranked; 8-byte keys with indices have no
+// room for that with two workgroups on a compute unit.
+template <typename K, bool PAIRS, int WAVES>
+constexpr bool kKeepBins = !(PAIRS && sizeof(K) == 8 && WAVES == 8);
+
+template <typename K, bool PAIRS, int WAVES>
+struct FinishShared {
+    uint32_t bins[finish_bins(WAVES) / 2];     // two 16-bit counters a word: counts, then bin starts, then bin ends
+    K keys[finish_cap(WAVES)];
+    uint32_t vals[PAIRS ? finish_cap(WAVES) : 1];
+    uint16_t bin_at[kKeepBins<K, PAIRS, WAVES> ? finish_cap(WAVES) : 1];
+    K red_key[WAVES];
+    uint32_t red_val[WAVES], red32[WAVES];
+    uint32_t crowded;
+};
+
+// Where bucket `id` = row * 256 + b lies: {row, first position in the row, entries, id}.
+__device__ __forceinline__ uint4 bucket_at(const SplitRow* __restrict__ infos, uint32_t id) {
+    const uint32_t row = id / kMaxBuckets, b = id % kMaxBuckets;
+    const SplitRow& info = infos[row];
+    const uint32_t b0 = info.begin[b];
+    return make_uint4(row, b0, info.begin[b + 1] - b0, id);
+}
+
+// Entry `at` of the sorted row goes to the strided outputs.
+template <typename K, bool PAIRS>
+__device__ __forceinline__ void emit_entry(const PassIo<K>& io, const K* xrow, K* yrow, int64_t irow, int64_t at, K key, uint32_t val) {
+    if (yrow) {
+        K bits = decode_key<K>(key, io.kind, io.descending);
+        if constexpr (PAIRS) {
+            if (io.restore_zero && static_cast<K>(bits << 1) == 0) bits = xrow[static_cast<int64_t>(val) * io.sx];
+        }
+        yrow[at * io.sy] = bits;
+    }
+    if constexpr (PAIRS) {
+        if (io.idx) {
+            if (io.idx64) static_cast<int64_t*>(io.idx)[irow + at * io.si] = static_cast<int64_t>(val);
+            else static_cast<int32_t*>(io.idx)[irow + at * io.si] = static_cast<int32_t>(val);
+        }
+    }
+}
+
+// Workgroup g takes entries g, g + G, ... of the bucket list (what split_plan wrote: row, first
+// position, size of every bucket); once a bucket lies in LDS the registers already receive the
+// next one's entries.  A bucket whose bins are too crowded to rank by comparison is put on
+// `crowded_list` (counters[1] entries) for split_finish_crowded.
+template <typename K, bool PAIRS, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4))) void split_finish(PassIo<K> io, int64_t n,
+                                                             uint32_t compare_max, uint32_t* __restrict__ counters,
+                                                             const uint4* __restrict__ bucket_list, uint32_t* __restrict__ crowded_list) {
+    constexpr int ITEMS = kFinishItems;
+    constexpr int T = WAVES * kWave;
+    constexpr int kBins = finish_bins(WAVES);
+    constexpr int kBinBits = WAVES == 8 ? 13 : 12;
+    static_assert(kBins == 1 << kBinBits, "bins and their bits");
+    constexpr int WORDS = kBins / 2 / T;       // counter words a thread scans (8)
+    constexpr bool KEEP = kKeepBins<K, PAIRS, WAVES>;
+    __shared__ FinishShared<K, PAIRS, WAVES> sm;
+    const int tid = threadIdx.x;
+    const int lane = lane_id();
+    const int w = tid / kWave;
+    const int seg = w * kWave * ITEMS + lane;              // item k of this thread is entry seg + 64 k of the bucket
+    const int64_t total = counters[2];                     // buckets on the list
+    const int64_t step = gridDim.x;
+
+    // (no branches: an entry beyond the bucket's end reads its first entry instead and is never used)
+    auto load_bucket = [&](const uint4& d, K (&key)[ITEMS], uint32_t (&val)[PAIRS ? ITEMS : 1]) __attribute__((always_inline)) {
+        const K* src = io.kbuf[0] + static_cast<int64_t>(d.x) * n + d.y;
+        const uint32_t* vsrc = PAIRS ? io.vbuf[0] + static_cast<int64_t>(d.x) * n + d.y : nullptr;
+        const int size = static_cast<int>(d.z);
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const int e = seg + k * kWave;
+            key[k] = src[e < size ? e : 0];
+            if constexpr (PAIRS) val[k] = vsrc[e < size ? e : 0];
+        }
+    };
+
+    int64_t v = blockIdx.x;
+    if (v >= total) return;
+    uint4 cur = bucket_list[v];
+    K key[ITEMS];
+    uint32_t val[PAIRS ? ITEMS : 1];
+    load_bucket(cur, key, val);
+    for (;;) {
+        SPLIT_PHASE_BEGIN();
+        const int64_t vn = v + step;
+        uint4 nxt = cur;
+        if (vn < total) nxt = bucket_list[vn];             // on its way while this bucket is counted
+        const int valid = static_cast<int>(cur.z);
+        const int64_t begin = cur.y;
+        const int64_t row = cur.x;
+
+        // ---- smallest key (and index): the origin of the offsets
+        K lo = ~K(0);
+        uint32_t vlo = ~0u;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            if (seg + k * kWave < valid) {
+                lo = key[k] < lo ? key[k] : lo;
+                if constexpr (PAIRS) vlo = val[k] < vlo ? val[k] : vlo;
+            }
+        }
+        for (int i = tid; i < kBins / 2; i += T) sm.bins[i] = 0u;
+        lo = wave_reduce(lo, [](K a, K c) { return a < c ? a : c; });
+        if constexpr (PAIRS) vlo = wave_reduce(vlo, [](uint32_t a, uint32_t c) { return a < c ? a : c; });
+        if (lane == 0) {
+            sm.red_key[w] = lo;
+            if constexpr (PAIRS) sm.red_val[w] = vlo;
+        }
+        if (tid == 0) sm.crowded = 0u;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < WAVES; ++i) {
+            lo = sm.red_key[i] < lo ? sm.red_key[i] : lo;
+            if constexpr (PAIRS) vlo = sm.red_val[i] < vlo ? sm.red_val[i] : vlo;
+        }
+        __syncthreads();                                   // red_key / red_val are reused at once
+        // ---- OR of all offsets: its leading bit bounds them, its trailing zeros carry nothing (quantised values)
+        K ors = 0;
+        uint32_t vors = 0;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k)
+            if (seg + k * kWave < valid) {
+                ors |= static_cast<K>(key[k] - lo);
+                if constexpr (PAIRS) vors |= val[k] - vlo;
+            }
+        ors = wave_reduce(ors, [](K a, K c) { return static_cast<K>(a | c); });
+        if constexpr (PAIRS) vors = wave_reduce(vors, [](uint32_t a, uint32_t c) { return a | c; });
+        if (lane == 0) {
+            sm.red_key[w] = ors;
+            if constexpr (PAIRS) sm.red_val[w] = vors;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < WAVES; ++i) {
+            ors |= sm.red_key[i];
+            if constexpr (PAIRS) vors |= sm.red_val[i];
+        }
+
+        // The word an entry is binned by: its key's offset from the smallest key without the
+        // zero bits; for pairs, when there is room, that offset with the index's offset below it,
+        // so that equal keys spread over bins in index order instead of crowding one.
+        const int zeros = ors ? __builtin_ctzll(static_cast<unsigned long long>(ors)) : 0;
+        const int key_bits = ors ? 64 - __builtin_clzll(static_cast<unsigned long long>(ors)) - zeros : 0;
+        int idx_bits = 0;
+        if constexpr (PAIRS) {
+            idx_bits = vors ? 32 - __builtin_clz(vors) : 0;
+            if (key_bits + idx_bits > 64) idx_bits = 0;    // wide keys seldom repeat
+        }
+        const int width = key_bits + idx_bits;
+        const int down = width > kBinBits ? width - kBinBits : 0;      // words >> down lie below kBins
+        auto bin_of = [&](K k1, uint32_t v1) __attribute__((always_inline)) -> uint32_t {
+            if constexpr (sizeof(K) == 4) {
+                if (width <= 32) {                         // (uniform) everything fits 32-bit arithmetic
+                    uint32_t word = static_cast<uint32_t>(k1 - lo) >> zeros;
+                    if constexpr (PAIRS) word = idx_bits ? ((word << idx_bits) | (v1 - vlo)) : word;
+                    return word >> down;
+                }
+            }
+            unsigned long long word = static_cast<unsigned long long>(static_cast<K>(k1 - lo) >> zeros);
+            if constexpr (PAIRS) {
+                if (idx_bits) word = (word << idx_bits) | static_cast<unsigned long long>(v1 - vlo);
+            }
+            return static_cast<uint32_t>(word >> down);
+        };
+        // entries that share a bin are told apart by comparison, unless the bin says it all
+        const bool compare = down != 0 || (PAIRS && idx_bits == 0 && vors != 0u);
+        SPLIT_PHASE(8);
+
+        // ---- count
+        uint32_t bin[ITEMS];
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) bin[k] = bin_of(key[k], PAIRS ? val[k] : 0u);
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k)
+            if (seg + k * kWave < valid) atomicAdd(&sm.bins[bin[k] >> 1], 1u << (16u * (bin[k] & 1u)));
+        __syncthreads();
+        SPLIT_PHASE(9);
+
+        // ---- counts -> bin starts (exclusive prefix over the 8192 bins), and the fullest bin
+        {
+            uint32_t words[WORDS];
+            uint32_t sum = 0, fullest = 0;
+#pragma unroll
+            for (int i = 0; i < WORDS; ++i) {
+                words[i] = sm.bins[tid * WORDS + i];
+                const uint32_t c0 = words[i] & 0xffffu, c1 = words[i] >> 16;
+                sum += c0 + c1;
+                fullest = c0 > fullest ? c0 : fullest;
+                fullest = c1 > fullest ? c1 : fullest;
+            }
+            const uint32_t incl = wave_scan_inclusive(sum, 0u, [](uint32_t a, uint32_t c) { return a + c; });
+            if (lane == kWave - 1) sm.red32[w] = incl;
+            fullest = wave_reduce(fullest, [](uint32_t a, uint32_t c) { return a > c ? a : c; });
+            if (lane == 0 && fullest > compare_max) atomicMax(&sm.crowded, fullest);
+            __syncthreads();
+            uint32_t run = incl - sum;
+            for (int i = 0; i < w; ++i) run += sm.red32[i];
+#pragma unroll
+            for (int i = 0; i < WORDS; ++i) {
+                const uint32_t c0 = words[i] & 0xffffu, c1 = words[i] >> 16;
+                sm.bins[tid * WORDS + i] = run | ((run + c0) << 16);
+                run += c0 + c1;
+            }
+        }
+        __syncthreads();
+        SPLIT_PHASE(10);
+
+        if (compare && sm.crowded != 0u) {
+            // many equal or clustered keys: the stable digit passes of split_finish_crowded take this bucket
+            if (tid == 0) crowded_list[atomicAdd(&counters[1], 1u)] = cur.w;
+            if (vn < total) load_bucket(nxt, key, val);
+        } else {
+            // ---- place: the atomic hands out the next free entry of the bin, whose word ends up at its end
+            {
+                uint32_t old[ITEMS];
+#pragma unroll
+                for (int k = 0; k < ITEMS; ++k)
+                    if (seg + k * kWave < valid) old[k] = atomicAdd(&sm.bins[bin[k] >> 1], 1u << (16u * (bin[k] & 1u)));
+#pragma unroll
+                for (int k = 0; k < ITEMS; ++k) {
+                    if (seg + k * kWave < valid) {
+                        const uint32_t pos = (old[k] >> (16u * (bin[k] & 1u))) & 0xffffu;
+                        sm.keys[pos] = key[k];
+                        if constexpr (PAIRS) sm.vals[pos] = val[k];
+                        if constexpr (KEEP) sm.bin_at[pos] = static_cast<uint16_t>(bin[k]);
+                    }
+                }
+            }
+            __syncthreads();
+            SPLIT_PHASE(11);
+            // the bucket is in LDS: the registers take the next bucket, whose entries arrive while
+            // this one is ranked and written
+            if (vn < total) load_bucket(nxt, key, val);
+
+            const K* xrow = io.x + io.xmap.at(row);
+            K* yrow = io.y ? io.y + io.ymap.at(row) : nullptr;
+            const int64_t irow = (PAIRS && io.idx) ? io.imap.at(row) : 0;
+            // ---- rank inside the bin and write: thread tid takes entries tid, tid + 512, ...; five at
+            // a time, each step reading for all five before the next step looks at what came back
+            constexpr int B = 5;
+            static_assert(ITEMS % B == 0, "whole batches");
+#pragma unroll 1
+            for (int k0 = 0; k0 < ITEMS; k0 += B) {
+                if (k0 * T >= valid) break;                // (uniform) nothing left
+                K mine[B];
+                uint32_t mine_v[PAIRS ? B : 1];
+                uint32_t mine_b[B];
+#pragma unroll
+                for (int j = 0; j < B; ++j) {
+                    const int pos = (k0 + j) * T + tid;
+                    const int at = pos < valid ? pos : 0;
+                    mine[j] = sm.keys[at];
+                    if constexpr (PAIRS) mine_v[j] = sm.vals[at];
+                    if constexpr (KEEP) mine_b[j] = sm.bin_at[at];
+                }
+                if (!compare) {
+#pragma unroll
+                    for (int j = 0; j < B; ++j)
+                        if ((k0 + j) * T + tid < valid)
+                            emit_entry<K, PAIRS>(io, xrow, yrow, irow, begin + (k0 + j) * T + tid, mine[j], PAIRS ? mine_v[j] : 0u);
+                    continue;
+                }
+                int first[B], end[B], ahead[B];
+#pragma unroll
+                for (int j = 0; j < B; ++j) {
+                    uint32_t b1;
+                    if constexpr (KEEP) b1 = mine_b[j];
+                    else b1 = bin_of(mine[j], PAIRS ? mine_v[j] : 0u);
+                    end[j] = static_cast<int>((sm.bins[b1 >> 1] >> (16u * (b1 & 1u))) & 0xffffu);
+                    const uint32_t b0 = b1 - 1u;
+                    first[j] = b1 == 0u ? 0 : static_cast<int>((sm.bins[b0 >> 1] >> (16u * (b0 & 1u))) & 0xffffu);
+                    ahead[j] = 0;
+                }
+                // the first kNear entries of the bin without a loop (a bin seldom holds more)
+#pragma unroll
+                for (int i = 0; i < kNear; ++i) {
+                    K other[B];
+                    uint32_t other_v[PAIRS ? B : 1];
+#pragma unroll
+                    for (int j = 0; j < B; ++j) {
+                        const int q = first[j] + i < valid ? first[j] + i : 0;
+                        other[j] = sm.keys[q];
+                        if constexpr (PAIRS) other_v[j] = sm.vals[q];
+                    }
+#pragma unroll
+                    for (int j = 0; j < B; ++j) {
+                        const int q = first[j] + i;
+                        bool before = other[j] < mine[j];
+                        if (other[j] == mine[j]) {
+                            if constexpr (PAIRS) before = other_v[j] < mine_v[j];
+                            else before = q < (k0 + j) * T + tid;
+                        }
+                        ahead[j] += (q < end[j] && before) ? 1 : 0;
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < B; ++j) {
+                    const int pos = (k0 + j) * T + tid;
+                    if (pos >= valid) continue;
+                    for (int q = first[j] + kNear; q < end[j]; ++q) {          // the rest of a fuller bin
+                        const K other = sm.keys[q];
+                        bool before = other < mine[j];
+                        if (other == mine[j]) {
+                            if constexpr (PAIRS) before = sm.vals[q] < mine_v[j];
+                            else before = q < pos;
+                        }
+                        ahead[j] += before ? 1 : 0;
+                    }
+                    emit_entry<K, PAIRS>(io, xrow, yrow, irow, begin + first[j] + ahead[j], mine[j], PAIRS ? mine_v[j] : 0u);
+                }
+            }
+            SPLIT_PHASE(12);
+        }
+        if (vn >= total) break;
+        v = vn;
+        cur = nxt;
+        __syncthreads();                                   // the bucket in LDS has left
+    }
+}
+
+// The buckets split_finish left: stable digit passes on chip - for pairs first by index (the
+// entries arrive in no particular order), then by key.
+template <typename K, bool PAIRS, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void split_finish_crowded(PassIo<K> io, int64_t n, const SplitRow* __restrict__ infos,
+                                                                     const uint32_t* __restrict__ counters,
+                                                                     const uint32_t* __restrict__ crowded_list) {
+    constexpr int ITEMS = kFinishItems;
+    __shared__ SmallShared<K, PAIRS, ITEMS, WAVES> sm;
+    const uint32_t listed = counters[1];
+    const int lane = lane_id();
+    const int seg = (threadIdx.x / kWave) * kWave * ITEMS + lane;
+    for (uint32_t i = blockIdx.x; i < listed; i += gridDim.x) {
+        const uint4 at = bucket_at(infos, crowded_list[i]);
+        const int valid = static_cast<int>(at.z);
+        const int64_t at_row = at.x, at_begin = at.y;
+        const K* src = io.kbuf[0] + at_row * n + at_begin;
+        const uint32_t* vsrc = PAIRS ? io.vbuf[0] + at_row * n + at_begin : nullptr;
+        K key[ITEMS];
+        uint32_t val[PAIRS ? ITEMS : 1];
+        K ors = 0, ands = ~K(0), vors = 0, vands = ~K(0);
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const int e = seg + k * kWave;
+            key[k] = ~K(0);                                    // padding sorts last, by index and by key
+            if constexpr (PAIRS) val[k] = ~0u;
+            if (e < valid) {
+                key[k] = src[e];
+                ors |= key[k];
+                ands &= key[k];
+                if constexpr (PAIRS) {
+                    val[k] = vsrc[e];
+                    vors |= static_cast<K>(val[k]);
+                    vands &= static_cast<K>(val[k]);
+                }
+            }
+        }
+        if constexpr (PAIRS) {
+            sort_in_workgroup<K, PAIRS, ITEMS, WAVES, true>(sm, key, val, vors, vands, valid, 4);
+            __syncthreads();
+        }
+        sort_in_workgroup<K, PAIRS, ITEMS, WAVES>(sm, key, val, ors, ands, valid, KeyTraits<K>::kPasses);
+        const K* xrow = io.x + io.xmap.at(at_row);
+        K* yrow = io.y ? io.y + io.ymap.at(at_row) : nullptr;
+        const int64_t irow = (PAIRS && io.idx) ? io.imap.at(at_row) : 0;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k)
+            if (seg + k * kWave < valid) emit_entry<K, PAIRS>(io, xrow, yrow, irow, at_begin + seg + k * kWave, key[k], PAIRS ? val[k] : 0u);
+        __syncthreads();
+    }
+}
+
+// Workgroups of `kernel` that the current device holds at once (0 when HIP cannot tell).
+template <typename Kernel>
+int64_t resident_workgroups(Kernel kernel, int block) {
+    int device = 0, units = 0, per_unit = 0;
+    if (hipGetDevice(&device) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_unit, kernel, block, 0) != hipSuccess) return 0;
+    return static_cast<int64_t>(units) * per_unit;
+}
+
+struct SplitLayout {
+    int64_t chunks_per_row;
+    size_t counters_off, rows_off, list_off, crowded_off, fine_off, base_off, total;
+};
+
+SplitLayout split_layout(int64_t m, int64_t n) {
+    SplitLayout l;
+    l.chunks_per_row = ceil_div(n, static_cast<int64_t>(kChunk));
+    size_t off = 0;
+    l.counters_off = off;        // [0] rows that keep the digit passes, [1] crowded buckets, [2] listed buckets
+    off += 256;
+    l.rows_off = off;
+    off += align_up(static_cast<size_t>(m) * sizeof(SplitRow), 256);
+    l.list_off = off;            // {row, begin, size, id} of every bucket
+    off += align_up(static_cast<size_t>(m) * kMaxBuckets * 16, 256);
+    l.crowded_off = off;
+    off += align_up(static_cast<size_t>(m) * kMaxBuckets * 4, 256);
+    l.fine_off = off;            // fine-bin histogram of every chunk, two counts a word
+    off += align_up(static_cast<size_t>(m) * l.chunks_per_row * (kFine / 2) * 4, 256);
+    l.base_off = off;            // where every chunk writes each bucket
+    off += align_up(static_cast<size_t>(m) * l.chunks_per_row * kMaxBuckets * 4, 256);
+    l.total = off;
+    return l;
+}
+
+}  // namespace
+
+// Whether rows of n keys can take the bucket route at all (each row then decides on the device).
+bool split_route_takes(size_t key_size, int64_t m, int64_t n) {
+    return (key_size == 4 || key_size == 8) && n <= static_cast<int64_t>(kMaxBuckets - 1) * kCapLarge &&
+           m * kMaxBuckets <= 0x7fffffffLL && m * ceil_div(n, static_cast<int64_t>(kChunk)) <= 0x7fffffffLL;
+}
+
+size_t split_scratch_bytes(size_t key_size, bool pairs, int64_t m, int64_t n) {
+    (void)key_size;
+    (void)pairs;              // keys and indices travel through the caller's first ping-pong buffers
+    return split_layout(m, n).total;
+}
+
+// Enqueues the bucket route for every row; keys (and indices) travel through io.kbuf[0] (and
+// io.vbuf[0]).  Rows it does not take are counted in **other_rows (device memory inside
+// `scratch`) and marked in the row records at *route_records (*route_stride bytes apart, first
+// word 1 when the row was taken).
+template <typename K>
+int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, int64_t n, void* scratch, int poll_limit,
+              int compare_max, const uint32_t** other_rows, const uint32_t** route_records, size_t* route_stride) {
+    const SplitLayout l = split_layout(m, n);
+    char* base = static_cast<char*>(scratch);
+    uint32_t* counters = reinterpret_cast<uint32_t*>(base + l.counters_off);
+    SplitRow* rows = reinterpret_cast<SplitRow*>(base + l.rows_off);
+    uint4* list = reinterpret_cast<uint4*>(base + l.list_off);
+    uint32_t* crowded = reinterpret_cast<uint32_t*>(base + l.crowded_off);
+    uint32_t* fine = reinterpret_cast<uint32_t*>(base + l.fine_off);
+    uint32_t* chunk_base = reinterpret_cast<uint32_t*>(base + l.base_off);
+    *other_rows = counters;
+    *route_records = reinterpret_cast<const uint32_t*>(rows);
+    *route_stride = sizeof(SplitRow);
+    (void)poll_limit;            // nothing waits for anything on this route
+
+    split_clear<<<dim3(1), dim3(256), 0, stream>>>(counters, 64);
+    DLFX_CHECK_LAUNCH();
+    split_sample<K><<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(io, n, rows);
+    DLFX_CHECK_LAUNCH();
+    const dim3 chunks(static_cast<unsigned>(m * l.chunks_per_row));
+    split_histogram<K><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine);
+    DLFX_CHECK_LAUNCH();
+    const bool small = n <= kSmallCapRows;
+    split_plan<<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(n, static_cast<uint32_t>(small ? kCapSmall : kCapLarge), l.chunks_per_row, fine, rows, counters, list, chunk_base);
+    DLFX_CHECK_LAUNCH();
+    // split_finish: as many workgroups as the device holds at once, each walking its share of the buckets
+    const int64_t buckets = m * kMaxBuckets;
+    const uint32_t limit = static_cast<uint32_t>(compare_max);
+    auto launch = [&](auto pairs_tag, auto waves_tag) -> int {
+        constexpr bool PAIRS = decltype(pairs_tag)::value;
+        constexpr int WAVES = decltype(waves_tag)::value;
+        const int64_t finish_room = resident_workgroups(split_finish<K, PAIRS, WAVES>, WAVES * kWave);
+        if (finish_room <= 0) return DLFX_ERR_LAUNCH;
+        const dim3 fgrid(static_cast<unsigned>(buckets < finish_room ? buckets : finish_room));
+        split_pass<K, PAIRS><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, chunk_base);
+        DLFX_CHECK_LAUNCH();
+        split_finish<K, PAIRS, WAVES><<<fgrid, dim3(WAVES * kWave), 0, stream>>>(io, n, limit, counters, list, crowded);
+        DLFX_CHECK_LAUNCH();
+        split_finish_crowded<K, PAIRS, WAVES><<<fgrid, dim3(WAVES * kWave), 0, stream>>>(io, n, rows, counters, crowded);
+        DLFX_CHECK_LAUNCH();
+        return DLFX_OK;
+    };
+    using Large = std::integral_constant<int, 8>;
+    using Small = std::integral_constant<int, 4>;
+    if (pairs) return small ? launch(std::true_type(), Small()) : launch(std::true_type(), Large());
+    return small ? launch(std::false_type(), Small()) : launch(std::false_type(), Large());
+}
+
+template int run_split<uint32_t>(hipStream_t, const PassIo<uint32_t>&, bool, int64_t, int64_t, void*, int, int, const uint32_t**,
+                                 const uint32_t**, size_t*);
+template int run_split<uint64_t>(hipStream_t, const PassIo<uint64_t>&, bool, int64_t, int64_t, void*, int, int, const uint32_t**,
+                                 const uint32_t**, size_t*);
+
+}  // namespace dlfx
+
+#ifdef SPLIT_TIMING
+extern "C" void dlfx_debug_split_phases(unsigned long long* out, int reset) {
+    static unsigned long long host[dlfx::kPhaseSlots * 16];
+    if (out) {
+        (void)hipMemcpyFromSymbol(host, HIP_SYMBOL(dlfx::g_split_cycles), sizeof(host));
+        for (int i = 0; i < 16; ++i) out[i] = 0;
+        for (int b = 0; b < dlfx::kPhaseSlots; ++b)
+            for (int i = 0; i < 16; ++i) out[i] += host[b * 16 + i];
+    }
+    if (reset) {
+        for (auto& v : host) v = 0;
+        (void)hipMemcpyToSymbol(HIP_SYMBOL(dlfx::g_split_cycles), host, sizeof(host));
+    }
+}
+#endif

@@ -80,17 +80,13 @@ int dlfx_last_hip_error(void);
  *   "sort_poll_limit"  the same bound for the per-digit tile chaining of a radix pass.
  *   "sort_wave_rows"   longest row (64, 128, 256 or 512; default 512) sorted by one wavefront
  *                      in registers; longer rows of up to 4096 elements take one workgroup.
- *   "sort_buckets"     1 (default): rows of 4- and 8-byte keys whose most significant varying
- *                      digit spreads them evenly are sorted on that digit first and each run
- *                      of equal digits is finished on chip; 0: every row takes the
- *                      least-significant-digit-first passes.  Same results either way.
- *   "sort_bucket_min"  shortest mean run (row length / 256) for which "sort_buckets" applies;
- *                      0 (default): 128 / 512 for 8- / 4-byte integers, 64 / 128 when
- *                      indices travel with them, 1024 for floating-point keys.
- *   "sort_leading_launch" 1 (default): rows of 8-byte keys with indices that "sort_buckets" sends
- *                      most significant digit first run that digit's pass in a launch of
- *                      their own with 4096-key tiles; 0: inside the launch of that pass, with
- *                      the 2048-key tiles of the other rows.  Same results either way.
+ *   "sort_buckets"     1 (default): rows of 4- and 8-byte keys longer than 4096 elements are cut into
+ *                      buckets of equal depth by value and each bucket is sorted on chip, wherever
+ *                      a row's keys allow it (each row decides on the device); 0: every row takes
+ *                      the least-significant-digit-first passes.  Same results either way.
+ *   "sort_compare_max" fullest counting bin (default 96) of a bucket whose entries are still ranked
+ *                      by comparing them; fuller bins send the bucket through stable digit passes
+ *                      (0: every bucket).  Same results for every value.
  *   "topk_thread_rows" longest row (default 256; half of it for 8-byte keys) for which top_k
  *                      with a limit of at most 8 over at least 16384 contiguous rows gives
  *                      each row to one thread.

@@ -163,18 +163,10 @@ def test_rows_leave_out_passes_that_move_nothing(hip_backend, oracle_backend, dt
 
 @pytest.mark.parametrize("dtype", [np.int64, np.float32, np.int32, np.float64])
 @pytest.mark.parametrize("n", [5000, 40000, 150000, 300000, 600000, 1 << 20])
-def test_long_rows_sorted_leading_digit_first(hip_backend, dtype, n):
-    hip_backend.set_tuning("sort_bucket_min", 1)     # every run length takes the route (the lengths cover each bucket kernel)
-    try:
-        _leading_digit_first(hip_backend, dtype, n)
-    finally:
-        hip_backend.set_tuning("sort_bucket_min", 0)
-
-
-def _leading_digit_first(hip_backend, dtype, n):
-    """Rows whose leading digit spreads them evenly take one tiled pass on
-    that digit and finish every run of equal digits on chip; rows it does not spread (or that
-    vary in one digit only) take the least-significant-digit-first passes in the same call.
+def test_long_rows_cut_into_buckets(hip_backend, dtype, n):
+    """Rows longer than one workgroup sorts are cut into buckets of equal depth by value and
+    each bucket is finished on chip; rows whose keys do not allow that (one value taking more
+    than a bucket holds, ...) take the least-significant-digit-first passes in the same call.
     Checked against numpy's stable sort and against the same call with that route switched off."""
     if np.dtype(dtype).kind == "i":
         wide = full_range_i64(300, n).astype(dtype)                   # even leading digit
@@ -226,36 +218,43 @@ def _leading_digit_first(hip_backend, dtype, n):
     assert np.array_equal(np.ascontiguousarray(Zh.numpy()).view(np.uint8), np.sort(x[:, 0:n:2], axis=-1).view(np.uint8))
 
 
-@pytest.mark.parametrize("dtype", [np.int64, np.float64])
-@pytest.mark.parametrize("n", [40000, 300000, 1 << 20])
-def test_leading_digit_pass_in_its_own_launch_or_not(hip_backend, dtype, n):
-    """Stable argsort of 8-byte keys: the rows sorted most significant digit first run their one
-    tiled pass in a launch of their own (larger tiles) beside rows that take every pass; the same
-    indices and values come out when that launch is switched off, and both match numpy."""
+@pytest.mark.parametrize("dtype", [np.int64, np.float64, np.int32, np.float32])
+@pytest.mark.parametrize("n", [6000, 40000, 300000])
+def test_buckets_ranked_by_comparison_or_by_digit_passes(hip_backend, dtype, n):
+    """A bucket whose counting bins are crowded (many equal or clustered keys) is finished by the
+    stable digit passes - for argsort first by index, then by key - instead of by comparing the
+    entries of a bin.  Forcing that for every bucket ("sort_compare_max" 0), and allowing bins of
+    any size to be compared (4096), gives the same values and indices, and both match numpy."""
     spread = full_range_i64(320, 3 * n).reshape(3, n)
     spread[1, 1::2] = spread[1, 0::2][: spread[1, 1::2].size]                   # every key twice
-    lopsided = (full_range_i64(321, 2 * n).reshape(2, n) >> 40)
-    raw = np.concatenate([spread, lopsided])
+    spread[2] = np.repeat(spread[2, : (n + 99) // 100], 100)[:n]                # runs of 100 equal keys
+    clustered = (full_range_i64(321, 2 * n).reshape(2, n) >> 40)
+    clustered[1] = clustered[1] // 1000 * 1000                                  # few distinct values
+    raw = np.concatenate([spread, clustered])
+    if np.dtype(dtype).itemsize == 4:
+        raw = (raw >> 32).astype(np.int32)
     if np.dtype(dtype).kind == "f":
-        x = raw.view(np.float64).copy()
+        x = raw.view(dtype).copy()
         x[np.isnan(x)] = 0.0
     else:
-        x = raw
+        x = raw.astype(dtype)
     Xh = Tensor.from_numpy(hip_backend, x)
     order = np.argsort(x, axis=-1, kind="stable")
     want = np.take_along_axis(x, order, -1)
-    for own in (0, 1):
-        hip_backend.set_tuning("sort_leading_launch", own)
+    for limit in (0, 96, 4096):
+        hip_backend.set_tuning("sort_compare_max", limit)
         try:
             Yh, Ih = F.argsort(Xh, -1, False, with_values=True)
             Id = F.argsort(Xh, -1, True).numpy().astype(np.int64)
+            Sh = F.sort(Xh, -1).numpy()
         finally:
-            hip_backend.set_tuning("sort_leading_launch", 1)
-        assert np.array_equal(Ih.numpy(), order) and np.array_equal(Yh.numpy().view(np.uint8), want.view(np.uint8))
+            hip_backend.set_tuning("sort_compare_max", 96)
+        assert np.array_equal(Ih.numpy(), order) and np.array_equal(Yh.numpy().view(np.uint8), want.view(np.uint8)), limit
+        assert np.array_equal(np.sort(x, axis=-1).view(np.uint8), Sh.view(np.uint8)), limit
         got = np.take_along_axis(x, Id, -1)
-        assert np.array_equal(got.view(np.uint8), np.ascontiguousarray(want[:, ::-1]).view(np.uint8))
+        assert np.array_equal(got.view(np.uint8), np.ascontiguousarray(want[:, ::-1]).view(np.uint8)), limit
         same = got[:, 1:] == got[:, :-1]
-        assert np.all(Id[:, 1:][same] > Id[:, :-1][same])
+        assert np.all(Id[:, 1:][same] > Id[:, :-1][same]), limit
 
 
 @pytest.mark.parametrize("dtype", [np.int64, np.float64])
