@@ -70,18 +70,20 @@ struct RowRoutes {
 // serialise all 64 lanes on one LDS word; a digit that is the same in a whole batch of
 // keys (constant bytes: small integers, narrow float ranges) is added once per wave.
 template <typename K>
-__global__ __launch_bounds__(kBlock) void sort_histogram(PassIo<K> io, int64_t n, int64_t chunk, int64_t chunks_per_row,
+__global__ __launch_bounds__(kBlock) void sort_histogram(PassIo<K> io, int64_t n, int64_t chunk, int64_t chunks_per_row, int64_t units,
                                                          RowRoutes routes, uint32_t* __restrict__ ghist) {
     constexpr int P = KeyTraits<K>::kPasses;
     constexpr int U = 32 / sizeof(K);                 // keys in flight per thread
     constexpr int R = 32 / P;                         // copies: 8 (32-bit keys) or 4 (64-bit keys): 32 KB
     __shared__ uint32_t hist[P * kRadix * R];
     if (routes.none_here()) return;
-    const int64_t row = blockIdx.x / chunks_per_row;
-    if (routes.elsewhere(row)) return;
+    for (int64_t unit = blockIdx.x; unit < units; unit += gridDim.x) {       // (row, chunk) pairs
+    const int64_t row = unit / chunks_per_row;
+    if (routes.elsewhere(row)) continue;
+    __syncthreads();                                   // the previous unit's histogram has left
     for (int i = threadIdx.x; i < P * kRadix * R; i += kBlock) hist[i] = 0;
     __syncthreads();
-    const int64_t c = blockIdx.x - row * chunks_per_row;
+    const int64_t c = unit - row * chunks_per_row;
     const K* xrow = io.x + io.xmap.at(row);
     const int64_t lo = c * chunk;
     const int64_t hi = (lo + chunk < n) ? lo + chunk : n;
@@ -131,6 +133,7 @@ __global__ __launch_bounds__(kBlock) void sort_histogram(PassIo<K> io, int64_t n
         for (int r = 0; r < R; ++r) v += hist[i * R + r];
         if (v) atomicAdd(&g[i], v);
     }
+    }
 }
 
 // In place: histogram -> exclusive prefix (start of each digit's run in the row).  Workgroup
@@ -170,9 +173,11 @@ __global__ __launch_bounds__(kRadix) void sort_bases(uint32_t* __restrict__ ghis
 
 __global__ __launch_bounds__(kBlock) void sort_clear(uint32_t* __restrict__ p, int64_t words, RowRoutes routes) {
     if (routes.none_here()) return;
-    const int64_t i = (static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x) * 4;
-    if (i + 4 <= words) *reinterpret_cast<uint4*>(p + i) = make_uint4(0u, 0u, 0u, 0u);
-    else for (int64_t j = i; j < words; ++j) p[j] = 0u;
+    for (int64_t b = blockIdx.x; b * (kBlock * 4) < words; b += gridDim.x) {
+        const int64_t i = (b * kBlock + threadIdx.x) * 4;
+        if (i + 4 <= words) *reinterpret_cast<uint4*>(p + i) = make_uint4(0u, 0u, 0u, 0u);
+        else for (int64_t j = i; j < words; ++j) p[j] = 0u;
+    }
 }
 
 // ------------------------------------------------------------------ one pass
@@ -207,15 +212,19 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
     // workgroups are handed out in index order and dealt round-robin over the chip's eight
     // parts: tile t of every row comes before tile t + 1 of any row, so a tile's predecessors
     // in its row have usually finished when it looks back, and the tiles of a row share a
-    // second-level cache when the number of rows is a multiple of eight
-    const int64_t t = blockIdx.x / rows;
-    const int64_t row = blockIdx.x - t * rows;
-    if (routes.elsewhere(row)) return;
+    // second-level cache when the number of rows is a multiple of eight.  With fewer workgroups
+    // than tiles (a launch sized to what the device holds at once) workgroup g takes tiles
+    // g, g + G, ... in that numbering.
+    for (int64_t unit = blockIdx.x; unit < rows * tiles_per_row; unit += gridDim.x) {
+    if (unit != static_cast<int64_t>(blockIdx.x)) __syncthreads();      // the previous tile has left LDS
+    const int64_t t = unit / rows;
+    const int64_t row = unit - t * rows;
+    if (routes.elsewhere(row)) continue;
     const uint32_t* row_moves = moves + row * P;
     const int tag = pass;
     int ran = 0;            // passes before this one that this row ran
     for (int p = 0; p < pass; ++p) ran += row_moves[p] ? 1 : 0;
-    if (!LAST && row_moves[pass] == 0u) return;
+    if (!LAST && row_moves[pass] == 0u) continue;
     const bool first = ran == 0;
     const K* __restrict__ src_keys = first ? nullptr : io.kbuf[(ran - 1) & 1];
     const uint32_t* __restrict__ src_vals = first ? nullptr : io.vbuf[(ran - 1) & 1];
@@ -517,6 +526,7 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
         }
     }
     DLFX_PHASE(5);
+    }
 }
 
 // ------------------------------------------------------------------ rows that fit one workgroup
@@ -906,20 +916,29 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     uint32_t* ghist = reinterpret_cast<uint32_t*>(base + l.hist_off);
     uint32_t* status = reinterpret_cast<uint32_t*>(base + l.status_off);
     const int64_t clear_words = static_cast<int64_t>((l.status_off + l.status_bytes - l.hist_off) / 4);   // histograms + status
-    sort_clear<<<dim3(static_cast<unsigned>(ceil_div(clear_words, kBlock * 4))), dim3(kBlock), 0, stream>>>(ghist, clear_words, routes);
+    // When the bucket route runs, these launches only take the rows it left - usually none - so
+    // they are sized to what the device holds at once and walk their work; an idle launch then
+    // costs a few microseconds however long the rows are.
+    const bool bounded = routes.records != nullptr;
+    auto sized = [&](int64_t units, int64_t room) { return dim3(static_cast<unsigned>(bounded && room > 0 && room < units ? room : units)); };
+    sort_clear<<<sized(ceil_div(clear_words, kBlock * 4), 2048), dim3(kBlock), 0, stream>>>(ghist, clear_words, routes);
     DLFX_CHECK_LAUNCH();
 
     const int64_t chunk = 32768;
     const int64_t chunks_per_row = ceil_div(n, chunk);
     if (m * chunks_per_row > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
-    sort_histogram<K><<<dim3(static_cast<unsigned>(m * chunks_per_row)), dim3(kBlock), 0, stream>>>(io, n, chunk, chunks_per_row, routes, ghist);
+    sort_histogram<K><<<sized(m * chunks_per_row, 1024), dim3(kBlock), 0, stream>>>(io, n, chunk, chunks_per_row, m * chunks_per_row, routes, ghist);
     DLFX_CHECK_LAUNCH();
     // a pass that moves nothing may only be left out when no pass reads the input while
     // another tile of the same pass writes the output over it
     sort_bases<<<dim3(static_cast<unsigned>(m * P)), dim3(kRadix), 0, stream>>>(ghist, moves, y_over_x ? 1 : 0, routes);
     DLFX_CHECK_LAUNCH();
 
-    const dim3 grid(static_cast<unsigned>(m * l.tiles_per_row));
+    // (a tile waits for tiles of workgroups that run beside it: no more workgroups than fit at once)
+    const int64_t room = !bounded ? 0
+                         : a.pairs ? resident_workgroups(sort_pass<K, true, IP, false>, kPassBlock)
+                                   : resident_workgroups(sort_pass<K, false, IK, false>, kPassBlock);
+    const dim3 grid = sized(m * l.tiles_per_row, room);
     for (int p = 0; p < P; ++p) {
         if (p < P - 1) {
             if (a.pairs)

@@ -237,54 +237,92 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
     uint32_t before = incl - sum;
     for (int i = 0; i < static_cast<int>(threadIdx.x / kWave); ++i) before += red[i];
 
-    // every fine bin leaves room in a bucket, and 256 buckets are enough
-    bool ok = biggest < cap;
-    uint32_t target = 1;
-    if (ok) {
-        target = cap - biggest;
-        ok = static_cast<uint64_t>(n) / target + 1 <= static_cast<uint64_t>(kMaxBuckets);
+    // every fine bin leaves room in a bucket
+    const bool fits = biggest < cap;
+    const uint32_t target = fits ? cap - biggest : 1u;
+
+    // A bin goes to bucket (keys before it) / target, so that every bucket holds fewer than
+    // target + biggest = cap keys; and where at least kGapBins empty bins lie between two
+    // populated ones a new bucket starts as well: stray keys far from the rest (a few zeros below
+    // positive values) then do not stretch the range of the bucket next to them, which
+    // split_finish resolves with a fixed number of counting bins.
+    constexpr int kGapBins = 64;
+    int last = -1;                                     // last populated bin of this thread
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+        if (cnt[i]) last = static_cast<int>(threadIdx.x) * PER + i;
+    int seen = wave_scan_inclusive(last, -1, [](int a, int b) { return a > b ? a : b; });
+    __syncthreads();
+    if (lane_id() == kWave - 1) red[threadIdx.x / kWave] = static_cast<uint32_t>(seen);
+    __syncthreads();
+    int populated_before = __shfl_up(seen, 1, kWave);  // last populated bin before this thread's first
+    if (lane_id() == 0) populated_before = -1;
+    for (int i = 0; i < static_cast<int>(threadIdx.x / kWave); ++i)
+        populated_before = static_cast<int>(red[i]) > populated_before ? static_cast<int>(red[i]) : populated_before;
+    uint32_t cuts = 0;                                 // gaps that end in this thread's bins
+    uint32_t cut_at = 0;                               // bit i: bin i of this thread starts a bucket after a gap
+    {
+        int prev = populated_before;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int bin = static_cast<int>(threadIdx.x) * PER + i;
+            if (cnt[i]) {
+                if (prev >= 0 && bin - prev > kGapBins) {
+                    cut_at |= 1u << i;
+                    ++cuts;
+                }
+                prev = bin;
+            }
+        }
     }
-    if (!ok) {
+    const uint32_t cuts_incl = wave_scan_inclusive(cuts, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+    __syncthreads();
+    if (lane_id() == kWave - 1) red[threadIdx.x / kWave] = cuts_incl;
+    __syncthreads();
+    uint32_t cuts_before = cuts_incl - cuts;
+    for (int i = 0; i < static_cast<int>(threadIdx.x / kWave); ++i) cuts_before += red[i];
+
+    uint32_t bucket[PER];
+    {
+        uint32_t run = before, extra = cuts_before;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            extra += (cut_at >> i) & 1u;
+            bucket[i] = run / target + extra;
+            run += cnt[i];
+        }
+    }
+    // the bucket of the bin before this thread's first, and the number of buckets
+    __shared__ uint32_t last_bucket[kSplitBlock];
+    last_bucket[threadIdx.x] = bucket[PER - 1];
+    __syncthreads();
+    const uint32_t n_buckets = last_bucket[kSplitBlock - 1] + 1;
+    if (!fits || n_buckets > static_cast<uint32_t>(kMaxBuckets)) {
         if (threadIdx.x == 0) {
             info.route = 0u;
             atomicAdd(&counters[0], 1u);
         }
         return;
     }
-    // a bin goes to bucket (keys before it) / target: every bucket then holds fewer than
-    // target + biggest = cap keys; a bin opens every bucket after its predecessor's up to its own
-    uint32_t prev_bucket = 0;                          // bucket of the bin before this thread's first
+    // a bin opens every bucket after its predecessor's up to its own
     {
-        // (the last count of the thread before this one: the prefix before this thread's first bin minus that count)
-        const uint32_t prev_cnt = __shfl_up(cnt[PER - 1], 1, kWave);
-        uint32_t carried = prev_cnt;
-        if (lane_id() == 0 && threadIdx.x != 0) {
-            // first lane of a wave: the count lives in the wave before; take it from the chunk histograms again
-            carried = 0;
-            const uint32_t* g = chunk_fine + row * chunks_per_row * (kFine / 2) + (threadIdx.x * PER - 1) / 2;
-            for (int64_t c = 0; c < chunks_per_row; ++c) carried += g[c * (kFine / 2)] >> 16;
-        }
-        if (threadIdx.x != 0) prev_bucket = (before - carried) / target;
-        else info.begin[0] = 0u;
-    }
-    uint32_t bucket[PER];
-    uint32_t run = before;
+        uint32_t prev_bucket = threadIdx.x == 0 ? 0u : last_bucket[threadIdx.x - 1];
+        if (threadIdx.x == 0) info.begin[0] = 0u;
+        uint32_t run = before;
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-        const uint32_t b = run / target;
-        bucket[i] = b;
-        info.bucket_of[threadIdx.x * PER + i] = static_cast<uint8_t>(b);
-        for (uint32_t k = prev_bucket + 1; k <= b; ++k) info.begin[k] = run;
-        prev_bucket = b;
-        run += cnt[i];
+        for (int i = 0; i < PER; ++i) {
+            info.bucket_of[threadIdx.x * PER + i] = static_cast<uint8_t>(bucket[i]);
+            for (uint32_t k = prev_bucket + 1; k <= bucket[i]; ++k) info.begin[k] = run;
+            prev_bucket = bucket[i];
+            run += cnt[i];
+        }
     }
     if (threadIdx.x == kSplitBlock - 1) {
-        // (run == n here) the last bin's bucket is the last one
-        info.n_buckets = prev_bucket + 1;
-        info.begin[prev_bucket + 1] = static_cast<uint32_t>(n);
+        info.n_buckets = n_buckets;
+        info.begin[n_buckets] = static_cast<uint32_t>(n);
         info.route = 1u;
-        listed[0] = prev_bucket + 1;
-        listed[1] = atomicAdd(&counters[2], prev_bucket + 1);
+        listed[0] = n_buckets;
+        listed[1] = atomicAdd(&counters[2], n_buckets);
     }
     per_bucket[threadIdx.x] = 0u;
     __syncthreads();
@@ -839,16 +877,6 @@ __global__ __launch_bounds__(WAVES * kWave) void split_finish_crowded(PassIo<K> 
             if (seg + k * kWave < valid) emit_entry<K, PAIRS>(io, xrow, yrow, irow, at_begin + seg + k * kWave, key[k], PAIRS ? val[k] : 0u);
         __syncthreads();
     }
-}
-
-// Workgroups of `kernel` that the current device holds at once (0 when HIP cannot tell).
-template <typename Kernel>
-int64_t resident_workgroups(Kernel kernel, int block) {
-    int device = 0, units = 0, per_unit = 0;
-    if (hipGetDevice(&device) != hipSuccess) return 0;
-    if (hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_unit, kernel, block, 0) != hipSuccess) return 0;
-    return static_cast<int64_t>(units) * per_unit;
 }
 
 struct SplitLayout {
