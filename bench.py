@@ -27,14 +27,52 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the step's kernels, from two profiler runs of this script with
-# --copy-calibration (rocprofv3 --pmc FETCH_SIZE, then --pmc WRITE_SIZE; KiB per dispatch, each
-# scaled by what the counter reads for the 1 GiB device copy: 2.000 and 1.000).  A counter cannot
-# be read from inside the timed run, so the figures are constants of the kernels as committed.
-MEASURED_TRAFFIC_BYTES = {
-    "reduce_rows_block": 4295020345,      # 2^30 fp32: 1.0000 x the algorithmic bytes
-    "scan_rows_chained": 539300000,       # [64, 2^20] 4-byte elements: 1.0045 x
-}
+# HBM bytes per launch of the library's kernels come from the committed profiler summary (two
+# rocprofv3 --pmc runs of this script, FETCH_SIZE then WRITE_SIZE, each scaled by what the
+# counter reads for a plain 1 GiB device copy): a counter cannot be read from inside the timed
+# run, so the figures are those of the kernels as profiled, looked up by kernel name.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_all_configs_hbm_traffic_pmc.txt")
+
+
+def profiled_traffic():
+    """{kernel name as the profile prints it: HBM bytes per launch} from the lines
+    `traffic_bytes_per_launch <bytes> <kernel>` of the committed summary ({} when it is absent)."""
+    out = {}
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch "):
+                    _, nbytes, name = line.rstrip("\n").split(" ", 2)
+                    out[name] = int(nbytes)
+    except OSError:
+        pass
+    return out
+
+
+def traffic_of(kernels, table):
+    """Sum over the kernels of one call (name prefixes); None when any is missing from the profile."""
+    if not kernels or not table:
+        return None
+    total = 0
+    for k in ([kernels] if isinstance(kernels, str) else kernels):
+        hit = [v for name, v in table.items() if name.startswith(k)]
+        if not hit:
+            return None
+        total += hit[0]
+    return total
+
+
+FAMILY_OF = (("top_k", "top_k"), ("argsort", "sort"), ("sort", "sort"), ("cumsum", "scan"),
+             ("reduce_", "reduce"), ("argmax", "reduce"), ("log_sum_exp", "reduce"))
+
+
+def family_of(op_name):
+    for prefix, family in FAMILY_OF:
+        if op_name.startswith(prefix):
+            return family
+    return None
+
+
 METRIC = "HBM GB/s (% of ~8 TB/s peak) + Gelem/s per op: reduce, scan, top_k, sort"
 
 
@@ -119,6 +157,29 @@ def make_ops(be, which):
 
     ops = []
 
+    # ---------------- ceilings: what the memory system gives a plain two-way and a one-way stream
+    # at the sizes of C2 and C5 (dlfx_copy of a dense view = one 128-bit non-temporal load and
+    # store per thread; the one-way stream is the library's own long-row reduce_max)
+    if on("ceil"):
+        for label, shape in (("[64,2^20]", (64, 1 << 20)), ("[32,512,56,56]", (32, 512, 56, 56))):
+            xs = gen(shape, torch.float32, lambda c: synth.normal(900 + c), 4)
+            y = empty(shape, torch.float32)
+            count = xs[0].numel()
+            dense = [count]
+            calls = [be.copy(dtype_code(np.float32), dense, x.view(-1), 0, [1], y.view(-1), 0, [1], defer=True) for x in xs]
+
+            def v_copy(x=xs[0], y=y, call=calls[0]):
+                call()
+                assert torch.equal(x, y), "copy"
+            ops.append(Op("ceil", "copy_f32_" + label, count, 8 * count, calls, v_copy, "copy_dense"))
+            flat = [x.view(1, -1) for x in xs]
+            calls, outs = reduce_calls("reduce_max", flat, [1])
+
+            def v_read(x=xs[0], out=outs[0], call=calls[0]):
+                call()
+                assert float(out.storage[0]) == float(x.max()), "reduce_max"
+            ops.append(Op("ceil", "read_f32_" + label, count, 4 * count + 4, calls, v_read, "reduce_rows_block"))
+
     # ---------------- C2: scans and the long reduce (the step)
     if on("all", "step", "c2"):
         xi = gen((64, 1 << 20), torch.int32, lambda c: synth.randint(2 + 100 * c, 0, 100), 4)
@@ -192,19 +253,19 @@ def make_ops(be, which):
         def v_mean(x=x5[0], out=outs[0], call=calls[0]):
             call()
             assert torch.allclose(out.storage[:16384].double(), x.double().mean((2, 3)).view(-1), rtol=1e-5, atol=1e-6)
-        ops.append(Op("C5", "reduce_mean{2,3}_f32_[32,512,56,56]", n5, 4 * n5 + 65536, calls, v_mean))
+        ops.append(Op("C5", "reduce_mean{2,3}_f32_[32,512,56,56]", n5, 4 * n5 + 65536, calls, v_mean, "reduce_rows_group<ValueReducer<float, 0, 0>"))
         calls, outs = reduce_calls("reduce_max", x5, [1])
 
         def v_max(x=x5[0], out=outs[0], call=calls[0]):
             call()
             assert torch.equal(out.storage[:100352], x.amax(1).reshape(-1))
-        ops.append(Op("C5", "reduce_max{1}_f32_[32,512,56,56]", n5, 4 * n5 + 401408, calls, v_max))
+        ops.append(Op("C5", "reduce_max{1}_f32_[32,512,56,56]", n5, 4 * n5 + 401408, calls, v_max, "reduce_cols<ValueReducer<float, 2, 0>"))
         calls, outs = argmax_calls(x5, 1)
 
         def v_arg(x=x5[0], out=outs[0], call=calls[0]):
             call()
             assert torch.equal(out.storage[:100352].long(), torch.argmax(x, 1).reshape(-1))
-        ops.append(Op("C5", "argmax{1}_f32_[32,512,56,56]", n5, 4 * n5 + 401408, calls, v_arg))
+        ops.append(Op("C5", "argmax{1}_f32_[32,512,56,56]", n5, 4 * n5 + 401408, calls, v_arg, "reduce_cols<ArgReducer<float, true, int>"))
         calls, y5 = scan_calls(x5, 1)
 
         def v_cs(x=x5[0], y=y5, call=calls[0]):
@@ -213,7 +274,7 @@ def make_ops(be, which):
             mag = torch.cumsum(x.double().abs(), 1)
             tol = 4 * 9 * float(np.finfo(np.float32).eps) * torch.maximum(want.abs(), mag)
             assert bool(((y.double() - want).abs() <= tol).all())
-        ops.append(Op("C5", "cumsum{1}_f32_[32,512,56,56]", n5, 8 * n5, calls, v_cs))
+        ops.append(Op("C5", "cumsum{1}_f32_[32,512,56,56]", n5, 8 * n5, calls, v_cs, "scan_cols<float"))
 
     # ---------------- N1: count and nonzero (the callers next to reduce and scan)
     if on("all", "n1"):
@@ -373,6 +434,14 @@ def topk_ops(be, tensor, xs, ks, config, shape_text):
     return ops
 
 
+def split_kernels(es, pairs, n):
+    """The kernels that move the data of one sort / argsort of rows the bucket route takes."""
+    key = "unsigned int" if es == 4 else "unsigned long"
+    waves = 4 if n <= 131072 else 8
+    flag = "true" if pairs else "false"
+    return ["split_histogram<%s>" % key, "split_pass<%s, %s>" % (key, flag), "split_finish<%s, %s, %d>" % (key, flag, waves)]
+
+
 def sort_ops(be, tensor, xs, config, text):
     import numpy as np
     import torch
@@ -394,7 +463,7 @@ def sort_ops(be, tensor, xs, config, text):
             call()
             assert torch.equal(y, torch.sort(x, dim=1, descending=bool(desc)).values), "sort"
         ops.append(Op(config, "sort_%s_%s" % ("desc" if desc else "asc", text), rows * n, 2 * es * rows * n, calls, v,
-                      "sort_pass"))
+                      split_kernels(es, False, n)))
         calls = []
         for x in xs:
             X = tensor(x)
@@ -413,7 +482,7 @@ def sort_ops(be, tensor, xs, config, text):
             else:
                 assert bool((g[:, 1:] <= g[:, :-1]).all() if desc else (g[:, 1:] >= g[:, :-1]).all())
         ops.append(Op(config, "argsort_%s_%s" % ("desc" if desc else "asc", text), rows * n, (es + 4) * rows * n,
-                      calls, va, "sort_pass"))
+                      calls, va, split_kernels(es, True, n)))
     return ops
 
 
@@ -507,7 +576,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3 | short (many short rows and an outer axis; not part of all)")
+    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3 | short (many short rows and an outer axis; not part of all) | ceil (copy and read-only streams at the C2 and C5 sizes; not part of all)")
     ap.add_argument("--cpu-all", action="store_true",
                     help="also time the CPU restatement on a bounded sample of every configuration")
     ap.add_argument("--no-cpu", action="store_true")
@@ -531,6 +600,8 @@ def main():
                 op.verify()
         torch.cuda.synchronize()
         log("parity gates passed")
+
+    traffic_table = profiled_traffic()
 
     # ---- the step: C2a + C2b + C2c back to back
     step_ops = [op for op in ops if op.config in ("C2a", "C2b", "C2c")]
@@ -571,7 +642,7 @@ def main():
         result["roofline"] = {"bound": "hbm", "kernel": dom.kernel, "op": dom.name, "achieved": round(achieved, 1),
                               "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                               "avg_launch_us": round(avg_us, 2),
-                              "traffic": next((v for k, v in MEASURED_TRAFFIC_BYTES.items() if k in dom.kernel), None)}
+                              "traffic": traffic_of(dom.kernel, traffic_table)}
     else:
         result.update({"value": None, "ms_per_step": None, "config": {"workload": args.configs}})
 
@@ -589,6 +660,24 @@ def main():
         per_op.append(entry)
         log("%-4s %-44s %10.1f us %9.1f GB/s %6.1f%%" % (op.config, op.name, med, gbs, 100 * gbs / HBM_PEAK_GBS))
     result["per_op"] = per_op
+
+    # ---- each family's worst case over the bandwidth-bound configurations (C2 - C5; C1 moves
+    # 1 MB and is bound by launch latency: it is reported by c1_graph below)
+    by_family = {}
+    for op, entry in zip(ops, per_op):
+        fam = family_of(op.name)
+        if fam is None or op.config not in ("C2a", "C2b", "C2c", "C3", "C4a", "C4b", "C5"):
+            continue
+        if fam not in by_family or entry["frac_hbm"] < by_family[fam]["frac"]:
+            traffic = traffic_of(op.kernel, traffic_table)
+            by_family[fam] = {"config": op.config, "op": op.name, "kernels": op.kernel, "us": entry["us"],
+                              "achieved": entry["gb_s"], "unit": "GB/s", "peak": HBM_PEAK_GBS, "frac": entry["frac_hbm"],
+                              "algorithmic_bytes": op.alg_bytes, "traffic": traffic,
+                              "traffic_ratio": None if traffic is None else round(traffic / op.alg_bytes, 3)}
+    if by_family:
+        result["roofline_by_family"] = by_family
+        for fam, e in by_family.items():
+            log("worst %-7s %-4s %-40s %6.1f%% of peak, HBM traffic x%s" % (fam, e["config"], e["op"], 100 * e["frac"], e["traffic_ratio"]))
 
     # ---- the launch-bound configuration recorded once and replayed as a HIP graph
     c1 = [op for op in ops if op.config == "C1"]

@@ -99,9 +99,10 @@ __device__ __forceinline__ T block_reduce(T v, Join join, T* lds, int waves) {
 
 // ------------------------------------------------------------------ 1. the range of a row's keys
 template <typename K>
-__global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_t n, SplitRow* __restrict__ rows) {
+__global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_t n, SplitRow* __restrict__ rows, uint32_t* __restrict__ counters) {
     __shared__ K red[kSplitBlock / kWave];
     const int64_t row = blockIdx.x;
+    if (row == 0 && threadIdx.x < 4) counters[threadIdx.x] = 0u;      // what the later launches of this sort count up from
     const K* xrow = io.x + io.xmap.at(row);
     // 1024 evenly spaced keys, each wave's 256 spread over the whole row (the last one is the
     // row's last key: a sorted row shows its whole range)
@@ -136,12 +137,6 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
         rows[row].shift = shift;
         rows[row].base = static_cast<unsigned long long>(lo > margin ? static_cast<K>(lo - margin) : K(0));
     }
-}
-
-__global__ __launch_bounds__(256) void split_clear(uint32_t* __restrict__ p, int64_t words) {
-    const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
-    if (i + 4 <= words) *reinterpret_cast<uint4*>(p + i) = make_uint4(0u, 0u, 0u, 0u);
-    else for (int64_t j = i; j < words; ++j) p[j] = 0u;
 }
 
 // ------------------------------------------------------------------ 2. fine-bin histograms
@@ -530,7 +525,8 @@ __device__ __forceinline__ uint4 bucket_at(const SplitRow* __restrict__ infos, u
     return make_uint4(row, b0, info.begin[b + 1] - b0, id);
 }
 
-// Entry `at` of the sorted row goes to the strided outputs.
+// Entry `at` of the sorted row goes to the strided outputs (unit strides: plain 32-bit offsets
+// from the row's start, the case every contiguous output takes).
 template <typename K, bool PAIRS>
 __device__ __forceinline__ void emit_entry(const PassIo<K>& io, const K* xrow, K* yrow, int64_t irow, int64_t at, K key, uint32_t val) {
     if (yrow) {
@@ -538,11 +534,13 @@ __device__ __forceinline__ void emit_entry(const PassIo<K>& io, const K* xrow, K
         if constexpr (PAIRS) {
             if (io.restore_zero && static_cast<K>(bits << 1) == 0) bits = xrow[static_cast<int64_t>(val) * io.sx];
         }
-        yrow[at * io.sy] = bits;
+        if (io.sy == 1) yrow[static_cast<uint32_t>(at)] = bits;
+        else yrow[at * io.sy] = bits;
     }
     if constexpr (PAIRS) {
         if (io.idx) {
-            if (io.idx64) static_cast<int64_t*>(io.idx)[irow + at * io.si] = static_cast<int64_t>(val);
+            if (io.si == 1 && !io.idx64) (static_cast<int32_t*>(io.idx) + irow)[static_cast<uint32_t>(at)] = static_cast<int32_t>(val);
+            else if (io.idx64) static_cast<int64_t*>(io.idx)[irow + at * io.si] = static_cast<int64_t>(val);
             else static_cast<int32_t*>(io.idx)[irow + at * io.si] = static_cast<int32_t>(val);
         }
     }
@@ -732,7 +730,9 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
                         const uint32_t pos = (old[k] >> (16u * (bin[k] & 1u))) & 0xffffu;
                         sm.keys[pos] = key[k];
                         if constexpr (PAIRS) sm.vals[pos] = val[k];
-                        if constexpr (KEEP) sm.bin_at[pos] = static_cast<uint16_t>(bin[k]);
+                        if constexpr (KEEP) {
+                            if (compare) sm.bin_at[pos] = static_cast<uint16_t>(bin[k]);
+                        }
                     }
                 }
             }
@@ -938,9 +938,7 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
     *route_stride = sizeof(SplitRow);
     (void)poll_limit;            // nothing waits for anything on this route
 
-    split_clear<<<dim3(1), dim3(256), 0, stream>>>(counters, 64);
-    DLFX_CHECK_LAUNCH();
-    split_sample<K><<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(io, n, rows);
+    split_sample<K><<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(io, n, rows, counters);
     DLFX_CHECK_LAUNCH();
     const dim3 chunks(static_cast<unsigned>(m * l.chunks_per_row));
     split_histogram<K><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine);
