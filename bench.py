@@ -35,27 +35,30 @@ TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_all_configs_hbm_traffic_
 
 
 def profiled_traffic():
-    """{kernel name as the profile prints it: HBM bytes per launch} from the lines
-    `traffic_bytes_per_launch <bytes> <kernel>` of the committed summary ({} when it is absent)."""
+    """{(configuration, kernel name as the profile prints it): HBM bytes per launch} from the lines
+    `traffic_bytes_per_launch <bytes> <configuration> <kernel>` of the committed summary ({} when
+    it is absent).  The profile is taken one configuration (C1 ... C5) at a time, so a kernel that
+    several configurations launch at different sizes has a figure for each."""
     out = {}
     try:
         with open(TRAFFIC_PROFILE) as f:
             for line in f:
                 if line.startswith("traffic_bytes_per_launch "):
-                    _, nbytes, name = line.rstrip("\n").split(" ", 2)
-                    out[name] = int(nbytes)
+                    _, nbytes, config, name = line.rstrip("\n").split(" ", 3)
+                    out[(config, name)] = int(nbytes)
     except OSError:
         pass
     return out
 
 
-def traffic_of(kernels, table):
-    """Sum over the kernels of one call (name prefixes); None when any is missing from the profile."""
+def traffic_of(kernels, table, config):
+    """Sum over the kernels of one call (name prefixes) as profiled for the operation's
+    configuration; None when any is missing from the profile."""
     if not kernels or not table:
         return None
     total = 0
     for k in ([kernels] if isinstance(kernels, str) else kernels):
-        hit = [v for name, v in table.items() if name.startswith(k)]
+        hit = [v for (c, name), v in table.items() if c == config[:2] and name.startswith(k)]
         if not hit:
             return None
         total += hit[0]
@@ -159,7 +162,7 @@ def make_ops(be, which):
 
     # ---------------- ceilings: what the memory system gives a plain two-way and a one-way stream
     # at the sizes of C2 and C5 (dlfx_copy of a dense view = one 128-bit non-temporal load and
-    # store per thread; the one-way stream is the library's own long-row reduce_max)
+    # store per thread; the one-way stream is the library's reduce_max over rows of 4096, a workgroup a row)
     if on("ceil"):
         for label, shape in (("[64,2^20]", (64, 1 << 20)), ("[32,512,56,56]", (32, 512, 56, 56))):
             xs = gen(shape, torch.float32, lambda c: synth.normal(900 + c), 4)
@@ -172,13 +175,13 @@ def make_ops(be, which):
                 call()
                 assert torch.equal(x, y), "copy"
             ops.append(Op("ceil", "copy_f32_" + label, count, 8 * count, calls, v_copy, "copy_dense"))
-            flat = [x.view(1, -1) for x in xs]
-            calls, outs = reduce_calls("reduce_max", flat, [1])
+            rows = [x.view(-1, 4096) for x in xs]
+            calls, outs = reduce_calls("reduce_max", rows, [1])
 
-            def v_read(x=xs[0], out=outs[0], call=calls[0]):
+            def v_read(x=rows[0], out=outs[0], call=calls[0]):
                 call()
-                assert float(out.storage[0]) == float(x.max()), "reduce_max"
-            ops.append(Op("ceil", "read_f32_" + label, count, 4 * count + 4, calls, v_read, "reduce_rows_block"))
+                assert torch.equal(out.storage.view(-1), x.max(dim=1).values), "reduce_max"
+            ops.append(Op("ceil", "read_f32_" + label, count, 4 * count + 4 * (count // 4096), calls, v_read, "reduce_rows_block"))
 
     # ---------------- C2: scans and the long reduce (the step)
     if on("all", "step", "c2"):
@@ -439,7 +442,8 @@ def split_kernels(es, pairs, n):
     key = "unsigned int" if es == 4 else "unsigned long"
     waves = 4 if n <= 131072 else 8
     flag = "true" if pairs else "false"
-    return ["split_histogram<%s>" % key, "split_pass<%s, %s>" % (key, flag), "split_finish<%s, %s, %d>" % (key, flag, waves)]
+    return ["split_sample<%s>" % key, "split_histogram<%s>" % key, "split_plan", "split_pass<%s, %s>" % (key, flag),
+            "split_finish<%s, %s, %d>" % (key, flag, waves)]
 
 
 def sort_ops(be, tensor, xs, config, text):
@@ -642,7 +646,7 @@ def main():
         result["roofline"] = {"bound": "hbm", "kernel": dom.kernel, "op": dom.name, "achieved": round(achieved, 1),
                               "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                               "avg_launch_us": round(avg_us, 2),
-                              "traffic": traffic_of(dom.kernel, traffic_table)}
+                              "traffic": traffic_of(dom.kernel, traffic_table, dom.config)}
     else:
         result.update({"value": None, "ms_per_step": None, "config": {"workload": args.configs}})
 
@@ -669,7 +673,7 @@ def main():
         if fam is None or op.config not in ("C2a", "C2b", "C2c", "C3", "C4a", "C4b", "C5"):
             continue
         if fam not in by_family or entry["frac_hbm"] < by_family[fam]["frac"]:
-            traffic = traffic_of(op.kernel, traffic_table)
+            traffic = traffic_of(op.kernel, traffic_table, op.config)
             by_family[fam] = {"config": op.config, "op": op.name, "kernels": op.kernel, "us": entry["us"],
                               "achieved": entry["gb_s"], "unit": "GB/s", "peak": HBM_PEAK_GBS, "frac": entry["frac_hbm"],
                               "algorithmic_bytes": op.alg_bytes, "traffic": traffic,

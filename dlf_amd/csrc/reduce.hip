@@ -392,13 +392,21 @@ __global__ __launch_bounds__(kBlock) void reduce_cols(
         if (red.rank == 1) {
             const int64_t s = red.strides[0];
             int64_t j = lo + ty;
-            for (; j + 7 * TY < hi; j += 8 * TY) {
-                typename R::in_t v[8];
+            // row loads a lane keeps in flight: four when the launch fills the chip several times
+            // over (measured: deeper queues then only slow the memory system down), eight when
+            // few wavefronts have to cover the latency
+            auto rows_at_once = [&](auto depth) __attribute__((always_inline)) {
+                constexpr int U = decltype(depth)::value;
+                for (; j + (U - 1) * TY < hi; j += U * TY) {
+                    typename R::in_t v[U];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) v[u] = load_stream(&p[(j + u * TY) * s]);
+                    for (int u = 0; u < U; ++u) v[u] = load_stream(&p[(j + u * TY) * s]);
 #pragma unroll
-                for (int u = 0; u < 8; ++u) acc = R::join(acc, R::map(v[u], j + u * TY, prm));
-            }
+                    for (int u = 0; u < U; ++u) acc = R::join(acc, R::map(v[u], j + u * TY, prm));
+                }
+            };
+            if (gridDim.x >= 1024) rows_at_once(std::integral_constant<int, 4>());
+            else rows_at_once(std::integral_constant<int, 8>());
             for (; j < hi; j += TY) acc = R::join(acc, R::map(load_stream(&p[j * s]), j, prm));
         } else {
             for (int64_t j = lo + ty; j < hi; j += TY) acc = R::join(acc, R::map(p[red.at(j)], j, prm));

@@ -15,9 +15,13 @@
 //     cumsum over C of NCHW).  Lanes run along the kept axis so each load is a
 //     contiguous segment, the four waves of a workgroup take consecutive
 //     chunks of the scanned axis and exchange chunk totals through LDS.
+#include <atomic>
+#include <chrono>
 #include <cstring>
 #include <limits>
 #include <type_traits>
+
+#include <unistd.h>
 
 #include "common.hip.h"
 
@@ -70,6 +74,8 @@ struct TileState<T, 4> {
     static size_t bytes(int64_t tiles) { return static_cast<size_t>(tiles) * 8; }
     __host__ __device__ void bind(void* base, int64_t) { words = static_cast<unsigned long long*>(base); }
     __device__ __forceinline__ void clear(int64_t i) { words[i] = 0ull; }
+    // the same from inside the launch that goes on to use the states
+    __device__ __forceinline__ void clear_shared(int64_t i) { __hip_atomic_store(&words[i], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
     __device__ __forceinline__ void publish(int64_t i, uint32_t flag, T v) {
         unsigned long long w = (static_cast<unsigned long long>(flag) << 32) | bit_cast<uint32_t>(v);
         __hip_atomic_store(&words[i], w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -98,6 +104,10 @@ struct TileStateWords {
     __device__ __forceinline__ void clear(int64_t i) {
 #pragma unroll
         for (int k = 0; k < WORDS; ++k) words[i * WORDS + k] = 0ull;
+    }
+    __device__ __forceinline__ void clear_shared(int64_t i) {
+#pragma unroll
+        for (int k = 0; k < WORDS; ++k) __hip_atomic_store(&words[i * WORDS + k], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __device__ __forceinline__ void publish(int64_t i, uint32_t flag, T v) {
         const Parts p = bit_cast<Parts>(v);
@@ -133,6 +143,35 @@ __global__ __launch_bounds__(kBlock) void scan_init(unsigned* ticket, int64_t ro
     if (i < tiles) st.clear(i);
 }
 
+// Tile states cleared by the scan launch itself.  The states are cut into slices of kSliceTiles;
+// workgroup s of the launch clears slice s before anything else and then stores the call's
+// nonce into ready[s].  A state is published, or read, only once its slice's word has been seen
+// to hold the nonce: what the scratch held before the call (anything) cannot pass for a state
+// of this call.  Workgroups are dispatched in index order and workgroup s never waits before it
+// clears, so the slice of tile g (s = g / kSliceTiles <= g) is cleared by a workgroup that
+// started no later than tile g's.  The nonce is a kernel argument: a recorded launch replayed
+// from a graph would meet its own nonce from the replay before, so launches under stream
+// capture clear the states with a launch of their own (ready == nullptr), as do in-place
+// scans, whose tickets need clearing too.
+constexpr int64_t kSliceTiles = 1024;
+struct ClearedBy {
+    unsigned long long* ready;
+    unsigned long long nonce;
+    __device__ __forceinline__ bool seen(int64_t slice) const {
+        return __hip_atomic_load(&ready[slice], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nonce;
+    }
+    // Returns once slice `slice` is cleared; `early` is an earlier load of its word.
+    __device__ __forceinline__ void await(int64_t slice, unsigned long long early) const {
+        if (early != nonce)
+            while (!seen(slice)) __builtin_amdgcn_s_sleep(1);
+        // What follows are agent-scope atomics on the states, which the hardware issues after
+        // this load has returned and which go to the same coherence point: the compiler alone
+        // has to keep them behind it (a cache-invalidating agent-scope fence here costs more
+        // than the separate clearing launch did).
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+};
+
 // Elements per memory access: 16 bytes of the arithmetic type, or of the stored type when input
 // and output are both 16-bit (half scans compute in fp32 but should still move 16 bytes at a time).
 template <typename T, typename X, typename Y>
@@ -162,7 +201,7 @@ template <typename T, int K, int ITEMS, bool CHAINED, bool SELF_HELP, int BLOCK 
 __device__ __forceinline__ void scan_tile(
     const X* __restrict__ x, Y* __restrict__ y, const DimMap& xmap, const DimMap& ymap, int64_t sx, int64_t sy,
     const DimMap& xaxis, int64_t n, int64_t tiles_per_row, int exclusive, int64_t row, int64_t t, int poll_limit,
-    TileState<T>& st, RowScanShared<T>& sm) {
+    TileState<T>& st, RowScanShared<T>& sm, const ClearedBy& cb = ClearedBy{nullptr, 0ull}, unsigned long long ready_early = 0ull) {
     // where element i of a row lives: i * sx, or (scan_nonzero over a flattened view whose
     // dimensions do not merge) wherever the row-major walk of `xaxis` puts it
     auto x_at = [&](int64_t i) -> int64_t {
@@ -243,11 +282,25 @@ __device__ __forceinline__ void scan_tile(
     if (CHAINED) {
         if (w == 0) {
             const int64_t sbase = row * tiles_per_row;
+            // states from here on are known to be cleared (when this launch clears them itself)
+            int64_t cleared_from = 0;
+            if (cb.ready) {
+                const int64_t slice = (sbase + t) / kSliceTiles;
+                cb.await(slice, ready_early);
+                cleared_from = slice * kSliceTiles;
+            }
             if (lane == 0) st.publish(sbase + t, t == 0 ? kInclusive : kAggregate, aggregate);
             T excl = Op::identity();
             if (t > 0) {
                 int64_t pos = t - 1;
                 for (;;) {
+                    // the states this round reads reach back to pos - 63 or to the row's first
+                    const int64_t lowest = sbase + (pos >= kWave - 1 ? pos - (kWave - 1) : 0);
+                    while (lowest < cleared_from) {
+                        const int64_t slice = (cleared_from - 1) / kSliceTiles;
+                        cb.await(slice, 0ull);
+                        cleared_from = slice * kSliceTiles;
+                    }
                     const int64_t idx = pos - lane;
                     T v = Op::identity();
                     uint32_t f = kInclusive;          // before the row: an inclusive identity
@@ -455,28 +508,52 @@ __global__ __launch_bounds__(kBlock) void scan_rows_group(
 template <typename T, int K, int ITEMS, bool TICKET, int BLOCK, typename X, bool NZ, typename Y>
 __global__ __launch_bounds__(BLOCK) void scan_rows_chained(
     const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy, DimMap xaxis,
-    int64_t n, int64_t tiles_per_row, int exclusive, int poll_limit, unsigned* ticket, TileState<T> st) {
+    int64_t n, int64_t tiles_per_row, int exclusive, int poll_limit, unsigned* ticket, TileState<T> st, ClearedBy cb) {
     __shared__ RowScanShared<T> sm;
     const int64_t row = blockIdx.x / tiles_per_row;
     int64_t t = blockIdx.x - row * tiles_per_row;
+    unsigned long long ready_early = 0ull;
+    if constexpr (!TICKET) {
+        if (cb.ready) {
+            const int64_t tiles = gridDim.x;
+            if (static_cast<int64_t>(blockIdx.x) * kSliceTiles < tiles) {
+                // this workgroup's slice of the states: cleared, made visible, announced
+                for (int64_t i = threadIdx.x; i < kSliceTiles; i += BLOCK) {
+                    const int64_t idx = static_cast<int64_t>(blockIdx.x) * kSliceTiles + i;
+                    if (idx < tiles) st.clear_shared(idx);
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+                __syncthreads();
+                if (threadIdx.x == 0) __hip_atomic_store(&cb.ready[blockIdx.x], cb.nonce, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            // asked for now, looked at when the tile has been loaded and scanned
+            ready_early = __hip_atomic_load(&cb.ready[blockIdx.x / kSliceTiles], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
     if constexpr (TICKET) {
         if (threadIdx.x == 0) sm.next_tile = atomicAdd(&ticket[row], 1u);
         __syncthreads();
         t = sm.next_tile;
     }
-    scan_tile<T, K, ITEMS, true, !TICKET, BLOCK, X, NZ, Y>(x, y, xmap, ymap, sx, sy, xaxis, n, tiles_per_row, exclusive, row, t, poll_limit, st, sm);
+    scan_tile<T, K, ITEMS, true, !TICKET, BLOCK, X, NZ, Y>(x, y, xmap, ymap, sx, sy, xaxis, n, tiles_per_row, exclusive, row, t, poll_limit, st, sm,
+                                                           TICKET ? ClearedBy{nullptr, 0ull} : cb, ready_early);
 }
 
 // ------------------------------------------------------------------ column kernel
 // One lane per row ("column"), four waves along the scanned axis.  Each pass of
 // the loop covers kWaves * chunk positions of the axis: thread (lx, ty) scans
 // positions [s + ty*chunk, s + (ty+1)*chunk) in registers.
+#ifndef DLFX_SCAN_COLS_CHUNK
+#define DLFX_SCAN_COLS_CHUNK 16
+#endif
+constexpr int kColsChunk = DLFX_SCAN_COLS_CHUNK;      // rows of a column a wave scans per round
+
 template <typename T, int K, typename X, bool NZ, typename Y>
 __global__ __launch_bounds__(kBlock) void scan_cols(
     const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
     int64_t m, int64_t n, int chunk, int exclusive) {
     using Op = ScanOp<T, K>;
-    constexpr int R = 16;
+    constexpr int R = kColsChunk;
     __shared__ T totals[2][kWaves][kWave];
 
     const int lx = threadIdx.x & (kWave - 1);
@@ -488,14 +565,25 @@ __global__ __launch_bounds__(kBlock) void scan_cols(
 
     T carry = Op::identity();
     int buf = 0;
-    for (int64_t s = 0; s < n; s += static_cast<int64_t>(kWaves) * chunk, buf ^= 1) {
+    const int waves = static_cast<int>(blockDim.x) / kWave;       // 4, or 1 when every column block has a wave of its own
+    const int64_t step = static_cast<int64_t>(waves) * chunk;
+    // the wave's chunk of the next round is on its way while this round is scanned and stored
+    auto load_chunk = [&](int64_t s, T* v) __attribute__((always_inline)) {
         const int64_t p0 = s + static_cast<int64_t>(ty) * chunk;
-        T v[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int64_t p = p0 + r;
             v[r] = (live && r < chunk && p < n) ? scan_input<T, X, NZ>(load_stream(&xc[p * sx])) : Op::identity();
         }
+    };
+    T ahead[R];
+    load_chunk(0, ahead);
+    for (int64_t s = 0; s < n; s += step, buf ^= 1) {
+        const int64_t p0 = s + static_cast<int64_t>(ty) * chunk;
+        T v[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) v[r] = ahead[r];
+        if (s + step < n) load_chunk(s + step, ahead);
 #pragma unroll
         for (int r = 1; r < R; ++r) v[r] = Op::apply(v[r - 1], v[r]);
         totals[buf][ty][lx] = v[R - 1];
@@ -504,9 +592,11 @@ __global__ __launch_bounds__(kBlock) void scan_cols(
         T all = Op::identity();
 #pragma unroll
         for (int i = 0; i < kWaves; ++i) {
-            const T tv = totals[buf][i][lx];
-            if (i < ty) pre = Op::apply(pre, tv);
-            all = Op::apply(all, tv);
+            if (i < waves) {
+                const T tv = totals[buf][i][lx];
+                if (i < ty) pre = Op::apply(pre, tv);
+                all = Op::apply(all, tv);
+            }
         }
         carry = Op::apply(carry, all);
         if (live) {
@@ -559,10 +649,10 @@ bool make_dim_map2(const int64_t* dims, const int64_t* sx, const int64_t* sy, in
 }
 
 #ifndef DLFX_SCAN_CHAIN_BLOCK
-#define DLFX_SCAN_CHAIN_BLOCK 256
+#define DLFX_SCAN_CHAIN_BLOCK 512
 #endif
 #ifndef DLFX_SCAN_CHAIN_BYTES
-#define DLFX_SCAN_CHAIN_BYTES 65536
+#define DLFX_SCAN_CHAIN_BYTES 131072
 #endif
 constexpr int kChainBlock = DLFX_SCAN_CHAIN_BLOCK;
 constexpr int64_t kChainTileBytes = DLFX_SCAN_CHAIN_BYTES;
@@ -578,21 +668,25 @@ int64_t tile_elems(size_t elem_size, int64_t n) {
 }
 
 struct ScanLayout {
+    bool chained;                          // rows too long for one workgroup's registers: tiles with states
     int64_t tiles_per_row, tiles;
-    size_t ticket_off, state_off, total;
+    size_t ticket_off, state_off, ready_off, total;
 };
 
 ScanLayout scan_layout(size_t elem_size, int64_t m, int64_t n) {
     ScanLayout l;
+    l.chained = n > 256 * (256 / static_cast<int64_t>(elem_size));
     l.tiles_per_row = ceil_div(n, tile_elems(elem_size, n));
     l.tiles = m * l.tiles_per_row;
     l.ticket_off = 0;
     l.state_off = align_up(static_cast<size_t>(m) * 4, 256);
-    if (l.tiles_per_row <= 1) {
+    l.ready_off = 0;
+    if (!l.chained) {
         l.total = 0;
     } else {
         const size_t sb = static_cast<size_t>(l.tiles) * 2 * elem_size;      // a 64-bit word per 32 bits of the value
-        l.total = l.state_off + align_up(sb, 256);
+        l.ready_off = l.state_off + align_up(sb, 256);                       // a word per slice of states
+        l.total = l.ready_off + align_up(static_cast<size_t>(ceil_div(l.tiles, kSliceTiles)) * 8, 256);
     }
     return l;
 }
@@ -611,6 +705,33 @@ bool views_overlap(int rank, const int64_t* dims, const X* x, const int64_t* sx,
     const char* yb = reinterpret_cast<const char*>(y + ylo);
     const char* ye = reinterpret_cast<const char*>(y + yhi + 1);
     return xb < ye && yb < xe;
+}
+
+// True when launches into `stream` are being recorded into a graph (or that cannot be told).
+bool stream_is_capturing(hipStream_t stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;
+    }
+    return status != hipStreamCaptureStatusNone;
+}
+
+// A 64-bit value no earlier call of this process has used and, started from the clock and the
+// process, no other process is likely to have left in reused memory; never zero.
+unsigned long long next_nonce() {
+    static std::atomic<unsigned long long> counter{[] {
+        unsigned long long z = static_cast<unsigned long long>(std::chrono::steady_clock::now().time_since_epoch().count());
+        z ^= static_cast<unsigned long long>(reinterpret_cast<uintptr_t>(&g_poll_limit)) << 17;
+        z ^= static_cast<unsigned long long>(getpid()) << 40;
+        z += 0x9e3779b97f4a7c15ull;                       // splitmix64
+        z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+        z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+        return z ^ (z >> 31);
+    }()};
+    unsigned long long v;
+    do v = counter.fetch_add(0x9e3779b97f4a7c15ull, std::memory_order_relaxed); while (v == 0ull);
+    return v;
 }
 
 template <typename T, int K, typename X = T, bool NZ = false, typename Y = T>
@@ -661,10 +782,15 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     const bool short_rows = n <= 64 && m >= 256;
     const bool use_cols = !axis_general && (short_rows || (!axis_unit && m >= 64 && (inner_unit || n < 4096)));
     if (use_cols) {
-        int chunk = static_cast<int>(ceil_div(n, kWaves) < 16 ? ceil_div(n, kWaves) : 16);
+#ifdef DLFX_SCAN_COLS_ONE_WAVE
+        const int waves = (ceil_div(m, kWave) >= 1024 && n >= 64) ? 1 : kWaves;
+#else
+        const int waves = kWaves;
+#endif
+        int chunk = static_cast<int>(ceil_div(n, waves) < kColsChunk ? ceil_div(n, waves) : kColsChunk);
         const int64_t blocks = ceil_div(m, kWave);
         if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
-        scan_cols<T, K, X, NZ, Y><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
+        scan_cols<T, K, X, NZ, Y><<<dim3(static_cast<unsigned>(blocks)), dim3(waves * kWave), 0, stream>>>(
             x, y, xmap, ymap, sx, sy, m, n, chunk, exclusive);
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
@@ -676,7 +802,7 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     const int64_t tile = tile_elems(sizeof(T), n);
     constexpr int FULL = 256 / sizeof(T);
     const dim3 block(kBlock);
-    if (l.tiles_per_row == 1) {
+    if (!l.chained) {
         const dim3 grid(static_cast<unsigned>(m));
         auto single = [&](auto items) {
             constexpr int ITEMS = decltype(items)::value;
@@ -697,17 +823,27 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     unsigned* ticket = reinterpret_cast<unsigned*>(static_cast<char*>(scratch) + l.ticket_off);
     TileState<T> st;
     st.bind(static_cast<char*>(scratch) + l.state_off, l.tiles);
-    scan_init<T><<<dim3(static_cast<unsigned>(ceil_div(l.tiles, kBlock))), block, 0, stream>>>(ticket, m, st, l.tiles);
-    DLFX_CHECK_LAUNCH();
+    const bool in_place = views_overlap(rank, dims, x, x_strides, y, y_strides);
+    // The scan launch clears the tile states itself, except where that cannot work: under stream
+    // capture (a replayed launch would carry the nonce of the replay before it) and in place
+    // (the rows' tickets need clearing before any workgroup runs).
+    ClearedBy cb{nullptr, 0ull};
+    if (!in_place && !stream_is_capturing(stream)) {
+        cb.ready = reinterpret_cast<unsigned long long*>(static_cast<char*>(scratch) + l.ready_off);
+        cb.nonce = next_nonce();
+    } else {
+        scan_init<T><<<dim3(static_cast<unsigned>(ceil_div(l.tiles, kBlock))), block, 0, stream>>>(ticket, m, st, l.tiles);
+        DLFX_CHECK_LAUNCH();
+    }
     const dim3 grid(static_cast<unsigned>(l.tiles));
     constexpr int CI = static_cast<int>(kChainTileBytes / sizeof(T) / kChainBlock);
     const dim3 cblock(kChainBlock);
-    if (views_overlap(rank, dims, x, x_strides, y, y_strides))
+    if (in_place)
         scan_rows_chained<T, K, CI, true, kChainBlock, X, NZ, Y><<<grid, cblock, 0, stream>>>(
-            x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st);
+            x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st, cb);
     else
         scan_rows_chained<T, K, CI, false, kChainBlock, X, NZ, Y><<<grid, cblock, 0, stream>>>(
-            x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st);
+            x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st, cb);
     DLFX_CHECK_LAUNCH();
     return DLFX_OK;
 }

@@ -1,34 +1,38 @@
 // The bucket route of sort / argsort for rows longer than one workgroup holds (gfx950).
 //
-// A row is cut into at most 256 buckets of at most 5120 (shorter rows: 2560) keys by value, each bucket is then
-// sorted on chip, so the keys cross HBM four times (plus one read for the histogram) however
-// wide they are:
-//   1. split_sample     1024 keys of every row, evenly spaced, give the range of its keys (a few
-//                       stray keys at either end left aside); 4096 "fine bins" resolve that range.
-//   2. split_histogram  one read of the input: fine-bin histogram of every row (LDS atomics)
-//                       and the OR / AND of all its keys.
-//   3. split_plan       per row: neighbouring fine bins are merged into buckets of equal depth
-//                       (bucket of a bin = keys before it / target), so skewed rows - floats
-//                       with their exponents, clustered integers - still give even buckets.
-//                       A row whose sample missed a varying bit, whose largest fine bin does
-//                       not fit a workgroup, or that would need more than 256 buckets keeps
-//                       the least-significant-digit-first passes of sort.hip (decided here, on
-//                       the device, row by row).
-//   4. split_pass       a tile of 4096 keys finds each key's bucket (table in LDS) and its slot
-//                       among the tile's keys of that bucket with one LDS atomic, lays the tile
-//                       out by bucket in LDS and writes it as runs; a tile's offset inside each
-//                       bucket comes from the earlier tiles of the row through chained status
-//                       words (decoupled look-back, bounded waits).  The order inside a run is
-//                       whatever the atomics gave: not stable, and it need not be.
-//   5. split_finish     one workgroup per bucket: the keys' offsets from the bucket minimum,
-//                       scaled to 8192 bins, are counted and placed with LDS atomics; what
-//                       shares a bin (about one other key) is ranked by comparing whole
-//                       (key, index) entries, which also restores the stable order of equal
-//                       keys; the bucket leaves for the strided outputs.  Bins too crowded for
-//                       that (many equal or clustered keys) fall back to the stable digit
-//                       passes of sort_in_workgroup, for pairs first by index, then by key.
+// A row is cut by value into at most 256 buckets of at most 5120 keys (rows of up to 131072 keys:
+// 2560), and every bucket is then sorted on chip, so the keys cross HBM four times (plus one read
+// for the histogram) however wide they are:
+//   1. split_sample     1024 keys of every row, from 256 evenly spaced places, give the range of
+//                       its keys (a few stray keys at either end left aside); 4096 "fine bins"
+//                       resolve that range, keys outside it share the first or the last bin.
+//   2. split_histogram  one read of the input: a fine-bin histogram of every chunk of 32768 keys
+//                       (LDS atomics).
+//   3. split_plan       per row: the chunks' histograms add up to the row's; neighbouring fine
+//                       bins are merged into buckets of equal depth (bucket of a bin = keys
+//                       before it / target, and a new bucket after a long run of empty bins), so
+//                       skewed rows - floats with their exponents, clustered integers - still
+//                       give even buckets.  Every chunk's histogram becomes the place of its keys
+//                       inside each bucket, and the buckets of all rows are listed for the last
+//                       step.  A row whose largest fine bin does not fit a workgroup, or that
+//                       would need more than 256 buckets, keeps the least-significant-digit-first
+//                       passes of sort.hip (decided here, on the device, row by row).
+//   4. split_pass       one workgroup per chunk: a tile of 4096 keys finds each key's bucket
+//                       (table in LDS) and its slot among the tile's keys of that bucket with one
+//                       LDS atomic, lays the tile out by bucket in LDS and writes it as runs to
+//                       where split_plan said the chunk's keys of each bucket go: workgroups
+//                       exchange nothing.  The order inside a run is whatever the atomics gave:
+//                       not stable, and it need not be.
+//   5. split_finish     resident workgroups take buckets from the list: the keys' offsets from
+//                       the bucket minimum, scaled to 8192 (4096) bins, are counted and placed
+//                       with LDS atomics; what shares a bin (about one other key) is ranked by
+//                       comparing whole (key, index) entries, which also restores the stable
+//                       order of equal keys; the bucket leaves for the strided outputs.
+//   6. split_finish_crowded  buckets with a bin too crowded for that (many equal or clustered
+//                       keys) take the stable digit passes of sort_in_workgroup instead, for
+//                       pairs first by index, then by key.
 // Ranking with an LDS atomic costs a few instructions per key where wave-wide digit matching
-// costs about fifty per digit, which is what bounded the digit passes.
+// costs about fifty per digit, which is what bounds the digit passes.
 #include <cstddef>
 #include <cstring>
 
@@ -104,15 +108,17 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
     const int64_t row = blockIdx.x;
     if (row == 0 && threadIdx.x < 4) counters[threadIdx.x] = 0u;      // what the later launches of this sort count up from
     const K* xrow = io.x + io.xmap.at(row);
-    // 1024 evenly spaced keys, each wave's 256 spread over the whole row (the last one is the
-    // row's last key: a sorted row shows its whole range)
+    // 1024 keys: four neighbours (one memory line when the row is contiguous) at each of 256
+    // evenly spaced places, the last of them the row's last keys, so that a sorted row shows
+    // its whole range
     K key[4];
     uint32_t unused[4] = {0u, 0u, 0u, 0u};
+    int64_t e0 = (static_cast<int64_t>(threadIdx.x) * n) / kSplitBlock;
+    if (threadIdx.x == kSplitBlock - 1 || e0 > n - 4) e0 = n - 4;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-        const int64_t j = static_cast<int64_t>(threadIdx.x) + u * kSplitBlock;
-        int64_t e = n >= 1024 ? (j * n) / 1024 : (j < n ? j : n - 1);
-        if (j == 1023) e = n - 1;
+        const int64_t j = static_cast<int64_t>(threadIdx.x) * 4 + u;
+        const int64_t e = n >= 1024 ? e0 + u : (j < n ? j : n - 1);
         key[u] = key_of_element<K>(io, xrow[e * io.sx]);
     }
     // every wave orders its 256 keys and offers its 4th smallest and 4th largest: three stray

@@ -14,7 +14,7 @@ from oracle import oracle as O
 
 pytestmark = pytest.mark.gpu
 
-SIZES = [1, 2, 63, 64, 65, 255, 256, 257, 1000, 1024, 1025, 4095, 4096, 4097, 8192, 12289, 100000]
+SIZES = [1, 2, 63, 64, 65, 255, 256, 257, 1000, 1024, 1025, 4095, 4096, 4097, 8192, 12289, 16384, 16385, 20000, 32768, 32769, 100000]
 
 
 def both(hip, orc, x):
@@ -112,6 +112,24 @@ def test_many_rows_of_one_tile_and_long_single_row(hip_backend, oracle_backend):
     y = randint(50, 3_000_001, 0, 100).astype(np.int32).reshape(1, 3_000_001)
     Yh = Tensor.from_numpy(hip_backend, y)
     assert np.array_equal(F.cumsum(Yh, 1).numpy(), np.cumsum(y, axis=1, dtype=np.int32))
+
+
+def test_tile_states_cleared_slice_by_slice(hip_backend):
+    # Rows of 33 tiles: the tiles' states fill more than one slice of 1024 and a row straddles
+    # the slice boundary, so its look-back reads states that two different workgroups cleared.
+    # Twice over the same scratch: the second call meets the first call's states and must not
+    # take them for its own.
+    n = 33 * 32768
+    x = randint(54, 40 * n, -100, 100).astype(np.int32).reshape(40, n)
+    Xh = Tensor.from_numpy(hip_backend, x)
+    want = np.cumsum(x, axis=1, dtype=np.int32)
+    assert np.array_equal(F.cumsum(Xh, 1).numpy(), want)
+    x2 = (x[::-1] * 3).astype(np.int32).copy()
+    Xh2 = Tensor.from_numpy(hip_backend, x2)
+    assert np.array_equal(F.cumsum(Xh2, 1).numpy(), np.cumsum(x2, axis=1, dtype=np.int32))
+    y = normal(55, 40 * n).astype(np.float64).reshape(40, n)[:6]
+    Yh = Tensor.from_numpy(hip_backend, y)
+    assert np.array_equal(F.cummax(Yh, 1).numpy(), np.maximum.accumulate(y, axis=1))
 
 
 def test_bounded_wait_self_help_path(hip_backend, oracle_backend):
