@@ -656,74 +656,89 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
         const int zeros = ors ? __builtin_ctzll(static_cast<unsigned long long>(ors)) : 0;
         const int key_bits = ors ? 64 - __builtin_clzll(static_cast<unsigned long long>(ors)) - zeros : 0;
         int idx_bits = 0;
+        bool packed = false;                               // the word fits a key's width
         if constexpr (PAIRS) {
             idx_bits = vors ? 32 - __builtin_clz(vors) : 0;
+            packed = idx_bits != 0 && key_bits + idx_bits <= static_cast<int>(8 * sizeof(K));
             if (key_bits + idx_bits > 64) idx_bits = 0;    // wide keys seldom repeat
         }
         const int width = key_bits + idx_bits;
         const int down = width > kBinBits ? width - kBinBits : 0;      // words >> down lie below kBins
-        auto bin_of = [&](K k1, uint32_t v1) __attribute__((always_inline)) -> uint32_t {
-            if constexpr (sizeof(K) == 4) {
-                if (width <= 32) {                         // (uniform) everything fits 32-bit arithmetic
-                    uint32_t word = static_cast<uint32_t>(k1 - lo) >> zeros;
-                    if constexpr (PAIRS) word = idx_bits ? ((word << idx_bits) | (v1 - vlo)) : word;
-                    return word >> down;
-                }
-            }
-            unsigned long long word = static_cast<unsigned long long>(static_cast<K>(k1 - lo) >> zeros);
-            if constexpr (PAIRS) {
-                if (idx_bits) word = (word << idx_bits) | static_cast<unsigned long long>(v1 - vlo);
-            }
-            return static_cast<uint32_t>(word >> down);
-        };
-        // entries that share a bin are told apart by comparison, unless the bin says it all
-        const bool compare = down != 0 || (PAIRS && idx_bits == 0 && vors != 0u);
         SPLIT_PHASE(8);
 
-        // ---- count
-        uint32_t bin[ITEMS];
+        // The rest of the bucket's work in two forms.  PACKED (pairs whose word fits a key's
+        // width): the word alone stands for the entry from here on - it is unique, orders the
+        // entries as (key, index) does, and gives both back when the entry leaves - so LDS holds
+        // one word per entry and ranking is one comparison.  Otherwise keys (and indices) are
+        // kept as they are and entries of a bin are told apart by comparing them whole.
+        auto finish = [&](auto packed_tag) __attribute__((always_inline)) {
+            constexpr bool PACKED = decltype(packed_tag)::value;
+            constexpr bool VALS = PAIRS && !PACKED;              // indices travel beside the keys
+            constexpr bool KEPT = KEEP && !PACKED;               // bins kept beside the entries
+            auto bin_of = [&](K k1, uint32_t v1) __attribute__((always_inline)) -> uint32_t {
+                if constexpr (PACKED) {
+                    return static_cast<uint32_t>(k1 >> down);
+                } else {
+                    unsigned long long word = static_cast<unsigned long long>(static_cast<K>(k1 - lo) >> zeros);
+                    if constexpr (PAIRS) {
+                        if (idx_bits) word = (word << idx_bits) | static_cast<unsigned long long>(v1 - vlo);
+                    }
+                    return static_cast<uint32_t>(word >> down);
+                }
+            };
+            // entries that share a bin are told apart by comparison, unless the bin says it all
+            const bool compare = down != 0 || (VALS && idx_bits == 0 && vors != 0u);
+            if constexpr (PACKED) {
 #pragma unroll
-        for (int k = 0; k < ITEMS; ++k) bin[k] = bin_of(key[k], PAIRS ? val[k] : 0u);
-#pragma unroll
-        for (int k = 0; k < ITEMS; ++k)
-            if (seg + k * kWave < valid) atomicAdd(&sm.bins[bin[k] >> 1], 1u << (16u * (bin[k] & 1u)));
-        __syncthreads();
-        SPLIT_PHASE(9);
-
-        // ---- counts -> bin starts (exclusive prefix over the 8192 bins), and the fullest bin
-        {
-            uint32_t words[WORDS];
-            uint32_t sum = 0, fullest = 0;
-#pragma unroll
-            for (int i = 0; i < WORDS; ++i) {
-                words[i] = sm.bins[tid * WORDS + i];
-                const uint32_t c0 = words[i] & 0xffffu, c1 = words[i] >> 16;
-                sum += c0 + c1;
-                fullest = c0 > fullest ? c0 : fullest;
-                fullest = c1 > fullest ? c1 : fullest;
+                for (int k = 0; k < ITEMS; ++k)
+                    key[k] = static_cast<K>(static_cast<K>(static_cast<K>(key[k] - lo) >> zeros) << idx_bits) | static_cast<K>(val[k] - vlo);
             }
-            const uint32_t incl = wave_scan_inclusive(sum, 0u, [](uint32_t a, uint32_t c) { return a + c; });
-            if (lane == kWave - 1) sm.red32[w] = incl;
-            fullest = wave_reduce(fullest, [](uint32_t a, uint32_t c) { return a > c ? a : c; });
-            if (lane == 0 && fullest > compare_max) atomicMax(&sm.crowded, fullest);
+
+            // ---- count
+            uint32_t bin[ITEMS];
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) bin[k] = bin_of(key[k], VALS ? val[k] : 0u);
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k)
+                if (seg + k * kWave < valid) atomicAdd(&sm.bins[bin[k] >> 1], 1u << (16u * (bin[k] & 1u)));
             __syncthreads();
-            uint32_t run = incl - sum;
-            for (int i = 0; i < w; ++i) run += sm.red32[i];
-#pragma unroll
-            for (int i = 0; i < WORDS; ++i) {
-                const uint32_t c0 = words[i] & 0xffffu, c1 = words[i] >> 16;
-                sm.bins[tid * WORDS + i] = run | ((run + c0) << 16);
-                run += c0 + c1;
-            }
-        }
-        __syncthreads();
-        SPLIT_PHASE(10);
+            SPLIT_PHASE(9);
 
-        if (compare && sm.crowded != 0u) {
-            // many equal or clustered keys: the stable digit passes of split_finish_crowded take this bucket
-            if (tid == 0) crowded_list[atomicAdd(&counters[1], 1u)] = cur.w;
-            if (vn < total) load_bucket(nxt, key, val);
-        } else {
+            // ---- counts -> bin starts (exclusive prefix over the bins), and the fullest bin
+            {
+                uint32_t words[WORDS];
+                uint32_t sum = 0, fullest = 0;
+#pragma unroll
+                for (int i = 0; i < WORDS; ++i) {
+                    words[i] = sm.bins[tid * WORDS + i];
+                    const uint32_t c0 = words[i] & 0xffffu, c1 = words[i] >> 16;
+                    sum += c0 + c1;
+                    fullest = c0 > fullest ? c0 : fullest;
+                    fullest = c1 > fullest ? c1 : fullest;
+                }
+                const uint32_t incl = wave_scan_inclusive(sum, 0u, [](uint32_t a, uint32_t c) { return a + c; });
+                if (lane == kWave - 1) sm.red32[w] = incl;
+                fullest = wave_reduce(fullest, [](uint32_t a, uint32_t c) { return a > c ? a : c; });
+                if (lane == 0 && fullest > compare_max) atomicMax(&sm.crowded, fullest);
+                __syncthreads();
+                uint32_t run = incl - sum;
+                for (int i = 0; i < w; ++i) run += sm.red32[i];
+#pragma unroll
+                for (int i = 0; i < WORDS; ++i) {
+                    const uint32_t c0 = words[i] & 0xffffu, c1 = words[i] >> 16;
+                    sm.bins[tid * WORDS + i] = run | ((run + c0) << 16);
+                    run += c0 + c1;
+                }
+            }
+            __syncthreads();
+            SPLIT_PHASE(10);
+
+            if (compare && sm.crowded != 0u) {
+                // many equal or clustered keys: the stable digit passes of split_finish_crowded take this bucket
+                if (tid == 0) crowded_list[atomicAdd(&counters[1], 1u)] = cur.w;
+                if (vn < total) load_bucket(nxt, key, val);
+                return;
+            }
             // ---- place: the atomic hands out the next free entry of the bin, whose word ends up at its end
             {
                 uint32_t old[ITEMS];
@@ -735,8 +750,8 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
                     if (seg + k * kWave < valid) {
                         const uint32_t pos = (old[k] >> (16u * (bin[k] & 1u))) & 0xffffu;
                         sm.keys[pos] = key[k];
-                        if constexpr (PAIRS) sm.vals[pos] = val[k];
-                        if constexpr (KEEP) {
+                        if constexpr (VALS) sm.vals[pos] = val[k];
+                        if constexpr (KEPT) {
                             if (compare) sm.bin_at[pos] = static_cast<uint16_t>(bin[k]);
                         }
                     }
@@ -751,7 +766,16 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
             const K* xrow = io.x + io.xmap.at(row);
             K* yrow = io.y ? io.y + io.ymap.at(row) : nullptr;
             const int64_t irow = (PAIRS && io.idx) ? io.imap.at(row) : 0;
-            // ---- rank inside the bin and write: thread tid takes entries tid, tid + 512, ...; five at
+            const K idx_mask = static_cast<K>((K(1) << idx_bits) - 1);
+            // entry `at` of the row leaves: a packed word gives its key and index back first
+            auto emit = [&](int64_t at, K k1, uint32_t v1) __attribute__((always_inline)) {
+                if constexpr (PACKED)
+                    emit_entry<K, PAIRS>(io, xrow, yrow, irow, at, static_cast<K>(lo + static_cast<K>(static_cast<K>(k1 >> idx_bits) << zeros)),
+                                         vlo + static_cast<uint32_t>(k1 & idx_mask));
+                else
+                    emit_entry<K, PAIRS>(io, xrow, yrow, irow, at, k1, v1);
+            };
+            // ---- rank inside the bin and write: thread tid takes entries tid, tid + T, ...; five at
             // a time, each step reading for all five before the next step looks at what came back
             constexpr int B = 5;
             static_assert(ITEMS % B == 0, "whole batches");
@@ -759,29 +783,28 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
             for (int k0 = 0; k0 < ITEMS; k0 += B) {
                 if (k0 * T >= valid) break;                // (uniform) nothing left
                 K mine[B];
-                uint32_t mine_v[PAIRS ? B : 1];
+                uint32_t mine_v[VALS ? B : 1] = {};
                 uint32_t mine_b[B];
 #pragma unroll
                 for (int j = 0; j < B; ++j) {
                     const int pos = (k0 + j) * T + tid;
                     const int at = pos < valid ? pos : 0;
                     mine[j] = sm.keys[at];
-                    if constexpr (PAIRS) mine_v[j] = sm.vals[at];
-                    if constexpr (KEEP) mine_b[j] = sm.bin_at[at];
+                    if constexpr (VALS) mine_v[j] = sm.vals[at];
+                    if constexpr (KEPT) mine_b[j] = sm.bin_at[at];
                 }
                 if (!compare) {
 #pragma unroll
                     for (int j = 0; j < B; ++j)
-                        if ((k0 + j) * T + tid < valid)
-                            emit_entry<K, PAIRS>(io, xrow, yrow, irow, begin + (k0 + j) * T + tid, mine[j], PAIRS ? mine_v[j] : 0u);
+                        if ((k0 + j) * T + tid < valid) emit(begin + (k0 + j) * T + tid, mine[j], VALS ? mine_v[j] : 0u);
                     continue;
                 }
                 int first[B], end[B], ahead[B];
 #pragma unroll
                 for (int j = 0; j < B; ++j) {
                     uint32_t b1;
-                    if constexpr (KEEP) b1 = mine_b[j];
-                    else b1 = bin_of(mine[j], PAIRS ? mine_v[j] : 0u);
+                    if constexpr (KEPT) b1 = mine_b[j];
+                    else b1 = bin_of(mine[j], VALS ? mine_v[j] : 0u);
                     end[j] = static_cast<int>((sm.bins[b1 >> 1] >> (16u * (b1 & 1u))) & 0xffffu);
                     const uint32_t b0 = b1 - 1u;
                     first[j] = b1 == 0u ? 0 : static_cast<int>((sm.bins[b0 >> 1] >> (16u * (b0 & 1u))) & 0xffffu);
@@ -791,20 +814,22 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
 #pragma unroll
                 for (int i = 0; i < kNear; ++i) {
                     K other[B];
-                    uint32_t other_v[PAIRS ? B : 1];
+                    uint32_t other_v[VALS ? B : 1] = {};
 #pragma unroll
                     for (int j = 0; j < B; ++j) {
                         const int q = first[j] + i < valid ? first[j] + i : 0;
                         other[j] = sm.keys[q];
-                        if constexpr (PAIRS) other_v[j] = sm.vals[q];
+                        if constexpr (VALS) other_v[j] = sm.vals[q];
                     }
 #pragma unroll
                     for (int j = 0; j < B; ++j) {
                         const int q = first[j] + i;
                         bool before = other[j] < mine[j];
-                        if (other[j] == mine[j]) {
-                            if constexpr (PAIRS) before = other_v[j] < mine_v[j];
-                            else before = q < (k0 + j) * T + tid;
+                        if constexpr (!PACKED) {               // (packed words are all different)
+                            if (other[j] == mine[j]) {
+                                if constexpr (VALS) before = other_v[j] < mine_v[j];
+                                else before = q < (k0 + j) * T + tid;
+                            }
                         }
                         ahead[j] += (q < end[j] && before) ? 1 : 0;
                     }
@@ -816,17 +841,21 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
                     for (int q = first[j] + kNear; q < end[j]; ++q) {          // the rest of a fuller bin
                         const K other = sm.keys[q];
                         bool before = other < mine[j];
-                        if (other == mine[j]) {
-                            if constexpr (PAIRS) before = sm.vals[q] < mine_v[j];
-                            else before = q < pos;
+                        if constexpr (!PACKED) {
+                            if (other == mine[j]) {
+                                if constexpr (VALS) before = sm.vals[q] < mine_v[j];
+                                else before = q < pos;
+                            }
                         }
                         ahead[j] += before ? 1 : 0;
                     }
-                    emit_entry<K, PAIRS>(io, xrow, yrow, irow, begin + first[j] + ahead[j], mine[j], PAIRS ? mine_v[j] : 0u);
+                    emit(begin + first[j] + ahead[j], mine[j], VALS ? mine_v[j] : 0u);
                 }
             }
             SPLIT_PHASE(12);
-        }
+        };
+        if (PAIRS && packed) finish(std::integral_constant<bool, PAIRS>());
+        else finish(std::false_type());
         if (vn >= total) break;
         v = vn;
         cur = nxt;
