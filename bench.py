@@ -234,6 +234,22 @@ def make_ops(be, which):
             assert torch.equal(out.storage[:256].long(), torch.argmax(x, 1))
         ops.append(Op("C1", "argmax_f32_[256,1000]", 256000, 1024000 + 1024, calls, v_am))
         ops += topk_ops(be, tensor, x1, [5], "C1", "[256,1000]")
+        # the same five results from one launch (dlfx_logits_head); reported beside C1, not part of it
+        hs, hm, hl = (empty((256,), torch.float32) for _ in range(3))
+        ha = torch.empty(256, dtype=torch.int32, device=dev)
+        hv = empty((256, 5), torch.float32)
+        hi = torch.empty((256, 5), dtype=torch.int32, device=dev)
+        calls = [be.logits_head(dtype_code(np.float32), 256, 1000, x.view(-1), 0, 1000, hs, hm, ha, hl, 5, hv, hi, defer=True) for x in x1]
+
+        def v_head(x=x1[0], call=calls[0]):
+            call()
+            assert torch.allclose(hs.double(), x.double().sum(1), rtol=1e-5, atol=1e-5)
+            assert torch.equal(hm, x.amax(1)) and torch.equal(ha.long(), torch.argmax(x, 1))
+            assert torch.allclose(hl.double(), torch.logsumexp(x.double(), 1), rtol=1e-5, atol=1e-5)
+            top = torch.topk(x, 5, dim=1)
+            assert torch.equal(hv, top.values) and torch.equal(torch.gather(x, 1, hi.long()), hv)
+        ops.append(Op("C1f", "logits_head(sum,max,argmax,lse,top_k5)_f32_[256,1000]", 256000, 1024000 + 256 * 56, calls, v_head,
+                      "logits_head_rows"))
 
     # ---------------- C3: top_k
     if on("all", "c3"):
@@ -706,6 +722,16 @@ def main():
         us = e0.elapsed_time(e1) * 1e3 / reps
         result["c1_graph"] = {"ops": len(c1), "us_per_replay": round(us, 2), "us_per_op": round(us / len(c1), 2)}
         log("C1   %d ops replayed as one HIP graph: %.1f us per replay, %.1f us per op" % (len(c1), us, us / len(c1)))
+        # the floor of this way of measuring: a one-element fill (a kernel that does nothing to
+        # speak of), issued and timed exactly like the operations above
+        one = torch.zeros(1, dtype=torch.float32, device=be.device)
+        floor = Op("C1", "floor", 1, 4, [be.fill(0, [1], [1], one, 0, 1.0, defer=True)])
+        result["c1_floor_us"] = round(time_op(torch, floor, 50)[0], 2)
+        log("C1   launch floor (one-element fill, timed the same way): %.1f us" % result["c1_floor_us"])
+        fused = [e for e in per_op if e["config"] == "C1f"]
+        if fused:
+            separate = sum(e["us"] for e in per_op if e["config"] == "C1")
+            result["c1_fused"] = {"us": fused[0]["us"], "us_five_separate_calls": round(separate, 2)}
 
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device=be.device).normal_()

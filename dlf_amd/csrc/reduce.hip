@@ -424,6 +424,88 @@ __global__ __launch_bounds__(kBlock) void reduce_cols(
 }
 
 // --------------------------------------------------------------------------
+// The classification head in one read: per row of logits its sum, maximum, first arg-maximum,
+// log-sum-exp and `limit` best entries, each exactly what the separate reduce / arg_reduce /
+// top_k call gives (the same reducers; the same order among the best: larger value first,
+// -0.0 and +0.0 one value, NaNs by their bit pattern, lower index first among equals).
+// One wavefront holds one row (element i * 64 + lane is item i of the lane).
+template <int ITEMS>
+__global__ __launch_bounds__(kWave) void logits_head_rows(
+    const float* __restrict__ x, int64_t row_stride, int64_t m, int64_t n, float* __restrict__ sum_out,
+    float* __restrict__ max_out, int32_t* __restrict__ argmax_out, float* __restrict__ lse_out, int limit,
+    float* __restrict__ best_out, int32_t* __restrict__ best_idx) {
+    using Sum = ValueReducer<float, kAdd, kMapId>;
+    using Max = ValueReducer<float, kMax, kMapId>;
+    using Lse = ValueReducer<float, kAdd, kMapExp>;
+    using Arg = ArgReducer<float, true, int32_t>;
+    const int64_t row = blockIdx.x;
+    const int lane = lane_id();
+    const float* xr = x + row * row_stride;
+    const uint32_t n32 = static_cast<uint32_t>(n);
+    float v[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        const uint32_t e = static_cast<uint32_t>(i * kWave + lane);
+        v[i] = xr[e < n32 ? e : 0u];                         // (past the row: its first element again, never used)
+    }
+    Sum::acc_t a_sum = Sum::identity();
+    Max::acc_t a_max = Max::identity();
+    Lse::acc_t a_lse = Lse::identity();
+    Arg::acc_t a_arg = Arg::identity();
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        const uint32_t e = static_cast<uint32_t>(i * kWave + lane);
+        if (e < n32) {
+            a_sum = Sum::join(a_sum, Sum::map(v[i], e, 0));
+            a_max = Max::join(a_max, Max::map(v[i], e, 0));
+            if (lse_out) a_lse = Lse::join(a_lse, Lse::map(v[i], e, 0));
+            a_arg = Arg::join(a_arg, Arg::map(v[i], e, 0));
+        }
+    }
+    a_sum = wave_reduce(a_sum, [](Sum::acc_t a, Sum::acc_t b) { return Sum::join(a, b); });
+    a_max = wave_reduce(a_max, [](Max::acc_t a, Max::acc_t b) { return Max::join(a, b); });
+    if (lse_out) a_lse = wave_reduce(a_lse, [](Lse::acc_t a, Lse::acc_t b) { return Lse::join(a, b); });
+    a_arg = wave_reduce(a_arg, [](Arg::acc_t a, Arg::acc_t b) { return Arg::join(a, b); });
+    if (lane == 0) {
+        if (sum_out) sum_out[row] = Sum::finish(a_sum, n, kFinalId);
+        if (max_out) max_out[row] = Max::finish(a_max, n, kFinalId);
+        if (lse_out) lse_out[row] = Lse::finish(a_lse, n, kFinalLog);
+        if (argmax_out) argmax_out[row] = Arg::finish(a_arg, n, kFinalId);
+    }
+    if (limit <= 0) return;
+
+    // ---- the best `limit` entries: `limit` times the best entry that comes after the one taken
+    // last, entries ordered by image (larger first), then by lower index
+    uint32_t ord[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        uint32_t bits = bit_cast<uint32_t>(v[i]);
+        if ((bits << 1) == 0u) bits = 0u;                    // -0.0 and +0.0 are one value
+        ord[i] = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+    }
+    struct Entry {
+        uint32_t o, x;
+    };
+    auto beats = [](uint32_t oa, uint32_t xa, uint32_t ob, uint32_t xb) { return oa > ob || (oa == ob && xa < xb); };
+    Entry last = {0xffffffffu, 0u};
+    for (int j = 0; j < limit; ++j) {
+        Entry mine = {0u, 0xffffffffu};
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const uint32_t e = static_cast<uint32_t>(i * kWave + lane);
+            const bool after = j == 0 || beats(last.o, last.x, ord[i], e);       // not taken yet
+            if (e < n32 && after && beats(ord[i], e, mine.o, mine.x)) mine = {ord[i], e};
+        }
+        const Entry top = wave_reduce(mine, [beats](Entry a, Entry b) { return beats(b.o, b.x, a.o, a.x) ? b : a; });
+        if (lane == 0) {
+            if (best_out) best_out[row * limit + j] = xr[top.x];                 // the element itself (a zero keeps its sign)
+            if (best_idx) best_idx[row * limit + j] = static_cast<int32_t>(top.x);
+        }
+        last = top;
+    }
+}
+
+// --------------------------------------------------------------------------
 // Host-side planning.
 
 struct ReducePlan {
@@ -801,4 +883,29 @@ extern "C" int dlfx_count(dlfx_stream_t stream, int dtype, int64_t m, int64_t n,
     if (dtype == DLFX_C64) return count_as(Cx<float>());
     if (dtype == DLFX_C128) return count_as(Cx<double>());
     return dispatch_dtype_half(dtype, count_as);
+}
+
+extern "C" int dlfx_logits_head(dlfx_stream_t stream, int dtype, int64_t m, int64_t n,
+                                const void* x, int64_t x_offset, int64_t row_stride,
+                                void* sum, void* max, int32_t* argmax, void* log_sum_exp,
+                                int64_t k, void* best_values, int32_t* best_indices) {
+    if (!x || m <= 0 || n <= 0 || k < 0 || row_stride < n) return DLFX_ERR_INVALID_ARGUMENT;
+    if (dtype != DLFX_F32) return DLFX_ERR_UNSUPPORTED_DTYPE;
+    if (n > DLFX_LOGITS_HEAD_MAX_N || k > DLFX_LOGITS_HEAD_MAX_K || k > n || m > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+    if (k > 0 && !best_values && !best_indices) return DLFX_ERR_INVALID_ARGUMENT;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const float* xp = static_cast<const float*>(x) + x_offset;
+    const dim3 grid(static_cast<unsigned>(m)), block(kWave);
+    auto launch = [&](auto items) {
+        constexpr int ITEMS = decltype(items)::value;
+        logits_head_rows<ITEMS><<<grid, block, 0, s>>>(xp, row_stride, m, n, static_cast<float*>(sum), static_cast<float*>(max), argmax,
+                                                        static_cast<float*>(log_sum_exp), static_cast<int>(k),
+                                                        static_cast<float*>(best_values), best_indices);
+    };
+    if (n <= 4 * kWave) launch(std::integral_constant<int, 4>());
+    else if (n <= 8 * kWave) launch(std::integral_constant<int, 8>());
+    else if (n <= 16 * kWave) launch(std::integral_constant<int, 16>());
+    else launch(std::integral_constant<int, 32>());
+    DLFX_CHECK_LAUNCH();
+    return DLFX_OK;
 }

@@ -43,6 +43,10 @@ def _declare(lib):
     lib.dlfx_reduce_static.argtypes = ([c_void_p, c_char_p, c_int, c_int64, c_int64] + view + [c_void_p, c_int64]
                                        + view + [c_void_p, c_int64])
 
+    lib.dlfx_logits_head.restype = c_int
+    lib.dlfx_logits_head.argtypes = [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int64, c_int64,
+                                     c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p]
+
     lib.dlfx_arg_reduce_scratch_bytes.restype = c_size_t
     lib.dlfx_arg_reduce_scratch_bytes.argtypes = [c_int, c_int64, c_int64]
     lib.dlfx_arg_reduce.restype = c_int
@@ -110,7 +114,7 @@ _lib = None
 
 # Every symbol include/dlfx.h declares.
 EXPORTS = ("dlfx_version", "dlfx_status_string", "dlfx_last_hip_error", "dlfx_set_tuning",
-           "dlfx_reduce_scratch_bytes", "dlfx_reduce", "dlfx_reduce_static",
+           "dlfx_reduce_scratch_bytes", "dlfx_reduce", "dlfx_reduce_static", "dlfx_logits_head",
            "dlfx_arg_reduce_scratch_bytes", "dlfx_arg_reduce",
            "dlfx_scan_scratch_bytes", "dlfx_scan",
            "dlfx_sort_scratch_bytes", "dlfx_sort",
@@ -261,6 +265,17 @@ class HipBackend:
                            (name.encode(), dtype, m, n),
                            (xs.rank, _arr(xs.extents), _arr(xs.strides), x.data_ptr(), xs.offset,
                             ys.rank, _arr(ys.extents), _arr(ys.strides), y.data_ptr(), ys.offset), defer, (x, y))
+
+    def logits_head(self, dtype, m, n, x, x_offset, row_stride, sums, maxs, argmaxs, lses, k, best_values, best_indices,
+                    defer=False):
+        """dlfx_logits_head: sum, max, argmax, log-sum-exp and the k best of every row in one launch;
+        any output (a device tensor) may be None."""
+        def ptr(t):
+            return None if t is None else t.data_ptr()
+        return self._issue(self.lib.dlfx_logits_head, "dlfx_logits_head", (dtype, m, n),
+                           (x.data_ptr(), x_offset, row_stride, ptr(sums), ptr(maxs), ptr(argmaxs), ptr(lses), k,
+                            ptr(best_values), ptr(best_indices)), defer,
+                           (x, sums, maxs, argmaxs, lses, best_values, best_indices))
 
     def arg_reduce(self, name, dtype, index_dtype, rows, k, xs, x, ys, y, defer=False):
         sp, sb = self.scratch(self.lib.dlfx_arg_reduce_scratch_bytes(dtype, rows, k))

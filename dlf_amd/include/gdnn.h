@@ -70,6 +70,23 @@ void reduce(const std::string& name, const size_t m, const size_t n,
     ev.done();
 }
 
+// Not in the reference: sum, max, first arg-maximum, log-sum-exp and the k best entries of
+// every row of an [m, n] fp32 matrix in one launch (dlfx_logits_head).  Row r starts at
+// x_offset + r * row_stride; outputs are dense and any may be null.
+inline void logits_head(const size_t m, const size_t n,
+                        const Buffer<float>& x_buffer, const size_t x_offset, const size_t row_stride,
+                        Buffer<float>* sum, Buffer<float>* max, Buffer<int>* argmax, Buffer<float>* log_sum_exp,
+                        const size_t k, Buffer<float>* best_values, Buffer<int>* best_indices,
+                        const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
+    detail::EventScope ev(queue, event);
+    check_status(dlfx_logits_head(queue.stream(), DLFX_F32, m, n, x_buffer.data(), x_offset, row_stride,
+                                  sum ? sum->data() : nullptr, max ? max->data() : nullptr,
+                                  argmax ? argmax->data() : nullptr, log_sum_exp ? log_sum_exp->data() : nullptr, k,
+                                  best_values ? best_values->data() : nullptr, best_indices ? best_indices->data() : nullptr),
+                 "gpgpu::dnn::logits_head");
+    ev.done();
+}
+
 template <typename T>
 void arg_reduce(const std::string& name, const size_t n, const size_t k,
                 const std::vector<size_t>& x_dims, const std::vector<size_t>& x_strides,

@@ -135,6 +135,27 @@ int dlfx_reduce_static(dlfx_stream_t stream, const char* name, int dtype, int64_
                        int y_rank, const int64_t* y_dims, const int64_t* y_strides,
                        void* y, int64_t y_offset);
 
+/* ---------------------------------------------------------------- logits head
+ * No counterpart in the reference: the five calls its classification heads make on one
+ * [m, n] matrix of logits -- reduce_sum, reduce_max, argmax, reduce_log_sum_exp and top_k
+ * (largest, sorted) along the last axis -- in one launch and one read, for callers bound by
+ * launch latency (m * n of a megabyte or so).  Every result equals what the separate call
+ * writes (dlfx_reduce / dlfx_arg_reduce / dlfx_top_k on the same rows): the same fp64
+ * accumulation rounded once, the first maximum, and among the k best larger values first,
+ * -0.0 and +0.0 as one value, lower index first among equals.
+ * x: m rows of n fp32 elements, row r at x + x_offset + r * row_stride (row_stride >= n).
+ * Outputs are dense and any may be NULL: sum, max, log_sum_exp [m] fp32; argmax [m] int32;
+ * best_values [m, k] fp32 and best_indices [m, k] int32 (k == 0: neither is written).
+ * DLFX_F32 only; n <= DLFX_LOGITS_HEAD_MAX_N and k <= DLFX_LOGITS_HEAD_MAX_K (a row lives in
+ * the registers of one wavefront), otherwise DLFX_ERR_TOO_LARGE: use the separate calls.
+ */
+#define DLFX_LOGITS_HEAD_MAX_N 2048
+#define DLFX_LOGITS_HEAD_MAX_K 8
+int dlfx_logits_head(dlfx_stream_t stream, int dtype, int64_t m, int64_t n,
+                     const void* x, int64_t x_offset, int64_t row_stride,
+                     void* sum, void* max, int32_t* argmax, void* log_sum_exp,
+                     int64_t k, void* best_values, int32_t* best_indices);
+
 /* ---------------------------------------------------------------- arg_reduce
  * Replaces gpgpu::dnn::arg_reduce<T> (gdnn.h:138-144; caller
  * reduce_detail.h:134-147).  The reduced axis is the last one of x_dims

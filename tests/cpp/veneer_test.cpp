@@ -426,6 +426,24 @@ static void test_layout_steps_stay_on_the_device() {
 
 // ONNX nodes as the interpreter binds them (predict.h:1078-1201, 1486-1510, 2031-2044):
 // attribute defaults, output shapes and order.
+static void test_logits_head() {
+    // one launch against the five front-end calls on the same logits
+    std::mt19937 rng(11);
+    std::vector<float> v(40 * 1000);
+    for (auto& e : v) e = static_cast<float>(static_cast<int>(rng() % 2001) - 1000) / 64.0f;      // many equal values
+    auto X = dev(Tensor<float>({40, 1000}, v));
+    DevTensor<float> S({40}), M({40}), L({40}), BV({40, 5});
+    DevTensor<int> A({40}), BI({40, 5});
+    gpgpu::dnn::logits_head(40, 1000, X.data(), 0, 1000, &S.data(), &M.data(), &A.data(), &L.data(), 5, &BV.data(), &BI.data());
+    CHECK(M.read() == reduce_max(X, {1}).read());
+    CHECK(A.read() == argmax(X, 1, false).read());
+    CHECK(near(S.read(), reduce_sum(X, {1}).read()));
+    CHECK(near(L.read(), reduce_log_sum_exp(X, {1}).read()));
+    auto r = top_k(X, 5);
+    CHECK(BV.read() == r.first.read());
+    CHECK(BI.read() == r.second.read());
+}
+
 static void test_onnx_nodes() {
     using namespace dlf::predict;
     // PredictTest.cpp:290-319
@@ -600,6 +618,7 @@ int main() {
     test_softmax_scratch_is_its_own_slice();
     test_layout_steps_stay_on_the_device();
     test_onnx_nodes();
+    test_logits_head();
     std::printf("veneer_test: %d checks, %d failed\n", g_checked, g_failed);
     return g_failed ? 1 : 0;
 }
