@@ -435,6 +435,16 @@ int record_hip_error(hipError_t e);
         if (e_ != hipSuccess) return dlfx::record_hip_error(e_); \
     } while (0)
 
+// True when launches into `stream` are being recorded into a graph (or that cannot be told).
+inline bool stream_is_capturing(hipStream_t stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;
+    }
+    return status != hipStreamCaptureStatusNone;
+}
+
 // Common argument validation for a strided view.
 inline bool view_ok(int rank, const int64_t* dims, const int64_t* strides) {
     if (rank < 0 || rank > 64) return false;

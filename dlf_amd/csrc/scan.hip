@@ -707,16 +707,6 @@ bool views_overlap(int rank, const int64_t* dims, const X* x, const int64_t* sx,
     return xb < ye && yb < xe;
 }
 
-// True when launches into `stream` are being recorded into a graph (or that cannot be told).
-bool stream_is_capturing(hipStream_t stream) {
-    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
-        (void)hipGetLastError();
-        return true;
-    }
-    return status != hipStreamCaptureStatusNone;
-}
-
 // A 64-bit value no earlier call of this process has used and, started from the clock and the
 // process, no other process is likely to have left in reused memory; never zero.
 unsigned long long next_nonce() {

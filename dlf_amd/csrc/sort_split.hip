@@ -52,6 +52,9 @@ __device__ unsigned long long g_split_cycles[kPhaseSlots * 16];
 #define SPLIT_PHASE_BEGIN() do { } while (0)
 #endif
 
+#ifndef SPLIT_HIST_BYTES
+#define SPLIT_HIST_BYTES 32
+#endif
 constexpr int kFineBits = 12;
 constexpr int kFine = 1 << kFineBits;                 // fine bins per row
 constexpr int kMaxBuckets = 256;
@@ -153,7 +156,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
 template <typename K>
 __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int64_t n, int64_t chunks_per_row,
                                                                const SplitRow* __restrict__ rows, uint32_t* __restrict__ chunk_fine) {
-    constexpr int U = 32 / sizeof(K);                 // keys in flight per thread
+    constexpr int U = SPLIT_HIST_BYTES / sizeof(K);   // keys per thread and batch
     __shared__ uint32_t hist[kFine];
     for (int i = threadIdx.x; i < kFine; i += kSplitBlock) hist[i] = 0;
     __syncthreads();
@@ -164,32 +167,54 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
     const K base = static_cast<K>(rows[row].base);
     const int64_t lo = c * kChunk;
     const int64_t hi = (lo + kChunk < n) ? lo + kChunk : n;
-    for (int64_t b0 = lo; b0 < hi; b0 += static_cast<int64_t>(kSplitBlock) * U) {
-        const int64_t i0 = b0 + threadIdx.x;
-        if (b0 + static_cast<int64_t>(kSplitBlock) * U <= hi) {
-            K key[U];
+    // batches of 256 x U keys; the next batch's keys are on their way while this one is counted
+    // (no branches in the loads: a key beyond the chunk's end reads the chunk's first key and is never counted)
+    constexpr int64_t BATCH = static_cast<int64_t>(kSplitBlock) * U;
+    // (whole batches of a contiguous, aligned row move as 16-byte accesses: which thread counts
+    // which key does not matter here)
+    constexpr int VK = 16 / sizeof(K);
+    using VecK = Vec<K, VK>;
+    const bool vectors = io.sx == 1 && reinterpret_cast<uintptr_t>(xrow + lo) % 16 == 0;
+    auto load_batch = [&](int64_t b0, K (&key)[U]) __attribute__((always_inline)) {
+        if (vectors && b0 + BATCH <= hi) {
+            const VecK* src = reinterpret_cast<const VecK*>(xrow + b0);
 #pragma unroll
-            for (int u = 0; u < U; ++u) key[u] = xrow[(i0 + static_cast<int64_t>(u) * kSplitBlock) * io.sx];
-            uint32_t f[U];
+            for (int v = 0; v < U / VK; ++v) {
+                const VecK a = src[threadIdx.x + v * kSplitBlock];
 #pragma unroll
-            for (int u = 0; u < U; ++u) f[u] = fine_bin(key_of_element<K>(io, key[u]), base, shift);
-            // a wave whose keys all share one fine bin (narrow ranges, few distinct values) adds once
-            const uint32_t f0 = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(f[0])));
-            bool same = true;
-#pragma unroll
-            for (int u = 0; u < U; ++u) same = same && f[u] == f0;
-            if (__ballot(!same) == 0ull) {
-                if (lane_id() == 0) atomicAdd(&hist[f0], static_cast<uint32_t>(U * kWave));
-            } else {
-#pragma unroll
-                for (int u = 0; u < U; ++u) atomicAdd(&hist[f[u]], 1u);
+                for (int e = 0; e < VK; ++e) key[v * VK + e] = a.v[e];
             }
-        } else {
-            for (int u = 0; u < U; ++u) {
-                const int64_t i = i0 + static_cast<int64_t>(u) * kSplitBlock;
-                if (i < hi) atomicAdd(&hist[fine_bin(key_of_element<K>(io, xrow[i * io.sx]), base, shift)], 1u);
-            }
+            return;
         }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t i = b0 + threadIdx.x + static_cast<int64_t>(u) * kSplitBlock;
+            key[u] = xrow[(i < hi ? i : lo) * io.sx];
+        }
+    };
+    K key[U];
+    load_batch(lo, key);
+    for (int64_t b0 = lo; b0 < hi; b0 += BATCH) {
+        K ahead[U];
+        if (b0 + BATCH < hi) load_batch(b0 + BATCH, ahead);
+        const bool full = b0 + BATCH <= hi;
+        uint32_t f[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) f[u] = fine_bin(key_of_element<K>(io, key[u]), base, shift);
+        // a wave whose keys all share one fine bin (narrow ranges, few distinct values) adds once
+        const uint32_t f0 = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(f[0])));
+        bool same = full;
+#pragma unroll
+        for (int u = 0; u < U; ++u) same = same && f[u] == f0;
+        if (__ballot(!same) == 0ull) {
+            if (lane_id() == 0) atomicAdd(&hist[f0], static_cast<uint32_t>(U * kWave));
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (full || b0 + threadIdx.x + static_cast<int64_t>(u) * kSplitBlock < hi) atomicAdd(&hist[f[u]], 1u);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) key[u] = ahead[u];
     }
     __syncthreads();
     uint32_t* g = chunk_fine + static_cast<int64_t>(blockIdx.x) * (kFine / 2);

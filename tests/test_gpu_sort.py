@@ -257,6 +257,26 @@ def test_buckets_ranked_by_comparison_or_by_digit_passes(hip_backend, dtype, n):
         assert np.all(Id[:, 1:][same] > Id[:, :-1][same]), limit
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_rows_left_to_the_digit_passes_beside_rows_on_the_bucket_route(hip_backend, dtype):
+    """Rows the bucket route does not take (one value repeated, a handful of values: a fine bin
+    larger than a workgroup holds) are sorted by the digit passes in the same call that sends
+    its other rows through the bucket route; several calls in a row over one scratch buffer."""
+    n = 70000
+    x = (full_range_i64(330, 9 * n).reshape(9, n) >> (40 if np.dtype(dtype).itemsize == 8 else 36)).astype(dtype)
+    x[1, :] = 7                                   # one value
+    x[4, :] = x[4, :] % 5                         # five values
+    x[6, : n // 2] = -3                           # half the row one value
+    Xh = Tensor.from_numpy(hip_backend, x)
+    order = np.argsort(x, axis=-1, kind="stable")
+    for _ in range(2):
+        Yh, Ih = F.argsort(Xh, -1, False, with_values=True)
+        Sh = F.sort(Xh, -1, True)
+        assert np.array_equal(Ih.numpy(), order)
+        assert np.array_equal(Yh.numpy(), np.take_along_axis(x, order, -1))
+        assert np.array_equal(Sh.numpy(), np.sort(x, axis=-1)[:, ::-1])
+
+
 @pytest.mark.parametrize("dtype", [np.int64, np.float64])
 @pytest.mark.parametrize("n", [100, 700, 2048, 4096])
 def test_wide_keys_in_short_rows_settle_on_their_leading_digits_or_run_every_digit(hip_backend, dtype, n):
