@@ -62,6 +62,21 @@ constexpr int kSplitBlock = 256;
 constexpr int kSplitItems = 16;                       // keys per thread of a split_pass tile
 constexpr int kSplitTile = kSplitBlock * kSplitItems;
 constexpr int kChunk = 8 * kSplitTile;                // keys one split_pass workgroup takes (32768)
+// Threads of a split_pass workgroup (16 keys each make its tile): 256, 512 or 1024.  A tile leaves
+// as one run per bucket, so its keys spread over the row's buckets decide how long the runs
+// are; short runs (128 bytes for 8-byte keys in 256 buckets) cost write bandwidth, larger tiles
+// cost LDS and occupancy.  Measured on [256, 2^20] int64: 1476 / 1235 / 1044 us (keys),
+// 2197 / 1698 us (pairs: 1024 threads do not fit LDS); on [1024, 65536] fp32 (32 buckets):
+// 118 / 118 / 157 us (keys), 193 / 178 / 203 us (pairs).
+template <typename K, bool PAIRS>
+constexpr int kPassBlockMax = (sizeof(K) == 8 && !PAIRS) ? 1024 : 512;
+template <typename K, bool PAIRS>
+int pass_block(int64_t n, int cap) {
+    const int64_t buckets = ceil_div(n * 5, static_cast<int64_t>(cap) * 4);       // buckets fill to about 4/5
+    int block = 256;
+    while (block < kPassBlockMax<K, PAIRS> && static_cast<int64_t>(block) * kSplitItems * static_cast<int64_t>(sizeof(K)) < 1024 * buckets) block *= 2;
+    return block;
+}
 // split_finish comes in two sizes: eight wavefronts for buckets of up to 5120 keys (rows of up
 // to about 1.2 M keys), four wavefronts for buckets of up to 2560 (rows of up to 131072 keys:
 // more, smaller workgroups on a compute unit hide each other's waits better).
@@ -382,15 +397,15 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
 }
 
 // ------------------------------------------------------------------ 4. one pass: chunk -> buckets
-template <typename K, bool PAIRS>
+template <typename K, bool PAIRS, int BLOCK>
 struct SplitShared {
     uint32_t table[kFine / 4];                 // bucket_of, four fine bins a word
     uint32_t hist[kMaxBuckets];                // keys of the tile per bucket
     uint32_t start[kMaxBuckets];               // where each bucket begins in the tile
     int32_t dst_base[kMaxBuckets];             // row position of a bucket's share of this tile minus start
-    uint32_t scan_tmp[kSplitBlock / kWave];
-    K keys[kSplitTile];
-    uint32_t vals[PAIRS ? kSplitTile : 1];
+    uint32_t scan_tmp[kMaxBuckets / kWave];
+    K keys[BLOCK * kSplitItems];
+    uint32_t vals[PAIRS ? BLOCK * kSplitItems : 1];
 };
 
 // One workgroup per chunk (kChunk keys, tiles of 4096): where the chunk's keys of each bucket
@@ -399,12 +414,13 @@ struct SplitShared {
 // and their slot among the tile's keys of that bucket with one LDS atomic each, the tile is laid
 // out by bucket in LDS and written as runs; once it lies in LDS the registers already receive
 // the next tile's keys.  The order inside a run is whatever the atomics gave.
-template <typename K, bool PAIRS>
-__global__ __launch_bounds__(kSplitBlock) __attribute__((amdgpu_waves_per_eu(4))) void split_pass(PassIo<K> io, int64_t n, int64_t chunks_per_row,
+template <typename K, bool PAIRS, int BLOCK>
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void split_pass(PassIo<K> io, int64_t n, int64_t chunks_per_row,
                                                           const SplitRow* __restrict__ infos, const uint32_t* __restrict__ chunk_base) {
     constexpr int ITEMS = kSplitItems;
-    constexpr int TILE = kSplitTile;
-    __shared__ SplitShared<K, PAIRS> sm;
+    constexpr int TILE = BLOCK * kSplitItems;
+    static_assert(kChunk % TILE == 0, "whole tiles a chunk");
+    __shared__ SplitShared<K, PAIRS, BLOCK> sm;
     const int tid = threadIdx.x;
     const int lane = lane_id();
     const int w = tid / kWave;
@@ -425,16 +441,21 @@ __global__ __launch_bounds__(kSplitBlock) __attribute__((amdgpu_waves_per_eu(4))
         const K* src = xrow + tile_base * io.sx;
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
-            const int e = tid + k * kSplitBlock;
+            const int e = tid + k * BLOCK;
             key[k] = src[static_cast<int64_t>(e < valid ? e : 0) * io.sx];
         }
     };
 
     K key[ITEMS];
     load_tile(chunk_lo, key);
-    reinterpret_cast<uint4*>(sm.table)[tid] = reinterpret_cast<const uint4*>(info.bucket_of)[tid];   // 256 threads x 16 bytes
-    sm.hist[tid] = 0u;
-    uint32_t next = chunk_base[static_cast<int64_t>(blockIdx.x) * kMaxBuckets + tid];   // where this chunk's coming keys of bucket tid go
+    // threads 0 .. 255 each own a bucket (and 16 bytes of the table)
+    const bool owner = tid < kMaxBuckets;
+    uint32_t next = 0;                                 // where this chunk's coming keys of bucket tid go
+    if (owner) {
+        reinterpret_cast<uint4*>(sm.table)[tid] = reinterpret_cast<const uint4*>(info.bucket_of)[tid];
+        sm.hist[tid] = 0u;
+        next = chunk_base[static_cast<int64_t>(blockIdx.x) * kMaxBuckets + tid];
+    }
     __syncthreads();
 
     for (int64_t tile_base = chunk_lo; tile_base < chunk_hi; tile_base += TILE) {
@@ -457,24 +478,29 @@ __global__ __launch_bounds__(kSplitBlock) __attribute__((amdgpu_waves_per_eu(4))
             }
 #pragma unroll
             for (int k = k0; k < k0 + 8; ++k)
-                if (full || tid + k * kSplitBlock < valid) where[k] = (where[k] << 16) | atomicAdd(&sm.hist[where[k]], 1u);
+                if (full || tid + k * BLOCK < valid) where[k] = (where[k] << 16) | atomicAdd(&sm.hist[where[k]], 1u);
         }
         __syncthreads();
         SPLIT_PHASE(1);
 
         // ---- thread b owns bucket b: its place in the tile and in the row
         {
-            const uint32_t count = sm.hist[tid];
-            const uint32_t incl = wave_scan_inclusive(count, 0u, [](uint32_t a, uint32_t b) { return a + b; });
-            if (lane == kWave - 1) sm.scan_tmp[w] = incl;
-            sm.hist[tid] = 0u;                             // for the next tile
+            uint32_t count = 0, incl = 0;
+            if (owner) {
+                count = sm.hist[tid];
+                incl = wave_scan_inclusive(count, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+                if (lane == kWave - 1) sm.scan_tmp[w] = incl;
+                sm.hist[tid] = 0u;                         // for the next tile
+            }
             __syncthreads();
-            uint32_t pre = 0;
-            for (int i = 0; i < w; ++i) pre += sm.scan_tmp[i];
-            const uint32_t start = pre + incl - count;
-            sm.start[tid] = start;
-            sm.dst_base[tid] = static_cast<int32_t>(next) - static_cast<int32_t>(start);
-            next += count;
+            if (owner) {
+                uint32_t pre = 0;
+                for (int i = 0; i < w; ++i) pre += sm.scan_tmp[i];
+                const uint32_t start = pre + incl - count;
+                sm.start[tid] = start;
+                sm.dst_base[tid] = static_cast<int32_t>(next) - static_cast<int32_t>(start);
+                next += count;
+            }
         }
         __syncthreads();
         SPLIT_PHASE(2);
@@ -484,9 +510,9 @@ __global__ __launch_bounds__(kSplitBlock) __attribute__((amdgpu_waves_per_eu(4))
         for (int k = 0; k < ITEMS; ++k) where[k] = sm.start[where[k] >> 16] + (where[k] & 0xffffu);
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
-            if (full || tid + k * kSplitBlock < valid) {
+            if (full || tid + k * BLOCK < valid) {
                 sm.keys[where[k]] = key[k];
-                if constexpr (PAIRS) sm.vals[where[k]] = static_cast<uint32_t>(tile_base) + static_cast<uint32_t>(tid + k * kSplitBlock);
+                if constexpr (PAIRS) sm.vals[where[k]] = static_cast<uint32_t>(tile_base) + static_cast<uint32_t>(tid + k * BLOCK);
             }
         }
         __syncthreads();
@@ -504,24 +530,24 @@ __global__ __launch_bounds__(kSplitBlock) __attribute__((amdgpu_waves_per_eu(4))
                 K out[8];
                 int32_t at[8];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) out[j] = sm.keys[(k0 + j) * kSplitBlock + tid];
+                for (int j = 0; j < 8; ++j) out[j] = sm.keys[(k0 + j) * BLOCK + tid];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const uint32_t f = fine_bin(out[j], base, shift);
                     at[j] = static_cast<int32_t>((sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu);
                 }
 #pragma unroll
-                for (int j = 0; j < 8; ++j) at[j] = sm.dst_base[at[j]] + ((k0 + j) * kSplitBlock + tid);
+                for (int j = 0; j < 8; ++j) at[j] = sm.dst_base[at[j]] + ((k0 + j) * BLOCK + tid);
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
-                    if (full || (k0 + j) * kSplitBlock + tid < valid) dk[at[j]] = out[j];
+                    if (full || (k0 + j) * BLOCK + tid < valid) dk[at[j]] = out[j];
                 if constexpr (PAIRS) {
                     uint32_t pay[8];
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) pay[j] = sm.vals[(k0 + j) * kSplitBlock + tid];
+                    for (int j = 0; j < 8; ++j) pay[j] = sm.vals[(k0 + j) * BLOCK + tid];
 #pragma unroll
                     for (int j = 0; j < 8; ++j)
-                        if (full || (k0 + j) * kSplitBlock + tid < valid) dv[at[j]] = pay[j];
+                        if (full || (k0 + j) * BLOCK + tid < valid) dv[at[j]] = pay[j];
                 }
             }
         }
@@ -1015,7 +1041,10 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         const int64_t finish_room = resident_workgroups(split_finish<K, PAIRS, WAVES>, WAVES * kWave);
         if (finish_room <= 0) return DLFX_ERR_LAUNCH;
         const dim3 fgrid(static_cast<unsigned>(buckets < finish_room ? buckets : finish_room));
-        split_pass<K, PAIRS><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, chunk_base);
+        const int block = pass_block<K, PAIRS>(n, small ? kCapSmall : kCapLarge);
+        if (block == 256) split_pass<K, PAIRS, 256><<<chunks, dim3(256), 0, stream>>>(io, n, l.chunks_per_row, rows, chunk_base);
+        else if (block == 512) split_pass<K, PAIRS, 512><<<chunks, dim3(512), 0, stream>>>(io, n, l.chunks_per_row, rows, chunk_base);
+        else if constexpr (kPassBlockMax<K, PAIRS> >= 1024) split_pass<K, PAIRS, 1024><<<chunks, dim3(1024), 0, stream>>>(io, n, l.chunks_per_row, rows, chunk_base);
         DLFX_CHECK_LAUNCH();
         split_finish<K, PAIRS, WAVES><<<fgrid, dim3(WAVES * kWave), 0, stream>>>(io, n, limit, counters, list, crowded);
         DLFX_CHECK_LAUNCH();
