@@ -1,7 +1,7 @@
 // The bucket route of sort / argsort for rows longer than one workgroup holds (gfx950).
 //
 // A row is cut by value into at most 256 buckets of at most 5120 keys (rows of up to 131072 keys:
-// 2560), and every bucket is then sorted on chip, so the keys cross HBM four times (plus one read
+// 2560; rows longer than 1.1 M keys: 10240), and every bucket is then sorted on chip, so the keys cross HBM four times (plus one read
 // for the histogram) however wide they are:
 //   1. split_sample     1024 keys of every row, from 256 evenly spaced places, give the range of
 //                       its keys (a few stray keys at either end left aside); 4096 "fine bins"
@@ -77,14 +77,23 @@ int pass_block(int64_t n, int cap) {
     while (block < kPassBlockMax<K, PAIRS> && static_cast<int64_t>(block) * kSplitItems * static_cast<int64_t>(sizeof(K)) < 1024 * buckets) block *= 2;
     return block;
 }
-// split_finish comes in two sizes: eight wavefronts for buckets of up to 5120 keys (rows of up
-// to about 1.2 M keys), four wavefronts for buckets of up to 2560 (rows of up to 131072 keys:
-// more, smaller workgroups on a compute unit hide each other's waits better).
+// split_finish comes in three sizes: four wavefronts for buckets of up to 2560 keys (rows of up
+// to 131072 keys: more, smaller workgroups on a compute unit hide each other's waits better),
+// eight for buckets of up to 5120 (rows of up to 1.1 M keys), sixteen for buckets of up to 10240
+// (rows of up to about 2.4 M keys; measured at 2^20 int64 keys: the scatter pass gains from the
+// longer runs, 1049 -> 973 us, but the finish loses more, 1413 -> 1577 us, so the size is kept
+// for rows the eight-wavefront size cannot take).
 constexpr int kFinishItems = 10;
 constexpr int finish_cap(int waves) { return waves * kWave * kFinishItems; }      // keys a bucket may hold
 constexpr int finish_bins(int waves) { return waves * 1024; }                     // counting bins, two 16-bit counters a word
-constexpr int kCapLarge = finish_cap(8), kCapSmall = finish_cap(4);
+constexpr int kCapHuge = finish_cap(16), kCapLarge = finish_cap(8), kCapSmall = finish_cap(4);
 constexpr int64_t kSmallCapRows = 131072;             // longest row that takes the small size
+#ifndef SPLIT_HUGE_FROM
+#define SPLIT_HUGE_FROM 1100000
+#endif
+constexpr int64_t kLargeCapRows = SPLIT_HUGE_FROM;    // longest row that takes the eight-wavefront size
+// Wavefronts of the finishing workgroup for rows of n keys, and what a bucket may hold then.
+inline int finish_waves(int64_t n) { return n <= kSmallCapRows ? 4 : n <= kLargeCapRows ? 8 : 16; }
 constexpr int kNear = 2;                              // entries of a bin compared without a loop
 
 // What split_sample and split_plan decide for a row.
@@ -561,7 +570,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
 // working it out again from the key when the entry is ranked; 8-byte keys with indices have no
 // room for that with two workgroups on a compute unit.
 template <typename K, bool PAIRS, int WAVES>
-constexpr bool kKeepBins = !(PAIRS && sizeof(K) == 8 && WAVES == 8);
+constexpr bool kKeepBins = !(PAIRS && sizeof(K) == 8 && WAVES >= 8);
 
 template <typename K, bool PAIRS, int WAVES>
 struct FinishShared {
@@ -614,7 +623,7 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
     constexpr int ITEMS = kFinishItems;
     constexpr int T = WAVES * kWave;
     constexpr int kBins = finish_bins(WAVES);
-    constexpr int kBinBits = WAVES == 8 ? 13 : 12;
+    constexpr int kBinBits = WAVES == 16 ? 14 : WAVES == 8 ? 13 : 12;
     static_assert(kBins == 1 << kBinBits, "bins and their bits");
     constexpr int WORDS = kBins / 2 / T;       // counter words a thread scans (8)
     constexpr bool KEEP = kKeepBins<K, PAIRS, WAVES>;
@@ -994,7 +1003,7 @@ SplitLayout split_layout(int64_t m, int64_t n) {
 
 // Whether rows of n keys can take the bucket route at all (each row then decides on the device).
 bool split_route_takes(size_t key_size, int64_t m, int64_t n) {
-    return (key_size == 4 || key_size == 8) && n <= static_cast<int64_t>(kMaxBuckets - 1) * kCapLarge &&
+    return (key_size == 4 || key_size == 8) && n <= static_cast<int64_t>(kMaxBuckets - 1) * kCapHuge &&
            m * kMaxBuckets <= 0x7fffffffLL && m * ceil_div(n, static_cast<int64_t>(kChunk)) <= 0x7fffffffLL;
 }
 
@@ -1029,8 +1038,9 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
     const dim3 chunks(static_cast<unsigned>(m * l.chunks_per_row));
     split_histogram<K><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine);
     DLFX_CHECK_LAUNCH();
-    const bool small = n <= kSmallCapRows;
-    split_plan<<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(n, static_cast<uint32_t>(small ? kCapSmall : kCapLarge), l.chunks_per_row, fine, rows, counters, list, chunk_base);
+    const int waves = finish_waves(n);
+    const int cap = finish_cap(waves);
+    split_plan<<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(n, static_cast<uint32_t>(cap), l.chunks_per_row, fine, rows, counters, list, chunk_base);
     DLFX_CHECK_LAUNCH();
     // split_finish: as many workgroups as the device holds at once, each walking its share of the buckets
     const int64_t buckets = m * kMaxBuckets;
@@ -1041,7 +1051,7 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         const int64_t finish_room = resident_workgroups(split_finish<K, PAIRS, WAVES>, WAVES * kWave);
         if (finish_room <= 0) return DLFX_ERR_LAUNCH;
         const dim3 fgrid(static_cast<unsigned>(buckets < finish_room ? buckets : finish_room));
-        const int block = pass_block<K, PAIRS>(n, small ? kCapSmall : kCapLarge);
+        const int block = pass_block<K, PAIRS>(n, cap);
         if (block == 256) split_pass<K, PAIRS, 256><<<chunks, dim3(256), 0, stream>>>(io, n, l.chunks_per_row, rows, chunk_base);
         else if (block == 512) split_pass<K, PAIRS, 512><<<chunks, dim3(512), 0, stream>>>(io, n, l.chunks_per_row, rows, chunk_base);
         else if constexpr (kPassBlockMax<K, PAIRS> >= 1024) split_pass<K, PAIRS, 1024><<<chunks, dim3(1024), 0, stream>>>(io, n, l.chunks_per_row, rows, chunk_base);
@@ -1052,10 +1062,11 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
     };
+    using Huge = std::integral_constant<int, 16>;
     using Large = std::integral_constant<int, 8>;
     using Small = std::integral_constant<int, 4>;
-    if (pairs) return small ? launch(std::true_type(), Small()) : launch(std::true_type(), Large());
-    return small ? launch(std::false_type(), Small()) : launch(std::false_type(), Large());
+    if (pairs) return waves == 4 ? launch(std::true_type(), Small()) : waves == 8 ? launch(std::true_type(), Large()) : launch(std::true_type(), Huge());
+    return waves == 4 ? launch(std::false_type(), Small()) : waves == 8 ? launch(std::false_type(), Large()) : launch(std::false_type(), Huge());
 }
 
 template int run_split<uint32_t>(hipStream_t, const PassIo<uint32_t>&, bool, int64_t, int64_t, void*, int, int, const uint32_t**,

@@ -257,6 +257,21 @@ def test_buckets_ranked_by_comparison_or_by_digit_passes(hip_backend, dtype, n):
         assert np.all(Id[:, 1:][same] > Id[:, :-1][same]), limit
 
 
+@pytest.mark.parametrize("dtype", [np.int64, np.float32])
+def test_rows_beyond_a_million_keys_take_the_largest_buckets(hip_backend, dtype):
+    """Rows longer than 1.1 M keys are cut into buckets of up to 10240 keys, finished by workgroups
+    of sixteen wavefronts (up to about 2.4 M keys a row; longer rows keep the digit passes)."""
+    for n in (1_500_000, 2_700_001):
+        raw = full_range_i64(340 + n % 7, 2 * n).reshape(2, n)
+        x = raw.astype(dtype) if np.dtype(dtype).kind == "i" else (raw >> 40).astype(np.float32) / np.float32(64.0)
+        Xh = Tensor.from_numpy(hip_backend, x)
+        order = np.argsort(x, axis=-1, kind="stable")
+        Yh, Ih = F.argsort(Xh, -1, False, with_values=True)
+        assert np.array_equal(Ih.numpy(), order)
+        assert np.array_equal(Yh.numpy(), np.take_along_axis(x, order, -1))
+        assert np.array_equal(F.sort(Xh, -1, True).numpy(), np.sort(x, axis=-1)[:, ::-1])
+
+
 @pytest.mark.parametrize("dtype", [np.int32, np.int64])
 def test_rows_left_to_the_digit_passes_beside_rows_on_the_bucket_route(hip_backend, dtype):
     """Rows the bucket route does not take (one value repeated, a handful of values: a fine bin
