@@ -74,7 +74,8 @@ template <typename K, bool PAIRS>
 int pass_block(int64_t n, int cap) {
     const int64_t buckets = ceil_div(n * 5, static_cast<int64_t>(cap) * 4);       // buckets fill to about 4/5
     int block = 256;
-    while (block < kPassBlockMax<K, PAIRS> && static_cast<int64_t>(block) * kSplitItems * static_cast<int64_t>(sizeof(K)) < 1024 * buckets) block *= 2;
+    const int64_t run_bytes = 1024;                        // what a tile should write per bucket at least
+    while (block < kPassBlockMax<K, PAIRS> && static_cast<int64_t>(block) * kSplitItems * static_cast<int64_t>(sizeof(K)) < run_bytes * buckets) block *= 2;
     return block;
 }
 // split_finish comes in three sizes: four wavefronts for buckets of up to 2560 keys (rows of up
@@ -92,30 +93,73 @@ constexpr int64_t kSmallCapRows = 131072;             // longest row that takes 
 #define SPLIT_HUGE_FROM 1100000
 #endif
 constexpr int64_t kLargeCapRows = SPLIT_HUGE_FROM;    // longest row that takes the eight-wavefront size
+constexpr int64_t kLargeCapFloatRows = 700000;        // ... of floats, which seldom fill their fine bins as evenly as integers do
 // Wavefronts of the finishing workgroup for rows of n keys, and what a bucket may hold then.
-inline int finish_waves(int64_t n) { return n <= kSmallCapRows ? 4 : n <= kLargeCapRows ? 8 : 16; }
+inline int finish_waves(int64_t n, bool floats) {
+    return n <= kSmallCapRows ? 4 : n <= (floats ? kLargeCapFloatRows : kLargeCapRows) ? 8 : 16;
+}
 constexpr int kNear = 2;                              // entries of a bin compared without a loop
 
 // What split_sample and split_plan decide for a row.
 struct alignas(16) SplitRow {
     uint32_t route;                        // 1: this row takes the bucket route, 0: the digit passes
-    uint32_t shift;                        // fine bin of a key: min((key - base) >> shift, kFine - 1), 0 below base
-    unsigned long long base;
+    uint32_t shift;                        // by key image: fine bin = min((key - base) >> shift, kFine - 1), 0 below base
+    unsigned long long base;               // keys below share the first fine bin (both ways)
     uint32_t n_buckets;
-    uint32_t reserved[3];
+    uint32_t by_value;                     // 1 (floats only): fine bin = (value - lo) * scale between base and top
+    unsigned long long top;                // by value: keys from here up share the last fine bin
+    unsigned long long lo_bits, scale_bits;    // by value: lo and scale as a float's / double's bits
     uint32_t begin[kMaxBuckets + 4];       // first position of each bucket in the row; begin[n_buckets] = n
     uint8_t bucket_of[kFine];              // fine bin -> bucket (16-byte aligned: tiles load it as vectors)
 };
 static_assert(offsetof(SplitRow, bucket_of) % 16 == 0 && sizeof(SplitRow) % 16 == 0, "vector loads of the table");
 
-// Monotone in the key whatever the key: keys outside the sampled range land in the first or
-// last bins, so nothing has to be verified afterwards - a poor sample costs balance, not order.
+template <typename K> struct FloatOf;
+template <> struct FloatOf<uint32_t> { using type = float; };
+template <> struct FloatOf<uint64_t> { using type = double; };
+
+// The fine bin of a key, monotone in the key whatever the key: keys outside the sampled range
+// land in the first or last bins, so nothing has to be verified afterwards - a poor sample costs
+// balance, not order.  Two ways to spread the range over the bins: evenly over the key images
+// (integers; floats whose magnitudes spread over many binades - an image is about the
+// logarithm of its float), or evenly over the values (floats that spread evenly as numbers:
+// uniform or bell-shaped data, data on both sides of zero, where most images would crowd into
+// the few bins of the largest binades).  split_sample picks per row.
 template <typename K>
-__device__ __forceinline__ uint32_t fine_bin(K key, K base, uint32_t shift) {
-    const K off = static_cast<K>(key - base) >> shift;
-    const uint32_t f = off < static_cast<K>(kFine - 1) ? static_cast<uint32_t>(off) : static_cast<uint32_t>(kFine - 1);
-    return key < base ? 0u : f;
-}
+struct FineMap {
+    using F = typename FloatOf<K>::type;
+    K base, top;
+    F lo, scale;
+    uint32_t shift, by_value;
+    int descending;
+    __device__ FineMap(const SplitRow& r, int desc)
+        : base(static_cast<K>(r.base)), top(static_cast<K>(r.top)), lo(bit_cast<F>(static_cast<K>(r.lo_bits))),
+          scale(bit_cast<F>(static_cast<K>(r.scale_bits))), shift(r.shift), by_value(r.by_value), descending(desc) {}
+    // the number a float key stands for, increasing with the key (so negated for descending sorts)
+    __device__ __forceinline__ static F value_of(K key, int desc) {
+        const F x = bit_cast<F>(decode_key<K>(key, kKeyFloat, desc));
+        return desc ? -x : x;
+    }
+    // BY_VALUE must equal by_value: the kernels branch once per workgroup, not once per key
+    template <bool BY_VALUE>
+    __device__ __forceinline__ uint32_t bin(K key) const {
+        uint32_t f;
+        if constexpr (BY_VALUE) {
+            // between base and top the value is finite; subtraction, scaling and truncation are
+            // all monotone, so the bin never decreases as the key grows
+            const F t = (value_of(key, descending) - lo) * scale;
+            int b = static_cast<int>(t);
+            b = b < 0 ? 0 : b;
+            f = b < kFine - 1 ? static_cast<uint32_t>(b) : static_cast<uint32_t>(kFine - 1);
+            f = key >= top ? static_cast<uint32_t>(kFine - 1) : f;
+        } else {
+            const K off = static_cast<K>(key - base) >> shift;
+            f = off < static_cast<K>(kFine - 1) ? static_cast<uint32_t>(off) : static_cast<uint32_t>(kFine - 1);
+        }
+        return key < base ? 0u : f;
+    }
+    __device__ __forceinline__ uint32_t operator()(K key) const { return by_value ? bin<true>(key) : bin<false>(key); }
+};
 
 template <typename T, typename Join>
 __device__ __forceinline__ T block_reduce(T v, Join join, T* lds, int waves) {
@@ -129,8 +173,10 @@ __device__ __forceinline__ T block_reduce(T v, Join join, T* lds, int waves) {
 }
 
 // ------------------------------------------------------------------ 1. the range of a row's keys
-template <typename K>
-__global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_t n, SplitRow* __restrict__ rows, uint32_t* __restrict__ counters) {
+// VAL: float rows long enough for the value map to matter (the host knows); without it the row
+// is spread by key image and the kernels carry no code for anything else.
+template <typename K, bool VAL>
+__global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_t n, uint32_t cap, SplitRow* __restrict__ rows, uint32_t* __restrict__ counters) {
     __shared__ K red[kSplitBlock / kWave];
     const int64_t row = blockIdx.x;
     if (row == 0 && threadIdx.x < 4) counters[threadIdx.x] = 0u;      // what the later launches of this sort count up from
@@ -159,16 +205,63 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
     }
     lo = block_reduce(lo, [](K a, K b) { return a < b ? a : b; }, red, kSplitBlock / kWave);
     hi = block_reduce(hi, [](K a, K b) { return a > b ? a : b; }, red, kSplitBlock / kWave);
-    if (threadIdx.x == 0) {
-        // that range takes the middle half of the fine bins; a quarter on either side is left for
-        // keys outside it (beyond those, keys share the first or last bin)
+    // that range takes the middle half of the fine bins; a quarter on either side is left for
+    // keys outside it (beyond those, keys share the first or last bin)
+    SplitRow map;
+    {
         const unsigned long long range = static_cast<unsigned long long>(static_cast<K>(hi - lo));
         const int width = range ? 64 - __builtin_clzll(range) : 0;
-        const uint32_t shift = width > kFineBits - 1 ? static_cast<uint32_t>(width - (kFineBits - 1)) : 0u;
-        const K margin = static_cast<K>(K(kFine / 4) << shift);
-        rows[row].route = 0u;
-        rows[row].shift = shift;
-        rows[row].base = static_cast<unsigned long long>(lo > margin ? static_cast<K>(lo - margin) : K(0));
+        map.shift = width > kFineBits - 1 ? static_cast<uint32_t>(width - (kFineBits - 1)) : 0u;
+        const K margin = static_cast<K>(K(kFine / 4) << map.shift);
+        map.base = static_cast<unsigned long long>(lo > margin ? static_cast<K>(lo - margin) : K(0));
+        map.by_value = 0u;
+        map.top = 0ull;
+        map.lo_bits = map.scale_bits = 0ull;
+    }
+    if constexpr (VAL) {
+        // the same range spread evenly over the values instead - taken when, by key image, the
+        // sample's fullest cell of 16 bins promises a fine bin of more than a quarter of what a
+        // bucket holds (the row might not fit the route, or only in lopsided buckets) and the
+        // values crowd their fullest cell less; otherwise the cheaper image arithmetic stays
+        using F = typename FloatOf<K>::type;
+        const F xl = FineMap<K>::value_of(lo, io.descending), xh = FineMap<K>::value_of(hi, io.descending);
+        const F w = xh - xl;
+        const F first = xl - w * F(0.5), last = xh + w * F(0.5);
+        if (w > F(0) && w - w == F(0) && first - first == F(0) && last - last == F(0)) {       // all finite
+            SplitRow by_value = map;
+            by_value.by_value = 1u;
+            by_value.lo_bits = static_cast<unsigned long long>(bit_cast<K>(first));
+            by_value.scale_bits = static_cast<unsigned long long>(bit_cast<K>(static_cast<F>(kFine) / (w * F(2))));
+            // the keys of `first` and `last` (the element value is the negated one when descending)
+            by_value.base = static_cast<unsigned long long>(key_of_element<K>(io, bit_cast<K>(io.descending ? -first : first)));
+            by_value.top = static_cast<unsigned long long>(key_of_element<K>(io, bit_cast<K>(io.descending ? -last : last)));
+            static_assert(kFine / 16 == kSplitBlock, "a thread per cell");
+            __shared__ uint32_t cells[2][kFine / 16];
+            for (int i = threadIdx.x; i < 2 * (kFine / 16); i += kSplitBlock) (&cells[0][0])[i] = 0u;
+            __syncthreads();
+            const FineMap<K> by_image_map(map, io.descending), by_value_map(by_value, io.descending);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                atomicAdd(&cells[0][by_image_map(key[u]) >> 4], 1u);
+                atomicAdd(&cells[1][by_value_map(key[u]) >> 4], 1u);
+            }
+            __syncthreads();
+            uint32_t worst_image = cells[0][threadIdx.x], worst_value = cells[1][threadIdx.x];      // kFine / 16 == kSplitBlock
+            __shared__ uint32_t red32[kSplitBlock / kWave];
+            worst_image = block_reduce(worst_image, [](uint32_t a, uint32_t b) { return a > b ? a : b; }, red32, kSplitBlock / kWave);
+            worst_value = block_reduce(worst_value, [](uint32_t a, uint32_t b) { return a > b ? a : b; }, red32, kSplitBlock / kWave);
+            if (worst_value < worst_image && static_cast<unsigned long long>(worst_image) * static_cast<unsigned long long>(n) > static_cast<unsigned long long>(cap) * kFine) map = by_value;
+        }
+    }
+    if (threadIdx.x == 0) {
+        SplitRow& out = rows[row];
+        out.route = 0u;
+        out.shift = map.shift;
+        out.base = map.base;
+        out.by_value = map.by_value;
+        out.top = map.top;
+        out.lo_bits = map.lo_bits;
+        out.scale_bits = map.scale_bits;
     }
 }
 
@@ -177,7 +270,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
 // counts a word (a count is at most kChunk).  split_plan adds the chunks up for the row's
 // histogram and turns each chunk's into its keys per bucket, so that split_pass needs no
 // communication between workgroups.
-template <typename K>
+template <typename K, bool VAL>
 __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int64_t n, int64_t chunks_per_row,
                                                                const SplitRow* __restrict__ rows, uint32_t* __restrict__ chunk_fine) {
     constexpr int U = SPLIT_HIST_BYTES / sizeof(K);   // keys per thread and batch
@@ -187,8 +280,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
     const int64_t row = blockIdx.x / chunks_per_row;
     const int64_t c = blockIdx.x - row * chunks_per_row;
     const K* xrow = io.x + io.xmap.at(row);
-    const uint32_t shift = rows[row].shift;
-    const K base = static_cast<K>(rows[row].base);
+    const FineMap<K> fine_of(rows[row], io.descending);
     const int64_t lo = c * kChunk;
     const int64_t hi = (lo + kChunk < n) ? lo + kChunk : n;
     // batches of 256 x U keys; the next batch's keys are on their way while this one is counted
@@ -216,6 +308,8 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
             key[u] = xrow[(i < hi ? i : lo) * io.sx];
         }
     };
+    auto count_chunk = [&](auto by_value_tag) __attribute__((always_inline)) {
+    constexpr bool BY_VALUE = decltype(by_value_tag)::value;
     K key[U];
     load_batch(lo, key);
     for (int64_t b0 = lo; b0 < hi; b0 += BATCH) {
@@ -224,7 +318,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
         const bool full = b0 + BATCH <= hi;
         uint32_t f[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) f[u] = fine_bin(key_of_element<K>(io, key[u]), base, shift);
+        for (int u = 0; u < U; ++u) f[u] = fine_of.template bin<BY_VALUE>(key_of_element<K>(io, key[u]));
         // a wave whose keys all share one fine bin (narrow ranges, few distinct values) adds once
         const uint32_t f0 = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(f[0])));
         bool same = full;
@@ -240,6 +334,9 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
 #pragma unroll
         for (int u = 0; u < U; ++u) key[u] = ahead[u];
     }
+    };
+    if (VAL && fine_of.by_value) count_chunk(std::integral_constant<bool, VAL>());
+    else count_chunk(std::false_type());
     __syncthreads();
     uint32_t* g = chunk_fine + static_cast<int64_t>(blockIdx.x) * (kFine / 2);
     for (int i = threadIdx.x; i < kFine / 2; i += kSplitBlock) g[i] = hist[2 * i] | (hist[2 * i + 1] << 16);
@@ -423,7 +520,7 @@ struct SplitShared {
 // and their slot among the tile's keys of that bucket with one LDS atomic each, the tile is laid
 // out by bucket in LDS and written as runs; once it lies in LDS the registers already receive
 // the next tile's keys.  The order inside a run is whatever the atomics gave.
-template <typename K, bool PAIRS, int BLOCK>
+template <typename K, bool PAIRS, int BLOCK, bool VAL>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void split_pass(PassIo<K> io, int64_t n, int64_t chunks_per_row,
                                                           const SplitRow* __restrict__ infos, const uint32_t* __restrict__ chunk_base) {
     constexpr int ITEMS = kSplitItems;
@@ -437,8 +534,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
     const int64_t c = blockIdx.x - row * chunks_per_row;
     const SplitRow& info = infos[row];
     if (info.route != 1u) return;
-    const uint32_t shift = info.shift;
-    const K base = static_cast<K>(info.base);
+    const FineMap<K> fine_of(info, io.descending);
     const K* xrow = io.x + io.xmap.at(row);
     const int64_t row_off = row * n;
     const int64_t chunk_lo = c * kChunk;
@@ -467,6 +563,8 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
     }
     __syncthreads();
 
+    auto move_chunk = [&](auto by_value_tag) __attribute__((always_inline)) {
+    constexpr bool BY_VALUE = decltype(by_value_tag)::value;
     for (int64_t tile_base = chunk_lo; tile_base < chunk_hi; tile_base += TILE) {
         const int valid = static_cast<int>((chunk_hi - tile_base < TILE) ? chunk_hi - tile_base : TILE);
         const bool full = valid == TILE;
@@ -482,7 +580,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
         for (int k0 = 0; k0 < ITEMS; k0 += 8) {
 #pragma unroll
             for (int k = k0; k < k0 + 8; ++k) {
-                const uint32_t f = fine_bin(key[k], base, shift);
+                const uint32_t f = fine_of.template bin<BY_VALUE>(key[k]);
                 where[k] = (sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu;
             }
 #pragma unroll
@@ -542,7 +640,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
                 for (int j = 0; j < 8; ++j) out[j] = sm.keys[(k0 + j) * BLOCK + tid];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    const uint32_t f = fine_bin(out[j], base, shift);
+                    const uint32_t f = fine_of.template bin<BY_VALUE>(out[j]);
                     at[j] = static_cast<int32_t>((sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu);
                 }
 #pragma unroll
@@ -563,6 +661,9 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
         SPLIT_PHASE(5);
         __syncthreads();                                   // the tile in LDS has left
     }
+    };
+    if (VAL && fine_of.by_value) move_chunk(std::integral_constant<bool, VAL>());
+    else move_chunk(std::false_type());
 }
 
 // ------------------------------------------------------------------ 5. a bucket, on chip
@@ -1033,13 +1134,17 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
     *route_stride = sizeof(SplitRow);
     (void)poll_limit;            // nothing waits for anything on this route
 
-    split_sample<K><<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(io, n, rows, counters);
+    const int waves = finish_waves(n, io.kind == kKeyFloat);
+    const int cap = finish_cap(waves);
+    // float rows beyond the smallest size may be spread by value (split_sample decides per row)
+    const bool val = io.kind == kKeyFloat && waves > 4;
+    if (val) split_sample<K, true><<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(io, n, static_cast<uint32_t>(cap), rows, counters);
+    else split_sample<K, false><<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(io, n, static_cast<uint32_t>(cap), rows, counters);
     DLFX_CHECK_LAUNCH();
     const dim3 chunks(static_cast<unsigned>(m * l.chunks_per_row));
-    split_histogram<K><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine);
+    if (val) split_histogram<K, true><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine);
+    else split_histogram<K, false><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine);
     DLFX_CHECK_LAUNCH();
-    const int waves = finish_waves(n);
-    const int cap = finish_cap(waves);
     split_plan<<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(n, static_cast<uint32_t>(cap), l.chunks_per_row, fine, rows, counters, list, chunk_base);
     DLFX_CHECK_LAUNCH();
     // split_finish: as many workgroups as the device holds at once, each walking its share of the buckets
@@ -1052,9 +1157,18 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         if (finish_room <= 0) return DLFX_ERR_LAUNCH;
         const dim3 fgrid(static_cast<unsigned>(buckets < finish_room ? buckets : finish_room));
         const int block = pass_block<K, PAIRS>(n, cap);
-        if (block == 256) split_pass<K, PAIRS, 256><<<chunks, dim3(256), 0, stream>>>(io, n, l.chunks_per_row, rows, chunk_base);
-        else if (block == 512) split_pass<K, PAIRS, 512><<<chunks, dim3(512), 0, stream>>>(io, n, l.chunks_per_row, rows, chunk_base);
-        else if constexpr (kPassBlockMax<K, PAIRS> >= 1024) split_pass<K, PAIRS, 1024><<<chunks, dim3(1024), 0, stream>>>(io, n, l.chunks_per_row, rows, chunk_base);
+        auto pass = [&](auto block_tag, auto val_tag) {
+            constexpr int BLOCK = decltype(block_tag)::value;
+            constexpr bool VAL = decltype(val_tag)::value;
+            split_pass<K, PAIRS, BLOCK, VAL><<<chunks, dim3(BLOCK), 0, stream>>>(io, n, l.chunks_per_row, rows, chunk_base);
+        };
+        auto pass_of = [&](auto block_tag) {
+            if (val) pass(block_tag, std::true_type());
+            else pass(block_tag, std::false_type());
+        };
+        if (block == 256) pass_of(std::integral_constant<int, 256>());
+        else if (block == 512) pass_of(std::integral_constant<int, 512>());
+        else if constexpr (kPassBlockMax<K, PAIRS> >= 1024) pass_of(std::integral_constant<int, 1024>());
         DLFX_CHECK_LAUNCH();
         split_finish<K, PAIRS, WAVES><<<fgrid, dim3(WAVES * kWave), 0, stream>>>(io, n, limit, counters, list, crowded);
         DLFX_CHECK_LAUNCH();

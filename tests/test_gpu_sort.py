@@ -257,6 +257,39 @@ def test_buckets_ranked_by_comparison_or_by_digit_passes(hip_backend, dtype, n):
         assert np.all(Id[:, 1:][same] > Id[:, :-1][same]), limit
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n", [70000, 1 << 20])
+def test_float_rows_spread_by_value_or_by_image(hip_backend, dtype, n):
+    """Float rows choose how their range is spread over the fine bins: evenly over the values
+    (bell-shaped data on both sides of zero, uniform data) or over the key images (magnitudes over
+    many binades).  Either way the order is exact, with infinities, NaNs and zeros of both signs
+    in the row, ascending and descending."""
+    bell = normal(350, 2 * n).astype(dtype).reshape(2, n)
+    bell[1] = bell[1] * dtype(1e-3) + dtype(5.0)                       # a narrow bell far from zero
+    decades = np.exp(normal(351, n).astype(np.float64) * 12.0).astype(dtype).reshape(1, n)      # magnitudes over many binades
+    decades[0, ::2] *= dtype(-1.0)
+    mixed = normal(352, n).astype(dtype).reshape(1, n)
+    mixed[0, 5:2000:7] = np.inf
+    mixed[0, 6:2000:7] = -np.inf
+    mixed[0, 7:3000:11] = np.nan
+    mixed[0, 100:200] = 0.0
+    mixed[0, 150:250:2] = -0.0
+    flat = np.full((1, n), dtype(2.5))
+    flat[0, n // 2] = dtype(-1.0)
+    x = np.concatenate([bell, decades, mixed, flat])
+    Xh = Tensor.from_numpy(hip_backend, x)
+    want = np.sort(x, axis=-1)
+    got = F.sort(Xh, -1).numpy()
+    assert np.array_equal(got, want, equal_nan=True)
+    assert np.array_equal(F.sort(Xh, -1, True).numpy(), want[:, ::-1], equal_nan=True)
+    plain = [0, 1, 2, 4]                                                # rows without NaNs: the stable order is numpy's
+    order = np.argsort(x[plain], axis=-1, kind="stable")
+    Ih = F.argsort(Tensor.from_numpy(hip_backend, x[plain]), -1, False)
+    assert np.array_equal(Ih.numpy(), order)
+    Yh, Jh = F.argsort(Xh, -1, True, with_values=True)
+    assert np.array_equal(np.take_along_axis(x, Jh.numpy().astype(np.int64), -1).view(np.uint8), Yh.numpy().view(np.uint8))
+
+
 @pytest.mark.parametrize("dtype", [np.int64, np.float32])
 def test_rows_beyond_a_million_keys_take_the_largest_buckets(hip_backend, dtype):
     """Rows longer than 1.1 M keys are cut into buckets of up to 10240 keys, finished by workgroups
