@@ -458,7 +458,7 @@ def split_kernels(es, pairs, n):
     key = "unsigned int" if es == 4 else "unsigned long"
     waves = 4 if n <= 131072 else 8
     flag = "true" if pairs else "false"
-    return ["split_sample<%s>" % key, "split_histogram<%s>" % key, "split_plan", "split_pass<%s, %s," % (key, flag),
+    return ["split_sample<%s," % key, "split_histogram<%s," % key, "split_plan", "split_pass<%s, %s," % (key, flag),
             "split_finish<%s, %s, %d>" % (key, flag, waves)]
 
 
