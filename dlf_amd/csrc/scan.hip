@@ -543,10 +543,7 @@ __global__ __launch_bounds__(BLOCK) void scan_rows_chained(
 // One lane per row ("column"), four waves along the scanned axis.  Each pass of
 // the loop covers kWaves * chunk positions of the axis: thread (lx, ty) scans
 // positions [s + ty*chunk, s + (ty+1)*chunk) in registers.
-#ifndef DLFX_SCAN_COLS_CHUNK
-#define DLFX_SCAN_COLS_CHUNK 16
-#endif
-constexpr int kColsChunk = DLFX_SCAN_COLS_CHUNK;      // rows of a column a wave scans per round
+constexpr int kColsChunk = 16;      // rows of a column a wave scans per round (4, 8 and 32 measured: slower)
 
 template <typename T, int K, typename X, bool NZ, typename Y>
 __global__ __launch_bounds__(kBlock) void scan_cols(
@@ -565,8 +562,7 @@ __global__ __launch_bounds__(kBlock) void scan_cols(
 
     T carry = Op::identity();
     int buf = 0;
-    const int waves = static_cast<int>(blockDim.x) / kWave;       // 4, or 1 when every column block has a wave of its own
-    const int64_t step = static_cast<int64_t>(waves) * chunk;
+    const int64_t step = static_cast<int64_t>(kWaves) * chunk;
     // the wave's chunk of the next round is on its way while this round is scanned and stored
     auto load_chunk = [&](int64_t s, T* v) __attribute__((always_inline)) {
         const int64_t p0 = s + static_cast<int64_t>(ty) * chunk;
@@ -592,11 +588,9 @@ __global__ __launch_bounds__(kBlock) void scan_cols(
         T all = Op::identity();
 #pragma unroll
         for (int i = 0; i < kWaves; ++i) {
-            if (i < waves) {
-                const T tv = totals[buf][i][lx];
-                if (i < ty) pre = Op::apply(pre, tv);
-                all = Op::apply(all, tv);
-            }
+            const T tv = totals[buf][i][lx];
+            if (i < ty) pre = Op::apply(pre, tv);
+            all = Op::apply(all, tv);
         }
         carry = Op::apply(carry, all);
         if (live) {
@@ -772,15 +766,10 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     const bool short_rows = n <= 64 && m >= 256;
     const bool use_cols = !axis_general && (short_rows || (!axis_unit && m >= 64 && (inner_unit || n < 4096)));
     if (use_cols) {
-#ifdef DLFX_SCAN_COLS_ONE_WAVE
-        const int waves = (ceil_div(m, kWave) >= 1024 && n >= 64) ? 1 : kWaves;
-#else
-        const int waves = kWaves;
-#endif
-        int chunk = static_cast<int>(ceil_div(n, waves) < kColsChunk ? ceil_div(n, waves) : kColsChunk);
+        int chunk = static_cast<int>(ceil_div(n, kWaves) < kColsChunk ? ceil_div(n, kWaves) : kColsChunk);
         const int64_t blocks = ceil_div(m, kWave);
         if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
-        scan_cols<T, K, X, NZ, Y><<<dim3(static_cast<unsigned>(blocks)), dim3(waves * kWave), 0, stream>>>(
+        scan_cols<T, K, X, NZ, Y><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
             x, y, xmap, ymap, sx, sy, m, n, chunk, exclusive);
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;

@@ -52,9 +52,6 @@ __device__ unsigned long long g_split_cycles[kPhaseSlots * 16];
 #define SPLIT_PHASE_BEGIN() do { } while (0)
 #endif
 
-#ifndef SPLIT_HIST_BYTES
-#define SPLIT_HIST_BYTES 32
-#endif
 constexpr int kFineBits = 12;
 constexpr int kFine = 1 << kFineBits;                 // fine bins per row
 constexpr int kMaxBuckets = 256;
@@ -89,10 +86,7 @@ constexpr int finish_cap(int waves) { return waves * kWave * kFinishItems; }    
 constexpr int finish_bins(int waves) { return waves * 1024; }                     // counting bins, two 16-bit counters a word
 constexpr int kCapHuge = finish_cap(16), kCapLarge = finish_cap(8), kCapSmall = finish_cap(4);
 constexpr int64_t kSmallCapRows = 131072;             // longest row that takes the small size
-#ifndef SPLIT_HUGE_FROM
-#define SPLIT_HUGE_FROM 1100000
-#endif
-constexpr int64_t kLargeCapRows = SPLIT_HUGE_FROM;    // longest row that takes the eight-wavefront size
+constexpr int64_t kLargeCapRows = 1100000;            // longest row that takes the eight-wavefront size
 constexpr int64_t kLargeCapFloatRows = 700000;        // ... of floats, which seldom fill their fine bins as evenly as integers do
 // Wavefronts of the finishing workgroup for rows of n keys, and what a bucket may hold then.
 inline int finish_waves(int64_t n, bool floats) {
@@ -273,7 +267,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
 template <typename K, bool VAL>
 __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int64_t n, int64_t chunks_per_row,
                                                                const SplitRow* __restrict__ rows, uint32_t* __restrict__ chunk_fine) {
-    constexpr int U = SPLIT_HIST_BYTES / sizeof(K);   // keys per thread and batch
+    constexpr int U = 32 / sizeof(K);                 // keys per thread and batch (64 bytes measured: no faster)
     __shared__ uint32_t hist[kFine];
     for (int i = threadIdx.x; i < kFine; i += kSplitBlock) hist[i] = 0;
     __syncthreads();
