@@ -349,6 +349,30 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block(
     }
 }
 
+// Second stage for few rows: a workgroup per row, every thread's loads of partials in flight at
+// once (one wave walking 2048 partials of a single row took 10 us, as long as a fiftieth of the
+// first stage over 4 GB).
+template <typename R>
+__global__ __launch_bounds__(kBlock) void reduce_finalize_block(
+    const typename R::acc_t* __restrict__ partial, int64_t n, int64_t parts,
+    typename R::out_t* __restrict__ y, DimMap ymap, int final_op) {
+    using acc_t = typename R::acc_t;
+    const int64_t row = blockIdx.x;
+    const acc_t* p = partial + row * parts;
+    acc_t acc = R::identity();
+    int64_t i = threadIdx.x;
+    for (; i + 7 * kBlock < parts; i += 8 * kBlock) {
+        acc_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = p[i + u * kBlock];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc = R::join(acc, v[u]);
+    }
+    for (; i < parts; i += kBlock) acc = R::join(acc, p[i]);
+    acc = block_reduce<R>(acc);
+    if (threadIdx.x == 0) y[ymap.at(row)] = R::finish(acc, n, final_op);
+}
+
 // Second stage: one wave per row folds that row's `parts` partials.
 template <typename R>
 __global__ __launch_bounds__(kBlock) void reduce_finalize(
@@ -607,8 +631,11 @@ int launch_reduce(hipStream_t stream, const ReducePlan& pl, const typename R::in
             x, pl.kept, pl.red, n, parts, y, pl.ymap, final_op, partial, prm);
     DLFX_CHECK_LAUNCH();
     if (parts > 1) {
-        reduce_finalize<R><<<dim3(static_cast<unsigned>(ceil_div(m, kBlock / kWave))), dim3(kBlock), 0, stream>>>(
-            partial, m, n, parts, y, pl.ymap, final_op);
+        if (m <= 64 && parts >= 256)
+            reduce_finalize_block<R><<<dim3(static_cast<unsigned>(m)), dim3(kBlock), 0, stream>>>(partial, n, parts, y, pl.ymap, final_op);
+        else
+            reduce_finalize<R><<<dim3(static_cast<unsigned>(ceil_div(m, kBlock / kWave))), dim3(kBlock), 0, stream>>>(
+                partial, m, n, parts, y, pl.ymap, final_op);
         DLFX_CHECK_LAUNCH();
     }
     return DLFX_OK;
