@@ -192,7 +192,16 @@ def test_long_rows_cut_into_buckets(hip_backend, dtype, n):
         for j in range(1, group):
             at = np.arange(0, n - group, step) + j
             bits[at] = bits[at - j] ^ randint(307 + j, at.size, 0, 1 << 20).astype(bits.dtype)
-    x = np.stack([wide, lopsided, ties, one_digit, narrow, wide[::-1].copy(), close, few])
+    # rows whose order is not random: sorted, a sawtooth of sorted runs, and one value with a few
+    # strays at both ends (the sample reads evenly spaced places; the strays must not stretch
+    # the range the buckets divide)
+    in_order = np.sort(wide)
+    sawtooth = np.sort(narrow.reshape(-1, 250) if n % 250 == 0 else narrow[: n // 250 * 250].reshape(-1, 250), axis=1).reshape(-1)
+    sawtooth = np.concatenate([sawtooth, narrow[sawtooth.size:]])
+    strays = np.full(n, narrow[0])
+    strays[[1, n // 3, n - 2]] = [wide.min(), wide.max(), wide.min()]
+    strays[n // 2: n // 2 + 300] = narrow[:300]
+    x = np.stack([wide, lopsided, ties, one_digit, narrow, wide[::-1].copy(), close, few, in_order, sawtooth, strays])
     Xh = Tensor.from_numpy(hip_backend, x)
     want = np.sort(x, axis=-1, kind="stable")
     order = np.argsort(x, axis=-1, kind="stable")
