@@ -18,7 +18,7 @@ SOURCES = ["lib.hip", "reduce.hip", "scan.hip", "sort.hip", "sort_split.hip", "t
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wall", "-Wno-unused-function",
+    "-Wall", "-Wno-unused-function", "-Wno-pass-failed",
 ]
 
 

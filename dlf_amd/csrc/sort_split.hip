@@ -84,7 +84,7 @@ int pass_block(int64_t n, int cap) {
 constexpr int kFinishItems = 10;
 constexpr int finish_cap(int waves) { return waves * kWave * kFinishItems; }      // keys a bucket may hold
 constexpr int finish_bins(int waves) { return waves * 1024; }                     // counting bins, two 16-bit counters a word
-constexpr int kCapHuge = finish_cap(16), kCapLarge = finish_cap(8), kCapSmall = finish_cap(4);
+constexpr int kCapHuge = finish_cap(16);
 constexpr int64_t kSmallCapRows = 131072;             // longest row that takes the small size
 constexpr int64_t kLargeCapRows = 1100000;            // longest row that takes the eight-wavefront size
 constexpr int64_t kLargeCapFloatRows = 700000;        // ... of floats, which seldom fill their fine bins as evenly as integers do
