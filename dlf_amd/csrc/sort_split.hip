@@ -63,10 +63,10 @@ constexpr int kChunk = 8 * kSplitTile;                // keys one split_pass wor
 // as one run per bucket, so its keys spread over the row's buckets decide how long the runs
 // are; short runs (128 bytes for 8-byte keys in 256 buckets) cost write bandwidth, larger tiles
 // cost LDS and occupancy.  Measured on [256, 2^20] int64: 1476 / 1235 / 1044 us (keys),
-// 2197 / 1698 us (pairs: 1024 threads do not fit LDS); on [1024, 65536] fp32 (32 buckets):
-// 118 / 118 / 157 us (keys), 193 / 178 / 203 us (pairs).
+// 2197 / 1698 / 1540 us (pairs; at 1024 threads the indices pass through LDS after the keys); on
+// [1024, 65536] fp32 (32 buckets): 118 / 118 / 157 us (keys), 193 / 178 / 203 us (pairs).
 template <typename K, bool PAIRS>
-constexpr int kPassBlockMax = (sizeof(K) == 8 && !PAIRS) ? 1024 : 512;
+constexpr int kPassBlockMax = sizeof(K) == 8 ? 1024 : 512;
 template <typename K, bool PAIRS>
 int pass_block(int64_t n, int cap) {
     const int64_t buckets = ceil_div(n * 5, static_cast<int64_t>(cap) * 4);       // buckets fill to about 4/5
@@ -497,6 +497,11 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
 }
 
 // ------------------------------------------------------------------ 4. one pass: chunk -> buckets
+// The largest tile of 8-byte keys with indices does not fit LDS twice over: its indices pass
+// through the space its keys have left (the threads keep where everything goes in registers).
+template <typename K, bool PAIRS, int BLOCK>
+constexpr bool kPassInTurn = PAIRS && sizeof(K) == 8 && BLOCK == 1024;
+
 template <typename K, bool PAIRS, int BLOCK>
 struct SplitShared {
     uint32_t table[kFine / 4];                 // bucket_of, four fine bins a word
@@ -505,7 +510,7 @@ struct SplitShared {
     int32_t dst_base[kMaxBuckets];             // row position of a bucket's share of this tile minus start
     uint32_t scan_tmp[kMaxBuckets / kWave];
     K keys[BLOCK * kSplitItems];
-    uint32_t vals[PAIRS ? BLOCK * kSplitItems : 1];
+    uint32_t vals[PAIRS && !kPassInTurn<K, PAIRS, BLOCK> ? BLOCK * kSplitItems : 1];
 };
 
 // One workgroup per chunk (kChunk keys, tiles of 4096): where the chunk's keys of each bucket
@@ -519,6 +524,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
                                                           const SplitRow* __restrict__ infos, const uint32_t* __restrict__ chunk_base) {
     constexpr int ITEMS = kSplitItems;
     constexpr int TILE = BLOCK * kSplitItems;
+    constexpr bool IN_TURN = kPassInTurn<K, PAIRS, BLOCK>;
     static_assert(kChunk % TILE == 0, "whole tiles a chunk");
     __shared__ SplitShared<K, PAIRS, BLOCK> sm;
     const int tid = threadIdx.x;
@@ -613,7 +619,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
         for (int k = 0; k < ITEMS; ++k) {
             if (full || tid + k * BLOCK < valid) {
                 sm.keys[where[k]] = key[k];
-                if constexpr (PAIRS) sm.vals[where[k]] = static_cast<uint32_t>(tile_base) + static_cast<uint32_t>(tid + k * BLOCK);
+                if constexpr (PAIRS && !IN_TURN) sm.vals[where[k]] = static_cast<uint32_t>(tile_base) + static_cast<uint32_t>(tid + k * BLOCK);
             }
         }
         __syncthreads();
@@ -621,34 +627,52 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
         // the tile is in LDS: the registers take the next tile, whose keys arrive while this one is written
         if (tile_base + TILE < chunk_hi) load_tile(tile_base + TILE, key);
 
-        // ---- write runs: thread tid takes tile positions tid, tid + 256, ...; eight at a time, the
+        // ---- write runs: thread tid takes tile positions tid, tid + BLOCK, ...; eight at a time, the
         // reads of each step issued for all eight before the next step uses them
         {
             K* dk = io.kbuf[0] + row_off;
             uint32_t* dv = PAIRS ? io.vbuf[0] + row_off : nullptr;
+            int32_t at[ITEMS];                         // where tile position k * BLOCK + tid goes in the row
 #pragma unroll
             for (int k0 = 0; k0 < ITEMS; k0 += 8) {
                 K out[8];
-                int32_t at[8];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) out[j] = sm.keys[(k0 + j) * BLOCK + tid];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const uint32_t f = fine_of.template bin<BY_VALUE>(out[j]);
-                    at[j] = static_cast<int32_t>((sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu);
+                    at[k0 + j] = static_cast<int32_t>((sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu);
                 }
 #pragma unroll
-                for (int j = 0; j < 8; ++j) at[j] = sm.dst_base[at[j]] + ((k0 + j) * BLOCK + tid);
+                for (int j = 0; j < 8; ++j) at[k0 + j] = sm.dst_base[at[k0 + j]] + ((k0 + j) * BLOCK + tid);
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
-                    if (full || (k0 + j) * BLOCK + tid < valid) dk[at[j]] = out[j];
-                if constexpr (PAIRS) {
+                    if (full || (k0 + j) * BLOCK + tid < valid) dk[at[k0 + j]] = out[j];
+                if constexpr (PAIRS && !IN_TURN) {
                     uint32_t pay[8];
 #pragma unroll
                     for (int j = 0; j < 8; ++j) pay[j] = sm.vals[(k0 + j) * BLOCK + tid];
 #pragma unroll
                     for (int j = 0; j < 8; ++j)
-                        if (full || (k0 + j) * BLOCK + tid < valid) dv[at[j]] = pay[j];
+                        if (full || (k0 + j) * BLOCK + tid < valid) dv[at[k0 + j]] = pay[j];
+                }
+            }
+            if constexpr (IN_TURN) {
+                // the keys have left: their space takes the indices, laid out the same way
+                uint32_t* turn = reinterpret_cast<uint32_t*>(sm.keys);
+                __syncthreads();
+#pragma unroll
+                for (int k = 0; k < ITEMS; ++k)
+                    if (full || tid + k * BLOCK < valid) turn[where[k]] = static_cast<uint32_t>(tile_base) + static_cast<uint32_t>(tid + k * BLOCK);
+                __syncthreads();
+#pragma unroll
+                for (int k0 = 0; k0 < ITEMS; k0 += 8) {
+                    uint32_t pay[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) pay[j] = turn[(k0 + j) * BLOCK + tid];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (full || (k0 + j) * BLOCK + tid < valid) dv[at[k0 + j]] = pay[j];
                 }
             }
         }
