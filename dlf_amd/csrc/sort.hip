@@ -1,5 +1,11 @@
 // sort / argsort along the last axis of strided views for gfx950.
 //
+// Which way a row goes: rows of up to 64 / 512 elements are sorted by one wavefront in
+// registers, rows of up to 4096 by one workgroup on chip, longer rows of 4- and 8-byte keys by
+// the bucket route of sort_split.hip (run_split below enqueues it first; every row decides on
+// the device whether it can take it).  What is left - rows the bucket route cannot take,
+// 16-bit keys - is sorted here:
+//
 // Segmented least-significant-digit radix sort, 8 bits per pass, every row an
 // independent segment:
 //   1. sort_histogram: one read of the input builds, per row, the digit
