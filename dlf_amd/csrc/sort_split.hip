@@ -290,7 +290,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
             const VecK* src = reinterpret_cast<const VecK*>(xrow + b0);
 #pragma unroll
             for (int v = 0; v < U / VK; ++v) {
-                const VecK a = src[threadIdx.x + v * kSplitBlock];
+                const VecK a = load_stream(&src[threadIdx.x + v * kSplitBlock]);      // (non-temporal: 71 -> 50 us on [1024, 65536] fp32)
 #pragma unroll
                 for (int e = 0; e < VK; ++e) key[v * VK + e] = a.v[e];
             }
@@ -547,7 +547,9 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
             const int e = tid + k * BLOCK;
-            key[k] = src[static_cast<int64_t>(e < valid ? e : 0) * io.sx];
+            const K* at = &src[static_cast<int64_t>(e < valid ? e : 0) * io.sx];
+            if constexpr (sizeof(K) == 4) key[k] = load_stream(at);       // (non-temporal loads measured: a gain for 4-byte keys,
+            else key[k] = *at;                                            // a loss of 7 % for 8-byte keys)
         }
     };
 
