@@ -294,7 +294,7 @@ __device__ __forceinline__ void scan_tile(
             if (t > 0) {
                 int64_t pos = t - 1;
                 for (;;) {
-                    // the states this round reads reach back to pos - 63 or to the row's first
+                    // the states this step of the look-back reads reach back to pos - 63 or to the row's first
                     const int64_t lowest = sbase + (pos >= kWave - 1 ? pos - (kWave - 1) : 0);
                     while (lowest < cleared_from) {
                         const int64_t slice = (cleared_from - 1) / kSliceTiles;
