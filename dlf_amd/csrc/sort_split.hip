@@ -103,6 +103,8 @@ struct alignas(16) SplitRow {
     uint32_t by_value;                     // 1 (floats only): fine bin = (value - lo) * scale between base and top
     unsigned long long top;                // by value: keys from here up share the last fine bin
     unsigned long long lo_bits, scale_bits;    // by value: lo and scale as a float's / double's bits
+    unsigned long long gap_lo, gap_hi;     // by key image, floats: keys in [gap_lo, gap_hi) count as gap_lo and the keys above move down by
+                                           // the width of the gap (none: both all ones)
     uint32_t begin[kMaxBuckets + 4];       // first position of each bucket in the row; begin[n_buckets] = n
     uint8_t bucket_of[kFine];              // fine bin -> bucket (16-byte aligned: tiles load it as vectors)
 };
@@ -118,24 +120,32 @@ template <> struct FloatOf<uint64_t> { using type = double; };
 // (integers; floats whose magnitudes spread over many binades - an image is about the
 // logarithm of its float), or evenly over the values (floats that spread evenly as numbers:
 // uniform or bell-shaped data, data on both sides of zero, where most images would crowd into
-// the few bins of the largest binades).  split_sample picks per row.
+// the few bins of the largest binades).  split_sample picks per row.  By key image, a float row
+// with values on both sides of zero would spend most bins on the images between its smallest
+// negative and positive magnitudes, where it has next to no keys: split_sample finds that gap
+// and the map closes it up.
 template <typename K>
 struct FineMap {
     using F = typename FloatOf<K>::type;
-    K base, top;
+    K base, top, gap_lo, gap_hi, less;     // less: -(gap_hi + base), what the image with the gap taken out is short of
     F lo, scale;
     uint32_t shift, by_value;
     int descending;
     __device__ FineMap(const SplitRow& r, int desc)
-        : base(static_cast<K>(r.base)), top(static_cast<K>(r.top)), lo(bit_cast<F>(static_cast<K>(r.lo_bits))),
-          scale(bit_cast<F>(static_cast<K>(r.scale_bits))), shift(r.shift), by_value(r.by_value), descending(desc) {}
+        : base(static_cast<K>(r.base)), top(static_cast<K>(r.top)), gap_lo(static_cast<K>(r.gap_lo)), gap_hi(static_cast<K>(r.gap_hi)),
+          less(static_cast<K>(K(0) - static_cast<K>(r.gap_hi) - static_cast<K>(r.base))),
+          lo(bit_cast<F>(static_cast<K>(r.lo_bits))), scale(bit_cast<F>(static_cast<K>(r.scale_bits))), shift(r.shift),
+          by_value(r.by_value), descending(desc) {}
     // the number a float key stands for, increasing with the key (so negated for descending sorts)
     __device__ __forceinline__ static F value_of(K key, int desc) {
         const F x = bit_cast<F>(decode_key<K>(key, kKeyFloat, desc));
         return desc ? -x : x;
     }
-    // BY_VALUE must equal by_value: the kernels branch once per workgroup, not once per key
-    template <bool BY_VALUE>
+    // BY_VALUE must equal by_value: the kernels branch once per workgroup, not once per key.
+    // GAP: the row may have a gap (the host knows which rows can) - otherwise no code for it.
+    // With the gap taken out, the image of a key is min(key, gap_lo) + max(key, gap_hi) - gap_hi:
+    // monotone, the key itself below the gap (where base lies) and when there is no gap.
+    template <bool BY_VALUE, bool GAP>
     __device__ __forceinline__ uint32_t bin(K key) const {
         uint32_t f;
         if constexpr (BY_VALUE) {
@@ -146,13 +156,31 @@ struct FineMap {
             b = b < 0 ? 0 : b;
             f = b < kFine - 1 ? static_cast<uint32_t>(b) : static_cast<uint32_t>(kFine - 1);
             f = key >= top ? static_cast<uint32_t>(kFine - 1) : f;
+        } else if constexpr (GAP) {
+            // base lies below the gap: a key held between base and gap_lo, plus one held above
+            // gap_hi, less gap_hi and base, is the image's distance from base - no test for keys
+            // under base, and as many operations as without a gap
+            const K below = clamp_between(key, base, gap_lo), above = key > gap_hi ? key : gap_hi;
+            const K off = static_cast<K>(below + above + less) >> shift;
+            return off < static_cast<K>(kFine - 1) ? static_cast<uint32_t>(off) : static_cast<uint32_t>(kFine - 1);
         } else {
             const K off = static_cast<K>(key - base) >> shift;
             f = off < static_cast<K>(kFine - 1) ? static_cast<uint32_t>(off) : static_cast<uint32_t>(kFine - 1);
         }
         return key < base ? 0u : f;
     }
-    __device__ __forceinline__ uint32_t operator()(K key) const { return by_value ? bin<true>(key) : bin<false>(key); }
+    // min(max(x, lo), hi) for lo <= hi: one instruction for 32-bit keys (the compiler cannot know that lo <= hi)
+    __device__ __forceinline__ static K clamp_between(K x, K lo, K hi) {
+        if constexpr (sizeof(K) == 4) {
+            uint32_t r;
+            asm("v_med3_u32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(lo), "v"(hi));      // (one scalar operand an instruction)
+            return r;
+        } else {
+            const K up = x > lo ? x : lo;
+            return up < hi ? up : hi;
+        }
+    }
+    __device__ __forceinline__ uint32_t operator()(K key) const { return by_value ? bin<true, true>(key) : bin<false, true>(key); }
 };
 
 template <typename T, typename Join>
@@ -167,9 +195,13 @@ __device__ __forceinline__ T block_reduce(T v, Join join, T* lds, int waves) {
 }
 
 // ------------------------------------------------------------------ 1. the range of a row's keys
-// VAL: float rows long enough for the value map to matter (the host knows); without it the row
-// is spread by key image and the kernels carry no code for anything else.
-template <typename K, bool VAL>
+// MAP (the host knows): 0 for rows spread by key image and nothing else (integers, short float
+// rows); 1 for float rows of middling length, whose images may have the gap around zero closed
+// up; 2 for longer float rows, by key image as they are or by value.  The kernels carry no code for what their
+// MAP leaves out.
+constexpr int kMapPlain = 0, kMapGap = 1, kMapValue = 2;
+
+template <typename K, int MAP>
 __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_t n, uint32_t cap, SplitRow* __restrict__ rows, uint32_t* __restrict__ counters) {
     __shared__ K red[kSplitBlock / kWave];
     const int64_t row = blockIdx.x;
@@ -199,11 +231,53 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
     }
     lo = block_reduce(lo, [](K a, K b) { return a < b ? a : b; }, red, kSplitBlock / kWave);
     hi = block_reduce(hi, [](K a, K b) { return a > b ? a : b; }, red, kSplitBlock / kWave);
+    // Float rows: the images of negative and of positive values lie either side of the middle
+    // of the key range, those of the smallest magnitudes next to it and the two zeros at it.
+    // Every wave offers the nearest of its keys below the zeros and the nearest above them; the
+    // second nearest of the four on each side bound the gap (one stray tiny value a side does not
+    // count, and zeros never do).  Keys inside it - zeros, a few tiny values - share a fine bin.
+    K gap_lo = ~K(0), gap_hi = ~K(0);
+    if constexpr (MAP == kMapGap) {
+        constexpr K zero_hi = K(1) << (8 * sizeof(K) - 1), zero_lo = zero_hi - 1;      // keys of +0.0 and -0.0 (either way round)
+        int below = 0, upto = 0;                       // entries 0 .. below - 1 lie under the zeros, entries from upto on above them
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            below += __popcll(__ballot(key[u] < zero_lo));
+            upto += __popcll(__ballot(key[u] <= zero_hi));
+        }
+        auto entry = [&](int at) {                     // at: the same in every lane
+            const K mine = at < kWave ? key[0] : at < 2 * kWave ? key[1] : at < 3 * kWave ? key[2] : key[3];
+            return lane_read(mine, at % kWave);
+        };
+        __shared__ K near[2][kSplitBlock / kWave];
+        const K wave_under = below >= 1 ? entry(below - 1) : K(0), wave_over = upto < 4 * kWave ? entry(upto) : ~K(0);
+        if (lane_id() == 0) {
+            near[0][threadIdx.x / kWave] = wave_under;
+            near[1][threadIdx.x / kWave] = wave_over;
+        }
+        __syncthreads();
+        K under[2] = {K(0), K(0)}, over[2] = {~K(0), ~K(0)};       // nearest and second nearest
+        for (int w = 0; w < kSplitBlock / kWave; ++w) {
+            const K a = near[0][w], b = near[1][w];
+            if (a > under[0]) { under[1] = under[0]; under[0] = a; } else if (a > under[1]) under[1] = a;
+            if (b < over[0]) { over[1] = over[0]; over[0] = b; } else if (b < over[1]) over[1] = b;
+        }
+        const K nearest_under = under[1], nearest_over = over[1];
+        // worth closing when it lies inside the range and is at least half of it (a bit of bin width or more)
+        if (n >= 1024 && nearest_under != K(0) && nearest_under >= lo && nearest_over <= hi &&
+            static_cast<K>(nearest_over - nearest_under) >= static_cast<K>(static_cast<K>(hi - lo) / 2)) {
+            gap_lo = nearest_under;
+            gap_hi = nearest_over;
+        }
+    }
     // that range takes the middle half of the fine bins; a quarter on either side is left for
     // keys outside it (beyond those, keys share the first or last bin)
     SplitRow map;
     {
-        const unsigned long long range = static_cast<unsigned long long>(static_cast<K>(hi - lo));
+        map.gap_lo = static_cast<unsigned long long>(gap_lo);
+        map.gap_hi = static_cast<unsigned long long>(gap_hi);
+        const K gap = static_cast<K>(gap_hi - gap_lo);         // lo is below the gap, hi above it
+        const unsigned long long range = static_cast<unsigned long long>(static_cast<K>(hi - lo - gap));
         const int width = range ? 64 - __builtin_clzll(range) : 0;
         map.shift = width > kFineBits - 1 ? static_cast<uint32_t>(width - (kFineBits - 1)) : 0u;
         const K margin = static_cast<K>(K(kFine / 4) << map.shift);
@@ -212,7 +286,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
         map.top = 0ull;
         map.lo_bits = map.scale_bits = 0ull;
     }
-    if constexpr (VAL) {
+    if constexpr (MAP == kMapValue) {
         // the same range spread evenly over the values instead - taken when, by key image, the
         // sample's fullest cell of 16 bins promises a fine bin of more than a quarter of what a
         // bucket holds (the row might not fit the route, or only in lopsided buckets) and the
@@ -253,6 +327,8 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
         out.shift = map.shift;
         out.base = map.base;
         out.by_value = map.by_value;
+        out.gap_lo = map.gap_lo;
+        out.gap_hi = map.gap_hi;
         out.top = map.top;
         out.lo_bits = map.lo_bits;
         out.scale_bits = map.scale_bits;
@@ -264,7 +340,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
 // counts a word (a count is at most kChunk).  split_plan adds the chunks up for the row's
 // histogram and turns each chunk's into its keys per bucket, so that split_pass needs no
 // communication between workgroups.
-template <typename K, bool VAL>
+template <typename K, int MAP>
 __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int64_t n, int64_t chunks_per_row,
                                                                const SplitRow* __restrict__ rows, uint32_t* __restrict__ chunk_fine) {
     constexpr int U = 32 / sizeof(K);                 // keys per thread and batch (64 bytes measured: no faster)
@@ -304,6 +380,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
     };
     auto count_chunk = [&](auto by_value_tag) __attribute__((always_inline)) {
     constexpr bool BY_VALUE = decltype(by_value_tag)::value;
+    constexpr bool GAP = MAP == kMapGap;               // (a branch per workgroup on whether the row has a gap: more registers, slower)
     K key[U];
     load_batch(lo, key);
     for (int64_t b0 = lo; b0 < hi; b0 += BATCH) {
@@ -312,7 +389,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
         const bool full = b0 + BATCH <= hi;
         uint32_t f[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) f[u] = fine_of.template bin<BY_VALUE>(key_of_element<K>(io, key[u]));
+        for (int u = 0; u < U; ++u) f[u] = fine_of.template bin<BY_VALUE, GAP>(key_of_element<K>(io, key[u]));
         // a wave whose keys all share one fine bin (narrow ranges, few distinct values) adds once
         const uint32_t f0 = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(f[0])));
         bool same = full;
@@ -329,7 +406,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
         for (int u = 0; u < U; ++u) key[u] = ahead[u];
     }
     };
-    if (VAL && fine_of.by_value) count_chunk(std::integral_constant<bool, VAL>());
+    if (MAP == kMapValue && fine_of.by_value) count_chunk(std::integral_constant<bool, MAP == kMapValue>());
     else count_chunk(std::false_type());
     __syncthreads();
     uint32_t* g = chunk_fine + static_cast<int64_t>(blockIdx.x) * (kFine / 2);
@@ -519,7 +596,7 @@ struct SplitShared {
 // and their slot among the tile's keys of that bucket with one LDS atomic each, the tile is laid
 // out by bucket in LDS and written as runs; once it lies in LDS the registers already receive
 // the next tile's keys.  The order inside a run is whatever the atomics gave.
-template <typename K, bool PAIRS, int BLOCK, bool VAL>
+template <typename K, bool PAIRS, int BLOCK, int MAP>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void split_pass(PassIo<K> io, int64_t n, int64_t chunks_per_row,
                                                           const SplitRow* __restrict__ infos, const uint32_t* __restrict__ chunk_base) {
     constexpr int ITEMS = kSplitItems;
@@ -567,6 +644,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
 
     auto move_chunk = [&](auto by_value_tag) __attribute__((always_inline)) {
     constexpr bool BY_VALUE = decltype(by_value_tag)::value;
+    constexpr bool GAP = MAP == kMapGap;
     for (int64_t tile_base = chunk_lo; tile_base < chunk_hi; tile_base += TILE) {
         const int valid = static_cast<int>((chunk_hi - tile_base < TILE) ? chunk_hi - tile_base : TILE);
         const bool full = valid == TILE;
@@ -582,7 +660,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
         for (int k0 = 0; k0 < ITEMS; k0 += 8) {
 #pragma unroll
             for (int k = k0; k < k0 + 8; ++k) {
-                const uint32_t f = fine_of.template bin<BY_VALUE>(key[k]);
+                const uint32_t f = fine_of.template bin<BY_VALUE, GAP>(key[k]);
                 where[k] = (sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu;
             }
 #pragma unroll
@@ -642,7 +720,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
                 for (int j = 0; j < 8; ++j) out[j] = sm.keys[(k0 + j) * BLOCK + tid];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    const uint32_t f = fine_of.template bin<BY_VALUE>(out[j]);
+                    const uint32_t f = fine_of.template bin<BY_VALUE, GAP>(out[j]);
                     at[k0 + j] = static_cast<int32_t>((sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu);
                 }
 #pragma unroll
@@ -682,7 +760,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
         __syncthreads();                                   // the tile in LDS has left
     }
     };
-    if (VAL && fine_of.by_value) move_chunk(std::integral_constant<bool, VAL>());
+    if (MAP == kMapValue && fine_of.by_value) move_chunk(std::integral_constant<bool, MAP == kMapValue>());
     else move_chunk(std::false_type());
 }
 
@@ -1156,14 +1234,26 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
 
     const int waves = finish_waves(n, io.kind == kKeyFloat);
     const int cap = finish_cap(waves);
-    // float rows beyond the smallest size may be spread by value (split_sample decides per row)
-    const bool val = io.kind == kKeyFloat && waves > 4;
-    if (val) split_sample<K, true><<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(io, n, static_cast<uint32_t>(cap), rows, counters);
-    else split_sample<K, false><<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(io, n, static_cast<uint32_t>(cap), rows, counters);
+    // Float rows beyond the smallest size may be spread by value (split_sample decides per row).
+    // The smallest may have the gap around zero closed up once they are long enough for it to
+    // pay: a quarter of a binade, the bin of an open gap, holds some 4 % of a bell-shaped row -
+    // not much beside a bucket while the row has under a dozen buckets' worth of keys, and the
+    // finer bins of the closed gap would only split the thin tails into many small buckets
+    // (measured on normal rows: open gap ahead up to 24 000 keys, closed from 32 768).
+    const int map = io.kind != kKeyFloat ? kMapPlain : waves > 4 ? kMapValue : n >= 12 * static_cast<int64_t>(cap) ? kMapGap : kMapPlain;
+    auto with_map = [&](auto&& launch_with) {
+        if (map == kMapPlain) launch_with(std::integral_constant<int, kMapPlain>());
+        else if (map == kMapGap) launch_with(std::integral_constant<int, kMapGap>());
+        else launch_with(std::integral_constant<int, kMapValue>());
+    };
+    with_map([&](auto map_tag) {
+        split_sample<K, decltype(map_tag)::value><<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(io, n, static_cast<uint32_t>(cap), rows, counters);
+    });
     DLFX_CHECK_LAUNCH();
     const dim3 chunks(static_cast<unsigned>(m * l.chunks_per_row));
-    if (val) split_histogram<K, true><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine);
-    else split_histogram<K, false><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine);
+    with_map([&](auto map_tag) {
+        split_histogram<K, decltype(map_tag)::value><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine);
+    });
     DLFX_CHECK_LAUNCH();
     split_plan<<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(n, static_cast<uint32_t>(cap), l.chunks_per_row, fine, rows, counters, list, chunk_base);
     DLFX_CHECK_LAUNCH();
@@ -1177,14 +1267,11 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         if (finish_room <= 0) return DLFX_ERR_LAUNCH;
         const dim3 fgrid(static_cast<unsigned>(buckets < finish_room ? buckets : finish_room));
         const int block = pass_block<K, PAIRS>(n, cap);
-        auto pass = [&](auto block_tag, auto val_tag) {
-            constexpr int BLOCK = decltype(block_tag)::value;
-            constexpr bool VAL = decltype(val_tag)::value;
-            split_pass<K, PAIRS, BLOCK, VAL><<<chunks, dim3(BLOCK), 0, stream>>>(io, n, l.chunks_per_row, rows, chunk_base);
-        };
         auto pass_of = [&](auto block_tag) {
-            if (val) pass(block_tag, std::true_type());
-            else pass(block_tag, std::false_type());
+            with_map([&](auto map_tag) {
+                split_pass<K, PAIRS, decltype(block_tag)::value, decltype(map_tag)::value><<<chunks, dim3(decltype(block_tag)::value), 0, stream>>>(
+                    io, n, l.chunks_per_row, rows, chunk_base);
+            });
         };
         if (block == 256) pass_of(std::integral_constant<int, 256>());
         else if (block == 512) pass_of(std::integral_constant<int, 512>());

@@ -299,6 +299,45 @@ def test_float_rows_spread_by_value_or_by_image(hip_backend, dtype, n):
     assert np.array_equal(np.take_along_axis(x, Jh.numpy().astype(np.int64), -1).view(np.uint8), Yh.numpy().view(np.uint8))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n", [31000, 65536, 131072])
+def test_float_rows_either_side_of_zero_close_the_gap_between_their_images(hip_backend, dtype, n):
+    """Float rows of 30 720 to 131 072 elements with values on both sides of zero leave the images
+    between their smallest negative and positive magnitudes out of the fine bins.  Rows where that
+    applies (bell-shaped, with a few zeros, with one stray tiny value a side), rows where it does
+    not (half zeros, tiny values all over, one sign only, magnitudes over many binades) and rows
+    with infinities and NaNs, ascending and descending, against numpy."""
+    rows = normal(360, 8 * n).astype(dtype).reshape(8, n)
+    rows[1, ::97] = 0.0
+    rows[1, 5::97] = -0.0
+    rows[2, 17] = dtype(1e-30)
+    rows[2, 4711] = dtype(-1e-30)
+    rows[3, rows[3] < 0] = 0.0                                            # half the row zeros
+    rows[4, ::3] *= dtype(1e-20)                                          # a third of the row tiny, both signs
+    rows[5] = np.abs(rows[5]) + dtype(0.25)                               # one sign only
+    rows[6] = (np.exp(normal(361, n).astype(np.float64) * 10.0) * np.sign(rows[6])).astype(dtype)
+    rows[7, 5:2000:7] = np.inf
+    rows[7, 6:2000:7] = -np.inf
+    rows[7, 7:3000:11] = np.nan
+    rows[7, 8:3000:11] = -np.nan
+    Xh = Tensor.from_numpy(hip_backend, rows)
+    want = np.sort(rows, axis=-1)
+    got = F.sort(Xh, -1).numpy()
+    assert np.array_equal(got[:7], want[:7])
+    nans = np.isnan(got[7])                                               # negative NaNs first, positive ones last; numpy: all last
+    assert nans.sum() == np.isnan(rows[7]).sum()
+    assert np.array_equal(got[7][~nans], want[7][: (~nans).sum()])
+    assert np.array_equal(F.sort(Tensor.from_numpy(hip_backend, rows[:7]), -1, True).numpy(), want[:7, ::-1])
+    order = np.argsort(rows[:7], axis=-1, kind="stable")
+    Yh, Ih = F.argsort(Tensor.from_numpy(hip_backend, rows[:7]), -1, False, with_values=True)
+    assert np.array_equal(Ih.numpy(), order)
+    assert np.array_equal(Yh.numpy().view(np.uint8), np.take_along_axis(rows[:7], order, -1).view(np.uint8))
+    Yd, Jd = F.argsort(Xh, -1, True, with_values=True)
+    assert np.array_equal(np.take_along_axis(rows, Jd.numpy().astype(np.int64), -1).view(np.uint8), Yd.numpy().view(np.uint8))
+    d = Yd.numpy()[:7]
+    assert bool((d[:, 1:] <= d[:, :-1]).all())
+
+
 @pytest.mark.parametrize("dtype", [np.int64, np.float32])
 def test_rows_beyond_a_million_keys_take_the_largest_buckets(hip_backend, dtype):
     """Rows longer than 1.1 M keys are cut into buckets of up to 10240 keys, finished by workgroups
