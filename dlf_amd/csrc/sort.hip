@@ -9,10 +9,10 @@
 // Segmented least-significant-digit radix sort, 8 bits per pass, every row an
 // independent segment:
 //   1. sort_histogram: one read of the input builds, per row, the digit
-//      histograms of every pass (they do not depend on the order of the keys).
-//   2. sort_bases: exclusive scan of each histogram -> where each digit's run
-//      starts inside the row.
-//   3. sort_pass (once per digit): a tile of keys is ranked with wave-wide
+//      histograms of every pass (they do not depend on the order of the keys);
+//      the workgroup that adds a row's last chunk turns each histogram into its
+//      exclusive scan -> where each digit's run starts inside the row.
+//   2. sort_pass (once per digit): a tile of keys is ranked with wave-wide
 //      digit matching (stable), gathered in LDS in its locally sorted order and
 //      written out in runs; the offset of a tile inside a digit's run comes from
 //      the counts of the row's earlier tiles, chained with decoupled look-back
@@ -69,6 +69,41 @@ struct RowRoutes {
     __device__ __forceinline__ bool elsewhere(int64_t row) const { return records && records[row * stride_words] == 1u; }
 };
 
+// ------------------------------------------------------------------ bases
+// In place: one histogram of a row -> exclusive prefix (start of each digit's run in the row),
+// by the 256 threads of a workgroup.  *moves receives the bits of the digit that are not the
+// same in all keys of the row: none means the pass would not change the order of the row (the
+// row then skips it), and the ranking only needs to look at those bits.  `all_bits` forces
+// every pass of every row to run.  The counts were added by other workgroups of this launch:
+// they are read where those additions were made, past this part's own cache.
+__device__ __forceinline__ void bases_of_pass(uint32_t* __restrict__ g, uint32_t* __restrict__ moves, int all_bits) {
+    __shared__ uint32_t wave_tot[kRadix / kWave];
+    __shared__ uint32_t wave_or[kRadix / kWave], wave_and[kRadix / kWave];
+    __syncthreads();                                   // the pass before has left these words
+    const uint32_t v = __hip_atomic_load(g + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t incl = wave_scan_inclusive(v, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+    const uint32_t ors = wave_reduce(v ? threadIdx.x : 0u, [](uint32_t a, uint32_t b) { return a | b; });
+    const uint32_t ands = wave_reduce(v ? threadIdx.x : 0xffu, [](uint32_t a, uint32_t b) { return a & b; });
+    const int w = threadIdx.x / kWave;
+    if (lane_id() == kWave - 1) {
+        wave_tot[w] = incl;
+        wave_or[w] = ors;
+        wave_and[w] = ands;
+    }
+    __syncthreads();
+    uint32_t pre = 0;
+    for (int i = 0; i < w; ++i) pre += wave_tot[i];
+    g[threadIdx.x] = pre + incl - v;
+    if (threadIdx.x == 0) {
+        uint32_t o = 0, a = 0xffu;
+        for (int i = 0; i < kRadix / kWave; ++i) {
+            o |= wave_or[i];
+            a &= wave_and[i];
+        }
+        *moves = all_bits ? 0xffu : (o ^ a);
+    }
+}
+
 // ------------------------------------------------------------------ histograms
 // One read of the input builds the digit histograms of every pass for a chunk of a row.
 // Each workgroup keeps kHistCopies interleaved copies of every histogram (a lane adds to copy
@@ -77,8 +112,11 @@ struct RowRoutes {
 // keys (constant bytes: small integers, narrow float ranges) is added once per wave.
 template <typename K>
 __global__ __launch_bounds__(kBlock) void sort_histogram(PassIo<K> io, int64_t n, int64_t chunk, int64_t chunks_per_row, int64_t units,
-                                                         RowRoutes routes, uint32_t* __restrict__ ghist) {
+                                                         RowRoutes routes, uint32_t* __restrict__ ghist, uint32_t* __restrict__ arrived,
+                                                         uint32_t* __restrict__ moves, int all_bits) {
     constexpr int P = KeyTraits<K>::kPasses;
+    static_assert(kBlock == kRadix, "a thread per digit when the row's histograms are scanned");
+    __shared__ uint32_t last_chunk;
     constexpr int U = 32 / sizeof(K);                 // keys in flight per thread
     constexpr int R = 32 / P;                         // copies: 8 (32-bit keys) or 4 (64-bit keys): 32 KB
     __shared__ uint32_t hist[P * kRadix * R];
@@ -139,51 +177,25 @@ __global__ __launch_bounds__(kBlock) void sort_histogram(PassIo<K> io, int64_t n
         for (int r = 0; r < R; ++r) v += hist[i * R + r];
         if (v) atomicAdd(&g[i], v);
     }
-    }
-}
-
-// In place: histogram -> exclusive prefix (start of each digit's run in the row).  Workgroup
-// b handles one (row, pass) pair.  moves[b] receives the bits of the digit that are not the
-// same in all keys of the row: none means the pass would not change the order of the row (the
-// row then skips it), and the ranking only needs to look at those bits.  `all_bits` forces
-// every pass of every row to run.
-__global__ __launch_bounds__(kRadix) void sort_bases(uint32_t* __restrict__ ghist, uint32_t* __restrict__ moves, int all_bits,
-                                                     RowRoutes routes) {
-    __shared__ uint32_t wave_tot[kRadix / kWave];
-    __shared__ uint32_t wave_or[kRadix / kWave], wave_and[kRadix / kWave];
-    if (routes.none_here()) return;
-    uint32_t* g = ghist + static_cast<int64_t>(blockIdx.x) * kRadix;
-    const uint32_t v = g[threadIdx.x];
-    const uint32_t incl = wave_scan_inclusive(v, 0u, [](uint32_t a, uint32_t b) { return a + b; });
-    const uint32_t ors = wave_reduce(v ? threadIdx.x : 0u, [](uint32_t a, uint32_t b) { return a | b; });
-    const uint32_t ands = wave_reduce(v ? threadIdx.x : 0xffu, [](uint32_t a, uint32_t b) { return a & b; });
-    const int w = threadIdx.x / kWave;
-    if (lane_id() == kWave - 1) {
-        wave_tot[w] = incl;
-        wave_or[w] = ors;
-        wave_and[w] = ands;
-    }
+    // The workgroup that brings the row's last chunk scans the row's histograms.  The additions
+    // are made where the whole device sees them, so it is enough that each workgroup's have
+    // been carried out before it counts its chunk (no cache is written back or emptied for
+    // this: with thousands of workgroups that costs more than the histograms), and that the
+    // last one reads the sums in the same place (bases_of_pass does).
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
-    uint32_t pre = 0;
-    for (int i = 0; i < w; ++i) pre += wave_tot[i];
-    g[threadIdx.x] = pre + incl - v;
-    if (threadIdx.x == 0) {
-        uint32_t o = 0, a = 0xffu;
-        for (int i = 0; i < kRadix / kWave; ++i) {
-            o |= wave_or[i];
-            a &= wave_and[i];
-        }
-        moves[blockIdx.x] = all_bits ? 0xffu : (o ^ a);
+    if (threadIdx.x == 0) last_chunk = atomicAdd(&arrived[row], 1u) == static_cast<uint32_t>(chunks_per_row - 1) ? 1u : 0u;
+    __syncthreads();
+    if (last_chunk) {
+        for (int p = 0; p < P; ++p) bases_of_pass(g + p * kRadix, moves + row * P + p, all_bits);
+    }
     }
 }
 
-__global__ __launch_bounds__(kBlock) void sort_clear(uint32_t* __restrict__ p, int64_t words, RowRoutes routes) {
-    if (routes.none_here()) return;
-    for (int64_t b = blockIdx.x; b * (kBlock * 4) < words; b += gridDim.x) {
-        const int64_t i = (b * kBlock + threadIdx.x) * 4;
-        if (i + 4 <= words) *reinterpret_cast<uint4*>(p + i) = make_uint4(0u, 0u, 0u, 0u);
-        else for (int64_t j = i; j < words; ++j) p[j] = 0u;
-    }
+__global__ __launch_bounds__(kBlock) void sort_clear(uint32_t* __restrict__ p, int64_t words) {
+    const int64_t i = (static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x) * 4;
+    if (i + 4 <= words) *reinterpret_cast<uint4*>(p + i) = make_uint4(0u, 0u, 0u, 0u);
+    else for (int64_t j = i; j < words; ++j) p[j] = 0u;
 }
 
 // ------------------------------------------------------------------ one pass
@@ -799,7 +811,7 @@ constexpr int tile_items(size_t key_size, bool pairs) { return ((key_size == 8 &
 
 struct SortLayout {
     int64_t tiles_per_row;
-    size_t moves_off, hist_off, hist_bytes, status_off, status_bytes, split_off, split_bytes, keys_off[2], vals_off[2], total;
+    size_t moves_off, arrived_off, hist_off, hist_bytes, status_off, status_bytes, split_off, split_bytes, keys_off[2], vals_off[2], total;
 };
 
 SortLayout sort_layout(size_t key_size, bool pairs, int64_t m, int64_t n) {
@@ -810,6 +822,8 @@ SortLayout sort_layout(size_t key_size, bool pairs, int64_t m, int64_t n) {
     size_t off = 0;
     l.moves_off = off;           // one word per (row, pass): does the pass move the row's keys
     off += align_up(static_cast<size_t>(m) * passes * 4, 256);
+    l.arrived_off = off;         // chunks of each row counted so far; cleared with the histograms and the status words after it
+    off += align_up(static_cast<size_t>(m) * 4, 256);
     l.hist_off = off;
     l.hist_bytes = static_cast<size_t>(m) * passes * kRadix * 4;
     off += align_up(l.hist_bytes, 256);
@@ -904,40 +918,45 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     io.vbuf[0] = a.pairs ? reinterpret_cast<uint32_t*>(base + l.vals_off[0]) : nullptr;
     io.vbuf[1] = a.pairs ? reinterpret_cast<uint32_t*>(base + l.vals_off[1]) : nullptr;
 
+    uint32_t* moves = reinterpret_cast<uint32_t*>(base + l.moves_off);
+    uint32_t* arrived = reinterpret_cast<uint32_t*>(base + l.arrived_off);
+    uint32_t* ghist = reinterpret_cast<uint32_t*>(base + l.hist_off);
+    uint32_t* status = reinterpret_cast<uint32_t*>(base + l.status_off);
     // The bucket route first: every row it can take goes that way (decided on the device, row by
     // row); the digit passes below take the others and leave at once when there are none.  The
     // routes share the first ping-pong buffer: their rows are different rows.
     RowRoutes routes = {nullptr, 0, nullptr};
     if constexpr (sizeof(K) >= 4) {
         if (l.split_bytes != 0 && g_sort_buckets) {
+            // (the route clears the tables of the rows it leaves)
+            const LeftTables tables = {arrived, ghist, static_cast<uint32_t>(P * kRadix), status,
+                                       l.status_bytes ? l.tiles_per_row * kRadix : 0};
             size_t stride = 0;
-            const int st = run_split<K>(stream, io, a.pairs, m, n, base + l.split_off, g_sort_poll_limit, g_sort_compare_max,
+            const int st = run_split<K>(stream, io, a.pairs, m, n, base + l.split_off, g_sort_poll_limit, g_sort_compare_max, tables,
                                         &routes.other_rows, &routes.records, &stride);
             if (st != DLFX_OK) return st;
             routes.stride_words = stride / 4;
         }
     }
 
-    uint32_t* moves = reinterpret_cast<uint32_t*>(base + l.moves_off);
-    uint32_t* ghist = reinterpret_cast<uint32_t*>(base + l.hist_off);
-    uint32_t* status = reinterpret_cast<uint32_t*>(base + l.status_off);
-    const int64_t clear_words = static_cast<int64_t>((l.status_off + l.status_bytes - l.hist_off) / 4);   // histograms + status
     // When the bucket route runs, these launches only take the rows it left - usually none - so
     // they are sized to what the device holds at once and walk their work; an idle launch then
     // costs a few microseconds however long the rows are.
     const bool bounded = routes.records != nullptr;
     auto sized = [&](int64_t units, int64_t room) { return dim3(static_cast<unsigned>(bounded && room > 0 && room < units ? room : units)); };
-    sort_clear<<<sized(ceil_div(clear_words, kBlock * 4), 2048), dim3(kBlock), 0, stream>>>(ghist, clear_words, routes);
-    DLFX_CHECK_LAUNCH();
+    if (!bounded) {
+        const int64_t clear_words = static_cast<int64_t>((l.status_off + l.status_bytes - l.arrived_off) / 4);   // counts, histograms, status
+        sort_clear<<<dim3(static_cast<unsigned>(ceil_div(clear_words, kBlock * 4))), dim3(kBlock), 0, stream>>>(arrived, clear_words);
+        DLFX_CHECK_LAUNCH();
+    }
 
     const int64_t chunk = 32768;
     const int64_t chunks_per_row = ceil_div(n, chunk);
     if (m * chunks_per_row > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
-    sort_histogram<K><<<sized(m * chunks_per_row, 1024), dim3(kBlock), 0, stream>>>(io, n, chunk, chunks_per_row, m * chunks_per_row, routes, ghist);
-    DLFX_CHECK_LAUNCH();
     // a pass that moves nothing may only be left out when no pass reads the input while
     // another tile of the same pass writes the output over it
-    sort_bases<<<dim3(static_cast<unsigned>(m * P)), dim3(kRadix), 0, stream>>>(ghist, moves, y_over_x ? 1 : 0, routes);
+    sort_histogram<K><<<sized(m * chunks_per_row, 1024), dim3(kBlock), 0, stream>>>(io, n, chunk, chunks_per_row, m * chunks_per_row, routes, ghist,
+                                                                                    arrived, moves, y_over_x ? 1 : 0);
     DLFX_CHECK_LAUNCH();
 
     // (a tile waits for tiles of workgroups that run beside it: no more workgroups than fit at once)

@@ -97,6 +97,16 @@ int64_t resident_workgroups(Kernel kernel, int block) {
 }
 
 // ------------------------------------------------------------------ the bucket route (sort_split.hip)
+// The tables of the digit passes that must start at zero for a row those passes sort; the
+// bucket route clears them for every row it leaves.
+struct LeftTables {
+    uint32_t* arrived;                   // one word a row
+    uint32_t* hist;                      // hist_words a row
+    uint32_t hist_words;
+    uint32_t* status;                    // status_words a row (none for rows of one tile)
+    int64_t status_words;
+};
+
 // Whether rows of n keys may take it at all, the scratch it needs, and its launch: rows it does
 // not take are counted in **other_rows (device memory) and marked by a first word other than 1
 // in the per-row records at *route_records (*route_stride bytes apart).
@@ -104,7 +114,7 @@ bool split_route_takes(size_t key_size, int64_t m, int64_t n);
 size_t split_scratch_bytes(size_t key_size, bool pairs, int64_t m, int64_t n);
 template <typename K>
 int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, int64_t n, void* scratch, int poll_limit,
-              int compare_max, const uint32_t** other_rows, const uint32_t** route_records, size_t* route_stride);
+              int compare_max, const LeftTables& tables, const uint32_t** other_rows, const uint32_t** route_records, size_t* route_stride);
 
 // ------------------------------------------------------------------ a sort that stays in one workgroup
 constexpr int kSmallMoves = 256;         // keys that the run walk of sort_in_workgroup may move (one thread each)

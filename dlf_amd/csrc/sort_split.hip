@@ -415,11 +415,12 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
 
 // ------------------------------------------------------------------ 3. buckets of equal depth
 // One workgroup per row; thread t owns fine bins [16 t, 16 t + 16).  counters[0] counts the rows
-// that keep the digit passes, counters[2] the buckets listed for split_finish.  For a row that
+// that keep the digit passes (their tables of those passes are cleared here), counters[2] the
+// buckets listed for split_finish.  For a row that
 // takes the route, chunk_base[chunk][b] receives the row position where that chunk's keys of
 // bucket b go: the bucket's start plus what the row's earlier chunks hold of it.
 __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t cap, int64_t chunks_per_row, const uint32_t* __restrict__ chunk_fine,
-                                                          SplitRow* __restrict__ rows, uint32_t* __restrict__ counters,
+                                                          SplitRow* __restrict__ rows, uint32_t* __restrict__ counters, LeftTables left,
                                                           uint4* __restrict__ bucket_list, uint32_t* __restrict__ chunk_base) {
     constexpr int PER = kFine / kSplitBlock;          // 16
     __shared__ uint32_t red[kSplitBlock / kWave];
@@ -519,7 +520,13 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
         if (threadIdx.x == 0) {
             info.route = 0u;
             atomicAdd(&counters[0], 1u);
+            left.arrived[row] = 0u;
         }
+        // the digit passes sort this row: their tables for it start at zero
+        uint4* hist = reinterpret_cast<uint4*>(left.hist + row * left.hist_words);
+        for (uint32_t i = threadIdx.x; i < left.hist_words / 4; i += kSplitBlock) hist[i] = make_uint4(0u, 0u, 0u, 0u);
+        uint4* status = reinterpret_cast<uint4*>(left.status + row * left.status_words);
+        for (int64_t i = threadIdx.x; i < left.status_words / 4; i += kSplitBlock) status[i] = make_uint4(0u, 0u, 0u, 0u);
         return;
     }
     // a bin opens every bucket after its predecessor's up to its own
@@ -1218,7 +1225,7 @@ size_t split_scratch_bytes(size_t key_size, bool pairs, int64_t m, int64_t n) {
 // word 1 when the row was taken).
 template <typename K>
 int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, int64_t n, void* scratch, int poll_limit,
-              int compare_max, const uint32_t** other_rows, const uint32_t** route_records, size_t* route_stride) {
+              int compare_max, const LeftTables& tables, const uint32_t** other_rows, const uint32_t** route_records, size_t* route_stride) {
     const SplitLayout l = split_layout(m, n);
     char* base = static_cast<char*>(scratch);
     uint32_t* counters = reinterpret_cast<uint32_t*>(base + l.counters_off);
@@ -1255,7 +1262,7 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         split_histogram<K, decltype(map_tag)::value><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine);
     });
     DLFX_CHECK_LAUNCH();
-    split_plan<<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(n, static_cast<uint32_t>(cap), l.chunks_per_row, fine, rows, counters, list, chunk_base);
+    split_plan<<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(n, static_cast<uint32_t>(cap), l.chunks_per_row, fine, rows, counters, tables, list, chunk_base);
     DLFX_CHECK_LAUNCH();
     // split_finish: as many workgroups as the device holds at once, each walking its share of the buckets
     const int64_t buckets = m * kMaxBuckets;
@@ -1290,10 +1297,10 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
     return waves == 4 ? launch(std::false_type(), Small()) : waves == 8 ? launch(std::false_type(), Large()) : launch(std::false_type(), Huge());
 }
 
-template int run_split<uint32_t>(hipStream_t, const PassIo<uint32_t>&, bool, int64_t, int64_t, void*, int, int, const uint32_t**,
-                                 const uint32_t**, size_t*);
-template int run_split<uint64_t>(hipStream_t, const PassIo<uint64_t>&, bool, int64_t, int64_t, void*, int, int, const uint32_t**,
-                                 const uint32_t**, size_t*);
+template int run_split<uint32_t>(hipStream_t, const PassIo<uint32_t>&, bool, int64_t, int64_t, void*, int, int, const LeftTables&,
+                                 const uint32_t**, const uint32_t**, size_t*);
+template int run_split<uint64_t>(hipStream_t, const PassIo<uint64_t>&, bool, int64_t, int64_t, void*, int, int, const LeftTables&,
+                                 const uint32_t**, const uint32_t**, size_t*);
 
 }  // namespace dlfx
 
