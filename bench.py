@@ -263,6 +263,16 @@ def make_ops(be, which):
         x4b = gen((256, 1 << 20), torch.int64, lambda c: synth.full_range_i64(7), 1)
         ops += sort_ops(be, tensor, x4b, "C4b", "i64_[256,2^20]")
 
+    # ---------------- beside the baseline's configurations: float rows on both sides of zero
+    # (N(0,1) values at the C4a shape, at the row length from which the images of such rows have
+    # the gap around zero closed, and doubles); not part of all
+    if on("spread"):
+        for shape, dtype, text in (((1024, 65536), torch.float32, "f32_normal_[1024,65536]"),
+                                   ((2048, 32768), torch.float32, "f32_normal_[2048,32768]"),
+                                   ((512, 65536), torch.float64, "f64_normal_[512,65536]")):
+            xs = gen(shape, dtype, lambda c: synth.normal(9 + 100 * c), 4)
+            ops += sort_ops(be, tensor, xs, "C4n", text)
+
     # ---------------- C5: strided NCHW
     if on("all", "c5"):
         x5 = gen((32, 512, 56, 56), torch.float32, lambda c: synth.normal(8 + 100 * c), 6)
@@ -469,7 +479,7 @@ def sort_ops(be, tensor, xs, config, text):
     ops = []
     rows, n = xs[0].shape
     es = xs[0].element_size()
-    npd = np.float32 if xs[0].dtype == torch.float32 else np.int64
+    npd = {torch.float32: np.float32, torch.float64: np.float64, torch.int64: np.int64}[xs[0].dtype]
     y = torch.empty_like(xs[0])
     Y = tensor(y)
     I = Tensor.empty(be, [rows, n], np.int32)
@@ -596,7 +606,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3 | short (many short rows and an outer axis; not part of all) | ceil (copy and read-only streams at the C2 and C5 sizes; not part of all)")
+    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3 | short (many short rows and an outer axis; not part of all) | spread (sorts of N(0,1) rows; not part of all) | ceil (copy and read-only streams at the C2 and C5 sizes; not part of all)")
     ap.add_argument("--cpu-all", action="store_true",
                     help="also time the CPU restatement on a bounded sample of every configuration")
     ap.add_argument("--no-cpu", action="store_true")
