@@ -860,6 +860,7 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
     K key[ITEMS];
     uint32_t val[PAIRS ? ITEMS : 1];
     load_bucket(cur, key, val);
+    int dirty_words = kBins / 2;                           // counter words that are not zero
     for (;;) {
         SPLIT_PHASE_BEGIN();
         const int64_t vn = v + step;
@@ -879,7 +880,12 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
                 if constexpr (PAIRS) vlo = val[k] < vlo ? val[k] : vlo;
             }
         }
-        for (int i = tid; i < kBins / 2; i += T) sm.bins[i] = 0u;
+        if (dirty_words == kBins / 2) {                    // what the bucket before used
+#pragma unroll
+            for (int i = 0; i < kBins / 2 / T; ++i) sm.bins[tid + i * T] = 0u;
+        } else {
+            for (int i = tid; i < dirty_words; i += T) sm.bins[i] = 0u;
+        }
         lo = wave_reduce(lo, [](K a, K c) { return a < c ? a : c; });
         if constexpr (PAIRS) vlo = wave_reduce(vlo, [](uint32_t a, uint32_t c) { return a < c ? a : c; });
         if (lane == 0) {
@@ -930,6 +936,12 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
         }
         const int width = key_bits + idx_bits;
         const int down = width > kBinBits ? width - kBinBits : 0;      // words >> down lie below kBins
+        // a bucket whose words are narrower than that (quantised values, small integers) uses the
+        // first 2^width bins only: the others are neither scanned now nor cleared afterwards
+        // (the smallest buckets only: the larger ones measured 2.5 % slower with the test in their loops)
+        constexpr bool kNarrow = WAVES == 4;
+        const int used_words = (!kNarrow || width >= kBinBits) ? kBins / 2 : (width > 4 ? (1 << width) / 2 : WORDS);
+        dirty_words = used_words;
         SPLIT_PHASE(8);
 
         // The rest of the bucket's work in two forms.  PACKED (pairs whose word fits a key's
@@ -972,11 +984,15 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
 
             // ---- counts -> bin starts (exclusive prefix over the bins), and the fullest bin
             {
-                uint32_t words[WORDS];
+                uint32_t words[WORDS] = {};
                 uint32_t sum = 0, fullest = 0;
+                const bool in_use = !kNarrow || tid * WORDS < used_words;
+                if (in_use) {
+#pragma unroll
+                    for (int i = 0; i < WORDS; ++i) words[i] = sm.bins[tid * WORDS + i];
+                }
 #pragma unroll
                 for (int i = 0; i < WORDS; ++i) {
-                    words[i] = sm.bins[tid * WORDS + i];
                     const uint32_t c0 = words[i] & 0xffffu, c1 = words[i] >> 16;
                     sum += c0 + c1;
                     fullest = c0 > fullest ? c0 : fullest;
@@ -989,11 +1005,13 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
                 __syncthreads();
                 uint32_t run = incl - sum;
                 for (int i = 0; i < w; ++i) run += sm.red32[i];
+                if (in_use) {
 #pragma unroll
-                for (int i = 0; i < WORDS; ++i) {
-                    const uint32_t c0 = words[i] & 0xffffu, c1 = words[i] >> 16;
-                    sm.bins[tid * WORDS + i] = run | ((run + c0) << 16);
-                    run += c0 + c1;
+                    for (int i = 0; i < WORDS; ++i) {
+                        const uint32_t c0 = words[i] & 0xffffu, c1 = words[i] >> 16;
+                        sm.bins[tid * WORDS + i] = run | ((run + c0) << 16);
+                        run += c0 + c1;
+                    }
                 }
             }
             __syncthreads();
