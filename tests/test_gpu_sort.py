@@ -338,6 +338,33 @@ def test_float_rows_either_side_of_zero_close_the_gap_between_their_images(hip_b
     assert bool((d[:, 1:] <= d[:, :-1]).all())
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.float32, np.int64])
+def test_buckets_of_narrow_and_of_wide_keys_in_turn(hip_backend, dtype):
+    """A bucket whose keys differ in fewer bits than the finishing workgroup has counting bins uses
+    (scans, clears) only the first of them; buckets of full-width keys use all.  Rows that mix
+    the two kinds - so that one workgroup meets them in turn - and rows of every width from one
+    bit up, keys only and with indices, against numpy."""
+    n = 60000
+    widths = [1, 3, 5, 8, 11, 12, 13, 20]
+    rows = np.stack([randint(370 + w, n, 0, 1 << w) for w in widths]).astype(np.int64)
+    wide = full_range_i64(371, 3 * n).reshape(3, n) >> (33 if np.dtype(dtype).itemsize == 4 else 1)
+    mixed = wide.copy()
+    mixed[0, ::2] = randint(372, n // 2, 0, 50)                          # every other key one of 50 values
+    mixed[1, : n // 2] = randint(373, n // 2, 1000, 1004)                # half the row four values, the rest wide
+    mixed[2, n // 3:] = (mixed[2, n // 3:] >> 12) << 12                  # low bits all zero in two thirds
+    raw = np.concatenate([rows, mixed, wide[:1]])
+    x = raw.astype(dtype)
+    Xh = Tensor.from_numpy(hip_backend, x)
+    want = np.sort(x, axis=-1)
+    for _ in range(2):                                                    # a second call over the same scratch
+        assert np.array_equal(F.sort(Xh, -1).numpy(), want)
+        assert np.array_equal(F.sort(Xh, -1, True).numpy(), want[:, ::-1])
+    order = np.argsort(x, axis=-1, kind="stable")
+    Yh, Ih = F.argsort(Xh, -1, False, with_values=True)
+    assert np.array_equal(Ih.numpy(), order)
+    assert np.array_equal(Yh.numpy(), want)
+
+
 @pytest.mark.parametrize("dtype", [np.int64, np.float32])
 def test_rows_beyond_a_million_keys_take_the_largest_buckets(hip_backend, dtype):
     """Rows longer than 1.1 M keys are cut into buckets of up to 10240 keys, finished by workgroups
