@@ -432,13 +432,23 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
     uint32_t cnt[PER];
 #pragma unroll
     for (int i = 0; i < PER; ++i) cnt[i] = 0;
-    for (int64_t c = 0; c < chunks_per_row; ++c) {
+    auto chunk_words = [&](int64_t c, uint32_t (&w)[PER / 2]) __attribute__((always_inline)) {
         const uint4 a = reinterpret_cast<const uint4*>(f + c * (kFine / 2))[0], b = reinterpret_cast<const uint4*>(f + c * (kFine / 2))[1];
-        const uint32_t w[PER / 2] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w; w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w;
+    };
+    for (int64_t c0 = 0; c0 < chunks_per_row; c0 += 4) {             // four chunks' loads in flight
+        uint32_t w[4][PER / 2];
 #pragma unroll
-        for (int i = 0; i < PER / 2; ++i) {
-            cnt[2 * i] += w[i] & 0xffffu;
-            cnt[2 * i + 1] += w[i] >> 16;
+        for (int j = 0; j < 4; ++j)
+            if (c0 + j < chunks_per_row) chunk_words(c0 + j, w[j]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (c0 + j >= chunks_per_row) break;
+#pragma unroll
+            for (int i = 0; i < PER / 2; ++i) {
+                cnt[2 * i] += w[j][i] & 0xffffu;
+                cnt[2 * i + 1] += w[j][i] >> 16;
+            }
         }
     }
     uint32_t sum = 0, biggest = 0;
@@ -529,39 +539,48 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
         for (int64_t i = threadIdx.x; i < left.status_words / 4; i += kSplitBlock) status[i] = make_uint4(0u, 0u, 0u, 0u);
         return;
     }
-    // a bin opens every bucket after its predecessor's up to its own
+    // a bin opens every bucket after its predecessor's up to its own (the starts are put together
+    // in LDS: the threads read one another's just below)
+    __shared__ uint32_t begin[kMaxBuckets + 1];
     {
         uint32_t prev_bucket = threadIdx.x == 0 ? 0u : last_bucket[threadIdx.x - 1];
-        if (threadIdx.x == 0) info.begin[0] = 0u;
+        if (threadIdx.x == 0) begin[0] = 0u;
         uint32_t run = before;
+        uint32_t packed[PER / 4];                     // this thread's 16 table bytes: one store
+#pragma unroll
+        for (int i = 0; i < PER / 4; ++i) packed[i] = 0u;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            info.bucket_of[threadIdx.x * PER + i] = static_cast<uint8_t>(bucket[i]);
-            for (uint32_t k = prev_bucket + 1; k <= bucket[i]; ++k) info.begin[k] = run;
+            packed[i / 4] |= bucket[i] << (8 * (i % 4));
+            for (uint32_t k = prev_bucket + 1; k <= bucket[i]; ++k) begin[k] = run;
             prev_bucket = bucket[i];
             run += cnt[i];
         }
+        static_assert(PER == 16 && offsetof(SplitRow, bucket_of) % 16 == 0, "a thread's bins are one aligned 16-byte piece of the table");
+        reinterpret_cast<uint4*>(info.bucket_of)[threadIdx.x] = make_uint4(packed[0], packed[1], packed[2], packed[3]);
     }
     if (threadIdx.x == kSplitBlock - 1) {
         info.n_buckets = n_buckets;
-        info.begin[n_buckets] = static_cast<uint32_t>(n);
+        begin[n_buckets] = static_cast<uint32_t>(n);
         info.route = 1u;
         listed[0] = n_buckets;
         listed[1] = atomicAdd(&counters[2], n_buckets);
     }
     per_bucket[threadIdx.x] = 0u;
     __syncthreads();
+    for (uint32_t k = threadIdx.x; k <= n_buckets; k += kSplitBlock) info.begin[k] = begin[k];
     // the buckets of every such row, in no particular order: what split_finish walks
     uint32_t next = 0;                                 // where the coming chunk's keys of bucket threadIdx.x go
     if (threadIdx.x < listed[0]) {
-        const uint32_t b0 = info.begin[threadIdx.x], b1 = info.begin[threadIdx.x + 1];
+        const uint32_t b0 = begin[threadIdx.x], b1 = begin[threadIdx.x + 1];
         bucket_list[listed[1] + threadIdx.x] = make_uint4(static_cast<uint32_t>(row), b0, b1 - b0, static_cast<uint32_t>(row) * kMaxBuckets + threadIdx.x);
         next = b0;
     }
     // each chunk's keys per bucket, and from them where the chunk writes each bucket
+    uint32_t w[PER / 2], ahead[PER / 2];
+    chunk_words(0, w);
     for (int64_t c = 0; c < chunks_per_row; ++c) {
-        const uint4 a = reinterpret_cast<const uint4*>(f + c * (kFine / 2))[0], b = reinterpret_cast<const uint4*>(f + c * (kFine / 2))[1];
-        const uint32_t w[PER / 2] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        if (c + 1 < chunks_per_row) chunk_words(c + 1, ahead);        // on its way across this chunk's barriers
         // this thread's bins lie in few buckets: sum runs of equal buckets before touching LDS
         uint32_t acc = 0;
 #pragma unroll
@@ -577,6 +596,8 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
         next += per_bucket[threadIdx.x];
         per_bucket[threadIdx.x] = 0u;
         __syncthreads();
+#pragma unroll
+        for (int i = 0; i < PER / 2; ++i) w[i] = ahead[i];
     }
 }
 
