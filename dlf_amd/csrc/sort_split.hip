@@ -194,6 +194,34 @@ __device__ __forceinline__ T block_reduce(T v, Join join, T* lds, int waves) {
     return r;
 }
 
+// The fourth smallest (SMALLEST) or fourth largest of the 256 keys a wavefront holds, four a
+// lane: the best is found and one instance of it struck out, three times over, and the best of
+// what is left is the answer (a full sort of the 256 keys cost three times as much).
+template <bool SMALLEST, typename K>
+__device__ __forceinline__ K wave_fourth(const K (&key)[4]) {
+    constexpr K out = SMALLEST ? ~K(0) : K(0);         // a struck-out entry: never better than a key
+    auto better = [](K a, K b) { return SMALLEST ? (a < b ? a : b) : (a > b ? a : b); };
+    K left[4] = {key[0], key[1], key[2], key[3]};
+    K best = out;
+#pragma unroll
+    for (int round = 0; round < 4; ++round) {
+        const K mine = better(better(left[0], left[1]), better(left[2], left[3]));
+        best = wave_reduce(mine, better);
+        if (round == 3) break;
+        const unsigned long long holders = __ballot(mine == best);
+        if (lane_id() == __ffsll(static_cast<long long>(holders)) - 1) {     // the first lane that holds it strikes one out
+            bool struck = false;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const bool hit = !struck && left[u] == best;
+                left[u] = hit ? out : left[u];
+                struck = struck || hit;
+            }
+        }
+    }
+    return best;
+}
+
 // ------------------------------------------------------------------ 1. the range of a row's keys
 // MAP (the host knows): 0 for rows spread by key image and nothing else (integers, short float
 // rows); 1 for float rows of middling length, whose images may have the gap around zero closed
@@ -211,7 +239,6 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
     // evenly spaced places, the last of them the row's last keys, so that a sorted row shows
     // its whole range
     K key[4];
-    uint32_t unused[4] = {0u, 0u, 0u, 0u};
     int64_t e0 = (static_cast<int64_t>(threadIdx.x) * n) / kSplitBlock;
     if (threadIdx.x == kSplitBlock - 1 || e0 > n - 4) e0 = n - 4;
 #pragma unroll
@@ -220,17 +247,21 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
         const int64_t e = n >= 1024 ? e0 + u : (j < n ? j : n - 1);
         key[u] = key_of_element<K>(io, xrow[e * io.sx]);
     }
-    // every wave orders its 256 keys and offers its 4th smallest and 4th largest: three stray
-    // keys per wave at either end (a few zeros among positive values, a few huge ones) do not
-    // stretch the range the fine bins resolve
-    wave_bitonic_items<false, 4>(key, unused, [](K ka, uint32_t, K kb, uint32_t) { return ka < kb; });
-    K lo = lane_read(key[0], 3), hi = lane_read(key[3], kWave - 4);
+    // every wave offers the 4th smallest and the 4th largest of its 256 keys: three stray keys
+    // per wave at either end (a few zeros among positive values, a few huge ones) do not stretch
+    // the range the fine bins resolve
+    auto smaller = [](K a, K b) { return a < b ? a : b; };
+    auto larger = [](K a, K b) { return a > b ? a : b; };
+    K lo, hi;
     if (n < 64) {                                      // too few keys for that: the plain range
-        lo = lane_read(key[0], 0);
-        hi = lane_read(key[3], kWave - 1);
+        lo = wave_reduce(smaller(smaller(key[0], key[1]), smaller(key[2], key[3])), smaller);
+        hi = wave_reduce(larger(larger(key[0], key[1]), larger(key[2], key[3])), larger);
+    } else {
+        lo = wave_fourth<true>(key);
+        hi = wave_fourth<false>(key);
     }
-    lo = block_reduce(lo, [](K a, K b) { return a < b ? a : b; }, red, kSplitBlock / kWave);
-    hi = block_reduce(hi, [](K a, K b) { return a > b ? a : b; }, red, kSplitBlock / kWave);
+    lo = block_reduce(lo, smaller, red, kSplitBlock / kWave);
+    hi = block_reduce(hi, larger, red, kSplitBlock / kWave);
     // Float rows: the images of negative and of positive values lie either side of the middle
     // of the key range, those of the smallest magnitudes next to it and the two zeros at it.
     // Every wave offers the nearest of its keys below the zeros and the nearest above them; the
@@ -239,18 +270,14 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
     K gap_lo = ~K(0), gap_hi = ~K(0);
     if constexpr (MAP == kMapGap) {
         constexpr K zero_hi = K(1) << (8 * sizeof(K) - 1), zero_lo = zero_hi - 1;      // keys of +0.0 and -0.0 (either way round)
-        int below = 0, upto = 0;                       // entries 0 .. below - 1 lie under the zeros, entries from upto on above them
+        K under_mine = K(0), over_mine = ~K(0);        // this lane's nearest key below the zeros, and above them
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            below += __popcll(__ballot(key[u] < zero_lo));
-            upto += __popcll(__ballot(key[u] <= zero_hi));
+            if (key[u] < zero_lo) under_mine = larger(under_mine, key[u]);
+            if (key[u] > zero_hi) over_mine = smaller(over_mine, key[u]);
         }
-        auto entry = [&](int at) {                     // at: the same in every lane
-            const K mine = at < kWave ? key[0] : at < 2 * kWave ? key[1] : at < 3 * kWave ? key[2] : key[3];
-            return lane_read(mine, at % kWave);
-        };
         __shared__ K near[2][kSplitBlock / kWave];
-        const K wave_under = below >= 1 ? entry(below - 1) : K(0), wave_over = upto < 4 * kWave ? entry(upto) : ~K(0);
+        const K wave_under = wave_reduce(under_mine, larger), wave_over = wave_reduce(over_mine, smaller);
         if (lane_id() == 0) {
             near[0][threadIdx.x / kWave] = wave_under;
             near[1][threadIdx.x / kWave] = wave_over;
