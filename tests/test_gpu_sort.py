@@ -300,7 +300,7 @@ def test_float_rows_spread_by_value_or_by_image(hip_backend, dtype, n):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-@pytest.mark.parametrize("n", [31000, 65536, 131072])
+@pytest.mark.parametrize("n", [30720, 31000, 65536, 131072])
 def test_float_rows_either_side_of_zero_close_the_gap_between_their_images(hip_backend, dtype, n):
     """Float rows of 30 720 to 131 072 elements with values on both sides of zero leave the images
     between their smallest negative and positive magnitudes out of the fine bins.  Rows where that
