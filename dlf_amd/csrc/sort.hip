@@ -1,7 +1,7 @@
 // sort / argsort along the last axis of strided views for gfx950.
 //
 // Which way a row goes: rows of up to 64 / 512 elements are sorted by one wavefront in
-// registers, rows of up to 4096 by one workgroup on chip, longer rows of 4- and 8-byte keys by
+// registers, rows of up to 4096 (16-bit keys) or 8192 by one workgroup on chip, longer rows of 4- and 8-byte keys by
 // the bucket route of sort_split.hip (run_split below enqueues it first; every row decides on
 // the device whether it can take it).  What is left - rows the bucket route cannot take,
 // 16-bit keys - is sorted here:
@@ -548,18 +548,18 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
 }
 
 // ------------------------------------------------------------------ rows that fit one workgroup
-// A row of at most 256 * ITEMS keys is read once, sorted through all its passes in LDS and
+// A row of at most 64 * WAVES * ITEMS keys is read once, sorted through all its passes in LDS and
 // registers and written once: no histogram pass, no scratch traffic, no chaining between
 // tiles.  The passes are those of sort_pass without the parts that connect tiles: rank inside
-// the wave with ballots over the digit bits that vary in the row, digit starts from the four
-// waves' counts, scatter through LDS, reload in element order.  Digits that are the same in
+// the wave with ballots over the digit bits that vary in the row, digit starts from the
+// waves' counts (four waves, or eight for rows beyond 4096 keys), scatter through LDS, reload in element order.  Digits that are the same in
 // the whole row are skipped.  Element e of the row is item e / 64 % ITEMS of lane e % 64 of
 // wave e / (64 * ITEMS), before and after every pass.
-template <typename K, bool PAIRS, int ITEMS>
-__global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t rows, int64_t n) {
+template <typename K, bool PAIRS, int ITEMS, int WAVES = 4>
+__global__ __launch_bounds__(WAVES * kWave) void sort_rows_small(PassIo<K> io, int64_t rows, int64_t n) {
     constexpr int P = KeyTraits<K>::kPasses;
     static_assert(ITEMS % 2 == 0, "items are ranked in pairs");
-    __shared__ SmallShared<K, PAIRS, ITEMS> sm;
+    __shared__ SmallShared<K, PAIRS, ITEMS, WAVES> sm;
     const int tid = threadIdx.x;
     const int lane = lane_id();
     const int w = tid / kWave;
@@ -583,7 +583,7 @@ __global__ __launch_bounds__(256) void sort_rows_small(PassIo<K> io, int64_t row
         }
         if constexpr (PAIRS) val[k] = static_cast<uint32_t>(e);
     }
-    sort_in_workgroup<K, PAIRS, ITEMS>(sm, key, val, ors, ands, valid, P);
+    sort_in_workgroup<K, PAIRS, ITEMS, WAVES>(sm, key, val, ors, ands, valid, P);
 
     // ---- write
     if (io.y) {
@@ -765,7 +765,11 @@ __global__ __launch_bounds__(256) void sort_cols_wave(PassIo<K> io, int64_t rows
 // longest row sorted by one wavefront (dlfx_set_tuning "sort_wave_rows": 64, 128, 256 or 512)
 int g_sort_wave_rows = 512;
 
-constexpr int64_t kSmallRow = 4096;      // longest row sort_rows_small takes
+// longest row sort_rows_small takes: four wavefronts hold 4096 keys, eight hold 8192 (4- and
+// 8-byte keys: [4096, 8192] fp32 sorts in 245 us against 485 us by the bucket route, argsort
+// 260 against 590; int64 235 against 280, argsort 260 against 340; sixteen wavefronts with
+// 16384 4-byte keys only win when the row fills them)
+constexpr int64_t small_row(size_t key_size) { return key_size >= 4 ? 8192 : 4096; }
 
 int g_sort_buckets = 1;                  // 1: rows the bucket route takes go that way (dlfx_set_tuning "sort_buckets")
 int g_sort_compare_max = 96;             // fullest counting bin of a bucket that is still ranked by comparison
@@ -799,7 +803,14 @@ int launch_small(hipStream_t stream, const PassIo<K>& io_in, int64_t m, int64_t 
     else if (n <= 512) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 2><<<g, block, 0, stream>>>(io, m, n); }
     else if (n <= 1024) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 4><<<g, block, 0, stream>>>(io, m, n); }
     else if (n <= 2048) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 8><<<g, block, 0, stream>>>(io, m, n); }
-    else { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 16><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 4096) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 16><<<g, block, 0, stream>>>(io, m, n); }
+    else if constexpr (sizeof(K) >= 4) {
+        // eight wavefronts, 10, 12 or 16 keys a thread: 5120, 6144 or 8192 slots
+        const dim3 g = grid_for(1), wide(8 * kWave);
+        if (n <= 5120) sort_rows_small<K, PAIRS, 10, 8><<<g, wide, 0, stream>>>(io, m, n);
+        else if (n <= 6144) sort_rows_small<K, PAIRS, 12, 8><<<g, wide, 0, stream>>>(io, m, n);
+        else sort_rows_small<K, PAIRS, 16, 8><<<g, wide, 0, stream>>>(io, m, n);
+    }
     DLFX_CHECK_LAUNCH();
     return DLFX_OK;
 }
@@ -831,7 +842,7 @@ SortLayout sort_layout(size_t key_size, bool pairs, int64_t m, int64_t n) {
     l.status_bytes = l.tiles_per_row > 1 ? static_cast<size_t>(m) * l.tiles_per_row * kRadix * 4 : 0;
     off += align_up(l.status_bytes, 256);
     l.split_off = off;           // tables of the bucket route (rows longer than one workgroup sorts on chip)
-    l.split_bytes = (n > kSmallRow && split_route_takes(key_size, m, n)) ? split_scratch_bytes(key_size, pairs, m, n) : 0;
+    l.split_bytes = (n > small_row(key_size) && split_route_takes(key_size, m, n)) ? split_scratch_bytes(key_size, pairs, m, n) : 0;
     off += align_up(l.split_bytes, 256);
     for (int i = 0; i < 2; ++i) {
         l.keys_off[i] = off;
@@ -907,7 +918,7 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     // (one row's output over another row's input) takes the general path.
     bool same_view = a.y == a.x;
     for (int i = 0; i < a.rank && same_view; ++i) same_view = a.xs[i] == a.ys[i] || a.dims[i] == 1;
-    if (n <= kSmallRow && (!y_over_x || same_view)) {
+    if (n <= small_row(sizeof(K)) && (!y_over_x || same_view)) {
         if (m > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
         return a.pairs ? launch_small<K, true>(stream, io, m, n) : launch_small<K, false>(stream, io, m, n);
     }
