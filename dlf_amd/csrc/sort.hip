@@ -1,7 +1,8 @@
 // sort / argsort along the last axis of strided views for gfx950.
 //
 // Which way a row goes: rows of up to 64 / 512 elements are sorted by one wavefront in
-// registers, rows of up to 4096 (16-bit keys) or 8192 by one workgroup on chip, longer rows of 4- and 8-byte keys by
+// registers, rows of up to 4096 (16-bit keys), 8192 (8-byte) or 16384 (4-byte keys) by one workgroup
+// on chip, longer rows of 4- and 8-byte keys by
 // the bucket route of sort_split.hip (run_split below enqueues it first; every row decides on
 // the device whether it can take it).  What is left - rows the bucket route cannot take,
 // 16-bit keys - is sorted here:
@@ -552,7 +553,7 @@ __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX
 // registers and written once: no histogram pass, no scratch traffic, no chaining between
 // tiles.  The passes are those of sort_pass without the parts that connect tiles: rank inside
 // the wave with ballots over the digit bits that vary in the row, digit starts from the
-// waves' counts (four waves, or eight for rows beyond 4096 keys), scatter through LDS, reload in element order.  Digits that are the same in
+// waves' counts (four waves; eight or sixteen for rows beyond 4096 keys), scatter through LDS, reload in element order.  Digits that are the same in
 // the whole row are skipped.  Element e of the row is item e / 64 % ITEMS of lane e % 64 of
 // wave e / (64 * ITEMS), before and after every pass.
 template <typename K, bool PAIRS, int ITEMS, int WAVES = 4>
@@ -767,9 +768,10 @@ int g_sort_wave_rows = 512;
 
 // longest row sort_rows_small takes: four wavefronts hold 4096 keys, eight hold 8192 (4- and
 // 8-byte keys: [4096, 8192] fp32 sorts in 245 us against 485 us by the bucket route, argsort
-// 260 against 590; int64 235 against 280, argsort 260 against 340; sixteen wavefronts with
-// 16384 4-byte keys only win when the row fills them)
-constexpr int64_t small_row(size_t key_size) { return key_size >= 4 ? 8192 : 4096; }
+// 260 against 590; int64 235 against 280, argsort 260 against 340), sixteen hold 16384 4-byte
+// keys ([2048, 16384] fp32 301 against 362 us, argsort 355 against 434; [2796, 12000] 333
+// against 401; int32 the same within 5 %)
+constexpr int64_t small_row(size_t key_size) { return key_size == 4 ? 16384 : key_size == 8 ? 8192 : 4096; }
 
 int g_sort_buckets = 1;                  // 1: rows the bucket route takes go that way (dlfx_set_tuning "sort_buckets")
 int g_sort_compare_max = 96;             // fullest counting bin of a bucket that is still ranked by comparison
@@ -805,11 +807,19 @@ int launch_small(hipStream_t stream, const PassIo<K>& io_in, int64_t m, int64_t 
     else if (n <= 2048) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 8><<<g, block, 0, stream>>>(io, m, n); }
     else if (n <= 4096) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 16><<<g, block, 0, stream>>>(io, m, n); }
     else if constexpr (sizeof(K) >= 4) {
-        // eight wavefronts, 10, 12 or 16 keys a thread: 5120, 6144 or 8192 slots
+        // eight wavefronts, 10, 12 or 16 keys a thread: 5120, 6144 or 8192 slots; sixteen for 4-byte
+        // keys beyond that, 10, 12, 14 or 16 keys a thread: 10240, 12288, 14336 or 16384 slots
         const dim3 g = grid_for(1), wide(8 * kWave);
         if (n <= 5120) sort_rows_small<K, PAIRS, 10, 8><<<g, wide, 0, stream>>>(io, m, n);
         else if (n <= 6144) sort_rows_small<K, PAIRS, 12, 8><<<g, wide, 0, stream>>>(io, m, n);
-        else sort_rows_small<K, PAIRS, 16, 8><<<g, wide, 0, stream>>>(io, m, n);
+        else if (n <= 8192) sort_rows_small<K, PAIRS, 16, 8><<<g, wide, 0, stream>>>(io, m, n);
+        else if constexpr (sizeof(K) == 4) {
+            const dim3 widest(16 * kWave);
+            if (n <= 10240) sort_rows_small<K, PAIRS, 10, 16><<<g, widest, 0, stream>>>(io, m, n);
+            else if (n <= 12288) sort_rows_small<K, PAIRS, 12, 16><<<g, widest, 0, stream>>>(io, m, n);
+            else if (n <= 14336) sort_rows_small<K, PAIRS, 14, 16><<<g, widest, 0, stream>>>(io, m, n);
+            else sort_rows_small<K, PAIRS, 16, 16><<<g, widest, 0, stream>>>(io, m, n);
+        }
     }
     DLFX_CHECK_LAUNCH();
     return DLFX_OK;

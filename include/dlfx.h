@@ -79,9 +79,10 @@ int dlfx_last_hip_error(void);
  *                      (default 2048; 0 makes every tile help itself at once).
  *   "sort_poll_limit"  the same bound for the per-digit tile chaining of a radix pass.
  *   "sort_wave_rows"   longest row (64, 128, 256 or 512; default 512) sorted by one wavefront
- *                      in registers; longer rows of up to 8192 elements (16-bit keys: 4096) take
- *                      one workgroup.
- *   "sort_buckets"     1 (default): rows of 4- and 8-byte keys longer than 8192 elements are cut into
+ *                      in registers; longer rows of up to 16384 elements (8-byte keys: 8192,
+ *                      16-bit keys: 4096) take one workgroup.
+ *   "sort_buckets"     1 (default): rows of 4-byte keys longer than 16384 elements and of 8-byte
+ *                      keys longer than 8192 are cut into
  *                      buckets of equal depth by value and each bucket is sorted on chip, wherever
  *                      a row's keys allow it (each row decides on the device); 0: every row takes
  *                      the least-significant-digit-first passes.  Same results either way.

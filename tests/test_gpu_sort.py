@@ -162,7 +162,7 @@ def test_rows_leave_out_passes_that_move_nothing(hip_backend, oracle_backend, dt
 
 
 @pytest.mark.parametrize("dtype", [np.int64, np.float32, np.int32, np.float64])
-@pytest.mark.parametrize("n", [5000, 9000, 40000, 150000, 300000, 600000, 1 << 20])
+@pytest.mark.parametrize("n", [5000, 9000, 17000, 40000, 150000, 300000, 600000, 1 << 20])
 def test_long_rows_cut_into_buckets(hip_backend, dtype, n):
     """Rows longer than one workgroup sorts are cut into buckets of equal depth by value and
     each bucket is finished on chip; rows whose keys do not allow that (one value taking more
@@ -228,7 +228,7 @@ def test_long_rows_cut_into_buckets(hip_backend, dtype, n):
 
 
 @pytest.mark.parametrize("dtype", [np.int64, np.float64, np.int32, np.float32])
-@pytest.mark.parametrize("n", [9000, 40000, 300000])
+@pytest.mark.parametrize("n", [9000, 17000, 40000, 300000])
 def test_buckets_ranked_by_comparison_or_by_digit_passes(hip_backend, dtype, n):
     """A bucket whose counting bins are crowded (many equal or clustered keys) is finished by the
     stable digit passes - for argsort first by index, then by key - instead of by comparing the
@@ -469,13 +469,13 @@ def test_nans_take_the_place_of_their_bit_pattern(hip_backend, dtype):
 
 
 @pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8, 9, 16, 17, 32, 33, 63, 64, 65, 100, 127, 128, 129, 255, 256, 257, 300, 511, 512, 513, 1023, 1024, 1025, 2047, 2048, 2049, 4095,
-                               4096, 4097, 5119, 5120, 5121, 6144, 6145, 8191, 8192, 8193])
+                               4096, 4097, 5119, 5120, 5121, 6144, 6145, 8191, 8192, 8193, 10240, 10241, 12288, 12289, 14336, 14337, 16383, 16384, 16385])
 def test_rows_around_the_one_workgroup_limits(hip_backend, oracle_backend, n):
     """Rows of up to 64, 128, 256 (512 for values only or 8-byte keys) elements are sorted by one
-    wavefront in registers, rows of up to 4096 elements - 8192 for 4- and 8-byte keys - by one
-    workgroup on chip (512, 1024, 2048, 4096, 5120, 6144 or 8192 slots); longer rows take the tiled
-    passes or the bucket route.  Every boundary, all key widths, both directions, values, indices
-    (32- and 64-bit) and in place."""
+    wavefront in registers, rows of up to 4096 elements - 8192 for 8-byte keys, 16384 for 4-byte
+    keys - by one workgroup on chip (512 to 16384 slots); longer rows take the tiled passes or the
+    bucket route.  Every boundary, all key widths, both directions, values, indices (32- and
+    64-bit) and in place."""
     for dtype in (np.float32, np.int64, np.float64, np.int16, np.float16, np.int32):
         x = (normal(200 + n, 5 * n) * 50).astype(dtype).reshape(5, n)
         x[1] = x[1, 0]                                   # a constant row: no pass runs
