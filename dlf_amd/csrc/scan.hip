@@ -201,7 +201,8 @@ template <typename T, int K, int ITEMS, bool CHAINED, bool SELF_HELP, int BLOCK 
 __device__ __forceinline__ void scan_tile(
     const X* __restrict__ x, Y* __restrict__ y, const DimMap& xmap, const DimMap& ymap, int64_t sx, int64_t sy,
     const DimMap& xaxis, int64_t n, int64_t tiles_per_row, int exclusive, int64_t row, int64_t t, int poll_limit,
-    TileState<T>& st, RowScanShared<T>& sm, const ClearedBy& cb = ClearedBy{nullptr, 0ull}, unsigned long long ready_early = 0ull) {
+    TileState<T>& st, RowScanShared<T>& sm, const ClearedBy& cb = ClearedBy{nullptr, 0ull}, unsigned long long ready_early = 0ull,
+    int pad = 0) {
     // where element i of a row lives: i * sx, or (scan_nonzero over a flattened view whose
     // dimensions do not merge) wherever the row-major walk of `xaxis` puts it
     auto x_at = [&](int64_t i) -> int64_t {
@@ -220,15 +221,21 @@ __device__ __forceinline__ void scan_tile(
 
     const X* xr = x + xmap.at(row);
     Y* yr = y + ymap.at(row);
+    // A unit-stride row that does not start on a vector boundary (pad != 0: the host found such
+    // rows) is tiled from the boundary before it: position j of that tiling is element
+    // j - shift of the row, positions below `shift` hold the identity, and every whole vector
+    // of the row is aligned in memory.  Elsewhere shift is 0 and positions are elements.
+    const int shift = pad ? static_cast<int>((reinterpret_cast<uintptr_t>(xr) / sizeof(X)) % V) : 0;
+    const int64_t n_pos = n + shift;                       // positions of the row: [shift, n_pos)
     const int64_t seg = tile_base + static_cast<int64_t>(w) * kWave * ITEMS;
 
     // ---- load
     T vals[ITEMS];
-    // whole vectors of an aligned unit-stride row move as one access; the row's last, partial
-    // vector (and what lies past the row in its last tile) element by element
-    const bool x_vec = sx == 1 && (reinterpret_cast<uintptr_t>(xr + seg) % (sizeof(X) * V) == 0);
-    const VecX* pv = reinterpret_cast<const VecX*>(xr + seg);
-    const bool full = n - tile_base >= TILE;               // every element of the tile lies in the row
+    // whole vectors of an aligned unit-stride row move as one access; the row's first and last,
+    // partial vectors (and what lies past the row in its last tile) element by element
+    const bool x_vec = sx == 1 && (reinterpret_cast<uintptr_t>(xr - shift + seg) % (sizeof(X) * V) == 0);
+    const VecX* pv = reinterpret_cast<const VecX*>(xr - shift + seg);
+    const bool full = tile_base >= shift && n_pos - tile_base >= TILE;      // every position of the tile is an element of the row
     if (full && x_vec) {
         // the common case apart: all loads issued back to back, nothing to test per vector
 #pragma unroll
@@ -241,13 +248,14 @@ __device__ __forceinline__ void scan_tile(
 #pragma unroll
     for (int k = 0; k < KV; ++k) {
         const int64_t i0 = seg + static_cast<int64_t>(k * kWave + lane) * V;
-        if (x_vec && i0 + V <= n) {
+        if (x_vec && i0 >= shift && i0 + V <= n_pos) {
             VecX a = load_stream(&pv[k * kWave + lane]);
 #pragma unroll
             for (int e = 0; e < V; ++e) vals[k * V + e] = scan_input<T, X, NZ>(a.v[e]);
         } else {
 #pragma unroll
-            for (int e = 0; e < V; ++e) vals[k * V + e] = (i0 + e < n) ? scan_input<T, X, NZ>(xr[x_at(i0 + e)]) : Op::identity();
+            for (int e = 0; e < V; ++e)
+                vals[k * V + e] = (i0 + e >= shift && i0 + e < n_pos) ? scan_input<T, X, NZ>(xr[x_at(i0 + e - shift)]) : Op::identity();
         }
     }
     // ---- scan inside the wave: vals[] become inclusive prefixes within the wave segment
@@ -325,10 +333,11 @@ __device__ __forceinline__ void scan_tile(
                         while (stuck != 0ull) {
                             const int l = __ffsll(static_cast<long long>(stuck)) - 1;
                             stuck &= stuck - 1;
-                            const int64_t pbase = (pos - l) * TILE;
-                            const int64_t cnt = (n - pbase < TILE) ? n - pbase : TILE;
+                            const int64_t pfirst = (pos - l) * TILE;                       // positions [pfirst, pfirst + TILE)
+                            const int64_t pbase = pfirst > shift ? pfirst - shift : 0;     // elements [pbase, pend)
+                            const int64_t pend = pfirst + TILE - shift < n ? pfirst + TILE - shift : n;
                             T a = Op::identity();
-                            for (int64_t i = lane; i < cnt; i += kWave) a = Op::apply(a, scan_input<T, X, NZ>(xr[x_at(pbase + i)]));
+                            for (int64_t i = pbase + lane; i < pend; i += kWave) a = Op::apply(a, scan_input<T, X, NZ>(xr[x_at(i)]));
                             a = wave_reduce(a, [](T p, T q) { return Op::apply(p, q); });
                             if (lane == l) {
                                 v = a;
@@ -372,8 +381,8 @@ __device__ __forceinline__ void scan_tile(
     for (int i = 0; i < ITEMS; ++i) vals[i] = Op::apply(pre, vals[i]);
 
     using VecY = Vec<Y, V>;
-    const bool y_vec = sy == 1 && (reinterpret_cast<uintptr_t>(yr + seg) % (sizeof(Y) * V) == 0);
-    VecY* qv = reinterpret_cast<VecY*>(yr + seg);
+    const bool y_vec = sy == 1 && (reinterpret_cast<uintptr_t>(yr - shift + seg) % (sizeof(Y) * V) == 0);
+    VecY* qv = reinterpret_cast<VecY*>(yr - shift + seg);
     if (full && y_vec) {
 #pragma unroll
         for (int k = 0; k < KV; ++k) {
@@ -386,7 +395,7 @@ __device__ __forceinline__ void scan_tile(
 #pragma unroll
     for (int k = 0; k < KV; ++k) {
         const int64_t i0 = seg + static_cast<int64_t>(k * kWave + lane) * V;
-        if (y_vec && i0 + V <= n) {
+        if (y_vec && i0 >= shift && i0 + V <= n_pos) {
             VecY a;
 #pragma unroll
             for (int e = 0; e < V; ++e) a.v[e] = static_cast<Y>(vals[k * V + e]);
@@ -394,7 +403,7 @@ __device__ __forceinline__ void scan_tile(
         } else {
 #pragma unroll
             for (int e = 0; e < V; ++e)
-                if (i0 + e < n) yr[(i0 + e) * sy] = static_cast<Y>(vals[k * V + e]);
+                if (i0 + e >= shift && i0 + e < n_pos) yr[(i0 + e - shift) * sy] = static_cast<Y>(vals[k * V + e]);
         }
     }
 }
@@ -403,10 +412,11 @@ __device__ __forceinline__ void scan_tile(
 template <typename T, int K, int ITEMS, typename X, bool NZ, typename Y>
 __global__ __launch_bounds__(kBlock) void scan_rows_single(
     const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy, DimMap xaxis,
-    int64_t n, int exclusive) {
+    int64_t n, int exclusive, int pad) {
     __shared__ RowScanShared<T> sm;
     TileState<T> st;
-    scan_tile<T, K, ITEMS, false, false, kBlock, X, NZ, Y>(x, y, xmap, ymap, sx, sy, xaxis, n, 1, exclusive, blockIdx.x, 0, 0, st, sm);
+    scan_tile<T, K, ITEMS, false, false, kBlock, X, NZ, Y>(x, y, xmap, ymap, sx, sy, xaxis, n, 1, exclusive, blockIdx.x, 0, 0, st, sm,
+                                                           ClearedBy{nullptr, 0ull}, 0ull, pad);
 }
 
 // Short rows: LANES lanes per row (one lane, a quad, a DPP row of 16 lanes, or a whole wavefront), ITEMS elements
@@ -415,7 +425,7 @@ __global__ __launch_bounds__(kBlock) void scan_rows_single(
 template <typename T, int K, int LANES, int ITEMS, typename X, bool NZ, typename Y>
 __global__ __launch_bounds__(kBlock) void scan_rows_group(
     const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
-    int64_t rows, int64_t n, int exclusive) {
+    int64_t rows, int64_t n, int exclusive, int pad) {
     static_assert(LANES == 1 || LANES == 4 || LANES == 16 || LANES == kWave, "a thread, a quad, a DPP row or a wavefront");
     using Op = ScanOp<T, K>;
     constexpr int V = (scan_vec<T, X, Y>() < ITEMS) ? scan_vec<T, X, Y>() : ITEMS;
@@ -428,23 +438,27 @@ __global__ __launch_bounds__(kBlock) void scan_rows_group(
     const bool live = row < rows;                       // whole groups are live or not
     const X* xr = x + (live ? xmap.at(row) : 0);
     Y* yr = y + (live ? ymap.at(row) : 0);
-    const int64_t count = live ? n : 0;
+    // a row that does not start on a vector boundary (pad != 0: the host found such rows) is laid
+    // out from the boundary before it, as in scan_tile: position e is element e - shift
+    const int shift = pad ? static_cast<int>((reinterpret_cast<uintptr_t>(xr) / sizeof(X)) % V) : 0;
+    const int64_t count = live ? n + shift : 0;            // positions [shift, count) are the row
 
-    // whole vectors of an aligned unit-stride row move as one access, the row's last, partial
-    // vector element by element
-    const bool x_vec = sx == 1 && reinterpret_cast<uintptr_t>(xr) % (sizeof(X) * V) == 0;
-    const bool y_vec = sy == 1 && reinterpret_cast<uintptr_t>(yr) % (sizeof(Y) * V) == 0;
+    // whole vectors of an aligned unit-stride row move as one access, the row's first and last,
+    // partial vectors element by element
+    const bool x_vec = sx == 1 && reinterpret_cast<uintptr_t>(xr - shift) % (sizeof(X) * V) == 0;
+    const bool y_vec = sy == 1 && reinterpret_cast<uintptr_t>(yr - shift) % (sizeof(Y) * V) == 0;
     T vals[ITEMS];
 #pragma unroll
     for (int v = 0; v < KV; ++v) {
         const int64_t e0 = static_cast<int64_t>(v * LANES + l) * V;
-        if (x_vec && e0 + V <= count) {
-            const VecX a = load_stream(reinterpret_cast<const VecX*>(xr + e0));
+        if (x_vec && e0 >= shift && e0 + V <= count) {
+            const VecX a = load_stream(reinterpret_cast<const VecX*>(xr - shift + e0));
 #pragma unroll
             for (int j = 0; j < V; ++j) vals[v * V + j] = scan_input<T, X, NZ>(a.v[j]);
         } else {
 #pragma unroll
-            for (int j = 0; j < V; ++j) vals[v * V + j] = (e0 + j < count) ? scan_input<T, X, NZ>(xr[(e0 + j) * sx]) : Op::identity();
+            for (int j = 0; j < V; ++j)
+                vals[v * V + j] = (e0 + j >= shift && e0 + j < count) ? scan_input<T, X, NZ>(xr[(e0 + j - shift) * sx]) : Op::identity();
         }
     }
     auto combine = [](T a, T b) { return Op::apply(a, b); };
@@ -488,15 +502,15 @@ __global__ __launch_bounds__(kBlock) void scan_rows_group(
 #pragma unroll
     for (int v = 0; v < KV; ++v) {
         const int64_t e0 = static_cast<int64_t>(v * LANES + l) * V;
-        if (y_vec && e0 + V <= count) {
+        if (y_vec && e0 >= shift && e0 + V <= count) {
             VecY a;
 #pragma unroll
             for (int j = 0; j < V; ++j) a.v[j] = static_cast<Y>(vals[v * V + j]);
-            store_stream(reinterpret_cast<VecY*>(yr + e0), a);
+            store_stream(reinterpret_cast<VecY*>(yr - shift + e0), a);
         } else {
 #pragma unroll
             for (int j = 0; j < V; ++j)
-                if (e0 + j < count) yr[(e0 + j) * sy] = static_cast<Y>(vals[v * V + j]);
+                if (e0 + j >= shift && e0 + j < count) yr[(e0 + j - shift) * sy] = static_cast<Y>(vals[v * V + j]);
         }
     }
 }
@@ -508,7 +522,7 @@ __global__ __launch_bounds__(kBlock) void scan_rows_group(
 template <typename T, int K, int ITEMS, bool TICKET, int BLOCK, typename X, bool NZ, typename Y>
 __global__ __launch_bounds__(BLOCK) void scan_rows_chained(
     const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy, DimMap xaxis,
-    int64_t n, int64_t tiles_per_row, int exclusive, int poll_limit, unsigned* ticket, TileState<T> st, ClearedBy cb) {
+    int64_t n, int64_t tiles_per_row, int exclusive, int poll_limit, unsigned* ticket, TileState<T> st, ClearedBy cb, int pad) {
     __shared__ RowScanShared<T> sm;
     const int64_t row = blockIdx.x / tiles_per_row;
     int64_t t = blockIdx.x - row * tiles_per_row;
@@ -536,7 +550,7 @@ __global__ __launch_bounds__(BLOCK) void scan_rows_chained(
         t = sm.next_tile;
     }
     scan_tile<T, K, ITEMS, true, !TICKET, BLOCK, X, NZ, Y>(x, y, xmap, ymap, sx, sy, xaxis, n, tiles_per_row, exclusive, row, t, poll_limit, st, sm,
-                                                           TICKET ? ClearedBy{nullptr, 0ull} : cb, ready_early);
+                                                           TICKET ? ClearedBy{nullptr, 0ull} : cb, ready_early, pad);
 }
 
 // ------------------------------------------------------------------ column kernel
@@ -651,6 +665,8 @@ bool make_dim_map2(const int64_t* dims, const int64_t* sx, const int64_t* sy, in
 constexpr int kChainBlock = DLFX_SCAN_CHAIN_BLOCK;
 constexpr int64_t kChainTileBytes = DLFX_SCAN_CHAIN_BYTES;
 
+constexpr int64_t kMaxPad = 15;        // the most positions a row gains when it is tiled from the vector boundary before it
+
 // Elements per tile: 256 bytes per thread for chained rows, less for short rows.
 int64_t tile_elems(size_t elem_size, int64_t n) {
     const int64_t full = 256 * (256 / static_cast<int64_t>(elem_size));
@@ -744,20 +760,32 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     const bool axis_unit = (sx == 1 || sx == -1 || n == 1) && (sy == 1 || sy == -1 || n == 1);
     const bool inner_unit = xmap.rank >= 1 && xmap.strides[xmap.rank - 1] == 1 && ymap.strides[ymap.rank - 1] == 1 &&
                             xmap.dims[xmap.rank - 1] >= 16;
+    // Unit-stride rows that do not all start on a vector boundary are laid out from the boundary
+    // before each row (scan_tile, scan_rows_group), which can make a row up to one vector less
+    // one element longer.
+    int pad = 0;
+    if (!NZ && !axis_general && sx == 1 && sy == 1) {
+        constexpr int VX = scan_vec<T, X, Y>();
+        bool aligned = reinterpret_cast<uintptr_t>(x) % (sizeof(X) * VX) == 0;
+        for (int i = 0; i < xmap.rank; ++i) aligned = aligned && xmap.strides[i] % VX == 0;
+        if (!aligned) pad = VX - 1;
+    }
     // Short rows along a unit-stride axis: a group of lanes per row (rows of up to 512 elements;
     // a workgroup per row would leave most of its threads, or of the chip, idle).
-    if (!axis_general && axis_unit && n <= 512 && m >= 4) {
-        const int64_t lanes = n <= 4 ? 1 : n <= 32 ? 4 : n <= 64 ? 16 : kWave;
+    if (!axis_general && axis_unit && n + pad <= 512 && m >= 4) {
+        const int64_t np = n + pad;
+        const int64_t lanes = np <= 4 ? 1 : np <= 32 ? 4 : np <= 128 ? 16 : kWave;
         const int64_t blocks = ceil_div(m * lanes, kBlock);
         if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
         const dim3 grid(static_cast<unsigned>(blocks)), block(kBlock);
 #define DLFX_SCAN_GROUP(LANES, ITEMS) \
-    scan_rows_group<T, K, LANES, ITEMS, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, m, n, exclusive)
-        if (n <= 4) DLFX_SCAN_GROUP(1, 4);
-        else if (n <= 16) DLFX_SCAN_GROUP(4, 4);
-        else if (n <= 32) DLFX_SCAN_GROUP(4, 8);
-        else if (n <= 64) DLFX_SCAN_GROUP(16, 4);
-        else if (n <= 256) DLFX_SCAN_GROUP(kWave, 4);
+    scan_rows_group<T, K, LANES, ITEMS, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, m, n, exclusive, pad)
+        if (np <= 4) DLFX_SCAN_GROUP(1, 4);
+        else if (np <= 16) DLFX_SCAN_GROUP(4, 4);
+        else if (np <= 32) DLFX_SCAN_GROUP(4, 8);
+        else if (np <= 64) DLFX_SCAN_GROUP(16, 4);
+        else if (np <= 128) DLFX_SCAN_GROUP(16, 8);
+        else if (np <= 256) DLFX_SCAN_GROUP(kWave, 4);
         else DLFX_SCAN_GROUP(kWave, 8);
 #undef DLFX_SCAN_GROUP
         DLFX_CHECK_LAUNCH();
@@ -775,10 +803,10 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
         return DLFX_OK;
     }
 
-    const ScanLayout l = scan_layout(sizeof(T), m, n);
+    const ScanLayout l = scan_layout(sizeof(T), m, n + pad);
     if (l.tiles > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
     if (scratch_bytes < l.total || (l.total && !scratch)) return DLFX_ERR_SCRATCH_TOO_SMALL;
-    const int64_t tile = tile_elems(sizeof(T), n);
+    const int64_t tile = tile_elems(sizeof(T), n + pad);
     constexpr int FULL = 256 / sizeof(T);
     const dim3 block(kBlock);
     if (!l.chained) {
@@ -786,7 +814,7 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
         auto single = [&](auto items) {
             constexpr int ITEMS = decltype(items)::value;
             if constexpr (ITEMS <= FULL)
-                scan_rows_single<T, K, ITEMS, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
+                scan_rows_single<T, K, ITEMS, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive, pad);
         };
         switch (tile / 256) {
         case 1: single(std::integral_constant<int, 1>()); break;
@@ -819,10 +847,10 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     const dim3 cblock(kChainBlock);
     if (in_place)
         scan_rows_chained<T, K, CI, true, kChainBlock, X, NZ, Y><<<grid, cblock, 0, stream>>>(
-            x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st, cb);
+            x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st, cb, pad);
     else
         scan_rows_chained<T, K, CI, false, kChainBlock, X, NZ, Y><<<grid, cblock, 0, stream>>>(
-            x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st, cb);
+            x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st, cb, pad);
     DLFX_CHECK_LAUNCH();
     return DLFX_OK;
 }
@@ -846,7 +874,7 @@ extern "C" size_t dlfx_scan_scratch_bytes(int dtype, int64_t m, int64_t n) {
     size_t es = dtype_size(dtype);
     if (dtype == DLFX_F16) es = 4;                  // scanned as fp32
     if (es < 4 || m <= 0 || n <= 0) return 0;
-    return scan_layout(es, m, n).total;
+    return scan_layout(es, m, n + kMaxPad).total;       // rows off a vector boundary take up to a vector more
 }
 
 extern "C" int dlfx_scan(dlfx_stream_t stream, const char* name, int dtype, int64_t m, int64_t n,
@@ -902,7 +930,7 @@ extern "C" int dlfx_scan(dlfx_stream_t stream, const char* name, int dtype, int6
 
 extern "C" size_t dlfx_scan_nonzero_scratch_bytes(int dtype, int64_t m, int64_t n) {
     if (!dtype_size(dtype) || m <= 0 || n <= 0) return 0;
-    return scan_layout(4, m, n).total;
+    return scan_layout(4, m, n + kMaxPad).total;
 }
 
 extern "C" int dlfx_scan_nonzero(dlfx_stream_t stream, int dtype, int64_t m, int64_t n,

@@ -206,3 +206,41 @@ def test_short_rows_one_lane_group_per_row(hip_backend, oracle_backend, n):
         assert np.array_equal(F.cumsum(V, 1).numpy(), np.cumsum(xi[:, 1:], axis=1, dtype=np.int32))
     # the same rows as columns of the transposed view: the axis is no longer unit-stride
     assert np.array_equal(F.cumsum(Xi.transpose(), 0).numpy(), np.cumsum(xi, axis=1, dtype=np.int32).T)
+
+
+@pytest.mark.parametrize("n", [9, 70, 300, 1000, 5000, 16383, 16387, 40001, 150003])
+def test_rows_off_a_vector_boundary(hip_backend, oracle_backend, n):
+    """Unit-stride rows that do not start on a 16-byte boundary - odd row lengths, views cut one or
+    two elements into a row - are laid out from the boundary before each row, so that their whole
+    vectors still move as one access.  Input and output off the boundary by the same or by
+    different amounts, every kernel size class, 4-, 8- and 2-byte elements, exclusive and reversed,
+    and (long rows) with tiles that never wait for their predecessors."""
+    m = 5
+    for dtype in (np.int32, np.int64):
+        x = randint(230 + n, m * (n + 3), -50, 50).astype(dtype).reshape(m, n + 3)
+        Xh, Xo = both(hip_backend, oracle_backend, x)
+        for cut in (1, 2, 3):
+            Vh, Vo = Xh.slice([cut], [cut + n], [1]), Xo.slice([cut], [cut + n], [1])
+            for exclusive in (False, True):
+                for reverse in (False, True):
+                    assert np.array_equal(F.cumsum(Vh, 1, exclusive, reverse).numpy(), F.cumsum(Vo, 1, exclusive, reverse).numpy()), (dtype, cut, exclusive, reverse)
+        # the output off the boundary by another amount than the input
+        Yh = Tensor.from_numpy(hip_backend, np.zeros((m, n + 3), dtype))
+        F.cumsum(Xh.slice([1], [1 + n], [1]), 1, out=Yh.slice([2], [2 + n], [1]))
+        got = Yh.numpy()
+        assert np.array_equal(got[:, 2: 2 + n], np.cumsum(x[:, 1: 1 + n], axis=1, dtype=dtype))
+        assert not got[:, :2].any() and not got[:, 2 + n:].any()          # nothing written beside the rows
+        assert np.array_equal(F.cummax(Xh.slice([3], [3 + n], [1]), 1).numpy(), np.maximum.accumulate(x[:, 3: 3 + n], axis=1))
+    xh = (normal(231 + n, m * (n + 1)) * 0.25).astype(np.float16).reshape(m, n + 1)
+    got = F.cumsum(Tensor.from_numpy(hip_backend, xh).slice([1], [1 + n], [1]), 1).numpy().astype(np.float64)
+    x64 = xh[:, 1:].astype(np.float64)
+    want, mag = np.cumsum(x64, axis=1), np.cumsum(np.abs(x64), axis=1)
+    assert (np.abs(got - want) <= 4 * max(1.0, np.log2(n)) * np.finfo(np.float32).eps * mag + 2.0 ** -10 * np.abs(want) + 1e-30).all()
+    if n > 20000:
+        hip_backend.set_tuning("scan_poll_limit", 0)
+        try:
+            x = randint(232 + n, m * (n + 1), -50, 50).astype(np.int32).reshape(m, n + 1)
+            Xh = Tensor.from_numpy(hip_backend, x)
+            assert np.array_equal(F.cumsum(Xh.slice([1], [1 + n], [1]), 1).numpy(), np.cumsum(x[:, 1:], axis=1, dtype=np.int32))
+        finally:
+            hip_backend.set_tuning("scan_poll_limit", 2048)
