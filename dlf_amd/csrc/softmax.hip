@@ -74,15 +74,20 @@ __device__ __forceinline__ V team_reduce(V v, Join join, V* lds) {
     return v;
 }
 
-// Rows held in registers.  TEAM threads per row, ITEMS elements per thread; element (k, t) of
-// the row is ((k / V) * TEAM + t) * V + k % V with V elements per 128-bit access when VEC.
-template <typename S, int TEAM, int ITEMS, int KIND, bool VEC>
+// Rows held in registers.  TEAM threads per row, ITEMS elements per thread in 128-bit accesses
+// of V elements: item k of thread t sits at position ((k / V) * TEAM + t) * V + k % V of its
+// row.  A row that starts on a 16-byte boundary has element i at position i.  Rows that do not
+// (pad != 0: the host found that rows may not - a row length that is no multiple of V, a base
+// off the boundary) are laid out from the boundary before them: element i at position
+// i + shift, so that every whole vector of the row is still one aligned access; the vectors at
+// a row's two ends, when partial, move element by element.
+template <typename S, int TEAM, int ITEMS, int KIND>
 __global__ __launch_bounds__(TEAM > 256 ? TEAM : 256)
 __attribute__((amdgpu_waves_per_eu(TEAM >= 1024 && sizeof(typename ComputeOf<S>::type) * ITEMS <= 128 ? 8 : 1)))      // two 1024-thread rows per CU
-void softmax_rows(const S* x, S* y, int64_t m, int64_t n) {          // y may be x: no restrict
+void softmax_rows(const S* x, S* y, int64_t m, int64_t n, int pad) {          // y may be x: no restrict
     using T = typename ComputeOf<S>::type;
     constexpr int BLOCK = TEAM > 256 ? TEAM : 256;
-    constexpr int V = VEC ? 16 / static_cast<int>(sizeof(S)) : 1;
+    constexpr int V = 16 / static_cast<int>(sizeof(S));
     static_assert(ITEMS % V == 0, "whole vectors per thread");
     constexpr int G = ITEMS / V;
     using VecT = Vec<S, V>;
@@ -94,24 +99,30 @@ void softmax_rows(const S* x, S* y, int64_t m, int64_t n) {          // y may be
     const S* xr = x + (live ? row : 0) * n;
     S* yr = y + (live ? row : 0) * n;
     const T lowest = std::is_integral<T>::value ? std::numeric_limits<T>::lowest() : -std::numeric_limits<T>::infinity();
+    const int32_t shift = pad ? static_cast<int32_t>((reinterpret_cast<uintptr_t>(xr) / sizeof(S)) % V) : 0;
+    const bool y_like_x = !pad || static_cast<int32_t>((reinterpret_cast<uintptr_t>(yr) / sizeof(S)) % V) == shift;
     const int32_t n32 = static_cast<int32_t>(n);          // rows here have at most 32768 elements
-    auto index_of = [&](int k) -> int32_t { return ((k / V) * TEAM + t) * V + k % V; };
+    const int32_t end32 = n32 + shift;                    // positions [shift, end32) are the row
+    auto index_of = [&](int k) -> int32_t { return ((k / V) * TEAM + t) * V + k % V - shift; };
+    auto in_row = [&](int k) -> bool { return static_cast<uint32_t>(index_of(k)) < static_cast<uint32_t>(n32); };
 
+    // A vector that holds the row's first or last elements also holds the neighbouring row's:
+    // it is read whole all the same (and what is not the row's dropped) unless it reaches
+    // outside the tensor, which only the first and the last row's end vectors can.
+    const S* const tensor_end = x + m * n;
     T v[ITEMS];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        const int64_t i0 = (static_cast<int64_t>(g) * TEAM + t) * V;
-        if (VEC) {
-            if (live && i0 < n) {                         // n is a multiple of V here
-                const VecT a = load_stream(reinterpret_cast<const VecT*>(xr + i0));
+        const int32_t p0 = (g * TEAM + t) * V;
+        const S* at = xr - shift + p0;
+        if (live && p0 + V > shift && p0 < end32 && at >= x && at + V <= tensor_end) {
+            const VecT a = load_stream(reinterpret_cast<const VecT*>(at));
 #pragma unroll
-                for (int e = 0; e < V; ++e) v[g * V + e] = static_cast<T>(a.v[e]);
-            } else {
-#pragma unroll
-                for (int e = 0; e < V; ++e) v[g * V + e] = lowest;
-            }
+            for (int e = 0; e < V; ++e) v[g * V + e] = (p0 + e >= shift && p0 + e < end32) ? static_cast<T>(a.v[e]) : lowest;
         } else {
-            v[g] = (live && i0 < n) ? static_cast<T>(load_stream(&xr[i0])) : lowest;
+#pragma unroll
+            for (int e = 0; e < V; ++e)
+                v[g * V + e] = (live && p0 + e >= shift && p0 + e < end32) ? static_cast<T>(load_stream(&xr[p0 + e - shift])) : lowest;
         }
     }
 
@@ -130,7 +141,7 @@ void softmax_rows(const S* x, S* y, int64_t m, int64_t n) {          // y may be
         int32_t hot = std::numeric_limits<int32_t>::max();
 #pragma unroll
         for (int k = ITEMS - 1; k >= 0; --k)
-            if (v[k] == mx && index_of(k) < n32) hot = index_of(k);      // this thread's indices grow with k
+            if (v[k] == mx && in_row(k)) hot = index_of(k);      // this thread's indices grow with k
         hot = team_reduce<TEAM>(hot, [](int32_t a, int32_t b) { return a < b ? a : b; }, reinterpret_cast<int32_t*>(lds_raw));
         if (hot >= n32 || leading_nan) hot = 0;                            // all NaN or -inf, or a leading NaN
 #pragma unroll
@@ -146,7 +157,7 @@ void softmax_rows(const S* x, S* y, int64_t m, int64_t n) {          // y may be
         T sum = T(0);
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
-            const T e = index_of(k) < n32 ? exp_of<T>(v[k] - mx) : T(0);
+            const T e = in_row(k) ? exp_of<T>(v[k] - mx) : T(0);
             if constexpr (KIND == kSoftmax) v[k] = e;
             sum += e;
         }
@@ -165,16 +176,17 @@ void softmax_rows(const S* x, S* y, int64_t m, int64_t n) {          // y may be
 
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        const int64_t i0 = (static_cast<int64_t>(g) * TEAM + t) * V;
-        if (live && i0 < n) {
-            if (VEC) {
-                VecT a;
+        const int32_t p0 = (g * TEAM + t) * V;
+        if (!live) continue;
+        if (y_like_x && p0 >= shift && p0 + V <= end32) {
+            VecT a;
 #pragma unroll
-                for (int e = 0; e < V; ++e) a.v[e] = static_cast<S>(v[g * V + e]);
-                store_stream(reinterpret_cast<VecT*>(yr + i0), a);
-            } else {
-                store_stream(&yr[i0], static_cast<S>(v[g]));
-            }
+            for (int e = 0; e < V; ++e) a.v[e] = static_cast<S>(v[g * V + e]);
+            store_stream(reinterpret_cast<VecT*>(yr - shift + p0), a);
+        } else {
+#pragma unroll
+            for (int e = 0; e < V; ++e)
+                if (p0 + e >= shift && p0 + e < end32) store_stream(&yr[p0 + e - shift], static_cast<S>(v[g * V + e]));
         }
     }
 }
@@ -392,47 +404,55 @@ template <typename T, int KIND>
 int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y, void* scratch, size_t scratch_bytes) {
     constexpr int V = 16 / static_cast<int>(sizeof(T));
     constexpr int kRegisterBytes = static_cast<int>(sizeof(typename ComputeOf<T>::type));
-    const bool vec = n % V == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
+    // rows all start on a 16-byte boundary, or are laid out from the boundary before them (softmax_rows),
+    // which can make a row up to V - 1 positions longer
+    const bool aligned = n % V == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
+    const int pad = aligned ? 0 : V - 1;
+    const int64_t np = n + pad;
     // wavefront teams: 4 rows per workgroup
 #define DLFX_WAVE_ROWS(ITEMS)                                                                                   \
     do {                                                                                                        \
         const dim3 grid(static_cast<unsigned>(ceil_div(m, 4)));                                                 \
-        if (vec) softmax_rows<T, kWave, ITEMS, KIND, true><<<grid, dim3(256), 0, stream>>>(x, y, m, n);         \
-        else softmax_rows<T, kWave, ITEMS, KIND, false><<<grid, dim3(256), 0, stream>>>(x, y, m, n);            \
+        softmax_rows<T, kWave, ITEMS, KIND><<<grid, dim3(256), 0, stream>>>(x, y, m, n, pad);                   \
         DLFX_CHECK_LAUNCH();                                                                                    \
         return DLFX_OK;                                                                                         \
     } while (0)
 #define DLFX_BLOCK_ROWS(ITEMS)                                                                                  \
     do {                                                                                                        \
         const dim3 grid(static_cast<unsigned>(m));                                                              \
-        if (vec) softmax_rows<T, 1024, ITEMS, KIND, true><<<grid, dim3(1024), 0, stream>>>(x, y, m, n);         \
-        else softmax_rows<T, 1024, ITEMS, KIND, false><<<grid, dim3(1024), 0, stream>>>(x, y, m, n);            \
+        softmax_rows<T, 1024, ITEMS, KIND><<<grid, dim3(1024), 0, stream>>>(x, y, m, n, pad);                   \
         DLFX_CHECK_LAUNCH();                                                                                    \
         return DLFX_OK;                                                                                         \
     } while (0)
     if (ceil_div(m, 4) > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
     // very short rows: one, four or sixteen lanes per row (V elements each), 256, 64 or 16 rows per workgroup
-#define DLFX_LANE_ROWS(TEAM)                                                                                    \
+#define DLFX_LANE_ROWS(TEAM, ITEMS)                                                                             \
     do {                                                                                                        \
         const dim3 grid(static_cast<unsigned>(ceil_div(m, 256 / TEAM)));                                        \
-        if (vec) softmax_rows<T, TEAM, V, KIND, true><<<grid, dim3(256), 0, stream>>>(x, y, m, n);              \
-        else softmax_rows<T, TEAM, V, KIND, false><<<grid, dim3(256), 0, stream>>>(x, y, m, n);                 \
+        softmax_rows<T, TEAM, ITEMS, KIND><<<grid, dim3(256), 0, stream>>>(x, y, m, n, pad);                    \
         DLFX_CHECK_LAUNCH();                                                                                    \
         return DLFX_OK;                                                                                         \
     } while (0)
-    if (n <= V) DLFX_LANE_ROWS(1);
-    if (n <= 4 * V) DLFX_LANE_ROWS(4);
-    if (n <= 16 * V) DLFX_LANE_ROWS(16);
+    // (slots of a row: V, 4 V, 16 V, 32 V, 64 V, 128 V, 256 V, then 2048 and 4096 to 32768 in steps of at most half)
+    if (np <= V) DLFX_LANE_ROWS(1, V);
+    if (np <= 4 * V) DLFX_LANE_ROWS(4, V);
+    if (np <= 16 * V) DLFX_LANE_ROWS(16, V);
+    if (np <= 32 * V) DLFX_LANE_ROWS(16, 2 * V);
 #undef DLFX_LANE_ROWS
-    if (n <= kWave * V) DLFX_WAVE_ROWS(V);
-    if (n <= kWave * 4 * V) DLFX_WAVE_ROWS(4 * V);
-    if (n <= kWave * 32) DLFX_WAVE_ROWS(32);
+    if (np <= kWave * V) DLFX_WAVE_ROWS(V);
+    if (np <= kWave * 2 * V) DLFX_WAVE_ROWS(2 * V);
+    if (np <= kWave * 4 * V) DLFX_WAVE_ROWS(4 * V);
+    if (np <= kWave * 32) DLFX_WAVE_ROWS(32);
     if constexpr (V <= 4) {
-        if (n <= 1024 * 4) DLFX_BLOCK_ROWS(4);
+        if (np <= 1024 * 4) DLFX_BLOCK_ROWS(4);
     }
-    if (n <= 1024 * 8) DLFX_BLOCK_ROWS(8);
-    if (n <= 1024 * 16) DLFX_BLOCK_ROWS(16);
-    if (n <= 1024 * 32 && kRegisterBytes == 4) DLFX_BLOCK_ROWS(32);
+    if (np <= 1024 * 8) DLFX_BLOCK_ROWS(8);
+    if constexpr (V <= 4) {
+        if (np <= 1024 * 12) DLFX_BLOCK_ROWS(12);
+    }
+    if (np <= 1024 * 16) DLFX_BLOCK_ROWS(16);
+    if (np <= 1024 * 24 && kRegisterBytes == 4) DLFX_BLOCK_ROWS(24);
+    if (np <= 1024 * 32 && kRegisterBytes == 4) DLFX_BLOCK_ROWS(32);
 #undef DLFX_WAVE_ROWS
 #undef DLFX_BLOCK_ROWS
     const size_t need = split_scratch_bytes<T>(m, n);

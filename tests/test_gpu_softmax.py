@@ -95,11 +95,15 @@ def test_hardmax_of_integer_rows(hip_backend, oracle_backend, dtype, n):
         F.softmax(Tensor.from_numpy(hip_backend, x), 1)
 
 
-@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8, 10, 15, 16, 17, 31, 32, 33, 63, 64, 65, 4095, 4096, 4097])
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8, 10, 15, 16, 17, 31, 32, 33, 61, 63, 64, 65, 66, 125, 128, 129, 253, 255, 257, 509, 512, 513, 1021, 1025,
+                               2045, 2047, 2051, 4095, 4096, 4097, 8189, 8193, 12285, 12289, 16381, 16385, 24573, 24577, 32765])
 def test_row_lengths_around_the_team_sizes(hip_backend, oracle_backend, n):
     """One lane per row up to 4 (fp32) / 2 (fp64) / 8 (half) elements, four lanes up to four times
-    that, sixteen lanes per row up to 64 (fp32) / 32 (fp64) / 128 (half) elements, a wavefront up to
-    2048, a workgroup of 1024 threads with 4 elements each up to 4096: the boundaries of each."""
+    that, sixteen lanes per row up to 128 (fp32) elements, a wavefront up to 2048, a workgroup of
+    1024 threads up to 32768: the boundaries of each class.  Rows that do not start on a 16-byte
+    boundary (odd lengths) are laid out from the boundary before them, which moves those
+    boundaries down by up to a vector less one element; the output rows here start on other
+    boundaries than the input rows (a view that begins one row into its buffer)."""
     m = 700 if n <= 16 else 70 if n < 1000 else 9     # several workgroups of one- and four-lane teams
     for dtype in (np.float32, np.float64, np.float16):
         x = (normal(230 + n, m * n) * 2).astype(dtype).reshape(m, n)
@@ -118,6 +122,10 @@ def test_row_lengths_around_the_team_sizes(hip_backend, oracle_backend, n):
         want = sp_log_softmax(x64, axis=1)
         assert (np.abs(got - want) <= slack * (1 + np.abs(want)) + out_ulp * np.abs(want)).all(), dtype
         assert np.array_equal(F.hardmax(Xh).numpy(), F.hardmax(Xo).numpy()), dtype
+        if dtype == np.float32 and n > 1:
+            Vh, Vo = Xh.slice([1], [m], [0]), Xo.slice([1], [m], [0])          # the same rows from the second on
+            assert np.array_equal(F.softmax(Vh).numpy(), F.softmax(Xh).numpy()[1:], equal_nan=True)
+            assert np.array_equal(F.hardmax(Vh).numpy(), F.hardmax(Vo).numpy())
 
 
 @pytest.mark.parametrize("m,n,dtype", [(1, 200000, np.float32), (3, 70001, np.float32), (7, 40000, np.float64), (2, 32769, np.float32),
