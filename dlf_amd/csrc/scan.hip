@@ -197,12 +197,11 @@ struct RowScanShared {
 // [w*64*ITEMS, (w+1)*64*ITEMS); within it, vector k of lane l covers elements
 // (k*64 + l)*V .. +V.  CHAINED tiles publish / look back through `st`.
 template <typename T, int K, int ITEMS, bool CHAINED, bool SELF_HELP, int BLOCK = kBlock, typename X = T, bool NZ = false,
-          typename Y = T>
+          typename Y = T, bool PAD = false>
 __device__ __forceinline__ void scan_tile(
     const X* __restrict__ x, Y* __restrict__ y, const DimMap& xmap, const DimMap& ymap, int64_t sx, int64_t sy,
     const DimMap& xaxis, int64_t n, int64_t tiles_per_row, int exclusive, int64_t row, int64_t t, int poll_limit,
-    TileState<T>& st, RowScanShared<T>& sm, const ClearedBy& cb = ClearedBy{nullptr, 0ull}, unsigned long long ready_early = 0ull,
-    int pad = 0) {
+    TileState<T>& st, RowScanShared<T>& sm, const ClearedBy& cb = ClearedBy{nullptr, 0ull}, unsigned long long ready_early = 0ull) {
     // where element i of a row lives: i * sx, or (scan_nonzero over a flattened view whose
     // dimensions do not merge) wherever the row-major walk of `xaxis` puts it
     auto x_at = [&](int64_t i) -> int64_t {
@@ -221,11 +220,11 @@ __device__ __forceinline__ void scan_tile(
 
     const X* xr = x + xmap.at(row);
     Y* yr = y + ymap.at(row);
-    // A unit-stride row that does not start on a vector boundary (pad != 0: the host found such
+    // A unit-stride row that does not start on a vector boundary (PAD: the host found such
     // rows) is tiled from the boundary before it: position j of that tiling is element
     // j - shift of the row, positions below `shift` hold the identity, and every whole vector
     // of the row is aligned in memory.  Elsewhere shift is 0 and positions are elements.
-    const int shift = pad ? static_cast<int>((reinterpret_cast<uintptr_t>(xr) / sizeof(X)) % V) : 0;
+    const int shift = PAD ? static_cast<int>((reinterpret_cast<uintptr_t>(xr) / sizeof(X)) % V) : 0;
     const int64_t n_pos = n + shift;                       // positions of the row: [shift, n_pos)
     const int64_t seg = tile_base + static_cast<int64_t>(w) * kWave * ITEMS;
 
@@ -409,14 +408,13 @@ __device__ __forceinline__ void scan_tile(
 }
 
 // Rows of a single tile: workgroup b scans row b.
-template <typename T, int K, int ITEMS, typename X, bool NZ, typename Y>
+template <typename T, int K, int ITEMS, typename X, bool NZ, typename Y, bool PAD>
 __global__ __launch_bounds__(kBlock) void scan_rows_single(
     const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy, DimMap xaxis,
-    int64_t n, int exclusive, int pad) {
+    int64_t n, int exclusive) {
     __shared__ RowScanShared<T> sm;
     TileState<T> st;
-    scan_tile<T, K, ITEMS, false, false, kBlock, X, NZ, Y>(x, y, xmap, ymap, sx, sy, xaxis, n, 1, exclusive, blockIdx.x, 0, 0, st, sm,
-                                                           ClearedBy{nullptr, 0ull}, 0ull, pad);
+    scan_tile<T, K, ITEMS, false, false, kBlock, X, NZ, Y, PAD>(x, y, xmap, ymap, sx, sy, xaxis, n, 1, exclusive, blockIdx.x, 0, 0, st, sm);
 }
 
 // Short rows: LANES lanes per row (one lane, a quad, a DPP row of 16 lanes, or a whole wavefront), ITEMS elements
@@ -519,10 +517,10 @@ __global__ __launch_bounds__(kBlock) void scan_rows_group(
 // TICKET the tile of the row is drawn from that row's atomic counter (in-place
 // scans); without, it is the workgroup's position in the row and waits are
 // bounded by self-help.
-template <typename T, int K, int ITEMS, bool TICKET, int BLOCK, typename X, bool NZ, typename Y>
+template <typename T, int K, int ITEMS, bool TICKET, int BLOCK, typename X, bool NZ, typename Y, bool PAD>
 __global__ __launch_bounds__(BLOCK) void scan_rows_chained(
     const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy, DimMap xaxis,
-    int64_t n, int64_t tiles_per_row, int exclusive, int poll_limit, unsigned* ticket, TileState<T> st, ClearedBy cb, int pad) {
+    int64_t n, int64_t tiles_per_row, int exclusive, int poll_limit, unsigned* ticket, TileState<T> st, ClearedBy cb) {
     __shared__ RowScanShared<T> sm;
     const int64_t row = blockIdx.x / tiles_per_row;
     int64_t t = blockIdx.x - row * tiles_per_row;
@@ -549,8 +547,8 @@ __global__ __launch_bounds__(BLOCK) void scan_rows_chained(
         __syncthreads();
         t = sm.next_tile;
     }
-    scan_tile<T, K, ITEMS, true, !TICKET, BLOCK, X, NZ, Y>(x, y, xmap, ymap, sx, sy, xaxis, n, tiles_per_row, exclusive, row, t, poll_limit, st, sm,
-                                                           TICKET ? ClearedBy{nullptr, 0ull} : cb, ready_early, pad);
+    scan_tile<T, K, ITEMS, true, !TICKET, BLOCK, X, NZ, Y, PAD>(x, y, xmap, ymap, sx, sy, xaxis, n, tiles_per_row, exclusive, row, t, poll_limit, st, sm,
+                                                                TICKET ? ClearedBy{nullptr, 0ull} : cb, ready_early);
 }
 
 // ------------------------------------------------------------------ column kernel
@@ -813,8 +811,15 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
         const dim3 grid(static_cast<unsigned>(m));
         auto single = [&](auto items) {
             constexpr int ITEMS = decltype(items)::value;
-            if constexpr (ITEMS <= FULL)
-                scan_rows_single<T, K, ITEMS, X, NZ, Y><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive, pad);
+            if constexpr (ITEMS <= FULL) {
+                if constexpr (!NZ) {
+                    if (pad) {
+                        scan_rows_single<T, K, ITEMS, X, NZ, Y, true><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
+                        return;
+                    }
+                }
+                scan_rows_single<T, K, ITEMS, X, NZ, Y, false><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, xaxis, n, exclusive);
+            }
         };
         switch (tile / 256) {
         case 1: single(std::integral_constant<int, 1>()); break;
@@ -845,12 +850,23 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     const dim3 grid(static_cast<unsigned>(l.tiles));
     constexpr int CI = static_cast<int>(kChainTileBytes / sizeof(T) / kChainBlock);
     const dim3 cblock(kChainBlock);
-    if (in_place)
-        scan_rows_chained<T, K, CI, true, kChainBlock, X, NZ, Y><<<grid, cblock, 0, stream>>>(
-            x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st, cb, pad);
-    else
-        scan_rows_chained<T, K, CI, false, kChainBlock, X, NZ, Y><<<grid, cblock, 0, stream>>>(
-            x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st, cb, pad);
+    // rows off a vector boundary have kernels of their own: the aligned ones carry none of that arithmetic
+    auto chained = [&](auto ticketed, auto padded) {
+        scan_rows_chained<T, K, CI, decltype(ticketed)::value, kChainBlock, X, NZ, Y, decltype(padded)::value><<<grid, cblock, 0, stream>>>(
+            x, y, xmap, ymap, sx, sy, xaxis, n, l.tiles_per_row, exclusive, g_poll_limit, ticket, st, cb);
+    };
+    bool launched = false;
+    if constexpr (!NZ) {
+        if (pad) {
+            if (in_place) chained(std::true_type(), std::true_type());
+            else chained(std::false_type(), std::true_type());
+            launched = true;
+        }
+    }
+    if (!launched) {
+        if (in_place) chained(std::true_type(), std::false_type());
+        else chained(std::false_type(), std::false_type());
+    }
     DLFX_CHECK_LAUNCH();
     return DLFX_OK;
 }

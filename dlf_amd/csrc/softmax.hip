@@ -77,14 +77,15 @@ __device__ __forceinline__ V team_reduce(V v, Join join, V* lds) {
 // Rows held in registers.  TEAM threads per row, ITEMS elements per thread in 128-bit accesses
 // of V elements: item k of thread t sits at position ((k / V) * TEAM + t) * V + k % V of its
 // row.  A row that starts on a 16-byte boundary has element i at position i.  Rows that do not
-// (pad != 0: the host found that rows may not - a row length that is no multiple of V, a base
+// (PAD: the host found that rows may not - a row length that is no multiple of V, a base
 // off the boundary) are laid out from the boundary before them: element i at position
 // i + shift, so that every whole vector of the row is still one aligned access; the vectors at
-// a row's two ends, when partial, move element by element.
-template <typename S, int TEAM, int ITEMS, int KIND>
+// a row's two ends, when partial, move element by element.  Without PAD none of that arithmetic
+// is compiled in: n is a multiple of V and a vector lies in the row or past it.
+template <typename S, int TEAM, int ITEMS, int KIND, bool PAD>
 __global__ __launch_bounds__(TEAM > 256 ? TEAM : 256)
 __attribute__((amdgpu_waves_per_eu(TEAM >= 1024 && sizeof(typename ComputeOf<S>::type) * ITEMS <= 128 ? 8 : 1)))      // two 1024-thread rows per CU
-void softmax_rows(const S* x, S* y, int64_t m, int64_t n, int pad) {          // y may be x: no restrict
+void softmax_rows(const S* x, S* y, int64_t m, int64_t n) {          // y may be x: no restrict
     using T = typename ComputeOf<S>::type;
     constexpr int BLOCK = TEAM > 256 ? TEAM : 256;
     constexpr int V = 16 / static_cast<int>(sizeof(S));
@@ -99,8 +100,8 @@ void softmax_rows(const S* x, S* y, int64_t m, int64_t n, int pad) {          //
     const S* xr = x + (live ? row : 0) * n;
     S* yr = y + (live ? row : 0) * n;
     const T lowest = std::is_integral<T>::value ? std::numeric_limits<T>::lowest() : -std::numeric_limits<T>::infinity();
-    const int32_t shift = pad ? static_cast<int32_t>((reinterpret_cast<uintptr_t>(xr) / sizeof(S)) % V) : 0;
-    const bool y_like_x = !pad || static_cast<int32_t>((reinterpret_cast<uintptr_t>(yr) / sizeof(S)) % V) == shift;
+    const int32_t shift = PAD ? static_cast<int32_t>((reinterpret_cast<uintptr_t>(xr) / sizeof(S)) % V) : 0;
+    const bool y_like_x = !PAD || static_cast<int32_t>((reinterpret_cast<uintptr_t>(yr) / sizeof(S)) % V) == shift;
     const int32_t n32 = static_cast<int32_t>(n);          // rows here have at most 32768 elements
     const int32_t end32 = n32 + shift;                    // positions [shift, end32) are the row
     auto index_of = [&](int k) -> int32_t { return ((k / V) * TEAM + t) * V + k % V - shift; };
@@ -115,7 +116,16 @@ void softmax_rows(const S* x, S* y, int64_t m, int64_t n, int pad) {          //
     for (int g = 0; g < G; ++g) {
         const int32_t p0 = (g * TEAM + t) * V;
         const S* at = xr - shift + p0;
-        if (live && p0 + V > shift && p0 < end32 && at >= x && at + V <= tensor_end) {
+        if constexpr (!PAD) {
+            if (live && p0 < n32) {
+                const VecT a = load_stream(reinterpret_cast<const VecT*>(at));
+#pragma unroll
+                for (int e = 0; e < V; ++e) v[g * V + e] = static_cast<T>(a.v[e]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < V; ++e) v[g * V + e] = lowest;
+            }
+        } else if (live && p0 + V > shift && p0 < end32 && at >= x && at + V <= tensor_end) {
             const VecT a = load_stream(reinterpret_cast<const VecT*>(at));
 #pragma unroll
             for (int e = 0; e < V; ++e) v[g * V + e] = (p0 + e >= shift && p0 + e < end32) ? static_cast<T>(a.v[e]) : lowest;
@@ -178,7 +188,14 @@ void softmax_rows(const S* x, S* y, int64_t m, int64_t n, int pad) {          //
     for (int g = 0; g < G; ++g) {
         const int32_t p0 = (g * TEAM + t) * V;
         if (!live) continue;
-        if (y_like_x && p0 >= shift && p0 + V <= end32) {
+        if constexpr (!PAD) {
+            if (p0 < n32) {
+                VecT a;
+#pragma unroll
+                for (int e = 0; e < V; ++e) a.v[e] = static_cast<S>(v[g * V + e]);
+                store_stream(reinterpret_cast<VecT*>(yr + p0), a);
+            }
+        } else if (y_like_x && p0 >= shift && p0 + V <= end32) {
             VecT a;
 #pragma unroll
             for (int e = 0; e < V; ++e) a.v[e] = static_cast<S>(v[g * V + e]);
@@ -413,14 +430,16 @@ int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y, v
 #define DLFX_WAVE_ROWS(ITEMS)                                                                                   \
     do {                                                                                                        \
         const dim3 grid(static_cast<unsigned>(ceil_div(m, 4)));                                                 \
-        softmax_rows<T, kWave, ITEMS, KIND><<<grid, dim3(256), 0, stream>>>(x, y, m, n, pad);                   \
+        if (pad) softmax_rows<T, kWave, ITEMS, KIND, true><<<grid, dim3(256), 0, stream>>>(x, y, m, n);         \
+        else softmax_rows<T, kWave, ITEMS, KIND, false><<<grid, dim3(256), 0, stream>>>(x, y, m, n);            \
         DLFX_CHECK_LAUNCH();                                                                                    \
         return DLFX_OK;                                                                                         \
     } while (0)
 #define DLFX_BLOCK_ROWS(ITEMS)                                                                                  \
     do {                                                                                                        \
         const dim3 grid(static_cast<unsigned>(m));                                                              \
-        softmax_rows<T, 1024, ITEMS, KIND><<<grid, dim3(1024), 0, stream>>>(x, y, m, n, pad);                   \
+        if (pad) softmax_rows<T, 1024, ITEMS, KIND, true><<<grid, dim3(1024), 0, stream>>>(x, y, m, n);         \
+        else softmax_rows<T, 1024, ITEMS, KIND, false><<<grid, dim3(1024), 0, stream>>>(x, y, m, n);            \
         DLFX_CHECK_LAUNCH();                                                                                    \
         return DLFX_OK;                                                                                         \
     } while (0)
@@ -429,7 +448,8 @@ int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y, v
 #define DLFX_LANE_ROWS(TEAM, ITEMS)                                                                             \
     do {                                                                                                        \
         const dim3 grid(static_cast<unsigned>(ceil_div(m, 256 / TEAM)));                                        \
-        softmax_rows<T, TEAM, ITEMS, KIND><<<grid, dim3(256), 0, stream>>>(x, y, m, n, pad);                    \
+        if (pad) softmax_rows<T, TEAM, ITEMS, KIND, true><<<grid, dim3(256), 0, stream>>>(x, y, m, n);          \
+        else softmax_rows<T, TEAM, ITEMS, KIND, false><<<grid, dim3(256), 0, stream>>>(x, y, m, n);             \
         DLFX_CHECK_LAUNCH();                                                                                    \
         return DLFX_OK;                                                                                         \
     } while (0)
