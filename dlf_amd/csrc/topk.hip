@@ -630,7 +630,10 @@ template <> struct BitsOf<int16_t> { using type = uint32_t; using storage = uint
 // counting, when there is only a handful).  When more than 64 elements reach the bound (long
 // runs of equal values), the wave takes the `limit` best one after the other instead: exact
 // for any input, and only slow where it is needed.
-constexpr int kWaveRowMax = 4096;       // longest row topk_rows_wave takes
+#ifndef DLFX_TOPK_WAVE_ROW_MAX
+#define DLFX_TOPK_WAVE_ROW_MAX 4096
+#endif
+constexpr int kWaveRowMax = DLFX_TOPK_WAVE_ROW_MAX;       // longest row topk_rows_wave takes
 constexpr int kWaveRowLimit = 16;       // largest limit (the limit-th of 64 lane maxima is a weak bound beyond)
 constexpr int kWaveSortItems = 4;       // rows of up to 64 * this many elements can be ordered whole by the wave
 
