@@ -630,11 +630,8 @@ template <> struct BitsOf<int16_t> { using type = uint32_t; using storage = uint
 // counting, when there is only a handful).  When more than 64 elements reach the bound (long
 // runs of equal values), the wave takes the `limit` best one after the other instead: exact
 // for any input, and only slow where it is needed.
-#ifndef DLFX_TOPK_WAVE_ROW_MAX
-#define DLFX_TOPK_WAVE_ROW_MAX 4096
-#endif
-constexpr int kWaveRowMax = DLFX_TOPK_WAVE_ROW_MAX;       // longest row topk_rows_wave takes
-constexpr int kWaveRowLimit = 16;       // largest limit (the limit-th of 64 lane maxima is a weak bound beyond)
+constexpr int kWaveRowMax = 2048;       // longest row topk_rows_wave takes (beyond, the row in 64 registers a lane costs twice the time of topk_select)
+constexpr int kWaveRowLimit = 32;       // largest limit: the limit-th of 64 lane maxima lets about 45 entries through at 32, more than the 64 the buffer holds from 40 on
 constexpr int kWaveSortItems = 4;       // rows of up to 64 * this many elements can be ordered whole by the wave
 
 template <typename E, int ITEMS>
@@ -1015,8 +1012,9 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
     };
 
     constexpr int CAP = cand_cap<K>();
-    if constexpr (BLOCK * ITEMS <= CAP) {
-        // short rows: select straight from registers
+    constexpr bool kShort = BLOCK * ITEMS <= CAP;          // a row's items are no more than the candidates LDS holds
+    if constexpr (kShort && WAVES != 16) {
+        // short rows of small workgroups: select straight from registers
         K ord[ITEMS];
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) ord[i] = load_ord(i);
@@ -1071,13 +1069,17 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
         if (tid == 0) sm.count = 0u;
         DLFX_PHASE(0);            // loads and thread maxima
         auto larger = [](T a, T b) { return a > b ? a : b; };
+        // (a row shorter than the workgroup's first vectors leaves the last waves and 16-lane rows
+        // without elements: a sample from there bounds nothing, so only the full ones count)
+        const int full_waves = static_cast<int>(n32 / static_cast<uint32_t>(kWave * V));
+        const int full_rows = static_cast<int>(n32 / static_cast<uint32_t>(16 * V));
         int samples, mth;
-        if (limit <= WAVES) {
+        if (limit <= WAVES && limit <= full_waves) {
             const T wmax = wave_reduce(tmax, larger);
             if (lane == 0) red[w] = wmax;
             samples = WAVES;
             mth = limit;
-        } else if (limit <= 4 * WAVES) {
+        } else if (limit <= 4 * WAVES && limit <= full_rows) {
             const T rmax = group_reduce(tmax, 16, larger);
             if ((lane & 15) == 0) red[w * 4 + (lane >> 4)] = rmax;
             samples = 4 * WAVES;
@@ -1169,6 +1171,13 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
             merge_rank_emit<BLOCK, K>(sm.cand_ord, sm.cand_idx, sm.pack, static_cast<int>(total), limit, io, row, xr,
                                       [&](K bits) { return ord_of(bit_cast<T>(bits)); });
             DLFX_PHASE(3);        // ordering and output
+        } else if constexpr (kShort) {
+            // a short row whose survivors are too many to rank (or that holds a NaN): exact
+            // selection from the registers, no second kernel
+            __syncthreads();                          // every thread has read the count select_and_emit clears
+            if (tid == 0) row_state[row] = kRowDone;
+            select_and_emit<BLOCK, ITEMS, false>(sm, io, row, xr, limit, ITEMS,
+                                                 [&](int i) { return index_of(i) < n32 ? ord_of(sc[i]) : K(0); }, index_of);
         } else if (total <= CAP && limit <= BLOCK) {
             if (tid == 0) row_state[row] = total;
             K* so = spill_ord + row * CAP;
@@ -1302,8 +1311,7 @@ int launch_select(hipStream_t stream, const TopkIo<typename BitsOf<T>::type, typ
         else if (n <= 256) DLFX_TOPK_WAVE(4);
         else if (n <= 512) DLFX_TOPK_WAVE(8);
         else if (n <= 1024) DLFX_TOPK_WAVE(16);
-        else if (n <= 2048) DLFX_TOPK_WAVE(32);
-        else DLFX_TOPK_WAVE(64);
+        else DLFX_TOPK_WAVE(32);
 #undef DLFX_TOPK_WAVE
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
