@@ -110,7 +110,7 @@ constexpr int kAmbMax = 64;        // members of the deciding digit that are ran
 constexpr int kSelectThreads = 256; // threads that run the exact selection among candidates
 constexpr uint32_t kRowDone = 0u, kRowWhole = 0xffffffffu;   // per-row hand-over state (else: candidate count)
 
-template <typename K>
+template <typename K, int CAND = cand_cap<K>()>
 struct TopkShared {
     uint32_t hist[kRadix];
     uint32_t wave_tot[kRadix / kWave];
@@ -123,8 +123,8 @@ struct TopkShared {
     uint32_t amb_idx[kAmbMax];
     K and_bits[16], or_bits[16];
     uint32_t amb_count;
-    K cand_ord[cand_cap<K>()];
-    uint32_t cand_idx[cand_cap<K>()];
+    K cand_ord[CAND];                       // (rows no longer than the capacity keep at most what is merged by rank)
+    uint32_t cand_idx[CAND];
     unsigned long long pack[sizeof(K) == 4 ? 512 : 1];      // sorted runs of (image, ~index) words, 4-byte keys
 };
 
@@ -159,8 +159,8 @@ __device__ __forceinline__ uint32_t wave_append(uint32_t* counter, bool take) {
 // participating value.  Results: sm.sel_digit, sm.sel_k (rank inside that
 // digit), sm.sel_ties (its population).  sm.hist must be all zero on entry and is
 // all zero again on return.
-template <int BLOCK, int ITEMS, bool ROLLED, typename K, typename Val, typename Part>
-__device__ __forceinline__ void select_digit(TopkShared<K>& sm, int nitems, int shift, uint32_t kk, Val val, Part part) {
+template <int BLOCK, int ITEMS, bool ROLLED, typename K, int CAND, typename Val, typename Part>
+__device__ __forceinline__ void select_digit(TopkShared<K, CAND>& sm, int nitems, int shift, uint32_t kk, Val val, Part part) {
     const int tid = threadIdx.x;
     const int lane = lane_id();
     (void)lane;
@@ -205,8 +205,8 @@ __device__ __forceinline__ void select_digit(TopkShared<K>& sm, int nitems, int 
 // The kk-th largest of the values val(i) over the items with part(i): most significant
 // byte first.  Returns the value; *rank_in_ties / *ties describe how many of the elements
 // equal to it still have to be taken and how many there are.
-template <int BLOCK, int ITEMS, bool ROLLED, typename V, typename K, typename Val, typename Valid>
-__device__ __forceinline__ V kth_largest(TopkShared<K>& sm, int nitems, uint32_t kk, Val val, Valid valid,
+template <int BLOCK, int ITEMS, bool ROLLED, typename V, typename K, int CAND, typename Val, typename Valid>
+__device__ __forceinline__ V kth_largest(TopkShared<K, CAND>& sm, int nitems, uint32_t kk, Val val, Valid valid,
                                          uint32_t* rank_in_ties, uint32_t* ties,
                                          int first_pass = static_cast<int>(sizeof(V)) - 1, V known_high = 0) {
     // bytes above first_pass are the same (known_high) in every participating value
@@ -251,8 +251,8 @@ __device__ __forceinline__ uint32_t beats(K oj, uint32_t xj, K o, uint32_t x) {
 
 // For each of `count` (image, index) entries held in LDS: sm.rank[e] = number of entries that
 // beat it (entries are distinct).  Quadratic: small counts.  Ends with a barrier.
-template <int BLOCK, typename K>
-__device__ __forceinline__ void compute_ranks(TopkShared<K>& sm, const K* e_ord, const uint32_t* e_idx, int count) {
+template <int BLOCK, typename K, int CAND>
+__device__ __forceinline__ void compute_ranks(TopkShared<K, CAND>& sm, const K* e_ord, const uint32_t* e_idx, int count) {
     const int tid = threadIdx.x;
     for (int i = tid; i < count; i += BLOCK) sm.rank[i] = 0;
     team_sync<BLOCK>();
@@ -444,8 +444,8 @@ __device__ __forceinline__ void merge_rank_emit(K* e_ord, uint32_t* e_idx, unsig
 // Radix select from the first byte in which the items differ; as soon as the digit that
 // holds the limit-th best has at most kAmbMax members, those members are ranked
 // directly (by image, then index) instead of refining further.
-template <int BLOCK, int ITEMS, bool ROLLED, typename K, typename S, typename Ord, typename Idx>
-__device__ __forceinline__ void select_and_emit(TopkShared<K>& sm, const TopkIo<K, S>& io, int64_t row, const S* xr,
+template <int BLOCK, int ITEMS, bool ROLLED, typename K, int CAND, typename S, typename Ord, typename Idx>
+__device__ __forceinline__ void select_and_emit(TopkShared<K, CAND>& sm, const TopkIo<K, S>& io, int64_t row, const S* xr,
                                                 int limit, int nitems, Ord ord, Idx idx) {
     const int tid = threadIdx.x;
     const int lane = lane_id();
@@ -630,7 +630,7 @@ template <> struct BitsOf<int16_t> { using type = uint32_t; using storage = uint
 // counting, when there is only a handful).  When more than 64 elements reach the bound (long
 // runs of equal values), the wave takes the `limit` best one after the other instead: exact
 // for any input, and only slow where it is needed.
-constexpr int kWaveRowMax = 2048;       // longest row topk_rows_wave takes (beyond, the row in 64 registers a lane costs twice the time of topk_select)
+constexpr int kWaveRowMax = 1024;       // longest row topk_rows_wave takes (beyond, the pre-filter of topk_select with 256 threads a row is as fast or faster)
 constexpr int kWaveRowLimit = 32;       // largest limit: the limit-th of 64 lane maxima lets about 45 entries through at 32, more than the 64 the buffer holds from 40 on
 constexpr int kWaveSortItems = 4;       // rows of up to 64 * this many elements can be ordered whole by the wave
 
@@ -984,7 +984,13 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
     constexpr int G = ITEMS / V;
     constexpr int WAVES = BLOCK / kWave;
     using VecT = Vec<S, V>;
-    __shared__ TopkShared<K> sm;
+    constexpr int CAP = cand_cap<K>();
+    // A row whose items are no more than the candidates a longer row may leave never hands
+    // anything to a second kernel: it keeps the survivors it can rank here (kMergeMax) and
+    // otherwise selects from its registers.
+    constexpr bool kShort = BLOCK * ITEMS <= CAP;
+    constexpr uint32_t kCap = static_cast<uint32_t>(kShort ? kMergeMax : CAP);
+    __shared__ TopkShared<K, static_cast<int>(kCap)> sm;
 
     const int tid = threadIdx.x;
     const int lane = lane_id();
@@ -1006,189 +1012,177 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
     auto score_of = [&](S stored) -> T { return bit_cast<T>(static_cast<K>(widen_bits<K, S>(stored, kind) ^ flip)); };
     // order-preserving unsigned image of a score (scores are always maximised)
     auto ord_of = [&](T sc) -> K { return to_ord<K>(bit_cast<K>(sc), kind, 1); };
-    auto load_ord = [&](int i) -> K {        // straight from memory; padding -> 0
-        const uint32_t ix = index_of(i);
-        return ix < n32 ? ord_of(score_of(xr[static_cast<int64_t>(ix) * io.sx])) : K(0);
-    };
 
-    constexpr int CAP = cand_cap<K>();
-    constexpr bool kShort = BLOCK * ITEMS <= CAP;          // a row's items are no more than the candidates LDS holds
-    if constexpr (kShort && WAVES != 16) {
-        // short rows of small workgroups: select straight from registers
-        K ord[ITEMS];
+    T sc[ITEMS];
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) ord[i] = load_ord(i);
-        __syncthreads();
-        if (tid == 0) row_state[row] = kRowDone;
-        select_and_emit<BLOCK, ITEMS, false>(sm, io, row, xr, limit, ITEMS, [&](int i) { return ord[i]; }, index_of);
+    for (int g = 0; g < G; ++g) {
+        const uint32_t i0 = tid_v + static_cast<uint32_t>(g * (BLOCK * V));
+        if (ALIGNED && i0 + V <= n32) {
+            const VecT a = load_stream(reinterpret_cast<const VecT*>(xr + i0));
+#pragma unroll
+            for (int e = 0; e < V; ++e) sc[g * V + e] = score_of(a.v[e]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const int64_t at = ALIGNED ? static_cast<int64_t>(i0 + e) : static_cast<int64_t>(i0 + e) * io.sx;
+                sc[g * V + e] = (i0 + e < n32) ? score_of(xr[at]) : worst;
+            }
+        }
+    }
+    // ---- pre-filter.  The largest element of each thread is a distinct element of the
+    // row, and so is the largest of any group of threads.  A bound that provably has at
+    // least `limit` elements at or above it comes from 16 or 64 such samples:
+    //   * limit <= the number of waves: the limit-th largest of the wave maxima;
+    //   * limit <= four times that: the limit-th largest of the maxima of 16-lane rows;
+    //   * above: every wave sorts its 64 thread maxima; the value at position p*s - 1 of a
+    //     wave has p*s elements at or above it.  SPW such samples per wave (p = 1..SPW, four
+    //     from each of sixteen waves, sixteen from each of four: 64 in all) are
+    //     sorted together: the m-th largest sample has at least m*s elements at or above
+    //     it (q samples of one wave among the first m stand for q*s elements of that
+    //     wave), so with m*s >= limit it cannot exceed the limit-th largest element.
+    // Everything below the bound is out; what is left is usually 1 to 2 times `limit`.
+    constexpr int SPW = kWave / WAVES;                 // samples a wave gives in the third form: 64 in all
+    static_assert(WAVES <= 16 && SPW * WAVES == kWave, "the samples of all waves fill one wave");
+    T tmax = worst;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) tmax = sc[i] > tmax ? sc[i] : tmax;
+    // NaNs compare false with everything, so the comparisons below would drop them, while
+    // the radix selection (and the sort) place them by their bit pattern, above +inf or
+    // below -inf.  A row that holds one is therefore selected exactly (short rows from the
+    // registers below, long rows by topk_finish from the row itself); the sum of a thread's scores is NaN exactly when one of them is, or when
+    // infinities of both signs meet, which only costs that row the slower path.
+    bool nan_seen = false;
+    if constexpr (!std::is_integral<T>::value) {
+        T sum = T(0);
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) sum += sc[i];
+        nan_seen = sum != sum;
+    }
+    T* red = reinterpret_cast<T*>(sm.out_ord);
+    if (tid == 0) sm.count = 0u;
+    DLFX_PHASE(0);            // loads and thread maxima
+    auto larger = [](T a, T b) { return a > b ? a : b; };
+    // (a row shorter than the workgroup's first vectors leaves the last waves and 16-lane rows
+    // without elements: a sample from there bounds nothing, so only the full ones count)
+    const int full_waves = static_cast<int>(n32 / static_cast<uint32_t>(kWave * V));
+    const int full_rows = static_cast<int>(n32 / static_cast<uint32_t>(16 * V));
+    int samples, mth;
+    if (limit <= WAVES && limit <= full_waves) {
+        const T wmax = wave_reduce(tmax, larger);
+        if (lane == 0) red[w] = wmax;
+        samples = WAVES;
+        mth = limit;
+    } else if (limit <= 4 * WAVES && limit <= full_rows) {
+        const T rmax = group_reduce(tmax, 16, larger);
+        if ((lane & 15) == 0) red[w * 4 + (lane >> 4)] = rmax;
+        samples = 4 * WAVES;
+        mth = limit;
     } else {
-        T sc[ITEMS];
+        // (the last sample of a wave is its thread maximum number SPW * stride <= 64; a limit
+        // above the workgroup's size has no bound and is given none below)
+        constexpr int kMaxStride = kWave / SPW;
+        const int stride = (limit + 31) / 32 <= kMaxStride ? (limit + 31) / 32 : (limit + 63) / 64;
+        const T sorted = wave_sort_descending(tmax);
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
-            const uint32_t i0 = tid_v + static_cast<uint32_t>(g * (BLOCK * V));
-            if (ALIGNED && i0 + V <= n32) {
-                const VecT a = load_stream(reinterpret_cast<const VecT*>(xr + i0));
-#pragma unroll
-                for (int e = 0; e < V; ++e) sc[g * V + e] = score_of(a.v[e]);
-            } else {
-#pragma unroll
-                for (int e = 0; e < V; ++e) {
-                    const int64_t at = ALIGNED ? static_cast<int64_t>(i0 + e) : static_cast<int64_t>(i0 + e) * io.sx;
-                    sc[g * V + e] = (i0 + e < n32) ? score_of(xr[at]) : worst;
-                }
-            }
-        }
-        // ---- pre-filter.  The largest element of each thread is a distinct element of the
-        // row, and so is the largest of any group of threads.  A bound that provably has at
-        // least `limit` elements at or above it comes from 16 or 64 such samples:
-        //   * limit <= 16: the limit-th largest of the 16 wave maxima;
-        //   * limit <= 64: the limit-th largest of the 64 maxima of 16-lane rows;
-        //   * above: every wave sorts its 64 thread maxima; the value at position p*s - 1 of a
-        //     wave has p*s elements at or above it.  Four such samples per wave (p = 1..4) are
-        //     sorted together: the m-th largest sample has at least m*s elements at or above
-        //     it (q samples of one wave among the first m stand for q*s elements of that
-        //     wave), so with m*s >= limit it cannot exceed the limit-th largest element.
-        // Everything below the bound is out; what is left is usually 1 to 2 times `limit`.
-        static_assert(WAVES == 16, "four samples from each of sixteen waves fill one wave");
-        T tmax = worst;
-#pragma unroll
-        for (int i = 0; i < ITEMS; ++i) tmax = sc[i] > tmax ? sc[i] : tmax;
-        // NaNs compare false with everything, so the comparisons below would drop them, while
-        // the radix selection (and the sort) place them by their bit pattern, above +inf or
-        // below -inf.  A row that holds one is therefore selected by topk_finish from the row
-        // itself; the sum of a thread's scores is NaN exactly when one of them is, or when
-        // infinities of both signs meet, which only costs that row the slower path.
-        bool nan_seen = false;
-        if constexpr (!std::is_integral<T>::value) {
-            T sum = T(0);
-#pragma unroll
-            for (int i = 0; i < ITEMS; ++i) sum += sc[i];
-            nan_seen = sum != sum;
-        }
-        T* red = reinterpret_cast<T*>(sm.out_ord);
-        if (tid == 0) sm.count = 0u;
-        DLFX_PHASE(0);            // loads and thread maxima
-        auto larger = [](T a, T b) { return a > b ? a : b; };
-        // (a row shorter than the workgroup's first vectors leaves the last waves and 16-lane rows
-        // without elements: a sample from there bounds nothing, so only the full ones count)
-        const int full_waves = static_cast<int>(n32 / static_cast<uint32_t>(kWave * V));
-        const int full_rows = static_cast<int>(n32 / static_cast<uint32_t>(16 * V));
-        int samples, mth;
-        if (limit <= WAVES && limit <= full_waves) {
-            const T wmax = wave_reduce(tmax, larger);
-            if (lane == 0) red[w] = wmax;
-            samples = WAVES;
-            mth = limit;
-        } else if (limit <= 4 * WAVES && limit <= full_rows) {
-            const T rmax = group_reduce(tmax, 16, larger);
-            if ((lane & 15) == 0) red[w * 4 + (lane >> 4)] = rmax;
-            samples = 4 * WAVES;
-            mth = limit;
-        } else {
-            const int stride = limit <= 512 ? (limit + 31) / 32 : (limit + 63) / 64;     // <= 16
-            const T sorted = wave_sort_descending(tmax);
-#pragma unroll
-            for (int p = 1; p <= 4; ++p)
-                if (lane + 1 == p * stride) red[w * 4 + p - 1] = sorted;
-            samples = 4 * WAVES;
-            mth = (limit + stride - 1) / stride;                                       // <= 64
+        for (int p = 1; p <= SPW; ++p)
+            if (lane + 1 == p * stride) red[w * SPW + p - 1] = sorted;
+        samples = kWave;
+        mth = (limit + stride - 1) / stride;                                       // <= 64
+    }
+    __syncthreads();
+    T bound;
+    if (samples == WAVES) {
+        // sixteen samples: every wave orders them itself (ten exchange steps)
+        bound = lane < WAVES ? red[lane] : worst;
+        bound = lane_get(wave_sort_descending<16>(bound), mth - 1);
+    } else {
+        // one wave orders the samples; the others wait (sixteen waves sorting the same
+        // samples would only compete for the issue slots of the row that shares this
+        // compute unit)
+        if (w == 0) {
+            T b = wave_sort_descending(lane < samples ? red[lane] : worst);
+            b = lane_get(b, (mth - 1) & (kWave - 1));
+            if (limit > BLOCK) b = worst;
+            if (lane == 0) red[kWave] = b;
         }
         __syncthreads();
-        T bound;
-        if (samples == WAVES) {
-            // sixteen samples: every wave orders them itself (ten exchange steps)
-            bound = lane < WAVES ? red[lane] : worst;
-            bound = lane_get(wave_sort_descending<16>(bound), mth - 1);
-        } else {
-            // one wave orders the samples; the others wait (sixteen waves sorting the same
-            // samples would only compete for the issue slots of the row that shares this
-            // compute unit)
-            if (w == 0) {
-                T b = wave_sort_descending(red[lane]);
-                b = lane_get(b, mth - 1);
-                if (limit > BLOCK) b = worst;
-                if (lane == 0) red[4 * WAVES] = b;
-            }
-            __syncthreads();
-            bound = red[4 * WAVES];
+        bound = red[kWave];
+    }
+    DLFX_PHASE(1);            // bound
+    // ---- survivors go to LDS as (image, index).  A wave counts its survivors with one
+    // ballot per item, reserves that many slots with one atomic and places every survivor
+    // at the wave's base + the number of the wave's survivors before it; their order in
+    // LDS does not matter (they are ranked by image and index afterwards).  The ballots
+    // are kept in scalar registers for the second sweep while there are few enough.  What
+    // is stored is the score's bit pattern; its image is formed when the few survivors
+    // are read back.  A wave none of whose thread maxima reaches the bound has none.
+    constexpr bool kKeepMasks = ITEMS <= 32;
+    unsigned long long masks[kKeepMasks ? ITEMS : 1];
+    uint32_t wave_count = 0;
+    if (__ballot(tmax >= bound) != 0ull) {
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const unsigned long long m = __ballot(sc[i] >= bound);
+            if constexpr (kKeepMasks) masks[i] = m;
+            wave_count += static_cast<uint32_t>(__popcll(m));
         }
-        DLFX_PHASE(1);            // bound
-        // ---- survivors go to LDS as (image, index).  A wave counts its survivors with one
-        // ballot per item, reserves that many slots with one atomic and places every survivor
-        // at the wave's base + the number of the wave's survivors before it; their order in
-        // LDS does not matter (they are ranked by image and index afterwards).  The ballots
-        // are kept in scalar registers for the second sweep while there are few enough.  What
-        // is stored is the score's bit pattern; its image is formed when the few survivors
-        // are read back.  A wave none of whose thread maxima reaches the bound has none.
-        constexpr uint32_t kCap = static_cast<uint32_t>(CAP);
-        constexpr bool kKeepMasks = ITEMS <= 32;
-        unsigned long long masks[kKeepMasks ? ITEMS : 1];
-        uint32_t wave_count = 0;
-        if (__ballot(tmax >= bound) != 0ull) {
+    }
+    if (__ballot(nan_seen) != 0ull) wave_count = kCap + 1u;       // more than fits: the row goes to topk_finish
+    if (wave_count != 0u) {
+        uint32_t base = 0;
+        if (lane == 0) base = atomicAdd(&sm.count, wave_count);
+        base = lane_read(base, 0);
+        if (base + wave_count <= kCap) {
+            const unsigned long long lt_mask = (1ull << lane) - 1ull;
 #pragma unroll
             for (int i = 0; i < ITEMS; ++i) {
-                const unsigned long long m = __ballot(sc[i] >= bound);
-                if constexpr (kKeepMasks) masks[i] = m;
-                wave_count += static_cast<uint32_t>(__popcll(m));
-            }
-        }
-        if (__ballot(nan_seen) != 0ull) wave_count = kCap + 1u;       // more than fits: the row goes to topk_finish
-        if (wave_count != 0u) {
-            uint32_t base = 0;
-            if (lane == 0) base = atomicAdd(&sm.count, wave_count);
-            base = lane_read(base, 0);
-            if (base + wave_count <= kCap) {
-                const unsigned long long lt_mask = (1ull << lane) - 1ull;
-#pragma unroll
-                for (int i = 0; i < ITEMS; ++i) {
-                    unsigned long long m;
-                    if constexpr (kKeepMasks) m = masks[i];
-                    else m = __ballot(sc[i] >= bound);
-                    if (m != 0ull) {
-                        if (sc[i] >= bound) {
-                            const uint32_t slot = base + static_cast<uint32_t>(__popcll(m & lt_mask));
-                            sm.cand_ord[slot] = bit_cast<K>(sc[i]);
-                            sm.cand_idx[slot] = index_of(i);
-                        }
-                        base += static_cast<uint32_t>(__popcll(m));
+                unsigned long long m;
+                if constexpr (kKeepMasks) m = masks[i];
+                else m = __ballot(sc[i] >= bound);
+                if (m != 0ull) {
+                    if (sc[i] >= bound) {
+                        const uint32_t slot = base + static_cast<uint32_t>(__popcll(m & lt_mask));
+                        sm.cand_ord[slot] = bit_cast<K>(sc[i]);
+                        sm.cand_idx[slot] = index_of(i);
                     }
+                    base += static_cast<uint32_t>(__popcll(m));
                 }
             }
         }
-        __syncthreads();
-        const uint32_t total = sm.count;              // above the capacity: not all were stored
-        DLFX_PHASE(2);            // compaction
-        // What happens next depends on how many survived:
-        //   * up to kMergeMax: ordered here by sorted runs and ranks, answer written (handing
-        //     them to a second kernel with small workgroups was measured: slower);
-        //   * up to kCandCap: they are handed, through global memory, to topk_finish, whose
-        //     small workgroups hide the latency of an exact radix selection much better than
-        //     this one (which holds a whole row) could;
-        //   * more (long runs of equal values, adversarial order), or a limit the bound does
-        //     not hold for: topk_finish selects from the row itself.
-        if (total <= static_cast<uint32_t>(kMergeMax) && limit <= BLOCK) {
-            if (tid == 0) row_state[row] = kRowDone;
-            merge_rank_emit<BLOCK, K>(sm.cand_ord, sm.cand_idx, sm.pack, static_cast<int>(total), limit, io, row, xr,
-                                      [&](K bits) { return ord_of(bit_cast<T>(bits)); });
-            DLFX_PHASE(3);        // ordering and output
-        } else if constexpr (kShort) {
-            // a short row whose survivors are too many to rank (or that holds a NaN): exact
-            // selection from the registers, no second kernel
-            __syncthreads();                          // every thread has read the count select_and_emit clears
-            if (tid == 0) row_state[row] = kRowDone;
-            select_and_emit<BLOCK, ITEMS, false>(sm, io, row, xr, limit, ITEMS,
-                                                 [&](int i) { return index_of(i) < n32 ? ord_of(sc[i]) : K(0); }, index_of);
-        } else if (total <= CAP && limit <= BLOCK) {
-            if (tid == 0) row_state[row] = total;
-            K* so = spill_ord + row * CAP;
-            uint32_t* si = spill_idx + row * CAP;
-            for (uint32_t i = tid; i < total; i += BLOCK) {
-                so[i] = ord_of(bit_cast<T>(sm.cand_ord[i]));
-                si[i] = sm.cand_idx[i];
-            }
-        } else {
-            if (tid == 0) row_state[row] = kRowWhole;
+    }
+    __syncthreads();
+    const uint32_t total = sm.count;              // above the capacity: not all were stored
+    DLFX_PHASE(2);            // compaction
+    // What happens next depends on how many survived:
+    //   * up to kMergeMax: ordered here by sorted runs and ranks, answer written (handing
+    //     them to a second kernel with small workgroups was measured: slower);
+    //   * up to kCandCap: they are handed, through global memory, to topk_finish, whose
+    //     small workgroups hide the latency of an exact radix selection much better than
+    //     this one (which holds a whole row) could;
+    //   * more (long runs of equal values, adversarial order), or a limit the bound does
+    //     not hold for: topk_finish selects from the row itself.
+    if (total <= static_cast<uint32_t>(kMergeMax) && limit <= BLOCK) {
+        if (tid == 0) row_state[row] = kRowDone;
+        merge_rank_emit<BLOCK, K>(sm.cand_ord, sm.cand_idx, sm.pack, static_cast<int>(total), limit, io, row, xr,
+                                  [&](K bits) { return ord_of(bit_cast<T>(bits)); });
+        DLFX_PHASE(3);        // ordering and output
+    } else if constexpr (kShort) {
+        // a short row whose survivors are too many to rank (or that holds a NaN): exact
+        // selection from the registers, no second kernel
+        __syncthreads();                          // every thread has read the count select_and_emit clears
+        if (tid == 0) row_state[row] = kRowDone;
+        select_and_emit<BLOCK, ITEMS, false>(sm, io, row, xr, limit, ITEMS,
+                                             [&](int i) { return index_of(i) < n32 ? ord_of(sc[i]) : K(0); }, index_of);
+    } else if (total <= CAP && limit <= BLOCK) {
+        if (tid == 0) row_state[row] = total;
+        K* so = spill_ord + row * CAP;
+        uint32_t* si = spill_idx + row * CAP;
+        for (uint32_t i = tid; i < total; i += BLOCK) {
+            so[i] = ord_of(bit_cast<T>(sm.cand_ord[i]));
+            si[i] = sm.cand_idx[i];
         }
+    } else {
+        if (tid == 0) row_state[row] = kRowWhole;
     }
 }
 
@@ -1310,8 +1304,7 @@ int launch_select(hipStream_t stream, const TopkIo<typename BitsOf<T>::type, typ
         else if (n <= 128) DLFX_TOPK_WAVE(2);
         else if (n <= 256) DLFX_TOPK_WAVE(4);
         else if (n <= 512) DLFX_TOPK_WAVE(8);
-        else if (n <= 1024) DLFX_TOPK_WAVE(16);
-        else DLFX_TOPK_WAVE(32);
+        else DLFX_TOPK_WAVE(16);
 #undef DLFX_TOPK_WAVE
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
@@ -1323,8 +1316,14 @@ do {                                                                            
 } while (0)
     if (n <= 256) DLFX_TOPK(256, 1);
     else if (n <= 1024) DLFX_TOPK(256, 4);
-    else if (n <= 2048) DLFX_TOPK(1024, 2);
-    else if (n <= 4096) DLFX_TOPK(1024, 4);
+    else if (n <= 2048) {
+        // (a limit above the workgroup's size has no bound from the pre-filter: the larger workgroup takes those)
+        if (lim <= 256) DLFX_TOPK(256, 8);
+        else DLFX_TOPK(1024, 2);
+    } else if (n <= 4096) {
+        if (lim <= 256 && sizeof(K) == 4) DLFX_TOPK(256, 16);
+        else DLFX_TOPK(1024, 4);
+    }
     else if (n <= 8192) DLFX_TOPK(1024, 8);
     else if (n <= 16384) DLFX_TOPK(1024, 16);
     else if (n <= 32768) {

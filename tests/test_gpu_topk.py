@@ -136,12 +136,12 @@ def test_top_k_with_nans_agrees_with_the_sort(hip_backend, dtype, n, k):
 
 @pytest.mark.parametrize("n", [1, 5, 63, 64, 65, 128, 129, 255, 256, 257, 1000, 1024, 1025, 1300, 2048, 2049, 2300, 3000, 4096])
 def test_short_rows_one_wave_per_row(hip_backend, oracle_backend, n):
-    """Rows of up to 2048 elements with limits up to 32, and rows of up to 256 elements with any
+    """Rows of up to 1024 elements with limits up to 32, and rows of up to 256 elements with any
     limit (the wave then orders the whole row), are selected by one wavefront each; beyond
-    (rows of up to 4096 elements, larger limits) a workgroup per row pre-filters with a bound
-    from its full waves' maxima (a row of 2049 to 4096 elements leaves the workgroup's last
-    waves empty, and a limit above the number of full ones must not take its bound from them)
-    and selects from its registers when too many survive.
+    (rows of up to 4096 elements, larger limits) a workgroup of 256 or 1024 threads per row
+    pre-filters with a bound from its full waves' maxima (a row that does not fill the
+    workgroup leaves its last waves empty, and a limit above the number of full ones must not
+    take its bound from them) and selects from its registers when too many survive.
     Every size class, limits up to the cap, both directions, all element types, and the rows
     that defeat the bound (all equal, few distinct values, sorted either way)."""
     for dtype in (np.float32, np.int32, np.float64, np.int64, np.float16, np.int16):
@@ -151,7 +151,7 @@ def test_short_rows_one_wave_per_row(hip_backend, oracle_backend, n):
         x[3] = np.sort(x[3])
         x[4] = np.sort(x[4])[::-1]
         Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
-        for k in sorted({1, min(n, 5), min(n, 9), min(n, 16), min(n, 17), min(n, 32), min(n, 33), min(n, 64), min(n, 65), min(n, 200)}):
+        for k in sorted({1, min(n, 5), min(n, 9), min(n, 16), min(n, 17), min(n, 32), min(n, 33), min(n, 64), min(n, 65), min(n, 200), min(n, 256), min(n, 257), min(n, 700)}):
             for largest in (True, False):
                 Yh, Ih = F.top_k(Xh, k, -1, largest)
                 Yo, Io = F.top_k(Xo, k, -1, largest)
