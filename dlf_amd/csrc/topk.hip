@@ -1077,6 +1077,29 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
         if ((lane & 15) == 0) red[w * 4 + (lane >> 4)] = rmax;
         samples = 4 * WAVES;
         mth = limit;
+    } else if (ITEMS >= 2 && 2 * limit > BLOCK) {
+        // A limit above half the number of threads would take its bound from the weakest thread
+        // maxima of every wave, which most of the row exceeds.  The two halves of a thread's
+        // items are sampled as threads of their own instead: twice as many waves of maxima,
+        // half as many samples from each, all from the upper half of its 64.
+        constexpr int HALF = SPW / 2;
+        const int stride = (limit + 63) / 64;
+        T first_half = worst, second_half = worst;
+#pragma unroll
+        for (int i = 0; i < ITEMS; i += 2) {               // (every other item: a short row fills both halves)
+            first_half = larger(first_half, sc[i]);
+            if (i + 1 < ITEMS) second_half = larger(second_half, sc[i + 1]);
+        }
+        const T sorted_first = wave_sort_descending(first_half), sorted_second = wave_sort_descending(second_half);
+#pragma unroll
+        for (int p = 1; p <= HALF; ++p) {
+            if (lane + 1 == p * stride) {
+                red[w * SPW + p - 1] = sorted_first;
+                red[w * SPW + HALF + p - 1] = sorted_second;
+            }
+        }
+        samples = kWave;
+        mth = (limit + stride - 1) / stride;                                       // <= 64
     } else {
         // (the last sample of a wave is its thread maximum number SPW * stride <= 64; a limit
         // above the workgroup's size has no bound and is given none below)
@@ -1272,6 +1295,9 @@ SelectLayout select_layout(size_t key_size, int64_t m, int64_t n) {
 
 bool selection_fits(size_t key_size, int64_t n, int64_t limit) {
     if (limit > kMaxLimit) return false;
+    // more than an eighth of a short row: no bound keeps few enough candidates, and the row's
+    // whole sort on chip (one workgroup, one read) takes half the time of the exact selection
+    if (n <= 4096 && limit > 256 && limit * 8 > n) return false;
     return n <= (key_size == 4 ? 65536 : 32768);
 }
 
