@@ -804,8 +804,17 @@ int launch_small(hipStream_t stream, const PassIo<K>& io_in, int64_t m, int64_t 
     else if (n <= 8 * kWave && wave_items8) { const dim3 g = grid_for(4); sort_rows_wave_items<K, PAIRS, 8><<<g, block, 0, stream>>>(io, m, n); }
     else if (n <= 512) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 2><<<g, block, 0, stream>>>(io, m, n); }
     else if (n <= 1024) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 4><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 1536) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 6><<<g, block, 0, stream>>>(io, m, n); }
     else if (n <= 2048) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 8><<<g, block, 0, stream>>>(io, m, n); }
-    else if (n <= 4096) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 16><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 2560) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 10><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 3072) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 12><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 3584 && !(PAIRS && sizeof(K) == 8)) { const dim3 g = grid_for(1); sort_rows_small<K, PAIRS, 14><<<g, block, 0, stream>>>(io, m, n); }
+    else if (n <= 4096) {
+        // (16 8-byte keys a thread with their indices: eight wavefronts of 8 keep them in registers)
+        const dim3 g = grid_for(1);
+        if constexpr (PAIRS && sizeof(K) == 8) sort_rows_small<K, PAIRS, 8, 8><<<g, dim3(8 * kWave), 0, stream>>>(io, m, n);
+        else sort_rows_small<K, PAIRS, 16><<<g, block, 0, stream>>>(io, m, n);
+    }
     else if constexpr (sizeof(K) >= 4) {
         // eight wavefronts, 10, 12 or 16 keys a thread: 5120, 6144 or 8192 slots; sixteen for 4-byte
         // keys beyond that, 10, 12, 14 or 16 keys a thread: 10240, 12288, 14336 or 16384 slots

@@ -468,8 +468,8 @@ def test_nans_take_the_place_of_their_bit_pattern(hip_backend, dtype):
     assert (np.diff(idx[:, :200], axis=1) > 0).all()                                # equal keys keep their order
 
 
-@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8, 9, 16, 17, 32, 33, 63, 64, 65, 100, 127, 128, 129, 255, 256, 257, 300, 511, 512, 513, 1023, 1024, 1025, 2047, 2048, 2049, 4095,
-                               4096, 4097, 5119, 5120, 5121, 6144, 6145, 8191, 8192, 8193, 10240, 10241, 12288, 12289, 14336, 14337, 16383, 16384, 16385])
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8, 9, 16, 17, 32, 33, 63, 64, 65, 100, 127, 128, 129, 255, 256, 257, 300, 511, 512, 513, 1023, 1024, 1025, 1535, 1536, 1537, 2047, 2048, 2049, 2560, 2561, 3072, 3073, 3584, 3585,
+                               4095, 4096, 4097, 5119, 5120, 5121, 6144, 6145, 8191, 8192, 8193, 10240, 10241, 12288, 12289, 14336, 14337, 16383, 16384, 16385])
 def test_rows_around_the_one_workgroup_limits(hip_backend, oracle_backend, n):
     """Rows of up to 64, 128, 256 (512 for values only or 8-byte keys) elements are sorted by one
     wavefront in registers, rows of up to 4096 elements - 8192 for 8-byte keys, 16384 for 4-byte
