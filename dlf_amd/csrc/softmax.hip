@@ -453,7 +453,7 @@ int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y, v
         DLFX_CHECK_LAUNCH();                                                                                    \
         return DLFX_OK;                                                                                         \
     } while (0)
-    // (slots of a row: V, 4 V, 16 V, 32 V, 64 V, 128 V, 256 V, then 2048 and 4096 to 32768 in steps of at most half)
+    // (slots of a row: V, 4 V, 16 V, 32 V, 64 V, 128 V, 256 V, then 2048, 3072, 4096, 6144 and 8192 to 32768 in steps of at most half)
     if (np <= V) DLFX_LANE_ROWS(1, V);
     if (np <= 4 * V) DLFX_LANE_ROWS(4, V);
     if (np <= 16 * V) DLFX_LANE_ROWS(16, V);
@@ -463,9 +463,24 @@ int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y, v
     if (np <= kWave * 2 * V) DLFX_WAVE_ROWS(2 * V);
     if (np <= kWave * 4 * V) DLFX_WAVE_ROWS(4 * V);
     if (np <= kWave * 32) DLFX_WAVE_ROWS(32);
+    // a workgroup of 256 threads per row up to 8192 slots: a row of 2049 elements would leave
+    // most of 1024 threads without any
+#define DLFX_TEAM_ROWS(ITEMS)                                                                                   \
+    do {                                                                                                        \
+        const dim3 grid(static_cast<unsigned>(m));                                                              \
+        if (pad) softmax_rows<T, 256, ITEMS, KIND, true><<<grid, dim3(256), 0, stream>>>(x, y, m, n);           \
+        else softmax_rows<T, 256, ITEMS, KIND, false><<<grid, dim3(256), 0, stream>>>(x, y, m, n);              \
+        DLFX_CHECK_LAUNCH();                                                                                    \
+        return DLFX_OK;                                                                                         \
+    } while (0)
     if constexpr (V <= 4) {
-        if (np <= 1024 * 4) DLFX_BLOCK_ROWS(4);
+        if (np <= 256 * 12) DLFX_TEAM_ROWS(12);
     }
+    if (np <= 256 * 16) DLFX_TEAM_ROWS(16);
+    if constexpr (kRegisterBytes == 4) {
+        if (np <= 256 * 24) DLFX_TEAM_ROWS(24);
+    }
+#undef DLFX_TEAM_ROWS
     if (np <= 1024 * 8) DLFX_BLOCK_ROWS(8);
     if constexpr (V <= 4) {
         if (np <= 1024 * 12) DLFX_BLOCK_ROWS(12);

@@ -96,11 +96,11 @@ def test_hardmax_of_integer_rows(hip_backend, oracle_backend, dtype, n):
 
 
 @pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8, 10, 15, 16, 17, 31, 32, 33, 61, 63, 64, 65, 66, 125, 128, 129, 253, 255, 257, 509, 512, 513, 1021, 1025,
-                               2045, 2047, 2051, 4095, 4096, 4097, 8189, 8193, 12285, 12289, 16381, 16385, 24573, 24577, 32765])
+                               2045, 2047, 2051, 3069, 3072, 3073, 4095, 4096, 4097, 6141, 6144, 6145, 8189, 8193, 12285, 12289, 16381, 16385, 24573, 24577, 32765])
 def test_row_lengths_around_the_team_sizes(hip_backend, oracle_backend, n):
     """One lane per row up to 4 (fp32) / 2 (fp64) / 8 (half) elements, four lanes up to four times
     that, sixteen lanes per row up to 128 (fp32) elements, a wavefront up to 2048, a workgroup of
-    1024 threads up to 32768: the boundaries of each class.  Rows that do not start on a 16-byte
+    256 threads up to 6144 and of 1024 threads up to 32768: the boundaries of each class.  Rows that do not start on a 16-byte
     boundary (odd lengths) are laid out from the boundary before them, which moves those
     boundaries down by up to a vector less one element; the output rows here start on other
     boundaries than the input rows (a view that begins one row into its buffer)."""
