@@ -965,13 +965,19 @@ __global__ __launch_bounds__(256) void topk_cols_wave(TopkIo<typename BitsOf<E>:
     for (int a = w; a < limit; a += 4) emit_one<K>(io, yr, ir, xr, a, images[a * kPitch + r], places[a * kPitch + r]);
 }
 
-// E: the element type.  ALIGNED: the axis is contiguous and every row starts on a 16-byte
-// boundary (checked on the host), so rows are read with 128-bit loads off one base register.
+// E: the element type.  LOAD says how a row is read (the host decides): kLoadAligned - the axis
+// is contiguous and every row starts on a 16-byte boundary, so rows are read with 128-bit loads
+// off one base register; kLoadShifted - contiguous rows that start anywhere (an odd row length)
+// are laid out from the boundary before them: position p of that layout is element p - shift,
+// the positions below `shift` are padding, and every whole vector of the row is still one
+// aligned load; kLoadStrided - element by element, any stride.
 //
 // Elements are held as scores of type T: the element itself when the largest are wanted,
 // its order-reversing image otherwise (sign flip for floats, complement for integers), so
 // the kernel always looks for the largest scores and compares them natively.
-template <typename E, int BLOCK, int ITEMS, bool ALIGNED>
+constexpr int kLoadStrided = 0, kLoadAligned = 1, kLoadShifted = 2;
+
+template <typename E, int BLOCK, int ITEMS, int LOAD>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(BLOCK >= 1024 && sizeof(typename BitsOf<E>::type) == 4 && ITEMS <= 32 ? 8 : 1)))
 void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> io, int64_t n, int limit,
                  uint32_t* __restrict__ row_state, typename BitsOf<E>::type* __restrict__ spill_ord,
@@ -1001,11 +1007,14 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
     if (tid < kRadix) sm.hist[tid] = 0;
     DLFX_PHASE_BEGIN();
 
-    // item (g, e) of thread t is element ((g*BLOCK + t)*V + e) of the row
+    // item (g, e) of thread t is position ((g*BLOCK + t)*V + e) of the row: element position - shift
+    // (padding before the row gets an index far beyond it, like the padding behind it)
     const uint32_t n32 = static_cast<uint32_t>(n);        // rows here have at most 65536 elements
+    const uint32_t shift = LOAD == kLoadShifted ? static_cast<uint32_t>((reinterpret_cast<uintptr_t>(xr) / sizeof(S)) % V) : 0u;
+    const uint32_t end32 = n32 + shift;                   // positions [shift, end32) are the row
     const uint32_t tid_v = static_cast<uint32_t>(tid) * V;
     auto index_of = [&](int i) -> uint32_t {
-        return tid_v + static_cast<uint32_t>((i / V) * (BLOCK * V) + (i % V));
+        return tid_v + static_cast<uint32_t>((i / V) * (BLOCK * V) + (i % V)) - shift;
     };
     const K flip = io.largest ? K(0) : (kind == kKeyFloat ? KeyBits<K>::kSign : ~K(0));
     const T worst = std::is_integral<T>::value ? std::numeric_limits<T>::lowest() : -std::numeric_limits<T>::infinity();
@@ -1017,15 +1026,16 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
 #pragma unroll
     for (int g = 0; g < G; ++g) {
         const uint32_t i0 = tid_v + static_cast<uint32_t>(g * (BLOCK * V));
-        if (ALIGNED && i0 + V <= n32) {
-            const VecT a = load_stream(reinterpret_cast<const VecT*>(xr + i0));
+        if (LOAD != kLoadStrided && i0 >= shift && i0 + V <= end32) {
+            const VecT a = load_stream(reinterpret_cast<const VecT*>(xr + i0 - shift));
 #pragma unroll
             for (int e = 0; e < V; ++e) sc[g * V + e] = score_of(a.v[e]);
         } else {
 #pragma unroll
             for (int e = 0; e < V; ++e) {
-                const int64_t at = ALIGNED ? static_cast<int64_t>(i0 + e) : static_cast<int64_t>(i0 + e) * io.sx;
-                sc[g * V + e] = (i0 + e < n32) ? score_of(xr[at]) : worst;
+                const uint32_t ix = i0 + e - shift;
+                const int64_t at = LOAD != kLoadStrided ? static_cast<int64_t>(ix) : static_cast<int64_t>(ix) * io.sx;
+                sc[g * V + e] = (ix < n32) ? score_of(xr[at]) : worst;
             }
         }
     }
@@ -1064,8 +1074,8 @@ void topk_select(TopkIo<typename BitsOf<E>::type, typename BitsOf<E>::storage> i
     auto larger = [](T a, T b) { return a > b ? a : b; };
     // (a row shorter than the workgroup's first vectors leaves the last waves and 16-lane rows
     // without elements: a sample from there bounds nothing, so only the full ones count)
-    const int full_waves = static_cast<int>(n32 / static_cast<uint32_t>(kWave * V));
-    const int full_rows = static_cast<int>(n32 / static_cast<uint32_t>(16 * V));
+    const int full_waves = static_cast<int>(end32 / static_cast<uint32_t>(kWave * V));
+    const int full_rows = static_cast<int>(end32 / static_cast<uint32_t>(16 * V));
     int samples, mth;
     if (limit <= WAVES && limit <= full_waves) {
         const T wmax = wave_reduce(tmax, larger);
@@ -1337,22 +1347,36 @@ int launch_select(hipStream_t stream, const TopkIo<typename BitsOf<T>::type, typ
     }
 #define DLFX_TOPK(BLOCK, ITEMS)                                                                     \
 do {                                                                                            \
-    if (aligned) topk_select<T, BLOCK, ITEMS, true><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx); \
-    else topk_select<T, BLOCK, ITEMS, false><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx);      \
+    if (load == kLoadAligned) topk_select<T, BLOCK, ITEMS, kLoadAligned><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx); \
+    else if (load == kLoadShifted) topk_select<T, BLOCK, ITEMS, kLoadShifted><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx); \
+    else topk_select<T, BLOCK, ITEMS, kLoadStrided><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx);      \
 } while (0)
-    if (n <= 256) DLFX_TOPK(256, 1);
-    else if (n <= 1024) DLFX_TOPK(256, 4);
-    else if (n <= 2048) {
+    // Contiguous rows off a 16-byte boundary are laid out from the boundary before them, which
+    // takes up to a vector less one element more room: the size class is picked for that, unless
+    // it would take the row beyond what the kernel holds or into the classes that hand
+    // candidates to topk_finish through scratch the caller was not asked for.
+    int load = aligned ? kLoadAligned : kLoadStrided;
+    int64_t np = n;
+    if (!aligned && io.sx == 1 && n > 8192) {           // (shorter rows measured the same or faster element by element)
+        const int64_t padded = n + 16 / static_cast<int64_t>(sizeof(S)) - 1;
+        if (padded <= (sizeof(K) == 4 ? 65536 : 32768) && (padded <= cand_cap<K>() || n > cand_cap<K>())) {
+            load = kLoadShifted;
+            np = padded;
+        }
+    }
+    if (np <= 256) DLFX_TOPK(256, 1);
+    else if (np <= 1024) DLFX_TOPK(256, 4);
+    else if (np <= 2048) {
         // (a limit above the workgroup's size has no bound from the pre-filter: the larger workgroup takes those)
         if (lim <= 256) DLFX_TOPK(256, 8);
         else DLFX_TOPK(1024, 2);
-    } else if (n <= 4096) {
+    } else if (np <= 4096) {
         if (lim <= 256 && sizeof(K) == 4) DLFX_TOPK(256, 16);
         else DLFX_TOPK(1024, 4);
     }
-    else if (n <= 8192) DLFX_TOPK(1024, 8);
-    else if (n <= 16384) DLFX_TOPK(1024, 16);
-    else if (n <= 32768) {
+    else if (np <= 8192) DLFX_TOPK(1024, 8);
+    else if (np <= 16384) DLFX_TOPK(1024, 16);
+    else if (np <= 32768) {
         DLFX_TOPK(1024, 32);
     } else {
         if constexpr (sizeof(K) == 4) DLFX_TOPK(1024, 64);

@@ -48,6 +48,34 @@ def test_row_lengths(hip_backend, n):
         check(hip_backend, x, k, -1, False)
 
 
+@pytest.mark.parametrize("n", [1027, 4099, 8191, 8193, 8199, 16381, 16387, 32765, 32771, 50257, 65533, 65535])
+def test_rows_off_a_vector_boundary(hip_backend, oracle_backend, n):
+    """Contiguous rows of an odd length start at every offset within a 16-byte vector; beyond 8192
+    elements they are read as whole vectors from the boundary before each row, which makes a
+    row up to a vector less one element longer (a longer size class just below a class limit;
+    no change where that would take the row past what one workgroup holds, or from the rows
+    that finish in one launch into those that may spill).  Ties across the padding on either
+    side of a row, the row's first and last elements among the winners, a view that starts
+    mid-buffer, all element widths."""
+    for dtype in (np.float32, np.int64, np.float16, np.int16, np.float64):
+        x = (normal(300 + n, 6 * n) * 300).astype(dtype).reshape(6, n)
+        x[1, 0] = x[1].max() + 1                       # the first element wins
+        x[2, n - 1] = x[2].max() + 1                   # ... the last
+        x[3] = x[3, 0]                                 # all equal: the lowest indices win
+        x[4, ::3] = x[4].min()                         # a third of the row ties at the bottom
+        Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
+        for k in (1, 5, 40, 300):
+            for largest in (True, False):
+                Yh, Ih = F.top_k(Xh, k, -1, largest)
+                Yo, Io = F.top_k(Xo, k, -1, largest)
+                assert np.array_equal(Ih.numpy(), Io.numpy()), (dtype, k, largest)
+                assert np.array_equal(Yh.numpy().view(np.uint8), Yo.numpy().view(np.uint8)), (dtype, k, largest)
+        Vh, Vo = Xh.slice([1], [6], [0]), Xo.slice([1], [6], [0])      # the rows from the second on
+        Yh, Ih = F.top_k(Vh, 7, -1, True)
+        Yo, Io = F.top_k(Vo, 7, -1, True)
+        assert np.array_equal(Ih.numpy(), Io.numpy()) and np.array_equal(Yh.numpy().view(np.uint8), Yo.numpy().view(np.uint8))
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int64])
 def test_dtypes_and_axes(hip_backend, dtype):
     if np.dtype(dtype).kind == "f":
