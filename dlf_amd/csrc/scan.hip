@@ -426,7 +426,9 @@ __global__ __launch_bounds__(kBlock) void scan_rows_group(
     int64_t rows, int64_t n, int exclusive, int pad) {
     static_assert(LANES == 1 || LANES == 4 || LANES == 16 || LANES == kWave, "a thread, a quad, a DPP row or a wavefront");
     using Op = ScanOp<T, K>;
-    constexpr int V = (scan_vec<T, X, Y>() < ITEMS) ? scan_vec<T, X, Y>() : ITEMS;
+    constexpr int V0 = (scan_vec<T, X, Y>() < ITEMS) ? scan_vec<T, X, Y>() : ITEMS;
+    constexpr int V = ITEMS % V0 == 0 ? V0 : V0 / 2;      // (12 items of a 16-bit type: vectors of 4)
+    static_assert(ITEMS % V == 0, "whole vectors per lane");
     constexpr int KV = ITEMS / V;
     using VecX = Vec<X, V>;
     using VecY = Vec<Y, V>;
@@ -663,6 +665,10 @@ bool make_dim_map2(const int64_t* dims, const int64_t* sx, const int64_t* sy, in
 constexpr int kChainBlock = DLFX_SCAN_CHAIN_BLOCK;
 constexpr int64_t kChainTileBytes = DLFX_SCAN_CHAIN_BYTES;
 
+#ifndef DLFX_SCAN_GROUP_ROW_MAX
+#define DLFX_SCAN_GROUP_ROW_MAX 768
+#endif
+constexpr int64_t kGroupRowMax = DLFX_SCAN_GROUP_ROW_MAX;      // longest row (in slots) a group of lanes scans
 constexpr int64_t kMaxPad = 15;        // the most positions a row gains when it is tiled from the vector boundary before it
 
 // Elements per tile: 256 bytes per thread for chained rows, less for short rows.
@@ -768,11 +774,11 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
         for (int i = 0; i < xmap.rank; ++i) aligned = aligned && xmap.strides[i] % VX == 0;
         if (!aligned) pad = VX - 1;
     }
-    // Short rows along a unit-stride axis: a group of lanes per row (rows of up to 512 elements;
+    // Short rows along a unit-stride axis: a group of lanes per row (rows of up to 768 elements;
     // a workgroup per row would leave most of its threads, or of the chip, idle).
-    if (!axis_general && axis_unit && n + pad <= 512 && m >= 4) {
+    if (!axis_general && axis_unit && n + pad <= kGroupRowMax && m >= 4) {
         const int64_t np = n + pad;
-        const int64_t lanes = np <= 4 ? 1 : np <= 32 ? 4 : np <= 128 ? 16 : kWave;
+        const int64_t lanes = np <= 4 ? 1 : np <= 32 ? 4 : np <= 192 ? 16 : kWave;
         const int64_t blocks = ceil_div(m * lanes, kBlock);
         if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
         const dim3 grid(static_cast<unsigned>(blocks)), block(kBlock);
@@ -783,8 +789,10 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
         else if (np <= 32) DLFX_SCAN_GROUP(4, 8);
         else if (np <= 64) DLFX_SCAN_GROUP(16, 4);
         else if (np <= 128) DLFX_SCAN_GROUP(16, 8);
+        else if (np <= 192) DLFX_SCAN_GROUP(16, 12);
         else if (np <= 256) DLFX_SCAN_GROUP(kWave, 4);
-        else DLFX_SCAN_GROUP(kWave, 8);
+        else if (np <= 512) DLFX_SCAN_GROUP(kWave, 8);
+        else DLFX_SCAN_GROUP(kWave, 12);
 #undef DLFX_SCAN_GROUP
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;

@@ -453,15 +453,18 @@ int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y, v
         DLFX_CHECK_LAUNCH();                                                                                    \
         return DLFX_OK;                                                                                         \
     } while (0)
-    // (slots of a row: V, 4 V, 16 V, 32 V, 64 V, 128 V, 256 V, then 2048, 3072, 4096, 6144 and 8192 to 32768 in steps of at most half)
+    // (slots of a row: V, 4 V, 16 V, 32 V, 48 V, 64 V, 128 V, 192 V, 256 V, 384 V, then 2048, 3072, 4096, 6144 and 8192 to 32768 in steps of at most half)
     if (np <= V) DLFX_LANE_ROWS(1, V);
     if (np <= 4 * V) DLFX_LANE_ROWS(4, V);
     if (np <= 16 * V) DLFX_LANE_ROWS(16, V);
     if (np <= 32 * V) DLFX_LANE_ROWS(16, 2 * V);
+    if (np <= 48 * V) DLFX_LANE_ROWS(16, 3 * V);
 #undef DLFX_LANE_ROWS
     if (np <= kWave * V) DLFX_WAVE_ROWS(V);
     if (np <= kWave * 2 * V) DLFX_WAVE_ROWS(2 * V);
+    if (np <= kWave * 3 * V) DLFX_WAVE_ROWS(3 * V);
     if (np <= kWave * 4 * V) DLFX_WAVE_ROWS(4 * V);
+    if (np <= kWave * 6 * V && kWave * 6 * V < kWave * 32) DLFX_WAVE_ROWS(6 * V);
     if (np <= kWave * 32) DLFX_WAVE_ROWS(32);
     // a workgroup of 256 threads per row up to 8192 slots: a row of 2049 elements would leave
     // most of 1024 threads without any

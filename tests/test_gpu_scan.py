@@ -167,9 +167,9 @@ def test_in_place_long_rows_use_tickets(hip_backend, oracle_backend):
     assert not np.array_equal(Xo.numpy(), Xh.numpy())     # the restated reference loop reproduces the slip
 
 
-@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 7, 8, 9, 13, 15, 16, 17, 63, 64, 65, 255, 256, 257, 511, 512, 513])
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 7, 8, 9, 13, 15, 16, 17, 63, 64, 65, 127, 128, 129, 191, 192, 193, 255, 256, 257, 511, 512, 513, 767, 768, 769])
 def test_short_rows_one_lane_group_per_row(hip_backend, oracle_backend, n):
-    """Rows of up to 512 elements along a unit-stride axis are scanned by a group of 1, 4, 16 or
+    """Rows of up to 768 elements along a unit-stride axis are scanned by a group of 1, 4, 16 or
     64 lanes each.  Every size class; all four scans; exclusive and reversed; integer results are
     exact, floating ones within the usual bound of the fp64 evaluation."""
     m = 37 if n > 16 else 1037                       # several workgroups of thread- and quad-sized groups
@@ -208,7 +208,7 @@ def test_short_rows_one_lane_group_per_row(hip_backend, oracle_backend, n):
     assert np.array_equal(F.cumsum(Xi.transpose(), 0).numpy(), np.cumsum(xi, axis=1, dtype=np.int32).T)
 
 
-@pytest.mark.parametrize("n", [9, 70, 300, 1000, 5000, 16383, 16387, 40001, 150003])
+@pytest.mark.parametrize("n", [9, 70, 130, 190, 300, 601, 766, 1000, 5000, 16383, 16387, 40001, 150003])
 def test_rows_off_a_vector_boundary(hip_backend, oracle_backend, n):
     """Unit-stride rows that do not start on a 16-byte boundary - odd row lengths, views cut one or
     two elements into a row - are laid out from the boundary before each row, so that their whole

@@ -95,7 +95,7 @@ def test_hardmax_of_integer_rows(hip_backend, oracle_backend, dtype, n):
         F.softmax(Tensor.from_numpy(hip_backend, x), 1)
 
 
-@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8, 10, 15, 16, 17, 31, 32, 33, 61, 63, 64, 65, 66, 125, 128, 129, 253, 255, 257, 509, 512, 513, 1021, 1025,
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8, 10, 15, 16, 17, 31, 32, 33, 61, 63, 64, 65, 66, 125, 128, 129, 189, 192, 193, 253, 255, 257, 509, 512, 513, 765, 768, 769, 1021, 1025, 1533, 1536, 1537,
                                2045, 2047, 2051, 3069, 3072, 3073, 4095, 4096, 4097, 6141, 6144, 6145, 8189, 8193, 12285, 12289, 16381, 16385, 24573, 24577, 32765])
 def test_row_lengths_around_the_team_sizes(hip_backend, oracle_backend, n):
     """One lane per row up to 4 (fp32) / 2 (fp64) / 8 (half) elements, four lanes up to four times
