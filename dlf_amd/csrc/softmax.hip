@@ -491,6 +491,20 @@ int launch_softmax(hipStream_t stream, int64_t m, int64_t n, const T* x, T* y, v
     if (np <= 1024 * 16) DLFX_BLOCK_ROWS(16);
     if (np <= 1024 * 24 && kRegisterBytes == 4) DLFX_BLOCK_ROWS(24);
     if (np <= 1024 * 32 && kRegisterBytes == 4) DLFX_BLOCK_ROWS(32);
+    // Longer rows, when there is at least one for every compute unit: up to 64 registers a thread
+    // hold the row (one workgroup on a compute unit), which reads it once where the streamed
+    // kernel reads it twice.
+    if (m >= kSplitMaxRows) {
+        if constexpr (kRegisterBytes == 4) {
+            if (np <= 1024 * 40) DLFX_BLOCK_ROWS(40);
+            if (np <= 1024 * 48) DLFX_BLOCK_ROWS(48);
+            if (np <= 1024 * 56) DLFX_BLOCK_ROWS(56);
+            if (np <= 1024 * 64) DLFX_BLOCK_ROWS(64);
+        } else {
+            if (np <= 1024 * 24) DLFX_BLOCK_ROWS(24);
+            if (np <= 1024 * 32) DLFX_BLOCK_ROWS(32);
+        }
+    }
 #undef DLFX_WAVE_ROWS
 #undef DLFX_BLOCK_ROWS
     const size_t need = split_scratch_bytes<T>(m, n);

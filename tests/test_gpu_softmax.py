@@ -128,6 +128,38 @@ def test_row_lengths_around_the_team_sizes(hip_backend, oracle_backend, n):
             assert np.array_equal(F.hardmax(Vh).numpy(), F.hardmax(Vo).numpy())
 
 
+@pytest.mark.parametrize("n,dtype", [(32769, np.float32), (40957, np.float32), (40960, np.float32), (49153, np.float32), (50257, np.float32),
+                                     (57344, np.float32), (65533, np.float32), (65536, np.float32), (65537, np.float32), (50257, np.float16),
+                                     (65536, np.float16), (16385, np.float64), (24577, np.float64), (32765, np.float64), (32768, np.float64)])
+def test_many_long_rows_are_held_in_registers(hip_backend, oracle_backend, n, dtype):
+    """With at least 256 rows, rows of up to 65536 4-byte (32768 8-byte) elements are held in the
+    registers of one workgroup, 40 to 64 a thread, and read once; longer ones are streamed.
+    All three kinds, rows that start off a 16-byte boundary, a NaN in position 0 and elsewhere,
+    -inf entries, a constant row."""
+    m = 257
+    x = (normal(280 + n, m * n) * 3).astype(dtype).reshape(m, n)
+    x[0, n // 3] = -np.inf
+    x[1, 0] = np.nan
+    x[2, n - 5] = np.nan
+    x[3] = 2.5
+    Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
+    eps = float(np.finfo(np.float32 if dtype == np.float16 else dtype).eps)
+    out_ulp = 2.0 ** -10 if dtype == np.float16 else 0.0
+    slack = 8 * np.log2(n) * eps + out_ulp
+    clean = [r for r in range(m) if r not in (1, 2)]
+    x64 = x[clean].astype(np.float64)
+    got = F.softmax(Xh).numpy().astype(np.float64)
+    want = sp_softmax(x64, axis=1)
+    assert (np.abs(got[clean] - want) <= want * slack + 1e-30 + (2.0 ** -24 if dtype == np.float16 else 0)).all()
+    assert np.isnan(got[1]).all() and np.isnan(got[2]).all()
+    got = F.logsoftmax(Xh).numpy().astype(np.float64)
+    want = sp_log_softmax(x64, axis=1)
+    fin = np.isfinite(want)
+    assert (np.abs(got[clean][fin] - want[fin]) <= slack * (1 + np.abs(want[fin])) + out_ulp * np.abs(want[fin])).all()
+    assert np.array_equal(np.isneginf(got[clean]), np.isneginf(want))
+    assert np.array_equal(F.hardmax(Xh).numpy(), F.hardmax(Xo).numpy())
+
+
 @pytest.mark.parametrize("m,n,dtype", [(1, 200000, np.float32), (3, 70001, np.float32), (7, 40000, np.float64), (2, 32769, np.float32),
                                        (5, 16385, np.float64), (2, 100000, np.float16), (200, 33000, np.float32)])
 def test_few_long_rows_are_cut_into_tiles(hip_backend, oracle_backend, m, n, dtype):
