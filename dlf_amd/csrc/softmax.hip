@@ -4,10 +4,12 @@
 // hardmax a one at the first occurrence of the maximum and zeros elsewhere; hardmax also takes
 // int32 / int64 rows, gpgpu/src/gdnn.cpp:1888-1900).
 //
-// A row is read once: it lives in the registers of a team of threads (one wavefront for rows
-// up to 2048 elements, a 1024-thread workgroup up to 32768 four-byte elements) between the
-// load, the two team-wide reductions and the store.  Longer rows are streamed twice (running
-// maximum and rescaled sum first, then the outputs).  Bandwidth bound; exp and log in the
+// A row is read once: it lives in the registers of a team of threads (1, 4 or 16 lanes for
+// the shortest rows, one wavefront up to 2048 elements, a 256-thread workgroup up to 6144, a
+// 1024-thread workgroup up to 32768 four-byte elements, and up to 65536 when there are
+// enough rows for every compute unit) between the load, the two team-wide reductions and the
+// store.  Longer rows are streamed twice (running maximum and rescaled sum first, then the
+// outputs), a few long rows cut into tiles over the whole device.  Bandwidth bound; exp and log in the
 // element type, sums in it as well (tree order), as the reference's row loops do.  IEEE half
 // rows are widened to float at the load and rounded once at the store.
 #include <cmath>

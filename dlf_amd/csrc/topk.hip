@@ -1,15 +1,19 @@
 // top_k along the last axis of strided views for gfx950.
 //
-// Selection kernel (rows up to 65536 elements, limit up to 1024): one workgroup
-// per row reads the row exactly once into registers as order-preserving
-// unsigned keys, finds the limit-th best key with a most-significant-digit
-// radix select over LDS histograms (no further global reads), breaks ties at
-// the threshold by lowest source index with the same select over the indices,
-// compacts the winners into LDS, orders them with a bitonic network and writes
-// values and indices.  Among equal values the lowest index always comes first.
+// Selection kernel (rows up to 65536 elements, limit up to 1024): one workgroup of 256 or
+// 1024 threads per row reads the row exactly once into registers, takes a bound that at
+// least `limit` elements reach from samples of its threads' maxima, compacts the elements
+// that reach it into LDS and orders those few by sorted runs and rank merging; a row with
+// too many survivors (long runs of equal values, a limit that is a large part of the row)
+// is selected exactly, by a most-significant-digit radix select over LDS histograms: from
+// its registers when the row is short, by a second kernel from spilled candidates or the
+// row itself otherwise.  Among equal values the lowest index always comes first.
 //
-// Anything larger goes through the stable segmented argsort and keeps the first
-// `limit` entries of each row.
+// Around it: one wavefront per row for rows of up to 1024 elements and limits up to 32, one
+// thread per row for many very short rows, kernels for rows that lie side by side in memory
+// (an outer axis), two levels of selection for rows longer than one workgroup holds.
+// Limits above 1024, or that are a large part of a short row, go through the stable
+// argsort and keep the first `limit` entries of each row.
 #include <cstring>
 #include <limits>
 #include <type_traits>
