@@ -20,6 +20,14 @@
 
 #include "common.hip.h"
 
+// This file is compiled three times, once for each width of element, so that the three sets of
+// kernels compile side by side: part 0 (this file on its own) holds the 32-bit elements and
+// everything that is not a template, the entry points included; topk_wide.hip includes it as
+// part 1 for the 64-bit elements, topk_narrow.hip as part 2 for the 16-bit ones.
+#ifndef DLFX_TOPK_PART
+#define DLFX_TOPK_PART 0
+#endif
+
 namespace dlfx {
 
 // from sort.hip
@@ -767,7 +775,13 @@ constexpr int kColsLimit = 16;         // largest limit topk_cols takes
 constexpr int kThreadRowLimit = 8;     // ... and topk_rows_thread
 // longest row topk_rows_thread takes with 4-byte keys, half of it with 8-byte keys
 // (dlfx_set_tuning "topk_thread_rows"); beyond, a wave per row has enough rows in flight and wins
+}  // namespace
+#if DLFX_TOPK_PART == 0
 int g_topk_thread_rows = 256;
+#else
+extern int g_topk_thread_rows;
+#endif
+namespace {
 
 template <typename K, int KMAX>
 __device__ __forceinline__ void cols_insert(K (&lo)[KMAX], uint32_t (&li)[KMAX], K o, uint32_t x) {
@@ -1368,17 +1382,23 @@ do {                                                                            
             np = padded;
         }
     }
-    if (np <= 256) DLFX_TOPK(256, 1);
-    else if (np <= 1024) DLFX_TOPK(256, 4);
+    // (rows of up to 8192 elements are never read in the shifted layout)
+#define DLFX_TOPK_SHORT(BLOCK, ITEMS)                                                               \
+do {                                                                                            \
+    if (load == kLoadAligned) topk_select<T, BLOCK, ITEMS, kLoadAligned><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx); \
+    else topk_select<T, BLOCK, ITEMS, kLoadStrided><<<grid, dim3(BLOCK), 0, stream>>>(io, n, lim, row_state, spill_ord, spill_idx);      \
+} while (0)
+    if (np <= 1024) DLFX_TOPK_SHORT(256, 4);
     else if (np <= 2048) {
         // (a limit above the workgroup's size has no bound from the pre-filter: the larger workgroup takes those)
-        if (lim <= 256) DLFX_TOPK(256, 8);
-        else DLFX_TOPK(1024, 2);
+        if (lim <= 256) DLFX_TOPK_SHORT(256, 8);
+        else DLFX_TOPK_SHORT(1024, 2);
     } else if (np <= 4096) {
-        if (lim <= 256 && sizeof(K) == 4) DLFX_TOPK(256, 16);
-        else DLFX_TOPK(1024, 4);
+        if (lim <= 256 && sizeof(K) == 4) DLFX_TOPK_SHORT(256, 16);
+        else DLFX_TOPK_SHORT(1024, 4);
     }
-    else if (np <= 8192) DLFX_TOPK(1024, 8);
+    else if (np <= 8192) DLFX_TOPK_SHORT(1024, 8);
+#undef DLFX_TOPK_SHORT
     else if (np <= 16384) DLFX_TOPK(1024, 16);
     else if (np <= 32768) {
         DLFX_TOPK(1024, 32);
@@ -1590,6 +1610,7 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
 
 }  // namespace
 
+#if DLFX_TOPK_PART == 0
 bool set_topk_tuning(const char* key, int64_t value) {
     if (!std::strcmp(key, "topk_thread_rows") && value >= 0 && value <= 65536) {
         g_topk_thread_rows = static_cast<int>(value);
@@ -1597,11 +1618,30 @@ bool set_topk_tuning(const char* key, int64_t value) {
     }
     return false;
 }
+#endif
+
+// the other widths' translation units
+#define DLFX_TOPK_ARGS                                                                                              \
+    hipStream_t s, int64_t limit, int dir, int dtype, int index_dtype, int rank, const int64_t *x_dims,             \
+        const int64_t *y_dims, const void *xp, const int64_t *x_strides, void *yp, const int64_t *y_strides, void *ip, \
+        const int64_t *i_strides, void *scratch, size_t scratch_bytes
+#define DLFX_TOPK_PASS s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes
+int top_k_wide(DLFX_TOPK_ARGS);
+int top_k_narrow(DLFX_TOPK_ARGS);
+#if DLFX_TOPK_PART == 1
+int top_k_wide(DLFX_TOPK_ARGS) {
+    return dtype == DLFX_F64 ? run_top_k<double>(DLFX_TOPK_PASS) : run_top_k<int64_t>(DLFX_TOPK_PASS);
+}
+#elif DLFX_TOPK_PART == 2
+int top_k_narrow(DLFX_TOPK_ARGS) {
+    return dtype == DLFX_F16 ? run_top_k<half_t>(DLFX_TOPK_PASS) : run_top_k<int16_t>(DLFX_TOPK_PASS);
+}
+#endif
 }  // namespace dlfx
 
 using namespace dlfx;
 
-#ifdef DLFX_TOPK_TIMING
+#if defined(DLFX_TOPK_TIMING) && DLFX_TOPK_PART == 0
 extern "C" void dlfx_debug_topk_phases(unsigned long long* out, int reset) {
     static unsigned long long host[dlfx::kPhaseSlots * 8];
     if (out) {
@@ -1632,6 +1672,7 @@ size_t top_k_scratch_impl(int dtype, int64_t m, int64_t n, int64_t limit) {
 }  // namespace
 }  // namespace dlfx
 
+#if DLFX_TOPK_PART == 0
 extern "C" size_t dlfx_top_k_scratch_bytes(int dtype, int64_t m, int64_t n, int64_t limit) {
     return top_k_scratch_impl(dtype, m, n, limit);
 }
@@ -1657,12 +1698,13 @@ extern "C" int dlfx_top_k(dlfx_stream_t stream, int64_t limit, int dir, int dtyp
     void* ip = static_cast<char*>(idx) + i_offset * (index_dtype == DLFX_I64 ? 8 : 4);
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (dtype) {
-    case DLFX_F32: return run_top_k<float>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
-    case DLFX_I32: return run_top_k<int32_t>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
-    case DLFX_F64: return run_top_k<double>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
-    case DLFX_I64: return run_top_k<int64_t>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
-    case DLFX_F16: return run_top_k<half_t>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
-    case DLFX_I16: return run_top_k<int16_t>(s, limit, dir, dtype, index_dtype, rank, x_dims, y_dims, xp, x_strides, yp, y_strides, ip, i_strides, scratch, scratch_bytes);
+    case DLFX_F32: return run_top_k<float>(DLFX_TOPK_PASS);
+    case DLFX_I32: return run_top_k<int32_t>(DLFX_TOPK_PASS);
+    case DLFX_F64:
+    case DLFX_I64: return top_k_wide(DLFX_TOPK_PASS);
+    case DLFX_F16:
+    case DLFX_I16: return top_k_narrow(DLFX_TOPK_PASS);
     default: return DLFX_ERR_UNSUPPORTED_DTYPE;
     }
 }
+#endif
