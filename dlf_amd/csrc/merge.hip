@@ -50,11 +50,12 @@ struct MergeViews {
     int64_t na, nb;
 };
 
-// Eight lanes per tile boundary probe eight evenly spaced split candidates at once: a boundary
-// takes about log9 of the row length dependent memory round trips instead of log2, for 2.4
-// times the probes (64 lanes per boundary cut the round trips further but fetched as many
-// cache lines as the merge itself moves).
-constexpr int kProbe = 8;
+// Four lanes per tile boundary probe four evenly spaced split candidates at once: a boundary
+// takes about log5 of the row length dependent memory round trips instead of log2.  The kernel
+// is bound by the cache lines its probes fetch as much as by those round trips: with 16 384
+// boundaries, 8 lanes each (log9) measured 3 to 4 % slower, 16 lanes 7 % slower, 64 lanes
+// fetched as many cache lines as the merge itself moves; 1 lane (plain bisection) 5 % slower.
+constexpr int kProbe = 4;
 
 template <typename T, bool DESC>
 __global__ __launch_bounds__(kBlock) void merge_partition(const T* __restrict__ x, const T* __restrict__ y, MergeViews v,
