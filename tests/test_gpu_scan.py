@@ -156,6 +156,12 @@ def test_in_place_long_rows_use_tickets(hip_backend, oracle_backend):
     F.cumsum(Xh, 1, out=Xh)
     F.cumsum(Xo, 1, out=Xo)
     assert np.array_equal(Xh.numpy(), Xo.numpy())
+    # ... and rows off a 16-byte boundary (an odd length), whose tiles start before the row
+    for n in (300001, 70003):
+        z = randint(54 + n, 5 * n, -100, 100).astype(np.int32).reshape(5, n)
+        Z = Tensor.from_numpy(hip_backend, z)
+        F.cumsum(Z, 1, out=Z)
+        assert np.array_equal(Z.numpy(), np.cumsum(z, axis=1, dtype=np.int32))
     # In-place *exclusive* scans: the reference's CPU loop stores the running value
     # into y before it reads x (reduce_detail.h:183-187), so with y aliasing x it
     # loses the input it has yet to read.  That is a read-after-write slip, not a

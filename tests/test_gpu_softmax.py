@@ -213,10 +213,12 @@ def test_few_long_rows_are_cut_into_tiles(hip_backend, oracle_backend, m, n, dty
     assert (np.abs(a - b) <= b * 2 * slack + 1e-30 + (2.0 ** -23 if dtype == np.float16 else 0)).all()
 
 
-@pytest.mark.parametrize("n", [3000, 20000, 32768])
+@pytest.mark.parametrize("n", [3000, 3001, 5001, 20000, 20003, 32766, 32768, 50257])
 def test_hardmax_in_place_with_a_leading_nan(hip_backend, n):
     """In place (the reference's routine, gdnn.h:253-264, only works in place) on rows held by a
-    1024-thread workgroup: a row that starts with a NaN keeps position 0 hot (nothing compares
+    workgroup of 256 or 1024 threads, rows off a 16-byte boundary among them (odd lengths: the
+    first and last vectors of a row are then shared with its neighbours, which other workgroups
+    rewrite at the same time): a row that starts with a NaN keeps position 0 hot (nothing compares
     larger than a NaN in the serial loop, dnn_detail.h:334-346), and exactly one element is hot,
     whichever wave stores element 0 first."""
     x = (normal(171 + n, 64 * n) * 3).astype(np.float32).reshape(64, n)
@@ -229,3 +231,9 @@ def test_hardmax_in_place_with_a_leading_nan(hip_backend, n):
         y = X.numpy()
         assert (y.sum(axis=1) == 1).all()
         assert (y[::2, 0] == 1).all() and (y[1::2, n - 1] == 1).all()
+    # softmax in place agrees with softmax out of place
+    x[::2, 0] = 0.5
+    X.storage.copy_(Tensor.from_numpy(hip_backend, x).storage)
+    want = F.softmax(Tensor.from_numpy(hip_backend, x)).numpy()
+    hip_backend.softmax("softmax", F.dtype_code(np.float32), 64, n, X.storage, 0, X.storage, 0)
+    assert np.array_equal(X.numpy(), want)
