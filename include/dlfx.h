@@ -86,7 +86,7 @@ int dlfx_last_hip_error(void);
  *                      buckets of equal depth by value and each bucket is sorted on chip, wherever
  *                      a row's keys allow it (each row decides on the device); 0: every row takes
  *                      the least-significant-digit-first passes.  Same results either way.
- *   "sort_compare_max" fullest counting bin (default 96) of a bucket whose entries are still ranked
+ *   "sort_compare_max" fullest counting bin (default 32) of a bucket whose entries are still ranked
  *                      by comparing them; fuller bins send the bucket through stable digit passes
  *                      (0: every bucket).  Same results for every value.
  *   "topk_thread_rows" longest row (default 256; half of it for 8-byte keys) for which top_k

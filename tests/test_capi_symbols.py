@@ -52,7 +52,7 @@ def test_host_only_calls():
     assert lib.dlfx_sort_scratch_bytes(3, 256, 1 << 20) >= 2 * 256 * (1 << 20) * 8
     assert lib.dlfx_set_tuning(b"no_such_knob", 1) == -3
     assert lib.dlfx_set_tuning(b"scan_poll_limit", 2048) == 0
-    for knob, value in ((b"sort_poll_limit", 2048), (b"sort_wave_rows", 512), (b"sort_buckets", 1), (b"sort_compare_max", 96), (b"topk_thread_rows", 256)):
+    for knob, value in ((b"sort_poll_limit", 2048), (b"sort_wave_rows", 512), (b"sort_buckets", 1), (b"sort_compare_max", 32), (b"topk_thread_rows", 256)):
         assert lib.dlfx_set_tuning(knob, value) == 0
     assert lib.dlfx_set_tuning(b"sort_wave_rows", 100000) == -3
 

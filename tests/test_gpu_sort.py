@@ -250,14 +250,14 @@ def test_buckets_ranked_by_comparison_or_by_digit_passes(hip_backend, dtype, n):
     Xh = Tensor.from_numpy(hip_backend, x)
     order = np.argsort(x, axis=-1, kind="stable")
     want = np.take_along_axis(x, order, -1)
-    for limit in (0, 96, 4096):
+    for limit in (0, 32, 96, 4096):
         hip_backend.set_tuning("sort_compare_max", limit)
         try:
             Yh, Ih = F.argsort(Xh, -1, False, with_values=True)
             Id = F.argsort(Xh, -1, True).numpy().astype(np.int64)
             Sh = F.sort(Xh, -1).numpy()
         finally:
-            hip_backend.set_tuning("sort_compare_max", 96)
+            hip_backend.set_tuning("sort_compare_max", 32)
         assert np.array_equal(Ih.numpy(), order) and np.array_equal(Yh.numpy().view(np.uint8), want.view(np.uint8)), limit
         assert np.array_equal(np.sort(x, axis=-1).view(np.uint8), Sh.view(np.uint8)), limit
         got = np.take_along_axis(x, Id, -1)
