@@ -87,7 +87,7 @@ def build_veneer_test(force=False):
     if not force and os.path.exists(out) and os.path.getmtime(out) > newest:
         return out
     cmd = [_hipcc(), "-O2", "-std=c++17", "-I", inc, "-I", os.path.join(HERE, "..", "include"), src, "-o", out,
-           "-L", os.path.dirname(LIB), "-ldlfx", "-Wl,-rpath,$ORIGIN/../../dlf_amd/lib"]
+           "-pthread", "-L", os.path.dirname(LIB), "-ldlfx", "-Wl,-rpath,$ORIGIN/../../dlf_amd/lib"]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("veneer test build failed:\n" + r.stderr)

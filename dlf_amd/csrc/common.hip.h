@@ -435,6 +435,16 @@ int record_hip_error(hipError_t e);
         if (e_ != hipSuccess) return dlfx::record_hip_error(e_); \
     } while (0)
 
+// Workgroups of `kernel` that the current device holds at once (0 when HIP cannot tell).
+template <typename Kernel>
+int64_t resident_workgroups(Kernel kernel, int block) {
+    int device = 0, units = 0, per_unit = 0;
+    if (hipGetDevice(&device) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_unit, kernel, block, 0) != hipSuccess) return 0;
+    return static_cast<int64_t>(units) * per_unit;
+}
+
 // True when launches into `stream` are being recorded into a graph (or that cannot be told).
 inline bool stream_is_capturing(hipStream_t stream) {
     hipStreamCaptureStatus status = hipStreamCaptureStatusNone;

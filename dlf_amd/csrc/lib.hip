@@ -38,6 +38,7 @@ extern "C" const char* dlfx_status_string(int status) {
     case DLFX_ERR_RANK: return "view rank exceeds DLFX_MAX_RANK";
     case DLFX_ERR_LAUNCH: return "HIP launch failed";
     case DLFX_ERR_TOO_LARGE: return "extent too large for this kernel";
+    case DLFX_ERR_CAPTURING: return "the first call on a device cannot be recorded into a graph";
     default: return "unknown status";
     }
 }

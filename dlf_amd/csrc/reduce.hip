@@ -774,13 +774,15 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 constexpr int kMaxDevices = 64;
 std::atomic<void*> g_static_scratch[kMaxDevices];
 
-int static_scratch_of_current_device(void** out) {
+int static_scratch_of_current_device(hipStream_t stream, void** out) {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return record_hip_error(e);
     if (dev < 0 || dev >= kMaxDevices) return DLFX_ERR_INVALID_ARGUMENT;
     void* p = g_static_scratch[dev].load(std::memory_order_acquire);
     if (!p) {
+        // the lookup may load the code object: not something to do while a graph is being recorded
+        if (stream_is_capturing(stream)) return DLFX_ERR_CAPTURING;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         if (e != hipSuccess) return record_hip_error(e);
         if (!p) return record_hip_error(hipErrorInvalidSymbol);
@@ -810,7 +812,7 @@ extern "C" int dlfx_reduce_static(dlfx_stream_t stream, const char* name, int dt
     // Same bound as the caller of dlfx_reduce would have to provide; beyond the array: refuse.
     if (partial_bound_bytes(m) > kStaticScratchBytes) return DLFX_ERR_TOO_LARGE;
     void* ptr = nullptr;
-    const int st = static_scratch_of_current_device(&ptr);
+    const int st = static_scratch_of_current_device(static_cast<hipStream_t>(stream), &ptr);
     if (st != DLFX_OK) return st;
     // Partials are written by the first kernel before the second reads them: nothing to clear.
     return reduce_entry(stream, name, dtype, m, n, x_rank, x_dims, x_strides, x, x_offset,

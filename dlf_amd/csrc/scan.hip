@@ -6,11 +6,15 @@
 //     once.  Inside a tile each wave owns a contiguous segment that it loads
 //     with 128-bit accesses and scans with DPP row shifts / broadcasts; tiles of
 //     one row are chained with decoupled look-back (aggregate / inclusive-prefix
-//     words published with agent-scope atomics).  No wait is unbounded: when the
-//     output does not overlap the input, a tile that polled a predecessor's
-//     state too long computes that predecessor's aggregate from the input
-//     itself; when it does overlap (in-place scan) tile numbers are drawn from a
-//     per-row atomic ticket, so a tile only waits for tiles that are running.
+//     words published with agent-scope atomics).  Waits when the output does not
+//     overlap the input are bounded by a poll limit: a tile that polled a
+//     predecessor's state too long computes that predecessor's aggregate from
+//     the input itself, and a tile that polled too long for the word that says
+//     a slice of states has been cleared reads and publishes no state of that
+//     slice (its predecessors there are folded from the input, its successors
+//     time out on it the same way).  When the output does overlap the input
+//     (in-place scan) tile numbers are drawn from a per-row atomic ticket, so a
+//     tile only waits for tiles that are running; that wait has no limit.
 //   * scan_cols: many rows, scanned axis strided, a kept axis contiguous (e.g.
 //     cumsum over C of NCHW).  Lanes run along the kept axis so each load is a
 //     contiguous segment, the four waves of a workgroup take consecutive
@@ -147,12 +151,14 @@ __global__ __launch_bounds__(kBlock) void scan_init(unsigned* ticket, int64_t ro
 // workgroup s of the launch clears slice s before anything else and then stores the call's
 // nonce into ready[s].  A state is published, or read, only once its slice's word has been seen
 // to hold the nonce: what the scratch held before the call (anything) cannot pass for a state
-// of this call.  Workgroups are dispatched in index order and workgroup s never waits before it
-// clears, so the slice of tile g (s = g / kSliceTiles <= g) is cleared by a workgroup that
-// started no later than tile g's.  The nonce is a kernel argument: a recorded launch replayed
-// from a graph would meet its own nonce from the replay before, so launches under stream
-// capture clear the states with a launch of their own (ready == nullptr), as do in-place
-// scans, whose tickets need clearing too.
+// of this call.  Workgroup s never waits before it clears and the host takes this path only when
+// the clearing workgroups are fewer than the device holds at once, so they should all be running
+// when any tile asks; nothing in HIP promises the order in which workgroups start, though, so
+// the wait gives up after `limit` polls and the tile then leaves that slice's states alone
+// (scan_tile).  The nonce is a kernel argument: a recorded launch replayed from a graph would
+// meet its own nonce from the replay before, so launches under stream capture clear the states
+// with a launch of their own (ready == nullptr), as do in-place scans, whose tickets need
+// clearing too.
 constexpr int64_t kSliceTiles = 1024;
 struct ClearedBy {
     unsigned long long* ready;
@@ -160,15 +166,22 @@ struct ClearedBy {
     __device__ __forceinline__ bool seen(int64_t slice) const {
         return __hip_atomic_load(&ready[slice], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nonce;
     }
-    // Returns once slice `slice` is cleared; `early` is an earlier load of its word.
-    __device__ __forceinline__ void await(int64_t slice, unsigned long long early) const {
-        if (early != nonce)
-            while (!seen(slice)) __builtin_amdgcn_s_sleep(1);
-        // What follows are agent-scope atomics on the states, which the hardware issues after
-        // this load has returned and which go to the same coherence point: the compiler alone
-        // has to keep them behind it (a cache-invalidating agent-scope fence here costs more
-        // than the separate clearing launch did).
+    // True once slice `slice` is known to be cleared (`early` is an earlier load of its word),
+    // false when `limit` polls did not show it.
+    __device__ __forceinline__ bool await(int64_t slice, unsigned long long early, int limit) const {
+        if (early != nonce) {
+            int polls = 0;
+            while (!seen(slice)) {
+                if (polls++ >= limit) return false;
+                __builtin_amdgcn_s_sleep(1);
+            }
+        }
+        // What follows are agent-scope atomics on the states, which go to the same coherence
+        // point as this load and are issued after it has returned (every later access depends on
+        // the branch above): the compiler alone has to keep them behind it (a cache-invalidating
+        // agent-scope fence here costs more than the separate clearing launch did).
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        return true;
     }
 };
 
@@ -289,29 +302,41 @@ __device__ __forceinline__ void scan_tile(
     if (CHAINED) {
         if (w == 0) {
             const int64_t sbase = row * tiles_per_row;
-            // states from here on are known to be cleared (when this launch clears them itself)
-            int64_t cleared_from = 0;
+            // States [cleared_from, this tile's] are known to be cleared (when this launch clears
+            // them itself); states below dead_below are never read: the word of their slice did
+            // not show the nonce in time, so whatever they hold may be older than this call.
+            int64_t cleared_from = 0, dead_below = 0;
+            bool publishes = true;
             if (cb.ready) {
                 const int64_t slice = (sbase + t) / kSliceTiles;
-                cb.await(slice, ready_early);
-                cleared_from = slice * kSliceTiles;
+                if (cb.await(slice, ready_early, poll_limit)) {
+                    cleared_from = slice * kSliceTiles;
+                } else {
+                    // not even this tile's own slice: nothing is published (the slice's clearing
+                    // would wipe it or, worse, come first and leave it) and every predecessor
+                    // is folded from the input
+                    publishes = false;
+                    cleared_from = dead_below = sbase + t;
+                }
             }
-            if (lane == 0) st.publish(sbase + t, t == 0 ? kInclusive : kAggregate, aggregate);
+            if (lane == 0 && publishes) st.publish(sbase + t, t == 0 ? kInclusive : kAggregate, aggregate);
             T excl = Op::identity();
             if (t > 0) {
                 int64_t pos = t - 1;
                 for (;;) {
                     // the states this step of the look-back reads reach back to pos - 63 or to the row's first
                     const int64_t lowest = sbase + (pos >= kWave - 1 ? pos - (kWave - 1) : 0);
-                    while (lowest < cleared_from) {
+                    while (lowest < cleared_from && cleared_from > dead_below) {
                         const int64_t slice = (cleared_from - 1) / kSliceTiles;
-                        cb.await(slice, 0ull);
-                        cleared_from = slice * kSliceTiles;
+                        if (cb.await(slice, 0ull, poll_limit)) cleared_from = slice * kSliceTiles;
+                        else dead_below = cleared_from;
                     }
                     const int64_t idx = pos - lane;
                     T v = Op::identity();
                     uint32_t f = kInclusive;          // before the row: an inclusive identity
-                    if (idx >= 0) {
+                    if (idx >= 0 && sbase + idx < dead_below) {
+                        f = kInvalid;                  // (only with SELF_HELP: this launch clears its states only then)
+                    } else if (idx >= 0) {
                         f = st.read(sbase + idx, &v);
                         if constexpr (SELF_HELP) {
                             for (int polls = 0; f == kInvalid && polls < poll_limit; ++polls) {
@@ -352,7 +377,7 @@ __device__ __forceinline__ void scan_tile(
                     if (incl_mask != 0ull) break;
                     pos -= kWave;
                 }
-                if (lane == 0) st.publish(sbase + t, kInclusive, Op::apply(excl, aggregate));
+                if (lane == 0 && publishes) st.publish(sbase + t, kInclusive, Op::apply(excl, aggregate));
             }
             if (lane == 0) sm.tile_prefix = excl;
         }
@@ -844,11 +869,24 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     TileState<T> st;
     st.bind(static_cast<char*>(scratch) + l.state_off, l.tiles);
     const bool in_place = views_overlap(rank, dims, x, x_strides, y, y_strides);
+    constexpr int CI = static_cast<int>(kChainTileBytes / sizeof(T) / kChainBlock);
+    const bool padded = !NZ && pad != 0;
     // The scan launch clears the tile states itself, except where that cannot work: under stream
-    // capture (a replayed launch would carry the nonce of the replay before it) and in place
-    // (the rows' tickets need clearing before any workgroup runs).
+    // capture (a replayed launch would carry the nonce of the replay before it), in place (the
+    // rows' tickets need clearing before any workgroup runs), and when there are more slices to
+    // clear than the device holds workgroups at once (the clearing workgroups, the first of the
+    // launch, should all be running when a tile asks for their word; 256 run on any gfx950).
     ClearedBy cb{nullptr, 0ull};
-    if (!in_place && !stream_is_capturing(stream)) {
+    bool clears_itself = !in_place && !stream_is_capturing(stream);
+    if (clears_itself && ceil_div(l.tiles, kSliceTiles) > 256) {
+        int64_t room = 0;
+        if constexpr (!NZ) {
+            if (padded) room = resident_workgroups(scan_rows_chained<T, K, CI, false, kChainBlock, X, NZ, Y, true>, kChainBlock);
+        }
+        if (!padded) room = resident_workgroups(scan_rows_chained<T, K, CI, false, kChainBlock, X, NZ, Y, false>, kChainBlock);
+        clears_itself = ceil_div(l.tiles, kSliceTiles) <= room;
+    }
+    if (clears_itself) {
         cb.ready = reinterpret_cast<unsigned long long*>(static_cast<char*>(scratch) + l.ready_off);
         cb.nonce = next_nonce();
     } else {
@@ -856,7 +894,6 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
         DLFX_CHECK_LAUNCH();
     }
     const dim3 grid(static_cast<unsigned>(l.tiles));
-    constexpr int CI = static_cast<int>(kChainTileBytes / sizeof(T) / kChainBlock);
     const dim3 cblock(kChainBlock);
     // rows off a vector boundary have kernels of their own: the aligned ones carry none of that arithmetic
     auto chained = [&](auto ticketed, auto padded) {

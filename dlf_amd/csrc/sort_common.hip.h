@@ -86,16 +86,6 @@ __device__ __forceinline__ uint32_t make_status(int tag, bool inclusive, uint32_
 
 constexpr int kRadix = 256;
 
-// Workgroups of `kernel` that the current device holds at once (0 when HIP cannot tell).
-template <typename Kernel>
-int64_t resident_workgroups(Kernel kernel, int block) {
-    int device = 0, units = 0, per_unit = 0;
-    if (hipGetDevice(&device) != hipSuccess) return 0;
-    if (hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_unit, kernel, block, 0) != hipSuccess) return 0;
-    return static_cast<int64_t>(units) * per_unit;
-}
-
 // ------------------------------------------------------------------ the bucket route (sort_split.hip)
 // The tables of the digit passes that must start at zero for a row those passes sort; the
 // bucket route clears them for every row it leaves.

@@ -199,6 +199,8 @@ class HipBackend:
     def copy_view(self, storage, shape):
         """Row-major device copy of a strided view (dlfx_copy: the reference's reorder(X, Y))."""
         out = self.torch.empty(max(1, shape.size), dtype=storage.dtype, device=self.device)
+        if shape.size == 0:              # an empty slice: nothing to move
+            return out
         dense = []
         size = 1
         for e in reversed(shape.extents):

@@ -385,13 +385,17 @@ inline void cumsum(const DevTensor<T>& X, DevTensor<T>& Y, int axis = -1, bool e
 // row-major order in Y, copied on the device (gpgpu::dnn::copy).
 template <typename T>
 void reorder(const DevTensor<T>& X, DevTensor<T>& Y) {
+    // Y may be X itself or another tensor over X's buffer (a view): the copy kernels do not take
+    // overlapping views, so the elements then go through a tensor of their own
+    const bool shared = &X == &Y || (!X.empty() && !Y.empty() && X.data().data() == Y.data().data());
     if (&X == &Y && X.shape().is_contiguous()) return;
     DevTensor<T> out;
-    DevTensor<T>& dst = (&X == &Y) ? out : Y;
+    DevTensor<T>& dst = shared ? out : Y;
     dst.resize(X.shape());
-    gpgpu::dnn::copy(X.size(), X.shape().extents(), X.data(), X.shape().offset(), X.shape().strides(),
-                     dst.data(), dst.shape().offset(), dst.shape().strides());
-    if (&X == &Y) Y = std::move(out);
+    if (X.size() != 0)
+        gpgpu::dnn::copy(X.size(), X.shape().extents(), X.data(), X.shape().offset(), X.shape().strides(),
+                         dst.data(), dst.shape().offset(), dst.shape().strides());
+    if (shared) Y = std::move(out);
 }
 
 // ---------------------------------------------------------------- sort / argsort / top_k

@@ -264,8 +264,9 @@ void copy(const size_t n, const std::vector<size_t>& dims,
     if (size != n || x_stride.size() != dims.size() || y_stride.size() != dims.size())
         throw LogicError("gpgpu::dnn::copy: extents, strides and n disagree");
     detail::EventScope ev(queue, event);
-    check_status(dlfx_copy(queue.stream(), detail::dtype_of<T>::value, static_cast<int>(d.size()), d.data(),
-                           x_buffer.data(), x_offset, xs.data(), y_buffer.data(), y_offset, ys.data()), "gpgpu::dnn::copy");
+    if (n != 0)            // an empty view: nothing to move
+        check_status(dlfx_copy(queue.stream(), detail::dtype_of<T>::value, static_cast<int>(d.size()), d.data(),
+                               x_buffer.data(), x_offset, xs.data(), y_buffer.data(), y_offset, ys.data()), "gpgpu::dnn::copy");
     ev.done();
 }
 
@@ -302,8 +303,9 @@ void fill(const size_t n, Buffer<T>& x_buffer, const size_t x_offset, const T va
           const Queue& queue = gpgpu::current::queue(), Event* event = nullptr) {
     const int64_t d[1] = {static_cast<int64_t>(n)}, one[1] = {1};
     detail::EventScope ev(queue, event);
-    check_status(dlfx_fill(queue.stream(), detail::dtype_of<T>::value, 1, d, one, x_buffer.data(), x_offset, &value),
-                 "gpgpu::dnn::fill");
+    if (n != 0)
+        check_status(dlfx_fill(queue.stream(), detail::dtype_of<T>::value, 1, d, one, x_buffer.data(), x_offset, &value),
+                     "gpgpu::dnn::fill");
     ev.done();
 }
 
@@ -317,8 +319,9 @@ void fill(const size_t n, const std::vector<size_t>& dims, const std::vector<siz
     for (auto e : dims) size *= e;
     if (size != n || strides.size() != dims.size()) throw LogicError("gpgpu::dnn::fill: extents, strides and n disagree");
     detail::EventScope ev(queue, event);
-    check_status(dlfx_fill(queue.stream(), detail::dtype_of<T>::value, static_cast<int>(d.size()), d.data(), st.data(),
-                           x_buffer.data(), x_offset, &value), "gpgpu::dnn::fill");
+    if (n != 0)
+        check_status(dlfx_fill(queue.stream(), detail::dtype_of<T>::value, static_cast<int>(d.size()), d.data(), st.data(),
+                               x_buffer.data(), x_offset, &value), "gpgpu::dnn::fill");
     ev.done();
 }
 

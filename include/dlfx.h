@@ -63,7 +63,8 @@ typedef enum dlfx_status {
     DLFX_ERR_SCRATCH_TOO_SMALL = -4,
     DLFX_ERR_RANK = -5,              /* view rank above DLFX_MAX_RANK */
     DLFX_ERR_LAUNCH = -6,            /* HIP reported an error; see dlfx_last_hip_error */
-    DLFX_ERR_TOO_LARGE = -7          /* an extent exceeds what the kernels index */
+    DLFX_ERR_TOO_LARGE = -7,         /* an extent exceeds what the kernels index */
+    DLFX_ERR_CAPTURING = -8          /* a first call on a device that may not be recorded into a graph */
 } dlfx_status;
 
 /* Library version: major*10000 + minor*100 + patch. */
@@ -126,7 +127,10 @@ int dlfx_reduce(dlfx_stream_t stream, const char* name, int dtype, int64_t m, in
  * nothing.  The array covers every shape dlfx_reduce accepts (its scratch query never asks for
  * more); a shape whose partials would not fit is refused with DLFX_ERR_TOO_LARGE and nothing
  * is enqueued.  The first call on a device looks the array's address up (the device that is
- * current must be the one the stream belongs to).  All calls on one GPU share that GPU's
+ * current must be the one the stream belongs to), which may load the library's device code:
+ * that call must come before any stream capture -- while `stream` is being captured it is
+ * refused with DLFX_ERR_CAPTURING and nothing is enqueued; later calls on the device record
+ * like any other launch.  All calls on one GPU share that GPU's
  * array: calls that overlap in time on one GPU -- different streams, or different host threads
  * -- race on it and must be serialised by the caller.
  */

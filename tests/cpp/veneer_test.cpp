@@ -13,6 +13,7 @@
 #include <cmath>
 #include <complex>
 #include <cstdio>
+#include <future>
 #include <random>
 
 #include "dev_tensor.h"
@@ -602,6 +603,61 @@ static void test_onnx_nodes() {
     CHECK(threw);
 }
 
+// Two host threads, each on the queue and context its first use creates for it
+// (dlf/test/GPGPUTest.cpp:716-733; gpgpu/src/gpgpu.cpp:139-185): a long-row reduction, a chained
+// scan and an argsort of long rows per thread, all three with scratch from the thread's own
+// arena, running at the same time; results equal the single-thread ones.
+struct ThreadResult {
+    Tensor<int32_t> sums, scan, order;
+    bool own_queue = false;
+    size_t left_in_use = 1;
+};
+static ThreadResult thread_work(const std::vector<int32_t>& xs, size_t m, size_t n, const gpgpu::Queue* main_queue) {
+    ThreadResult r;
+    const gpgpu::Queue& mine = gpgpu::current::queue();
+    r.own_queue = main_queue == nullptr || (mine != *main_queue && mine.context() != main_queue->context());
+    auto X = dev(Tensor<int32_t>({m, n}, xs));
+    for (int round = 0; round < 3; ++round) {            // several rounds so that the threads' launches interleave
+        r.sums = reduce_sum(X, {1}).read();
+        r.scan = cumsum(X, 1).read();
+        r.order = argsort(X, 1).read();
+    }
+    mine.finish();
+    r.left_in_use = mine.context().temporary_bytes_in_use();
+    return r;
+}
+static void test_two_threads() {
+    const size_t m = 4, n = 300000;
+    std::vector<int32_t> a(m * n), b(m * n);
+    std::mt19937 rng(23);
+    for (auto& v : a) v = static_cast<int32_t>(rng() % 1000);
+    for (auto& v : b) v = static_cast<int32_t>(rng() % 50) - 25;
+    const gpgpu::Queue& main_queue = gpgpu::current::queue();
+    const ThreadResult alone_a = thread_work(a, m, n, nullptr), alone_b = thread_work(b, m, n, nullptr);
+    auto fa = std::async(std::launch::async, thread_work, std::cref(a), m, n, &main_queue);
+    auto fb = std::async(std::launch::async, thread_work, std::cref(b), m, n, &main_queue);
+    const ThreadResult ta = fa.get(), tb = fb.get();
+    CHECK(ta.own_queue && tb.own_queue);
+    CHECK(ta.left_in_use == 0 && tb.left_in_use == 0);
+    CHECK(ta.sums == alone_a.sums && ta.scan == alone_a.scan && ta.order == alone_a.order);
+    CHECK(tb.sums == alone_b.sums && tb.scan == alone_b.scan && tb.order == alone_b.order);
+    // ... and the single-thread results are right: serial host scan, stable order
+    bool ok = true;
+    for (size_t r = 0; r < m; ++r) {
+        int32_t acc = 0;
+        for (size_t j = 0; j < n; ++j) {
+            acc += a[r * n + j];
+            ok = ok && alone_a.scan.values()[r * n + j] == acc;
+        }
+        ok = ok && alone_a.sums.values()[r] == acc;
+        for (size_t j = 1; j < n; ++j) {
+            const int32_t p = alone_a.order.values()[r * n + j - 1], q = alone_a.order.values()[r * n + j];
+            ok = ok && (a[r * n + p] < a[r * n + q] || (a[r * n + p] == a[r * n + q] && p < q));
+        }
+    }
+    CHECK(ok);
+}
+
 int main() {
     test_reduce();
     test_arg_reduce();
@@ -619,6 +675,7 @@ int main() {
     test_layout_steps_stay_on_the_device();
     test_onnx_nodes();
     test_logits_head();
+    test_two_threads();
     std::printf("veneer_test: %d checks, %d failed\n", g_checked, g_failed);
     return g_failed ? 1 : 0;
 }

@@ -51,3 +51,42 @@ def test_capture_and_replay_matches_eager(hip_backend):
         assert np.array_equal(got[6], np.cumsum(lr, axis=1, dtype=np.int32))
         assert np.array_equal(got[7], np.sort(lr, axis=1))
         assert np.array_equal(got[13], (zr == 0).sum(axis=1))
+
+
+def test_reduce_static_records_and_replays(hip_backend):
+    # dlfx_reduce_static is meant for callers under capture: once its first call on the device
+    # has been made (outside any capture), recorded calls replay like any other launch and
+    # allocate nothing (the caching allocator's count of allocations does not move across the
+    # recording; a first recording that holds one fill kernel takes what torch itself sets up
+    # once per process).
+    import torch
+    from dlf_amd.frontend import prepare_reduce
+    x0 = normal(173, 3 * (1 << 20)).astype(np.float32).reshape(3, 1 << 20)
+    X = Tensor.from_numpy(hip_backend, x0)
+    view, out_dims, m, n = prepare_reduce(X.shape, [1], False)
+    code = F.dtype_code(X.dtype)
+    Y = Tensor.empty(hip_backend, out_dims, X.dtype)
+    Ye = Tensor.empty(hip_backend, out_dims, X.dtype)
+    hip_backend.reduce_static("reduce_sum", code, m, n, view, X.storage, Y.shape, Y.storage)     # the first call: eager
+    torch.cuda.synchronize()
+    def allocations():
+        return torch.cuda.memory_stats(hip_backend.device)["allocation.all.allocated"]
+    first = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(first):
+        Ye.storage.zero_()
+    before = allocations()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        hip_backend.reduce_static("reduce_sum", code, m, n, view, X.storage, Y.shape, Y.storage)
+        hip_backend.reduce_static("reduce_max", code, m, n, view, X.storage, Ye.shape, Ye.storage)
+    assert allocations() == before
+    for r in range(3):
+        xr = np.roll(x0, 5 * r + 1, axis=1) * (r + 2)
+        X.storage.copy_(torch.from_numpy(np.ascontiguousarray(xr).reshape(-1)))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got_sum, got_max = Y.numpy().copy(), Ye.numpy().copy()
+        want = F.reduce("reduce_sum", X, (1,)).numpy()                  # dlfx_reduce, eagerly, same input
+        assert np.array_equal(got_sum, want), r
+        assert np.array_equal(got_max, xr.max(axis=1)), r

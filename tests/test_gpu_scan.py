@@ -132,6 +132,61 @@ def test_tile_states_cleared_slice_by_slice(hip_backend):
     assert np.array_equal(F.cummax(Yh, 1).numpy(), np.maximum.accumulate(y, axis=1))
 
 
+def test_two_streams_with_stale_scratch(hip_backend):
+    # Two chained scans at once on two streams, each with scratch of its own that is not clean:
+    # all ones before the first round, afterwards whatever the round before left (the states and
+    # slice words of an earlier call).  Every launch clears its own states while the other
+    # stream's launch competes for the compute units, so workgroups need not start in index order.
+    torch = hip_backend.torch
+    lib = hip_backend.lib
+    from dlf_amd.hip_backend import _arr, _check
+    m, n = 64, 1 << 20
+    a = randint(56, m * n, 0, 100).astype(np.int32).reshape(m, n)
+    want = [np.cumsum(a, axis=1, dtype=np.int32), np.cumsum(a[::-1], axis=1, dtype=np.int32)]
+    xs = [torch.from_numpy(a).to(hip_backend.device), torch.from_numpy(a[::-1].copy()).to(hip_backend.device)]
+    ys = [torch.empty_like(x) for x in xs]
+    nbytes = lib.dlfx_scan_scratch_bytes(2, m, n)
+    scratch = [torch.full((nbytes,), 0xFF, dtype=torch.uint8, device=hip_backend.device) for _ in range(2)]
+    streams = [torch.cuda.Stream(device=hip_backend.device) for _ in range(2)]
+    torch.cuda.synchronize(hip_backend.device)
+    dims, strides = _arr([m, n]), _arr([n, 1])
+    for it in range(24):
+        for k in range(2):
+            ys[k].zero_()
+        torch.cuda.synchronize(hip_backend.device)
+        for k in range(2):
+            _check(lib.dlfx_scan(streams[k].cuda_stream, b"cumsum", 2, m, n, 0, 2, dims, xs[k].data_ptr(), 0, strides,
+                                 ys[k].data_ptr(), 0, strides, scratch[k].data_ptr(), nbytes), "dlfx_scan")
+        torch.cuda.synchronize(hip_backend.device)
+        for k in range(2):
+            assert np.array_equal(ys[k].cpu().numpy(), want[k]), (it, k)
+
+
+def test_clearing_not_seen_in_time_folds_the_input(hip_backend):
+    # With a poll limit of 0 a tile that has not seen its slice's word at its first look gives up
+    # at once: it publishes nothing and folds every predecessor from the input; tiles behind it
+    # time out on it the same way.  Dirty scratch, so that a state read by mistake would show.
+    torch = hip_backend.torch
+    lib = hip_backend.lib
+    from dlf_amd.hip_backend import _arr, _check
+    m, n = 6, 40 * 32768 + 77
+    a = randint(57, m * n, -100, 100).astype(np.int32).reshape(m, n)
+    x = torch.from_numpy(a).to(hip_backend.device)
+    y = torch.empty_like(x)
+    nbytes = lib.dlfx_scan_scratch_bytes(2, m, n)
+    scratch = torch.full((nbytes,), 0xFF, dtype=torch.uint8, device=hip_backend.device)
+    stream = torch.cuda.current_stream(hip_backend.device).cuda_stream
+    hip_backend.set_tuning("scan_poll_limit", 0)
+    try:
+        for _ in range(3):
+            _check(lib.dlfx_scan(stream, b"cumsum", 2, m, n, 0, 2, _arr([m, n]), x.data_ptr(), 0, _arr([n, 1]),
+                                 y.data_ptr(), 0, _arr([n, 1]), scratch.data_ptr(), nbytes), "dlfx_scan")
+            torch.cuda.synchronize(hip_backend.device)
+            assert np.array_equal(y.cpu().numpy(), np.cumsum(a, axis=1, dtype=np.int32))
+    finally:
+        hip_backend.set_tuning("scan_poll_limit", 2048)
+
+
 def test_bounded_wait_self_help_path(hip_backend, oracle_backend):
     # With a poll limit of 0 a tile never waits: whatever predecessor has not
     # published yet is folded from the input by the waiting tile itself.
