@@ -2,10 +2,9 @@
 //
 // Which way a row goes: rows of up to 64 / 512 elements are sorted by one wavefront in
 // registers, rows of up to 4096 (16-bit keys), 8192 (8-byte) or 16384 (4-byte keys) by one workgroup
-// on chip, longer rows of 4- and 8-byte keys by
-// the bucket route of sort_split.hip (run_split below enqueues it first; every row decides on
-// the device whether it can take it).  What is left - rows the bucket route cannot take,
-// 16-bit keys - is sorted here:
+// on chip, longer rows of 4- and 8-byte keys by the bucket route of sort_split.hip (run_split),
+// which sorts every row of such a call.  What is left - 16-bit keys, rows longer than 256 of the
+// largest buckets hold (about 2.6 million keys) - is sorted here:
 //
 // Segmented least-significant-digit radix sort, 8 bits per pass, every row an
 // independent segment:
@@ -59,17 +58,6 @@ __device__ unsigned long long g_phase_cycles[kPhaseSlots * 8];
 #define DLFX_PHASE_BEGIN() do { } while (0)
 #endif
 
-// Which rows of a call the digit passes take: the bucket route (sort_split.hip) marks the rows
-// it sorts with a first word of 1 in its per-row records and counts the others; with no
-// records every row is taken here.
-struct RowRoutes {
-    const uint32_t* records;      // null: every row
-    size_t stride_words;
-    const uint32_t* other_rows;   // how many rows the bucket route left
-    __device__ __forceinline__ bool none_here() const { return records && *other_rows == 0u; }
-    __device__ __forceinline__ bool elsewhere(int64_t row) const { return records && records[row * stride_words] == 1u; }
-};
-
 // ------------------------------------------------------------------ bases
 // In place: one histogram of a row -> exclusive prefix (start of each digit's run in the row),
 // by the 256 threads of a workgroup.  *moves receives the bits of the digit that are not the
@@ -113,7 +101,7 @@ __device__ __forceinline__ void bases_of_pass(uint32_t* __restrict__ g, uint32_t
 // keys (constant bytes: small integers, narrow float ranges) is added once per wave.
 template <typename K>
 __global__ __launch_bounds__(kBlock) void sort_histogram(PassIo<K> io, int64_t n, int64_t chunk, int64_t chunks_per_row, int64_t units,
-                                                         RowRoutes routes, uint32_t* __restrict__ ghist, uint32_t* __restrict__ arrived,
+                                                         uint32_t* __restrict__ ghist, uint32_t* __restrict__ arrived,
                                                          uint32_t* __restrict__ moves, int all_bits) {
     constexpr int P = KeyTraits<K>::kPasses;
     static_assert(kBlock == kRadix, "a thread per digit when the row's histograms are scanned");
@@ -121,10 +109,8 @@ __global__ __launch_bounds__(kBlock) void sort_histogram(PassIo<K> io, int64_t n
     constexpr int U = 32 / sizeof(K);                 // keys in flight per thread
     constexpr int R = 32 / P;                         // copies: 8 (32-bit keys) or 4 (64-bit keys): 32 KB
     __shared__ uint32_t hist[P * kRadix * R];
-    if (routes.none_here()) return;
     for (int64_t unit = blockIdx.x; unit < units; unit += gridDim.x) {       // (row, chunk) pairs
     const int64_t row = unit / chunks_per_row;
-    if (routes.elsewhere(row)) continue;
     __syncthreads();                                   // the previous unit's histogram has left
     for (int i = threadIdx.x; i < P * kRadix * R; i += kBlock) hist[i] = 0;
     __syncthreads();
@@ -220,25 +206,20 @@ template <typename K, bool PAIRS, int ITEMS, bool LAST>
 __global__ __launch_bounds__(kPassBlock) __attribute__((amdgpu_waves_per_eu(DLFX_SORT_WAVES))) void sort_pass(PassIo<K> io, int pass, int64_t rows, int64_t n, int64_t tiles_per_row,
                                                     const uint32_t* __restrict__ gbase,
                                                     const uint32_t* __restrict__ moves,
-                                                    RowRoutes routes,
                                                     uint32_t* __restrict__ status, int poll_limit) {
     constexpr int P = KeyTraits<K>::kPasses;
     constexpr int TILE = kPassBlock * ITEMS;
     constexpr int W = 4;    // status words of earlier tiles fetched per look-back step
     __shared__ PassShared<K, PAIRS, ITEMS> sm;
 
-    if (routes.none_here()) return;
     // workgroups are handed out in index order and dealt round-robin over the chip's eight
     // parts: tile t of every row comes before tile t + 1 of any row, so a tile's predecessors
     // in its row have usually finished when it looks back, and the tiles of a row share a
-    // second-level cache when the number of rows is a multiple of eight.  With fewer workgroups
-    // than tiles (a launch sized to what the device holds at once) workgroup g takes tiles
-    // g, g + G, ... in that numbering.
+    // second-level cache when the number of rows is a multiple of eight.
     for (int64_t unit = blockIdx.x; unit < rows * tiles_per_row; unit += gridDim.x) {
     if (unit != static_cast<int64_t>(blockIdx.x)) __syncthreads();      // the previous tile has left LDS
     const int64_t t = unit / rows;
     const int64_t row = unit - t * rows;
-    if (routes.elsewhere(row)) continue;
     const uint32_t* row_moves = moves + row * P;
     const int tag = pass;
     int ran = 0;            // passes before this one that this row ran
@@ -844,35 +825,58 @@ struct SortLayout {
     size_t moves_off, arrived_off, hist_off, hist_bytes, status_off, status_bytes, split_off, split_bytes, keys_off[2], vals_off[2], total;
 };
 
+// Rows longer than one workgroup sorts on chip take the bucket route when their shape allows
+// it (and dlfx_set_tuning has not switched it off): it sorts every row of the call, needs one
+// pair of ping-pong buffers and its own tables, and none of the digit passes' tables.
+bool takes_bucket_route(size_t key_size, int64_t m, int64_t n) {
+    return key_size >= 4 && g_sort_buckets != 0 && n > small_row(key_size) && split_route_takes(key_size, m, n);
+}
+
 SortLayout sort_layout(size_t key_size, bool pairs, int64_t m, int64_t n) {
     SortLayout l;
     const int passes = static_cast<int>(key_size);          // one per key byte
     const int64_t tile = kPassBlock * tile_items(key_size, pairs);
+    const bool buckets = takes_bucket_route(key_size, m, n);
     l.tiles_per_row = ceil_div(n, tile);
     size_t off = 0;
     l.moves_off = off;           // one word per (row, pass): does the pass move the row's keys
-    off += align_up(static_cast<size_t>(m) * passes * 4, 256);
+    if (!buckets) off += align_up(static_cast<size_t>(m) * passes * 4, 256);
     l.arrived_off = off;         // chunks of each row counted so far; cleared with the histograms and the status words after it
-    off += align_up(static_cast<size_t>(m) * 4, 256);
+    if (!buckets) off += align_up(static_cast<size_t>(m) * 4, 256);
     l.hist_off = off;
-    l.hist_bytes = static_cast<size_t>(m) * passes * kRadix * 4;
+    l.hist_bytes = buckets ? 0 : static_cast<size_t>(m) * passes * kRadix * 4;
     off += align_up(l.hist_bytes, 256);
     l.status_off = off;
-    l.status_bytes = l.tiles_per_row > 1 ? static_cast<size_t>(m) * l.tiles_per_row * kRadix * 4 : 0;
+    l.status_bytes = (!buckets && l.tiles_per_row > 1) ? static_cast<size_t>(m) * l.tiles_per_row * kRadix * 4 : 0;
     off += align_up(l.status_bytes, 256);
-    l.split_off = off;           // tables of the bucket route (rows longer than one workgroup sorts on chip)
-    l.split_bytes = (n > small_row(key_size) && split_route_takes(key_size, m, n)) ? split_scratch_bytes(key_size, pairs, m, n) : 0;
+    l.split_off = off;           // tables of the bucket route
+    l.split_bytes = buckets ? split_scratch_bytes(key_size, pairs, m, n) : 0;
     off += align_up(l.split_bytes, 256);
     for (int i = 0; i < 2; ++i) {
         l.keys_off[i] = off;
-        off += align_up(static_cast<size_t>(m) * n * key_size, 256);
+        if (i == 0 || !buckets) off += align_up(static_cast<size_t>(m) * n * key_size, 256);
     }
     for (int i = 0; i < 2; ++i) {
         l.vals_off[i] = off;
-        if (pairs) off += align_up(static_cast<size_t>(m) * n * 4, 256);
+        if (pairs && (i == 0 || !buckets)) off += align_up(static_cast<size_t>(m) * n * 4, 256);
     }
     l.total = off;
     return l;
+}
+
+// True when the bytes the two views touch intersect (views of different element types).
+bool bytes_overlap(int rank, const int64_t* dims, const void* x, const int64_t* sx, size_t ex, const void* y, const int64_t* sy, size_t ey) {
+    int64_t xlo = 0, xhi = 0, ylo = 0, yhi = 0;
+    for (int i = 0; i < rank; ++i) {
+        const int64_t dx = (dims[i] - 1) * sx[i], dy = (dims[i] - 1) * sy[i];
+        if (dx > 0) xhi += dx; else xlo += dx;
+        if (dy > 0) yhi += dy; else ylo += dy;
+    }
+    const char* xb = static_cast<const char*>(x) + xlo * static_cast<int64_t>(ex);
+    const char* xe = static_cast<const char*>(x) + (xhi + 1) * static_cast<int64_t>(ex);
+    const char* yb = static_cast<const char*>(y) + ylo * static_cast<int64_t>(ey);
+    const char* ye = static_cast<const char*>(y) + (yhi + 1) * static_cast<int64_t>(ey);
+    return xb < ye && yb < xe;
 }
 
 template <typename T>
@@ -931,6 +935,8 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     const bool y_over_x = a.y && ranges_overlap<K>(a.rank, a.dims, static_cast<const K*>(a.x), a.xs, static_cast<const K*>(a.y), a.ys);
     io.canon_zero = (a.pairs && a.kind == kKeyFloat && !y_over_x) ? 1 : 0;
     io.restore_zero = (io.canon_zero && a.y) ? 1 : 0;
+    const bool i_over_x = a.idx && bytes_overlap(a.rank, a.dims, a.x, a.xs, sizeof(K), a.idx, a.is, a.idx64 ? 8 : 4);
+    io.x_intact = (!y_over_x && !i_over_x) ? 1 : 0;
 
     // short rows: one workgroup sorts a row on chip.  A workgroup reads its whole row before it
     // writes, so sorting in place is fine; an output that overlaps the input in any other way
@@ -948,33 +954,17 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     io.vbuf[0] = a.pairs ? reinterpret_cast<uint32_t*>(base + l.vals_off[0]) : nullptr;
     io.vbuf[1] = a.pairs ? reinterpret_cast<uint32_t*>(base + l.vals_off[1]) : nullptr;
 
+    // The bucket route sorts every row of the call (rows that do not cut into buckets a workgroup
+    // holds are finished by one workgroup per oversized bucket, decided on the device).
+    if constexpr (sizeof(K) >= 4) {
+        if (l.split_bytes != 0) return run_split<K>(stream, io, a.pairs, m, n, base + l.split_off, g_sort_compare_max);
+    }
+
     uint32_t* moves = reinterpret_cast<uint32_t*>(base + l.moves_off);
     uint32_t* arrived = reinterpret_cast<uint32_t*>(base + l.arrived_off);
     uint32_t* ghist = reinterpret_cast<uint32_t*>(base + l.hist_off);
     uint32_t* status = reinterpret_cast<uint32_t*>(base + l.status_off);
-    // The bucket route first: every row it can take goes that way (decided on the device, row by
-    // row); the digit passes below take the others and leave at once when there are none.  The
-    // routes share the first ping-pong buffer: their rows are different rows.
-    RowRoutes routes = {nullptr, 0, nullptr};
-    if constexpr (sizeof(K) >= 4) {
-        if (l.split_bytes != 0 && g_sort_buckets) {
-            // (the route clears the tables of the rows it leaves)
-            const LeftTables tables = {arrived, ghist, static_cast<uint32_t>(P * kRadix), status,
-                                       l.status_bytes ? l.tiles_per_row * kRadix : 0};
-            size_t stride = 0;
-            const int st = run_split<K>(stream, io, a.pairs, m, n, base + l.split_off, g_sort_poll_limit, g_sort_compare_max, tables,
-                                        &routes.other_rows, &routes.records, &stride);
-            if (st != DLFX_OK) return st;
-            routes.stride_words = stride / 4;
-        }
-    }
-
-    // When the bucket route runs, these launches only take the rows it left - usually none - so
-    // they are sized to what the device holds at once and walk their work; an idle launch then
-    // costs a few microseconds however long the rows are.
-    const bool bounded = routes.records != nullptr;
-    auto sized = [&](int64_t units, int64_t room) { return dim3(static_cast<unsigned>(bounded && room > 0 && room < units ? room : units)); };
-    if (!bounded) {
+    {
         const int64_t clear_words = static_cast<int64_t>((l.status_off + l.status_bytes - l.arrived_off) / 4);   // counts, histograms, status
         sort_clear<<<dim3(static_cast<unsigned>(ceil_div(clear_words, kBlock * 4))), dim3(kBlock), 0, stream>>>(arrived, clear_words);
         DLFX_CHECK_LAUNCH();
@@ -985,26 +975,22 @@ int run_sort(hipStream_t stream, const SortArgs& a, void* scratch, size_t scratc
     if (m * chunks_per_row > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
     // a pass that moves nothing may only be left out when no pass reads the input while
     // another tile of the same pass writes the output over it
-    sort_histogram<K><<<sized(m * chunks_per_row, 1024), dim3(kBlock), 0, stream>>>(io, n, chunk, chunks_per_row, m * chunks_per_row, routes, ghist,
+    sort_histogram<K><<<dim3(static_cast<unsigned>(m * chunks_per_row)), dim3(kBlock), 0, stream>>>(io, n, chunk, chunks_per_row, m * chunks_per_row, ghist,
                                                                                     arrived, moves, y_over_x ? 1 : 0);
     DLFX_CHECK_LAUNCH();
 
-    // (a tile waits for tiles of workgroups that run beside it: no more workgroups than fit at once)
-    const int64_t room = !bounded ? 0
-                         : a.pairs ? resident_workgroups(sort_pass<K, true, IP, false>, kPassBlock)
-                                   : resident_workgroups(sort_pass<K, false, IK, false>, kPassBlock);
-    const dim3 grid = sized(m * l.tiles_per_row, room);
+    const dim3 grid(static_cast<unsigned>(m * l.tiles_per_row));
     for (int p = 0; p < P; ++p) {
         if (p < P - 1) {
             if (a.pairs)
-                sort_pass<K, true, IP, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, routes, status, g_sort_poll_limit);
+                sort_pass<K, true, IP, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
             else
-                sort_pass<K, false, IK, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, routes, status, g_sort_poll_limit);
+                sort_pass<K, false, IK, false><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
         } else {
             if (a.pairs)
-                sort_pass<K, true, IP, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, routes, status, g_sort_poll_limit);
+                sort_pass<K, true, IP, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
             else
-                sort_pass<K, false, IK, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, routes, status, g_sort_poll_limit);
+                sort_pass<K, false, IK, true><<<grid, dim3(kPassBlock), 0, stream>>>(io, p, m, n, l.tiles_per_row, ghist, moves, status, g_sort_poll_limit);
         }
         DLFX_CHECK_LAUNCH();
     }

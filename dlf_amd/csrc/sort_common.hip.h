@@ -58,6 +58,7 @@ struct PassIo {
     int kind, descending;
     int canon_zero;           // argsort of floats: -0.0 and +0.0 are one key
     int restore_zero;         // ... and the value written for a zero key is re-read from x
+    int x_intact;             // no output overlaps the input: x can still be read once outputs are being written
     // rows side by side in memory (the axis is an outer dimension): workgroups are dealt to the
     // 8 XCDs in turn, so workgroup b takes block (b % 8) * xcd_blocks + b / 8 and neighbouring
     // rows, which share cache lines, meet in one L2 (0: workgroup b takes block b)
@@ -87,24 +88,40 @@ __device__ __forceinline__ uint32_t make_status(int tag, bool inclusive, uint32_
 constexpr int kRadix = 256;
 
 // ------------------------------------------------------------------ the bucket route (sort_split.hip)
-// The tables of the digit passes that must start at zero for a row those passes sort; the
-// bucket route clears them for every row it leaves.
-struct LeftTables {
-    uint32_t* arrived;                   // one word a row
-    uint32_t* hist;                      // hist_words a row
-    uint32_t hist_words;
-    uint32_t* status;                    // status_words a row (none for rows of one tile)
-    int64_t status_words;
-};
-
-// Whether rows of n keys may take it at all, the scratch it needs, and its launch: rows it does
-// not take are counted in **other_rows (device memory) and marked by a first word other than 1
-// in the per-row records at *route_records (*route_stride bytes apart).
+// Whether rows of n keys may take it, the scratch it needs beside the caller's first pair of
+// ping-pong buffers, and its launches: every row of the call is sorted by it.
 bool split_route_takes(size_t key_size, int64_t m, int64_t n);
 size_t split_scratch_bytes(size_t key_size, bool pairs, int64_t m, int64_t n);
 template <typename K>
-int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, int64_t n, void* scratch, int poll_limit,
-              int compare_max, const LeftTables& tables, const uint32_t** other_rows, const uint32_t** route_records, size_t* route_stride);
+int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, int64_t n, void* scratch, int compare_max);
+
+// ------------------------------------------------------------------ stable ranks by digit
+// Every wavefront of a workgroup ranks its ITEMS x 64 elements, item k of lane l being element
+// k * 64 + l of the wavefront's share: rank[k] = how many earlier elements of the wavefront
+// carry the same digit d[k] (wave-wide matching over the bits of `vary`; all other bits must
+// agree in every element).  wave_hist[w][*] must be zero on entry (and that visible); on return
+// (no barrier inside) row w holds the wavefront's count of every digit.
+template <int ITEMS>
+__device__ __forceinline__ void rank_by_digit(uint32_t* __restrict__ wave_hist_row, const uint32_t (&d)[ITEMS], uint32_t vary, uint32_t (&rank)[ITEMS]) {
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        uint32_t peers_lo = 0xffffffffu, peers_hi = 0xffffffffu;
+        for (uint32_t bits = vary; bits != 0u; bits &= bits - 1u) {
+            const uint32_t b = static_cast<uint32_t>(__builtin_ctz(bits));
+            const int32_t ones = __builtin_amdgcn_sbfe(static_cast<int32_t>(d[k]), b, 1u);
+            const unsigned long long vote = __ballot(ones < 0);
+            peers_lo &= ~(static_cast<uint32_t>(vote) ^ static_cast<uint32_t>(ones));
+            peers_hi &= ~(static_cast<uint32_t>(vote >> 32) ^ static_cast<uint32_t>(ones));
+        }
+        const uint32_t before = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
+        const uint32_t cnt = static_cast<uint32_t>(__popc(peers_lo) + __popc(peers_hi));
+        const uint32_t seen = wave_hist_row[d[k]];
+        rank[k] = seen + before;
+        __builtin_amdgcn_wave_barrier();
+        if (before == 0) wave_hist_row[d[k]] = seen + cnt;
+        __builtin_amdgcn_wave_barrier();
+    }
+}
 
 // ------------------------------------------------------------------ a sort that stays in one workgroup
 constexpr int kSmallMoves = 256;         // keys that the run walk of sort_in_workgroup may move (one thread each)

@@ -14,9 +14,11 @@
 //                       skewed rows - floats with their exponents, clustered integers - still
 //                       give even buckets.  Every chunk's histogram becomes the place of its keys
 //                       inside each bucket, and the buckets of all rows are listed for the last
-//                       step.  A row whose largest fine bin does not fit a workgroup, or that
-//                       would need more than 256 buckets, keeps the least-significant-digit-first
-//                       passes of sort.hip (decided here, on the device, row by row).
+//                       step.  A row with a fine bin fuller than a workgroup holds (one value
+//                       repeated many times, keys packed more tightly than the bins resolve)
+//                       gets buckets larger than that - each such bin one to itself where the
+//                       bucket numbers allow - which step 6 finishes (decided here, on the
+//                       device, row by row).
 //   4. split_pass       one workgroup per chunk: a tile of 4096 keys finds each key's bucket
 //                       (table in LDS) and its slot among the tile's keys of that bucket with one
 //                       LDS atomic, lays the tile out by bucket in LDS and writes it as runs to
@@ -30,7 +32,13 @@
 //                       order of equal keys; the bucket leaves for the strided outputs.
 //   6. split_finish_crowded  buckets with a bin too crowded for that (many equal or clustered
 //                       keys) take the stable digit passes of sort_in_workgroup instead, for
-//                       pairs first by index, then by key.
+//                       pairs first by index, then by key.  A bucket larger than a workgroup
+//                       holds is sorted by the one workgroup that draws it: stable digit passes
+//                       over the digits that vary in it (none for one repeated value: a copy),
+//                       window by window, between the scratch buffer and the bucket's place
+//                       in the outputs.  Pairs of such a row were moved by split_pass_stable
+//                       (ranks in element order instead of atomics), so they arrive in index
+//                       order.
 // Ranking with an LDS atomic costs a few instructions per key where wave-wide digit matching
 // costs about fifty per digit, which is what bounds the digit passes.
 #include <cstddef>
@@ -441,19 +449,26 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
 }
 
 // ------------------------------------------------------------------ 3. buckets of equal depth
-// One workgroup per row; thread t owns fine bins [16 t, 16 t + 16).  counters[0] counts the rows
-// that keep the digit passes (their tables of those passes are cleared here), counters[2] the
-// buckets listed for split_finish.  For a row that
-// takes the route, chunk_base[chunk][b] receives the row position where that chunk's keys of
-// bucket b go: the bucket's start plus what the row's earlier chunks hold of it.
+// One workgroup per row; thread t owns fine bins [16 t, 16 t + 16).  For every row,
+// chunk_base[chunk][b] receives the row position where that chunk's keys of bucket b go: the
+// bucket's start plus what the row's earlier chunks hold of it.  Buckets that a workgroup of
+// split_finish holds are appended to bucket_list (counters[2] entries); a row with a fine bin
+// fuller than that (one value repeated many times, keys clustered more tightly than the fine
+// bins resolve) has buckets that are larger: those go on the list split_finish_crowded walks
+// (counters[1] entries) and the row is marked route 2, which for pairs makes split_pass_stable
+// move it, so that every bucket of the row arrives in index order.
 __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t cap, int64_t chunks_per_row, const uint32_t* __restrict__ chunk_fine,
-                                                          SplitRow* __restrict__ rows, uint32_t* __restrict__ counters, LeftTables left,
-                                                          uint4* __restrict__ bucket_list, uint32_t* __restrict__ chunk_base) {
+                                                          SplitRow* __restrict__ rows, uint32_t* __restrict__ counters,
+                                                          uint4* __restrict__ bucket_list, uint32_t* __restrict__ crowded_list,
+                                                          uint32_t* __restrict__ chunk_base) {
     constexpr int PER = kFine / kSplitBlock;          // 16
-    __shared__ uint32_t red[kSplitBlock / kWave];
-    __shared__ uint32_t listed[2];                    // buckets of this row, and where they go in the list
+    constexpr int WAVES = kSplitBlock / kWave;
+    __shared__ uint32_t red[WAVES];
+    __shared__ uint32_t listed[2][WAVES + 1];         // buckets of this row for either list by wavefront, and where they go
     __shared__ uint32_t per_bucket[kMaxBuckets];
+    __shared__ uint32_t last_count[kSplitBlock];      // every thread's last fine bin
     const int64_t row = blockIdx.x;
+    const int w = threadIdx.x / kWave;
     const uint32_t* f = chunk_fine + row * chunks_per_row * (kFine / 2) + threadIdx.x * (PER / 2);
     SplitRow& info = rows[row];
     uint32_t cnt[PER];
@@ -484,87 +499,95 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
         sum += cnt[i];
         biggest = cnt[i] > biggest ? cnt[i] : biggest;
     }
-    biggest = block_reduce(biggest, [](uint32_t a, uint32_t b) { return a > b ? a : b; }, red, kSplitBlock / kWave);
+    last_count[threadIdx.x] = cnt[PER - 1];
+    biggest = block_reduce(biggest, [](uint32_t a, uint32_t b) { return a > b ? a : b; }, red, WAVES);
     // exclusive prefix of the thread sums
     const uint32_t incl = wave_scan_inclusive(sum, 0u, [](uint32_t a, uint32_t b) { return a + b; });
     __syncthreads();
-    if (lane_id() == kWave - 1) red[threadIdx.x / kWave] = incl;
+    if (lane_id() == kWave - 1) red[w] = incl;
     __syncthreads();
     uint32_t before = incl - sum;
-    for (int i = 0; i < static_cast<int>(threadIdx.x / kWave); ++i) before += red[i];
+    for (int i = 0; i < w; ++i) before += red[i];
 
-    // every fine bin leaves room in a bucket
-    const bool fits = biggest < cap;
-    const uint32_t target = fits ? cap - biggest : 1u;
-
-    // A bin goes to bucket (keys before it) / target, so that every bucket holds fewer than
-    // target + biggest = cap keys; and where at least kGapBins empty bins lie between two
-    // populated ones a new bucket starts as well: stray keys far from the rest (a few zeros below
-    // positive values) then do not stretch the range of the bucket next to them, which
-    // split_finish resolves with a fixed number of counting bins.
-    constexpr int kGapBins = 64;
-    int last = -1;                                     // last populated bin of this thread
-#pragma unroll
-    for (int i = 0; i < PER; ++i)
-        if (cnt[i]) last = static_cast<int>(threadIdx.x) * PER + i;
-    int seen = wave_scan_inclusive(last, -1, [](int a, int b) { return a > b ? a : b; });
-    __syncthreads();
-    if (lane_id() == kWave - 1) red[threadIdx.x / kWave] = static_cast<uint32_t>(seen);
-    __syncthreads();
-    int populated_before = __shfl_up(seen, 1, kWave);  // last populated bin before this thread's first
-    if (lane_id() == 0) populated_before = -1;
-    for (int i = 0; i < static_cast<int>(threadIdx.x / kWave); ++i)
-        populated_before = static_cast<int>(red[i]) > populated_before ? static_cast<int>(red[i]) : populated_before;
-    uint32_t cuts = 0;                                 // gaps that end in this thread's bins
-    uint32_t cut_at = 0;                               // bit i: bin i of this thread starts a bucket after a gap
-    {
-        int prev = populated_before;
-#pragma unroll
-        for (int i = 0; i < PER; ++i) {
-            const int bin = static_cast<int>(threadIdx.x) * PER + i;
-            if (cnt[i]) {
-                if (prev >= 0 && bin - prev > kGapBins) {
-                    cut_at |= 1u << i;
-                    ++cuts;
-                }
-                prev = bin;
-            }
-        }
-    }
-    const uint32_t cuts_incl = wave_scan_inclusive(cuts, 0u, [](uint32_t a, uint32_t b) { return a + b; });
-    __syncthreads();
-    if (lane_id() == kWave - 1) red[threadIdx.x / kWave] = cuts_incl;
-    __syncthreads();
-    uint32_t cuts_before = cuts_incl - cuts;
-    for (int i = 0; i < static_cast<int>(threadIdx.x / kWave); ++i) cuts_before += red[i];
-
+    // A bin goes to bucket (keys before it) / target plus the cuts at or before it: bit i of
+    // `cut_at` makes bin i of this thread open a new bucket whatever the count says.  Returns
+    // the number of buckets.
     uint32_t bucket[PER];
-    {
-        uint32_t run = before, extra = cuts_before;
+    __shared__ uint32_t last_bucket[kSplitBlock];
+    auto assign = [&](uint32_t target, uint32_t cut_at) __attribute__((always_inline)) -> uint32_t {
+        const uint32_t cuts = static_cast<uint32_t>(__popc(cut_at));
+        const uint32_t cuts_incl = wave_scan_inclusive(cuts, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+        __syncthreads();
+        if (lane_id() == kWave - 1) red[w] = cuts_incl;
+        __syncthreads();
+        uint32_t extra = cuts_incl - cuts;
+        for (int i = 0; i < w; ++i) extra += red[i];
+        uint32_t run = before;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
             extra += (cut_at >> i) & 1u;
             bucket[i] = run / target + extra;
             run += cnt[i];
         }
-    }
-    // the bucket of the bin before this thread's first, and the number of buckets
-    __shared__ uint32_t last_bucket[kSplitBlock];
-    last_bucket[threadIdx.x] = bucket[PER - 1];
-    __syncthreads();
-    const uint32_t n_buckets = last_bucket[kSplitBlock - 1] + 1;
-    if (!fits || n_buckets > static_cast<uint32_t>(kMaxBuckets)) {
-        if (threadIdx.x == 0) {
-            info.route = 0u;
-            atomicAdd(&counters[0], 1u);
-            left.arrived[row] = 0u;
+        last_bucket[threadIdx.x] = bucket[PER - 1];
+        __syncthreads();
+        return last_bucket[kSplitBlock - 1] + 1;
+    };
+
+    // Where at least kGapBins empty bins lie between two populated ones a new bucket starts
+    // whatever the counts say: stray keys far from the rest (a few zeros below positive values)
+    // then do not stretch the range of the bucket next to them, which split_finish resolves with
+    // a fixed number of counting bins.
+    constexpr int kGapBins = 64;
+    uint32_t gap_cuts = 0;
+    {
+        int last = -1;                                 // last populated bin of this thread
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+            if (cnt[i]) last = static_cast<int>(threadIdx.x) * PER + i;
+        int seen = wave_scan_inclusive(last, -1, [](int a, int b) { return a > b ? a : b; });
+        __syncthreads();
+        if (lane_id() == kWave - 1) red[w] = static_cast<uint32_t>(seen);
+        __syncthreads();
+        int prev = __shfl_up(seen, 1, kWave);          // last populated bin before this thread's first
+        if (lane_id() == 0) prev = -1;
+        for (int i = 0; i < w; ++i) prev = static_cast<int>(red[i]) > prev ? static_cast<int>(red[i]) : prev;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int bin = static_cast<int>(threadIdx.x) * PER + i;
+            if (cnt[i]) {
+                if (prev >= 0 && bin - prev > kGapBins) gap_cuts |= 1u << i;
+                prev = bin;
+            }
         }
-        // the digit passes sort this row: their tables for it start at zero
-        uint4* hist = reinterpret_cast<uint4*>(left.hist + row * left.hist_words);
-        for (uint32_t i = threadIdx.x; i < left.hist_words / 4; i += kSplitBlock) hist[i] = make_uint4(0u, 0u, 0u, 0u);
-        uint4* status = reinterpret_cast<uint4*>(left.status + row * left.status_words);
-        for (int64_t i = threadIdx.x; i < left.status_words / 4; i += kSplitBlock) status[i] = make_uint4(0u, 0u, 0u, 0u);
-        return;
+    }
+
+    // Every fine bin leaves room in a bucket: buckets of (keys before) / (cap - largest bin) hold
+    // fewer than cap keys each.
+    uint32_t route = 1u, n_buckets = kMaxBuckets + 1;
+    if (biggest < cap) {
+        n_buckets = assign(cap - biggest, gap_cuts);
+        if (n_buckets > static_cast<uint32_t>(kMaxBuckets)) n_buckets = assign(cap - biggest, 0u);
+    }
+    if (n_buckets > static_cast<uint32_t>(kMaxBuckets)) {
+        // Some fine bin does not (or too many buckets would be needed): the row gets buckets of
+        // cap * 3/4 keys plus a bin of less than cap / 4 - or of n / 224 keys when that is more,
+        // which 256 buckets always hold - and every fuller bin a bucket to itself while the
+        // bucket numbers allow it; a bucket larger than cap is finished by split_finish_crowded
+        // (a bucket of one value costs next to nothing there).
+        route = 2u;
+        const uint32_t heavy = cap / 4;
+        uint32_t heavy_cuts = 0;
+        uint32_t prev = threadIdx.x == 0 ? 0u : last_count[threadIdx.x - 1];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            if (cnt[i] >= heavy || prev >= heavy) heavy_cuts |= 1u << i;
+            prev = cnt[i];
+        }
+        const uint32_t by_count = static_cast<uint32_t>((n + 223) / 224);
+        const uint32_t target = cap - heavy > by_count ? cap - heavy : by_count;
+        n_buckets = assign(target, heavy_cuts);
+        if (n_buckets > static_cast<uint32_t>(kMaxBuckets)) n_buckets = assign(target, 0u);      // at most 224
     }
     // a bin opens every bucket after its predecessor's up to its own (the starts are put together
     // in LDS: the threads read one another's just below)
@@ -589,30 +612,55 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
     if (threadIdx.x == kSplitBlock - 1) {
         info.n_buckets = n_buckets;
         begin[n_buckets] = static_cast<uint32_t>(n);
-        info.route = 1u;
-        listed[0] = n_buckets;
-        listed[1] = atomicAdd(&counters[2], n_buckets);
+        info.route = route;
+        if (route == 2u) atomicAdd(&counters[3], 1u);      // split_pass_stable has something to do
     }
     per_bucket[threadIdx.x] = 0u;
     __syncthreads();
     for (uint32_t k = threadIdx.x; k <= n_buckets; k += kSplitBlock) info.begin[k] = begin[k];
-    // the buckets of every such row, in no particular order: what split_finish walks
+    // The buckets that hold anything, in no particular order, on the list of the kernel that
+    // finishes them: split_finish those that fit its workgroup, split_finish_crowded the others.
     uint32_t next = 0;                                 // where the coming chunk's keys of bucket threadIdx.x go
-    if (threadIdx.x < listed[0]) {
-        const uint32_t b0 = begin[threadIdx.x], b1 = begin[threadIdx.x + 1];
-        bucket_list[listed[1] + threadIdx.x] = make_uint4(static_cast<uint32_t>(row), b0, b1 - b0, static_cast<uint32_t>(row) * kMaxBuckets + threadIdx.x);
-        next = b0;
+    {
+        uint32_t b0 = 0, size = 0;
+        if (threadIdx.x < n_buckets) {
+            b0 = begin[threadIdx.x];
+            size = begin[threadIdx.x + 1] - b0;
+            next = b0;
+        }
+        const bool fits_finish = size != 0u && size <= cap, oversized = size > cap;
+        const unsigned long long fit_lanes = __ballot(fits_finish), over_lanes = __ballot(oversized);
+        if (lane_id() == 0) {
+            listed[0][w] = static_cast<uint32_t>(__popcll(fit_lanes));
+            listed[1][w] = static_cast<uint32_t>(__popcll(over_lanes));
+        }
+        __syncthreads();
+        if (threadIdx.x < 2) {
+            uint32_t total = 0;
+            for (int i = 0; i < WAVES; ++i) {
+                const uint32_t c = listed[threadIdx.x][i];
+                listed[threadIdx.x][i] = total;
+                total += c;
+            }
+            listed[threadIdx.x][WAVES] = total ? atomicAdd(&counters[threadIdx.x == 0 ? 2 : 1], total) : 0u;
+        }
+        __syncthreads();
+        const unsigned long long below = (1ull << lane_id()) - 1ull;
+        const uint32_t id = static_cast<uint32_t>(row) * kMaxBuckets + threadIdx.x;
+        if (fits_finish)
+            bucket_list[listed[0][WAVES] + listed[0][w] + static_cast<uint32_t>(__popcll(fit_lanes & below))] = make_uint4(static_cast<uint32_t>(row), b0, size, id);
+        if (oversized) crowded_list[listed[1][WAVES] + listed[1][w] + static_cast<uint32_t>(__popcll(over_lanes & below))] = id;
     }
     // each chunk's keys per bucket, and from them where the chunk writes each bucket
-    uint32_t w[PER / 2], ahead[PER / 2];
-    chunk_words(0, w);
+    uint32_t w8[PER / 2], ahead[PER / 2];
+    chunk_words(0, w8);
     for (int64_t c = 0; c < chunks_per_row; ++c) {
         if (c + 1 < chunks_per_row) chunk_words(c + 1, ahead);        // on its way across this chunk's barriers
         // this thread's bins lie in few buckets: sum runs of equal buckets before touching LDS
         uint32_t acc = 0;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            acc += (i & 1) ? (w[i / 2] >> 16) : (w[i / 2] & 0xffffu);
+            acc += (i & 1) ? (w8[i / 2] >> 16) : (w8[i / 2] & 0xffffu);
             if (i == PER - 1 || bucket[i + 1] != bucket[i]) {
                 if (acc) atomicAdd(&per_bucket[bucket[i]], acc);
                 acc = 0;
@@ -624,7 +672,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
         per_bucket[threadIdx.x] = 0u;
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < PER / 2; ++i) w[i] = ahead[i];
+        for (int i = 0; i < PER / 2; ++i) w8[i] = ahead[i];
     }
 }
 
@@ -665,7 +713,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
     const int64_t row = blockIdx.x / chunks_per_row;
     const int64_t c = blockIdx.x - row * chunks_per_row;
     const SplitRow& info = infos[row];
-    if (info.route != 1u) return;
+    if (PAIRS && info.route != 1u) return;             // (a row with buckets larger than a workgroup holds: split_pass_stable)
     const FineMap<K> fine_of(info, io.descending);
     const K* xrow = io.x + io.xmap.at(row);
     const int64_t row_off = row * n;
@@ -817,6 +865,91 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
     };
     if (MAP == kMapValue && fine_of.by_value) move_chunk(std::integral_constant<bool, MAP == kMapValue>());
     else move_chunk(std::false_type());
+}
+
+// The same pass for the rows (of pairs) that have buckets larger than a workgroup holds
+// (SplitRow::route 2): every key's slot among the tile's keys of its bucket is its rank in
+// element order (wave-wide matching of bucket numbers, as the digit passes rank), so each bucket
+// receives its entries in index order and a bucket of one repeated value arrives sorted.  Entries
+// go straight to their places in the row; a tile is 256 threads x 16 keys, wavefront w taking
+// elements [1024 w, 1024 w + 1024) of it.
+template <typename K>
+__global__ __launch_bounds__(kSplitBlock) void split_pass_stable(PassIo<K> io, int64_t n, int64_t chunks_per_row, int64_t chunks,
+                                                                 const SplitRow* __restrict__ infos, const uint32_t* __restrict__ counters,
+                                                                 const uint32_t* __restrict__ chunk_base) {
+    constexpr int ITEMS = kSplitItems;
+    constexpr int WAVES = kSplitBlock / kWave;
+    constexpr int TILE = kSplitBlock * ITEMS;
+    __shared__ uint32_t table[kFine / 4];
+    __shared__ uint32_t wave_hist[WAVES][kMaxBuckets];
+    __shared__ uint32_t place[kMaxBuckets];            // row position of the tile's first entry of each bucket
+    const int tid = threadIdx.x;
+    const int lane = lane_id();
+    const int w = tid / kWave;
+    if (counters[3] == 0u) return;                     // no such row in this call (the usual case)
+    // (a small grid walks the chunks: the launch costs little when there is nothing to do)
+    for (int64_t unit = blockIdx.x; unit < chunks; unit += gridDim.x) {
+    const int64_t row = unit / chunks_per_row;
+    const int64_t c = unit - row * chunks_per_row;
+    const SplitRow& info = infos[row];
+    if (info.route != 2u) continue;
+    __syncthreads();                                   // the chunk before has left the table
+    const FineMap<K> fine_of(info, io.descending);
+    const K* xrow = io.x + io.xmap.at(row);
+    K* dk = io.kbuf[0] + row * n;
+    uint32_t* dv = io.vbuf[0] + row * n;
+    const int64_t chunk_lo = c * kChunk;
+    const int64_t chunk_hi = (chunk_lo + kChunk < n) ? chunk_lo + kChunk : n;
+    // bucket numbers lie below n_buckets: only those bits are matched
+    const uint32_t vary = info.n_buckets > 1u ? (2u << (31 - __builtin_clz(info.n_buckets - 1u))) - 1u : 0u;
+    static_assert(kSplitBlock == kMaxBuckets, "a thread per bucket");
+    reinterpret_cast<uint4*>(table)[tid] = reinterpret_cast<const uint4*>(info.bucket_of)[tid];
+    uint32_t next = chunk_base[unit * kMaxBuckets + tid];      // where this chunk's coming keys of bucket tid go
+    for (int64_t tile_base = chunk_lo; tile_base < chunk_hi; tile_base += TILE) {
+        for (int i = tid; i < WAVES * kMaxBuckets; i += kSplitBlock) (&wave_hist[0][0])[i] = 0u;
+        K key[ITEMS];
+        uint32_t bucket[ITEMS], rank[ITEMS];
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const int64_t e = tile_base + w * (kWave * ITEMS) + k * kWave + lane;
+            key[k] = key_of_element<K>(io, xrow[(e < chunk_hi ? e : chunk_lo) * io.sx]);
+        }
+        __syncthreads();                               // table and zeroed counts are in place
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const uint32_t f = fine_of(key[k]);
+            bucket[k] = (table[f >> 2] >> (8u * (f & 3u))) & 0xffu;
+            // (elements beyond the chunk's end come after every element of it: whatever bucket
+            // they are counted in, no rank of an element of the chunk changes, and the counts are
+            // never used again after a chunk's last tile)
+        }
+        rank_by_digit<ITEMS>(wave_hist[w], bucket, vary, rank);
+        __syncthreads();
+        {
+            // thread b owns bucket b: each wavefront's share of it starts after the shares of the wavefronts before
+            uint32_t run = 0;
+#pragma unroll
+            for (int i = 0; i < WAVES; ++i) {
+                const uint32_t count = wave_hist[i][tid];
+                wave_hist[i][tid] = run;
+                run += count;
+            }
+            place[tid] = next;
+            next += run;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const int64_t e = tile_base + w * (kWave * ITEMS) + k * kWave + lane;
+            if (e < chunk_hi) {
+                const uint32_t at = place[bucket[k]] + wave_hist[w][bucket[k]] + rank[k];
+                dk[at] = key[k];
+                dv[at] = static_cast<uint32_t>(e);
+            }
+        }
+        __syncthreads();                               // the counts and places have been read
+    }
+    }
 }
 
 // ------------------------------------------------------------------ 5. a bucket, on chip
@@ -1195,8 +1328,192 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
     }
 }
 
+// ------------------------------------------------------------------ 6. what split_finish does not take
+// A bucket larger than a workgroup holds, sorted by the one workgroup that drew it from the list.
+// Its entries lie in kbuf[0] / vbuf[0] ("side A"), pairs in index order (split_pass_stable).  The
+// bucket's place in the outputs ("side B": the value output and / or the index output, whatever
+// their strides) is the only other memory that is certainly there, so the stable digit passes
+// below ping-pong between the two: key images travel through the value output as they are and
+// are decoded by the last pass, which always goes from A to B; without a value output the keys
+// of side B are read again from the input through the indices (possible while the input is
+// intact).  Digits that are the same in the whole bucket are left out - a bucket of one repeated
+// value is just copied - and an even number of passes is preceded by a plain copy to B.
+template <typename K, bool PAIRS>
+struct OversizedIo {
+    const PassIo<K>& io;
+    const K* xrow;
+    K* yrow;
+    int64_t irow;
+    K* ak;                                             // side A
+    uint32_t* av;
+    __device__ __forceinline__ void read(bool side_b, int64_t at, K* key, uint32_t* val) const {
+        if (!side_b) {
+            *key = ak[at];
+            if constexpr (PAIRS) *val = av[at];
+            return;
+        }
+        if constexpr (PAIRS) {
+            *val = io.idx64 ? static_cast<uint32_t>(static_cast<const int64_t*>(io.idx)[irow + at * io.si])
+                            : static_cast<uint32_t>(static_cast<const int32_t*>(io.idx)[irow + at * io.si]);
+            *key = yrow ? yrow[at * io.sy] : key_of_element<K>(io, xrow[static_cast<int64_t>(*val) * io.sx]);
+        } else {
+            *key = yrow[at * io.sy];
+        }
+    }
+    __device__ __forceinline__ void write(bool side_b, int64_t at, K key, uint32_t val) const {
+        if (!side_b) {
+            ak[at] = key;
+            if constexpr (PAIRS) av[at] = val;
+            return;
+        }
+        if (yrow) yrow[at * io.sy] = key;
+        if constexpr (PAIRS) {
+            if (io.idx64) static_cast<int64_t*>(io.idx)[irow + at * io.si] = static_cast<int64_t>(val);
+            else static_cast<int32_t*>(io.idx)[irow + at * io.si] = static_cast<int32_t>(val);
+        }
+    }
+};
+
+// Returns false, having done nothing, for the one case it does not take: an index-only argsort
+// whose index output overwrites the input (side B cannot hold keys and they cannot be read again
+// either); the caller then sorts the bucket where it lies.
+template <typename K, bool PAIRS, int WAVES>
+__device__ __forceinline__ bool sort_oversized(SmallShared<K, PAIRS, kFinishItems, WAVES>& sm, const PassIo<K>& io, int64_t n, int64_t row, int64_t begin, int64_t size) {
+    constexpr int ITEMS = kFinishItems;
+    constexpr int T = WAVES * kWave;
+    constexpr int WINDOW = T * ITEMS;
+    __shared__ uint32_t digit_at[kRadix];              // where the next entry of each digit goes
+    const int tid = threadIdx.x;
+    const int lane = lane_id();
+    const int w = tid / kWave;
+    const int seg = w * kWave * ITEMS + lane;
+    OversizedIo<K, PAIRS> mem{io, io.x + io.xmap.at(row), io.y ? io.y + io.ymap.at(row) : nullptr, (PAIRS && io.idx) ? io.imap.at(row) : 0,
+                              io.kbuf[0] + row * n, PAIRS ? io.vbuf[0] + row * n : nullptr};
+
+    // ---- which bits differ inside the bucket
+    K ors = 0, ands = ~K(0);
+    for (int64_t i = tid; i < size; i += T) {
+        const K k1 = mem.ak[begin + i];
+        ors |= k1;
+        ands &= k1;
+    }
+    ors = wave_reduce(ors, [](K a, K b) { return static_cast<K>(a | b); });
+    ands = wave_reduce(ands, [](K a, K b) { return static_cast<K>(a & b); });
+    __syncthreads();
+    if (lane == 0) {
+        sm.wave_or[w] = ors;
+        sm.wave_and[w] = ands;
+    }
+    __syncthreads();
+    K any = 0, all = ~K(0);
+#pragma unroll
+    for (int i = 0; i < WAVES; ++i) {
+        any |= sm.wave_or[i];
+        all &= sm.wave_and[i];
+    }
+    const K differ = static_cast<K>(any & ~all);
+    int passes = 0;
+    for (int p = 0; p < KeyTraits<K>::kPasses; ++p) passes += (static_cast<uint32_t>(differ >> (8 * p)) & 0xffu) != 0u ? 1 : 0;
+
+    // entry `at` of the sorted row leaves for good
+    auto emit = [&](int64_t at, K k1, uint32_t v1) __attribute__((always_inline)) {
+        emit_entry<K, PAIRS>(io, mem.xrow, mem.yrow, mem.irow, at, k1, v1);
+    };
+    if (passes == 0) {                                 // one value: pairs are in index order already
+        for (int64_t i = tid; i < size; i += T) {
+            K k1;
+            uint32_t v1 = 0;
+            mem.read(false, begin + i, &k1, &v1);
+            emit(begin + i, k1, v1);
+        }
+        return true;
+    }
+    if (PAIRS && !mem.yrow && !io.x_intact) return false;
+
+    bool from_b = false;
+    if (passes % 2 == 0) {                             // so that the last pass goes from A to B
+        for (int64_t i = tid; i < size; i += T) {
+            K k1;
+            uint32_t v1 = 0;
+            mem.read(false, begin + i, &k1, &v1);
+            mem.write(true, begin + i, k1, v1);
+        }
+        from_b = true;
+        __syncthreads();
+    }
+    int left = passes;
+    for (int p = 0; p < KeyTraits<K>::kPasses; ++p) {
+        const int shift = 8 * p;
+        const uint32_t vary = static_cast<uint32_t>(differ >> shift) & 0xffu;
+        if (vary == 0u) continue;
+        const bool last = --left == 0;
+        // ---- how many entries carry each digit, and from that where each digit's run starts
+        for (int i = tid; i < kRadix; i += T) digit_at[i] = 0u;
+        __syncthreads();
+        for (int64_t i = tid; i < size; i += T) {
+            K k1;
+            uint32_t v1 = 0;
+            mem.read(from_b, begin + i, &k1, &v1);
+            atomicAdd(&digit_at[static_cast<uint32_t>(k1 >> shift) & 0xffu], 1u);
+        }
+        __syncthreads();
+        {
+            const uint32_t count = tid < kRadix ? digit_at[tid] : 0u;
+            const uint32_t incl = wave_scan_inclusive(count, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+            if (tid < kRadix && lane == kWave - 1) sm.scan_tmp[w] = incl;
+            __syncthreads();
+            if (tid < kRadix) {
+                uint32_t run = incl - count;
+                for (int i = 0; i < w; ++i) run += sm.scan_tmp[i];
+                digit_at[tid] = run;
+            }
+        }
+        // ---- window by window, in order: stable ranks inside the window, runs carried along
+        for (int64_t lo = 0; lo < size; lo += WINDOW) {
+            for (int i = tid; i < WAVES * kRadix; i += T) (&sm.wave_hist[0][0])[i] = 0u;
+            K key[ITEMS];
+            uint32_t val[PAIRS ? ITEMS : 1];
+            uint32_t digit[ITEMS], rank[ITEMS];
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) {
+                const int64_t e = lo + seg + k * kWave;
+                key[k] = all;                          // padding agrees with the bucket in every bit that does not vary
+                if constexpr (PAIRS) val[k] = 0u;
+                if (e < size) mem.read(from_b, begin + e, &key[k], &val[PAIRS ? k : 0]);
+                digit[k] = static_cast<uint32_t>(key[k] >> shift) & 0xffu;
+            }
+            __syncthreads();                           // zeroed counts and digit_at are in place
+            rank_by_digit<ITEMS>(sm.wave_hist[w], digit, vary, rank);
+            __syncthreads();
+            if (tid < kRadix) {
+                uint32_t run = digit_at[tid];
+#pragma unroll
+                for (int i = 0; i < WAVES; ++i) {
+                    const uint32_t count = sm.wave_hist[i][tid];
+                    sm.wave_hist[i][tid] = run;
+                    run += count;
+                }
+                digit_at[tid] = run;                   // (padding of the last window counts too: never used again)
+            }
+            __syncthreads();
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) {
+                if (lo + seg + k * kWave < size) {
+                    const int64_t at = begin + sm.wave_hist[w][digit[k]] + rank[k];
+                    if (last) emit(at, key[k], PAIRS ? val[k] : 0u);
+                    else mem.write(!from_b, at, key[k], PAIRS ? val[k] : 0u);
+                }
+            }
+            __syncthreads();
+        }
+        from_b = !from_b;
+    }
+    return true;
+}
+
 // The buckets split_finish left: stable digit passes on chip - for pairs first by index (the
-// entries arrive in no particular order), then by key.
+// entries arrive in no particular order), then by key - and the buckets larger than a workgroup
+// holds, which split_plan put on the same list.
 template <typename K, bool PAIRS, int WAVES>
 __global__ __launch_bounds__(WAVES * kWave) void split_finish_crowded(PassIo<K> io, int64_t n, const SplitRow* __restrict__ infos,
                                                                      const uint32_t* __restrict__ counters,
@@ -1208,8 +1525,13 @@ __global__ __launch_bounds__(WAVES * kWave) void split_finish_crowded(PassIo<K> 
     const int seg = (threadIdx.x / kWave) * kWave * ITEMS + lane;
     for (uint32_t i = blockIdx.x; i < listed; i += gridDim.x) {
         const uint4 at = bucket_at(infos, crowded_list[i]);
-        const int valid = static_cast<int>(at.z);
         const int64_t at_row = at.x, at_begin = at.y;
+        if (at.z > static_cast<uint32_t>(finish_cap(WAVES))) {
+            (void)sort_oversized<K, PAIRS, WAVES>(sm, io, n, at_row, at_begin, at.z);      // (what it does not take: split_finish_in_place)
+            __syncthreads();
+            continue;
+        }
+        const int valid = static_cast<int>(at.z);
         const K* src = io.kbuf[0] + at_row * n + at_begin;
         const uint32_t* vsrc = PAIRS ? io.vbuf[0] + at_row * n + at_begin : nullptr;
         K key[ITEMS];
@@ -1246,6 +1568,96 @@ __global__ __launch_bounds__(WAVES * kWave) void split_finish_crowded(PassIo<K> 
     }
 }
 
+// The oversized buckets of several values that sort_oversized leaves: an index-only argsort
+// whose index output overwrites its input (the host launches this kernel for such calls only).
+// The bucket is sorted where it lies - neighbouring halves of windows sorted together on chip,
+// odd and even pairs in turn, as many rounds as there are halves - and then copied out: slow
+// (the work grows with the square of the bucket), and only for this combination.
+template <typename K, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void split_finish_in_place(PassIo<K> io, int64_t n, const SplitRow* __restrict__ infos,
+                                                                      const uint32_t* __restrict__ counters,
+                                                                      const uint32_t* __restrict__ crowded_list) {
+    constexpr int ITEMS = kFinishItems;
+    constexpr int T = WAVES * kWave, WINDOW = T * ITEMS, HALF = WINDOW / 2;
+    __shared__ SmallShared<K, true, ITEMS, WAVES> sm;
+    const uint32_t listed = counters[1];
+    const int lane = lane_id();
+    const int w = threadIdx.x / kWave;
+    const int seg = w * kWave * ITEMS + lane;
+    for (uint32_t i = blockIdx.x; i < listed; i += gridDim.x) {
+        const uint4 at = bucket_at(infos, crowded_list[i]);
+        const int64_t size = at.z;
+        if (size <= WINDOW) continue;
+        K* ak = io.kbuf[0] + static_cast<int64_t>(at.x) * n + at.y;
+        uint32_t* av = io.vbuf[0] + static_cast<int64_t>(at.x) * n + at.y;
+        // a bucket of one value was copied out by split_finish_crowded
+        K kor = 0, kand = ~K(0);
+        for (int64_t e = threadIdx.x; e < size; e += T) {
+            kor |= ak[e];
+            kand &= ak[e];
+        }
+        kor = wave_reduce(kor, [](K a, K b) { return static_cast<K>(a | b); });
+        kand = wave_reduce(kand, [](K a, K b) { return static_cast<K>(a & b); });
+        __syncthreads();
+        if (lane == 0) {
+            sm.wave_or[w] = kor;
+            sm.wave_and[w] = kand;
+        }
+        __syncthreads();
+        K any = 0, all = ~K(0);
+#pragma unroll
+        for (int j = 0; j < WAVES; ++j) {
+            any |= sm.wave_or[j];
+            all &= sm.wave_and[j];
+        }
+        __syncthreads();
+        if (any == all) continue;
+        const int64_t halves = (size + HALF - 1) / HALF;
+#pragma unroll 1
+        for (int64_t round = 0; round < halves; ++round) {
+#pragma unroll 1
+            for (int64_t h = round & 1; h < halves; h += 2) {
+                const int64_t lo = h * HALF;
+                const int valid = static_cast<int>(size - lo < WINDOW ? size - lo : WINDOW);
+                if (valid <= HALF && round > 0) continue;       // a lone last half: sorted since the first round
+                K key[ITEMS];
+                uint32_t val[ITEMS];
+                K ors = 0, ands = ~K(0), vors = 0, vands = ~K(0);
+#pragma unroll
+                for (int k = 0; k < ITEMS; ++k) {
+                    const int e = seg + k * kWave;
+                    key[k] = ~K(0);                            // padding sorts last, by index and by key
+                    val[k] = ~0u;
+                    if (e < valid) {
+                        key[k] = ak[lo + e];
+                        val[k] = av[lo + e];
+                        ors |= key[k];
+                        ands &= key[k];
+                        vors |= static_cast<K>(val[k]);
+                        vands &= static_cast<K>(val[k]);
+                    }
+                }
+                sort_in_workgroup<K, true, ITEMS, WAVES, true>(sm, key, val, vors, vands, valid, 4);
+                __syncthreads();
+                sort_in_workgroup<K, true, ITEMS, WAVES>(sm, key, val, ors, ands, valid, KeyTraits<K>::kPasses);
+#pragma unroll
+                for (int k = 0; k < ITEMS; ++k) {
+                    const int e = seg + k * kWave;
+                    if (e < valid) {
+                        ak[lo + e] = key[k];
+                        av[lo + e] = val[k];
+                    }
+                }
+                __syncthreads();
+            }
+        }
+        const K* xrow = io.x + io.xmap.at(at.x);
+        const int64_t irow = io.imap.at(at.x);
+        for (int64_t e = threadIdx.x; e < size; e += T) emit_entry<K, true>(io, xrow, nullptr, irow, static_cast<int64_t>(at.y) + e, ak[e], av[e]);
+        __syncthreads();
+    }
+}
+
 struct SplitLayout {
     int64_t chunks_per_row;
     size_t counters_off, rows_off, list_off, crowded_off, fine_off, base_off, total;
@@ -1255,7 +1667,7 @@ SplitLayout split_layout(int64_t m, int64_t n) {
     SplitLayout l;
     l.chunks_per_row = ceil_div(n, static_cast<int64_t>(kChunk));
     size_t off = 0;
-    l.counters_off = off;        // [0] rows that keep the digit passes, [1] crowded buckets, [2] listed buckets
+    l.counters_off = off;        // [1] buckets on the list of split_finish_crowded, [2] on that of split_finish
     off += 256;
     l.rows_off = off;
     off += align_up(static_cast<size_t>(m) * sizeof(SplitRow), 256);
@@ -1285,13 +1697,10 @@ size_t split_scratch_bytes(size_t key_size, bool pairs, int64_t m, int64_t n) {
     return split_layout(m, n).total;
 }
 
-// Enqueues the bucket route for every row; keys (and indices) travel through io.kbuf[0] (and
-// io.vbuf[0]).  Rows it does not take are counted in **other_rows (device memory inside
-// `scratch`) and marked in the row records at *route_records (*route_stride bytes apart, first
-// word 1 when the row was taken).
+// Enqueues the bucket route, which sorts every row of the call; keys (and indices) travel through
+// io.kbuf[0] (and io.vbuf[0]).
 template <typename K>
-int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, int64_t n, void* scratch, int poll_limit,
-              int compare_max, const LeftTables& tables, const uint32_t** other_rows, const uint32_t** route_records, size_t* route_stride) {
+int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, int64_t n, void* scratch, int compare_max) {
     const SplitLayout l = split_layout(m, n);
     char* base = static_cast<char*>(scratch);
     uint32_t* counters = reinterpret_cast<uint32_t*>(base + l.counters_off);
@@ -1300,10 +1709,6 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
     uint32_t* crowded = reinterpret_cast<uint32_t*>(base + l.crowded_off);
     uint32_t* fine = reinterpret_cast<uint32_t*>(base + l.fine_off);
     uint32_t* chunk_base = reinterpret_cast<uint32_t*>(base + l.base_off);
-    *other_rows = counters;
-    *route_records = reinterpret_cast<const uint32_t*>(rows);
-    *route_stride = sizeof(SplitRow);
-    (void)poll_limit;            // nothing waits for anything on this route
 
     const int waves = finish_waves(n, io.kind == kKeyFloat);
     const int cap = finish_cap(waves);
@@ -1328,7 +1733,7 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         split_histogram<K, decltype(map_tag)::value><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine);
     });
     DLFX_CHECK_LAUNCH();
-    split_plan<<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(n, static_cast<uint32_t>(cap), l.chunks_per_row, fine, rows, counters, tables, list, chunk_base);
+    split_plan<<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(n, static_cast<uint32_t>(cap), l.chunks_per_row, fine, rows, counters, list, crowded, chunk_base);
     DLFX_CHECK_LAUNCH();
     // split_finish: as many workgroups as the device holds at once, each walking its share of the buckets
     const int64_t buckets = m * kMaxBuckets;
@@ -1350,10 +1755,25 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         else if (block == 512) pass_of(std::integral_constant<int, 512>());
         else if constexpr (kPassBlockMax<K, PAIRS> >= 1024) pass_of(std::integral_constant<int, 1024>());
         DLFX_CHECK_LAUNCH();
+        if constexpr (PAIRS) {
+            // rows with buckets larger than a workgroup holds (as a rule none: every workgroup leaves at once)
+            const int64_t units = m * l.chunks_per_row;
+            split_pass_stable<K><<<dim3(static_cast<unsigned>(units < 1024 ? units : 1024)), dim3(kSplitBlock), 0, stream>>>(
+                io, n, l.chunks_per_row, units, rows, counters, chunk_base);
+            DLFX_CHECK_LAUNCH();
+        }
         split_finish<K, PAIRS, WAVES><<<fgrid, dim3(WAVES * kWave), 0, stream>>>(io, n, limit, counters, list, crowded);
         DLFX_CHECK_LAUNCH();
+        // (a smaller grid for this launch, which as a rule finds little to do, was measured: the
+        // same for the benchmark rows, up to 15 % slower on bell-shaped rows, whose buckets are often crowded)
         split_finish_crowded<K, PAIRS, WAVES><<<fgrid, dim3(WAVES * kWave), 0, stream>>>(io, n, rows, counters, crowded);
         DLFX_CHECK_LAUNCH();
+        if constexpr (PAIRS) {
+            if (!io.y && !io.x_intact) {       // what sort_oversized cannot take (an index-only argsort written over its input)
+                split_finish_in_place<K, WAVES><<<fgrid, dim3(WAVES * kWave), 0, stream>>>(io, n, rows, counters, crowded);
+                DLFX_CHECK_LAUNCH();
+            }
+        }
         return DLFX_OK;
     };
     using Huge = std::integral_constant<int, 16>;
@@ -1363,10 +1783,8 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
     return waves == 4 ? launch(std::false_type(), Small()) : waves == 8 ? launch(std::false_type(), Large()) : launch(std::false_type(), Huge());
 }
 
-template int run_split<uint32_t>(hipStream_t, const PassIo<uint32_t>&, bool, int64_t, int64_t, void*, int, int, const LeftTables&,
-                                 const uint32_t**, const uint32_t**, size_t*);
-template int run_split<uint64_t>(hipStream_t, const PassIo<uint64_t>&, bool, int64_t, int64_t, void*, int, int, const LeftTables&,
-                                 const uint32_t**, const uint32_t**, size_t*);
+template int run_split<uint32_t>(hipStream_t, const PassIo<uint32_t>&, bool, int64_t, int64_t, void*, int);
+template int run_split<uint64_t>(hipStream_t, const PassIo<uint64_t>&, bool, int64_t, int64_t, void*, int);
 
 }  // namespace dlfx
 

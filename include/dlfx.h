@@ -83,10 +83,13 @@ int dlfx_last_hip_error(void);
  *                      in registers; longer rows of up to 16384 elements (8-byte keys: 8192,
  *                      16-bit keys: 4096) take one workgroup.
  *   "sort_buckets"     1 (default): rows of 4-byte keys longer than 16384 elements and of 8-byte
- *                      keys longer than 8192 are cut into
- *                      buckets of equal depth by value and each bucket is sorted on chip, wherever
- *                      a row's keys allow it (each row decides on the device); 0: every row takes
- *                      the least-significant-digit-first passes.  Same results either way.
+ *                      keys longer than 8192 (up to about 2.6 million elements) are cut into
+ *                      buckets of equal depth by value and each bucket is sorted on chip; 0: every
+ *                      row takes the least-significant-digit-first passes.  Same results either
+ *                      way, but not the same scratch: the bucket route needs one pair of
+ *                      ping-pong buffers where the digit passes need two, so set this before
+ *                      dlfx_sort_scratch_bytes / dlfx_argsort_scratch_bytes / dlfx_top_k_scratch_bytes
+ *                      of the calls it is to hold for.
  *   "sort_compare_max" fullest counting bin (default 32) of a bucket whose entries are still ranked
  *                      by comparing them; fuller bins send the bucket through stable digit passes
  *                      (0: every bucket).  Same results for every value.

@@ -165,9 +165,8 @@ def test_rows_leave_out_passes_that_move_nothing(hip_backend, oracle_backend, dt
 @pytest.mark.parametrize("n", [5000, 9000, 17000, 40000, 150000, 300000, 600000, 1 << 20])
 def test_long_rows_cut_into_buckets(hip_backend, dtype, n):
     """Rows longer than one workgroup sorts are cut into buckets of equal depth by value and
-    each bucket is finished on chip; rows whose keys do not allow that (one value taking more
-    than a bucket holds, ...) take the least-significant-digit-first passes in the same call.
-    Checked against numpy's stable sort and against the same call with that route switched off."""
+    each bucket is finished on chip.  Checked against numpy's stable sort and against the
+    least-significant-digit-first passes (the same call with the bucket route switched off)."""
     if np.dtype(dtype).kind == "i":
         wide = full_range_i64(300, n).astype(dtype)                   # even leading digit
         lopsided = (full_range_i64(301, n) >> 40).astype(dtype)       # (int64) three digits vary, the top one in two values
@@ -381,10 +380,11 @@ def test_rows_beyond_a_million_keys_take_the_largest_buckets(hip_backend, dtype)
 
 
 @pytest.mark.parametrize("dtype", [np.int32, np.int64])
-def test_rows_left_to_the_digit_passes_beside_rows_on_the_bucket_route(hip_backend, dtype):
-    """Rows the bucket route does not take (one value repeated, a handful of values: a fine bin
-    larger than a workgroup holds) are sorted by the digit passes in the same call that sends
-    its other rows through the bucket route; several calls in a row over one scratch buffer."""
+def test_rows_with_oversized_buckets_beside_rows_that_cut_evenly(hip_backend, dtype):
+    """Rows that do not cut into buckets a workgroup holds (one value repeated, a handful of
+    values: a fine bin fuller than a bucket) get buckets of their own size, finished by one
+    workgroup each, in the same call that sorts its other rows the usual way; several calls in
+    a row over one scratch buffer."""
     n = 70000
     x = (full_range_i64(330, 9 * n).reshape(9, n) >> (40 if np.dtype(dtype).itemsize == 8 else 36)).astype(dtype)
     x[1, :] = 7                                   # one value
@@ -398,6 +398,78 @@ def test_rows_left_to_the_digit_passes_beside_rows_on_the_bucket_route(hip_backe
         assert np.array_equal(Ih.numpy(), order)
         assert np.array_equal(Yh.numpy(), np.take_along_axis(x, order, -1))
         assert np.array_equal(Sh.numpy(), np.sort(x, axis=-1)[:, ::-1])
+
+
+def oversized_rows(dtype, n, seed):
+    """Rows whose keys defeat cutting by value: repeated values, and distinct values packed more
+    tightly than the fine bins of the row's range resolve."""
+    dt = np.dtype(dtype)
+    if dt.kind == "i":
+        wide = full_range_i64(seed, n).astype(dtype)
+        cluster = wide.copy()                                         # nine keys in ten within 1000 of one another
+        near = randint(seed + 1, n, 0, 1000).astype(dtype) + dtype(12345)
+        pick = randint(seed + 2, n, 0, 10) > 0
+        cluster[pick] = near[pick]
+        pair = (randint(seed + 3, n, 0, 2) + 40).astype(dtype)        # two neighbouring values
+        pair[:: 97] = wide[:: 97]
+    else:
+        wide = (normal(seed, n) * 1e3).astype(dtype)
+        cluster = wide.copy()
+        eps = np.finfo(dtype).eps
+        near = (dtype(3.25) * (1 + randint(seed + 1, n, 0, 1000).astype(dtype) * eps)).astype(dtype)
+        pick = randint(seed + 2, n, 0, 10) > 0
+        cluster[pick] = near[pick]
+        pair = np.where(randint(seed + 3, n, 0, 2) > 0, dtype(0.0), dtype(-0.0)).astype(dtype)       # the two zeros: one key for a stable argsort
+        pair[:: 97] = wide[:: 97]
+    constant = np.full(n, wide[0], dtype=dtype)
+    few = wide[randint(seed + 4, n, 0, 5)]                            # five values
+    many = np.sort(wide[:300])[randint(seed + 5, n, 0, 300)]          # 300 values: more heavy bins than buckets
+    half = wide.copy()
+    half[randint(seed + 6, n, 0, 2) > 0] = wide[1]
+    return np.stack([constant, cluster, few, wide, pair, many, half])
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.int64, np.float32, np.float64])
+@pytest.mark.parametrize("n", [20000, 70000, 300000, 1 << 20])
+def test_buckets_larger_than_a_workgroup_holds(hip_backend, dtype, n):
+    x = oversized_rows(dtype, n, 340)
+    Xh = Tensor.from_numpy(hip_backend, x)
+    want = np.sort(x, axis=-1, kind="stable")
+    for desc in (False, True):
+        key = -x if (desc and np.dtype(dtype).kind == "f") else x
+        order = np.argsort(key, axis=-1, kind="stable") if not desc or np.dtype(dtype).kind == "f" else np.argsort(~x, axis=-1, kind="stable")
+        got = F.sort(Xh, -1, desc).numpy()
+        ref = want[:, ::-1] if desc else want
+        assert np.array_equal(got, ref), desc                              # (== : the two zeros are one value)
+        Ih = F.argsort(Xh, -1, desc)                                       # indices alone: keys of the far side come from the input
+        assert np.array_equal(Ih.numpy(), order), desc
+        Yh, I64 = F.argsort(Xh, -1, desc, with_values=True, index_dtype=np.int64)
+        assert np.array_equal(I64.numpy(), order), desc
+        assert np.array_equal(Yh.numpy().view(np.uint8), np.take_along_axis(x, order, -1).view(np.uint8)), desc
+    # in place, and onto a transposed destination
+    Zh = Tensor.from_numpy(hip_backend, x)
+    F.sort(Zh, -1, out=Zh)
+    assert np.array_equal(Zh.numpy(), want)
+    xp = x + dtype(0) if np.dtype(dtype).kind == "f" else x               # (-0.0 + 0.0 = +0.0: written over the input, the two zeros order by sign)
+    Zh = Tensor.from_numpy(hip_backend, xp)
+    Yh, Ih = F.argsort(Zh, -1, values=Zh)
+    assert np.array_equal(Ih.numpy(), np.argsort(xp, axis=-1, kind="stable"))
+    assert np.array_equal(Yh.numpy(), want)
+    Th = Tensor.from_numpy(hip_backend, np.zeros((n, x.shape[0]), dtype=dtype)).transpose([1, 0])
+    F.sort(Xh, -1, out=Th)
+    assert np.array_equal(np.ascontiguousarray(Th.numpy()), want)
+
+
+@pytest.mark.parametrize("n", [70000, 300000])
+def test_index_only_argsort_written_over_its_input(hip_backend, n):
+    # argsort(X, X) of int32 (UniformTest.cpp:2461-2466 does this with short rows): there is no value
+    # output and the input is gone once indices are written, so an oversized bucket of several
+    # values is sorted where it lies
+    from dlf_amd.frontend import dtype_code
+    x = oversized_rows(np.int32, n, 350)
+    Xh = Tensor.from_numpy(hip_backend, x)
+    hip_backend.argsort(0, dtype_code(np.int32), dtype_code(np.int32), Xh.shape, Xh.storage, None, None, Xh.shape, Xh.storage)
+    assert np.array_equal(Xh.numpy(), np.argsort(x, axis=-1, kind="stable"))
 
 
 @pytest.mark.parametrize("dtype", [np.int64, np.float64])
