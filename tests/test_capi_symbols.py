@@ -49,7 +49,12 @@ def test_host_only_calls():
     assert lib.dlfx_softmax_scratch_bytes(0, 256, 262144) == 0
     assert lib.dlfx_softmax_scratch_bytes(2, 8, 262144) > 0            # hardmax of int32
     assert lib.dlfx_softmax_scratch_bytes(5, 8, 262144) == 0           # no int16 softmax family
-    assert lib.dlfx_sort_scratch_bytes(3, 256, 1 << 20) >= 2 * 256 * (1 << 20) * 8
+    # long rows on the bucket route: one pair of ping-pong buffers (with indices: at most 1.6 x the input)
+    keys = 256 * (1 << 20) * 8
+    assert keys <= lib.dlfx_sort_scratch_bytes(3, 256, 1 << 20) < int(1.1 * keys)
+    assert keys + keys // 2 <= lib.dlfx_argsort_scratch_bytes(3, 256, 1 << 20) <= int(1.6 * keys)
+    # 16-bit keys keep the digit passes and both pairs
+    assert lib.dlfx_sort_scratch_bytes(5, 64, 1 << 16) >= 2 * 64 * (1 << 16) * 2
     assert lib.dlfx_set_tuning(b"no_such_knob", 1) == -3
     assert lib.dlfx_set_tuning(b"scan_poll_limit", 2048) == 0
     for knob, value in ((b"sort_poll_limit", 2048), (b"sort_wave_rows", 512), (b"sort_buckets", 1), (b"sort_compare_max", 32), (b"topk_thread_rows", 256)):
