@@ -101,6 +101,7 @@ inline int finish_waves(int64_t n, bool floats) {
     return n <= kSmallCapRows ? 4 : n <= (floats ? kLargeCapFloatRows : kLargeCapRows) ? 8 : 16;
 }
 constexpr int kNear = 2;                              // entries of a bin compared without a loop
+constexpr int64_t kFrontRows = 512;                   // fewest rows of a call that split_front takes (two a compute unit)
 
 // What split_sample and split_plan decide for a row.
 struct alignas(16) SplitRow {
@@ -139,7 +140,8 @@ struct FineMap {
     F lo, scale;
     uint32_t shift, by_value;
     int descending;
-    __device__ FineMap(const SplitRow& r, int desc)
+    template <typename Row>                // a SplitRow, or the FineRange that goes into one
+    __device__ FineMap(const Row& r, int desc)
         : base(static_cast<K>(r.base)), top(static_cast<K>(r.top)), gap_lo(static_cast<K>(r.gap_lo)), gap_hi(static_cast<K>(r.gap_hi)),
           less(static_cast<K>(K(0) - static_cast<K>(r.gap_hi) - static_cast<K>(r.base))),
           lo(bit_cast<F>(static_cast<K>(r.lo_bits))), scale(bit_cast<F>(static_cast<K>(r.scale_bits))), shift(r.shift),
@@ -237,21 +239,40 @@ __device__ __forceinline__ K wave_fourth(const K (&key)[4]) {
 // MAP leaves out.
 constexpr int kMapPlain = 0, kMapGap = 1, kMapValue = 2;
 
-template <typename K, int MAP>
-__global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_t n, uint32_t cap, SplitRow* __restrict__ rows, uint32_t* __restrict__ counters) {
-    __shared__ K red[kSplitBlock / kWave];
-    const int64_t row = blockIdx.x;
-    if (row == 0 && threadIdx.x < 4) counters[threadIdx.x] = 0u;      // what the later launches of this sort count up from
-    const K* xrow = io.x + io.xmap.at(row);
+// How a row's keys spread over its fine bins (the part of SplitRow that split_sample decides).
+struct FineRange {
+    uint32_t shift, by_value;
+    unsigned long long base, top, lo_bits, scale_bits, gap_lo, gap_hi;
+    __device__ __forceinline__ void store(SplitRow& out) const {
+        out.shift = shift;
+        out.base = base;
+        out.by_value = by_value;
+        out.gap_lo = gap_lo;
+        out.gap_hi = gap_hi;
+        out.top = top;
+        out.lo_bits = lo_bits;
+        out.scale_bits = scale_bits;
+    }
+};
+
+// The sample of row `xrow` and what it says, worked out by a workgroup of BLOCK threads (every
+// thread returns the same answer).  The sample is that of 256 threads whatever BLOCK is: further
+// wavefronts repeat the first four, which changes no minimum or maximum, and the lists of what
+// every wavefront offers are those of the first four.
+template <typename K, int MAP, int BLOCK>
+__device__ __forceinline__ FineRange sample_row(const PassIo<K>& io, const K* __restrict__ xrow, int64_t n, uint32_t cap) {
+    static_assert(BLOCK % kSplitBlock == 0 && (MAP != kMapValue || BLOCK == kSplitBlock), "whole repeats of the sampling threads");
+    __shared__ K red[BLOCK / kWave];
+    const int st = threadIdx.x % kSplitBlock;          // the sampling thread this one is (or repeats)
     // 1024 keys: four neighbours (one memory line when the row is contiguous) at each of 256
     // evenly spaced places, the last of them the row's last keys, so that a sorted row shows
     // its whole range
     K key[4];
-    int64_t e0 = (static_cast<int64_t>(threadIdx.x) * n) / kSplitBlock;
-    if (threadIdx.x == kSplitBlock - 1 || e0 > n - 4) e0 = n - 4;
+    int64_t e0 = (static_cast<int64_t>(st) * n) / kSplitBlock;
+    if (st == kSplitBlock - 1 || e0 > n - 4) e0 = n - 4;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-        const int64_t j = static_cast<int64_t>(threadIdx.x) * 4 + u;
+        const int64_t j = static_cast<int64_t>(st) * 4 + u;
         const int64_t e = n >= 1024 ? e0 + u : (j < n ? j : n - 1);
         key[u] = key_of_element<K>(io, xrow[e * io.sx]);
     }
@@ -268,8 +289,8 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
         lo = wave_fourth<true>(key);
         hi = wave_fourth<false>(key);
     }
-    lo = block_reduce(lo, smaller, red, kSplitBlock / kWave);
-    hi = block_reduce(hi, larger, red, kSplitBlock / kWave);
+    lo = block_reduce(lo, smaller, red, BLOCK / kWave);
+    hi = block_reduce(hi, larger, red, BLOCK / kWave);
     // Float rows: the images of negative and of positive values lie either side of the middle
     // of the key range, those of the smallest magnitudes next to it and the two zeros at it.
     // Every wave offers the nearest of its keys below the zeros and the nearest above them; the
@@ -286,7 +307,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
         }
         __shared__ K near[2][kSplitBlock / kWave];
         const K wave_under = wave_reduce(under_mine, larger), wave_over = wave_reduce(over_mine, smaller);
-        if (lane_id() == 0) {
+        if (lane_id() == 0 && threadIdx.x < kSplitBlock) {
             near[0][threadIdx.x / kWave] = wave_under;
             near[1][threadIdx.x / kWave] = wave_over;
         }
@@ -307,7 +328,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
     }
     // that range takes the middle half of the fine bins; a quarter on either side is left for
     // keys outside it (beyond those, keys share the first or last bin)
-    SplitRow map;
+    FineRange map;
     {
         map.gap_lo = static_cast<unsigned long long>(gap_lo);
         map.gap_hi = static_cast<unsigned long long>(gap_hi);
@@ -331,7 +352,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
         const F w = xh - xl;
         const F first = xl - w * F(0.5), last = xh + w * F(0.5);
         if (w > F(0) && w - w == F(0) && first - first == F(0) && last - last == F(0)) {       // all finite
-            SplitRow by_value = map;
+            FineRange by_value = map;
             by_value.by_value = 1u;
             by_value.lo_bits = static_cast<unsigned long long>(bit_cast<K>(first));
             by_value.scale_bits = static_cast<unsigned long long>(bit_cast<K>(static_cast<F>(kFine) / (w * F(2))));
@@ -356,17 +377,17 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
             if (worst_value < worst_image && static_cast<unsigned long long>(worst_image) * static_cast<unsigned long long>(n) > static_cast<unsigned long long>(cap) * kFine) map = by_value;
         }
     }
+    return map;
+}
+
+template <typename K, int MAP>
+__global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_t n, uint32_t cap, SplitRow* __restrict__ rows, uint32_t* __restrict__ counters) {
+    const int64_t row = blockIdx.x;
+    if (row == 0 && threadIdx.x < 4) counters[threadIdx.x] = 0u;      // what the later launches of this sort count up from
+    const FineRange map = sample_row<K, MAP, kSplitBlock>(io, io.x + io.xmap.at(row), n, cap);
     if (threadIdx.x == 0) {
-        SplitRow& out = rows[row];
-        out.route = 0u;
-        out.shift = map.shift;
-        out.base = map.base;
-        out.by_value = map.by_value;
-        out.gap_lo = map.gap_lo;
-        out.gap_hi = map.gap_hi;
-        out.top = map.top;
-        out.lo_bits = map.lo_bits;
-        out.scale_bits = map.scale_bits;
+        rows[row].route = 0u;
+        map.store(rows[row]);
     }
 }
 
@@ -375,22 +396,15 @@ __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_
 // counts a word (a count is at most kChunk).  split_plan adds the chunks up for the row's
 // histogram and turns each chunk's into its keys per bucket, so that split_pass needs no
 // communication between workgroups.
-template <typename K, int MAP>
-__global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int64_t n, int64_t chunks_per_row,
-                                                               const SplitRow* __restrict__ rows, uint32_t* __restrict__ chunk_fine) {
+// Elements [lo, hi) of a row counted into hist[kFine] (LDS, which the caller has cleared) by a
+// workgroup of BLOCK threads.  STREAM: the elements are not read again soon (non-temporal loads).
+template <typename K, int MAP, int BLOCK, bool STREAM>
+__device__ __forceinline__ void count_fine_bins(const PassIo<K>& io, const K* __restrict__ xrow, int64_t lo, int64_t hi,
+                                                const FineMap<K>& fine_of, uint32_t* __restrict__ hist) {
     constexpr int U = 32 / sizeof(K);                 // keys per thread and batch (64 bytes measured: no faster)
-    __shared__ uint32_t hist[kFine];
-    for (int i = threadIdx.x; i < kFine; i += kSplitBlock) hist[i] = 0;
-    __syncthreads();
-    const int64_t row = blockIdx.x / chunks_per_row;
-    const int64_t c = blockIdx.x - row * chunks_per_row;
-    const K* xrow = io.x + io.xmap.at(row);
-    const FineMap<K> fine_of(rows[row], io.descending);
-    const int64_t lo = c * kChunk;
-    const int64_t hi = (lo + kChunk < n) ? lo + kChunk : n;
-    // batches of 256 x U keys; the next batch's keys are on their way while this one is counted
-    // (no branches in the loads: a key beyond the chunk's end reads the chunk's first key and is never counted)
-    constexpr int64_t BATCH = static_cast<int64_t>(kSplitBlock) * U;
+    // batches of BLOCK x U keys; the next batch's keys are on their way while this one is counted
+    // (no branches in the loads: a key beyond the range's end reads its first key and is never counted)
+    constexpr int64_t BATCH = static_cast<int64_t>(BLOCK) * U;
     // (whole batches of a contiguous, aligned row move as 16-byte accesses: which thread counts
     // which key does not matter here)
     constexpr int VK = 16 / sizeof(K);
@@ -401,7 +415,9 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
             const VecK* src = reinterpret_cast<const VecK*>(xrow + b0);
 #pragma unroll
             for (int v = 0; v < U / VK; ++v) {
-                const VecK a = load_stream(&src[threadIdx.x + v * kSplitBlock]);      // (non-temporal: 71 -> 50 us on [1024, 65536] fp32)
+                VecK a;
+                if constexpr (STREAM) a = load_stream(&src[threadIdx.x + v * BLOCK]);      // (non-temporal: 71 -> 50 us on [1024, 65536] fp32)
+                else a = src[threadIdx.x + v * BLOCK];
 #pragma unroll
                 for (int e = 0; e < VK; ++e) key[v * VK + e] = a.v[e];
             }
@@ -409,7 +425,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int64_t i = b0 + threadIdx.x + static_cast<int64_t>(u) * kSplitBlock;
+            const int64_t i = b0 + threadIdx.x + static_cast<int64_t>(u) * BLOCK;
             key[u] = xrow[(i < hi ? i : lo) * io.sx];
         }
     };
@@ -435,7 +451,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
         } else {
 #pragma unroll
             for (int u = 0; u < U; ++u)
-                if (full || b0 + threadIdx.x + static_cast<int64_t>(u) * kSplitBlock < hi) atomicAdd(&hist[f[u]], 1u);
+                if (full || b0 + threadIdx.x + static_cast<int64_t>(u) * BLOCK < hi) atomicAdd(&hist[f[u]], 1u);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) key[u] = ahead[u];
@@ -443,6 +459,21 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
     };
     if (MAP == kMapValue && fine_of.by_value) count_chunk(std::integral_constant<bool, MAP == kMapValue>());
     else count_chunk(std::false_type());
+}
+
+template <typename K, int MAP>
+__global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int64_t n, int64_t chunks_per_row,
+                                                               const SplitRow* __restrict__ rows, uint32_t* __restrict__ chunk_fine) {
+    __shared__ uint32_t hist[kFine];
+    for (int i = threadIdx.x; i < kFine; i += kSplitBlock) hist[i] = 0;
+    __syncthreads();
+    const int64_t row = blockIdx.x / chunks_per_row;
+    const int64_t c = blockIdx.x - row * chunks_per_row;
+    const K* xrow = io.x + io.xmap.at(row);
+    const FineMap<K> fine_of(rows[row], io.descending);
+    const int64_t lo = c * kChunk;
+    const int64_t hi = (lo + kChunk < n) ? lo + kChunk : n;
+    count_fine_bins<K, MAP, kSplitBlock, true>(io, xrow, lo, hi, fine_of, hist);
     __syncthreads();
     uint32_t* g = chunk_fine + static_cast<int64_t>(blockIdx.x) * (kFine / 2);
     for (int i = threadIdx.x; i < kFine / 2; i += kSplitBlock) g[i] = hist[2 * i] | (hist[2 * i + 1] << 16);
@@ -457,71 +488,55 @@ __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int
 // bins resolve) has buckets that are larger: those go on the list split_finish_crowded walks
 // (counters[1] entries) and the row is marked route 2, which for pairs makes split_pass_stable
 // move it, so that every bucket of the row arrives in index order.
-__global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t cap, int64_t chunks_per_row, const uint32_t* __restrict__ chunk_fine,
-                                                          SplitRow* __restrict__ rows, uint32_t* __restrict__ counters,
-                                                          uint4* __restrict__ bucket_list, uint32_t* __restrict__ crowded_list,
-                                                          uint32_t* __restrict__ chunk_base) {
+template <int BLOCK>
+struct PlanShared {
+    uint32_t red[BLOCK / kWave];
+    uint32_t listed[2][kSplitBlock / kWave + 1];      // buckets of this row for either list by wavefront, and where they go
+    uint32_t last_count[kSplitBlock];                 // every planning thread's last fine bin
+    uint32_t last_bucket[kSplitBlock];
+    uint32_t begin[kMaxBuckets + 1];
+};
+
+// The buckets of row `row` from its fine-bin counts: planning thread t (the first 256 threads of
+// a workgroup of BLOCK) brings the counts of fine bins [16 t, 16 t + 16) in cnt[] and receives
+// their buckets in bucket[]; the other threads bring zeros and only keep the barriers company.
+// The row's record, its table and its buckets' places (also sm.begin) are written, the buckets
+// listed.  Returns the number of buckets.
+template <int BLOCK>
+__device__ __forceinline__ uint32_t plan_buckets(PlanShared<BLOCK>& sm, const uint32_t (&cnt)[kFine / kSplitBlock], uint32_t (&bucket)[kFine / kSplitBlock],
+                                                 int64_t n, uint32_t cap, int64_t row, SplitRow& info, uint32_t* __restrict__ counters,
+                                                 uint4* __restrict__ bucket_list, uint32_t* __restrict__ crowded_list, uint32_t* route_out = nullptr) {
     constexpr int PER = kFine / kSplitBlock;          // 16
-    constexpr int WAVES = kSplitBlock / kWave;
-    __shared__ uint32_t red[WAVES];
-    __shared__ uint32_t listed[2][WAVES + 1];         // buckets of this row for either list by wavefront, and where they go
-    __shared__ uint32_t per_bucket[kMaxBuckets];
-    __shared__ uint32_t last_count[kSplitBlock];      // every thread's last fine bin
-    const int64_t row = blockIdx.x;
+    constexpr int WAVES = BLOCK / kWave;
     const int w = threadIdx.x / kWave;
-    const uint32_t* f = chunk_fine + row * chunks_per_row * (kFine / 2) + threadIdx.x * (PER / 2);
-    SplitRow& info = rows[row];
-    uint32_t cnt[PER];
-#pragma unroll
-    for (int i = 0; i < PER; ++i) cnt[i] = 0;
-    auto chunk_words = [&](int64_t c, uint32_t (&w)[PER / 2]) __attribute__((always_inline)) {
-        const uint4 a = reinterpret_cast<const uint4*>(f + c * (kFine / 2))[0], b = reinterpret_cast<const uint4*>(f + c * (kFine / 2))[1];
-        w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w; w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w;
-    };
-    for (int64_t c0 = 0; c0 < chunks_per_row; c0 += 4) {             // four chunks' loads in flight
-        uint32_t w[4][PER / 2];
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (c0 + j < chunks_per_row) chunk_words(c0 + j, w[j]);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            if (c0 + j >= chunks_per_row) break;
-#pragma unroll
-            for (int i = 0; i < PER / 2; ++i) {
-                cnt[2 * i] += w[j][i] & 0xffffu;
-                cnt[2 * i + 1] += w[j][i] >> 16;
-            }
-        }
-    }
+    const bool planner = threadIdx.x < kSplitBlock;
     uint32_t sum = 0, biggest = 0;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
         sum += cnt[i];
         biggest = cnt[i] > biggest ? cnt[i] : biggest;
     }
-    last_count[threadIdx.x] = cnt[PER - 1];
-    biggest = block_reduce(biggest, [](uint32_t a, uint32_t b) { return a > b ? a : b; }, red, WAVES);
+    if (planner) sm.last_count[threadIdx.x] = cnt[PER - 1];
+    biggest = block_reduce(biggest, [](uint32_t a, uint32_t b) { return a > b ? a : b; }, sm.red, WAVES);
     // exclusive prefix of the thread sums
     const uint32_t incl = wave_scan_inclusive(sum, 0u, [](uint32_t a, uint32_t b) { return a + b; });
     __syncthreads();
-    if (lane_id() == kWave - 1) red[w] = incl;
+    if (lane_id() == kWave - 1) sm.red[w] = incl;
     __syncthreads();
     uint32_t before = incl - sum;
-    for (int i = 0; i < w; ++i) before += red[i];
+    for (int i = 0; i < w; ++i) before += sm.red[i];
 
     // A bin goes to bucket (keys before it) / target plus the cuts at or before it: bit i of
     // `cut_at` makes bin i of this thread open a new bucket whatever the count says.  Returns
     // the number of buckets.
-    uint32_t bucket[PER];
-    __shared__ uint32_t last_bucket[kSplitBlock];
     auto assign = [&](uint32_t target, uint32_t cut_at) __attribute__((always_inline)) -> uint32_t {
         const uint32_t cuts = static_cast<uint32_t>(__popc(cut_at));
         const uint32_t cuts_incl = wave_scan_inclusive(cuts, 0u, [](uint32_t a, uint32_t b) { return a + b; });
         __syncthreads();
-        if (lane_id() == kWave - 1) red[w] = cuts_incl;
+        if (lane_id() == kWave - 1) sm.red[w] = cuts_incl;
         __syncthreads();
         uint32_t extra = cuts_incl - cuts;
-        for (int i = 0; i < w; ++i) extra += red[i];
+        for (int i = 0; i < w; ++i) extra += sm.red[i];
         uint32_t run = before;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
@@ -529,9 +544,9 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
             bucket[i] = run / target + extra;
             run += cnt[i];
         }
-        last_bucket[threadIdx.x] = bucket[PER - 1];
+        if (planner) sm.last_bucket[threadIdx.x] = bucket[PER - 1];
         __syncthreads();
-        return last_bucket[kSplitBlock - 1] + 1;
+        return sm.last_bucket[kSplitBlock - 1] + 1;
     };
 
     // Where at least kGapBins empty bins lie between two populated ones a new bucket starts
@@ -547,11 +562,11 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
             if (cnt[i]) last = static_cast<int>(threadIdx.x) * PER + i;
         int seen = wave_scan_inclusive(last, -1, [](int a, int b) { return a > b ? a : b; });
         __syncthreads();
-        if (lane_id() == kWave - 1) red[w] = static_cast<uint32_t>(seen);
+        if (lane_id() == kWave - 1) sm.red[w] = static_cast<uint32_t>(seen);
         __syncthreads();
         int prev = __shfl_up(seen, 1, kWave);          // last populated bin before this thread's first
         if (lane_id() == 0) prev = -1;
-        for (int i = 0; i < w; ++i) prev = static_cast<int>(red[i]) > prev ? static_cast<int>(red[i]) : prev;
+        for (int i = 0; i < w; ++i) prev = static_cast<int>(sm.red[i]) > prev ? static_cast<int>(sm.red[i]) : prev;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
             const int bin = static_cast<int>(threadIdx.x) * PER + i;
@@ -578,12 +593,13 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
         route = 2u;
         const uint32_t heavy = cap / 4;
         uint32_t heavy_cuts = 0;
-        uint32_t prev = threadIdx.x == 0 ? 0u : last_count[threadIdx.x - 1];
+        uint32_t prev = (planner && threadIdx.x != 0) ? sm.last_count[threadIdx.x - 1] : 0u;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
             if (cnt[i] >= heavy || prev >= heavy) heavy_cuts |= 1u << i;
             prev = cnt[i];
         }
+        if (!planner) heavy_cuts = 0u;
         const uint32_t by_count = static_cast<uint32_t>((n + 223) / 224);
         const uint32_t target = cap - heavy > by_count ? cap - heavy : by_count;
         n_buckets = assign(target, heavy_cuts);
@@ -591,10 +607,9 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
     }
     // a bin opens every bucket after its predecessor's up to its own (the starts are put together
     // in LDS: the threads read one another's just below)
-    __shared__ uint32_t begin[kMaxBuckets + 1];
-    {
-        uint32_t prev_bucket = threadIdx.x == 0 ? 0u : last_bucket[threadIdx.x - 1];
-        if (threadIdx.x == 0) begin[0] = 0u;
+    if (planner) {
+        uint32_t prev_bucket = threadIdx.x == 0 ? 0u : sm.last_bucket[threadIdx.x - 1];
+        if (threadIdx.x == 0) sm.begin[0] = 0u;
         uint32_t run = before;
         uint32_t packed[PER / 4];                     // this thread's 16 table bytes: one store
 #pragma unroll
@@ -602,55 +617,91 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
             packed[i / 4] |= bucket[i] << (8 * (i % 4));
-            for (uint32_t k = prev_bucket + 1; k <= bucket[i]; ++k) begin[k] = run;
+            for (uint32_t k = prev_bucket + 1; k <= bucket[i]; ++k) sm.begin[k] = run;
             prev_bucket = bucket[i];
             run += cnt[i];
         }
         static_assert(PER == 16 && offsetof(SplitRow, bucket_of) % 16 == 0, "a thread's bins are one aligned 16-byte piece of the table");
         reinterpret_cast<uint4*>(info.bucket_of)[threadIdx.x] = make_uint4(packed[0], packed[1], packed[2], packed[3]);
     }
+    if (route_out) *route_out = route;
     if (threadIdx.x == kSplitBlock - 1) {
         info.n_buckets = n_buckets;
-        begin[n_buckets] = static_cast<uint32_t>(n);
+        sm.begin[n_buckets] = static_cast<uint32_t>(n);
         info.route = route;
         if (route == 2u) atomicAdd(&counters[3], 1u);      // split_pass_stable has something to do
     }
-    per_bucket[threadIdx.x] = 0u;
     __syncthreads();
-    for (uint32_t k = threadIdx.x; k <= n_buckets; k += kSplitBlock) info.begin[k] = begin[k];
+    for (uint32_t k = threadIdx.x; k <= n_buckets; k += BLOCK) info.begin[k] = sm.begin[k];
     // The buckets that hold anything, in no particular order, on the list of the kernel that
     // finishes them: split_finish those that fit its workgroup, split_finish_crowded the others.
-    uint32_t next = 0;                                 // where the coming chunk's keys of bucket threadIdx.x go
     {
         uint32_t b0 = 0, size = 0;
         if (threadIdx.x < n_buckets) {
-            b0 = begin[threadIdx.x];
-            size = begin[threadIdx.x + 1] - b0;
-            next = b0;
+            b0 = sm.begin[threadIdx.x];
+            size = sm.begin[threadIdx.x + 1] - b0;
         }
         const bool fits_finish = size != 0u && size <= cap, oversized = size > cap;
         const unsigned long long fit_lanes = __ballot(fits_finish), over_lanes = __ballot(oversized);
-        if (lane_id() == 0) {
-            listed[0][w] = static_cast<uint32_t>(__popcll(fit_lanes));
-            listed[1][w] = static_cast<uint32_t>(__popcll(over_lanes));
+        if (lane_id() == 0 && planner) {
+            sm.listed[0][w] = static_cast<uint32_t>(__popcll(fit_lanes));
+            sm.listed[1][w] = static_cast<uint32_t>(__popcll(over_lanes));
         }
         __syncthreads();
         if (threadIdx.x < 2) {
             uint32_t total = 0;
-            for (int i = 0; i < WAVES; ++i) {
-                const uint32_t c = listed[threadIdx.x][i];
-                listed[threadIdx.x][i] = total;
+            for (int i = 0; i < kSplitBlock / kWave; ++i) {
+                const uint32_t c = sm.listed[threadIdx.x][i];
+                sm.listed[threadIdx.x][i] = total;
                 total += c;
             }
-            listed[threadIdx.x][WAVES] = total ? atomicAdd(&counters[threadIdx.x == 0 ? 2 : 1], total) : 0u;
+            sm.listed[threadIdx.x][kSplitBlock / kWave] = total ? atomicAdd(&counters[threadIdx.x == 0 ? 2 : 1], total) : 0u;
         }
         __syncthreads();
         const unsigned long long below = (1ull << lane_id()) - 1ull;
         const uint32_t id = static_cast<uint32_t>(row) * kMaxBuckets + threadIdx.x;
         if (fits_finish)
-            bucket_list[listed[0][WAVES] + listed[0][w] + static_cast<uint32_t>(__popcll(fit_lanes & below))] = make_uint4(static_cast<uint32_t>(row), b0, size, id);
-        if (oversized) crowded_list[listed[1][WAVES] + listed[1][w] + static_cast<uint32_t>(__popcll(over_lanes & below))] = id;
+            bucket_list[sm.listed[0][kSplitBlock / kWave] + sm.listed[0][w] + static_cast<uint32_t>(__popcll(fit_lanes & below))] = make_uint4(static_cast<uint32_t>(row), b0, size, id);
+        if (oversized) crowded_list[sm.listed[1][kSplitBlock / kWave] + sm.listed[1][w] + static_cast<uint32_t>(__popcll(over_lanes & below))] = id;
     }
+    return n_buckets;
+}
+
+__global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t cap, int64_t chunks_per_row, const uint32_t* __restrict__ chunk_fine,
+                                                          SplitRow* __restrict__ rows, uint32_t* __restrict__ counters,
+                                                          uint4* __restrict__ bucket_list, uint32_t* __restrict__ crowded_list,
+                                                          uint32_t* __restrict__ chunk_base) {
+    constexpr int PER = kFine / kSplitBlock;          // 16
+    __shared__ PlanShared<kSplitBlock> sm;
+    __shared__ uint32_t per_bucket[kMaxBuckets];
+    const int64_t row = blockIdx.x;
+    const uint32_t* f = chunk_fine + row * chunks_per_row * (kFine / 2) + threadIdx.x * (PER / 2);
+    uint32_t cnt[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) cnt[i] = 0;
+    auto chunk_words = [&](int64_t c, uint32_t (&w)[PER / 2]) __attribute__((always_inline)) {
+        const uint4 a = reinterpret_cast<const uint4*>(f + c * (kFine / 2))[0], b = reinterpret_cast<const uint4*>(f + c * (kFine / 2))[1];
+        w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w; w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w;
+    };
+    for (int64_t c0 = 0; c0 < chunks_per_row; c0 += 4) {             // four chunks' loads in flight
+        uint32_t w[4][PER / 2];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (c0 + j < chunks_per_row) chunk_words(c0 + j, w[j]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (c0 + j >= chunks_per_row) break;
+#pragma unroll
+            for (int i = 0; i < PER / 2; ++i) {
+                cnt[2 * i] += w[j][i] & 0xffffu;
+                cnt[2 * i + 1] += w[j][i] >> 16;
+            }
+        }
+    }
+    uint32_t bucket[PER];
+    per_bucket[threadIdx.x] = 0u;
+    const uint32_t n_buckets = plan_buckets<kSplitBlock>(sm, cnt, bucket, n, cap, row, rows[row], counters, bucket_list, crowded_list);
+    uint32_t next = threadIdx.x < n_buckets ? sm.begin[threadIdx.x] : 0u;      // where the coming chunk's keys of bucket threadIdx.x go
     // each chunk's keys per bucket, and from them where the chunk writes each bucket
     uint32_t w8[PER / 2], ahead[PER / 2];
     chunk_words(0, w8);
@@ -693,32 +744,24 @@ struct SplitShared {
     uint32_t vals[PAIRS && !kPassInTurn<K, PAIRS, BLOCK> ? BLOCK * kSplitItems : 1];
 };
 
-// One workgroup per chunk (kChunk keys, tiles of 4096): where the chunk's keys of each bucket
-// go is known (chunk_base), so the workgroup carries the running positions itself from tile to
-// tile and nothing passes between workgroups.  A tile's keys find their bucket (table in LDS)
+// A workgroup moves a range of a row (split_pass: a chunk of kChunk keys) in tiles of BLOCK x 16
+// keys: where the range's keys of each bucket go is known (chunk_base), so the workgroup carries
+// the running positions itself from tile to tile and nothing passes between workgroups.  A tile's keys find their bucket (table in LDS)
 // and their slot among the tile's keys of that bucket with one LDS atomic each, the tile is laid
 // out by bucket in LDS and written as runs; once it lies in LDS the registers already receive
 // the next tile's keys.  The order inside a run is whatever the atomics gave.
-template <typename K, bool PAIRS, int BLOCK, int MAP>
-__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void split_pass(PassIo<K> io, int64_t n, int64_t chunks_per_row,
-                                                          const SplitRow* __restrict__ infos, const uint32_t* __restrict__ chunk_base) {
+template <typename K, bool PAIRS, int BLOCK, int MAP, bool STREAM>
+__device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK>& sm, const PassIo<K>& io, int64_t n, int64_t row, const SplitRow& info,
+                                                   int64_t chunk_lo, int64_t chunk_hi, const uint32_t* __restrict__ places) {
     constexpr int ITEMS = kSplitItems;
     constexpr int TILE = BLOCK * kSplitItems;
     constexpr bool IN_TURN = kPassInTurn<K, PAIRS, BLOCK>;
-    static_assert(kChunk % TILE == 0, "whole tiles a chunk");
-    __shared__ SplitShared<K, PAIRS, BLOCK> sm;
     const int tid = threadIdx.x;
     const int lane = lane_id();
     const int w = tid / kWave;
-    const int64_t row = blockIdx.x / chunks_per_row;
-    const int64_t c = blockIdx.x - row * chunks_per_row;
-    const SplitRow& info = infos[row];
-    if (PAIRS && info.route != 1u) return;             // (a row with buckets larger than a workgroup holds: split_pass_stable)
     const FineMap<K> fine_of(info, io.descending);
     const K* xrow = io.x + io.xmap.at(row);
     const int64_t row_off = row * n;
-    const int64_t chunk_lo = c * kChunk;
-    const int64_t chunk_hi = (chunk_lo + kChunk < n) ? chunk_lo + kChunk : n;
 
     // (no branches: an element beyond the chunk's end reads the tile's first element instead and is never used)
     auto load_tile = [&](int64_t tile_base, K (&key)[ITEMS]) __attribute__((always_inline)) {
@@ -728,8 +771,8 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
         for (int k = 0; k < ITEMS; ++k) {
             const int e = tid + k * BLOCK;
             const K* at = &src[static_cast<int64_t>(e < valid ? e : 0) * io.sx];
-            if constexpr (sizeof(K) == 4) key[k] = load_stream(at);       // (non-temporal loads measured: a gain for 4-byte keys,
-            else key[k] = *at;                                            // a loss of 7 % for 8-byte keys)
+            if constexpr (sizeof(K) == 4 && STREAM) key[k] = load_stream(at);       // (non-temporal loads measured: a gain for 4-byte keys,
+            else key[k] = *at;                                                      // a loss of 7 % for 8-byte keys)
         }
     };
 
@@ -741,7 +784,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
     if (owner) {
         reinterpret_cast<uint4*>(sm.table)[tid] = reinterpret_cast<const uint4*>(info.bucket_of)[tid];
         sm.hist[tid] = 0u;
-        next = chunk_base[static_cast<int64_t>(blockIdx.x) * kMaxBuckets + tid];
+        next = places[tid];
     }
     __syncthreads();
 
@@ -867,6 +910,63 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
     else move_chunk(std::false_type());
 }
 
+// One workgroup per chunk (kChunk keys): elements [chunk_lo, chunk_hi) of row `row` go to their
+// buckets, places[b] being the row position of the first of them that belongs to bucket b.
+template <typename K, bool PAIRS, int BLOCK, int MAP>
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void split_pass(PassIo<K> io, int64_t n, int64_t chunks_per_row,
+                                                          const SplitRow* __restrict__ infos, const uint32_t* __restrict__ chunk_base) {
+    static_assert(kChunk % (BLOCK * kSplitItems) == 0, "whole tiles a chunk");
+    __shared__ SplitShared<K, PAIRS, BLOCK> sm;
+    const int64_t row = blockIdx.x / chunks_per_row;
+    const int64_t c = blockIdx.x - row * chunks_per_row;
+    const SplitRow& info = infos[row];
+    if (PAIRS && info.route != 1u) return;             // (a row with buckets larger than a workgroup holds: split_pass_stable)
+    const int64_t chunk_lo = c * kChunk;
+    const int64_t chunk_hi = (chunk_lo + kChunk < n) ? chunk_lo + kChunk : n;
+    scatter_to_buckets<K, PAIRS, BLOCK, MAP, true>(sm, io, n, row, info, chunk_lo, chunk_hi, chunk_base + static_cast<int64_t>(blockIdx.x) * kMaxBuckets);
+}
+
+// Steps 1 to 4 for a whole row by one workgroup, for calls of many rows that are not too long
+// (at least two rows per compute unit, rows of up to 131072 keys): the row's range from its
+// sample, its fine-bin histogram in LDS (no chunks, no tables in memory), its buckets, and the
+// scatter, for which the row is read a second time - out of the caches as a rule, the same
+// workgroup having just read it.  Three launches fewer, one crossing of HBM less, and what one
+// workgroup waits for (the sample, the dependent steps of the plan) the others on its compute
+// unit fill.  Rows of pairs with buckets larger than a workgroup holds are left to
+// split_pass_stable.
+template <typename K, bool PAIRS, int BLOCK, int MAP>
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void split_front(PassIo<K> io, int64_t n, uint32_t cap, SplitRow* __restrict__ rows,
+                                                           uint32_t* __restrict__ counters, uint4* __restrict__ bucket_list,
+                                                           uint32_t* __restrict__ crowded_list) {
+    static_assert(MAP != kMapValue, "rows short enough for the smallest buckets");
+    __shared__ SplitShared<K, PAIRS, BLOCK> sm;
+    __shared__ PlanShared<BLOCK> plan;
+    static_assert(sizeof(sm.keys) >= kFine * sizeof(uint32_t), "the histogram lies where the tiles will");
+    uint32_t* hist = reinterpret_cast<uint32_t*>(sm.keys);
+    const int64_t row = blockIdx.x;
+    const K* xrow = io.x + io.xmap.at(row);
+    SplitRow& info = rows[row];
+    const FineRange range = sample_row<K, MAP, BLOCK>(io, xrow, n, cap);
+    if (threadIdx.x == 0) range.store(info);
+    for (int i = threadIdx.x; i < kFine; i += BLOCK) hist[i] = 0u;
+    __syncthreads();
+    count_fine_bins<K, MAP, BLOCK, false>(io, xrow, 0, n, FineMap<K>(range, io.descending), hist);
+    __syncthreads();
+    constexpr int PER = kFine / kSplitBlock;
+    uint32_t cnt[PER], bucket[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) cnt[i] = threadIdx.x < kSplitBlock ? hist[threadIdx.x * PER + i] : 0u;
+    uint32_t route = 0;
+    (void)plan_buckets<BLOCK>(plan, cnt, bucket, n, cap, row, info, counters, bucket_list, crowded_list, &route);
+    if (PAIRS && route != 1u) return;
+    __syncthreads();                                   // the row's record and table are in memory, the histogram has been read
+    scatter_to_buckets<K, PAIRS, BLOCK, MAP, true>(sm, io, n, row, info, 0, n, plan.begin);
+}
+
+__global__ void split_clear(uint32_t* __restrict__ counters) {
+    if (threadIdx.x < 4) counters[threadIdx.x] = 0u;
+}
+
 // The same pass for the rows (of pairs) that have buckets larger than a workgroup holds
 // (SplitRow::route 2): every key's slot among the tile's keys of its bucket is its rank in
 // element order (wave-wide matching of bucket numbers, as the digit passes rank), so each bucket
@@ -888,9 +988,10 @@ __global__ __launch_bounds__(kSplitBlock) void split_pass_stable(PassIo<K> io, i
     const int w = tid / kWave;
     if (counters[3] == 0u) return;                     // no such row in this call (the usual case)
     // (a small grid walks the chunks: the launch costs little when there is nothing to do)
+    // (without chunk tables - split_front made the plan - a unit is a whole row)
     for (int64_t unit = blockIdx.x; unit < chunks; unit += gridDim.x) {
-    const int64_t row = unit / chunks_per_row;
-    const int64_t c = unit - row * chunks_per_row;
+    const int64_t row = chunk_base ? unit / chunks_per_row : unit;
+    const int64_t c = chunk_base ? unit - row * chunks_per_row : 0;
     const SplitRow& info = infos[row];
     if (info.route != 2u) continue;
     __syncthreads();                                   // the chunk before has left the table
@@ -899,12 +1000,12 @@ __global__ __launch_bounds__(kSplitBlock) void split_pass_stable(PassIo<K> io, i
     K* dk = io.kbuf[0] + row * n;
     uint32_t* dv = io.vbuf[0] + row * n;
     const int64_t chunk_lo = c * kChunk;
-    const int64_t chunk_hi = (chunk_lo + kChunk < n) ? chunk_lo + kChunk : n;
+    const int64_t chunk_hi = (chunk_base && chunk_lo + kChunk < n) ? chunk_lo + kChunk : n;
     // bucket numbers lie below n_buckets: only those bits are matched
     const uint32_t vary = info.n_buckets > 1u ? (2u << (31 - __builtin_clz(info.n_buckets - 1u))) - 1u : 0u;
     static_assert(kSplitBlock == kMaxBuckets, "a thread per bucket");
     reinterpret_cast<uint4*>(table)[tid] = reinterpret_cast<const uint4*>(info.bucket_of)[tid];
-    uint32_t next = chunk_base[unit * kMaxBuckets + tid];      // where this chunk's coming keys of bucket tid go
+    uint32_t next = chunk_base ? chunk_base[unit * kMaxBuckets + tid] : info.begin[tid];      // where this unit's coming keys of bucket tid go
     for (int64_t tile_base = chunk_lo; tile_base < chunk_hi; tile_base += TILE) {
         for (int i = tid; i < WAVES * kMaxBuckets; i += kSplitBlock) (&wave_hist[0][0])[i] = 0u;
         K key[ITEMS];
@@ -1724,17 +1825,27 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         else if (map == kMapGap) launch_with(std::integral_constant<int, kMapGap>());
         else launch_with(std::integral_constant<int, kMapValue>());
     };
-    with_map([&](auto map_tag) {
-        split_sample<K, decltype(map_tag)::value><<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(io, n, static_cast<uint32_t>(cap), rows, counters);
-    });
-    DLFX_CHECK_LAUNCH();
+    // Many rows of 4-byte keys that take the smallest buckets: one workgroup makes a row's plan and
+    // moves the row (split_front); otherwise the steps are launches of their own, a workgroup a chunk.
+    const bool front = sizeof(K) == 4 && waves == 4 && m >= kFrontRows;
+    if (!front) {
+        with_map([&](auto map_tag) {
+            split_sample<K, decltype(map_tag)::value><<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(io, n, static_cast<uint32_t>(cap), rows, counters);
+        });
+        DLFX_CHECK_LAUNCH();
+    } else {
+        split_clear<<<dim3(1), dim3(kWave), 0, stream>>>(counters);
+        DLFX_CHECK_LAUNCH();
+    }
     const dim3 chunks(static_cast<unsigned>(m * l.chunks_per_row));
-    with_map([&](auto map_tag) {
-        split_histogram<K, decltype(map_tag)::value><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine);
-    });
-    DLFX_CHECK_LAUNCH();
-    split_plan<<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(n, static_cast<uint32_t>(cap), l.chunks_per_row, fine, rows, counters, list, crowded, chunk_base);
-    DLFX_CHECK_LAUNCH();
+    if (!front) {
+        with_map([&](auto map_tag) {
+            split_histogram<K, decltype(map_tag)::value><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine);
+        });
+        DLFX_CHECK_LAUNCH();
+        split_plan<<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(n, static_cast<uint32_t>(cap), l.chunks_per_row, fine, rows, counters, list, crowded, chunk_base);
+        DLFX_CHECK_LAUNCH();
+    }
     // split_finish: as many workgroups as the device holds at once, each walking its share of the buckets
     const int64_t buckets = m * kMaxBuckets;
     const uint32_t limit = static_cast<uint32_t>(compare_max);
@@ -1746,9 +1857,17 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         const dim3 fgrid(static_cast<unsigned>(buckets < finish_room ? buckets : finish_room));
         const int block = pass_block<K, PAIRS>(n, cap);
         auto pass_of = [&](auto block_tag) {
+            constexpr int BLOCK = decltype(block_tag)::value;
             with_map([&](auto map_tag) {
-                split_pass<K, PAIRS, decltype(block_tag)::value, decltype(map_tag)::value><<<chunks, dim3(decltype(block_tag)::value), 0, stream>>>(
-                    io, n, l.chunks_per_row, rows, chunk_base);
+                constexpr int MAP = decltype(map_tag)::value;
+                if constexpr (sizeof(K) == 4 && WAVES == 4 && MAP != kMapValue && BLOCK <= 512) {
+                    if (front) {
+                        split_front<K, PAIRS, BLOCK, MAP><<<dim3(static_cast<unsigned>(m)), dim3(BLOCK), 0, stream>>>(
+                            io, n, static_cast<uint32_t>(cap), rows, counters, list, crowded);
+                        return;
+                    }
+                }
+                split_pass<K, PAIRS, BLOCK, MAP><<<chunks, dim3(BLOCK), 0, stream>>>(io, n, l.chunks_per_row, rows, chunk_base);
             });
         };
         if (block == 256) pass_of(std::integral_constant<int, 256>());
@@ -1757,9 +1876,9 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         DLFX_CHECK_LAUNCH();
         if constexpr (PAIRS) {
             // rows with buckets larger than a workgroup holds (as a rule none: every workgroup leaves at once)
-            const int64_t units = m * l.chunks_per_row;
+            const int64_t units = front ? m : m * l.chunks_per_row;
             split_pass_stable<K><<<dim3(static_cast<unsigned>(units < 1024 ? units : 1024)), dim3(kSplitBlock), 0, stream>>>(
-                io, n, l.chunks_per_row, units, rows, counters, chunk_base);
+                io, n, l.chunks_per_row, units, rows, counters, front ? nullptr : chunk_base);
             DLFX_CHECK_LAUNCH();
         }
         split_finish<K, PAIRS, WAVES><<<fgrid, dim3(WAVES * kWave), 0, stream>>>(io, n, limit, counters, list, crowded);

@@ -460,6 +460,33 @@ def test_buckets_larger_than_a_workgroup_holds(hip_backend, dtype, n):
     assert np.array_equal(np.ascontiguousarray(Th.numpy()), want)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.int32])
+@pytest.mark.parametrize("n", [17000, 40000, 70000, 131072])
+def test_many_rows_each_planned_and_moved_by_one_workgroup(hip_backend, dtype, n):
+    # calls of at least 512 rows of 4-byte keys of up to 131072 elements: one workgroup takes a
+    # row from its sample to its scatter; rows that cut evenly beside rows with oversized buckets
+    m = 530
+    kinds = oversized_rows(dtype, n, 360)                               # 7 kinds of awkward rows
+    if np.dtype(dtype).kind == "f":
+        wide = (normal(361, m * n) * 3).astype(dtype).reshape(m, n)
+        wide[::3] = np.floor(uniform01(362, ((m + 2) // 3) * n) * 4096).astype(dtype).reshape(-1, n) / dtype(4096)      # the benchmark's quantised rows
+    else:
+        wide = (full_range_i64(361, m * n) >> 33).astype(dtype).reshape(m, n)
+    x = wide
+    x[5::40] = kinds[np.arange(x[5::40].shape[0]) % kinds.shape[0]]
+    Xh = Tensor.from_numpy(hip_backend, x)
+    want = np.sort(x, axis=-1, kind="stable")
+    assert np.array_equal(F.sort(Xh, -1).numpy(), want)
+    order = np.argsort(x, axis=-1, kind="stable")
+    assert np.array_equal(F.argsort(Xh, -1).numpy(), order)
+    Yh, Ih = F.argsort(Xh, -1, True, with_values=True)
+    rev = np.argsort(-x if np.dtype(dtype).kind == "f" else ~x, axis=-1, kind="stable")
+    assert np.array_equal(Ih.numpy(), rev)
+    assert np.array_equal(Yh.numpy().view(np.uint8), np.take_along_axis(x, rev, -1).view(np.uint8))
+    F.sort(Xh, -1, True, out=Xh)                                        # in place
+    assert np.array_equal(Xh.numpy(), want[:, ::-1])
+
+
 @pytest.mark.parametrize("n", [70000, 300000])
 def test_index_only_argsort_written_over_its_input(hip_backend, n):
     # argsort(X, X) of int32 (UniformTest.cpp:2461-2466 does this with short rows): there is no value
