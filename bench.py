@@ -398,6 +398,19 @@ def make_ops(be, which):
             call()
             assert torch.equal(zm, torch.sort(torch.cat([a, b], dim=1), dim=1).values)
         ops.append(Op("N2", "merge_f32_[64,2^19]+[64,2^19]", 64 * 2 * half, 2 * 4 * 64 * 2 * half, calls, v_merge))
+    # ---------------- L1 (only on request): a few very long rows (a sampling head over a huge vocabulary)
+    if on("long"):
+        for rows_l, n_l in ((1, 1 << 26), (64, 1 << 20)):
+            text = "[%d,2^%d]" % (rows_l, n_l.bit_length() - 1)
+            xl_ = gen((rows_l, n_l), torch.float32, lambda c: synth.normal(30 + 100 * c), 2)
+            yl_ = empty((rows_l, n_l), torch.float32)
+            calls = [be.softmax("softmax", dtype_code(np.float32), rows_l, n_l, x.view(-1), 0, yl_.view(-1), 0, defer=True) for x in xl_]
+
+            def v_sl(x=xl_[0], y=yl_, call=calls[0]):
+                call()
+                assert torch.allclose(y.double(), torch.softmax(x.double(), 1), rtol=1e-5, atol=1e-14)
+            ops.append(Op("L1", "softmax_f32_" + text, rows_l * n_l, 8 * rows_l * n_l, calls, v_sl))
+            ops += topk_ops(be, tensor, xl_, (5, 100), "L1", text)
     # ---------------- S1 (only on request): many short rows, and top_k along an outer axis
     if on("short"):
         for rows_s, n_s in ((1 << 20, 64), (1 << 18, 256), (1 << 16, 1024)):
@@ -479,13 +492,15 @@ def topk_ops(be, tensor, xs, ks, config, shape_text):
     return ops
 
 
-def split_kernels(es, pairs, n):
+def split_kernels(es, pairs, rows, n):
     """The kernels that move the data of one sort / argsort of rows the bucket route takes."""
     key = "unsigned int" if es == 4 else "unsigned long"
     waves = 4 if n <= 131072 else 8
     flag = "true" if pairs else "false"
-    return ["split_sample<%s," % key, "split_histogram<%s," % key, "split_plan", "split_pass<%s, %s," % (key, flag),
-            "split_finish<%s, %s, %d>" % (key, flag, waves)]
+    finish = "split_finish<%s, %s, %d>" % (key, flag, waves)
+    if es == 4 and waves == 4 and rows >= 512:            # one workgroup plans and moves a whole row
+        return ["split_front<%s, %s," % (key, flag), finish]
+    return ["split_sample<%s," % key, "split_histogram<%s," % key, "split_plan", "split_pass<%s, %s," % (key, flag), finish]
 
 
 def sort_ops(be, tensor, xs, config, text):
@@ -509,7 +524,7 @@ def sort_ops(be, tensor, xs, config, text):
             call()
             assert torch.equal(y, torch.sort(x, dim=1, descending=bool(desc)).values), "sort"
         ops.append(Op(config, "sort_%s_%s" % ("desc" if desc else "asc", text), rows * n, 2 * es * rows * n, calls, v,
-                      split_kernels(es, False, n)))
+                      split_kernels(es, False, rows, n)))
         calls = []
         for x in xs:
             X = tensor(x)
@@ -528,7 +543,7 @@ def sort_ops(be, tensor, xs, config, text):
             else:
                 assert bool((g[:, 1:] <= g[:, :-1]).all() if desc else (g[:, 1:] >= g[:, :-1]).all())
         ops.append(Op(config, "argsort_%s_%s" % ("desc" if desc else "asc", text), rows * n, (es + 4) * rows * n,
-                      calls, va, split_kernels(es, True, n)))
+                      calls, va, split_kernels(es, True, rows, n)))
     return ops
 
 
@@ -622,7 +637,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3 | short (many short rows and an outer axis; not part of all) | spread (sorts of N(0,1) rows; not part of all) | ceil (copy and read-only streams at the C2 and C5 sizes; part of all) | ceilbig (the same streams at 1 GiB and 4 GiB; not part of all)")
+    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3 | short (many short rows and an outer axis; not part of all) | spread (sorts of N(0,1) rows; not part of all) | ceil (copy and read-only streams at the C2 and C5 sizes; part of all) | ceilbig (the same streams at 1 GiB and 4 GiB; not part of all) | long (softmax and top_k over a few very long rows; not part of all)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
