@@ -24,7 +24,9 @@ struct DimMap {
     int64_t dims[kMaxRank];
     int64_t strides[kMaxRank];
 
-    __host__ __device__ int64_t at(int64_t flat) const {
+    // (always inlined: an out-of-line call takes the address of its map, and a kernel whose
+    // argument block holds the map then keeps a private copy of the whole block in scratch memory)
+    __host__ __device__ __attribute__((always_inline)) int64_t at(int64_t flat) const {
         if (rank == 1) return flat * strides[0];
         int64_t off = 0;
         for (int i = rank - 1; i > 0; --i) {

@@ -102,6 +102,17 @@ inline int finish_waves(int64_t n, bool floats) {
 }
 constexpr int kNear = 2;                              // entries of a bin compared without a loop
 constexpr int64_t kFrontRows = 512;                   // fewest rows of a call that split_front takes (two a compute unit)
+// A bucket larger than a workgroup holds is listed once per window of this many entries, so that
+// a bucket of one repeated value (a constant row is one bucket) is copied out by many workgroups.
+constexpr uint32_t kOverWindow = 32768;
+constexpr uint32_t kNoWindow = 0xffffffffu;           // an entry of the list that is a whole (crowded) bucket
+// What split_finish_crowded walks: {bucket id = row * 256 + b, window} entries, and the OR and
+// the AND of the keys of every oversized bucket (split_plan sets them to zero and all ones,
+// split_pass_stable gathers them): equal means one repeated value.
+struct CrowdedList {
+    uint2* items;
+    unsigned long long* range;             // [2 id]: OR of the bucket's keys, [2 id + 1]: AND
+};
 
 // What split_sample and split_plan decide for a row.
 struct alignas(16) SplitRow {
@@ -237,7 +248,7 @@ __device__ __forceinline__ K wave_fourth(const K (&key)[4]) {
 // rows); 1 for float rows of middling length, whose images may have the gap around zero closed
 // up; 2 for longer float rows, by key image as they are or by value.  The kernels carry no code for what their
 // MAP leaves out.
-constexpr int kMapPlain = 0, kMapGap = 1, kMapValue = 2;
+constexpr int kMapPlain = 0, kMapGap = 1, kMapValue = 2, kMapAny = 3;      // (any: decided per row as the kernel runs)
 
 // How a row's keys spread over its fine bins (the part of SplitRow that split_sample decides).
 struct FineRange {
@@ -505,7 +516,7 @@ struct PlanShared {
 template <int BLOCK>
 __device__ __forceinline__ uint32_t plan_buckets(PlanShared<BLOCK>& sm, const uint32_t (&cnt)[kFine / kSplitBlock], uint32_t (&bucket)[kFine / kSplitBlock],
                                                  int64_t n, uint32_t cap, int64_t row, SplitRow& info, uint32_t* __restrict__ counters,
-                                                 uint4* __restrict__ bucket_list, uint32_t* __restrict__ crowded_list, uint32_t* route_out = nullptr) {
+                                                 uint4* __restrict__ bucket_list, CrowdedList crowded, uint32_t* route_out = nullptr) {
     constexpr int PER = kFine / kSplitBlock;          // 16
     constexpr int WAVES = BLOCK / kWave;
     const int w = threadIdx.x / kWave;
@@ -641,11 +652,13 @@ __device__ __forceinline__ uint32_t plan_buckets(PlanShared<BLOCK>& sm, const ui
             b0 = sm.begin[threadIdx.x];
             size = sm.begin[threadIdx.x + 1] - b0;
         }
-        const bool fits_finish = size != 0u && size <= cap, oversized = size > cap;
-        const unsigned long long fit_lanes = __ballot(fits_finish), over_lanes = __ballot(oversized);
-        if (lane_id() == 0 && planner) {
-            sm.listed[0][w] = static_cast<uint32_t>(__popcll(fit_lanes));
-            sm.listed[1][w] = static_cast<uint32_t>(__popcll(over_lanes));
+        const bool fits_finish = size != 0u && size <= cap;
+        const uint32_t windows = size > cap ? (size + kOverWindow - 1) / kOverWindow : 0u;      // list entries of an oversized bucket
+        const unsigned long long fit_lanes = __ballot(fits_finish);
+        const uint32_t windows_incl = wave_scan_inclusive(windows, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+        if (planner) {
+            if (lane_id() == 0) sm.listed[0][w] = static_cast<uint32_t>(__popcll(fit_lanes));
+            if (lane_id() == kWave - 1) sm.listed[1][w] = windows_incl;
         }
         __syncthreads();
         if (threadIdx.x < 2) {
@@ -662,14 +675,19 @@ __device__ __forceinline__ uint32_t plan_buckets(PlanShared<BLOCK>& sm, const ui
         const uint32_t id = static_cast<uint32_t>(row) * kMaxBuckets + threadIdx.x;
         if (fits_finish)
             bucket_list[sm.listed[0][kSplitBlock / kWave] + sm.listed[0][w] + static_cast<uint32_t>(__popcll(fit_lanes & below))] = make_uint4(static_cast<uint32_t>(row), b0, size, id);
-        if (oversized) crowded_list[sm.listed[1][kSplitBlock / kWave] + sm.listed[1][w] + static_cast<uint32_t>(__popcll(over_lanes & below))] = id;
+        if (windows != 0u) {
+            uint2* at = crowded.items + sm.listed[1][kSplitBlock / kWave] + sm.listed[1][w] + (windows_incl - windows);
+            for (uint32_t i = 0; i < windows; ++i) at[i] = make_uint2(id, i);
+            crowded.range[2 * id] = 0ull;
+            crowded.range[2 * id + 1] = ~0ull;
+        }
     }
     return n_buckets;
 }
 
 __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t cap, int64_t chunks_per_row, const uint32_t* __restrict__ chunk_fine,
                                                           SplitRow* __restrict__ rows, uint32_t* __restrict__ counters,
-                                                          uint4* __restrict__ bucket_list, uint32_t* __restrict__ crowded_list,
+                                                          uint4* __restrict__ bucket_list, CrowdedList crowded,
                                                           uint32_t* __restrict__ chunk_base) {
     constexpr int PER = kFine / kSplitBlock;          // 16
     __shared__ PlanShared<kSplitBlock> sm;
@@ -700,7 +718,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
     }
     uint32_t bucket[PER];
     per_bucket[threadIdx.x] = 0u;
-    const uint32_t n_buckets = plan_buckets<kSplitBlock>(sm, cnt, bucket, n, cap, row, rows[row], counters, bucket_list, crowded_list);
+    const uint32_t n_buckets = plan_buckets<kSplitBlock>(sm, cnt, bucket, n, cap, row, rows[row], counters, bucket_list, crowded);
     uint32_t next = threadIdx.x < n_buckets ? sm.begin[threadIdx.x] : 0u;      // where the coming chunk's keys of bucket threadIdx.x go
     // each chunk's keys per bucket, and from them where the chunk writes each bucket
     uint32_t w8[PER / 2], ahead[PER / 2];
@@ -727,13 +745,42 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
     }
 }
 
+// Where bucket `id` = row * 256 + b lies: {row, first position in the row, entries, id}.
+__device__ __forceinline__ uint4 bucket_at(const SplitRow* __restrict__ infos, uint32_t id) {
+    const uint32_t row = id / kMaxBuckets, b = id % kMaxBuckets;
+    const SplitRow& info = infos[row];
+    const uint32_t b0 = info.begin[b];
+    return make_uint4(row, b0, info.begin[b + 1] - b0, id);
+}
+
+// Entry `at` of the sorted row goes to the strided outputs (unit strides: plain 32-bit offsets
+// from the row's start, the case every contiguous output takes).
+template <typename K, bool PAIRS>
+__device__ __forceinline__ void emit_entry(const PassIo<K>& io, const K* xrow, K* yrow, int64_t irow, int64_t at, K key, uint32_t val) {
+    if (yrow) {
+        K bits = decode_key<K>(key, io.kind, io.descending);
+        if constexpr (PAIRS) {
+            if (io.restore_zero && static_cast<K>(bits << 1) == 0) bits = xrow[static_cast<int64_t>(val) * io.sx];
+        }
+        if (io.sy == 1) yrow[static_cast<uint32_t>(at)] = bits;
+        else yrow[at * io.sy] = bits;
+    }
+    if constexpr (PAIRS) {
+        if (io.idx) {
+            if (io.si == 1 && !io.idx64) (static_cast<int32_t*>(io.idx) + irow)[static_cast<uint32_t>(at)] = static_cast<int32_t>(val);
+            else if (io.idx64) static_cast<int64_t*>(io.idx)[irow + at * io.si] = static_cast<int64_t>(val);
+            else static_cast<int32_t*>(io.idx)[irow + at * io.si] = static_cast<int32_t>(val);
+        }
+    }
+}
+
 // ------------------------------------------------------------------ 4. one pass: chunk -> buckets
 // The largest tile of 8-byte keys with indices does not fit LDS twice over: its indices pass
 // through the space its keys have left (the threads keep where everything goes in registers).
 template <typename K, bool PAIRS, int BLOCK>
 constexpr bool kPassInTurn = PAIRS && sizeof(K) == 8 && BLOCK == 1024;
 
-template <typename K, bool PAIRS, int BLOCK>
+template <typename K, bool PAIRS, int BLOCK, bool STABLE = false>
 struct SplitShared {
     uint32_t table[kFine / 4];                 // bucket_of, four fine bins a word
     uint32_t hist[kMaxBuckets];                // keys of the tile per bucket
@@ -742,6 +789,35 @@ struct SplitShared {
     uint32_t scan_tmp[kMaxBuckets / kWave];
     K keys[BLOCK * kSplitItems];
     uint32_t vals[PAIRS && !kPassInTurn<K, PAIRS, BLOCK> ? BLOCK * kSplitItems : 1];
+    // the stable pass: every wavefront's count of each bucket, which buckets are larger than a
+    // workgroup holds, and
+    uint32_t wave_hist[STABLE ? BLOCK / kWave : 1][kMaxBuckets];
+    uint32_t oversized[STABLE ? kMaxBuckets : 1];
+    K mixed[STABLE ? kMaxBuckets : 1];        // ... the bits in which neighbouring entries of such a bucket differ in this tile
+};
+
+// What the stable pass needs beyond the plain one.
+template <typename K>
+struct StablePass {
+    uint32_t cap = 0;                          // the most entries of a bucket that split_finish takes
+    unsigned long long* range = nullptr;       // CrowdedList::range
+    // the row's outputs (what emit_entry reads from PassIo, by value)
+    K* yrow = nullptr;                         // the row of the value output, if there is one
+    void* idx = nullptr;                       // the index output, if there is one
+    int64_t irow = 0, sx = 1, sy = 1, si = 1;  // where its row starts; the strides
+    int idx64 = 0, kind = 0, descending = 0, restore_zero = 0;
+    bool direct = false;                       // the oversized buckets' entries go straight to the outputs
+    __device__ __forceinline__ void emit(const K* xrow, int64_t at, K key, uint32_t val) const {
+        if (yrow) {
+            K bits = decode_key<K>(key, kind, descending);
+            if (restore_zero && static_cast<K>(bits << 1) == 0) bits = xrow[static_cast<int64_t>(val) * sx];
+            yrow[at * sy] = bits;
+        }
+        if (idx) {
+            if (idx64) static_cast<int64_t*>(idx)[irow + at * si] = static_cast<int64_t>(val);
+            else static_cast<int32_t*>(idx)[irow + at * si] = static_cast<int32_t>(val);
+        }
+    }
 };
 
 // A workgroup moves a range of a row (split_pass: a chunk of kChunk keys) in tiles of BLOCK x 16
@@ -750,18 +826,30 @@ struct SplitShared {
 // and their slot among the tile's keys of that bucket with one LDS atomic each, the tile is laid
 // out by bucket in LDS and written as runs; once it lies in LDS the registers already receive
 // the next tile's keys.  The order inside a run is whatever the atomics gave.
-template <typename K, bool PAIRS, int BLOCK, int MAP, bool STREAM>
-__device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK>& sm, const PassIo<K>& io, int64_t n, int64_t row, const SplitRow& info,
-                                                   int64_t chunk_lo, int64_t chunk_hi, const uint32_t* __restrict__ places) {
+//
+// STABLE (rows with buckets larger than a workgroup holds, SplitRow::route 2): a key's slot is
+// its rank in element order instead (wave-wide matching of bucket numbers, as the digit passes
+// rank; wavefront w takes elements [1024 w, 1024 w + 1024) of the tile), so every bucket receives
+// its entries in index order and a bucket of one repeated value arrives sorted.  The entries of
+// the oversized buckets go straight to their places in the outputs when those do not overlap
+// the input (a bucket of one value is then done: a constant row costs one crossing), and the
+// OR and the AND of the keys of every oversized bucket are left in `range`.
+template <typename K, bool PAIRS, int BLOCK, int MAP, bool STREAM, bool STABLE = false>
+__device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK, STABLE>& sm, const PassIo<K>& io, int64_t n, int64_t row, const SplitRow& info,
+                                                   int64_t chunk_lo, int64_t chunk_hi, const uint32_t* __restrict__ places, StablePass<K> stable = {}) {
     constexpr int ITEMS = kSplitItems;
     constexpr int TILE = BLOCK * kSplitItems;
+    constexpr int WAVES = BLOCK / kWave;
     constexpr bool IN_TURN = kPassInTurn<K, PAIRS, BLOCK>;
+    static_assert(!(STABLE && IN_TURN), "the stable pass writes keys and indices together");
     const int tid = threadIdx.x;
     const int lane = lane_id();
     const int w = tid / kWave;
     const FineMap<K> fine_of(info, io.descending);
     const K* xrow = io.x + io.xmap.at(row);
     const int64_t row_off = row * n;
+    // element of the tile that this thread's item k is
+    auto element_of = [&](int k) __attribute__((always_inline)) { return STABLE ? w * (kWave * ITEMS) + k * kWave + lane : tid + k * BLOCK; };
 
     // (no branches: an element beyond the chunk's end reads the tile's first element instead and is never used)
     auto load_tile = [&](int64_t tile_base, K (&key)[ITEMS]) __attribute__((always_inline)) {
@@ -769,7 +857,7 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK>&
         const K* src = xrow + tile_base * io.sx;
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
-            const int e = tid + k * BLOCK;
+            const int e = element_of(k);
             const K* at = &src[static_cast<int64_t>(e < valid ? e : 0) * io.sx];
             if constexpr (sizeof(K) == 4 && STREAM) key[k] = load_stream(at);       // (non-temporal loads measured: a gain for 4-byte keys,
             else key[k] = *at;                                                      // a loss of 7 % for 8-byte keys)
@@ -785,12 +873,23 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK>&
         reinterpret_cast<uint4*>(sm.table)[tid] = reinterpret_cast<const uint4*>(info.bucket_of)[tid];
         sm.hist[tid] = 0u;
         next = places[tid];
+        if constexpr (STABLE) {
+            sm.oversized[tid] = (tid < static_cast<int>(info.n_buckets) && info.begin[tid + 1] - info.begin[tid] > stable.cap) ? 1u : 0u;
+            sm.mixed[tid] = K(0);
+        }
     }
+    if constexpr (STABLE)
+        for (int i = tid; i < WAVES * kMaxBuckets; i += BLOCK) (&sm.wave_hist[0][0])[i] = 0u;
+    // (stable) bucket numbers lie below n_buckets: only those bits are matched; elements beyond the
+    // chunk's end count as the last bucket's, after every element of the chunk
+    const uint32_t last_bucket = info.n_buckets - 1u;
+    const uint32_t vary = last_bucket != 0u ? (2u << (31 - __builtin_clz(last_bucket))) - 1u : 0u;
+    const bool direct = STABLE && stable.direct;
     __syncthreads();
 
     auto move_chunk = [&](auto by_value_tag) __attribute__((always_inline)) {
     constexpr bool BY_VALUE = decltype(by_value_tag)::value;
-    constexpr bool GAP = MAP == kMapGap;
+    constexpr bool GAP = MAP == kMapGap || MAP == kMapAny;
     for (int64_t tile_base = chunk_lo; tile_base < chunk_hi; tile_base += TILE) {
         const int valid = static_cast<int>((chunk_hi - tile_base < TILE) ? chunk_hi - tile_base : TILE);
         const bool full = valid == TILE;
@@ -802,6 +901,18 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK>&
         // ---- bucket of every key (table), then its slot among the tile's keys of that bucket:
         // one LDS atomic each, eight lookups issued before their eight atomics
         uint32_t where[ITEMS];                     // bucket << 16 | slot, later the key's place in the tile
+        if constexpr (STABLE) {
+            uint32_t rank[ITEMS];
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) {
+                const uint32_t f = fine_of.template bin<BY_VALUE, GAP>(key[k]);
+                where[k] = (sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu;
+                if (!full && element_of(k) >= valid) where[k] = last_bucket;
+            }
+            rank_by_digit<ITEMS>(sm.wave_hist[w], where, vary, rank);
+#pragma unroll
+            for (int k = 0; k < ITEMS; ++k) where[k] = (where[k] << 16) | rank[k];
+        } else {
 #pragma unroll
         for (int k0 = 0; k0 < ITEMS; k0 += 8) {
 #pragma unroll
@@ -813,14 +924,26 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK>&
             for (int k = k0; k < k0 + 8; ++k)
                 if (full || tid + k * BLOCK < valid) where[k] = (where[k] << 16) | atomicAdd(&sm.hist[where[k]], 1u);
         }
+        }
         __syncthreads();
         SPLIT_PHASE(1);
 
         // ---- thread b owns bucket b: its place in the tile and in the row
+        uint32_t own_start = 0, own_count = 0;         // (stable) ... and how many entries of the chunk it has in the tile
         {
             uint32_t count = 0, incl = 0;
             if (owner) {
-                count = sm.hist[tid];
+                if constexpr (STABLE) {
+                    // each wavefront's share of the bucket starts after the shares of the wavefronts before
+#pragma unroll
+                    for (int i = 0; i < WAVES; ++i) {
+                        const uint32_t c = sm.wave_hist[i][tid];
+                        sm.wave_hist[i][tid] = count;
+                        count += c;
+                    }
+                } else {
+                    count = sm.hist[tid];
+                }
                 incl = wave_scan_inclusive(count, 0u, [](uint32_t a, uint32_t b) { return a + b; });
                 if (lane == kWave - 1) sm.scan_tmp[w] = incl;
                 sm.hist[tid] = 0u;                         // for the next tile
@@ -833,6 +956,10 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK>&
                 sm.start[tid] = start;
                 sm.dst_base[tid] = static_cast<int32_t>(next) - static_cast<int32_t>(start);
                 next += count;
+                if constexpr (STABLE) {
+                    own_start = start;
+                    own_count = (!full && tid == static_cast<int>(last_bucket)) ? count - static_cast<uint32_t>(TILE - valid) : count;
+                }
             }
         }
         __syncthreads();
@@ -840,22 +967,80 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK>&
 
         // ---- lay the tile out by bucket (bucket starts read first, then the stores)
 #pragma unroll
-        for (int k = 0; k < ITEMS; ++k) where[k] = sm.start[where[k] >> 16] + (where[k] & 0xffffu);
+        for (int k = 0; k < ITEMS; ++k) {
+            if constexpr (STABLE) where[k] = sm.start[where[k] >> 16] + sm.wave_hist[w][where[k] >> 16] + (where[k] & 0xffffu);
+            else where[k] = sm.start[where[k] >> 16] + (where[k] & 0xffffu);
+        }
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
-            if (full || tid + k * BLOCK < valid) {
+            if (full || element_of(k) < valid) {
                 sm.keys[where[k]] = key[k];
-                if constexpr (PAIRS && !IN_TURN) sm.vals[where[k]] = static_cast<uint32_t>(tile_base) + static_cast<uint32_t>(tid + k * BLOCK);
+                if constexpr (PAIRS && !IN_TURN) sm.vals[where[k]] = static_cast<uint32_t>(tile_base) + static_cast<uint32_t>(element_of(k));
             }
         }
         __syncthreads();
         SPLIT_PHASE(3);
+        if constexpr (STABLE)
+            for (int i = tid; i < WAVES * kMaxBuckets; i += BLOCK) (&sm.wave_hist[0][0])[i] = 0u;      // for the next tile
         // the tile is in LDS: the registers take the next tile, whose keys arrive while this one is written
         if (tile_base + TILE < chunk_hi) load_tile(tile_base + TILE, key);
 
         // ---- write runs: thread tid takes tile positions tid, tid + BLOCK, ...; eight at a time, the
         // reads of each step issued for all eight before the next step uses them
-        {
+        if constexpr (STABLE) {
+            K* dk = io.kbuf[0] + row_off;
+            uint32_t* dv = PAIRS ? io.vbuf[0] + row_off : nullptr;
+            constexpr int G = sizeof(K) == 8 ? 4 : 8;          // tile positions a thread handles at a time (registers)
+            const K own_first = (owner && own_count != 0u) ? sm.keys[own_start] : K(0);
+#pragma unroll
+            for (int k0 = 0; k0 < ITEMS; k0 += G) {
+                K out[G], before[G];
+                uint32_t pay[PAIRS ? G : 1], b[G], first[G], big[G];
+                int32_t at[G];
+#pragma unroll
+                for (int j = 0; j < G; ++j) {
+                    const int p = (k0 + j) * BLOCK + tid;
+                    out[j] = sm.keys[p];
+                    before[j] = sm.keys[p > 0 ? p - 1 : 0];
+                    if constexpr (PAIRS) pay[j] = sm.vals[p];
+                }
+#pragma unroll
+                for (int j = 0; j < G; ++j) {
+                    const uint32_t f = fine_of.template bin<BY_VALUE, GAP>(out[j]);
+                    b[j] = (sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu;
+                }
+#pragma unroll
+                for (int j = 0; j < G; ++j) {
+                    at[j] = sm.dst_base[b[j]] + ((k0 + j) * BLOCK + tid);
+                    first[j] = sm.start[b[j]];
+                    big[j] = sm.oversized[b[j]];
+                }
+#pragma unroll
+                for (int j = 0; j < G; ++j) {
+                    const uint32_t p = static_cast<uint32_t>((k0 + j) * BLOCK + tid);
+                    if (!full && p >= static_cast<uint32_t>(valid)) continue;
+                    if (big[j] != 0u) {
+                        if (p > first[j] && before[j] != out[j]) atomicOr(&sm.mixed[b[j]], static_cast<K>(before[j] ^ out[j]));
+                        if (direct) {
+                            stable.emit(xrow, at[j], out[j], PAIRS ? pay[j] : 0u);
+                            continue;
+                        }
+                    }
+                    dk[at[j]] = out[j];
+                    if constexpr (PAIRS) dv[at[j]] = pay[j];
+                }
+            }
+            __syncthreads();                               // the tile in LDS has left, every mixed bucket is marked
+            if (owner && own_count != 0u && sm.oversized[tid] != 0u) {
+                // the OR and the AND of the bucket's keys in this tile, from one of them and the bits that vary
+                const K vary_here = sm.mixed[tid];
+                sm.mixed[tid] = K(0);
+                const uint32_t id = static_cast<uint32_t>(row) * kMaxBuckets + tid;
+                atomicOr(&stable.range[2 * id], static_cast<unsigned long long>(static_cast<K>(own_first | vary_here)));
+                atomicAnd(&stable.range[2 * id + 1], static_cast<unsigned long long>(static_cast<K>(own_first & ~vary_here)) | ~static_cast<unsigned long long>(~K(0)));
+            }
+            continue;
+        } else {
             K* dk = io.kbuf[0] + row_off;
             uint32_t* dv = PAIRS ? io.vbuf[0] + row_off : nullptr;
             int32_t at[ITEMS];                         // where tile position k * BLOCK + tid goes in the row
@@ -906,7 +1091,7 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK>&
         __syncthreads();                                   // the tile in LDS has left
     }
     };
-    if (MAP == kMapValue && fine_of.by_value) move_chunk(std::integral_constant<bool, MAP == kMapValue>());
+    if ((MAP == kMapValue || MAP == kMapAny) && fine_of.by_value) move_chunk(std::integral_constant<bool, MAP == kMapValue || MAP == kMapAny>());
     else move_chunk(std::false_type());
 }
 
@@ -920,7 +1105,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
     const int64_t row = blockIdx.x / chunks_per_row;
     const int64_t c = blockIdx.x - row * chunks_per_row;
     const SplitRow& info = infos[row];
-    if (PAIRS && info.route != 1u) return;             // (a row with buckets larger than a workgroup holds: split_pass_stable)
+    if (info.route != 1u) return;                      // (a row with buckets larger than a workgroup holds: split_pass_stable)
     const int64_t chunk_lo = c * kChunk;
     const int64_t chunk_hi = (chunk_lo + kChunk < n) ? chunk_lo + kChunk : n;
     scatter_to_buckets<K, PAIRS, BLOCK, MAP, true>(sm, io, n, row, info, chunk_lo, chunk_hi, chunk_base + static_cast<int64_t>(blockIdx.x) * kMaxBuckets);
@@ -937,7 +1122,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
 template <typename K, bool PAIRS, int BLOCK, int MAP>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void split_front(PassIo<K> io, int64_t n, uint32_t cap, SplitRow* __restrict__ rows,
                                                            uint32_t* __restrict__ counters, uint4* __restrict__ bucket_list,
-                                                           uint32_t* __restrict__ crowded_list) {
+                                                           CrowdedList crowded) {
     static_assert(MAP != kMapValue, "rows short enough for the smallest buckets");
     __shared__ SplitShared<K, PAIRS, BLOCK> sm;
     __shared__ PlanShared<BLOCK> plan;
@@ -957,8 +1142,8 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
 #pragma unroll
     for (int i = 0; i < PER; ++i) cnt[i] = threadIdx.x < kSplitBlock ? hist[threadIdx.x * PER + i] : 0u;
     uint32_t route = 0;
-    (void)plan_buckets<BLOCK>(plan, cnt, bucket, n, cap, row, info, counters, bucket_list, crowded_list, &route);
-    if (PAIRS && route != 1u) return;
+    (void)plan_buckets<BLOCK>(plan, cnt, bucket, n, cap, row, info, counters, bucket_list, crowded, &route);
+    if (route != 1u) return;
     __syncthreads();                                   // the row's record and table are in memory, the histogram has been read
     scatter_to_buckets<K, PAIRS, BLOCK, MAP, true>(sm, io, n, row, info, 0, n, plan.begin);
 }
@@ -967,89 +1152,30 @@ __global__ void split_clear(uint32_t* __restrict__ counters) {
     if (threadIdx.x < 4) counters[threadIdx.x] = 0u;
 }
 
-// The same pass for the rows (of pairs) that have buckets larger than a workgroup holds
-// (SplitRow::route 2): every key's slot among the tile's keys of its bucket is its rank in
-// element order (wave-wide matching of bucket numbers, as the digit passes rank), so each bucket
-// receives its entries in index order and a bucket of one repeated value arrives sorted.  Entries
-// go straight to their places in the row; a tile is 256 threads x 16 keys, wavefront w taking
-// elements [1024 w, 1024 w + 1024) of it.
-template <typename K>
-__global__ __launch_bounds__(kSplitBlock) void split_pass_stable(PassIo<K> io, int64_t n, int64_t chunks_per_row, int64_t chunks,
-                                                                 const SplitRow* __restrict__ infos, const uint32_t* __restrict__ counters,
-                                                                 const uint32_t* __restrict__ chunk_base) {
-    constexpr int ITEMS = kSplitItems;
-    constexpr int WAVES = kSplitBlock / kWave;
-    constexpr int TILE = kSplitBlock * ITEMS;
-    __shared__ uint32_t table[kFine / 4];
-    __shared__ uint32_t wave_hist[WAVES][kMaxBuckets];
-    __shared__ uint32_t place[kMaxBuckets];            // row position of the tile's first entry of each bucket
-    const int tid = threadIdx.x;
-    const int lane = lane_id();
-    const int w = tid / kWave;
-    if (counters[3] == 0u) return;                     // no such row in this call (the usual case)
-    // (a small grid walks the chunks: the launch costs little when there is nothing to do)
-    // (without chunk tables - split_front made the plan - a unit is a whole row)
-    for (int64_t unit = blockIdx.x; unit < chunks; unit += gridDim.x) {
-    const int64_t row = chunk_base ? unit / chunks_per_row : unit;
-    const int64_t c = chunk_base ? unit - row * chunks_per_row : 0;
-    const SplitRow& info = infos[row];
-    if (info.route != 2u) continue;
-    __syncthreads();                                   // the chunk before has left the table
-    const FineMap<K> fine_of(info, io.descending);
-    const K* xrow = io.x + io.xmap.at(row);
-    K* dk = io.kbuf[0] + row * n;
-    uint32_t* dv = io.vbuf[0] + row * n;
-    const int64_t chunk_lo = c * kChunk;
-    const int64_t chunk_hi = (chunk_base && chunk_lo + kChunk < n) ? chunk_lo + kChunk : n;
-    // bucket numbers lie below n_buckets: only those bits are matched
-    const uint32_t vary = info.n_buckets > 1u ? (2u << (31 - __builtin_clz(info.n_buckets - 1u))) - 1u : 0u;
-    static_assert(kSplitBlock == kMaxBuckets, "a thread per bucket");
-    reinterpret_cast<uint4*>(table)[tid] = reinterpret_cast<const uint4*>(info.bucket_of)[tid];
-    uint32_t next = chunk_base ? chunk_base[unit * kMaxBuckets + tid] : info.begin[tid];      // where this unit's coming keys of bucket tid go
-    for (int64_t tile_base = chunk_lo; tile_base < chunk_hi; tile_base += TILE) {
-        for (int i = tid; i < WAVES * kMaxBuckets; i += kSplitBlock) (&wave_hist[0][0])[i] = 0u;
-        K key[ITEMS];
-        uint32_t bucket[ITEMS], rank[ITEMS];
-#pragma unroll
-        for (int k = 0; k < ITEMS; ++k) {
-            const int64_t e = tile_base + w * (kWave * ITEMS) + k * kWave + lane;
-            key[k] = key_of_element<K>(io, xrow[(e < chunk_hi ? e : chunk_lo) * io.sx]);
-        }
-        __syncthreads();                               // table and zeroed counts are in place
-#pragma unroll
-        for (int k = 0; k < ITEMS; ++k) {
-            const uint32_t f = fine_of(key[k]);
-            bucket[k] = (table[f >> 2] >> (8u * (f & 3u))) & 0xffu;
-            // (elements beyond the chunk's end come after every element of it: whatever bucket
-            // they are counted in, no rank of an element of the chunk changes, and the counts are
-            // never used again after a chunk's last tile)
-        }
-        rank_by_digit<ITEMS>(wave_hist[w], bucket, vary, rank);
-        __syncthreads();
-        {
-            // thread b owns bucket b: each wavefront's share of it starts after the shares of the wavefronts before
-            uint32_t run = 0;
-#pragma unroll
-            for (int i = 0; i < WAVES; ++i) {
-                const uint32_t count = wave_hist[i][tid];
-                wave_hist[i][tid] = run;
-                run += count;
-            }
-            place[tid] = next;
-            next += run;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int k = 0; k < ITEMS; ++k) {
-            const int64_t e = tile_base + w * (kWave * ITEMS) + k * kWave + lane;
-            if (e < chunk_hi) {
-                const uint32_t at = place[bucket[k]] + wave_hist[w][bucket[k]] + rank[k];
-                dk[at] = key[k];
-                dv[at] = static_cast<uint32_t>(e);
-            }
-        }
-        __syncthreads();                               // the counts and places have been read
-    }
+// The stable pass for the rows that have buckets larger than a workgroup holds (SplitRow::route
+// 2).  A small grid walks the units - chunks, or whole rows when split_front made the plan and
+// left no chunk tables - so the launch costs little in the usual case of no such row.
+constexpr int kStableBlock = 512;
+template <typename K, bool PAIRS>
+__global__ __launch_bounds__(kStableBlock) void split_pass_stable(PassIo<K> io, int64_t n, uint32_t cap, int64_t chunks_per_row, int64_t units,
+                                                                  const SplitRow* __restrict__ infos, const uint32_t* __restrict__ counters,
+                                                                  const uint32_t* __restrict__ chunk_base, unsigned long long* __restrict__ range) {
+    static_assert(kChunk % (kStableBlock * kSplitItems) == 0, "whole tiles a chunk");
+    __shared__ SplitShared<K, PAIRS, kStableBlock, true> sm;
+    if (counters[3] == 0u) return;                     // no such row in this call
+    for (int64_t unit = blockIdx.x; unit < units; unit += gridDim.x) {
+        const int64_t row = chunk_base ? unit / chunks_per_row : unit;
+        const int64_t c = chunk_base ? unit - row * chunks_per_row : 0;
+        const SplitRow& info = infos[row];
+        if (info.route != 2u) continue;
+        const int64_t chunk_lo = c * kChunk;
+        const int64_t chunk_hi = (chunk_base && chunk_lo + kChunk < n) ? chunk_lo + kChunk : n;
+        __syncthreads();                               // the unit before has left the tables
+        scatter_to_buckets<K, PAIRS, kStableBlock, kMapAny, false, true>(sm, io, n, row, info, chunk_lo, chunk_hi,
+                                                                        chunk_base ? chunk_base + unit * kMaxBuckets : info.begin,
+                                                                        StablePass<K>{cap, range, io.y ? io.y + io.ymap.at(row) : nullptr, PAIRS ? io.idx : nullptr,
+                                                                                      (PAIRS && io.idx) ? io.imap.at(row) : 0, io.sx, io.sy, io.si, io.idx64,
+                                                                                      io.kind, io.descending, PAIRS ? io.restore_zero : 0, io.x_intact != 0});
     }
 }
 
@@ -1071,35 +1197,6 @@ struct FinishShared {
     uint32_t crowded;
 };
 
-// Where bucket `id` = row * 256 + b lies: {row, first position in the row, entries, id}.
-__device__ __forceinline__ uint4 bucket_at(const SplitRow* __restrict__ infos, uint32_t id) {
-    const uint32_t row = id / kMaxBuckets, b = id % kMaxBuckets;
-    const SplitRow& info = infos[row];
-    const uint32_t b0 = info.begin[b];
-    return make_uint4(row, b0, info.begin[b + 1] - b0, id);
-}
-
-// Entry `at` of the sorted row goes to the strided outputs (unit strides: plain 32-bit offsets
-// from the row's start, the case every contiguous output takes).
-template <typename K, bool PAIRS>
-__device__ __forceinline__ void emit_entry(const PassIo<K>& io, const K* xrow, K* yrow, int64_t irow, int64_t at, K key, uint32_t val) {
-    if (yrow) {
-        K bits = decode_key<K>(key, io.kind, io.descending);
-        if constexpr (PAIRS) {
-            if (io.restore_zero && static_cast<K>(bits << 1) == 0) bits = xrow[static_cast<int64_t>(val) * io.sx];
-        }
-        if (io.sy == 1) yrow[static_cast<uint32_t>(at)] = bits;
-        else yrow[at * io.sy] = bits;
-    }
-    if constexpr (PAIRS) {
-        if (io.idx) {
-            if (io.si == 1 && !io.idx64) (static_cast<int32_t*>(io.idx) + irow)[static_cast<uint32_t>(at)] = static_cast<int32_t>(val);
-            else if (io.idx64) static_cast<int64_t*>(io.idx)[irow + at * io.si] = static_cast<int64_t>(val);
-            else static_cast<int32_t*>(io.idx)[irow + at * io.si] = static_cast<int32_t>(val);
-        }
-    }
-}
-
 // Workgroup g takes entries g, g + G, ... of the bucket list (what split_plan wrote: row, first
 // position, size of every bucket); once a bucket lies in LDS the registers already receive the
 // next one's entries.  A bucket whose bins are too crowded to rank by comparison is put on
@@ -1107,7 +1204,7 @@ __device__ __forceinline__ void emit_entry(const PassIo<K>& io, const K* xrow, K
 template <typename K, bool PAIRS, int WAVES>
 __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4))) void split_finish(PassIo<K> io, int64_t n,
                                                              uint32_t compare_max, uint32_t* __restrict__ counters,
-                                                             const uint4* __restrict__ bucket_list, uint32_t* __restrict__ crowded_list) {
+                                                             const uint4* __restrict__ bucket_list, uint2* __restrict__ crowded_list) {
     constexpr int ITEMS = kFinishItems;
     constexpr int T = WAVES * kWave;
     constexpr int kBins = finish_bins(WAVES);
@@ -1301,7 +1398,7 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
 
             if (compare && sm.crowded != 0u) {
                 // many equal or clustered keys: the stable digit passes of split_finish_crowded take this bucket
-                if (tid == 0) crowded_list[atomicAdd(&counters[1], 1u)] = cur.w;
+                if (tid == 0) crowded_list[atomicAdd(&counters[1], 1u)] = make_uint2(cur.w, kNoWindow);
                 if (vn < total) load_bucket(nxt, key, val);
                 return;
             }
@@ -1441,25 +1538,34 @@ __global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4
 // value is just copied - and an even number of passes is preceded by a plain copy to B.
 template <typename K, bool PAIRS>
 struct OversizedIo {
-    const PassIo<K>& io;
+    // (what it needs of PassIo, by value: a reference to the kernel's argument block made the
+    // compiler keep a private copy of the whole block in scratch memory)
     const K* xrow;
     K* yrow;
-    int64_t irow;
+    void* idx;
+    int64_t irow, sx, sy, si;
+    int idx64, kind, descending, canon_zero, restore_zero;
     K* ak;                                             // side A
     uint32_t* av;
-    __device__ __forceinline__ void read(bool side_b, int64_t at, K* key, uint32_t* val) const {
+    __device__ __forceinline__ K image_of(K bits) const {
+        if (canon_zero && static_cast<K>(bits << 1) == 0) bits = 0;
+        return encode_key<K>(bits, kind, descending);
+    }
+    // (values: side B holds what split_pass_stable emitted - values, not key images)
+    __device__ __forceinline__ void read(bool side_b, int64_t at, K* key, uint32_t* val, bool values = false) const {
         if (!side_b) {
             *key = ak[at];
             if constexpr (PAIRS) *val = av[at];
             return;
         }
         if constexpr (PAIRS) {
-            *val = io.idx64 ? static_cast<uint32_t>(static_cast<const int64_t*>(io.idx)[irow + at * io.si])
-                            : static_cast<uint32_t>(static_cast<const int32_t*>(io.idx)[irow + at * io.si]);
-            *key = yrow ? yrow[at * io.sy] : key_of_element<K>(io, xrow[static_cast<int64_t>(*val) * io.sx]);
+            *val = idx64 ? static_cast<uint32_t>(static_cast<const int64_t*>(idx)[irow + at * si])
+                         : static_cast<uint32_t>(static_cast<const int32_t*>(idx)[irow + at * si]);
+            *key = yrow ? yrow[at * sy] : image_of(xrow[static_cast<int64_t>(*val) * sx]);
         } else {
-            *key = yrow[at * io.sy];
+            *key = yrow[at * sy];
         }
+        if (values && yrow) *key = image_of(*key);
     }
     __device__ __forceinline__ void write(bool side_b, int64_t at, K key, uint32_t val) const {
         if (!side_b) {
@@ -1467,10 +1573,26 @@ struct OversizedIo {
             if constexpr (PAIRS) av[at] = val;
             return;
         }
-        if (yrow) yrow[at * io.sy] = key;
+        if (yrow) yrow[at * sy] = key;
         if constexpr (PAIRS) {
-            if (io.idx64) static_cast<int64_t*>(io.idx)[irow + at * io.si] = static_cast<int64_t>(val);
-            else static_cast<int32_t*>(io.idx)[irow + at * io.si] = static_cast<int32_t>(val);
+            if (idx64) static_cast<int64_t*>(idx)[irow + at * si] = static_cast<int64_t>(val);
+            else static_cast<int32_t*>(idx)[irow + at * si] = static_cast<int32_t>(val);
+        }
+    }
+    // entry `at` of the sorted row leaves for good
+    __device__ __forceinline__ void emit(int64_t at, K key, uint32_t val) const {
+        if (yrow) {
+            K bits = decode_key<K>(key, kind, descending);
+            if constexpr (PAIRS) {
+                if (restore_zero && static_cast<K>(bits << 1) == 0) bits = xrow[static_cast<int64_t>(val) * sx];
+            }
+            yrow[at * sy] = bits;
+        }
+        if constexpr (PAIRS) {
+            if (idx) {
+                if (idx64) static_cast<int64_t*>(idx)[irow + at * si] = static_cast<int64_t>(val);
+                else static_cast<int32_t*>(idx)[irow + at * si] = static_cast<int32_t>(val);
+            }
         }
     }
 };
@@ -1479,7 +1601,8 @@ struct OversizedIo {
 // whose index output overwrites the input (side B cannot hold keys and they cannot be read again
 // either); the caller then sorts the bucket where it lies.
 template <typename K, bool PAIRS, int WAVES>
-__device__ __forceinline__ bool sort_oversized(SmallShared<K, PAIRS, kFinishItems, WAVES>& sm, const PassIo<K>& io, int64_t n, int64_t row, int64_t begin, int64_t size) {
+__device__ __forceinline__ bool sort_oversized(SmallShared<K, PAIRS, kFinishItems, WAVES>& sm, const PassIo<K>& io, int64_t n, int64_t row, int64_t begin, int64_t size, bool in_b,
+                                               unsigned long long ors, unsigned long long ands, const K* xrow, K* yrow, int64_t irow) {
     constexpr int ITEMS = kFinishItems;
     constexpr int T = WAVES * kWave;
     constexpr int WINDOW = T * ITEMS;
@@ -1488,39 +1611,20 @@ __device__ __forceinline__ bool sort_oversized(SmallShared<K, PAIRS, kFinishItem
     const int lane = lane_id();
     const int w = tid / kWave;
     const int seg = w * kWave * ITEMS + lane;
-    OversizedIo<K, PAIRS> mem{io, io.x + io.xmap.at(row), io.y ? io.y + io.ymap.at(row) : nullptr, (PAIRS && io.idx) ? io.imap.at(row) : 0,
-                              io.kbuf[0] + row * n, PAIRS ? io.vbuf[0] + row * n : nullptr};
+    OversizedIo<K, PAIRS> mem{xrow, yrow, PAIRS ? io.idx : nullptr, irow, io.sx, io.sy, io.si, io.idx64, io.kind, io.descending, io.canon_zero,
+                              io.restore_zero, io.kbuf[0] + row * n, PAIRS ? io.vbuf[0] + row * n : nullptr};
+    const bool x_intact = io.x_intact != 0;
 
-    // ---- which bits differ inside the bucket
-    K ors = 0, ands = ~K(0);
-    for (int64_t i = tid; i < size; i += T) {
-        const K k1 = mem.ak[begin + i];
-        ors |= k1;
-        ands &= k1;
-    }
-    ors = wave_reduce(ors, [](K a, K b) { return static_cast<K>(a | b); });
-    ands = wave_reduce(ands, [](K a, K b) { return static_cast<K>(a & b); });
-    __syncthreads();
-    if (lane == 0) {
-        sm.wave_or[w] = ors;
-        sm.wave_and[w] = ands;
-    }
-    __syncthreads();
-    K any = 0, all = ~K(0);
-#pragma unroll
-    for (int i = 0; i < WAVES; ++i) {
-        any |= sm.wave_or[i];
-        all &= sm.wave_and[i];
-    }
-    const K differ = static_cast<K>(any & ~all);
+    // ---- the bits that differ inside the bucket (split_pass_stable gathered its keys' OR and AND)
+    const K all = static_cast<K>(ands);
+    const K differ = static_cast<K>(static_cast<K>(ors) & ~all);
+    constexpr int U = WAVES >= 16 ? 2 : 8;             // entries in flight a thread where the bucket is only streamed
     int passes = 0;
     for (int p = 0; p < KeyTraits<K>::kPasses; ++p) passes += (static_cast<uint32_t>(differ >> (8 * p)) & 0xffu) != 0u ? 1 : 0;
 
-    // entry `at` of the sorted row leaves for good
-    auto emit = [&](int64_t at, K k1, uint32_t v1) __attribute__((always_inline)) {
-        emit_entry<K, PAIRS>(io, mem.xrow, mem.yrow, mem.irow, at, k1, v1);
-    };
+    auto emit = [&](int64_t at, K k1, uint32_t v1) __attribute__((always_inline)) { mem.emit(at, k1, v1); };
     if (passes == 0) {                                 // one value: pairs are in index order already
+        if (in_b) return true;
         for (int64_t i = tid; i < size; i += T) {
             K k1;
             uint32_t v1 = 0;
@@ -1529,17 +1633,27 @@ __device__ __forceinline__ bool sort_oversized(SmallShared<K, PAIRS, kFinishItem
         }
         return true;
     }
-    if (PAIRS && !mem.yrow && !io.x_intact) return false;
+    if (PAIRS && !mem.yrow && !x_intact) return false;
 
-    bool from_b = false;
-    if (passes % 2 == 0) {                             // so that the last pass goes from A to B
-        for (int64_t i = tid; i < size; i += T) {
-            K k1;
-            uint32_t v1 = 0;
-            mem.read(false, begin + i, &k1, &v1);
-            mem.write(true, begin + i, k1, v1);
+    bool from_b = in_b, b_values = in_b;               // (values: side B still holds what split_pass_stable emitted)
+    if ((passes % 2 == 0) != in_b) {                   // so that the last pass goes from A to B
+        for (int64_t i0 = 0; i0 < size; i0 += U * T) {
+            K k1[U];
+            uint32_t v1[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t i = i0 + u * T + tid;
+                v1[u] = 0u;
+                mem.read(from_b, begin + (i < size ? i : 0), &k1[u], &v1[u], b_values);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t i = i0 + u * T + tid;
+                if (i < size) mem.write(!from_b, begin + i, k1[u], v1[u]);
+            }
         }
-        from_b = true;
+        from_b = !from_b;
+        b_values = false;
         __syncthreads();
     }
     int left = passes;
@@ -1551,11 +1665,17 @@ __device__ __forceinline__ bool sort_oversized(SmallShared<K, PAIRS, kFinishItem
         // ---- how many entries carry each digit, and from that where each digit's run starts
         for (int i = tid; i < kRadix; i += T) digit_at[i] = 0u;
         __syncthreads();
-        for (int64_t i = tid; i < size; i += T) {
-            K k1;
-            uint32_t v1 = 0;
-            mem.read(from_b, begin + i, &k1, &v1);
-            atomicAdd(&digit_at[static_cast<uint32_t>(k1 >> shift) & 0xffu], 1u);
+        for (int64_t i0 = 0; i0 < size; i0 += U * T) {
+            K k1[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t i = i0 + u * T + tid;
+                uint32_t v1 = 0;
+                mem.read(from_b, begin + (i < size ? i : 0), &k1[u], &v1, b_values);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (i0 + u * T + tid < size) atomicAdd(&digit_at[static_cast<uint32_t>(k1[u] >> shift) & 0xffu], 1u);
         }
         __syncthreads();
         {
@@ -1580,7 +1700,7 @@ __device__ __forceinline__ bool sort_oversized(SmallShared<K, PAIRS, kFinishItem
                 const int64_t e = lo + seg + k * kWave;
                 key[k] = all;                          // padding agrees with the bucket in every bit that does not vary
                 if constexpr (PAIRS) val[k] = 0u;
-                if (e < size) mem.read(from_b, begin + e, &key[k], &val[PAIRS ? k : 0]);
+                if (e < size) mem.read(from_b, begin + e, &key[k], &val[PAIRS ? k : 0], b_values);
                 digit[k] = static_cast<uint32_t>(key[k] >> shift) & 0xffu;
             }
             __syncthreads();                           // zeroed counts and digit_at are in place
@@ -1608,28 +1728,65 @@ __device__ __forceinline__ bool sort_oversized(SmallShared<K, PAIRS, kFinishItem
             __syncthreads();
         }
         from_b = !from_b;
+        b_values = false;
     }
     return true;
 }
 
 // The buckets split_finish left: stable digit passes on chip - for pairs first by index (the
 // entries arrive in no particular order), then by key - and the buckets larger than a workgroup
-// holds, which split_plan put on the same list.
+// holds, which split_plan put on the same list, an entry per window of kOverWindow entries.
+//
+// split_pass_stable left the smallest and the largest key of every oversized bucket: when they
+// are equal - one repeated value, whose pairs arrived in index order - every window of the bucket
+// is copied out as it lies, by as many workgroups as the bucket has windows; otherwise the
+// workgroup that draws the bucket's first window sorts it whole (sort_oversized).
 template <typename K, bool PAIRS, int WAVES>
 __global__ __launch_bounds__(WAVES * kWave) void split_finish_crowded(PassIo<K> io, int64_t n, const SplitRow* __restrict__ infos,
-                                                                     const uint32_t* __restrict__ counters,
-                                                                     const uint32_t* __restrict__ crowded_list) {
+                                                                     const uint32_t* __restrict__ counters, CrowdedList crowded) {
     constexpr int ITEMS = kFinishItems;
+    constexpr int T = WAVES * kWave;
     __shared__ SmallShared<K, PAIRS, ITEMS, WAVES> sm;
     const uint32_t listed = counters[1];
     const int lane = lane_id();
     const int seg = (threadIdx.x / kWave) * kWave * ITEMS + lane;
     for (uint32_t i = blockIdx.x; i < listed; i += gridDim.x) {
-        const uint4 at = bucket_at(infos, crowded_list[i]);
+        const uint2 item = crowded.items[i];
+        const uint4 at = bucket_at(infos, item.x);
         const int64_t at_row = at.x, at_begin = at.y;
-        if (at.z > static_cast<uint32_t>(finish_cap(WAVES))) {
-            (void)sort_oversized<K, PAIRS, WAVES>(sm, io, n, at_row, at_begin, at.z);      // (what it does not take: split_finish_in_place)
-            __syncthreads();
+        if (item.y != kNoWindow) {
+            const int64_t size = at.z;
+            const K* ak = io.kbuf[0] + at_row * n + at_begin;
+            const uint32_t* av = PAIRS ? io.vbuf[0] + at_row * n + at_begin : nullptr;
+            const K* xrow = io.x + io.xmap.at(at_row);
+            K* yrow = io.y ? io.y + io.ymap.at(at_row) : nullptr;
+            const int64_t irow = (PAIRS && io.idx) ? io.imap.at(at_row) : 0;
+            if (static_cast<K>(crowded.range[2 * item.x]) != static_cast<K>(crowded.range[2 * item.x + 1])) {
+                if (item.y == 0u) {
+                    (void)sort_oversized<K, PAIRS, WAVES>(sm, io, n, at_row, at_begin, size, io.x_intact != 0, crowded.range[2 * item.x], crowded.range[2 * item.x + 1], xrow, yrow, irow);      // (what it does not take: split_finish_in_place)
+                    __syncthreads();
+                }
+                continue;
+            }
+            if (io.x_intact) continue;                 // one value, and split_pass_stable wrote it to the outputs
+            const int64_t lo = static_cast<int64_t>(item.y) * kOverWindow;
+            const int64_t hi = lo + kOverWindow < size ? lo + kOverWindow : size;
+            constexpr int U = WAVES >= 16 ? 2 : 8;                     // entries in flight a thread (the registers of 1024 threads allow two)
+            for (int64_t e0 = lo; e0 < hi; e0 += U * T) {
+                K key[U];
+                uint32_t val[PAIRS ? U : 1];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int64_t e = e0 + u * T + threadIdx.x;
+                    key[u] = ak[e < hi ? e : lo];
+                    if constexpr (PAIRS) val[u] = av[e < hi ? e : lo];
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int64_t e = e0 + u * T + threadIdx.x;
+                    if (e < hi) emit_entry<K, PAIRS>(io, xrow, yrow, irow, at_begin + e, key[u], PAIRS ? val[u] : 0u);
+                }
+            }
             continue;
         }
         const int valid = static_cast<int>(at.z);
@@ -1676,8 +1833,7 @@ __global__ __launch_bounds__(WAVES * kWave) void split_finish_crowded(PassIo<K> 
 // (the work grows with the square of the bucket), and only for this combination.
 template <typename K, int WAVES>
 __global__ __launch_bounds__(WAVES * kWave) void split_finish_in_place(PassIo<K> io, int64_t n, const SplitRow* __restrict__ infos,
-                                                                      const uint32_t* __restrict__ counters,
-                                                                      const uint32_t* __restrict__ crowded_list) {
+                                                                      const uint32_t* __restrict__ counters, CrowdedList crowded) {
     constexpr int ITEMS = kFinishItems;
     constexpr int T = WAVES * kWave, WINDOW = T * ITEMS, HALF = WINDOW / 2;
     __shared__ SmallShared<K, true, ITEMS, WAVES> sm;
@@ -1686,33 +1842,13 @@ __global__ __launch_bounds__(WAVES * kWave) void split_finish_in_place(PassIo<K>
     const int w = threadIdx.x / kWave;
     const int seg = w * kWave * ITEMS + lane;
     for (uint32_t i = blockIdx.x; i < listed; i += gridDim.x) {
-        const uint4 at = bucket_at(infos, crowded_list[i]);
+        // the first window's entry stands for its bucket; a bucket of one value has been copied out
+        const uint2 item = crowded.items[i];
+        if (item.y != 0u || static_cast<K>(crowded.range[2 * item.x]) == static_cast<K>(crowded.range[2 * item.x + 1])) continue;
+        const uint4 at = bucket_at(infos, item.x);
         const int64_t size = at.z;
-        if (size <= WINDOW) continue;
         K* ak = io.kbuf[0] + static_cast<int64_t>(at.x) * n + at.y;
         uint32_t* av = io.vbuf[0] + static_cast<int64_t>(at.x) * n + at.y;
-        // a bucket of one value was copied out by split_finish_crowded
-        K kor = 0, kand = ~K(0);
-        for (int64_t e = threadIdx.x; e < size; e += T) {
-            kor |= ak[e];
-            kand &= ak[e];
-        }
-        kor = wave_reduce(kor, [](K a, K b) { return static_cast<K>(a | b); });
-        kand = wave_reduce(kand, [](K a, K b) { return static_cast<K>(a & b); });
-        __syncthreads();
-        if (lane == 0) {
-            sm.wave_or[w] = kor;
-            sm.wave_and[w] = kand;
-        }
-        __syncthreads();
-        K any = 0, all = ~K(0);
-#pragma unroll
-        for (int j = 0; j < WAVES; ++j) {
-            any |= sm.wave_or[j];
-            all &= sm.wave_and[j];
-        }
-        __syncthreads();
-        if (any == all) continue;
         const int64_t halves = (size + HALF - 1) / HALF;
 #pragma unroll 1
         for (int64_t round = 0; round < halves; ++round) {
@@ -1761,7 +1897,7 @@ __global__ __launch_bounds__(WAVES * kWave) void split_finish_in_place(PassIo<K>
 
 struct SplitLayout {
     int64_t chunks_per_row;
-    size_t counters_off, rows_off, list_off, crowded_off, fine_off, base_off, total;
+    size_t counters_off, rows_off, list_off, crowded_off, state_off, fine_off, base_off, total;
 };
 
 SplitLayout split_layout(int64_t m, int64_t n) {
@@ -1774,8 +1910,11 @@ SplitLayout split_layout(int64_t m, int64_t n) {
     off += align_up(static_cast<size_t>(m) * sizeof(SplitRow), 256);
     l.list_off = off;            // {row, begin, size, id} of every bucket
     off += align_up(static_cast<size_t>(m) * kMaxBuckets * 16, 256);
-    l.crowded_off = off;
-    off += align_up(static_cast<size_t>(m) * kMaxBuckets * 4, 256);
+    l.crowded_off = off;         // {id, window}: a bucket is crowded or oversized, and an oversized one has a window per kOverWindow entries
+    static_assert(kOverWindow == kChunk, "as many windows a row as chunks, at most");
+    off += align_up(static_cast<size_t>(m) * (kMaxBuckets + l.chunks_per_row) * 8, 256);
+    l.state_off = off;           // OR and AND of the keys of every (oversized) bucket
+    off += align_up(static_cast<size_t>(m) * kMaxBuckets * 16, 256);
     l.fine_off = off;            // fine-bin histogram of every chunk, two counts a word
     off += align_up(static_cast<size_t>(m) * l.chunks_per_row * (kFine / 2) * 4, 256);
     l.base_off = off;            // where every chunk writes each bucket
@@ -1807,7 +1946,7 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
     uint32_t* counters = reinterpret_cast<uint32_t*>(base + l.counters_off);
     SplitRow* rows = reinterpret_cast<SplitRow*>(base + l.rows_off);
     uint4* list = reinterpret_cast<uint4*>(base + l.list_off);
-    uint32_t* crowded = reinterpret_cast<uint32_t*>(base + l.crowded_off);
+    const CrowdedList crowded = {reinterpret_cast<uint2*>(base + l.crowded_off), reinterpret_cast<unsigned long long*>(base + l.state_off)};
     uint32_t* fine = reinterpret_cast<uint32_t*>(base + l.fine_off);
     uint32_t* chunk_base = reinterpret_cast<uint32_t*>(base + l.base_off);
 
@@ -1874,14 +2013,14 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         else if (block == 512) pass_of(std::integral_constant<int, 512>());
         else if constexpr (kPassBlockMax<K, PAIRS> >= 1024) pass_of(std::integral_constant<int, 1024>());
         DLFX_CHECK_LAUNCH();
-        if constexpr (PAIRS) {
+        {
             // rows with buckets larger than a workgroup holds (as a rule none: every workgroup leaves at once)
             const int64_t units = front ? m : m * l.chunks_per_row;
-            split_pass_stable<K><<<dim3(static_cast<unsigned>(units < 1024 ? units : 1024)), dim3(kSplitBlock), 0, stream>>>(
-                io, n, l.chunks_per_row, units, rows, counters, front ? nullptr : chunk_base);
+            split_pass_stable<K, PAIRS><<<dim3(static_cast<unsigned>(units < 1024 ? units : 1024)), dim3(kStableBlock), 0, stream>>>(
+                io, n, static_cast<uint32_t>(cap), l.chunks_per_row, units, rows, counters, front ? nullptr : chunk_base, crowded.range);
             DLFX_CHECK_LAUNCH();
         }
-        split_finish<K, PAIRS, WAVES><<<fgrid, dim3(WAVES * kWave), 0, stream>>>(io, n, limit, counters, list, crowded);
+        split_finish<K, PAIRS, WAVES><<<fgrid, dim3(WAVES * kWave), 0, stream>>>(io, n, limit, counters, list, crowded.items);
         DLFX_CHECK_LAUNCH();
         // (a smaller grid for this launch, which as a rule finds little to do, was measured: the
         // same for the benchmark rows, up to 15 % slower on bell-shaped rows, whose buckets are often crowded)
