@@ -114,6 +114,19 @@ struct CrowdedList {
     unsigned long long* range;             // [2 id]: OR of the bucket's keys, [2 id + 1]: AND
 };
 
+// A row whose keys cluster more tightly than evenly spaced fine bins resolve gets a map made from
+// the quantiles of a sample instead: the sorted sample's every 16th key bounds a segment, 256 of
+// them, and a segment has 16 fine bins - the first for the bounding key itself (a value repeated
+// so often that it bounds segments gets a bin, and then a bucket, to itself), the others spread
+// evenly over the keys up to the next bound.
+constexpr int kSegments = 256;
+constexpr int kSegmentBins = kFine / kSegments;
+constexpr int kQuantileSample = kSegments * 16;       // keys sampled for the bounds
+struct alignas(16) PiecewiseMap {
+    unsigned long long bound[kSegments];   // bound[0] = 0: every key has a segment
+    uint8_t shift[kSegments];              // bin of a key above its bound: 1 + min((key - bound - 1) >> shift, 14)
+};
+
 // What split_sample and split_plan decide for a row.
 struct alignas(16) SplitRow {
     uint32_t route;                        // 1: this row takes the bucket route, 0: the digit passes
@@ -125,6 +138,7 @@ struct alignas(16) SplitRow {
     unsigned long long lo_bits, scale_bits;    // by value: lo and scale as a float's / double's bits
     unsigned long long gap_lo, gap_hi;     // by key image, floats: keys in [gap_lo, gap_hi) count as gap_lo and the keys above move down by
                                            // the width of the gap (none: both all ones)
+    uint32_t piecewise, unused[3];         // 1: none of the above - the row's PiecewiseMap says where a key goes
     uint32_t begin[kMaxBuckets + 4];       // first position of each bucket in the row; begin[n_buckets] = n
     uint8_t bucket_of[kFine];              // fine bin -> bucket (16-byte aligned: tiles load it as vectors)
 };
@@ -149,14 +163,31 @@ struct FineMap {
     using F = typename FloatOf<K>::type;
     K base, top, gap_lo, gap_hi, less;     // less: -(gap_hi + base), what the image with the gap taken out is short of
     F lo, scale;
-    uint32_t shift, by_value;
+    uint32_t shift, by_value, piecewise;
     int descending;
+    const K* bound = nullptr;              // piecewise: the map's bounds and shifts (in LDS)
+    const uint8_t* bound_shift = nullptr;
     template <typename Row>                // a SplitRow, or the FineRange that goes into one
     __device__ FineMap(const Row& r, int desc)
         : base(static_cast<K>(r.base)), top(static_cast<K>(r.top)), gap_lo(static_cast<K>(r.gap_lo)), gap_hi(static_cast<K>(r.gap_hi)),
           less(static_cast<K>(K(0) - static_cast<K>(r.gap_hi) - static_cast<K>(r.base))),
           lo(bit_cast<F>(static_cast<K>(r.lo_bits))), scale(bit_cast<F>(static_cast<K>(r.scale_bits))), shift(r.shift),
-          by_value(r.by_value), descending(desc) {}
+          by_value(r.by_value), piecewise(r.piecewise), descending(desc) {}
+    // by the row's PiecewiseMap: the last segment whose bound is not above the key, then the bin inside it
+    __device__ __forceinline__ uint32_t bin_piecewise(K key) const {
+        uint32_t j = 0;
+#pragma unroll
+        for (int step = kSegments / 2; step > 0; step >>= 1) j += bound[j + step] <= key ? static_cast<uint32_t>(step) : 0u;
+        const K above = static_cast<K>(key - bound[j]);
+        const K sub = static_cast<K>(static_cast<K>(above - 1) >> bound_shift[j]);
+        return j * kSegmentBins + (above == 0 ? 0u : 1u + (sub < K(kSegmentBins - 2) ? static_cast<uint32_t>(sub) : static_cast<uint32_t>(kSegmentBins - 2)));
+    }
+    // MODE: 0 by key image, 1 by value, 2 piecewise (what the row's record says; the kernels branch once per workgroup)
+    template <int MODE, bool GAP>
+    __device__ __forceinline__ uint32_t bin_as(K key) const {
+        if constexpr (MODE == 2) return bin_piecewise(key);
+        else return bin<MODE == 1, GAP>(key);
+    }
     // the number a float key stands for, increasing with the key (so negated for descending sorts)
     __device__ __forceinline__ static F value_of(K key, int desc) {
         const F x = bit_cast<F>(decode_key<K>(key, kKeyFloat, desc));
@@ -248,13 +279,14 @@ __device__ __forceinline__ K wave_fourth(const K (&key)[4]) {
 // rows); 1 for float rows of middling length, whose images may have the gap around zero closed
 // up; 2 for longer float rows, by key image as they are or by value.  The kernels carry no code for what their
 // MAP leaves out.
-constexpr int kMapPlain = 0, kMapGap = 1, kMapValue = 2, kMapAny = 3;      // (any: decided per row as the kernel runs)
+constexpr int kMapPlain = 0, kMapGap = 1, kMapValue = 2, kMapAny = 3, kMapPiecewise = 4;      // (any: what the row's record says, as the kernel runs)
 
 // How a row's keys spread over its fine bins (the part of SplitRow that split_sample decides).
 struct FineRange {
-    uint32_t shift, by_value;
+    uint32_t shift, by_value, piecewise;
     unsigned long long base, top, lo_bits, scale_bits, gap_lo, gap_hi;
     __device__ __forceinline__ void store(SplitRow& out) const {
+        out.piecewise = piecewise;
         out.shift = shift;
         out.base = base;
         out.by_value = by_value;
@@ -270,8 +302,14 @@ struct FineRange {
 // thread returns the same answer).  The sample is that of 256 threads whatever BLOCK is: further
 // wavefronts repeat the first four, which changes no minimum or maximum, and the lists of what
 // every wavefront offers are those of the first four.
+//
+// The sample also shows whether the row's keys cluster more tightly than the chosen map resolves:
+// a fine bin that holds so many of the sample's keys that it promises twice what a bucket may
+// hold, and keys that differ among them (one value repeated is no trouble: its bucket is done
+// when it has been moved).  Such a row is marked `piecewise`.  sample_hist: kFine words of LDS,
+// zero on entry and on return.
 template <typename K, int MAP, int BLOCK>
-__device__ __forceinline__ FineRange sample_row(const PassIo<K>& io, const K* __restrict__ xrow, int64_t n, uint32_t cap) {
+__device__ __forceinline__ FineRange sample_row(const PassIo<K>& io, const K* __restrict__ xrow, int64_t n, uint32_t cap, uint32_t* __restrict__ sample_hist) {
     static_assert(BLOCK % kSplitBlock == 0 && (MAP != kMapValue || BLOCK == kSplitBlock), "whole repeats of the sampling threads");
     __shared__ K red[BLOCK / kWave];
     const int st = threadIdx.x % kSplitBlock;          // the sampling thread this one is (or repeats)
@@ -388,17 +426,57 @@ __device__ __forceinline__ FineRange sample_row(const PassIo<K>& io, const K* __
             if (worst_value < worst_image && static_cast<unsigned long long>(worst_image) * static_cast<unsigned long long>(n) > static_cast<unsigned long long>(cap) * kFine) map = by_value;
         }
     }
+    map.piecewise = 0u;
+    if (n > static_cast<int64_t>(cap)) {
+        const FineMap<K> chosen(map, io.descending);
+        const bool sampler = threadIdx.x < kSplitBlock;    // (further threads repeat these keys)
+        uint32_t f[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            f[u] = chosen(key[u]);
+            if (sampler) atomicAdd(&sample_hist[f[u]], 1u);
+        }
+        __syncthreads();
+        const unsigned long long by_size = (2ull * cap * 1024ull + static_cast<unsigned long long>(n) - 1ull) / static_cast<unsigned long long>(n);
+        const uint32_t many = by_size > 8ull ? static_cast<uint32_t>(by_size) : 8u;       // (eight: never reached by chance on evenly spread keys)
+        bool crowded[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) crowded[u] = sampler && sample_hist[f[u]] >= many;
+        __syncthreads();
+        // every crowded bin's word now takes one of the bin's keys (folded to 32 bits), whichever lands last ...
+        auto folded = [](K k) { return static_cast<uint32_t>(k) ^ static_cast<uint32_t>(static_cast<unsigned long long>(k) >> 32); };
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (crowded[u]) sample_hist[f[u]] = folded(key[u]);
+        __syncthreads();
+        // ... and a key of the bin that differs from it says that the bin holds more than one value
+        bool mixed = false;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) mixed = mixed || (crowded[u] && sample_hist[f[u]] != folded(key[u]));
+        map.piecewise = __syncthreads_or(mixed ? 1 : 0) ? 1u : 0u;
+        if (sampler) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) sample_hist[f[u]] = 0u;
+        }
+        __syncthreads();
+    }
     return map;
 }
 
 template <typename K, int MAP>
 __global__ __launch_bounds__(kSplitBlock) void split_sample(PassIo<K> io, int64_t n, uint32_t cap, SplitRow* __restrict__ rows, uint32_t* __restrict__ counters) {
+    __shared__ uint32_t sample_hist[kFine];
     const int64_t row = blockIdx.x;
     if (row == 0 && threadIdx.x < 4) counters[threadIdx.x] = 0u;      // what the later launches of this sort count up from
-    const FineRange map = sample_row<K, MAP, kSplitBlock>(io, io.x + io.xmap.at(row), n, cap);
+    for (int i = threadIdx.x; i < kFine; i += kSplitBlock) sample_hist[i] = 0u;
+    const FineRange map = sample_row<K, MAP, kSplitBlock>(io, io.x + io.xmap.at(row), n, cap, sample_hist);
     if (threadIdx.x == 0) {
         rows[row].route = 0u;
         map.store(rows[row]);
+        // counters[4]: not zero when some row of the call has a piecewise map.  split_plan leaves
+        // it zero for the next sort; whatever else it may hold at first (new scratch memory)
+        // only makes split_remap look at every row's record once.
+        if (map.piecewise != 0u) atomicOr(&counters[4], 1u);
     }
 }
 
@@ -440,8 +518,8 @@ __device__ __forceinline__ void count_fine_bins(const PassIo<K>& io, const K* __
             key[u] = xrow[(i < hi ? i : lo) * io.sx];
         }
     };
-    auto count_chunk = [&](auto by_value_tag) __attribute__((always_inline)) {
-    constexpr bool BY_VALUE = decltype(by_value_tag)::value;
+    auto count_chunk = [&](auto mode_tag) __attribute__((always_inline)) {
+    constexpr int MODE = decltype(mode_tag)::value;
     constexpr bool GAP = MAP == kMapGap;               // (a branch per workgroup on whether the row has a gap: more registers, slower)
     K key[U];
     load_batch(lo, key);
@@ -451,7 +529,7 @@ __device__ __forceinline__ void count_fine_bins(const PassIo<K>& io, const K* __
         const bool full = b0 + BATCH <= hi;
         uint32_t f[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) f[u] = fine_of.template bin<BY_VALUE, GAP>(key_of_element<K>(io, key[u]));
+        for (int u = 0; u < U; ++u) f[u] = fine_of.template bin_as<MODE, GAP>(key_of_element<K>(io, key[u]));
         // a wave whose keys all share one fine bin (narrow ranges, few distinct values) adds once
         const uint32_t f0 = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(f[0])));
         bool same = full;
@@ -468,23 +546,37 @@ __device__ __forceinline__ void count_fine_bins(const PassIo<K>& io, const K* __
         for (int u = 0; u < U; ++u) key[u] = ahead[u];
     }
     };
-    if (MAP == kMapValue && fine_of.by_value) count_chunk(std::integral_constant<bool, MAP == kMapValue>());
-    else count_chunk(std::false_type());
+    if constexpr (MAP == kMapPiecewise) count_chunk(std::integral_constant<int, 2>());
+    else if (MAP == kMapValue && fine_of.by_value) count_chunk(std::integral_constant<int, MAP == kMapValue ? 1 : 0>());
+    else count_chunk(std::integral_constant<int, 0>());
 }
 
 template <typename K, int MAP>
 __global__ __launch_bounds__(kSplitBlock) void split_histogram(PassIo<K> io, int64_t n, int64_t chunks_per_row,
-                                                               const SplitRow* __restrict__ rows, uint32_t* __restrict__ chunk_fine) {
+                                                               const SplitRow* __restrict__ rows, uint32_t* __restrict__ chunk_fine,
+                                                               const PiecewiseMap* __restrict__ maps) {
     __shared__ uint32_t hist[kFine];
     for (int i = threadIdx.x; i < kFine; i += kSplitBlock) hist[i] = 0;
     __syncthreads();
     const int64_t row = blockIdx.x / chunks_per_row;
     const int64_t c = blockIdx.x - row * chunks_per_row;
     const K* xrow = io.x + io.xmap.at(row);
-    const FineMap<K> fine_of(rows[row], io.descending);
+    FineMap<K> fine_of(rows[row], io.descending);
     const int64_t lo = c * kChunk;
     const int64_t hi = (lo + kChunk < n) ? lo + kChunk : n;
-    count_fine_bins<K, MAP, kSplitBlock, true>(io, xrow, lo, hi, fine_of, hist);
+    if (fine_of.piecewise != 0u) {                     // (seldom) by the map split_remap made for the row
+        __shared__ K bound[kSegments];
+        __shared__ uint8_t bound_shift[kSegments];
+        static_assert(kSplitBlock == kSegments, "a thread a segment");
+        bound[threadIdx.x] = static_cast<K>(maps[row].bound[threadIdx.x]);
+        bound_shift[threadIdx.x] = maps[row].shift[threadIdx.x];
+        __syncthreads();
+        fine_of.bound = bound;
+        fine_of.bound_shift = bound_shift;
+        count_fine_bins<K, kMapPiecewise, kSplitBlock, true>(io, xrow, lo, hi, fine_of, hist);
+    } else {
+        count_fine_bins<K, MAP, kSplitBlock, true>(io, xrow, lo, hi, fine_of, hist);
+    }
     __syncthreads();
     uint32_t* g = chunk_fine + static_cast<int64_t>(blockIdx.x) * (kFine / 2);
     for (int i = threadIdx.x; i < kFine / 2; i += kSplitBlock) g[i] = hist[2 * i] | (hist[2 * i + 1] << 16);
@@ -516,7 +608,7 @@ struct PlanShared {
 template <int BLOCK>
 __device__ __forceinline__ uint32_t plan_buckets(PlanShared<BLOCK>& sm, const uint32_t (&cnt)[kFine / kSplitBlock], uint32_t (&bucket)[kFine / kSplitBlock],
                                                  int64_t n, uint32_t cap, int64_t row, SplitRow& info, uint32_t* __restrict__ counters,
-                                                 uint4* __restrict__ bucket_list, CrowdedList crowded, uint32_t* route_out = nullptr) {
+                                                 uint4* __restrict__ bucket_list, CrowdedList crowded, uint32_t* route_out = nullptr, bool piecewise = false) {
     constexpr int PER = kFine / kSplitBlock;          // 16
     constexpr int WAVES = BLOCK / kWave;
     const int w = threadIdx.x / kWave;
@@ -590,7 +682,8 @@ __device__ __forceinline__ uint32_t plan_buckets(PlanShared<BLOCK>& sm, const ui
 
     // Every fine bin leaves room in a bucket: buckets of (keys before) / (cap - largest bin) hold
     // fewer than cap keys each.
-    uint32_t route = 1u, n_buckets = kMaxBuckets + 1;
+    // (a row with a piecewise map is moved by split_pass_stable whatever its buckets: the plain pass carries no code for that map)
+    uint32_t route = piecewise ? 2u : 1u, n_buckets = kMaxBuckets + 1;
     if (biggest < cap) {
         n_buckets = assign(cap - biggest, gap_cuts);
         if (n_buckets > static_cast<uint32_t>(kMaxBuckets)) n_buckets = assign(cap - biggest, 0u);
@@ -685,14 +778,11 @@ __device__ __forceinline__ uint32_t plan_buckets(PlanShared<BLOCK>& sm, const ui
     return n_buckets;
 }
 
-__global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t cap, int64_t chunks_per_row, const uint32_t* __restrict__ chunk_fine,
-                                                          SplitRow* __restrict__ rows, uint32_t* __restrict__ counters,
-                                                          uint4* __restrict__ bucket_list, CrowdedList crowded,
-                                                          uint32_t* __restrict__ chunk_base) {
+// The plan of row `row` from its chunks' fine-bin histograms, by a workgroup of kSplitBlock threads.
+__device__ __forceinline__ void plan_row(PlanShared<kSplitBlock>& sm, uint32_t* __restrict__ per_bucket, int64_t row, int64_t n, uint32_t cap, int64_t chunks_per_row,
+                                         const uint32_t* __restrict__ chunk_fine, SplitRow* __restrict__ rows, uint32_t* __restrict__ counters,
+                                         uint4* __restrict__ bucket_list, CrowdedList crowded, uint32_t* __restrict__ chunk_base, bool piecewise) {
     constexpr int PER = kFine / kSplitBlock;          // 16
-    __shared__ PlanShared<kSplitBlock> sm;
-    __shared__ uint32_t per_bucket[kMaxBuckets];
-    const int64_t row = blockIdx.x;
     const uint32_t* f = chunk_fine + row * chunks_per_row * (kFine / 2) + threadIdx.x * (PER / 2);
     uint32_t cnt[PER];
 #pragma unroll
@@ -718,7 +808,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
     }
     uint32_t bucket[PER];
     per_bucket[threadIdx.x] = 0u;
-    const uint32_t n_buckets = plan_buckets<kSplitBlock>(sm, cnt, bucket, n, cap, row, rows[row], counters, bucket_list, crowded);
+    const uint32_t n_buckets = plan_buckets<kSplitBlock>(sm, cnt, bucket, n, cap, row, rows[row], counters, bucket_list, crowded, nullptr, piecewise);
     uint32_t next = threadIdx.x < n_buckets ? sm.begin[threadIdx.x] : 0u;      // where the coming chunk's keys of bucket threadIdx.x go
     // each chunk's keys per bucket, and from them where the chunk writes each bucket
     uint32_t w8[PER / 2], ahead[PER / 2];
@@ -742,6 +832,104 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < PER / 2; ++i) w8[i] = ahead[i];
+    }
+}
+
+__global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t cap, int64_t chunks_per_row, const uint32_t* __restrict__ chunk_fine,
+                                                          SplitRow* __restrict__ rows, uint32_t* __restrict__ counters,
+                                                          uint4* __restrict__ bucket_list, CrowdedList crowded,
+                                                          uint32_t* __restrict__ chunk_base) {
+    __shared__ PlanShared<kSplitBlock> sm;
+    __shared__ uint32_t per_bucket[kMaxBuckets];
+    const int64_t row = blockIdx.x;
+    if (row == 0 && threadIdx.x == 0) counters[4] = 0u;       // split_remap has read it: zero again for the next sort that uses this memory
+    plan_row(sm, per_bucket, row, n, cap, chunks_per_row, chunk_fine, rows, counters, bucket_list, crowded, chunk_base, rows[row].piecewise != 0u);
+}
+
+// ------------------------------------------------------------------ 3b. rows whose keys cluster
+// The rows split_sample marked `piecewise` (as a rule none: counters[4] is then zero and every
+// workgroup leaves at once).  split_remap, a workgroup per such row: a sample of 4096 of the
+// row's keys sorted on chip, and the row's PiecewiseMap from it; split_histogram and split_plan
+// then treat the row like any other, by that map.  Where split_front stands for those launches
+// (it leaves such a row alone), split_replan does their part: a workgroup counts the whole row
+// into the fine bins of its map and plans it.
+template <typename K>
+__global__ __launch_bounds__(kSplitBlock) void split_remap(PassIo<K> io, int64_t m, int64_t n, const SplitRow* __restrict__ rows,
+                                                           const uint32_t* __restrict__ counters, PiecewiseMap* __restrict__ maps) {
+    constexpr int ITEMS = kQuantileSample / kSplitBlock;      // 16
+    static_assert(kQuantileSample / kSegments == 16 && kSplitBlock == kSegments, "every 16th key of the sorted sample bounds a segment; a thread a segment");
+    __shared__ SmallShared<K, false, ITEMS, kSplitBlock / kWave> sorter;
+    __shared__ K bound[kSegments + 1];                 // [kSegments]: the sample's largest key
+    if (counters[4] == 0u) return;
+    const int tid = threadIdx.x;
+    const int seg = (tid / kWave) * kWave * ITEMS + lane_id();
+    for (int64_t row = blockIdx.x; row < m; row += gridDim.x) {
+        if (rows[row].piecewise == 0u) continue;
+        const K* xrow = io.x + io.xmap.at(row);
+        __syncthreads();                               // the row before has left LDS
+        // ---- the sample: 4096 keys at even distances, sorted
+        K key[ITEMS];
+        uint32_t none[1] = {0u};
+        K ors = 0, ands = ~K(0);
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const int64_t e = (static_cast<int64_t>(seg + k * kWave) * n) / kQuantileSample;
+            key[k] = key_of_element<K>(io, xrow[e * io.sx]);
+            ors |= key[k];
+            ands &= key[k];
+        }
+        sort_in_workgroup<K, false, ITEMS, kSplitBlock / kWave>(sorter, key, none, ors, ands, kQuantileSample, KeyTraits<K>::kPasses);
+        // ---- bounds: key k of this thread is the sorted sample's entry seg + 64 k
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            const int at = seg + k * kWave;
+            if (at % 16 == 0) bound[at / 16] = at == 0 ? K(0) : key[k];
+            if (at == kQuantileSample - 1) bound[kSegments] = key[k];
+        }
+        __syncthreads();
+        // the keys above a bound, up to the next one, share 15 bins: 1 + ((key - bound - 1) >> shift), at most 15
+        const K lo = bound[tid], hi = bound[tid + 1];
+        uint32_t shift = 0;
+        if (hi > lo) {
+            const unsigned long long widest = static_cast<unsigned long long>(static_cast<K>(hi - lo - 1));
+            const int bits = widest ? 64 - __builtin_clzll(widest) : 0;
+            shift = bits > 4 ? static_cast<uint32_t>(bits - 4) : 0u;
+        }
+        maps[row].bound[tid] = static_cast<unsigned long long>(lo);
+        maps[row].shift[tid] = static_cast<uint8_t>(shift);
+    }
+}
+
+template <typename K>
+__global__ __launch_bounds__(kSplitBlock) void split_replan(PassIo<K> io, int64_t m, int64_t n, uint32_t cap, SplitRow* __restrict__ rows,
+                                                            uint32_t* __restrict__ counters, uint4* __restrict__ bucket_list, CrowdedList crowded,
+                                                            const PiecewiseMap* __restrict__ maps) {
+    __shared__ uint32_t hist[kFine];
+    __shared__ PlanShared<kSplitBlock> plan;
+    __shared__ K bound[kSegments];
+    __shared__ uint8_t bound_shift[kSegments];
+    if (counters[4] == 0u) return;
+    const int tid = threadIdx.x;
+    for (int64_t row = blockIdx.x; row < m; row += gridDim.x) {
+        SplitRow& info = rows[row];
+        if (info.piecewise == 0u) continue;
+        const K* xrow = io.x + io.xmap.at(row);
+        __syncthreads();                               // the row before has left LDS
+        static_assert(kSplitBlock == kSegments, "a thread a segment");
+        bound[tid] = static_cast<K>(maps[row].bound[tid]);
+        bound_shift[tid] = maps[row].shift[tid];
+        for (int i = tid; i < kFine; i += kSplitBlock) hist[i] = 0u;
+        __syncthreads();
+        FineMap<K> fine_of(info, io.descending);
+        fine_of.bound = bound;
+        fine_of.bound_shift = bound_shift;
+        count_fine_bins<K, kMapPiecewise, kSplitBlock, false>(io, xrow, 0, n, fine_of, hist);
+        __syncthreads();
+        constexpr int PER = kFine / kSplitBlock;
+        uint32_t cnt[PER], bucket[PER];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) cnt[i] = hist[tid * PER + i];
+        (void)plan_buckets<kSplitBlock>(plan, cnt, bucket, n, cap, row, info, counters, bucket_list, crowded, nullptr, true);
     }
 }
 
@@ -794,6 +982,9 @@ struct SplitShared {
     uint32_t wave_hist[STABLE ? BLOCK / kWave : 1][kMaxBuckets];
     uint32_t oversized[STABLE ? kMaxBuckets : 1];
     K mixed[STABLE ? kMaxBuckets : 1];        // ... the bits in which neighbouring entries of such a bucket differ in this tile
+    K bound[STABLE ? kSegments : 1];           // the row's PiecewiseMap, if it has one
+    uint8_t bound_shift[STABLE ? kSegments : 4];
+    uint8_t bucket_at[STABLE ? BLOCK * kSplitItems : 4];      // the bucket of every entry of the tile as laid out
 };
 
 // What the stable pass needs beyond the plain one.
@@ -801,6 +992,7 @@ template <typename K>
 struct StablePass {
     uint32_t cap = 0;                          // the most entries of a bucket that split_finish takes
     unsigned long long* range = nullptr;       // CrowdedList::range
+    const PiecewiseMap* map = nullptr;         // the row's, if SplitRow::piecewise says so
     // the row's outputs (what emit_entry reads from PassIo, by value)
     K* yrow = nullptr;                         // the row of the value output, if there is one
     void* idx = nullptr;                       // the index output, if there is one
@@ -845,9 +1037,17 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK, 
     const int tid = threadIdx.x;
     const int lane = lane_id();
     const int w = tid / kWave;
-    const FineMap<K> fine_of(info, io.descending);
+    FineMap<K> fine_of(info, io.descending);
     const K* xrow = io.x + io.xmap.at(row);
     const int64_t row_off = row * n;
+    if constexpr (STABLE) {
+        fine_of.bound = sm.bound;
+        fine_of.bound_shift = sm.bound_shift;
+        if (fine_of.piecewise != 0u && tid < kSegments) {
+            sm.bound[tid] = static_cast<K>(stable.map->bound[tid]);
+            sm.bound_shift[tid] = stable.map->shift[tid];
+        }
+    }
     // element of the tile that this thread's item k is
     auto element_of = [&](int k) __attribute__((always_inline)) { return STABLE ? w * (kWave * ITEMS) + k * kWave + lane : tid + k * BLOCK; };
 
@@ -887,8 +1087,8 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK, 
     const bool direct = STABLE && stable.direct;
     __syncthreads();
 
-    auto move_chunk = [&](auto by_value_tag) __attribute__((always_inline)) {
-    constexpr bool BY_VALUE = decltype(by_value_tag)::value;
+    auto move_chunk = [&](auto mode_tag) __attribute__((always_inline)) {
+    constexpr int MODE = decltype(mode_tag)::value;
     constexpr bool GAP = MAP == kMapGap || MAP == kMapAny;
     for (int64_t tile_base = chunk_lo; tile_base < chunk_hi; tile_base += TILE) {
         const int valid = static_cast<int>((chunk_hi - tile_base < TILE) ? chunk_hi - tile_base : TILE);
@@ -905,7 +1105,7 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK, 
             uint32_t rank[ITEMS];
 #pragma unroll
             for (int k = 0; k < ITEMS; ++k) {
-                const uint32_t f = fine_of.template bin<BY_VALUE, GAP>(key[k]);
+                const uint32_t f = fine_of.template bin_as<MODE, GAP>(key[k]);
                 where[k] = (sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu;
                 if (!full && element_of(k) >= valid) where[k] = last_bucket;
             }
@@ -917,7 +1117,7 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK, 
         for (int k0 = 0; k0 < ITEMS; k0 += 8) {
 #pragma unroll
             for (int k = k0; k < k0 + 8; ++k) {
-                const uint32_t f = fine_of.template bin<BY_VALUE, GAP>(key[k]);
+                const uint32_t f = fine_of.template bin_as<MODE, GAP>(key[k]);
                 where[k] = (sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu;
             }
 #pragma unroll
@@ -968,14 +1168,17 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK, 
         // ---- lay the tile out by bucket (bucket starts read first, then the stores)
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
-            if constexpr (STABLE) where[k] = sm.start[where[k] >> 16] + sm.wave_hist[w][where[k] >> 16] + (where[k] & 0xffffu);
+            // (stable: the bucket stays in the upper half, for the table of buckets beside the tile)
+            if constexpr (STABLE) where[k] = (where[k] & 0xffff0000u) | (sm.start[where[k] >> 16] + sm.wave_hist[w][where[k] >> 16] + (where[k] & 0xffffu));
             else where[k] = sm.start[where[k] >> 16] + (where[k] & 0xffffu);
         }
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
             if (full || element_of(k) < valid) {
-                sm.keys[where[k]] = key[k];
-                if constexpr (PAIRS && !IN_TURN) sm.vals[where[k]] = static_cast<uint32_t>(tile_base) + static_cast<uint32_t>(element_of(k));
+                const uint32_t at_tile = STABLE ? (where[k] & 0xffffu) : where[k];
+                sm.keys[at_tile] = key[k];
+                if constexpr (PAIRS && !IN_TURN) sm.vals[at_tile] = static_cast<uint32_t>(tile_base) + static_cast<uint32_t>(element_of(k));
+                if constexpr (STABLE) sm.bucket_at[at_tile] = static_cast<uint8_t>(where[k] >> 16);
             }
         }
         __syncthreads();
@@ -990,7 +1193,7 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK, 
         if constexpr (STABLE) {
             K* dk = io.kbuf[0] + row_off;
             uint32_t* dv = PAIRS ? io.vbuf[0] + row_off : nullptr;
-            constexpr int G = sizeof(K) == 8 ? 4 : 8;          // tile positions a thread handles at a time (registers)
+            constexpr int G = sizeof(K) == 8 ? (PAIRS ? 2 : 4) : 8;      // tile positions a thread handles at a time (registers)
             const K own_first = (owner && own_count != 0u) ? sm.keys[own_start] : K(0);
 #pragma unroll
             for (int k0 = 0; k0 < ITEMS; k0 += G) {
@@ -1005,10 +1208,7 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK, 
                     if constexpr (PAIRS) pay[j] = sm.vals[p];
                 }
 #pragma unroll
-                for (int j = 0; j < G; ++j) {
-                    const uint32_t f = fine_of.template bin<BY_VALUE, GAP>(out[j]);
-                    b[j] = (sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu;
-                }
+                for (int j = 0; j < G; ++j) b[j] = sm.bucket_at[(k0 + j) * BLOCK + tid];
 #pragma unroll
                 for (int j = 0; j < G; ++j) {
                     at[j] = sm.dst_base[b[j]] + ((k0 + j) * BLOCK + tid);
@@ -1051,7 +1251,7 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK, 
                 for (int j = 0; j < 8; ++j) out[j] = sm.keys[(k0 + j) * BLOCK + tid];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    const uint32_t f = fine_of.template bin<BY_VALUE, GAP>(out[j]);
+                    const uint32_t f = fine_of.template bin_as<MODE, GAP>(out[j]);
                     at[k0 + j] = static_cast<int32_t>((sm.table[f >> 2] >> (8u * (f & 3u))) & 0xffu);
                 }
 #pragma unroll
@@ -1091,8 +1291,14 @@ __device__ __forceinline__ void scatter_to_buckets(SplitShared<K, PAIRS, BLOCK, 
         __syncthreads();                                   // the tile in LDS has left
     }
     };
-    if ((MAP == kMapValue || MAP == kMapAny) && fine_of.by_value) move_chunk(std::integral_constant<bool, MAP == kMapValue || MAP == kMapAny>());
-    else move_chunk(std::false_type());
+    if constexpr (MAP == kMapAny) {
+        if (fine_of.piecewise) move_chunk(std::integral_constant<int, 2>());
+        else if (fine_of.by_value) move_chunk(std::integral_constant<int, 1>());
+        else move_chunk(std::integral_constant<int, 0>());
+    } else {
+        if (MAP == kMapValue && fine_of.by_value) move_chunk(std::integral_constant<int, MAP == kMapValue ? 1 : 0>());
+        else move_chunk(std::integral_constant<int, 0>());
+    }
 }
 
 // One workgroup per chunk (kChunk keys): elements [chunk_lo, chunk_hi) of row `row` go to their
@@ -1131,10 +1337,16 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
     const int64_t row = blockIdx.x;
     const K* xrow = io.x + io.xmap.at(row);
     SplitRow& info = rows[row];
-    const FineRange range = sample_row<K, MAP, BLOCK>(io, xrow, n, cap);
-    if (threadIdx.x == 0) range.store(info);
     for (int i = threadIdx.x; i < kFine; i += BLOCK) hist[i] = 0u;
-    __syncthreads();
+    const FineRange range = sample_row<K, MAP, BLOCK>(io, xrow, n, cap, hist);
+    if (threadIdx.x == 0) {
+        range.store(info);
+        if (range.piecewise != 0u) {                   // split_replan counts and plans such a row
+            info.route = 0u;
+            atomicOr(&counters[4], 1u);
+        }
+    }
+    if (range.piecewise != 0u) return;
     count_fine_bins<K, MAP, BLOCK, false>(io, xrow, 0, n, FineMap<K>(range, io.descending), hist);
     __syncthreads();
     constexpr int PER = kFine / kSplitBlock;
@@ -1149,7 +1361,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
 }
 
 __global__ void split_clear(uint32_t* __restrict__ counters) {
-    if (threadIdx.x < 4) counters[threadIdx.x] = 0u;
+    if (threadIdx.x < 8) counters[threadIdx.x] = 0u;      // what the later launches of this sort count up from
 }
 
 // The stable pass for the rows that have buckets larger than a workgroup holds (SplitRow::route
@@ -1159,7 +1371,8 @@ constexpr int kStableBlock = 512;
 template <typename K, bool PAIRS>
 __global__ __launch_bounds__(kStableBlock) void split_pass_stable(PassIo<K> io, int64_t n, uint32_t cap, int64_t chunks_per_row, int64_t units,
                                                                   const SplitRow* __restrict__ infos, const uint32_t* __restrict__ counters,
-                                                                  const uint32_t* __restrict__ chunk_base, unsigned long long* __restrict__ range) {
+                                                                  const uint32_t* __restrict__ chunk_base, unsigned long long* __restrict__ range,
+                                                                  const PiecewiseMap* __restrict__ maps) {
     static_assert(kChunk % (kStableBlock * kSplitItems) == 0, "whole tiles a chunk");
     __shared__ SplitShared<K, PAIRS, kStableBlock, true> sm;
     if (counters[3] == 0u) return;                     // no such row in this call
@@ -1173,7 +1386,7 @@ __global__ __launch_bounds__(kStableBlock) void split_pass_stable(PassIo<K> io, 
         __syncthreads();                               // the unit before has left the tables
         scatter_to_buckets<K, PAIRS, kStableBlock, kMapAny, false, true>(sm, io, n, row, info, chunk_lo, chunk_hi,
                                                                         chunk_base ? chunk_base + unit * kMaxBuckets : info.begin,
-                                                                        StablePass<K>{cap, range, io.y ? io.y + io.ymap.at(row) : nullptr, PAIRS ? io.idx : nullptr,
+                                                                        StablePass<K>{cap, range, maps + row, io.y ? io.y + io.ymap.at(row) : nullptr, PAIRS ? io.idx : nullptr,
                                                                                       (PAIRS && io.idx) ? io.imap.at(row) : 0, io.sx, io.sy, io.si, io.idx64,
                                                                                       io.kind, io.descending, PAIRS ? io.restore_zero : 0, io.x_intact != 0});
     }
@@ -1897,7 +2110,7 @@ __global__ __launch_bounds__(WAVES * kWave) void split_finish_in_place(PassIo<K>
 
 struct SplitLayout {
     int64_t chunks_per_row;
-    size_t counters_off, rows_off, list_off, crowded_off, state_off, fine_off, base_off, total;
+    size_t counters_off, rows_off, list_off, crowded_off, state_off, fine_off, base_off, maps_off, total;
 };
 
 SplitLayout split_layout(int64_t m, int64_t n) {
@@ -1919,6 +2132,8 @@ SplitLayout split_layout(int64_t m, int64_t n) {
     off += align_up(static_cast<size_t>(m) * l.chunks_per_row * (kFine / 2) * 4, 256);
     l.base_off = off;            // where every chunk writes each bucket
     off += align_up(static_cast<size_t>(m) * l.chunks_per_row * kMaxBuckets * 4, 256);
+    l.maps_off = off;            // the maps of rows whose keys cluster
+    off += align_up(static_cast<size_t>(m) * sizeof(PiecewiseMap), 256);
     l.total = off;
     return l;
 }
@@ -1949,6 +2164,7 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
     const CrowdedList crowded = {reinterpret_cast<uint2*>(base + l.crowded_off), reinterpret_cast<unsigned long long*>(base + l.state_off)};
     uint32_t* fine = reinterpret_cast<uint32_t*>(base + l.fine_off);
     uint32_t* chunk_base = reinterpret_cast<uint32_t*>(base + l.base_off);
+    PiecewiseMap* maps = reinterpret_cast<PiecewiseMap*>(base + l.maps_off);
 
     const int waves = finish_waves(n, io.kind == kKeyFloat);
     const int cap = finish_cap(waves);
@@ -1977,9 +2193,17 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         DLFX_CHECK_LAUNCH();
     }
     const dim3 chunks(static_cast<unsigned>(m * l.chunks_per_row));
+    // rows whose keys cluster get their maps (as a rule none: every workgroup leaves at once)
+    auto remap_rows = [&]() -> int {
+        split_remap<K><<<dim3(static_cast<unsigned>(m < 1024 ? m : 1024)), dim3(kSplitBlock), 0, stream>>>(io, m, n, rows, counters, maps);
+        DLFX_CHECK_LAUNCH();
+        return DLFX_OK;
+    };
     if (!front) {
+        const int status = remap_rows();
+        if (status != DLFX_OK) return status;
         with_map([&](auto map_tag) {
-            split_histogram<K, decltype(map_tag)::value><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine);
+            split_histogram<K, decltype(map_tag)::value><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine, maps);
         });
         DLFX_CHECK_LAUNCH();
         split_plan<<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(n, static_cast<uint32_t>(cap), l.chunks_per_row, fine, rows, counters, list, crowded, chunk_base);
@@ -2013,11 +2237,18 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         else if (block == 512) pass_of(std::integral_constant<int, 512>());
         else if constexpr (kPassBlockMax<K, PAIRS> >= 1024) pass_of(std::integral_constant<int, 1024>());
         DLFX_CHECK_LAUNCH();
+        if (front) {
+            const int status = remap_rows();
+            if (status != DLFX_OK) return status;
+            split_replan<K><<<dim3(static_cast<unsigned>(m < 1024 ? m : 1024)), dim3(kSplitBlock), 0, stream>>>(
+                io, m, n, static_cast<uint32_t>(cap), rows, counters, list, crowded, maps);
+            DLFX_CHECK_LAUNCH();
+        }
         {
             // rows with buckets larger than a workgroup holds (as a rule none: every workgroup leaves at once)
             const int64_t units = front ? m : m * l.chunks_per_row;
             split_pass_stable<K, PAIRS><<<dim3(static_cast<unsigned>(units < 1024 ? units : 1024)), dim3(kStableBlock), 0, stream>>>(
-                io, n, static_cast<uint32_t>(cap), l.chunks_per_row, units, rows, counters, front ? nullptr : chunk_base, crowded.range);
+                io, n, static_cast<uint32_t>(cap), l.chunks_per_row, units, rows, counters, front ? nullptr : chunk_base, crowded.range, maps);
             DLFX_CHECK_LAUNCH();
         }
         split_finish<K, PAIRS, WAVES><<<fgrid, dim3(WAVES * kWave), 0, stream>>>(io, n, limit, counters, list, crowded.items);

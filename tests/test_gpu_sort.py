@@ -487,6 +487,63 @@ def test_many_rows_each_planned_and_moved_by_one_workgroup(hip_backend, dtype, n
     assert np.array_equal(Xh.numpy(), want[:, ::-1])
 
 
+def clustered_rows(dtype, n, seed):
+    """Rows whose distinct keys crowd parts of their range: the evenly spaced fine bins of the
+    bucket route cannot cut them, a map made from the quantiles of a sample can."""
+    dt = np.dtype(dtype)
+    u = uniform01(seed, n)
+    g = normal(seed + 1, n)
+    if dt.kind == "i":
+        top = float(np.iinfo(dtype).max)
+        zipf = np.minimum(np.floor(1.0 / np.maximum(u, 1e-12) ** 1.3), top / 2).astype(dtype)      # most keys small, a long tail
+        two = np.where(randint(seed + 2, n, 0, 2) > 0, 1000 + randint(seed + 3, n, 0, 5000), int(top / 3) + randint(seed + 4, n, 0, 5000)).astype(dtype)
+        tail = np.where(randint(seed + 5, n, 0, 20) > 0, randint(seed + 6, n, -3000, 3000), (g * top / 8).astype(np.int64)).astype(dtype)
+        steps = (np.floor(u * 64).astype(np.int64) * int(top / 80) + randint(seed + 7, n, 0, 300)).astype(dtype)     # 64 narrow clusters
+    else:
+        zipf = np.exp(g * 6).astype(dtype)                                                # log-normal: twenty binades
+        two = np.where(randint(seed + 2, n, 0, 2) > 0, 1.0 + g * 1e-5, -250.0 + g * 1e-4).astype(dtype)
+        tail = np.where(randint(seed + 5, n, 0, 20) > 0, g * 1e-3, g * 1e6).astype(dtype)
+        steps = (np.floor(u * 64) * 1000 + g * 1e-2).astype(dtype)
+    return np.stack([zipf, two, tail, steps, np.sort(zipf), np.sort(two)[::-1]])
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.int64, np.float32, np.float64])
+@pytest.mark.parametrize("n", [30000, 131072, 1 << 20, 2500000])
+def test_rows_whose_keys_cluster(hip_backend, dtype, n):
+    x = clustered_rows(dtype, n, 370)
+    Xh = Tensor.from_numpy(hip_backend, x)
+    want = np.sort(x, axis=-1, kind="stable")
+    assert np.array_equal(F.sort(Xh, -1).numpy(), want)
+    order = np.argsort(x, axis=-1, kind="stable")
+    assert np.array_equal(F.argsort(Xh, -1).numpy(), order)
+    Yh, Ih = F.argsort(Xh, -1, True, with_values=True)
+    rev = np.argsort(-x if np.dtype(dtype).kind == "f" else ~x, axis=-1, kind="stable")
+    assert np.array_equal(Ih.numpy(), rev)
+    assert np.array_equal(Yh.numpy().view(np.uint8), np.take_along_axis(x, rev, -1).view(np.uint8))
+    one = Tensor.from_numpy(hip_backend, x[2:3])                         # a single row: every workgroup on it
+    assert np.array_equal(F.sort(one, -1).numpy(), want[2:3])
+    F.sort(Xh, -1, out=Xh)                                              # in place: nothing goes straight to the outputs
+    assert np.array_equal(Xh.numpy(), want)
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.float32])
+def test_many_rows_whose_keys_cluster(hip_backend, dtype):
+    # the calls of many short rows (one workgroup plans and moves a row): clustered rows among plain ones
+    m, n = 600, 40000
+    kinds = clustered_rows(dtype, n, 380)
+    if np.dtype(dtype).kind == "f":
+        x = normal(381, m * n).astype(dtype).reshape(m, n)
+    else:
+        x = (full_range_i64(381, m * n) >> 34).astype(dtype).reshape(m, n)
+    x[3::7] = kinds[np.arange(x[3::7].shape[0]) % kinds.shape[0]]
+    Xh = Tensor.from_numpy(hip_backend, x)
+    assert np.array_equal(F.sort(Xh, -1).numpy(), np.sort(x, axis=-1))
+    order = np.argsort(x, axis=-1, kind="stable")
+    Yh, Ih = F.argsort(Xh, -1, with_values=True)
+    assert np.array_equal(Ih.numpy(), order)
+    assert np.array_equal(Yh.numpy().view(np.uint8), np.take_along_axis(x, order, -1).view(np.uint8))
+
+
 @pytest.mark.parametrize("n", [70000, 300000])
 def test_index_only_argsort_written_over_its_input(hip_backend, n):
     # argsort(X, X) of int32 (UniformTest.cpp:2461-2466 does this with short rows): there is no value
