@@ -851,63 +851,76 @@ __global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t ca
 // workgroup leaves at once).  split_remap, a workgroup per such row: a sample of 4096 of the
 // row's keys sorted on chip, and the row's PiecewiseMap from it; split_histogram and split_plan
 // then treat the row like any other, by that map.  Where split_front stands for those launches
-// (it leaves such a row alone), split_replan does their part: a workgroup counts the whole row
-// into the fine bins of its map and plans it.
+// (it leaves such a row alone), split_replan does the whole of it instead: a workgroup makes the
+// row's map, counts the row into the map's fine bins and plans it.
+template <typename K>
+struct RemapShared {
+    SmallShared<K, false, kQuantileSample / kSplitBlock, kSplitBlock / kWave> sorter;
+    K bound[kSegments + 1];                            // [kSegments]: the sample's largest key
+    uint8_t bound_shift[kSegments];
+};
+
+// The PiecewiseMap of a row into sm.bound / sm.bound_shift, by a workgroup of kSplitBlock threads
+// (no barrier after the last writes).
+template <typename K>
+__device__ __forceinline__ void piecewise_map_of(RemapShared<K>& sm, const PassIo<K>& io, const K* __restrict__ xrow, int64_t n) {
+    constexpr int ITEMS = kQuantileSample / kSplitBlock;      // 16
+    static_assert(kQuantileSample / kSegments == 16 && kSplitBlock == kSegments, "every 16th key of the sorted sample bounds a segment; a thread a segment");
+    const int tid = threadIdx.x;
+    const int seg = (tid / kWave) * kWave * ITEMS + lane_id();
+    // ---- the sample: 4096 keys at even distances, sorted
+    K key[ITEMS];
+    uint32_t none[1] = {0u};
+    K ors = 0, ands = ~K(0);
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const int64_t e = (static_cast<int64_t>(seg + k * kWave) * n) / kQuantileSample;
+        key[k] = key_of_element<K>(io, xrow[e * io.sx]);
+        ors |= key[k];
+        ands &= key[k];
+    }
+    sort_in_workgroup<K, false, ITEMS, kSplitBlock / kWave>(sm.sorter, key, none, ors, ands, kQuantileSample, KeyTraits<K>::kPasses);
+    // ---- bounds: key k of this thread is the sorted sample's entry seg + 64 k
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const int at = seg + k * kWave;
+        if (at % 16 == 0) sm.bound[at / 16] = at == 0 ? K(0) : key[k];
+        if (at == kQuantileSample - 1) sm.bound[kSegments] = key[k];
+    }
+    __syncthreads();
+    // the keys above a bound, up to the next one, share 15 bins: 1 + ((key - bound - 1) >> shift), at most 15
+    const K lo = sm.bound[tid], hi = sm.bound[tid + 1];
+    uint32_t shift = 0;
+    if (hi > lo) {
+        const unsigned long long widest = static_cast<unsigned long long>(static_cast<K>(hi - lo - 1));
+        const int bits = widest ? 64 - __builtin_clzll(widest) : 0;
+        shift = bits > 4 ? static_cast<uint32_t>(bits - 4) : 0u;
+    }
+    sm.bound_shift[tid] = static_cast<uint8_t>(shift);
+}
+
 template <typename K>
 __global__ __launch_bounds__(kSplitBlock) void split_remap(PassIo<K> io, int64_t m, int64_t n, const SplitRow* __restrict__ rows,
                                                            const uint32_t* __restrict__ counters, PiecewiseMap* __restrict__ maps) {
-    constexpr int ITEMS = kQuantileSample / kSplitBlock;      // 16
-    static_assert(kQuantileSample / kSegments == 16 && kSplitBlock == kSegments, "every 16th key of the sorted sample bounds a segment; a thread a segment");
-    __shared__ SmallShared<K, false, ITEMS, kSplitBlock / kWave> sorter;
-    __shared__ K bound[kSegments + 1];                 // [kSegments]: the sample's largest key
+    __shared__ RemapShared<K> sm;
     if (counters[4] == 0u) return;
     const int tid = threadIdx.x;
-    const int seg = (tid / kWave) * kWave * ITEMS + lane_id();
     for (int64_t row = blockIdx.x; row < m; row += gridDim.x) {
         if (rows[row].piecewise == 0u) continue;
-        const K* xrow = io.x + io.xmap.at(row);
         __syncthreads();                               // the row before has left LDS
-        // ---- the sample: 4096 keys at even distances, sorted
-        K key[ITEMS];
-        uint32_t none[1] = {0u};
-        K ors = 0, ands = ~K(0);
-#pragma unroll
-        for (int k = 0; k < ITEMS; ++k) {
-            const int64_t e = (static_cast<int64_t>(seg + k * kWave) * n) / kQuantileSample;
-            key[k] = key_of_element<K>(io, xrow[e * io.sx]);
-            ors |= key[k];
-            ands &= key[k];
-        }
-        sort_in_workgroup<K, false, ITEMS, kSplitBlock / kWave>(sorter, key, none, ors, ands, kQuantileSample, KeyTraits<K>::kPasses);
-        // ---- bounds: key k of this thread is the sorted sample's entry seg + 64 k
-#pragma unroll
-        for (int k = 0; k < ITEMS; ++k) {
-            const int at = seg + k * kWave;
-            if (at % 16 == 0) bound[at / 16] = at == 0 ? K(0) : key[k];
-            if (at == kQuantileSample - 1) bound[kSegments] = key[k];
-        }
-        __syncthreads();
-        // the keys above a bound, up to the next one, share 15 bins: 1 + ((key - bound - 1) >> shift), at most 15
-        const K lo = bound[tid], hi = bound[tid + 1];
-        uint32_t shift = 0;
-        if (hi > lo) {
-            const unsigned long long widest = static_cast<unsigned long long>(static_cast<K>(hi - lo - 1));
-            const int bits = widest ? 64 - __builtin_clzll(widest) : 0;
-            shift = bits > 4 ? static_cast<uint32_t>(bits - 4) : 0u;
-        }
-        maps[row].bound[tid] = static_cast<unsigned long long>(lo);
-        maps[row].shift[tid] = static_cast<uint8_t>(shift);
+        piecewise_map_of<K>(sm, io, io.x + io.xmap.at(row), n);
+        maps[row].bound[tid] = static_cast<unsigned long long>(sm.bound[tid]);
+        maps[row].shift[tid] = sm.bound_shift[tid];
     }
 }
 
 template <typename K>
 __global__ __launch_bounds__(kSplitBlock) void split_replan(PassIo<K> io, int64_t m, int64_t n, uint32_t cap, SplitRow* __restrict__ rows,
                                                             uint32_t* __restrict__ counters, uint4* __restrict__ bucket_list, CrowdedList crowded,
-                                                            const PiecewiseMap* __restrict__ maps) {
+                                                            PiecewiseMap* __restrict__ maps) {
+    __shared__ RemapShared<K> sm;
     __shared__ uint32_t hist[kFine];
     __shared__ PlanShared<kSplitBlock> plan;
-    __shared__ K bound[kSegments];
-    __shared__ uint8_t bound_shift[kSegments];
     if (counters[4] == 0u) return;
     const int tid = threadIdx.x;
     for (int64_t row = blockIdx.x; row < m; row += gridDim.x) {
@@ -915,14 +928,14 @@ __global__ __launch_bounds__(kSplitBlock) void split_replan(PassIo<K> io, int64_
         if (info.piecewise == 0u) continue;
         const K* xrow = io.x + io.xmap.at(row);
         __syncthreads();                               // the row before has left LDS
-        static_assert(kSplitBlock == kSegments, "a thread a segment");
-        bound[tid] = static_cast<K>(maps[row].bound[tid]);
-        bound_shift[tid] = maps[row].shift[tid];
+        piecewise_map_of<K>(sm, io, xrow, n);
+        maps[row].bound[tid] = static_cast<unsigned long long>(sm.bound[tid]);      // (split_pass_stable reads it)
+        maps[row].shift[tid] = sm.bound_shift[tid];
         for (int i = tid; i < kFine; i += kSplitBlock) hist[i] = 0u;
         __syncthreads();
         FineMap<K> fine_of(info, io.descending);
-        fine_of.bound = bound;
-        fine_of.bound_shift = bound_shift;
+        fine_of.bound = sm.bound;
+        fine_of.bound_shift = sm.bound_shift;
         count_fine_bins<K, kMapPiecewise, kSplitBlock, false>(io, xrow, 0, n, fine_of, hist);
         __syncthreads();
         constexpr int PER = kFine / kSplitBlock;
@@ -2238,8 +2251,6 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
         else if constexpr (kPassBlockMax<K, PAIRS> >= 1024) pass_of(std::integral_constant<int, 1024>());
         DLFX_CHECK_LAUNCH();
         if (front) {
-            const int status = remap_rows();
-            if (status != DLFX_OK) return status;
             split_replan<K><<<dim3(static_cast<unsigned>(m < 1024 ? m : 1024)), dim3(kSplitBlock), 0, stream>>>(
                 io, m, n, static_cast<uint32_t>(cap), rows, counters, list, crowded, maps);
             DLFX_CHECK_LAUNCH();
