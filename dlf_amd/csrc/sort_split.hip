@@ -14,11 +14,9 @@
 //                       skewed rows - floats with their exponents, clustered integers - still
 //                       give even buckets.  Every chunk's histogram becomes the place of its keys
 //                       inside each bucket, and the buckets of all rows are listed for the last
-//                       step.  A row with a fine bin fuller than a workgroup holds (one value
-//                       repeated many times, keys packed more tightly than the bins resolve)
-//                       gets buckets larger than that - each such bin one to itself where the
-//                       bucket numbers allow - which step 6 finishes (decided here, on the
-//                       device, row by row).
+//                       step.  A row with a fine bin fuller than a workgroup holds gets buckets
+//                       larger than that - each such bin one to itself where the bucket
+//                       numbers allow (decided here, on the device, row by row; below).
 //   4. split_pass       one workgroup per chunk: a tile of 4096 keys finds each key's bucket
 //                       (table in LDS) and its slot among the tile's keys of that bucket with one
 //                       LDS atomic, lays the tile out by bucket in LDS and writes it as runs to
@@ -32,13 +30,19 @@
 //                       order of equal keys; the bucket leaves for the strided outputs.
 //   6. split_finish_crowded  buckets with a bin too crowded for that (many equal or clustered
 //                       keys) take the stable digit passes of sort_in_workgroup instead, for
-//                       pairs first by index, then by key.  A bucket larger than a workgroup
-//                       holds is sorted by the one workgroup that draws it: stable digit passes
-//                       over the digits that vary in it (none for one repeated value: a copy),
-//                       window by window, between the scratch buffer and the bucket's place
-//                       in the outputs.  Pairs of such a row were moved by split_pass_stable
-//                       (ranks in element order instead of atomics), so they arrive in index
-//                       order.
+//                       pairs first by index, then by key.
+// Rows that evenly spaced fine bins do not cut:
+//   * one value repeated more often than a workgroup holds makes a bucket larger than that.  The
+//     row is then moved by split_pass_stable (ranks in element order instead of atomics), which
+//     writes the entries of such buckets straight to the outputs: a bucket of one value arrives
+//     sorted, in index order, and is done.
+//   * distinct keys packed more tightly than the bins resolve: split_sample sees them in its
+//     sample and marks the row, split_remap gives it a map made from the quantiles of a larger
+//     sample (PiecewiseMap), and steps 2 to 6 run as for any row, the stable pass moving it.
+//   * what is left - an oversized bucket of several values that the sample did not show - is
+//     sorted by the one workgroup of split_finish_crowded that draws it: stable digit passes over
+//     the digits that vary in it, window by window, between the scratch buffer and the bucket's
+//     place in the outputs.
 // Ranking with an LDS atomic costs a few instructions per key where wave-wide digit matching
 // costs about fifty per digit, which is what bounds the digit passes.
 #include <cstddef>
