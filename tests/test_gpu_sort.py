@@ -544,6 +544,40 @@ def test_many_rows_whose_keys_cluster(hip_backend, dtype):
     assert np.array_equal(Yh.numpy().view(np.uint8), np.take_along_axis(x, order, -1).view(np.uint8))
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.float64])
+def test_repeated_and_clustered_keys_on_strided_views(hip_backend, dtype):
+    # the rows of the two tests above read through a view with a step, backwards, and written to
+    # transposed outputs: the stable pass writes oversized buckets straight to such outputs, and an
+    # index-only argsort reads its keys back from such an input
+    n = 80000
+    x2 = np.concatenate([oversized_rows(dtype, 2 * n, 390), clustered_rows(dtype, 2 * n, 391)])
+    m = x2.shape[0]
+    view = x2[:, ::2][:, ::-1]
+    Xh = Tensor.from_numpy(hip_backend, x2).slice([0], [2 * n], [1], [2]).flip([1])
+    assert np.array_equal(Xh.numpy().view(np.uint8), np.ascontiguousarray(view).view(np.uint8))
+    from dlf_amd.frontend import dtype_code
+
+    def argsort_into(desc, Y, I):                       # the boundary call, with outputs that are views
+        hip_backend.argsort(int(desc), dtype_code(Xh.dtype), dtype_code(I.dtype), Xh.shape, Xh.storage,
+                            Y.shape if Y is not None else None, Y.storage if Y is not None else None, I.shape, I.storage)
+
+    for desc in (False, True):
+        key = view if not desc else (-view if np.dtype(dtype).kind == "f" else ~view)
+        order = np.argsort(key, axis=-1, kind="stable")
+        Ih = Tensor.from_numpy(hip_backend, np.zeros((n, m), dtype=np.int64)).transpose([1, 0])
+        argsort_into(desc, None, Ih)
+        assert np.array_equal(np.ascontiguousarray(Ih.numpy()), order), desc
+        Yh = Tensor.from_numpy(hip_backend, np.zeros((n, m), dtype=dtype)).transpose([1, 0])
+        I32 = Tensor.from_numpy(hip_backend, np.zeros((n, m), dtype=np.int32)).transpose([1, 0])
+        argsort_into(desc, Yh, I32)
+        assert np.array_equal(np.ascontiguousarray(I32.numpy()), order), desc
+        assert np.array_equal(np.ascontiguousarray(Yh.numpy()).view(np.uint8), np.ascontiguousarray(np.take_along_axis(view, order, -1)).view(np.uint8)), desc
+        Zh = Tensor.from_numpy(hip_backend, np.zeros((n, m), dtype=dtype)).transpose([1, 0])
+        F.sort(Xh, -1, desc, out=Zh)
+        want = np.sort(view, axis=-1)
+        assert np.array_equal(np.ascontiguousarray(Zh.numpy()), want[:, ::-1] if desc else want), desc
+
+
 @pytest.mark.parametrize("n", [70000, 300000])
 def test_index_only_argsort_written_over_its_input(hip_backend, n):
     # argsort(X, X) of int32 (UniformTest.cpp:2461-2466 does this with short rows): there is no value
