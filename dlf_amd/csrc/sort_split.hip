@@ -782,27 +782,41 @@ __device__ __forceinline__ uint32_t plan_buckets(PlanShared<BLOCK>& sm, const ui
     return n_buckets;
 }
 
-// The plan of row `row` from its chunks' fine-bin histograms, by a workgroup of kSplitBlock threads.
-__device__ __forceinline__ void plan_row(PlanShared<kSplitBlock>& sm, uint32_t* __restrict__ per_bucket, int64_t row, int64_t n, uint32_t cap, int64_t chunks_per_row,
+// The plan of row `row` from its chunks' fine-bin histograms, by a workgroup of BLOCK threads:
+// groups of 256 threads take the chunks in turn (thread t of a group owns fine bins [16 t,
+// 16 t + 16) of its chunks), each with the histograms of eight chunks in flight - what bounds the
+// plan of a long row is the latency of these loads (they miss the L2: other compute units'
+// workgroups wrote them), not their number.  per_chunk: chunks_per_row x 256 words of LDS.
+constexpr int kPlanChunks = 8;
+template <int BLOCK>
+__device__ __forceinline__ void plan_row(PlanShared<BLOCK>& sm, uint32_t* __restrict__ row_hist, uint32_t* __restrict__ per_chunk, int64_t row, int64_t n,
+                                         uint32_t cap, int64_t chunks_per_row,
                                          const uint32_t* __restrict__ chunk_fine, SplitRow* __restrict__ rows, uint32_t* __restrict__ counters,
                                          uint4* __restrict__ bucket_list, CrowdedList crowded, uint32_t* __restrict__ chunk_base, bool piecewise) {
     constexpr int PER = kFine / kSplitBlock;          // 16
-    const uint32_t* f = chunk_fine + row * chunks_per_row * (kFine / 2) + threadIdx.x * (PER / 2);
-    uint32_t cnt[PER];
-#pragma unroll
-    for (int i = 0; i < PER; ++i) cnt[i] = 0;
+    constexpr int GROUPS = BLOCK / kSplitBlock;
+    const int group = threadIdx.x / kSplitBlock, t = threadIdx.x % kSplitBlock;
+    const uint32_t* f = chunk_fine + row * chunks_per_row * (kFine / 2) + t * (PER / 2);
     auto chunk_words = [&](int64_t c, uint32_t (&w)[PER / 2]) __attribute__((always_inline)) {
         const uint4 a = reinterpret_cast<const uint4*>(f + c * (kFine / 2))[0], b = reinterpret_cast<const uint4*>(f + c * (kFine / 2))[1];
         w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w; w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w;
     };
-    for (int64_t c0 = 0; c0 < chunks_per_row; c0 += 4) {             // four chunks' loads in flight
-        uint32_t w[4][PER / 2];
+    // ---- the row's histogram: every group adds up its chunks, the groups add up in LDS
+    uint32_t cnt[PER];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (c0 + j < chunks_per_row) chunk_words(c0 + j, w[j]);
+    for (int i = 0; i < PER; ++i) cnt[i] = 0;
+    if constexpr (GROUPS > 1) {
+        for (int i = threadIdx.x; i < kFine; i += BLOCK) row_hist[i] = 0u;
+    }
+    for (int64_t i = threadIdx.x; i < chunks_per_row * kMaxBuckets; i += BLOCK) per_chunk[i] = 0u;
+    for (int64_t c0 = group; c0 < chunks_per_row; c0 += kPlanChunks * GROUPS) {
+        uint32_t w[kPlanChunks][PER / 2];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            if (c0 + j >= chunks_per_row) break;
+        for (int j = 0; j < kPlanChunks; ++j)
+            if (c0 + j * GROUPS < chunks_per_row) chunk_words(c0 + j * GROUPS, w[j]);
+#pragma unroll
+        for (int j = 0; j < kPlanChunks; ++j) {
+            if (c0 + j * GROUPS >= chunks_per_row) break;
 #pragma unroll
             for (int i = 0; i < PER / 2; ++i) {
                 cnt[2 * i] += w[j][i] & 0xffffu;
@@ -810,44 +824,97 @@ __device__ __forceinline__ void plan_row(PlanShared<kSplitBlock>& sm, uint32_t* 
             }
         }
     }
-    uint32_t bucket[PER];
-    per_bucket[threadIdx.x] = 0u;
-    const uint32_t n_buckets = plan_buckets<kSplitBlock>(sm, cnt, bucket, n, cap, row, rows[row], counters, bucket_list, crowded, nullptr, piecewise);
-    uint32_t next = threadIdx.x < n_buckets ? sm.begin[threadIdx.x] : 0u;      // where the coming chunk's keys of bucket threadIdx.x go
-    // each chunk's keys per bucket, and from them where the chunk writes each bucket
-    uint32_t w8[PER / 2], ahead[PER / 2];
-    chunk_words(0, w8);
-    for (int64_t c = 0; c < chunks_per_row; ++c) {
-        if (c + 1 < chunks_per_row) chunk_words(c + 1, ahead);        // on its way across this chunk's barriers
-        // this thread's bins lie in few buckets: sum runs of equal buckets before touching LDS
-        uint32_t acc = 0;
+    if constexpr (GROUPS > 1) {
+        __syncthreads();
 #pragma unroll
-        for (int i = 0; i < PER; ++i) {
-            acc += (i & 1) ? (w8[i / 2] >> 16) : (w8[i / 2] & 0xffffu);
-            if (i == PER - 1 || bucket[i + 1] != bucket[i]) {
-                if (acc) atomicAdd(&per_bucket[bucket[i]], acc);
-                acc = 0;
-            }
+        for (int i = 0; i < PER; ++i)
+            if (cnt[i]) atomicAdd(&row_hist[t * PER + i], cnt[i]);
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < PER; ++i) cnt[i] = group == 0 ? row_hist[t * PER + i] : 0u;
+        __syncthreads();                               // row_hist is free: the planners' buckets go there next
+    }
+    uint32_t bucket[PER];
+    const uint32_t n_buckets = plan_buckets<BLOCK>(sm, cnt, bucket, n, cap, row, rows[row], counters, bucket_list, crowded, nullptr, piecewise);
+    if constexpr (GROUPS > 1) {
+        // every group needs the buckets of its threads' bins
+        if (group == 0) {
+#pragma unroll
+            for (int i = 0; i < PER; ++i) row_hist[t * PER + i] = bucket[i];
         }
         __syncthreads();
-        chunk_base[(row * chunks_per_row + c) * kMaxBuckets + threadIdx.x] = next;
-        next += per_bucket[threadIdx.x];
-        per_bucket[threadIdx.x] = 0u;
-        __syncthreads();
 #pragma unroll
-        for (int i = 0; i < PER / 2; ++i) w8[i] = ahead[i];
+        for (int i = 0; i < PER; ++i) bucket[i] = row_hist[t * PER + i];
+    }
+    // ---- each chunk's keys per bucket.  A thread's 16 bins lie in two buckets at most as a rule -
+    // the bins up to the first change of bucket (left_bins) and the rest: two sums and two LDS
+    // atomics a chunk.
+    uint32_t left_bins = (1u << PER) - 1u;
+    int changes = 0;
+#pragma unroll
+    for (int i = 0; i + 1 < PER; ++i) {
+        if (bucket[i + 1] != bucket[i]) {
+            if (changes == 0) left_bins = (2u << i) - 1u;
+            ++changes;
+        }
+    }
+    const bool two_at_most = changes <= 1;
+    for (int64_t c0 = group; c0 < chunks_per_row; c0 += kPlanChunks * GROUPS) {
+        uint32_t w[kPlanChunks][PER / 2];
+#pragma unroll
+        for (int j = 0; j < kPlanChunks; ++j)
+            if (c0 + j * GROUPS < chunks_per_row) chunk_words(c0 + j * GROUPS, w[j]);
+#pragma unroll
+        for (int j = 0; j < kPlanChunks; ++j) {
+            const int64_t c = c0 + j * GROUPS;
+            if (c >= chunks_per_row) break;
+            uint32_t* into = per_chunk + c * kMaxBuckets;
+            if (two_at_most) {
+                uint32_t total = 0, left = 0;
+#pragma unroll
+                for (int i = 0; i < PER; ++i) {
+                    const uint32_t count = (i & 1) ? (w[j][i / 2] >> 16) : (w[j][i / 2] & 0xffffu);
+                    total += count;
+                    left += ((left_bins >> i) & 1u) ? count : 0u;
+                }
+                if (left) atomicAdd(&into[bucket[0]], left);
+                if (total != left) atomicAdd(&into[bucket[PER - 1]], total - left);
+            } else {
+                uint32_t acc = 0;
+#pragma unroll
+                for (int i = 0; i < PER; ++i) {
+                    acc += (i & 1) ? (w[j][i / 2] >> 16) : (w[j][i / 2] & 0xffffu);
+                    if (i == PER - 1 || bucket[i + 1] != bucket[i]) {
+                        if (acc) atomicAdd(&into[bucket[i]], acc);
+                        acc = 0;
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+    // ---- and from them where every chunk writes each bucket: thread b carries bucket b through the chunks
+    if (threadIdx.x < kMaxBuckets) {
+        uint32_t next = threadIdx.x < n_buckets ? sm.begin[threadIdx.x] : 0u;
+        for (int64_t c = 0; c < chunks_per_row; ++c) {
+            chunk_base[(row * chunks_per_row + c) * kMaxBuckets + threadIdx.x] = next;
+            next += per_chunk[c * kMaxBuckets + threadIdx.x];
+        }
     }
 }
 
-__global__ __launch_bounds__(kSplitBlock) void split_plan(int64_t n, uint32_t cap, int64_t chunks_per_row, const uint32_t* __restrict__ chunk_fine,
-                                                          SplitRow* __restrict__ rows, uint32_t* __restrict__ counters,
-                                                          uint4* __restrict__ bucket_list, CrowdedList crowded,
-                                                          uint32_t* __restrict__ chunk_base) {
-    __shared__ PlanShared<kSplitBlock> sm;
-    __shared__ uint32_t per_bucket[kMaxBuckets];
+// (BLOCK: 256 for rows of up to eight chunks - all their histograms are in flight at once anyway - and 1024 beyond)
+template <int BLOCK>
+__global__ __launch_bounds__(BLOCK) void split_plan(int64_t n, uint32_t cap, int64_t chunks_per_row, const uint32_t* __restrict__ chunk_fine,
+                                                    SplitRow* __restrict__ rows, uint32_t* __restrict__ counters,
+                                                    uint4* __restrict__ bucket_list, CrowdedList crowded,
+                                                    uint32_t* __restrict__ chunk_base) {
+    __shared__ PlanShared<BLOCK> sm;
+    __shared__ uint32_t row_hist[BLOCK > kSplitBlock ? kFine : 1];
+    extern __shared__ uint32_t per_chunk[];            // chunks_per_row x 256 words
     const int64_t row = blockIdx.x;
     if (row == 0 && threadIdx.x == 0) counters[4] = 0u;       // split_remap has read it: zero again for the next sort that uses this memory
-    plan_row(sm, per_bucket, row, n, cap, chunks_per_row, chunk_fine, rows, counters, bucket_list, crowded, chunk_base, rows[row].piecewise != 0u);
+    plan_row<BLOCK>(sm, row_hist, per_chunk, row, n, cap, chunks_per_row, chunk_fine, rows, counters, bucket_list, crowded, chunk_base, rows[row].piecewise != 0u);
 }
 
 // ------------------------------------------------------------------ 3b. rows whose keys cluster
@@ -2223,7 +2290,11 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
             split_histogram<K, decltype(map_tag)::value><<<chunks, dim3(kSplitBlock), 0, stream>>>(io, n, l.chunks_per_row, rows, fine, maps);
         });
         DLFX_CHECK_LAUNCH();
-        split_plan<<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), 0, stream>>>(n, static_cast<uint32_t>(cap), l.chunks_per_row, fine, rows, counters, list, crowded, chunk_base);
+        const size_t per_chunk_bytes = static_cast<size_t>(l.chunks_per_row) * kMaxBuckets * sizeof(uint32_t);      // (at most 80 chunks: 80 KB)
+        if (l.chunks_per_row <= kPlanChunks)
+            split_plan<kSplitBlock><<<dim3(static_cast<unsigned>(m)), dim3(kSplitBlock), per_chunk_bytes, stream>>>(n, static_cast<uint32_t>(cap), l.chunks_per_row, fine, rows, counters, list, crowded, chunk_base);
+        else
+            split_plan<1024><<<dim3(static_cast<unsigned>(m)), dim3(1024), per_chunk_bytes, stream>>>(n, static_cast<uint32_t>(cap), l.chunks_per_row, fine, rows, counters, list, crowded, chunk_base);
         DLFX_CHECK_LAUNCH();
     }
     // split_finish: as many workgroups as the device holds at once, each walking its share of the buckets
