@@ -939,13 +939,18 @@ __device__ __forceinline__ void piecewise_map_of(RemapShared<K>& sm, const PassI
     static_assert(kQuantileSample / kSegments == 16 && kSplitBlock == kSegments, "every 16th key of the sorted sample bounds a segment; a thread a segment");
     const int tid = threadIdx.x;
     const int seg = (tid / kWave) * kWave * ITEMS + lane_id();
-    // ---- the sample: 4096 keys at even distances, sorted
+    // ---- the sample, sorted: one key from each of 4096 equal stretches of the row, at a place
+    // inside the stretch that changes from stretch to stretch (a row that repeats with some period
+    // shows all its phases)
     K key[ITEMS];
     uint32_t none[1] = {0u};
     K ors = 0, ands = ~K(0);
+    const int64_t stretch = n / kQuantileSample;
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
-        const int64_t e = (static_cast<int64_t>(seg + k * kWave) * n) / kQuantileSample;
+        const uint32_t p = static_cast<uint32_t>(seg + k * kWave);
+        int64_t e = (static_cast<int64_t>(p) * n) / kQuantileSample;
+        if (stretch > 1) e += static_cast<int64_t>((p * 2654435761u) >> 8) % stretch;
         key[k] = key_of_element<K>(io, xrow[e * io.sx]);
         ors |= key[k];
         ands &= key[k];
