@@ -287,6 +287,22 @@ def make_ops(be, which):
             xs = gen(shape, dtype, lambda c: synth.normal(9 + 100 * c), 4)
             ops += sort_ops(be, tensor, xs, "C4n", text)
 
+    # ---------------- beside the baseline's configurations: rows that evenly spaced bins do not cut -
+    # one value, ten values, and nine keys in ten inside a window of 1000 values with the rest
+    # spread over the whole range (at the C4 shapes and as one long row); not part of all
+    if on("repeats"):
+        def clustered(seed):
+            wide, near, pick = synth.full_range_i64(seed), synth.randint(seed + 1, 0, 1000), synth.randint(seed + 2, 0, 10)
+            return lambda idx: torch.where(pick(idx) > 0, near(idx) + 12345, wide(idx))
+        for shape, dtype, fn, text in (((1024, 65536), torch.float32, lambda c: synth.randint(40 + 100 * c, 0, 10), "f32_ten_values_[1024,65536]"),
+                                       ((256, 1 << 20), torch.int64, lambda c: (lambda idx: torch.full_like(idx, 7)), "i64_one_value_[256,2^20]"),
+                                       ((256, 1 << 20), torch.int64, lambda c: synth.randint(41 + 100 * c, 0, 10), "i64_ten_values_[256,2^20]"),
+                                       ((256, 1 << 20), torch.int64, lambda c: clustered(42 + 100 * c), "i64_clustered_[256,2^20]"),
+                                       ((1, 2500000), torch.int64, lambda c: clustered(43 + 100 * c), "i64_clustered_[1,2500000]"),
+                                       ((1, 2500000), torch.int64, lambda c: synth.full_range_i64(44 + 100 * c), "i64_[1,2500000]")):
+            xs = gen(shape, dtype, fn, 2)
+            ops += [op for op in sort_ops(be, tensor, xs, "C4r", text) if "_asc_" in op.name]
+
     # ---------------- C5: strided NCHW
     if on("all", "c5"):
         x5 = gen((32, 512, 56, 56), torch.float32, lambda c: synth.normal(8 + 100 * c), 6)
@@ -637,7 +653,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3 | short (many short rows and an outer axis; not part of all) | spread (sorts of N(0,1) rows; not part of all) | ceil (copy and read-only streams at the C2 and C5 sizes; part of all) | ceilbig (the same streams at 1 GiB and 4 GiB; not part of all) | long (softmax and top_k over a few very long rows; not part of all)")
+    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3 | short (many short rows and an outer axis; not part of all) | spread (sorts of N(0,1) rows; not part of all) | ceil (copy and read-only streams at the C2 and C5 sizes; part of all) | ceilbig (the same streams at 1 GiB and 4 GiB; not part of all) | long (softmax and top_k over a few very long rows; not part of all) | repeats (sorts of rows of one value, of ten values and of clustered keys; not part of all)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
