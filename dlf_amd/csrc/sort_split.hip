@@ -604,6 +604,15 @@ struct PlanShared {
     uint32_t begin[kMaxBuckets + 1];
 };
 
+// What packing a row's fine bins into buckets one by one needs (plan_buckets, when its formula
+// asks for more buckets than there are).
+struct PackShared {
+    uint32_t prefix[kFine + 1];                        // keys before every fine bin
+    uint16_t next[kFine];                              // the bin after the fullest bucket that starts at a bin
+    uint16_t start[kMaxBuckets + 2];                   // first bin of every bucket
+    uint32_t buckets;
+};
+
 // The buckets of row `row` from its fine-bin counts: planning thread t (the first 256 threads of
 // a workgroup of BLOCK) brings the counts of fine bins [16 t, 16 t + 16) in cnt[] and receives
 // their buckets in bucket[]; the other threads bring zeros and only keep the barriers company.
@@ -612,7 +621,8 @@ struct PlanShared {
 template <int BLOCK>
 __device__ __forceinline__ uint32_t plan_buckets(PlanShared<BLOCK>& sm, const uint32_t (&cnt)[kFine / kSplitBlock], uint32_t (&bucket)[kFine / kSplitBlock],
                                                  int64_t n, uint32_t cap, int64_t row, SplitRow& info, uint32_t* __restrict__ counters,
-                                                 uint4* __restrict__ bucket_list, CrowdedList crowded, uint32_t* route_out = nullptr, bool piecewise = false) {
+                                                 uint4* __restrict__ bucket_list, CrowdedList crowded, uint32_t* route_out = nullptr, bool piecewise = false,
+                                                 PackShared* pack = nullptr) {
     constexpr int PER = kFine / kSplitBlock;          // 16
     constexpr int WAVES = BLOCK / kWave;
     const int w = threadIdx.x / kWave;
@@ -691,6 +701,69 @@ __device__ __forceinline__ uint32_t plan_buckets(PlanShared<BLOCK>& sm, const ui
     if (biggest < cap) {
         n_buckets = assign(cap - biggest, gap_cuts);
         if (n_buckets > static_cast<uint32_t>(kMaxBuckets)) n_buckets = assign(cap - biggest, 0u);
+    }
+    if (n_buckets > static_cast<uint32_t>(kMaxBuckets) && biggest < cap && pack != nullptr) {
+        // Too many buckets that way (a long row: the formula leaves room for the row's largest bin
+        // in every bucket): the bins are packed one bucket after the other instead, each bucket
+        // taking bins while they fit.  Every bin finds where the fullest bucket that starts
+        // with it ends (bisection over the prefix sums); one thread then walks from bucket to
+        // bucket - 256 dependent steps at most, on this path only.
+        if (planner) {
+            uint32_t run = before;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) {
+                pack->prefix[threadIdx.x * PER + i] = run;
+                run += cnt[i];
+            }
+            if (threadIdx.x == kSplitBlock - 1) pack->prefix[kFine] = run;
+        }
+        __syncthreads();
+        if (planner) {
+#pragma unroll 1
+            for (int i = 0; i < PER; ++i) {
+                const int bin = static_cast<int>(threadIdx.x) * PER + i;
+                const uint32_t most = pack->prefix[bin] + cap;
+                int lo = bin + 1, hi = kFine;                          // the answer lies in [lo, hi]: every bin alone fits
+                while (lo < hi) {
+                    const int mid = (lo + hi + 1) >> 1;
+                    if (pack->prefix[mid] <= most) lo = mid;
+                    else hi = mid - 1;
+                }
+                pack->next[bin] = static_cast<uint16_t>(lo);
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            uint32_t b = 0;
+            int pos = 0;
+            while (pos < kFine && b <= static_cast<uint32_t>(kMaxBuckets)) {
+                pack->start[b++] = static_cast<uint16_t>(pos);
+                pos = pack->next[pos];
+            }
+            pack->start[b < static_cast<uint32_t>(kMaxBuckets) + 1u ? b : static_cast<uint32_t>(kMaxBuckets) + 1u] = static_cast<uint16_t>(kFine);
+            pack->buckets = pos < kFine ? static_cast<uint32_t>(kMaxBuckets) + 1u : b;
+        }
+        __syncthreads();
+        const uint32_t packed = pack->buckets;
+        if (packed <= static_cast<uint32_t>(kMaxBuckets)) {
+            if (planner) {
+                const int first_bin = static_cast<int>(threadIdx.x) * PER;
+                uint32_t lo = 0, hi = packed - 1u;                     // the bucket of this thread's first bin
+                while (lo < hi) {
+                    const uint32_t mid = (lo + hi + 1u) >> 1;
+                    if (static_cast<int>(pack->start[mid]) <= first_bin) lo = mid;
+                    else hi = mid - 1u;
+                }
+#pragma unroll
+                for (int i = 0; i < PER; ++i) {
+                    while (lo + 1u < packed && first_bin + i >= static_cast<int>(pack->start[lo + 1u])) ++lo;
+                    bucket[i] = lo;
+                }
+                sm.last_bucket[threadIdx.x] = bucket[PER - 1];
+            }
+            __syncthreads();
+            n_buckets = packed;
+        }
     }
     if (n_buckets > static_cast<uint32_t>(kMaxBuckets)) {
         // Some fine bin does not (or too many buckets would be needed): the row gets buckets of
@@ -789,7 +862,7 @@ __device__ __forceinline__ uint32_t plan_buckets(PlanShared<BLOCK>& sm, const ui
 // workgroups wrote them), not their number.  per_chunk: chunks_per_row x 256 words of LDS.
 constexpr int kPlanChunks = 8;
 template <int BLOCK>
-__device__ __forceinline__ void plan_row(PlanShared<BLOCK>& sm, uint32_t* __restrict__ row_hist, uint32_t* __restrict__ per_chunk, int64_t row, int64_t n,
+__device__ __forceinline__ void plan_row(PlanShared<BLOCK>& sm, PackShared& pack, uint32_t* __restrict__ row_hist, uint32_t* __restrict__ per_chunk, int64_t row, int64_t n,
                                          uint32_t cap, int64_t chunks_per_row,
                                          const uint32_t* __restrict__ chunk_fine, SplitRow* __restrict__ rows, uint32_t* __restrict__ counters,
                                          uint4* __restrict__ bucket_list, CrowdedList crowded, uint32_t* __restrict__ chunk_base, bool piecewise) {
@@ -835,7 +908,7 @@ __device__ __forceinline__ void plan_row(PlanShared<BLOCK>& sm, uint32_t* __rest
         __syncthreads();                               // row_hist is free: the planners' buckets go there next
     }
     uint32_t bucket[PER];
-    const uint32_t n_buckets = plan_buckets<BLOCK>(sm, cnt, bucket, n, cap, row, rows[row], counters, bucket_list, crowded, nullptr, piecewise);
+    const uint32_t n_buckets = plan_buckets<BLOCK>(sm, cnt, bucket, n, cap, row, rows[row], counters, bucket_list, crowded, nullptr, piecewise, &pack);
     if constexpr (GROUPS > 1) {
         // every group needs the buckets of its threads' bins
         if (group == 0) {
@@ -910,11 +983,12 @@ __global__ __launch_bounds__(BLOCK) void split_plan(int64_t n, uint32_t cap, int
                                                     uint4* __restrict__ bucket_list, CrowdedList crowded,
                                                     uint32_t* __restrict__ chunk_base) {
     __shared__ PlanShared<BLOCK> sm;
+    __shared__ PackShared pack;
     __shared__ uint32_t row_hist[BLOCK > kSplitBlock ? kFine : 1];
     extern __shared__ uint32_t per_chunk[];            // chunks_per_row x 256 words
     const int64_t row = blockIdx.x;
     if (row == 0 && threadIdx.x == 0) counters[4] = 0u;       // split_remap has read it: zero again for the next sort that uses this memory
-    plan_row<BLOCK>(sm, row_hist, per_chunk, row, n, cap, chunks_per_row, chunk_fine, rows, counters, bucket_list, crowded, chunk_base, rows[row].piecewise != 0u);
+    plan_row<BLOCK>(sm, pack, row_hist, per_chunk, row, n, cap, chunks_per_row, chunk_fine, rows, counters, bucket_list, crowded, chunk_base, rows[row].piecewise != 0u);
 }
 
 // ------------------------------------------------------------------ 3b. rows whose keys cluster
@@ -2230,8 +2304,11 @@ SplitLayout split_layout(int64_t m, int64_t n) {
 }  // namespace
 
 // Whether rows of n keys can take the bucket route at all (each row then decides on the device).
+// (the longest rows: nine tenths of what 256 of the largest buckets hold - fine bins do not fill
+// buckets to the brim, and a row that needs more buckets than there are gets oversized ones)
+constexpr int64_t kLongestRow = static_cast<int64_t>(kMaxBuckets) * kCapHuge / 10 * 9;
 bool split_route_takes(size_t key_size, int64_t m, int64_t n) {
-    return (key_size == 4 || key_size == 8) && n <= static_cast<int64_t>(kMaxBuckets - 1) * kCapHuge &&
+    return (key_size == 4 || key_size == 8) && n <= kLongestRow &&
            m * kMaxBuckets <= 0x7fffffffLL && m * ceil_div(n, static_cast<int64_t>(kChunk)) <= 0x7fffffffLL;
 }
 
