@@ -308,7 +308,7 @@ struct FineRange {
 // every wavefront offers are those of the first four.
 //
 // The sample also shows whether the row's keys cluster more tightly than the chosen map resolves:
-// a fine bin that holds so many of the sample's keys that it promises twice what a bucket may
+// a fine bin that holds so many of the sample's keys that it promises more than a bucket may
 // hold, and keys that differ among them (one value repeated is no trouble: its bucket is done
 // when it has been moved).  Such a row is marked `piecewise`.  sample_hist: kFine words of LDS,
 // zero on entry and on return.
@@ -441,8 +441,12 @@ __device__ __forceinline__ FineRange sample_row(const PassIo<K>& io, const K* __
             if (sampler) atomicAdd(&sample_hist[f[u]], 1u);
         }
         __syncthreads();
-        const unsigned long long by_size = (2ull * cap * 1024ull + static_cast<unsigned long long>(n) - 1ull) / static_cast<unsigned long long>(n);
-        const uint32_t many = by_size > 8ull ? static_cast<uint32_t>(by_size) : 8u;       // (eight: never reached by chance on evenly spread keys)
+        // (what a full bucket's worth of keys shows in the sample, and four standard deviations of
+        // that count more - twice that at most; eight at least, which evenly spread keys never reach by chance)
+        const float full = static_cast<float>(cap) * 1024.0f / static_cast<float>(n);
+        const float margin = 4.0f * sqrtf(full) + 1.0f;
+        const uint32_t by_size = static_cast<uint32_t>(full + (margin < full ? margin : full)) + 1u;
+        const uint32_t many = by_size > 8u ? by_size : 8u;
         bool crowded[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) crowded[u] = sampler && sample_hist[f[u]] >= many;
@@ -2340,7 +2344,10 @@ int run_split(hipStream_t stream, const PassIo<K>& io, bool pairs, int64_t m, in
     // not much beside a bucket while the row has under a dozen buckets' worth of keys, and the
     // finer bins of the closed gap would only split the thin tails into many small buckets
     // (measured on normal rows: open gap ahead up to 24 000 keys, closed from 32 768).
-    const int map = io.kind != kKeyFloat ? kMapPlain : waves > 4 ? kMapValue : n >= 12 * static_cast<int64_t>(cap) ? kMapGap : kMapPlain;
+    // Doubles always: their sign and exponent alone fill the 12 bits of a fine bin's number, so with
+    // the gap open a row on both sides of zero has one bin to a binade or less, and a bell-shaped
+    // row a bin fuller than a bucket (N(0,1) doubles, rows of 10 000: 15 Gkeys/s with the gap open).
+    const int map = io.kind != kKeyFloat ? kMapPlain : waves > 4 ? kMapValue : (sizeof(K) == 8 || n >= 12 * static_cast<int64_t>(cap)) ? kMapGap : kMapPlain;
     auto with_map = [&](auto&& launch_with) {
         if (map == kMapPlain) launch_with(std::integral_constant<int, kMapPlain>());
         else if (map == kMapGap) launch_with(std::integral_constant<int, kMapGap>());
