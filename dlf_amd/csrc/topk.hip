@@ -1424,6 +1424,7 @@ do {                                                                            
 struct LongPlan {
     bool ok;
     int64_t seg_len, segs, last_n;
+    int64_t keep;                      // what every segment leaves: `limit`, or one more (below)
     size_t val_off, idx_off, pos_off, rest_off, total;
 };
 
@@ -1437,28 +1438,35 @@ LongPlan long_plan(int dtype, size_t elem_size, size_t key_size, int64_t m, int6
     p.seg_len = align_up(static_cast<size_t>(ceil_div(n, segs)), 8);      // segments start on 16-byte boundaries when the row does
     p.segs = ceil_div(n, p.seg_len);
     p.last_n = n - (p.segs - 1) * p.seg_len;
-    if (p.segs < 2 || p.last_n < limit || p.segs * limit > n / 2 || m * p.segs > 0x7fffffffLL) return p;
-    const size_t cands = static_cast<size_t>(m) * p.segs * limit;
+    // The winners lie in the candidate array as sorted runs, one per segment.  The selection
+    // kernel gives a thread four neighbouring elements out of every 4096, so with runs of a length
+    // that divides 4096 a thread would hold the same ranks of every run - a few threads all the
+    // heads - and the bound it takes from samples of the threads' maxima would let thousands
+    // through ([1, 2^24], limit 256: 250 us; limit 257: 68 us).  An even limit therefore keeps one
+    // winner more per segment: runs of odd length, which shift from one group of 4096 to the next.
+    p.keep = (limit % 2 == 0 && limit < kMaxLimit) ? limit + 1 : limit;
+    if (p.segs < 2 || p.last_n < p.keep || p.segs * p.keep > n / 2 || m * p.segs > 0x7fffffffLL) return p;
+    const size_t cands = static_cast<size_t>(m) * p.segs * p.keep;
     p.val_off = 0;
     p.idx_off = align_up(cands * elem_size, 256);
     p.pos_off = p.idx_off + align_up(cands * 4, 256);
     p.rest_off = p.pos_off + align_up(static_cast<size_t>(m) * limit * 4, 256);
     const size_t first = select_layout(key_size, m * p.segs, p.seg_len).total;
-    const size_t second = top_k_scratch_impl(dtype, m, p.segs * limit, limit);
+    const size_t second = top_k_scratch_impl(dtype, m, p.segs * p.keep, limit);
     p.total = p.rest_off + (first > second ? first : second);
     p.ok = true;
     return p;
 }
 
 __global__ __launch_bounds__(256) void topk_places_to_indices(const int32_t* __restrict__ place, const uint32_t* __restrict__ cand_idx,
-                                                              int64_t rows, int limit, int64_t segs, int64_t seg_len,
+                                                              int64_t rows, int limit, int64_t keep, int64_t segs, int64_t seg_len,
                                                               void* idx, DimMap imap, int64_t si, int idx64) {
     const int64_t g = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (g >= rows * limit) return;
     const int64_t row = g / limit;
     const int j = static_cast<int>(g - row * limit);
-    const int64_t p = place[g];
-    const int64_t ix = (p / limit) * seg_len + cand_idx[row * segs * limit + p];
+    const int64_t p = place[g];                        // among the row's segs * keep candidates
+    const int64_t ix = (p / keep) * seg_len + cand_idx[row * segs * keep + p];
     const int64_t at = imap.at(row) + j * si;
     if (idx64) static_cast<int64_t*>(idx)[at] = ix;
     else static_cast<int32_t*>(idx)[at] = static_cast<int32_t>(ix);
@@ -1563,16 +1571,16 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
         io1.idx = cand_idx;
         io1.ymap.rank = io1.imap.rank = 1;
         io1.ymap.dims[0] = io1.imap.dims[0] = m * lp.segs;
-        io1.ymap.strides[0] = io1.imap.strides[0] = limit;
+        io1.ymap.strides[0] = io1.imap.strides[0] = lp.keep;
         io1.sy = io1.si = 1;
         io1.idx64 = 0;
         io1.segs = lp.segs;
         io1.last_n = lp.last_n;
-        int st = launch_select<T>(stream, io1, m * lp.segs, lp.seg_len, limit, base + lp.rest_off, scratch_bytes - lp.rest_off);
+        int st = launch_select<T>(stream, io1, m * lp.segs, lp.seg_len, lp.keep, base + lp.rest_off, scratch_bytes - lp.rest_off);
         if (st != DLFX_OK) return st;
         int64_t c_dims[64], c_strides[64], p_strides[64];
         for (int i = 0; i < rank; ++i) c_dims[i] = x_dims[i];
-        c_dims[rank - 1] = lp.segs * limit;
+        c_dims[rank - 1] = lp.segs * lp.keep;
         int64_t cs = 1, ps = 1;
         for (int i = rank - 1; i >= 0; --i) {
             c_strides[i] = cs;
@@ -1585,7 +1593,7 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
         if (st != DLFX_OK) return st;
         const int64_t outs = m * limit;
         topk_places_to_indices<<<dim3(static_cast<unsigned>(ceil_div(outs, 256))), dim3(256), 0, stream>>>(
-            place, cand_idx, m, lim, lp.segs, lp.seg_len, idx, io.imap, io.si, io.idx64);
+            place, cand_idx, m, lim, lp.keep, lp.segs, lp.seg_len, idx, io.imap, io.si, io.idx64);
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
     }
