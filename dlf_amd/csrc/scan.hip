@@ -584,22 +584,81 @@ __global__ __launch_bounds__(BLOCK) void scan_rows_chained(
 // positions [s + ty*chunk, s + (ty+1)*chunk) in registers.
 constexpr int kColsChunk = 16;      // rows of a column a wave scans per round (4, 8 and 32 measured: slower)
 
+// Few columns and a long axis would leave the chip to a handful of workgroups walking the whole
+// axis one round after the other: the axis is then cut into segments of seg_len positions, a
+// workgroup per (block of 64 columns, segment).  scan_cols_partials leaves every segment's
+// total per column in `partials` ([segment][column]); scan_cols starts a segment from what the
+// segments before it add up to.  The input is read twice - three crossings instead of two -
+// by as many workgroups as fill the device.
+struct ColSegments {
+    int64_t seg_len, segs, col_blocks;     // one segment: seg_len = n, segs = 1
+};
+
+template <typename T, int K, typename X, bool NZ>
+__global__ __launch_bounds__(kBlock) void scan_cols_partials(
+    const X* __restrict__ x, DimMap xmap, int64_t sx, int64_t m, int64_t n, ColSegments cut, T* __restrict__ partials) {
+    using Op = ScanOp<T, K>;
+    constexpr int R = kColsChunk;
+    __shared__ T totals[kWaves][kWave];
+    const int lx = threadIdx.x & (kWave - 1);
+    const int ty = threadIdx.x / kWave;
+    const int64_t col_block = blockIdx.x % cut.col_blocks, seg = blockIdx.x / cut.col_blocks;
+    const int64_t col = col_block * kWave + lx;
+    const bool live = col < m;
+    const X* xc = x + (live ? xmap.at(col) : 0);
+    const int64_t lo = seg * cut.seg_len;
+    const int64_t hi = lo + cut.seg_len < n ? lo + cut.seg_len : n;
+    T sum = Op::identity();
+    // wave ty takes positions lo + 16 ty, + 64, ...: sixteen loads in flight a lane
+    for (int64_t p0 = lo + static_cast<int64_t>(ty) * R; p0 < hi; p0 += static_cast<int64_t>(kWaves) * R) {
+        T v[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t p = p0 + r;
+            v[r] = (live && p < hi) ? scan_input<T, X, NZ>(load_stream(&xc[p * sx])) : Op::identity();
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) sum = Op::apply(sum, v[r]);
+    }
+    totals[ty][lx] = sum;
+    __syncthreads();
+    if (ty == 0 && live) {
+        T all = totals[0][lx];
+#pragma unroll
+        for (int i = 1; i < kWaves; ++i) all = Op::apply(all, totals[i][lx]);
+        partials[seg * m + col] = all;
+    }
+}
+
 template <typename T, int K, typename X, bool NZ, typename Y>
 __global__ __launch_bounds__(kBlock) void scan_cols(
     const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
-    int64_t m, int64_t n, int chunk, int exclusive) {
+    int64_t m, int64_t n, int chunk, int exclusive, ColSegments cut, const T* __restrict__ partials) {
     using Op = ScanOp<T, K>;
     constexpr int R = kColsChunk;
     __shared__ T totals[2][kWaves][kWave];
 
     const int lx = threadIdx.x & (kWave - 1);
     const int ty = threadIdx.x / kWave;
-    const int64_t col = static_cast<int64_t>(blockIdx.x) * kWave + lx;
+    const int64_t col_block = blockIdx.x % cut.col_blocks, seg = blockIdx.x / cut.col_blocks;
+    const int64_t col = col_block * kWave + lx;
     const bool live = col < m;
     const X* xc = x + (live ? xmap.at(col) : 0);
     Y* yc = y + (live ? ymap.at(col) : 0);
+    const int64_t lo = seg * cut.seg_len;
+    const int64_t hi = lo + cut.seg_len < n ? lo + cut.seg_len : n;        // this workgroup scans positions [lo, hi)
 
     T carry = Op::identity();
+    if (cut.segs > 1 && live) {
+        // what the segments before this one add up to (their totals, in order: four loads in flight)
+        for (int64_t s0 = 0; s0 < seg; s0 += 4) {
+            T part[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) part[j] = s0 + j < seg ? partials[(s0 + j) * m + col] : Op::identity();
+#pragma unroll
+            for (int j = 0; j < 4; ++j) carry = Op::apply(carry, part[j]);
+        }
+    }
     int buf = 0;
     const int64_t step = static_cast<int64_t>(kWaves) * chunk;
     // the wave's chunk of the next round is on its way while this round is scanned and stored
@@ -608,17 +667,17 @@ __global__ __launch_bounds__(kBlock) void scan_cols(
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int64_t p = p0 + r;
-            v[r] = (live && r < chunk && p < n) ? scan_input<T, X, NZ>(load_stream(&xc[p * sx])) : Op::identity();
+            v[r] = (live && r < chunk && p < hi) ? scan_input<T, X, NZ>(load_stream(&xc[p * sx])) : Op::identity();
         }
     };
     T ahead[R];
-    load_chunk(0, ahead);
-    for (int64_t s = 0; s < n; s += step, buf ^= 1) {
+    load_chunk(lo, ahead);
+    for (int64_t s = lo; s < hi; s += step, buf ^= 1) {
         const int64_t p0 = s + static_cast<int64_t>(ty) * chunk;
         T v[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) v[r] = ahead[r];
-        if (s + step < n) load_chunk(s + step, ahead);
+        if (s + step < hi) load_chunk(s + step, ahead);
 #pragma unroll
         for (int r = 1; r < R; ++r) v[r] = Op::apply(v[r - 1], v[r]);
         totals[buf][ty][lx] = v[R - 1];
@@ -638,13 +697,13 @@ __global__ __launch_bounds__(kBlock) void scan_cols(
                 for (int r = 0; r < R; ++r) {
                     const int64_t p = p0 + r;
                     const T prev = (r == 0) ? pre : Op::apply(pre, v[r > 0 ? r - 1 : 0]);
-                    if (r < chunk && p < n) store_stream(&yc[p * sy], static_cast<Y>(prev));
+                    if (r < chunk && p < hi) store_stream(&yc[p * sy], static_cast<Y>(prev));
                 }
             } else {
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const int64_t p = p0 + r;
-                    if (r < chunk && p < n) store_stream(&yc[p * sy], static_cast<Y>(Op::apply(pre, v[r])));
+                    if (r < chunk && p < hi) store_stream(&yc[p * sy], static_cast<Y>(Op::apply(pre, v[r])));
                 }
             }
         }
@@ -704,6 +763,33 @@ int64_t tile_elems(size_t elem_size, int64_t n) {
     for (int64_t tile = 256; tile < full; tile *= (tile == 256 ? 4 : 2))
         if (n <= tile) return tile;
     return full;
+}
+
+// How scan_cols cuts the axis of m columns of n positions: not at all while the blocks of 64
+// columns alone give the device enough workgroups (or the axis is short); otherwise into segments
+// of whole rounds (64 positions), about 1024 workgroups in all, no segment under 512 positions.
+ColSegments col_segments(int64_t m, int64_t n) {
+    ColSegments c;
+    c.col_blocks = ceil_div(m, static_cast<int64_t>(kWave));
+    c.seg_len = n;
+    c.segs = 1;
+    if (c.col_blocks >= 512 || n < 2048) return c;
+    int64_t want = ceil_div(static_cast<int64_t>(1024), c.col_blocks);
+    const int64_t most = n / 512;
+    if (want > most) want = most;
+    if (want < 2) return c;
+    c.seg_len = align_up(static_cast<size_t>(ceil_div(n, want)), static_cast<size_t>(kWaves * kColsChunk));
+    c.segs = ceil_div(n, c.seg_len);
+    if (c.segs < 2) {
+        c.seg_len = n;
+        c.segs = 1;
+    }
+    return c;
+}
+
+size_t col_partials_bytes(size_t elem_size, int64_t m, int64_t n) {
+    const ColSegments c = col_segments(m, n);
+    return c.segs > 1 ? static_cast<size_t>(c.segs) * static_cast<size_t>(m) * elem_size : 0;
 }
 
 struct ScanLayout {
@@ -823,13 +909,23 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
         return DLFX_OK;
     }
     const bool short_rows = n <= 64 && m >= 256;
-    const bool use_cols = !axis_general && (short_rows || (!axis_unit && m >= 64 && (inner_unit || n < 4096)));
+    // (columns side by side in memory: from 64 of them; from 8 when the axis has a million positions or more -
+    // [4194304, 16] fp32 along the first axis: 309 GB/s as strided rows, 1643 GB/s as columns, three lanes in
+    // four idle; [262144, 16]: 674 against 497)
+    const ColSegments cut = col_segments(m, n);
+    const bool use_cols = !axis_general && (short_rows || (!axis_unit && (m >= 64 || (m >= 8 && n >= (1 << 20))) && (inner_unit || n < 4096)));
     if (use_cols) {
         int chunk = static_cast<int>(ceil_div(n, kWaves) < kColsChunk ? ceil_div(n, kWaves) : kColsChunk);
-        const int64_t blocks = ceil_div(m, kWave);
+        const int64_t blocks = cut.col_blocks * cut.segs;
         if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
+        T* partials = static_cast<T*>(scratch);
+        if (cut.segs > 1) {
+            if (!scratch || scratch_bytes < col_partials_bytes(sizeof(T), m, n)) return DLFX_ERR_SCRATCH_TOO_SMALL;
+            scan_cols_partials<T, K, X, NZ><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(x, xmap, sx, m, n, cut, partials);
+            DLFX_CHECK_LAUNCH();
+        }
         scan_cols<T, K, X, NZ, Y><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
-            x, y, xmap, ymap, sx, sy, m, n, chunk, exclusive);
+            x, y, xmap, ymap, sx, sy, m, n, chunk, exclusive, cut, partials);
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
     }
@@ -935,7 +1031,9 @@ extern "C" size_t dlfx_scan_scratch_bytes(int dtype, int64_t m, int64_t n) {
     size_t es = dtype_size(dtype);
     if (dtype == DLFX_F16) es = 4;                  // scanned as fp32
     if (es < 4 || m <= 0 || n <= 0) return 0;
-    return scan_layout(es, m, n + kMaxPad).total;       // rows off a vector boundary take up to a vector more
+    const size_t rows = dlfx::scan_layout(es, m, n + dlfx::kMaxPad).total;       // rows off a vector boundary take up to a vector more
+    const size_t cols = dlfx::col_partials_bytes(es, m, n);                       // (an axis that is not the innermost, cut into segments)
+    return rows > cols ? rows : cols;
 }
 
 extern "C" int dlfx_scan(dlfx_stream_t stream, const char* name, int dtype, int64_t m, int64_t n,

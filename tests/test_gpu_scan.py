@@ -305,3 +305,28 @@ def test_rows_off_a_vector_boundary(hip_backend, oracle_backend, n):
             assert np.array_equal(F.cumsum(Xh.slice([1], [1 + n], [1]), 1).numpy(), np.cumsum(x[:, 1:], axis=1, dtype=np.int32))
         finally:
             hip_backend.set_tuning("scan_poll_limit", 2048)
+
+
+@pytest.mark.parametrize("shape,axis", [((40000, 64), 0), ((100000, 17), 0), ((3, 9000, 100), 1), ((2050, 1000), 0), ((262144, 8), 0), ((5000, 7), 0)])
+def test_long_axis_beside_few_columns_is_cut_into_segments(hip_backend, shape, axis):
+    # an axis that is not the innermost, long, with too few columns beside it to fill the device:
+    # workgroups take segments of the axis and start from the totals of the segments before them
+    # (the last shape has too few columns for that kernel and keeps the strided rows)
+    x = randint(480, int(np.prod(shape)), -50, 50).astype(np.int32).reshape(shape)
+    Xh = Tensor.from_numpy(hip_backend, x)
+    assert np.array_equal(F.cumsum(Xh, axis).numpy(), np.cumsum(x, axis=axis, dtype=np.int32))
+    ex = np.cumsum(x, axis=axis, dtype=np.int32) - x
+    assert np.array_equal(F.cumsum(Xh, axis, True).numpy(), ex)
+    rev = np.flip(np.cumsum(np.flip(x, axis), axis=axis, dtype=np.int32), axis)
+    assert np.array_equal(F.cumsum(Xh, axis, False, True).numpy(), rev)
+    assert np.array_equal(F.cummax(Xh, axis).numpy(), np.maximum.accumulate(x, axis=axis))
+    assert np.array_equal(F.cummin(Xh, axis).numpy(), np.minimum.accumulate(x, axis=axis))
+    y = (normal(481, int(np.prod(shape))) * 3).astype(np.float32).reshape(shape)
+    Yh = Tensor.from_numpy(hip_backend, y)
+    got = F.cumsum(Yh, axis).numpy().astype(np.float64)
+    want = np.cumsum(y.astype(np.float64), axis=axis)
+    mag = np.cumsum(np.abs(y.astype(np.float64)), axis=axis)
+    n = shape[axis]
+    assert np.all(np.abs(got - want) <= 4 * np.log2(n) * np.finfo(np.float32).eps * np.maximum(np.abs(want), mag))
+    F.cumsum(Xh, axis, out=Xh)                                          # in place
+    assert np.array_equal(Xh.numpy(), np.cumsum(x, axis=axis, dtype=np.int32))
