@@ -239,7 +239,7 @@ struct CountReducer {
 template <typename R>
 __device__ __forceinline__ typename R::acc_t
 row_partial_contig(const typename R::in_t* __restrict__ p, int64_t n, int g, int width,
-                   int64_t part, int64_t parts, typename R::param_t prm) {
+                   int64_t part, int64_t parts, typename R::param_t prm, int64_t first_index = 0) {
     using T = typename R::in_t;
     using acc_t = typename R::acc_t;
     constexpr int V = vec_width<T>();
@@ -262,7 +262,7 @@ row_partial_contig(const typename R::in_t* __restrict__ p, int64_t n, int g, int
     for (; v + 3 * static_cast<int64_t>(width) < v_hi; v += 4 * static_cast<int64_t>(width)) {
         VecT a = load_stream(&pv[v]), b = load_stream(&pv[v + width]), c = load_stream(&pv[v + 2 * width]),
              d = load_stream(&pv[v + 3 * width]);
-        const int64_t j0 = head + v * V;
+        const int64_t j0 = first_index + head + v * V;
 #pragma unroll
         for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(a.v[e], j0 + e, prm));
 #pragma unroll
@@ -274,14 +274,14 @@ row_partial_contig(const typename R::in_t* __restrict__ p, int64_t n, int g, int
     }
     for (; v < v_hi; v += width) {
         VecT a = load_stream(&pv[v]);
-        const int64_t j0 = head + v * V;
+        const int64_t j0 = first_index + head + v * V;
 #pragma unroll
         for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(a.v[e], j0 + e, prm));
     }
     if (part == 0)
-        for (int64_t j = g; j < head; j += width) acc = R::join(acc, R::map(p[j], j, prm));
+        for (int64_t j = g; j < head; j += width) acc = R::join(acc, R::map(p[j], first_index + j, prm));
     if (part == parts - 1)
-        for (int64_t j = tail_start + g; j < n; j += width) acc = R::join(acc, R::map(p[j], j, prm));
+        for (int64_t j = tail_start + g; j < n; j += width) acc = R::join(acc, R::map(p[j], first_index + j, prm));
     return acc;
 }
 
@@ -331,7 +331,12 @@ __device__ __forceinline__ typename R::acc_t block_reduce(typename R::acc_t acc)
 
 // Long rows: `parts` workgroups per row.  parts == 1 writes the result,
 // otherwise each workgroup leaves one partial accumulator in `partial`.
-template <typename R, bool CONTIG>
+// LAYOUT of a row: kRowStrided - any view of the reduced dimensions, element by element;
+// kRowContig - one contiguous run; kRowRuns - contiguous runs of the innermost reduced dimension
+// (statistics per channel of an NCHW tensor: 32 runs of 3136 elements a row), a group of lanes
+// taking a run at a time with the vector loads of the contiguous case.
+constexpr int kRowStrided = 0, kRowContig = 1, kRowRuns = 2;
+template <typename R, int LAYOUT>
 __global__ __launch_bounds__(kBlock) void reduce_rows_block(
     const typename R::in_t* __restrict__ x, DimMap kept, DimMap red, int64_t n, int64_t parts,
     typename R::out_t* __restrict__ y, DimMap ymap, int final_op,
@@ -340,8 +345,22 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block(
     const int64_t part = blockIdx.x - row * parts;
     const typename R::in_t* p = x + kept.at(row);
     typename R::acc_t acc;
-    if constexpr (CONTIG) acc = row_partial_contig<R>(p, n, threadIdx.x, kBlock, part, parts, prm);
-    else acc = row_partial_strided<R>(p, red, n, threadIdx.x, kBlock, part, parts, prm);
+    if constexpr (LAYOUT == kRowContig) {
+        acc = row_partial_contig<R>(p, n, threadIdx.x, kBlock, part, parts, prm);
+    } else if constexpr (LAYOUT == kRowRuns) {
+        acc = R::identity();
+        const int last = red.rank - 1;
+        const int64_t run = red.dims[last], runs = n / run;
+        DimMap outer = red;
+        outer.rank = last;
+        // 64 lanes a run from 256 elements, 16 from 64, 4 below
+        const int lanes = run >= 256 ? kWave : run >= 64 ? 16 : 4;
+        const int64_t groups = kBlock / lanes;
+        for (int64_t r = part * groups + threadIdx.x / lanes; r < runs; r += parts * groups)
+            acc = R::join(acc, row_partial_contig<R>(p + outer.at(r), run, threadIdx.x % lanes, lanes, 0, 1, prm, r * run));
+    } else {
+        acc = row_partial_strided<R>(p, red, n, threadIdx.x, kBlock, part, parts, prm);
+    }
     acc = block_reduce<R>(acc);
     if (threadIdx.x == 0) {
         if (parts == 1) y[ymap.at(row)] = R::finish(acc, n, final_op);
@@ -623,11 +642,16 @@ int launch_reduce(hipStream_t stream, const ReducePlan& pl, const typename R::in
     if (m * parts > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
     if (parts > 1 && scratch_bytes < static_cast<size_t>(m * parts) * sizeof(acc_t))
         return DLFX_ERR_SCRATCH_TOO_SMALL;
+    // rows made of contiguous runs (the innermost reduced dimension has stride 1 and at least 16 elements)
+    const bool runs = !contig && pl.red.rank >= 2 && pl.red.strides[pl.red.rank - 1] == 1 && pl.red.dims[pl.red.rank - 1] >= 16;
     if (contig)
-        reduce_rows_block<R, true><<<dim3(static_cast<unsigned>(m * parts)), dim3(kBlock), 0, stream>>>(
+        reduce_rows_block<R, kRowContig><<<dim3(static_cast<unsigned>(m * parts)), dim3(kBlock), 0, stream>>>(
+            x, pl.kept, pl.red, n, parts, y, pl.ymap, final_op, partial, prm);
+    else if (runs)
+        reduce_rows_block<R, kRowRuns><<<dim3(static_cast<unsigned>(m * parts)), dim3(kBlock), 0, stream>>>(
             x, pl.kept, pl.red, n, parts, y, pl.ymap, final_op, partial, prm);
     else
-        reduce_rows_block<R, false><<<dim3(static_cast<unsigned>(m * parts)), dim3(kBlock), 0, stream>>>(
+        reduce_rows_block<R, kRowStrided><<<dim3(static_cast<unsigned>(m * parts)), dim3(kBlock), 0, stream>>>(
             x, pl.kept, pl.red, n, parts, y, pl.ymap, final_op, partial, prm);
     DLFX_CHECK_LAUNCH();
     if (parts > 1) {
