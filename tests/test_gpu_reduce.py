@@ -208,3 +208,20 @@ def test_int64_mean_of_many_short_rows_truncates_exactly(hip_backend, oracle_bac
         wrapped = [((s + 2**63) % 2**64) - 2**63 for s in sums]
         exact = [abs(s) // n * (1 if s >= 0 else -1) for s in wrapped]
         assert got[5:50].tolist() == exact
+
+
+@pytest.mark.parametrize("shape,axes", [((6, 40, 70, 65), [0, 2, 3]), ((5, 64, 9, 300, 20), [0, 2, 4]), ((3, 7, 4000, 17), [0, 2, 3]),
+                                        ((2, 3, 40, 50, 20), [0, 2, 4]), ((20, 96, 56, 56), [0, 2, 3])])
+def test_long_rows_made_of_contiguous_runs(hip_backend, oracle_backend, shape, axes):
+    # rows longer than 8192 elements whose reduced dimensions end in a contiguous one (statistics
+    # per channel of an NCHW tensor): read run by run; runs of 4550, 20, 68000, 20 and 3136 elements
+    x = randint(190, int(np.prod(shape)), -100, 100).astype(np.int32).reshape(shape)
+    Xh = Tensor.from_numpy(hip_backend, x)
+    for name, fn in (("reduce_sum", np.sum), ("reduce_max", np.max), ("reduce_min", np.min)):
+        got = F.reduce(name, Xh, axes).numpy()
+        assert np.array_equal(got, fn(x.astype(np.int64), axis=tuple(axes)).astype(np.int32)), name
+    y = (normal(191, int(np.prod(shape))) * 2).astype(np.float32).reshape(shape)
+    Yh, Yo = both(hip_backend, oracle_backend, y)
+    for name in ("reduce_sum", "reduce_mean", "reduce_max", "reduce_log_sum_exp", "reduce_sum_square", "reduce_nrm2"):
+        check_float_reduce(name, Yh, Yo, axes)
+    assert np.array_equal(F.count(Xh, np.int32(3), tuple(axes)).numpy(), (x == 3).sum(axis=tuple(axes)))
