@@ -225,3 +225,24 @@ def test_long_rows_made_of_contiguous_runs(hip_backend, oracle_backend, shape, a
     for name in ("reduce_sum", "reduce_mean", "reduce_max", "reduce_log_sum_exp", "reduce_sum_square", "reduce_nrm2"):
         check_float_reduce(name, Yh, Yo, axes)
     assert np.array_equal(F.count(Xh, np.int32(3), tuple(axes)).numpy(), (x == 3).sum(axis=tuple(axes)))
+
+
+@pytest.mark.parametrize("shape,axis", [((8, 21, 64, 64), 1), ((64, 3, 50, 50), 1), ((5000, 2, 3), 1), ((3, 32, 5000), 1), ((2, 33, 5000), 1),
+                                        ((17, 8000), 0), ((4, 5, 6, 700), 2)])
+def test_short_axis_beside_many_columns_one_lane_per_column(hip_backend, oracle_backend, shape, axis):
+    # a reduced axis of up to 32 elements that is not the innermost, beside thousands of columns: a lane
+    # reduces a column on its own (33 elements: the kernel of four wavefronts per 64 columns)
+    x = randint(192, int(np.prod(shape)), -9, 9).astype(np.int32).reshape(shape)       # ties: the first extremum counts
+    Xh = Tensor.from_numpy(hip_backend, x)
+    assert np.array_equal(F.reduce("reduce_sum", Xh, [axis]).numpy(), x.sum(axis=axis, dtype=np.int32))
+    assert np.array_equal(F.reduce("reduce_max", Xh, [axis], True).numpy(), x.max(axis=axis, keepdims=True))
+    assert np.array_equal(F.reduce("reduce_prod", Xh, [axis]).numpy(), np.prod(x, axis=axis, dtype=np.int32))
+    assert np.array_equal(F.argmax(Xh, axis).numpy().reshape(-1), np.argmax(x, axis=axis).reshape(-1))
+    assert np.array_equal(F.argmin(Xh, axis).numpy().reshape(-1), np.argmin(x, axis=axis).reshape(-1))
+    assert np.array_equal(F.count(Xh, np.int32(0), (axis,)).numpy().reshape(-1), (x == 0).sum(axis=axis).reshape(-1))
+    y = (normal(193, int(np.prod(shape))) * 2).astype(np.float32).reshape(shape)
+    Yh, Yo = both(hip_backend, oracle_backend, y)
+    for name in ("reduce_sum", "reduce_mean", "reduce_min", "reduce_log_sum_exp", "reduce_nrm2"):
+        check_float_reduce(name, Yh, Yo, [axis])
+    sl = Xh.slice([0], [shape[-1] - 1], [len(shape) - 1], [2])            # every other innermost element: the general kernels
+    assert np.array_equal(F.reduce("reduce_sum", sl, [axis]).numpy(), x[..., 0:shape[-1] - 1:2].sum(axis=axis, dtype=np.int32))

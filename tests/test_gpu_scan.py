@@ -330,3 +330,25 @@ def test_long_axis_beside_few_columns_is_cut_into_segments(hip_backend, shape, a
     assert np.all(np.abs(got - want) <= 4 * np.log2(n) * np.finfo(np.float32).eps * np.maximum(np.abs(want), mag))
     F.cumsum(Xh, axis, out=Xh)                                          # in place
     assert np.array_equal(Xh.numpy(), np.cumsum(x, axis=axis, dtype=np.int32))
+
+
+@pytest.mark.parametrize("shape,axis", [((8, 21, 64, 64), 1), ((64, 3, 50, 50), 1), ((5000, 2, 3), 1), ((3, 32, 5000), 1), ((2, 33, 5000), 1),
+                                        ((17, 8000), 0), ((4, 5, 6, 700), 2)])
+def test_short_axis_beside_many_columns_one_lane_per_column(hip_backend, shape, axis):
+    # an axis of up to 32 positions that is not the innermost, beside thousands of columns: every lane
+    # scans a column in registers (33 positions: the kernel of four wavefronts a round)
+    x = randint(490, int(np.prod(shape)), -50, 50).astype(np.int32).reshape(shape)
+    Xh = Tensor.from_numpy(hip_backend, x)
+    inc = np.cumsum(x, axis=axis, dtype=np.int32)
+    assert np.array_equal(F.cumsum(Xh, axis).numpy(), inc)
+    assert np.array_equal(F.cumsum(Xh, axis, True).numpy(), inc - x)
+    assert np.array_equal(F.cumsum(Xh, axis, True, True).numpy(), np.flip(np.cumsum(np.flip(x, axis), axis=axis, dtype=np.int32), axis) - x)
+    assert np.array_equal(F.cummax(Xh, axis).numpy(), np.maximum.accumulate(x, axis=axis))
+    assert np.array_equal(F.cumprod(Xh, axis).numpy(), np.cumprod(x, axis=axis, dtype=np.int32))
+    y = (normal(491, int(np.prod(shape))) * 3).astype(np.float64).reshape(shape)
+    Yh = Tensor.from_numpy(hip_backend, y)
+    assert np.allclose(F.cumsum(Yh, axis).numpy(), np.cumsum(y, axis=axis), rtol=1e-12, atol=1e-12)
+    sl = Xh.slice([0], [shape[-1] - 1], [len(shape) - 1], [2])            # every other innermost element: columns with a step
+    assert np.array_equal(F.cumsum(sl, axis).numpy(), np.cumsum(x[..., 0:shape[-1] - 1:2], axis=axis, dtype=np.int32))
+    F.cumsum(Xh, axis, out=Xh)
+    assert np.array_equal(Xh.numpy(), inc)
