@@ -303,6 +303,38 @@ def make_ops(be, which):
             xs = gen(shape, dtype, fn, 2)
             ops += [op for op in sort_ops(be, tensor, xs, "C4r", text) if "_asc_" in op.name]
 
+    # ---------------- beside the baseline's configurations: shapes at which a sweep found a step in the
+    # time per element (each named with what takes it now); not part of all
+    if on("beside"):
+        def timed_only(call):
+            def v(call=call):
+                call()
+            return v
+        # scans and reductions along an axis that is not the innermost
+        for shape, axis, what in (((262144, 64), 0, "few columns: the axis cut into segments"), ((4194304, 16), 0, "few columns: the axis cut into segments"),
+                                  ((16384, 1000), 0, "the axis cut into segments"), ((8, 21, 512, 512), 1, "a short axis: a lane per column"),
+                                  ((64, 3, 224, 224), 1, "a short axis: a lane per column")):
+            xs = gen(shape, torch.float32, lambda c: synth.normal(50 + 100 * c), 2)
+            text = "_f32_[%s]" % ",".join(str(e) for e in shape)
+            count = int(np.prod(shape))
+            calls, _ = scan_calls(xs, axis)
+            ops.append(Op("B1", "cumsum{%d}%s" % (axis, text), count, 8 * count, calls, timed_only(calls[0])))
+            calls, _ = argmax_calls(xs, axis)
+            ops.append(Op("B1", "argmax{%d}%s" % (axis, text), count, 4 * count, calls, timed_only(calls[0])))
+        # statistics per channel: rows made of contiguous runs
+        xs = gen((32, 512, 56, 56), torch.float32, lambda c: synth.normal(51 + 100 * c), 2)
+        calls, _ = reduce_calls("reduce_sum", xs, [0, 2, 3])
+        ops.append(Op("B2", "reduce_sum{0,2,3}_f32_[32,512,56,56]", 32 * 512 * 3136, 4 * 32 * 512 * 3136, calls, timed_only(calls[0])))
+        # long rows near the end of the bucket route (bins packed bucket by bucket), doubles with the gap closed
+        for shape, dtype, text in (((16, 2300000), torch.float32, "f32_normal_[16,2300000]"), ((16, 2400000), torch.float32, "f32_normal_[16,2400000]"),
+                                   ((3355, 10000), torch.float64, "f64_normal_[3355,10000]")):
+            xs = gen(shape, dtype, lambda c: synth.normal(52 + 100 * c), 2)
+            ops += [op for op in sort_ops(be, tensor, xs, "B3", text) if "_asc_" in op.name]
+        # top_k of very long rows
+        for rows_l, n_l in ((1, 1 << 24), (1, 1 << 23)):
+            xl_ = gen((rows_l, n_l), torch.float32, lambda c: synth.normal(53 + 100 * c), 2)
+            ops += topk_ops(be, tensor, xl_, (256, 257), "B4", "[%d,2^%d]" % (rows_l, n_l.bit_length() - 1))
+
     # ---------------- C5: strided NCHW
     if on("all", "c5"):
         x5 = gen((32, 512, 56, 56), torch.float32, lambda c: synth.normal(8 + 100 * c), 6)
@@ -653,7 +685,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3 | short (many short rows and an outer axis; not part of all) | spread (sorts of N(0,1) rows; not part of all) | ceil (copy and read-only streams at the C2 and C5 sizes; part of all) | ceilbig (the same streams at 1 GiB and 4 GiB; not part of all) | long (softmax and top_k over a few very long rows; not part of all) | repeats (sorts of rows of one value, of ten values and of clustered keys; not part of all)")
+    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3 | short (many short rows and an outer axis; not part of all) | spread (sorts of N(0,1) rows; not part of all) | ceil (copy and read-only streams at the C2 and C5 sizes; part of all) | ceilbig (the same streams at 1 GiB and 4 GiB; not part of all) | long (softmax and top_k over a few very long rows; not part of all) | repeats (sorts of rows of one value, of ten values and of clustered keys; not part of all) | beside (shapes beside the baseline's at which sweeps found steps: outer-axis scans and reductions, statistics per channel, rows near the end of the bucket route, top_k of very long rows; not part of all)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
