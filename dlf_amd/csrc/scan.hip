@@ -248,6 +248,10 @@ __device__ __forceinline__ void scan_tile(
     const bool x_vec = sx == 1 && (reinterpret_cast<uintptr_t>(xr - shift + seg) % (sizeof(X) * V) == 0);
     const VecX* pv = reinterpret_cast<const VecX*>(xr - shift + seg);
     const bool full = tile_base >= shift && n_pos - tile_base >= TILE;      // every position of the tile is an element of the row
+    // A row walked backwards (stride -1: the reverse scans): elements [i, i + V) of the row are the
+    // vector that ends at xr - i in memory, last element first.
+    const bool x_rev = !PAD && sx == -1 && (reinterpret_cast<uintptr_t>(xr - seg - (V - 1)) % (sizeof(X) * V) == 0);
+    const VecX* pr = reinterpret_cast<const VecX*>(xr - seg - (V - 1));
     if (full && x_vec) {
         // the common case apart: all loads issued back to back, nothing to test per vector
 #pragma unroll
@@ -255,6 +259,13 @@ __device__ __forceinline__ void scan_tile(
             VecX a = load_stream(&pv[k * kWave + lane]);
 #pragma unroll
             for (int e = 0; e < V; ++e) vals[k * V + e] = scan_input<T, X, NZ>(a.v[e]);
+        }
+    } else if (full && x_rev) {
+#pragma unroll
+        for (int k = 0; k < KV; ++k) {
+            VecX a = load_stream(pr - (k * kWave + lane));
+#pragma unroll
+            for (int e = 0; e < V; ++e) vals[k * V + e] = scan_input<T, X, NZ>(a.v[V - 1 - e]);
         }
     } else
 #pragma unroll
@@ -264,6 +275,10 @@ __device__ __forceinline__ void scan_tile(
             VecX a = load_stream(&pv[k * kWave + lane]);
 #pragma unroll
             for (int e = 0; e < V; ++e) vals[k * V + e] = scan_input<T, X, NZ>(a.v[e]);
+        } else if (x_rev && i0 + V <= n_pos) {
+            VecX a = load_stream(pr - (k * kWave + lane));
+#pragma unroll
+            for (int e = 0; e < V; ++e) vals[k * V + e] = scan_input<T, X, NZ>(a.v[V - 1 - e]);
         } else {
 #pragma unroll
             for (int e = 0; e < V; ++e)
@@ -407,6 +422,8 @@ __device__ __forceinline__ void scan_tile(
     using VecY = Vec<Y, V>;
     const bool y_vec = sy == 1 && (reinterpret_cast<uintptr_t>(yr - shift + seg) % (sizeof(Y) * V) == 0);
     VecY* qv = reinterpret_cast<VecY*>(yr - shift + seg);
+    const bool y_rev = !PAD && sy == -1 && (reinterpret_cast<uintptr_t>(yr - seg - (V - 1)) % (sizeof(Y) * V) == 0);
+    VecY* qr = reinterpret_cast<VecY*>(yr - seg - (V - 1));
     if (full && y_vec) {
 #pragma unroll
         for (int k = 0; k < KV; ++k) {
@@ -414,6 +431,14 @@ __device__ __forceinline__ void scan_tile(
 #pragma unroll
             for (int e = 0; e < V; ++e) a.v[e] = static_cast<Y>(vals[k * V + e]);
             store_stream(&qv[k * kWave + lane], a);
+        }
+    } else if (full && y_rev) {
+#pragma unroll
+        for (int k = 0; k < KV; ++k) {
+            VecY a;
+#pragma unroll
+            for (int e = 0; e < V; ++e) a.v[V - 1 - e] = static_cast<Y>(vals[k * V + e]);
+            store_stream(qr - (k * kWave + lane), a);
         }
     } else
 #pragma unroll
@@ -424,6 +449,11 @@ __device__ __forceinline__ void scan_tile(
 #pragma unroll
             for (int e = 0; e < V; ++e) a.v[e] = static_cast<Y>(vals[k * V + e]);
             store_stream(&qv[k * kWave + lane], a);
+        } else if (y_rev && i0 + V <= n_pos) {
+            VecY a;
+#pragma unroll
+            for (int e = 0; e < V; ++e) a.v[V - 1 - e] = static_cast<Y>(vals[k * V + e]);
+            store_stream(qr - (k * kWave + lane), a);
         } else {
 #pragma unroll
             for (int e = 0; e < V; ++e)
@@ -472,6 +502,9 @@ __global__ __launch_bounds__(kBlock) void scan_rows_group(
     // partial vectors element by element
     const bool x_vec = sx == 1 && reinterpret_cast<uintptr_t>(xr - shift) % (sizeof(X) * V) == 0;
     const bool y_vec = sy == 1 && reinterpret_cast<uintptr_t>(yr - shift) % (sizeof(Y) * V) == 0;
+    // a row walked backwards that ends on a vector boundary: whole vectors, last element first
+    const bool x_rev = !pad && sx == -1 && reinterpret_cast<uintptr_t>(xr - (V - 1)) % (sizeof(X) * V) == 0;
+    const bool y_rev = !pad && sy == -1 && reinterpret_cast<uintptr_t>(yr - (V - 1)) % (sizeof(Y) * V) == 0;
     T vals[ITEMS];
 #pragma unroll
     for (int v = 0; v < KV; ++v) {
@@ -480,6 +513,10 @@ __global__ __launch_bounds__(kBlock) void scan_rows_group(
             const VecX a = load_stream(reinterpret_cast<const VecX*>(xr - shift + e0));
 #pragma unroll
             for (int j = 0; j < V; ++j) vals[v * V + j] = scan_input<T, X, NZ>(a.v[j]);
+        } else if (x_rev && e0 + V <= count) {
+            const VecX a = load_stream(reinterpret_cast<const VecX*>(xr - e0 - (V - 1)));
+#pragma unroll
+            for (int j = 0; j < V; ++j) vals[v * V + j] = scan_input<T, X, NZ>(a.v[V - 1 - j]);
         } else {
 #pragma unroll
             for (int j = 0; j < V; ++j)
@@ -532,6 +569,11 @@ __global__ __launch_bounds__(kBlock) void scan_rows_group(
 #pragma unroll
             for (int j = 0; j < V; ++j) a.v[j] = static_cast<Y>(vals[v * V + j]);
             store_stream(reinterpret_cast<VecY*>(yr - shift + e0), a);
+        } else if (y_rev && e0 + V <= count) {
+            VecY a;
+#pragma unroll
+            for (int j = 0; j < V; ++j) a.v[V - 1 - j] = static_cast<Y>(vals[v * V + j]);
+            store_stream(reinterpret_cast<VecY*>(yr - e0 - (V - 1)), a);
         } else {
 #pragma unroll
             for (int j = 0; j < V; ++j)

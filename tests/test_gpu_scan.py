@@ -307,6 +307,45 @@ def test_rows_off_a_vector_boundary(hip_backend, oracle_backend, n):
             hip_backend.set_tuning("scan_poll_limit", 2048)
 
 
+@pytest.mark.parametrize("n", [8, 64, 200, 512, 776, 1024, 4096, 16384, 40000, 150008, 1 << 20])
+def test_rows_walked_backwards_move_whole_vectors(hip_backend, oracle_backend, n):
+    """A reversed scan walks a unit-stride row with stride -1; rows that end on a 16-byte boundary
+    load and store whole vectors, last element first.  Input and output reversed together (the
+    reverse scans), only one of them (a flipped view scanned into a forward result and the other
+    way round), in place, 2-, 4- and 8-byte elements, every kernel size class; rows that end off
+    the boundary (views cut short by one to three elements) take the element-wise path in the
+    same launch."""
+    m = 5 if n < 100000 else 2
+    for dtype in (np.int32, np.int64):
+        x = randint(260 + n, m * n, -50, 50).astype(dtype).reshape(m, n)
+        Xh, Xo = both(hip_backend, oracle_backend, x)
+        for exclusive in (False, True):
+            assert np.array_equal(F.cumsum(Xh, 1, exclusive, True).numpy(), F.cumsum(Xo, 1, exclusive, True).numpy()), (dtype, exclusive)
+        want = np.cumsum(x[:, ::-1], axis=1, dtype=dtype)
+        assert np.array_equal(F.cumsum(Xh.flip([1]), 1).numpy(), want), dtype                 # reversed in, forward out
+        Yh = Tensor.from_numpy(hip_backend, np.zeros((m, n), dtype))
+        F.cumsum(Xh, 1, out=Yh.flip([1]))                                                     # forward in, reversed out
+        assert np.array_equal(Yh.numpy(), np.cumsum(x, axis=1, dtype=dtype)[:, ::-1]), dtype
+        assert np.array_equal(F.cummax(Xh, 1, True).numpy(), np.maximum.accumulate(x[:, ::-1], axis=1)[:, ::-1]), dtype
+        assert np.array_equal(F.cumprod(Xh, 1, False, True).numpy(), F.cumprod(Xo, 1, False, True).numpy()), dtype
+        for cut in (1, 2, 3):
+            if n > cut:
+                Vh, Vo = Xh.slice([0], [n - cut], [1]), Xo.slice([0], [n - cut], [1])
+                assert np.array_equal(F.cumsum(Vh, 1, False, True).numpy(), F.cumsum(Vo, 1, False, True).numpy()), (dtype, cut)
+        Zh = Tensor.from_numpy(hip_backend, x)
+        F.cumsum(Zh, 1, False, True, out=Zh)                                                  # in place
+        assert np.array_equal(Zh.numpy(), np.cumsum(x[:, ::-1], axis=1, dtype=dtype)[:, ::-1]), dtype
+    xh = (normal(261 + n, m * n) * 0.25).astype(np.float16).reshape(m, n)
+    got = F.cumsum(Tensor.from_numpy(hip_backend, xh), 1, False, True).numpy().astype(np.float64)
+    x64 = xh[:, ::-1].astype(np.float64)
+    want, mag = np.cumsum(x64, axis=1)[:, ::-1], np.cumsum(np.abs(x64), axis=1)[:, ::-1]
+    assert (np.abs(got - want) <= 4 * max(1.0, np.log2(n)) * np.finfo(np.float32).eps * mag + 2.0 ** -10 * np.abs(want) + 1e-30).all()
+    xb = (randint(262 + n, m * n, 0, 3) == 0)
+    xb = xb.reshape(m, n)
+    assert np.array_equal(F.cumsum(Tensor.from_numpy(hip_backend, xb.astype(np.int64)), 1, True, True).numpy(),
+                          (np.cumsum(xb[:, ::-1], axis=1, dtype=np.int64) - xb[:, ::-1])[:, ::-1])
+
+
 @pytest.mark.parametrize("shape,axis", [((40000, 64), 0), ((100000, 17), 0), ((3, 9000, 100), 1), ((2050, 1000), 0), ((262144, 8), 0), ((5000, 7), 0)])
 def test_long_axis_beside_few_columns_is_cut_into_segments(hip_backend, shape, axis):
     # an axis that is not the innermost, long, with too few columns beside it to fill the device:
