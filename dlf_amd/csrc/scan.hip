@@ -632,120 +632,200 @@ constexpr int kColsChunk = 16;      // rows of a column a wave scans per round (
 // total per column in `partials` ([segment][column]); scan_cols starts a segment from what the
 // segments before it add up to.  The input is read twice - three crossings instead of two -
 // by as many workgroups as fill the device.
+// Where a lane's column is at a position of the axis.  A position is the same for a whole
+// wavefront, so with NARROW (every column starts less than 4 GB after the base: the host checks
+// the view) the address is a scalar base - the position's offset, worked out once a wavefront -
+// plus the lane's 32-bit offset, the form that a global access takes as it is: no pair of vector
+// registers per access in flight for its address, which is what kept these kernels at 118
+// registers and four wavefronts a SIMD.
+template <typename P, bool NARROW>
+struct ColumnAt {
+    P* base;
+    uint32_t lane_bytes;
+    int64_t step_bytes;
+    __device__ __forceinline__ ColumnAt(P* origin, int64_t column_offset, int64_t axis_stride) {
+        if constexpr (NARROW) {
+            base = origin;
+            lane_bytes = static_cast<uint32_t>(column_offset * static_cast<int64_t>(sizeof(P)));
+        } else {
+            base = origin + column_offset;
+            lane_bytes = 0;
+        }
+        step_bytes = axis_stride * static_cast<int64_t>(sizeof(P));
+    }
+    __device__ __forceinline__ P* at(int64_t position) const {
+        using Byte = std::conditional_t<std::is_const<P>::value, const char, char>;
+        Byte* row = reinterpret_cast<Byte*>(base) + position * step_bytes;
+        if constexpr (NARROW) return reinterpret_cast<P*>(row + static_cast<uint64_t>(lane_bytes));
+        else return reinterpret_cast<P*>(row);
+    }
+};
+
 struct ColSegments {
     int64_t seg_len, segs, col_blocks;     // one segment: seg_len = n, segs = 1
 };
 
-template <typename T, int K, typename X, bool NZ>
+template <typename T, int K, typename X, bool NZ, int C, bool NARROW>
 __global__ __launch_bounds__(kBlock) void scan_cols_partials(
     const X* __restrict__ x, DimMap xmap, int64_t sx, int64_t m, int64_t n, ColSegments cut, T* __restrict__ partials) {
     using Op = ScanOp<T, K>;
+    using VecX = Vec<X, C>;
     constexpr int R = kColsChunk;
-    __shared__ T totals[kWaves][kWave];
+    __shared__ T totals[kWaves][C][kWave];
     const int lx = threadIdx.x & (kWave - 1);
-    const int ty = threadIdx.x / kWave;
+    // (NARROW: the wavefront's number as a scalar, so that positions and their offsets are scalars too)
+    const int ty = NARROW ? __builtin_amdgcn_readfirstlane(threadIdx.x / kWave) : threadIdx.x / kWave;
     const int64_t col_block = blockIdx.x % cut.col_blocks, seg = blockIdx.x / cut.col_blocks;
-    const int64_t col = col_block * kWave + lx;
+    const int64_t col = (col_block * kWave + lx) * C;
     const bool live = col < m;
-    const X* xc = x + (live ? xmap.at(col) : 0);
+    const ColumnAt<const X, NARROW> xc(x, live ? xmap.at(col) : 0, sx);
     const int64_t lo = seg * cut.seg_len;
     const int64_t hi = lo + cut.seg_len < n ? lo + cut.seg_len : n;
-    T sum = Op::identity();
+    T sum[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) sum[c] = Op::identity();
     // wave ty takes positions lo + 16 ty, + 64, ...: sixteen loads in flight a lane
     for (int64_t p0 = lo + static_cast<int64_t>(ty) * R; p0 < hi; p0 += static_cast<int64_t>(kWaves) * R) {
-        T v[R];
+        T v[R * C];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int64_t p = p0 + r;
-            v[r] = (live && p < hi) ? scan_input<T, X, NZ>(load_stream(&xc[p * sx])) : Op::identity();
+            if (live && p < hi) {
+                const VecX a = load_stream(reinterpret_cast<const VecX*>(xc.at(p)));
+#pragma unroll
+                for (int c = 0; c < C; ++c) v[r * C + c] = scan_input<T, X, NZ>(a.v[c]);
+            } else {
+#pragma unroll
+                for (int c = 0; c < C; ++c) v[r * C + c] = Op::identity();
+            }
         }
 #pragma unroll
-        for (int r = 0; r < R; ++r) sum = Op::apply(sum, v[r]);
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int c = 0; c < C; ++c) sum[c] = Op::apply(sum[c], v[r * C + c]);
     }
-    totals[ty][lx] = sum;
+#pragma unroll
+    for (int c = 0; c < C; ++c) totals[ty][c][lx] = sum[c];
     __syncthreads();
     if (ty == 0 && live) {
-        T all = totals[0][lx];
 #pragma unroll
-        for (int i = 1; i < kWaves; ++i) all = Op::apply(all, totals[i][lx]);
-        partials[seg * m + col] = all;
+        for (int c = 0; c < C; ++c) {
+            T all = totals[0][c][lx];
+#pragma unroll
+            for (int i = 1; i < kWaves; ++i) all = Op::apply(all, totals[i][c][lx]);
+            partials[seg * m + col + c] = all;
+        }
     }
 }
 
-template <typename T, int K, typename X, bool NZ, typename Y>
-__global__ __launch_bounds__(kBlock) void scan_cols(
+// C columns that lie side by side in memory per lane (one access of C elements: a wavefront's
+// access to a position of the axis is then 64 C elements wide - with one two-byte element per
+// lane it is 128 bytes, and such scans ran at the element rate of fp32 or below).
+#ifndef DLFX_SCAN_COLS_WAVES
+#define DLFX_SCAN_COLS_WAVES 5
+#endif
+template <typename T, int K, typename X, bool NZ, typename Y, int C, bool NARROW>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(1, DLFX_SCAN_COLS_WAVES))) void scan_cols(
     const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy,
     int64_t m, int64_t n, int chunk, int exclusive, ColSegments cut, const T* __restrict__ partials) {
     using Op = ScanOp<T, K>;
+    using VecX = Vec<X, C>;
+    using VecY = Vec<Y, C>;
     constexpr int R = kColsChunk;
-    __shared__ T totals[2][kWaves][kWave];
+    __shared__ T totals[2][kWaves][C][kWave];
 
     const int lx = threadIdx.x & (kWave - 1);
-    const int ty = threadIdx.x / kWave;
+    // (NARROW: the wavefront's number as a scalar, so that positions and their offsets are scalars too)
+    const int ty = NARROW ? __builtin_amdgcn_readfirstlane(threadIdx.x / kWave) : threadIdx.x / kWave;
     const int64_t col_block = blockIdx.x % cut.col_blocks, seg = blockIdx.x / cut.col_blocks;
-    const int64_t col = col_block * kWave + lx;
+    const int64_t col = (col_block * kWave + lx) * C;
     const bool live = col < m;
-    const X* xc = x + (live ? xmap.at(col) : 0);
-    Y* yc = y + (live ? ymap.at(col) : 0);
+    const ColumnAt<const X, NARROW> xc(x, live ? xmap.at(col) : 0, sx);
+    const ColumnAt<Y, NARROW> yc(y, live ? ymap.at(col) : 0, sy);
     const int64_t lo = seg * cut.seg_len;
     const int64_t hi = lo + cut.seg_len < n ? lo + cut.seg_len : n;        // this workgroup scans positions [lo, hi)
 
-    T carry = Op::identity();
+    T carry[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) carry[c] = Op::identity();
     if (cut.segs > 1 && live) {
         // what the segments before this one add up to (their totals, in order: four loads in flight)
         for (int64_t s0 = 0; s0 < seg; s0 += 4) {
-            T part[4];
+            T part[4 * C];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) part[j] = s0 + j < seg ? partials[(s0 + j) * m + col] : Op::identity();
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) carry = Op::apply(carry, part[j]);
+                for (int c = 0; c < C; ++c) part[j * C + c] = s0 + j < seg ? partials[(s0 + j) * m + col + c] : Op::identity();
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int c = 0; c < C; ++c) carry[c] = Op::apply(carry[c], part[j * C + c]);
         }
     }
     int buf = 0;
     const int64_t step = static_cast<int64_t>(kWaves) * chunk;
     // the wave's chunk of the next round is on its way while this round is scanned and stored
-    auto load_chunk = [&](int64_t s, T* v) __attribute__((always_inline)) {
+    // (kept as loaded: two-byte elements wait two to a register)
+    auto load_chunk = [&](int64_t s, VecX* v) __attribute__((always_inline)) {
         const int64_t p0 = s + static_cast<int64_t>(ty) * chunk;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int64_t p = p0 + r;
-            v[r] = (live && r < chunk && p < hi) ? scan_input<T, X, NZ>(load_stream(&xc[p * sx])) : Op::identity();
+            if (live && r < chunk && p < hi) {
+                v[r] = load_stream(reinterpret_cast<const VecX*>(xc.at(p)));
+            } else {
+#pragma unroll
+                for (int c = 0; c < C; ++c) v[r].v[c] = static_cast<X>(Op::identity());      // (folds as the identity, also where scan_input maps elements to 0 / 1)
+            }
         }
     };
-    T ahead[R];
+    VecX ahead[R];
     load_chunk(lo, ahead);
     for (int64_t s = lo; s < hi; s += step, buf ^= 1) {
         const int64_t p0 = s + static_cast<int64_t>(ty) * chunk;
-        T v[R];
+        T v[R * C];
 #pragma unroll
-        for (int r = 0; r < R; ++r) v[r] = ahead[r];
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int c = 0; c < C; ++c) v[r * C + c] = scan_input<T, X, NZ>(ahead[r].v[c]);
         if (s + step < hi) load_chunk(s + step, ahead);
 #pragma unroll
-        for (int r = 1; r < R; ++r) v[r] = Op::apply(v[r - 1], v[r]);
-        totals[buf][ty][lx] = v[R - 1];
-        __syncthreads();
-        T pre = carry;
-        T all = Op::identity();
+        for (int i = C; i < R * C; ++i) v[i] = Op::apply(v[i - C], v[i]);
 #pragma unroll
-        for (int i = 0; i < kWaves; ++i) {
-            const T tv = totals[buf][i][lx];
-            if (i < ty) pre = Op::apply(pre, tv);
-            all = Op::apply(all, tv);
+        for (int c = 0; c < C; ++c) totals[buf][ty][c][lx] = v[(R - 1) * C + c];
+        __syncthreads();
+        T pre[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            pre[c] = carry[c];
+            T all = Op::identity();
+#pragma unroll
+            for (int i = 0; i < kWaves; ++i) {
+                const T tv = totals[buf][i][c][lx];
+                if (i < ty) pre[c] = Op::apply(pre[c], tv);
+                all = Op::apply(all, tv);
+            }
+            carry[c] = Op::apply(carry[c], all);
         }
-        carry = Op::apply(carry, all);
         if (live) {
             if (exclusive) {
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const int64_t p = p0 + r;
-                    const T prev = (r == 0) ? pre : Op::apply(pre, v[r > 0 ? r - 1 : 0]);
-                    if (r < chunk && p < hi) store_stream(&yc[p * sy], static_cast<Y>(prev));
+                    VecY out;
+#pragma unroll
+                    for (int c = 0; c < C; ++c)
+                        out.v[c] = static_cast<Y>((r == 0) ? pre[c] : Op::apply(pre[c], v[(r > 0 ? r - 1 : 0) * C + c]));
+                    if (r < chunk && p < hi) store_stream(reinterpret_cast<VecY*>(yc.at(p)), out);
                 }
             } else {
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const int64_t p = p0 + r;
-                    if (r < chunk && p < hi) store_stream(&yc[p * sy], static_cast<Y>(Op::apply(pre, v[r])));
+                    VecY out;
+#pragma unroll
+                    for (int c = 0; c < C; ++c) out.v[c] = static_cast<Y>(Op::apply(pre[c], v[r * C + c]));
+                    if (r < chunk && p < hi) store_stream(reinterpret_cast<VecY*>(yc.at(p)), out);
                 }
             }
         }
@@ -756,23 +836,41 @@ __global__ __launch_bounds__(kBlock) void scan_cols(
 // all its loads in flight at once, 256 columns a workgroup and no barrier (the kernel above
 // gives such an axis to four wavefronts a position or two each: fp32 [8, 21, 512, 512] along
 // axis 1 141 us, [64, 3, 224, 224] 184 us).
-template <typename T, int K, typename X, bool NZ, typename Y, int N>
+template <typename T, int K, typename X, bool NZ, typename Y, int N, int C, bool NARROW>
 __global__ __launch_bounds__(kBlock) void scan_cols_thread(
     const X* __restrict__ x, Y* __restrict__ y, DimMap xmap, DimMap ymap, int64_t sx, int64_t sy, int64_t m, int n, int exclusive) {
     using Op = ScanOp<T, K>;
-    const int64_t col = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    using VecX = Vec<X, C>;
+    using VecY = Vec<Y, C>;
+    const int64_t col = (static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x) * C;
     if (col >= m) return;
-    const X* xc = x + xmap.at(col);
-    Y* yc = y + ymap.at(col);
-    T v[N];
-#pragma unroll
-    for (int r = 0; r < N; ++r) v[r] = r < n ? scan_input<T, X, NZ>(load_stream(&xc[r * sx])) : Op::identity();
-    T run = Op::identity();
+    const ColumnAt<const X, NARROW> xc(x, xmap.at(col), sx);
+    const ColumnAt<Y, NARROW> yc(y, ymap.at(col), sy);
+    T v[N * C];
 #pragma unroll
     for (int r = 0; r < N; ++r) {
-        const T before = run;
-        run = Op::apply(run, v[r]);
-        if (r < n) store_stream(&yc[r * sy], static_cast<Y>(exclusive ? before : run));
+        if (r < n) {
+            const VecX a = load_stream(reinterpret_cast<const VecX*>(xc.at(r)));
+#pragma unroll
+            for (int c = 0; c < C; ++c) v[r * C + c] = scan_input<T, X, NZ>(a.v[c]);
+        } else {
+#pragma unroll
+            for (int c = 0; c < C; ++c) v[r * C + c] = Op::identity();
+        }
+    }
+    T run[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) run[c] = Op::identity();
+#pragma unroll
+    for (int r = 0; r < N; ++r) {
+        VecY out;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const T before = run[c];
+            run[c] = Op::apply(run[c], v[r * C + c]);
+            out.v[c] = static_cast<Y>(exclusive ? before : run[c]);
+        }
+        if (r < n) store_stream(reinterpret_cast<VecY*>(yc.at(r)), out);
     }
 }
 
@@ -834,14 +932,27 @@ int64_t tile_elems(size_t elem_size, int64_t n) {
 // How scan_cols cuts the axis of m columns of n positions: not at all while the blocks of 64
 // columns alone give the device enough workgroups (or the axis is short); otherwise into segments
 // of whole rounds (64 positions), about 1024 workgroups in all, no segment under 512 positions.
-ColSegments col_segments(int64_t m, int64_t n) {
+#ifndef DLFX_SCAN_COLS_WANT
+#define DLFX_SCAN_COLS_WANT 1024
+#endif
+#ifndef DLFX_SCAN_COLS_FEW
+#define DLFX_SCAN_COLS_FEW 64
+#endif
+#ifndef DLFX_SCAN_COLS_MIN_SEG
+#define DLFX_SCAN_COLS_MIN_SEG 512
+#endif
+ColSegments col_segments(int64_t m, int64_t n, int per_lane = 1) {
     ColSegments c;
-    c.col_blocks = ceil_div(m, static_cast<int64_t>(kWave));
+    c.col_blocks = ceil_div(m, static_cast<int64_t>(kWave) * per_lane);
     c.seg_len = n;
     c.segs = 1;
     if (c.col_blocks >= 512 || n < 2048) return c;
-    int64_t want = ceil_div(static_cast<int64_t>(1024), c.col_blocks);
-    const int64_t most = n / 512;
+    int64_t want = ceil_div(static_cast<int64_t>(DLFX_SCAN_COLS_WANT), c.col_blocks);
+    // (a segment starts from the totals of those before it, read one after the other: up to 32 segments
+    // may be as short as 128 positions, more than that only of 512 and more)
+    int64_t most = n / DLFX_SCAN_COLS_MIN_SEG;
+    const int64_t few = n / 128 < DLFX_SCAN_COLS_FEW ? n / 128 : DLFX_SCAN_COLS_FEW;
+    if (most < few) most = few;
     if (want > most) want = most;
     if (want < 2) return c;
     c.seg_len = align_up(static_cast<size_t>(ceil_div(n, want)), static_cast<size_t>(kWaves * kColsChunk));
@@ -853,9 +964,22 @@ ColSegments col_segments(int64_t m, int64_t n) {
     return c;
 }
 
+constexpr int kColsPerLaneMax = 2;
+int g_cols_per_lane = 0;           // dlfx_set_tuning "scan_cols_per_lane": at most so many (0: as the kernels choose)
+#ifndef DLFX_SCAN_COLS_BYTES
+#define DLFX_SCAN_COLS_BYTES 4
+#endif
+constexpr size_t kColsAccessBytes = DLFX_SCAN_COLS_BYTES;      // widest access of a lane to its columns
+
+// (the most that any number of columns per lane asks for: the query does not see the strides)
 size_t col_partials_bytes(size_t elem_size, int64_t m, int64_t n) {
-    const ColSegments c = col_segments(m, n);
-    return c.segs > 1 ? static_cast<size_t>(c.segs) * static_cast<size_t>(m) * elem_size : 0;
+    size_t most = 0;
+    for (int per_lane = 1; per_lane <= kColsPerLaneMax; per_lane *= 2) {
+        const ColSegments c = col_segments(m, n, per_lane);
+        const size_t bytes = c.segs > 1 ? static_cast<size_t>(c.segs) * static_cast<size_t>(m) * elem_size : 0;
+        if (bytes > most) most = bytes;
+    }
+    return most;
 }
 
 struct ScanLayout {
@@ -978,18 +1102,64 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
     // (columns side by side in memory: from 64 of them; from 8 when the axis has a million positions or more -
     // [4194304, 16] fp32 along the first axis: 309 GB/s as strided rows, 1643 GB/s as columns, three lanes in
     // four idle; [262144, 16]: 674 against 497)
-    const ColSegments cut = col_segments(m, n);
     const bool use_cols = !axis_general && (short_rows || (!axis_unit && (m >= 64 || (m >= 8 && n >= (1 << 20))) && (inner_unit || n < 4096)));
-    if (use_cols && n <= 32 && m >= 4096) {
-        const int64_t blocks = ceil_div(m, static_cast<int64_t>(kBlock));
+    // Columns per lane: as many neighbours in memory as make an access of DLFX_SCAN_COLS_BYTES, where every
+    // such group of columns starts on a boundary of its own size at every position of the axis.
+    int per_lane = 1;
+    if (use_cols && !std::is_class<X>::value && !std::is_class<Y>::value) {
+        for (int c = g_cols_per_lane ? g_cols_per_lane : kColsPerLaneMax; c > 1 && per_lane == 1; c /= 2) {
+            if (sizeof(X) * c > kColsAccessBytes || sizeof(Y) * c > kColsAccessBytes) continue;
+            bool ok = xmap.rank >= 1 && xmap.strides[xmap.rank - 1] == 1 && ymap.strides[ymap.rank - 1] == 1 &&
+                      xmap.dims[xmap.rank - 1] % c == 0 && sx % c == 0 && sy % c == 0 &&
+                      reinterpret_cast<uintptr_t>(x) % (sizeof(X) * c) == 0 && reinterpret_cast<uintptr_t>(y) % (sizeof(Y) * c) == 0;
+            for (int i = 0; ok && i + 1 < xmap.rank; ++i) ok = xmap.strides[i] % c == 0 && ymap.strides[i] % c == 0;
+            if (ok) per_lane = c;
+        }
+    }
+    // Every column within 4 GB after the base, in input and output: scalar base + 32-bit lane offset.
+    bool narrow = use_cols;
+    {
+        int64_t span_x = 0, span_y = 0;
+        for (int i = 0; narrow && i < xmap.rank; ++i) {
+            narrow = xmap.strides[i] >= 0 && ymap.strides[i] >= 0;
+            span_x += (xmap.dims[i] - 1) * xmap.strides[i];
+            span_y += (ymap.dims[i] - 1) * ymap.strides[i];
+        }
+        narrow = narrow && static_cast<uint64_t>(span_x) * sizeof(X) < (1ull << 32) && static_cast<uint64_t>(span_y) * sizeof(Y) < (1ull << 32);
+    }
+    if (!narrow) per_lane = 1;
+    const ColSegments cut = col_segments(m, n, per_lane);
+    // One column a lane: the kernel that walks the axis in rounds is faster with an address of its own
+    // per lane and access (fp32 [32, 512, 56, 56] along axis 1: 77 against 82 us with scalar bases - the
+    // compiler runs out of scalar registers for the bases of 32 accesses and parks them in vector
+    // registers), the kernel that holds a short axis whole with scalar bases (60 against 65 us at
+    // [8, 21, 512, 512]).  Two columns a lane need the registers that the scalar bases leave free.
+    const bool thread_kernel = use_cols && n <= 32 && m >= 4096;
+    auto with_cols = [&](auto&& launch) {
+        constexpr bool kScalars = !std::is_class<X>::value && !std::is_class<Y>::value;
+        if constexpr (kScalars && sizeof(X) * 4 <= kColsAccessBytes && sizeof(Y) * 4 <= kColsAccessBytes) {
+            if (per_lane == 4) { launch(std::integral_constant<int, 4>(), std::true_type()); return; }
+        }
+        if constexpr (kScalars && sizeof(X) * 2 <= kColsAccessBytes && sizeof(Y) * 2 <= kColsAccessBytes) {
+            if (per_lane == 2) { launch(std::integral_constant<int, 2>(), std::true_type()); return; }
+        }
+        if (narrow && thread_kernel) launch(std::integral_constant<int, 1>(), std::true_type());
+        else launch(std::integral_constant<int, 1>(), std::false_type());
+    };
+    if (thread_kernel) {
+        const int64_t blocks = ceil_div(m, static_cast<int64_t>(kBlock) * per_lane);
         if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
         const dim3 grid(static_cast<unsigned>(blocks)), block(kBlock);
-#define DLFX_SCAN_THREAD(N) scan_cols_thread<T, K, X, NZ, Y, N><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, m, static_cast<int>(n), exclusive)
-        if (n <= 4) DLFX_SCAN_THREAD(4);
-        else if (n <= 8) DLFX_SCAN_THREAD(8);
-        else if (n <= 16) DLFX_SCAN_THREAD(16);
-        else DLFX_SCAN_THREAD(32);
+        with_cols([&](auto c, auto nw) {
+            constexpr int C = decltype(c)::value;
+            constexpr bool NW = decltype(nw)::value;
+#define DLFX_SCAN_THREAD(N) scan_cols_thread<T, K, X, NZ, Y, N, C, NW><<<grid, block, 0, stream>>>(x, y, xmap, ymap, sx, sy, m, static_cast<int>(n), exclusive)
+            if (n <= 4) DLFX_SCAN_THREAD(4);
+            else if (n <= 8) DLFX_SCAN_THREAD(8);
+            else if (n <= 16) DLFX_SCAN_THREAD(16);
+            else DLFX_SCAN_THREAD(32);
 #undef DLFX_SCAN_THREAD
+        });
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
     }
@@ -1000,11 +1170,17 @@ int launch_scan(hipStream_t stream, int64_t m, int64_t n, int exclusive, int ran
         T* partials = static_cast<T*>(scratch);
         if (cut.segs > 1) {
             if (!scratch || scratch_bytes < col_partials_bytes(sizeof(T), m, n)) return DLFX_ERR_SCRATCH_TOO_SMALL;
-            scan_cols_partials<T, K, X, NZ><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(x, xmap, sx, m, n, cut, partials);
+            with_cols([&](auto c, auto nw) {
+                if constexpr (decltype(c)::value == 1 && decltype(nw)::value) return;        // (the short-axis kernel's combination)
+                else scan_cols_partials<T, K, X, NZ, decltype(c)::value, decltype(nw)::value><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(x, xmap, sx, m, n, cut, partials);
+            });
             DLFX_CHECK_LAUNCH();
         }
-        scan_cols<T, K, X, NZ, Y><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
-            x, y, xmap, ymap, sx, sy, m, n, chunk, exclusive, cut, partials);
+        with_cols([&](auto c, auto nw) {
+            if constexpr (decltype(c)::value == 1 && decltype(nw)::value) return;
+            else scan_cols<T, K, X, NZ, Y, decltype(c)::value, decltype(nw)::value><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
+                x, y, xmap, ymap, sx, sy, m, n, chunk, exclusive, cut, partials);
+        });
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
     }
@@ -1098,6 +1274,10 @@ using namespace dlfx;
 
 namespace dlfx {
 bool set_scan_tuning(const char* key, int64_t value) {
+    if (!std::strcmp(key, "scan_cols_per_lane") && (value == 0 || value == 1 || value == 2 || value == 4)) {
+        g_cols_per_lane = static_cast<int>(value);
+        return true;
+    }
     if (!std::strcmp(key, "scan_poll_limit") && value >= 0 && value <= (1 << 30)) {
         g_poll_limit = static_cast<int>(value);
         return true;
@@ -1130,6 +1310,20 @@ extern "C" int dlfx_scan(dlfx_stream_t stream, const char* name, int dtype, int6
     else if (!std::strcmp(name, "cummin")) kind = kScanMin;
     else return DLFX_ERR_UNKNOWN_OP;
     hipStream_t s = static_cast<hipStream_t>(stream);
+#ifdef DLFX_SCAN_FEW_TYPES
+    // (a build for experiments, minutes faster to compile: running sums of fp32 and half only)
+    if (dtype == DLFX_F16 && kind == kScanMax)
+        return launch_scan<float, kScanMax, half_t, false, half_t>(s, m, n, exclusive, rank, dims, static_cast<const half_t*>(x) + x_offset, x_strides,
+                                                                  static_cast<half_t*>(y) + y_offset, y_strides, scratch, scratch_bytes);
+    if (kind != kScanAdd) return DLFX_ERR_UNSUPPORTED_DTYPE;
+    if (dtype == DLFX_F16)
+        return launch_scan<float, kScanAdd, half_t, false, half_t>(s, m, n, exclusive, rank, dims, static_cast<const half_t*>(x) + x_offset, x_strides,
+                                                                  static_cast<half_t*>(y) + y_offset, y_strides, scratch, scratch_bytes);
+    if (dtype == DLFX_F32)
+        return launch_scan<float, kScanAdd>(s, m, n, exclusive, rank, dims, static_cast<const float*>(x) + x_offset, x_strides,
+                                            static_cast<float*>(y) + y_offset, y_strides, scratch, scratch_bytes);
+    return DLFX_ERR_UNSUPPORTED_DTYPE;
+#else
     if (dtype == DLFX_F16) {
         // half elements are scanned in fp32: one rounding per output instead of one per step
         const half_t* xp = static_cast<const half_t*>(x) + x_offset;
@@ -1164,6 +1358,7 @@ extern "C" int dlfx_scan(dlfx_stream_t stream, const char* name, int dtype, int6
         default:       return launch_scan<T, kScanMin>(s, m, n, exclusive, rank, dims, xp, x_strides, yp, y_strides, scratch, scratch_bytes);
         }
     });
+#endif
 }
 
 extern "C" size_t dlfx_scan_nonzero_scratch_bytes(int dtype, int64_t m, int64_t n) {
@@ -1206,6 +1401,9 @@ extern "C" int dlfx_scan_nonzero(dlfx_stream_t stream, int dtype, int64_t m, int
     xs2[split] = xaxis.rank == 1 ? xaxis.strides[0] : 0;
     ys2[split] = yaxis.rank == 1 ? yaxis.strides[0] : 1;
     hipStream_t s = static_cast<hipStream_t>(stream);
+#ifdef DLFX_SCAN_FEW_TYPES
+    return DLFX_ERR_UNSUPPORTED_DTYPE;
+#endif
     auto run = [&](auto tag) {
         using X = decltype(tag);
         return launch_scan<int32_t, kScanAdd, X, true>(s, m, n, exclusive, split + 1, d2, static_cast<const X*>(x) + x_offset,

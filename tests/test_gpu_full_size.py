@@ -169,6 +169,12 @@ def test_tensors_of_more_than_2_32_elements(hip_backend):
     am = dev(F.argmax(wrap(hip_backend, xr), 1)).long().reshape(-1)
     first = (xr == xr.amax(dim=1, keepdim=True)).to(torch.int8).argmax(dim=1)
     assert torch.equal(am, first)
+    # columns that start up to 4.7 GB after the base (scan along the middle axis: lanes keep 64-bit offsets)
+    xc = x[:70 * 64 * (1 << 18)].view(70, 64, 1 << 18)
+    yc = dev(F.cumsum(wrap(hip_backend, xc), 1))
+    for rows in (slice(0, 2), slice(-2, None)):
+        assert torch.equal(yc[rows], torch.cumsum(xc[rows], 1, dtype=torch.int32))
+    del yc
     xt = x[:135000 * 32000].view(135000, 32000)
     Y, I = F.top_k(wrap(hip_backend, xt), 5, 1, True)
     for rows in (slice(0, 32), slice(-32, None)):

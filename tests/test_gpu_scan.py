@@ -371,6 +371,63 @@ def test_long_axis_beside_few_columns_is_cut_into_segments(hip_backend, shape, a
     assert np.array_equal(Xh.numpy(), np.cumsum(x, axis=axis, dtype=np.int32))
 
 
+@pytest.mark.parametrize("shape,axis", [((8, 21, 64, 64), 1), ((4, 100, 30, 30), 1), ((4096, 128), 0), ((3, 5000, 66), 1), ((5000, 67), 0),
+                                        ((64, 3, 25, 25), 1), ((2, 40, 6, 10, 12), 1), ((70000, 6), 0)])
+def test_two_byte_columns_go_two_to_a_lane(hip_backend, shape, axis):
+    """Half elements along an axis that is not the innermost: a lane takes two columns that lie
+    side by side (one 4-byte access) where every such pair starts on a 4-byte boundary - an even
+    number of columns in the innermost run, even strides, an aligned base - and one column
+    otherwise (odd extents, views that start at an odd element).  Running maxima and minima are
+    exact, running sums held to the fp32 bound; short axes, long axes cut into segments, views,
+    in place, exclusive and reversed."""
+    x = (normal(500, int(np.prod(shape))) * 2).astype(np.float16).reshape(shape)
+    Xh = Tensor.from_numpy(hip_backend, x)
+    n = shape[axis]
+
+    def check_sum(got, src, ax, exclusive=False, reverse=False):
+        s64 = src.astype(np.float64)
+        if reverse:
+            s64 = np.flip(s64, ax)
+        want, mag = np.cumsum(s64, axis=ax), np.cumsum(np.abs(s64), axis=ax)
+        if exclusive:
+            want, mag = want - s64, mag
+        if reverse:
+            want, mag = np.flip(want, ax), np.flip(mag, ax)
+        err = np.abs(got.astype(np.float64) - want)
+        assert (err <= 4 * max(1.0, np.log2(n)) * np.finfo(np.float32).eps * mag + 2.0 ** -10 * np.abs(want) + 1e-30).all()
+
+    assert np.array_equal(F.cummax(Xh, axis).numpy(), np.maximum.accumulate(x, axis=axis))
+    assert np.array_equal(F.cummin(Xh, axis).numpy(), np.minimum.accumulate(x, axis=axis))
+    assert np.array_equal(F.cummax(Xh, axis, True).numpy(), np.flip(np.maximum.accumulate(np.flip(x, axis), axis=axis), axis))
+    check_sum(F.cumsum(Xh, axis).numpy(), x, axis)
+    check_sum(F.cumsum(Xh, axis, True).numpy(), x, axis, exclusive=True)
+    check_sum(F.cumsum(Xh, axis, False, True).numpy(), x, axis, reverse=True)
+    # views of the innermost dimension: an even start keeps the pairs, an odd start or an odd length does not
+    last = len(shape) - 1
+    w = shape[last]
+    for lo, hi in ((2, w), (1, w - 1), (0, w - 1), (2, w - 2)):
+        if hi - lo < 1:
+            continue
+        Vh = Xh.slice([lo], [hi], [last])
+        v = x[..., lo:hi]
+        assert np.array_equal(F.cummax(Vh, axis).numpy(), np.maximum.accumulate(v, axis=axis)), (lo, hi)
+        check_sum(F.cumsum(Vh, axis).numpy(), v, axis)
+        # into a view of a larger result: nothing is written beside it
+        Yh = Tensor.from_numpy(hip_backend, np.full(shape, 7, np.float16))
+        F.cummin(Vh, axis, out=Yh.slice([lo], [hi], [last]))
+        got = Yh.numpy()
+        assert np.array_equal(got[..., lo:hi], np.minimum.accumulate(v, axis=axis)), (lo, hi)
+        assert (got[..., :lo] == 7).all() and (got[..., hi:] == 7).all(), (lo, hi)
+    # every other column (stride 2 in the innermost dimension: no neighbours to pair)
+    Sh = Xh.slice([0], [w], [last], [2])
+    assert np.array_equal(F.cummax(Sh, axis).numpy(), np.maximum.accumulate(x[..., ::2], axis=axis))
+    # the columns walked backwards
+    assert np.array_equal(F.cummax(Xh.flip([last]), axis).numpy(), np.maximum.accumulate(x[..., ::-1], axis=axis))
+    Zh = Tensor.from_numpy(hip_backend, x)
+    F.cummax(Zh, axis, out=Zh)                                           # in place
+    assert np.array_equal(Zh.numpy(), np.maximum.accumulate(x, axis=axis))
+
+
 @pytest.mark.parametrize("shape,axis", [((8, 21, 64, 64), 1), ((64, 3, 50, 50), 1), ((5000, 2, 3), 1), ((3, 32, 5000), 1), ((2, 33, 5000), 1),
                                         ((17, 8000), 0), ((4, 5, 6, 700), 2)])
 def test_short_axis_beside_many_columns_one_lane_per_column(hip_backend, shape, axis):
