@@ -408,14 +408,19 @@ __global__ __launch_bounds__(kBlock) void reduce_finalize(
 
 // Columns: kept axis of extent L is contiguous, lanes run along it; the four
 // waves of a workgroup take reduced indices ty, ty+4, ... of slice `part`.
-template <typename R>
+// A lane takes C neighbouring columns in one access (C = 2 for two-byte elements where every
+// pair starts on a 4-byte boundary: with one such element per lane a wavefront's access is
+// 128 bytes wide and the kernel runs at the element rate of fp32).
+template <typename R, int C>
 __global__ __launch_bounds__(kBlock) void reduce_cols(
     const typename R::in_t* __restrict__ x, DimMap outer, int64_t L, DimMap red, int64_t n,
     int64_t col_blocks, int64_t parts, typename R::out_t* __restrict__ y, DimMap ymap, int final_op,
     typename R::acc_t* __restrict__ partial, typename R::param_t prm) {
     using acc_t = typename R::acc_t;
+    using in_t = typename R::in_t;
+    using VecIn = Vec<in_t, C>;
     constexpr int TY = kBlock / kWave;
-    __shared__ acc_t sm[TY][kWave];
+    __shared__ acc_t sm[TY][C][kWave];
     const int lx = threadIdx.x & (kWave - 1);
     const int ty = threadIdx.x / kWave;
     int64_t b = blockIdx.x;
@@ -423,15 +428,21 @@ __global__ __launch_bounds__(kBlock) void reduce_cols(
     b /= parts;
     const int64_t cb = b % col_blocks;
     const int64_t o = b / col_blocks;
-    const int64_t c = cb * kWave + lx;
+    const int64_t c = (cb * kWave + lx) * C;
 
     const int64_t per = (n + parts - 1) / parts;
     const int64_t lo = part * per;
     const int64_t hi = (lo + per < n) ? lo + per : n;
 
-    acc_t acc = R::identity();
+    acc_t acc[C];
+#pragma unroll
+    for (int k = 0; k < C; ++k) acc[k] = R::identity();
     if (c < L) {
-        const typename R::in_t* __restrict__ p = x + outer.at(o) + c;
+        const in_t* __restrict__ p = x + outer.at(o) + c;
+        auto fold = [&](const VecIn& v, int64_t j) __attribute__((always_inline)) {
+#pragma unroll
+            for (int k = 0; k < C; ++k) acc[k] = R::join(acc[k], R::map(v.v[k], j, prm));
+        };
         if (red.rank == 1) {
             const int64_t s = red.strides[0];
             int64_t j = lo + ty;
@@ -441,51 +452,60 @@ __global__ __launch_bounds__(kBlock) void reduce_cols(
             auto rows_at_once = [&](auto depth) __attribute__((always_inline)) {
                 constexpr int U = decltype(depth)::value;
                 for (; j + (U - 1) * TY < hi; j += U * TY) {
-                    typename R::in_t v[U];
+                    VecIn v[U];
 #pragma unroll
-                    for (int u = 0; u < U; ++u) v[u] = load_stream(&p[(j + u * TY) * s]);
+                    for (int u = 0; u < U; ++u) v[u] = load_stream(reinterpret_cast<const VecIn*>(&p[(j + u * TY) * s]));
 #pragma unroll
-                    for (int u = 0; u < U; ++u) acc = R::join(acc, R::map(v[u], j + u * TY, prm));
+                    for (int u = 0; u < U; ++u) fold(v[u], j + u * TY);
                 }
             };
             if (gridDim.x >= 1024) rows_at_once(std::integral_constant<int, 4>());
             else rows_at_once(std::integral_constant<int, 8>());
-            for (; j < hi; j += TY) acc = R::join(acc, R::map(load_stream(&p[j * s]), j, prm));
+            for (; j < hi; j += TY) fold(load_stream(reinterpret_cast<const VecIn*>(&p[j * s])), j);
         } else {
-            for (int64_t j = lo + ty; j < hi; j += TY) acc = R::join(acc, R::map(p[red.at(j)], j, prm));
+            for (int64_t j = lo + ty; j < hi; j += TY) fold(*reinterpret_cast<const VecIn*>(&p[red.at(j)]), j);
         }
     }
-    sm[ty][lx] = acc;
+#pragma unroll
+    for (int k = 0; k < C; ++k) sm[ty][k][lx] = acc[k];
     __syncthreads();
     if (ty == 0 && c < L) {
 #pragma unroll
-        for (int i = 1; i < TY; ++i) acc = R::join(acc, sm[i][lx]);
-        const int64_t row = o * L + c;
-        if (parts == 1) y[ymap.at(row)] = R::finish(acc, n, final_op);
-        else partial[row * parts + part] = acc;
+        for (int k = 0; k < C; ++k) {
+            acc_t all = acc[k];
+#pragma unroll
+            for (int i = 1; i < TY; ++i) all = R::join(all, sm[i][k][lx]);
+            const int64_t row = o * L + c + k;
+            if (parts == 1) y[ymap.at(row)] = R::finish(all, n, final_op);
+            else partial[row * parts + part] = all;
+        }
     }
 }
 
 // Columns beside a short reduced axis (up to 32 elements, one stride): a lane reduces a whole
 // column, all its loads in flight at once, 256 columns a workgroup and no barrier (reduce_cols
 // gives such an axis to four wavefronts an element or two each: fp32 [64, 3, 224, 224] over
-// axis 1 54 us, [8, 21, 512, 512] 60 us).
-template <typename R, int N>
+// axis 1 54 us, [8, 21, 512, 512] 60 us).  C neighbouring columns a lane, as above.
+template <typename R, int N, int C>
 __global__ __launch_bounds__(kBlock) void reduce_cols_thread(
     const typename R::in_t* __restrict__ x, DimMap outer, int64_t L, int64_t stride, int n, int64_t col_blocks,
     typename R::out_t* __restrict__ y, DimMap ymap, int final_op, typename R::param_t prm) {
+    using VecIn = Vec<typename R::in_t, C>;
     const int64_t cb = blockIdx.x % col_blocks, o = blockIdx.x / col_blocks;
-    const int64_t c = cb * kBlock + threadIdx.x;
+    const int64_t c = (cb * kBlock + threadIdx.x) * C;
     if (c >= L) return;
     const typename R::in_t* __restrict__ p = x + outer.at(o) + c;
-    typename R::in_t v[N];
+    VecIn v[N];
 #pragma unroll
-    for (int j = 0; j < N; ++j) v[j] = load_stream(&p[(j < n ? j : 0) * stride]);
-    typename R::acc_t acc = R::identity();
+    for (int j = 0; j < N; ++j) v[j] = load_stream(reinterpret_cast<const VecIn*>(&p[(j < n ? j : 0) * stride]));
 #pragma unroll
-    for (int j = 0; j < N; ++j)
-        if (j < n) acc = R::join(acc, R::map(v[j], j, prm));
-    y[ymap.at(o * L + c)] = R::finish(acc, n, final_op);
+    for (int k = 0; k < C; ++k) {
+        typename R::acc_t acc = R::identity();
+#pragma unroll
+        for (int j = 0; j < N; ++j)
+            if (j < n) acc = R::join(acc, R::map(v[j].v[k], j, prm));
+        y[ymap.at(o * L + c + k)] = R::finish(acc, n, final_op);
+    }
 }
 
 // --------------------------------------------------------------------------
@@ -626,28 +646,44 @@ int launch_reduce(hipStream_t stream, const ReducePlan& pl, const typename R::in
         outer.rank -= 1;
         outer.dims[outer.rank] = 1;
         outer.strides[outer.rank] = 0;
+        // two-byte elements: two neighbouring columns a lane where every pair starts on a 4-byte boundary
+        bool pairs = sizeof(T) == 2 && !std::is_class<T>::value && L % 2 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0;
+        for (int i = 0; pairs && i < outer.rank; ++i) pairs = outer.strides[i] % 2 == 0;
+        for (int i = 0; pairs && i < pl.red.rank; ++i) pairs = pl.red.strides[i] % 2 == 0;
+        auto with_cols = [&](auto&& launch) {
+            if constexpr (sizeof(T) == 2 && !std::is_class<T>::value) {
+                if (pairs) { launch(std::integral_constant<int, 2>()); return; }
+            }
+            launch(std::integral_constant<int, 1>());
+        };
+        const int per_lane = pairs ? 2 : 1;
         if (n <= 32 && pl.red.rank == 1 && m >= 4096) {
-            const int64_t wide_blocks = ceil_div(L, static_cast<int64_t>(kBlock));
+            const int64_t wide_blocks = ceil_div(L, static_cast<int64_t>(kBlock) * per_lane);
             const int64_t blocks = (m / L) * wide_blocks;
             if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
             const dim3 grid(static_cast<unsigned>(blocks)), block(kBlock);
-#define DLFX_REDUCE_THREAD(N) reduce_cols_thread<R, N><<<grid, block, 0, stream>>>(x, outer, L, pl.red.strides[0], static_cast<int>(n), wide_blocks, y, pl.ymap, final_op, prm)
-            if (n <= 4) DLFX_REDUCE_THREAD(4);
-            else if (n <= 8) DLFX_REDUCE_THREAD(8);
-            else if (n <= 16) DLFX_REDUCE_THREAD(16);
-            else DLFX_REDUCE_THREAD(32);
+            with_cols([&](auto cols_per_lane) {
+                constexpr int C = decltype(cols_per_lane)::value;
+#define DLFX_REDUCE_THREAD(N) reduce_cols_thread<R, N, C><<<grid, block, 0, stream>>>(x, outer, L, pl.red.strides[0], static_cast<int>(n), wide_blocks, y, pl.ymap, final_op, prm)
+                if (n <= 4) DLFX_REDUCE_THREAD(4);
+                else if (n <= 8) DLFX_REDUCE_THREAD(8);
+                else if (n <= 16) DLFX_REDUCE_THREAD(16);
+                else DLFX_REDUCE_THREAD(32);
 #undef DLFX_REDUCE_THREAD
+            });
             DLFX_CHECK_LAUNCH();
             return DLFX_OK;
         }
-        const int64_t col_blocks = ceil_div(L, kWave);
+        const int64_t col_blocks = ceil_div(L, static_cast<int64_t>(kWave) * per_lane);
         const int64_t base_blocks = (m / L) * col_blocks;
-        const int64_t parts = col_parts(base_blocks, n);
+        const int64_t parts = col_parts(base_blocks * per_lane, n);      // (as many slices as one column a lane would get: what the scratch query allows for)
         if (base_blocks * parts > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
         if (parts > 1 && scratch_bytes < static_cast<size_t>(m * parts) * sizeof(acc_t))
             return DLFX_ERR_SCRATCH_TOO_SMALL;
-        reduce_cols<R><<<dim3(static_cast<unsigned>(base_blocks * parts)), dim3(kBlock), 0, stream>>>(
-            x, outer, L, pl.red, n, col_blocks, parts, y, pl.ymap, final_op, partial, prm);
+        with_cols([&](auto cols_per_lane) {
+            reduce_cols<R, decltype(cols_per_lane)::value><<<dim3(static_cast<unsigned>(base_blocks * parts)), dim3(kBlock), 0, stream>>>(
+                x, outer, L, pl.red, n, col_blocks, parts, y, pl.ymap, final_op, partial, prm);
+        });
         DLFX_CHECK_LAUNCH();
         if (parts > 1) {
             reduce_finalize<R><<<dim3(static_cast<unsigned>(ceil_div(m, kBlock / kWave))), dim3(kBlock), 0, stream>>>(

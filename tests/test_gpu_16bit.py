@@ -88,6 +88,41 @@ def test_argmax_argmin_half_and_int16(hip_backend, oracle_backend):
     assert np.array_equal(F.argmax(Xh, 1).numpy(), F.argmax(Xo, 1).numpy())
 
 
+@pytest.mark.parametrize("shape,axes", [((8, 21, 64, 64), (1,)), ((4, 100, 30, 30), (1,)), ((4096, 128), (0,)), ((5000, 67), (0,)), ((64, 3, 25, 25), (1,)),
+                                        ((16, 50, 6, 20), (0, 2)), ((3, 70000, 6), (1,)), ((2, 9, 5000), (1,))])
+def test_two_byte_columns_reduced_in_pairs(hip_backend, oracle_backend, shape, axes):
+    """Reductions and arg-reductions over axes that are not the innermost: a lane takes two
+    neighbouring two-byte columns in one 4-byte access where every pair starts on a 4-byte
+    boundary (an even innermost extent, even strides, an aligned base) and one column otherwise
+    (odd extents, views that start at an odd element).  Extrema, counts and positions are exact;
+    sums are held to the half-ulp + fp32 bound."""
+    n = int(np.prod([shape[a] for a in axes]))
+    last = len(shape) - 1
+    w = shape[last]
+    xh = np.round(halfs(130, shape, 3) * 4) / 4                     # quarter steps: ties among the extrema
+    xs = shorts(131, shape, -40, 40)
+    for x in (xh, xs):
+        Xh, Xo = both(hip_backend, oracle_backend, x)
+        views = [(Xh, Xo, x)]
+        for lo, hi in ((2, w), (1, w - 1), (0, w - 1)):
+            if hi - lo >= 1:
+                views.append((Xh.slice([lo], [hi], [last]), Xo.slice([lo], [hi], [last]), x[..., lo:hi]))
+        views.append((Xh.slice([0], [w], [last], [2]), Xo.slice([0], [w], [last], [2]), x[..., ::2]))
+        for Vh, Vo, v in views:
+            if len(axes) == 1:
+                assert np.array_equal(F.argmax(Vh, axes[0]).numpy(), F.argmax(Vo, axes[0]).numpy())
+                assert np.array_equal(F.argmin(Vh, axes[0], False).numpy(), F.argmin(Vo, axes[0], False).numpy())
+                assert np.array_equal(F.argmax(Vh, axes[0], True, np.int64).numpy(), F.argmax(Vo, axes[0], True, np.int64).numpy())
+            if x.dtype == np.float16:
+                assert np.array_equal(F.reduce("reduce_max", Vh, axes).numpy(), v.max(axis=axes))
+                assert np.array_equal(F.reduce("reduce_min", Vh, axes, True).numpy(), v.min(axis=axes, keepdims=True))
+                assert np.array_equal(F.count(Vh, np.float16(0.25), axes).numpy(), (v == np.float16(0.25)).sum(axis=axes))
+                got = F.reduce("reduce_sum", Vh, axes).numpy().astype(np.float64)
+                exact, mag = v.astype(np.float64).sum(axis=axes), np.abs(v.astype(np.float64)).sum(axis=axes)
+                bound = np.abs(exact) * 2.0 ** -10 + 2.0 ** -24 + 4 * max(1.0, np.log2(n)) * np.finfo(np.float32).eps * mag
+                assert (np.abs(got - exact) <= bound).all()
+
+
 @pytest.mark.parametrize("n", [5, 300, 5000, 70000])
 def test_half_scans(hip_backend, oracle_backend, n):
     x = halfs(129 + n, (3, n), 0.5)
