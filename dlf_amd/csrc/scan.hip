@@ -653,6 +653,16 @@ struct ColumnAt {
         }
         step_bytes = axis_stride * static_cast<int64_t>(sizeof(P));
     }
+    // the same by a running pointer: `row` is where position p starts, `next` moves it one position on
+    // (an address worked out per position from p * stride keeps a product per position in scalar
+    // registers for the whole loop once the compiler has unrolled it)
+    using Row = std::conditional_t<std::is_const<P>::value, const char, char>*;
+    __device__ __forceinline__ Row row(int64_t position) const { return reinterpret_cast<Row>(base) + position * step_bytes; }
+    __device__ __forceinline__ Row next(Row r) const { return r + step_bytes; }
+    __device__ __forceinline__ P* in_row(Row r) const {
+        if constexpr (NARROW) return reinterpret_cast<P*>(r + static_cast<uint64_t>(lane_bytes));
+        else return reinterpret_cast<P*>(r);
+    }
     __device__ __forceinline__ P* at(int64_t position) const {
         using Byte = std::conditional_t<std::is_const<P>::value, const char, char>;
         Byte* row = reinterpret_cast<Byte*>(base) + position * step_bytes;
@@ -768,11 +778,12 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(1, DLFX_
     // (kept as loaded: two-byte elements wait two to a register)
     auto load_chunk = [&](int64_t s, VecX* v) __attribute__((always_inline)) {
         const int64_t p0 = s + static_cast<int64_t>(ty) * chunk;
+        auto xrow = xc.row(p0);
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
+        for (int r = 0; r < R; ++r, xrow = xc.next(xrow)) {
             const int64_t p = p0 + r;
             if (live && r < chunk && p < hi) {
-                v[r] = load_stream(reinterpret_cast<const VecX*>(xc.at(p)));
+                v[r] = load_stream(reinterpret_cast<const VecX*>(xc.in_row(xrow)));
             } else {
 #pragma unroll
                 for (int c = 0; c < C; ++c) v[r].v[c] = static_cast<X>(Op::identity());      // (folds as the identity, also where scan_input maps elements to 0 / 1)
@@ -808,24 +819,25 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(1, DLFX_
             carry[c] = Op::apply(carry[c], all);
         }
         if (live) {
+            auto yrow = yc.row(p0);
             if (exclusive) {
 #pragma unroll
-                for (int r = 0; r < R; ++r) {
+                for (int r = 0; r < R; ++r, yrow = yc.next(yrow)) {
                     const int64_t p = p0 + r;
                     VecY out;
 #pragma unroll
                     for (int c = 0; c < C; ++c)
                         out.v[c] = static_cast<Y>((r == 0) ? pre[c] : Op::apply(pre[c], v[(r > 0 ? r - 1 : 0) * C + c]));
-                    if (r < chunk && p < hi) store_stream(reinterpret_cast<VecY*>(yc.at(p)), out);
+                    if (r < chunk && p < hi) store_stream(reinterpret_cast<VecY*>(yc.in_row(yrow)), out);
                 }
             } else {
 #pragma unroll
-                for (int r = 0; r < R; ++r) {
+                for (int r = 0; r < R; ++r, yrow = yc.next(yrow)) {
                     const int64_t p = p0 + r;
                     VecY out;
 #pragma unroll
                     for (int c = 0; c < C; ++c) out.v[c] = static_cast<Y>(Op::apply(pre[c], v[r * C + c]));
-                    if (r < chunk && p < hi) store_stream(reinterpret_cast<VecY*>(yc.at(p)), out);
+                    if (r < chunk && p < hi) store_stream(reinterpret_cast<VecY*>(yc.in_row(yrow)), out);
                 }
             }
         }
