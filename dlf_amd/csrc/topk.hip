@@ -778,8 +778,10 @@ constexpr int kThreadRowLimit = 8;     // ... and topk_rows_thread
 }  // namespace
 #if DLFX_TOPK_PART == 0
 int g_topk_thread_rows = 256;
+int g_topk_cols_waves = 0;            // dlfx_set_tuning "topk_cols_waves": 1, 4 or 8 wavefronts a block of 64 rows in topk_cols (0: by the shape)
 #else
 extern int g_topk_thread_rows;
+extern int g_topk_cols_waves;
 #endif
 namespace {
 
@@ -789,6 +791,25 @@ __device__ __forceinline__ void cols_insert(K (&lo)[KMAX], uint32_t (&li)[KMAX],
 #pragma unroll
     for (int p = 0; p < KMAX; ++p) {
         const bool b = beats<K>(o, x, lo[p], li[p]) != 0u;
+        const K to = lo[p];
+        const uint32_t tx = li[p];
+        lo[p] = b ? o : to;
+        li[p] = b ? x : tx;
+        o = b ? to : o;
+        x = b ? tx : x;
+    }
+}
+
+// The same for an element that comes after every entry of a full list (a higher index than all
+// of them, no placeholder left): it enters before the entries with a smaller image, and a tie
+// never moves it forward - one comparison per entry instead of the (image, index) pair's.
+template <typename K, int KMAX>
+__device__ __forceinline__ void cols_insert_later(K (&lo)[KMAX], uint32_t (&li)[KMAX], K o, uint32_t x) {
+    if (!(o > lo[KMAX - 1])) return;
+    bool b = false;
+#pragma unroll
+    for (int p = 0; p < KMAX; ++p) {
+        b = b || o > lo[p];                 // (behind the place where it entered every entry moves down one place, ties included)
         const K to = lo[p];
         const uint32_t tx = li[p];
         lo[p] = b ? o : to;
@@ -828,6 +849,11 @@ __global__ __launch_bounds__(kWave * SEG) void topk_cols(TopkIo<typename BitsOf<
     const int64_t chunk = (n + SEG - 1) / SEG;
     const int64_t j0 = seg * chunk;
     const int64_t j1 = j0 + chunk < n ? j0 + chunk : n;
+    // (a wavefront runs an insertion wherever one of its 64 rows needs it, which is nearly
+    // everywhere: the kernel is bound by vector ALU work - fp32 [32, 512, 56, 56] along axis 1,
+    // limit 5: 5700 instructions a wavefront and 64 positions - so the list is exactly as long as
+    // the limit asks and, once it is full, entries are compared by their images alone)
+    constexpr int kFill = (KMAX + kUnroll - 1) / kUnroll * kUnroll;      // the list is full after so many elements
     for (int64_t j = j0; j < j1; j += kUnroll) {
         K o[kUnroll];
 #pragma unroll
@@ -835,9 +861,16 @@ __global__ __launch_bounds__(kWave * SEG) void topk_cols(TopkIo<typename BitsOf<
             const bool in = live && j + u < j1;
             o[u] = in ? to_ord<K>(static_cast<K>(widen_bits<K, S>(load_stream(xr + (j + u) * io.sx), kind) ^ flip), kind, 1) : K(0);
         }
+        // (lists of more than 8 entries keep the one insertion: two unrolled copies of it cost them
+        // registers and a wavefront per SIMD - int64 [16, 80, 160, 160], limit 16: 406 -> 650 us)
+        if (KMAX > 8 || j - j0 < kFill) {
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
-            cols_insert<K, KMAX>(lo, li, o[u], (live && j + u < j1) ? static_cast<uint32_t>(j + u) : 0xffffffffu);
+            for (int u = 0; u < kUnroll; ++u)
+                cols_insert<K, KMAX>(lo, li, o[u], (live && j + u < j1) ? static_cast<uint32_t>(j + u) : 0xffffffffu);
+        } else {
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) cols_insert_later<K, KMAX>(lo, li, o[u], static_cast<uint32_t>(j + u));
+        }
     }
     if constexpr (SEG > 1) {
         if (seg > 0) {
@@ -1503,7 +1536,11 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
         io.xmap.strides[io.xmap.rank - 1] == 1 && io.xmap.dims[io.xmap.rank - 1] >= kWave) {
         const int lim = static_cast<int>(limit);
         const int64_t blocks = ceil_div(m, static_cast<int64_t>(kWave));
-        const int seg = (blocks >= 8192 || n < 64) ? 1 : (blocks >= 2048 || n < 512) ? 4 : 8;
+        // wavefronts that share a block of 64 rows, each with a piece of the axis (measured on fp32, axes of 64 to
+        // 2048 positions, 500 to 16400 blocks: eight while the blocks are few - and for limits of one or two, whose
+        // lists are cheap to merge, up to 5000 blocks -, four beyond; one only for axes too short to cut)
+        int seg = n < 64 ? 1 : blocks < (lim <= 2 ? 5000 : 1024) ? 8 : 4;
+        if (g_topk_cols_waves) seg = g_topk_cols_waves;
         const dim3 cgrid(static_cast<unsigned>(ceil_div(blocks, 8) * 8));
 #define DLFX_TOPK_COLS(KMAX)                                                                        \
     do {                                                                                            \
@@ -1513,8 +1550,12 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
     } while (0)
         if (lim <= 1) DLFX_TOPK_COLS(1);
         else if (lim <= 2) DLFX_TOPK_COLS(2);
+        else if (lim <= 3) DLFX_TOPK_COLS(3);
         else if (lim <= 4) DLFX_TOPK_COLS(4);
+        else if (lim <= 5) DLFX_TOPK_COLS(5);
+        else if (lim <= 6) DLFX_TOPK_COLS(6);
         else if (lim <= 8) DLFX_TOPK_COLS(8);
+        else if (lim <= 12) DLFX_TOPK_COLS(12);
         else DLFX_TOPK_COLS(16);
 #undef DLFX_TOPK_COLS
         DLFX_CHECK_LAUNCH();
@@ -1620,6 +1661,10 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
 
 #if DLFX_TOPK_PART == 0
 bool set_topk_tuning(const char* key, int64_t value) {
+    if (!std::strcmp(key, "topk_cols_waves") && (value == 0 || value == 1 || value == 4 || value == 8)) {
+        g_topk_cols_waves = static_cast<int>(value);
+        return true;
+    }
     if (!std::strcmp(key, "topk_thread_rows") && value >= 0 && value <= 65536) {
         g_topk_thread_rows = static_cast<int>(value);
         return true;
