@@ -1586,7 +1586,10 @@ int run_top_k(hipStream_t stream, int64_t limit, int dir, int dtype, int index_d
     } while (0)
         if (lim <= 1) DLFX_TOPK_THREAD(1);
         else if (lim <= 2) DLFX_TOPK_THREAD(2);
+        else if (lim <= 3) DLFX_TOPK_THREAD(3);
         else if (lim <= 4) DLFX_TOPK_THREAD(4);
+        else if (lim <= 5) DLFX_TOPK_THREAD(5);
+        else if (lim <= 6) DLFX_TOPK_THREAD(6);
         else DLFX_TOPK_THREAD(8);
 #undef DLFX_TOPK_THREAD
         DLFX_CHECK_LAUNCH();
