@@ -112,7 +112,7 @@ def make_ops(be, which):
     from dlf_amd.shape import Shape
 
     dev = be.device
-    np_of = {torch.float32: np.float32, torch.int32: np.int32, torch.int64: np.int64, torch.float64: np.float64}
+    np_of = {torch.float32: np.float32, torch.int32: np.int32, torch.int64: np.int64, torch.float64: np.float64, torch.float16: np.float16}
 
     def tensor(t):
         return Tensor(be, Shape(list(t.shape)), t.view(-1), np_of[t.dtype])
@@ -330,6 +330,31 @@ def make_ops(be, which):
                                    ((3355, 10000), torch.float64, "f64_normal_[3355,10000]")):
             xs = gen(shape, dtype, lambda c: synth.normal(52 + 100 * c), 2)
             ops += [op for op in sort_ops(be, tensor, xs, "B3", text) if "_asc_" in op.name]
+        # half elements along an axis that is not the innermost: two neighbouring columns a lane
+        for shape, axis in (((32, 512, 56, 56), 1), ((64, 1 << 20), 0), ((8, 21, 512, 512), 1)):
+            xs = gen(shape, torch.float16, lambda c: synth.normal(54 + 100 * c), 2)
+            text = "_f16_[%s]" % ",".join(str(e) for e in shape)
+            count = int(np.prod(shape))
+            calls, _ = scan_calls(xs, axis)
+            ops.append(Op("B5", "cumsum{%d}%s" % (axis, text), count, 4 * count, calls, timed_only(calls[0])))
+            calls, _ = reduce_calls("reduce_sum", xs, [axis])
+            ops.append(Op("B5", "reduce_sum{%d}%s" % (axis, text), count, 2 * count, calls, timed_only(calls[0])))
+            calls, _ = argmax_calls(xs, axis)
+            ops.append(Op("B5", "argmax{%d}%s" % (axis, text), count, 2 * count, calls, timed_only(calls[0])))
+        # top_k along an axis that is not the innermost (register lists, a lane per column)
+        for shape, axis in (((32, 512, 56, 56), 1), ((16, 80, 160, 160), 1)):
+            xs = gen(shape, torch.float32, lambda c: synth.normal(55 + 100 * c), 2)
+            count = int(np.prod(shape))
+            for k in (1, 5):
+                out_dims = [k if i == axis else e for i, e in enumerate(shape)]
+                Yk = Tensor.empty(be, out_dims, np.float32)
+                Ik = Tensor.empty(be, out_dims, np.int32)
+                calls = []
+                for x in xs:
+                    X = tensor(x)
+                    calls.append(be.top_k(k, 1, dtype_code(np.float32), 2, X.shape.moveaxis(axis, -1), X.storage, Yk.shape.moveaxis(axis, -1), Yk.storage,
+                                          Ik.shape.moveaxis(axis, -1), Ik.storage, defer=True))
+                ops.append(Op("B6", "top_k%d{%d}_f32_[%s]" % (k, axis, ",".join(str(e) for e in shape)), count, 4 * count, calls, timed_only(calls[0])))
         # top_k of very long rows
         for rows_l, n_l in ((1, 1 << 24), (1, 1 << 23)):
             xl_ = gen((rows_l, n_l), torch.float32, lambda c: synth.normal(53 + 100 * c), 2)
@@ -685,7 +710,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3 | short (many short rows and an outer axis; not part of all) | spread (sorts of N(0,1) rows; not part of all) | ceil (copy and read-only streams at the C2 and C5 sizes; part of all) | ceilbig (the same streams at 1 GiB and 4 GiB; not part of all) | long (softmax and top_k over a few very long rows; not part of all) | repeats (sorts of rows of one value, of ten values and of clustered keys; not part of all) | beside (shapes beside the baseline's at which sweeps found steps: outer-axis scans and reductions, statistics per channel, rows near the end of the bucket route, top_k of very long rows; not part of all)")
+    ap.add_argument("--configs", default="all", help="all | step | comma-separated subset of c1,c2,c3,c4,c5,n1,n2,n3 | short (many short rows and an outer axis; not part of all) | spread (sorts of N(0,1) rows; not part of all) | ceil (copy and read-only streams at the C2 and C5 sizes; part of all) | ceilbig (the same streams at 1 GiB and 4 GiB; not part of all) | long (softmax and top_k over a few very long rows; not part of all) | repeats (sorts of rows of one value, of ten values and of clustered keys; not part of all) | beside (shapes beside the baseline's at which sweeps found steps: outer-axis scans and reductions, statistics per channel, rows near the end of the bucket route, half elements along an outer axis, top_k along an outer axis and of very long rows; not part of all)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
