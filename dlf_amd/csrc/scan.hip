@@ -1286,7 +1286,7 @@ using namespace dlfx;
 
 namespace dlfx {
 bool set_scan_tuning(const char* key, int64_t value) {
-    if (!std::strcmp(key, "scan_cols_per_lane") && (value == 0 || value == 1 || value == 2 || value == 4)) {
+    if (!std::strcmp(key, "scan_cols_per_lane") && (value == 0 || value == 1 || value == 2)) {
         g_cols_per_lane = static_cast<int>(value);
         return true;
     }

@@ -96,6 +96,12 @@ int dlfx_last_hip_error(void);
  *   "topk_thread_rows" longest row (default 256; half of it for 8-byte keys) for which top_k
  *                      with a limit of at most 8 over at least 16384 contiguous rows gives
  *                      each row to one thread.
+ *   "topk_cols_waves"  wavefronts (1, 4 or 8; 0, the default: by the shape) that share a block of
+ *                      64 neighbouring rows, each with a piece of the axis, when top_k with a
+ *                      small limit runs along an axis that is not the innermost.
+ *   "scan_cols_per_lane" the most neighbouring columns (1 or 2; 0, the default: 2 where the
+ *                      layout allows) that a lane takes in one access when two-byte elements
+ *                      are scanned along an axis that is not the innermost.
  * Returns DLFX_ERR_UNKNOWN_OP for an unknown key or out-of-range value.  No
  * counterpart in the reference (its database/ tuning tables play this role). */
 int dlfx_set_tuning(const char* key, int64_t value);

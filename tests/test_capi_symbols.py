@@ -57,9 +57,11 @@ def test_host_only_calls():
     assert lib.dlfx_sort_scratch_bytes(5, 64, 1 << 16) >= 2 * 64 * (1 << 16) * 2
     assert lib.dlfx_set_tuning(b"no_such_knob", 1) == -3
     assert lib.dlfx_set_tuning(b"scan_poll_limit", 2048) == 0
-    for knob, value in ((b"sort_poll_limit", 2048), (b"sort_wave_rows", 512), (b"sort_buckets", 1), (b"sort_compare_max", 32), (b"topk_thread_rows", 256)):
+    for knob, value in ((b"sort_poll_limit", 2048), (b"sort_wave_rows", 512), (b"sort_buckets", 1), (b"sort_compare_max", 32), (b"topk_thread_rows", 256),
+                        (b"topk_cols_waves", 0), (b"scan_cols_per_lane", 0)):
         assert lib.dlfx_set_tuning(knob, value) == 0
     assert lib.dlfx_set_tuning(b"sort_wave_rows", 100000) == -3
+    assert lib.dlfx_set_tuning(b"topk_cols_waves", 3) == -3 and lib.dlfx_set_tuning(b"scan_cols_per_lane", 4) == -3
 
 
 def test_argument_errors_are_reported_without_a_gpu():

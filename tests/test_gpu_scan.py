@@ -426,6 +426,14 @@ def test_two_byte_columns_go_two_to_a_lane(hip_backend, shape, axis):
     Zh = Tensor.from_numpy(hip_backend, x)
     F.cummax(Zh, axis, out=Zh)                                           # in place
     assert np.array_equal(Zh.numpy(), np.maximum.accumulate(x, axis=axis))
+    # one column a lane gives the same, sums included (the same additions in the same order)
+    pairs = F.cumsum(Xh, axis).numpy()
+    hip_backend.set_tuning("scan_cols_per_lane", 1)
+    try:
+        singles = F.cumsum(Xh, axis).numpy()
+    finally:
+        hip_backend.set_tuning("scan_cols_per_lane", 0)
+    assert np.array_equal(pairs.view(np.uint16), singles.view(np.uint16))
 
 
 @pytest.mark.parametrize("shape,axis", [((8, 21, 64, 64), 1), ((64, 3, 50, 50), 1), ((5000, 2, 3), 1), ((3, 32, 5000), 1), ((2, 33, 5000), 1),

@@ -232,6 +232,30 @@ def test_rows_side_by_side_in_memory(hip_backend, oracle_backend, n):
     assert np.array_equal(Ih.numpy()[ok], Io.numpy()[ok]) and np.array_equal(Yh.numpy()[ok], Yo.numpy()[ok])
 
 
+@pytest.mark.parametrize("n", [64, 200, 513])
+def test_rows_side_by_side_any_number_of_waves(hip_backend, oracle_backend, n):
+    """The wavefronts that share a block of 64 neighbouring rows each take a piece of the axis and
+    merge their lists: one, four and eight of them give what the oracle gives, for every list
+    length, with ties (lower index first) inside a piece and across pieces."""
+    cols = 16384 + 70
+    for dtype, spread in ((np.float32, 3), (np.int64, 2), (np.int16, 40), (np.float64, 1000)):
+        x = np.round(normal(240 + n, n * cols) * spread).astype(dtype).reshape(n, cols)
+        x[:, 5] = 1                                                    # one value: the first `limit` positions win
+        x[n // 2:, 6] = x[: n - n // 2, 6]                             # every value twice, in different pieces
+        Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
+        for k in (1, 2, 3, 5, 6, 7, 8):
+            for largest in (True, False):
+                Yo, Io = F.top_k(Xo, k, 0, largest)
+                for waves in (1, 4, 8, 0):
+                    hip_backend.set_tuning("topk_cols_waves", waves)
+                    try:
+                        Yh, Ih = F.top_k(Xh, k, 0, largest)
+                    finally:
+                        hip_backend.set_tuning("topk_cols_waves", 0)
+                    assert np.array_equal(Ih.numpy(), Io.numpy()), (dtype, k, largest, waves)
+                    assert np.array_equal(Yh.numpy(), Yo.numpy()), (dtype, k, largest, waves)
+
+
 @pytest.mark.parametrize("n", [17, 33, 63, 64])
 def test_short_rows_side_by_side_with_a_long_list(hip_backend, oracle_backend, n):
     """top_k along an outer axis of at most 64 elements with a limit beyond the register lists:
