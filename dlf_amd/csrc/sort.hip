@@ -744,6 +744,72 @@ __global__ __launch_bounds__(256) void sort_cols_wave(PassIo<K> io, int64_t rows
     }
 }
 
+// The same for rows of 65 to 64 * ITEMS elements (4-byte keys): a tile of 16 neighbouring rows,
+// read 16 rows wide (64 bytes a position, where a wavefront per row reads every element of its
+// row from a cache line of its own: fp32 [32, 512, 56, 56] along axis 1 440 us), each wavefront
+// sorts four of them with the network of sort_rows_wave_items (pitch 17: a wavefront's accesses
+// to one row of the tile fall into different banks), and the tile leaves the way it came.
+template <typename K, bool PAIRS, int ITEMS>
+__global__ __launch_bounds__(256) void sort_cols_tile(PassIo<K> io, int64_t rows, int64_t n) {
+    constexpr int kTile = 16, kPitch = kTile + 1;
+    __shared__ K keys[ITEMS * kWave * kPitch];
+    __shared__ uint32_t places[PAIRS ? ITEMS * kWave * kPitch : 1];
+    const int lane = lane_id();
+    const int w = threadIdx.x / kWave;
+    const int64_t row0 = block_of(io) * kTile;
+    if (row0 >= rows) return;
+    const int r = threadIdx.x % kTile;                     // this thread's row of the tile in the load and store phases
+    const int a0 = threadIdx.x / kTile;                    // ... and its first position of the axis
+    const bool row_live = row0 + r < rows;
+    const int n32 = static_cast<int>(n);
+    const K* xrow = io.x + (row_live ? io.xmap.at(row0 + r) : 0);
+    for (int a = a0; a < n32; a += 256 / kTile)
+        keys[a * kPitch + r] = row_live ? key_of_element<K>(io, xrow[static_cast<int64_t>(a) * io.sx]) : ~K(0);
+    __syncthreads();
+    for (int q = w; q < kTile; q += 4) {                   // row q of the tile: element i * 64 + lane is item i of the lane
+        K key[ITEMS];
+        uint32_t idx[ITEMS];
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const int e = i * kWave + lane;
+            key[i] = e < n32 ? keys[e * kPitch + q] : ~K(0);       // padding sorts last
+            idx[i] = static_cast<uint32_t>(e);
+        }
+        wave_bitonic_items<PAIRS, ITEMS>(key, idx, [](K ka, uint32_t ia, K kb, uint32_t ib) {      // a strictly before b
+            if constexpr (PAIRS) return ka < kb || (ka == kb && ia < ib);
+            else return ka < kb;
+        });
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const int e = i * kWave + lane;
+            if (e >= n32) continue;
+            K bits = decode_key<K>(key[i], io.kind, io.descending);
+            if constexpr (PAIRS) {
+                if (io.restore_zero && static_cast<K>(bits << 1) == 0 && row0 + q < rows)
+                    bits = io.x[io.xmap.at(row0 + q) + static_cast<int64_t>(idx[i]) * io.sx];
+                places[e * kPitch + q] = idx[i];
+            }
+            keys[e * kPitch + q] = bits;
+        }
+    }
+    __syncthreads();
+    if (!row_live) return;
+    if (io.y) {
+        K* yrow = io.y + io.ymap.at(row0 + r);
+        for (int a = a0; a < n32; a += 256 / kTile) yrow[static_cast<int64_t>(a) * io.sy] = keys[a * kPitch + r];
+    }
+    if constexpr (PAIRS) {
+        if (io.idx) {
+            const int64_t irow = io.imap.at(row0 + r);
+            for (int a = a0; a < n32; a += 256 / kTile) {
+                const int64_t at = irow + static_cast<int64_t>(a) * io.si;
+                if (io.idx64) static_cast<int64_t*>(io.idx)[at] = static_cast<int64_t>(places[a * kPitch + r]);
+                else static_cast<int32_t*>(io.idx)[at] = static_cast<int32_t>(places[a * kPitch + r]);
+            }
+        }
+    }
+}
+
 // longest row sorted by one wavefront (dlfx_set_tuning "sort_wave_rows": 64, 128, 256 or 512)
 int g_sort_wave_rows = 512;
 
@@ -774,7 +840,22 @@ int launch_small(hipStream_t stream, const PassIo<K>& io_in, int64_t m, int64_t 
     };
     // eight items per lane pay off except for 4-byte keys that carry an index
     const bool wave_items8 = g_sort_wave_rows >= 8 * kWave && !(PAIRS && sizeof(K) == 4);
+    // (tiles of 16 rows: the innermost run of rows at least that long, and rows enough for a few tiles a compute
+    // unit.  Keys alone, rows of up to 256 elements: fp32 [8, 128, 256, 256] along axis 1 482 -> 268 us,
+    // [256, 100000] along axis 0 183 -> 112 us.  With indices the tile costs LDS that the wavefront-per-row
+    // kernels do not need and was slower from 129 elements on (317 -> 353 us at 200, 527 -> 609 us at 256) and
+    // within 8 % below; eight items a lane lost both ways at 300 elements (222 -> 282 us); a row that fills
+    // little of four items a lane - 129 to 160 elements - gains nothing either)
+    const bool tiles = !PAIRS && side_by_side && sizeof(K) == 4 && n > kWave && n <= 4 * kWave && !(n > 2 * kWave && n <= 160) && m >= 4096 &&
+                       io.xmap.dims[io.xmap.rank - 1] >= 16;
     if (side_by_side && n <= kWave && m >= 4096) sort_cols_wave<K, PAIRS><<<dim3(static_cast<unsigned>(ceil_div(m, kWave))), block, 0, stream>>>(io, m, n);
+    else if (tiles) {
+        if constexpr (sizeof(K) == 4) {
+            const dim3 g = grid_for(16);
+            if (n <= 2 * kWave) sort_cols_tile<K, PAIRS, 2><<<g, block, 0, stream>>>(io, m, n);
+            else sort_cols_tile<K, PAIRS, 4><<<g, block, 0, stream>>>(io, m, n);
+        }
+    }
     else if (n <= 4) { const dim3 g = grid_for(64); sort_rows_wave<K, PAIRS, 4><<<g, block, 0, stream>>>(io, m, n); }
     else if (n <= 8) { const dim3 g = grid_for(32); sort_rows_wave<K, PAIRS, 8><<<g, block, 0, stream>>>(io, m, n); }
     else if (n <= 16) { const dim3 g = grid_for(16); sort_rows_wave<K, PAIRS, 16><<<g, block, 0, stream>>>(io, m, n); }

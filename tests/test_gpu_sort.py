@@ -779,3 +779,43 @@ def test_short_rows_side_by_side_in_memory(hip_backend, oracle_backend, n):
     Y, I = F.argsort(T, 1, True, with_values=True)
     Yo, Io = F.argsort(O, 1, True, with_values=True)
     assert np.array_equal(I.numpy(), Io.numpy()) and np.array_equal(Y.numpy().view(np.uint32), Yo.numpy().view(np.uint32))
+
+
+@pytest.mark.parametrize("n", [65, 100, 128, 129, 161, 200, 255, 256, 257])
+def test_rows_of_up_to_256_keys_side_by_side_in_memory(hip_backend, oracle_backend, n):
+    """sort along an outer axis of 65 to 256 elements with thousands of rows side by side: 4-byte
+    keys pass through LDS in tiles of 16 rows (129 to 160 elements and every argsort keep a
+    wavefront per row).  Both directions, a row count that leaves the last tile ragged, a middle
+    axis whose innermost run is shorter than a tile, in place, signed zeros and NaNs, a view
+    that steps over every other row; the other key widths and argsort beside it."""
+    cols = 4099
+    for dtype in (np.float32, np.int32, np.int64, np.float16):
+        x = (normal(290 + n, n * cols) * 50).astype(dtype).reshape(n, cols)
+        x[:, 1] = x[0, 1]
+        x[: n // 2, 3] = x[n // 2: 2 * (n // 2), 3]
+        Xh, Xo = Tensor.from_numpy(hip_backend, x), Tensor.from_numpy(oracle_backend, x)
+        for desc in (False, True):
+            want = np.sort(x, axis=0, kind="stable")
+            want = want[::-1] if desc else want
+            assert np.array_equal(F.sort(Xh, 0, desc).numpy(), want), (dtype, desc)
+            I, Io = F.argsort(Xh, 0, desc), F.argsort(Xo, 0, desc)
+            assert np.array_equal(I.numpy(), Io.numpy()), (dtype, desc)
+        Z = Tensor.from_numpy(hip_backend, x)
+        F.sort(Z, 0, False, out=Z)                                     # in place
+        assert np.array_equal(Z.numpy(), np.sort(x, axis=0, kind="stable"))
+        V = Xh.slice([0], [cols], [1], [2])                            # every other row
+        assert np.array_equal(F.sort(V, 0).numpy(), np.sort(x[:, ::2], axis=0, kind="stable"))
+    a = (normal(291 + n, 5 * n * 900) * 9).astype(np.float32).reshape(5, n, 900)
+    a[1, 0, :] = 0.0
+    a[1, n - 1, :] = -0.0
+    a[2, 5, ::7] = np.nan
+    # (comparisons do not order NaNs, nor -0.0 against +0.0: the keys' order-preserving images do - negative NaNs
+    # first, -0.0 before +0.0, positive NaNs last -, and descending is that order reversed)
+    bits = a.view(np.uint32)
+    image = np.where(bits >> 31 != 0, ~bits, bits | np.uint32(0x80000000))
+    by_image = np.take_along_axis(a, np.argsort(image, axis=1, kind="stable"), 1)
+    T = Tensor.from_numpy(hip_backend, a)
+    assert np.array_equal(F.sort(T, 1).numpy().view(np.uint32), by_image.view(np.uint32))
+    assert np.array_equal(F.sort(T, 1, True).numpy().view(np.uint32), by_image[:, ::-1].view(np.uint32))
+    b = (normal(292 + n, 700 * n * 6) * 9).astype(np.float32).reshape(700, n, 6)       # innermost runs of 6 rows
+    assert np.array_equal(F.sort(Tensor.from_numpy(hip_backend, b), 1).numpy(), np.sort(b, axis=1, kind="stable"))
