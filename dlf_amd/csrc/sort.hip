@@ -744,7 +744,7 @@ __global__ __launch_bounds__(256) void sort_cols_wave(PassIo<K> io, int64_t rows
     }
 }
 
-// The same for rows of 65 to 64 * ITEMS elements (4-byte keys): a tile of 16 neighbouring rows,
+// The same for rows of 65 to 64 * ITEMS elements (4-byte keys; 8-byte keys with two items): a tile of 16 neighbouring rows,
 // read 16 rows wide (64 bytes a position, where a wavefront per row reads every element of its
 // row from a cache line of its own: fp32 [32, 512, 56, 56] along axis 1 440 us), each wavefront
 // sorts four of them with the network of sort_rows_wave_items (pitch 17: a wavefront's accesses
@@ -846,14 +846,14 @@ int launch_small(hipStream_t stream, const PassIo<K>& io_in, int64_t m, int64_t 
     // kernels do not need and was slower from 129 elements on (317 -> 353 us at 200, 527 -> 609 us at 256) and
     // within 8 % below; eight items a lane lost both ways at 300 elements (222 -> 282 us); a row that fills
     // little of four items a lane - 129 to 160 elements - gains nothing either)
-    const bool tiles = !PAIRS && side_by_side && sizeof(K) == 4 && n > kWave && n <= 4 * kWave && !(n > 2 * kWave && n <= 160) && m >= 4096 &&
-                       io.xmap.dims[io.xmap.rank - 1] >= 16;
+    const bool tiles = !PAIRS && side_by_side && (sizeof(K) == 4 || sizeof(K) == 8) && n > kWave && n <= (sizeof(K) == 4 ? 4 : 2) * kWave &&
+                       !(n > 2 * kWave && n <= 160) && m >= 4096 && io.xmap.dims[io.xmap.rank - 1] >= 16;
     if (side_by_side && n <= kWave && m >= 4096) sort_cols_wave<K, PAIRS><<<dim3(static_cast<unsigned>(ceil_div(m, kWave))), block, 0, stream>>>(io, m, n);
     else if (tiles) {
-        if constexpr (sizeof(K) == 4) {
+        if constexpr (!PAIRS && sizeof(K) >= 4) {
             const dim3 g = grid_for(16);
             if (n <= 2 * kWave) sort_cols_tile<K, PAIRS, 2><<<g, block, 0, stream>>>(io, m, n);
-            else sort_cols_tile<K, PAIRS, 4><<<g, block, 0, stream>>>(io, m, n);
+            else if constexpr (sizeof(K) == 4) sort_cols_tile<K, PAIRS, 4><<<g, block, 0, stream>>>(io, m, n);
         }
     }
     else if (n <= 4) { const dim3 g = grid_for(64); sort_rows_wave<K, PAIRS, 4><<<g, block, 0, stream>>>(io, m, n); }

@@ -784,12 +784,12 @@ def test_short_rows_side_by_side_in_memory(hip_backend, oracle_backend, n):
 @pytest.mark.parametrize("n", [65, 100, 128, 129, 161, 200, 255, 256, 257])
 def test_rows_of_up_to_256_keys_side_by_side_in_memory(hip_backend, oracle_backend, n):
     """sort along an outer axis of 65 to 256 elements with thousands of rows side by side: 4-byte
-    keys pass through LDS in tiles of 16 rows (129 to 160 elements and every argsort keep a
-    wavefront per row).  Both directions, a row count that leaves the last tile ragged, a middle
+    keys (8-byte keys up to 128 elements) pass through LDS in tiles of 16 rows (129 to 160
+    elements and every argsort keep a wavefront per row).  Both directions, a row count that leaves the last tile ragged, a middle
     axis whose innermost run is shorter than a tile, in place, signed zeros and NaNs, a view
     that steps over every other row; the other key widths and argsort beside it."""
     cols = 4099
-    for dtype in (np.float32, np.int32, np.int64, np.float16):
+    for dtype in (np.float32, np.int32, np.int64, np.float64, np.float16):
         x = (normal(290 + n, n * cols) * 50).astype(dtype).reshape(n, cols)
         x[:, 1] = x[0, 1]
         x[: n // 2, 3] = x[n // 2: 2 * (n // 2), 3]
