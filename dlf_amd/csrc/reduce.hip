@@ -236,7 +236,7 @@ struct CountReducer {
 // One row's contiguous elements, visited by `width` cooperating lanes (lane
 // `g` of the group) restricted to 128-bit vectors [v_lo, v_hi) of the aligned
 // body; with_head / with_tail add the unaligned ends of the row.
-template <typename R>
+template <typename R, bool STREAM = true>
 __device__ __forceinline__ typename R::acc_t
 row_partial_contig(const typename R::in_t* __restrict__ p, int64_t n, int g, int width,
                    int64_t part, int64_t parts, typename R::param_t prm, int64_t first_index = 0) {
@@ -245,6 +245,7 @@ row_partial_contig(const typename R::in_t* __restrict__ p, int64_t n, int g, int
     constexpr int V = vec_width<T>();
     using VecT = Vec<T, V>;
 
+    auto fetch = [](const VecT* q) __attribute__((always_inline)) { if constexpr (STREAM) return load_stream(q); else return *q; };
     acc_t acc = R::identity();
     const uintptr_t addr = reinterpret_cast<uintptr_t>(p) / sizeof(T);
     int64_t head = (V - static_cast<int64_t>(addr % V)) % V;
@@ -260,8 +261,8 @@ row_partial_contig(const typename R::in_t* __restrict__ p, int64_t n, int g, int
     int64_t v = v_lo + g;
     // four independent 128-bit loads in flight per lane
     for (; v + 3 * static_cast<int64_t>(width) < v_hi; v += 4 * static_cast<int64_t>(width)) {
-        VecT a = load_stream(&pv[v]), b = load_stream(&pv[v + width]), c = load_stream(&pv[v + 2 * width]),
-             d = load_stream(&pv[v + 3 * width]);
+        VecT a = fetch(&pv[v]), b = fetch(&pv[v + width]), c = fetch(&pv[v + 2 * width]),
+             d = fetch(&pv[v + 3 * width]);
         const int64_t j0 = first_index + head + v * V;
 #pragma unroll
         for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(a.v[e], j0 + e, prm));
@@ -272,11 +273,24 @@ row_partial_contig(const typename R::in_t* __restrict__ p, int64_t n, int g, int
 #pragma unroll
         for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(d.v[e], j0 + 3 * static_cast<int64_t>(width) * V + e, prm));
     }
-    for (; v < v_hi; v += width) {
-        VecT a = load_stream(&pv[v]);
+    // what is left, at most three vectors a lane, again with all loads in flight (rows of a few
+    // vectors a lane - many short rows - consist of little else)
+    if (v < v_hi) {
+        const bool two = v + static_cast<int64_t>(width) < v_hi, three = v + 2 * static_cast<int64_t>(width) < v_hi;
+        VecT a = fetch(&pv[v]), b = a, c = a;
+        if (two) b = fetch(&pv[v + width]);
+        if (three) c = fetch(&pv[v + 2 * width]);
         const int64_t j0 = first_index + head + v * V;
 #pragma unroll
         for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(a.v[e], j0 + e, prm));
+        if (two) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(b.v[e], j0 + static_cast<int64_t>(width) * V + e, prm));
+        }
+        if (three) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) acc = R::join(acc, R::map(c.v[e], j0 + 2 * static_cast<int64_t>(width) * V + e, prm));
+        }
     }
     if (part == 0)
         for (int64_t j = g; j < head; j += width) acc = R::join(acc, R::map(p[j], first_index + j, prm));
@@ -298,7 +312,13 @@ row_partial_strided(const typename R::in_t* __restrict__ p, const DimMap& red, i
 }
 
 // Short rows: 2^log2g lanes per row, 256 >> log2g rows per workgroup.
-template <typename R, bool CONTIG>
+// STREAM: the loads carry the non-temporal hint.  Not where a wavefront's access takes part of a
+// cache line and another access the rest (rows that are not whole lines, or shorter than the 64
+// bytes a lane group reads of each row at a time times a few): the line was then fetched twice -
+// fp32 [2867200, 56] 229 us with the hint, 148 us without, [4194304, 16] 77 against 46 us,
+// [500000, 100] 59 against 34 us; rows of whole lines from 512 bytes on are faster with it
+// (int64 [1048576, 64] 81 against 92 us).
+template <typename R, bool CONTIG, bool STREAM>
 __global__ __launch_bounds__(kBlock) void reduce_rows_group(
     const typename R::in_t* __restrict__ x, DimMap kept, DimMap red, int64_t m, int64_t n, int log2g,
     typename R::out_t* __restrict__ y, DimMap ymap, int final_op, typename R::param_t prm) {
@@ -308,7 +328,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_group(
     typename R::acc_t acc = R::identity();
     if (row < m) {
         const typename R::in_t* p = x + kept.at(row);
-        if constexpr (CONTIG) acc = row_partial_contig<R>(p, n, g, width, 0, 1, prm);
+        if constexpr (CONTIG) acc = row_partial_contig<R, STREAM>(p, n, g, width, 0, 1, prm);
         else acc = row_partial_strided<R>(p, red, n, g, width, 0, 1, prm);
     }
     acc = group_reduce(acc, width, [](typename R::acc_t a, typename R::acc_t b) { return R::join(a, b); });
@@ -336,7 +356,7 @@ __device__ __forceinline__ typename R::acc_t block_reduce(typename R::acc_t acc)
 // (statistics per channel of an NCHW tensor: 32 runs of 3136 elements a row), a group of lanes
 // taking a run at a time with the vector loads of the contiguous case.
 constexpr int kRowStrided = 0, kRowContig = 1, kRowRuns = 2;
-template <typename R, int LAYOUT>
+template <typename R, int LAYOUT, bool STREAM = true>
 __global__ __launch_bounds__(kBlock) void reduce_rows_block(
     const typename R::in_t* __restrict__ x, DimMap kept, DimMap red, int64_t n, int64_t parts,
     typename R::out_t* __restrict__ y, DimMap ymap, int final_op,
@@ -356,8 +376,16 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block(
         // 64 lanes a run from 256 elements, 16 from 64, 4 below
         const int lanes = run >= 256 ? kWave : run >= 64 ? 16 : 4;
         const int64_t groups = kBlock / lanes;
-        for (int64_t r = part * groups + threadIdx.x / lanes; r < runs; r += parts * groups)
-            acc = R::join(acc, row_partial_contig<R>(p + outer.at(r), run, threadIdx.x % lanes, lanes, 0, 1, prm, r * run));
+        // long runs are handed out in pieces of 4096 elements: a few long runs a row (statistics per
+        // channel of [64, 3, 224, 224]: 64 runs of 50176 elements, of [8, 16, 32, 64, 64]: 8 runs of
+        // 131072) would otherwise leave most groups of most of the row's workgroups without work
+        const int64_t piece = run > 8192 ? 4096 : run;
+        const int64_t pieces = (run + piece - 1) / piece;
+        for (int64_t it = part * groups + threadIdx.x / lanes; it < runs * pieces; it += parts * groups) {
+            const int64_t r = it / pieces, at = (it - r * pieces) * piece;
+            const int64_t len = run - at < piece ? run - at : piece;
+            acc = R::join(acc, row_partial_contig<R, STREAM>(p + outer.at(r) + at, len, threadIdx.x % lanes, lanes, 0, 1, prm, r * run + at));
+        }
     } else {
         acc = row_partial_strided<R>(p, red, n, threadIdx.x, kBlock, part, parts, prm);
     }
@@ -463,7 +491,16 @@ __global__ __launch_bounds__(kBlock) void reduce_cols(
             else rows_at_once(std::integral_constant<int, 8>());
             for (; j < hi; j += TY) fold(load_stream(reinterpret_cast<const VecIn*>(&p[j * s])), j);
         } else {
-            for (int64_t j = lo + ty; j < hi; j += TY) fold(*reinterpret_cast<const VecIn*>(&p[red.at(j)]), j);
+            // several reduced dimensions that do not merge (batch and height of an NCHW tensor): four loads in flight
+            int64_t j = lo + ty;
+            for (; j + 3 * TY < hi; j += 4 * TY) {
+                VecIn v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = load_stream(reinterpret_cast<const VecIn*>(&p[red.at(j + u * TY)]));
+#pragma unroll
+                for (int u = 0; u < 4; ++u) fold(v[u], j + u * TY);
+            }
+            for (; j < hi; j += TY) fold(*reinterpret_cast<const VecIn*>(&p[red.at(j)]), j);
         }
     }
 #pragma unroll
@@ -614,6 +651,9 @@ int64_t row_parts(int64_t m, int64_t n) {
     return want < cap ? want : cap;
 }
 
+#ifndef DLFX_REDUCE_SHORT_RUNS
+#define DLFX_REDUCE_SHORT_RUNS 1024
+#endif
 int64_t col_parts(int64_t base_blocks, int64_t n) {
     if (base_blocks >= 1024) return 1;
     int64_t want = ceil_div(2048, base_blocks);
@@ -694,17 +734,25 @@ int launch_reduce(hipStream_t stream, const ReducePlan& pl, const typename R::in
     }
 
     const int64_t short_limit = 8192;
-    if (n <= short_limit) {
+    // rows made of contiguous runs (the innermost reduced dimension has stride 1 and at least 16 elements)
+    const bool runs = !contig && pl.red.rank >= 2 && pl.red.strides[pl.red.rank - 1] == 1 && pl.red.dims[pl.red.rank - 1] >= 16;
+    // (short rows of runs take the long rows' kernel, a workgroup a row, from 1024 elements: element by element
+    // with a division per element - fp32 [32, 512, 56, 56] over {0, 3} - they took 76 us)
+    if (n <= short_limit && !(runs && n >= DLFX_REDUCE_SHORT_RUNS)) {
         const int per_lane = contig ? vec_width<T>() * 4 : 8;
         int log2g = next_pow2_log(ceil_div(n, per_lane));
         if (log2g > 6) log2g = 6;
         const int64_t blocks = ceil_div(m, kBlock >> log2g);
         if (blocks > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
-        if (contig)
-            reduce_rows_group<R, true><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
+        const int64_t row_bytes = n * static_cast<int64_t>(sizeof(T));
+        if (contig && row_bytes >= 512 && row_bytes % 128 == 0)
+            reduce_rows_group<R, true, true><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
+                x, pl.kept, pl.red, m, n, log2g, y, pl.ymap, final_op, prm);
+        else if (contig)
+            reduce_rows_group<R, true, false><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
                 x, pl.kept, pl.red, m, n, log2g, y, pl.ymap, final_op, prm);
         else
-            reduce_rows_group<R, false><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
+            reduce_rows_group<R, false, true><<<dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream>>>(
                 x, pl.kept, pl.red, m, n, log2g, y, pl.ymap, final_op, prm);
         DLFX_CHECK_LAUNCH();
         return DLFX_OK;
@@ -714,10 +762,12 @@ int launch_reduce(hipStream_t stream, const ReducePlan& pl, const typename R::in
     if (m * parts > 0x7fffffffLL) return DLFX_ERR_TOO_LARGE;
     if (parts > 1 && scratch_bytes < static_cast<size_t>(m * parts) * sizeof(acc_t))
         return DLFX_ERR_SCRATCH_TOO_SMALL;
-    // rows made of contiguous runs (the innermost reduced dimension has stride 1 and at least 16 elements)
-    const bool runs = !contig && pl.red.rank >= 2 && pl.red.strides[pl.red.rank - 1] == 1 && pl.red.dims[pl.red.rank - 1] >= 16;
     if (contig)
         reduce_rows_block<R, kRowContig><<<dim3(static_cast<unsigned>(m * parts)), dim3(kBlock), 0, stream>>>(
+            x, pl.kept, pl.red, n, parts, y, pl.ymap, final_op, partial, prm);
+    else if (runs && (pl.red.dims[pl.red.rank - 1] * static_cast<int64_t>(sizeof(T)) < 512 || pl.red.dims[pl.red.rank - 1] * static_cast<int64_t>(sizeof(T)) % 128 != 0))
+        // (runs that are not whole cache lines: without the non-temporal hint, as in reduce_rows_group)
+        reduce_rows_block<R, kRowRuns, false><<<dim3(static_cast<unsigned>(m * parts)), dim3(kBlock), 0, stream>>>(
             x, pl.kept, pl.red, n, parts, y, pl.ymap, final_op, partial, prm);
     else if (runs)
         reduce_rows_block<R, kRowRuns><<<dim3(static_cast<unsigned>(m * parts)), dim3(kBlock), 0, stream>>>(

@@ -211,10 +211,14 @@ def test_int64_mean_of_many_short_rows_truncates_exactly(hip_backend, oracle_bac
 
 
 @pytest.mark.parametrize("shape,axes", [((6, 40, 70, 65), [0, 2, 3]), ((5, 64, 9, 300, 20), [0, 2, 4]), ((3, 7, 4000, 17), [0, 2, 3]),
-                                        ((2, 3, 40, 50, 20), [0, 2, 4]), ((20, 96, 56, 56), [0, 2, 3])])
+                                        ((2, 3, 40, 50, 20), [0, 2, 4]), ((20, 96, 56, 56), [0, 2, 3]), ((9, 3, 150, 151), [0, 2, 3]),
+                                        ((3, 5, 20001), [0, 2]), ((2, 16, 8, 64, 64), [0, 2, 3, 4]), ((32, 7, 9, 56), [0, 3]),
+                                        ((6, 50, 4, 128), [0, 3]), ((5, 33, 64, 16), [0, 2, 3])])
 def test_long_rows_made_of_contiguous_runs(hip_backend, oracle_backend, shape, axes):
-    # rows longer than 8192 elements whose reduced dimensions end in a contiguous one (statistics
-    # per channel of an NCHW tensor): read run by run; runs of 4550, 20, 68000, 20 and 3136 elements
+    # rows whose reduced dimensions end in a contiguous one (statistics per channel of an NCHW tensor): read
+    # run by run; runs of 4550, 20, 68000, 20 and 3136 elements; then a few long runs a row, handed out in
+    # pieces of 4096 elements (22650, 20001 and 32768 elements, the middle one off every boundary), and rows
+    # of 1024 to 8192 elements made of runs (56, 128 and 1024 elements: whole cache lines or not)
     x = randint(190, int(np.prod(shape)), -100, 100).astype(np.int32).reshape(shape)
     Xh = Tensor.from_numpy(hip_backend, x)
     for name, fn in (("reduce_sum", np.sum), ("reduce_max", np.max), ("reduce_min", np.min)):
@@ -246,3 +250,25 @@ def test_short_axis_beside_many_columns_one_lane_per_column(hip_backend, oracle_
         check_float_reduce(name, Yh, Yo, [axis])
     sl = Xh.slice([0], [shape[-1] - 1], [len(shape) - 1], [2])            # every other innermost element: the general kernels
     assert np.array_equal(F.reduce("reduce_sum", sl, [axis]).numpy(), x[..., 0:shape[-1] - 1:2].sum(axis=axis, dtype=np.int32))
+
+
+@pytest.mark.parametrize("shape", [(40000, 56), (30000, 100), (100000, 7), (20000, 64), (70000, 16), (3000, 200), (9000, 31)])
+def test_many_short_rows_whole_cache_lines_or_not(hip_backend, oracle_backend, shape):
+    # rows of a few hundred bytes: a group of lanes a row; rows that are whole cache lines (from 512 bytes) are
+    # loaded with the non-temporal hint, the others without - both for every element type here
+    for dtype in (np.int32, np.int64, np.float16):
+        x = randint(196, int(np.prod(shape)), -20, 20).astype(dtype).reshape(shape)
+        Xh = Tensor.from_numpy(hip_backend, x)
+        if dtype != np.float16:
+            assert np.array_equal(F.reduce("reduce_sum", Xh, [1]).numpy(), x.sum(axis=1, dtype=dtype))
+            assert np.array_equal(F.count(Xh, dtype(3), (1,)).numpy(), (x == 3).sum(axis=1))
+        assert np.array_equal(F.reduce("reduce_max", Xh, [1]).numpy(), x.max(axis=1))
+        assert np.array_equal(F.reduce("reduce_min", Xh, [1], True).numpy(), x.min(axis=1, keepdims=True))
+        assert np.array_equal(F.argmax(Xh, 1, False).numpy(), np.argmax(x, axis=1))
+        assert np.array_equal(F.argmin(Xh, 1, False).numpy(), np.argmin(x, axis=1))
+        V = Xh.slice([1], [shape[1]], [1])                              # rows that start off every boundary
+        assert np.array_equal(F.reduce("reduce_max", V, [1]).numpy(), x[:, 1:].max(axis=1))
+    y = (normal(197, int(np.prod(shape))) * 2).astype(np.float32).reshape(shape)
+    Yh, Yo = both(hip_backend, oracle_backend, y)
+    for name in ("reduce_sum", "reduce_mean", "reduce_log_sum_exp", "reduce_nrm2"):
+        check_float_reduce(name, Yh, Yo, [1])
