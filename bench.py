@@ -310,11 +310,16 @@ def make_ops(be, which):
             def v(call=call):
                 call()
             return v
+
+        def enough(shape, dtype):
+            # copies to rotate through: a working set of 1.3 GB, so that the 256 MB cache in front of HBM holds none of them
+            size = int(np.prod(shape)) * torch.empty((), dtype=dtype).element_size()
+            return max(2, min(12, -(-1300000000 // size)))
         # scans and reductions along an axis that is not the innermost
         for shape, axis, what in (((262144, 64), 0, "few columns: the axis cut into segments"), ((4194304, 16), 0, "few columns: the axis cut into segments"),
                                   ((16384, 1000), 0, "the axis cut into segments"), ((8, 21, 512, 512), 1, "a short axis: a lane per column"),
                                   ((64, 3, 224, 224), 1, "a short axis: a lane per column")):
-            xs = gen(shape, torch.float32, lambda c: synth.normal(50 + 100 * c), 2)
+            xs = gen(shape, torch.float32, lambda c: synth.normal(50 + 100 * c), enough(shape, torch.float32))
             text = "_f32_[%s]" % ",".join(str(e) for e in shape)
             count = int(np.prod(shape))
             calls, _ = scan_calls(xs, axis)
@@ -322,17 +327,22 @@ def make_ops(be, which):
             calls, _ = argmax_calls(xs, axis)
             ops.append(Op("B1", "argmax{%d}%s" % (axis, text), count, 4 * count, calls, timed_only(calls[0])))
         # statistics per channel: rows made of contiguous runs
-        xs = gen((32, 512, 56, 56), torch.float32, lambda c: synth.normal(51 + 100 * c), 2)
+        xs = gen((32, 512, 56, 56), torch.float32, lambda c: synth.normal(51 + 100 * c), enough((32, 512, 56, 56), torch.float32))
         calls, _ = reduce_calls("reduce_sum", xs, [0, 2, 3])
         ops.append(Op("B2", "reduce_sum{0,2,3}_f32_[32,512,56,56]", 32 * 512 * 3136, 4 * 32 * 512 * 3136, calls, timed_only(calls[0])))
+        # many short rows that are not whole cache lines; rows of a few long runs; rows of 1024 to 8192 elements made of runs
+        for shape, axes in (((2867200, 56), [1]), ((4194304, 16), [1]), ((8, 16, 32, 64, 64), [0, 2, 3, 4]), ((16, 64, 128, 128), [1, 3]), ((32, 512, 56, 56), [3])):
+            xs = gen(shape, torch.float32, lambda c: synth.normal(56 + 100 * c), enough(shape, torch.float32))
+            calls, _ = reduce_calls("reduce_sum", xs, axes)
+            ops.append(Op("B2", "reduce_sum{%s}_f32_[%s]" % (",".join(str(a) for a in axes), ",".join(str(e) for e in shape)), int(np.prod(shape)), 4 * int(np.prod(shape)), calls, timed_only(calls[0])))
         # long rows near the end of the bucket route (bins packed bucket by bucket), doubles with the gap closed
         for shape, dtype, text in (((16, 2300000), torch.float32, "f32_normal_[16,2300000]"), ((16, 2400000), torch.float32, "f32_normal_[16,2400000]"),
                                    ((3355, 10000), torch.float64, "f64_normal_[3355,10000]")):
-            xs = gen(shape, dtype, lambda c: synth.normal(52 + 100 * c), 2)
+            xs = gen(shape, dtype, lambda c: synth.normal(52 + 100 * c), enough(shape, dtype))
             ops += [op for op in sort_ops(be, tensor, xs, "B3", text) if "_asc_" in op.name]
         # half elements along an axis that is not the innermost: two neighbouring columns a lane
         for shape, axis in (((32, 512, 56, 56), 1), ((64, 1 << 20), 0), ((8, 21, 512, 512), 1)):
-            xs = gen(shape, torch.float16, lambda c: synth.normal(54 + 100 * c), 2)
+            xs = gen(shape, torch.float16, lambda c: synth.normal(54 + 100 * c), enough(shape, torch.float16))
             text = "_f16_[%s]" % ",".join(str(e) for e in shape)
             count = int(np.prod(shape))
             calls, _ = scan_calls(xs, axis)
@@ -343,7 +353,7 @@ def make_ops(be, which):
             ops.append(Op("B5", "argmax{%d}%s" % (axis, text), count, 2 * count, calls, timed_only(calls[0])))
         # top_k along an axis that is not the innermost (register lists, a lane per column)
         for shape, axis in (((32, 512, 56, 56), 1), ((16, 80, 160, 160), 1)):
-            xs = gen(shape, torch.float32, lambda c: synth.normal(55 + 100 * c), 2)
+            xs = gen(shape, torch.float32, lambda c: synth.normal(55 + 100 * c), enough(shape, torch.float32))
             count = int(np.prod(shape))
             for k in (1, 5):
                 out_dims = [k if i == axis else e for i, e in enumerate(shape)]
@@ -357,7 +367,7 @@ def make_ops(be, which):
                 ops.append(Op("B6", "top_k%d{%d}_f32_[%s]" % (k, axis, ",".join(str(e) for e in shape)), count, 4 * count, calls, timed_only(calls[0])))
         # top_k of very long rows
         for rows_l, n_l in ((1, 1 << 24), (1, 1 << 23)):
-            xl_ = gen((rows_l, n_l), torch.float32, lambda c: synth.normal(53 + 100 * c), 2)
+            xl_ = gen((rows_l, n_l), torch.float32, lambda c: synth.normal(53 + 100 * c), enough((rows_l, n_l), torch.float32))
             ops += topk_ops(be, tensor, xl_, (256, 257), "B4", "[%d,2^%d]" % (rows_l, n_l.bit_length() - 1))
 
     # ---------------- C5: strided NCHW
