@@ -940,7 +940,7 @@ __global__ __launch_bounds__(256) void topk_rows_thread(TopkIo<typename BitsOf<E
 #pragma unroll
             for (int t = 0; t < C; ++t) {
                 const int f = t * kWave + lane;
-                in[t] = (t < n32 && f < run) ? load_stream(io.x + row0 * row_pitch + f) : S(0);
+                in[t] = (t < n32 && f < run) ? io.x[row0 * row_pitch + f] : S(0);
             }
 #pragma unroll
             for (int t = 0; t < C; ++t) {
@@ -953,7 +953,9 @@ __global__ __launch_bounds__(256) void topk_rows_thread(TopkIo<typename BitsOf<E
             for (int t = 0; t < C; ++t) {
                 const int r = 2 * t + half;
                 const bool ok = row0 + r < rows && c0 + col < n32;
-                in[t] = ok ? load_stream(io.x + (row0 + r) * row_pitch + (c0 + col)) : S(0);
+                // (no non-temporal hint: pieces of rows that are not whole cache lines share lines, and a line two
+                // such loads share is fetched twice - fp32 [500000, 200], limit 1: 117 us with the hint, 107 without)
+                in[t] = ok ? io.x[(row0 + r) * row_pitch + (c0 + col)] : S(0);
             }
 #pragma unroll
             for (int t = 0; t < C; ++t) mine[(2 * t + half) * (C + 1) + col] = in[t];
