@@ -491,16 +491,27 @@ __global__ __launch_bounds__(kBlock) void reduce_cols(
             else rows_at_once(std::integral_constant<int, 8>());
             for (; j < hi; j += TY) fold(load_stream(reinterpret_cast<const VecIn*>(&p[j * s])), j);
         } else {
-            // several reduced dimensions that do not merge (batch and height of an NCHW tensor): four loads in flight
+            // several reduced dimensions that do not merge (batch and height of an NCHW tensor): eight loads in
+            // flight; two dimensions of fewer than 2^32 elements are told apart with one 32-bit division
+            const bool two = red.rank == 2 && n <= 0xffffffffLL;
+            const uint32_t inner = static_cast<uint32_t>(red.dims[1]);
+            auto where = [&](int64_t j) __attribute__((always_inline)) -> int64_t {
+                if (two) {
+                    const uint32_t q = static_cast<uint32_t>(j) / inner, r = static_cast<uint32_t>(j) - q * inner;
+                    return static_cast<int64_t>(q) * red.strides[0] + static_cast<int64_t>(r) * red.strides[1];
+                }
+                return red.at(j);
+            };
+            constexpr int U = 8;
             int64_t j = lo + ty;
-            for (; j + 3 * TY < hi; j += 4 * TY) {
-                VecIn v[4];
+            for (; j + (U - 1) * TY < hi; j += U * TY) {
+                VecIn v[U];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) v[u] = load_stream(reinterpret_cast<const VecIn*>(&p[red.at(j + u * TY)]));
+                for (int u = 0; u < U; ++u) v[u] = load_stream(reinterpret_cast<const VecIn*>(&p[where(j + u * TY)]));
 #pragma unroll
-                for (int u = 0; u < 4; ++u) fold(v[u], j + u * TY);
+                for (int u = 0; u < U; ++u) fold(v[u], j + u * TY);
             }
-            for (; j < hi; j += TY) fold(*reinterpret_cast<const VecIn*>(&p[red.at(j)]), j);
+            for (; j < hi; j += TY) fold(*reinterpret_cast<const VecIn*>(&p[where(j)]), j);
         }
     }
 #pragma unroll
@@ -687,7 +698,8 @@ int launch_reduce(hipStream_t stream, const ReducePlan& pl, const typename R::in
         outer.dims[outer.rank] = 1;
         outer.strides[outer.rank] = 0;
         // two-byte elements: two neighbouring columns a lane where every pair starts on a 4-byte boundary
-        bool pairs = sizeof(T) == 2 && !std::is_class<T>::value && L % 2 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0;
+        // (from 128 columns on: fewer leave half the lanes of the one block of columns without work)
+        bool pairs = sizeof(T) == 2 && !std::is_class<T>::value && L % 2 == 0 && L >= 128 && reinterpret_cast<uintptr_t>(x) % 4 == 0;
         for (int i = 0; pairs && i < outer.rank; ++i) pairs = outer.strides[i] % 2 == 0;
         for (int i = 0; pairs && i < pl.red.rank; ++i) pairs = pl.red.strides[i] % 2 == 0;
         auto with_cols = [&](auto&& launch) {
