@@ -307,7 +307,25 @@ row_partial_strided(const typename R::in_t* __restrict__ p, const DimMap& red, i
     const int64_t per = (n + parts - 1) / parts;
     const int64_t lo = part * per;
     const int64_t hi = (lo + per < n) ? lo + per : n;
-    for (int64_t j = lo + g; j < hi; j += width) acc = R::join(acc, R::map(p[red.at(j)], j, prm));
+    // (two dimensions of fewer than 2^32 elements are told apart with one 32-bit division; four loads in flight)
+    const bool two = red.rank == 2 && n <= 0xffffffffLL;
+    const uint32_t inner = static_cast<uint32_t>(red.rank == 2 ? red.dims[1] : 1);
+    auto where = [&](int64_t j) __attribute__((always_inline)) -> int64_t {
+        if (two) {
+            const uint32_t q = static_cast<uint32_t>(j) / inner, r = static_cast<uint32_t>(j) - q * inner;
+            return static_cast<int64_t>(q) * red.strides[0] + static_cast<int64_t>(r) * red.strides[1];
+        }
+        return red.at(j);
+    };
+    int64_t j = lo + g;
+    for (; j + 3 * static_cast<int64_t>(width) < hi; j += 4 * static_cast<int64_t>(width)) {
+        typename R::in_t v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = p[where(j + u * static_cast<int64_t>(width))];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc = R::join(acc, R::map(v[u], j + u * static_cast<int64_t>(width), prm));
+    }
+    for (; j < hi; j += width) acc = R::join(acc, R::map(p[where(j)], j, prm));
     return acc;
 }
 
@@ -662,6 +680,12 @@ int64_t row_parts(int64_t m, int64_t n) {
     return want < cap ? want : cap;
 }
 
+#ifndef DLFX_REDUCE_COLS_MIN_RUN
+#define DLFX_REDUCE_COLS_MIN_RUN 48
+#endif
+#ifndef DLFX_REDUCE_COLS_SHORT_AXIS
+#define DLFX_REDUCE_COLS_SHORT_AXIS 8
+#endif
 #ifndef DLFX_REDUCE_SHORT_RUNS
 #define DLFX_REDUCE_SHORT_RUNS 1024
 #endif
@@ -689,7 +713,10 @@ int launch_reduce(hipStream_t stream, const ReducePlan& pl, const typename R::in
 
     const bool contig = pl.red.rank == 0 || (pl.red.rank == 1 && pl.red.strides[0] == 1);
     const bool cols = !contig && pl.kept.rank >= 1 && pl.kept.strides[pl.kept.rank - 1] == 1 &&
-                      pl.kept.dims[pl.kept.rank - 1] >= 16;
+                      pl.kept.dims[pl.kept.rank - 1] >= 16 &&
+                      // (a short run of columns beside a short reduced axis: a lane a row keeps the lanes busy, where a
+                      // block of 64 columns a workgroup leaves most of them idle - fp32 [4096, 50, 3, 17] over axis 2: 78 us)
+                      (pl.kept.dims[pl.kept.rank - 1] >= DLFX_REDUCE_COLS_MIN_RUN || n > DLFX_REDUCE_COLS_SHORT_AXIS);
 
     if (cols) {
         DimMap outer = pl.kept;

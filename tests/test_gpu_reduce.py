@@ -232,10 +232,12 @@ def test_long_rows_made_of_contiguous_runs(hip_backend, oracle_backend, shape, a
 
 
 @pytest.mark.parametrize("shape,axis", [((8, 21, 64, 64), 1), ((64, 3, 50, 50), 1), ((5000, 2, 3), 1), ((3, 32, 5000), 1), ((2, 33, 5000), 1),
-                                        ((17, 8000), 0), ((4, 5, 6, 700), 2)])
+                                        ((17, 8000), 0), ((4, 5, 6, 700), 2),
+                                        ((600, 50, 3, 17), 2), ((9000, 8, 20), 1), ((20000, 4, 16), 1), ((9000, 9, 20), 1), ((3000, 8, 47), 1), ((3000, 8, 48), 1)])
 def test_short_axis_beside_many_columns_one_lane_per_column(hip_backend, oracle_backend, shape, axis):
     # a reduced axis of up to 32 elements that is not the innermost, beside thousands of columns: a lane
-    # reduces a column on its own (33 elements: the kernel of four wavefronts per 64 columns)
+    # reduces a column on its own (33 elements: the kernel of four wavefronts per 64 columns); beside runs of
+    # fewer than 48 columns an axis of up to 8 elements goes a lane a row through the strided-row kernel instead
     x = randint(192, int(np.prod(shape)), -9, 9).astype(np.int32).reshape(shape)       # ties: the first extremum counts
     Xh = Tensor.from_numpy(hip_backend, x)
     assert np.array_equal(F.reduce("reduce_sum", Xh, [axis]).numpy(), x.sum(axis=axis, dtype=np.int32))
